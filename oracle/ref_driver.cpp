@@ -1,0 +1,470 @@
+// TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+// C-ABI driver over the reference's own CPU backend (compiled from the reference sources by
+// oracle/Makefile into oracle/_ref/libodl_ref.so). It only *calls* the reference's public
+// Tensor/Operator/Mat API — no algorithm is restated here — so that tests can check the plain-C
+// oracle against the real thing bit for bit, tests/golden/make_golden.py can write fixtures, and
+// the benchmark can time the reference CPU path beside the GPU.
+// Every entry point returns 0, or -1 for std::invalid_argument, -2 for any other std::exception.
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <vector>
+
+#include "origin/core/operator.h"
+#include "origin/core/parameter.h"
+#include "origin/core/tensor.h"
+#include "origin/mat/origin/origin_mat.h"
+#include "origin/nn/layers/conv2d.h"
+#include "origin/nn/layers/flatten.h"
+#include "origin/nn/layers/linear.h"
+#include "origin/nn/layers/max_pool2d.h"
+#include "origin/nn/layers/relu.h"
+#include "origin/nn/sequential.h"
+#include "origin/operators/activation/relu.h"
+#include "origin/operators/activation/softmax.h"
+#include "origin/operators/conv/conv2d.h"
+#include "origin/operators/loss/softmax_cross_entropy.h"
+#include "origin/operators/math/add.h"
+#include "origin/operators/math/broadcast_to.h"
+#include "origin/operators/math/compare.h"
+#include "origin/operators/math/div.h"
+#include "origin/operators/math/exp.h"
+#include "origin/operators/math/log.h"
+#include "origin/operators/math/mat_mul.h"
+#include "origin/operators/math/mul.h"
+#include "origin/operators/math/neg.h"
+#include "origin/operators/math/pow.h"
+#include "origin/operators/math/square.h"
+#include "origin/operators/math/sub.h"
+#include "origin/operators/math/sum.h"
+#include "origin/operators/math/sum_to.h"
+#include "origin/operators/pooling/max_pool2d.h"
+#include "origin/optim/adam.h"
+#include "origin/optim/hooks.h"
+#include "origin/optim/sgd.h"
+#include "origin/utils/metrics.h"
+
+using namespace origin;
+namespace F = origin::functional;
+
+namespace
+{
+Shape make_shape(const int64_t *dims, int n)
+{
+    std::vector<size_t> d(dims, dims + n);
+    return Shape(d);
+}
+
+Tensor f32(const float *p, const Shape &s, bool grad = false)
+{
+    std::vector<float> v(p, p + s.elements());
+    return Tensor(v, s, dtype(DataType::kFloat32).requires_grad(grad));
+}
+
+Tensor labels(const void *p, int is64, int64_t n)
+{
+    if (is64)
+    {
+        std::vector<int64_t> v((const int64_t *)p, (const int64_t *)p + n);
+        return Tensor(v, Shape{(size_t)n}, dtype(DataType::kInt64));
+    }
+    std::vector<int32_t> v((const int32_t *)p, (const int32_t *)p + n);
+    return Tensor(v, Shape{(size_t)n}, dtype(DataType::kInt32));
+}
+
+std::unique_ptr<origin::Mat> mat_f32(const float *p, const Shape &s)
+{
+    return OriginMat::from_memory(p, DataType::kFloat32, s, TensorOptions(DataType::kFloat32));
+}
+
+std::unique_ptr<origin::Mat> mat_labels(const void *p, int is64, int64_t n)
+{
+    return OriginMat::from_memory(p, is64 ? DataType::kInt64 : DataType::kInt32, Shape{(size_t)n},
+                                  TensorOptions(is64 ? DataType::kInt64 : DataType::kInt32));
+}
+
+void out(const Tensor &t, float *dst)
+{
+    auto v = t.to_vector<float>();
+    std::memcpy(dst, v.data(), v.size() * sizeof(float));
+}
+
+void out(const origin::Mat &m, float *dst)
+{
+    auto v = static_cast<const OriginMat &>(m).to_vector<float>();
+    std::memcpy(dst, v.data(), v.size() * sizeof(float));
+}
+
+template <typename Fn>
+int guarded(Fn &&fn)
+{
+    try
+    {
+        fn();
+        return 0;
+    }
+    catch (const std::invalid_argument &)
+    {
+        return -1;
+    }
+    catch (const std::exception &)
+    {
+        return -2;
+    }
+}
+}  // namespace
+
+extern "C" {
+
+int odl_ref_ping()
+{
+    return 1;
+}
+
+int odl_ref_matmul(const float *a, const float *b, float *c, int64_t m, int64_t n, int64_t k)
+{
+    return guarded([&] {
+        auto y = F::mat_mul(f32(a, Shape{(size_t)m, (size_t)k}), f32(b, Shape{(size_t)k, (size_t)n}));
+        out(y, c);
+    });
+}
+
+int odl_ref_matmul_batched(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t n, int64_t k,
+                           int b_is_batched)
+{
+    return guarded([&] {
+        auto A = f32(a, Shape{(size_t)batch, (size_t)m, (size_t)k});
+        auto B = b_is_batched ? f32(b, Shape{(size_t)batch, (size_t)k, (size_t)n}) : f32(b, Shape{(size_t)k, (size_t)n});
+        out(F::mat_mul(A, B), c);
+    });
+}
+
+// forward + backward with an injected upstream gradient: z = y * dC; z.backward() seeds ones.
+int odl_ref_matmul_fwd_bwd(const float *x, const float *w, const float *gy, float *y, float *gx, float *gw, int64_t m,
+                           int64_t k, int64_t n)
+{
+    return guarded([&] {
+        auto X = f32(x, Shape{(size_t)m, (size_t)k}, true);
+        auto W = f32(w, Shape{(size_t)k, (size_t)n}, true);
+        auto G = f32(gy, Shape{(size_t)m, (size_t)n});
+        auto Y = F::mat_mul(X, W);
+        auto Z = Y * G;
+        Z.backward();
+        out(Y, y);
+        out(X.grad(), gx);
+        out(W.grad(), gw);
+    });
+}
+
+int odl_ref_transpose(const float *src, float *dst, const int64_t *shape, int nd)
+{
+    return guarded([&] { out(f32(src, make_shape(shape, nd)).transpose(), dst); });
+}
+
+int odl_ref_im2col(const float *img, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
+                   int PW, int to_matrix, float *col)
+{
+    return guarded([&] {
+        auto m = mat_f32(img, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
+        out(*m->im2col({KH, KW}, {SH, SW}, {PH, PW}, to_matrix != 0), col);
+    });
+}
+
+int odl_ref_col2im(const float *col, const int64_t *col_shape, int col_nd, int64_t N, int64_t C, int64_t H, int64_t W,
+                   int KH, int KW, int SH, int SW, int PH, int PW, int to_matrix, float *img)
+{
+    return guarded([&] {
+        auto m = mat_f32(col, make_shape(col_shape, col_nd));
+        out(*m->col2im(Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W}, {KH, KW}, {SH, SW}, {PH, PW}, to_matrix != 0),
+            img);
+    });
+}
+
+int odl_ref_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                   int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *y)
+{
+    return guarded([&] {
+        auto X  = f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
+        auto Wt = f32(w, Shape{(size_t)OC, (size_t)C, (size_t)KH, (size_t)KW});
+        Tensor B;
+        if (b)
+            B = f32(b, Shape{(size_t)OC});
+        out(F::conv2d(X, Wt, b ? &B : nullptr, {SH, SW}, {PH, PW}), y);
+    });
+}
+
+// full operator path: y = conv2d(x, W, b); (y * gy).backward()
+int odl_ref_conv2d_backward(const float *gy, const float *x, const float *w, const float *b, int64_t N, int64_t C,
+                            int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *gx,
+                            float *gw, float *gb)
+{
+    return guarded([&] {
+        auto X  = f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W}, true);
+        auto Wt = f32(w, Shape{(size_t)OC, (size_t)C, (size_t)KH, (size_t)KW}, true);
+        Tensor B;
+        if (b)
+            B = f32(b, Shape{(size_t)OC}, true);
+        auto Y = F::conv2d(X, Wt, b ? &B : nullptr, {SH, SW}, {PH, PW});
+        auto G = f32(gy, Y.shape());
+        auto Z = Y * G;
+        Z.backward();
+        out(X.grad(), gx);
+        out(Wt.grad(), gw);
+        if (b && gb)
+            out(B.grad(), gb);
+    });
+}
+
+int odl_ref_sum(const float *src, const int64_t *shape, int nd, int axis, int keepdim, float *dst)
+{
+    return guarded([&] { out(F::sum(f32(src, make_shape(shape, nd)), axis, keepdim != 0), dst); });
+}
+
+int odl_ref_max(const float *src, const int64_t *shape, int nd, int axis, float *dst)
+{
+    return guarded([&] { out(*mat_f32(src, make_shape(shape, nd))->max(axis), dst); });
+}
+
+int odl_ref_sum_to(const float *src, const int64_t *sshape, int sn, const int64_t *tshape, int tn, float *dst)
+{
+    return guarded([&] { out(F::sum_to(f32(src, make_shape(sshape, sn)), make_shape(tshape, tn)), dst); });
+}
+
+int odl_ref_broadcast_to(const float *src, const int64_t *sshape, int sn, const int64_t *dshape, int dn, float *dst)
+{
+    return guarded([&] { out(F::broadcast_to(f32(src, make_shape(sshape, sn)), make_shape(dshape, dn)), dst); });
+}
+
+// backward of broadcast_to with upstream gradient g (left-aligned sum_to inside the reference)
+int odl_ref_broadcast_to_backward(const float *src, const int64_t *sshape, int sn, const int64_t *dshape, int dn,
+                                  const float *g, float *gsrc)
+{
+    return guarded([&] {
+        auto X = f32(src, make_shape(sshape, sn), true);
+        auto Y = F::broadcast_to(X, make_shape(dshape, dn));
+        auto Z = Y * f32(g, make_shape(dshape, dn));
+        Z.backward();
+        out(X.grad(), gsrc);
+    });
+}
+
+int odl_ref_softmax(const float *x, const int64_t *shape, int nd, int axis, float *y)
+{
+    return guarded([&] { out(F::softmax(f32(x, make_shape(shape, nd)), axis), y); });
+}
+
+int odl_ref_gather(const float *in, const void *idx, int is64, int64_t N, int64_t C, float *o)
+{
+    return guarded([&] {
+        auto m = mat_f32(in, Shape{(size_t)N, (size_t)C});
+        out(*m->gather(*mat_labels(idx, is64, N)), o);
+    });
+}
+
+int odl_ref_one_hot(const void *idx, int is64, int64_t N, int64_t C, float *o)
+{
+    return guarded([&] {
+        auto t = mat_labels(idx, is64, N);
+        out(*t->one_hot(*t, (int)C), o);
+    });
+}
+
+int odl_ref_softmax_ce(const float *x, const void *t, int is64, int64_t N, int64_t C, float *loss, float *gx)
+{
+    return guarded([&] {
+        auto X = f32(x, Shape{(size_t)N, (size_t)C}, true);
+        auto T = labels(t, is64, N);
+        auto L = F::softmax_cross_entropy(X, T);
+        *loss  = L.item<float>();
+        if (gx)
+        {
+            L.backward();
+            out(X.grad(), gx);
+        }
+    });
+}
+
+int odl_ref_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+                       int PH, int PW, float *y, uint64_t *idx)
+{
+    return guarded([&] {
+        auto m = mat_f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
+        std::vector<size_t> ind;
+        out(*m->max_pool2d({KH, KW}, {SH, SW}, {PH, PW}, &ind), y);
+        for (size_t i = 0; i < ind.size(); ++i)
+            idx[i] = ind[i];
+    });
+}
+
+int odl_ref_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N, int64_t C, int64_t H, int64_t W,
+                                int KH, int KW, int SH, int SW, int PH, int PW, float *gx)
+{
+    return guarded([&] {
+        int OH = (int)((H + 2 * PH - KH) / SH + 1), OW = (int)((W + 2 * PW - KW) / SW + 1);
+        std::vector<float> zeros((size_t)(N * C * H * W), 0.0f);
+        auto xm = mat_f32(zeros.data(), Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
+        auto gm = mat_f32(gy, Shape{(size_t)N, (size_t)C, (size_t)OH, (size_t)OW});
+        std::vector<size_t> ind(idx, idx + (size_t)(N * C * OH * OW));
+        out(*xm->max_pool2d_backward(*gm, {KH, KW}, {SH, SW}, {PH, PW}, ind), gx);
+    });
+}
+
+int odl_ref_accuracy(const float *y, const int32_t *t, int64_t N, int64_t C, float *acc)
+{
+    return guarded([&] {
+        std::vector<int32_t> tv(t, t + N);
+        auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt32));
+        *acc   = accuracy(f32(y, Shape{(size_t)N, (size_t)C}), T).item<float>();
+    });
+}
+
+// op: 0 add 1 sub 2 mul 3 div 4 gt
+int odl_ref_binary(int op, const float *a, const int64_t *ashape, int an, const float *b, const int64_t *bshape, int bn,
+                   float *o)
+{
+    return guarded([&] {
+        auto A = f32(a, make_shape(ashape, an));
+        auto B = f32(b, make_shape(bshape, bn));
+        Tensor R;
+        switch (op)
+        {
+            case 0: R = A + B; break;
+            case 1: R = A - B; break;
+            case 2: R = A * B; break;
+            case 3: R = A / B; break;
+            default: R = A > B; break;
+        }
+        out(R, o);
+    });
+}
+
+// op: 0 relu 1 exp 2 log 3 neg 4 square
+int odl_ref_unary(int op, const float *a, int64_t n, float *o)
+{
+    return guarded([&] {
+        auto A = f32(a, Shape{(size_t)n});
+        Tensor R;
+        switch (op)
+        {
+            case 0: R = F::relu(A); break;
+            case 1: R = F::exp(A); break;
+            case 2: R = F::log(A); break;
+            case 3: R = -A; break;
+            default: R = F::square(A); break;
+        }
+        out(R, o);
+    });
+}
+
+int odl_ref_pow_scalar(const float *a, int64_t n, float e, float *o)
+{
+    return guarded([&] { out(F::pow(f32(a, Shape{(size_t)n}), Scalar(e)), o); });
+}
+
+// MLP D -> Hd -> C (Linear, ReLU, Linear), softmax CE, WeightDecay hook, Adam; `steps` steps on the same batch.
+// Parameters are read and written in place; loss/grads/logits of the LAST step are returned.
+int odl_ref_mlp_train(const float *x, const void *t, int is64, int64_t N, int64_t D, int64_t Hd, int64_t C, float *W1,
+                      float *b1, float *W2, float *b2, int steps, float lr, float beta1, float beta2, float eps,
+                      float wd, float *loss, float *gW1, float *gb1, float *gW2, float *gb2, float *logits)
+{
+    return guarded([&] {
+        Sequential model;
+        model.add(std::make_unique<nn::Linear>((int)D, (int)Hd, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::Linear>((int)Hd, (int)C, true));
+        auto &l1 = dynamic_cast<nn::Linear &>(model[0]);
+        auto &l2 = dynamic_cast<nn::Linear &>(model[2]);
+        Adam opt(model, lr, beta1, beta2, eps);
+        if (wd != 0.0f)
+            opt.register_hook(WeightDecay(wd).hook());
+        *l1.weight() = Parameter(f32(W1, Shape{(size_t)D, (size_t)Hd}, true));
+        *l1.bias()   = Parameter(f32(b1, Shape{1, (size_t)Hd}, true));
+        *l2.weight() = Parameter(f32(W2, Shape{(size_t)Hd, (size_t)C}, true));
+        *l2.bias()   = Parameter(f32(b2, Shape{1, (size_t)C}, true));
+        auto X = f32(x, Shape{(size_t)N, (size_t)D});
+        auto T = labels(t, is64, N);
+        model.train();
+        for (int s = 0; s < steps; ++s)
+        {
+            opt.zero_grad();
+            auto y = model(X);
+            auto L = F::softmax_cross_entropy(y, T);
+            L.backward();
+            *loss = L.item<float>();
+            out(y, logits);
+            out(l1.weight()->grad(), gW1);
+            out(l1.bias()->grad(), gb1);
+            out(l2.weight()->grad(), gW2);
+            out(l2.bias()->grad(), gb2);
+            opt.step();
+        }
+        out(*l1.weight(), W1);
+        out(*l1.bias(), b1);
+        out(*l2.weight(), W2);
+        out(*l2.bias(), b2);
+    });
+}
+
+// CNN of BASELINE config 4 (no BatchNorm), SGD without momentum/weight decay, one step.
+int odl_ref_cnn_train(const float *x, const void *t, int is64, int64_t N, int64_t S, int64_t C1, int64_t C2, int64_t Hd,
+                      int64_t Cc, float *Wc1, float *bc1, float *Wc2, float *bc2, float *Wl1, float *bl1, float *Wl2,
+                      float *bl2, float lr, float *loss, float *gWc1, float *gbc1, float *gWc2, float *gbc2,
+                      float *gWl1, float *gbl1, float *gWl2, float *gbl2, float *logits)
+{
+    return guarded([&] {
+        int64_t Fdim = C2 * (S / 4) * (S / 4);
+        Sequential model;
+        model.add(std::make_unique<nn::Conv2d>(1, (int)C1, 3, 1, 1, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::MaxPool2d>(2, 2, 0));
+        model.add(std::make_unique<nn::Conv2d>((int)C1, (int)C2, 3, 1, 1, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::MaxPool2d>(2, 2, 0));
+        model.add(std::make_unique<nn::Flatten>());
+        model.add(std::make_unique<nn::Linear>((int)Fdim, (int)Hd, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::Linear>((int)Hd, (int)Cc, true));
+        auto &c1 = dynamic_cast<nn::Conv2d &>(model[0]);
+        auto &c2 = dynamic_cast<nn::Conv2d &>(model[3]);
+        auto &l1 = dynamic_cast<nn::Linear &>(model[7]);
+        auto &l2 = dynamic_cast<nn::Linear &>(model[9]);
+        SGD opt(model, lr);
+        *c1.weight() = Parameter(f32(Wc1, Shape{(size_t)C1, 1, 3, 3}, true));
+        *c1.bias()   = Parameter(f32(bc1, Shape{(size_t)C1}, true));
+        *c2.weight() = Parameter(f32(Wc2, Shape{(size_t)C2, (size_t)C1, 3, 3}, true));
+        *c2.bias()   = Parameter(f32(bc2, Shape{(size_t)C2}, true));
+        *l1.weight() = Parameter(f32(Wl1, Shape{(size_t)Fdim, (size_t)Hd}, true));
+        *l1.bias()   = Parameter(f32(bl1, Shape{1, (size_t)Hd}, true));
+        *l2.weight() = Parameter(f32(Wl2, Shape{(size_t)Hd, (size_t)Cc}, true));
+        *l2.bias()   = Parameter(f32(bl2, Shape{1, (size_t)Cc}, true));
+        auto X = f32(x, Shape{(size_t)N, 1, (size_t)S, (size_t)S});
+        auto T = labels(t, is64, N);
+        model.train();
+        opt.zero_grad();
+        auto y = model(X);
+        auto L = F::softmax_cross_entropy(y, T);
+        L.backward();
+        *loss = L.item<float>();
+        out(y, logits);
+        out(c1.weight()->grad(), gWc1);
+        out(c1.bias()->grad(), gbc1);
+        out(c2.weight()->grad(), gWc2);
+        out(c2.bias()->grad(), gbc2);
+        out(l1.weight()->grad(), gWl1);
+        out(l1.bias()->grad(), gbl1);
+        out(l2.weight()->grad(), gWl2);
+        out(l2.bias()->grad(), gbl2);
+        opt.step();
+        out(*c1.weight(), Wc1);
+        out(*c1.bias(), bc1);
+        out(*c2.weight(), Wc2);
+        out(*c2.bias(), bc2);
+        out(*l1.weight(), Wl1);
+        out(*l1.bias(), bl1);
+        out(*l2.weight(), Wl2);
+        out(*l2.bias(), bl2);
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,146 @@
+"""ctypes bindings of the CPU oracle (oracle/liboracle.so) and, where it was built, of the compiled
+reference CPU backend (oracle/_ref/libodl_ref.so). Test infrastructure only: imported by tests, by the
+smoke check and by the CPU-baseline leg of the benchmark, never by the shipped package."""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_SO = os.path.join(ORACLE_DIR, "liboracle.so")
+REF_SO = os.path.join(ORACLE_DIR, "_ref", "libodl_ref.so")
+
+_T = {"p": ctypes.c_void_p, "l": ctypes.c_int64, "i": ctypes.c_int, "f": ctypes.c_float}
+
+# signature strings: p pointer, l int64, i int, f float; return type after '>' (i int, f float, l int64, v void)
+_ORC_SIGS = {
+    "orc_matmul": "ppplll>v",
+    "orc_matmul_batched": "ppplllli>v",
+    "orc_matmul_rows": "pppllll>v",
+    "orc_transpose": "pplll>v",
+    "orc_matmul_backward": "ppppplll>v",
+    "orc_conv_outsize": "llll>l",
+    "orc_im2col": "plllliiiiiiip>i",
+    "orc_col2im": "plllliiiiiiip>i",
+    "orc_conv2d": "ppplllll" + "iiiiii" + "p>i",
+    "orc_conv2d_backward": "ppplllll" + "iiiiii" + "ppp>i",
+    "orc_sum_axis": "plllp>v",
+    "orc_sum_all": "pl>f",
+    "orc_max_axis": "plllp>v",
+    "orc_max_all": "pl>f",
+    "orc_sum_to": "ppipip>i",
+    "orc_broadcast_to": "ppipip>v",
+    "orc_softmax": "plllp>v",
+    "orc_gather": "ppillp>i",
+    "orc_one_hot": "pillp>i",
+    "orc_softmax_ce_loss": "ppillp>i",
+    "orc_softmax_ce_grad": "ppillfp>i",
+    "orc_max_pool2d": "plllliiiiiipp>i",
+    "orc_max_pool2d_backward": "ppllll" + "iiiiii" + "p>i",
+    "orc_argmax_rows": "pllp>v",
+    "orc_accuracy": "ppll>f",
+    "orc_binary": "iplplp>i",
+    "orc_unary": "iplp>v",
+    "orc_pow_scalar": "plfp>v",
+    "orc_mlp_train_step": "ppillll" + "p" * 12 + "ifffff" + "pppppp>i",
+    "orc_cnn_train_step": "ppillllll" + "p" * 8 + "f" + "p" + "pp" + "p" * 8 + "p>i",
+}
+
+_REF_SIGS = {
+    "odl_ref_ping": ">i",
+    "odl_ref_matmul": "ppplll>i",
+    "odl_ref_matmul_batched": "pppllll" + "i>i",
+    "odl_ref_matmul_fwd_bwd": "pppppplll>i",
+    "odl_ref_transpose": "pppi>i",
+    "odl_ref_im2col": "plllliiiiiiip>i",
+    "odl_ref_col2im": "ppillll" + "iiiiiii" + "p>i",
+    "odl_ref_conv2d": "ppplllll" + "iiiiii" + "p>i",
+    "odl_ref_conv2d_backward": "pppplllll" + "iiiiii" + "ppp>i",
+    "odl_ref_sum": "ppiiip>i",
+    "odl_ref_max": "ppiip>i",
+    "odl_ref_sum_to": "ppipip>i",
+    "odl_ref_broadcast_to": "ppipip>i",
+    "odl_ref_broadcast_to_backward": "ppipipp>i",
+    "odl_ref_softmax": "ppiip>i",
+    "odl_ref_gather": "ppillp>i",
+    "odl_ref_one_hot": "pillp>i",
+    "odl_ref_softmax_ce": "ppillpp>i",
+    "odl_ref_max_pool2d": "plllliiiiiipp>i",
+    "odl_ref_max_pool2d_backward": "ppllll" + "iiiiii" + "p>i",
+    "odl_ref_accuracy": "ppllp>i",
+    "odl_ref_binary": "ippippip>i",
+    "odl_ref_unary": "iplp>i",
+    "odl_ref_pow_scalar": "plfp>i",
+    "odl_ref_mlp_train": "ppillll" + "pppp" + "ifffff" + "pppppp>i",
+    "odl_ref_cnn_train": "ppillllll" + "p" * 8 + "f" + "p" + "p" * 8 + "p>i",
+}
+
+
+def _ret(c):
+    return {"v": None, "i": ctypes.c_int, "f": ctypes.c_float, "l": ctypes.c_int64}[c]
+
+
+class _Lib:
+    def __init__(self, path, sigs):
+        self._lib = ctypes.CDLL(path)
+        self._keep = []
+        for name, sig in sigs.items():
+            args, ret = sig.split(">")
+            fn = getattr(self._lib, name)
+            fn.argtypes = [_T[c] for c in args]
+            fn.restype = _ret(ret)
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+
+        def call(*args):
+            conv = []
+            for a in args:
+                if isinstance(a, np.ndarray):
+                    assert a.flags["C_CONTIGUOUS"], "oracle arrays must be C-contiguous"
+                    conv.append(a.ctypes.data)
+                elif a is None:
+                    conv.append(None)
+                else:
+                    conv.append(a)
+            return fn(*conv)
+
+        return call
+
+
+def build_oracle(force=False):
+    """Compile the plain-C oracle (seconds). Building the checker is not using it."""
+    src = os.path.join(ORACLE_DIR, "oracle.c")
+    if force or not os.path.exists(ORACLE_SO) or os.path.getmtime(ORACLE_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", ORACLE_DIR, "liboracle.so"], stdout=subprocess.DEVNULL)
+    return ORACLE_SO
+
+
+_oracle = None
+_ref = None
+
+
+def oracle():
+    global _oracle
+    if _oracle is None:
+        build_oracle()
+        _oracle = _Lib(ORACLE_SO, _ORC_SIGS)
+    return _oracle
+
+
+def have_ref():
+    return os.path.exists(REF_SO)
+
+
+def ref():
+    """The compiled reference CPU backend; only present where oracle/Makefile's `ref` target was built."""
+    global _ref
+    if _ref is None:
+        _ref = _Lib(REF_SO, _REF_SIGS)
+    return _ref
+
+
+def shape_arr(shape):
+    return np.asarray(list(shape), dtype=np.int64)
