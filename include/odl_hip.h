@@ -1,0 +1,185 @@
+/*
+ * odl_hip.h — C ABI of the gfx950 (MI355X) compute backend for OriginDL's hot path.
+ *
+ * This is the boundary a maintainer of the reference binds to: each entry point below stands where one
+ * `origin::cuda::*` free function (include/origin/mat/origin/cuda/cuda_ops.cuh, cuda/factory.cuh) or one
+ * device-runtime call of the reference's Storage/Allocator (src/mat/origin/memory) stands today. Plain
+ * pointers and sizes only; no C++ types, no torch types.
+ *
+ * Conventions
+ *  - All buffers are DEVICE pointers unless a parameter is named host_*. Tensors are dense, row-major,
+ *    float32 unless the name says otherwise; dimensions are int64_t; labels are int32 or int64
+ *    (idx_is_i64 selects), max-pool indices are uint64 (the reference's std::vector<size_t>).
+ *  - `stream` is a hipStream_t passed as void*; NULL is the null stream, which is what the reference uses
+ *    for everything (its host is single-threaded and uses one ordered queue). Launches are asynchronous.
+ *  - Every function returns ODL_OK or a negative code and records a message readable through
+ *    odl_hip_last_error() (thread-local). ODL_ERR_INVALID_ARG corresponds to the reference's
+ *    std::invalid_argument (THROW_INVALID_ARG), ODL_ERR_RUNTIME to std::runtime_error (THROW_RUNTIME_ERROR,
+ *    CUDA_CHECK), include/origin/utils/exception.h:37-57.
+ *  - Functions that need scratch take (workspace, workspace_bytes); the matching *_workspace_bytes query
+ *    says how much. The library never keeps a buffer it hands out or receives.
+ *  - There is no CPU fallback: without a visible gfx950 device every compute entry point fails with
+ *    ODL_ERR_RUNTIME.
+ */
+#ifndef ODL_HIP_H
+#define ODL_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ODL_OK 0
+#define ODL_ERR_INVALID_ARG (-1)
+#define ODL_ERR_RUNTIME (-2)
+
+/* ------------------------------------------------------------------ device runtime ----------------- */
+/* include/origin/cuda/cuda.h:25-105 — is_available / device_count / current_device / set_device /
+ * device_info / synchronize; src/mat/origin/cuda/cuda_utils.cu:37-91 */
+int odl_hip_device_count(int *count);
+int odl_hip_set_device(int device);
+int odl_hip_get_device(int *device);
+int odl_hip_synchronize(void);
+/* writes "name | gcnArch | CUs | clock MHz | global MiB" into buf (NUL-terminated, truncated to len) */
+int odl_hip_device_info(int device, char *buf, size_t len);
+const char *odl_hip_last_error(void);
+/* src/mat/origin/memory/allocator.cpp:53-107 (cudaSetDevice + cudaMalloc / cudaFree / cudaMemGetInfo) */
+int odl_hip_malloc(void **ptr, size_t bytes);
+int odl_hip_free(void *ptr);
+int odl_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
+/* src/mat/origin/memory/storage.cpp:69-145 — synchronous copies, device-synchronised before D2H */
+int odl_hip_memcpy_h2d(void *dst, const void *host_src, size_t bytes);
+int odl_hip_memcpy_d2h(void *host_dst, const void *src, size_t bytes);
+int odl_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+int odl_hip_memset(void *dst, int value, size_t bytes, void *stream);
+
+/* ------------------------------------------------------------------ GEMM ---------------------------- */
+/* General row-major SGEMM on FP32 MFMA: C[M,N] = op(A)[M,K] . op(B)[K,N] (+ bias[N] broadcast over rows
+ * when bias != NULL). trans_a: A is stored [K,M] (lda >= M) else [M,K] (lda >= K); trans_b: B is stored
+ * [N,K] (ldb >= K) else [K,N] (ldb >= N). Replaces origin::cuda::matmul (cuda_ops.cuh matmul;
+ * src/mat/origin/cuda/math/mat_mul.cu:1833-1970) and makes the reference's materialised transposes
+ * (src/operators/math/mat_mul.cpp:171-174) unnecessary.
+ * split_k: 0 = choose automatically, 1 = none, >1 = that many K slices reduced in a fixed order
+ * (needs workspace of odl_hip_sgemm_workspace_bytes). */
+int odl_hip_sgemm(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                  const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int split_k,
+                  void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_sgemm_workspace_bytes(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, int split_k);
+
+/* Mat::matmul — 2-D x 2-D (batch = 1), 3-D x 2-D (b_is_batched = 0), 3-D x 3-D (b_is_batched = 1);
+ * src/mat/origin/cpu/math/matmul.cpp:113-218. */
+int odl_hip_matmul(const float *a, const float *b, float *c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                   int b_is_batched, void *stream);
+/* MatMul::backward (src/operators/math/mat_mul.cpp:123-182): gx[M,K] = gy[M,N] . w[K,N]^T and
+ * gw[K,N] = x[M,K]^T . gy[M,N], as NT and TN GEMMs with no transpose copy. Either output may be NULL. */
+int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M,
+                            int64_t K, int64_t N, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_matmul_backward_workspace_bytes(int64_t M, int64_t K, int64_t N);
+/* Mat::transpose (src/mat/origin/cpu/shape/transpose.cpp:27-77): last two dims of [outer, rows, cols] */
+int odl_hip_transpose(const float *src, float *dst, int64_t outer, int64_t rows, int64_t cols, void *stream);
+
+/* ------------------------------------------------------------------ convolution --------------------- */
+/* Mat::im2col / Mat::col2im (include/origin/mat/mat.h:462-483; src/mat/origin/cpu/conv/conv2d.cpp:39-377).
+ * to_matrix != 0: col is [N*OH*OW, C*KH*KW]; else [N,C,KH,KW,OH,OW]. Zero padding. col2im accumulates each
+ * image pixel's taps in ascending (kh, kw) order, as the reference's scatter loop does, so results are
+ * bit-identical to it and independent of scheduling (no atomics). */
+int odl_hip_im2col(const float *img, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+                   int PH, int PW, int to_matrix, float *col, void *stream);
+int odl_hip_col2im(const float *col, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+                   int PH, int PW, int to_matrix, float *img, void *stream);
+/* Mat::conv2d (mat.h:490; conv2d.cpp:404-512): y[N,OC,OH,OW] = NCHW(im2col(x) . W2d^T + b). b may be NULL. */
+int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                   int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *y, void *workspace,
+                   size_t workspace_bytes, void *stream);
+size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                                      int SH, int SW, int PH, int PW);
+/* Mat::conv2d_backward (mat.h:505; conv2d.cpp:514-599) -> gx, gW and (when gb != NULL) gb.
+ * Reference-faithful: gy's NCHW buffer is read as a row-major [N*OH*OW, OC] matrix with no permutation
+ * (conv2d.cpp:548) for gW and gx; gb is the true per-channel sum of gy (571-578). */
+int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int64_t N, int64_t C, int64_t H,
+                            int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *gx,
+                            float *gw, float *gb, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_conv2d_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH,
+                                               int KW, int SH, int SW, int PH, int PW);
+
+/* ------------------------------------------------------------------ reductions / broadcast ---------- */
+/* Mat::sum(axis) seen as [outer, axis, inner] -> [outer, inner]
+ * (src/mat/origin/cpu/math/sum.cpp:15-90; operation_templates.h:270-333). */
+int odl_hip_sum_axis(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *workspace,
+                     size_t workspace_bytes, void *stream);
+size_t odl_hip_sum_axis_workspace_bytes(int64_t outer, int64_t axis, int64_t inner);
+/* Mat::sum(-1): all elements -> dst[0] (operation_templates.h:342-357) */
+int odl_hip_sum_all(const float *src, int64_t n, float *dst, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_sum_all_workspace_bytes(int64_t n);
+/* Mat::max(axis) / Mat::max(-1) (src/mat/origin/cpu/math/max.cpp:20-121) */
+int odl_hip_max_axis(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *stream);
+int odl_hip_max_all(const float *src, int64_t n, float *dst, void *stream);
+/* Mat::sum_to (mat.h:217; src/mat/origin/cpu/math/sum_to.cpp:11-76): LEFT-aligned shape comparison, one
+ * fused pass per contiguous run of reduced dims. Equal shapes copy. A target with more elements ->
+ * ODL_ERR_RUNTIME; a reduced shape that cannot be reshaped to the target -> ODL_ERR_INVALID_ARG. */
+int odl_hip_sum_to(const float *src, const int64_t *host_src_shape, int src_ndim, const int64_t *host_dst_shape,
+                   int dst_ndim, float *dst, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_sum_to_workspace_bytes(const int64_t *host_src_shape, int src_ndim, const int64_t *host_dst_shape,
+                                      int dst_ndim);
+/* conv bias gradient gy[N,OC,P] -> gb[OC] (conv2d.cpp:566-580) in one pass over gy */
+int odl_hip_sum_nchw_channels(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
+                              size_t workspace_bytes, void *stream);
+size_t odl_hip_sum_nchw_channels_workspace_bytes(int64_t N, int64_t OC, int64_t P);
+/* Mat::broadcast_to (mat.h:210; operation_templates.h:433-493): RIGHT-aligned, up to 8 dims */
+int odl_hip_broadcast_to(const float *src, const int64_t *host_src_shape, int src_ndim,
+                         const int64_t *host_dst_shape, int dst_ndim, float *dst, void *stream);
+
+/* ------------------------------------------------------------------ softmax / cross entropy --------- */
+/* Softmax::forward over [outer, axis, inner] (src/operators/activation/softmax.cpp:14-76) in one kernel */
+int odl_hip_softmax(const float *x, int64_t outer, int64_t axis, int64_t inner, float *y, void *stream);
+/* Mat::gather / Mat::one_hot (mat.h:697,705; src/mat/origin/cpu/nn/gather.cpp). gather validates the labels
+ * (a device flag read back, one 4-byte D2H, like the reference CUDA backend's label check
+ * src/mat/origin/cuda/nn/gather.cu:146-175) and returns ODL_ERR_INVALID_ARG for an out-of-range label;
+ * one_hot skips out-of-range labels silently. */
+int odl_hip_gather(const float *in, const void *idx, int idx_is_i64, int64_t N, int64_t C, float *out, void *stream);
+int odl_hip_one_hot(const void *idx, int idx_is_i64, int64_t N, int64_t C, float *out, void *stream);
+/* SoftmaxCrossEntropy::forward (src/operators/loss/softmax_cross_entropy.cpp:17-75), fused:
+ * *host_loss = -(1/N) sum_i log(softmax(x)[i, t_i] + 1e-8). Synchronises (the reference's .item<float>()).
+ * workspace: N floats + 16 bytes. Out-of-range label -> ODL_ERR_INVALID_ARG. */
+int odl_hip_softmax_ce_loss(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float *host_loss,
+                            void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_softmax_ce_loss_workspace_bytes(int64_t N);
+/* SoftmaxCrossEntropy::backward (softmax_cross_entropy.cpp:77-111), one pass:
+ * gx = (softmax(x) - one_hot(t)) * (gy / N); gy is the host scalar the reference reads with .item<float>() */
+int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float gy, float *gx,
+                            void *stream);
+
+/* ------------------------------------------------------------------ pooling ------------------------- */
+/* Mat::max_pool2d / max_pool2d_backward (mat.h:560-578; src/mat/origin/cpu/pooling/max_pool2d.cpp:40-224).
+ * idx[n,c,oh,ow] = kh*KW+kw of the first maximum (strict >, scan starts at window cell (0,0));
+ * padding cells are 0.0, not -inf. idx may be NULL in the forward. */
+int odl_hip_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+                       int PH, int PW, float *y, uint64_t *idx, void *stream);
+int odl_hip_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N, int64_t C, int64_t H, int64_t W,
+                                int KH, int KW, int SH, int SW, int PH, int PW, float *gx, void *stream);
+
+/* ------------------------------------------------------------------ metrics ------------------------- */
+/* argmax per row, first maximum (src/utils/metrics.cpp:40-53), and accuracy() (metrics.cpp:11-70) with
+ * int32 labels; *host_acc = correct / N. */
+int odl_hip_argmax_rows(const float *y, int64_t N, int64_t C, int64_t *out, void *stream);
+int odl_hip_accuracy(const float *y, const int32_t *t, int64_t N, int64_t C, float *host_acc, void *workspace,
+                     size_t workspace_bytes, void *stream);
+size_t odl_hip_accuracy_workspace_bytes(int64_t N);
+
+/* ------------------------------------------------------------------ elementwise --------------------- */
+/* origin::cuda::{add,subtract,multiply,divide,gt} (cuda_ops.cuh:57-140): op 0 add, 1 sub, 2 mul, 3 div,
+ * 4 greater-than mask (1.0f / 0.0f). na == nb, or one side has a single element; anything else is the
+ * reference's "complex broadcasting" runtime_error. out may alias a or b (add_inplace). */
+int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t nb, float *out, void *stream);
+/* origin::cuda::{relu,exp,log,negate,square,sqrt}: op 0 relu, 1 exp, 2 log, 3 neg, 4 square, 5 sqrt */
+int odl_hip_unary(int op, const float *a, int64_t n, float *out, void *stream);
+/* origin::cuda::pow with a float32 scalar exponent (src/mat/origin/cpu/math/pow.cpp:35-43) */
+int odl_hip_pow_scalar(const float *a, int64_t n, float exponent, float *out, void *stream);
+/* origin::cuda::{zeros,ones,full} (cuda/factory.cuh:23-50) */
+int odl_hip_fill(float *dst, int64_t n, float value, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

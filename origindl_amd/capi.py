@@ -1,0 +1,438 @@
+"""Thin convenience layer over the C ABI (include/odl_hip.h) for tests, the smoke check and the benchmark.
+
+torch is used for exactly two things: device memory (tensors own the buffers whose raw pointers go through the
+C ABI) and the stream the kernels are launched on. No torch operator computes anything here, and nothing
+falls back to torch or to the CPU: every function below is one call into libodl_hip.so.
+
+Names and argument meaning follow the reference's Mat interface (include/origin/mat/mat.h) and operators
+(src/operators/**): mat_mul, mat_mul_backward, im2col, col2im, conv2d, conv2d_backward, sum, sum_to,
+broadcast_to, max, softmax, gather, one_hot, softmax_cross_entropy(+_backward), max_pool2d(+_backward),
+accuracy, and the elementwise set. Errors surface as OdlInvalidArgument / OdlRuntimeError, the counterparts of
+the reference's std::invalid_argument / std::runtime_error."""
+import builtins as _builtins
+import ctypes
+
+import numpy as np
+import torch
+
+from ._lib import OdlInvalidArgument, OdlRuntimeError, lib  # noqa: F401
+
+_f32 = torch.float32
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _chk(t, name="tensor", dtype=_f32):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.is_contiguous() and t.dtype == dtype):
+        raise OdlInvalidArgument("%s must be a contiguous %s device tensor" % (name, dtype))
+    return t
+
+
+def _empty(shape, dtype=_f32):
+    return torch.empty(tuple(int(s) for s in shape), dtype=dtype, device="cuda")
+
+
+def _ws(nbytes):
+    nbytes = int(nbytes)
+    if nbytes == 0:
+        return None, 0
+    buf = torch.empty((nbytes + 3) // 4, dtype=torch.int32, device="cuda")
+    return buf, nbytes
+
+
+def _shape_arr(shape):
+    arr = (ctypes.c_int64 * _builtins.max(len(shape), 1))(*[int(s) for s in shape])
+    return arr
+
+
+def _labels(t):
+    if t.dtype == torch.int64:
+        return _chk(t, "labels", torch.int64), 1
+    if t.dtype == torch.int32:
+        return _chk(t, "labels", torch.int32), 0
+    raise OdlInvalidArgument("indices must be int32 or int64, but got %s" % t.dtype)
+
+
+def conv_outsize(i, k, s, p):
+    return (i + 2 * p - k) // s + 1
+
+
+def _pair(v):
+    return (int(v), int(v)) if isinstance(v, int) else (int(v[0]), int(v[1]))
+
+
+# ------------------------------------------------------------------------------------------ runtime
+def device_count():
+    n = ctypes.c_int(0)
+    lib().call("odl_hip_device_count", ctypes.byref(n))
+    return n.value
+
+
+def is_available():
+    return device_count() > 0
+
+
+def device_info(device=0):
+    buf = ctypes.create_string_buffer(256)
+    lib().call("odl_hip_device_info", device, buf, 256)
+    return buf.value.decode()
+
+
+def synchronize():
+    lib().call("odl_hip_synchronize")
+
+
+# --------------------------------------------------------------------------------------------- GEMM
+def sgemm(a, b, trans_a=False, trans_b=False, bias=None, split_k=0, out=None):
+    """C = op(A) . op(B) (+ bias per column)."""
+    _chk(a, "A"), _chk(b, "B")
+    M, K = (a.shape[1], a.shape[0]) if trans_a else (a.shape[0], a.shape[1])
+    K2, N = (b.shape[1], b.shape[0]) if trans_b else (b.shape[0], b.shape[1])
+    if K != K2:
+        raise OdlInvalidArgument("Matrix dimensions must be compatible for multiplication: K=%d vs %d" % (K, K2))
+    c = out if out is not None else _empty((M, N))
+    need = lib().query("odl_hip_sgemm_workspace_bytes", int(trans_a), int(trans_b), M, N, K, split_k)
+    ws, nb = _ws(need)
+    lib().call("odl_hip_sgemm", int(trans_a), int(trans_b), M, N, K, _p(a), a.shape[1], _p(b), b.shape[1], _p(c), N,
+               _p(bias), split_k, _p(ws), nb, _stream())
+    return c
+
+
+def mat_mul(a, b):
+    """Mat::matmul: 2-D x 2-D, 3-D x 2-D, 3-D x 3-D (src/mat/origin/cpu/math/matmul.cpp:113-218)."""
+    _chk(a, "a"), _chk(b, "b")
+    if a.dim() < 2 or b.dim() < 2:
+        raise OdlInvalidArgument("Matrix multiplication requires at least 2D tensors")
+    if a.dim() == 2 and b.dim() == 2:
+        batch, M, K, bb = 1, a.shape[0], a.shape[1], 0
+        oshape = (M, b.shape[1])
+    elif a.dim() == 3 and b.dim() == 2:
+        batch, M, K, bb = a.shape[0], a.shape[1], a.shape[2], 0
+        oshape = (batch, M, b.shape[1])
+    elif a.dim() == 3 and b.dim() == 3:
+        if a.shape[0] != b.shape[0]:
+            raise OdlInvalidArgument("Matrix dimensions must be compatible: batch %d vs %d" % (a.shape[0], b.shape[0]))
+        batch, M, K, bb = a.shape[0], a.shape[1], a.shape[2], 1
+        oshape = (batch, M, b.shape[2])
+    else:
+        raise OdlInvalidArgument("Matrix multiplication requires compatible dimensions")
+    if b.shape[-2] != K:
+        raise OdlInvalidArgument("Matrix dimensions must be compatible for multiplication: %s x %s"
+                                 % (tuple(a.shape), tuple(b.shape)))
+    N = b.shape[-1]
+    c = _empty(oshape)
+    lib().call("odl_hip_matmul", _p(a), _p(b), _p(c), batch, M, N, K, bb, _stream())
+    return c
+
+
+def mat_mul_backward(x, w, gy, need_gx=True, need_gw=True):
+    """MatMul::backward (src/operators/math/mat_mul.cpp:123-182) -> (gx, gw)."""
+    _chk(x, "x"), _chk(w, "w"), _chk(gy, "gy")
+    M, K = x.shape
+    N = w.shape[1]
+    gx = _empty((M, K)) if need_gx else None
+    gw = _empty((K, N)) if need_gw else None
+    ws, nb = _ws(lib().query("odl_hip_matmul_backward_workspace_bytes", M, K, N))
+    lib().call("odl_hip_matmul_backward", _p(x), _p(w), _p(gy), _p(gx), _p(gw), M, K, N, _p(ws), nb, _stream())
+    return gx, gw
+
+
+def transpose(x):
+    _chk(x, "x")
+    if x.dim() < 2:
+        return x.clone()
+    rows, cols = x.shape[-2], x.shape[-1]
+    outer = int(np.prod(x.shape[:-2])) if x.dim() > 2 else 1
+    out = _empty(tuple(x.shape[:-2]) + (cols, rows))
+    lib().call("odl_hip_transpose", _p(x), _p(out), outer, rows, cols, _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------- conv
+def im2col(img, kernel_size, stride, pad, to_matrix=True):
+    _chk(img, "img")
+    if img.dim() != 4:
+        raise OdlInvalidArgument("im2col: input must be 4D (N, C, H, W)")
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = img.shape
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    shape = (N * OH * OW, C * KH * KW) if to_matrix else (N, C, KH, KW, OH, OW)
+    col = _empty([_builtins.max(s, 0) for s in shape])
+    lib().call("odl_hip_im2col", _p(img), N, C, H, W, KH, KW, SH, SW, PH, PW, int(to_matrix), _p(col), _stream())
+    return col
+
+
+def col2im(col, input_shape, kernel_size, stride, pad, to_matrix=True):
+    _chk(col, "col")
+    if len(input_shape) != 4:
+        raise OdlInvalidArgument("col2im: input_shape must be 4D (N, C, H, W)")
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = [int(s) for s in input_shape]
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    want = (N * OH * OW, C * KH * KW) if to_matrix else (N, C, KH, KW, OH, OW)
+    if tuple(col.shape) != want:
+        raise OdlInvalidArgument("col2im: invalid col shape %s for input_shape %s" % (tuple(col.shape), (N, C, H, W)))
+    img = _empty((N, C, H, W))
+    lib().call("odl_hip_col2im", _p(col), N, C, H, W, KH, KW, SH, SW, PH, PW, int(to_matrix), _p(img), _stream())
+    return img
+
+
+def conv2d(x, w, b=None, stride=1, pad=0):
+    """Mat::conv2d (src/mat/origin/cpu/conv/conv2d.cpp:404-512)."""
+    _chk(x, "x"), _chk(w, "W")
+    if x.dim() != 4:
+        raise OdlInvalidArgument("conv2d: x must be 4D (N, C, H, W)")
+    if w.dim() != 4:
+        raise OdlInvalidArgument("conv2d: W must be 4D (OC, C, KH, KW)")
+    N, C, H, W = x.shape
+    OC, Cw, KH, KW = w.shape
+    if C != Cw:
+        raise OdlInvalidArgument("conv2d: channel mismatch - x has %d channels, but W expects %d" % (C, Cw))
+    if b is not None and (b.dim() != 1 or b.shape[0] != OC):
+        raise OdlInvalidArgument("conv2d: b must be 1D with size %d" % OC)
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    y = _empty((N, OC, _builtins.max(OH, 0), _builtins.max(OW, 0)))
+    ws, nb = _ws(lib().query("odl_hip_conv2d_workspace_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW))
+    lib().call("odl_hip_conv2d", _p(x), _p(w), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, _p(y), _p(ws), nb,
+               _stream())
+    return y
+
+
+def conv2d_backward(gy, x, w, has_bias=True, stride=1, pad=0):
+    """Mat::conv2d_backward (conv2d.cpp:514-599) -> (gx, gW, gb or None)."""
+    _chk(gy, "gy"), _chk(x, "x"), _chk(w, "W")
+    if gy.dim() != 4 or x.dim() != 4 or w.dim() != 4:
+        raise OdlInvalidArgument("conv2d_backward: gy, x and W must be 4D")
+    N, C, H, W = x.shape
+    OC, _, KH, KW = w.shape
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    gx, gw = _empty(x.shape), _empty(w.shape)
+    gb = _empty((OC,)) if has_bias else None
+    ws, nb = _ws(lib().query("odl_hip_conv2d_backward_workspace_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW))
+    lib().call("odl_hip_conv2d_backward", _p(gy), _p(x), _p(w), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, _p(gx), _p(gw),
+               _p(gb), _p(ws), nb, _stream())
+    return gx, gw, gb
+
+
+# ------------------------------------------------------------------------------- reductions / broadcast
+def _split_axis(shape, axis):
+    outer = int(np.prod(shape[:axis])) if axis > 0 else 1
+    inner = int(np.prod(shape[axis + 1:])) if axis + 1 < len(shape) else 1
+    return outer, int(shape[axis]), inner
+
+
+def sum(x, axis=-1, keepdim=False):  # noqa: A001 - the reference's name
+    """Mat::sum (src/mat/origin/cpu/math/sum.cpp:15-90): axis -1 sums everything into shape {1}."""
+    _chk(x, "x")
+    if axis == -1:
+        out = _empty([1] * x.dim() if keepdim else (1,))
+        ws, nb = _ws(lib().query("odl_hip_sum_all_workspace_bytes", x.numel()))
+        lib().call("odl_hip_sum_all", _p(x), x.numel(), _p(out), _p(ws), nb, _stream())
+        return out
+    if axis < 0 or axis >= x.dim():
+        raise OdlInvalidArgument("Invalid axis %d for sum operation. Tensor has %d dimensions" % (axis, x.dim()))
+    outer, ax, inner = _split_axis(x.shape, axis)
+    oshape = [1 if i == axis else s for i, s in enumerate(x.shape)] if keepdim else \
+        [s for i, s in enumerate(x.shape) if i != axis]
+    out = _empty(oshape)
+    ws, nb = _ws(lib().query("odl_hip_sum_axis_workspace_bytes", outer, ax, inner))
+    lib().call("odl_hip_sum_axis", _p(x), outer, ax, inner, _p(out), _p(ws), nb, _stream())
+    return out
+
+
+def max(x, axis=-1):  # noqa: A001
+    """Mat::max (src/mat/origin/cpu/math/max.cpp:20-121)."""
+    _chk(x, "x")
+    if axis == -1:
+        out = _empty((1,))
+        lib().call("odl_hip_max_all", _p(x), x.numel(), _p(out), _stream())
+        return out
+    if axis < 0 or axis >= x.dim():
+        raise OdlInvalidArgument("Invalid axis %d for max operation. Tensor has %d dimensions" % (axis, x.dim()))
+    outer, ax, inner = _split_axis(x.shape, axis)
+    out = _empty([s for i, s in enumerate(x.shape) if i != axis])
+    lib().call("odl_hip_max_axis", _p(x), outer, ax, inner, _p(out), _stream())
+    return out
+
+
+def sum_to(x, shape):
+    """Mat::sum_to (src/mat/origin/cpu/math/sum_to.cpp:11-76), left-aligned."""
+    _chk(x, "x")
+    shape = tuple(int(s) for s in shape)
+    ss, ts = _shape_arr(x.shape), _shape_arr(shape)
+    out = _empty(shape)
+    ws, nb = _ws(lib().query("odl_hip_sum_to_workspace_bytes", ss, x.dim(), ts, len(shape)))
+    lib().call("odl_hip_sum_to", _p(x), ss, x.dim(), ts, len(shape), _p(out), _p(ws), nb, _stream())
+    return out
+
+
+def sum_nchw_channels(gy):
+    _chk(gy, "gy")
+    N, OC = gy.shape[0], gy.shape[1]
+    P = int(np.prod(gy.shape[2:]))
+    out = _empty((OC,))
+    ws, nb = _ws(lib().query("odl_hip_sum_nchw_channels_workspace_bytes", N, OC, P))
+    lib().call("odl_hip_sum_nchw_channels", _p(gy), N, OC, P, _p(out), _p(ws), nb, _stream())
+    return out
+
+
+def broadcast_to(x, shape):
+    _chk(x, "x")
+    shape = tuple(int(s) for s in shape)
+    out = _empty(shape)
+    lib().call("odl_hip_broadcast_to", _p(x), _shape_arr(x.shape), x.dim(), _shape_arr(shape), len(shape), _p(out),
+               _stream())
+    return out
+
+
+# --------------------------------------------------------------------------------- softmax / CE
+def softmax(x, axis=-1):
+    _chk(x, "x")
+    if axis < 0:
+        axis += x.dim()
+    if axis < 0 or axis >= x.dim():
+        raise OdlInvalidArgument("Invalid axis for softmax. Tensor has %d dimensions" % x.dim())
+    outer, ax, inner = _split_axis(x.shape, axis)
+    y = _empty(x.shape)
+    lib().call("odl_hip_softmax", _p(x), outer, ax, inner, _p(y), _stream())
+    return y
+
+
+def gather(x, idx):
+    _chk(x, "input")
+    idx, is64 = _labels(idx)
+    if x.dim() != 2:
+        raise OdlInvalidArgument("gather: input must be 2D (N, C)")
+    if idx.dim() != 1:
+        raise OdlInvalidArgument("gather: indices must be 1D (N,)")
+    if x.shape[0] != idx.shape[0]:
+        raise OdlInvalidArgument("gather: batch size mismatch")
+    out = _empty((x.shape[0],))
+    lib().call("odl_hip_gather", _p(x), _p(idx), is64, x.shape[0], x.shape[1], _p(out), _stream())
+    return out
+
+
+def one_hot(idx, num_classes):
+    idx, is64 = _labels(idx)
+    if idx.dim() != 1:
+        raise OdlInvalidArgument("one_hot: indices must be 1D (N,)")
+    if num_classes <= 0:
+        raise OdlInvalidArgument("one_hot: num_classes must be positive, but got %d" % num_classes)
+    out = _empty((idx.shape[0], num_classes))
+    lib().call("odl_hip_one_hot", _p(idx), is64, idx.shape[0], num_classes, _p(out), _stream())
+    return out
+
+
+def _ce_check(x, t):
+    _chk(x, "x")
+    t, is64 = _labels(t)
+    if x.dim() != 2:
+        raise OdlInvalidArgument("SoftmaxCrossEntropy expects x to be 2D (N, C)")
+    if t.dim() != 1:
+        raise OdlInvalidArgument("SoftmaxCrossEntropy expects target to be 1D (N,)")
+    if x.shape[0] != t.shape[0]:
+        raise OdlInvalidArgument("SoftmaxCrossEntropy: batch size mismatch")
+    return t, is64
+
+
+def softmax_cross_entropy(x, t):
+    """SoftmaxCrossEntropy::forward -> python float (the reference reads the sum back to the host too)."""
+    t, is64 = _ce_check(x, t)
+    N, C = x.shape
+    ws, nb = _ws(lib().query("odl_hip_softmax_ce_loss_workspace_bytes", N))
+    loss = ctypes.c_float(0)
+    lib().call("odl_hip_softmax_ce_loss", _p(x), _p(t), is64, N, C, ctypes.byref(loss), _p(ws), nb, _stream())
+    return loss.value
+
+
+def softmax_cross_entropy_backward(x, t, gy=1.0):
+    t, is64 = _ce_check(x, t)
+    N, C = x.shape
+    gx = _empty(x.shape)
+    lib().call("odl_hip_softmax_ce_grad", _p(x), _p(t), is64, N, C, ctypes.c_float(gy), _p(gx), _stream())
+    return gx
+
+
+# ----------------------------------------------------------------------------------------- pooling
+def max_pool2d(x, kernel_size, stride, pad, with_indices=True):
+    _chk(x, "x")
+    if x.dim() != 4:
+        raise OdlInvalidArgument("max_pool2d: x must be 4D (N, C, H, W)")
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = x.shape
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    y = _empty((N, C, _builtins.max(OH, 0), _builtins.max(OW, 0)))
+    idx = torch.empty(y.shape, dtype=torch.int64, device="cuda") if with_indices else None  # uint64 bit pattern
+    lib().call("odl_hip_max_pool2d", _p(x), N, C, H, W, KH, KW, SH, SW, PH, PW, _p(y), _p(idx), _stream())
+    return y, idx
+
+
+def max_pool2d_backward(gy, idx, input_shape, kernel_size, stride, pad):
+    _chk(gy, "gy")
+    if gy.dim() != 4:
+        raise OdlInvalidArgument("max_pool2d_backward: gy must be 4D (N, C, OH, OW)")
+    if idx is None or idx.numel() != gy.numel():
+        raise OdlInvalidArgument("max_pool2d_backward: indices size mismatch")
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = [int(s) for s in input_shape]
+    gx = _empty((N, C, H, W))
+    lib().call("odl_hip_max_pool2d_backward", _p(gy), _p(idx), N, C, H, W, KH, KW, SH, SW, PH, PW, _p(gx), _stream())
+    return gx
+
+
+# ----------------------------------------------------------------------------------------- metrics
+def argmax_rows(y):
+    _chk(y, "y")
+    out = torch.empty((y.shape[0],), dtype=torch.int64, device="cuda")
+    lib().call("odl_hip_argmax_rows", _p(y), y.shape[0], y.shape[1], _p(out), _stream())
+    return out
+
+
+def accuracy(y, t):
+    _chk(y, "y"), _chk(t, "target", torch.int32)
+    if y.dim() != 2 or t.dim() != 1 or y.shape[0] != t.shape[0]:
+        raise OdlInvalidArgument("accuracy expects y (N, C) and target (N,)")
+    ws, nb = _ws(lib().query("odl_hip_accuracy_workspace_bytes", y.shape[0]))
+    acc = ctypes.c_float(0)
+    lib().call("odl_hip_accuracy", _p(y), _p(t), y.shape[0], y.shape[1], ctypes.byref(acc), _p(ws), nb, _stream())
+    return acc.value
+
+
+# -------------------------------------------------------------------------------------- elementwise
+_BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "gt": 4}
+_UN = {"relu": 0, "exp": 1, "log": 2, "neg": 3, "square": 4, "sqrt": 5}
+
+
+def binary(op, a, b, out=None):
+    _chk(a, "a"), _chk(b, "b")
+    big = a if a.numel() >= b.numel() else b
+    out = out if out is not None else _empty(big.shape)
+    lib().call("odl_hip_binary", _BIN[op], _p(a), a.numel(), _p(b), b.numel(), _p(out), _stream())
+    return out
+
+
+def unary(op, a):
+    _chk(a, "a")
+    out = _empty(a.shape)
+    lib().call("odl_hip_unary", _UN[op], _p(a), a.numel(), _p(out), _stream())
+    return out
+
+
+def pow_scalar(a, e):
+    _chk(a, "a")
+    out = _empty(a.shape)
+    lib().call("odl_hip_pow_scalar", _p(a), a.numel(), ctypes.c_float(e), _p(out), _stream())
+    return out
+
+
+def fill(shape, value):
+    out = _empty(shape)
+    lib().call("odl_hip_fill", _p(out), out.numel(), ctypes.c_float(value), _stream())
+    return out

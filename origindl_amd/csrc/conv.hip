@@ -1,0 +1,335 @@
+// Convolution path of the backend: im2col / col2im in both of the reference's layouts, and conv2d forward /
+// backward composed from them and the MFMA GEMM (src/mat/origin/cpu/conv/conv2d.cpp:39-599 is the behaviour
+// being matched; nothing of the reference's CUDA design is kept).
+//
+//   forward : col = im2col(x); y^T[OC, N*OH*OW] = W2d[OC,K] . col^T  — computed as an "NT" GEMM whose epilogue
+//             adds the bias per row and stores straight into NCHW, so neither the W transpose, nor the
+//             broadcast bias matrix, nor the NHWC->NCHW pass of the reference exist here.
+//   backward: gW[OC,K] = gy2d^T . col as a "TN" GEMM with split-K (the reduction runs over N*OH*OW rows);
+//             gx = col2im(gy2d . W2d); gb = per-channel sum of gy. gy2d is gy's buffer read as a row-major
+//             [N*OH*OW, OC] matrix exactly as it lies (conv2d.cpp:548) — free on the GPU: it is the same pointer.
+//   col2im is a gather: one thread owns one image pixel and adds its taps in ascending (kh, kw) order, which
+//   is the order in which the reference's scatter loop reaches that pixel — bit-identical sums, no atomics.
+#include "odl_common.h"
+
+namespace odl
+{
+int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                 const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int epi, int64_t P,
+                 int split_k, void *workspace, size_t workspace_bytes, hipStream_t st);
+size_t sgemm_workspace(int64_t M, int64_t N, int64_t K, int split_k);
+int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
+                             size_t workspace_bytes, hipStream_t st);
+size_t sum_nchw_channels_workspace(int64_t N, int64_t OC, int64_t P);
+}  // namespace odl
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace
+{
+struct ConvGeom
+{
+    int64_t N, C, H, W;
+    int KH, KW, SH, SW, PH, PW;
+    int64_t OH, OW;
+};
+
+inline int64_t outsize(int64_t in, int k, int s, int p)
+{
+    return (in + 2 * (int64_t)p - k) / s + 1;  // include/origin/utils/conv_utils.h
+}
+
+inline size_t align256(size_t b)
+{
+    return (b + 255) & ~(size_t)255;
+}
+
+// col[m][ck] (m = (n,oh,ow), ck = (c,kh,kw)); one thread produces VEC consecutive ck of one row.
+template <int VEC>
+__global__ void im2col_matrix_kernel(const float *__restrict__ img, float *__restrict__ col, ConvGeom g)
+{
+    const int64_t K = g.C * g.KH * g.KW;
+    const int64_t kq = K / VEC;
+    const int64_t total = g.N * g.OH * g.OW * kq;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    const int64_t m = t / kq;
+    const int ck0 = (int)(t % kq) * VEC;
+    const int64_t ow = m % g.OW, oh = (m / g.OW) % g.OH, n = m / (g.OW * g.OH);
+    float v[VEC];
+    int kw = ck0 % g.KW, kh = (ck0 / g.KW) % g.KH;
+    int64_t c = ck0 / (g.KW * g.KH);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+    {
+        const int64_t h = oh * g.SH + kh - g.PH, w = ow * g.SW + kw - g.PW;
+        v[e] = (h >= 0 && h < g.H && w >= 0 && w < g.W) ? img[((n * g.C + c) * g.H + h) * g.W + w] : 0.f;
+        if (++kw == g.KW)
+        {
+            kw = 0;
+            if (++kh == g.KH)
+            {
+                kh = 0;
+                ++c;
+            }
+        }
+    }
+    if (VEC == 4)
+    {
+        f32x4 o = {v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<f32x4 *>(col + m * K + ck0) = o;
+    }
+    else
+    {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+            col[m * K + ck0 + e] = v[e];
+    }
+}
+
+// col[n][c][kh][kw][oh][ow]; one thread per element, consecutive threads along ow.
+__global__ void im2col_6d_kernel(const float *__restrict__ img, float *__restrict__ col, ConvGeom g)
+{
+    const int64_t total = g.N * g.C * g.KH * g.KW * g.OH * g.OW;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    int64_t r = t;
+    const int64_t ow = r % g.OW;
+    r /= g.OW;
+    const int64_t oh = r % g.OH;
+    r /= g.OH;
+    const int kw = (int)(r % g.KW);
+    r /= g.KW;
+    const int kh = (int)(r % g.KH);
+    r /= g.KH;  // r = n*C + c
+    const int64_t h = oh * g.SH + kh - g.PH, w = ow * g.SW + kw - g.PW;
+    col[t] = (h >= 0 && h < g.H && w >= 0 && w < g.W) ? img[(r * g.H + h) * g.W + w] : 0.f;
+}
+
+// one thread per image pixel; taps added in ascending (kh, kw), starting from +0.0f like the reference's
+// zero-filled padded image (conv2d.cpp:316-349).
+template <bool MATRIX>
+__global__ void col2im_kernel(const float *__restrict__ col, float *__restrict__ img, ConvGeom g)
+{
+    const int64_t total = g.N * g.C * g.H * g.W;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    const int64_t w = t % g.W, h = (t / g.W) % g.H;
+    const int64_t nc = t / (g.W * g.H);
+    const int64_t c = nc % g.C, n = nc / g.C;
+    const int64_t K = g.C * g.KH * g.KW;
+    float acc = 0.f;
+    for (int kh = 0; kh < g.KH; ++kh)
+    {
+        const int64_t hp = h + g.PH - kh;
+        if (hp < 0 || hp % g.SH != 0)
+            continue;
+        const int64_t oh = hp / g.SH;
+        if (oh >= g.OH)
+            continue;
+        for (int kw = 0; kw < g.KW; ++kw)
+        {
+            const int64_t wp = w + g.PW - kw;
+            if (wp < 0 || wp % g.SW != 0)
+                continue;
+            const int64_t ow = wp / g.SW;
+            if (ow >= g.OW)
+                continue;
+            float v;
+            if (MATRIX)
+                v = col[((n * g.OH + oh) * g.OW + ow) * K + (c * g.KH + kh) * g.KW + kw];
+            else
+                v = col[(((nc * g.KH + kh) * g.KW + kw) * g.OH + oh) * g.OW + ow];
+            acc += v;
+        }
+    }
+    img[t] = acc;
+}
+
+int make_geom(ConvGeom &g, const char *who, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+              int PH, int PW)
+{
+    ODL_REQUIRE(N >= 0 && C >= 0 && H > 0 && W > 0, "%s: bad image shape (%lld,%lld,%lld,%lld)", who, (long long)N,
+                (long long)C, (long long)H, (long long)W);
+    ODL_REQUIRE(KH > 0 && KW > 0 && SH > 0 && SW > 0 && PH >= 0 && PW >= 0, "%s: bad kernel/stride/pad", who);
+    g = ConvGeom{N, C, H, W, KH, KW, SH, SW, PH, PW, outsize(H, KH, SH, PH), outsize(W, KW, SW, PW)};
+    ODL_REQUIRE(g.OH > 0 && g.OW > 0,
+                "%s: invalid output size OH=%lld, OW=%lld for input H=%lld, W=%lld, kernel=(%d,%d), stride=(%d,%d), "
+                "pad=(%d,%d)",
+                who, (long long)g.OH, (long long)g.OW, (long long)H, (long long)W, KH, KW, SH, SW, PH, PW);
+    return ODL_OK;
+}
+
+int im2col_launch(const float *img, float *col, const ConvGeom &g, int to_matrix, hipStream_t st)
+{
+    const int64_t K = g.C * g.KH * g.KW;
+    const int64_t total = g.N * g.OH * g.OW * K;
+    if (total == 0)
+        return ODL_OK;
+    if (to_matrix)
+    {
+        const bool v4 = (K % 4 == 0) && (reinterpret_cast<uintptr_t>(col) % 16 == 0);
+        const int64_t threads = v4 ? total / 4 : total;
+        const dim3 grid((unsigned)odl::ceil_div(threads, 256));
+        if (v4)
+            hipLaunchKernelGGL(im2col_matrix_kernel<4>, grid, dim3(256), 0, st, img, col, g);
+        else
+            hipLaunchKernelGGL(im2col_matrix_kernel<1>, grid, dim3(256), 0, st, img, col, g);
+    }
+    else
+    {
+        hipLaunchKernelGGL(im2col_6d_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, img, col, g);
+    }
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int col2im_launch(const float *col, float *img, const ConvGeom &g, int to_matrix, hipStream_t st)
+{
+    const int64_t total = g.N * g.C * g.H * g.W;
+    if (total == 0)
+        return ODL_OK;
+    const dim3 grid((unsigned)odl::ceil_div(total, 256));
+    if (to_matrix)
+        hipLaunchKernelGGL(col2im_kernel<true>, grid, dim3(256), 0, st, col, img, g);
+    else
+        hipLaunchKernelGGL(col2im_kernel<false>, grid, dim3(256), 0, st, col, img, g);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int odl_hip_im2col(const float *img, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
+                   int PW, int to_matrix, float *col, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ConvGeom g;
+    int rc = make_geom(g, "im2col", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(g.N * g.OH * g.OW * g.C * g.KH * g.KW < (1ll << 40), "im2col: column matrix too large");
+    return im2col_launch(img, col, g, to_matrix, odl::as_stream(stream));
+}
+
+int odl_hip_col2im(const float *col, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
+                   int PW, int to_matrix, float *img, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ConvGeom g;
+    int rc = make_geom(g, "col2im", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    return col2im_launch(col, img, g, to_matrix, odl::as_stream(stream));
+}
+
+size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                                      int SW, int PH, int PW)
+{
+    (void)OC;
+    if (KH <= 0 || KW <= 0 || SH <= 0 || SW <= 0)
+        return 0;
+    const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
+    if (OH <= 0 || OW <= 0)
+        return 0;
+    return align256((size_t)(N * OH * OW * C * KH * KW) * sizeof(float));
+}
+
+int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                   int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *y, void *workspace,
+                   size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ConvGeom g;
+    int rc = make_geom(g, "conv2d", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(OC > 0, "conv2d: OC must be positive");
+    const int64_t M = N * g.OH * g.OW, K = C * KH * KW;
+    if (M == 0)
+        return ODL_OK;
+    const size_t need = odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need, "conv2d: workspace of %zu bytes required, got %zu",
+                need, workspace_bytes);
+    hipStream_t st = odl::as_stream(stream);
+    float *col = static_cast<float *>(workspace);
+    rc = im2col_launch(x, col, g, 1, st);
+    if (rc != ODL_OK)
+        return rc;
+    // y^T[OC, M] = W2d[OC,K] . col[M,K]^T, stored as y[n][oc][p] with the bias added per output channel
+    return odl::sgemm_launch(0, 1, OC, M, K, w, K, col, K, y, 0, b, /*EPI_NCHW_ROWB*/ 2, g.OH * g.OW, 1, nullptr, 0,
+                             st);
+}
+
+size_t odl_hip_conv2d_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                                               int SH, int SW, int PH, int PW)
+{
+    if (KH <= 0 || KW <= 0 || SH <= 0 || SW <= 0)
+        return 0;
+    const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
+    if (OH <= 0 || OW <= 0)
+        return 0;
+    const int64_t M = N * OH * OW, K = C * KH * KW;
+    return align256((size_t)(M * K) * sizeof(float)) + align256(odl::sgemm_workspace(OC, K, M, 0)) +
+           align256(odl::sum_nchw_channels_workspace(N, OC, OH * OW));
+}
+
+int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int64_t N, int64_t C, int64_t H, int64_t W,
+                            int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *gx, float *gw, float *gb,
+                            void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ConvGeom g;
+    int rc = make_geom(g, "conv2d_backward", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(OC > 0, "conv2d_backward: OC must be positive");
+    const int64_t M = N * g.OH * g.OW, K = C * KH * KW;
+    if (M == 0)
+        return ODL_OK;
+    const size_t need = odl_hip_conv2d_backward_workspace_bytes(N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
+                "conv2d_backward: workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    hipStream_t st = odl::as_stream(stream);
+    char *ws = static_cast<char *>(workspace);
+    float *col = reinterpret_cast<float *>(ws);
+    const size_t col_bytes = align256((size_t)(M * K) * sizeof(float));
+    void *splitk_ws = ws + col_bytes;
+    const size_t splitk_bytes = align256(odl::sgemm_workspace(OC, K, M, 0));
+    void *red_ws = ws + col_bytes + splitk_bytes;
+    const size_t red_bytes = align256(odl::sum_nchw_channels_workspace(N, OC, g.OH * g.OW));
+
+    if (gw)
+    {
+        rc = im2col_launch(x, col, g, 1, st);
+        if (rc != ODL_OK)
+            return rc;
+        // gW[OC,K] = gy2d[M,OC]^T . col[M,K]
+        rc = odl::sgemm_launch(1, 0, OC, K, M, gy, OC, col, K, gw, K, nullptr, 0, 0, 0, splitk_ws, splitk_bytes, st);
+        if (rc != ODL_OK)
+            return rc;
+    }
+    if (gb)
+    {
+        rc = odl::sum_nchw_channels_launch(gy, N, OC, g.OH * g.OW, gb, red_ws, red_bytes, st);
+        if (rc != ODL_OK)
+            return rc;
+    }
+    if (gx)
+    {
+        // gx_col[M,K] = gy2d[M,OC] . W2d[OC,K], then the gather back to the image
+        rc = odl::sgemm_launch(0, 0, M, K, OC, gy, OC, w, K, col, K, nullptr, 0, 0, 1, nullptr, 0, st);
+        if (rc != ODL_OK)
+            return rc;
+        rc = col2im_launch(col, gx, g, 1, st);
+        if (rc != ODL_OK)
+            return rc;
+    }
+    return ODL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,228 @@
+// Elementwise plumbing between the hot kernels: add/sub/mul/div (same shape or single-element broadcast, the
+// only cases the reference supports, src/mat/origin/cpu/math/add.cpp:56-93), the > mask, relu/exp/log/neg/
+// square/sqrt, pow with a scalar exponent, and fills. 16 bytes per lane when the buffers allow it.
+// Built with floating-point contraction off: every arithmetic step rounds like the reference's separate ops.
+#include "odl_common.h"
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace
+{
+constexpr int kBlock = 256;
+
+template <int OP>
+__device__ inline float bin(float a, float b)
+{
+    if (OP == 0) return a + b;
+    if (OP == 1) return a - b;
+    if (OP == 2) return a * b;
+    if (OP == 3) return a / b;
+    return (a > b) ? 1.f : 0.f;
+}
+
+template <int OP>
+__device__ inline float un(float v)
+{
+    if (OP == 0) return v > 0.f ? v : 0.f;
+    if (OP == 1) return expf(v);
+    if (OP == 2) return logf(v);
+    if (OP == 3) return -v;
+    if (OP == 4) return v * v;
+    return sqrtf(v);
+}
+
+// MODE 0: a[i] op b[i]; 1: a[i] op b[0]; 2: a[0] op b[i]. Each thread handles 4 consecutive elements.
+template <int OP, int MODE, bool VEC>
+__global__ void binary_kernel(const float *a, const float *b, float *out, int64_t n)
+{
+    const int64_t i0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i0 >= n)
+        return;
+    float av[4], bv[4], ov[4];
+    const bool full = VEC && (i0 + 4 <= n);
+    if (full)
+    {
+        if (MODE != 2)
+        {
+            const f32x4 q = *reinterpret_cast<const f32x4 *>(a + i0);
+            av[0] = q[0], av[1] = q[1], av[2] = q[2], av[3] = q[3];
+        }
+        if (MODE != 1)
+        {
+            const f32x4 q = *reinterpret_cast<const f32x4 *>(b + i0);
+            bv[0] = q[0], bv[1] = q[1], bv[2] = q[2], bv[3] = q[3];
+        }
+    }
+    else
+    {
+        for (int e = 0; e < 4; ++e)
+        {
+            const bool in = i0 + e < n;
+            if (MODE != 2)
+                av[e] = in ? a[i0 + e] : 0.f;
+            if (MODE != 1)
+                bv[e] = in ? b[i0 + e] : 1.f;
+        }
+    }
+    if (MODE == 1)
+        bv[0] = bv[1] = bv[2] = bv[3] = b[0];
+    if (MODE == 2)
+        av[0] = av[1] = av[2] = av[3] = a[0];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        ov[e] = bin<OP>(av[e], bv[e]);
+    if (full)
+    {
+        f32x4 q = {ov[0], ov[1], ov[2], ov[3]};
+        *reinterpret_cast<f32x4 *>(out + i0) = q;
+    }
+    else
+        for (int e = 0; e < 4 && i0 + e < n; ++e)
+            out[i0 + e] = ov[e];
+}
+
+template <int OP>
+__global__ void unary_kernel(const float *a, float *out, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        out[i] = un<OP>(a[i]);
+}
+
+__global__ void pow_kernel(const float *a, float *out, int64_t n, float e)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        out[i] = powf(a[i], e);
+}
+
+__global__ void fill_kernel(float *dst, int64_t n, float v)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        dst[i] = v;
+}
+
+__global__ void fill_bytes_kernel(unsigned char *dst, size_t n, unsigned char v)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        dst[i] = v;
+}
+
+template <int OP>
+int launch_binary(const float *a, int64_t na, const float *b, int64_t nb, float *out, hipStream_t st)
+{
+    const int64_t n = na > nb ? na : nb;
+    const int mode = (na == nb) ? 0 : (nb == 1 ? 1 : 2);
+    auto aligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const bool vec = aligned(out) && (mode == 2 || aligned(a)) && (mode == 1 || aligned(b));
+    const dim3 grid((unsigned)odl::ceil_div(odl::ceil_div(n, 4), kBlock));
+#define ODL_BIN_CASE(M, V)                                                                          \
+    if (mode == M && vec == V)                                                                      \
+        hipLaunchKernelGGL((binary_kernel<OP, M, V>), grid, dim3(kBlock), 0, st, a, b, out, n);
+    ODL_BIN_CASE(0, true)
+    ODL_BIN_CASE(0, false)
+    ODL_BIN_CASE(1, true)
+    ODL_BIN_CASE(1, false)
+    ODL_BIN_CASE(2, true)
+    ODL_BIN_CASE(2, false)
+#undef ODL_BIN_CASE
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace
+
+namespace odl
+{
+int fill_launch(float *dst, int64_t n, float value, hipStream_t st)
+{
+    if (n <= 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(fill_kernel, dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, st, dst, n, value);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+// byte fill as a kernel: a memset node inside a captured graph is avoided on purpose
+int fill_bytes_launch(void *dst, int value, size_t bytes, hipStream_t st)
+{
+    if (bytes == 0)
+        return ODL_OK;
+    const unsigned char b = (unsigned char)value;
+    if (reinterpret_cast<uintptr_t>(dst) % 4 == 0 && bytes % 4 == 0)
+    {
+        const unsigned int w = b * 0x01010101u;
+        float f;
+        __builtin_memcpy(&f, &w, 4);
+        return fill_launch(static_cast<float *>(dst), (int64_t)(bytes / 4), f, st);
+    }
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)ceil_div((int64_t)bytes, kBlock)), dim3(kBlock), 0, st,
+                       static_cast<unsigned char *>(dst), bytes, b);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace odl
+
+extern "C" {
+
+int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t nb, float *out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(op >= 0 && op <= 4, "binary: unknown op %d", op);
+    ODL_REQUIRE(na >= 0 && nb >= 0, "binary: negative extent");
+    if (!(na == nb || na == 1 || nb == 1))
+        return odl::fail(ODL_ERR_RUNTIME, "Complex broadcasting not yet implemented (%lld vs %lld elements)",
+                         (long long)na, (long long)nb);
+    if (na == 0 || nb == 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    switch (op)
+    {
+        case 0: return launch_binary<0>(a, na, b, nb, out, st);
+        case 1: return launch_binary<1>(a, na, b, nb, out, st);
+        case 2: return launch_binary<2>(a, na, b, nb, out, st);
+        case 3: return launch_binary<3>(a, na, b, nb, out, st);
+        default: return launch_binary<4>(a, na, b, nb, out, st);
+    }
+}
+
+int odl_hip_unary(int op, const float *a, int64_t n, float *out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(op >= 0 && op <= 5, "unary: unknown op %d", op);
+    if (n <= 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    const dim3 grid((unsigned)odl::ceil_div(n, kBlock));
+    switch (op)
+    {
+        case 0: hipLaunchKernelGGL(unary_kernel<0>, grid, dim3(kBlock), 0, st, a, out, n); break;
+        case 1: hipLaunchKernelGGL(unary_kernel<1>, grid, dim3(kBlock), 0, st, a, out, n); break;
+        case 2: hipLaunchKernelGGL(unary_kernel<2>, grid, dim3(kBlock), 0, st, a, out, n); break;
+        case 3: hipLaunchKernelGGL(unary_kernel<3>, grid, dim3(kBlock), 0, st, a, out, n); break;
+        case 4: hipLaunchKernelGGL(unary_kernel<4>, grid, dim3(kBlock), 0, st, a, out, n); break;
+        default: hipLaunchKernelGGL(unary_kernel<5>, grid, dim3(kBlock), 0, st, a, out, n); break;
+    }
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_pow_scalar(const float *a, int64_t n, float exponent, float *out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    if (n <= 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(pow_kernel, dim3((unsigned)odl::ceil_div(n, kBlock)), dim3(kBlock), 0, odl::as_stream(stream), a,
+                       out, n, exponent);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_fill(float *dst, int64_t n, float value, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    return odl::fill_launch(dst, n, value, odl::as_stream(stream));
+}
+
+}  // extern "C"

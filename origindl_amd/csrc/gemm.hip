@@ -1,0 +1,528 @@
+// FP32 GEMM for gfx950 on the matrix cores (v_mfma_f32_32x32x2_f32), hand-written.
+//
+// C[M,N] = op(A)[M,K] . op(B)[K,N], row-major, all four transpose combinations, so that the backward
+// products dA = dC.B^T (NT) and dB = A^T.dC (TN) read their operands in place — the reference materialises
+// both transposes first (src/operators/math/mat_mul.cpp:171-174).
+//
+// Shape of the kernel (wave64, 256 threads = 4 waves in a 2x2 grid):
+//   * workgroup tile BM x BN x BK, wave tile (BM/2) x (BN/2) made of 32x32 MFMA blocks whose accumulators
+//     stay in registers for the whole K loop;
+//   * each operand tile is staged through LDS in the layout its global layout suggests, so the global->LDS
+//     copy is always a 16-byte load and a 16-byte store with no transposition:
+//       K-contiguous in memory  -> LDS [row][BK+4]  (fragment = one ds_read_b128 per lane),
+//       row-contiguous in memory -> LDS [k][rows+4] (fragment = four conflict-free ds_read_b32);
+//     both layouts give lane (i = lane%32, h = lane/32) the four values k = 4h..4h+3 of its row, and MFMA
+//     step s multiplies the k = {s, 4+s} pair — the K order inside a tile is permuted, which a sum allows;
+//   * two LDS buffers and register prefetch of the next K slab: one barrier per slab;
+//   * workgroup -> tile mapping that keeps each XCD (one L2 each, workgroups are dealt round-robin over the
+//     8 XCDs) on a contiguous band of tiles, walked in groups of 8 tile-rows so A and B panels are reused
+//     from that XCD's L2;
+//   * split-K (grid.y) writes partial tiles that a second kernel sums in slice order — deterministic.
+#include "odl_common.h"
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace
+{
+constexpr int kThreads = 256;
+constexpr int kXcds    = 8;
+constexpr int kGroupM  = 8;
+
+enum : int
+{
+    EPI_PLAIN     = 0,  // C[row*ldc + col]
+    EPI_BIAS_COL  = 1,  // + bias[col]
+    EPI_NCHW_ROWB = 2,  // conv forward: row = oc, col = n*P + p -> y[(n*OC + oc)*P + p] (+ bias[oc])
+};
+
+struct GemmArgs
+{
+    const float *A;
+    const float *B;
+    float *C;
+    const float *bias;
+    int64_t M, N, K;
+    int64_t lda, ldb, ldc;
+    int64_t k_per_split;     // K range of one grid.y slice (multiple of BK)
+    int64_t c_split_stride;  // elements between the partial outputs of consecutive slices (0 = none)
+    int64_t P;               // EPI_NCHW_ROWB: OH*OW
+    int tiles_m, tiles_n;
+};
+
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI>
+__global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g)
+{
+    // A tile: !TA -> memory is [M][K] (K-contiguous) -> LDS K-major; TA -> memory [K][M] -> LDS row-major.
+    // B tile: !TB -> memory is [K][N] (row-contiguous) -> LDS row-major; TB -> memory [N][K] -> LDS K-major.
+    constexpr bool A_KMAJOR = !TA;
+    constexpr bool B_KMAJOR = TB;
+    constexpr int LDA_S     = A_KMAJOR ? (BK + 4) : (BM + 4);
+    constexpr int LDB_S     = B_KMAJOR ? (BK + 4) : (BN + 4);
+    constexpr int A_SIZE    = A_KMAJOR ? BM * LDA_S : BK * LDA_S;
+    constexpr int B_SIZE    = B_KMAJOR ? BN * LDB_S : BK * LDB_S;
+    constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
+    constexpr int RB = WM / 32, CB = WN / 32;
+    constexpr int A_PER_T = BM * BK / kThreads;  // floats staged per thread
+    constexpr int B_PER_T = BN * BK / kThreads;
+    static_assert(BK % 8 == 0 && A_PER_T % 4 == 0 && B_PER_T % 4 == 0, "tile shape");
+
+    __shared__ __attribute__((aligned(16))) float As[2][A_SIZE];
+    __shared__ __attribute__((aligned(16))) float Bs[2][B_SIZE];
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+
+    // ---- workgroup -> tile: contiguous band per XCD, then groups of kGroupM tile-rows
+    int tm, tn;
+    {
+        const int nt = g.tiles_m * g.tiles_n;
+        const int bid = blockIdx.x;
+        const int xcd = bid % kXcds, loc = bid / kXcds;
+        const int full = nt / kXcds, rem = nt % kXcds;
+        const int t = xcd * full + (xcd < rem ? xcd : rem) + loc;
+        const int gsz = kGroupM * g.tiles_n;
+        const int grp = t / gsz, in_g = t % gsz;
+        const int first_m = grp * kGroupM;
+        const int gm = (g.tiles_m - first_m) < kGroupM ? (g.tiles_m - first_m) : kGroupM;
+        tm = first_m + in_g % gm;
+        tn = in_g / gm;
+    }
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t kbeg = (int64_t)blockIdx.y * g.k_per_split;
+    const int64_t kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
+    const int nkt = (int)((kend - kbeg + BK - 1) / BK);
+
+    float ra[A_PER_T], rb_[B_PER_T];
+
+    auto load_tile = [&](const float *__restrict__ src, int64_t ld, bool kmajor, int64_t row0, int64_t rows,
+                         int64_t k0, int brows, float *regs, int per_t) {
+        // kmajor: memory [rows][K]; else memory [K][rows]. `brows` = BM or BN.
+        if (VEC)
+        {
+            for (int u = 0; u < per_t / 4; ++u)
+            {
+                const int f = tid + u * kThreads;
+                int64_t r, k;
+                if (kmajor)
+                {
+                    r = row0 + f / (BK / 4);
+                    k = k0 + 4 * (f % (BK / 4));
+                }
+                else
+                {
+                    k = k0 + f / (brows / 4);
+                    r = row0 + 4 * (f % (brows / 4));
+                }
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (r < rows && k < kend)
+                    v = *reinterpret_cast<const f32x4 *>(src + (kmajor ? r * ld + k : k * ld + r));
+                regs[4 * u + 0] = v[0];
+                regs[4 * u + 1] = v[1];
+                regs[4 * u + 2] = v[2];
+                regs[4 * u + 3] = v[3];
+            }
+        }
+        else
+        {
+            for (int u = 0; u < per_t; ++u)
+            {
+                const int e = tid + u * kThreads;
+                int64_t r, k;
+                if (kmajor)
+                {
+                    r = row0 + e / BK;
+                    k = k0 + e % BK;
+                }
+                else
+                {
+                    k = k0 + e / brows;
+                    r = row0 + e % brows;
+                }
+                regs[u] = (r < rows && k < kend) ? src[kmajor ? r * ld + k : k * ld + r] : 0.f;
+            }
+        }
+    };
+
+    auto store_tile = [&](float *lds, int lds_ld, bool kmajor, int brows, const float *regs, int per_t) {
+        if (VEC)
+        {
+            for (int u = 0; u < per_t / 4; ++u)
+            {
+                const int f = tid + u * kThreads;
+                int off;
+                if (kmajor)
+                    off = (f / (BK / 4)) * lds_ld + 4 * (f % (BK / 4));
+                else
+                    off = (f / (brows / 4)) * lds_ld + 4 * (f % (brows / 4));
+                f32x4 v = {regs[4 * u], regs[4 * u + 1], regs[4 * u + 2], regs[4 * u + 3]};
+                *reinterpret_cast<f32x4 *>(lds + off) = v;
+            }
+        }
+        else
+        {
+            for (int u = 0; u < per_t; ++u)
+            {
+                const int e = tid + u * kThreads;
+                const int off = kmajor ? (e / BK) * lds_ld + e % BK : (e / brows) * lds_ld + e % brows;
+                lds[off] = regs[u];
+            }
+        }
+    };
+
+    f32x16 acc[RB][CB];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < CB; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0.f;
+
+    if (nkt > 0)
+    {
+        load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, kbeg, BM, ra, A_PER_T);
+        load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, kbeg, BN, rb_, B_PER_T);
+        store_tile(As[0], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
+        store_tile(Bs[0], LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < nkt; ++kt)
+    {
+        const int cur = kt & 1;
+        if (kt + 1 < nkt)
+        {
+            const int64_t k0 = kbeg + (int64_t)(kt + 1) * BK;
+            load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra, A_PER_T);
+            load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, k0, BN, rb_, B_PER_T);
+        }
+        const float *as = As[cur];
+        const float *bs = Bs[cur];
+#pragma unroll
+        for (int ks = 0; ks < BK / 8; ++ks)
+        {
+            float a[RB][4], b[CB][4];
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+            {
+                if (A_KMAJOR)
+                {
+                    const f32x4 v =
+                        *reinterpret_cast<const f32x4 *>(as + (wm + i * 32 + l32) * LDA_S + ks * 8 + 4 * lh);
+                    a[i][0] = v[0], a[i][1] = v[1], a[i][2] = v[2], a[i][3] = v[3];
+                }
+                else
+                {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        a[i][s] = as[(ks * 8 + 4 * lh + s) * LDA_S + wm + i * 32 + l32];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < CB; ++j)
+            {
+                if (B_KMAJOR)
+                {
+                    const f32x4 v =
+                        *reinterpret_cast<const f32x4 *>(bs + (wn + j * 32 + l32) * LDB_S + ks * 8 + 4 * lh);
+                    b[j][0] = v[0], b[j][1] = v[1], b[j][2] = v[2], b[j][3] = v[3];
+                }
+                else
+                {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        b[j][s] = bs[(ks * 8 + 4 * lh + s) * LDB_S + wn + j * 32 + l32];
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int i = 0; i < RB; ++i)
+#pragma unroll
+                    for (int j = 0; j < CB; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nkt)
+        {
+            store_tile(As[cur ^ 1], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
+            store_tile(Bs[cur ^ 1], LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
+    float *Cout = g.C + (int64_t)blockIdx.y * g.c_split_stride;
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < CB; ++j)
+        {
+            const int64_t col = n0 + wn + j * 32 + l32;
+            if (col >= g.N)
+                continue;
+            float bcol = 0.f;
+            if (EPI == EPI_BIAS_COL && g.bias)
+                bcol = g.bias[col];
+            int64_t nchw_base = 0;
+            if (EPI == EPI_NCHW_ROWB)
+            {
+                const int64_t n = col / g.P, p = col % g.P;
+                nchw_base = n * g.M * g.P + p;  // + oc * P
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                const int64_t row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+                if (row >= g.M)
+                    continue;
+                float v = acc[i][j][r];
+                if (EPI == EPI_NCHW_ROWB)
+                {
+                    if (g.bias)
+                        v = v + g.bias[row];
+                    Cout[nchw_base + row * g.P] = v;
+                }
+                else
+                {
+                    if (EPI == EPI_BIAS_COL)
+                        v = v + bcol;
+                    Cout[row * g.ldc + col] = v;
+                }
+            }
+        }
+}
+
+// out[i] = sum over slices (ascending) of part[s*stride + i] (+ bias by column or by row for the NCHW store)
+__global__ void splitk_reduce_kernel(const float *__restrict__ part, int splits, int64_t stride, float *out,
+                                     int64_t M, int64_t N, int64_t ldc, const float *bias)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= M * N)
+        return;
+    float s = 0.f;
+    for (int z = 0; z < splits; ++z)
+        s += part[(int64_t)z * stride + i];
+    const int64_t r = i / N, c = i % N;
+    if (bias)
+        s = s + bias[c];
+    out[r * ldc + c] = s;
+}
+
+__global__ void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows, int64_t cols)
+{
+    __shared__ float tile[32][33];
+    const int64_t o   = blockIdx.z;
+    const float *s    = src + o * rows * cols;
+    float *d          = dst + o * rows * cols;
+    const int64_t c0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
+    for (int i = threadIdx.y; i < 32; i += 8)
+    {
+        const int64_t r = r0 + i, c = c0 + threadIdx.x;
+        tile[i][threadIdx.x] = (r < rows && c < cols) ? s[r * cols + c] : 0.f;
+    }
+    __syncthreads();
+    for (int i = threadIdx.y; i < 32; i += 8)
+    {
+        const int64_t c = c0 + i, r = r0 + threadIdx.x;
+        if (r < rows && c < cols)
+            d[c * rows + r] = tile[threadIdx.x][i];
+    }
+}
+
+template <int BM, int BN, int BK, int EPI>
+int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g, int splits, hipStream_t st)
+{
+    dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits);
+    dim3 block(kThreads);
+#define ODL_GEMM_CASE(TA, TB, V)                                                                      \
+    if (ta == TA && tb == TB && vec == V)                                                             \
+    {                                                                                                 \
+        hipLaunchKernelGGL((sgemm_mfma_kernel<BM, BN, BK, TA, TB, V, EPI>), grid, block, 0, st, g);   \
+        return ODL_OK;                                                                                \
+    }
+    ODL_GEMM_CASE(false, false, true)
+    ODL_GEMM_CASE(false, true, true)
+    ODL_GEMM_CASE(true, false, true)
+    ODL_GEMM_CASE(true, true, true)
+    ODL_GEMM_CASE(false, false, false)
+    ODL_GEMM_CASE(false, true, false)
+    ODL_GEMM_CASE(true, false, false)
+    ODL_GEMM_CASE(true, true, false)
+#undef ODL_GEMM_CASE
+    return ODL_ERR_RUNTIME;
+}
+
+constexpr int kBM = 128, kBN = 128, kBK = 16;
+
+int pick_splits(int64_t M, int64_t N, int64_t K, int requested)
+{
+    if (requested >= 1)
+        return requested;
+    const int64_t tiles = odl::ceil_div(M, kBM) * odl::ceil_div(N, kBN);
+    const int64_t kt    = odl::ceil_div(K, kBK);
+    if (tiles >= 128 || kt < 64)
+        return 1;
+    int64_t s = odl::ceil_div(512, tiles);
+    if (s > kt / 16)
+        s = kt / 16;
+    if (s > 128)
+        s = 128;
+    return s < 1 ? 1 : (int)s;
+}
+}  // namespace
+
+namespace odl
+{
+// Shared by the convolution entry points. epi: 0 plain, 1 bias by column, 2 NCHW store with bias by row.
+int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                 const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int epi, int64_t P,
+                 int split_k, void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    if (M == 0 || N == 0)
+        return ODL_OK;
+    ODL_REQUIRE(M > 0 && N > 0 && K >= 0, "sgemm: bad dimensions M=%lld N=%lld K=%lld", (long long)M, (long long)N,
+                (long long)K);
+    ODL_REQUIRE(A && B && C, "sgemm: null operand");
+    ODL_REQUIRE(lda >= (trans_a ? M : K) && ldb >= (trans_b ? K : N) && (epi == EPI_NCHW_ROWB || ldc >= N),
+                "sgemm: leading dimension smaller than the row length");
+    ODL_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "sgemm: dimension exceeds 2^31");
+    GemmArgs g;
+    g.A = A, g.B = B, g.C = C, g.bias = bias;
+    g.M = M, g.N = N, g.K = K, g.lda = lda, g.ldb = ldb, g.ldc = ldc, g.P = P;
+    g.tiles_m = (int)ceil_div(M, kBM), g.tiles_n = (int)ceil_div(N, kBN);
+    ODL_REQUIRE((int64_t)g.tiles_m * g.tiles_n < (1ll << 31), "sgemm: too many tiles");
+
+    // 16-byte loads need 16-byte aligned rows: base pointers, leading dimensions and the contiguous extents
+    const bool vec = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) % 16 == 0) && lda % 4 == 0 &&
+                     ldb % 4 == 0 && (trans_a ? M : K) % 4 == 0 && (trans_b ? K : N) % 4 == 0;
+
+    int splits = (epi == EPI_NCHW_ROWB) ? 1 : pick_splits(M, N, K, split_k);
+    const int64_t kt = ceil_div(K > 0 ? K : 1, kBK);
+    if (splits > kt)
+        splits = (int)kt;
+    if (splits > 1)
+    {
+        const size_t need = (size_t)splits * M * N * sizeof(float);
+        if (workspace == nullptr || workspace_bytes < need)
+        {
+            if (split_k > 1)
+                return fail(ODL_ERR_INVALID_ARG, "sgemm: split_k=%d needs %zu workspace bytes, got %zu", split_k, need,
+                            workspace_bytes);
+            splits = 1;  // automatic choice falls back to a single pass
+        }
+    }
+    g.k_per_split    = ceil_div(kt, splits) * kBK;
+    g.c_split_stride = 0;
+    int rc;
+    if (splits > 1)
+    {
+        GemmArgs p = g;
+        p.C = static_cast<float *>(workspace), p.ldc = N, p.bias = nullptr, p.c_split_stride = M * N;
+        rc = launch_tile<kBM, kBN, kBK, EPI_PLAIN>(trans_a, trans_b, vec, p, splits, st);
+        if (rc != ODL_OK)
+            return fail(rc, "sgemm: no kernel variant");
+        ODL_LAUNCH_CHECK();
+        const int64_t total = M * N;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st,
+                           static_cast<const float *>(workspace), splits, M * N, C, M, N, ldc,
+                           epi == EPI_BIAS_COL ? bias : nullptr);
+        ODL_LAUNCH_CHECK();
+        return ODL_OK;
+    }
+    if (epi == EPI_NCHW_ROWB)
+        rc = launch_tile<kBM, kBN, kBK, EPI_NCHW_ROWB>(trans_a, trans_b, vec, g, 1, st);
+    else if (epi == EPI_BIAS_COL && bias)
+        rc = launch_tile<kBM, kBN, kBK, EPI_BIAS_COL>(trans_a, trans_b, vec, g, 1, st);
+    else
+        rc = launch_tile<kBM, kBN, kBK, EPI_PLAIN>(trans_a, trans_b, vec, g, 1, st);
+    if (rc != ODL_OK)
+        return fail(rc, "sgemm: no kernel variant");
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+size_t sgemm_workspace(int64_t M, int64_t N, int64_t K, int split_k)
+{
+    const int s = pick_splits(M, N, K, split_k);
+    return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+}
+}  // namespace odl
+
+extern "C" {
+
+int odl_hip_sgemm(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                  const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int split_k, void *workspace,
+                  size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    return odl::sgemm_launch(trans_a, trans_b, M, N, K, A, lda, B, ldb, C, ldc, bias, bias ? EPI_BIAS_COL : EPI_PLAIN,
+                             0, split_k, workspace, workspace_bytes, odl::as_stream(stream));
+}
+
+size_t odl_hip_sgemm_workspace_bytes(int, int, int64_t M, int64_t N, int64_t K, int split_k)
+{
+    return odl::sgemm_workspace(M, N, K, split_k);
+}
+
+int odl_hip_matmul(const float *a, const float *b, float *c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                   int b_is_batched, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(batch >= 1, "matmul: batch must be >= 1");
+    if (!b_is_batched)  // [batch*M, K] x [K, N]: one GEMM, the batch folds into the rows
+        return odl::sgemm_launch(0, 0, batch * M, N, K, a, K, b, N, c, N, nullptr, EPI_PLAIN, 0, 1, nullptr, 0,
+                                 odl::as_stream(stream));
+    for (int64_t i = 0; i < batch; ++i)
+    {
+        int rc = odl::sgemm_launch(0, 0, M, N, K, a + i * M * K, K, b + i * K * N, N, c + i * M * N, N, nullptr,
+                                   EPI_PLAIN, 0, 1, nullptr, 0, odl::as_stream(stream));
+        if (rc != ODL_OK)
+            return rc;
+    }
+    return ODL_OK;
+}
+
+size_t odl_hip_matmul_backward_workspace_bytes(int64_t M, int64_t K, int64_t N)
+{
+    const size_t a = odl::sgemm_workspace(M, K, N, 0), b = odl::sgemm_workspace(K, N, M, 0);
+    return a > b ? a : b;
+}
+
+int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M, int64_t K,
+                            int64_t N, void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    hipStream_t st = odl::as_stream(stream);
+    if (gx)  // gx[M,K] = gy[M,N] . w[K,N]^T
+    {
+        int rc = odl::sgemm_launch(0, 1, M, K, N, gy, N, w, N, gx, K, nullptr, EPI_PLAIN, 0, 0, workspace,
+                                   workspace_bytes, st);
+        if (rc != ODL_OK)
+            return rc;
+    }
+    if (gw)  // gw[K,N] = x[M,K]^T . gy[M,N]
+    {
+        int rc = odl::sgemm_launch(1, 0, K, N, M, x, K, gy, N, gw, N, nullptr, EPI_PLAIN, 0, 0, workspace,
+                                   workspace_bytes, st);
+        if (rc != ODL_OK)
+            return rc;
+    }
+    return ODL_OK;
+}
+
+int odl_hip_transpose(const float *src, float *dst, int64_t outer, int64_t rows, int64_t cols, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    if (outer * rows * cols == 0)
+        return ODL_OK;
+    ODL_REQUIRE(outer > 0 && rows > 0 && cols > 0 && outer < 65536, "transpose: bad dimensions");
+    dim3 grid((unsigned)odl::ceil_div(cols, 32), (unsigned)odl::ceil_div(rows, 32), (unsigned)outer);
+    hipLaunchKernelGGL(transpose_kernel, grid, dim3(32, 8), 0, odl::as_stream(stream), src, dst, rows, cols);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+}  // extern "C"

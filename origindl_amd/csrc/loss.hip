@@ -1,0 +1,365 @@
+// Softmax, gather / one-hot and the fused softmax-cross-entropy forward and gradient, plus the host-argmax
+// metric done on the device. The reference builds softmax from eight separate Mat ops with materialised
+// broadcasts and syncs twice inside the loss (src/operators/activation/softmax.cpp:14-76,
+// src/operators/loss/softmax_cross_entropy.cpp:17-111); here a row of logits is read once by one wave,
+// reduced with wave64 shuffles and written once.
+#include <cfloat>
+#include <vector>
+
+#include "odl_common.h"
+
+namespace
+{
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / 64;
+
+__device__ inline float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__device__ inline float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        const float u = __shfl_xor(v, o, 64);
+        v = (v < u) ? u : v;
+    }
+    return v;
+}
+
+__device__ inline int64_t label_at(const void *idx, int is64, int64_t i)
+{
+    return is64 ? static_cast<const int64_t *>(idx)[i] : (int64_t) static_cast<const int32_t *>(idx)[i];
+}
+
+// row statistics of one contiguous row handled by one wave: max, then sum of exp(x - max)
+__device__ inline void row_stats(const float *row, int64_t C, int lane, float &mx, float &sum)
+{
+    float m = -FLT_MAX;
+    for (int64_t j = lane; j < C; j += 64)
+        m = (m < row[j]) ? row[j] : m;
+    m = wave_max(m);
+    float s = 0.f;
+    for (int64_t j = lane; j < C; j += 64)
+        s += expf(row[j] - m);
+    mx = m;
+    sum = wave_sum(s);
+}
+
+__global__ void softmax_rows_kernel(const float *__restrict__ x, float *__restrict__ y, int64_t N, int64_t C)
+{
+    const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (row >= N)
+        return;
+    const int lane = threadIdx.x & 63;
+    float m, s;
+    row_stats(x + row * C, C, lane, m, s);
+    for (int64_t j = lane; j < C; j += 64)
+        y[row * C + j] = expf(x[row * C + j] - m) / s;
+}
+
+// softmax along the middle axis of [outer, axis, inner], one thread per (outer, inner) pair
+__global__ void softmax_strided_kernel(const float *__restrict__ x, float *__restrict__ y, int64_t outer, int64_t axis,
+                                       int64_t inner)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= outer * inner)
+        return;
+    const int64_t o = t / inner, i = t % inner;
+    const float *p = x + o * axis * inner + i;
+    float *q = y + o * axis * inner + i;
+    float m = -FLT_MAX;
+    for (int64_t a = 0; a < axis; ++a)
+        m = (m < p[a * inner]) ? p[a * inner] : m;
+    float s = 0.f;
+    for (int64_t a = 0; a < axis; ++a)
+        s += expf(p[a * inner] - m);
+    for (int64_t a = 0; a < axis; ++a)
+        q[a * inner] = expf(p[a * inner] - m) / s;
+}
+
+__global__ void gather_kernel(const float *__restrict__ in, const void *idx, int is64, int64_t N, int64_t C,
+                              float *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= N)
+        return;
+    const int64_t t = label_at(idx, is64, i);
+    out[i] = (t >= 0 && t < C) ? in[i * C + t] : 0.f;
+}
+
+__global__ void one_hot_kernel(const void *idx, int is64, int64_t N, int64_t C, float *__restrict__ out)
+{
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= N * C)
+        return;
+    const int64_t i = e / C, j = e % C;
+    out[e] = (label_at(idx, is64, i) == j) ? 1.f : 0.f;  // out-of-range labels match no column (gather.cpp:134)
+}
+
+// logp[i] = log(softmax(x)[i, t_i] + 1e-8); flag[0] |= 1 when a label is out of range
+__global__ void ce_row_logp_kernel(const float *__restrict__ x, const void *t, int is64, int64_t N, int64_t C,
+                                   float *__restrict__ logp, int *flag)
+{
+    const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (row >= N)
+        return;
+    const int lane = threadIdx.x & 63;
+    float m, s;
+    row_stats(x + row * C, C, lane, m, s);
+    if (lane == 0)
+    {
+        const int64_t lab = label_at(t, is64, row);
+        if (lab < 0 || lab >= C)
+        {
+            atomicOr(flag, 1);
+            logp[row] = 0.f;
+        }
+        else
+        {
+            const float p = expf(x[row * C + lab] - m) / s;
+            logp[row] = logf(p + 1e-8f);
+        }
+    }
+}
+
+// out[0] = -(sum of logp) / N   (softmax_cross_entropy.cpp:67-70); one workgroup
+__global__ void ce_finish_kernel(const float *__restrict__ logp, int64_t N, float *out)
+{
+    __shared__ float part[1024 / 64];
+    float acc = 0.f;
+    for (int64_t i = threadIdx.x; i < N; i += blockDim.x)
+        acc += logp[i];
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        float s = 0.f;
+        for (unsigned i = 0; i < blockDim.x / 64; ++i)
+            s += part[i];
+        out[0] = -s / (float)N;
+    }
+}
+
+// gx = (softmax(x) - one_hot(t)) * scale, one wave per row, one read and one write of the row
+__global__ void ce_grad_kernel(const float *__restrict__ x, const void *t, int is64, int64_t N, int64_t C, float scale,
+                               float *__restrict__ gx)
+{
+    const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (row >= N)
+        return;
+    const int lane = threadIdx.x & 63;
+    float m, s;
+    row_stats(x + row * C, C, lane, m, s);
+    const int64_t lab = label_at(t, is64, row);
+    for (int64_t j = lane; j < C; j += 64)
+    {
+        const float p = expf(x[row * C + j] - m) / s;
+        const float d = p - ((j == lab) ? 1.f : 0.f);
+        gx[row * C + j] = d * scale;
+    }
+}
+
+// first maximum of each row (strict >), sequential like src/utils/metrics.cpp:42-53
+__global__ void argmax_rows_kernel(const float *__restrict__ y, int64_t N, int64_t C, int64_t *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= N)
+        return;
+    const float *p = y + i * C;
+    int64_t mi = 0;
+    float mv = p[0];
+    for (int64_t j = 1; j < C; ++j)
+        if (p[j] > mv)
+        {
+            mv = p[j];
+            mi = j;
+        }
+    out[i] = mi;
+}
+
+__global__ void accuracy_count_kernel(const float *__restrict__ y, const int32_t *__restrict__ t, int64_t N, int64_t C,
+                                      unsigned int *count)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= N)
+        return;
+    const float *p = y + i * C;
+    int64_t mi = 0;
+    float mv = p[0];
+    for (int64_t j = 1; j < C; ++j)
+        if (p[j] > mv)
+        {
+            mv = p[j];
+            mi = j;
+        }
+    const int32_t lab = t[i];
+    if (lab >= 0 && lab < (int32_t)C && (int64_t)lab == mi)  // metrics.cpp:56-59
+        atomicAdd(count, 1u);
+}
+
+__global__ void zero_words_kernel(unsigned int *p, int n)
+{
+    if ((int)threadIdx.x < n)
+        p[threadIdx.x] = 0u;
+}
+
+inline size_t align256(size_t b)
+{
+    return (b + 255) & ~(size_t)255;
+}
+}  // namespace
+
+extern "C" {
+
+int odl_hip_softmax(const float *x, int64_t outer, int64_t axis, int64_t inner, float *y, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, "softmax: negative extent");
+    if (outer * axis * inner == 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    if (inner == 1)
+        hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)odl::ceil_div(outer, kWaves)), dim3(kBlock), 0, st, x, y,
+                           outer, axis);
+    else
+        hipLaunchKernelGGL(softmax_strided_kernel, dim3((unsigned)odl::ceil_div(outer * inner, kBlock)), dim3(kBlock), 0,
+                           st, x, y, outer, axis, inner);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_gather(const float *in, const void *idx, int idx_is_i64, int64_t N, int64_t C, float *out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C >= 0, "gather: negative extent");
+    if (N == 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    // the labels are validated on the host before the launch, so that an out-of-range label can be reported
+    // the way the reference reports it (gather.cpp:64-67; the CUDA backend does the same D2H copy)
+    const size_t esz = idx_is_i64 ? 8 : 4;
+    std::vector<char> host((size_t)N * esz);
+    ODL_HIP_CHECK(hipMemcpyAsync(host.data(), idx, host.size(), hipMemcpyDeviceToHost, st));
+    ODL_HIP_CHECK(hipStreamSynchronize(st));
+    for (int64_t i = 0; i < N; ++i)
+    {
+        const int64_t t = idx_is_i64 ? reinterpret_cast<const int64_t *>(host.data())[i]
+                                     : (int64_t) reinterpret_cast<const int32_t *>(host.data())[i];
+        if (t < 0 || t >= C)
+            return odl::fail(ODL_ERR_INVALID_ARG, "gather: index %lld out of range [0, %lld)", (long long)t,
+                             (long long)C);
+    }
+    hipLaunchKernelGGL(gather_kernel, dim3((unsigned)odl::ceil_div(N, kBlock)), dim3(kBlock), 0, st, in, idx, idx_is_i64,
+                       N, C, out);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_one_hot(const void *idx, int idx_is_i64, int64_t N, int64_t C, float *out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0, "one_hot: negative extent");
+    ODL_REQUIRE(C > 0, "one_hot: num_classes must be positive, but got %lld", (long long)C);
+    if (N == 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(one_hot_kernel, dim3((unsigned)odl::ceil_div(N * C, kBlock)), dim3(kBlock), 0,
+                       odl::as_stream(stream), idx, idx_is_i64, N, C, out);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+size_t odl_hip_softmax_ce_loss_workspace_bytes(int64_t N)
+{
+    return align256((size_t)(N > 0 ? N : 0) * sizeof(float)) + 256;
+}
+
+int odl_hip_softmax_ce_loss(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float *host_loss,
+                            void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N > 0 && C > 0, "softmax_cross_entropy: empty input");
+    ODL_REQUIRE(host_loss != nullptr, "softmax_cross_entropy: null output");
+    const size_t need = odl_hip_softmax_ce_loss_workspace_bytes(N);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
+                "softmax_cross_entropy: workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    hipStream_t st = odl::as_stream(stream);
+    float *logp = static_cast<float *>(workspace);
+    // tail of the workspace: [0] loss (float), [1] out-of-range flag (int)
+    unsigned int *tail = reinterpret_cast<unsigned int *>(static_cast<char *>(workspace) + need - 256);
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, tail, 2);
+    ODL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(ce_row_logp_kernel, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, st, x, t,
+                       idx_is_i64, N, C, logp, reinterpret_cast<int *>(tail + 1));
+    ODL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(ce_finish_kernel, dim3(1), dim3(1024), 0, st, logp, N, reinterpret_cast<float *>(tail));
+    ODL_LAUNCH_CHECK();
+    unsigned int host_tail[2] = {0, 0};
+    ODL_HIP_CHECK(hipMemcpyAsync(host_tail, tail, sizeof(host_tail), hipMemcpyDeviceToHost, st));
+    ODL_HIP_CHECK(hipStreamSynchronize(st));
+    if (host_tail[1] != 0)
+        return odl::fail(ODL_ERR_INVALID_ARG, "gather: index out of range [0, %lld)", (long long)C);
+    float loss;
+    __builtin_memcpy(&loss, &host_tail[0], sizeof(float));
+    *host_loss = loss;
+    return ODL_OK;
+}
+
+int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float gy, float *gx,
+                            void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N > 0 && C > 0, "softmax_cross_entropy backward: empty input");
+    const float scale = gy / (float)N;  // softmax_cross_entropy.cpp:105-106
+    hipLaunchKernelGGL(ce_grad_kernel, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, odl::as_stream(stream),
+                       x, t, idx_is_i64, N, C, scale, gx);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_argmax_rows(const float *y, int64_t N, int64_t C, int64_t *out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C > 0, "argmax: bad shape");
+    if (N == 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)odl::ceil_div(N, kBlock)), dim3(kBlock), 0,
+                       odl::as_stream(stream), y, N, C, out);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+size_t odl_hip_accuracy_workspace_bytes(int64_t)
+{
+    return 256;
+}
+
+int odl_hip_accuracy(const float *y, const int32_t *t, int64_t N, int64_t C, float *host_acc, void *workspace,
+                     size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N > 0 && C > 0, "accuracy: empty input");
+    ODL_REQUIRE(host_acc != nullptr, "accuracy: null output");
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= 256, "accuracy: workspace of 256 bytes required");
+    hipStream_t st = odl::as_stream(stream);
+    unsigned int *count = static_cast<unsigned int *>(workspace);
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, count, 1);
+    ODL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(accuracy_count_kernel, dim3((unsigned)odl::ceil_div(N, kBlock)), dim3(kBlock), 0, st, y, t, N, C,
+                       count);
+    ODL_LAUNCH_CHECK();
+    unsigned int host_count = 0;
+    ODL_HIP_CHECK(hipMemcpyAsync(&host_count, count, sizeof(host_count), hipMemcpyDeviceToHost, st));
+    ODL_HIP_CHECK(hipStreamSynchronize(st));
+    *host_acc = (float)host_count / (float)N;  // metrics.cpp:64
+    return ODL_OK;
+}
+
+}  // extern "C"

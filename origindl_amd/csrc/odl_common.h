@@ -1,0 +1,58 @@
+// Shared helpers of the gfx950 backend: status codes, thread-local error text, launch checks.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/odl_hip.h"
+
+namespace odl
+{
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+// true when the current device is a gfx950 part; the kernels in this library are built for nothing else
+int require_device();
+
+// small fills as kernels (a memset node inside a captured graph is avoided on purpose)
+int fill_launch(float *dst, int64_t n, float value, hipStream_t st);
+int fill_bytes_launch(void *dst, int value, size_t bytes, hipStream_t st);
+
+inline hipStream_t as_stream(void *s)
+{
+    return reinterpret_cast<hipStream_t>(s);
+}
+
+inline int64_t ceil_div(int64_t a, int64_t b)
+{
+    return (a + b - 1) / b;
+}
+}  // namespace odl
+
+#define ODL_HIP_CHECK(expr)                                                                          \
+    do                                                                                               \
+    {                                                                                                \
+        hipError_t e__ = (expr);                                                                     \
+        if (e__ != hipSuccess)                                                                       \
+            return odl::fail(ODL_ERR_RUNTIME, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e__), \
+                             __FILE__, __LINE__);                                                    \
+    } while (0)
+
+// after a kernel launch: surfaces launch-configuration errors without synchronising
+#define ODL_LAUNCH_CHECK() ODL_HIP_CHECK(hipGetLastError())
+
+#define ODL_REQUIRE(cond, ...)                                   \
+    do                                                           \
+    {                                                            \
+        if (!(cond))                                             \
+            return odl::fail(ODL_ERR_INVALID_ARG, __VA_ARGS__);  \
+    } while (0)
+
+#define ODL_REQUIRE_DEVICE()             \
+    do                                   \
+    {                                    \
+        int rc__ = odl::require_device(); \
+        if (rc__ != ODL_OK)              \
+            return rc__;                 \
+    } while (0)

@@ -1,0 +1,134 @@
+// Max pooling forward (values + window-local uint64 indices) and backward.
+// Matches src/mat/origin/cpu/pooling/max_pool2d.cpp:40-224: the window scan starts at cell (0,0), moves
+// kh-major, replaces only on strict >, and padding cells count as 0.0 (the reference pools over a zero-padded
+// im2col buffer). The reference materialises that 6-D buffer (KH*KW times the input); here each output reads
+// its window straight from x, and the backward is a gather per input pixel that adds the matching upstream
+// gradients in ascending (kh, kw) — the order of the reference's col2im — so gx is bit-identical.
+#include "odl_common.h"
+
+namespace
+{
+struct PoolGeom
+{
+    int64_t N, C, H, W, OH, OW;
+    int KH, KW, SH, SW, PH, PW;
+};
+
+__global__ void max_pool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, uint64_t *__restrict__ idx,
+                                    PoolGeom g)
+{
+    const int64_t total = g.N * g.C * g.OH * g.OW;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    const int64_t ow = t % g.OW, oh = (t / g.OW) % g.OH, nc = t / (g.OW * g.OH);
+    const float *p = x + nc * g.H * g.W;
+    const int64_t h0 = oh * g.SH - g.PH, w0 = ow * g.SW - g.PW;
+    float mv = 0.f;
+    uint64_t mi = 0;
+    for (int kh = 0; kh < g.KH; ++kh)
+    {
+        const int64_t h = h0 + kh;
+        for (int kw = 0; kw < g.KW; ++kw)
+        {
+            const int64_t w = w0 + kw;
+            const float v = (h >= 0 && h < g.H && w >= 0 && w < g.W) ? p[h * g.W + w] : 0.f;
+            if ((kh | kw) == 0)
+                mv = v;  // max_pool2d.cpp:110-113
+            else if (v > mv)
+            {
+                mv = v;
+                mi = (uint64_t)(kh * g.KW + kw);
+            }
+        }
+    }
+    y[t] = mv;
+    if (idx)
+        idx[t] = mi;
+}
+
+__global__ void max_pool_bwd_kernel(const float *__restrict__ gy, const uint64_t *__restrict__ idx,
+                                    float *__restrict__ gx, PoolGeom g)
+{
+    const int64_t total = g.N * g.C * g.H * g.W;
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    const int64_t w = t % g.W, h = (t / g.W) % g.H, nc = t / (g.W * g.H);
+    float acc = 0.f;
+    for (int kh = 0; kh < g.KH; ++kh)
+    {
+        const int64_t hp = h + g.PH - kh;
+        if (hp < 0 || hp % g.SH != 0)
+            continue;
+        const int64_t oh = hp / g.SH;
+        if (oh >= g.OH)
+            continue;
+        for (int kw = 0; kw < g.KW; ++kw)
+        {
+            const int64_t wp = w + g.PW - kw;
+            if (wp < 0 || wp % g.SW != 0)
+                continue;
+            const int64_t ow = wp / g.SW;
+            if (ow >= g.OW)
+                continue;
+            const int64_t o = (nc * g.OH + oh) * g.OW + ow;
+            // the reference decodes the index with int arithmetic (max_pool2d.cpp:203-205)
+            if ((int)idx[o] == kh * g.KW + kw)
+                acc += gy[o];
+        }
+    }
+    gx[t] = acc;
+}
+
+int make_geom(PoolGeom &g, const char *who, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+              int PH, int PW)
+{
+    ODL_REQUIRE(N >= 0 && C >= 0 && H > 0 && W > 0, "%s: bad input shape", who);
+    ODL_REQUIRE(KH > 0 && KW > 0 && SH > 0 && SW > 0 && PH >= 0 && PW >= 0, "%s: bad kernel/stride/pad", who);
+    g = PoolGeom{N, C, H, W, (H + 2 * (int64_t)PH - KH) / SH + 1, (W + 2 * (int64_t)PW - KW) / SW + 1,
+                 KH, KW, SH, SW, PH, PW};
+    ODL_REQUIRE(g.OH > 0 && g.OW > 0, "%s: invalid output size OH=%lld, OW=%lld", who, (long long)g.OH,
+                (long long)g.OW);
+    return ODL_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int odl_hip_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+                       int PH, int PW, float *y, uint64_t *idx, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    PoolGeom g;
+    int rc = make_geom(g, "max_pool2d", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    const int64_t total = N * C * g.OH * g.OW;
+    if (total == 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(max_pool_fwd_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0,
+                       odl::as_stream(stream), x, y, idx, g);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N, int64_t C, int64_t H, int64_t W,
+                                int KH, int KW, int SH, int SW, int PH, int PW, float *gx, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    PoolGeom g;
+    int rc = make_geom(g, "max_pool2d_backward", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(idx != nullptr, "max_pool2d_backward: indices not found");
+    const int64_t total = N * C * H * W;
+    if (total == 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(max_pool_bwd_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0,
+                       odl::as_stream(stream), gy, idx, gx, g);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,648 @@
+// Reductions and broadcast of the backend: Mat::sum / sum_to / max / broadcast_to and the conv bias gradient.
+// All of them are bandwidth-bound streams over HBM: loads are coalesced (16 bytes per lane where the layout
+// allows), partial sums are combined with wave64 shuffles and one LDS hop, and long reductions are split over
+// enough workgroups to fill 256 CUs, the partials being summed by a second small kernel in a fixed order —
+// results do not depend on scheduling (no float atomics anywhere).
+// Behaviour matched: src/mat/origin/cpu/math/{sum,sum_to,max,broadcast}.cpp and
+// include/origin/mat/origin/device_common/operation_templates.h:259-495.
+#include <cfloat>
+
+#include "odl_common.h"
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace
+{
+constexpr int kBlock = 256;
+constexpr int64_t kTargetThreads = 1 << 18;
+
+inline size_t align256(size_t b)
+{
+    return (b + 255) & ~(size_t)255;
+}
+
+__device__ inline float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__device__ inline float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        const float u = __shfl_xor(v, o, 64);
+        v = (v < u) ? u : v;
+    }
+    return v;
+}
+
+// sum over the whole workgroup (kBlock threads); the result is valid in thread 0
+__device__ inline float block_sum(float v)
+{
+    __shared__ float part[kBlock / 64];
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float s = 0.f;
+    if (threadIdx.x == 0)
+        for (int i = 0; i < kBlock / 64; ++i)
+            s += part[i];
+    __syncthreads();
+    return s;
+}
+
+// ---- rows: src[rows][len] (len contiguous) -> dst[rows]; grid (splits, rows); dst index = row*splits + split
+__global__ void row_sum_block_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t len,
+                                     int64_t chunk)
+{
+    const int64_t row = blockIdx.y;
+    const int64_t beg = (int64_t)blockIdx.x * chunk;
+    const int64_t end = (beg + chunk < len) ? beg + chunk : len;
+    const float *p = src + row * len;
+    float acc = 0.f;
+    // 16-byte loads once the pointer is aligned; head and tail one float at a time
+    int64_t i = beg + threadIdx.x;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(p + beg);
+    int64_t head = ((16 - (addr & 15)) & 15) / 4;
+    if (head > end - beg)
+        head = end - beg;
+    if ((int64_t)threadIdx.x < head)
+        acc += p[i];
+    const int64_t vbeg = beg + head;
+    const int64_t nvec = (end - vbeg) / 4;
+    const f32x4 *pv = reinterpret_cast<const f32x4 *>(p + vbeg);
+    f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t v = threadIdx.x; v < nvec; v += kBlock)
+        a4 += pv[v];
+    acc += (a4[0] + a4[1]) + (a4[2] + a4[3]);
+    for (int64_t t = vbeg + nvec * 4 + threadIdx.x; t < end; t += kBlock)
+        acc += p[t];
+    const float s = block_sum(acc);
+    if (threadIdx.x == 0)
+        dst[row * gridDim.x + blockIdx.x] = s;
+}
+
+// one wave per row, for many short rows
+__global__ void row_sum_wave_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows, int64_t len)
+{
+    const int64_t row = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (row >= rows)
+        return;
+    const float *p = src + row * len;
+    float acc = 0.f;
+    for (int64_t i = threadIdx.x & 63; i < len; i += 64)
+        acc += p[i];
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0)
+        dst[row] = acc;
+}
+
+// ---- columns: src[outer][axis][inner] -> dst[split][outer][inner]; lanes run along `inner`
+template <int VEC>
+__global__ void col_sum_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t outer, int64_t axis,
+                               int64_t inner, int64_t chunk)
+{
+    const int64_t iq = inner / VEC;  // VEC == 4 only when inner % 4 == 0
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= outer * iq)
+        return;
+    const int64_t o = t / iq, i = (t % iq) * VEC;
+    const int64_t beg = (int64_t)blockIdx.y * chunk;
+    const int64_t end = (beg + chunk < axis) ? beg + chunk : axis;
+    const float *p = src + (o * axis) * inner + i;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+        acc[e] = 0.f;
+    int64_t a = beg;
+    for (; a + 4 <= end; a += 4)
+    {
+        float v[4][VEC];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+        {
+            if (VEC == 4)
+            {
+                const f32x4 q = *reinterpret_cast<const f32x4 *>(p + (a + u) * inner);
+                v[u][0] = q[0], v[u][1 % VEC] = q[1], v[u][2 % VEC] = q[2], v[u][3 % VEC] = q[3];
+            }
+            else
+                v[u][0] = p[(a + u) * inner];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                acc[e] += v[u][e];
+    }
+    for (; a < end; ++a)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+            acc[e] += p[a * inner + e];
+    float *d = dst + ((int64_t)blockIdx.y * outer + o) * inner + i;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+        d[e] = acc[e];
+}
+
+// dst[i] = sum over s (ascending) of part[s*n + i]
+__global__ void fold_partials_kernel(const float *__restrict__ part, float *__restrict__ dst, int64_t n, int splits)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n)
+        return;
+    float s = 0.f;
+    for (int z = 0; z < splits; ++z)
+        s += part[(int64_t)z * n + i];
+    dst[i] = s;
+}
+
+// ---- conv bias gradient: gy[N][OC][P] -> part[oc][nsplit]; grid (nsplit, OC)
+__global__ void nchw_channel_sum_kernel(const float *__restrict__ gy, float *__restrict__ part, int64_t N, int64_t OC,
+                                        int64_t P, int64_t nchunk)
+{
+    const int64_t oc = blockIdx.y;
+    const int64_t nb = (int64_t)blockIdx.x * nchunk;
+    const int64_t ne = (nb + nchunk < N) ? nb + nchunk : N;
+    float acc = 0.f;
+    const bool v4 = (P % 4 == 0) && (reinterpret_cast<uintptr_t>(gy) % 16 == 0);
+    for (int64_t n = nb; n < ne; ++n)
+    {
+        const float *p = gy + (n * OC + oc) * P;
+        if (v4)
+        {
+            const f32x4 *pv = reinterpret_cast<const f32x4 *>(p);
+            f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
+            for (int64_t v = threadIdx.x; v < P / 4; v += kBlock)
+                a4 += pv[v];
+            acc += (a4[0] + a4[1]) + (a4[2] + a4[3]);
+        }
+        else
+            for (int64_t i = threadIdx.x; i < P; i += kBlock)
+                acc += p[i];
+    }
+    const float s = block_sum(acc);
+    if (threadIdx.x == 0)
+        part[oc * gridDim.x + blockIdx.x] = s;
+}
+
+// ---- max
+__global__ void row_max_wave_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows, int64_t len)
+{
+    const int64_t row = (int64_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (row >= rows)
+        return;
+    const float *p = src + row * len;
+    float m = -FLT_MAX;  // std::numeric_limits<float>::lowest(), max.cpp:96
+    for (int64_t i = threadIdx.x & 63; i < len; i += 64)
+        m = (m < p[i]) ? p[i] : m;
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0)
+        dst[row] = m;
+}
+
+__global__ void col_max_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t outer, int64_t axis,
+                               int64_t inner)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= outer * inner)
+        return;
+    const int64_t o = t / inner, i = t % inner;
+    const float *p = src + o * axis * inner + i;
+    float m = -FLT_MAX;
+    for (int64_t a = 0; a < axis; ++a)
+        m = (m < p[a * inner]) ? p[a * inner] : m;
+    dst[t] = m;
+}
+
+__global__ void max_all_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t n)
+{
+    __shared__ float part[1024 / 64];
+    float m = src[0];  // max.cpp:30-35 starts from the first element
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x)
+        m = (m < src[i]) ? src[i] : m;
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        for (unsigned i = 1; i < blockDim.x / 64; ++i)
+            m = (m < part[i]) ? part[i] : m;
+        dst[0] = m;
+    }
+}
+
+// ---- broadcast: right-aligned, a source dim of size 1 reads index 0
+struct BcastDims
+{
+    int nd;
+    int64_t dshape[8];
+    int64_t sstride[8];  // 0 where the source dim is 1 or absent
+};
+
+__global__ void broadcast_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t total, BcastDims d)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    int64_t r = t, si = 0;
+    for (int k = d.nd - 1; k >= 0; --k)
+    {
+        si += (r % d.dshape[k]) * d.sstride[k];
+        r /= d.dshape[k];
+    }
+    dst[t] = src[si];
+}
+
+int64_t prod(const int64_t *s, int n)
+{
+    int64_t p = 1;
+    for (int i = 0; i < n; ++i)
+        p *= s[i];
+    return p;
+}
+
+// how a [outer, axis, inner] sum is scheduled
+struct SumPlan
+{
+    bool rows;      // inner == 1
+    bool wave_rows; // many short rows: one wave each, no workspace
+    int splits;
+    int64_t chunk;
+    size_t ws_bytes;
+};
+
+SumPlan plan_sum(int64_t outer, int64_t axis, int64_t inner)
+{
+    SumPlan p{};
+    p.rows = (inner == 1);
+    if (p.rows)
+    {
+        if (outer >= 1024 || axis <= 2048)
+        {
+            p.wave_rows = true;
+            p.splits = 1;
+            return p;
+        }
+        int64_t s = odl::ceil_div(1024, outer);
+        const int64_t max_s = odl::ceil_div(axis, 4096);
+        if (s > max_s)
+            s = max_s;
+        if (s < 1)
+            s = 1;
+        p.chunk = odl::ceil_div(odl::ceil_div(axis, s), 4) * 4;
+        p.splits = (int)odl::ceil_div(axis, p.chunk);
+        p.ws_bytes = p.splits > 1 ? (size_t)(outer * p.splits) * sizeof(float) : 0;
+        return p;
+    }
+    const int64_t vec = (inner % 4 == 0) ? 4 : 1;
+    const int64_t cols = outer * (inner / vec);
+    int64_t s = kTargetThreads / (cols > 0 ? cols : 1);
+    if (s > axis / 16)
+        s = axis / 16;
+    if (s < 1)
+        s = 1;
+    if (s > 1024)
+        s = 1024;
+    p.chunk = odl::ceil_div(axis, s);
+    p.splits = (int)odl::ceil_div(axis, p.chunk > 0 ? p.chunk : 1);
+    if (p.splits < 1)
+        p.splits = 1;
+    p.ws_bytes = p.splits > 1 ? (size_t)p.splits * outer * inner * sizeof(float) : 0;
+    return p;
+}
+
+int sum_axis_launch(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *workspace,
+                    size_t workspace_bytes, hipStream_t st)
+{
+    const int64_t nout = outer * inner;
+    if (nout == 0)
+        return ODL_OK;
+    if (axis == 0)
+    {
+        return odl::fill_launch(dst, nout, 0.f, st);
+    }
+    SumPlan p = plan_sum(outer, axis, inner);
+    if (p.splits > 1 && (workspace == nullptr || workspace_bytes < p.ws_bytes))
+        return odl::fail(ODL_ERR_INVALID_ARG, "sum: workspace of %zu bytes required, got %zu", p.ws_bytes,
+                         workspace_bytes);
+    if (p.rows)
+    {
+        if (p.wave_rows)
+        {
+            hipLaunchKernelGGL(row_sum_wave_kernel, dim3((unsigned)odl::ceil_div(outer, kBlock / 64)), dim3(kBlock), 0,
+                               st, src, dst, outer, axis);
+            ODL_LAUNCH_CHECK();
+            return ODL_OK;
+        }
+        ODL_REQUIRE(outer < 65536, "sum: too many rows for the split schedule");
+        float *part = p.splits > 1 ? static_cast<float *>(workspace) : dst;
+        hipLaunchKernelGGL(row_sum_block_kernel, dim3((unsigned)p.splits, (unsigned)outer), dim3(kBlock), 0, st, src,
+                           part, axis, p.chunk);
+        ODL_LAUNCH_CHECK();
+        if (p.splits > 1)
+        {
+            hipLaunchKernelGGL(row_sum_wave_kernel, dim3((unsigned)odl::ceil_div(outer, kBlock / 64)), dim3(kBlock), 0,
+                               st, part, dst, outer, (int64_t)p.splits);
+            ODL_LAUNCH_CHECK();
+        }
+        return ODL_OK;
+    }
+    const bool v4 = (inner % 4 == 0) && (reinterpret_cast<uintptr_t>(src) % 16 == 0);
+    const int64_t threads = outer * (v4 ? inner / 4 : inner);
+    float *part = p.splits > 1 ? static_cast<float *>(workspace) : dst;
+    const dim3 grid((unsigned)odl::ceil_div(threads, kBlock), (unsigned)p.splits);
+    if (v4)
+        hipLaunchKernelGGL(col_sum_kernel<4>, grid, dim3(kBlock), 0, st, src, part, outer, axis, inner, p.chunk);
+    else
+        hipLaunchKernelGGL(col_sum_kernel<1>, grid, dim3(kBlock), 0, st, src, part, outer, axis, inner, p.chunk);
+    ODL_LAUNCH_CHECK();
+    if (p.splits > 1)
+    {
+        hipLaunchKernelGGL(fold_partials_kernel, dim3((unsigned)odl::ceil_div(nout, kBlock)), dim3(kBlock), 0, st, part,
+                           dst, nout, p.splits);
+        ODL_LAUNCH_CHECK();
+    }
+    return ODL_OK;
+}
+
+// sum_to.cpp:36-72: which dims are reduced (LEFT-aligned), and the [outer,axis,inner] passes that do it,
+// one per maximal run of adjacent reduced dims, last run first so earlier extents stay valid.
+struct SumToPlan
+{
+    int rc;  // ODL_OK, or the error the reference would throw
+    bool copy;
+    int npass;
+    int64_t outer[8], axis[8], inner[8];
+    size_t ws_bytes;  // two ping-pong intermediates + the largest per-pass workspace
+    size_t inter_bytes;
+    size_t pass_ws;
+};
+
+SumToPlan plan_sum_to(const int64_t *ss, int sn, const int64_t *ts, int tn)
+{
+    SumToPlan p{};
+    p.rc = ODL_OK;
+    if (sn > 8 || tn > 8 || sn < 0 || tn < 0)
+    {
+        p.rc = ODL_ERR_INVALID_ARG;
+        return p;
+    }
+    bool same = (sn == tn);
+    for (int i = 0; same && i < sn; ++i)
+        same = (ss[i] == ts[i]);
+    if (same)
+    {
+        p.copy = true;
+        return p;
+    }
+    const int64_t se = prod(ss, sn), te = prod(ts, tn);
+    if (te > se)
+    {
+        p.rc = ODL_ERR_RUNTIME;  // sum_to.cpp:24-28
+        return p;
+    }
+    bool red[8] = {false};
+    const int mind = sn < tn ? sn : tn;
+    for (int i = 0; i < mind; ++i)
+        red[i] = (ts[i] == 1 && ss[i] > 1);
+    for (int i = tn; i < sn; ++i)
+        red[i] = true;
+    int64_t kept = 1;
+    for (int i = 0; i < sn; ++i)
+        if (!red[i])
+            kept *= ss[i];
+    if (kept != te)
+    {
+        p.rc = ODL_ERR_INVALID_ARG;  // the final reshape throws
+        return p;
+    }
+    int64_t cur[8];
+    for (int i = 0; i < sn; ++i)
+        cur[i] = ss[i];
+    int i = sn - 1;
+    size_t inter = 0;
+    while (i >= 0)
+    {
+        if (!red[i])
+        {
+            --i;
+            continue;
+        }
+        int j = i;
+        while (j - 1 >= 0 && red[j - 1])
+            --j;
+        const int q = p.npass++;
+        p.outer[q] = prod(cur, j);
+        p.axis[q]  = prod(cur + j, i - j + 1);
+        p.inner[q] = prod(cur + i + 1, sn - i - 1);
+        for (int d = j; d <= i; ++d)
+            cur[d] = 1;
+        const size_t w = plan_sum(p.outer[q], p.axis[q], p.inner[q]).ws_bytes;
+        if (w > p.pass_ws)
+            p.pass_ws = w;
+        const size_t ob = (size_t)(p.outer[q] * p.inner[q]) * sizeof(float);
+        if (ob > inter)
+            inter = ob;
+        i = j - 1;
+    }
+    p.inter_bytes = p.npass > 1 ? align256(inter) : 0;
+    p.ws_bytes = 2 * p.inter_bytes + align256(p.pass_ws);
+    return p;
+}
+}  // namespace
+
+namespace odl
+{
+size_t sum_nchw_channels_workspace(int64_t N, int64_t OC, int64_t P)
+{
+    (void)P;
+    int64_t ns = ceil_div(1024, OC > 0 ? OC : 1);
+    if (ns > N)
+        ns = N;
+    if (ns < 1)
+        ns = 1;
+    return (size_t)(OC * ns) * sizeof(float);
+}
+
+int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
+                             size_t workspace_bytes, hipStream_t st)
+{
+    if (OC == 0)
+        return ODL_OK;
+    ODL_REQUIRE(N >= 0 && OC > 0 && OC < 65536 && P >= 0, "conv bias gradient: bad shape");
+    int64_t ns = ceil_div(1024, OC);
+    if (ns > N)
+        ns = N;
+    if (ns < 1)
+        ns = 1;
+    const int64_t nchunk = ceil_div(N > 0 ? N : 1, ns);
+    ns = ceil_div(N > 0 ? N : 1, nchunk);
+    const size_t need = (size_t)(OC * ns) * sizeof(float);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
+                "conv bias gradient: workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    float *part = static_cast<float *>(workspace);
+    hipLaunchKernelGGL(nchw_channel_sum_kernel, dim3((unsigned)ns, (unsigned)OC), dim3(kBlock), 0, st, gy, part, N, OC,
+                       P, nchunk);
+    ODL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(row_sum_wave_kernel, dim3((unsigned)ceil_div(OC, kBlock / 64)), dim3(kBlock), 0, st, part, gb, OC,
+                       ns);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace odl
+
+extern "C" {
+
+size_t odl_hip_sum_axis_workspace_bytes(int64_t outer, int64_t axis, int64_t inner)
+{
+    if (outer <= 0 || axis <= 0 || inner <= 0)
+        return 0;
+    return plan_sum(outer, axis, inner).ws_bytes;
+}
+
+int odl_hip_sum_axis(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *workspace,
+                     size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, "sum: negative extent");
+    return sum_axis_launch(src, outer, axis, inner, dst, workspace, workspace_bytes, odl::as_stream(stream));
+}
+
+size_t odl_hip_sum_all_workspace_bytes(int64_t n)
+{
+    return odl_hip_sum_axis_workspace_bytes(1, n, 1);
+}
+
+int odl_hip_sum_all(const float *src, int64_t n, float *dst, void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(n >= 0, "sum: negative extent");
+    return sum_axis_launch(src, 1, n, 1, dst, workspace, workspace_bytes, odl::as_stream(stream));
+}
+
+int odl_hip_max_axis(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, "max: negative extent");
+    if (outer * inner == 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    if (inner == 1)
+        hipLaunchKernelGGL(row_max_wave_kernel, dim3((unsigned)odl::ceil_div(outer, kBlock / 64)), dim3(kBlock), 0, st,
+                           src, dst, outer, axis);
+    else
+        hipLaunchKernelGGL(col_max_kernel, dim3((unsigned)odl::ceil_div(outer * inner, kBlock)), dim3(kBlock), 0, st,
+                           src, dst, outer, axis, inner);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_max_all(const float *src, int64_t n, float *dst, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(n > 0, "max: empty input");
+    hipLaunchKernelGGL(max_all_kernel, dim3(1), dim3(1024), 0, odl::as_stream(stream), src, dst, n);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+size_t odl_hip_sum_to_workspace_bytes(const int64_t *host_src_shape, int src_ndim, const int64_t *host_dst_shape,
+                                      int dst_ndim)
+{
+    const SumToPlan p = plan_sum_to(host_src_shape, src_ndim, host_dst_shape, dst_ndim);
+    return p.rc == ODL_OK ? p.ws_bytes : 0;
+}
+
+int odl_hip_sum_to(const float *src, const int64_t *host_src_shape, int src_ndim, const int64_t *host_dst_shape,
+                   int dst_ndim, float *dst, void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    hipStream_t st = odl::as_stream(stream);
+    const SumToPlan p = plan_sum_to(host_src_shape, src_ndim, host_dst_shape, dst_ndim);
+    if (p.rc == ODL_ERR_RUNTIME)
+        return odl::fail(ODL_ERR_RUNTIME, "sum_to: Target shape cannot have more elements than source tensor");
+    if (p.rc != ODL_OK)
+        return odl::fail(p.rc, "sum_to: source shape cannot be reduced to the target shape (left-aligned rule)");
+    if (p.copy)
+    {
+        const int64_t n = prod(host_src_shape, src_ndim);
+        if (n && dst != src)
+            ODL_HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)n * sizeof(float), hipMemcpyDeviceToDevice, st));
+        return ODL_OK;
+    }
+    if (p.npass == 0)  // only size-1 dims differ: a reshape
+    {
+        const int64_t n = prod(host_src_shape, src_ndim);
+        if (n && dst != src)
+            ODL_HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)n * sizeof(float), hipMemcpyDeviceToDevice, st));
+        return ODL_OK;
+    }
+    ODL_REQUIRE(p.ws_bytes == 0 || (workspace != nullptr && workspace_bytes >= p.ws_bytes),
+                "sum_to: workspace of %zu bytes required, got %zu", p.ws_bytes, workspace_bytes);
+    char *ws = static_cast<char *>(workspace);
+    float *inter[2] = {reinterpret_cast<float *>(ws), reinterpret_cast<float *>(ws + p.inter_bytes)};
+    void *pass_ws = ws + 2 * p.inter_bytes;
+    const float *cur = src;
+    for (int q = 0; q < p.npass; ++q)
+    {
+        float *out = (q == p.npass - 1) ? dst : inter[q & 1];
+        int rc = sum_axis_launch(cur, p.outer[q], p.axis[q], p.inner[q], out, pass_ws, p.pass_ws, st);
+        if (rc != ODL_OK)
+            return rc;
+        cur = out;
+    }
+    return ODL_OK;
+}
+
+size_t odl_hip_sum_nchw_channels_workspace_bytes(int64_t N, int64_t OC, int64_t P)
+{
+    return odl::sum_nchw_channels_workspace(N, OC, P);
+}
+
+int odl_hip_sum_nchw_channels(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
+                              size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    return odl::sum_nchw_channels_launch(gy, N, OC, P, gb, workspace, workspace_bytes, odl::as_stream(stream));
+}
+
+int odl_hip_broadcast_to(const float *src, const int64_t *host_src_shape, int src_ndim, const int64_t *host_dst_shape,
+                         int dst_ndim, float *dst, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(src_ndim >= 0 && dst_ndim >= 0 && src_ndim <= 8 && dst_ndim <= 8, "broadcast_to: at most 8 dims");
+    ODL_REQUIRE(src_ndim <= dst_ndim, "broadcast_to: source has more dims than the target");
+    BcastDims d{};
+    d.nd = dst_ndim;
+    int64_t st = 1;
+    for (int i = 0; i < dst_ndim; ++i)
+    {
+        const int dd = dst_ndim - 1 - i, sd = src_ndim - 1 - i;
+        d.dshape[dd] = host_dst_shape[dd];
+        d.sstride[dd] = 0;
+        if (sd >= 0)
+        {
+            const int64_t ssz = host_src_shape[sd];
+            ODL_REQUIRE(ssz == 1 || ssz == host_dst_shape[dd], "broadcast_to: dim %d of size %lld cannot become %lld", sd,
+                        (long long)ssz, (long long)host_dst_shape[dd]);
+            d.sstride[dd] = (ssz == 1) ? 0 : st;
+            st *= ssz;
+        }
+    }
+    const int64_t total = prod(host_dst_shape, dst_ndim);
+    if (total == 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(broadcast_kernel, dim3((unsigned)odl::ceil_div(total, kBlock)), dim3(kBlock), 0,
+                       odl::as_stream(stream), src, dst, total, d);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+}  // extern "C"

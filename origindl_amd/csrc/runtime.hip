@@ -1,0 +1,171 @@
+// Device runtime entry points of the C ABI: device selection, memory, copies, error text.
+// They stand where the reference's CUDAAllocator / Storage / origin::cuda::* device API make their
+// runtime calls (src/mat/origin/memory/allocator.cpp:53-107, storage.cpp:69-145, cuda/cuda_utils.cu:37-91).
+#include <cstring>
+
+#include "odl_common.h"
+
+namespace
+{
+thread_local char g_error[512] = "";
+}
+
+namespace odl
+{
+void set_error(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int require_device()
+{
+    // one check per device; the kernels are compiled for gfx950 only and there is no other code path
+    static int checked[64] = {0};  // 0 unknown, 1 ok, -1 wrong architecture
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0)
+        return fail(ODL_ERR_RUNTIME, "no HIP device available: %s", hipGetErrorString(e));
+    if (dev < 64 && checked[dev] == 1)
+        return ODL_OK;
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess)
+        return fail(ODL_ERR_RUNTIME, "hipGetDeviceProperties failed: %s", hipGetErrorString(e));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    {
+        if (dev < 64)
+            checked[dev] = -1;
+        return fail(ODL_ERR_RUNTIME, "device %d is %s; this library contains gfx950 code only", dev, prop.gcnArchName);
+    }
+    if (dev < 64)
+        checked[dev] = 1;
+    return ODL_OK;
+}
+}  // namespace odl
+
+extern "C" {
+
+const char *odl_hip_last_error(void)
+{
+    return g_error;
+}
+
+int odl_hip_device_count(int *count)
+{
+    ODL_REQUIRE(count != nullptr, "device_count: null output");
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess)
+    {
+        (void)hipGetLastError();
+        n = 0;
+    }
+    *count = n;
+    return ODL_OK;
+}
+
+int odl_hip_set_device(int device)
+{
+    ODL_HIP_CHECK(hipSetDevice(device));
+    return ODL_OK;
+}
+
+int odl_hip_get_device(int *device)
+{
+    ODL_REQUIRE(device != nullptr, "get_device: null output");
+    ODL_HIP_CHECK(hipGetDevice(device));
+    return ODL_OK;
+}
+
+int odl_hip_synchronize(void)
+{
+    ODL_HIP_CHECK(hipDeviceSynchronize());
+    return ODL_OK;
+}
+
+int odl_hip_device_info(int device, char *buf, size_t len)
+{
+    ODL_REQUIRE(buf != nullptr && len > 0, "device_info: null buffer");
+    hipDeviceProp_t prop;
+    ODL_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+    snprintf(buf, len, "%s | %s | %d CUs | %d MHz | %zu MiB", prop.name, prop.gcnArchName, prop.multiProcessorCount,
+             prop.clockRate / 1000, (size_t)(prop.totalGlobalMem >> 20));
+    return ODL_OK;
+}
+
+int odl_hip_malloc(void **ptr, size_t bytes)
+{
+    ODL_REQUIRE(ptr != nullptr, "malloc: null output");
+    *ptr = nullptr;
+    if (bytes == 0)
+        return ODL_OK;
+    hipError_t e = hipMalloc(ptr, bytes);
+    if (e != hipSuccess)
+    {
+        size_t fr = 0, tot = 0;
+        (void)hipMemGetInfo(&fr, &tot);  // the reference reports free/total on OOM (allocator.cpp:69-80)
+        return odl::fail(ODL_ERR_RUNTIME, "hipMalloc(%zu) failed: %s (free %zu MiB of %zu MiB)", bytes,
+                         hipGetErrorString(e), fr >> 20, tot >> 20);
+    }
+    return ODL_OK;
+}
+
+int odl_hip_free(void *ptr)
+{
+    if (ptr)
+        ODL_HIP_CHECK(hipFree(ptr));
+    return ODL_OK;
+}
+
+int odl_hip_mem_info(size_t *free_bytes, size_t *total_bytes)
+{
+    size_t fr = 0, tot = 0;
+    ODL_HIP_CHECK(hipMemGetInfo(&fr, &tot));
+    if (free_bytes)
+        *free_bytes = fr;
+    if (total_bytes)
+        *total_bytes = tot;
+    return ODL_OK;
+}
+
+int odl_hip_memcpy_h2d(void *dst, const void *host_src, size_t bytes)
+{
+    if (bytes)
+        ODL_HIP_CHECK(hipMemcpy(dst, host_src, bytes, hipMemcpyHostToDevice));
+    return ODL_OK;
+}
+
+int odl_hip_memcpy_d2h(void *host_dst, const void *src, size_t bytes)
+{
+    if (bytes)
+    {
+        ODL_HIP_CHECK(hipDeviceSynchronize());  // storage.cpp:100-101
+        ODL_HIP_CHECK(hipMemcpy(host_dst, src, bytes, hipMemcpyDeviceToHost));
+    }
+    return ODL_OK;
+}
+
+int odl_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream)
+{
+    if (bytes)
+        ODL_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, odl::as_stream(stream)));
+    return ODL_OK;
+}
+
+int odl_hip_memset(void *dst, int value, size_t bytes, void *stream)
+{
+    return odl::fill_bytes_launch(dst, value, bytes, odl::as_stream(stream));
+}
+
+}  // extern "C"

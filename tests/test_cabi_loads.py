@@ -1,0 +1,53 @@
+"""CPU-side checks of the boundary: the header parses, the built library exports every declared symbol,
+argument validation that needs no GPU behaves, and compute entry points refuse to run without a device."""
+import ctypes
+import os
+
+import pytest
+
+from origindl_amd import _lib
+
+
+def test_header_declares_the_expected_surface():
+    protos = _lib.parse_header()
+    for name in ("odl_hip_sgemm", "odl_hip_matmul", "odl_hip_matmul_backward", "odl_hip_im2col", "odl_hip_col2im",
+                 "odl_hip_conv2d", "odl_hip_conv2d_backward", "odl_hip_sum_axis", "odl_hip_sum_all", "odl_hip_sum_to",
+                 "odl_hip_sum_nchw_channels", "odl_hip_broadcast_to", "odl_hip_max_axis", "odl_hip_softmax",
+                 "odl_hip_gather", "odl_hip_one_hot", "odl_hip_softmax_ce_loss", "odl_hip_softmax_ce_grad",
+                 "odl_hip_max_pool2d", "odl_hip_max_pool2d_backward", "odl_hip_argmax_rows", "odl_hip_accuracy",
+                 "odl_hip_binary", "odl_hip_unary", "odl_hip_pow_scalar", "odl_hip_fill", "odl_hip_malloc",
+                 "odl_hip_free", "odl_hip_memcpy_h2d", "odl_hip_memcpy_d2h", "odl_hip_device_count",
+                 "odl_hip_last_error"):
+        assert name in protos, name
+    ret, args = protos["odl_hip_sgemm"]
+    assert ret is ctypes.c_int and len(args) == 16
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(_lib.LIB_PATH), "build the library first: python -m origindl_amd.build"
+    cdll = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _lib.parse_header():
+        assert hasattr(cdll, name), "%s declared in include/odl_hip.h but not exported" % name
+
+
+def test_workspace_queries_need_no_gpu():
+    l = _lib.lib()
+    # conv C1 of the benchmark: col matrix [100352, 576] floats
+    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) == 100352 * 576 * 4
+    assert l.query("odl_hip_conv2d_workspace_bytes", 1, 1, 2, 2, 1, 3, 3, 1, 1, 0, 0) == 0  # no valid output
+    assert l.query("odl_hip_sum_axis_workspace_bytes", 4096, 10, 1) == 0
+    assert l.query("odl_hip_sum_axis_workspace_bytes", 1, 16384, 4096) > 0
+    src = (ctypes.c_int64 * 2)(512, 1000)
+    dst = (ctypes.c_int64 * 2)(1, 1000)
+    assert l.query("odl_hip_sum_to_workspace_bytes", src, 2, dst, 2) >= 0
+
+
+def test_compute_refuses_to_run_without_a_gpu():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    l = _lib.lib()
+    rc = l.cdll.odl_hip_fill(None, 4, ctypes.c_float(1.0), None)
+    assert rc == _lib.ODL_ERR_RUNTIME and "HIP device" in l.last_error()
+    with pytest.raises(_lib.OdlRuntimeError):
+        l.call("odl_hip_sgemm", 0, 0, 4, 4, 4, None, 4, None, 4, None, 4, None, 0, None, 0, None)

@@ -1,0 +1,542 @@
+"""GPU parity: every entry point of the C ABI against the CPU oracle on the same seeded inputs, against the
+fixtures written from the compiled reference, and — at the benchmark's full sizes, where the oracle cannot
+finish — through sampled rows and size-independent properties.
+
+Bars (from the benchmark contract): integer/index outputs bit-exact; FP32 GEMM-type outputs within
+|d| <= 1e-5 * ||a_row||_2 * ||b_col||_2 per element; plain sums within the same bound read as a dot product with
+a vector of ones; softmax/CE within 1e-6 absolute (exp/log of the device library vs glibc); copies, gathers,
+col2im and max-pool backward bit-exact (same additions in the same order)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oraclelib as ol
+
+pytestmark = pytest.mark.gpu
+
+f32 = np.float32
+G = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_vectors.npz"))
+
+
+@pytest.fixture(scope="module")
+def api():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from origindl_amd import capi
+    assert capi.is_available()
+    print("\n[device]", capi.device_info(0), flush=True)
+    return capi
+
+
+@pytest.fixture(scope="module")
+def o():
+    return ol.oracle()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def gemm_bound(a, b):
+    """1e-5 * ||a_row|| * ||b_col|| for C = a @ b (a [M,K], b [K,N])."""
+    return 1e-5 * np.outer(np.linalg.norm(a.astype(np.float64), axis=1), np.linalg.norm(b.astype(np.float64), axis=0))
+
+
+def assert_gemm_close(got, want, a, b, what):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    bound = gemm_bound(a, b) + 1e-30
+    worst = float((err / bound).max())
+    assert worst <= 1.0, "%s: max |d| / (1e-5 |a_row||b_col|) = %.3f" % (what, worst)
+
+
+# --------------------------------------------------------------------------------------------- GEMM
+GEMM_SHAPES = [(128, 128, 128), (256, 384, 128), (64, 100, 10), (33, 47, 29), (512, 784, 1000), (512, 1000, 10),
+               (1, 5, 1), (130, 16, 260), (4, 1000, 4), (257, 129, 131)]
+
+
+@pytest.mark.parametrize("m,k,n", GEMM_SHAPES)
+def test_matmul_forward_backward_vs_oracle(api, o, m, k, n):
+    print("\n[case] matmul fwd+bwd", m, k, n, flush=True)
+    rng = np.random.default_rng(m * 7 + k * 3 + n)
+    x, w, gy = (rng.standard_normal(s, dtype=f32) for s in ((m, k), (k, n), (m, n)))
+    y = host(api.mat_mul(dev(x), dev(w)))
+    gx, gw = (host(t) for t in api.mat_mul_backward(dev(x), dev(w), dev(gy)))
+    # the full oracle is O(mnk) scalar work: sample rows for the largest shapes
+    rows = np.arange(m) if m * k * n < 3e7 else np.sort(rng.choice(m, 24, replace=False))
+    yo = np.empty((len(rows), n), f32)
+    for i, r in enumerate(rows):
+        o.orc_matmul_rows(x, w, yo[i:i + 1], int(r), int(r) + 1, n, k)
+    assert_gemm_close(y[rows], yo, x[rows], w, "C")
+    # gx rows are independent too: gx[r] = gy[r] . w^T
+    wT = np.ascontiguousarray(w.T)
+    gxo = np.empty((len(rows), k), f32)
+    for i, r in enumerate(rows):
+        o.orc_matmul_rows(gy, wT, gxo[i:i + 1], int(r), int(r) + 1, k, n)
+    assert_gemm_close(gx[rows], gxo, gy[rows], wT, "dA")
+    # gw[K,N] = x^T . gy: rows of gw are columns of x
+    xT = np.ascontiguousarray(x.T)
+    krows = np.arange(k) if m * k * n < 3e7 else np.sort(rng.choice(k, 24, replace=False))
+    gwo = np.empty((len(krows), n), f32)
+    for i, r in enumerate(krows):
+        o.orc_matmul_rows(xT, gy, gwo[i:i + 1], int(r), int(r) + 1, n, m)
+    assert_gemm_close(gw[krows], gwo, xT[krows], gy, "dB")
+
+
+def test_matmul_reference_unit_test_vectors(api):
+    # tests/unit_test/operator/test_matmul.cpp:19-64, 119-143, 213-229
+    x, w = dev(np.array([[1, 2], [3, 4]], f32)), dev(np.array([[5, 6], [7, 8]], f32))
+    assert host(api.mat_mul(x, w)).ravel().tolist() == [19, 22, 43, 50]
+    gx, gw = api.mat_mul_backward(x, w, dev(np.ones((2, 2), f32)))
+    assert host(gx).ravel().tolist() == [11, 15, 11, 15] and host(gw).ravel().tolist() == [4, 4, 6, 6]
+    a = dev(np.arange(1, 7, dtype=f32).reshape(2, 3))
+    b = dev(np.arange(7, 13, dtype=f32).reshape(3, 2))
+    assert host(api.mat_mul(a, b)).ravel().tolist() == [58, 64, 139, 154]
+    assert (host(api.mat_mul(dev(np.ones((10, 10), f32)), dev(np.ones((10, 10), f32)))) == 10).all()
+    with pytest.raises(api.OdlInvalidArgument):  # test_matmul.cpp:337-355
+        api.mat_mul(dev(np.ones((2, 3), f32)), dev(np.ones((2, 3), f32)))
+
+
+@pytest.mark.parametrize("size", [512, 1024, 2048])
+def test_matmul_all_ones_gives_k(api, size):
+    # tests/unit_test/operator/test_matmul.cpp:359-421 (device-only): ones(M,K) @ ones(K,N) == K exactly
+    print("\n[case] ones", size, flush=True)
+    a = torch.ones((size, size), device="cuda")
+    assert bool((api.mat_mul(a, a) == float(size)).all())
+    a = torch.ones((512, 1024), device="cuda")
+    b = torch.ones((1024, 2048), device="cuda")
+    assert bool((api.mat_mul(a, b) == 1024.0).all())
+    assert api.mat_mul(torch.ones((1, 1000), device="cuda"), torch.ones((1000, 1), device="cuda")).item() == 1000.0
+
+
+def test_matmul_batched(api, o):
+    rng = np.random.default_rng(11)
+    a, b = rng.standard_normal((3, 40, 50), dtype=f32), rng.standard_normal((3, 50, 60), dtype=f32)
+    c = np.empty((3, 40, 60), f32)
+    o.orc_matmul_batched(a, b, c, 3, 40, 60, 50, 1)
+    got = host(api.mat_mul(dev(a), dev(b)))
+    for i in range(3):
+        assert_gemm_close(got[i], c[i], a[i], b[i], "bmm")
+    o.orc_matmul_batched(a, b[0].copy(), c, 3, 40, 60, 50, 0)
+    got = host(api.mat_mul(dev(a), dev(b[0].copy())))
+    for i in range(3):
+        assert_gemm_close(got[i], c[i], a[i], b[0], "3dx2d")
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_sgemm_all_layouts_split_k_and_bias(api, ta, tb):
+    rng = np.random.default_rng(5 + 2 * ta + tb)
+    M, N, K = 192, 136, 4096
+    a = rng.standard_normal((K, M) if ta else (M, K), dtype=f32)
+    b = rng.standard_normal((N, K) if tb else (K, N), dtype=f32)
+    bias = rng.standard_normal(N, dtype=f32)
+    A, B = (a.T if ta else a), (b.T if tb else b)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    for split in (1, 0, 7):
+        got = host(api.sgemm(dev(a), dev(b), bool(ta), bool(tb), split_k=split))
+        assert (np.abs(got - want) <= gemm_bound(A, B)).all(), (ta, tb, split)
+    got = host(api.sgemm(dev(a), dev(b), bool(ta), bool(tb), bias=dev(bias), split_k=1))
+    assert (np.abs(got - (want + bias)) <= gemm_bound(A, B) + 1e-6).all()
+    got = host(api.sgemm(dev(a), dev(b), bool(ta), bool(tb), bias=dev(bias), split_k=5))
+    assert (np.abs(got - (want + bias)) <= gemm_bound(A, B) + 1e-6).all()
+
+
+@pytest.mark.parametrize("size", [4096])
+def test_matmul_full_size_sampled_rows_and_linearity(api, o, size):
+    # BASELINE's 4096^3: the oracle runs a seeded sample of rows (rows are independent in its loop);
+    # plus a size-independent property: (a1 + a2) @ b == a1 @ b + a2 @ b within the GEMM bound.
+    print("\n[case] full size", size, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    a = torch.randn((size, size), device="cuda", generator=g)
+    b = torch.randn((size, size), device="cuda", generator=g)
+    gy = torch.randn((size, size), device="cuda", generator=g)
+    c = api.mat_mul(a, b)
+    gx, gw = api.mat_mul_backward(a, b, gy)
+    rng = np.random.default_rng(2)
+    rows = np.sort(rng.choice(size, 6, replace=False))
+    ah, bh, gyh = host(a), host(b), host(gy)
+    ch, gxh, gwh = host(c), host(gx), host(gw)
+    bT, aT = np.ascontiguousarray(bh.T), np.ascontiguousarray(ah.T)
+    for r in rows:
+        want = np.empty((1, size), f32)
+        o.orc_matmul_rows(ah, bh, want, int(r), int(r) + 1, size, size)
+        assert_gemm_close(ch[r:r + 1], want, ah[r:r + 1], bh, "C row %d" % r)
+        o.orc_matmul_rows(gyh, bT, want, int(r), int(r) + 1, size, size)
+        assert_gemm_close(gxh[r:r + 1], want, gyh[r:r + 1], bT, "dA row %d" % r)
+        o.orc_matmul_rows(aT, gyh, want, int(r), int(r) + 1, size, size)
+        assert_gemm_close(gwh[r:r + 1], want, aT[r:r + 1], gyh, "dB row %d" % r)
+    a2 = torch.randn((size, size), device="cuda", generator=g)
+    lhs = host(api.mat_mul(a + a2, b))
+    rhs = ch + host(api.mat_mul(a2, b))
+    bound = gemm_bound(np.abs(ah) + np.abs(host(a2)), bh)
+    assert (np.abs(lhs - rhs) <= 3 * bound).all()
+
+
+def test_transpose(api, o):
+    rng = np.random.default_rng(3)
+    for shape in ((37, 53), (2, 3, 5), (128, 64), (1, 7)):
+        x = rng.standard_normal(shape, dtype=f32)
+        want = np.empty(shape[:-2] + (shape[-1], shape[-2]), f32)
+        o.orc_transpose(x, want, int(np.prod(shape[:-2])) if len(shape) > 2 else 1, shape[-2], shape[-1])
+        assert np.array_equal(host(api.transpose(dev(x))), want)
+
+
+# -------------------------------------------------------------------------------------- convolution
+CONV_CASES = {"convA": ((1, 1), (1, 1)), "convB": ((2, 2), (1, 1)), "convC": ((1, 1), (0, 0)),
+              "convD": ((2, 1), (0, 2)), "convE": ((1, 1), (0, 0))}
+
+
+def conv_bounds(x, w, gy, s, p, o):
+    """Per-element 1e-5 |a_row||b_col| bounds of the three conv GEMMs, built from the oracle's col matrix."""
+    N, C, H, W = x.shape
+    OC, _, KH, KW = w.shape
+    OH, OW = gy.shape[2], gy.shape[3]
+    M, K = N * OH * OW, C * KH * KW
+    col = np.empty((M, K), f32)
+    o.orc_im2col(x, N, C, H, W, KH, KW, s[0], s[1], p[0], p[1], 1, col)
+    w2d = w.reshape(OC, K)
+    gy2d = gy.reshape(M, OC)  # the reference's reinterpretation: same buffer, no permutation
+    by = gemm_bound(col, w2d.T).reshape(N, OH, OW, OC).transpose(0, 3, 1, 2)
+    bgw = gemm_bound(gy2d.T, col).reshape(w.shape)
+    # gx sums up to KH*KW entries of gx_col: bound each by the largest gx_col bound of its row block
+    bcol = gemm_bound(gy2d, w2d)
+    bgx = np.empty((M, K), f32)
+    bgx[:] = bcol
+    gxb = np.empty_like(x)
+    o.orc_col2im(np.ascontiguousarray(bgx), N, C, H, W, KH, KW, s[0], s[1], p[0], p[1], 1, gxb)
+    return by, bgw, gxb
+
+
+@pytest.mark.parametrize("name", sorted(CONV_CASES))
+def test_conv_fixtures_from_the_compiled_reference(api, o, name):
+    print("\n[case] conv fixture", name, flush=True)
+    s, p = CONV_CASES[name]
+    x, w, gy = G[f"{name}_x"], G[f"{name}_w"], G[f"{name}_gy"]
+    b = G[f"{name}_b"] if f"{name}_b" in G else None
+    by, bgw, bgx = conv_bounds(x, w, gy, s, p, o)
+    y = host(api.conv2d(dev(x), dev(w), dev(b) if b is not None else None, s, p))
+    assert (np.abs(y - G[f"{name}_y"]) <= by + 1e-6).all()
+    gx, gw, gb = api.conv2d_backward(dev(gy), dev(x), dev(w), b is not None, s, p)
+    assert (np.abs(host(gw) - G[f"{name}_gw"]) <= bgw + 1e-6).all()
+    assert (np.abs(host(gx) - G[f"{name}_gx"]) <= bgx + 1e-6).all()
+    if b is not None:
+        n_terms = gy.size / gy.shape[1]
+        assert (np.abs(host(gb) - G[f"{name}_gb"]) <= 1e-5 * np.sqrt(n_terms) *
+                np.linalg.norm(gy.transpose(1, 0, 2, 3).reshape(gy.shape[1], -1), axis=1) + 1e-6).all()
+    # data movement is exact
+    KH, KW = w.shape[2], w.shape[3]
+    assert np.array_equal(host(api.im2col(dev(x), (KH, KW), s, p, True)), G[f"{name}_col"])
+    assert np.array_equal(host(api.im2col(dev(x), (KH, KW), s, p, False)), G[f"{name}_col6"])
+    assert np.array_equal(host(api.col2im(dev(G[f"{name}_gcol"]), x.shape, (KH, KW), s, p, True)), G[f"{name}_im"])
+    assert np.array_equal(host(api.col2im(dev(G[f"{name}_gcol6"]), x.shape, (KH, KW), s, p, False)), G[f"{name}_im6"])
+
+
+def test_conv_reference_unit_test_vectors(api):
+    # tests/unit_test/operator/test_conv2d.cpp:21-117, test_conv2d_transpose_output.cpp:54-94
+    x9 = dev(np.arange(1, 10, dtype=f32).reshape(1, 1, 3, 3))
+    ones = dev(np.ones((1, 1, 2, 2), f32))
+    assert host(api.conv2d(x9, ones, None, 1, 0)).ravel().tolist() == [12, 16, 24, 28]
+    assert host(api.conv2d(x9, ones, None, 2, 0)).ravel().tolist() == [12]
+    x4 = dev(np.arange(1, 5, dtype=f32).reshape(1, 1, 2, 2))
+    assert host(api.conv2d(x4, ones, dev(np.array([1], f32)), 1, 0)).ravel().tolist() == [11]
+    assert tuple(api.conv2d(x4, ones, None, 1, 1).shape) == (1, 1, 3, 3)
+    w2 = dev(np.array([1, 1, 1, 1, 2, 2, 2, 2], f32).reshape(2, 1, 2, 2))
+    assert host(api.conv2d(x9, w2, None, 1, 0)).ravel().tolist() == [12, 16, 24, 28, 24, 32, 48, 56]
+    # the reinterpretation vector recorded from the compiled reference
+    gy = dev(np.arange(1, 9, dtype=f32).reshape(1, 2, 2, 2))
+    w = dev(np.arange(1, 9, dtype=f32).reshape(2, 1, 2, 2))
+    _, gw, _ = api.conv2d_backward(gy, x9, w, False, 1, 0)
+    assert host(gw).ravel().tolist() == [62, 78, 110, 126, 74, 94, 134, 154]
+    with pytest.raises(api.OdlInvalidArgument):
+        api.conv2d(x4, dev(np.ones((1, 2, 2, 2), f32)), None, 1, 0)  # channel mismatch
+    with pytest.raises(api.OdlInvalidArgument):
+        api.conv2d(x4, dev(np.ones((1, 1, 3, 3), f32)), None, 1, 0)  # no valid output
+
+
+@pytest.mark.parametrize("N,C,H,OC,s,p", [(2, 16, 14, 24, 1, 1), (3, 8, 13, 12, 2, 1), (2, 1, 28, 32, 1, 1)])
+def test_conv_vs_oracle_seeded(api, o, N, C, H, OC, s, p):
+    print("\n[case] conv seeded", N, C, H, OC, s, p, flush=True)
+    rng = np.random.default_rng(N * 100 + C)
+    x = rng.standard_normal((N, C, H, H), dtype=f32)
+    w = (rng.standard_normal((OC, C, 3, 3), dtype=f32) * f32(np.sqrt(2.0 / (C * 9)))).astype(f32)
+    b = rng.standard_normal(OC, dtype=f32)
+    OH = (H + 2 * p - 3) // s + 1
+    gy = rng.standard_normal((N, OC, OH, OH), dtype=f32)
+    yo, gxo, gwo, gbo = np.empty((N, OC, OH, OH), f32), np.empty_like(x), np.empty_like(w), np.empty_like(b)
+    assert o.orc_conv2d(x, w, b, N, C, H, H, OC, 3, 3, s, s, p, p, yo) == 0
+    assert o.orc_conv2d_backward(gy, x, w, N, C, H, H, OC, 3, 3, s, s, p, p, gxo, gwo, gbo) == 0
+    by, bgw, bgx = conv_bounds(x, w, gy, (s, s), (p, p), o)
+    assert (np.abs(host(api.conv2d(dev(x), dev(w), dev(b), s, p)) - yo) <= by + 1e-6).all()
+    gx, gw, gb = api.conv2d_backward(dev(gy), dev(x), dev(w), True, s, p)
+    assert (np.abs(host(gw) - gwo) <= bgw + 1e-6).all()
+    assert (np.abs(host(gx) - gxo) <= bgx + 1e-6).all()
+    np.testing.assert_allclose(host(gb), gbo, atol=1e-5 * np.sqrt(N * OH * OH) * np.abs(gy).max() * np.sqrt(N * OH * OH))
+
+
+def test_conv_full_size_c2_properties(api, o):
+    # BASELINE config C2: x[32,128,28,28] -> 256 channels, 3x3, stride 2, pad 1. The oracle checks a sample of
+    # output pixels (each is one dot product of a col row with a weight row); im2col/col2im adjointness and the
+    # bias-gradient identity hold at any size.
+    print("\n[case] conv C2 full size", flush=True)
+    N, C, H, OC, s, p = 32, 128, 28, 256, 2, 1
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn((N, C, H, H), device="cuda", generator=g)
+    w = torch.randn((OC, C, 3, 3), device="cuda", generator=g) * float(np.sqrt(2.0 / (C * 9)))
+    b = torch.randn((OC,), device="cuda", generator=g)
+    y = api.conv2d(x, w, b, s, p)
+    OH = y.shape[2]
+    gy = torch.randn(y.shape, device="cuda", generator=g)
+    gx, gw, gb = api.conv2d_backward(gy, x, w, True, s, p)
+    xh, wh, bh, yh = host(x), host(w), host(b), host(y)
+    rng = np.random.default_rng(4)
+    xp = np.pad(xh, ((0, 0), (0, 0), (p, p), (p, p)))
+    for _ in range(40):
+        n, oc, oh, ow = (int(rng.integers(0, d)) for d in (N, OC, OH, OH))
+        win = xp[n, :, oh * s:oh * s + 3, ow * s:ow * s + 3].ravel()
+        want = np.empty((1, 1), f32)
+        o.orc_matmul(win.reshape(1, -1).copy(), wh[oc].reshape(-1, 1).copy(), want, 1, 1, win.size)
+        want = f32(want[0, 0] + bh[oc])
+        assert abs(yh[n, oc, oh, ow] - want) <= 1e-5 * np.linalg.norm(win) * np.linalg.norm(wh[oc]) + 1e-6
+    # gb == gy.sum over (n, oh, ow)
+    want_gb = host(gy).astype(np.float64).sum(axis=(0, 2, 3))
+    np.testing.assert_allclose(host(gb), want_gb, atol=1e-5 * np.sqrt(N * OH * OH) * 80)
+    # <im2col(x), c> == <x, col2im(c)>
+    col = api.im2col(x, 3, s, p, True)
+    c = torch.randn(col.shape, device="cuda", generator=g)
+    lhs = float((col.double() * c.double()).sum())
+    rhs = float((x.double() * api.col2im(c, x.shape, 3, s, p, True).double()).sum())
+    assert abs(lhs - rhs) <= 1e-6 * float(col.double().norm() * c.double().norm())
+    # gW and gx against float64 GEMMs on the reference's reinterpreted gy
+    M, K = N * OH * OH, C * 9
+    gy2d = gy.reshape(M, OC).double()
+    want_gw = (gy2d.t() @ col.double()).reshape(w.shape)
+    bnd = 1e-5 * torch.outer(gy2d.norm(dim=0), col.double().norm(dim=0)).reshape(w.shape)
+    assert bool(((gw.double() - want_gw).abs() <= bnd).all())
+    want_gx = api.col2im((gy2d @ w.reshape(OC, K).double()).float(), x.shape, 3, s, p, True)
+    assert float((gx - want_gx).abs().max()) <= 9 * 1e-5 * float(gy2d.norm(dim=1).max() * w.reshape(OC, K).norm(dim=0).max())
+
+
+# ------------------------------------------------------------------------------- reductions / broadcast
+def sum_bound(v, axis_len):
+    return 1e-5 * np.sqrt(axis_len) * np.linalg.norm(v.astype(np.float64)) + 1e-30
+
+
+@pytest.mark.parametrize("shape,axis", [((512, 1000), 0), ((512, 10), 0), ((64, 33), 1), ((3, 4, 5), 1),
+                                        ((8, 300, 7), 1), ((5000, 3), 0), ((2, 70000), 1), ((1, 9), 0)])
+def test_sum_axis_vs_oracle(api, o, shape, axis):
+    rng = np.random.default_rng(sum(shape) + axis)
+    x = rng.standard_normal(shape, dtype=f32)
+    outer, inner = int(np.prod(shape[:axis])), int(np.prod(shape[axis + 1:]))
+    want = np.empty((outer, inner), f32)
+    o.orc_sum_axis(x, outer, shape[axis], inner, want)
+    got = host(api.sum(dev(x), axis)).reshape(outer, inner)
+    xs = x.reshape(outer, shape[axis], inner)
+    bound = 1e-5 * np.sqrt(shape[axis]) * np.linalg.norm(xs.astype(np.float64), axis=1)
+    assert (np.abs(got - want) <= bound + 1e-30).all()
+    kd = api.sum(dev(x), axis, keepdim=True)
+    assert tuple(kd.shape) == tuple(1 if i == axis else s for i, s in enumerate(shape))
+    # max over the same axis is exact
+    wmax = np.empty((outer, inner), f32)
+    o.orc_max_axis(x, outer, shape[axis], inner, wmax)
+    assert np.array_equal(host(api.max(dev(x), axis)).reshape(outer, inner), wmax)
+
+
+def test_sum_all_and_max_all(api, o):
+    rng = np.random.default_rng(12)
+    for n in (1, 7, 4096, 1_000_003):
+        x = rng.standard_normal(n, dtype=f32)
+        assert abs(host(api.sum(dev(x)))[0] - o.orc_sum_all(x, n)) <= 2 * sum_bound(x, n)
+        assert host(api.max(dev(x)))[0] == o.orc_max_all(x, n)
+    assert tuple(api.sum(dev(rng.standard_normal((3, 4), dtype=f32)), -1, keepdim=True).shape) == (1, 1)
+    with pytest.raises(api.OdlInvalidArgument):
+        api.sum(dev(np.ones((2, 2), f32)), 2)
+
+
+def test_sum_to_fixtures_and_errors(api, o):
+    for name in sorted(k[:-3] for k in G.files if k.startswith("sumto") and k.endswith("_rc")):
+        x, ts, rc = G[f"{name}_x"], tuple(int(v) for v in G[f"{name}_t"]), int(G[f"{name}_rc"])
+        if rc == -2:
+            with pytest.raises(api.OdlRuntimeError):  # test_sum_to.cpp:53-60
+                api.sum_to(dev(x), ts)
+        elif rc != 0:
+            with pytest.raises((api.OdlInvalidArgument, api.OdlRuntimeError)):
+                api.sum_to(dev(x), ts)
+        else:
+            got = host(api.sum_to(dev(x), ts)).ravel()
+            np.testing.assert_allclose(got, G[f"{name}_y"], atol=1e-5 * np.sqrt(x.size) * np.abs(x).max(), rtol=0)
+    # tests/unit_test/operator/test_sum_to.cpp:179-191 and the left-alignment probe ({2,2} -> {2} = row sums)
+    assert host(api.sum_to(dev(np.arange(1, 9, dtype=f32).reshape(2, 2, 2)), (2, 1))).ravel().tolist() == [10, 26]
+    assert host(api.sum_to(dev(np.array([[1, 2], [3, 4]], f32)), (2,))).tolist() == [3, 7]
+    assert host(api.sum_to(dev(np.array([[1, 2], [3, 4]], f32)), (1, 1))).ravel().tolist() == [10]
+    # MLP bias gradients [512,1000] -> [1,1000] and [512,10] -> [1,10] against the oracle
+    rng = np.random.default_rng(13)
+    for shape, ts in (((512, 1000), (1, 1000)), ((512, 10), (1, 10)), ((3, 4, 5), (1, 4)), ((6, 5, 4, 3), (6, 1, 4))):
+        x = rng.standard_normal(shape, dtype=f32)
+        want = np.empty(int(np.prod(ts)), f32)
+        assert o.orc_sum_to(x, ol.shape_arr(shape), len(shape), ol.shape_arr(ts), len(ts), want) == 0
+        got = host(api.sum_to(dev(x), ts)).ravel()
+        np.testing.assert_allclose(got, want, atol=1e-5 * np.sqrt(x.size / want.size) * 40, rtol=0)
+    same = rng.standard_normal((4, 5), dtype=f32)
+    assert np.array_equal(host(api.sum_to(dev(same), (4, 5))), same)
+
+
+def test_bias_grad_large_column_reduction(api):
+    # scaled bias-gradient shape used for the HBM roofline: [16384, 4096] -> [1, 4096]
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn((16384, 4096), device="cuda", generator=g)
+    got = api.sum_to(x, (1, 4096)).double()
+    want = x.double().sum(dim=0, keepdim=True)
+    assert float((got - want).abs().max()) <= 1e-5 * float(np.sqrt(16384)) * float(x.double().norm(dim=0).max())
+    gy = torch.randn((32, 128, 56, 56), device="cuda", generator=g)
+    gb = api.sum_nchw_channels(gy).double()
+    assert float((gb - gy.double().sum(dim=(0, 2, 3))).abs().max()) <= 1e-5 * float(np.sqrt(32 * 56 * 56)) * 400
+
+
+def test_broadcast_fixtures(api):
+    for name in ("bcastA", "bcastB", "bcastC"):
+        x, ds = G[f"{name}_x"], tuple(int(v) for v in G[f"{name}_d"])
+        assert np.array_equal(host(api.broadcast_to(dev(x), ds)), G[f"{name}_y"])
+        if int(G[f"{name}_rc"]) == 0:  # BroadcastTo::backward = left-aligned sum_to
+            got = host(api.sum_to(dev(G[f"{name}_g"]), x.shape))
+            np.testing.assert_allclose(got, G[f"{name}_gx"], atol=1e-5)
+    x = np.arange(3, dtype=f32).reshape(3, 1)
+    assert np.array_equal(host(api.broadcast_to(dev(x), (2, 3, 4))), np.broadcast_to(x, (2, 3, 4)))
+
+
+# ------------------------------------------------------------------------------------ softmax / CE
+def test_softmax_and_ce_vs_oracle(api, o):
+    rng = np.random.default_rng(14)
+    for N, C, is64 in ((512, 10, 1), (256, 10, 0), (7, 1000, 1), (1, 3, 0), (300, 65, 1)):
+        x = (rng.standard_normal((N, C), dtype=f32) * 3).astype(f32)
+        t = rng.integers(0, C, size=N).astype(np.int64 if is64 else np.int32)
+        p, gx, loss = np.empty_like(x), np.empty_like(x), np.zeros(1, f32)
+        o.orc_softmax(x, N, C, 1, p)
+        assert o.orc_softmax_ce_loss(x, t, is64, N, C, loss) == 0
+        assert o.orc_softmax_ce_grad(x, t, is64, N, C, 1.0, gx) == 0
+        np.testing.assert_allclose(host(api.softmax(dev(x))), p, atol=1e-6, rtol=0)
+        got_loss = api.softmax_cross_entropy(dev(x), dev(t))
+        assert abs(got_loss - loss[0]) <= 1e-4 * abs(loss[0]) + 1e-6
+        np.testing.assert_allclose(host(api.softmax_cross_entropy_backward(dev(x), dev(t), 1.0)), gx, atol=1e-6, rtol=0)
+        sel, oh = np.empty(N, f32), np.empty((N, C), f32)
+        o.orc_gather(p, t, is64, N, C, sel)
+        o.orc_one_hot(t, is64, N, C, oh)
+        assert np.array_equal(host(api.gather(dev(p), dev(t))), sel)  # integer indexing: bit-exact
+        assert np.array_equal(host(api.one_hot(dev(t), C)), oh)
+    x3 = rng.standard_normal((4, 6, 5), dtype=f32)
+    p3 = np.empty_like(x3)
+    o.orc_softmax(x3, 4, 6, 5, p3)
+    np.testing.assert_allclose(host(api.softmax(dev(x3), 1)), p3, atol=1e-6, rtol=0)
+
+
+def test_ce_reference_unit_test_vectors_and_errors(api):
+    # tests/unit_test/operator/test_softmax_cross_entropy.cpp:71-83, 131-161, 227-234
+    loss = api.softmax_cross_entropy(dev(np.ones((1, 3), f32)), dev(np.array([1], np.int32)))
+    assert abs(loss - np.log(3.0)) < 1e-6
+    x = np.array([[1, 2, 3]], f32)
+    gx = host(api.softmax_cross_entropy_backward(dev(x), dev(np.array([2], np.int32))))
+    e = np.exp(x.astype(np.float64) - 3)
+    np.testing.assert_allclose(gx, e / e.sum() - np.array([[0, 0, 1]]), atol=1e-6)
+    with pytest.raises(api.OdlInvalidArgument):
+        api.softmax_cross_entropy(dev(x), dev(np.array([3], np.int32)))
+    with pytest.raises(api.OdlInvalidArgument):
+        api.softmax_cross_entropy(dev(x), dev(np.array([0, 1], np.int32)))  # batch mismatch
+    with pytest.raises(api.OdlInvalidArgument):
+        api.gather(dev(G["oob_x"]), dev(G["oob_t"]))
+    assert np.array_equal(host(api.one_hot(dev(G["oob_t"]), 3)), G["oob_onehot"])
+
+
+def test_ce_fixtures(api):
+    for name in ("ceA", "ceB", "ceC"):
+        x, t = G[f"{name}_x"], G[f"{name}_t"]
+        assert abs(api.softmax_cross_entropy(dev(x), dev(t)) - G[f"{name}_loss"][0]) <= 1e-4 * abs(G[f"{name}_loss"][0])
+        np.testing.assert_allclose(host(api.softmax_cross_entropy_backward(dev(x), dev(t))), G[f"{name}_gx"], atol=1e-6)
+
+
+def test_ce_grad_large_rows_sum_to_zero(api):
+    # scaled shape used for the HBM roofline: [16384, 1000]; each row of softmax - one_hot sums to 0
+    g = torch.Generator(device="cuda").manual_seed(6)
+    x = torch.randn((16384, 1000), device="cuda", generator=g) * 2
+    t = torch.randint(0, 1000, (16384,), device="cuda", generator=g)
+    gx = api.softmax_cross_entropy_backward(x, t, 1.0)
+    assert float(gx.double().sum(dim=1).abs().max()) < 1e-9 + 1e-6 / 16384 * 10
+    want = (torch.softmax(x.double(), dim=1) - torch.nn.functional.one_hot(t, 1000)) / 16384
+    assert float((gx.double() - want).abs().max()) < 1e-6 / 16384 * 20 + 1e-10
+
+
+# ----------------------------------------------------------------------------------------- pooling
+POOL_CASES = {"poolA": (2, 2, 2, 2, 0, 0), "poolB": (3, 3, 2, 2, 1, 1), "poolC": (5, 5, 1, 1, 2, 2),
+              "poolD": (3, 2, 1, 2, 1, 0)}
+
+
+@pytest.mark.parametrize("name", sorted(POOL_CASES))
+def test_max_pool_fixtures_bit_exact(api, name):
+    KH, KW, SH, SW, PH, PW = POOL_CASES[name]
+    x = G[f"{name}_x"]
+    y, idx = api.max_pool2d(dev(x), (KH, KW), (SH, SW), (PH, PW))
+    assert np.array_equal(host(y), G[f"{name}_y"])
+    assert np.array_equal(host(idx).view(np.uint64), G[f"{name}_idx"])
+    gx = api.max_pool2d_backward(dev(G[f"{name}_gy"]), idx, x.shape, (KH, KW), (SH, SW), (PH, PW))
+    assert np.array_equal(host(gx), G[f"{name}_gx"])
+
+
+def test_max_pool_cnn_shapes_vs_oracle_bit_exact(api, o):
+    # config 4's pools at reduced batch: [N,32,28,28] -> 14x14 and [N,64,14,14] -> 7x7, indices compared in full
+    rng = np.random.default_rng(15)
+    for N, C, H in ((8, 32, 28), (8, 64, 14)):
+        x = np.maximum(rng.standard_normal((N, C, H, H), dtype=f32), 0)  # post-ReLU: many exact ties at 0
+        y, idx = np.empty((N, C, H // 2, H // 2), f32), np.empty((N, C, H // 2, H // 2), np.uint64)
+        assert o.orc_max_pool2d(x, N, C, H, H, 2, 2, 2, 2, 0, 0, y, idx) == 0
+        gy = rng.standard_normal(y.shape, dtype=f32)
+        gx = np.empty_like(x)
+        assert o.orc_max_pool2d_backward(gy, idx, N, C, H, H, 2, 2, 2, 2, 0, 0, gx) == 0
+        yd, idxd = api.max_pool2d(dev(x), 2, 2, 0)
+        assert np.array_equal(host(yd), y) and np.array_equal(host(idxd).view(np.uint64), idx)
+        assert np.array_equal(host(api.max_pool2d_backward(dev(gy), idxd, x.shape, 2, 2, 0)), gx)
+    # tests/unit_test/operator/test_max_pool2d.cpp:20-45
+    y, _ = api.max_pool2d(dev(np.arange(1, 17, dtype=f32).reshape(1, 1, 4, 4)), 2, 2, 0)
+    assert host(y).ravel().tolist() == [6, 8, 14, 16]
+
+
+# ----------------------------------------------------------------------------------------- metrics
+def test_argmax_and_accuracy_bit_exact(api, o):
+    rng = np.random.default_rng(16)
+    y = rng.integers(0, 4, size=(1000, 10)).astype(f32)  # ties everywhere
+    t = rng.integers(0, 10, size=1000).astype(np.int32)
+    am = np.empty(1000, np.int64)
+    o.orc_argmax_rows(y, 1000, 10, am)
+    assert np.array_equal(host(api.argmax_rows(dev(y))), am)
+    assert api.accuracy(dev(y), dev(t)) == o.orc_accuracy(y, t, 1000, 10)
+
+
+# ------------------------------------------------------------------------------------- elementwise
+def test_elementwise_vs_oracle_and_fixtures(api, o):
+    a, b = G["ew_a"], G["ew_b"]
+    for i, op in enumerate(("add", "sub", "mul", "div", "gt")):
+        assert np.array_equal(host(api.binary(op, dev(a), dev(b))), G[f"ew_bin{i}"]), op
+    for i, op in enumerate(("relu", "exp", "log", "neg", "square")):
+        src = np.abs(a) + f32(0.1) if op == "log" else a
+        got = host(api.unary(op, dev(src)))
+        if op in ("exp", "log"):
+            np.testing.assert_allclose(got, G[f"ew_un{i}"], rtol=2e-7, atol=1e-7)
+        else:
+            assert np.array_equal(got, G[f"ew_un{i}"]), op
+    np.testing.assert_allclose(host(api.pow_scalar(dev(np.abs(a)), 0.5)), G["ew_pow05"], rtol=3e-7)
+    rng = np.random.default_rng(17)
+    big = rng.standard_normal(100003, dtype=f32)
+    s = np.array([1.5], f32)
+    want = np.empty_like(big)
+    for i, op in enumerate(("add", "sub", "mul", "div", "gt")):
+        o.orc_binary(i, big, big.size, s, 1, want)
+        assert np.array_equal(host(api.binary(op, dev(big), dev(s))), want)
+        o.orc_binary(i, s, 1, big, big.size, want)
+        assert np.array_equal(host(api.binary(op, dev(s), dev(big))), want)
+    with pytest.raises(api.OdlRuntimeError):
+        api.binary("add", dev(big), dev(big[:5].copy()))
+    acc = dev(big.copy())
+    api.binary("add", acc, dev(big), out=acc)  # add_inplace: output aliases an input
+    assert np.array_equal(host(acc), big + big)
+    assert bool((api.fill((3, 5), 2.5) == 2.5).all())
