@@ -1,0 +1,242 @@
+"""Benchmark of the hot path on one MI355X.
+
+Default workload (the one the headline metric is quoted on): standalone matmul forward + backward, fp32,
+M = N = K = 4096 — one step = C = A.B, dA = dC.B^T, dB = A^T.dC = 6*M*N*K FLOP — on synthetic N(0,1) operands
+already resident in HBM. Prints ONE JSON line: value = TFLOP/s of the whole step, plus
+  roofline      the MFMA GEMM kernel: 2*M*N*K FLOP per launch / average launch duration measured with events on the
+                launch stream over the timed region, against the 157.3 TFLOP/s FP32 matrix peak;
+  cpu_baseline  the reference's own CPU backend (oracle/_ref, when its build travelled with the tree) or the plain-C
+                port of it (oracle/), timed on this box's host cores on a bounded row slice of the same three products;
+  extras        the other hot-path kernels at the benchmark's shapes (conv C1/C2 fwd+bwd, im2col/col2im, bias-gradient
+                and softmax-CE-gradient streams) with their own roofline fractions, and MLP train-step GEMM time.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--size 4096] [--no-extras] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def time_region(torch, fn, steps, warmup):
+    """ms per call of fn, timed with events on the current stream (the stream the kernels are launched on)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def cpu_baseline_gemm(size, budget_s=18.0):
+    """Reference CPU algorithm on a row slice of each of the three products; rows are independent in its loop
+    (src/mat/origin/cpu/math/matmul.cpp:27-41), so time scales linearly with the number of rows."""
+    import numpy as np
+    import oraclelib as ol
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((size, size), dtype=np.float32)
+    b = rng.standard_normal((size, size), dtype=np.float32)
+    use_ref = ol.have_ref()
+
+    def run(rows):
+        out = np.empty((rows, size), np.float32)
+        sl = np.ascontiguousarray(a[:rows])
+        t0 = time.perf_counter()
+        for _ in range(3):  # C rows, dA rows, dB rows: three products of identical shape on a slice
+            if use_ref:
+                assert ol.ref().odl_ref_matmul(sl, b, out, rows, size, size) == 0
+            else:
+                ol.oracle().orc_matmul(sl, b, out, rows, size, size)
+        return time.perf_counter() - t0
+
+    probe_rows = 2
+    t_probe = run(probe_rows)
+    rows = int(max(2, min(size, probe_rows * budget_s / max(t_probe, 1e-6))))
+    t = run(rows)
+    flop = 3 * 2.0 * rows * size * size
+    return {
+        "value": flop / t / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "reference" if use_ref else "port",
+        "sample": "%d of %d rows of each of C, dA, dB (%.1f s; full step extrapolates to %.0f s)"
+                  % (rows, size, t, t * size / rows),
+    }
+
+
+def extras(torch, capi, steps, warmup):
+    out = {}
+    g = torch.Generator(device="cuda").manual_seed(0)
+
+    def rnd(*shape):
+        return torch.randn(shape, device="cuda", generator=g)
+
+    # conv2d forward + weight-grad + input-grad at BASELINE's C1 and C2
+    for name, (N, C, H, OC, s, p) in {"conv_c1": (32, 64, 56, 128, 1, 1), "conv_c2": (32, 128, 28, 256, 2, 1)}.items():
+        x, w, b = rnd(N, C, H, H), rnd(OC, C, 3, 3) * (2.0 / (C * 9)) ** 0.5, rnd(OC)
+        OH = (H + 2 * p - 3) // s + 1
+        gy = rnd(N, OC, OH, OH)
+        M, K = N * OH * OH, C * 9
+        ms_f = time_region(torch, lambda: capi.conv2d(x, w, b, s, p), steps, warmup)
+        ms_b = time_region(torch, lambda: capi.conv2d_backward(gy, x, w, True, s, p), steps, warmup)
+        flop = 6.0 * M * K * OC
+        tf = flop / (ms_f + ms_b) / 1e9
+        out[name] = {"fwd_ms": ms_f, "bwd_ms": ms_b, "tflops": tf, "frac_mfma_peak": tf / PEAK_FP32_MFMA_TFLOPS,
+                     "flop": flop}
+        ms_i = time_region(torch, lambda: capi.im2col(x, 3, s, p, True), steps, warmup)
+        col = capi.im2col(x, 3, s, p, True)
+        ms_c = time_region(torch, lambda: capi.col2im(col, x.shape, 3, s, p, True), steps, warmup)
+        nbytes = 4.0 * (x.numel() + M * K)
+        out[name + "_im2col"] = {"ms": ms_i, "gbs": nbytes / ms_i / 1e6, "frac_hbm": nbytes / ms_i / 1e6 / PEAK_HBM_GBS}
+        out[name + "_col2im"] = {"ms": ms_c, "gbs": nbytes / ms_c / 1e6, "frac_hbm": nbytes / ms_c / 1e6 / PEAK_HBM_GBS}
+        ms_gb = time_region(torch, lambda: capi.sum_nchw_channels(gy), steps, warmup)
+        nb = 4.0 * (gy.numel() + OC)
+        out[name + "_bias_grad"] = {"ms": ms_gb, "gbs": nb / ms_gb / 1e6, "frac_hbm": nb / ms_gb / 1e6 / PEAK_HBM_GBS}
+        del x, w, b, gy, col
+    # gradient reductions: the MLP's own shapes (launch-bound) and scaled shapes that can saturate HBM
+    for name, shape, target in (("bias_grad_512x1000", (512, 1000), (1, 1000)),
+                                ("bias_grad_16384x4096_scaled", (16384, 4096), (1, 4096))):
+        x = rnd(*shape)
+        ms = time_region(torch, lambda: capi.sum_to(x, target), steps, warmup)
+        nb = 4.0 * (x.numel() + target[1])
+        out[name] = {"ms": ms, "gbs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+    for name, (N, C) in (("softmax_ce_grad_512x10", (512, 10)), ("softmax_ce_grad_16384x1000_scaled", (16384, 1000))):
+        x = rnd(N, C)
+        t = torch.randint(0, C, (N,), device="cuda", generator=g)
+        ms = time_region(torch, lambda: capi.softmax_cross_entropy_backward(x, t, 1.0), steps, warmup)
+        nb = 8.0 * N * C + 8.0 * N
+        out[name] = {"ms": ms, "gbs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+    # the MLP's six GEMMs (config 1): 512x784x1000 and 512x1000x10, forward + backward
+    x1, w1, g1 = rnd(512, 784), rnd(784, 1000), rnd(512, 1000)
+    x2, w2, g2 = rnd(512, 1000), rnd(1000, 10), rnd(512, 10)
+
+    def mlp_gemms():
+        capi.mat_mul(x1, w1)
+        capi.mat_mul(x2, w2)
+        capi.mat_mul_backward(x2, w2, g2)
+        capi.mat_mul_backward(x1, w1, g1)
+
+    ms = time_region(torch, mlp_gemms, steps, warmup)
+    flop = 6.0 * 512 * (784 * 1000 + 1000 * 10)
+    out["mlp_gemms_fwd_bwd"] = {"ms": ms, "tflops": flop / ms / 1e9, "flop": flop}
+    return out
+
+
+def pmc_probe(torch, capi, gemm_step):
+    """A short, fixed launch sequence for counter runs (`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`):
+    first a plain elementwise copy-like kernel of known traffic (negate of 64 Mi floats: 256 MiB read, 256 MiB
+    written) that calibrates the counters, then each hot kernel a few times."""
+    g = torch.Generator(device="cuda").manual_seed(0)
+    cal = torch.randn((64 * 1024 * 1024,), device="cuda", generator=g)
+    for _ in range(3):
+        capi.unary("neg", cal)
+    for _ in range(3):
+        gemm_step()
+    x = torch.randn((32, 64, 56, 56), device="cuda", generator=g)
+    w = torch.randn((128, 64, 3, 3), device="cuda", generator=g) * 0.06
+    b = torch.randn((128,), device="cuda", generator=g)
+    gy = torch.randn((32, 128, 56, 56), device="cuda", generator=g)
+    for _ in range(2):
+        capi.conv2d(x, w, b, 1, 1)
+        capi.conv2d_backward(gy, x, w, True, 1, 1)
+    big = torch.randn((16384, 4096), device="cuda", generator=g)
+    logits = torch.randn((16384, 1000), device="cuda", generator=g)
+    t = torch.randint(0, 1000, (16384,), device="cuda", generator=g)
+    for _ in range(3):
+        capi.sum_to(big, (1, 4096))
+        capi.softmax_cross_entropy_backward(logits, t, 1.0)
+    torch.cuda.synchronize()
+    print("pmc probe done")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--size", type=int, default=4096)
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="few launches of each hot kernel plus a plain copy of known size, for rocprofv3 --pmc runs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; nothing here uses a second one (no collectives, no sharding). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from origindl_amd import capi  # raises if libodl_hip.so is missing: there is no fallback
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    torch.cuda.set_device(0)
+    S = args.size
+    g = torch.Generator(device="cuda").manual_seed(1)
+    a = torch.randn((S, S), device="cuda", generator=g)
+    b = torch.randn((S, S), device="cuda", generator=g)
+    dc = torch.randn((S, S), device="cuda", generator=g)
+    # outputs and the (possibly empty) workspace are allocated once: the timed region is kernels only
+    c, da, db = torch.empty_like(a), torch.empty_like(a), torch.empty_like(a)
+    import ctypes
+    lib = capi.lib()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ws_bytes = lib.query("odl_hip_matmul_backward_workspace_bytes", S, S, S)
+    ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.int32, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+
+    def step():
+        lib.call("odl_hip_matmul", p(a), p(b), p(c), 1, S, S, S, 0, st)
+        lib.call("odl_hip_matmul_backward", p(a), p(b), p(dc), p(da), p(db), S, S, S, p(ws), ws_bytes, st)
+
+    if args.pmc_probe:
+        pmc_probe(torch, capi, step)
+        return
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ev_ms = e0.elapsed_time(e1) / args.steps
+    ms = max(wall_ms, ev_ms)
+    flop_step = 6.0 * S * S * S
+    value = flop_step / ms / 1e9
+
+    # the dominant kernel: three launches of the MFMA GEMM per step (NN, NT, TN), each 2*S^3 FLOP
+    launch_ms = ev_ms / 3.0
+    achieved = 2.0 * S * S * S / launch_ms / 1e9
+    line = {
+        "metric": "fwd+bwd TFLOP/s (GEMM %d^3) fp32 at 1 GPU" % S,
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic N(0,1) operands, seeded, resident in HBM",
+        "config": {"workload": "matmul fwd+bwd: C=A.B, dA=dC.B^T, dB=A^T.dC, M=N=K=%d" % S, "flop_per_step": flop_step},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                     "kernel": "sgemm_mfma_kernel<128,128,16> (NN, NT, TN)", "launch_ms": launch_ms},
+        "device": capi.device_info(0),
+    }
+    if not args.no_extras:
+        line["extras"] = extras(torch, capi, max(3, args.steps // 2), max(2, args.warmup // 2))
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_gemm(S)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
