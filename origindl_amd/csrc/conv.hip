@@ -44,47 +44,86 @@ inline size_t align256(size_t b)
     return (b + 255) & ~(size_t)255;
 }
 
-// col[m][ck] (m = (n,oh,ow), ck = (c,kh,kw)); one thread produces VEC consecutive ck of one row.
-template <int VEC>
-__global__ void im2col_matrix_kernel(const float *__restrict__ img, float *__restrict__ col, ConvGeom g)
+// Workgroups are dealt round-robin over the 8 XCDs (one L2 each); unfolding the id this way gives every XCD
+// a contiguous band of virtual blocks, so neighbouring tiles — which read the same image lines — share an L2.
+__device__ inline int64_t xcd_contiguous_block(int64_t bid, int64_t nb)
 {
-    const int64_t K = g.C * g.KH * g.KW;
-    const int64_t kq = K / VEC;
-    const int64_t total = g.N * g.OH * g.OW * kq;
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= total)
-        return;
-    const int64_t m = t / kq;
-    const int ck0 = (int)(t % kq) * VEC;
-    const int64_t ow = m % g.OW, oh = (m / g.OW) % g.OH, n = m / (g.OW * g.OH);
-    float v[VEC];
-    int kw = ck0 % g.KW, kh = (ck0 / g.KW) % g.KH;
-    int64_t c = ck0 / (g.KW * g.KH);
-#pragma unroll
-    for (int e = 0; e < VEC; ++e)
+    const int64_t xcd = bid % 8, loc = bid / 8;
+    const int64_t full = nb / 8, rem = nb % 8;
+    return xcd * full + (xcd < rem ? xcd : rem) + loc;
+}
+
+constexpr int kImPix = 64;   // pixels (col rows) per tile
+constexpr int kImCk  = 144;  // col columns per tile at most
+
+// col[m][ck] (m = (n,oh,ow), ck = (c,kh,kw)), tile = 64 consecutive rows x up to 144 columns.
+// Read phase: for one ck at a time the 64 lanes of a wave read 64 consecutive pixels — contiguous image addresses
+// (stride SW) — into an LDS tile; write phase: the tile leaves row by row with 16-byte stores. The image is read
+// through coalesced loads and the 9x larger col matrix is written through full-width stores.
+__global__ __launch_bounds__(256) void im2col_matrix_kernel(const float *__restrict__ img, float *__restrict__ col,
+                                                             ConvGeom g, int tk, int ktiles, int64_t mtiles)
+{
+    __shared__ float sh[kImPix][kImCk + 1];
+    const int64_t vb = xcd_contiguous_block(blockIdx.x, mtiles * ktiles);
+    const int64_t mt = vb / ktiles;
+    const int kt = (int)(vb % ktiles);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t M = g.N * g.OH * g.OW;
+    const int K = (int)(g.C * g.KH * g.KW);
+    const int64_t m = mt * kImPix + lane;
+    const bool live = m < M;
+    const int64_t mm = live ? m : 0;
+    const int ow = (int)(mm % g.OW), oh = (int)((mm / g.OW) % g.OH);
+    const int64_t n = mm / (g.OW * g.OH);
+    const int h0 = oh * g.SH - g.PH, w0 = ow * g.SW - g.PW;
+    const float *base = img + n * g.C * g.H * g.W;
+    const int ck0 = kt * tk;
+    const int ckn = (K - ck0 < tk) ? K - ck0 : tk;
+    const int H = (int)g.H, W = (int)g.W;
+    constexpr int U = 6;  // independent loads in flight per lane
+    for (int j = wave; j < ckn; j += 4 * U)
     {
-        const int64_t h = oh * g.SH + kh - g.PH, w = ow * g.SW + kw - g.PW;
-        v[e] = (h >= 0 && h < g.H && w >= 0 && w < g.W) ? img[((n * g.C + c) * g.H + h) * g.W + w] : 0.f;
-        if (++kw == g.KW)
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
         {
-            kw = 0;
-            if (++kh == g.KH)
+            const int ck = ck0 + j + 4 * u;  // wave-uniform
+            const int kw = ck % g.KW, t2 = ck / g.KW;
+            const int kh = t2 % g.KH, c = t2 / g.KH;
+            const int h = h0 + kh, w = w0 + kw;
+            v[u] = 0.f;
+            if (j + 4 * u < ckn && live && h >= 0 && h < H && w >= 0 && w < W)
+                v[u] = base[((int64_t)c * H + h) * W + w];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (j + 4 * u < ckn)
+                sh[lane][j + 4 * u] = v[u];
+    }
+    __syncthreads();
+    const int64_t row0 = mt * kImPix;
+    if ((ckn & 3) == 0 && (K & 3) == 0 && (ck0 & 3) == 0 && (reinterpret_cast<uintptr_t>(col) & 15) == 0)
+    {
+        const int q4 = ckn >> 2;
+        for (int e = threadIdx.x; e < kImPix * q4; e += 256)
+        {
+            const int row = e / q4, q = e % q4;
+            if (row0 + row < M)
             {
-                kh = 0;
-                ++c;
+                f32x4 o = {sh[row][4 * q], sh[row][4 * q + 1], sh[row][4 * q + 2], sh[row][4 * q + 3]};
+                *reinterpret_cast<f32x4 *>(col + (row0 + row) * K + ck0 + 4 * q) = o;
             }
         }
     }
-    if (VEC == 4)
-    {
-        f32x4 o = {v[0], v[1], v[2], v[3]};
-        *reinterpret_cast<f32x4 *>(col + m * K + ck0) = o;
-    }
     else
     {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e)
-            col[m * K + ck0 + e] = v[e];
+        for (int e = threadIdx.x; e < kImPix * ckn; e += 256)
+        {
+            const int row = e / ckn, j = e % ckn;
+            if (row0 + row < M)
+                col[(row0 + row) * K + ck0 + j] = sh[row][j];
+        }
     }
 }
 
@@ -108,10 +147,11 @@ __global__ void im2col_6d_kernel(const float *__restrict__ img, float *__restric
     col[t] = (h >= 0 && h < g.H && w >= 0 && w < g.W) ? img[(r * g.H + h) * g.W + w] : 0.f;
 }
 
-// one thread per image pixel; taps added in ascending (kh, kw), starting from +0.0f like the reference's
-// zero-filled padded image (conv2d.cpp:316-349).
-template <bool MATRIX>
-__global__ void col2im_kernel(const float *__restrict__ col, float *__restrict__ img, ConvGeom g)
+// Taps of one image pixel are added in ascending (kh, kw), starting from +0.0f like the reference's zero-filled
+// padded image (conv2d.cpp:316-349): bit-identical sums, no atomics.
+//
+// 6-D layout [N,C,KH,KW,OH,OW]: one thread per pixel, lanes along w — reads and writes are contiguous.
+__global__ void col2im_6d_kernel(const float *__restrict__ col, float *__restrict__ img, ConvGeom g)
 {
     const int64_t total = g.N * g.C * g.H * g.W;
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -119,8 +159,6 @@ __global__ void col2im_kernel(const float *__restrict__ col, float *__restrict__
         return;
     const int64_t w = t % g.W, h = (t / g.W) % g.H;
     const int64_t nc = t / (g.W * g.H);
-    const int64_t c = nc % g.C, n = nc / g.C;
-    const int64_t K = g.C * g.KH * g.KW;
     float acc = 0.f;
     for (int kh = 0; kh < g.KH; ++kh)
     {
@@ -138,15 +176,110 @@ __global__ void col2im_kernel(const float *__restrict__ col, float *__restrict__
             const int64_t ow = wp / g.SW;
             if (ow >= g.OW)
                 continue;
-            float v;
-            if (MATRIX)
-                v = col[((n * g.OH + oh) * g.OW + ow) * K + (c * g.KH + kh) * g.KW + kw];
-            else
-                v = col[(((nc * g.KH + kh) * g.KW + kw) * g.OH + oh) * g.OW + ow];
-            acc += v;
+            acc += col[(((nc * g.KH + kh) * g.KW + kw) * g.OH + oh) * g.OW + ow];
         }
     }
     img[t] = acc;
+}
+
+// Matrix layout [N*OH*OW, C*KH*KW]: a workgroup owns 64 channels x 16 consecutive w of one image row. Lanes run
+// along the channel, where a col row is nearly contiguous (KH*KW floats apart), each thread sums 4 pixels, and the
+// 64x16 result tile is turned through LDS so that the image is written in 64-byte runs along w.
+template <int CKH, int CKW>
+__global__ __launch_bounds__(256) void col2im_matrix_kernel(const float *__restrict__ col, float *__restrict__ img,
+                                                             ConvGeom g, int wtiles, int ctiles)
+{
+    __shared__ float sh[64][17];
+    const int KH = CKH > 0 ? CKH : g.KH, KW = CKW > 0 ? CKW : g.KW;
+    const int64_t nb = g.N * g.H * wtiles * ctiles;
+    int64_t vb = xcd_contiguous_block(blockIdx.x, nb);
+    const int ct = (int)(vb % ctiles);
+    vb /= ctiles;
+    const int wt = (int)(vb % wtiles);
+    vb /= wtiles;
+    const int h = (int)(vb % g.H);
+    const int64_t n = vb / g.H;
+    const int cl = threadIdx.x & 63, wq = threadIdx.x >> 6;
+    const int c = ct * 64 + cl;
+    const int K = (int)(g.C * KH * KW);
+    const int W = (int)g.W, OH = (int)g.OH, OW = (int)g.OW;
+    if (c < g.C)
+    {
+        const float *cbase = col + (int64_t)c * KH * KW;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            const int w = wt * 16 + wq * 4 + i;
+            float acc = 0.f;
+            if (w < W)
+            {
+                if (CKH > 0)
+                {
+                    // all taps are loaded (or zeroed) first, then added in ascending (kh, kw)
+                    float v[(CKH > 0 ? CKH : 1) * (CKW > 0 ? CKW : 1)];
+#pragma unroll
+                    for (int kh = 0; kh < CKH; ++kh)
+                    {
+                        const int hp = h + g.PH - kh;
+                        const int oh = hp / g.SH;
+                        const bool hok = hp >= 0 && hp % g.SH == 0 && oh < OH;
+#pragma unroll
+                        for (int kw = 0; kw < CKW; ++kw)
+                        {
+                            const int wp = w + g.PW - kw;
+                            const int ow = wp / g.SW;
+                            const bool ok = hok && wp >= 0 && wp % g.SW == 0 && ow < OW;
+                            v[kh * CKW + kw] = ok ? cbase[((n * OH + oh) * OW + ow) * K + kh * CKW + kw] : 0.f;
+                        }
+                    }
+                    // a skipped tap contributes nothing in the reference; adding +0.0f instead leaves every
+                    // partial sum unchanged because the accumulator starts at +0.0f and never becomes -0.0f
+#pragma unroll
+                    for (int q = 0; q < CKH * CKW; ++q)
+                        acc += v[q];
+                }
+                else
+                {
+                    for (int kh = 0; kh < KH; ++kh)
+                    {
+                        const int hp = h + g.PH - kh;
+                        if (hp < 0 || hp % g.SH != 0)
+                            continue;
+                        const int oh = hp / g.SH;
+                        if (oh >= OH)
+                            continue;
+                        for (int kw = 0; kw < KW; ++kw)
+                        {
+                            const int wp = w + g.PW - kw;
+                            if (wp < 0 || wp % g.SW != 0)
+                                continue;
+                            const int ow = wp / g.SW;
+                            if (ow >= OW)
+                                continue;
+                            acc += cbase[((n * OH + oh) * OW + ow) * K + kh * KW + kw];
+                        }
+                    }
+                }
+            }
+            sh[cl][wq * 4 + i] = acc;
+        }
+    }
+    __syncthreads();
+    const int row = threadIdx.x >> 2, part = threadIdx.x & 3;
+    const int cc = ct * 64 + row;
+    const int wbase = wt * 16 + part * 4;
+    if (cc < g.C && wbase < W)
+    {
+        float *dst = img + ((n * g.C + cc) * g.H + h) * W + wbase;
+        if ((W & 3) == 0 && (reinterpret_cast<uintptr_t>(img) & 15) == 0)
+        {
+            f32x4 o = {sh[row][part * 4], sh[row][part * 4 + 1], sh[row][part * 4 + 2], sh[row][part * 4 + 3]};
+            *reinterpret_cast<f32x4 *>(dst) = o;
+        }
+        else
+            for (int i = 0; i < 4 && wbase + i < W; ++i)
+                dst[i] = sh[row][part * 4 + i];
+    }
 }
 
 int make_geom(ConvGeom &g, const char *who, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
@@ -171,13 +304,12 @@ int im2col_launch(const float *img, float *col, const ConvGeom &g, int to_matrix
         return ODL_OK;
     if (to_matrix)
     {
-        const bool v4 = (K % 4 == 0) && (reinterpret_cast<uintptr_t>(col) % 16 == 0);
-        const int64_t threads = v4 ? total / 4 : total;
-        const dim3 grid((unsigned)odl::ceil_div(threads, 256));
-        if (v4)
-            hipLaunchKernelGGL(im2col_matrix_kernel<4>, grid, dim3(256), 0, st, img, col, g);
-        else
-            hipLaunchKernelGGL(im2col_matrix_kernel<1>, grid, dim3(256), 0, st, img, col, g);
+        const int tk = K < kImCk ? (int)K : kImCk;
+        const int ktiles = (int)odl::ceil_div(K, tk);
+        const int64_t mtiles = odl::ceil_div(g.N * g.OH * g.OW, kImPix);
+        ODL_REQUIRE(mtiles * ktiles < (1ll << 31) && K < (1ll << 31), "im2col: too many tiles");
+        hipLaunchKernelGGL(im2col_matrix_kernel, dim3((unsigned)(mtiles * ktiles)), dim3(256), 0, st, img, col, g, tk,
+                           ktiles, mtiles);
     }
     else
     {
@@ -192,11 +324,20 @@ int col2im_launch(const float *col, float *img, const ConvGeom &g, int to_matrix
     const int64_t total = g.N * g.C * g.H * g.W;
     if (total == 0)
         return ODL_OK;
-    const dim3 grid((unsigned)odl::ceil_div(total, 256));
     if (to_matrix)
-        hipLaunchKernelGGL(col2im_kernel<true>, grid, dim3(256), 0, st, col, img, g);
+    {
+        const int wtiles = (int)odl::ceil_div(g.W, 16), ctiles = (int)odl::ceil_div(g.C, 64);
+        const int64_t nb = g.N * g.H * wtiles * ctiles;
+        ODL_REQUIRE(nb < (1ll << 31) && g.N * g.OH * g.OW * g.C * g.KH * g.KW < (1ll << 40), "col2im: too large");
+        if (g.KH == 3 && g.KW == 3)
+            hipLaunchKernelGGL((col2im_matrix_kernel<3, 3>), dim3((unsigned)nb), dim3(256), 0, st, col, img, g, wtiles,
+                               ctiles);
+        else
+            hipLaunchKernelGGL((col2im_matrix_kernel<0, 0>), dim3((unsigned)nb), dim3(256), 0, st, col, img, g, wtiles,
+                               ctiles);
+    }
     else
-        hipLaunchKernelGGL(col2im_kernel<false>, grid, dim3(256), 0, st, col, img, g);
+        hipLaunchKernelGGL(col2im_6d_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, col, img, g);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

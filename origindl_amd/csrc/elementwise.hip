@@ -81,12 +81,29 @@ __global__ void binary_kernel(const float *a, const float *b, float *out, int64_
             out[i0 + e] = ov[e];
 }
 
-template <int OP>
+// 16 bytes per lane when the buffers are 16-byte aligned; the tail and unaligned buffers go one float at a time
+template <int OP, bool VEC>
 __global__ void unary_kernel(const float *a, float *out, int64_t n)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n)
-        out[i] = un<OP>(a[i]);
+    if (VEC)
+    {
+        const int64_t i0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+        if (i0 + 4 <= n)
+        {
+            const f32x4 q = *reinterpret_cast<const f32x4 *>(a + i0);
+            f32x4 r = {un<OP>(q[0]), un<OP>(q[1]), un<OP>(q[2]), un<OP>(q[3])};
+            *reinterpret_cast<f32x4 *>(out + i0) = r;
+        }
+        else
+            for (int64_t i = i0; i < n; ++i)
+                out[i] = un<OP>(a[i]);
+    }
+    else
+    {
+        const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (i < n)
+            out[i] = un<OP>(a[i]);
+    }
 }
 
 __global__ void pow_kernel(const float *a, float *out, int64_t n, float e)
@@ -194,16 +211,26 @@ int odl_hip_unary(int op, const float *a, int64_t n, float *out, void *stream)
     if (n <= 0)
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
-    const dim3 grid((unsigned)odl::ceil_div(n, kBlock));
+    const bool vec = (reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(out)) % 16 == 0;
+    const dim3 grid((unsigned)odl::ceil_div(vec ? odl::ceil_div(n, 4) : n, kBlock));
+#define ODL_UN_CASE(OP)                                                                          \
+    case OP:                                                                                     \
+        if (vec)                                                                                 \
+            hipLaunchKernelGGL((unary_kernel<OP, true>), grid, dim3(kBlock), 0, st, a, out, n);  \
+        else                                                                                     \
+            hipLaunchKernelGGL((unary_kernel<OP, false>), grid, dim3(kBlock), 0, st, a, out, n); \
+        break;
     switch (op)
     {
-        case 0: hipLaunchKernelGGL(unary_kernel<0>, grid, dim3(kBlock), 0, st, a, out, n); break;
-        case 1: hipLaunchKernelGGL(unary_kernel<1>, grid, dim3(kBlock), 0, st, a, out, n); break;
-        case 2: hipLaunchKernelGGL(unary_kernel<2>, grid, dim3(kBlock), 0, st, a, out, n); break;
-        case 3: hipLaunchKernelGGL(unary_kernel<3>, grid, dim3(kBlock), 0, st, a, out, n); break;
-        case 4: hipLaunchKernelGGL(unary_kernel<4>, grid, dim3(kBlock), 0, st, a, out, n); break;
-        default: hipLaunchKernelGGL(unary_kernel<5>, grid, dim3(kBlock), 0, st, a, out, n); break;
+        ODL_UN_CASE(0)
+        ODL_UN_CASE(1)
+        ODL_UN_CASE(2)
+        ODL_UN_CASE(3)
+        ODL_UN_CASE(4)
+        default:
+        ODL_UN_CASE(5)
     }
+#undef ODL_UN_CASE
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

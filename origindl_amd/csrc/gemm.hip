@@ -295,20 +295,33 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g)
         }
 }
 
-// out[i] = sum over slices (ascending) of part[s*stride + i] (+ bias by column or by row for the NCHW store)
-__global__ void splitk_reduce_kernel(const float *__restrict__ part, int splits, int64_t stride, float *out,
-                                     int64_t M, int64_t N, int64_t ldc, const float *bias)
+// out[i] = sum over slices of part[s*stride + i] (+ bias by column). 64 outputs x 16 slice groups per workgroup:
+// group g adds slices g, g+16, ..., the group sums meet in LDS and are added in group order — a fixed order.
+constexpr int kRedGroups = 16;
+__global__ __launch_bounds__(64 * kRedGroups) void splitk_reduce_kernel(const float *__restrict__ part, int splits,
+                                                                         int64_t stride, float *out, int64_t M, int64_t N,
+                                                                         int64_t ldc, const float *bias)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= M * N)
-        return;
-    float s = 0.f;
-    for (int z = 0; z < splits; ++z)
-        s += part[(int64_t)z * stride + i];
-    const int64_t r = i / N, c = i % N;
-    if (bias)
-        s = s + bias[c];
-    out[r * ldc + c] = s;
+    __shared__ float sh[kRedGroups][64];
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int64_t i = (int64_t)blockIdx.x * 64 + lane;
+    float acc = 0.f;
+    if (i < M * N)
+        for (int z = grp; z < splits; z += kRedGroups)
+            acc += part[(int64_t)z * stride + i];
+    sh[grp][lane] = acc;
+    __syncthreads();
+    if (grp == 0 && i < M * N)
+    {
+        float s = sh[0][lane];
+#pragma unroll
+        for (int k = 1; k < kRedGroups; ++k)
+            s += sh[k][lane];
+        const int64_t r = i / N, c = i % N;
+        if (bias)
+            s = s + bias[c];
+        out[r * ldc + c] = s;
+    }
 }
 
 __global__ void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows, int64_t cols)
@@ -426,7 +439,7 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
             return fail(rc, "sgemm: no kernel variant");
         ODL_LAUNCH_CHECK();
         const int64_t total = M * N;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st,
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 64)), dim3(64 * kRedGroups), 0, st,
                            static_cast<const float *>(workspace), splits, M * N, C, M, N, ldc,
                            epi == EPI_BIAS_COL ? bias : nullptr);
         ODL_LAUNCH_CHECK();

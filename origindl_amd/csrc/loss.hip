@@ -148,22 +148,57 @@ __global__ void ce_finish_kernel(const float *__restrict__ logp, int64_t N, floa
     }
 }
 
-// gx = (softmax(x) - one_hot(t)) * scale, one wave per row, one read and one write of the row
-__global__ void ce_grad_kernel(const float *__restrict__ x, const void *t, int is64, int64_t N, int64_t C, float scale,
-                               float *__restrict__ gx)
+// gx = (softmax(x) - one_hot(t)) * scale, one wave per row. Rows of up to 64*REGS classes stay in registers
+// between the max, the sum and the write, so the logits are read from memory once; longer rows re-read them.
+template <int REGS>
+__global__ __launch_bounds__(kBlock) void ce_grad_kernel(const float *__restrict__ x, const void *t, int is64, int64_t N,
+                                                          int64_t C, float scale, float *__restrict__ gx)
 {
     const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
     if (row >= N)
         return;
     const int lane = threadIdx.x & 63;
-    float m, s;
-    row_stats(x + row * C, C, lane, m, s);
+    const float *xr = x + row * C;
+    float *gr = gx + row * C;
     const int64_t lab = label_at(t, is64, row);
-    for (int64_t j = lane; j < C; j += 64)
+    if (REGS > 0)
     {
-        const float p = expf(x[row * C + j] - m) / s;
-        const float d = p - ((j == lab) ? 1.f : 0.f);
-        gx[row * C + j] = d * scale;
+        float v[REGS > 0 ? REGS : 1];
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int u = 0; u < REGS; ++u)
+        {
+            const int64_t j = lane + 64 * u;
+            v[u] = (j < C) ? xr[j] : -FLT_MAX;
+            m = (m < v[u]) ? v[u] : m;
+        }
+        m = wave_max(m);
+        float s = 0.f;
+#pragma unroll
+        for (int u = 0; u < REGS; ++u)
+        {
+            const int64_t j = lane + 64 * u;
+            v[u] = (j < C) ? expf(v[u] - m) : 0.f;
+            s += v[u];
+        }
+        s = wave_sum(s);
+#pragma unroll
+        for (int u = 0; u < REGS; ++u)
+        {
+            const int64_t j = lane + 64 * u;
+            if (j < C)
+                gr[j] = (v[u] / s - ((j == lab) ? 1.f : 0.f)) * scale;
+        }
+    }
+    else
+    {
+        float m, s;
+        row_stats(xr, C, lane, m, s);
+        for (int64_t j = lane; j < C; j += 64)
+        {
+            const float p = expf(xr[j] - m) / s;
+            gr[j] = (p - ((j == lab) ? 1.f : 0.f)) * scale;
+        }
     }
 }
 
@@ -318,8 +353,16 @@ int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(N > 0 && C > 0, "softmax_cross_entropy backward: empty input");
     const float scale = gy / (float)N;  // softmax_cross_entropy.cpp:105-106
-    hipLaunchKernelGGL(ce_grad_kernel, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, odl::as_stream(stream),
-                       x, t, idx_is_i64, N, C, scale, gx);
+    const dim3 grid((unsigned)odl::ceil_div(N, kWaves));
+    hipStream_t st = odl::as_stream(stream);
+    if (C <= 64)
+        hipLaunchKernelGGL(ce_grad_kernel<1>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+    else if (C <= 256)
+        hipLaunchKernelGGL(ce_grad_kernel<4>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+    else if (C <= 1024)
+        hipLaunchKernelGGL(ce_grad_kernel<16>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+    else
+        hipLaunchKernelGGL(ce_grad_kernel<0>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

@@ -14,7 +14,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 namespace
 {
 constexpr int kBlock = 256;
-constexpr int64_t kTargetThreads = 1 << 18;
 
 inline size_t align256(size_t b)
 {
@@ -102,10 +101,12 @@ __global__ void row_sum_wave_kernel(const float *__restrict__ src, float *__rest
         dst[row] = acc;
 }
 
-// ---- columns: src[outer][axis][inner] -> dst[split][outer][inner]; lanes run along `inner`
+// ---- columns: src[outer][axis][inner] -> dst[split][outer][inner]
+// One thread owns VEC adjacent columns (a workgroup covers 256*VEC contiguous floats of every row it reads) and
+// walks its slice of the axis with eight independent loads in flight.
 template <int VEC>
-__global__ void col_sum_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t outer, int64_t axis,
-                               int64_t inner, int64_t chunk)
+__global__ __launch_bounds__(kBlock) void col_sum_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                          int64_t outer, int64_t axis, int64_t inner, int64_t chunk)
 {
     const int64_t iq = inner / VEC;  // VEC == 4 only when inner % 4 == 0
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -120,11 +121,11 @@ __global__ void col_sum_kernel(const float *__restrict__ src, float *__restrict_
     for (int e = 0; e < VEC; ++e)
         acc[e] = 0.f;
     int64_t a = beg;
-    for (; a + 4 <= end; a += 4)
+    for (; a + 8 <= end; a += 8)
     {
-        float v[4][VEC];
+        float v[8][VEC];
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < 8; ++u)
         {
             if (VEC == 4)
             {
@@ -135,7 +136,7 @@ __global__ void col_sum_kernel(const float *__restrict__ src, float *__restrict_
                 v[u][0] = p[(a + u) * inner];
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < 8; ++u)
 #pragma unroll
             for (int e = 0; e < VEC; ++e)
                 acc[e] += v[u][e];
@@ -150,16 +151,42 @@ __global__ void col_sum_kernel(const float *__restrict__ src, float *__restrict_
         d[e] = acc[e];
 }
 
-// dst[i] = sum over s (ascending) of part[s*n + i]
-__global__ void fold_partials_kernel(const float *__restrict__ part, float *__restrict__ dst, int64_t n, int splits)
+// dst[i] = sum over s of part[s*n + i]. 64 columns x 16 slice groups per workgroup: group g adds slices
+// g, g+16, ... (coalesced along i), the group sums meet in LDS and are added in group order — a fixed order.
+constexpr int kFoldGroups = 16;
+__global__ __launch_bounds__(64 * kFoldGroups) void fold_partials_kernel(const float *__restrict__ part,
+                                                                          float *__restrict__ dst, int64_t n, int splits)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n)
-        return;
-    float s = 0.f;
-    for (int z = 0; z < splits; ++z)
-        s += part[(int64_t)z * n + i];
-    dst[i] = s;
+    __shared__ float sh[kFoldGroups][64];
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int64_t i = (int64_t)blockIdx.x * 64 + lane;
+    float acc = 0.f;
+    if (i < n)
+    {
+        int z = grp;
+        for (; z + 3 * kFoldGroups < splits; z += 4 * kFoldGroups)
+        {
+            const float v0 = part[(int64_t)z * n + i], v1 = part[(int64_t)(z + kFoldGroups) * n + i];
+            const float v2 = part[(int64_t)(z + 2 * kFoldGroups) * n + i];
+            const float v3 = part[(int64_t)(z + 3 * kFoldGroups) * n + i];
+            acc += v0;
+            acc += v1;
+            acc += v2;
+            acc += v3;
+        }
+        for (; z < splits; z += kFoldGroups)
+            acc += part[(int64_t)z * n + i];
+    }
+    sh[grp][lane] = acc;
+    __syncthreads();
+    if (grp == 0 && i < n)
+    {
+        float s = sh[0][lane];
+#pragma unroll
+        for (int k = 1; k < kFoldGroups; ++k)
+            s += sh[k][lane];
+        dst[i] = s;
+    }
 }
 
 // ---- conv bias gradient: gy[N][OC][P] -> part[oc][nsplit]; grid (nsplit, OC)
@@ -302,15 +329,16 @@ SumPlan plan_sum(int64_t outer, int64_t axis, int64_t inner)
         return p;
     }
     const int64_t vec = (inner % 4 == 0) ? 4 : 1;
-    const int64_t cols = outer * (inner / vec);
-    int64_t s = kTargetThreads / (cols > 0 ? cols : 1);
+    const int64_t col_blocks = odl::ceil_div(outer * (inner / vec), kBlock);
+    // ~2048 workgroups (8 per CU) is where this access pattern streams fastest on 256 CUs
+    int64_t s = odl::ceil_div(2048, col_blocks);
     if (s > axis / 16)
         s = axis / 16;
     if (s < 1)
         s = 1;
-    if (s > 1024)
-        s = 1024;
-    p.chunk = odl::ceil_div(axis, s);
+    if (s > 512)
+        s = 512;
+    p.chunk = odl::ceil_div(odl::ceil_div(axis, s), 8) * 8;
     p.splits = (int)odl::ceil_div(axis, p.chunk > 0 ? p.chunk : 1);
     if (p.splits < 1)
         p.splits = 1;
@@ -355,9 +383,9 @@ int sum_axis_launch(const float *src, int64_t outer, int64_t axis, int64_t inner
         return ODL_OK;
     }
     const bool v4 = (inner % 4 == 0) && (reinterpret_cast<uintptr_t>(src) % 16 == 0);
-    const int64_t threads = outer * (v4 ? inner / 4 : inner);
+    const int64_t cols = outer * (v4 ? inner / 4 : inner);
     float *part = p.splits > 1 ? static_cast<float *>(workspace) : dst;
-    const dim3 grid((unsigned)odl::ceil_div(threads, kBlock), (unsigned)p.splits);
+    const dim3 grid((unsigned)odl::ceil_div(cols, kBlock), (unsigned)p.splits);
     if (v4)
         hipLaunchKernelGGL(col_sum_kernel<4>, grid, dim3(kBlock), 0, st, src, part, outer, axis, inner, p.chunk);
     else
@@ -365,8 +393,8 @@ int sum_axis_launch(const float *src, int64_t outer, int64_t axis, int64_t inner
     ODL_LAUNCH_CHECK();
     if (p.splits > 1)
     {
-        hipLaunchKernelGGL(fold_partials_kernel, dim3((unsigned)odl::ceil_div(nout, kBlock)), dim3(kBlock), 0, st, part,
-                           dst, nout, p.splits);
+        hipLaunchKernelGGL(fold_partials_kernel, dim3((unsigned)odl::ceil_div(nout, 64)), dim3(64 * kFoldGroups), 0, st,
+                           part, dst, nout, p.splits);
         ODL_LAUNCH_CHECK();
     }
     return ODL_OK;
