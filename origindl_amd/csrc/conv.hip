@@ -18,6 +18,23 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
                  const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int epi, int64_t P,
                  int split_k, void *workspace, size_t workspace_bytes, hipStream_t st);
 size_t sgemm_workspace(int64_t M, int64_t N, int64_t K, int split_k);
+bool conv_implicit_forward_ok(const float *w, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                              int64_t OH, int64_t OW);
+bool conv_implicit_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                            int64_t OH, int64_t OW);
+bool conv_implicit_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                            int SH, int SW);
+size_t conv_implicit_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
+size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW);
+int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
+                          int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
+                          hipStream_t st);
+int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W,
+                        int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
+                        void *workspace, size_t workspace_bytes, hipStream_t st);
+int conv_implicit_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W,
+                        int64_t OC, int KH, int KW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
+                        size_t workspace_bytes, hipStream_t st);
 int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
                              size_t workspace_bytes, hipStream_t st);
 size_t sum_nchw_channels_workspace(int64_t N, int64_t OC, int64_t P);
@@ -368,15 +385,19 @@ int odl_hip_col2im(const float *col, int64_t N, int64_t C, int64_t H, int64_t W,
     return col2im_launch(col, img, g, to_matrix, odl::as_stream(stream));
 }
 
+// 16-byte aligned stand-in used by the workspace queries, which see shapes only
+static const float *const kAlignedProbe = reinterpret_cast<const float *>(uintptr_t(256));
+
 size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
                                       int SW, int PH, int PW)
 {
-    (void)OC;
     if (KH <= 0 || KW <= 0 || SH <= 0 || SW <= 0)
         return 0;
     const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
     if (OH <= 0 || OW <= 0)
         return 0;
+    if (odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW))
+        return 0;  // the im2col matrix is never materialised
     return align256((size_t)(N * OH * OW * C * KH * KW) * sizeof(float));
 }
 
@@ -393,18 +414,46 @@ int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, in
     const int64_t M = N * g.OH * g.OW, K = C * KH * KW;
     if (M == 0)
         return ODL_OK;
-    const size_t need = odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
-    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need, "conv2d: workspace of %zu bytes required, got %zu",
-                need, workspace_bytes);
     hipStream_t st = odl::as_stream(stream);
+    if (odl::conv_implicit_forward_ok(w, N, C, H, W, OC, KH, KW, g.OH, g.OW))
+        return odl::conv_implicit_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, st);
+    // explicit path: col = im2col(x), then y^T[OC, M] = W2d[OC,K] . col[M,K]^T stored as y[n][oc][p] (+ bias per channel)
+    const size_t need = align256((size_t)(M * K) * sizeof(float));
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
+                "conv2d: this shape/alignment needs a workspace of %zu bytes, got %zu", need, workspace_bytes);
     float *col = static_cast<float *>(workspace);
     rc = im2col_launch(x, col, g, 1, st);
     if (rc != ODL_OK)
         return rc;
-    // y^T[OC, M] = W2d[OC,K] . col[M,K]^T, stored as y[n][oc][p] with the bias added per output channel
     return odl::sgemm_launch(0, 1, OC, M, K, w, K, col, K, y, 0, b, /*EPI_NCHW_ROWB*/ 2, g.OH * g.OW, 1, nullptr, 0,
                              st);
 }
+
+namespace
+{
+// workspace regions of conv2d_backward, in order: [col][split-K partials][permuted weights][bias partials]
+struct BwdPlan
+{
+    bool wgrad_implicit, dgrad_implicit;
+    size_t col_bytes, splitk_bytes, wp_bytes, red_bytes;
+    size_t total() const { return col_bytes + splitk_bytes + wp_bytes + red_bytes; }
+};
+
+BwdPlan plan_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                      int SW, int64_t OH, int64_t OW)
+{
+    BwdPlan p{};
+    const int64_t M = N * OH * OW, K = C * KH * KW;
+    p.wgrad_implicit = odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
+    p.dgrad_implicit = odl::conv_implicit_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW);
+    p.col_bytes = (p.wgrad_implicit && p.dgrad_implicit) ? 0 : align256((size_t)(M * K) * sizeof(float));
+    p.splitk_bytes = align256(p.wgrad_implicit ? odl::conv_implicit_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
+                                               : odl::sgemm_workspace(OC, K, M, 0));
+    p.wp_bytes = p.dgrad_implicit ? align256(odl::conv_implicit_dgrad_workspace(C, OC, KH, KW)) : 0;
+    p.red_bytes = align256(odl::sum_nchw_channels_workspace(N, OC, OH * OW));
+    return p;
+}
+}  // namespace
 
 size_t odl_hip_conv2d_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
                                                int SH, int SW, int PH, int PW)
@@ -414,9 +463,7 @@ size_t odl_hip_conv2d_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, 
     const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
     if (OH <= 0 || OW <= 0)
         return 0;
-    const int64_t M = N * OH * OW, K = C * KH * KW;
-    return align256((size_t)(M * K) * sizeof(float)) + align256(odl::sgemm_workspace(OC, K, M, 0)) +
-           align256(odl::sum_nchw_channels_workspace(N, OC, OH * OW));
+    return plan_backward(kAlignedProbe, N, C, H, W, OC, KH, KW, SH, SW, OH, OW).total();
 }
 
 int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int64_t N, int64_t C, int64_t H, int64_t W,
@@ -432,41 +479,50 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
     const int64_t M = N * g.OH * g.OW, K = C * KH * KW;
     if (M == 0)
         return ODL_OK;
-    const size_t need = odl_hip_conv2d_backward_workspace_bytes(N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
-    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
-                "conv2d_backward: workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    const BwdPlan p = plan_backward(gy, N, C, H, W, OC, KH, KW, SH, SW, g.OH, g.OW);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= p.total(),
+                "conv2d_backward: this shape/alignment needs a workspace of %zu bytes, got %zu", p.total(),
+                workspace_bytes);
     hipStream_t st = odl::as_stream(stream);
     char *ws = static_cast<char *>(workspace);
     float *col = reinterpret_cast<float *>(ws);
-    const size_t col_bytes = align256((size_t)(M * K) * sizeof(float));
-    void *splitk_ws = ws + col_bytes;
-    const size_t splitk_bytes = align256(odl::sgemm_workspace(OC, K, M, 0));
-    void *red_ws = ws + col_bytes + splitk_bytes;
-    const size_t red_bytes = align256(odl::sum_nchw_channels_workspace(N, OC, g.OH * g.OW));
+    void *splitk_ws = ws + p.col_bytes;
+    void *wp_ws = ws + p.col_bytes + p.splitk_bytes;
+    void *red_ws = ws + p.col_bytes + p.splitk_bytes + p.wp_bytes;
 
+    // gy2d: gy's NCHW buffer read as a row-major [M, OC] matrix exactly as it lies (conv2d.cpp:548)
     if (gw)
     {
-        rc = im2col_launch(x, col, g, 1, st);
-        if (rc != ODL_OK)
-            return rc;
-        // gW[OC,K] = gy2d[M,OC]^T . col[M,K]
-        rc = odl::sgemm_launch(1, 0, OC, K, M, gy, OC, col, K, gw, K, nullptr, 0, 0, 0, splitk_ws, splitk_bytes, st);
+        if (p.wgrad_implicit)
+            rc = odl::conv_implicit_wgrad(gy, x, gw, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, splitk_ws,
+                                          p.splitk_bytes, st);
+        else
+        {
+            rc = im2col_launch(x, col, g, 1, st);
+            if (rc == ODL_OK)  // gW[OC,K] = gy2d[M,OC]^T . col[M,K]
+                rc = odl::sgemm_launch(1, 0, OC, K, M, gy, OC, col, K, gw, K, nullptr, 0, 0, 0, splitk_ws,
+                                       p.splitk_bytes, st);
+        }
         if (rc != ODL_OK)
             return rc;
     }
     if (gb)
     {
-        rc = odl::sum_nchw_channels_launch(gy, N, OC, g.OH * g.OW, gb, red_ws, red_bytes, st);
+        rc = odl::sum_nchw_channels_launch(gy, N, OC, g.OH * g.OW, gb, red_ws, p.red_bytes, st);
         if (rc != ODL_OK)
             return rc;
     }
     if (gx)
     {
-        // gx_col[M,K] = gy2d[M,OC] . W2d[OC,K], then the gather back to the image
-        rc = odl::sgemm_launch(0, 0, M, K, OC, gy, OC, w, K, col, K, nullptr, 0, 0, 1, nullptr, 0, st);
-        if (rc != ODL_OK)
-            return rc;
-        rc = col2im_launch(col, gx, g, 1, st);
+        if (p.dgrad_implicit)
+            rc = odl::conv_implicit_dgrad(gy, w, gx, N, C, H, W, OC, KH, KW, PH, PW, g.OH, g.OW, wp_ws, p.wp_bytes, st);
+        else
+        {
+            // gx_col[M,K] = gy2d[M,OC] . W2d[OC,K], then the gather back to the image
+            rc = odl::sgemm_launch(0, 0, M, K, OC, gy, OC, w, K, col, K, nullptr, 0, 0, 1, nullptr, 0, st);
+            if (rc == ODL_OK)
+                rc = col2im_launch(col, gx, g, 1, st);
+        }
         if (rc != ODL_OK)
             return rc;
     }

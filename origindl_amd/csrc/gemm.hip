@@ -36,6 +36,22 @@ enum : int
     EPI_NCHW_ROWB = 2,  // conv forward: row = oc, col = n*P + p -> y[(n*OC + oc)*P + p] (+ bias[oc])
 };
 
+// Where the B operand comes from. Besides a plain matrix it can be gathered on the fly from an NCHW image
+// (the im2col matrix is then never materialised) or from the upstream gradient of a convolution.
+enum : int
+{
+    SB_PLAIN       = 0,
+    SB_CONV_FWD    = 1,  // B(row = output pixel m, k = (c,kh,kw)) = x[n, c, oh*SH-PH+kh, ow*SW-PW+kw]      (forward)
+    SB_CONV_WGRAD  = 2,  // B(k = output pixel m, row = (c,kh,kw)) = same element                            (weight grad)
+    SB_CONV_DGRAD  = 3,  // B(row = input pixel q, k = (kh,kw,oc)) = gy2d[(n, h+PH-kh, w+PW-kw), oc], stride 1 (input grad)
+};
+
+struct ConvSrc
+{
+    int C, H, W, OH, OW, OC;
+    int KH, KW, SH, SW, PH, PW;
+};
+
 struct GemmArgs
 {
     const float *A;
@@ -50,13 +66,17 @@ struct GemmArgs
     int tiles_m, tiles_n;
 };
 
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI>
-__global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g)
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI, int SB = SB_PLAIN, int CK = 0>
+__global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSrc cv)
 {
     // A tile: !TA -> memory is [M][K] (K-contiguous) -> LDS K-major; TA -> memory [K][M] -> LDS row-major.
     // B tile: !TB -> memory is [K][N] (row-contiguous) -> LDS row-major; TB -> memory [N][K] -> LDS K-major.
+    // A gathered B is laid out in LDS the way its gather runs: the forward gather has lanes along the pixels
+    // (rows of B) -> row-major; the weight-grad gather has lanes along the pixels (K of B) and the input-grad
+    // gather reads 16 bytes along oc (K of B) -> K-major.
     constexpr bool A_KMAJOR = !TA;
-    constexpr bool B_KMAJOR = TB;
+    constexpr bool B_KMAJOR = (SB == SB_PLAIN) ? TB : (SB != SB_CONV_FWD);
+    static_assert(SB == SB_PLAIN || BN == 128, "the gather mappings assume 128 B rows per tile");
     constexpr int LDA_S     = A_KMAJOR ? (BK + 4) : (BM + 4);
     constexpr int LDB_S     = B_KMAJOR ? (BK + 4) : (BN + 4);
     constexpr int A_SIZE    = A_KMAJOR ? BM * LDA_S : BK * LDA_S;
@@ -172,6 +192,140 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g)
         }
     };
 
+    // ---- gathered B operands: per-thread state that does not change along K
+    const int KH = CK > 0 ? CK : cv.KH, KW = CK > 0 ? CK : cv.KW;
+    const int KHW = KH * KW;
+    [[maybe_unused]] const float *fw_base = nullptr;  // forward: &x[n, 0, oh*SH-PH, ow*SW-PW] of this thread's pixel
+    [[maybe_unused]] int fw_hb = 0, fw_wb = 0;
+    [[maybe_unused]] bool fw_live = false;
+    [[maybe_unused]] int wg_off[B_PER_T], wg_kh[B_PER_T], wg_kw[B_PER_T];  // weight grad: this thread's 8 (c,kh,kw)
+    [[maybe_unused]] int dg_n[2], dg_h[2], dg_w[2];                        // input grad: this thread's 2 pixels
+    [[maybe_unused]] bool dg_live[2];
+    if constexpr (SB == SB_CONV_FWD)
+    {
+        const int64_t m = n0 + (tid & (BN - 1));
+        fw_live = m < g.N;
+        const int64_t mm = fw_live ? m : 0;
+        const int ow = (int)(mm % cv.OW), oh = (int)((mm / cv.OW) % cv.OH);
+        const int64_t n = mm / ((int64_t)cv.OW * cv.OH);
+        fw_hb = oh * cv.SH - cv.PH, fw_wb = ow * cv.SW - cv.PW;
+        fw_base = g.B + n * cv.C * cv.H * cv.W + (int64_t)fw_hb * cv.W + fw_wb;  // dereferenced only when in bounds
+    }
+    if constexpr (SB == SB_CONV_WGRAD)
+    {
+#pragma unroll
+        for (int u = 0; u < B_PER_T; ++u)
+        {
+            const int64_t ck = n0 + (tid >> 4) + 16 * u;
+            const bool ok = ck < g.N;
+            const int cki = ok ? (int)ck : 0;
+            const int c = cki / KHW, r = cki - c * KHW;
+            const int kh = r / KW, kw = r - kh * KW;
+            wg_off[u] = (c * cv.H + kh) * cv.W + kw;
+            wg_kh[u] = ok ? kh : (1 << 20);  // an out-of-range row fails every bounds check
+            wg_kw[u] = kw;
+        }
+    }
+    if constexpr (SB == SB_CONV_DGRAD)
+    {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+        {
+            const int64_t q = n0 + (tid >> 2) + 64 * u;
+            dg_live[u] = q < g.N;
+            const int64_t qq = dg_live[u] ? q : 0;
+            dg_w[u] = (int)(qq % cv.W);
+            dg_h[u] = (int)((qq / cv.W) % cv.H);
+            dg_n[u] = (int)(qq / ((int64_t)cv.W * cv.H));
+        }
+    }
+
+    auto load_b = [&](int64_t k0) {
+        if constexpr (SB == SB_PLAIN)
+        {
+            load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, k0, BN, rb_, B_PER_T);
+        }
+        else if constexpr (SB == SB_CONV_FWD)
+        {
+            // element u of this thread: row = tid % 128 (its pixel), k = k0 + tid/128 + 2u  (wave-uniform)
+            const int ksub = __builtin_amdgcn_readfirstlane(tid >> 7);
+#pragma unroll
+            for (int u = 0; u < B_PER_T; ++u)
+            {
+                const int k = (int)k0 + ksub + 2 * u;
+                const int c = k / KHW, r = k - c * KHW;
+                const int kh = r / KW, kw = r - kh * KW;
+                const int h = fw_hb + kh, w = fw_wb + kw;
+                const bool ok = fw_live && k < kend && (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
+                rb_[u] = ok ? fw_base[(c * cv.H + kh) * cv.W + kw] : 0.f;
+            }
+        }
+        else if constexpr (SB == SB_CONV_WGRAD)
+        {
+            // element u: k = k0 + tid % 16 (its pixel for this slab), row = tid/16 + 16u
+            const int64_t m = k0 + (tid & 15);
+            const bool live = m < kend;
+            const int64_t mm = live ? m : 0;
+            const int ow = (int)(mm % cv.OW), oh = (int)((mm / cv.OW) % cv.OH);
+            const int64_t n = mm / ((int64_t)cv.OW * cv.OH);
+            const int hb = oh * cv.SH - cv.PH, wb = ow * cv.SW - cv.PW;
+            const float *base = g.B + n * cv.C * cv.H * cv.W + (int64_t)hb * cv.W + wb;
+#pragma unroll
+            for (int u = 0; u < B_PER_T; ++u)
+            {
+                const int h = hb + wg_kh[u], w = wb + wg_kw[u];
+                const bool ok = live && (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
+                rb_[u] = ok ? base[wg_off[u]] : 0.f;
+            }
+        }
+        else
+        {
+            // float4 u: row = tid/4 + 64u (its pixel), k = k0 + 4*(tid%4) .. +3 = four consecutive oc of one tap
+            const int tap = (int)(k0 / cv.OC);  // block-uniform: OC is a multiple of BK, a slab never straddles taps
+            const int oc0 = (int)(k0 - (int64_t)tap * cv.OC) + 4 * (tid & 3);
+            const int kh = tap / KW, kw = tap - kh * KW;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                const int oh = dg_h[u] + cv.PH - kh, ow = dg_w[u] + cv.PW - kw;
+                const bool ok = dg_live[u] && k0 < kend && (unsigned)oh < (unsigned)cv.OH && (unsigned)ow < (unsigned)cv.OW;
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (ok)
+                    v = *reinterpret_cast<const f32x4 *>(g.B + (((int64_t)dg_n[u] * cv.OH + oh) * cv.OW + ow) * cv.OC + oc0);
+                rb_[4 * u] = v[0], rb_[4 * u + 1] = v[1], rb_[4 * u + 2] = v[2], rb_[4 * u + 3] = v[3];
+            }
+        }
+    };
+
+    auto store_b = [&](float *lds) {
+        if constexpr (SB == SB_PLAIN)
+        {
+            store_tile(lds, LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
+        }
+        else if constexpr (SB == SB_CONV_FWD)
+        {
+            const int ksub = tid >> 7;
+#pragma unroll
+            for (int u = 0; u < B_PER_T; ++u)
+                lds[(ksub + 2 * u) * LDB_S + (tid & (BN - 1))] = rb_[u];
+        }
+        else if constexpr (SB == SB_CONV_WGRAD)
+        {
+#pragma unroll
+            for (int u = 0; u < B_PER_T; ++u)
+                lds[((tid >> 4) + 16 * u) * LDB_S + (tid & 15)] = rb_[u];
+        }
+        else
+        {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                f32x4 v = {rb_[4 * u], rb_[4 * u + 1], rb_[4 * u + 2], rb_[4 * u + 3]};
+                *reinterpret_cast<f32x4 *>(lds + ((tid >> 2) + 64 * u) * LDB_S + 4 * (tid & 3)) = v;
+            }
+        }
+    };
+
     f32x16 acc[RB][CB];
 #pragma unroll
     for (int i = 0; i < RB; ++i)
@@ -184,9 +338,9 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g)
     if (nkt > 0)
     {
         load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, kbeg, BM, ra, A_PER_T);
-        load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, kbeg, BN, rb_, B_PER_T);
+        load_b(kbeg);
         store_tile(As[0], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
-        store_tile(Bs[0], LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
+        store_b(Bs[0]);
     }
     __syncthreads();
 
@@ -197,7 +351,7 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g)
         {
             const int64_t k0 = kbeg + (int64_t)(kt + 1) * BK;
             load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra, A_PER_T);
-            load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, k0, BN, rb_, B_PER_T);
+            load_b(k0);
         }
         const float *as = As[cur];
         const float *bs = Bs[cur];
@@ -248,7 +402,7 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g)
         if (kt + 1 < nkt)
         {
             store_tile(As[cur ^ 1], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
-            store_tile(Bs[cur ^ 1], LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
+            store_b(Bs[cur ^ 1]);
         }
         __syncthreads();
     }
@@ -353,7 +507,8 @@ int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g, int splits, hipSt
 #define ODL_GEMM_CASE(TA, TB, V)                                                                      \
     if (ta == TA && tb == TB && vec == V)                                                             \
     {                                                                                                 \
-        hipLaunchKernelGGL((sgemm_mfma_kernel<BM, BN, BK, TA, TB, V, EPI>), grid, block, 0, st, g);   \
+        hipLaunchKernelGGL((sgemm_mfma_kernel<BM, BN, BK, TA, TB, V, EPI>), grid, block, 0, st, g,   \
+                           ConvSrc{});                                                                \
         return ODL_OK;                                                                                \
     }
     ODL_GEMM_CASE(false, false, true)
@@ -453,6 +608,183 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
         rc = launch_tile<kBM, kBN, kBK, EPI_PLAIN>(trans_a, trans_b, vec, g, 1, st);
     if (rc != ODL_OK)
         return fail(rc, "sgemm: no kernel variant");
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+// ------------------------------------------------------------------------------------------------------
+// Convolution as implicit GEMM: the same kernel, its B operand gathered from the image / upstream gradient.
+namespace
+{
+template <int SB, bool TA, int EPI>
+int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, hipStream_t st)
+{
+    const int ck = (cv.KH == 3 && cv.KW == 3) ? 3 : ((cv.KH == 1 && cv.KW == 1) ? 1 : 0);
+    const bool bm64 = g.M <= 64;
+    g.tiles_m = (int)odl::ceil_div(g.M, bm64 ? 64 : 128);
+    g.tiles_n = (int)odl::ceil_div(g.N, 128);
+    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits), block(kThreads);
+#define ODL_CONV_CASE(BMV, CKV)                                                                                  \
+    if (bm64 == (BMV == 64) && ck == CKV)                                                                        \
+    {                                                                                                            \
+        hipLaunchKernelGGL((sgemm_mfma_kernel<BMV, 128, 16, TA, false, true, EPI, SB, CKV>), grid, block, 0, st, \
+                           g, cv);                                                                               \
+        return ODL_OK;                                                                                           \
+    }
+    ODL_CONV_CASE(128, 3)
+    ODL_CONV_CASE(128, 1)
+    ODL_CONV_CASE(128, 0)
+    ODL_CONV_CASE(64, 3)
+    ODL_CONV_CASE(64, 1)
+    ODL_CONV_CASE(64, 0)
+#undef ODL_CONV_CASE
+    return ODL_ERR_RUNTIME;
+}
+
+// wp[c][(kh*KW + kw)*OC + oc] = w[oc][c][kh][kw]
+__global__ void permute_weight_kernel(const float *__restrict__ w, float *__restrict__ wp, int OC, int C, int KHW)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (int64_t)OC * C * KHW)
+        return;
+    const int oc = (int)(t % OC);
+    const int tap = (int)((t / OC) % KHW);
+    const int c = (int)(t / ((int64_t)OC * KHW));
+    wp[t] = w[((int64_t)oc * C + c) * KHW + tap];
+}
+
+bool aligned16(const void *p)
+{
+    return reinterpret_cast<uintptr_t>(p) % 16 == 0;
+}
+
+int wgrad_splits(int64_t OC, int64_t K, int64_t M)
+{
+    const int64_t tiles = odl::ceil_div(OC, OC <= 64 ? 64 : 128) * odl::ceil_div(K, 128);
+    const int64_t kt = odl::ceil_div(M, kBK);
+    int64_t s = odl::ceil_div(768, tiles);
+    if (s > kt / 16)
+        s = kt / 16;
+    if (s > 256)
+        s = 256;
+    return s < 1 ? 1 : (int)s;
+}
+}  // namespace
+
+// shapes the gathered-operand kernels accept (everything else takes the explicit im2col path)
+bool conv_implicit_forward_ok(const float *w, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                              int64_t OH, int64_t OW)
+{
+    const int64_t K = C * KH * KW;
+    return K % 4 == 0 && aligned16(w) && K < (1 << 30) && C * H * W < (1ll << 30) && N * OH * OW < (1ll << 31) &&
+           OC < (1 << 30);
+}
+
+bool conv_implicit_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                            int64_t OH, int64_t OW)
+{
+    return OC % 4 == 0 && aligned16(gy) && C * KH * KW < (1 << 30) && C * H * W < (1ll << 30) &&
+           N * OH * OW < (1ll << 31);
+}
+
+bool conv_implicit_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                            int SH, int SW)
+{
+    return SH == 1 && SW == 1 && OC % 16 == 0 && aligned16(gy) && (int64_t)KH * KW * OC < (1 << 30) &&
+           N * H * W < (1ll << 31) && C < (1 << 30);
+}
+
+size_t conv_implicit_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW)
+{
+    const int64_t K = C * KH * KW, M = N * OH * OW;
+    const int s = wgrad_splits(OC, K, M);
+    return s > 1 ? (size_t)s * OC * K * sizeof(float) : 0;
+}
+
+size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW)
+{
+    return (size_t)C * KH * KW * OC * sizeof(float);
+}
+
+static ConvSrc make_src(int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW, int64_t OC, int KH, int KW, int SH,
+                        int SW, int PH, int PW)
+{
+    return ConvSrc{(int)C, (int)H, (int)W, (int)OH, (int)OW, (int)OC, KH, KW, SH, SW, PH, PW};
+}
+
+// y[n][oc][p] = sum_k W2d[oc][k] * x_gathered[(n,p)][k] + b[oc]
+int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
+                          int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
+                          hipStream_t st)
+{
+    GemmArgs g{};
+    g.A = w, g.B = x, g.C = y, g.bias = b;
+    g.M = OC, g.N = N * OH * OW, g.K = C * KH * KW;
+    g.lda = g.K, g.ldb = 0, g.ldc = 0, g.P = OH * OW;
+    g.k_per_split = ceil_div(g.K, kBK) * kBK, g.c_split_stride = 0;
+    int rc = launch_conv_tile<SB_CONV_FWD, false, EPI_NCHW_ROWB>(g, make_src(C, H, W, OH, OW, OC, KH, KW, SH, SW, PH, PW),
+                                                                 1, st);
+    if (rc != ODL_OK)
+        return fail(rc, "conv2d: no kernel variant");
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+// gW[oc][k] = sum_m gy2d[m][oc] * x_gathered[m][k]   (gy2d = gy's buffer as [N*OH*OW, OC])
+int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W,
+                        int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
+                        void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    const int64_t K = C * KH * KW, M = N * OH * OW;
+    int splits = wgrad_splits(OC, K, M);
+    const size_t need = splits > 1 ? (size_t)splits * OC * K * sizeof(float) : 0;
+    if (splits > 1 && (workspace == nullptr || workspace_bytes < need))
+        splits = 1;
+    GemmArgs g{};
+    g.A = gy, g.B = x, g.bias = nullptr;
+    g.M = OC, g.N = K, g.K = M;
+    g.lda = OC, g.ldb = 0, g.P = 0;
+    g.k_per_split = ceil_div(ceil_div(M, kBK), splits) * kBK;
+    splits = (int)ceil_div(M, g.k_per_split);
+    g.C = splits > 1 ? static_cast<float *>(workspace) : gw;
+    g.ldc = K;
+    g.c_split_stride = splits > 1 ? OC * K : 0;
+    int rc = launch_conv_tile<SB_CONV_WGRAD, true, EPI_PLAIN>(g, make_src(C, H, W, OH, OW, OC, KH, KW, SH, SW, PH, PW),
+                                                              splits, st);
+    if (rc != ODL_OK)
+        return fail(rc, "conv2d_backward: no kernel variant");
+    ODL_LAUNCH_CHECK();
+    if (splits > 1)
+    {
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(OC * K, 64)), dim3(64 * kRedGroups), 0, st,
+                           static_cast<const float *>(workspace), splits, OC * K, gw, OC, K, K, nullptr);
+        ODL_LAUNCH_CHECK();
+    }
+    return ODL_OK;
+}
+
+// gx[n][c][h][w] = sum_{kh,kw,oc} W[oc][c][kh][kw] * gy2d[(n, h+PH-kh, w+PW-kw)][oc]   (stride 1)
+int conv_implicit_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W,
+                        int64_t OC, int KH, int KW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
+                        size_t workspace_bytes, hipStream_t st)
+{
+    const size_t need = conv_implicit_dgrad_workspace(C, OC, KH, KW);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need, "conv2d_backward: workspace of %zu bytes required",
+                need);
+    float *wp = static_cast<float *>(workspace);
+    const int64_t total = OC * C * KH * KW;
+    hipLaunchKernelGGL(permute_weight_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, w, wp, (int)OC,
+                       (int)C, KH * KW);
+    ODL_LAUNCH_CHECK();
+    GemmArgs g{};
+    g.A = wp, g.B = gy, g.C = gx, g.bias = nullptr;
+    g.M = C, g.N = N * H * W, g.K = (int64_t)KH * KW * OC;
+    g.lda = g.K, g.ldb = 0, g.ldc = 0, g.P = H * W;
+    g.k_per_split = g.K, g.c_split_stride = 0;
+    int rc = launch_conv_tile<SB_CONV_DGRAD, false, EPI_NCHW_ROWB>(g, make_src(C, H, W, OH, OW, OC, KH, KW, 1, 1, PH, PW),
+                                                                   1, st);
+    if (rc != ODL_OK)
+        return fail(rc, "conv2d_backward: no kernel variant");
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

@@ -257,24 +257,44 @@ def test_conv_reference_unit_test_vectors(api):
         api.conv2d(x4, dev(np.ones((1, 1, 3, 3), f32)), None, 1, 0)  # no valid output
 
 
-@pytest.mark.parametrize("N,C,H,OC,s,p", [(2, 16, 14, 24, 1, 1), (3, 8, 13, 12, 2, 1), (2, 1, 28, 32, 1, 1)])
-def test_conv_vs_oracle_seeded(api, o, N, C, H, OC, s, p):
-    print("\n[case] conv seeded", N, C, H, OC, s, p, flush=True)
-    rng = np.random.default_rng(N * 100 + C)
-    x = rng.standard_normal((N, C, H, H), dtype=f32)
-    w = (rng.standard_normal((OC, C, 3, 3), dtype=f32) * f32(np.sqrt(2.0 / (C * 9)))).astype(f32)
+# Shapes chosen to reach every code path of the conv entry points: gathered-operand (implicit GEMM) forward needs
+# C*KH*KW % 4 == 0, weight-grad needs OC % 4 == 0, input-grad needs stride 1 and OC % 16 == 0; everything else
+# takes the explicit im2col / col2im path. Kernel sizes 3 and 1 are compiled in, others (5, 2x3) are generic;
+# OC <= 64 uses the 64-row tile, larger OC the 128-row tile.
+CONV_SEEDED = [
+    # N, C, H, W, OC, KH, KW, s, p
+    (2, 16, 14, 14, 24, 3, 3, 1, 1),   # fwd + wgrad implicit, dgrad explicit
+    (3, 8, 13, 13, 12, 3, 3, 2, 1),    # stride 2
+    (2, 1, 28, 28, 32, 3, 3, 1, 1),    # C*9 = 9: explicit forward; implicit wgrad/dgrad
+    (2, 16, 12, 10, 32, 3, 3, 1, 1),   # all three implicit, 64-row tiles, W != H
+    (1, 32, 9, 9, 144, 3, 3, 1, 1),    # all three implicit, 128-row tiles with a ragged second tile
+    (2, 8, 11, 11, 16, 1, 1, 1, 0),    # 1x1
+    (2, 4, 12, 12, 16, 5, 5, 1, 2),    # generic kernel size
+    (2, 6, 10, 9, 16, 2, 3, 1, 1),     # rectangular kernel, K = 36
+    (2, 16, 15, 15, 20, 3, 3, 2, 0),   # stride 2 without padding
+    (5, 64, 7, 7, 48, 3, 3, 1, 1),     # more pixels than one tile column, C = 64
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,OC,KH,KW,s,p", CONV_SEEDED)
+def test_conv_vs_oracle_seeded(api, o, N, C, H, W, OC, KH, KW, s, p):
+    print("\n[case] conv seeded", N, C, H, W, OC, KH, KW, s, p, flush=True)
+    rng = np.random.default_rng(N * 100 + C + OC)
+    x = rng.standard_normal((N, C, H, W), dtype=f32)
+    w = (rng.standard_normal((OC, C, KH, KW), dtype=f32) * f32(np.sqrt(2.0 / (C * KH * KW)))).astype(f32)
     b = rng.standard_normal(OC, dtype=f32)
-    OH = (H + 2 * p - 3) // s + 1
-    gy = rng.standard_normal((N, OC, OH, OH), dtype=f32)
-    yo, gxo, gwo, gbo = np.empty((N, OC, OH, OH), f32), np.empty_like(x), np.empty_like(w), np.empty_like(b)
-    assert o.orc_conv2d(x, w, b, N, C, H, H, OC, 3, 3, s, s, p, p, yo) == 0
-    assert o.orc_conv2d_backward(gy, x, w, N, C, H, H, OC, 3, 3, s, s, p, p, gxo, gwo, gbo) == 0
+    OH, OW = (H + 2 * p - KH) // s + 1, (W + 2 * p - KW) // s + 1
+    gy = rng.standard_normal((N, OC, OH, OW), dtype=f32)
+    yo, gxo, gwo, gbo = np.empty((N, OC, OH, OW), f32), np.empty_like(x), np.empty_like(w), np.empty_like(b)
+    assert o.orc_conv2d(x, w, b, N, C, H, W, OC, KH, KW, s, s, p, p, yo) == 0
+    assert o.orc_conv2d_backward(gy, x, w, N, C, H, W, OC, KH, KW, s, s, p, p, gxo, gwo, gbo) == 0
     by, bgw, bgx = conv_bounds(x, w, gy, (s, s), (p, p), o)
     assert (np.abs(host(api.conv2d(dev(x), dev(w), dev(b), s, p)) - yo) <= by + 1e-6).all()
+    assert (np.abs(host(api.conv2d(dev(x), dev(w), None, s, p)) - (yo - b[None, :, None, None])) <= by + 2e-6).all()
     gx, gw, gb = api.conv2d_backward(dev(gy), dev(x), dev(w), True, s, p)
     assert (np.abs(host(gw) - gwo) <= bgw + 1e-6).all()
     assert (np.abs(host(gx) - gxo) <= bgx + 1e-6).all()
-    np.testing.assert_allclose(host(gb), gbo, atol=1e-5 * np.sqrt(N * OH * OH) * np.abs(gy).max() * np.sqrt(N * OH * OH))
+    np.testing.assert_allclose(host(gb), gbo, atol=1e-5 * np.sqrt(N * OH * OW) * np.abs(gy).max() * np.sqrt(N * OH * OW))
 
 
 def test_conv_full_size_c2_properties(api, o):
