@@ -32,8 +32,11 @@ def test_library_exports_every_declared_symbol():
 
 def test_workspace_queries_need_no_gpu():
     l = _lib.lib()
-    # conv C1 of the benchmark: col matrix [100352, 576] floats
-    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) == 100352 * 576 * 4
+    # conv C1 of the benchmark runs as implicit GEMM: no col matrix, hence no forward workspace
+    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) == 0
+    # C*KH*KW = 9 is not a multiple of 4: explicit im2col path, workspace = the col matrix [N*OH*OW, 9]
+    assert l.query("odl_hip_conv2d_workspace_bytes", 256, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1) == 256 * 28 * 28 * 9 * 4
+    assert l.query("odl_hip_conv2d_backward_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) < 100352 * 576 * 4
     assert l.query("odl_hip_conv2d_workspace_bytes", 1, 1, 2, 2, 1, 3, 3, 1, 1, 0, 0) == 0  # no valid output
     assert l.query("odl_hip_sum_axis_workspace_bytes", 4096, 10, 1) == 0
     assert l.query("odl_hip_sum_axis_workspace_bytes", 1, 16384, 4096) > 0
