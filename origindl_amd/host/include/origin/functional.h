@@ -1,0 +1,64 @@
+// The operators that call the hot path (forward/backward pairs over Mat) and their functional:: wrappers and
+// arithmetic overloads. Names, argument meaning and gradients follow the reference's src/operators/** for:
+// add sub mul div neg pow exp log square sum sum_to broadcast_to mat_mul reshape transpose flatten relu softmax
+// softmax_cross_entropy conv2d max_pool2d.
+#pragma once
+#include "tensor.h"
+
+namespace origin
+{
+namespace functional
+{
+Tensor add(const Tensor &lhs, const Tensor &rhs);
+Tensor sub(const Tensor &lhs, const Tensor &rhs);
+Tensor mul(const Tensor &lhs, const Tensor &rhs);
+Tensor div(const Tensor &lhs, const Tensor &rhs);
+Tensor neg(const Tensor &x);
+Tensor pow(const Tensor &base, const Scalar &exponent);
+Tensor exp(const Tensor &x);
+Tensor log(const Tensor &x);
+Tensor square(const Tensor &x);
+Tensor sum(const Tensor &x, int axis = -1, bool keepdim = false);  // -1: all elements
+Tensor sum_to(const Tensor &x, const Shape &shape);
+Tensor broadcast_to(const Tensor &x, const Shape &shape);
+Tensor mat_mul(const Tensor &x, const Tensor &w);
+Tensor reshape(const Tensor &x, const Shape &shape);
+Tensor transpose(const Tensor &x);
+Tensor flatten(const Tensor &x, int start_dim = 1, int end_dim = -1);
+Tensor relu(const Tensor &x);
+Tensor softmax(const Tensor &x, int axis = -1);
+Tensor softmax_cross_entropy(const Tensor &x, const Tensor &target);
+Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b = nullptr, std::pair<int, int> stride = {1, 1},
+              std::pair<int, int> pad = {0, 0});
+Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b, int stride, int pad);
+Tensor max_pool2d(const Tensor &x, std::pair<int, int> kernel_size, std::pair<int, int> stride = {0, 0},
+                  std::pair<int, int> pad = {0, 0});
+Tensor max_pool2d(const Tensor &x, int kernel_size, int stride = 0, int pad = 0);
+}  // namespace functional
+
+using functional::conv2d;
+
+Tensor operator+(const Tensor &lhs, const Tensor &rhs);
+Tensor operator+(const Tensor &lhs, const Scalar &rhs);
+Tensor operator+(const Scalar &lhs, const Tensor &rhs);
+Tensor operator-(const Tensor &lhs, const Tensor &rhs);
+Tensor operator-(const Tensor &lhs, const Scalar &rhs);
+Tensor operator-(const Scalar &lhs, const Tensor &rhs);
+Tensor operator*(const Tensor &lhs, const Tensor &rhs);
+Tensor operator*(const Tensor &lhs, const Scalar &rhs);
+Tensor operator*(const Scalar &lhs, const Tensor &rhs);
+Tensor operator/(const Tensor &lhs, const Tensor &rhs);
+Tensor operator/(const Tensor &lhs, const Scalar &rhs);
+Tensor operator/(const Scalar &lhs, const Tensor &rhs);
+Tensor operator-(const Tensor &x);
+Tensor operator^(const Tensor &base, const Scalar &exponent);
+Tensor operator>(const Tensor &lhs, const Tensor &rhs);
+Tensor operator>(const Tensor &lhs, const Scalar &rhs);
+Tensor &operator+=(Tensor &lhs, const Tensor &rhs);
+Tensor &operator-=(Tensor &lhs, const Tensor &rhs);
+Tensor &operator*=(Tensor &lhs, const Tensor &rhs);
+Tensor &operator/=(Tensor &lhs, const Tensor &rhs);
+
+// mean(argmax(y, 1) == target) as a 0-dim tensor (src/utils/metrics.cpp:11-70)
+Tensor accuracy(const Tensor &y, const Tensor &target);
+}  // namespace origin

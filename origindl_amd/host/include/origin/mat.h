@@ -1,0 +1,234 @@
+// The Mat plugin boundary and its gfx950 implementation.
+//
+// `Mat` keeps the reference's abstract interface (include/origin/mat/mat.h:20-806) for every virtual the hot
+// path's callers use; `OriginMat` is the concrete class behind `Mat_t`. Where the reference's OriginMat
+// dispatches a device Mat to origin::cuda::* kernels, this one calls the C ABI of libodl_hip.so
+// (include/odl_hip.h). There is no CPU compute path: a Mat on the CPU can be created, copied, reshaped, read
+// and moved to the device — arithmetic on it throws. The CPU backend of the reference is this project's
+// oracle and is never linked into this library.
+#pragma once
+#include <memory>
+#include <utility>
+#include <vector>
+
+#include "base.h"
+
+namespace origin
+{
+constexpr int ORIGIN_BACKEND_TYPE = 0;
+
+// Owning buffer on the host or on the device (device memory comes from a caching pool over odl_hip_malloc,
+// as the reference's Storage sits on its MemoryPool, src/mat/origin/memory/*).
+class Storage
+{
+public:
+    static std::shared_ptr<Storage> create(size_t bytes, DeviceType type, int index = 0);
+    ~Storage();
+    Storage(const Storage &)            = delete;
+    Storage &operator=(const Storage &) = delete;
+    void *data() const { return data_; }
+    size_t size() const { return size_; }
+    DeviceType device_type() const { return type_; }
+    int device_index() const { return index_; }
+    std::shared_ptr<Storage> to_device(DeviceType type, int index) const;  // synchronous copy, like the reference
+
+private:
+    Storage(void *p, size_t n, size_t cap, DeviceType t, int i) : data_(p), size_(n), capacity_(cap), type_(t), index_(i) {}
+    void *data_;
+    size_t size_, capacity_;
+    DeviceType type_;
+    int index_;
+};
+
+class Mat
+{
+public:
+    virtual ~Mat() = default;
+    // ---- lifetime / shape
+    virtual std::unique_ptr<Mat> clone() const                         = 0;
+    virtual std::unique_ptr<Mat> view(const Shape &shape) const        = 0;
+    virtual bool is_contiguous() const                                 = 0;
+    virtual std::unique_ptr<Mat> contiguous() const                    = 0;
+    virtual std::unique_ptr<Mat> reshape(const Shape &shape) const     = 0;
+    virtual std::unique_ptr<Mat> transpose() const                     = 0;
+    virtual Shape shape() const                                        = 0;
+    virtual size_t elements() const                                    = 0;
+    virtual bool is_scalar() const                                     = 0;
+    virtual Scalar scalar_value() const                                = 0;
+    virtual void *data_ptr()                                           = 0;
+    virtual int backend_type() const                                   = 0;
+    virtual DataType dtype() const                                     = 0;
+    virtual std::unique_ptr<Mat> to(DataType target) const             = 0;
+    virtual Device device() const                                      = 0;
+    virtual std::unique_ptr<Mat> to_device(Device device) const        = 0;
+    virtual void print(const std::string &desc = "") const             = 0;
+    // ---- arithmetic (same shape, or one single-element operand)
+    virtual std::unique_ptr<Mat> operator+(const Mat &other) const     = 0;
+    virtual std::unique_ptr<Mat> operator-(const Mat &other) const     = 0;
+    virtual std::unique_ptr<Mat> operator*(const Mat &other) const     = 0;
+    virtual std::unique_ptr<Mat> operator/(const Mat &other) const     = 0;
+    virtual std::unique_ptr<Mat> operator>(const Mat &other) const     = 0;
+    virtual std::unique_ptr<Mat> operator-() const                     = 0;
+    virtual void add_inplace(const Mat &other)                         = 0;
+    virtual void sub_inplace(const Mat &other)                         = 0;
+    virtual void mul_inplace(const Mat &other)                         = 0;
+    virtual void div_inplace(const Mat &other)                         = 0;
+    virtual void neg_inplace()                                         = 0;
+    virtual Mat &operator+=(const Mat &other)                          = 0;
+    virtual Mat &operator-=(const Mat &other)                          = 0;
+    virtual Mat &operator*=(const Mat &other)                          = 0;
+    virtual Mat &operator/=(const Mat &other)                          = 0;
+    virtual std::unique_ptr<Mat> matmul(const Mat &other) const        = 0;
+    // ---- reductions / broadcast
+    virtual std::unique_ptr<Mat> broadcast_to(const Shape &shape) const           = 0;
+    virtual std::unique_ptr<Mat> sum_to(const Shape &shape) const                 = 0;
+    virtual std::unique_ptr<Mat> sum(int axis = -1, bool keepdim = false) const   = 0;
+    virtual std::unique_ptr<Mat> max(int axis = -1) const                         = 0;
+    // ---- math
+    virtual std::unique_ptr<Mat> exp() const                           = 0;
+    virtual std::unique_ptr<Mat> log() const                           = 0;
+    virtual std::unique_ptr<Mat> sqrt() const                          = 0;
+    virtual std::unique_ptr<Mat> square() const                        = 0;
+    virtual std::unique_ptr<Mat> pow(const Scalar &exponent) const     = 0;
+    virtual std::unique_ptr<Mat> relu() const                          = 0;
+    // ---- convolution / pooling
+    virtual std::unique_ptr<Mat> im2col(std::pair<int, int> kernel_size, std::pair<int, int> stride,
+                                        std::pair<int, int> pad, bool to_matrix = true) const = 0;
+    virtual std::unique_ptr<Mat> col2im(const Shape &input_shape, std::pair<int, int> kernel_size,
+                                        std::pair<int, int> stride, std::pair<int, int> pad,
+                                        bool to_matrix = true) const                           = 0;
+    virtual std::unique_ptr<Mat> conv2d(const Mat &W, const Mat *b, std::pair<int, int> stride,
+                                        std::pair<int, int> pad) const                         = 0;
+    virtual std::vector<std::unique_ptr<Mat>> conv2d_backward(const Mat &gy, const Mat &x, const Mat &W, const Mat *b,
+                                                              std::pair<int, int> stride,
+                                                              std::pair<int, int> pad) const   = 0;
+    virtual std::unique_ptr<Mat> max_pool2d(std::pair<int, int> kernel_size, std::pair<int, int> stride,
+                                            std::pair<int, int> pad, std::vector<size_t> *indices = nullptr) const = 0;
+    virtual std::unique_ptr<Mat> max_pool2d_backward(const Mat &gy, std::pair<int, int> kernel_size,
+                                                     std::pair<int, int> stride, std::pair<int, int> pad,
+                                                     const std::vector<size_t> &indices) const = 0;
+    // ---- indexing
+    virtual std::unique_ptr<Mat> gather(const Mat &indices) const                   = 0;
+    virtual std::unique_ptr<Mat> one_hot(const Mat &indices, int num_classes) const = 0;
+};
+
+class OriginMat : public Mat
+{
+public:
+    OriginMat(const Shape &shape, DataType dtype, Device device = Device());
+    OriginMat(std::shared_ptr<Storage> storage, const Shape &shape, DataType dtype);
+    OriginMat(const OriginMat &) = default;  // shares the storage, like the reference's copy
+
+    // factories required of Mat_t by the core (src/core/tensor_impl.cpp:20-43)
+    static std::unique_ptr<Mat> from_scalar(const Scalar &scalar, const Shape &shape, const TensorOptions &options);
+    static std::unique_ptr<Mat> from_memory(const void *data, DataType user_dtype, const Shape &shape,
+                                            const TensorOptions &options);
+    static std::unique_ptr<Mat> randn(const Shape &shape, const TensorOptions &options = TensorOptions());
+    static std::unique_ptr<Mat> zeros(const Shape &shape, const TensorOptions &options = TensorOptions());
+    static std::unique_ptr<Mat> ones(const Shape &shape, const TensorOptions &options = TensorOptions());
+    static std::unique_ptr<Mat> full(const Shape &shape, float value, const TensorOptions &options = TensorOptions());
+
+    std::unique_ptr<Mat> clone() const override;
+    std::unique_ptr<Mat> view(const Shape &shape) const override;
+    bool is_contiguous() const override { return true; }
+    std::unique_ptr<Mat> contiguous() const override;
+    std::unique_ptr<Mat> reshape(const Shape &shape) const override;
+    std::unique_ptr<Mat> transpose() const override;
+    Shape shape() const override { return shape_; }
+    size_t elements() const override { return shape_.elements(); }
+    bool is_scalar() const override { return shape_.elements() == 1; }
+    Scalar scalar_value() const override;
+    void *data_ptr() override { return storage_->data(); }
+    int backend_type() const override { return ORIGIN_BACKEND_TYPE; }
+    DataType dtype() const override { return dtype_; }
+    std::unique_ptr<Mat> to(DataType target) const override;
+    Device device() const override { return Device(storage_->device_type(), storage_->device_index()); }
+    std::unique_ptr<Mat> to_device(Device device) const override;
+    void print(const std::string &desc = "") const override;
+
+    std::unique_ptr<Mat> operator+(const Mat &other) const override;
+    std::unique_ptr<Mat> operator-(const Mat &other) const override;
+    std::unique_ptr<Mat> operator*(const Mat &other) const override;
+    std::unique_ptr<Mat> operator/(const Mat &other) const override;
+    std::unique_ptr<Mat> operator>(const Mat &other) const override;
+    std::unique_ptr<Mat> operator-() const override;
+    void add_inplace(const Mat &other) override;
+    void sub_inplace(const Mat &other) override;
+    void mul_inplace(const Mat &other) override;
+    void div_inplace(const Mat &other) override;
+    void neg_inplace() override;
+    Mat &operator+=(const Mat &other) override;
+    Mat &operator-=(const Mat &other) override;
+    Mat &operator*=(const Mat &other) override;
+    Mat &operator/=(const Mat &other) override;
+    std::unique_ptr<Mat> matmul(const Mat &other) const override;
+
+    std::unique_ptr<Mat> broadcast_to(const Shape &shape) const override;
+    std::unique_ptr<Mat> sum_to(const Shape &shape) const override;
+    std::unique_ptr<Mat> sum(int axis = -1, bool keepdim = false) const override;
+    std::unique_ptr<Mat> max(int axis = -1) const override;
+
+    std::unique_ptr<Mat> exp() const override;
+    std::unique_ptr<Mat> log() const override;
+    std::unique_ptr<Mat> sqrt() const override;
+    std::unique_ptr<Mat> square() const override;
+    std::unique_ptr<Mat> pow(const Scalar &exponent) const override;
+    std::unique_ptr<Mat> relu() const override;
+
+    std::unique_ptr<Mat> im2col(std::pair<int, int> kernel_size, std::pair<int, int> stride, std::pair<int, int> pad,
+                                bool to_matrix = true) const override;
+    std::unique_ptr<Mat> col2im(const Shape &input_shape, std::pair<int, int> kernel_size, std::pair<int, int> stride,
+                                std::pair<int, int> pad, bool to_matrix = true) const override;
+    std::unique_ptr<Mat> conv2d(const Mat &W, const Mat *b, std::pair<int, int> stride,
+                                std::pair<int, int> pad) const override;
+    std::vector<std::unique_ptr<Mat>> conv2d_backward(const Mat &gy, const Mat &x, const Mat &W, const Mat *b,
+                                                      std::pair<int, int> stride,
+                                                      std::pair<int, int> pad) const override;
+    std::unique_ptr<Mat> max_pool2d(std::pair<int, int> kernel_size, std::pair<int, int> stride, std::pair<int, int> pad,
+                                    std::vector<size_t> *indices = nullptr) const override;
+    std::unique_ptr<Mat> max_pool2d_backward(const Mat &gy, std::pair<int, int> kernel_size, std::pair<int, int> stride,
+                                             std::pair<int, int> pad,
+                                             const std::vector<size_t> &indices) const override;
+    std::unique_ptr<Mat> gather(const Mat &indices) const override;
+    std::unique_ptr<Mat> one_hot(const Mat &indices, int num_classes) const override;
+
+    // ---- beyond the reference's Mat: the fused kernels the operators above Mat may use on the device
+    std::unique_ptr<Mat> softmax(int axis) const;
+    float softmax_cross_entropy(const Mat &target) const;                      // loss value (host)
+    std::unique_ptr<Mat> softmax_cross_entropy_backward(const Mat &target, float gy) const;
+    float accuracy(const Mat &target_int32) const;
+
+    // ---- OriginMat-only helpers used by callers (origin_mat.h:442-559 in the reference)
+    const std::shared_ptr<Storage> &storage() const { return storage_; }
+    template <typename T>
+    T *data_ptr()
+    {
+        return static_cast<T *>(storage_->data());
+    }
+    template <typename T>
+    const T *data_ptr() const
+    {
+        return static_cast<const T *>(storage_->data());
+    }
+    template <typename T>
+    std::vector<T> to_vector() const
+    {
+        std::vector<double> d = to_doubles();
+        return std::vector<T>(d.begin(), d.end());
+    }
+    std::vector<float> to_vector() const { return to_vector<float>(); }
+
+private:
+    std::vector<double> to_doubles() const;  // synchronous D2H when on the device
+    Shape shape_;
+    DataType dtype_;
+    std::shared_ptr<Storage> storage_;
+};
+
+using Mat_t = OriginMat;
+
+inline std::unique_ptr<Mat> create_mat(const void *data, DataType dtype, const Shape &shape, const TensorOptions &o)
+{
+    return OriginMat::from_memory(data, dtype, shape, o);
+}
+}  // namespace origin

@@ -1,0 +1,196 @@
+// Module / Sequential / the layers of the benchmark's MLP and CNN, and the optimizers that finish a training
+// step. API as in the reference's include/origin/nn/** and include/origin/optim/**; these are callers of the hot
+// path (host glue), not kernels.
+#pragma once
+#include <functional>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "functional.h"
+
+namespace origin
+{
+class Module
+{
+public:
+    Module() : training_(true) {}
+    virtual ~Module() = default;
+    virtual Tensor forward(const Tensor &input) = 0;
+    Tensor operator()(const Tensor &input) { return forward(input); }
+    virtual std::vector<Parameter *> parameters();
+    void register_parameter(const std::string &name, Parameter &param);
+    void register_module(const std::string &name, std::unique_ptr<Module> module);
+    void train(bool mode = true);
+    void eval() { train(false); }
+    bool is_training() const { return training_; }
+    virtual void to(Device device);
+    void zero_grad();
+
+protected:
+    std::vector<std::pair<std::string, Parameter *>> parameters_;         // registration order
+    std::vector<std::pair<std::string, std::unique_ptr<Module>>> modules_;
+    bool training_;
+};
+
+class Sequential : public Module
+{
+public:
+    void add(std::unique_ptr<Module> module) { layers_.push_back(std::move(module)); }
+    Tensor forward(const Tensor &input) override;
+    std::vector<Parameter *> parameters() override;
+    void to(Device device) override;
+    Module &operator[](size_t index) { return *layers_.at(index); }
+    const Module &operator[](size_t index) const { return *layers_.at(index); }
+    size_t size() const { return layers_.size(); }
+
+private:
+    std::vector<std::unique_ptr<Module>> layers_;
+};
+
+namespace nn
+{
+// weight [in, out] = randn * sqrt(1/in), bias zeros [1, out] (src/nn/layers/linear.cpp:39-62)
+class Linear : public Module
+{
+public:
+    Linear(int in_features, int out_features, bool bias = true);
+    Tensor forward(const Tensor &input) override;
+    Parameter *weight() { return &weight_; }
+    Parameter *bias() { return use_bias_ ? &bias_ : nullptr; }
+    void reset_parameters();
+
+private:
+    int in_features_, out_features_;
+    bool use_bias_;
+    Parameter weight_, bias_;
+};
+
+// weight [OC, C, KH, KW] = randn * sqrt(2/fan_in), bias zeros [OC] (src/nn/layers/conv2d.cpp:78-103)
+class Conv2d : public Module
+{
+public:
+    Conv2d(int in_channels, int out_channels, std::pair<int, int> kernel_size, std::pair<int, int> stride = {1, 1},
+           std::pair<int, int> pad = {0, 0}, bool bias = true);
+    Conv2d(int in_channels, int out_channels, int kernel_size, int stride = 1, int pad = 0, bool bias = true);
+    Tensor forward(const Tensor &input) override;
+    Parameter *weight() { return &weight_; }
+    Parameter *bias() { return use_bias_ ? &bias_ : nullptr; }
+
+private:
+    int in_channels_, out_channels_;
+    std::pair<int, int> kernel_, stride_, pad_;
+    bool use_bias_;
+    Parameter weight_, bias_;
+};
+
+class MaxPool2d : public Module
+{
+public:
+    MaxPool2d(std::pair<int, int> kernel_size, std::pair<int, int> stride = {0, 0}, std::pair<int, int> pad = {0, 0});
+    MaxPool2d(int kernel_size, int stride = 0, int pad = 0);
+    Tensor forward(const Tensor &input) override { return functional::max_pool2d(input, kernel_, stride_, pad_); }
+
+private:
+    std::pair<int, int> kernel_, stride_, pad_;
+};
+
+class ReLU : public Module
+{
+public:
+    Tensor forward(const Tensor &input) override { return functional::relu(input); }
+};
+
+class Flatten : public Module
+{
+public:
+    explicit Flatten(int start_dim = 1, int end_dim = -1) : start_(start_dim), end_(end_dim) {}
+    Tensor forward(const Tensor &input) override { return functional::flatten(input, start_, end_); }
+
+private:
+    int start_, end_;
+};
+
+// MLP({784, 1000, 10}, relu): Linear layers with the activation between them, none after the last
+// (src/nn/models/mlp.cpp:11-61)
+class MLP : public Module
+{
+public:
+    MLP(const std::vector<int> &sizes, std::function<Tensor(const Tensor &)> activation = nullptr);
+    Tensor forward(const Tensor &input) override;
+    Linear &layer(size_t i) { return *layers_.at(i); }
+    size_t num_layers() const { return layers_.size(); }
+
+private:
+    std::vector<Linear *> layers_;
+    std::function<Tensor(const Tensor &)> activation_;
+};
+}  // namespace nn
+
+// ------------------------------------------------------------------------------------------ optimizers
+class Optimizer
+{
+public:
+    explicit Optimizer(Module &target);
+    virtual ~Optimizer() = default;
+    void step();       // filter params with a gradient -> hooks -> step_one each (src/optim/optimizer.cpp:19-53)
+    void zero_grad();
+    void register_hook(std::function<void(std::vector<Parameter *> &)> hook) { hooks_.push_back(std::move(hook)); }
+
+protected:
+    virtual void step_one(Parameter &param) = 0;
+    Module *target_;
+    std::vector<Parameter *> parameters_;
+    std::vector<std::function<void(std::vector<Parameter *> &)>> hooks_;
+};
+
+class SGD : public Optimizer  // src/optim/sgd.cpp:18-75
+{
+public:
+    SGD(Module &target, float lr, float momentum = 0.0f, float weight_decay = 0.0f, bool nesterov = false);
+
+protected:
+    void step_one(Parameter &param) override;
+
+private:
+    float lr_, momentum_, weight_decay_;
+    bool nesterov_;
+    std::unordered_map<Parameter *, Tensor> momentum_buffers_;
+};
+
+class Adam : public Optimizer  // src/optim/adam.cpp:19-114
+{
+public:
+    Adam(Module &target, float lr = 0.001f, float beta1 = 0.9f, float beta2 = 0.999f, float eps = 1e-8f);
+
+protected:
+    void step_one(Parameter &param) override;
+
+private:
+    float lr_, beta1_, beta2_, eps_;
+    std::unordered_map<Parameter *, Tensor> m_buffers_, v_buffers_;
+    std::unordered_map<Parameter *, int> step_counts_;
+};
+
+class WeightDecay  // include/origin/optim/hooks.h:37-66: grad += rate * param, for every parameter
+{
+public:
+    explicit WeightDecay(float rate = 1e-4f) : rate_(rate) {}
+    std::function<void(std::vector<Parameter *> &)> hook() const;
+
+private:
+    float rate_;
+};
+
+// ------------------------------------------------------------------------------------------ device API
+namespace cuda  // the reference's name for "the accelerator" (include/origin/cuda/cuda.h:25-105)
+{
+bool is_available();
+int device_count();
+int current_device();
+void set_device(int device);
+void device_info();
+void synchronize();
+}  // namespace cuda
+}  // namespace origin

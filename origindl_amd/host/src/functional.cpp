@@ -1,0 +1,461 @@
+// Operators over Mat. Gradients restate the reference's backward rules (cited per operator); softmax and
+// softmax-cross-entropy go to the fused device kernels instead of the reference's chain of eight Mat ops.
+#include "origin/functional.h"
+
+namespace origin
+{
+namespace functional
+{
+namespace
+{
+Tensor scalar_like(const Scalar &s, const Tensor &ref)
+{
+    // a Scalar operand becomes a 0-dim tensor on the other operand's device (src/operators/math/add.cpp:110-114);
+    // device tensors are float32 here, so the scalar is materialised as float32
+    const DataType dt = ref.device().type() == DeviceType::kCUDA ? DataType::kFloat32 : s.dtype();
+    return Tensor(s, Shape({}), dtype(dt).device(ref.device()));
+}
+
+// gradient of a broadcasting binary op: reduce back to the operand's shape (left-aligned sum_to, as the reference)
+Tensor fit(const Tensor &g, const Shape &shape)
+{
+    return g.shape() == shape ? g : sum_to(g, shape);
+}
+
+struct BinaryBase : Operator
+{
+    Shape s0, s1;
+    void remember(const std::vector<Tensor> &xs, const char *name)
+    {
+        if (xs.size() != 2)
+            THROW_RUNTIME_ERROR("{} operator requires exactly 2 inputs, but got {}", name, xs.size());
+        s0 = xs[0].shape();
+        s1 = xs[1].shape();
+    }
+};
+
+struct Add : BinaryBase  // src/operators/math/add.cpp:12-55
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        remember(xs, "Add");
+        return {wrap(mat(xs[0]) + mat(xs[1]))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {fit(gys[0], s0), fit(gys[0], s1)};
+    }
+};
+
+struct Sub : BinaryBase  // src/operators/math/sub.cpp
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        remember(xs, "Sub");
+        return {wrap(mat(xs[0]) - mat(xs[1]))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {fit(gys[0], s0), fit(wrap(-mat(gys[0])), s1)};
+    }
+};
+
+struct Mul : BinaryBase  // src/operators/math/mul.cpp:12-53
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        remember(xs, "Mul");
+        return {wrap(mat(xs[0]) * mat(xs[1]))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        const Mat &gy = mat(gys[0]);
+        return {fit(wrap(gy * mat(inputs_[1])), s0), fit(wrap(gy * mat(inputs_[0])), s1)};
+    }
+};
+
+struct Div : BinaryBase  // src/operators/math/div.cpp:28-60
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        remember(xs, "Div");
+        return {wrap(mat(xs[0]) / mat(xs[1]))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        const Mat &gy = mat(gys[0]), &x0 = mat(inputs_[0]), &x1 = mat(inputs_[1]);
+        auto gx0 = gy / x1;
+        auto sq  = x1 * x1;
+        auto gx1 = gy * x0;
+        *gx1 /= *sq;
+        gx1->neg_inplace();
+        return {fit(wrap(std::move(gx0)), s0), fit(wrap(std::move(gx1)), s1)};
+    }
+};
+
+struct Neg : Operator
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(-mat(xs[0]))}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override { return {wrap(-mat(gys[0]))}; }
+};
+
+struct Pow : Operator  // src/operators/math/pow.cpp
+{
+    Scalar e;
+    explicit Pow(const Scalar &s) : e(s) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).pow(e))}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        auto tmp = mat(inputs_[0]).pow(Scalar(e.to_float32() - 1.0f));
+        tmp->mul_inplace(mat(gys[0]));
+        tmp->mul_inplace(mat(scalar_like(Scalar(e.to_float32()), inputs_[0])));
+        return {wrap(std::move(tmp))};
+    }
+};
+
+struct Exp : Operator
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).exp())}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        auto y = mat(inputs_[0]).exp();
+        return {wrap(mat(gys[0]) * *y)};
+    }
+};
+
+struct Log : Operator
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).log())}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {wrap(mat(gys[0]) / mat(inputs_[0]))};
+    }
+};
+
+struct Square : Operator
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).square())}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        auto two_x = mat(inputs_[0]) * mat(scalar_like(Scalar(2.0f), inputs_[0]));
+        return {wrap(mat(gys[0]) * *two_x)};
+    }
+};
+
+struct Sum : Operator  // src/operators/math/sum.cpp: backward = broadcast_to(gy, x.shape)
+{
+    int axis;
+    bool keepdim;
+    Sum(int a, bool k) : axis(a), keepdim(k) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).sum(axis, keepdim))}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        const Shape xs = inputs_[0].shape();
+        if (axis >= 0 && !keepdim && xs.size() > 1)
+        {
+            // put the reduced dim back as size 1 so that the right-aligned broadcast lands on the right axis
+            std::vector<size_t> d = xs.dims();
+            d[axis] = 1;
+            return {wrap(mat(gys[0]).reshape(Shape(d))->broadcast_to(xs))};
+        }
+        return {wrap(mat(gys[0]).broadcast_to(xs))};
+    }
+};
+
+struct SumTo : Operator  // src/operators/math/sum_to.cpp
+{
+    Shape shape;
+    explicit SumTo(const Shape &s) : shape(s) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).sum_to(shape))}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {wrap(mat(gys[0]).broadcast_to(inputs_[0].shape()))};
+    }
+};
+
+struct BroadcastTo : Operator  // src/operators/math/broadcast_to.cpp:10-46: backward = sum_to(gy, x.shape)
+{
+    Shape shape, x_shape;
+    explicit BroadcastTo(const Shape &s) : shape(s) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        x_shape = xs[0].shape();
+        return {wrap(mat(xs[0]).broadcast_to(shape))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {wrap(mat(gys[0]).sum_to(x_shape))};
+    }
+};
+
+struct MatMul : Operator  // src/operators/math/mat_mul.cpp:12-182
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        if (xs.size() != 2)
+            THROW_RUNTIME_ERROR("MatMul operator requires exactly 2 inputs, but got {}", xs.size());
+        return {wrap(mat(xs[0]).matmul(mat(xs[1])))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        // gx = gy . w^T, gw = x^T . gy; the transposes are Mat::transpose() as in the reference — on this backend
+        // a caller that wants to skip the two copies uses odl_hip_matmul_backward (NT / TN GEMMs) directly
+        const Mat &x = mat(inputs_[0]), &w = mat(inputs_[1]), &gy = mat(gys[0]);
+        auto wT = w.transpose();
+        auto xT = x.transpose();
+        return {wrap(gy.matmul(*wT)), wrap(xT->matmul(gy))};
+    }
+};
+
+struct Reshape : Operator
+{
+    Shape shape;
+    explicit Reshape(const Shape &s) : shape(s) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).reshape(shape))}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {wrap(mat(gys[0]).reshape(inputs_[0].shape()))};
+    }
+};
+
+struct Transpose : Operator
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).transpose())}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override { return {wrap(mat(gys[0]).transpose())}; }
+};
+
+struct ReLU : Operator  // src/operators/activation/relu.cpp:13-54: mask = x > 0, gx = gy * mask
+{
+    Tensor mask;
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        if (xs[0].requires_grad())
+            mask = wrap(mat(xs[0]) > mat(scalar_like(Scalar(0.0f), xs[0])));
+        return {wrap(mat(xs[0]).relu())};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override { return {wrap(mat(gys[0]) * mat(mask))}; }
+};
+
+struct Softmax : Operator  // src/operators/activation/softmax.cpp:14-129
+{
+    int axis;
+    explicit Softmax(int a) : axis(a) {}
+    int resolved(const Tensor &x) const
+    {
+        const int nd = (int)x.shape().size();
+        const int a  = axis < 0 ? nd + axis : axis;
+        if (a < 0 || a >= nd)
+            THROW_INVALID_ARG("Invalid axis {} for softmax. Tensor has {} dimensions", axis, nd);
+        return a;
+    }
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        return {wrap(omat(xs[0]).softmax(resolved(xs[0])))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        // gx = y * (gy - sum(gy * y, axis))
+        const Tensor &x = inputs_[0];
+        const int a     = resolved(x);
+        auto y   = omat(x).softmax(a);
+        auto gyy = mat(gys[0]) * *y;
+        std::vector<size_t> d = x.shape().dims();
+        d[a] = 1;
+        auto s    = gyy->sum(a, false)->reshape(Shape(d))->broadcast_to(x.shape());
+        auto diff = mat(gys[0]) - *s;
+        return {wrap(*y * *diff)};
+    }
+};
+
+struct SoftmaxCrossEntropy : Operator  // src/operators/loss/softmax_cross_entropy.cpp:17-111
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        if (xs.size() != 2)
+            THROW_RUNTIME_ERROR("SoftmaxCrossEntropy operator requires exactly 2 inputs (x and target), but got {}",
+                                xs.size());
+        const Tensor &x = xs[0], &t = xs[1];
+        if (x.shape().size() != 2)
+            THROW_INVALID_ARG("SoftmaxCrossEntropy expects x to be 2D (N, C), but got shape {}", x.shape().to_string());
+        if (t.shape().size() != 1)
+            THROW_INVALID_ARG("SoftmaxCrossEntropy expects target to be 1D (N,), but got shape {}",
+                              t.shape().to_string());
+        if (x.shape()[0] != t.shape()[0])
+            THROW_INVALID_ARG("SoftmaxCrossEntropy: batch size mismatch. x has {} samples, target has {} samples",
+                              x.shape()[0], t.shape()[0]);
+        const float loss = omat(x).softmax_cross_entropy(mat(t));  // synchronises, as the reference's .item() does
+        return {Tensor({loss}, Shape{}, dtype(DataType::kFloat32).device(x.device()))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        const Tensor &x = inputs_[0], &t = inputs_[1];
+        const float gy  = gys[0].item<float>();
+        auto gx         = omat(x).softmax_cross_entropy_backward(mat(t), gy);
+        auto gt         = Tensor::zeros(t.shape(), dtype(DataType::kFloat32).device(t.device()));
+        return {wrap(std::move(gx)), gt};
+    }
+};
+
+struct Conv2dOp : Operator  // src/operators/conv/conv2d.cpp:14-89
+{
+    std::pair<int, int> stride, pad;
+    Conv2dOp(std::pair<int, int> s, std::pair<int, int> p) : stride(s), pad(p) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        if (xs.size() < 2 || xs.size() > 3)
+            THROW_RUNTIME_ERROR("Conv2d operator requires 2 or 3 inputs (x, W, [b]), but got {}", xs.size());
+        if (xs[0].shape().size() != 4)
+            THROW_RUNTIME_ERROR("Conv2d forward: x must be 4D (N, C, H, W), but got shape {}", xs[0].shape().to_string());
+        if (xs[1].shape().size() != 4)
+            THROW_RUNTIME_ERROR("Conv2d forward: W must be 4D (OC, C, KH, KW), but got shape {}",
+                                xs[1].shape().to_string());
+        if (xs[0].shape()[1] != xs[1].shape()[1])
+            THROW_RUNTIME_ERROR("Conv2d forward: channel mismatch - x has {} channels, but W expects {} channels",
+                                xs[0].shape()[1], xs[1].shape()[1]);
+        const Mat *b = xs.size() == 3 ? &mat(xs[2]) : nullptr;
+        return {wrap(mat(xs[0]).conv2d(mat(xs[1]), b, stride, pad))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        const Mat &gy = mat(gys[0]);
+        const Mat *b  = inputs_.size() == 3 ? &mat(inputs_[2]) : nullptr;
+        auto grads    = gy.conv2d_backward(gy, mat(inputs_[0]), mat(inputs_[1]), b, stride, pad);
+        std::vector<Tensor> out;
+        for (auto &g : grads)
+            out.push_back(wrap(std::move(g)));
+        return out;
+    }
+};
+
+struct MaxPool2d : Operator  // src/operators/pooling/max_pool2d.cpp:14-86
+{
+    std::pair<int, int> k, s, p;
+    std::vector<size_t> indices;
+    MaxPool2d(std::pair<int, int> kk, std::pair<int, int> ss, std::pair<int, int> pp) : k(kk), s(ss), p(pp) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        return {wrap(mat(xs[0]).max_pool2d(k, s, p, xs[0].requires_grad() ? &indices : nullptr))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        if (indices.empty())
+            THROW_RUNTIME_ERROR("MaxPool2d backward: indices not found. This should not happen when requires_grad=true");
+        return {wrap(mat(inputs_[0]).max_pool2d_backward(mat(gys[0]), k, s, p, indices))};
+    }
+};
+
+template <typename Op, typename... A>
+Tensor apply(const std::vector<Tensor> &xs, A &&...args)
+{
+    auto op = std::make_shared<Op>(std::forward<A>(args)...);
+    return (*op)(xs)[0];
+}
+}  // namespace
+
+Tensor add(const Tensor &a, const Tensor &b) { return apply<Add>({a, b}); }
+Tensor sub(const Tensor &a, const Tensor &b) { return apply<Sub>({a, b}); }
+Tensor mul(const Tensor &a, const Tensor &b) { return apply<Mul>({a, b}); }
+Tensor div(const Tensor &a, const Tensor &b) { return apply<Div>({a, b}); }
+Tensor neg(const Tensor &x) { return apply<Neg>({x}); }
+Tensor pow(const Tensor &x, const Scalar &e) { return apply<Pow>({x}, e); }
+Tensor exp(const Tensor &x) { return apply<Exp>({x}); }
+Tensor log(const Tensor &x) { return apply<Log>({x}); }
+Tensor square(const Tensor &x) { return apply<Square>({x}); }
+Tensor sum(const Tensor &x, int axis, bool keepdim) { return apply<Sum>({x}, axis, keepdim); }
+Tensor sum_to(const Tensor &x, const Shape &s) { return apply<SumTo>({x}, s); }
+Tensor broadcast_to(const Tensor &x, const Shape &s) { return apply<BroadcastTo>({x}, s); }
+Tensor mat_mul(const Tensor &x, const Tensor &w) { return apply<MatMul>({x, w}); }
+Tensor reshape(const Tensor &x, const Shape &s) { return apply<Reshape>({x}, s); }
+Tensor transpose(const Tensor &x) { return apply<Transpose>({x}); }
+Tensor relu(const Tensor &x) { return apply<ReLU>({x}); }
+Tensor softmax(const Tensor &x, int axis) { return apply<Softmax>({x}, axis); }
+Tensor softmax_cross_entropy(const Tensor &x, const Tensor &t) { return apply<SoftmaxCrossEntropy>({x, t}); }
+
+Tensor flatten(const Tensor &x, int start_dim, int end_dim)  // src/operators/shape/flatten.cpp
+{
+    const std::vector<size_t> d = x.shape().dims();
+    const int nd = (int)d.size();
+    const int s = start_dim < 0 ? nd + start_dim : start_dim, e = end_dim < 0 ? nd + end_dim : end_dim;
+    if (s < 0 || s >= nd || e < 0 || e >= nd || s > e)
+        THROW_INVALID_ARG("Flatten: invalid dims - start_dim={}, end_dim={}, shape={}", start_dim, end_dim,
+                          x.shape().to_string());
+    std::vector<size_t> out(d.begin(), d.begin() + s);
+    size_t flat = 1;
+    for (int i = s; i <= e; ++i)
+        flat *= d[i];
+    out.push_back(flat);
+    out.insert(out.end(), d.begin() + e + 1, d.end());
+    return reshape(x, Shape(out));
+}
+
+Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b, std::pair<int, int> stride, std::pair<int, int> pad)
+{
+    std::vector<Tensor> in{x, W};
+    if (b)
+        in.push_back(*b);
+    return apply<Conv2dOp>(in, stride, pad);
+}
+Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b, int stride, int pad)
+{
+    return conv2d(x, W, b, pair(stride), pair(pad));
+}
+Tensor max_pool2d(const Tensor &x, std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p)
+{
+    if (s.first == 0 && s.second == 0)
+        s = k;  // stride defaults to the kernel size
+    return apply<MaxPool2d>({x}, k, s, p);
+}
+Tensor max_pool2d(const Tensor &x, int k, int s, int p)
+{
+    return max_pool2d(x, pair(k), pair(s), pair(p));
+}
+}  // namespace functional
+
+namespace F = functional;
+namespace
+{
+Tensor scalar_of(const Scalar &s, const Tensor &ref)
+{
+    const DataType dt = ref.device().type() == DeviceType::kCUDA ? DataType::kFloat32 : s.dtype();
+    return Tensor(s, Shape({}), dtype(dt).device(ref.device()));
+}
+}  // namespace
+
+Tensor operator+(const Tensor &a, const Tensor &b) { return F::add(a, b); }
+Tensor operator+(const Tensor &a, const Scalar &b) { return F::add(a, scalar_of(b, a)); }
+Tensor operator+(const Scalar &a, const Tensor &b) { return F::add(scalar_of(a, b), b); }
+Tensor operator-(const Tensor &a, const Tensor &b) { return F::sub(a, b); }
+Tensor operator-(const Tensor &a, const Scalar &b) { return F::sub(a, scalar_of(b, a)); }
+Tensor operator-(const Scalar &a, const Tensor &b) { return F::sub(scalar_of(a, b), b); }
+Tensor operator*(const Tensor &a, const Tensor &b) { return F::mul(a, b); }
+Tensor operator*(const Tensor &a, const Scalar &b) { return F::mul(a, scalar_of(b, a)); }
+Tensor operator*(const Scalar &a, const Tensor &b) { return F::mul(scalar_of(a, b), b); }
+Tensor operator/(const Tensor &a, const Tensor &b) { return F::div(a, b); }
+Tensor operator/(const Tensor &a, const Scalar &b) { return F::div(a, scalar_of(b, a)); }
+Tensor operator/(const Scalar &a, const Tensor &b) { return F::div(scalar_of(a, b), b); }
+Tensor operator-(const Tensor &x) { return F::neg(x); }
+Tensor operator^(const Tensor &x, const Scalar &e) { return F::pow(x, e); }
+Tensor operator>(const Tensor &a, const Tensor &b) { return Tensor(*a.impl_->data_ > *b.impl_->data_); }
+Tensor operator>(const Tensor &a, const Scalar &b) { return a > scalar_of(b, a); }
+Tensor &operator+=(Tensor &a, const Tensor &b) { a = a + b; return a; }
+Tensor &operator-=(Tensor &a, const Tensor &b) { a = a - b; return a; }
+Tensor &operator*=(Tensor &a, const Tensor &b) { a = a * b; return a; }
+Tensor &operator/=(Tensor &a, const Tensor &b) { a = a / b; return a; }
+
+Tensor Tensor::reshape(const Shape &shape) const { return F::reshape(*this, shape); }
+Tensor Tensor::transpose() const { return F::transpose(*this); }
+
+Tensor accuracy(const Tensor &y, const Tensor &target)
+{
+    if (y.shape().size() != 2)
+        THROW_INVALID_ARG("accuracy expects y to be 2D (N, C), but got shape {}", y.shape().to_string());
+    if (target.shape().size() != 1)
+        THROW_INVALID_ARG("accuracy expects target to be 1D (N,), but got shape {}", target.shape().to_string());
+    if (y.shape()[0] != target.shape()[0])
+        THROW_INVALID_ARG("accuracy: batch size mismatch. y has {} samples, target has {} samples", y.shape()[0],
+                          target.shape()[0]);
+    const Tensor t32 = target.dtype() == DataType::kInt32 ? target : target.to(DataType::kInt32);
+    const float acc  = static_cast<const OriginMat &>(*y.impl_->data_).accuracy(*t32.impl_->data_);
+    return Tensor({acc}, Shape{}, dtype(DataType::kFloat32).device(y.device()));
+}
+}  // namespace origin

@@ -1,0 +1,844 @@
+// OriginMat over the C ABI of libodl_hip.so: every device operation below is one or two calls into
+// include/odl_hip.h. Validation and error text follow the reference's CPU ops (src/mat/origin/cpu/**) so that
+// callers see the same exceptions; the arithmetic itself lives in the HIP library only.
+#include "origin/mat.h"
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <random>
+
+#include "odl_hip.h"
+
+namespace origin
+{
+namespace
+{
+void check(int rc)
+{
+    if (rc == ODL_OK)
+        return;
+    if (rc == ODL_ERR_INVALID_ARG)
+        throw std::invalid_argument(odl_hip_last_error());
+    throw std::runtime_error(odl_hip_last_error());
+}
+
+// Caching allocator for device memory: freed blocks are kept in size bins (powers of two from 256 B up to 1 MiB,
+// whole MiB above) and handed out again. Everything runs on the null stream, so a block freed by the host is
+// reused only by work queued after every kernel that touched it.
+class DevicePool
+{
+public:
+    static DevicePool &get()
+    {
+        static DevicePool *p = new DevicePool();  // never destroyed: outlives every Storage
+        return *p;
+    }
+    static size_t bin(size_t bytes)
+    {
+        if (bytes <= 256)
+            return 256;
+        if (bytes <= (1u << 20))
+        {
+            size_t b = 256;
+            while (b < bytes)
+                b <<= 1;
+            return b;
+        }
+        return (bytes + (1u << 20) - 1) & ~(size_t)((1u << 20) - 1);
+    }
+    void *alloc(size_t cap)
+    {
+        {
+            std::lock_guard<std::mutex> lk(mu_);
+            auto it = free_.find(cap);
+            if (it != free_.end() && !it->second.empty())
+            {
+                void *p = it->second.back();
+                it->second.pop_back();
+                return p;
+            }
+        }
+        void *p = nullptr;
+        check(odl_hip_malloc(&p, cap));
+        return p;
+    }
+    void release(void *p, size_t cap)
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        free_[cap].push_back(p);
+    }
+
+private:
+    std::mutex mu_;
+    std::map<size_t, std::vector<void *>> free_;
+};
+
+const OriginMat &as_origin(const Mat &m)
+{
+    const auto *p = dynamic_cast<const OriginMat *>(&m);
+    if (!p)
+        THROW_RUNTIME_ERROR("expected an OriginMat, got backend_type={}", m.backend_type());
+    return *p;
+}
+
+// a float32 Mat living on the device: the only thing the kernels compute on
+const OriginMat &dev_f32(const Mat &m, const char *who)
+{
+    const OriginMat &o = as_origin(m);
+    if (o.device().type() != DeviceType::kCUDA)
+        THROW_RUNTIME_ERROR("{}: tensor is on {}; this backend computes on the GPU only (move it with .to(device))", who,
+                            o.device().to_string());
+    if (o.dtype() != DataType::kFloat32)
+        THROW_INVALID_ARG("{}: only float32 is supported on the device, got {}", who, dtype_to_string(o.dtype()));
+    return o;
+}
+
+const float *fp(const OriginMat &m)
+{
+    return m.data_ptr<float>();
+}
+
+std::unique_ptr<OriginMat> new_like(const OriginMat &ref, const Shape &shape, DataType dt = DataType::kFloat32)
+{
+    return std::make_unique<OriginMat>(shape, dt, ref.device());
+}
+
+struct Workspace
+{
+    std::shared_ptr<Storage> s;
+    size_t bytes = 0;
+    explicit Workspace(size_t n, int index) : bytes(n)
+    {
+        if (n)
+            s = Storage::create(n, DeviceType::kCUDA, index);
+    }
+    void *ptr() const { return s ? s->data() : nullptr; }
+};
+
+std::vector<int64_t> dims64(const Shape &s)
+{
+    std::vector<int64_t> d(s.dims().begin(), s.dims().end());
+    if (d.empty())
+        d.push_back(1);  // storage for the pointer; the count passed alongside stays 0
+    return d;
+}
+
+void same_dtype_device(const OriginMat &a, const OriginMat &b, const char *who)
+{
+    if (a.dtype() != b.dtype())
+        THROW_INVALID_ARG("Data type mismatch in {}: expected {} but got {}", who, dtype_to_string(a.dtype()),
+                          dtype_to_string(b.dtype()));
+    if (a.device() != b.device())
+        THROW_INVALID_ARG("Device mismatch in {}: {} vs {}", who, a.device().to_string(), b.device().to_string());
+}
+
+Shape broadcast_shape(const OriginMat &a, const OriginMat &b, const char *who)
+{
+    if (a.shape() == b.shape())
+        return a.shape();
+    if (b.elements() == 1)
+        return a.shape();
+    if (a.elements() == 1)
+        return b.shape();
+    THROW_RUNTIME_ERROR("Complex broadcasting not yet implemented for {} operation: {} vs {}", who,
+                        a.shape().to_string(), b.shape().to_string());
+}
+
+std::unique_ptr<Mat> binary(int op, const char *who, const OriginMat &a, const Mat &other, OriginMat *out = nullptr)
+{
+    const OriginMat &x = dev_f32(a, who);
+    const OriginMat &y = dev_f32(other, who);
+    same_dtype_device(x, y, who);
+    const Shape rs = broadcast_shape(x, y, who);
+    std::unique_ptr<OriginMat> fresh;
+    OriginMat *dst = out;
+    if (!dst)
+    {
+        fresh = new_like(x, rs);
+        dst   = fresh.get();
+    }
+    else if (dst->shape() != rs)
+        THROW_INVALID_ARG("Output tensor mismatch. Expected shape={}, got shape={}", rs.to_string(),
+                          dst->shape().to_string());
+    check(odl_hip_binary(op, fp(x), (int64_t)x.elements(), fp(y), (int64_t)y.elements(), dst->data_ptr<float>(),
+                         nullptr));
+    return fresh;
+}
+
+std::unique_ptr<Mat> unary(int op, const char *who, const OriginMat &a, OriginMat *out = nullptr)
+{
+    const OriginMat &x = dev_f32(a, who);
+    std::unique_ptr<OriginMat> fresh;
+    OriginMat *dst = out;
+    if (!dst)
+    {
+        fresh = new_like(x, x.shape());
+        dst   = fresh.get();
+    }
+    check(odl_hip_unary(op, fp(x), (int64_t)x.elements(), dst->data_ptr<float>(), nullptr));
+    return fresh;
+}
+
+void split_axis(const Shape &s, int axis, int64_t &outer, int64_t &ax, int64_t &inner)
+{
+    outer = inner = 1;
+    for (int i = 0; i < axis; ++i)
+        outer *= (int64_t)s[i];
+    ax = (int64_t)s[axis];
+    for (size_t i = axis + 1; i < s.size(); ++i)
+        inner *= (int64_t)s[i];
+}
+
+int label_kind(const OriginMat &idx, const char *who)
+{
+    if (idx.dtype() == DataType::kInt64)
+        return 1;
+    if (idx.dtype() == DataType::kInt32)
+        return 0;
+    THROW_INVALID_ARG("{}: indices must be int32 or int64, but got {}", who, dtype_to_string(idx.dtype()));
+}
+}  // namespace
+
+// ------------------------------------------------------------------------------------------- Storage
+std::shared_ptr<Storage> Storage::create(size_t bytes, DeviceType type, int index)
+{
+    if (type == DeviceType::kCPU)
+    {
+        const size_t cap = (bytes + 127) & ~(size_t)127;
+        void *p          = cap ? std::aligned_alloc(128, cap) : nullptr;
+        if (cap && !p)
+            THROW_RUNTIME_ERROR("host allocation of {} bytes failed", bytes);
+        return std::shared_ptr<Storage>(new Storage(p, bytes, cap, type, index));
+    }
+    check(odl_hip_set_device(index));
+    const size_t cap = DevicePool::bin(bytes ? bytes : 1);
+    void *p          = DevicePool::get().alloc(cap);
+    return std::shared_ptr<Storage>(new Storage(p, bytes, cap, type, index));
+}
+
+Storage::~Storage()
+{
+    if (!data_)
+        return;
+    if (type_ == DeviceType::kCPU)
+        std::free(data_);
+    else
+        DevicePool::get().release(data_, capacity_);
+}
+
+std::shared_ptr<Storage> Storage::to_device(DeviceType type, int index) const
+{
+    auto dst = Storage::create(size_, type, index);
+    if (size_ == 0)
+        return dst;
+    if (type_ == DeviceType::kCPU && type == DeviceType::kCPU)
+        std::memcpy(dst->data(), data_, size_);
+    else if (type_ == DeviceType::kCPU)
+        check(odl_hip_memcpy_h2d(dst->data(), data_, size_));
+    else if (type == DeviceType::kCPU)
+        check(odl_hip_memcpy_d2h(dst->data(), data_, size_));
+    else
+    {
+        check(odl_hip_memcpy_d2d(dst->data(), data_, size_, nullptr));
+    }
+    return dst;
+}
+
+// ------------------------------------------------------------------------------------------ factories
+OriginMat::OriginMat(const Shape &shape, DataType dtype, Device device)
+    : shape_(shape), dtype_(dtype), storage_(Storage::create(shape.elements() * dtype_size(dtype), device.type(),
+                                                             device.index()))
+{}
+
+OriginMat::OriginMat(std::shared_ptr<Storage> storage, const Shape &shape, DataType dtype)
+    : shape_(shape), dtype_(dtype), storage_(std::move(storage))
+{}
+
+namespace
+{
+// writes n values of `dt` converted from doubles into a host buffer
+void store_as(void *dst, DataType dt, const double *src, size_t n)
+{
+    for (size_t i = 0; i < n; ++i)
+    {
+        switch (dt)
+        {
+            case DataType::kFloat32: static_cast<float *>(dst)[i] = (float)src[i]; break;
+            case DataType::kFloat64: static_cast<double *>(dst)[i] = src[i]; break;
+            case DataType::kInt8: static_cast<int8_t *>(dst)[i] = (int8_t)src[i]; break;
+            case DataType::kInt32: static_cast<int32_t *>(dst)[i] = (int32_t)src[i]; break;
+            case DataType::kInt64: static_cast<int64_t *>(dst)[i] = (int64_t)src[i]; break;
+            default: static_cast<uint8_t *>(dst)[i] = (uint8_t)src[i]; break;
+        }
+    }
+}
+
+double load_as(const void *src, DataType dt, size_t i)
+{
+    switch (dt)
+    {
+        case DataType::kFloat32: return static_cast<const float *>(src)[i];
+        case DataType::kFloat64: return static_cast<const double *>(src)[i];
+        case DataType::kInt8: return static_cast<const int8_t *>(src)[i];
+        case DataType::kInt32: return static_cast<const int32_t *>(src)[i];
+        case DataType::kInt64: return (double)static_cast<const int64_t *>(src)[i];
+        default: return static_cast<const uint8_t *>(src)[i];
+    }
+}
+
+std::unique_ptr<Mat> upload(const void *host, DataType dt, const Shape &shape, Device dev)
+{
+    auto m = std::make_unique<OriginMat>(shape, dt, dev);
+    const size_t bytes = shape.elements() * dtype_size(dt);
+    if (bytes == 0)
+        return m;
+    if (dev.type() == DeviceType::kCPU)
+        std::memcpy(m->data_ptr(), host, bytes);
+    else
+        check(odl_hip_memcpy_h2d(m->data_ptr(), host, bytes));
+    return m;
+}
+}  // namespace
+
+std::unique_ptr<Mat> OriginMat::from_memory(const void *data, DataType user_dtype, const Shape &shape,
+                                            const TensorOptions &options)
+{
+    const size_t n = shape.elements();
+    if (user_dtype == options.dtype())
+        return upload(data, user_dtype, shape, options.device());
+    std::vector<double> tmp(n);
+    for (size_t i = 0; i < n; ++i)
+        tmp[i] = load_as(data, user_dtype, i);
+    std::vector<char> conv(n * dtype_size(options.dtype()));
+    store_as(conv.data(), options.dtype(), tmp.data(), n);
+    return upload(conv.data(), options.dtype(), shape, options.device());
+}
+
+std::unique_ptr<Mat> OriginMat::from_scalar(const Scalar &scalar, const Shape &shape, const TensorOptions &options)
+{
+    const size_t n = shape.elements();
+    if (options.device().type() == DeviceType::kCUDA && options.dtype() == DataType::kFloat32)
+    {
+        auto m = std::make_unique<OriginMat>(shape, DataType::kFloat32, options.device());
+        check(odl_hip_fill(m->data_ptr<float>(), (int64_t)n, scalar.to_float32(), nullptr));
+        return m;
+    }
+    std::vector<double> tmp(n, scalar.to_float64());
+    std::vector<char> conv(n * dtype_size(options.dtype()));
+    store_as(conv.data(), options.dtype(), tmp.data(), n);
+    return upload(conv.data(), options.dtype(), shape, options.device());
+}
+
+std::unique_ptr<Mat> OriginMat::randn(const Shape &shape, const TensorOptions &options)
+{
+    // like the reference (src/mat/origin/cpu/factory.cpp:27-56): mt19937 + normal_distribution on the host,
+    // seeded from random_device — parameter initialisation, not part of the hot path
+    static std::mt19937 gen{std::random_device{}()};
+    std::normal_distribution<float> dist(0.f, 1.f);
+    std::vector<float> host(shape.elements());
+    for (auto &v : host)
+        v = dist(gen);
+    return from_memory(host.data(), DataType::kFloat32, shape, options);
+}
+
+std::unique_ptr<Mat> OriginMat::zeros(const Shape &shape, const TensorOptions &options)
+{
+    return from_scalar(Scalar(0.0f), shape, options);
+}
+
+std::unique_ptr<Mat> OriginMat::ones(const Shape &shape, const TensorOptions &options)
+{
+    return from_scalar(Scalar(1.0f), shape, options);
+}
+
+std::unique_ptr<Mat> OriginMat::full(const Shape &shape, float value, const TensorOptions &options)
+{
+    return from_scalar(Scalar(value), shape, options);
+}
+
+// ------------------------------------------------------------------------------------ lifetime / shape
+std::unique_ptr<Mat> OriginMat::clone() const
+{
+    return std::make_unique<OriginMat>(storage_->to_device(storage_->device_type(), storage_->device_index()), shape_,
+                                       dtype_);
+}
+
+std::unique_ptr<Mat> OriginMat::view(const Shape &shape) const
+{
+    if (shape.elements() != shape_.elements())
+        THROW_INVALID_ARG("view: cannot view shape {} as {}", shape_.to_string(), shape.to_string());
+    return std::make_unique<OriginMat>(storage_, shape, dtype_);  // zero-copy: same storage
+}
+
+std::unique_ptr<Mat> OriginMat::contiguous() const
+{
+    return std::make_unique<OriginMat>(*this);
+}
+
+std::unique_ptr<Mat> OriginMat::reshape(const Shape &shape) const
+{
+    if (shape.elements() != shape_.elements())
+        THROW_INVALID_ARG("reshape: cannot reshape {} ({} elements) to {} ({} elements)", shape_.to_string(),
+                          shape_.elements(), shape.to_string(), shape.elements());
+    return view(shape);
+}
+
+std::unique_ptr<Mat> OriginMat::transpose() const
+{
+    if (shape_.size() < 2)
+        return clone();
+    const OriginMat &x = dev_f32(*this, "transpose");
+    std::vector<size_t> d = shape_.dims();
+    const size_t rows = d[d.size() - 2], cols = d[d.size() - 1];
+    std::swap(d[d.size() - 2], d[d.size() - 1]);
+    auto out = new_like(x, Shape(d));
+    const int64_t outer = (int64_t)(shape_.elements() / ((rows * cols) != 0 ? rows * cols : 1));
+    check(odl_hip_transpose(fp(x), out->data_ptr<float>(), outer, (int64_t)rows, (int64_t)cols, nullptr));
+    return out;
+}
+
+std::vector<double> OriginMat::to_doubles() const
+{
+    const size_t n = shape_.elements();
+    std::vector<double> out(n);
+    if (n == 0)
+        return out;
+    const void *src = storage_->data();
+    std::vector<char> host;
+    if (storage_->device_type() != DeviceType::kCPU)
+    {
+        host.resize(n * dtype_size(dtype_));
+        check(odl_hip_memcpy_d2h(host.data(), storage_->data(), host.size()));
+        src = host.data();
+    }
+    for (size_t i = 0; i < n; ++i)
+        out[i] = load_as(src, dtype_, i);
+    return out;
+}
+
+Scalar OriginMat::scalar_value() const
+{
+    if (shape_.elements() != 1)
+        THROW_INVALID_ARG("scalar_value: tensor has {} elements", shape_.elements());
+    const double v = to_doubles()[0];
+    switch (dtype_)
+    {
+        case DataType::kFloat32: return Scalar((float)v);
+        case DataType::kFloat64: return Scalar(v);
+        case DataType::kInt64: return Scalar((int64_t)v);
+        default: return Scalar((int)v);
+    }
+}
+
+std::unique_ptr<Mat> OriginMat::to(DataType target) const
+{
+    if (target == dtype_)
+        return std::make_unique<OriginMat>(*this);
+    // dtype conversion is host-side plumbing (labels, metrics); it is not a device kernel of this backend
+    const std::vector<double> d = to_doubles();
+    std::vector<char> conv(d.size() * dtype_size(target));
+    store_as(conv.data(), target, d.data(), d.size());
+    return upload(conv.data(), target, shape_, device());
+}
+
+std::unique_ptr<Mat> OriginMat::to_device(Device dev) const
+{
+    if (dev == device())
+        return std::make_unique<OriginMat>(*this);
+    return std::make_unique<OriginMat>(storage_->to_device(dev.type(), dev.index()), shape_, dtype_);
+}
+
+void OriginMat::print(const std::string &desc) const
+{
+    const std::vector<double> d = to_doubles();
+    std::cout << desc << (desc.empty() ? "" : " ") << "Mat" << shape_.to_string() << " " << dtype_to_string(dtype_) << " "
+              << device().to_string() << " [";
+    for (size_t i = 0; i < d.size() && i < 16; ++i)
+        std::cout << (i ? ", " : "") << d[i];
+    std::cout << (d.size() > 16 ? ", ...]" : "]") << std::endl;
+}
+
+// ------------------------------------------------------------------------------------------ arithmetic
+std::unique_ptr<Mat> OriginMat::operator+(const Mat &o) const { return binary(0, "add", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator-(const Mat &o) const { return binary(1, "subtract", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator*(const Mat &o) const { return binary(2, "multiply", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator/(const Mat &o) const { return binary(3, "divide", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator>(const Mat &o) const { return binary(4, "gt", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator-() const { return unary(3, "negate", *this); }
+
+void OriginMat::add_inplace(const Mat &o) { binary(0, "add", *this, o, this); }
+void OriginMat::sub_inplace(const Mat &o) { binary(1, "subtract", *this, o, this); }
+void OriginMat::mul_inplace(const Mat &o) { binary(2, "multiply", *this, o, this); }
+void OriginMat::div_inplace(const Mat &o) { binary(3, "divide", *this, o, this); }
+void OriginMat::neg_inplace() { unary(3, "negate", *this, this); }
+Mat &OriginMat::operator+=(const Mat &o) { add_inplace(o); return *this; }
+Mat &OriginMat::operator-=(const Mat &o) { sub_inplace(o); return *this; }
+Mat &OriginMat::operator*=(const Mat &o) { mul_inplace(o); return *this; }
+Mat &OriginMat::operator/=(const Mat &o) { div_inplace(o); return *this; }
+
+std::unique_ptr<Mat> OriginMat::exp() const { return unary(1, "exp", *this); }
+std::unique_ptr<Mat> OriginMat::log() const { return unary(2, "log", *this); }
+std::unique_ptr<Mat> OriginMat::sqrt() const { return unary(5, "sqrt", *this); }
+std::unique_ptr<Mat> OriginMat::square() const { return unary(4, "square", *this); }
+std::unique_ptr<Mat> OriginMat::relu() const { return unary(0, "relu", *this); }
+
+std::unique_ptr<Mat> OriginMat::pow(const Scalar &exponent) const
+{
+    const OriginMat &x = dev_f32(*this, "pow");
+    auto out = new_like(x, shape_);
+    check(odl_hip_pow_scalar(fp(x), (int64_t)elements(), exponent.to_float32(), out->data_ptr<float>(), nullptr));
+    return out;
+}
+
+std::unique_ptr<Mat> OriginMat::matmul(const Mat &other) const
+{
+    const OriginMat &a = dev_f32(*this, "matmul");
+    const OriginMat &b = dev_f32(other, "matmul");
+    const Shape as = a.shape(), bs = b.shape();
+    if (as.size() < 2 || bs.size() < 2)
+        THROW_INVALID_ARG("Matrix multiplication requires at least 2D tensors. A shape: {}, B shape: {}", as.to_string(),
+                          bs.to_string());
+    int64_t batch = 1, M, K, N;
+    int b_batched = 0;
+    Shape rs;
+    if (as.size() == 2 && bs.size() == 2)
+    {
+        M = as[0], K = as[1], N = bs[1];
+        rs = Shape{as[0], bs[1]};
+    }
+    else if (as.size() == 3 && bs.size() == 2)
+    {
+        batch = as[0], M = as[1], K = as[2], N = bs[1];
+        rs = Shape{as[0], as[1], bs[1]};
+    }
+    else if (as.size() == 3 && bs.size() == 3)
+    {
+        if (as[0] != bs[0])
+            THROW_INVALID_ARG("Matrix dimensions must be compatible for multiplication. A[0]={} != B[0]={}", as[0], bs[0]);
+        batch = as[0], M = as[1], K = as[2], N = bs[2], b_batched = 1;
+        rs = Shape{as[0], as[1], bs[2]};
+    }
+    else
+        THROW_INVALID_ARG("Matrix multiplication requires compatible dimensions. A shape: {}, B shape: {}", as.to_string(),
+                          bs.to_string());
+    if ((int64_t)bs[bs.size() - 2] != K)
+        THROW_INVALID_ARG("Matrix dimensions must be compatible for multiplication. A shape: {}, B shape: {}",
+                          as.to_string(), bs.to_string());
+    auto c = new_like(a, rs);
+    check(odl_hip_matmul(fp(a), fp(b), c->data_ptr<float>(), batch, M, N, K, b_batched, nullptr));
+    return c;
+}
+
+// -------------------------------------------------------------------------------- reductions / broadcast
+std::unique_ptr<Mat> OriginMat::broadcast_to(const Shape &shape) const
+{
+    const OriginMat &x = dev_f32(*this, "broadcast_to");
+    auto out = new_like(x, shape);
+    const auto sd = dims64(shape_), dd = dims64(shape);
+    check(odl_hip_broadcast_to(fp(x), sd.data(), (int)shape_.size(), dd.data(), (int)shape.size(),
+                               out->data_ptr<float>(), nullptr));
+    return out;
+}
+
+std::unique_ptr<Mat> OriginMat::sum_to(const Shape &shape) const
+{
+    if (shape_ == shape)
+        return std::make_unique<OriginMat>(*this);  // storage-sharing copy, src/mat/origin/cpu/math/sum_to.cpp:14-18
+    const OriginMat &x = dev_f32(*this, "sum_to");
+    const auto sd = dims64(shape_), td = dims64(shape);
+    Workspace ws(odl_hip_sum_to_workspace_bytes(sd.data(), (int)shape_.size(), td.data(), (int)shape.size()),
+                 device().index());
+    auto out = new_like(x, shape);
+    check(odl_hip_sum_to(fp(x), sd.data(), (int)shape_.size(), td.data(), (int)shape.size(), out->data_ptr<float>(),
+                         ws.ptr(), ws.bytes, nullptr));
+    return out;
+}
+
+std::unique_ptr<Mat> OriginMat::sum(int axis, bool keepdim) const
+{
+    const OriginMat &x = dev_f32(*this, "sum");
+    if (axis == -1)
+    {
+        const Shape rs = keepdim ? Shape(std::vector<size_t>(shape_.size(), 1)) : Shape{1};
+        auto out = new_like(x, rs);
+        Workspace ws(odl_hip_sum_all_workspace_bytes((int64_t)elements()), device().index());
+        check(odl_hip_sum_all(fp(x), (int64_t)elements(), out->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+        return out;
+    }
+    if (axis < 0 || axis >= (int)shape_.size())
+        THROW_INVALID_ARG("Invalid axis {} for sum operation. Tensor has {} dimensions", axis, shape_.size());
+    std::vector<size_t> rd;
+    for (size_t i = 0; i < shape_.size(); ++i)
+    {
+        if ((int)i != axis)
+            rd.push_back(shape_[i]);
+        else if (keepdim)
+            rd.push_back(1);
+    }
+    int64_t outer, ax, inner;
+    split_axis(shape_, axis, outer, ax, inner);
+    auto out = new_like(x, Shape(rd));
+    Workspace ws(odl_hip_sum_axis_workspace_bytes(outer, ax, inner), device().index());
+    check(odl_hip_sum_axis(fp(x), outer, ax, inner, out->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+    return out;
+}
+
+std::unique_ptr<Mat> OriginMat::max(int axis) const
+{
+    const OriginMat &x = dev_f32(*this, "max");
+    if (axis == -1)
+    {
+        auto out = new_like(x, Shape{1});
+        check(odl_hip_max_all(fp(x), (int64_t)elements(), out->data_ptr<float>(), nullptr));
+        return out;
+    }
+    if (axis < 0 || axis >= (int)shape_.size())
+        THROW_INVALID_ARG("Invalid axis {} for max operation. Tensor has {} dimensions", axis, shape_.size());
+    std::vector<size_t> rd;
+    for (size_t i = 0; i < shape_.size(); ++i)
+        if ((int)i != axis)
+            rd.push_back(shape_[i]);
+    int64_t outer, ax, inner;
+    split_axis(shape_, axis, outer, ax, inner);
+    auto out = new_like(x, Shape(rd));
+    check(odl_hip_max_axis(fp(x), outer, ax, inner, out->data_ptr<float>(), nullptr));
+    return out;
+}
+
+// ----------------------------------------------------------------------------------- convolution / pooling
+std::unique_ptr<Mat> OriginMat::im2col(std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
+                                       bool to_matrix) const
+{
+    const OriginMat &x = dev_f32(*this, "im2col");
+    if (shape_.size() != 4)
+        THROW_INVALID_ARG("im2col: input must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
+    const int OH = get_conv_outsize((int)H, k.first, s.first, p.first);
+    const int OW = get_conv_outsize((int)W, k.second, s.second, p.second);
+    if (OH <= 0 || OW <= 0)
+        THROW_INVALID_ARG("im2col: invalid output size OH={}, OW={} for input H={}, W={}", OH, OW, H, W);
+    const Shape cs = to_matrix ? Shape{(size_t)(N * OH * OW), (size_t)(C * k.first * k.second)}
+                               : Shape{(size_t)N, (size_t)C, (size_t)k.first, (size_t)k.second, (size_t)OH, (size_t)OW};
+    auto col = new_like(x, cs);
+    check(odl_hip_im2col(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
+                         col->data_ptr<float>(), nullptr));
+    return col;
+}
+
+std::unique_ptr<Mat> OriginMat::col2im(const Shape &is, std::pair<int, int> k, std::pair<int, int> s,
+                                       std::pair<int, int> p, bool to_matrix) const
+{
+    const OriginMat &col = dev_f32(*this, "col2im");
+    if (is.size() != 4)
+        THROW_INVALID_ARG("col2im: input_shape must be 4D (N, C, H, W), but got shape {}", is.to_string());
+    const int64_t N = is[0], C = is[1], H = is[2], W = is[3];
+    const int OH = get_conv_outsize((int)H, k.first, s.first, p.first);
+    const int OW = get_conv_outsize((int)W, k.second, s.second, p.second);
+    const Shape want = to_matrix ? Shape{(size_t)(N * OH * OW), (size_t)(C * k.first * k.second)}
+                                 : Shape{(size_t)N, (size_t)C, (size_t)k.first, (size_t)k.second, (size_t)OH, (size_t)OW};
+    if (OH <= 0 || OW <= 0 || shape_ != want)
+        THROW_INVALID_ARG("col2im: invalid col shape {} for input_shape {}", shape_.to_string(), is.to_string());
+    auto img = new_like(col, is);
+    check(odl_hip_col2im(fp(col), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
+                         img->data_ptr<float>(), nullptr));
+    return img;
+}
+
+std::unique_ptr<Mat> OriginMat::conv2d(const Mat &Wm, const Mat *bm, std::pair<int, int> s, std::pair<int, int> p) const
+{
+    const OriginMat &x = dev_f32(*this, "conv2d");
+    const OriginMat &w = dev_f32(Wm, "conv2d");
+    if (shape_.size() != 4)
+        THROW_INVALID_ARG("conv2d: x must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
+    if (w.shape().size() != 4)
+        THROW_INVALID_ARG("conv2d: W must be 4D (OC, C, KH, KW), but got shape {}", w.shape().to_string());
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
+    const int64_t OC = w.shape()[0];
+    const int KH = (int)w.shape()[2], KW = (int)w.shape()[3];
+    if ((int64_t)w.shape()[1] != C)
+        THROW_INVALID_ARG("conv2d: channel mismatch - x has {} channels, but W expects {} channels", C, w.shape()[1]);
+    const int OH = get_conv_outsize((int)H, KH, s.first, p.first), OW = get_conv_outsize((int)W, KW, s.second, p.second);
+    if (OH <= 0 || OW <= 0)
+        THROW_INVALID_ARG("conv2d: invalid output size OH={}, OW={} for input H={}, W={}, kernel=({},{})", OH, OW, H, W,
+                          KH, KW);
+    const float *bias = nullptr;
+    if (bm)
+    {
+        const OriginMat &b = dev_f32(*bm, "conv2d");
+        if (b.shape().size() != 1 || (int64_t)b.shape()[0] != OC)
+            THROW_INVALID_ARG("conv2d: b must be 1D with size {}, but got shape {}", OC, b.shape().to_string());
+        bias = fp(b);
+    }
+    auto y = new_like(x, Shape{(size_t)N, (size_t)OC, (size_t)OH, (size_t)OW});
+    Workspace ws(odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
+                 device().index());
+    check(odl_hip_conv2d(fp(x), fp(w), bias, N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
+                         y->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+    return y;
+}
+
+std::vector<std::unique_ptr<Mat>> OriginMat::conv2d_backward(const Mat &gym, const Mat &xm, const Mat &Wm, const Mat *bm,
+                                                             std::pair<int, int> s, std::pair<int, int> p) const
+{
+    const OriginMat &gy = dev_f32(gym, "conv2d_backward");
+    const OriginMat &x  = dev_f32(xm, "conv2d_backward");
+    const OriginMat &w  = dev_f32(Wm, "conv2d_backward");
+    if (gy.shape().size() != 4)
+        THROW_INVALID_ARG("conv2d_backward: gy must be 4D (N, OC, OH, OW), but got shape {}", gy.shape().to_string());
+    if (x.shape().size() != 4)
+        THROW_INVALID_ARG("conv2d_backward: x must be 4D (N, C, H, W), but got shape {}", x.shape().to_string());
+    if (w.shape().size() != 4)
+        THROW_INVALID_ARG("conv2d_backward: W must be 4D (OC, C, KH, KW), but got shape {}", w.shape().to_string());
+    const int64_t N = x.shape()[0], C = x.shape()[1], H = x.shape()[2], W = x.shape()[3];
+    const int64_t OC = w.shape()[0];
+    const int KH = (int)w.shape()[2], KW = (int)w.shape()[3];
+    auto gx = new_like(x, x.shape());
+    auto gw = new_like(x, w.shape());
+    std::unique_ptr<OriginMat> gb;
+    if (bm)
+        gb = new_like(x, Shape{(size_t)OC});
+    Workspace ws(odl_hip_conv2d_backward_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
+                 device().index());
+    check(odl_hip_conv2d_backward(fp(gy), fp(x), fp(w), N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
+                                  gx->data_ptr<float>(), gw->data_ptr<float>(), gb ? gb->data_ptr<float>() : nullptr,
+                                  ws.ptr(), ws.bytes, nullptr));
+    std::vector<std::unique_ptr<Mat>> grads;  // {gx, gW, [gb]}
+    grads.push_back(std::move(gx));
+    grads.push_back(std::move(gw));
+    if (gb)
+        grads.push_back(std::move(gb));
+    return grads;
+}
+
+std::unique_ptr<Mat> OriginMat::max_pool2d(std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
+                                           std::vector<size_t> *indices) const
+{
+    const OriginMat &x = dev_f32(*this, "max_pool2d");
+    if (shape_.size() != 4)
+        THROW_INVALID_ARG("max_pool2d: x must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
+    const int OH = get_conv_outsize((int)H, k.first, s.first, p.first);
+    const int OW = get_conv_outsize((int)W, k.second, s.second, p.second);
+    if (OH <= 0 || OW <= 0)
+        THROW_INVALID_ARG("max_pool2d: invalid output size OH={}, OW={} for input H={}, W={}", OH, OW, H, W);
+    auto y = new_like(x, Shape{(size_t)N, (size_t)C, (size_t)OH, (size_t)OW});
+    const size_t n = y->elements();
+    std::shared_ptr<Storage> idx;
+    if (indices)
+        idx = Storage::create(n * sizeof(uint64_t), DeviceType::kCUDA, device().index());
+    check(odl_hip_max_pool2d(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second,
+                             y->data_ptr<float>(), idx ? static_cast<uint64_t *>(idx->data()) : nullptr, nullptr));
+    if (indices)
+    {
+        // the interface hands the window-local indices to the caller as a host vector (mat.h:560-566)
+        static_assert(sizeof(size_t) == sizeof(uint64_t), "size_t must be 64-bit");
+        indices->resize(n);
+        check(odl_hip_memcpy_d2h(indices->data(), idx->data(), n * sizeof(uint64_t)));
+    }
+    return y;
+}
+
+std::unique_ptr<Mat> OriginMat::max_pool2d_backward(const Mat &gym, std::pair<int, int> k, std::pair<int, int> s,
+                                                    std::pair<int, int> p, const std::vector<size_t> &indices) const
+{
+    const OriginMat &gy = dev_f32(gym, "max_pool2d_backward");
+    if (gy.shape().size() != 4)
+        THROW_INVALID_ARG("max_pool2d_backward: gy must be 4D (N, C, OH, OW), but got shape {}", gy.shape().to_string());
+    if (indices.size() != gy.elements())
+        THROW_INVALID_ARG("max_pool2d_backward: indices size mismatch. Expected {}, got {}", gy.elements(),
+                          indices.size());
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
+    auto idx = Storage::create(indices.size() * sizeof(uint64_t), DeviceType::kCUDA, gy.device().index());
+    check(odl_hip_memcpy_h2d(idx->data(), indices.data(), indices.size() * sizeof(uint64_t)));
+    auto gx = new_like(gy, shape_);
+    check(odl_hip_max_pool2d_backward(fp(gy), static_cast<const uint64_t *>(idx->data()), N, C, H, W, k.first, k.second,
+                                      s.first, s.second, p.first, p.second, gx->data_ptr<float>(), nullptr));
+    return gx;
+}
+
+// -------------------------------------------------------------------------------------------- indexing
+std::unique_ptr<Mat> OriginMat::gather(const Mat &indices) const
+{
+    const OriginMat &x   = dev_f32(*this, "gather");
+    const OriginMat &idx = as_origin(indices);
+    if (shape_.size() != 2)
+        THROW_INVALID_ARG("gather: input must be 2D (N, C), but got shape {}", shape_.to_string());
+    if (idx.shape().size() != 1)
+        THROW_INVALID_ARG("gather: indices must be 1D (N,), but got shape {}", idx.shape().to_string());
+    if (shape_[0] != idx.shape()[0])
+        THROW_INVALID_ARG("gather: batch size mismatch. input has {} samples, indices has {} samples", shape_[0],
+                          idx.shape()[0]);
+    if (idx.device() != device())
+        THROW_INVALID_ARG("gather: input and indices must be on the same device");
+    const int is64 = label_kind(idx, "gather");
+    auto out = new_like(x, Shape{shape_[0]});
+    check(odl_hip_gather(fp(x), idx.storage()->data(), is64, (int64_t)shape_[0], (int64_t)shape_[1],
+                         out->data_ptr<float>(), nullptr));
+    return out;
+}
+
+std::unique_ptr<Mat> OriginMat::one_hot(const Mat &indices, int num_classes) const
+{
+    const OriginMat &idx = as_origin(indices);
+    if (idx.shape().size() != 1)
+        THROW_INVALID_ARG("one_hot: indices must be 1D (N,), but got shape {}", idx.shape().to_string());
+    if (num_classes <= 0)
+        THROW_INVALID_ARG("one_hot: num_classes must be positive, but got {}", num_classes);
+    if (idx.device().type() != DeviceType::kCUDA)
+        THROW_RUNTIME_ERROR("one_hot: indices are on {}; this backend computes on the GPU only", idx.device().to_string());
+    const int is64 = label_kind(idx, "one_hot");
+    auto out = std::make_unique<OriginMat>(Shape{idx.shape()[0], (size_t)num_classes}, DataType::kFloat32, idx.device());
+    check(odl_hip_one_hot(idx.storage()->data(), is64, (int64_t)idx.shape()[0], num_classes, out->data_ptr<float>(),
+                          nullptr));
+    return out;
+}
+
+// ------------------------------------------------------------------------ fused paths above the Mat set
+std::unique_ptr<Mat> OriginMat::softmax(int axis) const
+{
+    const OriginMat &x = dev_f32(*this, "softmax");
+    int64_t outer, ax, inner;
+    split_axis(shape_, axis, outer, ax, inner);
+    auto y = new_like(x, shape_);
+    check(odl_hip_softmax(fp(x), outer, ax, inner, y->data_ptr<float>(), nullptr));
+    return y;
+}
+
+float OriginMat::softmax_cross_entropy(const Mat &target) const
+{
+    const OriginMat &x = dev_f32(*this, "softmax_cross_entropy");
+    const OriginMat &t = as_origin(target);
+    const int is64     = label_kind(t, "gather");
+    const int64_t N = shape_[0], C = shape_[1];
+    Workspace ws(odl_hip_softmax_ce_loss_workspace_bytes(N), device().index());
+    float loss = 0.f;
+    check(odl_hip_softmax_ce_loss(fp(x), t.storage()->data(), is64, N, C, &loss, ws.ptr(), ws.bytes, nullptr));
+    return loss;
+}
+
+std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_backward(const Mat &target, float gy) const
+{
+    const OriginMat &x = dev_f32(*this, "softmax_cross_entropy");
+    const OriginMat &t = as_origin(target);
+    const int is64     = label_kind(t, "one_hot");
+    auto gx = new_like(x, shape_);
+    check(odl_hip_softmax_ce_grad(fp(x), t.storage()->data(), is64, (int64_t)shape_[0], (int64_t)shape_[1], gy,
+                                  gx->data_ptr<float>(), nullptr));
+    return gx;
+}
+
+float OriginMat::accuracy(const Mat &target_int32) const
+{
+    const OriginMat &y = dev_f32(*this, "accuracy");
+    const OriginMat &t = as_origin(target_int32);
+    if (t.dtype() != DataType::kInt32 || t.device() != device())
+        THROW_INVALID_ARG("accuracy: target must be int32 on the same device");
+    Workspace ws(odl_hip_accuracy_workspace_bytes((int64_t)shape_[0]), device().index());
+    float acc = 0.f;
+    check(odl_hip_accuracy(fp(y), t.data_ptr<int32_t>(), (int64_t)shape_[0], (int64_t)shape_[1], &acc, ws.ptr(),
+                           ws.bytes, nullptr));
+    return acc;
+}
+}  // namespace origin

@@ -1,0 +1,319 @@
+// Host glue above the operators: modules, layers, optimizers, device API (see origin/nn.h).
+#include "origin/nn.h"
+
+#include <cmath>
+#include <random>
+
+#include "odl_hip.h"
+
+namespace origin
+{
+// ------------------------------------------------------------------------------------------- Module
+std::vector<Parameter *> Module::parameters()
+{
+    std::vector<Parameter *> out;
+    for (auto &p : parameters_)
+        out.push_back(p.second);
+    for (auto &m : modules_)
+        for (auto *p : m.second->parameters())
+            out.push_back(p);
+    return out;
+}
+
+void Module::register_parameter(const std::string &name, Parameter &param)
+{
+    parameters_.emplace_back(name, &param);
+}
+
+void Module::register_module(const std::string &name, std::unique_ptr<Module> module)
+{
+    modules_.emplace_back(name, std::move(module));
+}
+
+void Module::train(bool mode)
+{
+    training_ = mode;
+    for (auto &m : modules_)
+        m.second->train(mode);
+}
+
+void Module::to(Device device)
+{
+    for (auto *p : parameters())
+        if (p->defined() && p->device() != device)
+        {
+            Tensor moved = static_cast<const Tensor &>(*p).to(device);
+            moved.impl_->requires_grad_ = true;
+            *p = moved;
+        }
+}
+
+void Module::zero_grad()
+{
+    for (auto *p : parameters())
+        p->clear_grad();
+}
+
+Tensor Sequential::forward(const Tensor &input)
+{
+    Tensor x = input;
+    for (auto &l : layers_)
+        x = l->forward(x);
+    return x;
+}
+
+std::vector<Parameter *> Sequential::parameters()
+{
+    std::vector<Parameter *> out;
+    for (auto &l : layers_)
+        for (auto *p : l->parameters())
+            out.push_back(p);
+    return out;
+}
+
+void Sequential::to(Device device)
+{
+    for (auto &l : layers_)
+        l->to(device);
+}
+
+// ------------------------------------------------------------------------------------------- layers
+namespace
+{
+// randn * scale generated on the host (parameter initialisation is not a device kernel of this backend)
+Parameter scaled_randn(const Shape &shape, float scale)
+{
+    static std::mt19937 gen{std::random_device{}()};
+    std::normal_distribution<float> dist(0.f, 1.f);
+    std::vector<float> host(shape.elements());
+    for (auto &v : host)
+        v = dist(gen) * scale;
+    return Parameter(Tensor(host, shape, dtype(DataType::kFloat32).requires_grad(true)));
+}
+}  // namespace
+
+namespace nn
+{
+Linear::Linear(int in_features, int out_features, bool bias)
+    : in_features_(in_features), out_features_(out_features), use_bias_(bias)
+{
+    reset_parameters();
+    register_parameter("weight", weight_);
+    if (use_bias_)
+        register_parameter("bias", bias_);
+}
+
+void Linear::reset_parameters()
+{
+    weight_ = scaled_randn(Shape{(size_t)in_features_, (size_t)out_features_}, std::sqrt(1.0f / (float)in_features_));
+    if (use_bias_)
+        bias_ = Parameter(Tensor::zeros(Shape{1, (size_t)out_features_}, dtype(DataType::kFloat32).requires_grad(true)));
+}
+
+Tensor Linear::forward(const Tensor &input)
+{
+    if (weight_.shape().elements() == 0)
+        THROW_RUNTIME_ERROR("Weight is empty in forward! weight_.shape() = {}", weight_.shape().to_string());
+    auto output = functional::mat_mul(input, static_cast<const Tensor &>(weight_));
+    if (use_bias_)
+        output = output + functional::broadcast_to(bias_, output.shape());  // src/nn/layers/linear.cpp:96-102
+    return output;
+}
+
+Conv2d::Conv2d(int in_channels, int out_channels, std::pair<int, int> kernel_size, std::pair<int, int> stride,
+               std::pair<int, int> pad, bool bias)
+    : in_channels_(in_channels), out_channels_(out_channels), kernel_(kernel_size), stride_(stride), pad_(pad),
+      use_bias_(bias)
+{
+    const float fan_in = (float)(in_channels * kernel_.first * kernel_.second);
+    weight_ = scaled_randn(Shape{(size_t)out_channels, (size_t)in_channels, (size_t)kernel_.first, (size_t)kernel_.second},
+                           std::sqrt(2.0f / fan_in));
+    register_parameter("weight", weight_);
+    if (use_bias_)
+    {
+        bias_ = Parameter(Tensor::zeros(Shape{(size_t)out_channels}, dtype(DataType::kFloat32).requires_grad(true)));
+        register_parameter("bias", bias_);
+    }
+}
+
+Conv2d::Conv2d(int in_channels, int out_channels, int kernel_size, int stride, int pad, bool bias)
+    : Conv2d(in_channels, out_channels, pair(kernel_size), pair(stride), pair(pad), bias)
+{}
+
+Tensor Conv2d::forward(const Tensor &input)
+{
+    if (input.shape().size() != 4)
+        THROW_RUNTIME_ERROR("Conv2d forward: input must be 4D (N, C, H, W), but got shape {}", input.shape().to_string());
+    if (input.shape()[1] != (size_t)in_channels_)
+        THROW_RUNTIME_ERROR("Conv2d forward: input channel mismatch - input has {} channels, but layer expects {} channels",
+                            input.shape()[1], in_channels_);
+    const Tensor *b = use_bias_ ? &static_cast<const Tensor &>(bias_) : nullptr;
+    return functional::conv2d(input, static_cast<const Tensor &>(weight_), b, stride_, pad_);
+}
+
+MaxPool2d::MaxPool2d(std::pair<int, int> kernel_size, std::pair<int, int> stride, std::pair<int, int> pad)
+    : kernel_(kernel_size), stride_((stride.first == 0 && stride.second == 0) ? kernel_size : stride), pad_(pad)
+{}
+
+MaxPool2d::MaxPool2d(int kernel_size, int stride, int pad) : MaxPool2d(pair(kernel_size), pair(stride), pair(pad)) {}
+
+MLP::MLP(const std::vector<int> &sizes, std::function<Tensor(const Tensor &)> activation)
+    : activation_(activation ? std::move(activation) : [](const Tensor &x) { return functional::relu(x); })
+{
+    if (sizes.size() < 2)
+        THROW_INVALID_ARG("MLP needs at least an input and an output size");
+    for (size_t i = 0; i + 1 < sizes.size(); ++i)
+    {
+        auto l = std::make_unique<Linear>(sizes[i], sizes[i + 1], true);
+        layers_.push_back(l.get());
+        register_module("l" + std::to_string(i), std::move(l));
+    }
+}
+
+Tensor MLP::forward(const Tensor &input)
+{
+    Tensor x = input;
+    for (size_t i = 0; i < layers_.size(); ++i)
+    {
+        x = layers_[i]->forward(x);
+        if (i + 1 < layers_.size())
+            x = activation_(x);
+    }
+    return x;
+}
+}  // namespace nn
+
+// ---------------------------------------------------------------------------------------- optimizers
+Optimizer::Optimizer(Module &target) : target_(&target), parameters_(target.parameters()) {}
+
+void Optimizer::step()
+{
+    std::vector<Parameter *> with_grad;
+    for (auto *p : parameters_)
+        if (p->defined() && p->grad().defined())
+            with_grad.push_back(p);
+    for (auto &h : hooks_)
+        h(with_grad);
+    for (auto *p : with_grad)
+        step_one(*p);
+}
+
+void Optimizer::zero_grad()
+{
+    for (auto *p : parameters_)
+        p->clear_grad();
+}
+
+namespace
+{
+// The updated parameter starts a fresh graph: it must stay a leaf, otherwise every later backward would walk
+// back through all earlier optimizer steps.
+Parameter as_leaf(const Tensor &updated)
+{
+    Tensor t = updated.detach();
+    t.impl_->requires_grad_ = true;
+    return Parameter(t);
+}
+}  // namespace
+
+SGD::SGD(Module &target, float lr, float momentum, float weight_decay, bool nesterov)
+    : Optimizer(target), lr_(lr), momentum_(momentum), weight_decay_(weight_decay), nesterov_(nesterov)
+{}
+
+void SGD::step_one(Parameter &param)
+{
+    NoGradGuard guard;
+    Tensor grad = param.grad();
+    if (weight_decay_ > 0.0f)
+        grad = grad + param * Scalar(weight_decay_);
+    if (momentum_ > 0.0f)
+    {
+        auto it = momentum_buffers_.find(&param);
+        if (it == momentum_buffers_.end())
+            it = momentum_buffers_.emplace(&param, Tensor::zeros(grad.shape(), TensorOptions(grad.dtype()).device(grad.device()))).first;
+        Tensor &buf = it->second;
+        buf  = buf * Scalar(momentum_) + grad;
+        grad = nesterov_ ? grad + buf * Scalar(momentum_) : buf;
+    }
+    param = as_leaf(param - grad * Scalar(lr_));
+}
+
+Adam::Adam(Module &target, float lr, float beta1, float beta2, float eps)
+    : Optimizer(target), lr_(lr), beta1_(beta1), beta2_(beta2), eps_(eps)
+{}
+
+void Adam::step_one(Parameter &param)
+{
+    NoGradGuard guard;
+    const Tensor grad = param.grad();
+    auto zeros = [&] { return Tensor::zeros(grad.shape(), TensorOptions(grad.dtype()).device(grad.device())); };
+    if (!m_buffers_.count(&param))
+        m_buffers_.emplace(&param, zeros());
+    if (!v_buffers_.count(&param))
+        v_buffers_.emplace(&param, zeros());
+    int &t = step_counts_[&param];
+    ++t;
+    Tensor &m = m_buffers_.at(&param), &v = v_buffers_.at(&param);
+    // same sequence of elementwise steps, each rounded to float, as src/optim/adam.cpp:52-113
+    m = m * Scalar(beta1_) + grad * Scalar(1.0f - beta1_);
+    v = v * Scalar(beta2_) + (grad * grad) * Scalar(1.0f - beta2_);
+    const float b1p = std::pow(beta1_, static_cast<float>(t)), b2p = std::pow(beta2_, static_cast<float>(t));
+    const Tensor m_hat = m * Scalar(1.0f / (1.0f - b1p));
+    const Tensor v_hat = v * Scalar(1.0f / (1.0f - b2p));
+    const Tensor denom = functional::pow(v_hat, Scalar(0.5f)) + Scalar(eps_);
+    param = as_leaf(param - (m_hat / denom) * Scalar(lr_));
+}
+
+std::function<void(std::vector<Parameter *> &)> WeightDecay::hook() const
+{
+    const float rate = rate_;
+    return [rate](std::vector<Parameter *> &params) {
+        NoGradGuard guard;
+        for (auto *p : params)
+            if (p)
+                p->accumulate_grad(static_cast<const Tensor &>(*p) * Scalar(rate));
+    };
+}
+
+// ----------------------------------------------------------------------------------------- device API
+namespace cuda
+{
+int device_count()
+{
+    int n = 0;
+    odl_hip_device_count(&n);
+    return n;
+}
+bool is_available()
+{
+    return device_count() > 0;
+}
+int current_device()
+{
+    int d = 0;
+    if (odl_hip_get_device(&d) != ODL_OK)
+        THROW_RUNTIME_ERROR("{}", odl_hip_last_error());
+    return d;
+}
+void set_device(int device)
+{
+    if (odl_hip_set_device(device) != ODL_OK)
+        THROW_RUNTIME_ERROR("{}", odl_hip_last_error());
+}
+void device_info()
+{
+    const int n = device_count();
+    for (int i = 0; i < n; ++i)
+    {
+        char buf[256];
+        if (odl_hip_device_info(i, buf, sizeof(buf)) == ODL_OK)
+            loga("Device {}: {}", i, buf);
+    }
+}
+void synchronize()
+{
+    if (odl_hip_synchronize() != ODL_OK)
+        THROW_RUNTIME_ERROR("{}", odl_hip_last_error());
+}
+}  // namespace cuda
+}  // namespace origin

@@ -1,9 +1,12 @@
-// TEST INFRASTRUCTURE, NOT PRODUCT CODE.
-// C-ABI driver over the reference's own CPU backend (compiled from the reference sources by
-// oracle/Makefile into oracle/_ref/libodl_ref.so). It only *calls* the reference's public
-// Tensor/Operator/Mat API — no algorithm is restated here — so that tests can check the plain-C
-// oracle against the real thing bit for bit, tests/golden/make_golden.py can write fixtures, and
-// the benchmark can time the reference CPU path beside the GPU.
+// TEST INFRASTRUCTURE: one driver source, two backends.
+// A C-ABI driver written against OriginDL's public Tensor / Operator / Mat API only — no algorithm is restated
+// here. It is compiled twice:
+//   * against the reference's own headers and CPU backend (oracle/Makefile -> oracle/_ref/libodl_ref.so, entry
+//     points odl_ref_*, tensors on the CPU): the real reference, used to pin the plain-C oracle bit for bit, to
+//     write tests/golden fixtures and as the CPU baseline of the benchmark;
+//   * against this repository's host layer (origindl_amd/host, -DDRV_ON_DEVICE -DDRV_PREFIX=odl_host_, tensors on
+//     the GPU): the same calls then run on the gfx950 backend, which is what "drop-in behind the Tensor/Operator/
+//     Mat interfaces" means; tests compare its results with the fixtures and the oracle.
 // Every entry point returns 0, or -1 for std::invalid_argument, -2 for any other std::exception.
 #include <cstdint>
 #include <cstring>
@@ -48,8 +51,21 @@
 using namespace origin;
 namespace F = origin::functional;
 
+#ifndef DRV_PREFIX
+#    define DRV_PREFIX odl_ref_
+#endif
+#define DRV_CAT_(a, b) a##b
+#define DRV_CAT(a, b) DRV_CAT_(a, b)
+#define DRV(name) DRV_CAT(DRV_PREFIX, name)
+
 namespace
 {
+#ifdef DRV_ON_DEVICE
+const Device kDev(DeviceType::kCUDA, 0);
+#else
+const Device kDev(DeviceType::kCPU, 0);
+#endif
+
 Shape make_shape(const int64_t *dims, int n)
 {
     std::vector<size_t> d(dims, dims + n);
@@ -59,7 +75,7 @@ Shape make_shape(const int64_t *dims, int n)
 Tensor f32(const float *p, const Shape &s, bool grad = false)
 {
     std::vector<float> v(p, p + s.elements());
-    return Tensor(v, s, dtype(DataType::kFloat32).requires_grad(grad));
+    return Tensor(v, s, dtype(DataType::kFloat32).requires_grad(grad).device(kDev));
 }
 
 Tensor labels(const void *p, int is64, int64_t n)
@@ -67,21 +83,21 @@ Tensor labels(const void *p, int is64, int64_t n)
     if (is64)
     {
         std::vector<int64_t> v((const int64_t *)p, (const int64_t *)p + n);
-        return Tensor(v, Shape{(size_t)n}, dtype(DataType::kInt64));
+        return Tensor(v, Shape{(size_t)n}, dtype(DataType::kInt64).device(kDev));
     }
     std::vector<int32_t> v((const int32_t *)p, (const int32_t *)p + n);
-    return Tensor(v, Shape{(size_t)n}, dtype(DataType::kInt32));
+    return Tensor(v, Shape{(size_t)n}, dtype(DataType::kInt32).device(kDev));
 }
 
 std::unique_ptr<origin::Mat> mat_f32(const float *p, const Shape &s)
 {
-    return OriginMat::from_memory(p, DataType::kFloat32, s, TensorOptions(DataType::kFloat32));
+    return OriginMat::from_memory(p, DataType::kFloat32, s, TensorOptions(DataType::kFloat32).device(kDev));
 }
 
 std::unique_ptr<origin::Mat> mat_labels(const void *p, int is64, int64_t n)
 {
     return OriginMat::from_memory(p, is64 ? DataType::kInt64 : DataType::kInt32, Shape{(size_t)n},
-                                  TensorOptions(is64 ? DataType::kInt64 : DataType::kInt32));
+                                  TensorOptions(is64 ? DataType::kInt64 : DataType::kInt32).device(kDev));
 }
 
 void out(const Tensor &t, float *dst)
@@ -117,12 +133,12 @@ int guarded(Fn &&fn)
 
 extern "C" {
 
-int odl_ref_ping()
+int DRV(ping)()
 {
     return 1;
 }
 
-int odl_ref_matmul(const float *a, const float *b, float *c, int64_t m, int64_t n, int64_t k)
+int DRV(matmul)(const float *a, const float *b, float *c, int64_t m, int64_t n, int64_t k)
 {
     return guarded([&] {
         auto y = F::mat_mul(f32(a, Shape{(size_t)m, (size_t)k}), f32(b, Shape{(size_t)k, (size_t)n}));
@@ -130,7 +146,7 @@ int odl_ref_matmul(const float *a, const float *b, float *c, int64_t m, int64_t 
     });
 }
 
-int odl_ref_matmul_batched(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t n, int64_t k,
+int DRV(matmul_batched)(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t n, int64_t k,
                            int b_is_batched)
 {
     return guarded([&] {
@@ -141,7 +157,7 @@ int odl_ref_matmul_batched(const float *a, const float *b, float *c, int64_t bat
 }
 
 // forward + backward with an injected upstream gradient: z = y * dC; z.backward() seeds ones.
-int odl_ref_matmul_fwd_bwd(const float *x, const float *w, const float *gy, float *y, float *gx, float *gw, int64_t m,
+int DRV(matmul_fwd_bwd)(const float *x, const float *w, const float *gy, float *y, float *gx, float *gw, int64_t m,
                            int64_t k, int64_t n)
 {
     return guarded([&] {
@@ -157,12 +173,12 @@ int odl_ref_matmul_fwd_bwd(const float *x, const float *w, const float *gy, floa
     });
 }
 
-int odl_ref_transpose(const float *src, float *dst, const int64_t *shape, int nd)
+int DRV(transpose)(const float *src, float *dst, const int64_t *shape, int nd)
 {
     return guarded([&] { out(f32(src, make_shape(shape, nd)).transpose(), dst); });
 }
 
-int odl_ref_im2col(const float *img, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
+int DRV(im2col)(const float *img, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
                    int PW, int to_matrix, float *col)
 {
     return guarded([&] {
@@ -171,7 +187,7 @@ int odl_ref_im2col(const float *img, int64_t N, int64_t C, int64_t H, int64_t W,
     });
 }
 
-int odl_ref_col2im(const float *col, const int64_t *col_shape, int col_nd, int64_t N, int64_t C, int64_t H, int64_t W,
+int DRV(col2im)(const float *col, const int64_t *col_shape, int col_nd, int64_t N, int64_t C, int64_t H, int64_t W,
                    int KH, int KW, int SH, int SW, int PH, int PW, int to_matrix, float *img)
 {
     return guarded([&] {
@@ -181,7 +197,7 @@ int odl_ref_col2im(const float *col, const int64_t *col_shape, int col_nd, int64
     });
 }
 
-int odl_ref_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+int DRV(conv2d)(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
                    int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *y)
 {
     return guarded([&] {
@@ -195,7 +211,7 @@ int odl_ref_conv2d(const float *x, const float *w, const float *b, int64_t N, in
 }
 
 // full operator path: y = conv2d(x, W, b); (y * gy).backward()
-int odl_ref_conv2d_backward(const float *gy, const float *x, const float *w, const float *b, int64_t N, int64_t C,
+int DRV(conv2d_backward)(const float *gy, const float *x, const float *w, const float *b, int64_t N, int64_t C,
                             int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *gx,
                             float *gw, float *gb)
 {
@@ -216,28 +232,28 @@ int odl_ref_conv2d_backward(const float *gy, const float *x, const float *w, con
     });
 }
 
-int odl_ref_sum(const float *src, const int64_t *shape, int nd, int axis, int keepdim, float *dst)
+int DRV(sum)(const float *src, const int64_t *shape, int nd, int axis, int keepdim, float *dst)
 {
     return guarded([&] { out(F::sum(f32(src, make_shape(shape, nd)), axis, keepdim != 0), dst); });
 }
 
-int odl_ref_max(const float *src, const int64_t *shape, int nd, int axis, float *dst)
+int DRV(max)(const float *src, const int64_t *shape, int nd, int axis, float *dst)
 {
     return guarded([&] { out(*mat_f32(src, make_shape(shape, nd))->max(axis), dst); });
 }
 
-int odl_ref_sum_to(const float *src, const int64_t *sshape, int sn, const int64_t *tshape, int tn, float *dst)
+int DRV(sum_to)(const float *src, const int64_t *sshape, int sn, const int64_t *tshape, int tn, float *dst)
 {
     return guarded([&] { out(F::sum_to(f32(src, make_shape(sshape, sn)), make_shape(tshape, tn)), dst); });
 }
 
-int odl_ref_broadcast_to(const float *src, const int64_t *sshape, int sn, const int64_t *dshape, int dn, float *dst)
+int DRV(broadcast_to)(const float *src, const int64_t *sshape, int sn, const int64_t *dshape, int dn, float *dst)
 {
     return guarded([&] { out(F::broadcast_to(f32(src, make_shape(sshape, sn)), make_shape(dshape, dn)), dst); });
 }
 
 // backward of broadcast_to with upstream gradient g (left-aligned sum_to inside the reference)
-int odl_ref_broadcast_to_backward(const float *src, const int64_t *sshape, int sn, const int64_t *dshape, int dn,
+int DRV(broadcast_to_backward)(const float *src, const int64_t *sshape, int sn, const int64_t *dshape, int dn,
                                   const float *g, float *gsrc)
 {
     return guarded([&] {
@@ -249,12 +265,12 @@ int odl_ref_broadcast_to_backward(const float *src, const int64_t *sshape, int s
     });
 }
 
-int odl_ref_softmax(const float *x, const int64_t *shape, int nd, int axis, float *y)
+int DRV(softmax)(const float *x, const int64_t *shape, int nd, int axis, float *y)
 {
     return guarded([&] { out(F::softmax(f32(x, make_shape(shape, nd)), axis), y); });
 }
 
-int odl_ref_gather(const float *in, const void *idx, int is64, int64_t N, int64_t C, float *o)
+int DRV(gather)(const float *in, const void *idx, int is64, int64_t N, int64_t C, float *o)
 {
     return guarded([&] {
         auto m = mat_f32(in, Shape{(size_t)N, (size_t)C});
@@ -262,7 +278,7 @@ int odl_ref_gather(const float *in, const void *idx, int is64, int64_t N, int64_
     });
 }
 
-int odl_ref_one_hot(const void *idx, int is64, int64_t N, int64_t C, float *o)
+int DRV(one_hot)(const void *idx, int is64, int64_t N, int64_t C, float *o)
 {
     return guarded([&] {
         auto t = mat_labels(idx, is64, N);
@@ -270,7 +286,7 @@ int odl_ref_one_hot(const void *idx, int is64, int64_t N, int64_t C, float *o)
     });
 }
 
-int odl_ref_softmax_ce(const float *x, const void *t, int is64, int64_t N, int64_t C, float *loss, float *gx)
+int DRV(softmax_ce)(const float *x, const void *t, int is64, int64_t N, int64_t C, float *loss, float *gx)
 {
     return guarded([&] {
         auto X = f32(x, Shape{(size_t)N, (size_t)C}, true);
@@ -285,7 +301,7 @@ int odl_ref_softmax_ce(const float *x, const void *t, int is64, int64_t N, int64
     });
 }
 
-int odl_ref_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+int DRV(max_pool2d)(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
                        int PH, int PW, float *y, uint64_t *idx)
 {
     return guarded([&] {
@@ -297,7 +313,7 @@ int odl_ref_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t 
     });
 }
 
-int odl_ref_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N, int64_t C, int64_t H, int64_t W,
+int DRV(max_pool2d_backward)(const float *gy, const uint64_t *idx, int64_t N, int64_t C, int64_t H, int64_t W,
                                 int KH, int KW, int SH, int SW, int PH, int PW, float *gx)
 {
     return guarded([&] {
@@ -310,17 +326,17 @@ int odl_ref_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N,
     });
 }
 
-int odl_ref_accuracy(const float *y, const int32_t *t, int64_t N, int64_t C, float *acc)
+int DRV(accuracy)(const float *y, const int32_t *t, int64_t N, int64_t C, float *acc)
 {
     return guarded([&] {
         std::vector<int32_t> tv(t, t + N);
-        auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt32));
+        auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt32).device(kDev));
         *acc   = accuracy(f32(y, Shape{(size_t)N, (size_t)C}), T).item<float>();
     });
 }
 
 // op: 0 add 1 sub 2 mul 3 div 4 gt
-int odl_ref_binary(int op, const float *a, const int64_t *ashape, int an, const float *b, const int64_t *bshape, int bn,
+int DRV(binary)(int op, const float *a, const int64_t *ashape, int an, const float *b, const int64_t *bshape, int bn,
                    float *o)
 {
     return guarded([&] {
@@ -340,7 +356,7 @@ int odl_ref_binary(int op, const float *a, const int64_t *ashape, int an, const 
 }
 
 // op: 0 relu 1 exp 2 log 3 neg 4 square
-int odl_ref_unary(int op, const float *a, int64_t n, float *o)
+int DRV(unary)(int op, const float *a, int64_t n, float *o)
 {
     return guarded([&] {
         auto A = f32(a, Shape{(size_t)n});
@@ -357,14 +373,14 @@ int odl_ref_unary(int op, const float *a, int64_t n, float *o)
     });
 }
 
-int odl_ref_pow_scalar(const float *a, int64_t n, float e, float *o)
+int DRV(pow_scalar)(const float *a, int64_t n, float e, float *o)
 {
     return guarded([&] { out(F::pow(f32(a, Shape{(size_t)n}), Scalar(e)), o); });
 }
 
 // MLP D -> Hd -> C (Linear, ReLU, Linear), softmax CE, WeightDecay hook, Adam; `steps` steps on the same batch.
 // Parameters are read and written in place; loss/grads/logits of the LAST step are returned.
-int odl_ref_mlp_train(const float *x, const void *t, int is64, int64_t N, int64_t D, int64_t Hd, int64_t C, float *W1,
+int DRV(mlp_train)(const float *x, const void *t, int is64, int64_t N, int64_t D, int64_t Hd, int64_t C, float *W1,
                       float *b1, float *W2, float *b2, int steps, float lr, float beta1, float beta2, float eps,
                       float wd, float *loss, float *gW1, float *gb1, float *gW2, float *gb2, float *logits)
 {
@@ -407,7 +423,7 @@ int odl_ref_mlp_train(const float *x, const void *t, int is64, int64_t N, int64_
 }
 
 // CNN of BASELINE config 4 (no BatchNorm), SGD without momentum/weight decay, one step.
-int odl_ref_cnn_train(const float *x, const void *t, int is64, int64_t N, int64_t S, int64_t C1, int64_t C2, int64_t Hd,
+int DRV(cnn_train)(const float *x, const void *t, int is64, int64_t N, int64_t S, int64_t C1, int64_t C2, int64_t Hd,
                       int64_t Cc, float *Wc1, float *bc1, float *Wc2, float *bc2, float *Wl1, float *bl1, float *Wl2,
                       float *bl2, float lr, float *loss, float *gWc1, float *gbc1, float *gWc2, float *gbc2,
                       float *gWl1, float *gbl1, float *gWl2, float *gbl2, float *logits)

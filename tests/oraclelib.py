@@ -142,5 +142,22 @@ def ref():
     return _ref
 
 
+HOST_DRIVER_SO = os.path.join(ROOT, "origindl_amd", "lib", "libodl_host_driver.so")
+HOST_CPU_DRIVER_SO = os.path.join(ROOT, "origindl_amd", "lib", "libodl_hostcpu_driver.so")
+_host = {}
+
+
+def host_driver(cpu=False):
+    """tests/api_driver.cpp compiled against this repository's C++ host layer (origindl_amd/host): the same calls
+    the reference driver makes, running on the gfx950 backend (odl_host_*), or with tensors left on the CPU
+    (odl_hostcpu_*, where every compute call must refuse)."""
+    key = "hostcpu" if cpu else "host"
+    if key not in _host:
+        prefix = "odl_%s_" % key
+        sigs = {k.replace("odl_ref_", prefix): v for k, v in _REF_SIGS.items()}
+        _host[key] = _Lib(HOST_CPU_DRIVER_SO if cpu else HOST_DRIVER_SO, sigs)
+    return _host[key]
+
+
 def shape_arr(shape):
     return np.asarray(list(shape), dtype=np.int64)

@@ -54,3 +54,20 @@ def test_compute_refuses_to_run_without_a_gpu():
     assert rc == _lib.ODL_ERR_RUNTIME and "HIP device" in l.last_error()
     with pytest.raises(_lib.OdlRuntimeError):
         l.call("odl_hip_sgemm", 0, 0, 4, 4, 4, None, 4, None, 4, None, 4, None, 0, None, 0, None)
+
+
+def test_host_layer_refuses_cpu_compute():
+    """The C++ host layer has no CPU compute path: with tensors left on the CPU every operator call throws
+    runtime_error (the API driver reports -2), while creation / transfer of CPU tensors still works."""
+    import numpy as np
+    import oraclelib as ol
+    if not os.path.exists(ol.HOST_CPU_DRIVER_SO):
+        pytest.skip("host layer not built")
+    h = ol.host_driver(cpu=True)
+    assert h.odl_hostcpu_ping() == 1
+    a, b, c = np.ones((2, 3), np.float32), np.ones((3, 2), np.float32), np.zeros((2, 2), np.float32)
+    assert h.odl_hostcpu_matmul(a, b, c, 2, 2, 3) == -2
+    assert h.odl_hostcpu_unary(0, a, 6, np.zeros_like(a)) == -2
+    loss = np.zeros(1, np.float32)
+    assert h.odl_hostcpu_softmax_ce(a, np.zeros(2, np.int32), 0, 2, 3, loss, None) == -2
+    assert (c == 0).all()
