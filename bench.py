@@ -131,6 +131,32 @@ def extras(torch, capi, steps, warmup):
     return out
 
 
+def train_steps(steps, warmup, with_cpu):
+    """Configs 1 and 4 as whole training steps through the C++ host layer (Tensor/Operator/nn/optim over the C ABI):
+    forward, softmax-CE loss (read back each step, as the reference's loop does), backward, optimizer step, on
+    tensors resident in HBM. The same driver source compiled against the reference gives the CPU time beside it."""
+    import numpy as np
+    import oraclelib as ol
+    out = {}
+    if not os.path.exists(ol.HOST_DRIVER_SO):
+        return {"error": "host layer not built"}
+    h = ol.host_driver()
+    ms, loss = np.zeros(1, np.float32), np.zeros(1, np.float32)
+    rc = h.odl_host_mlp_bench(512, 784, 1000, 10, steps, warmup, ms, loss)
+    out["mlp_512x784x1000x10_adam"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss": float(loss[0]),
+                                       "gemm_flop_per_step": 6.0 * 512 * (784 * 1000 + 1000 * 10)}
+    rc = h.odl_host_cnn_bench(256, steps, warmup, ms, loss)
+    out["cnn_b256_sgd"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss": float(loss[0])}
+    if with_cpu and ol.have_ref():
+        r = ol.ref()
+        rc = r.odl_ref_mlp_bench(512, 784, 1000, 10, 1, 0, ms, loss)
+        out["mlp_512x784x1000x10_adam"]["cpu_reference_ms_per_step"] = float(ms[0])
+        out["mlp_512x784x1000x10_adam"]["cpu_reference_loss"] = float(loss[0])
+        rc = r.odl_ref_cnn_bench(4, 1, 0, ms, loss)
+        out["cnn_b256_sgd"]["cpu_reference_ms_per_step_extrapolated_from_batch_4"] = float(ms[0]) * 64.0
+    return out
+
+
 def pmc_probe(torch, capi, gemm_step):
     """A short, fixed launch sequence for counter runs (`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`):
     first a plain elementwise copy-like kernel of known traffic (negate of 64 Mi floats: 256 MiB read, 256 MiB
@@ -166,6 +192,8 @@ def main():
     ap.add_argument("--size", type=int, default=4096)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--train-probe", action="store_true",
+                    help="only the MLP/CNN training steps through the C++ host layer (for rocprofv3 --kernel-trace)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="few launches of each hot kernel plus a plain copy of known size, for rocprofv3 --pmc runs")
     args = ap.parse_args()
@@ -173,6 +201,10 @@ def main():
         print("bench.py: this build runs on ONE GPU; nothing here uses a second one (no collectives, no sharding). "
               "Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+
+    if args.train_probe:
+        print(json.dumps(train_steps(args.steps, args.warmup, False)))
+        return
 
     import torch
     from origindl_amd import capi  # raises if libodl_hip.so is missing: there is no fallback
@@ -189,12 +221,13 @@ def main():
     import ctypes
     lib = capi.lib()
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    ws_bytes = lib.query("odl_hip_matmul_backward_workspace_bytes", S, S, S)
+    ws_bytes = max(lib.query("odl_hip_matmul_backward_workspace_bytes", S, S, S),
+                   lib.query("odl_hip_matmul_workspace_bytes", 1, S, S, S, 0))
     ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.int32, device="cuda")
     p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
 
     def step():
-        lib.call("odl_hip_matmul", p(a), p(b), p(c), 1, S, S, S, 0, st)
+        lib.call("odl_hip_matmul", p(a), p(b), p(c), 1, S, S, S, 0, p(ws), ws_bytes, st)
         lib.call("odl_hip_matmul_backward", p(a), p(b), p(dc), p(da), p(db), S, S, S, p(ws), ws_bytes, st)
 
     if args.pmc_probe:
@@ -233,6 +266,7 @@ def main():
     }
     if not args.no_extras:
         line["extras"] = extras(torch, capi, max(3, args.steps // 2), max(2, args.warmup // 2))
+        line["extras"]["train_steps"] = train_steps(max(5, args.steps // 2), 3, not args.no_cpu)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_gemm(S)
     print(json.dumps(line))

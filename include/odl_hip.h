@@ -68,9 +68,11 @@ int odl_hip_sgemm(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, con
 size_t odl_hip_sgemm_workspace_bytes(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, int split_k);
 
 /* Mat::matmul — 2-D x 2-D (batch = 1), 3-D x 2-D (b_is_batched = 0), 3-D x 3-D (b_is_batched = 1);
- * src/mat/origin/cpu/math/matmul.cpp:113-218. */
+ * src/mat/origin/cpu/math/matmul.cpp:113-218. The workspace (may be NULL) lets small products be split along K
+ * so that they still fill the chip. */
 int odl_hip_matmul(const float *a, const float *b, float *c, int64_t batch, int64_t M, int64_t N, int64_t K,
-                   int b_is_batched, void *stream);
+                   int b_is_batched, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_matmul_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int b_is_batched);
 /* MatMul::backward (src/operators/math/mat_mul.cpp:123-182): gx[M,K] = gy[M,N] . w[K,N]^T and
  * gw[K,N] = x[M,K]^T . gy[M,N], as NT and TN GEMMs with no transpose copy. Either output may be NULL. */
 int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M,

@@ -127,7 +127,8 @@ def mat_mul(a, b):
                                  % (tuple(a.shape), tuple(b.shape)))
     N = b.shape[-1]
     c = _empty(oshape)
-    lib().call("odl_hip_matmul", _p(a), _p(b), _p(c), batch, M, N, K, bb, _stream())
+    ws, nb = _ws(lib().query("odl_hip_matmul_workspace_bytes", batch, M, N, K, bb))
+    lib().call("odl_hip_matmul", _p(a), _p(b), _p(c), batch, M, N, K, bb, _p(ws), nb, _stream())
     return c
 
 

@@ -523,22 +523,38 @@ int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g, int splits, hipSt
     return ODL_ERR_RUNTIME;
 }
 
-constexpr int kBM = 128, kBN = 128, kBK = 16;
+constexpr int kBK = 16;
 
+// Tile edge for a problem: 128x128 tiles when they can fill the chip (256 CUs), 64x64 tiles for smaller outputs so
+// that more workgroups exist.
+int pick_tile(int64_t M, int64_t N)
+{
+    return (odl::ceil_div(M, 128) * odl::ceil_div(N, 128) >= 256) ? 128 : 64;
+}
+
+// K slices for problems whose tiles alone cannot fill the chip: aim at ~512 workgroups, at least 4 K slabs each.
 int pick_splits(int64_t M, int64_t N, int64_t K, int requested)
 {
     if (requested >= 1)
         return requested;
-    const int64_t tiles = odl::ceil_div(M, kBM) * odl::ceil_div(N, kBN);
+    const int tile      = pick_tile(M, N);
+    const int64_t tiles = odl::ceil_div(M, tile) * odl::ceil_div(N, tile);
     const int64_t kt    = odl::ceil_div(K, kBK);
-    if (tiles >= 128 || kt < 64)
+    if (tiles >= 256 || kt < 8)
         return 1;
     int64_t s = odl::ceil_div(512, tiles);
-    if (s > kt / 16)
-        s = kt / 16;
+    if (s > kt / 4)
+        s = kt / 4;
     if (s > 128)
         s = 128;
     return s < 1 ? 1 : (int)s;
+}
+
+template <int EPI>
+int launch_any_tile(int tile, bool ta, bool tb, bool vec, const GemmArgs &g, int splits, hipStream_t st)
+{
+    return tile == 128 ? launch_tile<128, 128, kBK, EPI>(ta, tb, vec, g, splits, st)
+                       : launch_tile<64, 64, kBK, EPI>(ta, tb, vec, g, splits, st);
 }
 }  // namespace
 
@@ -560,7 +576,8 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
     GemmArgs g;
     g.A = A, g.B = B, g.C = C, g.bias = bias;
     g.M = M, g.N = N, g.K = K, g.lda = lda, g.ldb = ldb, g.ldc = ldc, g.P = P;
-    g.tiles_m = (int)ceil_div(M, kBM), g.tiles_n = (int)ceil_div(N, kBN);
+    const int tile = pick_tile(M, N);
+    g.tiles_m = (int)ceil_div(M, tile), g.tiles_n = (int)ceil_div(N, tile);
     ODL_REQUIRE((int64_t)g.tiles_m * g.tiles_n < (1ll << 31), "sgemm: too many tiles");
 
     // 16-byte loads need 16-byte aligned rows: base pointers, leading dimensions and the contiguous extents
@@ -589,7 +606,7 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
     {
         GemmArgs p = g;
         p.C = static_cast<float *>(workspace), p.ldc = N, p.bias = nullptr, p.c_split_stride = M * N;
-        rc = launch_tile<kBM, kBN, kBK, EPI_PLAIN>(trans_a, trans_b, vec, p, splits, st);
+        rc = launch_any_tile<EPI_PLAIN>(tile, trans_a, trans_b, vec, p, splits, st);
         if (rc != ODL_OK)
             return fail(rc, "sgemm: no kernel variant");
         ODL_LAUNCH_CHECK();
@@ -601,11 +618,11 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
         return ODL_OK;
     }
     if (epi == EPI_NCHW_ROWB)
-        rc = launch_tile<kBM, kBN, kBK, EPI_NCHW_ROWB>(trans_a, trans_b, vec, g, 1, st);
+        rc = launch_any_tile<EPI_NCHW_ROWB>(tile, trans_a, trans_b, vec, g, 1, st);
     else if (epi == EPI_BIAS_COL && bias)
-        rc = launch_tile<kBM, kBN, kBK, EPI_BIAS_COL>(trans_a, trans_b, vec, g, 1, st);
+        rc = launch_any_tile<EPI_BIAS_COL>(tile, trans_a, trans_b, vec, g, 1, st);
     else
-        rc = launch_tile<kBM, kBN, kBK, EPI_PLAIN>(trans_a, trans_b, vec, g, 1, st);
+        rc = launch_any_tile<EPI_PLAIN>(tile, trans_a, trans_b, vec, g, 1, st);
     if (rc != ODL_OK)
         return fail(rc, "sgemm: no kernel variant");
     ODL_LAUNCH_CHECK();
@@ -620,7 +637,7 @@ template <int SB, bool TA, int EPI>
 int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, hipStream_t st)
 {
     const int ck = (cv.KH == 3 && cv.KW == 3) ? 3 : ((cv.KH == 1 && cv.KW == 1) ? 1 : 0);
-    const bool bm64 = g.M <= 64;
+    const bool bm64 = g.M <= 64 || odl::ceil_div(g.M, 128) * odl::ceil_div(g.N, 128) * splits < 256;
     g.tiles_m = (int)odl::ceil_div(g.M, bm64 ? 64 : 128);
     g.tiles_n = (int)odl::ceil_div(g.N, 128);
     const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits), block(kThreads);
@@ -812,18 +829,23 @@ size_t odl_hip_sgemm_workspace_bytes(int, int, int64_t M, int64_t N, int64_t K, 
     return odl::sgemm_workspace(M, N, K, split_k);
 }
 
+size_t odl_hip_matmul_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int b_is_batched)
+{
+    return b_is_batched ? odl::sgemm_workspace(M, N, K, 0) : odl::sgemm_workspace(batch * M, N, K, 0);
+}
+
 int odl_hip_matmul(const float *a, const float *b, float *c, int64_t batch, int64_t M, int64_t N, int64_t K,
-                   int b_is_batched, void *stream)
+                   int b_is_batched, void *workspace, size_t workspace_bytes, void *stream)
 {
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(batch >= 1, "matmul: batch must be >= 1");
     if (!b_is_batched)  // [batch*M, K] x [K, N]: one GEMM, the batch folds into the rows
-        return odl::sgemm_launch(0, 0, batch * M, N, K, a, K, b, N, c, N, nullptr, EPI_PLAIN, 0, 1, nullptr, 0,
-                                 odl::as_stream(stream));
+        return odl::sgemm_launch(0, 0, batch * M, N, K, a, K, b, N, c, N, nullptr, EPI_PLAIN, 0, 0, workspace,
+                                 workspace_bytes, odl::as_stream(stream));
     for (int64_t i = 0; i < batch; ++i)
     {
         int rc = odl::sgemm_launch(0, 0, M, N, K, a + i * M * K, K, b + i * K * N, N, c + i * M * N, N, nullptr,
-                                   EPI_PLAIN, 0, 1, nullptr, 0, odl::as_stream(stream));
+                                   EPI_PLAIN, 0, 0, workspace, workspace_bytes, odl::as_stream(stream));
         if (rc != ODL_OK)
             return rc;
     }

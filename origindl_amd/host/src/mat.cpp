@@ -527,7 +527,8 @@ std::unique_ptr<Mat> OriginMat::matmul(const Mat &other) const
         THROW_INVALID_ARG("Matrix dimensions must be compatible for multiplication. A shape: {}, B shape: {}",
                           as.to_string(), bs.to_string());
     auto c = new_like(a, rs);
-    check(odl_hip_matmul(fp(a), fp(b), c->data_ptr<float>(), batch, M, N, K, b_batched, nullptr));
+    Workspace ws(odl_hip_matmul_workspace_bytes(batch, M, N, K, b_batched), device().index());
+    check(odl_hip_matmul(fp(a), fp(b), c->data_ptr<float>(), batch, M, N, K, b_batched, ws.ptr(), ws.bytes, nullptr));
     return c;
 }
 

@@ -9,8 +9,11 @@
 //     Mat interfaces" means; tests compare its results with the fixtures and the oracle.
 // Every entry point returns 0, or -1 for std::invalid_argument, -2 for any other std::exception.
 #include <cstdint>
+#include <chrono>
+#include <cmath>
 #include <cstring>
 #include <memory>
+#include <random>
 #include <stdexcept>
 #include <vector>
 
@@ -480,6 +483,127 @@ int DRV(cnn_train)(const float *x, const void *t, int is64, int64_t N, int64_t S
         out(*l1.bias(), bl1);
         out(*l2.weight(), Wl2);
         out(*l2.bias(), bl2);
+    });
+}
+
+}  // extern "C"
+
+// ---- whole training steps timed on resident tensors (benchmark configs 1 and 4): `warmup` untimed steps, then
+// `steps` timed ones; every step ends with the loss read back to the host (as the reference's loop does), which
+// also drains the device queue, so wall-clock time around the loop is the step time.
+namespace
+{
+std::vector<float> uniform_vec(std::mt19937 &gen, size_t n, float lo, float hi)
+{
+    std::uniform_real_distribution<float> d(lo, hi);
+    std::vector<float> v(n);
+    for (auto &e : v)
+        e = d(gen);
+    return v;
+}
+
+Parameter kaiming_uniform(std::mt19937 &gen, const Shape &s, size_t fan_in)
+{
+    const float bound = std::sqrt(6.0f / (float)fan_in);
+    return Parameter(Tensor(uniform_vec(gen, s.elements(), -bound, bound), s,
+                            dtype(DataType::kFloat32).requires_grad(true).device(kDev)));
+}
+
+Parameter zeros_param(const Shape &s)
+{
+    return Parameter(Tensor(std::vector<float>(s.elements(), 0.0f), s,
+                            dtype(DataType::kFloat32).requires_grad(true).device(kDev)));
+}
+
+template <typename Model, typename Opt>
+void timed_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T, int steps, int warmup, float *ms, float *loss)
+{
+    model.train();
+    auto one = [&] {
+        opt.zero_grad();
+        auto y = model(X);
+        auto L = F::softmax_cross_entropy(y, T);
+        L.backward();
+        opt.step();
+        return L.template item<float>();
+    };
+    for (int i = 0; i < warmup; ++i)
+        *loss = one();
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; ++i)
+        *loss = one();
+    // the parameters of the last step are still in flight: reading one back drains the queue
+    float sink = model.parameters()[0]->template to_vector<float>()[0];
+    (void)sink;
+    const auto t1 = std::chrono::steady_clock::now();
+    *ms = std::chrono::duration<float, std::milli>(t1 - t0).count() / (float)(steps > 0 ? steps : 1);
+}
+}  // namespace
+
+extern "C" {
+
+int DRV(mlp_bench)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, float *ms_per_step, float *loss)
+{
+    return guarded([&] {
+        std::mt19937 gen(1234);
+        Sequential model;
+        model.add(std::make_unique<nn::Linear>((int)D, (int)Hd, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::Linear>((int)Hd, (int)C, true));
+        auto &l1 = dynamic_cast<nn::Linear &>(model[0]);
+        auto &l2 = dynamic_cast<nn::Linear &>(model[2]);
+        Adam opt(model, 1e-3f, 0.9f, 0.999f, 1e-8f);
+        opt.register_hook(WeightDecay(1e-4f).hook());
+        *l1.weight() = kaiming_uniform(gen, Shape{(size_t)D, (size_t)Hd}, (size_t)D);
+        *l1.bias()   = zeros_param(Shape{1, (size_t)Hd});
+        *l2.weight() = kaiming_uniform(gen, Shape{(size_t)Hd, (size_t)C}, (size_t)Hd);
+        *l2.bias()   = zeros_param(Shape{1, (size_t)C});
+        auto X = Tensor(uniform_vec(gen, (size_t)(N * D), 0.0f, 1.0f), Shape{(size_t)N, (size_t)D},
+                        dtype(DataType::kFloat32).device(kDev));
+        std::vector<int64_t> tv((size_t)N);
+        for (auto &e : tv)
+            e = (int64_t)(gen() % (uint32_t)C);
+        auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt64).device(kDev));
+        timed_steps(model, opt, X, T, steps, warmup, ms_per_step, loss);
+    });
+}
+
+int DRV(cnn_bench)(int64_t N, int steps, int warmup, float *ms_per_step, float *loss)
+{
+    return guarded([&] {
+        std::mt19937 gen(4321);
+        const int64_t S = 28, C1 = 32, C2 = 64, Hd = 128, Cc = 10, Fdim = C2 * 7 * 7;
+        Sequential model;
+        model.add(std::make_unique<nn::Conv2d>(1, (int)C1, 3, 1, 1, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::MaxPool2d>(2, 2, 0));
+        model.add(std::make_unique<nn::Conv2d>((int)C1, (int)C2, 3, 1, 1, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::MaxPool2d>(2, 2, 0));
+        model.add(std::make_unique<nn::Flatten>());
+        model.add(std::make_unique<nn::Linear>((int)Fdim, (int)Hd, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::Linear>((int)Hd, (int)Cc, true));
+        auto &c1 = dynamic_cast<nn::Conv2d &>(model[0]);
+        auto &c2 = dynamic_cast<nn::Conv2d &>(model[3]);
+        auto &l1 = dynamic_cast<nn::Linear &>(model[7]);
+        auto &l2 = dynamic_cast<nn::Linear &>(model[9]);
+        SGD opt(model, 0.01f);
+        *c1.weight() = kaiming_uniform(gen, Shape{(size_t)C1, 1, 3, 3}, 9);
+        *c1.bias()   = zeros_param(Shape{(size_t)C1});
+        *c2.weight() = kaiming_uniform(gen, Shape{(size_t)C2, (size_t)C1, 3, 3}, (size_t)(9 * C1));
+        *c2.bias()   = zeros_param(Shape{(size_t)C2});
+        *l1.weight() = kaiming_uniform(gen, Shape{(size_t)Fdim, (size_t)Hd}, (size_t)Fdim);
+        *l1.bias()   = zeros_param(Shape{1, (size_t)Hd});
+        *l2.weight() = kaiming_uniform(gen, Shape{(size_t)Hd, (size_t)Cc}, (size_t)Hd);
+        *l2.bias()   = zeros_param(Shape{1, (size_t)Cc});
+        auto X = Tensor(uniform_vec(gen, (size_t)(N * S * S), 0.0f, 1.0f), Shape{(size_t)N, 1, (size_t)S, (size_t)S},
+                        dtype(DataType::kFloat32).device(kDev));
+        std::vector<int64_t> tv((size_t)N);
+        for (auto &e : tv)
+            e = (int64_t)(gen() % (uint32_t)Cc);
+        auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt64).device(kDev));
+        timed_steps(model, opt, X, T, steps, warmup, ms_per_step, loss);
     });
 }
 

@@ -75,6 +75,8 @@ _REF_SIGS = {
     "odl_ref_pow_scalar": "plfp>i",
     "odl_ref_mlp_train": "ppillll" + "pppp" + "ifffff" + "pppppp>i",
     "odl_ref_cnn_train": "ppillllll" + "p" * 8 + "f" + "p" + "p" * 8 + "p>i",
+    "odl_ref_mlp_bench": "lllliipp>i",
+    "odl_ref_cnn_bench": "liipp>i",
 }
 
 
