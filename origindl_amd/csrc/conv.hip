@@ -77,8 +77,10 @@ constexpr int kImCk  = 144;  // col columns per tile at most
 // Read phase: for one ck at a time the 64 lanes of a wave read 64 consecutive pixels — contiguous image addresses
 // (stride SW) — into an LDS tile; write phase: the tile leaves row by row with 16-byte stores. The image is read
 // through coalesced loads and the 9x larger col matrix is written through full-width stores.
-__global__ __launch_bounds__(256) void im2col_matrix_kernel(const float *__restrict__ img, float *__restrict__ col,
-                                                             ConvGeom g, int tk, int ktiles, int64_t mtiles)
+constexpr int kImThreads = 512;
+__global__ __launch_bounds__(kImThreads) void im2col_matrix_kernel(const float *__restrict__ img,
+                                                                    float *__restrict__ col, ConvGeom g, int tk,
+                                                                    int ktiles, int64_t mtiles)
 {
     __shared__ float sh[kImPix][kImCk + 1];
     const int64_t vb = xcd_contiguous_block(blockIdx.x, mtiles * ktiles);
@@ -98,32 +100,33 @@ __global__ __launch_bounds__(256) void im2col_matrix_kernel(const float *__restr
     const int ck0 = kt * tk;
     const int ckn = (K - ck0 < tk) ? K - ck0 : tk;
     const int H = (int)g.H, W = (int)g.W;
-    constexpr int U = 6;  // independent loads in flight per lane
-    for (int j = wave; j < ckn; j += 4 * U)
+    constexpr int U = 9;  // independent loads in flight per lane
+    constexpr int NW = kImThreads / 64;
+    for (int j = wave; j < ckn; j += NW * U)
     {
         float v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
         {
-            const int ck = ck0 + j + 4 * u;  // wave-uniform
+            const int ck = ck0 + j + NW * u;  // wave-uniform
             const int kw = ck % g.KW, t2 = ck / g.KW;
             const int kh = t2 % g.KH, c = t2 / g.KH;
             const int h = h0 + kh, w = w0 + kw;
             v[u] = 0.f;
-            if (j + 4 * u < ckn && live && h >= 0 && h < H && w >= 0 && w < W)
+            if (j + NW * u < ckn && live && h >= 0 && h < H && w >= 0 && w < W)
                 v[u] = base[((int64_t)c * H + h) * W + w];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            if (j + 4 * u < ckn)
-                sh[lane][j + 4 * u] = v[u];
+            if (j + NW * u < ckn)
+                sh[lane][j + NW * u] = v[u];
     }
     __syncthreads();
     const int64_t row0 = mt * kImPix;
     if ((ckn & 3) == 0 && (K & 3) == 0 && (ck0 & 3) == 0 && (reinterpret_cast<uintptr_t>(col) & 15) == 0)
     {
         const int q4 = ckn >> 2;
-        for (int e = threadIdx.x; e < kImPix * q4; e += 256)
+        for (int e = threadIdx.x; e < kImPix * q4; e += kImThreads)
         {
             const int row = e / q4, q = e % q4;
             if (row0 + row < M)
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(256) void im2col_matrix_kernel(const float *__restr
     }
     else
     {
-        for (int e = threadIdx.x; e < kImPix * ckn; e += 256)
+        for (int e = threadIdx.x; e < kImPix * ckn; e += kImThreads)
         {
             const int row = e / ckn, j = e % ckn;
             if (row0 + row < M)
@@ -325,8 +328,8 @@ int im2col_launch(const float *img, float *col, const ConvGeom &g, int to_matrix
         const int ktiles = (int)odl::ceil_div(K, tk);
         const int64_t mtiles = odl::ceil_div(g.N * g.OH * g.OW, kImPix);
         ODL_REQUIRE(mtiles * ktiles < (1ll << 31) && K < (1ll << 31), "im2col: too many tiles");
-        hipLaunchKernelGGL(im2col_matrix_kernel, dim3((unsigned)(mtiles * ktiles)), dim3(256), 0, st, img, col, g, tk,
-                           ktiles, mtiles);
+        hipLaunchKernelGGL(im2col_matrix_kernel, dim3((unsigned)(mtiles * ktiles)), dim3(kImThreads), 0, st, img, col, g,
+                           tk, ktiles, mtiles);
     }
     else
     {

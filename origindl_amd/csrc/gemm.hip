@@ -64,6 +64,7 @@ struct GemmArgs
     int64_t c_split_stride;  // elements between the partial outputs of consecutive slices (0 = none)
     int64_t P;               // EPI_NCHW_ROWB: OH*OW
     int tiles_m, tiles_n;
+    int splits;              // K slices (grid = tiles_m * tiles_n * splits workgroups)
 };
 
 template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI, int SB = SB_PLAIN, int CK = 0>
@@ -95,14 +96,20 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
     const int l32 = lane & 31, lh = lane >> 5;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
-    // ---- workgroup -> tile: contiguous band per XCD, then groups of kGroupM tile-rows
-    int tm, tn;
+    // ---- workgroup -> (K slice, tile). The grid is one-dimensional (tiles x slices). Workgroups are dealt
+    // round-robin over the 8 XCDs, so the id is first unfolded into a contiguous band per XCD; inside a band the
+    // tiles of one K slice are adjacent (they read the same K range of A and B, which then sits in that XCD's L2),
+    // and tiles are walked in groups of kGroupM tile-rows.
+    int tm, tn, kz;
     {
         const int nt = g.tiles_m * g.tiles_n;
-        const int bid = blockIdx.x;
-        const int xcd = bid % kXcds, loc = bid / kXcds;
-        const int full = nt / kXcds, rem = nt % kXcds;
-        const int t = xcd * full + (xcd < rem ? xcd : rem) + loc;
+        const int64_t total = (int64_t)nt * g.splits;
+        const int64_t bid = blockIdx.x;
+        const int64_t xcd = bid % kXcds, loc = bid / kXcds;
+        const int64_t full = total / kXcds, rem = total % kXcds;
+        const int64_t v = xcd * full + (xcd < rem ? xcd : rem) + loc;
+        kz = (int)(v / nt);
+        const int t = (int)(v % nt);
         const int gsz = kGroupM * g.tiles_n;
         const int grp = t / gsz, in_g = t % gsz;
         const int first_m = grp * kGroupM;
@@ -111,7 +118,7 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
         tn = in_g / gm;
     }
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-    const int64_t kbeg = (int64_t)blockIdx.y * g.k_per_split;
+    const int64_t kbeg = (int64_t)kz * g.k_per_split;
     const int64_t kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
     const int nkt = (int)((kend - kbeg + BK - 1) / BK);
 
@@ -280,9 +287,12 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
         }
         else
         {
-            // float4 u: row = tid/4 + 64u (its pixel), k = k0 + 4*(tid%4) .. +3 = four consecutive oc of one tap
-            const int tap = (int)(k0 / cv.OC);  // block-uniform: OC is a multiple of BK, a slab never straddles taps
-            const int oc0 = (int)(k0 - (int64_t)tap * cv.OC) + 4 * (tid & 3);
+            // float4 u: row = tid/4 + 64u (its pixel), k = k0 + 4*(tid%4) .. +3 = four consecutive oc of one tap.
+            // K runs as (oc slab of 16, tap, oc within the slab): the KH*KW taps of one 64-byte slab follow each
+            // other, and neighbouring pixels' taps re-read the same gy rows, so those reads hit in cache.
+            const int slab = (int)(k0 / BK);  // block-uniform
+            const int ocs = slab / KHW, tap = slab - ocs * KHW;
+            const int oc0 = ocs * BK + 4 * (tid & 3);
             const int kh = tap / KW, kw = tap - kh * KW;
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -408,7 +418,7 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
     }
 
     // ---- epilogue: accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
-    float *Cout = g.C + (int64_t)blockIdx.y * g.c_split_stride;
+    float *Cout = g.C + (int64_t)kz * g.c_split_stride;
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
@@ -500,9 +510,11 @@ __global__ void transpose_kernel(const float *__restrict__ src, float *__restric
 }
 
 template <int BM, int BN, int BK, int EPI>
-int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g, int splits, hipStream_t st)
+int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g_in, int splits, hipStream_t st)
 {
-    dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits);
+    GemmArgs g = g_in;
+    g.splits = splits;
+    dim3 grid((unsigned)((int64_t)g.tiles_m * g.tiles_n * splits));
     dim3 block(kThreads);
 #define ODL_GEMM_CASE(TA, TB, V)                                                                      \
     if (ta == TA && tb == TB && vec == V)                                                             \
@@ -640,7 +652,8 @@ int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, hipStream_t st)
     const bool bm64 = g.M <= 64 || odl::ceil_div(g.M, 128) * odl::ceil_div(g.N, 128) * splits < 256;
     g.tiles_m = (int)odl::ceil_div(g.M, bm64 ? 64 : 128);
     g.tiles_n = (int)odl::ceil_div(g.N, 128);
-    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)splits), block(kThreads);
+    g.splits = splits;
+    const dim3 grid((unsigned)((int64_t)g.tiles_m * g.tiles_n * splits)), block(kThreads);
 #define ODL_CONV_CASE(BMV, CKV)                                                                                  \
     if (bm64 == (BMV == 64) && ck == CKV)                                                                        \
     {                                                                                                            \
@@ -658,15 +671,16 @@ int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, hipStream_t st)
     return ODL_ERR_RUNTIME;
 }
 
-// wp[c][(kh*KW + kw)*OC + oc] = w[oc][c][kh][kw]
+// wp[c][((oc/16)*KHW + tap)*16 + oc%16] = w[oc][c][tap]: the K order of the input-grad GEMM (OC % 16 == 0)
 __global__ void permute_weight_kernel(const float *__restrict__ w, float *__restrict__ wp, int OC, int C, int KHW)
 {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (int64_t)OC * C * KHW)
         return;
-    const int oc = (int)(t % OC);
-    const int tap = (int)((t / OC) % KHW);
+    const int k = (int)(t % ((int64_t)OC * KHW));
     const int c = (int)(t / ((int64_t)OC * KHW));
+    const int lo = k % 16, tap = (k / 16) % KHW, ocs = k / (16 * KHW);
+    const int oc = ocs * 16 + lo;
     wp[t] = w[((int64_t)oc * C + c) * KHW + tap];
 }
 

@@ -8,6 +8,8 @@
 
 #include "odl_common.h"
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 namespace
 {
 constexpr int kBlock = 256;
@@ -202,6 +204,63 @@ __global__ __launch_bounds__(kBlock) void ce_grad_kernel(const float *__restrict
     }
 }
 
+// Same, for rows whose length is a multiple of 4 and whose base is 16-byte aligned: every lane moves 16 bytes
+// per access (QUADS float4 per lane, rows of up to 256*QUADS classes).
+template <int QUADS>
+__global__ __launch_bounds__(kBlock) void ce_grad_vec_kernel(const float *__restrict__ x, const void *t, int is64,
+                                                              int64_t N, int64_t C, float scale, float *__restrict__ gx)
+{
+    const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (row >= N)
+        return;
+    const int lane = threadIdx.x & 63;
+    const f32x4 *xr = reinterpret_cast<const f32x4 *>(x + row * C);
+    f32x4 *gr = reinterpret_cast<f32x4 *>(gx + row * C);
+    const int64_t lab = label_at(t, is64, row);
+    const int64_t cq = C / 4;
+    f32x4 v[QUADS];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u)
+    {
+        const int64_t q = lane + 64 * u;
+        if (q < cq)
+            v[u] = xr[q];
+        else
+            v[u] = f32x4{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            m = (m < v[u][e]) ? v[u][e] : m;
+    }
+    m = wave_max(m);
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u)
+    {
+        const bool in = lane + 64 * u < cq;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            v[u][e] = in ? expf(v[u][e] - m) : 0.f;
+            s += v[u][e];
+        }
+    }
+    s = wave_sum(s);
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u)
+    {
+        const int64_t q = lane + 64 * u;
+        if (q < cq)
+        {
+            f32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                o[e] = (v[u][e] / s - ((4 * q + e == lab) ? 1.f : 0.f)) * scale;
+            gr[q] = o;
+        }
+    }
+}
+
 // first maximum of each row (strict >), sequential like src/utils/metrics.cpp:42-53
 __global__ void argmax_rows_kernel(const float *__restrict__ y, int64_t N, int64_t C, int64_t *__restrict__ out)
 {
@@ -355,7 +414,17 @@ int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64
     const float scale = gy / (float)N;  // softmax_cross_entropy.cpp:105-106
     const dim3 grid((unsigned)odl::ceil_div(N, kWaves));
     hipStream_t st = odl::as_stream(stream);
-    if (C <= 64)
+    const bool vec = C % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gx)) & 15) == 0;
+    if (vec && C > 64 && C <= 1024)
+    {
+        if (C <= 256)
+            hipLaunchKernelGGL(ce_grad_vec_kernel<1>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+        else if (C <= 512)
+            hipLaunchKernelGGL(ce_grad_vec_kernel<2>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+        else
+            hipLaunchKernelGGL(ce_grad_vec_kernel<4>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+    }
+    else if (C <= 64)
         hipLaunchKernelGGL(ce_grad_kernel<1>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
     else if (C <= 256)
         hipLaunchKernelGGL(ce_grad_kernel<4>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);

@@ -430,7 +430,8 @@ def test_broadcast_fixtures(api):
 # ------------------------------------------------------------------------------------ softmax / CE
 def test_softmax_and_ce_vs_oracle(api, o):
     rng = np.random.default_rng(14)
-    for N, C, is64 in ((512, 10, 1), (256, 10, 0), (7, 1000, 1), (1, 3, 0), (300, 65, 1)):
+    for N, C, is64 in ((512, 10, 1), (256, 10, 0), (7, 1000, 1), (1, 3, 0), (300, 65, 1), (33, 128, 0), (9, 400, 1),
+                       (5, 2000, 0)):
         x = (rng.standard_normal((N, C), dtype=f32) * 3).astype(f32)
         t = rng.integers(0, C, size=N).astype(np.int64 if is64 else np.int32)
         p, gx, loss = np.empty_like(x), np.empty_like(x), np.zeros(1, f32)
