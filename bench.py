@@ -157,6 +157,11 @@ def train_steps(steps, warmup, with_cpu):
     return out
 
 
+# HBM-side bytes of one 4096^3 sgemm_mfma_kernel launch: FETCH_SIZE (scaled 2.000x by the calibration copy) 720.2 MiB
+# + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc` runs of `--pmc-probe` summarised under profiles/.
+GEMM_4096_TRAFFIC_BYTES = int((720.2 + 64.0) * 1024 * 1024)
+
+
 def pmc_probe(torch, capi, gemm_step):
     """A short, fixed launch sequence for counter runs (`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`):
     first a plain elementwise copy-like kernel of known traffic (negate of 64 Mi floats: 256 MiB read, 256 MiB
@@ -260,7 +265,8 @@ def main():
         "data": "synthetic N(0,1) operands, seeded, resident in HBM",
         "config": {"workload": "matmul fwd+bwd: C=A.B, dA=dC.B^T, dB=A^T.dC, M=N=K=%d" % S, "flop_per_step": flop_step},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+                     "traffic": GEMM_4096_TRAFFIC_BYTES if S == 4096 else None,
                      "kernel": "sgemm_mfma_kernel<128,128,16> (NN, NT, TN)", "launch_ms": launch_ms},
         "device": capi.device_info(0),
     }
