@@ -68,7 +68,7 @@ struct GemmArgs
 };
 
 template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI, int SB = SB_PLAIN, int CK = 0>
-__global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSrc cv)
+__global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_CONV_WGRAD ? 4 : 1)) void sgemm_mfma_kernel(GemmArgs g, ConvSrc cv)
 {
     // A tile: !TA -> memory is [M][K] (K-contiguous) -> LDS K-major; TA -> memory [K][M] -> LDS row-major.
     // B tile: !TB -> memory is [K][N] (row-contiguous) -> LDS row-major; TB -> memory [N][K] -> LDS K-major.
@@ -205,7 +205,10 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
     [[maybe_unused]] const float *fw_base = nullptr;  // forward: &x[n, 0, oh*SH-PH, ow*SW-PW] of this thread's pixel
     [[maybe_unused]] int fw_hb = 0, fw_wb = 0;
     [[maybe_unused]] bool fw_live = false;
-    [[maybe_unused]] int wg_off[B_PER_T], wg_kh[B_PER_T], wg_kw[B_PER_T];  // weight grad: this thread's 8 (c,kh,kw)
+    [[maybe_unused]] unsigned fw_mask = 0;
+    [[maybe_unused]] int wg_off[B_PER_T];  // weight grad: this thread's 8 (c,kh,kw) as offsets into an image ...
+    [[maybe_unused]] int wg_kh[CK > 0 ? 1 : B_PER_T], wg_kw[CK > 0 ? 1 : B_PER_T];  // ... and as taps (any kernel size)
+    [[maybe_unused]] unsigned wg_taps = 0;  // ... or as eight 4-bit tap numbers kh*KW+kw (3x3, 1x1; 15 = no such row)
     [[maybe_unused]] int dg_n[2], dg_h[2], dg_w[2];                        // input grad: this thread's 2 pixels
     [[maybe_unused]] bool dg_live[2];
     if constexpr (SB == SB_CONV_FWD)
@@ -217,6 +220,14 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
         const int64_t n = mm / ((int64_t)cv.OW * cv.OH);
         fw_hb = oh * cv.SH - cv.PH, fw_wb = ow * cv.SW - cv.PW;
         fw_base = g.B + n * cv.C * cv.H * cv.W + (int64_t)fw_hb * cv.W + fw_wb;  // dereferenced only when in bounds
+        if constexpr (CK > 0)
+        {
+            // bit kh*KW+kw: that tap of this thread's pixel lies inside the image
+            for (int kh = 0; kh < CK; ++kh)
+                for (int kw = 0; kw < CK; ++kw)
+                    if (fw_live && (unsigned)(fw_hb + kh) < (unsigned)cv.H && (unsigned)(fw_wb + kw) < (unsigned)cv.W)
+                        fw_mask |= 1u << (kh * CK + kw);
+        }
     }
     if constexpr (SB == SB_CONV_WGRAD)
     {
@@ -229,8 +240,13 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
             const int c = cki / KHW, r = cki - c * KHW;
             const int kh = r / KW, kw = r - kh * KW;
             wg_off[u] = (c * cv.H + kh) * cv.W + kw;
-            wg_kh[u] = ok ? kh : (1 << 20);  // an out-of-range row fails every bounds check
-            wg_kw[u] = kw;
+            if constexpr (CK > 0)
+                wg_taps |= (ok ? (unsigned)r : 15u) << (4 * u);
+            else
+            {
+                wg_kh[u] = ok ? kh : (1 << 20);  // an out-of-range row fails every bounds check
+                wg_kw[u] = kw;
+            }
         }
     }
     if constexpr (SB == SB_CONV_DGRAD)
@@ -262,8 +278,14 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
                 const int k = (int)k0 + ksub + 2 * u;
                 const int c = k / KHW, r = k - c * KHW;
                 const int kh = r / KW, kw = r - kh * KW;
-                const int h = fw_hb + kh, w = fw_wb + kw;
-                const bool ok = fw_live && k < kend && (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
+                bool ok;
+                if constexpr (CK > 0)
+                    ok = ((fw_mask >> r) & 1u) != 0 && k < kend;
+                else
+                {
+                    const int h = fw_hb + kh, w = fw_wb + kw;
+                    ok = fw_live && k < kend && (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
+                }
                 rb_[u] = ok ? fw_base[(c * cv.H + kh) * cv.W + kw] : 0.f;
             }
         }
@@ -277,12 +299,33 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g, ConvSr
             const int64_t n = mm / ((int64_t)cv.OW * cv.OH);
             const int hb = oh * cv.SH - cv.PH, wb = ow * cv.SW - cv.PW;
             const float *base = g.B + n * cv.C * cv.H * cv.W + (int64_t)hb * cv.W + wb;
-#pragma unroll
-            for (int u = 0; u < B_PER_T; ++u)
+            if constexpr (CK > 0)
             {
-                const int h = hb + wg_kh[u], w = wb + wg_kw[u];
-                const bool ok = live && (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
-                rb_[u] = ok ? base[wg_off[u]] : 0.f;
+                // bit kh*CK+kw of pm: that tap of this slab's pixel lies inside the image
+                unsigned colm = 0, pm = 0;
+#pragma unroll
+                for (int kw = 0; kw < CK; ++kw)
+                    colm |= ((unsigned)(wb + kw) < (unsigned)cv.W ? 1u : 0u) << kw;
+#pragma unroll
+                for (int kh = 0; kh < CK; ++kh)
+                    pm |= ((unsigned)(hb + kh) < (unsigned)cv.H ? colm : 0u) << (kh * CK);
+                pm = live ? pm : 0u;
+#pragma unroll
+                for (int u = 0; u < B_PER_T; ++u)
+                {
+                    const bool ok = ((pm >> ((wg_taps >> (4 * u)) & 15u)) & 1u) != 0;
+                    rb_[u] = ok ? base[wg_off[u]] : 0.f;
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int u = 0; u < B_PER_T; ++u)
+                {
+                    const int h = hb + wg_kh[u], w = wb + wg_kw[u];
+                    const bool ok = live && (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
+                    rb_[u] = ok ? base[wg_off[u]] : 0.f;
+                }
             }
         }
         else
@@ -691,9 +734,11 @@ bool aligned16(const void *p)
 
 int wgrad_splits(int64_t OC, int64_t K, int64_t M)
 {
+    // as many K slices as keep every workgroup resident at once (256 CUs x 3 or 4 workgroups by register use):
+    // one slice more and the last few workgroups run alone after all the others
     const int64_t tiles = odl::ceil_div(OC, OC <= 64 ? 64 : 128) * odl::ceil_div(K, 128);
     const int64_t kt = odl::ceil_div(M, kBK);
-    int64_t s = odl::ceil_div(768, tiles);
+    int64_t s = (OC <= 64 ? 1024 : 768) / tiles;
     if (s > kt / 16)
         s = kt / 16;
     if (s > 256)
