@@ -28,7 +28,8 @@ size_t conv_implicit_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, i
 size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW);
 int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
-                          hipStream_t st);
+                          void *workspace, size_t workspace_bytes, hipStream_t st);
+size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
 int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W,
                         int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
                         void *workspace, size_t workspace_bytes, hipStream_t st);
@@ -67,6 +68,13 @@ __device__ inline int64_t xcd_contiguous_block(int64_t bid, int64_t nb)
 {
     const int64_t xcd = bid % 8, loc = bid / 8;
     const int64_t full = nb / 8, rem = nb % 8;
+    return xcd * full + (xcd < rem ? xcd : rem) + loc;
+}
+
+__device__ inline unsigned xcd_contiguous_block32(unsigned bid, unsigned nb)
+{
+    const unsigned xcd = bid % 8u, loc = bid / 8u;
+    const unsigned full = nb / 8u, rem = nb % 8u;
     return xcd * full + (xcd < rem ? xcd : rem) + loc;
 }
 
@@ -147,6 +155,140 @@ __global__ __launch_bounds__(kImThreads) void im2col_matrix_kernel(const float *
     }
 }
 
+// Matrix layout, the fast path: tile = 64 consecutive col rows (pixels) x CT channels with all their taps.
+// Read phase: lanes run along the pixels, each wave takes every fourth channel and issues that channel's taps
+// together (a 3x3 window is unrolled and its in-image test is one bit of a per-lane mask computed once);
+// the tile is turned through LDS (odd row stride: no bank conflicts) and leaves as 16-byte stores along the
+// col rows. All index arithmetic is 32-bit, and the per-store division is a multiply by a precomputed reciprocal:
+// on a 64-wide wave integer address arithmetic, not memory, is what this kernel would otherwise wait for.
+struct Im2colTile
+{
+    int CT, ctiles, LS;      // channels per tile, channel tiles, LDS row stride (floats, odd)
+    unsigned mtiles;         // pixel tiles
+    unsigned q4_magic;       // ceil(2^32 / q4) for q4 = CT*KH*KW/4
+};
+
+template <int CK>
+__global__ __launch_bounds__(256) void im2col_tile_kernel(const float *__restrict__ img, float *__restrict__ col,
+                                                           ConvGeom g, Im2colTile t)
+{
+    extern __shared__ float sh_i2c[];
+    float *sh = sh_i2c;
+    const int KH = CK > 0 ? CK : g.KH, KW = CK > 0 ? CK : g.KW;
+    const int KHW = KH * KW;
+    const unsigned vb = xcd_contiguous_block32(blockIdx.x, t.mtiles * (unsigned)t.ctiles);
+    const unsigned mt = vb / (unsigned)t.ctiles;
+    const int ct = (int)(vb - mt * (unsigned)t.ctiles);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int H = (int)g.H, W = (int)g.W, C = (int)g.C, OW = (int)g.OW;
+    const unsigned P = (unsigned)(g.OH * g.OW);
+    const unsigned M = (unsigned)(g.N * g.OH * g.OW);
+    const unsigned m = mt * 64u + (unsigned)lane;
+    const bool live = m < M;
+    const unsigned mm = live ? m : 0u;
+    const unsigned n = mm / P, r = mm - n * P;
+    const int oh = (int)(r / (unsigned)OW), ow = (int)(r - (unsigned)oh * (unsigned)OW);
+    const int h0 = oh * g.SH - g.PH, w0 = ow * g.SW - g.PW;
+    const int c0 = ct * t.CT;
+    const int ccn = (C - c0 < t.CT) ? C - c0 : t.CT;
+    const int HW = H * W;
+    // first tap of this lane's window in channel c0; dereferenced only where the tap lies inside the image
+    const float *p = img + ((int64_t)n * C + c0) * HW + (int64_t)h0 * W + w0;
+    float *srow = sh + lane * t.LS;
+    if constexpr (CK > 0)
+    {
+        unsigned mask = 0;
+#pragma unroll
+        for (int kh = 0; kh < CK; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < CK; ++kw)
+                if (live && (unsigned)(h0 + kh) < (unsigned)H && (unsigned)(w0 + kw) < (unsigned)W)
+                    mask |= 1u << (kh * CK + kw);
+        for (int cl = wave; cl < ccn; cl += 4)
+        {
+            const float *pc = p + cl * HW;
+            float v[CK * CK];
+#pragma unroll
+            for (int kh = 0; kh < CK; ++kh)
+#pragma unroll
+                for (int kw = 0; kw < CK; ++kw)
+                    v[kh * CK + kw] = ((mask >> (kh * CK + kw)) & 1u) ? pc[kh * W + kw] : 0.f;
+#pragma unroll
+            for (int q = 0; q < CK * CK; ++q)
+                srow[cl * (CK * CK) + q] = v[q];
+        }
+    }
+    else
+    {
+        for (int cl = wave; cl < ccn; cl += 4)
+        {
+            const float *pc = p + cl * HW;
+            for (int kh = 0; kh < KH; ++kh)
+            {
+                const bool hok = live && (unsigned)(h0 + kh) < (unsigned)H;
+                for (int kw = 0; kw < KW; ++kw)
+                {
+                    const bool ok = hok && (unsigned)(w0 + kw) < (unsigned)W;
+                    srow[cl * KHW + kh * KW + kw] = ok ? pc[kh * W + kw] : 0.f;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int K = C * KHW;
+    const int run = ccn * KHW;
+    const unsigned row0 = mt * 64u;
+    const int rows = (M - row0 < 64u) ? (int)(M - row0) : 64;
+    float *dst0 = col + (int64_t)row0 * K + c0 * KHW;
+    if ((run & 3) == 0 && (K & 3) == 0 && ((c0 * KHW) & 3) == 0 && (reinterpret_cast<uintptr_t>(col) & 15) == 0)
+    {
+        const int q4 = run >> 2;
+        // row = e / q4 through the reciprocal: exact while e < 2^32 / q4, and e < 64 * q4 here. The reciprocal is that
+        // of a full tile's q4; a ragged last channel tile (smaller run) divides directly.
+        const bool full = ccn == t.CT && t.q4_magic != 0;
+        for (int e = threadIdx.x; e < rows * q4; e += 256)
+        {
+            const int row = full ? (int)__umulhi((unsigned)e, t.q4_magic) : e / q4;
+            const int q = e - row * q4;
+            const float *sr = sh + row * t.LS + 4 * q;
+            const f32x4 o = {sr[0], sr[1], sr[2], sr[3]};
+            *reinterpret_cast<f32x4 *>(dst0 + (int64_t)row * K + 4 * q) = o;
+        }
+    }
+    else
+    {
+        for (int e = threadIdx.x; e < rows * run; e += 256)
+        {
+            const int row = e / run, j = e - row * run;
+            dst0[(int64_t)row * K + j] = sh[row * t.LS + j];
+        }
+    }
+}
+
+// Tile shape for im2col_tile_kernel, or false when the shape needs the general kernel (64-bit indices, huge windows).
+bool plan_im2col_tile(const ConvGeom &g, Im2colTile &t)
+{
+    const int64_t KHW = (int64_t)g.KH * g.KW, M = g.N * g.OH * g.OW;
+    if (KHW > 160 || M >= (1ll << 31) - 64 || g.C * g.H * g.W >= (1ll << 31) || g.C * KHW >= (1ll << 31))
+        return false;
+    int CT = (int)(144 / KHW);
+    CT = CT < 1 ? 1 : (CT > 128 ? 128 : CT);
+    if (CT > g.C)
+        CT = (int)g.C;
+    if (CT >= 4)
+        CT &= ~3;  // a multiple of four channels keeps every tile's columns 16-byte aligned
+    t.CT = CT;
+    t.ctiles = (int)odl::ceil_div(g.C, CT);
+    t.LS = (int)(CT * KHW) | 1;
+    t.mtiles = (unsigned)odl::ceil_div(M, 64);
+    if ((int64_t)t.mtiles * t.ctiles >= (1ll << 31))
+        return false;
+    const unsigned q4 = (unsigned)(CT * KHW / 4);
+    t.q4_magic = q4 > 1 ? (unsigned)(((1ull << 32) + q4 - 1) / q4) : 0u;  // 0: the kernel divides directly
+    return true;
+}
+
 // col[n][c][kh][kw][oh][ow]; one thread per element, consecutive threads along ow.
 __global__ void im2col_6d_kernel(const float *__restrict__ img, float *__restrict__ col, ConvGeom g)
 {
@@ -205,12 +347,14 @@ __global__ void col2im_6d_kernel(const float *__restrict__ col, float *__restric
 // Matrix layout [N*OH*OW, C*KH*KW]: a workgroup owns 64 channels x 16 consecutive w of one image row. Lanes run
 // along the channel, where a col row is nearly contiguous (KH*KW floats apart), each thread sums 4 pixels, and the
 // 64x16 result tile is turned through LDS so that the image is written in 64-byte runs along w.
-template <int CKH, int CKW>
+// CS > 0 fixes both strides at compile time (the tap arithmetic divides by them).
+template <int CKH, int CKW, int CS>
 __global__ __launch_bounds__(256) void col2im_matrix_kernel(const float *__restrict__ col, float *__restrict__ img,
                                                              ConvGeom g, int wtiles, int ctiles)
 {
     __shared__ float sh[64][17];
     const int KH = CKH > 0 ? CKH : g.KH, KW = CKW > 0 ? CKW : g.KW;
+    const int SH = CS > 0 ? CS : g.SH, SW = CS > 0 ? CS : g.SW;
     const int64_t nb = g.N * g.H * wtiles * ctiles;
     int64_t vb = xcd_contiguous_block(blockIdx.x, nb);
     const int ct = (int)(vb % ctiles);
@@ -226,6 +370,7 @@ __global__ __launch_bounds__(256) void col2im_matrix_kernel(const float *__restr
     if (c < g.C)
     {
         const float *cbase = col + (int64_t)c * KH * KW;
+        const float *nbase = cbase + n * OH * OW * K;  // this image's rows; offsets below fit 32 bits (checked by the host)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
         {
@@ -241,15 +386,16 @@ __global__ __launch_bounds__(256) void col2im_matrix_kernel(const float *__restr
                     for (int kh = 0; kh < CKH; ++kh)
                     {
                         const int hp = h + g.PH - kh;
-                        const int oh = hp / g.SH;
-                        const bool hok = hp >= 0 && hp % g.SH == 0 && oh < OH;
+                        const int oh = hp / SH;
+                        const bool hok = hp >= 0 && hp % SH == 0 && oh < OH;
+                        const int ro = oh * OW;
 #pragma unroll
                         for (int kw = 0; kw < CKW; ++kw)
                         {
                             const int wp = w + g.PW - kw;
-                            const int ow = wp / g.SW;
-                            const bool ok = hok && wp >= 0 && wp % g.SW == 0 && ow < OW;
-                            v[kh * CKW + kw] = ok ? cbase[((n * OH + oh) * OW + ow) * K + kh * CKW + kw] : 0.f;
+                            const int ow = wp / SW;
+                            const bool ok = hok && wp >= 0 && wp % SW == 0 && ow < OW;
+                            v[kh * CKW + kw] = ok ? nbase[(ro + ow) * K + kh * CKW + kw] : 0.f;
                         }
                     }
                     // a skipped tap contributes nothing in the reference; adding +0.0f instead leaves every
@@ -263,17 +409,17 @@ __global__ __launch_bounds__(256) void col2im_matrix_kernel(const float *__restr
                     for (int kh = 0; kh < KH; ++kh)
                     {
                         const int hp = h + g.PH - kh;
-                        if (hp < 0 || hp % g.SH != 0)
+                        if (hp < 0 || hp % SH != 0)
                             continue;
-                        const int oh = hp / g.SH;
+                        const int oh = hp / SH;
                         if (oh >= OH)
                             continue;
                         for (int kw = 0; kw < KW; ++kw)
                         {
                             const int wp = w + g.PW - kw;
-                            if (wp < 0 || wp % g.SW != 0)
+                            if (wp < 0 || wp % SW != 0)
                                 continue;
-                            const int ow = wp / g.SW;
+                            const int ow = wp / SW;
                             if (ow >= OW)
                                 continue;
                             acc += cbase[((n * OH + oh) * OW + ow) * K + kh * KW + kw];
@@ -302,6 +448,220 @@ __global__ __launch_bounds__(256) void col2im_matrix_kernel(const float *__restr
     }
 }
 
+// Matrix layout, the fast path: a workgroup owns CT channels x TH x TW pixels of one image. It first copies the
+// rectangle of col rows those pixels draw from — ohr x owr output positions, CT*KH*KW consecutive floats of each —
+// into LDS with coalesced 16-byte loads, then sums each pixel's taps out of LDS in ascending (kh, kw) and writes the
+// image along w. Lanes run along w in both the LDS reads (odd row stride: distinct banks) and the image writes.
+// Index arithmetic is 32-bit with reciprocal multiplies, and the compute loop is wave-uniform over (channel, row).
+struct Col2imTile
+{
+    int TH, TW, CT;          // pixels and channels per workgroup
+    int htiles, wtiles, ctiles;
+    int ohr, owr;            // staged rectangle of output positions
+    int LS;                  // LDS row stride in floats (odd)
+    unsigned q4_magic;       // ceil(2^32 / (CT*KH*KW/4)), 0 = divide directly
+    unsigned owr_magic;      // ceil(2^32 / owr)
+};
+
+__device__ inline int ceil_div_signed(int a, int d)  // d > 0
+{
+    return a >= 0 ? (a + d - 1) / d : -((-a) / d);
+}
+
+template <int CK, int CS>
+__global__ __launch_bounds__(256) void col2im_tile_kernel(const float *__restrict__ col, float *__restrict__ img,
+                                                           ConvGeom g, Col2imTile t)
+{
+    extern __shared__ float sh_c2i[];
+    float *sh = sh_c2i;
+    const int KH = CK > 0 ? CK : g.KH, KW = CK > 0 ? CK : g.KW;
+    const int SH = CS > 0 ? CS : g.SH, SW = CS > 0 ? CS : g.SW;
+    const int KHW = KH * KW;
+    const int H = (int)g.H, W = (int)g.W, OH = (int)g.OH, OW = (int)g.OW, C = (int)g.C;
+    unsigned vb = xcd_contiguous_block32(blockIdx.x, (unsigned)g.N * t.htiles * t.wtiles * t.ctiles);
+    const int ct = (int)(vb % (unsigned)t.ctiles);
+    vb /= (unsigned)t.ctiles;
+    const int wt = (int)(vb % (unsigned)t.wtiles);
+    vb /= (unsigned)t.wtiles;
+    const int ht = (int)(vb % (unsigned)t.htiles);
+    const int n = (int)(vb / (unsigned)t.htiles);
+    const int h0 = ht * t.TH, w0 = wt * t.TW, c0 = ct * t.CT;
+    const int th = (H - h0 < t.TH) ? H - h0 : t.TH, tw = (W - w0 < t.TW) ? W - w0 : t.TW;
+    const int ccn = (C - c0 < t.CT) ? C - c0 : t.CT;
+    // first output position (possibly negative) whose window can reach this tile
+    const int oh_lo = ceil_div_signed(h0 + g.PH - (KH - 1), SH), ow_lo = ceil_div_signed(w0 + g.PW - (KW - 1), SW);
+    const int K = C * KHW;
+    const int run = ccn * KHW;
+    const float *src0 = col + (int64_t)n * OH * OW * K + c0 * KHW;  // offsets from here fit 32 bits (checked by the host)
+    const int R = t.ohr * t.owr;
+    if ((run & 3) == 0 && (K & 3) == 0 && ((c0 * KHW) & 3) == 0 && (reinterpret_cast<uintptr_t>(col) & 15) == 0)
+    {
+        const int q4 = run >> 2;
+        const bool recip = ccn == t.CT && t.q4_magic != 0;
+        constexpr int U = 8;  // independent 16-byte loads in flight per thread
+        for (int e0 = threadIdx.x; e0 < R * q4; e0 += 256 * U)
+        {
+            f32x4 v[U];
+            int doff[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+            {
+                const int e = e0 + 256 * u;
+                const int r = recip ? (int)__umulhi((unsigned)e, t.q4_magic) : e / q4;
+                const int q = e - r * q4;
+                const int ro = t.owr_magic ? (int)__umulhi((unsigned)r, t.owr_magic) : r;  // owr == 1: every row is its own
+                const int oh = oh_lo + ro, ow = ow_lo + (r - ro * t.owr);
+                const bool ok = e < R * q4 && (unsigned)oh < (unsigned)OH && (unsigned)ow < (unsigned)OW;
+                doff[u] = ok ? r * t.LS + 4 * q : -1;
+                v[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (ok)
+                    v[u] = *reinterpret_cast<const f32x4 *>(src0 + (oh * OW + ow) * K + 4 * q);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (doff[u] >= 0)
+                {
+                    float *d = sh + doff[u];
+                    d[0] = v[u][0], d[1] = v[u][1], d[2] = v[u][2], d[3] = v[u][3];
+                }
+        }
+    }
+    else
+    {
+        for (int e = threadIdx.x; e < R * run; e += 256)
+        {
+            const int r = e / run, j = e - r * run;
+            const int ro = t.owr_magic ? (int)__umulhi((unsigned)r, t.owr_magic) : r;  // owr == 1: every row is its own
+            const int oh = oh_lo + ro, ow = ow_lo + (r - ro * t.owr);
+            if ((unsigned)oh < (unsigned)OH && (unsigned)ow < (unsigned)OW)
+                sh[r * t.LS + j] = src0[(oh * OW + ow) * K + j];
+        }
+    }
+    __syncthreads();
+    // lanes: RW image rows of TW pixels per wave; waves walk (channel, row group) pairs
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int RW = 64 / t.TW;  // >= 1 (TW <= 64)
+    const int lr = lane / t.TW, lw = lane - lr * t.TW;
+    const int hgroups = (th + RW - 1) / RW;
+    const int w = w0 + lw;
+    const bool lane_ok = lr < RW && lw < tw;
+    float *dst0 = img + ((int64_t)n * C + c0) * H * W;
+    for (int idx = wave; idx < ccn * hgroups; idx += 4)
+    {
+        const int cl = idx / hgroups, hg = idx - cl * hgroups;  // wave-uniform
+        const int hh = hg * RW + lr;
+        if (!lane_ok || hh >= th)
+            continue;
+        const int h = h0 + hh;
+        const float *cs = sh + cl * KHW;
+        float acc = 0.f;
+        if constexpr (CK > 0)
+        {
+            // every tap is read (or zeroed) first, then added in ascending (kh, kw): a skipped tap contributes nothing
+            // in the reference, and adding +0.0f instead leaves each partial sum unchanged (the accumulator starts at
+            // +0.0f and never becomes -0.0f)
+            float v[CK * CK];
+#pragma unroll
+            for (int kh = 0; kh < CK; ++kh)
+            {
+                const int hp = h + g.PH - kh;
+                const int oh = hp / SH;
+                const bool hok = hp >= 0 && hp % SH == 0 && oh < OH;
+                const int rb = (oh - oh_lo) * t.owr - ow_lo;
+#pragma unroll
+                for (int kw = 0; kw < CK; ++kw)
+                {
+                    const int wp = w + g.PW - kw;
+                    const int ow = wp / SW;
+                    const bool ok = hok && wp >= 0 && wp % SW == 0 && ow < OW;
+                    v[kh * CK + kw] = ok ? cs[(rb + ow) * t.LS + kh * CK + kw] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < CK * CK; ++q)
+                acc += v[q];
+        }
+        else
+        {
+            for (int kh = 0; kh < KH; ++kh)
+            {
+                const int hp = h + g.PH - kh;
+                if (hp < 0 || hp % SH != 0)
+                    continue;
+                const int oh = hp / SH;
+                if (oh >= OH)
+                    continue;
+                for (int kw = 0; kw < KW; ++kw)
+                {
+                    const int wp = w + g.PW - kw;
+                    if (wp < 0 || wp % SW != 0)
+                        continue;
+                    const int ow = wp / SW;
+                    if (ow >= OW)
+                        continue;
+                    acc += cs[((oh - oh_lo) * t.owr + (ow - ow_lo)) * t.LS + kh * KW + kw];
+                }
+            }
+        }
+        dst0[(cl * H + h) * W + w] = acc;
+    }
+}
+
+// Tile shape for col2im_tile_kernel: the staged rectangle must fit in a third of a CU's LDS, there should be enough
+// workgroups to fill the chip, and among those the tile that re-reads the fewest col rows wins. False when the
+// shape needs the general kernel (64-bit offsets, windows too large to stage).
+bool plan_col2im_tile(const ConvGeom &g, Col2imTile &best)
+{
+    const int64_t KHW64 = (int64_t)g.KH * g.KW;
+    if (KHW64 > 160 || g.OH * g.OW * g.C * KHW64 >= (1ll << 31) || g.C * g.H * g.W >= (1ll << 31) || g.N >= (1 << 20))
+        return false;
+    const int KHW = (int)KHW64, H = (int)g.H, W = (int)g.W, C = (int)g.C;
+    double best_cost = 0;
+    bool found = false;
+    const int tw_opts[3] = {W <= 64 ? W : 64, (W <= 64 && W % 2 == 0 && W / 2 >= 8) ? W / 2 : 0, W > 64 ? 32 : 0};
+    for (int twi = 0; twi < 3; ++twi)
+    {
+        const int TW = tw_opts[twi];
+        if (TW <= 0)
+            continue;
+        for (int CT = 16; CT >= 1; CT >>= 1)
+        {
+            if (CT > C && CT != 1)
+                continue;
+            const int LS = (CT * KHW) | 1;
+            for (int TH = 1; TH <= H && TH <= 32; ++TH)
+            {
+                const int ohr = (TH + g.KH - 2) / g.SH + 1, owr = (TW + g.KW - 2) / g.SW + 1;
+                const size_t lds = (size_t)ohr * owr * LS * sizeof(float);
+                if (lds > 53 * 1024)
+                    break;
+                Col2imTile t{TH, TW, CT, (int)odl::ceil_div(H, TH), (int)odl::ceil_div(W, TW), (int)odl::ceil_div(C, CT),
+                             ohr, owr, LS, 0u, 0u};
+                const double blocks = (double)g.N * t.htiles * t.wtiles * t.ctiles;
+                if (blocks >= (double)(1ll << 31))
+                    continue;
+                // col rows staged per image pixel relative to the rows a pixel needs; short runs, idle lanes and a
+                // half-empty chip are charged on top
+                double cost = (double)ohr * owr * g.SH * g.SW / ((double)TH * TW);
+                if (CT * KHW * 4 < 256)
+                    cost *= 1.0 + 0.5 * (256.0 - CT * KHW * 4) / 256.0;
+                cost *= 64.0 / ((64 / TW) * TW);
+                if (blocks < 4096)
+                    cost *= 1.0 + 0.25 * (4096.0 / blocks - 1.0);
+                if (!found || cost < best_cost)
+                    best = t, best_cost = cost, found = true;
+            }
+        }
+    }
+    if (!found)
+        return false;
+    const unsigned q4 = (unsigned)(best.CT * KHW / 4);
+    best.q4_magic = q4 > 1 ? (unsigned)(((1ull << 32) + q4 - 1) / q4) : 0u;
+    best.owr_magic = best.owr > 1 ? (unsigned)(((1ull << 32) + best.owr - 1) / best.owr) : 0u;
+    return true;
+}
+
 int make_geom(ConvGeom &g, const char *who, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
               int PH, int PW)
 {
@@ -324,6 +684,20 @@ int im2col_launch(const float *img, float *col, const ConvGeom &g, int to_matrix
         return ODL_OK;
     if (to_matrix)
     {
+        Im2colTile t;
+        if (plan_im2col_tile(g, t))
+        {
+            const size_t lds = (size_t)64 * t.LS * sizeof(float);
+            const unsigned nbt = t.mtiles * (unsigned)t.ctiles;
+            if (g.KH == 3 && g.KW == 3)
+                hipLaunchKernelGGL((im2col_tile_kernel<3>), dim3(nbt), dim3(256), lds, st, img, col, g, t);
+            else if (g.KH == 1 && g.KW == 1)
+                hipLaunchKernelGGL((im2col_tile_kernel<1>), dim3(nbt), dim3(256), lds, st, img, col, g, t);
+            else
+                hipLaunchKernelGGL((im2col_tile_kernel<0>), dim3(nbt), dim3(256), lds, st, img, col, g, t);
+            ODL_LAUNCH_CHECK();
+            return ODL_OK;
+        }
         const int tk = K < kImCk ? (int)K : kImCk;
         const int ktiles = (int)odl::ceil_div(K, tk);
         const int64_t mtiles = odl::ceil_div(g.N * g.OH * g.OW, kImPix);
@@ -346,15 +720,43 @@ int col2im_launch(const float *col, float *img, const ConvGeom &g, int to_matrix
         return ODL_OK;
     if (to_matrix)
     {
+        const int cs = (g.SH == g.SW && (g.SH == 1 || g.SH == 2)) ? g.SH : 0;
+        Col2imTile t;
+        // the staged kernel pays off at stride 1, where neighbouring pixels share most of their col rows
+        if (cs == 1 && plan_col2im_tile(g, t))
+        {
+            const unsigned nbt = (unsigned)(g.N * t.htiles * t.wtiles * t.ctiles);
+            const size_t lds = (size_t)t.ohr * t.owr * t.LS * sizeof(float);
+#define ODL_COL2IM_TILE(CKV, CSV) \
+    hipLaunchKernelGGL((col2im_tile_kernel<CKV, CSV>), dim3(nbt), dim3(256), lds, st, col, img, g, t)
+            if (g.KH == 3 && g.KW == 3 && cs == 1)
+                ODL_COL2IM_TILE(3, 1);
+            else if (g.KH == 3 && g.KW == 3 && cs == 2)
+                ODL_COL2IM_TILE(3, 2);
+            else if (cs == 1)
+                ODL_COL2IM_TILE(0, 1);
+            else
+                ODL_COL2IM_TILE(0, 0);
+#undef ODL_COL2IM_TILE
+            ODL_LAUNCH_CHECK();
+            return ODL_OK;
+        }
         const int wtiles = (int)odl::ceil_div(g.W, 16), ctiles = (int)odl::ceil_div(g.C, 64);
         const int64_t nb = g.N * g.H * wtiles * ctiles;
         ODL_REQUIRE(nb < (1ll << 31) && g.N * g.OH * g.OW * g.C * g.KH * g.KW < (1ll << 40), "col2im: too large");
-        if (g.KH == 3 && g.KW == 3)
-            hipLaunchKernelGGL((col2im_matrix_kernel<3, 3>), dim3((unsigned)nb), dim3(256), 0, st, col, img, g, wtiles,
-                               ctiles);
+#define ODL_COL2IM_CASE(KHV, KWV, CSV)                                                                               \
+    hipLaunchKernelGGL((col2im_matrix_kernel<KHV, KWV, CSV>), dim3((unsigned)nb), dim3(256), 0, st, col, img, g, wtiles, \
+                       ctiles)
+        const bool k3 = g.KH == 3 && g.KW == 3 && g.OH * g.OW * g.C * 9 < (1ll << 31);  // 32-bit row offsets
+        if (k3 && cs == 1)
+            ODL_COL2IM_CASE(3, 3, 1);
+        else if (k3 && cs == 2)
+            ODL_COL2IM_CASE(3, 3, 2);
+        else if (k3)
+            ODL_COL2IM_CASE(3, 3, 0);
         else
-            hipLaunchKernelGGL((col2im_matrix_kernel<0, 0>), dim3((unsigned)nb), dim3(256), 0, st, col, img, g, wtiles,
-                               ctiles);
+            ODL_COL2IM_CASE(0, 0, 0);
+#undef ODL_COL2IM_CASE
     }
     else
         hipLaunchKernelGGL(col2im_6d_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, col, img, g);
@@ -400,7 +802,8 @@ size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W
     if (OH <= 0 || OW <= 0)
         return 0;
     if (odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW))
-        return 0;  // the im2col matrix is never materialised
+        return align256(odl::conv_implicit_forward_workspace(N, C, OC, KH, KW, OH, OW));  // no im2col matrix; K-slice
+                                                                                          // partials for small outputs
     return align256((size_t)(N * OH * OW * C * KH * KW) * sizeof(float));
 }
 
@@ -419,7 +822,8 @@ int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, in
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
     if (odl::conv_implicit_forward_ok(w, N, C, H, W, OC, KH, KW, g.OH, g.OW))
-        return odl::conv_implicit_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, st);
+        return odl::conv_implicit_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, workspace,
+                                          workspace_bytes, st);
     // explicit path: col = im2col(x), then y^T[OC, M] = W2d[OC,K] . col[M,K]^T stored as y[n][oc][p] (+ bias per channel)
     const size_t need = align256((size_t)(M * K) * sizeof(float));
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,

@@ -26,6 +26,11 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 namespace
 {
 constexpr int kThreads = 256;
+
+inline bool aligned16(const void *p)
+{
+    return reinterpret_cast<uintptr_t>(p) % 16 == 0;
+}
 constexpr int kXcds    = 8;
 constexpr int kGroupM  = 8;
 
@@ -507,7 +512,7 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
 constexpr int kRedGroups = 16;
 __global__ __launch_bounds__(64 * kRedGroups) void splitk_reduce_kernel(const float *__restrict__ part, int splits,
                                                                          int64_t stride, float *out, int64_t M, int64_t N,
-                                                                         int64_t ldc, const float *bias)
+                                                                         int64_t ldc, const float *bias, int64_t P)
 {
     __shared__ float sh[kRedGroups][64];
     const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
@@ -525,10 +530,72 @@ __global__ __launch_bounds__(64 * kRedGroups) void splitk_reduce_kernel(const fl
         for (int k = 1; k < kRedGroups; ++k)
             s += sh[k][lane];
         const int64_t r = i / N, c = i % N;
-        if (bias)
-            s = s + bias[c];
-        out[r * ldc + c] = s;
+        if (P > 0)
+        {
+            // convolution forward: row = output channel (bias by row), column = n*P + p -> y[n][row][p]
+            if (bias)
+                s = s + bias[r];
+            out[((c / P) * M + r) * P + c % P] = s;
+        }
+        else
+        {
+            if (bias)
+                s = s + bias[c];
+            out[r * ldc + c] = s;
+        }
     }
+}
+
+// The same sum for few slices of a large output: one thread per four consecutive outputs, slices added in
+// ascending order. Needs N % 4 == 0 (and P % 4 == 0) so that a quad stays inside one row (and one image).
+__global__ __launch_bounds__(256) void splitk_reduce_vec_kernel(const float *__restrict__ part, int splits,
+                                                                 int64_t stride, float *out, int64_t M, int64_t N,
+                                                                 int64_t ldc, const float *bias, int64_t P)
+{
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= M * N)
+        return;
+    f32x4 acc = *reinterpret_cast<const f32x4 *>(part + i);
+#pragma unroll 4
+    for (int z = 1; z < splits; ++z)
+    {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(part + (int64_t)z * stride + i);
+        acc[0] += v[0], acc[1] += v[1], acc[2] += v[2], acc[3] += v[3];
+    }
+    const int64_t r = i / N, c = i % N;
+    if (P > 0)
+    {
+        if (bias)
+        {
+            const float b = bias[r];
+            acc[0] = acc[0] + b, acc[1] = acc[1] + b, acc[2] = acc[2] + b, acc[3] = acc[3] + b;
+        }
+        *reinterpret_cast<f32x4 *>(out + ((c / P) * M + r) * P + c % P) = acc;
+    }
+    else
+    {
+        if (bias)
+        {
+            const f32x4 b = *reinterpret_cast<const f32x4 *>(bias + c);
+            acc[0] = acc[0] + b[0], acc[1] = acc[1] + b[1], acc[2] = acc[2] + b[2], acc[3] = acc[3] + b[3];
+        }
+        *reinterpret_cast<f32x4 *>(out + r * ldc + c) = acc;
+    }
+}
+
+// picks the reduction by shape: many slices of a small output -> slice groups in parallel; few slices of a large
+// output -> streaming quads
+void launch_splitk_reduce(const float *part, int splits, int64_t stride, float *out, int64_t M, int64_t N, int64_t ldc,
+                          const float *bias, int64_t P, hipStream_t st)
+{
+    const bool quads = splits <= 32 && M * N >= (1 << 16) && N % 4 == 0 && stride % 4 == 0 && ldc % 4 == 0 && P % 4 == 0 &&
+                       aligned16(part) && aligned16(out) && (bias == nullptr || P > 0 || aligned16(bias));
+    if (quads)
+        hipLaunchKernelGGL(splitk_reduce_vec_kernel, dim3((unsigned)odl::ceil_div(M * N, 1024)), dim3(256), 0, st, part,
+                           splits, stride, out, M, N, ldc, bias, P);
+    else
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)odl::ceil_div(M * N, 64)), dim3(64 * kRedGroups), 0, st,
+                           part, splits, stride, out, M, N, ldc, bias, P);
 }
 
 __global__ void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows, int64_t cols)
@@ -665,10 +732,8 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
         if (rc != ODL_OK)
             return fail(rc, "sgemm: no kernel variant");
         ODL_LAUNCH_CHECK();
-        const int64_t total = M * N;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(total, 64)), dim3(64 * kRedGroups), 0, st,
-                           static_cast<const float *>(workspace), splits, M * N, C, M, N, ldc,
-                           epi == EPI_BIAS_COL ? bias : nullptr);
+        launch_splitk_reduce(static_cast<const float *>(workspace), splits, M * N, C, M, N, ldc,
+                             epi == EPI_BIAS_COL ? bias : nullptr, 0, st);
         ODL_LAUNCH_CHECK();
         return ODL_OK;
     }
@@ -727,11 +792,6 @@ __global__ void permute_weight_kernel(const float *__restrict__ w, float *__rest
     wp[t] = w[((int64_t)oc * C + c) * KHW + tap];
 }
 
-bool aligned16(const void *p)
-{
-    return reinterpret_cast<uintptr_t>(p) % 16 == 0;
-}
-
 int wgrad_splits(int64_t OC, int64_t K, int64_t M)
 {
     // as many K slices as keep every workgroup resident at once (256 CUs x 3 or 4 workgroups by register use):
@@ -788,18 +848,58 @@ static ConvSrc make_src(int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
     return ConvSrc{(int)C, (int)H, (int)W, (int)OH, (int)OW, (int)OC, KH, KW, SH, SW, PH, PW};
 }
 
+// K slices of the forward product when its 128x128 tiles alone leave most of the chip idle
+static int forward_splits(int64_t OC, int64_t M, int64_t K)
+{
+    const int64_t tiles = ceil_div(OC, 128) * ceil_div(M, 128);
+    const int64_t kt = ceil_div(K, kBK);
+    if (OC <= 64 || tiles >= 200 || kt < 16)
+        return 1;
+    int64_t s = 768 / tiles;
+    if (s > kt / 8)
+        s = kt / 8;
+    if (s > 16)
+        s = 16;
+    return s < 2 ? 1 : (int)s;
+}
+
+size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW)
+{
+    const int64_t K = C * KH * KW, M = N * OH * OW;
+    const int s = forward_splits(OC, M, K);
+    return s > 1 ? (size_t)s * OC * M * sizeof(float) : 0;
+}
+
 // y[n][oc][p] = sum_k W2d[oc][k] * x_gathered[(n,p)][k] + b[oc]
 int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
-                          hipStream_t st)
+                          void *workspace, size_t workspace_bytes, hipStream_t st)
 {
     GemmArgs g{};
     g.A = w, g.B = x, g.C = y, g.bias = b;
     g.M = OC, g.N = N * OH * OW, g.K = C * KH * KW;
     g.lda = g.K, g.ldb = 0, g.ldc = 0, g.P = OH * OW;
     g.k_per_split = ceil_div(g.K, kBK) * kBK, g.c_split_stride = 0;
-    int rc = launch_conv_tile<SB_CONV_FWD, false, EPI_NCHW_ROWB>(g, make_src(C, H, W, OH, OW, OC, KH, KW, SH, SW, PH, PW),
-                                                                 1, st);
+    const ConvSrc cv = make_src(C, H, W, OH, OW, OC, KH, KW, SH, SW, PH, PW);
+    int splits = forward_splits(OC, g.N, g.K);
+    if (splits > 1 && (workspace == nullptr || workspace_bytes < (size_t)splits * OC * g.N * sizeof(float)))
+        splits = 1;  // a caller without the workspace still gets the single-pass kernel
+    int rc;
+    if (splits > 1)
+    {
+        // K slices into plain [OC, M] partials, then one pass that sums them in order, adds the bias and stores NCHW
+        g.k_per_split = ceil_div(ceil_div(g.K, kBK), splits) * kBK;
+        splits = (int)ceil_div(g.K, g.k_per_split);
+        g.C = static_cast<float *>(workspace), g.bias = nullptr, g.ldc = g.N, g.c_split_stride = OC * g.N;
+        rc = launch_conv_tile<SB_CONV_FWD, false, EPI_PLAIN>(g, cv, splits, st);
+        if (rc != ODL_OK)
+            return fail(rc, "conv2d: no kernel variant");
+        ODL_LAUNCH_CHECK();
+        launch_splitk_reduce(static_cast<const float *>(workspace), splits, OC * g.N, y, OC, g.N, g.N, b, g.P, st);
+        ODL_LAUNCH_CHECK();
+        return ODL_OK;
+    }
+    rc = launch_conv_tile<SB_CONV_FWD, false, EPI_NCHW_ROWB>(g, cv, 1, st);
     if (rc != ODL_OK)
         return fail(rc, "conv2d: no kernel variant");
     ODL_LAUNCH_CHECK();
@@ -832,8 +932,7 @@ int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, i
     ODL_LAUNCH_CHECK();
     if (splits > 1)
     {
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)ceil_div(OC * K, 64)), dim3(64 * kRedGroups), 0, st,
-                           static_cast<const float *>(workspace), splits, OC * K, gw, OC, K, K, nullptr);
+        launch_splitk_reduce(static_cast<const float *>(workspace), splits, OC * K, gw, OC, K, K, nullptr, 0, st);
         ODL_LAUNCH_CHECK();
     }
     return ODL_OK;
