@@ -25,7 +25,7 @@ bool conv_implicit_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, in
 bool conv_implicit_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
                             int SH, int SW);
 size_t conv_implicit_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
-size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW);
+size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW, int64_t pixels);
 int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
                           void *workspace, size_t workspace_bytes, hipStream_t st);
@@ -856,7 +856,7 @@ BwdPlan plan_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t 
     p.col_bytes = (p.wgrad_implicit && p.dgrad_implicit) ? 0 : align256((size_t)(M * K) * sizeof(float));
     p.splitk_bytes = align256(p.wgrad_implicit ? odl::conv_implicit_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
                                                : odl::sgemm_workspace(OC, K, M, 0));
-    p.wp_bytes = p.dgrad_implicit ? align256(odl::conv_implicit_dgrad_workspace(C, OC, KH, KW)) : 0;
+    p.wp_bytes = p.dgrad_implicit ? align256(odl::conv_implicit_dgrad_workspace(C, OC, KH, KW, N * H * W)) : 0;
     p.red_bytes = align256(odl::sum_nchw_channels_workspace(N, OC, OH * OW));
     return p;
 }

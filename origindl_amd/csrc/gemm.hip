@@ -70,7 +70,23 @@ struct GemmArgs
     int64_t P;               // EPI_NCHW_ROWB: OH*OW
     int tiles_m, tiles_n;
     int splits;              // K slices (grid = tiles_m * tiles_n * splits workgroups)
+    // Tail split (splits == 1 only): when the tile count is a little over a multiple of the CU count, the last
+    // `nt - tail_first` tiles would run alone after everything else. They are cut into tail_splits K pieces
+    // each — workgroups main_blocks.. — which write tile-local partials to tail_ws; tail_fixup_kernel sums them.
+    int main_blocks, tail_first, tail_splits;
+    int64_t tail_kps;
+    float *tail_ws;
 };
+
+__device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
+{
+    const int gsz = 8 * tiles_n;  // groups of 8 tile-rows
+    const int grp = t / gsz, in_g = t % gsz;
+    const int first_m = grp * 8;
+    const int gm = (tiles_m - first_m) < 8 ? (tiles_m - first_m) : 8;
+    tm = first_m + in_g % gm;
+    tn = in_g / gm;
+}
 
 template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI, int SB = SB_PLAIN, int CK = 0>
 __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_CONV_WGRAD ? 4 : 1)) void sgemm_mfma_kernel(GemmArgs g, ConvSrc cv)
@@ -105,26 +121,37 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
     // round-robin over the 8 XCDs, so the id is first unfolded into a contiguous band per XCD; inside a band the
     // tiles of one K slice are adjacent (they read the same K range of A and B, which then sits in that XCD's L2),
     // and tiles are walked in groups of kGroupM tile-rows.
-    int tm, tn, kz;
+    int tm, tn, kz = 0;
+    int64_t kbeg, kend;
+    float *tail_out = nullptr;
     {
         const int nt = g.tiles_m * g.tiles_n;
-        const int64_t total = (int64_t)nt * g.splits;
-        const int64_t bid = blockIdx.x;
-        const int64_t xcd = bid % kXcds, loc = bid / kXcds;
-        const int64_t full = total / kXcds, rem = total % kXcds;
-        const int64_t v = xcd * full + (xcd < rem ? xcd : rem) + loc;
-        kz = (int)(v / nt);
-        const int t = (int)(v % nt);
-        const int gsz = kGroupM * g.tiles_n;
-        const int grp = t / gsz, in_g = t % gsz;
-        const int first_m = grp * kGroupM;
-        const int gm = (g.tiles_m - first_m) < kGroupM ? (g.tiles_m - first_m) : kGroupM;
-        tm = first_m + in_g % gm;
-        tn = in_g / gm;
+        int t;
+        if (g.tail_splits > 0 && (int)blockIdx.x >= g.main_blocks)
+        {
+            // tail pieces keep the hardware's round-robin order: they are short and should spread over all XCDs
+            const int u = (int)blockIdx.x - g.main_blocks;
+            const int ti = u / g.tail_splits, piece = u - ti * g.tail_splits;
+            t = g.tail_first + ti;
+            kbeg = (int64_t)piece * g.tail_kps;
+            kend = (kbeg + g.tail_kps < g.K) ? kbeg + g.tail_kps : g.K;
+            tail_out = g.tail_ws + (int64_t)u * (BM * BN);
+        }
+        else
+        {
+            const int64_t total = g.tail_splits > 0 ? (int64_t)g.main_blocks : (int64_t)nt * g.splits;
+            const int64_t bid = blockIdx.x;
+            const int64_t xcd = bid % kXcds, loc = bid / kXcds;
+            const int64_t full = total / kXcds, rem = total % kXcds;
+            const int64_t v = xcd * full + (xcd < rem ? xcd : rem) + loc;
+            kz = (int)(v / nt);
+            t = (int)(v % nt);
+            kbeg = (int64_t)kz * g.k_per_split;
+            kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
+        }
+        tile_coords(t, g.tiles_m, g.tiles_n, tm, tn);
     }
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-    const int64_t kbeg = (int64_t)kz * g.k_per_split;
-    const int64_t kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
     const int nkt = (int)((kend - kbeg + BK - 1) / BK);
 
     float ra[A_PER_T], rb_[B_PER_T];
@@ -466,6 +493,18 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
     }
 
     // ---- epilogue: accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
+    if (tail_out)
+    {
+        // K piece of a tail tile: the whole BM x BN partial, tile-local (rows or columns past the matrix hold zeros)
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int j = 0; j < CB; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    tail_out[(wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4)) * BN + wn + j * 32 + l32] = acc[i][j][r];
+        return;
+    }
     float *Cout = g.C + (int64_t)kz * g.c_split_stride;
 #pragma unroll
     for (int i = 0; i < RB; ++i)
@@ -598,6 +637,105 @@ void launch_splitk_reduce(const float *part, int splits, int64_t stride, float *
                            part, splits, stride, out, M, N, ldc, bias, P);
 }
 
+// Sums the K pieces of each tail tile in piece order and stores the tile through the epilogue the main kernel
+// would have used. One thread per four consecutive columns of a tile row.
+__global__ __launch_bounds__(256) void tail_fixup_kernel(GemmArgs g, int BM, int BN, int epi)
+{
+    const int per_tile = BM * BN / 4;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    const int ti = idx / per_tile, e = idx - ti * per_tile;
+    const int nt = g.tiles_m * g.tiles_n;
+    if (g.tail_first + ti >= nt)
+        return;
+    const int row_l = e / (BN / 4), c4 = e - row_l * (BN / 4);
+    const float *p = g.tail_ws + ((int64_t)ti * g.tail_splits * BM + row_l) * BN + 4 * c4;
+    f32x4 acc = *reinterpret_cast<const f32x4 *>(p);
+    for (int z = 1; z < g.tail_splits; ++z)
+    {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(p + (int64_t)z * BM * BN);
+        acc[0] += v[0], acc[1] += v[1], acc[2] += v[2], acc[3] += v[3];
+    }
+    int tm, tn;
+    tile_coords(g.tail_first + ti, g.tiles_m, g.tiles_n, tm, tn);
+    const int64_t row = (int64_t)tm * BM + row_l;
+    if (row >= g.M)
+        return;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        const int64_t col = (int64_t)tn * BN + 4 * c4 + j;
+        if (col >= g.N)
+            continue;
+        float v = acc[j];
+        if (epi == EPI_NCHW_ROWB)
+        {
+            if (g.bias)
+                v = v + g.bias[row];
+            g.C[((col / g.P) * g.M + row) * g.P + col % g.P] = v;
+        }
+        else
+        {
+            if (epi == EPI_BIAS_COL && g.bias)
+                v = v + g.bias[col];
+            g.C[row * g.ldc + col] = v;
+        }
+    }
+}
+
+// Whether (and how) to split the last tiles: nt tiles over 256 CUs run in ceil(nt/256) rounds, and a last round of
+// only a few tiles leaves most CUs idle for a whole tile's time. Those few tiles are cut into K pieces instead.
+struct TailPlan
+{
+    int tiles = 0, splits = 0;  // tail tiles and K pieces of each (0: no tail split)
+    int64_t kps = 0;
+    size_t bytes = 0;
+};
+
+TailPlan plan_tail(int64_t nt, int64_t K, int BM, int BN)
+{
+    TailPlan p;
+    const int64_t kt = odl::ceil_div(K, 16);
+    const int64_t r = nt % 256;
+    if (nt <= 256 || nt > 256 * 8 || r == 0 || r > 128 || kt < 16)
+        return p;
+    int64_t s = 256 / r;
+    if (s > kt / 2)
+        s = kt / 2;
+    if (s > 32)
+        s = 32;
+    if (s < 2)
+        return p;
+    p.kps = odl::ceil_div(kt, s) * 16;
+    p.splits = (int)odl::ceil_div(K, p.kps);
+    p.tiles = (int)r;
+    p.bytes = (size_t)p.tiles * p.splits * BM * BN * sizeof(float);
+    return p;
+}
+
+// fills the tail fields of g (tiles_m/tiles_n set) when the workspace holds the partials; returns the grid size
+unsigned apply_tail(GemmArgs &g, int BM, int BN, void *tail_ws, size_t tail_bytes)
+{
+    const int64_t nt = (int64_t)g.tiles_m * g.tiles_n;
+    g.main_blocks = 0, g.tail_first = (int)nt, g.tail_splits = 0, g.tail_kps = 0, g.tail_ws = nullptr;
+    if (g.splits != 1 || tail_ws == nullptr || reinterpret_cast<uintptr_t>(tail_ws) % 16 != 0)
+        return (unsigned)(nt * g.splits);
+    const TailPlan p = plan_tail(nt, g.K, BM, BN);
+    if (p.splits == 0 || tail_bytes < p.bytes)
+        return (unsigned)nt;
+    g.tail_first = (int)(nt - p.tiles), g.main_blocks = g.tail_first, g.tail_splits = p.splits, g.tail_kps = p.kps;
+    g.tail_ws = static_cast<float *>(tail_ws);
+    return (unsigned)(g.main_blocks + p.tiles * p.splits);
+}
+
+void launch_tail_fixup(const GemmArgs &g, int BM, int BN, int epi, hipStream_t st)
+{
+    if (g.tail_splits <= 0)
+        return;
+    const int64_t nt = (int64_t)g.tiles_m * g.tiles_n;
+    const int64_t threads = (nt - g.tail_first) * (BM * BN / 4);
+    hipLaunchKernelGGL(tail_fixup_kernel, dim3((unsigned)odl::ceil_div(threads, 256)), dim3(256), 0, st, g, BM, BN, epi);
+}
+
 __global__ void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows, int64_t cols)
 {
     __shared__ float tile[32][33];
@@ -620,17 +758,19 @@ __global__ void transpose_kernel(const float *__restrict__ src, float *__restric
 }
 
 template <int BM, int BN, int BK, int EPI>
-int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g_in, int splits, hipStream_t st)
+int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g_in, int splits, void *tail_ws, size_t tail_bytes,
+                hipStream_t st)
 {
     GemmArgs g = g_in;
     g.splits = splits;
-    dim3 grid((unsigned)((int64_t)g.tiles_m * g.tiles_n * splits));
+    dim3 grid(apply_tail(g, BM, BN, tail_ws, tail_bytes));
     dim3 block(kThreads);
 #define ODL_GEMM_CASE(TA, TB, V)                                                                      \
     if (ta == TA && tb == TB && vec == V)                                                             \
     {                                                                                                 \
         hipLaunchKernelGGL((sgemm_mfma_kernel<BM, BN, BK, TA, TB, V, EPI>), grid, block, 0, st, g,   \
                            ConvSrc{});                                                                \
+        launch_tail_fixup(g, BM, BN, EPI, st);                                                        \
         return ODL_OK;                                                                                \
     }
     ODL_GEMM_CASE(false, false, true)
@@ -673,10 +813,11 @@ int pick_splits(int64_t M, int64_t N, int64_t K, int requested)
 }
 
 template <int EPI>
-int launch_any_tile(int tile, bool ta, bool tb, bool vec, const GemmArgs &g, int splits, hipStream_t st)
+int launch_any_tile(int tile, bool ta, bool tb, bool vec, const GemmArgs &g, int splits, void *tail_ws,
+                    size_t tail_bytes, hipStream_t st)
 {
-    return tile == 128 ? launch_tile<128, 128, kBK, EPI>(ta, tb, vec, g, splits, st)
-                       : launch_tile<64, 64, kBK, EPI>(ta, tb, vec, g, splits, st);
+    return tile == 128 ? launch_tile<128, 128, kBK, EPI>(ta, tb, vec, g, splits, tail_ws, tail_bytes, st)
+                       : launch_tile<64, 64, kBK, EPI>(ta, tb, vec, g, splits, nullptr, 0, st);
 }
 }  // namespace
 
@@ -728,7 +869,7 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
     {
         GemmArgs p = g;
         p.C = static_cast<float *>(workspace), p.ldc = N, p.bias = nullptr, p.c_split_stride = M * N;
-        rc = launch_any_tile<EPI_PLAIN>(tile, trans_a, trans_b, vec, p, splits, st);
+        rc = launch_any_tile<EPI_PLAIN>(tile, trans_a, trans_b, vec, p, splits, nullptr, 0, st);
         if (rc != ODL_OK)
             return fail(rc, "sgemm: no kernel variant");
         ODL_LAUNCH_CHECK();
@@ -738,11 +879,11 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
         return ODL_OK;
     }
     if (epi == EPI_NCHW_ROWB)
-        rc = launch_any_tile<EPI_NCHW_ROWB>(tile, trans_a, trans_b, vec, g, 1, st);
+        rc = launch_any_tile<EPI_NCHW_ROWB>(tile, trans_a, trans_b, vec, g, 1, workspace, workspace_bytes, st);
     else if (epi == EPI_BIAS_COL && bias)
-        rc = launch_any_tile<EPI_BIAS_COL>(tile, trans_a, trans_b, vec, g, 1, st);
+        rc = launch_any_tile<EPI_BIAS_COL>(tile, trans_a, trans_b, vec, g, 1, workspace, workspace_bytes, st);
     else
-        rc = launch_any_tile<EPI_PLAIN>(tile, trans_a, trans_b, vec, g, 1, st);
+        rc = launch_any_tile<EPI_PLAIN>(tile, trans_a, trans_b, vec, g, 1, workspace, workspace_bytes, st);
     if (rc != ODL_OK)
         return fail(rc, "sgemm: no kernel variant");
     ODL_LAUNCH_CHECK();
@@ -753,20 +894,26 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
 // Convolution as implicit GEMM: the same kernel, its B operand gathered from the image / upstream gradient.
 namespace
 {
+bool conv_tile_bm64(int64_t M, int64_t N, int splits)
+{
+    return M <= 64 || odl::ceil_div(M, 128) * odl::ceil_div(N, 128) * splits < 256;
+}
+
 template <int SB, bool TA, int EPI>
-int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, hipStream_t st)
+int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, void *tail_ws, size_t tail_bytes, hipStream_t st)
 {
     const int ck = (cv.KH == 3 && cv.KW == 3) ? 3 : ((cv.KH == 1 && cv.KW == 1) ? 1 : 0);
-    const bool bm64 = g.M <= 64 || odl::ceil_div(g.M, 128) * odl::ceil_div(g.N, 128) * splits < 256;
+    const bool bm64 = conv_tile_bm64(g.M, g.N, splits);
     g.tiles_m = (int)odl::ceil_div(g.M, bm64 ? 64 : 128);
     g.tiles_n = (int)odl::ceil_div(g.N, 128);
     g.splits = splits;
-    const dim3 grid((unsigned)((int64_t)g.tiles_m * g.tiles_n * splits)), block(kThreads);
+    const dim3 grid(apply_tail(g, bm64 ? 64 : 128, 128, tail_ws, tail_bytes)), block(kThreads);
 #define ODL_CONV_CASE(BMV, CKV)                                                                                  \
     if (bm64 == (BMV == 64) && ck == CKV)                                                                        \
     {                                                                                                            \
         hipLaunchKernelGGL((sgemm_mfma_kernel<BMV, 128, 16, TA, false, true, EPI, SB, CKV>), grid, block, 0, st, \
                            g, cv);                                                                               \
+        launch_tail_fixup(g, BMV, 128, EPI, st);                                                                 \
         return ODL_OK;                                                                                           \
     }
     ODL_CONV_CASE(128, 3)
@@ -837,9 +984,21 @@ size_t conv_implicit_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, i
     return s > 1 ? (size_t)s * OC * K * sizeof(float) : 0;
 }
 
-size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW)
+static size_t conv_tail_bytes(int64_t M, int64_t N, int64_t K)
 {
-    return (size_t)C * KH * KW * OC * sizeof(float);
+    const int bm = conv_tile_bm64(M, N, 1) ? 64 : 128;
+    return plan_tail(ceil_div(M, bm) * ceil_div(N, 128), K, bm, 128).bytes;
+}
+
+static size_t dgrad_wp_bytes(int64_t C, int64_t OC, int KH, int KW)
+{
+    return (((size_t)C * KH * KW * OC * sizeof(float)) + 255) & ~(size_t)255;
+}
+
+// permuted weights, then the tail-split partials of the input-grad GEMM [C, pixels, KH*KW*OC]
+size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW, int64_t pixels)
+{
+    return dgrad_wp_bytes(C, OC, KH, KW) + conv_tail_bytes(C, pixels, (int64_t)KH * KW * OC);
 }
 
 static ConvSrc make_src(int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW, int64_t OC, int KH, int KW, int SH,
@@ -867,7 +1026,7 @@ size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t OC, int KH,
 {
     const int64_t K = C * KH * KW, M = N * OH * OW;
     const int s = forward_splits(OC, M, K);
-    return s > 1 ? (size_t)s * OC * M * sizeof(float) : 0;
+    return s > 1 ? (size_t)s * OC * M * sizeof(float) : conv_tail_bytes(OC, M, K);
 }
 
 // y[n][oc][p] = sum_k W2d[oc][k] * x_gathered[(n,p)][k] + b[oc]
@@ -891,7 +1050,7 @@ int conv_implicit_forward(const float *x, const float *w, const float *b, float 
         g.k_per_split = ceil_div(ceil_div(g.K, kBK), splits) * kBK;
         splits = (int)ceil_div(g.K, g.k_per_split);
         g.C = static_cast<float *>(workspace), g.bias = nullptr, g.ldc = g.N, g.c_split_stride = OC * g.N;
-        rc = launch_conv_tile<SB_CONV_FWD, false, EPI_PLAIN>(g, cv, splits, st);
+        rc = launch_conv_tile<SB_CONV_FWD, false, EPI_PLAIN>(g, cv, splits, nullptr, 0, st);
         if (rc != ODL_OK)
             return fail(rc, "conv2d: no kernel variant");
         ODL_LAUNCH_CHECK();
@@ -899,7 +1058,7 @@ int conv_implicit_forward(const float *x, const float *w, const float *b, float 
         ODL_LAUNCH_CHECK();
         return ODL_OK;
     }
-    rc = launch_conv_tile<SB_CONV_FWD, false, EPI_NCHW_ROWB>(g, cv, 1, st);
+    rc = launch_conv_tile<SB_CONV_FWD, false, EPI_NCHW_ROWB>(g, cv, 1, workspace, workspace_bytes, st);
     if (rc != ODL_OK)
         return fail(rc, "conv2d: no kernel variant");
     ODL_LAUNCH_CHECK();
@@ -926,7 +1085,7 @@ int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, i
     g.ldc = K;
     g.c_split_stride = splits > 1 ? OC * K : 0;
     int rc = launch_conv_tile<SB_CONV_WGRAD, true, EPI_PLAIN>(g, make_src(C, H, W, OH, OW, OC, KH, KW, SH, SW, PH, PW),
-                                                              splits, st);
+                                                              splits, nullptr, 0, st);
     if (rc != ODL_OK)
         return fail(rc, "conv2d_backward: no kernel variant");
     ODL_LAUNCH_CHECK();
@@ -943,7 +1102,7 @@ int conv_implicit_dgrad(const float *gy, const float *w, float *gx, int64_t N, i
                         int64_t OC, int KH, int KW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
                         size_t workspace_bytes, hipStream_t st)
 {
-    const size_t need = conv_implicit_dgrad_workspace(C, OC, KH, KW);
+    const size_t need = dgrad_wp_bytes(C, OC, KH, KW);  // the tail partials behind it are optional
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need, "conv2d_backward: workspace of %zu bytes required",
                 need);
     float *wp = static_cast<float *>(workspace);
@@ -957,7 +1116,8 @@ int conv_implicit_dgrad(const float *gy, const float *w, float *gx, int64_t N, i
     g.lda = g.K, g.ldb = 0, g.ldc = 0, g.P = H * W;
     g.k_per_split = g.K, g.c_split_stride = 0;
     int rc = launch_conv_tile<SB_CONV_DGRAD, false, EPI_NCHW_ROWB>(g, make_src(C, H, W, OH, OW, OC, KH, KW, 1, 1, PH, PW),
-                                                                   1, st);
+                                                                   1, static_cast<char *>(workspace) + need,
+                                                                   workspace_bytes - need, st);
     if (rc != ODL_OK)
         return fail(rc, "conv2d_backward: no kernel variant");
     ODL_LAUNCH_CHECK();
@@ -967,7 +1127,9 @@ int conv_implicit_dgrad(const float *gy, const float *w, float *gx, int64_t N, i
 size_t sgemm_workspace(int64_t M, int64_t N, int64_t K, int split_k)
 {
     const int s = pick_splits(M, N, K, split_k);
-    return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+    if (s > 1)
+        return (size_t)s * M * N * sizeof(float);
+    return pick_tile(M, N) == 128 ? plan_tail(ceil_div(M, 128) * ceil_div(N, 128), K, 128, 128).bytes : 0;
 }
 }  // namespace odl
 
