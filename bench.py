@@ -74,11 +74,38 @@ def cpu_baseline_gemm(size, budget_s=18.0):
 
 
 def extras(torch, capi, steps, warmup):
+    """The other hot kernels at the benchmark's shapes. Outputs and workspaces are allocated once and every timed
+    call is one direct C-ABI call with prebuilt arguments, so that microsecond-scale kernels are not timed through
+    Python allocation and argument checking."""
+    import ctypes
+    from origindl_amd import _lib
     out = {}
     g = torch.Generator(device="cuda").manual_seed(0)
+    L = _lib.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    keep = []  # tensors behind the raw pointers
 
     def rnd(*shape):
         return torch.randn(shape, device="cuda", generator=g)
+
+    def ptr(t):
+        keep.append(t)
+        return ctypes.c_void_p(t.data_ptr())
+
+    def empty(*shape):
+        return torch.empty(shape, dtype=torch.float32, device="cuda")
+
+    def ws(nbytes):
+        nbytes = int(nbytes)
+        if nbytes == 0:
+            return None, 0
+        t = torch.empty((nbytes + 3) // 4, dtype=torch.int32, device="cuda")
+        return ptr(t), nbytes
+
+    def direct(name, *args):
+        fn = getattr(L.cdll, name)
+        L.check(fn(*args))  # argument errors surface here, once
+        return lambda: fn(*args)
 
     # conv2d forward + weight-grad + input-grad at BASELINE's C1 and C2
     for name, (N, C, H, OC, s, p) in {"conv_c1": (32, 64, 56, 128, 1, 1), "conv_c2": (32, 128, 28, 256, 2, 1)}.items():
@@ -86,33 +113,46 @@ def extras(torch, capi, steps, warmup):
         OH = (H + 2 * p - 3) // s + 1
         gy = rnd(N, OC, OH, OH)
         M, K = N * OH * OH, C * 9
-        ms_f = time_region(torch, lambda: capi.conv2d(x, w, b, s, p), steps, warmup)
-        ms_b = time_region(torch, lambda: capi.conv2d_backward(gy, x, w, True, s, p), steps, warmup)
+        geom = (N, C, H, H, OC, 3, 3, s, s, p, p)
+        y, gx, gw, gb = empty(N, OC, OH, OH), empty(N, C, H, H), empty(OC, C, 3, 3), empty(OC)
+        wf, nf = ws(L.query("odl_hip_conv2d_workspace_bytes", *geom))
+        wb, nbb = ws(L.query("odl_hip_conv2d_backward_workspace_bytes", *geom))
+        fwd = direct("odl_hip_conv2d", ptr(x), ptr(w), ptr(b), *geom, ptr(y), wf, nf, stream)
+        bwd = direct("odl_hip_conv2d_backward", ptr(gy), ptr(x), ptr(w), *geom, ptr(gx), ptr(gw), ptr(gb), wb, nbb,
+                     stream)
+        ms_f = time_region(torch, fwd, steps, warmup)
+        ms_b = time_region(torch, bwd, steps, warmup)
         flop = 6.0 * M * K * OC
         tf = flop / (ms_f + ms_b) / 1e9
         out[name] = {"fwd_ms": ms_f, "bwd_ms": ms_b, "tflops": tf, "frac_mfma_peak": tf / PEAK_FP32_MFMA_TFLOPS,
                      "flop": flop}
-        ms_i = time_region(torch, lambda: capi.im2col(x, 3, s, p, True), steps, warmup)
-        col = capi.im2col(x, 3, s, p, True)
-        ms_c = time_region(torch, lambda: capi.col2im(col, x.shape, 3, s, p, True), steps, warmup)
+        col, img = empty(M, K), empty(N, C, H, H)
+        ig = (N, C, H, H, 3, 3, s, s, p, p, 1)
+        ms_i = time_region(torch, direct("odl_hip_im2col", ptr(x), *ig, ptr(col), stream), steps, warmup)
+        ms_c = time_region(torch, direct("odl_hip_col2im", ptr(col), *ig, ptr(img), stream), steps, warmup)
         nbytes = 4.0 * (x.numel() + M * K)
         out[name + "_im2col"] = {"ms": ms_i, "gbs": nbytes / ms_i / 1e6, "frac_hbm": nbytes / ms_i / 1e6 / PEAK_HBM_GBS}
         out[name + "_col2im"] = {"ms": ms_c, "gbs": nbytes / ms_c / 1e6, "frac_hbm": nbytes / ms_c / 1e6 / PEAK_HBM_GBS}
-        ms_gb = time_region(torch, lambda: capi.sum_nchw_channels(gy), steps, warmup)
+        wr, nr = ws(L.query("odl_hip_sum_nchw_channels_workspace_bytes", N, OC, OH * OH))
+        ms_gb = time_region(torch, direct("odl_hip_sum_nchw_channels", ptr(gy), N, OC, OH * OH, ptr(gb), wr, nr, stream),
+                            steps, warmup)
         nb = 4.0 * (gy.numel() + OC)
         out[name + "_bias_grad"] = {"ms": ms_gb, "gbs": nb / ms_gb / 1e6, "frac_hbm": nb / ms_gb / 1e6 / PEAK_HBM_GBS}
-        del x, w, b, gy, col
+        del x, w, b, gy, col, img, y, gx, gw
+        keep.clear()
     # gradient reductions: the MLP's own shapes (launch-bound) and scaled shapes that can saturate HBM
-    for name, shape, target in (("bias_grad_512x1000", (512, 1000), (1, 1000)),
-                                ("bias_grad_16384x4096_scaled", (16384, 4096), (1, 4096))):
-        x = rnd(*shape)
-        ms = time_region(torch, lambda: capi.sum_to(x, target), steps, warmup)
-        nb = 4.0 * (x.numel() + target[1])
+    for name, shape in (("bias_grad_512x1000", (512, 1000)), ("bias_grad_16384x4096_scaled", (16384, 4096))):
+        x, o = rnd(*shape), empty(1, shape[1])
+        ss, ts = (ctypes.c_int64 * 2)(*shape), (ctypes.c_int64 * 2)(1, shape[1])
+        wr, nr = ws(L.query("odl_hip_sum_to_workspace_bytes", ss, 2, ts, 2))
+        ms = time_region(torch, direct("odl_hip_sum_to", ptr(x), ss, 2, ts, 2, ptr(o), wr, nr, stream), steps, warmup)
+        nb = 4.0 * (x.numel() + shape[1])
         out[name] = {"ms": ms, "gbs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
     for name, (N, C) in (("softmax_ce_grad_512x10", (512, 10)), ("softmax_ce_grad_16384x1000_scaled", (16384, 1000))):
-        x = rnd(N, C)
+        x, gx = rnd(N, C), empty(N, C)
         t = torch.randint(0, C, (N,), device="cuda", generator=g)
-        ms = time_region(torch, lambda: capi.softmax_cross_entropy_backward(x, t, 1.0), steps, warmup)
+        ms = time_region(torch, direct("odl_hip_softmax_ce_grad", ptr(x), ptr(t), 1, N, C, ctypes.c_float(1.0), ptr(gx),
+                                       stream), steps, warmup)
         nb = 8.0 * N * C + 8.0 * N
         out[name] = {"ms": ms, "gbs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
     # the MLP's six GEMMs (config 1): 512x784x1000 and 512x1000x10, forward + backward
