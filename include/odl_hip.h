@@ -178,6 +178,15 @@ int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t n
 int odl_hip_unary(int op, const float *a, int64_t n, float *out, void *stream);
 /* origin::cuda::pow with a float32 scalar exponent (src/mat/origin/cpu/math/pow.cpp:35-43) */
 int odl_hip_pow_scalar(const float *a, int64_t n, float exponent, float *out, void *stream);
+/* Fused optimizer steps. The reference has no Mat virtual for them: Adam::step_one (src/optim/adam.cpp:52-113) and
+ * SGD::step_one (src/optim/sgd.cpp:18-75) issue the same arithmetic as ~15 whole-tensor Mat operations per parameter.
+ * Each element goes through the identical sequence of separately rounded float operations
+ * (m = m*b1 + g*(1-b1); v = v*b2 + (g*g)*(1-b2); p_out = p - ((m*m_hat_scale) / (powf(v*v_hat_scale, 0.5) + eps))*lr),
+ * with m_hat_scale = 1/(1-b1^t) and v_hat_scale = 1/(1-b2^t) computed by the caller in float as the reference does.
+ * m and v are updated in place; p_out may be p. sgd_step: p_out = p - g*lr (no momentum, no weight decay). */
+int odl_hip_adam_step(const float *p, const float *g, float *m, float *v, int64_t n, float beta1, float beta2,
+                      float m_hat_scale, float v_hat_scale, float eps, float lr, float *p_out, void *stream);
+int odl_hip_sgd_step(const float *p, const float *g, int64_t n, float lr, float *p_out, void *stream);
 /* origin::cuda::{zeros,ones,full} (cuda/factory.cuh:23-50) */
 int odl_hip_fill(float *dst, int64_t n, float value, void *stream);
 

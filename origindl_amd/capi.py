@@ -433,6 +433,28 @@ def pow_scalar(a, e):
     return out
 
 
+def adam_step(p, g, m, v, t, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8):
+    """One fused Adam step (src/optim/adam.cpp:52-113): returns the new parameter, updates m and v in place.
+    The bias-correction scales are computed in float32 on the host exactly as the reference computes them."""
+    for name, x in (("p", p), ("g", g), ("m", m), ("v", v)):
+        _chk(x, name)
+    f = np.float32
+    b1p, b2p = f(np.power(f(beta1), f(t))), f(np.power(f(beta2), f(t)))
+    s1, s2 = f(1.0) / (f(1.0) - b1p), f(1.0) / (f(1.0) - b2p)
+    out = _empty(p.shape)
+    lib().call("odl_hip_adam_step", _p(p), _p(g), _p(m), _p(v), p.numel(), float(f(beta1)), float(f(beta2)), float(s1),
+               float(s2), float(f(eps)), float(f(lr)), _p(out), _stream())
+    return out
+
+
+def sgd_step(p, g, lr):
+    """p - g*lr in one launch (src/optim/sgd.cpp:18-75 without momentum or weight decay)."""
+    _chk(p, "p"), _chk(g, "g")
+    out = _empty(p.shape)
+    lib().call("odl_hip_sgd_step", _p(p), _p(g), p.numel(), float(np.float32(lr)), _p(out), _stream())
+    return out
+
+
 def fill(shape, value):
     out = _empty(shape)
     lib().call("odl_hip_fill", _p(out), out.numel(), ctypes.c_float(value), _stream())

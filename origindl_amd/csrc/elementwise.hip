@@ -113,6 +113,69 @@ __global__ void pow_kernel(const float *a, float *out, int64_t n, float e)
         out[i] = powf(a[i], e);
 }
 
+// One Adam step per element, as the same sequence of separately rounded float operations that the reference's
+// optimizer issues as whole-tensor ops (src/optim/adam.cpp:52-113): this file is compiled without contraction,
+// so m*b1 + g*(1-b1) is two products and a sum, and the square root is powf(v_hat, 0.5f) as there.
+struct AdamScalars
+{
+    float beta1, one_minus_beta1, beta2, one_minus_beta2, m_hat_scale, v_hat_scale, eps, lr;
+    float root;  // 0.5, passed at run time so that the call stays the powf the unfused pow kernel makes
+};
+
+__device__ inline void adam_one(float p, float g, float &m, float &v, float &p_out, const AdamScalars &a)
+{
+    const float mn = m * a.beta1 + g * a.one_minus_beta1;
+    const float gg = g * g;
+    const float vn = v * a.beta2 + gg * a.one_minus_beta2;
+    const float m_hat = mn * a.m_hat_scale;
+    const float v_hat = vn * a.v_hat_scale;
+    const float denom = powf(v_hat, a.root) + a.eps;
+    const float update = m_hat / denom;
+    p_out = p - update * a.lr;
+    m = mn, v = vn;
+}
+
+template <bool VEC>
+__global__ void adam_step_kernel(const float *p, const float *g, float *m, float *v, float *p_out, int64_t n, AdamScalars a)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (VEC)
+    {
+        const int64_t i = 4 * t;
+        if (i + 3 < n)
+        {
+            f32x4 pv = *reinterpret_cast<const f32x4 *>(p + i), gv = *reinterpret_cast<const f32x4 *>(g + i);
+            f32x4 mv = *reinterpret_cast<f32x4 *>(m + i), vv = *reinterpret_cast<f32x4 *>(v + i), ov;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                float mj = mv[j], vj = vv[j], oj;
+                adam_one(pv[j], gv[j], mj, vj, oj, a);
+                mv[j] = mj, vv[j] = vj, ov[j] = oj;
+            }
+            *reinterpret_cast<f32x4 *>(m + i) = mv;
+            *reinterpret_cast<f32x4 *>(v + i) = vv;
+            *reinterpret_cast<f32x4 *>(p_out + i) = ov;
+        }
+        else
+            for (int64_t k = i; k < n; ++k)
+                adam_one(p[k], g[k], m[k], v[k], p_out[k], a);
+    }
+    else if (t < n)
+        adam_one(p[t], g[t], m[t], v[t], p_out[t], a);
+}
+
+// p_out = p - g * lr, two separately rounded steps (src/optim/sgd.cpp:18-75 without momentum or weight decay)
+__global__ void sgd_step_kernel(const float *p, const float *g, float *p_out, int64_t n, float lr)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+    {
+        const float step = g[i] * lr;
+        p_out[i] = p[i] - step;
+    }
+}
+
 __global__ void fill_kernel(float *dst, int64_t n, float v)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -242,6 +305,40 @@ int odl_hip_pow_scalar(const float *a, int64_t n, float exponent, float *out, vo
         return ODL_OK;
     hipLaunchKernelGGL(pow_kernel, dim3((unsigned)odl::ceil_div(n, kBlock)), dim3(kBlock), 0, odl::as_stream(stream), a,
                        out, n, exponent);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_adam_step(const float *p, const float *g, float *m, float *v, int64_t n, float beta1, float beta2,
+                      float m_hat_scale, float v_hat_scale, float eps, float lr, float *p_out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(n >= 0, "adam_step: negative size");
+    if (n == 0)
+        return ODL_OK;
+    ODL_REQUIRE(p && g && m && v && p_out, "adam_step: null operand");
+    const AdamScalars a{beta1, 1.0f - beta1, beta2, 1.0f - beta2, m_hat_scale, v_hat_scale, eps, lr, 0.5f};
+    auto aligned = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+    hipStream_t st = odl::as_stream(stream);
+    if (aligned(p) && aligned(g) && aligned(m) && aligned(v) && aligned(p_out))
+        hipLaunchKernelGGL((adam_step_kernel<true>), dim3((unsigned)odl::ceil_div(odl::ceil_div(n, 4), kBlock)),
+                           dim3(kBlock), 0, st, p, g, m, v, p_out, n, a);
+    else
+        hipLaunchKernelGGL((adam_step_kernel<false>), dim3((unsigned)odl::ceil_div(n, kBlock)), dim3(kBlock), 0, st, p, g,
+                           m, v, p_out, n, a);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_sgd_step(const float *p, const float *g, int64_t n, float lr, float *p_out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(n >= 0, "sgd_step: negative size");
+    if (n == 0)
+        return ODL_OK;
+    ODL_REQUIRE(p && g && p_out, "sgd_step: null operand");
+    hipLaunchKernelGGL(sgd_step_kernel, dim3((unsigned)odl::ceil_div(n, kBlock)), dim3(kBlock), 0, odl::as_stream(stream),
+                       p, g, p_out, n, lr);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

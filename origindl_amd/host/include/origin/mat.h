@@ -196,6 +196,14 @@ public:
     std::unique_ptr<Mat> softmax(int axis) const;
     float softmax_cross_entropy(const Mat &target) const;                      // loss value (host)
     std::unique_ptr<Mat> softmax_cross_entropy_backward(const Mat &target, float gy) const;
+    // fused optimizer steps (one launch each; same per-element arithmetic as the op-by-op sequences of
+    // src/optim/adam.cpp:52-113 and src/optim/sgd.cpp:18-75). m and v are updated in place.
+    std::unique_ptr<Mat> adam_step(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, float m_hat_scale,
+                                   float v_hat_scale, float eps, float lr) const;
+    std::unique_ptr<Mat> sgd_step(const Mat &grad, float lr) const;
+    // {gy . w^T, x^T . gy} for 2-D operands, reading w and x in place (no transposed copies)
+    static std::pair<std::unique_ptr<Mat>, std::unique_ptr<Mat>> matmul_backward_2d(const Mat &x, const Mat &w,
+                                                                                   const Mat &gy);
     float accuracy(const Mat &target_int32) const;
 
     // ---- OriginMat-only helpers used by callers (origin_mat.h:442-559 in the reference)

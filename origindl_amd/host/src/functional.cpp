@@ -198,9 +198,14 @@ struct MatMul : Operator  // src/operators/math/mat_mul.cpp:12-182
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
-        // gx = gy . w^T, gw = x^T . gy; the transposes are Mat::transpose() as in the reference — on this backend
-        // a caller that wants to skip the two copies uses odl_hip_matmul_backward (NT / TN GEMMs) directly
+        // gx = gy . w^T, gw = x^T . gy. The reference copies both transposes first (mat_mul.cpp:171-174); for 2-D
+        // operands this backend's GEMM reads w and x in place instead — the same products, two copies fewer.
         const Mat &x = mat(inputs_[0]), &w = mat(inputs_[1]), &gy = mat(gys[0]);
+        if (x.shape().size() == 2 && w.shape().size() == 2 && gy.shape().size() == 2)
+        {
+            auto g = OriginMat::matmul_backward_2d(x, w, gy);
+            return {wrap(std::move(g.first)), wrap(std::move(g.second))};
+        }
         auto wT = w.transpose();
         auto xT = x.transpose();
         return {wrap(gy.matmul(*wT)), wrap(xT->matmul(gy))};

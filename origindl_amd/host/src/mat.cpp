@@ -830,6 +830,49 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_backward(const Mat &target
     return gx;
 }
 
+std::unique_ptr<Mat> OriginMat::adam_step(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, float m_hat_scale,
+                                          float v_hat_scale, float eps, float lr) const
+{
+    const OriginMat &p = dev_f32(*this, "adam_step");
+    const OriginMat &g = dev_f32(grad, "adam_step");
+    const OriginMat &mm = dev_f32(m, "adam_step");
+    const OriginMat &vv = dev_f32(v, "adam_step");
+    if (g.elements() != elements() || mm.elements() != elements() || vv.elements() != elements())
+        THROW_INVALID_ARG("adam_step: parameter, gradient and moment sizes differ");
+    auto out = new_like(p, shape_);
+    check(odl_hip_adam_step(fp(p), fp(g), const_cast<float *>(fp(mm)), const_cast<float *>(fp(vv)), (int64_t)elements(),
+                            beta1, beta2, m_hat_scale, v_hat_scale, eps, lr, out->data_ptr<float>(), nullptr));
+    return out;
+}
+
+std::unique_ptr<Mat> OriginMat::sgd_step(const Mat &grad, float lr) const
+{
+    const OriginMat &p = dev_f32(*this, "sgd_step");
+    const OriginMat &g = dev_f32(grad, "sgd_step");
+    if (g.elements() != elements())
+        THROW_INVALID_ARG("sgd_step: parameter and gradient sizes differ");
+    auto out = new_like(p, shape_);
+    check(odl_hip_sgd_step(fp(p), fp(g), (int64_t)elements(), lr, out->data_ptr<float>(), nullptr));
+    return out;
+}
+
+std::pair<std::unique_ptr<Mat>, std::unique_ptr<Mat>> OriginMat::matmul_backward_2d(const Mat &x_, const Mat &w_,
+                                                                                    const Mat &gy_)
+{
+    const OriginMat &x = dev_f32(x_, "matmul"), &w = dev_f32(w_, "matmul"), &gy = dev_f32(gy_, "matmul");
+    const Shape xs = x.shape(), ws_ = w.shape(), gs = gy.shape();
+    if (xs.size() != 2 || ws_.size() != 2 || gs.size() != 2 || xs[1] != ws_[0] || gs[0] != xs[0] || gs[1] != ws_[1])
+        THROW_INVALID_ARG("matmul backward: shapes {} {} {} do not form x[M,K] w[K,N] gy[M,N]", xs.to_string(),
+                          ws_.to_string(), gs.to_string());
+    const int64_t M = xs[0], K = xs[1], N = ws_[1];
+    auto gx = new_like(x, xs);
+    auto gw = new_like(w, ws_);
+    Workspace ws(odl_hip_matmul_backward_workspace_bytes(M, K, N), x.device().index());
+    check(odl_hip_matmul_backward(fp(x), fp(w), fp(gy), gx->data_ptr<float>(), gw->data_ptr<float>(), M, K, N, ws.ptr(),
+                                  ws.bytes, nullptr));
+    return {std::move(gx), std::move(gw)};
+}
+
 float OriginMat::accuracy(const Mat &target_int32) const
 {
     const OriginMat &y = dev_f32(*this, "accuracy");

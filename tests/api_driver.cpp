@@ -532,8 +532,14 @@ void timed_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T, int s
     const auto t0 = std::chrono::steady_clock::now();
     for (int i = 0; i < steps; ++i)
         *loss = one();
-    // the parameters of the last step are still in flight: reading one back drains the queue
-    float sink = model.parameters()[0]->template to_vector<float>()[0];
+    // the parameters of the last step are still in flight: reading the smallest one back drains the queue
+    // (a large one would add its own copy time to the steps)
+    auto params = model.parameters();
+    auto *smallest = params[0];
+    for (auto *p : params)
+        if (p->shape().elements() < smallest->shape().elements())
+            smallest = p;
+    float sink = smallest->template to_vector<float>()[0];
     (void)sink;
     const auto t1 = std::chrono::steady_clock::now();
     *ms = std::chrono::duration<float, std::milli>(t1 - t0).count() / (float)(steps > 0 ? steps : 1);

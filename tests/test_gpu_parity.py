@@ -561,3 +561,50 @@ def test_elementwise_vs_oracle_and_fixtures(api, o):
     api.binary("add", acc, dev(big), out=acc)  # add_inplace: output aliases an input
     assert np.array_equal(host(acc), big + big)
     assert bool((api.fill((3, 5), 2.5) == 2.5).all())
+
+
+def test_fused_optimizer_steps_match_the_op_by_op_sequence(api, o):
+    """odl_hip_adam_step / odl_hip_sgd_step against (1) the same arithmetic issued as separate whole-tensor ops, the
+    way the reference's optimizers issue it (src/optim/adam.cpp:52-113, sgd.cpp:18-75) — bit-identical — and
+    (2) the oracle's elementwise ops on the CPU (powf of glibc vs the device: a few ulp on the denominator)."""
+    rng = np.random.default_rng(23)
+    n = 100003  # not a multiple of four: the scalar tail runs too
+    p, g = rng.standard_normal(n, dtype=f32), rng.standard_normal(n, dtype=f32) * f32(0.1)
+    m, v = rng.standard_normal(n, dtype=f32) * f32(0.05), np.abs(rng.standard_normal(n, dtype=f32)) * f32(0.01)
+    b1, b2, eps, lr = f32(0.9), f32(0.999), f32(1e-8), f32(1e-3)
+    for t in (1, 7):
+        s1 = f32(1.0) / (f32(1.0) - f32(np.power(b1, f32(t))))
+        s2 = f32(1.0) / (f32(1.0) - f32(np.power(b2, f32(t))))
+        sc = lambda x: dev(np.array([x], f32))  # noqa: E731
+        dp, dg, dm, dv = dev(p), dev(g), dev(m), dev(v)
+        # separate ops
+        m2 = api.binary("add", api.binary("mul", dm, sc(b1)), api.binary("mul", dg, sc(f32(1.0) - b1)))
+        v2 = api.binary("add", api.binary("mul", dv, sc(b2)),
+                        api.binary("mul", api.binary("mul", dg, dg), sc(f32(1.0) - b2)))
+        den = api.binary("add", api.pow_scalar(api.binary("mul", v2, sc(s2)), 0.5), sc(eps))
+        p2 = api.binary("sub", dp, api.binary("mul", api.binary("div", api.binary("mul", m2, sc(s1)), den), sc(lr)))
+        # fused
+        fm, fv = dev(m), dev(v)
+        fp_ = api.adam_step(dp, dg, fm, fv, t, lr=lr, beta1=b1, beta2=b2, eps=eps)
+        assert np.array_equal(host(fm), host(m2)) and np.array_equal(host(fv), host(v2))
+        assert np.array_equal(host(fp_), host(p2))
+        # CPU: the oracle's elementwise ops chained the same way
+        def cpu(op, a, b):
+            a, b = np.atleast_1d(np.asarray(a, f32)), np.atleast_1d(np.asarray(b, f32))
+            out = np.empty(max(a.size, b.size), f32)
+            assert o.orc_binary(op, a, a.size, b, b.size, out) == 0
+            return out
+        cm = cpu(0, cpu(2, m, b1), cpu(2, g, f32(1.0) - b1))
+        cv = cpu(0, cpu(2, v, b2), cpu(2, cpu(2, g, g), f32(1.0) - b2))
+        assert np.array_equal(host(fm), cm) and np.array_equal(host(fv), cv)
+        cden = np.empty(n, f32)
+        o.orc_pow_scalar(cpu(2, cv, s2), n, f32(0.5), cden)
+        cp = cpu(1, p, cpu(2, cpu(3, cpu(2, cm, s1), cpu(0, cden, eps)), lr))
+        np.testing.assert_allclose(host(fp_), cp, rtol=0, atol=1e-6)  # an ulp of p (|p| < 8) around a step of ~1e-3
+    assert np.array_equal(host(api.sgd_step(dev(p), dev(g), 0.05)), p - g * f32(0.05))
+    big = rng.standard_normal(4096, dtype=f32)
+    dm0, dv0 = dev(np.zeros(4096, f32)), dev(np.zeros(4096, f32))
+    out = host(api.adam_step(dev(big), dev(big), dm0, dv0, 1))
+    # closed form at t = 1 from zero moments: m_hat = g and v_hat = g^2, so the step is lr * g / (|g| + eps)
+    b64 = big.astype(np.float64)
+    np.testing.assert_allclose(out, b64 - 1e-3 * b64 / (np.abs(b64) + 1e-8), rtol=0, atol=3e-7)
