@@ -196,6 +196,14 @@ public:
     std::unique_ptr<Mat> softmax(int axis) const;
     float softmax_cross_entropy(const Mat &target) const;                      // loss value (host)
     std::unique_ptr<Mat> softmax_cross_entropy_backward(const Mat &target, float gy) const;
+    // Max pooling with the window-local indices kept in device memory (uint64 per output). The Mat interface above
+    // hands them to the caller as a host vector, which costs a device-to-host copy in forward and a host-to-device
+    // copy in backward (the reference's device backend pays both); the pooling operator uses this pair instead.
+    std::unique_ptr<Mat> max_pool2d_device(std::pair<int, int> kernel_size, std::pair<int, int> stride,
+                                           std::pair<int, int> pad, std::shared_ptr<Storage> *indices) const;
+    std::unique_ptr<Mat> max_pool2d_backward_device(const Mat &gy, std::pair<int, int> kernel_size,
+                                                    std::pair<int, int> stride, std::pair<int, int> pad,
+                                                    const Storage &indices) const;
     // fused optimizer steps (one launch each; same per-element arithmetic as the op-by-op sequences of
     // src/optim/adam.cpp:52-113 and src/optim/sgd.cpp:18-75). m and v are updated in place.
     std::unique_ptr<Mat> adam_step(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, float m_hat_scale,

@@ -335,17 +335,24 @@ struct Conv2dOp : Operator  // src/operators/conv/conv2d.cpp:14-89
 struct MaxPool2d : Operator  // src/operators/pooling/max_pool2d.cpp:14-86
 {
     std::pair<int, int> k, s, p;
-    std::vector<size_t> indices;
+    std::shared_ptr<Storage> indices;  // window-local argmax per output, uint64, kept on the device
     MaxPool2d(std::pair<int, int> kk, std::pair<int, int> ss, std::pair<int, int> pp) : k(kk), s(ss), p(pp) {}
+    static const OriginMat &origin(const Mat &m)
+    {
+        const auto *o = dynamic_cast<const OriginMat *>(&m);
+        if (!o)
+            THROW_RUNTIME_ERROR("MaxPool2d: expected an OriginMat, got backend_type={}", m.backend_type());
+        return *o;
+    }
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
-        return {wrap(mat(xs[0]).max_pool2d(k, s, p, xs[0].requires_grad() ? &indices : nullptr))};
+        return {wrap(origin(mat(xs[0])).max_pool2d_device(k, s, p, xs[0].requires_grad() ? &indices : nullptr))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
-        if (indices.empty())
+        if (!indices)
             THROW_RUNTIME_ERROR("MaxPool2d backward: indices not found. This should not happen when requires_grad=true");
-        return {wrap(mat(inputs_[0]).max_pool2d_backward(mat(gys[0]), k, s, p, indices))};
+        return {wrap(origin(mat(inputs_[0])).max_pool2d_backward_device(mat(gys[0]), k, s, p, *indices))};
     }
 };
 

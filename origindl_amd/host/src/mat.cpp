@@ -713,8 +713,8 @@ std::vector<std::unique_ptr<Mat>> OriginMat::conv2d_backward(const Mat &gym, con
     return grads;
 }
 
-std::unique_ptr<Mat> OriginMat::max_pool2d(std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
-                                           std::vector<size_t> *indices) const
+std::unique_ptr<Mat> OriginMat::max_pool2d_device(std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
+                                                  std::shared_ptr<Storage> *indices) const
 {
     const OriginMat &x = dev_f32(*this, "max_pool2d");
     if (shape_.size() != 4)
@@ -725,38 +725,57 @@ std::unique_ptr<Mat> OriginMat::max_pool2d(std::pair<int, int> k, std::pair<int,
     if (OH <= 0 || OW <= 0)
         THROW_INVALID_ARG("max_pool2d: invalid output size OH={}, OW={} for input H={}, W={}", OH, OW, H, W);
     auto y = new_like(x, Shape{(size_t)N, (size_t)C, (size_t)OH, (size_t)OW});
-    const size_t n = y->elements();
     std::shared_ptr<Storage> idx;
     if (indices)
-        idx = Storage::create(n * sizeof(uint64_t), DeviceType::kCUDA, device().index());
+        idx = Storage::create(y->elements() * sizeof(uint64_t), DeviceType::kCUDA, device().index());
     check(odl_hip_max_pool2d(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second,
                              y->data_ptr<float>(), idx ? static_cast<uint64_t *>(idx->data()) : nullptr, nullptr));
+    if (indices)
+        *indices = idx;
+    return y;
+}
+
+std::unique_ptr<Mat> OriginMat::max_pool2d(std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
+                                           std::vector<size_t> *indices) const
+{
+    std::shared_ptr<Storage> idx;
+    auto y = max_pool2d_device(k, s, p, indices ? &idx : nullptr);
     if (indices)
     {
         // the interface hands the window-local indices to the caller as a host vector (mat.h:560-566)
         static_assert(sizeof(size_t) == sizeof(uint64_t), "size_t must be 64-bit");
-        indices->resize(n);
-        check(odl_hip_memcpy_d2h(indices->data(), idx->data(), n * sizeof(uint64_t)));
+        indices->resize(y->elements());
+        check(odl_hip_memcpy_d2h(indices->data(), idx->data(), y->elements() * sizeof(uint64_t)));
     }
     return y;
+}
+
+std::unique_ptr<Mat> OriginMat::max_pool2d_backward_device(const Mat &gym, std::pair<int, int> k, std::pair<int, int> s,
+                                                           std::pair<int, int> p, const Storage &indices) const
+{
+    const OriginMat &gy = dev_f32(gym, "max_pool2d_backward");
+    if (gy.shape().size() != 4)
+        THROW_INVALID_ARG("max_pool2d_backward: gy must be 4D (N, C, OH, OW), but got shape {}", gy.shape().to_string());
+    if (indices.size() < gy.elements() * sizeof(uint64_t) || indices.device_type() != DeviceType::kCUDA)
+        THROW_INVALID_ARG("max_pool2d_backward: indices size mismatch. Expected {}, got {}", gy.elements(),
+                          indices.size() / sizeof(uint64_t));
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
+    auto gx = new_like(gy, shape_);
+    check(odl_hip_max_pool2d_backward(fp(gy), static_cast<const uint64_t *>(indices.data()), N, C, H, W, k.first, k.second,
+                                      s.first, s.second, p.first, p.second, gx->data_ptr<float>(), nullptr));
+    return gx;
 }
 
 std::unique_ptr<Mat> OriginMat::max_pool2d_backward(const Mat &gym, std::pair<int, int> k, std::pair<int, int> s,
                                                     std::pair<int, int> p, const std::vector<size_t> &indices) const
 {
     const OriginMat &gy = dev_f32(gym, "max_pool2d_backward");
-    if (gy.shape().size() != 4)
-        THROW_INVALID_ARG("max_pool2d_backward: gy must be 4D (N, C, OH, OW), but got shape {}", gy.shape().to_string());
     if (indices.size() != gy.elements())
         THROW_INVALID_ARG("max_pool2d_backward: indices size mismatch. Expected {}, got {}", gy.elements(),
                           indices.size());
-    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
     auto idx = Storage::create(indices.size() * sizeof(uint64_t), DeviceType::kCUDA, gy.device().index());
     check(odl_hip_memcpy_h2d(idx->data(), indices.data(), indices.size() * sizeof(uint64_t)));
-    auto gx = new_like(gy, shape_);
-    check(odl_hip_max_pool2d_backward(fp(gy), static_cast<const uint64_t *>(idx->data()), N, C, H, W, k.first, k.second,
-                                      s.first, s.second, p.first, p.second, gx->data_ptr<float>(), nullptr));
-    return gx;
+    return max_pool2d_backward_device(gym, k, s, p, *idx);
 }
 
 // -------------------------------------------------------------------------------------------- indexing
