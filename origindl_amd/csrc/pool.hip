@@ -81,6 +81,123 @@ __global__ void max_pool_bwd_kernel(const float *__restrict__ gy, const uint64_t
     gx[t] = acc;
 }
 
+// The same two kernels with 32-bit index arithmetic and (for the usual windows)
+// kernel size and stride fixed at compile time: on a 64-wide wave the 64-bit divisions and modulos of the general
+// kernels above cost several times the memory traffic they serve.
+template <int CK, int CS>
+__global__ __launch_bounds__(256) void max_pool_fwd_plane_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                 uint64_t *__restrict__ idx, PoolGeom g)
+{
+    const int KH = CK > 0 ? CK : g.KH, KW = CK > 0 ? CK : g.KW;
+    const int SH = CS > 0 ? CS : g.SH, SW = CS > 0 ? CS : g.SW;
+    const int H = (int)g.H, W = (int)g.W, OW = (int)g.OW;
+    const unsigned plane = (unsigned)(g.OH * g.OW);
+    const unsigned t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= (unsigned)(g.N * g.C) * plane)
+        return;
+    const unsigned nc = t / plane, r = t - nc * plane;
+    const int oh = (int)(r / (unsigned)OW), ow = (int)r - oh * OW;
+    const int h0 = oh * SH - g.PH, w0 = ow * SW - g.PW;
+    {
+        const float *p = x + (int64_t)nc * H * W;
+        float mv = 0.f;
+        int mi = 0;
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh)
+        {
+            const int h = h0 + kh;
+#pragma unroll
+            for (int kw = 0; kw < KW; ++kw)
+            {
+                const int w = w0 + kw;
+                const float v = ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) ? p[h * W + w] : 0.f;
+                if ((kh | kw) == 0)
+                    mv = v;  // max_pool2d.cpp:110-113
+                else if (v > mv)
+                {
+                    mv = v;
+                    mi = kh * KW + kw;
+                }
+            }
+        }
+        y[t] = mv;
+        if (idx)
+            idx[t] = (uint64_t)mi;
+    }
+}
+
+template <int CK, int CS>
+__global__ __launch_bounds__(256) void max_pool_bwd_plane_kernel(const float *__restrict__ gy,
+                                                                 const uint64_t *__restrict__ idx,
+                                                                 float *__restrict__ gx, PoolGeom g)
+{
+    const int KH = CK > 0 ? CK : g.KH, KW = CK > 0 ? CK : g.KW;
+    const int SH = CS > 0 ? CS : g.SH, SW = CS > 0 ? CS : g.SW;
+    const int W = (int)g.W, OH = (int)g.OH, OW = (int)g.OW;
+    const unsigned plane = (unsigned)(g.H * g.W);
+    const int oplane = OH * OW;
+    const unsigned t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= (unsigned)(g.N * g.C) * plane)
+        return;
+    const unsigned nc = t / plane, r = t - nc * plane;
+    const int h = (int)(r / (unsigned)W), w = (int)r - h * W;
+    {
+        const float *gp = gy + (int64_t)nc * oplane;
+        const uint64_t *ip = idx + (int64_t)nc * oplane;
+        float acc = 0.f;
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh)
+        {
+            const int hp = h + g.PH - kh;
+            const int oh = hp / SH;
+            const bool hok = hp >= 0 && hp % SH == 0 && oh < OH;
+#pragma unroll
+            for (int kw = 0; kw < KW; ++kw)
+            {
+                const int wp = w + g.PW - kw;
+                const int ow = wp / SW;
+                if (hok && wp >= 0 && wp % SW == 0 && ow < OW)
+                {
+                    const int o = oh * OW + ow;
+                    // the reference decodes the index with int arithmetic (max_pool2d.cpp:203-205)
+                    if ((int)ip[o] == kh * KW + kw)
+                        acc += gp[o];
+                }
+            }
+        }
+        gx[t] = acc;
+    }
+}
+
+// the 32-bit kernels take everything whose element counts fit
+bool plane_ok(const PoolGeom &g)
+{
+    return g.N * g.C * g.H * g.W < (1ll << 31) - 256 && g.N * g.C * g.OH * g.OW < (1ll << 31) - 256 &&
+           (int64_t)g.KH * g.KW < (1 << 20);
+}
+
+dim3 plane_grid(int64_t plane, int64_t ncount)
+{
+    return dim3((unsigned)odl::ceil_div(plane * ncount, 256));
+}
+
+// CASE(kernel, stride) for the windows the networks on this path use; anything else runs with run-time sizes
+#define ODL_POOL_DISPATCH(KERNEL, ...)                                               \
+    do                                                                               \
+    {                                                                                \
+        const bool sq = g.KH == g.KW && g.SH == g.SW;                                \
+        if (sq && g.KH == 2 && g.SH == 2)                                            \
+            hipLaunchKernelGGL((KERNEL<2, 2>), grid, dim3(256), 0, st, __VA_ARGS__); \
+        else if (sq && g.KH == 3 && g.SH == 2)                                       \
+            hipLaunchKernelGGL((KERNEL<3, 2>), grid, dim3(256), 0, st, __VA_ARGS__); \
+        else if (sq && g.KH == 3 && g.SH == 1)                                       \
+            hipLaunchKernelGGL((KERNEL<3, 1>), grid, dim3(256), 0, st, __VA_ARGS__); \
+        else if (sq && g.KH == 5 && g.SH == 1)                                       \
+            hipLaunchKernelGGL((KERNEL<5, 1>), grid, dim3(256), 0, st, __VA_ARGS__); \
+        else                                                                         \
+            hipLaunchKernelGGL((KERNEL<0, 0>), grid, dim3(256), 0, st, __VA_ARGS__); \
+    } while (0)
+
 int make_geom(PoolGeom &g, const char *who, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
               int PH, int PW)
 {
@@ -107,8 +224,15 @@ int odl_hip_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t 
     const int64_t total = N * C * g.OH * g.OW;
     if (total == 0)
         return ODL_OK;
-    hipLaunchKernelGGL(max_pool_fwd_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0,
-                       odl::as_stream(stream), x, y, idx, g);
+    hipStream_t st = odl::as_stream(stream);
+    if (plane_ok(g))
+    {
+        const dim3 grid = plane_grid(g.OH * g.OW, N * C);
+        ODL_POOL_DISPATCH(max_pool_fwd_plane_kernel, x, y, idx, g);
+    }
+    else
+        hipLaunchKernelGGL(max_pool_fwd_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, x, y, idx,
+                           g);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
@@ -125,8 +249,15 @@ int odl_hip_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N,
     const int64_t total = N * C * H * W;
     if (total == 0)
         return ODL_OK;
-    hipLaunchKernelGGL(max_pool_bwd_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0,
-                       odl::as_stream(stream), gy, idx, gx, g);
+    hipStream_t st = odl::as_stream(stream);
+    if (plane_ok(g))
+    {
+        const dim3 grid = plane_grid(H * W, N * C);
+        ODL_POOL_DISPATCH(max_pool_bwd_plane_kernel, gy, idx, gx, g);
+    }
+    else
+        hipLaunchKernelGGL(max_pool_bwd_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, gy, idx, gx,
+                           g);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
