@@ -197,9 +197,10 @@ def train_steps(steps, warmup, with_cpu):
     return out
 
 
-# HBM-side bytes of one 4096^3 sgemm_mfma_kernel launch: FETCH_SIZE (scaled 2.000x by the calibration copy) 720.2 MiB
-# + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc` runs of `--pmc-probe` summarised under profiles/.
-GEMM_4096_TRAFFIC_BYTES = int((720.2 + 64.0) * 1024 * 1024)
+# HBM-side bytes of one 4096^3 sgemm_mfma_kernel launch: FETCH_SIZE (scaled 2.000x by the calibration copy) 805.2 MiB on
+# average over the NN / NT / TN variants (734 / 983 / 699) + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc`
+# runs of `--pmc-probe` summarised under profiles/.
+GEMM_4096_TRAFFIC_BYTES = int((805.2 + 64.0) * 1024 * 1024)
 
 
 def pmc_probe(torch, capi, gemm_step):
@@ -219,6 +220,10 @@ def pmc_probe(torch, capi, gemm_step):
     for _ in range(2):
         capi.conv2d(x, w, b, 1, 1)
         capi.conv2d_backward(gy, x, w, True, 1, 1)
+    for _ in range(2):
+        col = capi.im2col(x, 3, 1, 1, True)
+        capi.col2im(col, x.shape, 3, 1, 1, True)
+    del col
     big = torch.randn((16384, 4096), device="cuda", generator=g)
     logits = torch.randn((16384, 1000), device="cuda", generator=g)
     t = torch.randint(0, 1000, (16384,), device="cuda", generator=g)
