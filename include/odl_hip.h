@@ -174,10 +174,30 @@ size_t odl_hip_accuracy_workspace_bytes(int64_t N);
  * 4 greater-than mask (1.0f / 0.0f). na == nb, or one side has a single element; anything else is the
  * reference's "complex broadcasting" runtime_error. out may alias a or b (add_inplace). */
 int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t nb, float *out, void *stream);
-/* origin::cuda::{relu,exp,log,negate,square,sqrt}: op 0 relu, 1 exp, 2 log, 3 neg, 4 square, 5 sqrt */
+/* origin::cuda::{relu,exp,log,negate,square,sqrt,sigmoid,silu}: op 0 relu, 1 exp, 2 log, 3 neg, 4 square, 5 sqrt,
+ * 6 sigmoid = 1/(1+exp(-x)) (operation_templates.h:168-175), 7 silu = x*sigmoid(x) (src/mat/origin/cpu/activation/silu.cpp:49-56) */
 int odl_hip_unary(int op, const float *a, int64_t n, float *out, void *stream);
 /* origin::cuda::pow with a float32 scalar exponent (src/mat/origin/cpu/math/pow.cpp:35-43) */
 int odl_hip_pow_scalar(const float *a, int64_t n, float exponent, float *out, void *stream);
+/* ------------------------------------------------------------------ detector forward path ------------ */
+/* Mat::upsample, mode "nearest" (mat.h:770; src/mat/origin/cpu/nn/upsample.cpp:22-75):
+ * y[n,c,oh,ow] = x[n,c,oh/scale_h,ow/scale_w]. Unlike the reference, an output that would index past x is refused. */
+int odl_hip_upsample_nearest(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
+                             int scale_h, int scale_w, float *y, void *stream);
+/* Mat::cat (mat.h:797; src/mat/origin/cpu/shape/cat.cpp:20-140): inputs viewed as [outer, axis_size_i, inner] are laid
+ * side by side along the axis. host_inputs: `count` device pointers in a host array; host_axis_sizes: their axis extents. */
+int odl_hip_cat(const float *const *host_inputs, const int64_t *host_axis_sizes, int count, int64_t outer, int64_t inner,
+                float *out, void *stream);
+/* Mat::yolo_detect_forward (mat.h:719; src/mat/origin/cpu/custom/yolo_detect.cpp:28-166): 1x1 convolution
+ * [A*(classes+5), C] (+bias), view [N,A,classes+5,H,W] -> [N, A*H*W, classes+5], sigmoid, xy = (2s+grid)*stride,
+ * wh = (2s)^2*anchor. grid / anchor_grid are read with the reference's flat indexing ([A,H,W,2] and
+ * [A,anchor_H,anchor_W,2]); entries past grid_elems / anchor_elems count as 0 / 1 as there. */
+int odl_hip_yolo_detect_forward(const float *x, const float *conv_w, const float *conv_b, const float *grid,
+                                int64_t grid_elems, const float *anchor_grid, int64_t anchor_elems, int64_t anchor_H,
+                                int64_t anchor_W, int64_t N, int64_t C, int64_t H, int64_t W, float stride, int num_anchors,
+                                int num_classes, float *out, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_yolo_detect_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int num_anchors, int num_classes);
+
 /* Fused optimizer steps. The reference has no Mat virtual for them: Adam::step_one (src/optim/adam.cpp:52-113) and
  * SGD::step_one (src/optim/sgd.cpp:18-75) issue the same arithmetic as ~15 whole-tensor Mat operations per parameter.
  * Each element goes through the identical sequence of separately rounded float operations

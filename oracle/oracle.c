@@ -578,7 +578,14 @@ void orc_unary(int op, const float *a, int64_t n, float *out)
             case 2: out[i] = logf(v); break;             /* math/log.cpp */
             case 3: out[i] = -v; break;                  /* math/negate.cpp */
             case 4: out[i] = v * v; break;               /* math/square.cpp */
-            default: out[i] = sqrtf(v); break;           /* math/sqrt.cpp */
+            case 5: out[i] = sqrtf(v); break;            /* math/sqrt.cpp */
+            case 6: out[i] = 1.0f / (1.0f + expf(-v)); break; /* device_common/operation_templates.h:168-175 */
+            default: /* activation/silu.cpp:49-56 */
+            {
+                const float sg = 1.0f / (1.0f + expf(-v));
+                out[i] = v * sg;
+                break;
+            }
         }
     }
 }
@@ -588,6 +595,89 @@ void orc_pow_scalar(const float *a, int64_t n, float e, float *out)
 {
     for (int64_t i = 0; i < n; ++i)
         out[i] = powf(a[i], e);
+}
+
+/* ========================================================================== detector forward path */
+
+/* nn/upsample.cpp:22-75: nearest neighbour, ih = oh / scale_h, iw = ow / scale_w */
+int orc_upsample_nearest(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW, int scale_h,
+                         int scale_w, float *y)
+{
+    if (scale_h <= 0 || scale_w <= 0 || (OH - 1) / scale_h >= H || (OW - 1) / scale_w >= W)
+        return ORC_ERR_INVALID_ARG;
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < C; ++c)
+            for (int64_t oh = 0; oh < OH; ++oh)
+                for (int64_t ow = 0; ow < OW; ++ow)
+                    y[((n * C + c) * OH + oh) * OW + ow] = x[((n * C + c) * H + oh / scale_h) * W + ow / scale_w];
+    return ORC_OK;
+}
+
+/* shape/cat.cpp:20-140: every input viewed as [M, C_i, N]; chunk m of input i lands at out[m][off_i .. off_i + C_i) */
+int orc_cat(const float *const *inputs, const int64_t *axis_sizes, int count, int64_t outer, int64_t inner, float *out)
+{
+    int64_t total = 0, off = 0;
+    if (count < 1)
+        return ORC_ERR_RUNTIME;
+    for (int i = 0; i < count; ++i)
+        total += axis_sizes[i];
+    for (int i = 0; i < count; ++i)
+    {
+        const int64_t chunk = axis_sizes[i] * inner;
+        for (int64_t m = 0; m < outer; ++m)
+            memcpy(out + m * total * inner + off * inner, inputs[i] + m * chunk, sizeof(float) * (size_t)chunk);
+        off += axis_sizes[i];
+    }
+    return ORC_OK;
+}
+
+/* custom/yolo_detect.cpp:28-166. conv 1x1 (conv2d.cpp:404-512 through orc_conv2d), reshape [N,A,CI,H,W], permute to
+ * [N,A,H,W,CI], sigmoid as -x, exp, 1 + ., 1 / ., then xy = (2s + grid) * stride, wh = pow(2s, 2) * anchor. */
+int orc_yolo_detect_forward(const float *x, const float *conv_w, const float *conv_b, const float *grid, int64_t grid_elems,
+                            const float *anchor_grid, int64_t anchor_elems, int64_t anchor_H, int64_t anchor_W, int64_t N,
+                            int64_t C, int64_t H, int64_t W, float stride, int num_anchors, int num_classes, float *out)
+{
+    const int64_t CI = num_classes + 5, A = num_anchors, OC = A * CI, HW = H * W;
+    float *conv = (float *)malloc(sizeof(float) * (size_t)(N * OC * HW > 0 ? N * OC * HW : 1));
+    int rc = orc_conv2d(x, conv_w, conv_b, N, C, H, W, OC, 1, 1, 1, 1, 0, 0, conv);
+    if (rc != ORC_OK)
+    {
+        free(conv);
+        return rc;
+    }
+    for (int64_t b = 0; b < N; ++b)
+        for (int64_t i = 0; i < A * HW; ++i)
+        {
+            const int64_t a = i / HW, sp = i % HW, h = sp / W, w = sp % W;
+            float *o = out + (b * A * HW + i) * CI;
+            for (int64_t c = 0; c < CI; ++c)
+            {
+                const float v = conv[((b * A + a) * CI + c) * HW + sp];
+                const float e = expf(-v);
+                const float d = 1.0f + e;
+                o[c] = 1.0f / d;
+            }
+            {
+                const int64_t gb = a * HW * 2 + h * W * 2 + w * 2;
+                const float gx = gb < grid_elems ? grid[gb] : 0.0f, gy = gb + 1 < grid_elems ? grid[gb + 1] : 0.0f;
+                const int64_t sh = (anchor_H > 0 && H > anchor_H) ? H / anchor_H : 1;
+                const int64_t sw = (anchor_W > 0 && W > anchor_W) ? W / anchor_W : 1;
+                int64_t ah = h / sh, aw = w / sw;
+                if (ah > anchor_H - 1) ah = anchor_H - 1;
+                if (aw > anchor_W - 1) aw = anchor_W - 1;
+                const int64_t ab = a * anchor_H * anchor_W * 2 + ah * anchor_W * 2 + aw * 2;
+                const float anw = ab < anchor_elems ? anchor_grid[ab] : 1.0f;
+                const float anh = ab + 1 < anchor_elems ? anchor_grid[ab + 1] : 1.0f;
+                const float s0 = o[0], s1 = o[1], s2 = o[2], s3 = o[3];
+                float t;
+                t = s0 * 2.0f; t = t + gx; o[0] = t * stride;
+                t = s1 * 2.0f; t = t + gy; o[1] = t * stride;
+                o[2] = powf(s2 * 2.0f, 2.0f) * anw;
+                o[3] = powf(s3 * 2.0f, 2.0f) * anh;
+            }
+        }
+    free(conv);
+    return ORC_OK;
 }
 
 /* ========================================================================== training steps */

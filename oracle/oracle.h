@@ -112,6 +112,14 @@ int orc_binary(int op, const float *a, int64_t na, const float *b, int64_t nb, f
 void orc_unary(int op, const float *a, int64_t n, float *out);
 void orc_pow_scalar(const float *a, int64_t n, float e, float *out);
 
+/* detector forward path: nn/upsample.cpp:22-75, shape/cat.cpp:20-140, custom/yolo_detect.cpp:28-166 */
+int orc_upsample_nearest(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW, int scale_h,
+                         int scale_w, float *y);
+int orc_cat(const float *const *inputs, const int64_t *axis_sizes, int count, int64_t outer, int64_t inner, float *out);
+int orc_yolo_detect_forward(const float *x, const float *conv_w, const float *conv_b, const float *grid, int64_t grid_elems,
+                            const float *anchor_grid, int64_t anchor_elems, int64_t anchor_H, int64_t anchor_W, int64_t N,
+                            int64_t C, int64_t H, int64_t W, float stride, int num_anchors, int num_classes, float *out);
+
 /* ---- whole training steps (compositions restated from the reference's operators/optimizers) --------- */
 /* MLP: x[N,D] -> Linear(D,Hd)+ReLU -> Linear(Hd,C) -> softmax CE; backward; WeightDecay hook (grad += wd*p,
  * include/origin/optim/hooks.h:40-65); Adam step t (src/optim/adam.cpp:19-114). Parameters and Adam

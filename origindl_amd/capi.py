@@ -408,7 +408,7 @@ def accuracy(y, t):
 
 # -------------------------------------------------------------------------------------- elementwise
 _BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "gt": 4}
-_UN = {"relu": 0, "exp": 1, "log": 2, "neg": 3, "square": 4, "sqrt": 5}
+_UN = {"relu": 0, "exp": 1, "log": 2, "neg": 3, "square": 4, "sqrt": 5, "sigmoid": 6, "silu": 7}
 
 
 def binary(op, a, b, out=None):
@@ -430,6 +430,56 @@ def pow_scalar(a, e):
     _chk(a, "a")
     out = _empty(a.shape)
     lib().call("odl_hip_pow_scalar", _p(a), a.numel(), ctypes.c_float(e), _p(out), _stream())
+    return out
+
+
+def upsample(x, scale):
+    """Mat::upsample, nearest (src/mat/origin/cpu/nn/upsample.cpp:22-75): output is (H*scale_h, W*scale_w)."""
+    _chk(x, "x")
+    if x.dim() != 4:
+        raise OdlInvalidArgument("Upsample: input must be 4D (N, C, H, W)")
+    sh, sw = _pair(scale)
+    N, C, H, W = x.shape
+    y = _empty((N, C, H * sh, W * sw))
+    lib().call("odl_hip_upsample_nearest", _p(x), N, C, H, W, H * sh, W * sw, sh, sw, _p(y), _stream())
+    return y
+
+
+def cat(xs, dim=0):
+    """Mat::cat (src/mat/origin/cpu/shape/cat.cpp:20-140)."""
+    if len(xs) < 1:
+        raise OdlRuntimeError("cat: requires at least 1 input")
+    for x in xs:
+        _chk(x, "input")
+        if x.dim() != xs[0].dim():
+            raise OdlRuntimeError("cat: all inputs must have same number of dimensions")
+        for d in range(x.dim()):
+            if d != dim and x.shape[d] != xs[0].shape[d]:
+                raise OdlRuntimeError("cat: dimension %d mismatch: %d vs %d" % (d, x.shape[d], xs[0].shape[d]))
+    shape = list(xs[0].shape)
+    shape[dim] = _builtins.sum(int(x.shape[dim]) for x in xs)
+    outer, _, inner = _split_axis(shape, dim)
+    out = _empty(shape)
+    ptrs = (ctypes.c_void_p * len(xs))(*[x.data_ptr() for x in xs])
+    sizes = (ctypes.c_int64 * len(xs))(*[int(x.shape[dim]) for x in xs])
+    lib().call("odl_hip_cat", ptrs, sizes, len(xs), outer, inner, _p(out), _stream())
+    return out
+
+
+def yolo_detect_forward(x, conv_w, conv_b, grid, anchor_grid, stride, num_anchors, num_classes):
+    """Mat::yolo_detect_forward (src/mat/origin/cpu/custom/yolo_detect.cpp:28-166) -> [N, A*H*W, classes+5]."""
+    for name, t in (("x", x), ("conv_weight", conv_w), ("grid", grid), ("anchor_grid", anchor_grid)):
+        _chk(t, name)
+    if x.dim() != 4:
+        raise OdlInvalidArgument("yolo_detect_forward: input must be 4D (N, C, H, W)")
+    N, C, H, W = x.shape
+    aH = anchor_grid.shape[2] if anchor_grid.dim() >= 3 else H
+    aW = anchor_grid.shape[3] if anchor_grid.dim() >= 4 else W
+    out = _empty((N, H * W * num_anchors, num_classes + 5))
+    ws, nb = _ws(lib().query("odl_hip_yolo_detect_workspace_bytes", N, C, H, W, num_anchors, num_classes))
+    lib().call("odl_hip_yolo_detect_forward", _p(x), _p(conv_w), _p(conv_b), _p(grid), grid.numel(), _p(anchor_grid),
+               anchor_grid.numel(), aH, aW, N, C, H, W, float(stride), num_anchors, num_classes, _p(out), _p(ws), nb,
+               _stream())
     return out
 
 

@@ -1,0 +1,233 @@
+// Forward-only operators of the detector path: nearest-neighbour upsampling, concatenation, and the YOLO detect
+// head (1x1 convolution, then sigmoid and box decoding in one pass over the convolution's output).
+//   upsample  src/mat/origin/cpu/nn/upsample.cpp:22-75        y[n,c,oh,ow] = x[n,c,oh/scale_h,ow/scale_w]
+//   cat       src/mat/origin/cpu/shape/cat.cpp:20-140         [M, C_i, N] blocks copied side by side along C
+//   detect    src/mat/origin/cpu/custom/yolo_detect.cpp:28-166
+// All three are streams over HBM; index arithmetic is 32-bit where the sizes allow.
+#include "odl_common.h"
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+extern "C" int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                              int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *y, void *workspace,
+                              size_t workspace_bytes, void *stream);
+extern "C" size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                                                 int SH, int SW, int PH, int PW);
+
+namespace
+{
+constexpr int kBlock = 256;
+
+// one thread per output pixel; consecutive threads along ow
+__global__ __launch_bounds__(kBlock) void upsample_nearest_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                  unsigned planes, int H, int W, int OH, int OW, int sh,
+                                                                  int sw)
+{
+    const unsigned oplane = (unsigned)(OH * OW);
+    const unsigned t = blockIdx.x * (unsigned)kBlock + threadIdx.x;
+    if (t >= planes * oplane)
+        return;
+    const unsigned nc = t / oplane, r = t - nc * oplane;
+    const int oh = (int)(r / (unsigned)OW), ow = (int)r - oh * OW;
+    y[t] = x[(int64_t)nc * H * W + (oh / sh) * W + ow / sw];
+}
+
+// dst[m][off + j] = src[m][j] for j < chunk: `outer` contiguous runs; grid (run pieces, m)
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void cat_copy_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                          int64_t chunk, int64_t dst_stride, int64_t dst_off)
+{
+    const int64_t m = blockIdx.y;
+    const float *s = src + m * chunk;
+    float *d = dst + m * dst_stride + dst_off;
+    const int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * (VEC ? 4 : 1);
+    if (VEC)
+    {
+        if (i + 3 < chunk)
+            *reinterpret_cast<f32x4 *>(d + i) = *reinterpret_cast<const f32x4 *>(s + i);
+        else
+            for (int64_t k = i; k < chunk; ++k)
+                d[k] = s[k];
+    }
+    else if (i < chunk)
+        d[i] = s[i];
+}
+
+// conv[b][a*CI + c][h][w] -> out[b][(a*H + h)*W + w][c], sigmoid, then the box transform on c = 0..3.
+// A workgroup turns a tile of 64 spatial positions x CI channels through LDS: reads run along w, writes along c.
+struct DetectGeom
+{
+    int A, CI, H, W;
+    int anchor_H, anchor_W;
+    int64_t grid_elems, anchor_elems;
+    float stride;
+};
+
+__global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__restrict__ conv, const float *__restrict__ grid,
+                                                             const float *__restrict__ anchor_grid,
+                                                             float *__restrict__ out, DetectGeom g, int ptiles)
+{
+    extern __shared__ float sh_det[];  // [64][CI | 1]
+    const int LS = g.CI | 1;
+    const int HW = g.H * g.W;
+    unsigned vb = blockIdx.x;
+    const int pt = (int)(vb % (unsigned)ptiles);
+    vb /= (unsigned)ptiles;
+    const int a = (int)(vb % (unsigned)g.A);
+    const int b = (int)(vb / (unsigned)g.A);
+    const int p0 = pt * 64;
+    const int np = (HW - p0 < 64) ? HW - p0 : 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float *src = conv + ((int64_t)(b * g.A + a) * g.CI) * HW + p0;
+    for (int c = wave; c < g.CI; c += kBlock / 64)
+        if (lane < np)
+        {
+            const float v = src[(int64_t)c * HW + lane];
+            sh_det[lane * LS + c] = 1.0f / (1.0f + expf(-v));  // the reference's -x, exp, 1 + ., 1 / . steps
+        }
+    __syncthreads();
+    float *dst = out + ((int64_t)(b * g.A + a) * HW + p0) * g.CI;
+    for (int e = threadIdx.x; e < np * g.CI; e += kBlock)
+    {
+        const int pl = e / g.CI, c = e - pl * g.CI;
+        float v = sh_det[pl * LS + c];
+        if (c < 4)
+        {
+            const int p = p0 + pl;
+            const int h = p / g.W, w = p - h * g.W;
+            if (c < 2)
+            {
+                const int64_t gi = ((int64_t)a * HW + (int64_t)h * g.W + w) * 2 + c;
+                const float gv = gi < g.grid_elems ? grid[gi] : 0.0f;
+                const float t = v * 2.0f;
+                v = (t + gv) * g.stride;
+            }
+            else
+            {
+                const int sh_ = (g.anchor_H > 0 && g.H > g.anchor_H) ? g.H / g.anchor_H : 1;
+                const int sw_ = (g.anchor_W > 0 && g.W > g.anchor_W) ? g.W / g.anchor_W : 1;
+                int ah = h / sh_, aw = w / sw_;
+                ah = ah < g.anchor_H - 1 ? ah : g.anchor_H - 1;
+                aw = aw < g.anchor_W - 1 ? aw : g.anchor_W - 1;
+                const int64_t ai = ((int64_t)a * g.anchor_H * g.anchor_W + (int64_t)ah * g.anchor_W + aw) * 2 + (c - 2);
+                const float av = ai < g.anchor_elems ? anchor_grid[ai] : 1.0f;
+                const float t = v * 2.0f;
+                v = (t * t) * av;  // pow(2s, 2) * anchor
+            }
+        }
+        dst[e] = v;
+    }
+}
+}  // namespace
+
+extern "C" {
+
+int odl_hip_upsample_nearest(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
+                             int scale_h, int scale_w, float *y, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C >= 0 && H > 0 && W > 0 && OH > 0 && OW > 0, "upsample: bad shape");
+    ODL_REQUIRE(scale_h > 0 && scale_w > 0, "upsample: scale must be positive");
+    // the reference indexes x[oh/scale_h][ow/scale_w] without a bound; here the source pixel must exist
+    ODL_REQUIRE((OH - 1) / scale_h < H && (OW - 1) / scale_w < W,
+                "upsample: output (%lld,%lld) reaches past input (%lld,%lld) at scale (%d,%d)", (long long)OH,
+                (long long)OW, (long long)H, (long long)W, scale_h, scale_w);
+    const int64_t total = N * C * OH * OW;
+    if (total == 0)
+        return ODL_OK;
+    ODL_REQUIRE(total < (1ll << 32) - kBlock && H * W < (1ll << 31) && OH * OW < (1ll << 31), "upsample: too large");
+    hipLaunchKernelGGL(upsample_nearest_kernel, dim3((unsigned)odl::ceil_div(total, kBlock)), dim3(kBlock), 0,
+                       odl::as_stream(stream), x, y, (unsigned)(N * C), (int)H, (int)W, (int)OH, (int)OW, scale_h,
+                       scale_w);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_cat(const float *const *host_inputs, const int64_t *host_axis_sizes, int count, int64_t outer, int64_t inner,
+                float *out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(count >= 1, "cat: requires at least 1 input");
+    ODL_REQUIRE(host_inputs && host_axis_sizes && out, "cat: null argument");
+    ODL_REQUIRE(outer >= 0 && inner >= 0 && outer < 65536 * 32768ll, "cat: bad outer/inner extents");
+    int64_t total_axis = 0;
+    for (int i = 0; i < count; ++i)
+    {
+        ODL_REQUIRE(host_axis_sizes[i] >= 0, "cat: negative axis size");
+        total_axis += host_axis_sizes[i];
+    }
+    hipStream_t st = odl::as_stream(stream);
+    int64_t off = 0;
+    for (int i = 0; i < count; ++i)
+    {
+        const int64_t chunk = host_axis_sizes[i] * inner;
+        if (chunk > 0 && outer > 0)
+        {
+            ODL_REQUIRE(host_inputs[i] != nullptr, "cat: input %d is null", i);
+            const int64_t dst_stride = total_axis * inner, dst_off = off * inner;
+            const bool vec = chunk % 4 == 0 && dst_stride % 4 == 0 && dst_off % 4 == 0 &&
+                             reinterpret_cast<uintptr_t>(host_inputs[i]) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+            // grid.y carries the outer index in slabs of at most 65535
+            for (int64_t m0 = 0; m0 < outer; m0 += 65535)
+            {
+                const int64_t ms = outer - m0 < 65535 ? outer - m0 : 65535;
+                const float *s = host_inputs[i] + m0 * chunk;
+                float *d = out + m0 * dst_stride;
+                if (vec)
+                    hipLaunchKernelGGL((cat_copy_kernel<true>), dim3((unsigned)odl::ceil_div(chunk / 4, kBlock), (unsigned)ms),
+                                       dim3(kBlock), 0, st, s, d, chunk, dst_stride, dst_off);
+                else
+                    hipLaunchKernelGGL((cat_copy_kernel<false>), dim3((unsigned)odl::ceil_div(chunk, kBlock), (unsigned)ms),
+                                       dim3(kBlock), 0, st, s, d, chunk, dst_stride, dst_off);
+                ODL_LAUNCH_CHECK();
+            }
+        }
+        off += host_axis_sizes[i];
+    }
+    return ODL_OK;
+}
+
+size_t odl_hip_yolo_detect_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int num_anchors, int num_classes)
+{
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || num_anchors <= 0 || num_classes < 0)
+        return 0;
+    const int64_t OC = (int64_t)num_anchors * (num_classes + 5);
+    const size_t conv_out = ((size_t)(N * OC * H * W) * sizeof(float) + 255) & ~(size_t)255;
+    return conv_out + odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, 1, 1, 1, 1, 0, 0);
+}
+
+int odl_hip_yolo_detect_forward(const float *x, const float *conv_w, const float *conv_b, const float *grid,
+                                int64_t grid_elems, const float *anchor_grid, int64_t anchor_elems, int64_t anchor_H,
+                                int64_t anchor_W, int64_t N, int64_t C, int64_t H, int64_t W, float stride, int num_anchors,
+                                int num_classes, float *out, void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C > 0 && H > 0 && W > 0, "yolo_detect_forward: input must be 4D (N, C, H, W)");
+    ODL_REQUIRE(num_anchors > 0 && num_classes >= 0, "yolo_detect_forward: bad anchor/class counts");
+    ODL_REQUIRE(x && conv_w && grid && anchor_grid && out, "yolo_detect_forward: null operand");
+    ODL_REQUIRE(grid_elems >= 0 && anchor_elems >= 0 && anchor_H > 0 && anchor_W > 0, "yolo_detect_forward: bad grid sizes");
+    if (N == 0)
+        return ODL_OK;
+    const int CI = num_classes + 5;
+    const int64_t OC = (int64_t)num_anchors * CI;
+    ODL_REQUIRE(N * num_anchors * odl::ceil_div(H * W, 64) < (1ll << 31) && H * W < (1ll << 30) && CI < 8192,
+                "yolo_detect_forward: too large");
+    const size_t conv_bytes = ((size_t)(N * OC * H * W) * sizeof(float) + 255) & ~(size_t)255;
+    const size_t need = odl_hip_yolo_detect_workspace_bytes(N, C, H, W, num_anchors, num_classes);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need, "yolo_detect_forward: workspace of %zu bytes required, got %zu",
+                need, workspace_bytes);
+    float *conv = static_cast<float *>(workspace);
+    int rc = odl_hip_conv2d(x, conv_w, conv_b, N, C, H, W, OC, 1, 1, 1, 1, 0, 0, conv, static_cast<char *>(workspace) + conv_bytes,
+                            workspace_bytes - conv_bytes, stream);
+    if (rc != ODL_OK)
+        return rc;
+    const int ptiles = (int)odl::ceil_div(H * W, 64);
+    const DetectGeom g{num_anchors, CI, (int)H, (int)W, (int)anchor_H, (int)anchor_W, grid_elems, anchor_elems, stride};
+    const size_t lds = (size_t)64 * (CI | 1) * sizeof(float);
+    hipLaunchKernelGGL(yolo_decode_kernel, dim3((unsigned)(N * num_anchors * ptiles)), dim3(kBlock), lds,
+                       odl::as_stream(stream), conv, grid, anchor_grid, out, g, ptiles);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+}  // extern "C"

@@ -28,7 +28,10 @@ __device__ inline float un(float v)
     if (OP == 2) return logf(v);
     if (OP == 3) return -v;
     if (OP == 4) return v * v;
-    return sqrtf(v);
+    if (OP == 5) return sqrtf(v);
+    // sigmoid as 1/(1+exp(-x)) (operation_templates.h:168-175) and silu as x times that (cpu/activation/silu.cpp:49-56)
+    const float s = 1.0f / (1.0f + expf(-v));
+    return OP == 6 ? s : v * s;
 }
 
 // MODE 0: a[i] op b[i]; 1: a[i] op b[0]; 2: a[0] op b[i]. Each thread handles 4 consecutive elements.
@@ -270,7 +273,7 @@ int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t n
 int odl_hip_unary(int op, const float *a, int64_t n, float *out, void *stream)
 {
     ODL_REQUIRE_DEVICE();
-    ODL_REQUIRE(op >= 0 && op <= 5, "unary: unknown op %d", op);
+    ODL_REQUIRE(op >= 0 && op <= 7, "unary: unknown op %d", op);
     if (n <= 0)
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
@@ -290,8 +293,10 @@ int odl_hip_unary(int op, const float *a, int64_t n, float *out, void *stream)
         ODL_UN_CASE(2)
         ODL_UN_CASE(3)
         ODL_UN_CASE(4)
-        default:
         ODL_UN_CASE(5)
+        ODL_UN_CASE(6)
+        default:
+        ODL_UN_CASE(7)
     }
 #undef ODL_UN_CASE
     ODL_LAUNCH_CHECK();

@@ -8,6 +8,7 @@
 // oracle and is never linked into this library.
 #pragma once
 #include <memory>
+#include <string>
 #include <utility>
 #include <vector>
 
@@ -91,6 +92,15 @@ public:
     virtual std::unique_ptr<Mat> square() const                        = 0;
     virtual std::unique_ptr<Mat> pow(const Scalar &exponent) const     = 0;
     virtual std::unique_ptr<Mat> relu() const                          = 0;
+    virtual std::unique_ptr<Mat> sigmoid() const                       = 0;
+    virtual std::unique_ptr<Mat> silu() const                          = 0;
+    // ---- detector forward path (mat.h:719-797 of the reference)
+    virtual std::unique_ptr<Mat> upsample(const Shape &output_shape, int scale_h, int scale_w,
+                                          const std::string &mode = "nearest") const = 0;
+    virtual std::unique_ptr<Mat> cat(const std::vector<const Mat *> &others, int dim) const = 0;
+    virtual std::unique_ptr<Mat> yolo_detect_forward(const Mat &conv_weight, const Mat *conv_bias, const Mat &grid,
+                                                     const Mat &anchor_grid, float stride, int32_t num_anchors,
+                                                     int32_t num_classes) const = 0;
     // ---- convolution / pooling
     virtual std::unique_ptr<Mat> im2col(std::pair<int, int> kernel_size, std::pair<int, int> stride,
                                         std::pair<int, int> pad, bool to_matrix = true) const = 0;
@@ -174,6 +184,14 @@ public:
     std::unique_ptr<Mat> square() const override;
     std::unique_ptr<Mat> pow(const Scalar &exponent) const override;
     std::unique_ptr<Mat> relu() const override;
+    std::unique_ptr<Mat> sigmoid() const override;
+    std::unique_ptr<Mat> silu() const override;
+    std::unique_ptr<Mat> upsample(const Shape &output_shape, int scale_h, int scale_w,
+                                  const std::string &mode = "nearest") const override;
+    std::unique_ptr<Mat> cat(const std::vector<const Mat *> &others, int dim) const override;
+    std::unique_ptr<Mat> yolo_detect_forward(const Mat &conv_weight, const Mat *conv_bias, const Mat &grid,
+                                             const Mat &anchor_grid, float stride, int32_t num_anchors,
+                                             int32_t num_classes) const override;
 
     std::unique_ptr<Mat> im2col(std::pair<int, int> kernel_size, std::pair<int, int> stride, std::pair<int, int> pad,
                                 bool to_matrix = true) const override;

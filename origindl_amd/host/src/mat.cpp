@@ -483,6 +483,90 @@ std::unique_ptr<Mat> OriginMat::log() const { return unary(2, "log", *this); }
 std::unique_ptr<Mat> OriginMat::sqrt() const { return unary(5, "sqrt", *this); }
 std::unique_ptr<Mat> OriginMat::square() const { return unary(4, "square", *this); }
 std::unique_ptr<Mat> OriginMat::relu() const { return unary(0, "relu", *this); }
+std::unique_ptr<Mat> OriginMat::sigmoid() const { return unary(6, "sigmoid", *this); }
+std::unique_ptr<Mat> OriginMat::silu() const { return unary(7, "silu", *this); }
+
+// ------------------------------------------------------------------------------------ detector forward path
+std::unique_ptr<Mat> OriginMat::upsample(const Shape &output_shape, int scale_h, int scale_w, const std::string &) const
+{
+    const OriginMat &x = dev_f32(*this, "upsample");
+    if (shape_.size() != 4)
+        THROW_INVALID_ARG("Upsample: input must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
+    if (output_shape.size() != 4)
+        THROW_INVALID_ARG("Upsample: output_shape must be 4D (N, C, OH, OW), but got shape {}", output_shape.to_string());
+    auto y = new_like(x, output_shape);
+    check(odl_hip_upsample_nearest(fp(x), (int64_t)shape_[0], (int64_t)shape_[1], (int64_t)shape_[2], (int64_t)shape_[3],
+                                   (int64_t)output_shape[2], (int64_t)output_shape[3], scale_h, scale_w,
+                                   y->data_ptr<float>(), nullptr));
+    return y;
+}
+
+std::unique_ptr<Mat> OriginMat::cat(const std::vector<const Mat *> &others, int dim) const
+{
+    std::vector<const OriginMat *> in{&dev_f32(*this, "cat")};
+    for (const Mat *m : others)
+    {
+        if (!m)
+            THROW_RUNTIME_ERROR("cat: null input");
+        in.push_back(&dev_f32(*m, "cat"));
+    }
+    if (in.size() == 1)
+        return std::make_unique<OriginMat>(*this);  // shape/cat.cpp:29-33: a single input is returned as it is
+    if (dim < 0 || (size_t)dim >= shape_.size())
+        THROW_RUNTIME_ERROR("cat: dimension {} out of range for {} dimensions", dim, shape_.size());
+    size_t total = 0;
+    std::vector<const float *> ptrs;
+    std::vector<int64_t> sizes;
+    for (const OriginMat *m : in)
+    {
+        const Shape s = m->shape();
+        if (s.size() != shape_.size())
+            THROW_RUNTIME_ERROR("cat: all inputs must have same number of dimensions");
+        for (size_t d = 0; d < s.size(); ++d)
+            if (d != (size_t)dim && s[d] != shape_[d])
+                THROW_RUNTIME_ERROR("cat: dimension {} mismatch: {} vs {}", d, s[d], shape_[d]);
+        if (m->device() != device())
+            THROW_INVALID_ARG("cat: inputs live on different devices");
+        total += s[dim];
+        ptrs.push_back(fp(*m));
+        sizes.push_back((int64_t)s[dim]);
+    }
+    std::vector<size_t> od = shape_.dims();
+    od[dim] = total;
+    const Shape os(od);
+    int64_t outer, ax, inner;
+    split_axis(os, dim, outer, ax, inner);
+    auto y = new_like(*in[0], os);
+    check(odl_hip_cat(ptrs.data(), sizes.data(), (int)ptrs.size(), outer, inner, y->data_ptr<float>(), nullptr));
+    return y;
+}
+
+std::unique_ptr<Mat> OriginMat::yolo_detect_forward(const Mat &conv_weight, const Mat *conv_bias, const Mat &grid,
+                                                    const Mat &anchor_grid, float stride, int32_t num_anchors,
+                                                    int32_t num_classes) const
+{
+    const OriginMat &x = dev_f32(*this, "yolo_detect_forward");
+    if (shape_.size() != 4)
+        THROW_INVALID_ARG("yolo_detect_forward: input must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
+    const OriginMat &w = dev_f32(conv_weight, "yolo_detect_forward");
+    const OriginMat *b = conv_bias ? &dev_f32(*conv_bias, "yolo_detect_forward") : nullptr;
+    const OriginMat &g = dev_f32(grid, "yolo_detect_forward");
+    const OriginMat &ag = dev_f32(anchor_grid, "yolo_detect_forward");
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
+    const int64_t CI = num_classes + 5;
+    const Shape ws_ = w.shape();
+    if (ws_.size() != 4 || (int64_t)ws_[0] != num_anchors * CI || (int64_t)ws_[1] != C || ws_[2] != 1 || ws_[3] != 1)
+        THROW_INVALID_ARG("yolo_detect_forward: conv weight {} does not match [{}, {}, 1, 1]", ws_.to_string(),
+                          num_anchors * CI, C);
+    const Shape as = ag.shape();
+    const int64_t aH = as.size() >= 3 ? (int64_t)as[2] : H, aW = as.size() >= 4 ? (int64_t)as[3] : W;
+    auto y = new_like(x, Shape{(size_t)N, (size_t)(H * W * num_anchors), (size_t)CI});
+    Workspace ws(odl_hip_yolo_detect_workspace_bytes(N, C, H, W, num_anchors, num_classes), device().index());
+    check(odl_hip_yolo_detect_forward(fp(x), fp(w), b ? fp(*b) : nullptr, fp(g), (int64_t)g.elements(), fp(ag),
+                                      (int64_t)ag.elements(), aH, aW, N, C, H, W, stride, num_anchors, num_classes,
+                                      y->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+    return y;
+}
 
 std::unique_ptr<Mat> OriginMat::pow(const Scalar &exponent) const
 {

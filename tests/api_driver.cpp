@@ -376,6 +376,54 @@ int DRV(unary)(int op, const float *a, int64_t n, float *o)
     });
 }
 
+// ---- detector forward path, at the Mat interface (mat.h:392-405, 719-797)
+int DRV(activation)(int op, const float *a, int64_t n, float *o)  // 6 sigmoid, 7 silu
+{
+    return guarded([&] {
+        auto m = mat_f32(a, Shape{(size_t)n});
+        out(op == 6 ? *m->sigmoid() : *m->silu(), o);
+    });
+}
+
+int DRV(upsample)(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW, int sh, int sw,
+                  float *y)
+{
+    return guarded([&] {
+        auto m = mat_f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
+        out(*m->upsample(Shape{(size_t)N, (size_t)C, (size_t)OH, (size_t)OW}, sh, sw, "nearest"), y);
+    });
+}
+
+int DRV(cat)(const float *const *inputs, const int64_t *axis_sizes, int count, int64_t outer, int64_t inner, float *o)
+{
+    return guarded([&] {
+        std::vector<std::unique_ptr<origin::Mat>> mats;
+        for (int i = 0; i < count; ++i)
+            mats.push_back(mat_f32(inputs[i], Shape{(size_t)outer, (size_t)axis_sizes[i], (size_t)inner}));
+        std::vector<const origin::Mat *> others;
+        for (int i = 1; i < count; ++i)
+            others.push_back(mats[i].get());
+        out(*mats[0]->cat(others, 1), o);
+    });
+}
+
+int DRV(yolo_detect)(const float *x, const float *w, const float *b, const float *grid, const float *anchor_grid,
+                     int64_t anchor_H, int64_t anchor_W, int64_t N, int64_t C, int64_t H, int64_t W, float stride,
+                     int num_anchors, int num_classes, float *o)
+{
+    return guarded([&] {
+        const size_t A = (size_t)num_anchors, CI = (size_t)num_classes + 5;
+        auto xm = mat_f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
+        auto wm = mat_f32(w, Shape{A * CI, (size_t)C, 1, 1});
+        std::unique_ptr<origin::Mat> bm;
+        if (b)
+            bm = mat_f32(b, Shape{A * CI});
+        auto gm = mat_f32(grid, Shape{1, A, (size_t)H, (size_t)W, 2});
+        auto am = mat_f32(anchor_grid, Shape{1, A, (size_t)anchor_H, (size_t)anchor_W, 2});
+        out(*xm->yolo_detect_forward(*wm, bm.get(), *gm, *am, stride, num_anchors, num_classes), o);
+    });
+}
+
 int DRV(pow_scalar)(const float *a, int64_t n, float e, float *o)
 {
     return guarded([&] { out(F::pow(f32(a, Shape{(size_t)n}), Scalar(e)), o); });

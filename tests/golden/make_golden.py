@@ -222,6 +222,44 @@ def main():
     assert r.odl_ref_pow_scalar(np.abs(a), a.size, 0.5, o) == 0
     out["ew_pow05"] = o
 
+    # --- detector forward path: sigmoid / silu, nearest upsample, cat, yolo detect head ----------------------
+    rd = np.random.default_rng(20240902)
+    xa = (rd.standard_normal((301,), dtype=f32) * f32(3)).astype(f32)
+    out["det_act_x"] = xa
+    for op, nm in ((6, "sigmoid"), (7, "silu")):
+        o = np.empty_like(xa)
+        assert r.odl_ref_activation(op, xa, xa.size, o) == 0
+        out[f"det_{nm}"] = o
+    xu = rd.standard_normal((2, 3, 4, 5), dtype=f32)
+    for nm, (sh, sw) in (("up22", (2, 2)), ("up13", (1, 3))):
+        o = np.empty((2, 3, 4 * sh, 5 * sw), f32)
+        assert r.odl_ref_upsample(xu, 2, 3, 4, 5, 4 * sh, 5 * sw, sh, sw, o) == 0
+        out[f"det_{nm}"] = o
+    out["det_up_x"] = xu
+    parts = [rd.standard_normal((3, c, 7), dtype=f32) for c in (2, 5, 1)]
+    o = np.empty((3, 8, 7), f32)
+    keep = ol.ptr_arr(parts)
+    assert r.odl_ref_cat(keep, np.asarray([2, 5, 1], np.int64), 3, 3, 7, o) == 0
+    for i, pt in enumerate(parts):
+        out[f"det_cat_in{i}"] = pt
+    out["det_cat"] = o
+    # detect head: N=2, C=6, H=4, W=5, anchors=3, classes=2 (CI=7); the anchor grid is coarser than the map (2x5)
+    N, C, H, W, A, NC = 2, 6, 4, 5, 3, 2
+    CI = NC + 5
+    xd = rd.standard_normal((N, C, H, W), dtype=f32)
+    wd = (rd.standard_normal((A * CI, C, 1, 1), dtype=f32) * f32(0.5)).astype(f32)
+    bd = rd.standard_normal((A * CI,), dtype=f32)
+    gy_, gx_ = np.meshgrid(np.arange(H, dtype=f32), np.arange(W, dtype=f32), indexing="ij")
+    grid = np.broadcast_to(np.stack([gx_, gy_], -1) - f32(0.5), (1, A, H, W, 2)).astype(f32).copy()
+    for nm, (aH, aW) in (("detA", (H, W)), ("detB", (2, 5))):
+        anchors = (rd.random((A, 2), dtype=f32) * f32(30) + f32(4)).astype(f32)
+        ag = np.broadcast_to(anchors.reshape(1, A, 1, 1, 2), (1, A, aH, aW, 2)).astype(f32).copy()
+        ag += (rd.random(ag.shape, dtype=f32) * f32(0.25)).astype(f32)  # make every cell distinguishable
+        o = np.empty((N, A * H * W, CI), f32)
+        assert r.odl_ref_yolo_detect(xd, wd, bd if nm == "detA" else None, grid, ag, aH, aW, N, C, H, W, 8.0, A, NC, o) == 0
+        out[f"{nm}_anchor_grid"], out[f"{nm}_out"] = ag, o
+    out["det_x"], out["det_w"], out["det_b"], out["det_grid"] = xd, wd, bd, grid
+
     path = os.path.join(HERE, "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

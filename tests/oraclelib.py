@@ -44,6 +44,9 @@ _ORC_SIGS = {
     "orc_binary": "iplplp>i",
     "orc_unary": "iplp>v",
     "orc_pow_scalar": "plfp>v",
+    "orc_upsample_nearest": "p" + "llllll" + "ii" + "p>i",
+    "orc_cat": "ppillp>i",
+    "orc_yolo_detect_forward": "pppplp" + "lll" + "llll" + "f" + "ii" + "p>i",
     "orc_mlp_train_step": "ppillll" + "p" * 12 + "ifffff" + "pppppp>i",
     "orc_cnn_train_step": "ppillllll" + "p" * 8 + "f" + "p" + "pp" + "p" * 8 + "p>i",
 }
@@ -73,6 +76,10 @@ _REF_SIGS = {
     "odl_ref_binary": "ippippip>i",
     "odl_ref_unary": "iplp>i",
     "odl_ref_pow_scalar": "plfp>i",
+    "odl_ref_activation": "iplp>i",
+    "odl_ref_upsample": "p" + "llllll" + "ii" + "p>i",
+    "odl_ref_cat": "ppillp>i",
+    "odl_ref_yolo_detect": "ppppp" + "ll" + "llll" + "f" + "ii" + "p>i",
     "odl_ref_mlp_train": "ppillll" + "pppp" + "ifffff" + "pppppp>i",
     "odl_ref_cnn_train": "ppillllll" + "p" * 8 + "f" + "p" + "p" * 8 + "p>i",
     "odl_ref_mlp_bench": "lllliipp>i",
@@ -159,6 +166,11 @@ def host_driver(cpu=False):
         sigs = {k.replace("odl_ref_", prefix): v for k, v in _REF_SIGS.items()}
         _host[key] = _Lib(HOST_CPU_DRIVER_SO if cpu else HOST_DRIVER_SO, sigs)
     return _host[key]
+
+
+def ptr_arr(arrays):
+    """Host array of the data addresses of `arrays` (for entry points that take a pointer table)."""
+    return np.asarray([a.ctypes.data for a in arrays], dtype=np.uint64)
 
 
 def shape_arr(shape):

@@ -290,3 +290,29 @@ def test_reference_example_nn_linear_runs_unchanged_on_the_gpu():
     m = re.search(r"loss = ([-0-9.e]+), w = ([-0-9.e]+), b = ([-0-9.e]+)", last)
     loss, w, b = (float(v) for v in m.groups())
     assert abs(w - 2.0) < 0.1 and abs(b - 5.0) < 0.1 and loss < 0.05, last
+
+
+def test_detector_ops_through_the_mat_interface(h):
+    """sigmoid / silu / upsample / cat / yolo_detect_forward called on Mat objects exactly as the reference driver
+    called them to write the fixtures."""
+    x = G["det_act_x"]
+    for op, nm in ((6, "sigmoid"), (7, "silu")):
+        got = np.empty_like(x)
+        assert h.odl_host_activation(op, x, x.size, got) == 0
+        np.testing.assert_allclose(got, G[f"det_{nm}"], rtol=3e-7, atol=1e-9)
+    xu = G["det_up_x"]
+    for nm, (sh, sw) in (("up22", (2, 2)), ("up13", (1, 3))):
+        got = np.empty((2, 3, 4 * sh, 5 * sw), f32)
+        assert h.odl_host_upsample(xu, 2, 3, 4, 5, 4 * sh, 5 * sw, sh, sw, got) == 0
+        assert np.array_equal(got, G[f"det_{nm}"])
+    assert h.odl_host_upsample(xu, 2, 3, 4, 5, 9, 10, 2, 2, np.empty((2, 3, 9, 10), f32)) == -1  # row 8 -> input row 4
+    parts = [G[f"det_cat_in{i}"] for i in range(3)]
+    got = np.empty((3, 8, 7), f32)
+    assert h.odl_host_cat(ol.ptr_arr(parts), np.asarray([2, 5, 1], np.int64), 3, 3, 7, got) == 0
+    assert np.array_equal(got, G["det_cat"])
+    for name in ("detA", "detB"):
+        ag = G[f"{name}_anchor_grid"]
+        got = np.empty_like(G[f"{name}_out"])
+        assert h.odl_host_yolo_detect(G["det_x"], G["det_w"], G["det_b"] if name == "detA" else None, G["det_grid"], ag,
+                                      ag.shape[2], ag.shape[3], 2, 6, 4, 5, 8.0, 3, 2, got) == 0
+        np.testing.assert_allclose(got, G[f"{name}_out"], rtol=2e-6, atol=1e-6)

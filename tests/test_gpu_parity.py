@@ -273,6 +273,9 @@ CONV_SEEDED = [
     (2, 6, 10, 9, 16, 2, 3, 1, 1),     # rectangular kernel, K = 36
     (2, 16, 15, 15, 20, 3, 3, 2, 0),   # stride 2 without padding
     (5, 64, 7, 7, 48, 3, 3, 1, 1),     # more pixels than one tile column, C = 64
+    (2, 3, 64, 64, 16, 6, 6, 2, 2),    # the detector's stem: 6x6, stride 2, pad 2, three channels
+    (2, 32, 40, 40, 64, 3, 3, 2, 1),   # its down-sampling convolutions
+    (2, 64, 20, 20, 128, 1, 1, 1, 0),  # its 1x1 bottleneck convolutions
 ]
 
 
@@ -608,3 +611,71 @@ def test_fused_optimizer_steps_match_the_op_by_op_sequence(api, o):
     # closed form at t = 1 from zero moments: m_hat = g and v_hat = g^2, so the step is lr * g / (|g| + eps)
     b64 = big.astype(np.float64)
     np.testing.assert_allclose(out, b64 - 1e-3 * b64 / (np.abs(b64) + 1e-8), rtol=0, atol=3e-7)
+
+
+# ------------------------------------------------------------------ detector forward path (config 5's operators)
+def test_sigmoid_silu_vs_oracle_and_fixtures(api, o):
+    x = G["det_act_x"]
+    for op, nm in ((6, "sigmoid"), (7, "silu")):
+        np.testing.assert_allclose(host(api.unary(nm, dev(x))), G[f"det_{nm}"], rtol=3e-7, atol=1e-9)
+    rng = np.random.default_rng(31)
+    big = (rng.standard_normal(1 << 20, dtype=f32) * f32(5)).astype(f32)
+    for op, nm in ((6, "sigmoid"), (7, "silu")):
+        want = np.empty_like(big)
+        o.orc_unary(op, big, big.size, want)
+        np.testing.assert_allclose(host(api.unary(nm, dev(big))), want, rtol=3e-7, atol=1e-9)
+
+
+def test_upsample_and_cat_bit_exact(api, o):
+    xu = G["det_up_x"]
+    assert np.array_equal(host(api.upsample(dev(xu), 2)), G["det_up22"])
+    assert np.array_equal(host(api.upsample(dev(xu), (1, 3))), G["det_up13"])
+    parts = [G[f"det_cat_in{i}"] for i in range(3)]
+    assert np.array_equal(host(api.cat([dev(p) for p in parts], 1)), G["det_cat"])
+    # the detector's own shapes: P5 -> P4 upsample and the concatenation that follows it
+    rng = np.random.default_rng(32)
+    a, b = rng.standard_normal((4, 128, 10, 10), dtype=f32), rng.standard_normal((4, 128, 20, 20), dtype=f32)
+    up = host(api.upsample(dev(a), 2))
+    want = np.empty((4, 128, 20, 20), f32)
+    assert o.orc_upsample_nearest(a, 4, 128, 10, 10, 20, 20, 2, 2, want) == 0
+    assert np.array_equal(up, want)
+    cat = host(api.cat([dev(up), dev(b)], 1))
+    assert np.array_equal(cat, np.concatenate([up, b], axis=1))
+    odd = [rng.standard_normal((3, c, 5), dtype=f32) for c in (3, 1, 7)]  # runs that are not multiples of four floats
+    assert np.array_equal(host(api.cat([dev(p) for p in odd], 1)), np.concatenate(odd, axis=1))
+    same = [rng.standard_normal((2, 4, 6), dtype=f32) for _ in range(3)]
+    for dim in (0, 1, 2):
+        assert np.array_equal(host(api.cat([dev(p) for p in same], dim)), np.concatenate(same, axis=dim)), dim
+    with pytest.raises(api.OdlRuntimeError):
+        api.cat([dev(odd[0]), dev(same[0])], 1)
+    with pytest.raises(api.OdlInvalidArgument):  # an output row that would read past the input
+        api.lib().call("odl_hip_upsample_nearest", None, 1, 1, 2, 2, 5, 4, 2, 2, None, None)
+
+
+@pytest.mark.parametrize("name", ["detA", "detB"])
+def test_yolo_detect_fixtures(api, name):
+    ag = G[f"{name}_anchor_grid"]
+    b = dev(G["det_b"]) if name == "detA" else None
+    got = host(api.yolo_detect_forward(dev(G["det_x"]), dev(G["det_w"]), b, dev(G["det_grid"]), dev(ag), 8.0, 3, 2))
+    np.testing.assert_allclose(got, G[f"{name}_out"], rtol=2e-6, atol=1e-6)
+
+
+def test_yolo_detect_at_detector_size_vs_oracle(api, o):
+    # the P3 head of a width-0.25 YOLOv5: [4, 64, 40, 40] -> 3 anchors x 85
+    rng = np.random.default_rng(33)
+    N, C, H, W, A, NC = 4, 64, 40, 40, 3, 80
+    CI = NC + 5
+    x = rng.standard_normal((N, C, H, W), dtype=f32)
+    w = (rng.standard_normal((A * CI, C, 1, 1), dtype=f32) * f32(0.2)).astype(f32)
+    b = rng.standard_normal(A * CI, dtype=f32)
+    gyy, gxx = np.meshgrid(np.arange(H), np.arange(W), indexing="ij")
+    grid = np.broadcast_to(np.stack([gxx, gyy], -1).astype(f32) - f32(0.5), (1, A, H, W, 2)).copy()
+    anchors = np.array([[10, 13], [16, 30], [33, 23]], f32)
+    ag = np.broadcast_to(anchors.reshape(1, A, 1, 1, 2), (1, A, H, W, 2)).copy()
+    want = np.empty((N, A * H * W, CI), f32)
+    assert o.orc_yolo_detect_forward(x, w, b, grid, grid.size, ag, ag.size, H, W, N, C, H, W, 8.0, A, NC, want) == 0
+    got = host(api.yolo_detect_forward(dev(x), dev(w), dev(b), dev(grid), dev(ag), 8.0, A, NC))
+    # logits are sums of 64 products: the GEMM bound on the logit, carried through sigmoid (slope <= 1/4) and the box
+    # transform (at most x2*stride, or x4*2s*anchor)
+    np.testing.assert_allclose(got[..., 4:], want[..., 4:], rtol=0, atol=2e-6)
+    np.testing.assert_allclose(got[..., :4], want[..., :4], rtol=2e-5, atol=2e-4)

@@ -489,3 +489,73 @@ def test_adam_step_closed_form():
     W2, gW2 = G["mlp_W2"].astype(np.float64), g_[2].astype(np.float64)
     g = gW2 + 1e-4 * W2
     np.testing.assert_allclose(p[2], W2 - 1e-3 * g / (np.abs(g) + 1e-8), atol=2e-7)
+
+
+# ------------------------------------------------------------------ detector forward path (config 5's operators)
+def _detect_inputs(name):
+    aH, aW = G[f"{name}_anchor_grid"].shape[2:4]
+    return (G["det_x"], G["det_w"], G["det_b"] if name == "detA" else None, G["det_grid"], G[f"{name}_anchor_grid"],
+            int(aH), int(aW))
+
+
+def test_detector_ops_fixtures_bit_exact():
+    o = ol.oracle()
+    x = G["det_act_x"]
+    for op, nm in ((6, "sigmoid"), (7, "silu")):
+        got = np.empty_like(x)
+        o.orc_unary(op, x, x.size, got)
+        assert np.array_equal(got, G[f"det_{nm}"]), nm
+    xu = G["det_up_x"]
+    for nm, (sh, sw) in (("up22", (2, 2)), ("up13", (1, 3))):
+        got = np.empty((2, 3, 4 * sh, 5 * sw), f32)
+        assert o.orc_upsample_nearest(xu, 2, 3, 4, 5, 4 * sh, 5 * sw, sh, sw, got) == 0
+        assert np.array_equal(got, G[f"det_{nm}"]), nm
+    parts = [G[f"det_cat_in{i}"] for i in range(3)]
+    got = np.empty((3, 8, 7), f32)
+    assert o.orc_cat(ol.ptr_arr(parts), np.asarray([2, 5, 1], np.int64), 3, 3, 7, got) == 0
+    assert np.array_equal(got, G["det_cat"])
+    for name in ("detA", "detB"):
+        xd, wd, bd, grid, ag, aH, aW = _detect_inputs(name)
+        got = np.empty_like(G[f"{name}_out"])
+        assert o.orc_yolo_detect_forward(xd, wd, bd, grid, grid.size, ag, ag.size, aH, aW, 2, 6, 4, 5, 8.0, 3, 2, got) == 0
+        assert np.array_equal(got, G[f"{name}_out"]), name
+
+
+def test_detector_ops_against_plain_numpy():
+    """The same operators written independently: float64 formulas, np.repeat, np.concatenate, an einsum for the 1x1
+    convolution followed by the published YOLOv5 decoding (xy = (2s + grid) * stride, wh = (2s)^2 * anchor)."""
+    o = ol.oracle()
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(1000, dtype=f32) * f32(4)).astype(f32)
+    sg, si = np.empty_like(x), np.empty_like(x)
+    o.orc_unary(6, x, x.size, sg)
+    o.orc_unary(7, x, x.size, si)
+    x64 = x.astype(np.float64)
+    np.testing.assert_allclose(sg, 1 / (1 + np.exp(-x64)), rtol=3e-7)
+    np.testing.assert_allclose(si, x64 / (1 + np.exp(-x64)), rtol=3e-7, atol=1e-30)
+    xu = rng.standard_normal((2, 3, 5, 4), dtype=f32)
+    up = np.empty((2, 3, 15, 8), f32)
+    assert o.orc_upsample_nearest(xu, 2, 3, 5, 4, 15, 8, 3, 2, up) == 0
+    assert np.array_equal(up, np.repeat(np.repeat(xu, 3, axis=2), 2, axis=3))
+    assert o.orc_upsample_nearest(xu, 2, 3, 5, 4, 16, 8, 3, 2, np.empty((2, 3, 16, 8), f32)) == -1  # row 15 -> input row 5
+    parts = [rng.standard_normal((2, c, 3, 4), dtype=f32) for c in (4, 1, 6)]
+    cat = np.empty((2, 11, 3, 4), f32)
+    assert o.orc_cat(ol.ptr_arr(parts), np.asarray([4, 1, 6], np.int64), 3, 2, 12, cat) == 0
+    assert np.array_equal(cat, np.concatenate(parts, axis=1))
+    N, C, H, W, A, NC = 2, 5, 3, 4, 3, 4
+    CI = NC + 5
+    xd = rng.standard_normal((N, C, H, W), dtype=f32)
+    wd = rng.standard_normal((A * CI, C, 1, 1), dtype=f32)
+    bd = rng.standard_normal(A * CI, dtype=f32)
+    gyy, gxx = np.meshgrid(np.arange(H), np.arange(W), indexing="ij")
+    grid = np.broadcast_to(np.stack([gxx, gyy], -1).astype(f32) - f32(0.5), (1, A, H, W, 2)).copy()
+    anchors = (rng.random((A, 2), dtype=f32) * f32(20) + f32(2)).astype(f32)
+    ag = np.broadcast_to(anchors.reshape(1, A, 1, 1, 2), (1, A, H, W, 2)).copy()
+    got = np.empty((N, A * H * W, CI), f32)
+    assert o.orc_yolo_detect_forward(xd, wd, bd, grid, grid.size, ag, ag.size, H, W, N, C, H, W, 16.0, A, NC, got) == 0
+    conv = np.einsum("nchw,oc->nohw", xd.astype(np.float64), wd[:, :, 0, 0].astype(np.float64)) + bd[None, :, None, None]
+    s = 1 / (1 + np.exp(-conv.reshape(N, A, CI, H, W).transpose(0, 1, 3, 4, 2)))
+    want = s.copy()
+    want[..., 0:2] = (s[..., 0:2] * 2 + grid) * 16.0
+    want[..., 2:4] = (s[..., 2:4] * 2) ** 2 * ag
+    np.testing.assert_allclose(got, want.reshape(N, A * H * W, CI), rtol=2e-5, atol=2e-6)
