@@ -187,6 +187,7 @@ def train_steps(steps, warmup, with_cpu):
                                        "gemm_flop_per_step": 6.0 * 512 * (784 * 1000 + 1000 * 10)}
     rc = h.odl_host_cnn_bench(256, steps, warmup, ms, loss)
     out["cnn_b256_sgd"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss": float(loss[0])}
+    out["yolov5n_forward_4x3x320x320"] = yolo_forward(h, ol.ref() if with_cpu and ol.have_ref() else None, steps)
     if with_cpu and ol.have_ref():
         r = ol.ref()
         rc = r.odl_ref_mlp_bench(512, 784, 1000, 10, 1, 0, ms, loss)
@@ -195,6 +196,34 @@ def train_steps(steps, warmup, with_cpu):
         rc = r.odl_ref_cnn_bench(4, 1, 0, ms, loss)
         out["cnn_b256_sgd"]["cpu_reference_ms_per_step_extrapolated_from_batch_4"] = float(ms[0]) * 64.0
     return out
+
+
+def yolo_forward(h, ref, reps):
+    """Config 5: a YOLOv5n-architecture model (depth 0.33, width 0.25, random weights from a seed, written in PNNX's
+    file format by tests/pnnx_synth.py) run forward on [4,3,320,320] by the host layer's PNNX graph runner; the
+    reference's own runner on one CPU core beside it, at batch 1 (its time scales with the batch)."""
+    import tempfile
+    import numpy as np
+    import pnnx_synth
+    res = {}
+    with tempfile.TemporaryDirectory() as tmp:
+        def run(drv, name, batch, n):
+            param, binp, shp = pnnx_synth.write(os.path.join(tmp, "y5n_b%d" % batch), seed=0, batch=batch, size=320)
+            x = np.random.default_rng(0).random((batch, 3, 320, 320), dtype=np.float32)
+            o = np.empty(shp, np.float32)
+            oshape, nd, ms = np.zeros(8, np.int64), np.zeros(1, np.int32), np.zeros(1, np.float32)
+            t0 = time.perf_counter()
+            rc = getattr(drv, name)(param.encode(), binp.encode(), x, batch, 3, 320, 320, n, o, o.size, oshape, nd, ms)
+            return rc, float(ms[0]), time.perf_counter() - t0, o
+        rc, ms, _, o = run(h, "odl_host_pnnx_forward", 4, max(3, reps) + 1)
+        gflop = pnnx_synth.flops(4, 320) / 1e9
+        res.update({"rc": rc, "ms_per_forward": ms, "conv_gflop": gflop, "tflops": gflop / ms if ms > 0 else None,
+                    "output_shape": list(o.shape), "output_mean": float(o.mean())})
+        if ref is not None:
+            rc, _, wall, _ = run(ref, "odl_ref_pnnx_forward", 1, 1)
+            res["cpu_reference_ms_per_forward_batch_1"] = wall * 1e3
+            res["cpu_reference_ms_per_forward_extrapolated_to_batch_4"] = wall * 4e3
+    return res
 
 
 # HBM-side bytes of one 4096^3 sgemm_mfma_kernel launch: FETCH_SIZE (scaled 2.000x by the calibration copy) 805.2 MiB on

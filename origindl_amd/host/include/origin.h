@@ -5,3 +5,4 @@
 #include "origin/tensor.h"
 #include "origin/functional.h"
 #include "origin/nn.h"
+#include "origin/pnnx/pnnx_graph.h"

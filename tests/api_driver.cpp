@@ -27,6 +27,7 @@
 #include "origin/nn/layers/max_pool2d.h"
 #include "origin/nn/layers/relu.h"
 #include "origin/nn/sequential.h"
+#include "origin/pnnx/pnnx_graph.h"
 #include "origin/operators/activation/relu.h"
 #include "origin/operators/activation/softmax.h"
 #include "origin/operators/conv/conv2d.h"
@@ -421,6 +422,43 @@ int DRV(yolo_detect)(const float *x, const float *w, const float *b, const float
         auto gm = mat_f32(grid, Shape{1, A, (size_t)H, (size_t)W, 2});
         auto am = mat_f32(anchor_grid, Shape{1, A, (size_t)anchor_H, (size_t)anchor_W, 2});
         out(*xm->yolo_detect_forward(*wm, bm.get(), *gm, *am, stride, num_anchors, num_classes), o);
+    });
+}
+
+// A PNNX model (`.pnnx.param` + `.pnnx.bin`) run forward `reps` times on x[N,C,H,W]; the first output of
+// `pnnx_output_0` is copied to out (capacity in floats) and its shape to out_shape[0..out_nd). ms = mean time of the
+// forwards after the first (which also loads weights), read back included.
+int DRV(pnnx_forward)(const char *param_path, const char *bin_path, const float *x, int64_t N, int64_t C, int64_t H,
+                      int64_t W, int reps, float *o, int64_t capacity, int64_t *out_shape, int *out_nd, float *ms)
+{
+    return guarded([&] {
+        origin::pnnx::PNNXGraph graph(param_path, bin_path);
+        graph.build();
+        auto X = f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
+        std::vector<float> last;
+        Shape shp;
+        auto t0 = std::chrono::steady_clock::now();
+        for (int r = 0; r < (reps < 1 ? 1 : reps); ++r)
+        {
+            if (r == 1)
+                t0 = std::chrono::steady_clock::now();
+            graph.set_inputs("pnnx_input_0", {X});
+            graph.forward();
+            auto outs = graph.get_outputs("pnnx_output_0");
+            if (outs.empty())
+                throw std::runtime_error("pnnx_forward: the graph produced no output");
+            shp  = outs[0].shape();
+            last = outs[0].to_vector<float>();
+        }
+        const auto t1 = std::chrono::steady_clock::now();
+        if (ms)
+            *ms = reps > 1 ? std::chrono::duration<float, std::milli>(t1 - t0).count() / (float)(reps - 1) : 0.0f;
+        if ((int64_t)last.size() > capacity)
+            throw std::invalid_argument("pnnx_forward: output larger than the buffer");
+        std::memcpy(o, last.data(), last.size() * sizeof(float));
+        *out_nd = (int)shp.size();
+        for (size_t i = 0; i < shp.size(); ++i)
+            out_shape[i] = (int64_t)shp[i];
     });
 }
 

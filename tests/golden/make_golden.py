@@ -260,6 +260,18 @@ def main():
         out[f"{nm}_anchor_grid"], out[f"{nm}_out"] = ag, o
     out["det_x"], out["det_w"], out["det_b"], out["det_grid"] = xd, wd, bd, grid
 
+    # --- a whole YOLOv5n-architecture forward through the reference's PNNX runner (synthetic weights, 64x64 input) --
+    import tempfile
+    import pnnx_synth
+    with tempfile.TemporaryDirectory() as tmp:
+        param, binp, shp = pnnx_synth.write(os.path.join(tmp, "y5n"), seed=3, batch=1, size=64, num_classes=80)
+        xin = np.random.default_rng(7).random((1, 3, 64, 64), dtype=f32)
+        o = np.empty(shp, f32)
+        oshape, nd, ms = np.zeros(8, np.int64), np.zeros(1, np.int32), np.zeros(1, f32)
+        assert r.odl_ref_pnnx_forward(param.encode(), binp.encode(), xin, 1, 3, 64, 64, 1, o, o.size, oshape, nd, ms) == 0
+        assert tuple(oshape[:nd[0]]) == tuple(shp)
+    out["y5n64_x"], out["y5n64_out"] = xin, o
+
     path = os.path.join(HERE, "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

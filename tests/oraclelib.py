@@ -79,6 +79,7 @@ _REF_SIGS = {
     "odl_ref_activation": "iplp>i",
     "odl_ref_upsample": "p" + "llllll" + "ii" + "p>i",
     "odl_ref_cat": "ppillp>i",
+    "odl_ref_pnnx_forward": "ppplllliplppp>i",
     "odl_ref_yolo_detect": "ppppp" + "ll" + "llll" + "f" + "ii" + "p>i",
     "odl_ref_mlp_train": "ppillll" + "pppp" + "ifffff" + "pppppp>i",
     "odl_ref_cnn_train": "ppillllll" + "p" * 8 + "f" + "p" + "p" * 8 + "p>i",

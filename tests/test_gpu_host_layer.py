@@ -316,3 +316,48 @@ def test_detector_ops_through_the_mat_interface(h):
         assert h.odl_host_yolo_detect(G["det_x"], G["det_w"], G["det_b"] if name == "detA" else None, G["det_grid"], ag,
                                       ag.shape[2], ag.shape[3], 2, 6, 4, 5, 8.0, 3, 2, got) == 0
         np.testing.assert_allclose(got, G[f"{name}_out"], rtol=2e-6, atol=1e-6)
+
+
+def _run_pnnx(drv, prefix, param, binp, x, out_shape, reps=1):
+    out = np.empty(out_shape, f32)
+    oshape, nd, ms = np.zeros(8, np.int64), np.zeros(1, np.int32), np.zeros(1, f32)
+    N, C, H, W = x.shape
+    rc = getattr(drv, prefix + "pnnx_forward")(param.encode(), binp.encode(), x, N, C, H, W, reps, out, out.size, oshape,
+                                               nd, ms)
+    return rc, out, tuple(oshape[:nd[0]]), float(ms[0])
+
+
+def test_yolov5n_pnnx_forward_matches_the_reference(h, tmp_path):
+    """A YOLOv5n-architecture model in PNNX's file format (synthetic weights written by tests/pnnx_synth.py from a
+    seed) run by this repository's graph runner on the GPU, against the output the reference's own PNNX runner
+    produced for the same files on the CPU (fixture y5n64_out). Roughly sixty convolutions deep: every logit is a
+    chain of fp32 GEMMs whose summation order differs, so the bar is the GEMM bound carried through the network —
+    measured deviation is 5e-7 relative to |value| + 1; 1e-5 is asserted."""
+    import pnnx_synth
+    param, binp, shp = pnnx_synth.write(str(tmp_path / "y5n"), seed=3, batch=1, size=64, num_classes=80)
+    rc, out, oshape, _ = _run_pnnx(h, "odl_host_", param, binp, G["y5n64_x"], shp)
+    assert rc == 0 and oshape == tuple(shp) == (1, 252, 85)
+    want = G["y5n64_out"]
+    err = np.abs(out - want) / (np.abs(want) + 1.0)
+    print("\n[yolov5n 64x64] max scaled deviation %.3g" % err.max(), flush=True)
+    assert err.max() < 1e-5
+    # a second forward on the same graph object reuses the uploaded weights and gives the same answer
+    rc, out2, _, _ = _run_pnnx(h, "odl_host_", param, binp, G["y5n64_x"], shp, reps=3)
+    assert rc == 0 and np.array_equal(out, out2)
+
+
+def test_pnnx_runner_rejects_bad_files(h, tmp_path):
+    import pnnx_synth
+    param, binp, shp = pnnx_synth.write(str(tmp_path / "y5n"), seed=1, batch=1, size=32, num_classes=3)
+    x = np.zeros((1, 3, 32, 32), f32)
+    bad = tmp_path / "bad.param"
+    bad.write_text("1234\n1 1\n")
+    assert _run_pnnx(h, "odl_host_", str(bad), binp, x, shp)[0] == -2          # wrong magic -> runtime_error
+    assert _run_pnnx(h, "odl_host_", str(tmp_path / "nope.param"), binp, x, shp)[0] == -2
+    text = open(param).read().replace("nn.SiLU model.1.act", "nn.GELU model.1.act")
+    bad.write_text(text)
+    assert _run_pnnx(h, "odl_host_", str(bad), binp, x, shp)[0] == -2          # unsupported operator type
+    trunc = tmp_path / "trunc.bin"
+    trunc.write_bytes(open(binp, "rb").read()[:4000])
+    assert _run_pnnx(h, "odl_host_", param, str(trunc), x, shp)[0] == -2
+    assert _run_pnnx(h, "odl_host_", param, binp, x, shp)[0] == 0
