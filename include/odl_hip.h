@@ -94,6 +94,13 @@ int odl_hip_col2im(const float *col, int64_t N, int64_t C, int64_t H, int64_t W,
 int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
                    int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *y, void *workspace,
                    size_t workspace_bytes, void *stream);
+/* The same convolution with an activation applied to each output after the bias, in the kernel's epilogue:
+ * activation -1 none, 0 relu, 7 silu (the odl_hip_unary operator numbers). Bit-identical to odl_hip_conv2d followed by
+ * odl_hip_unary; the reference has no fused counterpart (its graphs hold nn.Conv2d and nn.SiLU as separate nodes,
+ * src/pnnx/operator_mapper.cpp:30-37). Same workspace as odl_hip_conv2d. */
+int odl_hip_conv2d_act(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                       int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int activation, float *y,
+                       void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
                                       int SH, int SW, int PH, int PW);
 /* Mat::conv2d_backward (mat.h:505; conv2d.cpp:514-599) -> gx, gW and (when gb != NULL) gb.

@@ -184,8 +184,8 @@ def col2im(col, input_shape, kernel_size, stride, pad, to_matrix=True):
     return img
 
 
-def conv2d(x, w, b=None, stride=1, pad=0):
-    """Mat::conv2d (src/mat/origin/cpu/conv/conv2d.cpp:404-512)."""
+def conv2d(x, w, b=None, stride=1, pad=0, activation=None):
+    """Mat::conv2d (src/mat/origin/cpu/conv/conv2d.cpp:404-512); activation "relu" / "silu" runs in the epilogue."""
     _chk(x, "x"), _chk(w, "W")
     if x.dim() != 4:
         raise OdlInvalidArgument("conv2d: x must be 4D (N, C, H, W)")
@@ -201,8 +201,9 @@ def conv2d(x, w, b=None, stride=1, pad=0):
     OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
     y = _empty((N, OC, _builtins.max(OH, 0), _builtins.max(OW, 0)))
     ws, nb = _ws(lib().query("odl_hip_conv2d_workspace_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW))
-    lib().call("odl_hip_conv2d", _p(x), _p(w), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, _p(y), _p(ws), nb,
-               _stream())
+    act = -1 if activation is None else _UN[activation]
+    lib().call("odl_hip_conv2d_act", _p(x), _p(w), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, act, _p(y), _p(ws),
+               nb, _stream())
     return y
 
 

@@ -16,7 +16,7 @@ namespace odl
 {
 int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                  const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int epi, int64_t P,
-                 int split_k, void *workspace, size_t workspace_bytes, hipStream_t st);
+                 int split_k, void *workspace, size_t workspace_bytes, hipStream_t st, int act = 0);
 size_t sgemm_workspace(int64_t M, int64_t N, int64_t K, int split_k);
 bool conv_implicit_forward_ok(const float *w, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
                               int64_t OH, int64_t OW);
@@ -28,7 +28,7 @@ size_t conv_implicit_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, i
 size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW, int64_t pixels);
 int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
-                          void *workspace, size_t workspace_bytes, hipStream_t st);
+                          int act, void *workspace, size_t workspace_bytes, hipStream_t st);
 size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
 int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W,
                         int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
@@ -807,11 +807,14 @@ size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W
     return align256((size_t)(N * OH * OW * C * KH * KW) * sizeof(float));
 }
 
-int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
-                   int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *y, void *workspace,
-                   size_t workspace_bytes, void *stream)
+int odl_hip_conv2d_act(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                       int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int activation, float *y,
+                       void *workspace, size_t workspace_bytes, void *stream)
 {
     ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(activation == -1 || activation == 0 || activation == 7,
+                "conv2d: activation must be -1 (none), 0 (relu) or 7 (silu), the unary operator numbers; got %d", activation);
+    const int act = activation == 0 ? 1 : (activation == 7 ? 2 : 0);
     ConvGeom g;
     int rc = make_geom(g, "conv2d", N, C, H, W, KH, KW, SH, SW, PH, PW);
     if (rc != ODL_OK)
@@ -822,7 +825,7 @@ int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, in
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
     if (odl::conv_implicit_forward_ok(w, N, C, H, W, OC, KH, KW, g.OH, g.OW))
-        return odl::conv_implicit_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, workspace,
+        return odl::conv_implicit_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, act, workspace,
                                           workspace_bytes, st);
     // explicit path: col = im2col(x), then y^T[OC, M] = W2d[OC,K] . col[M,K]^T stored as y[n][oc][p] (+ bias per channel)
     const size_t need = align256((size_t)(M * K) * sizeof(float));
@@ -833,7 +836,14 @@ int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, in
     if (rc != ODL_OK)
         return rc;
     return odl::sgemm_launch(0, 1, OC, M, K, w, K, col, K, y, 0, b, /*EPI_NCHW_ROWB*/ 2, g.OH * g.OW, 1, nullptr, 0,
-                             st);
+                             st, act);
+}
+
+int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                   int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, float *y, void *workspace,
+                   size_t workspace_bytes, void *stream)
+{
+    return odl_hip_conv2d_act(x, w, b, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, -1, y, workspace, workspace_bytes, stream);
 }
 
 namespace

@@ -68,6 +68,7 @@ struct GemmArgs
     int64_t k_per_split;     // K range of one grid.y slice (multiple of BK)
     int64_t c_split_stride;  // elements between the partial outputs of consecutive slices (0 = none)
     int64_t P;               // EPI_NCHW_ROWB: OH*OW
+    int act;                 // EPI_NCHW_ROWB: activation applied after the bias (0 none, 1 relu, 2 silu)
     int tiles_m, tiles_n;
     int splits;              // K slices (grid = tiles_m * tiles_n * splits workgroups)
     // Tail split (splits == 1 only): when the tile count is a little over a multiple of the CU count, the last
@@ -77,6 +78,19 @@ struct GemmArgs
     int64_t tail_kps;
     float *tail_ws;
 };
+
+// the activations a convolution's epilogue can apply; the expressions are those of the standalone unary kernels
+__device__ inline float apply_act(float v, int act)
+{
+    if (act == 1)
+        return v > 0.f ? v : 0.f;
+    if (act == 2)
+    {
+        const float s = 1.0f / (1.0f + expf(-v));
+        return v * s;
+    }
+    return v;
+}
 
 __device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
 {
@@ -534,7 +548,7 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
                 {
                     if (g.bias)
                         v = v + g.bias[row];
-                    Cout[nchw_base + row * g.P] = v;
+                    Cout[nchw_base + row * g.P] = apply_act(v, g.act);
                 }
                 else
                 {
@@ -551,7 +565,7 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
 constexpr int kRedGroups = 16;
 __global__ __launch_bounds__(64 * kRedGroups) void splitk_reduce_kernel(const float *__restrict__ part, int splits,
                                                                          int64_t stride, float *out, int64_t M, int64_t N,
-                                                                         int64_t ldc, const float *bias, int64_t P)
+                                                                         int64_t ldc, const float *bias, int64_t P, int act)
 {
     __shared__ float sh[kRedGroups][64];
     const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
@@ -574,7 +588,7 @@ __global__ __launch_bounds__(64 * kRedGroups) void splitk_reduce_kernel(const fl
             // convolution forward: row = output channel (bias by row), column = n*P + p -> y[n][row][p]
             if (bias)
                 s = s + bias[r];
-            out[((c / P) * M + r) * P + c % P] = s;
+            out[((c / P) * M + r) * P + c % P] = apply_act(s, act);
         }
         else
         {
@@ -589,7 +603,7 @@ __global__ __launch_bounds__(64 * kRedGroups) void splitk_reduce_kernel(const fl
 // ascending order. Needs N % 4 == 0 (and P % 4 == 0) so that a quad stays inside one row (and one image).
 __global__ __launch_bounds__(256) void splitk_reduce_vec_kernel(const float *__restrict__ part, int splits,
                                                                  int64_t stride, float *out, int64_t M, int64_t N,
-                                                                 int64_t ldc, const float *bias, int64_t P)
+                                                                 int64_t ldc, const float *bias, int64_t P, int act)
 {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= M * N)
@@ -609,6 +623,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_vec_kernel(const float *__r
             const float b = bias[r];
             acc[0] = acc[0] + b, acc[1] = acc[1] + b, acc[2] = acc[2] + b, acc[3] = acc[3] + b;
         }
+        acc[0] = apply_act(acc[0], act), acc[1] = apply_act(acc[1], act);
+        acc[2] = apply_act(acc[2], act), acc[3] = apply_act(acc[3], act);
         *reinterpret_cast<f32x4 *>(out + ((c / P) * M + r) * P + c % P) = acc;
     }
     else
@@ -625,16 +641,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_vec_kernel(const float *__r
 // picks the reduction by shape: many slices of a small output -> slice groups in parallel; few slices of a large
 // output -> streaming quads
 void launch_splitk_reduce(const float *part, int splits, int64_t stride, float *out, int64_t M, int64_t N, int64_t ldc,
-                          const float *bias, int64_t P, hipStream_t st)
+                          const float *bias, int64_t P, hipStream_t st, int act = 0)
 {
     const bool quads = splits <= 32 && M * N >= (1 << 16) && N % 4 == 0 && stride % 4 == 0 && ldc % 4 == 0 && P % 4 == 0 &&
                        aligned16(part) && aligned16(out) && (bias == nullptr || P > 0 || aligned16(bias));
     if (quads)
         hipLaunchKernelGGL(splitk_reduce_vec_kernel, dim3((unsigned)odl::ceil_div(M * N, 1024)), dim3(256), 0, st, part,
-                           splits, stride, out, M, N, ldc, bias, P);
+                           splits, stride, out, M, N, ldc, bias, P, act);
     else
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)odl::ceil_div(M * N, 64)), dim3(64 * kRedGroups), 0, st,
-                           part, splits, stride, out, M, N, ldc, bias, P);
+                           part, splits, stride, out, M, N, ldc, bias, P, act);
 }
 
 // Sums the K pieces of each tail tile in piece order and stores the tile through the epilogue the main kernel
@@ -671,7 +687,7 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(GemmArgs g, int BM, int
         {
             if (g.bias)
                 v = v + g.bias[row];
-            g.C[((col / g.P) * g.M + row) * g.P + col % g.P] = v;
+            g.C[((col / g.P) * g.M + row) * g.P + col % g.P] = apply_act(v, g.act);
         }
         else
         {
@@ -826,7 +842,7 @@ namespace odl
 // Shared by the convolution entry points. epi: 0 plain, 1 bias by column, 2 NCHW store with bias by row.
 int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                  const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int epi, int64_t P,
-                 int split_k, void *workspace, size_t workspace_bytes, hipStream_t st)
+                 int split_k, void *workspace, size_t workspace_bytes, hipStream_t st, int act = 0)
 {
     if (M == 0 || N == 0)
         return ODL_OK;
@@ -838,7 +854,7 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
     ODL_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "sgemm: dimension exceeds 2^31");
     GemmArgs g;
     g.A = A, g.B = B, g.C = C, g.bias = bias;
-    g.M = M, g.N = N, g.K = K, g.lda = lda, g.ldb = ldb, g.ldc = ldc, g.P = P;
+    g.M = M, g.N = N, g.K = K, g.lda = lda, g.ldb = ldb, g.ldc = ldc, g.P = P, g.act = act;
     const int tile = pick_tile(M, N);
     g.tiles_m = (int)ceil_div(M, tile), g.tiles_n = (int)ceil_div(N, tile);
     ODL_REQUIRE((int64_t)g.tiles_m * g.tiles_n < (1ll << 31), "sgemm: too many tiles");
@@ -1032,10 +1048,10 @@ size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t OC, int KH,
 // y[n][oc][p] = sum_k W2d[oc][k] * x_gathered[(n,p)][k] + b[oc]
 int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
-                          void *workspace, size_t workspace_bytes, hipStream_t st)
+                          int act, void *workspace, size_t workspace_bytes, hipStream_t st)
 {
     GemmArgs g{};
-    g.A = w, g.B = x, g.C = y, g.bias = b;
+    g.A = w, g.B = x, g.C = y, g.bias = b, g.act = act;
     g.M = OC, g.N = N * OH * OW, g.K = C * KH * KW;
     g.lda = g.K, g.ldb = 0, g.ldc = 0, g.P = OH * OW;
     g.k_per_split = ceil_div(g.K, kBK) * kBK, g.c_split_stride = 0;
@@ -1054,7 +1070,7 @@ int conv_implicit_forward(const float *x, const float *w, const float *b, float 
         if (rc != ODL_OK)
             return fail(rc, "conv2d: no kernel variant");
         ODL_LAUNCH_CHECK();
-        launch_splitk_reduce(static_cast<const float *>(workspace), splits, OC * g.N, y, OC, g.N, g.N, b, g.P, st);
+        launch_splitk_reduce(static_cast<const float *>(workspace), splits, OC * g.N, y, OC, g.N, g.N, b, g.P, st, act);
         ODL_LAUNCH_CHECK();
         return ODL_OK;
     }

@@ -214,6 +214,10 @@ public:
     std::unique_ptr<Mat> softmax(int axis) const;
     float softmax_cross_entropy(const Mat &target) const;                      // loss value (host)
     std::unique_ptr<Mat> softmax_cross_entropy_backward(const Mat &target, float gy) const;
+    // conv2d with an activation applied in the kernel's epilogue: -1 none, 0 relu, 7 silu. Bit-identical to conv2d()
+    // followed by relu() / silu().
+    std::unique_ptr<Mat> conv2d_act(const Mat &W, const Mat *b, std::pair<int, int> stride, std::pair<int, int> pad,
+                                    int activation) const;
     // Max pooling with the window-local indices kept in device memory (uint64 per output). The Mat interface above
     // hands them to the caller as a host vector, which costs a device-to-host copy in forward and a host-to-device
     // copy in backward (the reference's device backend pays both); the pooling operator uses this pair instead.

@@ -2,7 +2,7 @@
 // Same public surface as the reference's origin::pnnx::PNNXGraph (include/origin/pnnx/pnnx_graph.h:20-60):
 // construct with the two paths, build(), set_inputs(name, tensors), forward(), get_outputs(name).
 //
-// Differences that do not change results: weights are uploaded to the device once (at the first forward on that
+// Differences that do not change results: a convolution followed only by SiLU / ReLU runs as one kernel; weights are uploaded to the device once (at the first forward on that
 // device) and kept, where the reference rebuilds every weight tensor from host data on every forward
 // (src/pnnx/pnnx_graph.cpp:341-405); nodes run on Mat objects directly, without building an autograd graph.
 #pragma once
@@ -32,6 +32,11 @@ struct PNNXNode
     std::map<std::string, Attribute> attributes;
     std::map<int, std::vector<int>> shapes;
     int execution_order = -1;
+    // set by build(): a convolution whose only reader is an activation applies it in its own epilogue and writes that
+    // node's output; the activation node is then skipped
+    int fused_activation = -1;       // -1 none, 0 relu, 7 silu
+    std::string fused_output_name;   // the activation node's output
+    bool folded_into_producer = false;
 };
 
 class PNNXGraph

@@ -733,6 +733,12 @@ std::unique_ptr<Mat> OriginMat::col2im(const Shape &is, std::pair<int, int> k, s
 
 std::unique_ptr<Mat> OriginMat::conv2d(const Mat &Wm, const Mat *bm, std::pair<int, int> s, std::pair<int, int> p) const
 {
+    return conv2d_act(Wm, bm, s, p, -1);
+}
+
+std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pair<int, int> s, std::pair<int, int> p,
+                                           int activation) const
+{
     const OriginMat &x = dev_f32(*this, "conv2d");
     const OriginMat &w = dev_f32(Wm, "conv2d");
     if (shape_.size() != 4)
@@ -759,8 +765,8 @@ std::unique_ptr<Mat> OriginMat::conv2d(const Mat &Wm, const Mat *bm, std::pair<i
     auto y = new_like(x, Shape{(size_t)N, (size_t)OC, (size_t)OH, (size_t)OW});
     Workspace ws(odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
                  device().index());
-    check(odl_hip_conv2d(fp(x), fp(w), bias, N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
-                         y->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+    check(odl_hip_conv2d_act(fp(x), fp(w), bias, N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
+                             activation, y->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
     return y;
 }
 

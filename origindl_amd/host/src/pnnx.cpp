@@ -305,6 +305,24 @@ void PNNXGraph::build()
     for (auto &n : nodes_)
         if (n->type != "pnnx.Input" && n->execution_order < 0)
             THROW_RUNTIME_ERROR("PNNX: node {} is part of a cycle", n->name);
+    // conv -> activation pairs: the activation moves into the convolution's epilogue when nobody else reads the
+    // convolution's output
+    std::map<std::string, int> readers;
+    for (auto &n : nodes_)
+        for (auto &in : n->input_names)
+            ++readers[in];
+    for (auto &n : plan_)
+    {
+        if ((n->type != "nn.SiLU" && n->type != "nn.ReLU") || n->input_names.size() != 1 || n->output_names.size() != 1)
+            continue;
+        auto pit = producer.find(n->input_names[0]);
+        if (pit == producer.end() || pit->second->type != "nn.Conv2d" || readers[n->input_names[0]] != 1 ||
+            pit->second->output_names.size() != 1)
+            continue;
+        pit->second->fused_activation = n->type == "nn.SiLU" ? 7 : 0;
+        pit->second->fused_output_name = n->output_names[0];
+        n->folded_into_producer = true;
+    }
     static const char *known[] = {"nn.Conv2d",  "nn.SiLU",        "nn.ReLU",   "nn.Upsample",        "nn.MaxPool2d", "pnnx.Expression",
                                   "torch.cat",  "torch.flatten", "nn.Linear", "models.yolo.Detect"};
     for (auto &n : plan_)
@@ -359,6 +377,8 @@ std::vector<Tensor> PNNXGraph::get_outputs(const std::string &output_name) const
 
 void PNNXGraph::run(PNNXNode &node)
 {
+    if (node.folded_into_producer)
+        return;  // its producer already wrote this node's output
     std::vector<std::shared_ptr<Mat>> in;
     for (auto &name : node.input_names)
     {
@@ -386,7 +406,8 @@ void PNNXGraph::run(PNNXNode &node)
         if (!w)
             THROW_RUNTIME_ERROR("PNNX: node {} has no weight", node.name);
         auto b = weight("bias");
-        out = in[0]->conv2d(*w, b.get(), int_pair(node, "stride", {1, 1}), int_pair(node, "padding", {0, 0}));
+        out = origin_of(*in[0]).conv2d_act(*w, b.get(), int_pair(node, "stride", {1, 1}), int_pair(node, "padding", {0, 0}),
+                                          node.fused_activation);
     }
     else if (t == "nn.SiLU")
         out = in[0]->silu();
@@ -502,8 +523,7 @@ void PNNXGraph::run(PNNXNode &node)
     if (node.output_names.size() != 1)
         THROW_RUNTIME_ERROR("PNNX: node {} declares {} outputs; this runner's operators produce one", node.name,
                             node.output_names.size());
-    (void)origin_of(*out);
-    blobs_[node.output_names[0]] = std::move(out);
+    blobs_[node.fused_output_name.empty() ? node.output_names[0] : node.fused_output_name] = std::move(out);
 }
 }  // namespace pnnx
 }  // namespace origin

@@ -679,3 +679,22 @@ def test_yolo_detect_at_detector_size_vs_oracle(api, o):
     # transform (at most x2*stride, or x4*2s*anchor)
     np.testing.assert_allclose(got[..., 4:], want[..., 4:], rtol=0, atol=2e-6)
     np.testing.assert_allclose(got[..., :4], want[..., :4], rtol=2e-5, atol=2e-4)
+
+
+@pytest.mark.parametrize("N,C,H,OC,k,s,p", [
+    (2, 16, 14, 24, 3, 1, 1),     # implicit forward, one pass
+    (2, 1, 28, 32, 3, 1, 1),      # C*9 = 9: explicit im2col + GEMM
+    (8, 128, 14, 256, 3, 2, 1),   # few tiles: K slices summed by the reduction kernel
+    (4, 64, 56, 128, 3, 1, 1),    # tile count just over a multiple of the CU count: tail pieces and their fix-up
+    (2, 64, 20, 128, 1, 1, 0),    # 1x1
+])
+def test_conv_with_fused_activation_is_conv_then_activation(api, N, C, H, OC, k, s, p):
+    rng = np.random.default_rng(41)
+    x = dev(rng.standard_normal((N, C, H, H), dtype=f32))
+    w = dev((rng.standard_normal((OC, C, k, k), dtype=f32) * f32(np.sqrt(2.0 / (C * k * k)))).astype(f32))
+    b = dev(rng.standard_normal(OC, dtype=f32))
+    plain = api.conv2d(x, w, b, s, p)
+    for act in ("silu", "relu"):
+        assert np.array_equal(host(api.conv2d(x, w, b, s, p, activation=act)), host(api.unary(act, plain))), act
+    with pytest.raises(api.OdlInvalidArgument):
+        api.conv2d(x, w, b, s, p, activation="exp")
