@@ -155,6 +155,28 @@ def extras(torch, capi, steps, warmup):
                                        stream), steps, warmup)
         nb = 8.0 * N * C + 8.0 * N
         out[name] = {"ms": ms, "gbs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+    # config 2's other shapes: forward + both gradient GEMMs, 6*M*N*K FLOP per step
+    for (M, K, N) in ((1024, 1024, 1024), (2048, 2048, 2048), (8192, 8192, 8192), (512, 784, 1000), (512, 1000, 10)):
+        a, b, dc = rnd(M, K), rnd(K, N), rnd(M, N)
+        c, da, db = empty(M, N), empty(M, K), empty(K, N)
+        wsz = max(L.query("odl_hip_matmul_backward_workspace_bytes", M, K, N),
+                  L.query("odl_hip_matmul_workspace_bytes", 1, M, N, K, 0))
+        wp, nw = ws(wsz)
+        fwd = direct("odl_hip_matmul", ptr(a), ptr(b), ptr(c), 1, M, N, K, 0, wp, nw, stream)
+        bwd = direct("odl_hip_matmul_backward", ptr(a), ptr(b), ptr(dc), ptr(da), ptr(db), M, K, N, wp, nw, stream)
+        n = 3 if M >= 8192 else steps
+
+        def both():
+            fwd()
+            bwd()
+
+        ms = time_region(torch, both, n, 1 if M >= 8192 else warmup)
+        flop = 6.0 * M * N * K
+        tf = flop / ms / 1e9
+        out["gemm_fwd_bwd_%dx%dx%d" % (M, K, N)] = {"ms": ms, "tflops": tf, "frac_mfma_peak": tf / PEAK_FP32_MFMA_TFLOPS,
+                                                      "flop": flop}
+        del a, b, dc, c, da, db
+        keep.clear()
     # the MLP's six GEMMs (config 1): 512x784x1000 and 512x1000x10, forward + backward
     x1, w1, g1 = rnd(512, 784), rnd(784, 1000), rnd(512, 1000)
     x2, w2, g2 = rnd(512, 1000), rnd(1000, 10), rnd(512, 10)
