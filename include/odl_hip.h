@@ -177,8 +177,10 @@ int odl_hip_accuracy(const float *y, const int32_t *t, int64_t N, int64_t C, flo
 size_t odl_hip_accuracy_workspace_bytes(int64_t N);
 
 /* ------------------------------------------------------------------ elementwise --------------------- */
-/* origin::cuda::{add,subtract,multiply,divide,gt} (cuda_ops.cuh:57-140): op 0 add, 1 sub, 2 mul, 3 div,
- * 4 greater-than mask (1.0f / 0.0f). na == nb, or one side has a single element; anything else is the
+/* origin::cuda::{add,subtract,multiply,divide,gt,eq,ne,lt,le,ge} (cuda_ops.cuh:57-140): op 0 add, 1 sub, 2 mul, 3 div,
+ * 4 greater-than, 5 equal, 6 not-equal, 7 less, 8 less-equal, 9 greater-equal (masks of 1.0f / 0.0f);
+ * 10 sigmoid_backward(a = gy, b = y) = gy*y*(1-y) (mat.h:399), 11 silu_backward(a = gy, b = x) (mat.h:413).
+ * na == nb, or one side has a single element; anything else is the
  * reference's "complex broadcasting" runtime_error. out may alias a or b (add_inplace). */
 int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t nb, float *out, void *stream);
 /* origin::cuda::{relu,exp,log,negate,square,sqrt,sigmoid,silu}: op 0 relu, 1 exp, 2 log, 3 neg, 4 square, 5 sqrt,
@@ -193,6 +195,14 @@ int odl_hip_upsample_nearest(const float *x, int64_t N, int64_t C, int64_t H, in
                              int scale_h, int scale_w, float *y, void *stream);
 /* Mat::cat (mat.h:797; src/mat/origin/cpu/shape/cat.cpp:20-140): inputs viewed as [outer, axis_size_i, inner] are laid
  * side by side along the axis. host_inputs: `count` device pointers in a host array; host_axis_sizes: their axis extents. */
+/* Mat::upsample_backward (mat.h:784; nn/upsample.cpp:80-135): each input pixel sums the scale_h x scale_w block of gy
+ * it was copied to, rows then columns ascending (the reference's accumulation order: bit-identical). */
+int odl_hip_upsample_nearest_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
+                                      int scale_h, int scale_w, float *gx, void *stream);
+/* Mat::split, one piece (mat.h:805; src/mat/origin/cpu/shape/split.cpp) — the backward of cat: src viewed as
+ * [outer, axis_size, inner], dst = src[:, offset:offset+length, :]. */
+int odl_hip_slice_axis(const float *src, int64_t outer, int64_t axis_size, int64_t inner, int64_t offset, int64_t length,
+                       float *dst, void *stream);
 int odl_hip_cat(const float *const *host_inputs, const int64_t *host_axis_sizes, int count, int64_t outer, int64_t inner,
                 float *out, void *stream);
 /* Mat::yolo_detect_forward (mat.h:719; src/mat/origin/cpu/custom/yolo_detect.cpp:28-166): 1x1 convolution

@@ -32,13 +32,16 @@ __global__ __launch_bounds__(kBlock) void upsample_nearest_kernel(const float *_
     y[t] = x[(int64_t)nc * H * W + (oh / sh) * W + ow / sw];
 }
 
-// dst[m][off + j] = src[m][j] for j < chunk: `outer` contiguous runs; grid (run pieces, m)
+// dst[m*dst_stride + dst_off + j] = src[m*src_stride + src_off + j] for j < chunk: `outer` contiguous runs;
+// grid (run pieces, m). Concatenation scatters whole inputs (src_stride = chunk, src_off = 0); its backward, split,
+// gathers a slice (dst_stride = chunk, dst_off = 0).
 template <bool VEC>
 __global__ __launch_bounds__(kBlock) void cat_copy_kernel(const float *__restrict__ src, float *__restrict__ dst,
-                                                          int64_t chunk, int64_t dst_stride, int64_t dst_off)
+                                                          int64_t chunk, int64_t src_stride, int64_t src_off,
+                                                          int64_t dst_stride, int64_t dst_off)
 {
     const int64_t m = blockIdx.y;
-    const float *s = src + m * chunk;
+    const float *s = src + m * src_stride + src_off;
     float *d = dst + m * dst_stride + dst_off;
     const int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * (VEC ? 4 : 1);
     if (VEC)
@@ -51,6 +54,35 @@ __global__ __launch_bounds__(kBlock) void cat_copy_kernel(const float *__restric
     }
     else if (i < chunk)
         d[i] = s[i];
+}
+
+// gx[nc][h][w] = sum over the scale_h x scale_w block of gy it was copied to, rows then columns ascending — the order
+// in which the reference's loop over gy reaches that input pixel (nn/upsample.cpp:113-131)
+__global__ __launch_bounds__(kBlock) void upsample_nearest_bwd_kernel(const float *__restrict__ gy, float *__restrict__ gx,
+                                                                      unsigned planes, int H, int W, int OH, int OW, int sh,
+                                                                      int sw)
+{
+    const unsigned plane = (unsigned)(H * W);
+    const unsigned t = blockIdx.x * (unsigned)kBlock + threadIdx.x;
+    if (t >= planes * plane)
+        return;
+    const unsigned nc = t / plane, r = t - nc * plane;
+    const int h = (int)(r / (unsigned)W), w = (int)r - h * W;
+    const float *p = gy + (int64_t)nc * OH * OW;
+    float acc = 0.f;
+    for (int i = 0; i < sh; ++i)
+    {
+        const int oh = h * sh + i;
+        if (oh >= OH)
+            break;
+        for (int j = 0; j < sw; ++j)
+        {
+            const int ow = w * sw + j;
+            if (ow < OW)
+                acc += p[oh * OW + ow];
+        }
+    }
+    gx[t] = acc;
 }
 
 // conv[b][a*CI + c][h][w] -> out[b][(a*H + h)*W + w][c], sigmoid, then the box transform on c = 0..3.
@@ -175,15 +207,64 @@ int odl_hip_cat(const float *const *host_inputs, const int64_t *host_axis_sizes,
                 float *d = out + m0 * dst_stride;
                 if (vec)
                     hipLaunchKernelGGL((cat_copy_kernel<true>), dim3((unsigned)odl::ceil_div(chunk / 4, kBlock), (unsigned)ms),
-                                       dim3(kBlock), 0, st, s, d, chunk, dst_stride, dst_off);
+                                       dim3(kBlock), 0, st, s, d, chunk, chunk, (int64_t)0, dst_stride, dst_off);
                 else
                     hipLaunchKernelGGL((cat_copy_kernel<false>), dim3((unsigned)odl::ceil_div(chunk, kBlock), (unsigned)ms),
-                                       dim3(kBlock), 0, st, s, d, chunk, dst_stride, dst_off);
+                                       dim3(kBlock), 0, st, s, d, chunk, chunk, (int64_t)0, dst_stride, dst_off);
                 ODL_LAUNCH_CHECK();
             }
         }
         off += host_axis_sizes[i];
     }
+    return ODL_OK;
+}
+
+int odl_hip_slice_axis(const float *src, int64_t outer, int64_t axis_size, int64_t inner, int64_t offset, int64_t length,
+                       float *dst, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(outer >= 0 && axis_size >= 0 && inner >= 0 && outer < 65536 * 32768ll, "slice: bad extents");
+    ODL_REQUIRE(offset >= 0 && length >= 0 && offset + length <= axis_size, "slice: [%lld, %lld) lies outside an axis of %lld",
+                (long long)offset, (long long)(offset + length), (long long)axis_size);
+    const int64_t chunk = length * inner;
+    if (chunk == 0 || outer == 0)
+        return ODL_OK;
+    ODL_REQUIRE(src && dst, "slice: null operand");
+    hipStream_t st = odl::as_stream(stream);
+    const int64_t src_stride = axis_size * inner, src_off = offset * inner;
+    const bool vec = chunk % 4 == 0 && src_stride % 4 == 0 && src_off % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+    for (int64_t m0 = 0; m0 < outer; m0 += 65535)
+    {
+        const int64_t ms = outer - m0 < 65535 ? outer - m0 : 65535;
+        const float *s = src + m0 * src_stride;
+        float *d = dst + m0 * chunk;
+        if (vec)
+            hipLaunchKernelGGL((cat_copy_kernel<true>), dim3((unsigned)odl::ceil_div(chunk / 4, kBlock), (unsigned)ms), dim3(kBlock),
+                               0, st, s, d, chunk, src_stride, src_off, chunk, (int64_t)0);
+        else
+            hipLaunchKernelGGL((cat_copy_kernel<false>), dim3((unsigned)odl::ceil_div(chunk, kBlock), (unsigned)ms), dim3(kBlock), 0,
+                               st, s, d, chunk, src_stride, src_off, chunk, (int64_t)0);
+        ODL_LAUNCH_CHECK();
+    }
+    return ODL_OK;
+}
+
+int odl_hip_upsample_nearest_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
+                                      int scale_h, int scale_w, float *gx, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C >= 0 && H > 0 && W > 0 && OH > 0 && OW > 0, "upsample backward: bad shape");
+    ODL_REQUIRE(scale_h > 0 && scale_w > 0, "upsample backward: scale must be positive");
+    ODL_REQUIRE((OH - 1) / scale_h < H && (OW - 1) / scale_w < W, "upsample backward: gradient (%lld,%lld) reaches past input (%lld,%lld)",
+                (long long)OH, (long long)OW, (long long)H, (long long)W);
+    const int64_t total = N * C * H * W;
+    if (total == 0)
+        return ODL_OK;
+    ODL_REQUIRE(total < (1ll << 32) - kBlock && H * W < (1ll << 31) && OH * OW < (1ll << 31), "upsample backward: too large");
+    hipLaunchKernelGGL(upsample_nearest_bwd_kernel, dim3((unsigned)odl::ceil_div(total, kBlock)), dim3(kBlock), 0,
+                       odl::as_stream(stream), gy, gx, (unsigned)(N * C), (int)H, (int)W, (int)OH, (int)OW, scale_h, scale_w);
+    ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
 

@@ -17,7 +17,24 @@ __device__ inline float bin(float a, float b)
     if (OP == 1) return a - b;
     if (OP == 2) return a * b;
     if (OP == 3) return a / b;
-    return (a > b) ? 1.f : 0.f;
+    // comparisons give a 0/1 mask in the operands' own type (operation_templates.h:177-240)
+    if (OP == 4) return (a > b) ? 1.f : 0.f;
+    if (OP == 5) return (a == b) ? 1.f : 0.f;
+    if (OP == 6) return (a != b) ? 1.f : 0.f;
+    if (OP == 7) return (a < b) ? 1.f : 0.f;
+    if (OP == 8) return (a <= b) ? 1.f : 0.f;
+    if (OP == 9) return (a >= b) ? 1.f : 0.f;
+    // backward halves of the activations, a = upstream gradient:
+    if (OP == 10)  // sigmoid: b = y = sigmoid(x); gy*y*(1-y) (cpu/activation/sigmoid.cpp:93)
+    {
+        const float t = a * b;
+        return t * (1.0f - b);
+    }
+    // silu: b = x; gy*(s + x*s*(1-s)) with s = sigmoid(x) (cpu/activation/silu.cpp:87-90)
+    const float sg = 1.0f / (1.0f + expf(-b));
+    const float xs = b * sg;
+    const float g = sg + xs * (1.0f - sg);
+    return a * g;
 }
 
 template <int OP>
@@ -252,7 +269,7 @@ extern "C" {
 int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t nb, float *out, void *stream)
 {
     ODL_REQUIRE_DEVICE();
-    ODL_REQUIRE(op >= 0 && op <= 4, "binary: unknown op %d", op);
+    ODL_REQUIRE(op >= 0 && op <= 11, "binary: unknown op %d", op);
     ODL_REQUIRE(na >= 0 && nb >= 0, "binary: negative extent");
     if (!(na == nb || na == 1 || nb == 1))
         return odl::fail(ODL_ERR_RUNTIME, "Complex broadcasting not yet implemented (%lld vs %lld elements)",
@@ -266,7 +283,14 @@ int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t n
         case 1: return launch_binary<1>(a, na, b, nb, out, st);
         case 2: return launch_binary<2>(a, na, b, nb, out, st);
         case 3: return launch_binary<3>(a, na, b, nb, out, st);
-        default: return launch_binary<4>(a, na, b, nb, out, st);
+        case 4: return launch_binary<4>(a, na, b, nb, out, st);
+        case 5: return launch_binary<5>(a, na, b, nb, out, st);
+        case 6: return launch_binary<6>(a, na, b, nb, out, st);
+        case 7: return launch_binary<7>(a, na, b, nb, out, st);
+        case 8: return launch_binary<8>(a, na, b, nb, out, st);
+        case 9: return launch_binary<9>(a, na, b, nb, out, st);
+        case 10: return launch_binary<10>(a, na, b, nb, out, st);
+        default: return launch_binary<11>(a, na, b, nb, out, st);
     }
 }
 

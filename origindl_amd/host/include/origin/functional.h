@@ -3,6 +3,8 @@
 // add sub mul div neg pow exp log square sum sum_to broadcast_to mat_mul reshape transpose flatten relu softmax
 // softmax_cross_entropy conv2d max_pool2d.
 #pragma once
+#include <string>
+
 #include "tensor.h"
 
 namespace origin
@@ -26,6 +28,20 @@ Tensor reshape(const Tensor &x, const Shape &shape);
 Tensor transpose(const Tensor &x);
 Tensor flatten(const Tensor &x, int start_dim = 1, int end_dim = -1);
 Tensor relu(const Tensor &x);
+Tensor sigmoid(const Tensor &x);
+Tensor silu(const Tensor &x);
+Tensor cat(const std::vector<Tensor> &xs, int dim = 0);
+Tensor upsample(const Tensor &x, const std::string &mode = "nearest", std::pair<float, float> scale_factor = {2.0f, 2.0f});
+// in-place forms: overwrite the left operand's storage
+void add_(Tensor &lhs, const Tensor &rhs);
+void sub_(Tensor &lhs, const Tensor &rhs);
+void mul_(Tensor &lhs, const Tensor &rhs);
+void div_(Tensor &lhs, const Tensor &rhs);
+void neg_(Tensor &x);
+void exp_(Tensor &x);
+void log_(Tensor &x);
+void square_(Tensor &x);
+void relu_(Tensor &x);
 Tensor softmax(const Tensor &x, int axis = -1);
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &target);
 Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b = nullptr, std::pair<int, int> stride = {1, 1},
@@ -54,6 +70,20 @@ Tensor operator-(const Tensor &x);
 Tensor operator^(const Tensor &base, const Scalar &exponent);
 Tensor operator>(const Tensor &lhs, const Tensor &rhs);
 Tensor operator>(const Tensor &lhs, const Scalar &rhs);
+Tensor operator==(const Tensor &lhs, const Tensor &rhs);
+Tensor operator==(const Tensor &lhs, const Scalar &rhs);
+Tensor operator!=(const Tensor &lhs, const Tensor &rhs);
+Tensor operator!=(const Tensor &lhs, const Scalar &rhs);
+Tensor operator<(const Tensor &lhs, const Tensor &rhs);
+Tensor operator<(const Tensor &lhs, const Scalar &rhs);
+Tensor operator<=(const Tensor &lhs, const Tensor &rhs);
+Tensor operator<=(const Tensor &lhs, const Scalar &rhs);
+Tensor operator>=(const Tensor &lhs, const Tensor &rhs);
+Tensor operator>=(const Tensor &lhs, const Scalar &rhs);
+Tensor &operator+=(Tensor &lhs, const Scalar &rhs);
+Tensor &operator-=(Tensor &lhs, const Scalar &rhs);
+Tensor &operator*=(Tensor &lhs, const Scalar &rhs);
+Tensor &operator/=(Tensor &lhs, const Scalar &rhs);
 Tensor &operator+=(Tensor &lhs, const Tensor &rhs);
 Tensor &operator-=(Tensor &lhs, const Tensor &rhs);
 Tensor &operator*=(Tensor &lhs, const Tensor &rhs);

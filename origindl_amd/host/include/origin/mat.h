@@ -69,12 +69,21 @@ public:
     virtual std::unique_ptr<Mat> operator*(const Mat &other) const     = 0;
     virtual std::unique_ptr<Mat> operator/(const Mat &other) const     = 0;
     virtual std::unique_ptr<Mat> operator>(const Mat &other) const     = 0;
+    virtual std::unique_ptr<Mat> operator==(const Mat &other) const    = 0;
+    virtual std::unique_ptr<Mat> operator!=(const Mat &other) const    = 0;
+    virtual std::unique_ptr<Mat> operator<(const Mat &other) const     = 0;
+    virtual std::unique_ptr<Mat> operator<=(const Mat &other) const    = 0;
+    virtual std::unique_ptr<Mat> operator>=(const Mat &other) const    = 0;
     virtual std::unique_ptr<Mat> operator-() const                     = 0;
     virtual void add_inplace(const Mat &other)                         = 0;
     virtual void sub_inplace(const Mat &other)                         = 0;
     virtual void mul_inplace(const Mat &other)                         = 0;
     virtual void div_inplace(const Mat &other)                         = 0;
     virtual void neg_inplace()                                         = 0;
+    virtual void exp_inplace()                                         = 0;
+    virtual void log_inplace()                                         = 0;
+    virtual void square_inplace()                                      = 0;
+    virtual void relu_inplace()                                        = 0;
     virtual Mat &operator+=(const Mat &other)                          = 0;
     virtual Mat &operator-=(const Mat &other)                          = 0;
     virtual Mat &operator*=(const Mat &other)                          = 0;
@@ -94,6 +103,11 @@ public:
     virtual std::unique_ptr<Mat> relu() const                          = 0;
     virtual std::unique_ptr<Mat> sigmoid() const                       = 0;
     virtual std::unique_ptr<Mat> silu() const                          = 0;
+    virtual std::unique_ptr<Mat> sigmoid_backward(const Mat &y) const  = 0;  // this = gy, y = sigmoid(x)
+    virtual std::unique_ptr<Mat> silu_backward(const Mat &x) const     = 0;  // this = gy
+    virtual std::unique_ptr<Mat> upsample_backward(const Mat &gy, const Shape &x_shape, int scale_h, int scale_w,
+                                                   const std::string &mode = "nearest") const = 0;
+    virtual std::vector<std::unique_ptr<Mat>> split(const std::vector<size_t> &split_sizes, int dim) const = 0;
     // ---- detector forward path (mat.h:719-797 of the reference)
     virtual std::unique_ptr<Mat> upsample(const Shape &output_shape, int scale_h, int scale_w,
                                           const std::string &mode = "nearest") const = 0;
@@ -161,12 +175,21 @@ public:
     std::unique_ptr<Mat> operator*(const Mat &other) const override;
     std::unique_ptr<Mat> operator/(const Mat &other) const override;
     std::unique_ptr<Mat> operator>(const Mat &other) const override;
+    std::unique_ptr<Mat> operator==(const Mat &other) const override;
+    std::unique_ptr<Mat> operator!=(const Mat &other) const override;
+    std::unique_ptr<Mat> operator<(const Mat &other) const override;
+    std::unique_ptr<Mat> operator<=(const Mat &other) const override;
+    std::unique_ptr<Mat> operator>=(const Mat &other) const override;
     std::unique_ptr<Mat> operator-() const override;
     void add_inplace(const Mat &other) override;
     void sub_inplace(const Mat &other) override;
     void mul_inplace(const Mat &other) override;
     void div_inplace(const Mat &other) override;
     void neg_inplace() override;
+    void exp_inplace() override;
+    void log_inplace() override;
+    void square_inplace() override;
+    void relu_inplace() override;
     Mat &operator+=(const Mat &other) override;
     Mat &operator-=(const Mat &other) override;
     Mat &operator*=(const Mat &other) override;
@@ -186,6 +209,11 @@ public:
     std::unique_ptr<Mat> relu() const override;
     std::unique_ptr<Mat> sigmoid() const override;
     std::unique_ptr<Mat> silu() const override;
+    std::unique_ptr<Mat> sigmoid_backward(const Mat &y) const override;
+    std::unique_ptr<Mat> silu_backward(const Mat &x) const override;
+    std::unique_ptr<Mat> upsample_backward(const Mat &gy, const Shape &x_shape, int scale_h, int scale_w,
+                                           const std::string &mode = "nearest") const override;
+    std::vector<std::unique_ptr<Mat>> split(const std::vector<size_t> &split_sizes, int dim) const override;
     std::unique_ptr<Mat> upsample(const Shape &output_shape, int scale_h, int scale_w,
                                   const std::string &mode = "nearest") const override;
     std::unique_ptr<Mat> cat(const std::vector<const Mat *> &others, int dim) const override;

@@ -2,6 +2,9 @@
 // softmax-cross-entropy go to the fused device kernels instead of the reference's chain of eight Mat ops.
 #include "origin/functional.h"
 
+#include <cmath>
+#include <string>
+
 namespace origin
 {
 namespace functional
@@ -356,6 +359,85 @@ struct MaxPool2d : Operator  // src/operators/pooling/max_pool2d.cpp:14-86
     }
 };
 
+struct Sigmoid : Operator  // src/operators/activation/sigmoid.cpp:13-44: keeps y, gx = gy*y*(1-y)
+{
+    Tensor y;
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        y = wrap(mat(xs[0]).sigmoid());
+        return {y};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {wrap(mat(gys[0]).sigmoid_backward(mat(y)))};
+    }
+};
+
+struct SiLU : Operator  // src/operators/activation/silu.cpp: gx = gy*(s + x*s*(1-s))
+{
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).silu())}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {wrap(mat(gys[0]).silu_backward(mat(inputs_[0])))};
+    }
+};
+
+struct Cat : Operator  // src/operators/shape/cat.cpp: backward splits the gradient back along dim
+{
+    int dim;
+    std::vector<size_t> sizes;
+    explicit Cat(int d) : dim(d) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        if (xs.empty())
+            THROW_RUNTIME_ERROR("cat: requires at least 1 input");
+        std::vector<const Mat *> others;
+        sizes.clear();
+        for (size_t i = 0; i < xs.size(); ++i)
+        {
+            if (dim < 0 || (size_t)dim >= xs[i].shape().size())
+                THROW_RUNTIME_ERROR("cat: dimension {} out of range for shape {}", dim, xs[i].shape().to_string());
+            sizes.push_back(xs[i].shape()[dim]);
+            if (i)
+                others.push_back(&mat(xs[i]));
+        }
+        return {wrap(mat(xs[0]).cat(others, dim))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        std::vector<Tensor> out;
+        for (auto &piece : mat(gys[0]).split(sizes, dim))
+            out.push_back(wrap(std::move(piece)));
+        return out;
+    }
+};
+
+struct Upsample : Operator  // src/operators/nn/upsample.cpp:13-90
+{
+    std::string mode;
+    std::pair<float, float> scale;
+    std::pair<int, int> size;
+    int sh = 1, sw = 1;
+    Upsample(const std::string &m, std::pair<float, float> sc, std::pair<int, int> sz) : mode(m), scale(sc), size(sz) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        const Shape s = xs[0].shape();
+        if (s.size() != 4)
+            THROW_RUNTIME_ERROR("Upsample forward: x must be 4D (N, C, H, W), but got shape {}", s.to_string());
+        size_t OH, OW;
+        if (size.first > 0 && size.second > 0)
+            OH = (size_t)size.first, OW = (size_t)size.second;
+        else
+            OH = (size_t)std::lround(s[2] * scale.first), OW = (size_t)std::lround(s[3] * scale.second);
+        sh = (int)(OH / s[2]), sw = (int)(OW / s[3]);
+        return {wrap(mat(xs[0]).upsample(Shape{s[0], s[1], OH, OW}, sh, sw, mode))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {wrap(mat(inputs_[0]).upsample_backward(mat(gys[0]), inputs_[0].shape(), sh, sw, mode))};
+    }
+};
+
 template <typename Op, typename... A>
 Tensor apply(const std::vector<Tensor> &xs, A &&...args)
 {
@@ -380,6 +462,28 @@ Tensor mat_mul(const Tensor &x, const Tensor &w) { return apply<MatMul>({x, w});
 Tensor reshape(const Tensor &x, const Shape &s) { return apply<Reshape>({x}, s); }
 Tensor transpose(const Tensor &x) { return apply<Transpose>({x}); }
 Tensor relu(const Tensor &x) { return apply<ReLU>({x}); }
+Tensor sigmoid(const Tensor &x) { return apply<Sigmoid>({x}); }
+Tensor silu(const Tensor &x) { return apply<SiLU>({x}); }
+Tensor cat(const std::vector<Tensor> &xs, int dim) { return apply<Cat>(xs, dim); }
+Tensor upsample(const Tensor &x, const std::string &mode, std::pair<float, float> scale_factor)
+{
+    return apply<Upsample>({x}, mode, scale_factor, std::make_pair(0, 0));
+}
+
+// in-place forms: the left operand's storage is overwritten (src/operators/math/add.cpp:57-100 and its siblings)
+namespace
+{
+Mat &writable(Tensor &t) { return *t.impl_->data_; }
+}  // namespace
+void add_(Tensor &a, const Tensor &b) { writable(a).add_inplace(*b.impl_->data_); }
+void sub_(Tensor &a, const Tensor &b) { writable(a).sub_inplace(*b.impl_->data_); }
+void mul_(Tensor &a, const Tensor &b) { writable(a).mul_inplace(*b.impl_->data_); }
+void div_(Tensor &a, const Tensor &b) { writable(a).div_inplace(*b.impl_->data_); }
+void neg_(Tensor &x) { writable(x).neg_inplace(); }
+void exp_(Tensor &x) { writable(x).exp_inplace(); }
+void log_(Tensor &x) { writable(x).log_inplace(); }
+void square_(Tensor &x) { writable(x).square_inplace(); }
+void relu_(Tensor &x) { writable(x).relu_inplace(); }
 Tensor softmax(const Tensor &x, int axis) { return apply<Softmax>({x}, axis); }
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &t) { return apply<SoftmaxCrossEntropy>({x, t}); }
 
@@ -449,10 +553,24 @@ Tensor operator-(const Tensor &x) { return F::neg(x); }
 Tensor operator^(const Tensor &x, const Scalar &e) { return F::pow(x, e); }
 Tensor operator>(const Tensor &a, const Tensor &b) { return Tensor(*a.impl_->data_ > *b.impl_->data_); }
 Tensor operator>(const Tensor &a, const Scalar &b) { return a > scalar_of(b, a); }
-Tensor &operator+=(Tensor &a, const Tensor &b) { a = a + b; return a; }
-Tensor &operator-=(Tensor &a, const Tensor &b) { a = a - b; return a; }
-Tensor &operator*=(Tensor &a, const Tensor &b) { a = a * b; return a; }
-Tensor &operator/=(Tensor &a, const Tensor &b) { a = a / b; return a; }
+#define ODL_COMPARE(OP)                                                                                     \
+    Tensor operator OP(const Tensor &a, const Tensor &b) { return Tensor(*a.impl_->data_ OP * b.impl_->data_); } \
+    Tensor operator OP(const Tensor &a, const Scalar &b) { return a OP scalar_of(b, a); }
+ODL_COMPARE(==)
+ODL_COMPARE(!=)
+ODL_COMPARE(<)
+ODL_COMPARE(<=)
+ODL_COMPARE(>=)
+#undef ODL_COMPARE
+// compound assignment works in place on the left operand's storage, as the reference's does (add.cpp:121-133)
+Tensor &operator+=(Tensor &a, const Tensor &b) { F::add_(a, b); return a; }
+Tensor &operator-=(Tensor &a, const Tensor &b) { F::sub_(a, b); return a; }
+Tensor &operator*=(Tensor &a, const Tensor &b) { F::mul_(a, b); return a; }
+Tensor &operator/=(Tensor &a, const Tensor &b) { F::div_(a, b); return a; }
+Tensor &operator+=(Tensor &a, const Scalar &b) { F::add_(a, scalar_of(b, a)); return a; }
+Tensor &operator-=(Tensor &a, const Scalar &b) { F::sub_(a, scalar_of(b, a)); return a; }
+Tensor &operator*=(Tensor &a, const Scalar &b) { F::mul_(a, scalar_of(b, a)); return a; }
+Tensor &operator/=(Tensor &a, const Scalar &b) { F::div_(a, scalar_of(b, a)); return a; }
 
 Tensor Tensor::reshape(const Shape &shape) const { return F::reshape(*this, shape); }
 Tensor Tensor::transpose() const { return F::transpose(*this); }

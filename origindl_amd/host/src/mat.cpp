@@ -466,6 +466,11 @@ std::unique_ptr<Mat> OriginMat::operator-(const Mat &o) const { return binary(1,
 std::unique_ptr<Mat> OriginMat::operator*(const Mat &o) const { return binary(2, "multiply", *this, o); }
 std::unique_ptr<Mat> OriginMat::operator/(const Mat &o) const { return binary(3, "divide", *this, o); }
 std::unique_ptr<Mat> OriginMat::operator>(const Mat &o) const { return binary(4, "gt", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator==(const Mat &o) const { return binary(5, "eq", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator!=(const Mat &o) const { return binary(6, "ne", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator<(const Mat &o) const { return binary(7, "lt", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator<=(const Mat &o) const { return binary(8, "le", *this, o); }
+std::unique_ptr<Mat> OriginMat::operator>=(const Mat &o) const { return binary(9, "ge", *this, o); }
 std::unique_ptr<Mat> OriginMat::operator-() const { return unary(3, "negate", *this); }
 
 void OriginMat::add_inplace(const Mat &o) { binary(0, "add", *this, o, this); }
@@ -473,6 +478,10 @@ void OriginMat::sub_inplace(const Mat &o) { binary(1, "subtract", *this, o, this
 void OriginMat::mul_inplace(const Mat &o) { binary(2, "multiply", *this, o, this); }
 void OriginMat::div_inplace(const Mat &o) { binary(3, "divide", *this, o, this); }
 void OriginMat::neg_inplace() { unary(3, "negate", *this, this); }
+void OriginMat::exp_inplace() { unary(1, "exp", *this, this); }
+void OriginMat::log_inplace() { unary(2, "log", *this, this); }
+void OriginMat::square_inplace() { unary(4, "square", *this, this); }
+void OriginMat::relu_inplace() { unary(0, "relu", *this, this); }
 Mat &OriginMat::operator+=(const Mat &o) { add_inplace(o); return *this; }
 Mat &OriginMat::operator-=(const Mat &o) { sub_inplace(o); return *this; }
 Mat &OriginMat::operator*=(const Mat &o) { mul_inplace(o); return *this; }
@@ -485,6 +494,61 @@ std::unique_ptr<Mat> OriginMat::square() const { return unary(4, "square", *this
 std::unique_ptr<Mat> OriginMat::relu() const { return unary(0, "relu", *this); }
 std::unique_ptr<Mat> OriginMat::sigmoid() const { return unary(6, "sigmoid", *this); }
 std::unique_ptr<Mat> OriginMat::silu() const { return unary(7, "silu", *this); }
+
+std::unique_ptr<Mat> OriginMat::sigmoid_backward(const Mat &y) const
+{
+    if (y.shape() != shape_)
+        THROW_INVALID_ARG("sigmoid_backward: gy and y must have same shape and dtype");
+    return binary(10, "sigmoid_backward", *this, y);
+}
+
+std::unique_ptr<Mat> OriginMat::silu_backward(const Mat &x) const
+{
+    if (x.shape() != shape_)
+        THROW_INVALID_ARG("silu_backward: gy and x must have same shape and dtype");
+    return binary(11, "silu_backward", *this, x);
+}
+
+std::unique_ptr<Mat> OriginMat::upsample_backward(const Mat &gym, const Shape &xs, int scale_h, int scale_w,
+                                                  const std::string &) const
+{
+    const OriginMat &gy = dev_f32(gym, "upsample_backward");
+    if (gy.shape().size() != 4)
+        THROW_INVALID_ARG("Upsample backward: gradient must be 4D (N, C, OH, OW), but got shape {}", gy.shape().to_string());
+    if (xs.size() != 4)
+        THROW_INVALID_ARG("Upsample backward: x_shape must be 4D (N, C, H, W), but got shape {}", xs.to_string());
+    auto gx = new_like(gy, xs);
+    check(odl_hip_upsample_nearest_backward(fp(gy), (int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3],
+                                            (int64_t)gy.shape()[2], (int64_t)gy.shape()[3], scale_h, scale_w,
+                                            gx->data_ptr<float>(), nullptr));
+    return gx;
+}
+
+std::vector<std::unique_ptr<Mat>> OriginMat::split(const std::vector<size_t> &sizes, int dim) const
+{
+    const OriginMat &x = dev_f32(*this, "split");
+    if (dim < 0 || (size_t)dim >= shape_.size())
+        THROW_RUNTIME_ERROR("split: dimension {} out of range for {} dimensions", dim, shape_.size());
+    size_t total = 0;
+    for (size_t s : sizes)
+        total += s;
+    if (total != shape_[dim])
+        THROW_RUNTIME_ERROR("split: sizes sum to {}, but dimension {} has {} elements", total, dim, shape_[dim]);
+    int64_t outer, ax, inner;
+    split_axis(shape_, dim, outer, ax, inner);
+    std::vector<std::unique_ptr<Mat>> parts;
+    int64_t off = 0;
+    for (size_t sz : sizes)
+    {
+        std::vector<size_t> d = shape_.dims();
+        d[dim] = sz;
+        auto piece = new_like(x, Shape(d));
+        check(odl_hip_slice_axis(fp(x), outer, ax, inner, off, (int64_t)sz, piece->data_ptr<float>(), nullptr));
+        off += (int64_t)sz;
+        parts.push_back(std::move(piece));
+    }
+    return parts;
+}
 
 // ------------------------------------------------------------------------------------ detector forward path
 std::unique_ptr<Mat> OriginMat::upsample(const Shape &output_shape, int scale_h, int scale_w, const std::string &) const

@@ -361,3 +361,27 @@ def test_pnnx_runner_rejects_bad_files(h, tmp_path):
     trunc.write_bytes(open(binp, "rb").read()[:4000])
     assert _run_pnnx(h, "odl_host_", param, str(trunc), x, shp)[0] == -2
     assert _run_pnnx(h, "odl_host_", param, binp, x, shp)[0] == 0
+
+
+def test_the_references_own_operator_unit_tests_pass_on_this_backend():
+    """oracle/_ref/reference_operator_tests_hip is 27 of the reference's GoogleTest operator suites
+    (tests/unit_test/operator/test_{matmul,matmul_3d,conv2d,max_pool2d,softmax,softmax_cross_entropy,sum,sum_to,
+    broadcast_to,transpose,reshape,flatten,pow,add,sub,mul,div,neg,exp,log,square,relu,sigmoid,silu,cat,upsample,
+    compare}.cpp) compiled UNMODIFIED, from where they lie, against this repository's host layer and linked to the
+    gfx950 backend (make -C oracle ref-unit-tests; built only where the reference checkout exists). Every suite is
+    instantiated per device; the instances labelled CUDA — the device this backend answers to — run here. Left out by
+    name: the cases that need dtypes other than float32 on the device (type promotion, int/double inputs), which this
+    backend does not implement."""
+    import re
+    import subprocess
+    exe = os.path.join(ol.ORACLE_DIR, "_ref", "reference_operator_tests_hip")
+    if not os.path.exists(exe):
+        pytest.skip("the unit-test binary is built only where the reference checkout is present")
+    out = subprocess.run([exe, "--gtest_filter=*CUDA*-*TypePromotion*:*AllDtypes*:*TypeChecking*", "--gtest_brief=1"],
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    tail = out.stdout[-3000:]
+    print("\n" + "\n".join(tail.splitlines()[-4:]), flush=True)
+    assert out.returncode == 0, tail
+    ran = int(re.search(r"\[==========\] (\d+) tests from (\d+) test suites ran", out.stdout).group(1))
+    passed = int(re.search(r"\[  PASSED  \] (\d+) tests", out.stdout).group(1))
+    assert ran >= 400 and passed >= ran - 1, tail  # one case skips itself (it needs a second device)
