@@ -408,7 +408,8 @@ def accuracy(y, t):
 
 
 # -------------------------------------------------------------------------------------- elementwise
-_BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "gt": 4}
+_BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "gt": 4, "eq": 5, "ne": 6, "lt": 7, "le": 8, "ge": 9,
+        "sigmoid_backward": 10, "silu_backward": 11}
 _UN = {"relu": 0, "exp": 1, "log": 2, "neg": 3, "square": 4, "sqrt": 5, "sigmoid": 6, "silu": 7}
 
 
@@ -444,6 +445,34 @@ def upsample(x, scale):
     y = _empty((N, C, H * sh, W * sw))
     lib().call("odl_hip_upsample_nearest", _p(x), N, C, H, W, H * sh, W * sw, sh, sw, _p(y), _stream())
     return y
+
+
+def upsample_backward(gy, x_shape, scale):
+    """Mat::upsample_backward (src/mat/origin/cpu/nn/upsample.cpp:80-135)."""
+    _chk(gy, "gy")
+    sh, sw = _pair(scale)
+    N, C, H, W = (int(v) for v in x_shape)
+    gx = _empty((N, C, H, W))
+    lib().call("odl_hip_upsample_nearest_backward", _p(gy), N, C, H, W, gy.shape[2], gy.shape[3], sh, sw, _p(gx),
+               _stream())
+    return gx
+
+
+def split(x, sizes, dim):
+    """Mat::split (the backward of cat): pieces of the given sizes along dim."""
+    _chk(x, "x")
+    outer, ax, inner = _split_axis(x.shape, dim)
+    if _builtins.sum(sizes) != ax:
+        raise OdlRuntimeError("split: sizes sum to %d, but dimension %d has %d elements" % (_builtins.sum(sizes), dim, ax))
+    out, off = [], 0
+    for sz in sizes:
+        shape = list(x.shape)
+        shape[dim] = sz
+        piece = _empty(shape)
+        lib().call("odl_hip_slice_axis", _p(x), outer, ax, inner, off, sz, _p(piece), _stream())
+        out.append(piece)
+        off += sz
+    return out
 
 
 def cat(xs, dim=0):

@@ -652,6 +652,55 @@ def test_upsample_and_cat_bit_exact(api, o):
         api.lib().call("odl_hip_upsample_nearest", None, 1, 1, 2, 2, 5, 4, 2, 2, None, None)
 
 
+def test_compare_masks_activation_backward_split_and_upsample_backward(api):
+    rng = np.random.default_rng(34)
+    a = rng.integers(-3, 4, 100_003).astype(f32)
+    b = rng.integers(-3, 4, 100_003).astype(f32)
+    for nm, fn in (("gt", np.greater), ("eq", np.equal), ("ne", np.not_equal), ("lt", np.less), ("le", np.less_equal),
+                   ("ge", np.greater_equal)):
+        assert np.array_equal(host(api.binary(nm, dev(a), dev(b))), fn(a, b).astype(f32)), nm
+        assert np.array_equal(host(api.binary(nm, dev(a), dev(np.array([1.0], f32)))), fn(a, f32(1)).astype(f32)), nm
+    # activation gradients against the derivative in double precision: d sigmoid = y(1-y), d silu = s(1 + x(1-s))
+    x = (rng.standard_normal(1 << 18) * 4).astype(f32)
+    gy = rng.standard_normal(1 << 18).astype(f32)
+    x64, g64 = x.astype(np.float64), gy.astype(np.float64)
+    s64 = 1.0 / (1.0 + np.exp(-x64))
+    y = host(api.unary("sigmoid", dev(x)))
+    np.testing.assert_allclose(host(api.binary("sigmoid_backward", dev(gy), dev(y))), g64 * s64 * (1 - s64), rtol=2e-6,
+                               atol=5e-7)  # 1 - y in single precision is off by up to an ulp of 1, times |gy| <= 5
+    np.testing.assert_allclose(host(api.binary("silu_backward", dev(gy), dev(x))), g64 * s64 * (1 + x64 * (1 - s64)),
+                               rtol=2e-6, atol=2e-7)
+    # and against a centred difference of the forward kernel's own output at a few well-conditioned points
+    pts = np.array([-2.0, -0.5, 0.25, 1.0, 3.0], f32)
+    h = f32(1e-2)
+    for nm in ("sigmoid", "silu"):
+        hi, lo = host(api.unary(nm, dev(pts + h))), host(api.unary(nm, dev(pts - h)))
+        arg = host(api.unary("sigmoid", dev(pts))) if nm == "sigmoid" else pts
+        got = host(api.binary(nm + "_backward", dev(np.ones_like(pts)), dev(arg)))
+        np.testing.assert_allclose(got, (hi.astype(np.float64) - lo) / (2 * float(h)), rtol=2e-3)
+    # split undoes cat, along every axis and for ragged sizes
+    t = rng.standard_normal((4, 11, 6), dtype=f32)
+    for dim, sizes in ((0, [1, 3]), (1, [3, 1, 7]), (2, [2, 4])):
+        pieces = api.split(dev(t), sizes, dim)
+        want = np.split(t, np.cumsum(sizes)[:-1], axis=dim)
+        assert all(np.array_equal(host(g), w) for g, w in zip(pieces, want)), dim
+        assert np.array_equal(host(api.cat(pieces, dim)), t)
+    with pytest.raises(api.OdlRuntimeError):
+        api.split(dev(t), [3, 3], 1)
+    # upsample backward sums each scale_h x scale_w block in row-major order (cpu/nn/upsample.cpp:100-130)
+    g = rng.standard_normal((2, 5, 12, 18), dtype=f32)
+    for sh, sw in ((2, 2), (3, 1), (1, 3)):
+        H, W = 12 // sh, 18 // sw
+        blocks = g.reshape(2, 5, H, sh, W, sw)
+        want = np.zeros((2, 5, H, W), f32)
+        for i in range(sh):
+            for j in range(sw):
+                want = want + blocks[:, :, :, i, :, j]
+        assert np.array_equal(host(api.upsample_backward(dev(g), (2, 5, H, W), (sh, sw))), want), (sh, sw)
+    ones = np.ones((1, 2, 8, 8), f32)  # the adjoint of a copy-to-4 is a sum of 4
+    assert np.array_equal(host(api.upsample_backward(dev(ones), (1, 2, 4, 4), 2)), np.full((1, 2, 4, 4), 4, f32))
+
+
 @pytest.mark.parametrize("name", ["detA", "detB"])
 def test_yolo_detect_fixtures(api, name):
     ag = G[f"{name}_anchor_grid"]
