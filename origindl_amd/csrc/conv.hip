@@ -29,7 +29,8 @@ size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW, int6
 int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
                           int act, void *workspace, size_t workspace_bytes, hipStream_t st);
-size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
+size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                                       int64_t OH, int64_t OW);
 int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W,
                         int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
                         void *workspace, size_t workspace_bytes, hipStream_t st);
@@ -802,7 +803,7 @@ size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W
     if (OH <= 0 || OW <= 0)
         return 0;
     if (odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW))
-        return align256(odl::conv_implicit_forward_workspace(N, C, OC, KH, KW, OH, OW));  // no im2col matrix; K-slice
+        return align256(odl::conv_implicit_forward_workspace(N, C, H, W, OC, KH, KW, OH, OW));  // no im2col matrix; K-slice
                                                                                           // partials for small outputs
     return align256((size_t)(N * OH * OW * C * KH * KW) * sizeof(float));
 }

@@ -49,12 +49,40 @@ enum : int
     SB_CONV_FWD    = 1,  // B(row = output pixel m, k = (c,kh,kw)) = x[n, c, oh*SH-PH+kh, ow*SW-PW+kw]      (forward)
     SB_CONV_WGRAD  = 2,  // B(k = output pixel m, row = (c,kh,kw)) = same element                            (weight grad)
     SB_CONV_DGRAD  = 3,  // B(row = input pixel q, k = (kh,kw,oc)) = gy2d[(n, h+PH-kh, w+PW-kw), oc], stride 1 (input grad)
+    SB_CONV_FWD_TAP = 4,  // the forward operand with K ordered (kh,kw,c), C a multiple of 16: a slab of 16 k is one tap
 };
+
+// Division of a 32-bit unsigned number by a divisor fixed at launch: one multiply-high, a subtract, two shifts and
+// an add, exact for every 32-bit dividend (the round-up method: mul = floor(2^32 * (2^s - d) / d) + 1 with
+// s = ceil(log2 d)). A divisor of 1 has mul = 0 and no shifts.
+struct FastDiv
+{
+    unsigned mul, sh1, sh2;
+};
+
+inline FastDiv make_fastdiv(unsigned d)
+{
+    if (d <= 1)
+        return FastDiv{0u, 0u, 0u};
+    unsigned s = 0;
+    while ((1ull << s) < d)
+        ++s;
+    return FastDiv{(unsigned)((((1ull << 32) * ((1ull << s) - d)) / d) + 1), 1u, s - 1};
+}
+
+__device__ inline unsigned fastdiv(unsigned m, const FastDiv &f)
+{
+    const unsigned t = __umulhi(m, f.mul);
+    return (t + ((m - t) >> f.sh1)) >> f.sh2;
+}
 
 struct ConvSrc
 {
     int C, H, W, OH, OW, OC;
     int KH, KW, SH, SW, PH, PW;
+    FastDiv by_ow, by_oh;  // output pixel number -> (n, oh, ow)
+    FastDiv by_w, by_h;    // input pixel number -> (n, h, w)
+    FastDiv by_cslabs;     // K slab number -> (tap, channel slab) for the tap-ordered forward gather (C / 16 slabs a tap)
 };
 
 struct GemmArgs
@@ -111,7 +139,8 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
     // (rows of B) -> row-major; the weight-grad gather has lanes along the pixels (K of B) and the input-grad
     // gather reads 16 bytes along oc (K of B) -> K-major.
     constexpr bool A_KMAJOR = !TA;
-    constexpr bool B_KMAJOR = (SB == SB_PLAIN) ? TB : (SB != SB_CONV_FWD);
+    constexpr bool B_KMAJOR = (SB == SB_PLAIN) ? TB : (SB != SB_CONV_FWD && SB != SB_CONV_FWD_TAP);
+    static_assert(SB != SB_CONV_FWD_TAP || CK > 0, "the tap-ordered gather keeps its bounds as a per-lane tap mask");
     static_assert(SB == SB_PLAIN || BN == 128, "the gather mappings assume 128 B rows per tile");
     constexpr int LDA_S     = A_KMAJOR ? (BK + 4) : (BM + 4);
     constexpr int LDB_S     = B_KMAJOR ? (BK + 4) : (BN + 4);
@@ -252,20 +281,23 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
     [[maybe_unused]] int fw_hb = 0, fw_wb = 0;
     [[maybe_unused]] bool fw_live = false;
     [[maybe_unused]] unsigned fw_mask = 0;
+    [[maybe_unused]] unsigned fw_voff = 0;  // tap-ordered forward: byte offset of x[n, 0, oh*SH, ow*SW]
     [[maybe_unused]] int wg_off[B_PER_T];  // weight grad: this thread's 8 (c,kh,kw) as offsets into an image ...
     [[maybe_unused]] int wg_kh[CK > 0 ? 1 : B_PER_T], wg_kw[CK > 0 ? 1 : B_PER_T];  // ... and as taps (any kernel size)
     [[maybe_unused]] unsigned wg_taps = 0;  // ... or as eight 4-bit tap numbers kh*KW+kw (3x3, 1x1; 15 = no such row)
     [[maybe_unused]] int dg_n[2], dg_h[2], dg_w[2];                        // input grad: this thread's 2 pixels
     [[maybe_unused]] bool dg_live[2];
-    if constexpr (SB == SB_CONV_FWD)
+    if constexpr (SB == SB_CONV_FWD || SB == SB_CONV_FWD_TAP)
     {
         const int64_t m = n0 + (tid & (BN - 1));
         fw_live = m < g.N;
-        const int64_t mm = fw_live ? m : 0;
-        const int ow = (int)(mm % cv.OW), oh = (int)((mm / cv.OW) % cv.OH);
-        const int64_t n = mm / ((int64_t)cv.OW * cv.OH);
+        const unsigned mm = fw_live ? (unsigned)m : 0u;  // the pixel count is below 2^31
+        const unsigned q = fastdiv(mm, cv.by_ow);
+        const int64_t n = fastdiv(q, cv.by_oh);
+        const int ow = (int)(mm - q * (unsigned)cv.OW), oh = (int)(q - (unsigned)n * (unsigned)cv.OH);
         fw_hb = oh * cv.SH - cv.PH, fw_wb = ow * cv.SW - cv.PW;
         fw_base = g.B + n * cv.C * cv.H * cv.W + (int64_t)fw_hb * cv.W + fw_wb;  // dereferenced only when in bounds
+        fw_voff = (unsigned)(((n * cv.C * cv.H + oh * cv.SH) * cv.W + ow * cv.SW) * 4);  // the image is under 4 GiB
         if constexpr (CK > 0)
         {
             // bit kh*KW+kw: that tap of this thread's pixel lies inside the image
@@ -302,10 +334,11 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
         {
             const int64_t q = n0 + (tid >> 2) + 64 * u;
             dg_live[u] = q < g.N;
-            const int64_t qq = dg_live[u] ? q : 0;
-            dg_w[u] = (int)(qq % cv.W);
-            dg_h[u] = (int)((qq / cv.W) % cv.H);
-            dg_n[u] = (int)(qq / ((int64_t)cv.W * cv.H));
+            const unsigned qq = dg_live[u] ? (unsigned)q : 0u;  // the pixel count is below 2^31
+            const unsigned row = fastdiv(qq, cv.by_w), img = fastdiv(row, cv.by_h);
+            dg_w[u] = (int)(qq - row * (unsigned)cv.W);
+            dg_h[u] = (int)(row - img * (unsigned)cv.H);
+            dg_n[u] = (int)img;
         }
     }
 
@@ -335,16 +368,40 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
                 rb_[u] = ok ? fw_base[(c * cv.H + kh) * cv.W + kw] : 0.f;
             }
         }
+        else if constexpr (SB == SB_CONV_FWD_TAP)
+        {
+            // element u: row = tid % 128 (its pixel), k = k0 + tid/128 + 2u. The slab k0..k0+15 is one tap (kh,kw)
+            // and 16 consecutive channels, so the bounds test is one bit of the lane's tap mask for the whole slab
+            // and every address is a block-uniform base (channel plane + tap, minus the padding) plus the lane's
+            // constant pixel offset.
+            const int ksub = __builtin_amdgcn_readfirstlane(tid >> 7);
+            const int slab = __builtin_amdgcn_readfirstlane((int)(k0 / BK));
+            const int tap = (int)fastdiv((unsigned)slab, cv.by_cslabs), c0 = (slab - tap * (cv.C / BK)) * BK + ksub;
+            const int kh = tap / CK, kw = tap - kh * CK;
+            const int64_t plane = (int64_t)cv.H * cv.W;
+            const char *sb = reinterpret_cast<const char *>(g.B) +
+                             (c0 * plane + (int64_t)(kh - cv.PH) * cv.W + (kw - cv.PW)) * (int64_t)sizeof(float);
+#pragma unroll
+            for (int u = 0; u < B_PER_T; ++u)
+                rb_[u] = 0.f;
+            if (((fw_mask >> tap) & 1u) != 0)
+            {
+#pragma unroll
+                for (int u = 0; u < B_PER_T; ++u)
+                    rb_[u] = *reinterpret_cast<const float *>(sb + (int64_t)u * 2 * plane * (int64_t)sizeof(float) + fw_voff);
+            }
+        }
         else if constexpr (SB == SB_CONV_WGRAD)
         {
             // element u: k = k0 + tid % 16 (its pixel for this slab), row = tid/16 + 16u
-            const int64_t m = k0 + (tid & 15);
-            const bool live = m < kend;
-            const int64_t mm = live ? m : 0;
-            const int ow = (int)(mm % cv.OW), oh = (int)((mm / cv.OW) % cv.OH);
-            const int64_t n = mm / ((int64_t)cv.OW * cv.OH);
+            // (the pixel count is below 2^31, so the pixel number and its decomposition stay in 32 bits)
+            const unsigned m = (unsigned)k0 + (unsigned)(tid & 15);
+            const bool live = m < (unsigned)kend;
+            const unsigned mm = live ? m : 0u;
+            const unsigned q = fastdiv(mm, cv.by_ow), n = fastdiv(q, cv.by_oh);
+            const int ow = (int)(mm - q * (unsigned)cv.OW), oh = (int)(q - n * (unsigned)cv.OH);
             const int hb = oh * cv.SH - cv.PH, wb = ow * cv.SW - cv.PW;
-            const float *base = g.B + n * cv.C * cv.H * cv.W + (int64_t)hb * cv.W + wb;
+            const float *base = g.B + (int64_t)n * (cv.C * cv.H * cv.W) + (hb * cv.W + wb);
             if constexpr (CK > 0)
             {
                 // bit kh*CK+kw of pm: that tap of this slab's pixel lies inside the image
@@ -401,7 +458,7 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
         {
             store_tile(lds, LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
         }
-        else if constexpr (SB == SB_CONV_FWD)
+        else if constexpr (SB == SB_CONV_FWD || SB == SB_CONV_FWD_TAP)
         {
             const int ksub = tid >> 7;
 #pragma unroll
@@ -925,13 +982,14 @@ int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, void *tail_ws, s
     g.splits = splits;
     const dim3 grid(apply_tail(g, bm64 ? 64 : 128, 128, tail_ws, tail_bytes)), block(kThreads);
 #define ODL_CONV_CASE(BMV, CKV)                                                                                  \
-    if (bm64 == (BMV == 64) && ck == CKV)                                                                        \
-    {                                                                                                            \
-        hipLaunchKernelGGL((sgemm_mfma_kernel<BMV, 128, 16, TA, false, true, EPI, SB, CKV>), grid, block, 0, st, \
-                           g, cv);                                                                               \
-        launch_tail_fixup(g, BMV, 128, EPI, st);                                                                 \
-        return ODL_OK;                                                                                           \
-    }
+    if constexpr (SB != SB_CONV_FWD_TAP || CKV > 0)                                                              \
+        if (bm64 == (BMV == 64) && ck == CKV)                                                                    \
+        {                                                                                                        \
+            hipLaunchKernelGGL((sgemm_mfma_kernel<BMV, 128, 16, TA, false, true, EPI, SB, CKV>), grid, block, 0, \
+                               st, g, cv);                                                                       \
+            launch_tail_fixup(g, BMV, 128, EPI, st);                                                             \
+            return ODL_OK;                                                                                       \
+        }
     ODL_CONV_CASE(128, 3)
     ODL_CONV_CASE(128, 1)
     ODL_CONV_CASE(128, 0)
@@ -953,6 +1011,19 @@ __global__ void permute_weight_kernel(const float *__restrict__ w, float *__rest
     const int lo = k % 16, tap = (k / 16) % KHW, ocs = k / (16 * KHW);
     const int oc = ocs * 16 + lo;
     wp[t] = w[((int64_t)oc * C + c) * KHW + tap];
+}
+
+// wp[oc][tap*C + c] = w[oc][c][tap]: the K order of the tap-ordered forward gather
+__global__ void permute_weight_tap_kernel(const float *__restrict__ w, float *__restrict__ wp, int C, int KHW, int64_t total)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    const int K = C * KHW;
+    const int64_t oc = t / K;
+    const int k = (int)(t - oc * K);
+    const int tap = k / C, c = k - tap * C;
+    wp[t] = w[oc * K + c * KHW + tap];
 }
 
 int wgrad_splits(int64_t OC, int64_t K, int64_t M)
@@ -1020,7 +1091,8 @@ size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW, int6
 static ConvSrc make_src(int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW, int64_t OC, int KH, int KW, int SH,
                         int SW, int PH, int PW)
 {
-    return ConvSrc{(int)C, (int)H, (int)W, (int)OH, (int)OW, (int)OC, KH, KW, SH, SW, PH, PW};
+    return ConvSrc{(int)C, (int)H,  (int)W, (int)OH, (int)OW, (int)OC, KH, KW, SH, SW, PH, PW, make_fastdiv((unsigned)OW),
+                   make_fastdiv((unsigned)OH), make_fastdiv((unsigned)W), make_fastdiv((unsigned)H), make_fastdiv((unsigned)(C >= kBK ? C / kBK : 1))};
 }
 
 // K slices of the forward product when its tiles alone leave most of the chip idle: aim at ~512 workgroups of at
@@ -1041,11 +1113,29 @@ static int forward_splits(int64_t OC, int64_t M, int64_t K)
     return s < 2 ? 1 : (int)s;
 }
 
-size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW)
+// The tap-ordered gather: square 1x1 / 3x3 windows over a channel count that fills whole K slabs, image addressed
+// with 32-bit byte offsets. A 3x3 window needs the weights re-ordered to [OC][tap][C] first (a 1x1 window's order
+// is already that).
+static bool forward_tap_ok(int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW)
+{
+    return KH == KW && (KH == 1 || KH == 3) && C % kBK == 0 && N * C * H * W < (1ll << 30);
+}
+
+static size_t forward_wp_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW)
+{
+    if (!forward_tap_ok(N, C, H, W, KH, KW) || KH == 1)
+        return 0;
+    return (((size_t)OC * C * KH * KW * sizeof(float)) + 255) & ~(size_t)255;
+}
+
+// re-ordered weights (3x3 tap-ordered gather only), then K-slice partials or tail-split partials
+size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                                       int64_t OH, int64_t OW)
 {
     const int64_t K = C * KH * KW, M = N * OH * OW;
     const int s = forward_splits(OC, M, K);
-    return s > 1 ? (size_t)s * OC * M * sizeof(float) : conv_tail_bytes(OC, M, K);
+    return forward_wp_bytes(N, C, H, W, OC, KH, KW) +
+           (s > 1 ? (size_t)s * OC * M * sizeof(float) : conv_tail_bytes(OC, M, K));
 }
 
 // y[n][oc][p] = sum_k W2d[oc][k] * x_gathered[(n,p)][k] + b[oc]
@@ -1059,6 +1149,23 @@ int conv_implicit_forward(const float *x, const float *w, const float *b, float 
     g.lda = g.K, g.ldb = 0, g.ldc = 0, g.P = OH * OW;
     g.k_per_split = ceil_div(g.K, kBK) * kBK, g.c_split_stride = 0;
     const ConvSrc cv = make_src(C, H, W, OH, OW, OC, KH, KW, SH, SW, PH, PW);
+    bool tap = forward_tap_ok(N, C, H, W, KH, KW);
+    if (tap && KH > 1)
+    {
+        const size_t wp_bytes = forward_wp_bytes(N, C, H, W, OC, KH, KW);
+        if (workspace != nullptr && workspace_bytes >= wp_bytes)
+        {
+            float *wp = static_cast<float *>(workspace);
+            const int64_t total = OC * g.K;
+            hipLaunchKernelGGL(permute_weight_tap_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, w, wp,
+                               (int)C, KH * KW, total);
+            ODL_LAUNCH_CHECK();
+            g.A = wp;
+            workspace = static_cast<char *>(workspace) + wp_bytes, workspace_bytes -= wp_bytes;
+        }
+        else
+            tap = false;  // a caller without the workspace still gets the (c,kh,kw)-ordered gather
+    }
     int splits = forward_splits(OC, g.N, g.K);
     if (splits > 1 && (workspace == nullptr || workspace_bytes < (size_t)splits * OC * g.N * sizeof(float)))
         splits = 1;  // a caller without the workspace still gets the single-pass kernel
@@ -1069,7 +1176,8 @@ int conv_implicit_forward(const float *x, const float *w, const float *b, float 
         g.k_per_split = ceil_div(ceil_div(g.K, kBK), splits) * kBK;
         splits = (int)ceil_div(g.K, g.k_per_split);
         g.C = static_cast<float *>(workspace), g.bias = nullptr, g.ldc = g.N, g.c_split_stride = OC * g.N;
-        rc = launch_conv_tile<SB_CONV_FWD, false, EPI_PLAIN>(g, cv, splits, nullptr, 0, st);
+        rc = tap ? launch_conv_tile<SB_CONV_FWD_TAP, false, EPI_PLAIN>(g, cv, splits, nullptr, 0, st)
+                 : launch_conv_tile<SB_CONV_FWD, false, EPI_PLAIN>(g, cv, splits, nullptr, 0, st);
         if (rc != ODL_OK)
             return fail(rc, "conv2d: no kernel variant");
         ODL_LAUNCH_CHECK();
@@ -1077,7 +1185,8 @@ int conv_implicit_forward(const float *x, const float *w, const float *b, float 
         ODL_LAUNCH_CHECK();
         return ODL_OK;
     }
-    rc = launch_conv_tile<SB_CONV_FWD, false, EPI_NCHW_ROWB>(g, cv, 1, workspace, workspace_bytes, st);
+    rc = tap ? launch_conv_tile<SB_CONV_FWD_TAP, false, EPI_NCHW_ROWB>(g, cv, 1, workspace, workspace_bytes, st)
+             : launch_conv_tile<SB_CONV_FWD, false, EPI_NCHW_ROWB>(g, cv, 1, workspace, workspace_bytes, st);
     if (rc != ODL_OK)
         return fail(rc, "conv2d: no kernel variant");
     ODL_LAUNCH_CHECK();

@@ -32,10 +32,14 @@ def test_library_exports_every_declared_symbol():
 
 def test_workspace_queries_need_no_gpu():
     l = _lib.lib()
-    # conv C1 of the benchmark runs as implicit GEMM: no col matrix (231 MB); only the K pieces of its last 16 tiles
-    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) == 16 * 12 * 128 * 128 * 4
-    # a tile count that is a multiple of the CU count needs nothing at all
-    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 3, 3, 1, 1, 1, 1) == 0
+    # conv C1 of the benchmark runs as implicit GEMM: no col matrix (231 MB); only the weights re-ordered to
+    # [OC][tap][C] and the K pieces of its last 16 tiles
+    wp = 128 * 64 * 9 * 4
+    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) == wp + 16 * 12 * 128 * 128 * 4
+    # a tile count that is a multiple of the CU count needs no K pieces
+    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 3, 3, 1, 1, 1, 1) == wp
+    # a 1x1 window's weights are in tap order as they are
+    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 1, 1, 1, 1, 0, 0) == 0
     # C*KH*KW = 9 is not a multiple of 4: explicit im2col path, workspace = the col matrix [N*OH*OW, 9]
     assert l.query("odl_hip_conv2d_workspace_bytes", 256, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1) == 256 * 28 * 28 * 9 * 4
     assert l.query("odl_hip_conv2d_backward_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) < 100352 * 576 * 4
