@@ -52,29 +52,9 @@ enum : int
     SB_CONV_FWD_TAP = 4,  // the forward operand with K ordered (kh,kw,c), C a multiple of 16: a slab of 16 k is one tap
 };
 
-// Division of a 32-bit unsigned number by a divisor fixed at launch: one multiply-high, a subtract, two shifts and
-// an add, exact for every 32-bit dividend (the round-up method: mul = floor(2^32 * (2^s - d) / d) + 1 with
-// s = ceil(log2 d)). A divisor of 1 has mul = 0 and no shifts.
-struct FastDiv
-{
-    unsigned mul, sh1, sh2;
-};
-
-inline FastDiv make_fastdiv(unsigned d)
-{
-    if (d <= 1)
-        return FastDiv{0u, 0u, 0u};
-    unsigned s = 0;
-    while ((1ull << s) < d)
-        ++s;
-    return FastDiv{(unsigned)((((1ull << 32) * ((1ull << s) - d)) / d) + 1), 1u, s - 1};
-}
-
-__device__ inline unsigned fastdiv(unsigned m, const FastDiv &f)
-{
-    const unsigned t = __umulhi(m, f.mul);
-    return (t + ((m - t) >> f.sh1)) >> f.sh2;
-}
+using odl::FastDiv;
+using odl::fastdiv;
+using odl::make_fastdiv;
 
 struct ConvSrc
 {
@@ -629,8 +609,11 @@ __global__ __launch_bounds__(64 * kRedGroups) void splitk_reduce_kernel(const fl
     const int64_t i = (int64_t)blockIdx.x * 64 + lane;
     float acc = 0.f;
     if (i < M * N)
+    {
+#pragma unroll 4
         for (int z = grp; z < splits; z += kRedGroups)
             acc += part[(int64_t)z * stride + i];
+    }
     sh[grp][lane] = acc;
     __syncthreads();
     if (grp == 0 && i < M * N)
@@ -723,6 +706,7 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(GemmArgs g, int BM, int
     const int row_l = e / (BN / 4), c4 = e - row_l * (BN / 4);
     const float *p = g.tail_ws + ((int64_t)ti * g.tail_splits * BM + row_l) * BN + 4 * c4;
     f32x4 acc = *reinterpret_cast<const f32x4 *>(p);
+#pragma unroll 4
     for (int z = 1; z < g.tail_splits; ++z)
     {
         const f32x4 v = *reinterpret_cast<const f32x4 *>(p + (int64_t)z * BM * BN);

@@ -28,6 +28,30 @@ inline int64_t ceil_div(int64_t a, int64_t b)
 {
     return (a + b - 1) / b;
 }
+
+// Division of a 32-bit unsigned number by a divisor fixed at launch: one multiply-high, a subtract, two shifts and
+// an add, exact for every 32-bit dividend (the round-up method: mul = floor(2^32 * (2^s - d) / d) + 1 with
+// s = ceil(log2 d)). A divisor of 1 has mul = 0 and no shifts.
+struct FastDiv
+{
+    unsigned mul, sh1, sh2;
+};
+
+inline FastDiv make_fastdiv(unsigned d)
+{
+    if (d <= 1)
+        return FastDiv{0u, 0u, 0u};
+    unsigned s = 0;
+    while ((1ull << s) < d)
+        ++s;
+    return FastDiv{(unsigned)((((1ull << 32) * ((1ull << s) - d)) / d) + 1), 1u, s - 1};
+}
+
+__device__ inline unsigned fastdiv(unsigned m, const FastDiv &f)
+{
+    const unsigned t = __umulhi(m, f.mul);
+    return (t + ((m - t) >> f.sh1)) >> f.sh2;
+}
 }  // namespace odl
 
 #define ODL_HIP_CHECK(expr)                                                                          \

@@ -189,33 +189,61 @@ __global__ __launch_bounds__(64 * kFoldGroups) void fold_partials_kernel(const f
     }
 }
 
-// ---- conv bias gradient: gy[N][OC][P] -> part[oc][nsplit]; grid (nsplit, OC)
-__global__ void nchw_channel_sum_kernel(const float *__restrict__ gy, float *__restrict__ part, int64_t N, int64_t OC,
-                                        int64_t P, int64_t nchunk)
+// ---- conv bias gradient: gy[N][OC][P] -> part[oc][nsplit]; grid (nsplit, OC). A channel's N*P elements are one
+// flat range cut into nsplit equal chunks, so every thread has work whatever the size of one image plane; each
+// thread keeps four independent running sums (four loads in flight) that are added in a fixed order.
+struct ChannelSumPlan
 {
-    const int64_t oc = blockIdx.y;
-    const int64_t nb = (int64_t)blockIdx.x * nchunk;
-    const int64_t ne = (nb + nchunk < N) ? nb + nchunk : N;
-    float acc = 0.f;
-    const bool v4 = (P % 4 == 0) && (reinterpret_cast<uintptr_t>(gy) % 16 == 0);
-    for (int64_t n = nb; n < ne; ++n)
+    int64_t chunk;  // elements of one channel per workgroup (a multiple of 4)
+    int64_t ns;     // workgroups per channel
+};
+
+__host__ inline ChannelSumPlan plan_channel_sum(int64_t N, int64_t OC, int64_t P)
+{
+    const int64_t total = (N > 0 ? N : 0) * (P > 0 ? P : 0);
+    int64_t want = odl::ceil_div(2048, OC > 0 ? OC : 1);  // about eight workgroups per CU over all channels
+    int64_t chunk = odl::ceil_div(total > 0 ? total : 1, want);
+    if (chunk < 2048)
+        chunk = 2048;
+    chunk = odl::ceil_div(chunk, 4) * 4;
+    ChannelSumPlan p{chunk, odl::ceil_div(total > 0 ? total : 1, chunk)};
+    return p;
+}
+
+template <bool V4>
+__global__ __launch_bounds__(kBlock) void nchw_channel_sum_kernel(const float *__restrict__ gy, float *__restrict__ part,
+                                                                   unsigned total, unsigned P, unsigned OC,
+                                                                   unsigned chunk, odl::FastDiv by_plane)
+{
+    constexpr unsigned E = V4 ? 4 : 1;  // elements per load; V4 needs P % 4 == 0 and a 16-byte aligned gy
+    const unsigned oc = blockIdx.y;
+    const unsigned beg = blockIdx.x * chunk;
+    const unsigned end = (beg + chunk < total) ? beg + chunk : total;
+    const unsigned plane = P / E;  // loads per image plane
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (unsigned u0 = beg / E + threadIdx.x; u0 < end / E; u0 += 4 * kBlock)
     {
-        const float *p = gy + (n * OC + oc) * P;
-        if (v4)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
         {
-            const f32x4 *pv = reinterpret_cast<const f32x4 *>(p);
-            f32x4 a4 = {0.f, 0.f, 0.f, 0.f};
-            for (int64_t v = threadIdx.x; v < P / 4; v += kBlock)
-                a4 += pv[v];
-            acc += (a4[0] + a4[1]) + (a4[2] + a4[3]);
+            const unsigned u = u0 + j * kBlock;
+            if (u < end / E)
+            {
+                const unsigned n = odl::fastdiv(u, by_plane), v = u - n * plane;
+                const float *p = gy + ((int64_t)n * OC + oc) * P + (int64_t)v * E;
+                if (V4)
+                {
+                    const f32x4 q = *reinterpret_cast<const f32x4 *>(p);
+                    acc[j] += (q[0] + q[1]) + (q[2] + q[3]);
+                }
+                else
+                    acc[j] += *p;
+            }
         }
-        else
-            for (int64_t i = threadIdx.x; i < P; i += kBlock)
-                acc += p[i];
     }
-    const float s = block_sum(acc);
+    const float s = block_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
     if (threadIdx.x == 0)
-        part[oc * gridDim.x + blockIdx.x] = s;
+        part[(int64_t)oc * gridDim.x + blockIdx.x] = s;
 }
 
 // ---- max
@@ -490,13 +518,7 @@ namespace odl
 {
 size_t sum_nchw_channels_workspace(int64_t N, int64_t OC, int64_t P)
 {
-    (void)P;
-    int64_t ns = ceil_div(1024, OC > 0 ? OC : 1);
-    if (ns > N)
-        ns = N;
-    if (ns < 1)
-        ns = 1;
-    return (size_t)(OC * ns) * sizeof(float);
+    return (size_t)((OC > 0 ? OC : 0) * plan_channel_sum(N, OC, P).ns) * sizeof(float);
 }
 
 int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
@@ -505,22 +527,24 @@ int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, 
     if (OC == 0)
         return ODL_OK;
     ODL_REQUIRE(N >= 0 && OC > 0 && OC < 65536 && P >= 0, "conv bias gradient: bad shape");
-    int64_t ns = ceil_div(1024, OC);
-    if (ns > N)
-        ns = N;
-    if (ns < 1)
-        ns = 1;
-    const int64_t nchunk = ceil_div(N > 0 ? N : 1, ns);
-    ns = ceil_div(N > 0 ? N : 1, nchunk);
-    const size_t need = (size_t)(OC * ns) * sizeof(float);
+    ODL_REQUIRE(N * P < (1ll << 31), "conv bias gradient: more than 2^31 elements per channel");
+    const ChannelSumPlan pl = plan_channel_sum(N, OC, P);
+    ODL_REQUIRE(pl.ns < 65536, "conv bias gradient: too many workgroups per channel");
+    const size_t need = (size_t)(OC * pl.ns) * sizeof(float);
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
                 "conv bias gradient: workspace of %zu bytes required, got %zu", need, workspace_bytes);
     float *part = static_cast<float *>(workspace);
-    hipLaunchKernelGGL(nchw_channel_sum_kernel, dim3((unsigned)ns, (unsigned)OC), dim3(kBlock), 0, st, gy, part, N, OC,
-                       P, nchunk);
+    const bool v4 = P % 4 == 0 && reinterpret_cast<uintptr_t>(gy) % 16 == 0;
+    const dim3 grid((unsigned)pl.ns, (unsigned)OC), block(kBlock);
+    if (v4)
+        hipLaunchKernelGGL((nchw_channel_sum_kernel<true>), grid, block, 0, st, gy, part, (unsigned)(N * P), (unsigned)P,
+                           (unsigned)OC, (unsigned)pl.chunk, odl::make_fastdiv((unsigned)(P / 4)));
+    else
+        hipLaunchKernelGGL((nchw_channel_sum_kernel<false>), grid, block, 0, st, gy, part, (unsigned)(N * P), (unsigned)P,
+                           (unsigned)OC, (unsigned)pl.chunk, odl::make_fastdiv((unsigned)(P > 0 ? P : 1)));
     ODL_LAUNCH_CHECK();
     hipLaunchKernelGGL(row_sum_wave_kernel, dim3((unsigned)ceil_div(OC, kBlock / 64)), dim3(kBlock), 0, st, part, gb, OC,
-                       ns);
+                       pl.ns);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
