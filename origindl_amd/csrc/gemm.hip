@@ -1010,18 +1010,33 @@ __global__ void permute_weight_tap_kernel(const float *__restrict__ w, float *__
     wp[t] = w[oc * K + c * KHW + tap];
 }
 
+// K slices for a product whose tiles alone leave most of the chip idle. All workgroups are resident at once (at
+// most `slots` of them), so the launch lasts as long as the busiest CU: (workgroups on it) x (K slabs each, plus
+// about three slabs' worth of prologue and epilogue). A lone workgroup on a CU has nothing to overlap its memory
+// latency with and runs a quarter slower, three or more overlap a little better than two, and every slice adds one
+// more pass over the output (tiles x 64 KB) for the reduction that follows. The slice count with the smallest such
+// estimate wins.
+int pick_conv_splits(int64_t tiles, int64_t kt, int64_t slots, int64_t max_splits)
+{
+    int best = 1;
+    double best_cost = 0;
+    for (int64_t s = 1; s <= max_splits && tiles * s <= slots; ++s)
+    {
+        const int64_t per_cu = odl::ceil_div(tiles * s, 256);
+        const double overlap = per_cu == 1 ? 1.25 : (per_cu == 2 ? 1.0 : 0.95);
+        const double cost = (double)per_cu * (double)(odl::ceil_div(kt, s) + 3) * overlap + 0.014 * (double)tiles * (double)s;
+        if (s == 1 || cost < best_cost)
+            best = (int)s, best_cost = cost;
+    }
+    return best;
+}
+
 int wgrad_splits(int64_t OC, int64_t K, int64_t M)
 {
-    // as many K slices as keep every workgroup resident at once (256 CUs x 3 or 4 workgroups by register use):
-    // one slice more and the last few workgroups run alone after all the others
     const int64_t tiles = odl::ceil_div(OC, OC <= 64 ? 64 : 128) * odl::ceil_div(K, 128);
     const int64_t kt = odl::ceil_div(M, kBK);
-    int64_t s = (OC <= 64 ? 1024 : 768) / tiles;
-    if (s > kt / 16)
-        s = kt / 16;
-    if (s > 256)
-        s = 256;
-    return s < 1 ? 1 : (int)s;
+    const int64_t cap = kt / 8 < 256 ? kt / 8 : 256;
+    return pick_conv_splits(tiles, kt, OC <= 64 ? 1024 : 768, cap);
 }
 }  // namespace
 
@@ -1079,9 +1094,7 @@ static ConvSrc make_src(int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
                    make_fastdiv((unsigned)OH), make_fastdiv((unsigned)W), make_fastdiv((unsigned)H), make_fastdiv((unsigned)(C >= kBK ? C / kBK : 1))};
 }
 
-// K slices of the forward product when its tiles alone leave most of the chip idle: aim at ~512 workgroups of at
-// least four K slabs each (a lone workgroup per CU walks its slabs at memory latency, so short and many beats few
-// and long)
+// K slices of the forward product when its tiles alone leave most of the chip idle
 static int forward_splits(int64_t OC, int64_t M, int64_t K)
 {
     const int64_t tiles128 = ceil_div(OC, 128) * ceil_div(M, 128);
@@ -1089,12 +1102,8 @@ static int forward_splits(int64_t OC, int64_t M, int64_t K)
     const int64_t kt = ceil_div(K, kBK);
     if (tiles128 >= 200 || tiles >= 200 || kt < 8)
         return 1;
-    int64_t s = (OC <= 64 ? 512 : 768) / tiles;
-    if (s > kt / 4)
-        s = kt / 4;
-    if (s > 32)
-        s = 32;
-    return s < 2 ? 1 : (int)s;
+    const int64_t cap = kt / 4 < 32 ? kt / 4 : 32;
+    return pick_conv_splits(tiles, kt, OC <= 64 ? 1024 : 768, cap);
 }
 
 // The tap-ordered gather: square 1x1 / 3x3 windows over a channel count that fills whole K slabs, image addressed

@@ -206,6 +206,9 @@ __host__ inline ChannelSumPlan plan_channel_sum(int64_t N, int64_t OC, int64_t P
     if (chunk < 2048)
         chunk = 2048;
     chunk = odl::ceil_div(chunk, 4) * 4;
+    // a channel short enough for one workgroup (a few loads per thread) is summed in a single launch
+    if (total <= 16 * 1024 && OC >= 64)
+        chunk = odl::ceil_div(total > 0 ? total : 1, 4) * 4;
     ChannelSumPlan p{chunk, odl::ceil_div(total > 0 ? total : 1, chunk)};
     return p;
 }
@@ -243,7 +246,7 @@ __global__ __launch_bounds__(kBlock) void nchw_channel_sum_kernel(const float *_
     }
     const float s = block_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
     if (threadIdx.x == 0)
-        part[(int64_t)oc * gridDim.x + blockIdx.x] = s;
+        part[(int64_t)oc * gridDim.x + blockIdx.x] = s;  // with one workgroup per channel `part` is the result itself
 }
 
 // ---- max
@@ -531,9 +534,9 @@ int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, 
     const ChannelSumPlan pl = plan_channel_sum(N, OC, P);
     ODL_REQUIRE(pl.ns < 65536, "conv bias gradient: too many workgroups per channel");
     const size_t need = (size_t)(OC * pl.ns) * sizeof(float);
-    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
+    ODL_REQUIRE(pl.ns == 1 || (workspace != nullptr && workspace_bytes >= need),
                 "conv bias gradient: workspace of %zu bytes required, got %zu", need, workspace_bytes);
-    float *part = static_cast<float *>(workspace);
+    float *part = pl.ns == 1 ? gb : static_cast<float *>(workspace);
     const bool v4 = P % 4 == 0 && reinterpret_cast<uintptr_t>(gy) % 16 == 0;
     const dim3 grid((unsigned)pl.ns, (unsigned)OC), block(kBlock);
     if (v4)
@@ -543,9 +546,12 @@ int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, 
         hipLaunchKernelGGL((nchw_channel_sum_kernel<false>), grid, block, 0, st, gy, part, (unsigned)(N * P), (unsigned)P,
                            (unsigned)OC, (unsigned)pl.chunk, odl::make_fastdiv((unsigned)(P > 0 ? P : 1)));
     ODL_LAUNCH_CHECK();
-    hipLaunchKernelGGL(row_sum_wave_kernel, dim3((unsigned)ceil_div(OC, kBlock / 64)), dim3(kBlock), 0, st, part, gb, OC,
-                       pl.ns);
-    ODL_LAUNCH_CHECK();
+    if (pl.ns > 1)
+    {
+        hipLaunchKernelGGL(row_sum_wave_kernel, dim3((unsigned)ceil_div(OC, kBlock / 64)), dim3(kBlock), 0, st, part, gb,
+                           OC, pl.ns);
+        ODL_LAUNCH_CHECK();
+    }
     return ODL_OK;
 }
 }  // namespace odl

@@ -417,6 +417,13 @@ def test_bias_grad_large_column_reduction(api):
     gy = torch.randn((32, 128, 56, 56), device="cuda", generator=g)
     gb = api.sum_nchw_channels(gy).double()
     assert float((gb - gy.double().sum(dim=(0, 2, 3))).abs().max()) <= 1e-5 * float(np.sqrt(32 * 56 * 56)) * 400
+    # short channels (one workgroup each, a single launch), a plane that is not a multiple of four, and one image
+    for shape in ((32, 256, 14, 14), (5, 64, 7, 9), (1, 3, 5, 5), (3, 70, 33, 31)):
+        gy = torch.randn(shape, device="cuda", generator=g)
+        gb = api.sum_nchw_channels(gy).double()
+        want = gy.double().sum(dim=(0, 2, 3))
+        n = shape[0] * shape[2] * shape[3]
+        assert float((gb - want).abs().max()) <= 1e-5 * float(np.sqrt(n)) * 40, shape
 
 
 def test_broadcast_fixtures(api):
