@@ -215,6 +215,28 @@ int odl_hip_yolo_detect_forward(const float *x, const float *conv_w, const float
                                 int num_classes, float *out, void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_yolo_detect_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int num_anchors, int num_classes);
 
+/* Mat::batch_norm_forward / Mat::batch_norm (mat.h:603-631; src/mat/origin/cpu/normalization/batch_norm.cpp:31-258)
+ * over x[N, C, P]: P = H*W for num_dims 4, P = 1 for num_dims 2. training != 0: per-channel mean and biased variance
+ * of the batch (sum / count, then squared differences from that mean / count), written to mean[C] and var[C];
+ * training == 0: mean and var are copies of the running statistics. Then x_norm = (x - mean) / sqrt(var + eps) and
+ * y = gamma * x_norm + beta. x_norm may be NULL (the y-only Mat::batch_norm). running_mean / running_var may be NULL
+ * in training mode; the workspace is needed in training mode only. */
+int odl_hip_batch_norm_forward(const float *x, const float *gamma, const float *beta, const float *running_mean,
+                               const float *running_var, int training, float eps, int64_t N, int64_t C, int64_t P,
+                               float *y, float *mean, float *var, float *x_norm, void *workspace,
+                               size_t workspace_bytes, void *stream);
+/* Mat::batch_norm_backward (mat.h:643; batch_norm.cpp:279-418): dbeta = sum gy, dgamma = sum gy * x_norm per channel,
+ * gx = (gamma / sqrt(saved_var + eps)) * (gy - dbeta/count - x_norm * dgamma/count). */
+int odl_hip_batch_norm_backward(const float *gy, const float *gamma, const float *saved_var, const float *saved_x_norm,
+                                float eps, int64_t N, int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta,
+                                void *workspace, size_t workspace_bytes, void *stream);
+/* workspace of either call (partial channel sums) */
+size_t odl_hip_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t P);
+/* out = a*x + b*y, each product rounded before the sum: the running-statistics update of the BatchNorm layers
+ * (src/nn/layers/batch_norm2d.cpp:77-80, batch_norm1d.cpp), which the reference does on the host after four
+ * device-to-host copies. out may be x or y. */
+int odl_hip_axpby(float a, const float *x, float b, const float *y, int64_t n, float *out, void *stream);
+
 /* Fused optimizer steps. The reference has no Mat virtual for them: Adam::step_one (src/optim/adam.cpp:52-113) and
  * SGD::step_one (src/optim/sgd.cpp:18-75) issue the same arithmetic as ~15 whole-tensor Mat operations per parameter.
  * Each element goes through the identical sequence of separately rounded float operations

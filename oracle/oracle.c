@@ -597,6 +597,96 @@ void orc_pow_scalar(const float *a, int64_t n, float e, float *out)
         out[i] = powf(a[i], e);
 }
 
+/* ========================================================================== batch normalisation */
+
+/* normalization/batch_norm.cpp:31-258. x[N][C][P] (P = H*W; P = 1 is the two-dimensional [N][C] form). Training:
+ * per channel, a sequential float sum over (n, p) / count, then the sequential sum of squared differences from that
+ * mean / count. Evaluation: mean and var are copies of the running statistics. x_norm may be NULL. */
+int orc_batch_norm_forward(const float *x, const float *gamma, const float *beta, const float *running_mean,
+                           const float *running_var, int training, float eps, int64_t N, int64_t C, int64_t P, float *y,
+                           float *mean, float *var, float *x_norm)
+{
+    if (N < 0 || C <= 0 || P <= 0)
+        return ORC_ERR_INVALID_ARG;
+    const int64_t count = N * P;
+    for (int64_t c = 0; c < C; ++c)
+    {
+        if (training)
+        {
+            float sum = 0.f;
+            for (int64_t n = 0; n < N; ++n)
+                for (int64_t p = 0; p < P; ++p)
+                    sum += x[(n * C + c) * P + p];
+            if (count > 0)
+                mean[c] = sum / (float)count;
+            float sq = 0.f;
+            for (int64_t n = 0; n < N; ++n)
+                for (int64_t p = 0; p < P; ++p)
+                {
+                    const float d = x[(n * C + c) * P + p] - mean[c];
+                    sq += d * d;
+                }
+            if (count > 0)
+                var[c] = sq / (float)count;
+        }
+        else
+        {
+            mean[c] = running_mean[c];
+            var[c] = running_var[c];
+        }
+    }
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < C; ++c)
+        {
+            const float sd = sqrtf(var[c] + eps);
+            for (int64_t p = 0; p < P; ++p)
+            {
+                const int64_t i = (n * C + c) * P + p;
+                const float xn = (x[i] - mean[c]) / sd;
+                if (x_norm)
+                    x_norm[i] = xn;
+                const float t = gamma[c] * xn;
+                y[i] = t + beta[c];
+            }
+        }
+    return ORC_OK;
+}
+
+/* normalization/batch_norm.cpp:279-418 */
+int orc_batch_norm_backward(const float *gy, const float *gamma, const float *saved_var, const float *saved_x_norm,
+                            float eps, int64_t N, int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta)
+{
+    if (N < 0 || C <= 0 || P <= 0)
+        return ORC_ERR_INVALID_ARG;
+    const int64_t count = N * P;
+    for (int64_t c = 0; c < C; ++c)
+    {
+        float sum_gy = 0.f, sum_gy_xn = 0.f;
+        for (int64_t n = 0; n < N; ++n)
+            for (int64_t p = 0; p < P; ++p)
+            {
+                const int64_t i = (n * C + c) * P + p;
+                sum_gy += gy[i];
+                const float t = gy[i] * saved_x_norm[i];
+                sum_gy_xn += t;
+            }
+        const float mean_gy = count > 0 ? sum_gy / (float)count : 0.f;
+        const float mean_gy_xn = count > 0 ? sum_gy_xn / (float)count : 0.f;
+        const float sd = sqrtf(saved_var[c] + eps);
+        dgamma[c] = sum_gy_xn;
+        dbeta[c] = sum_gy;
+        const float scale = gamma[c] / sd;
+        for (int64_t n = 0; n < N; ++n)
+            for (int64_t p = 0; p < P; ++p)
+            {
+                const int64_t i = (n * C + c) * P + p;
+                const float t = saved_x_norm[i] * mean_gy_xn;
+                gx[i] = scale * ((gy[i] - mean_gy) - t);
+            }
+    }
+    return ORC_OK;
+}
+
 /* ========================================================================== detector forward path */
 
 /* nn/upsample.cpp:22-75: nearest neighbour, ih = oh / scale_h, iw = ow / scale_w */

@@ -120,6 +120,13 @@ int orc_yolo_detect_forward(const float *x, const float *conv_w, const float *co
                             const float *anchor_grid, int64_t anchor_elems, int64_t anchor_H, int64_t anchor_W, int64_t N,
                             int64_t C, int64_t H, int64_t W, float stride, int num_anchors, int num_classes, float *out);
 
+/* batch normalisation over x[N][C][P] (P = H*W, or 1 for [N][C]): normalization/batch_norm.cpp:31-258, 279-418 */
+int orc_batch_norm_forward(const float *x, const float *gamma, const float *beta, const float *running_mean,
+                           const float *running_var, int training, float eps, int64_t N, int64_t C, int64_t P, float *y,
+                           float *mean, float *var, float *x_norm);
+int orc_batch_norm_backward(const float *gy, const float *gamma, const float *saved_var, const float *saved_x_norm,
+                            float eps, int64_t N, int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta);
+
 /* ---- whole training steps (compositions restated from the reference's operators/optimizers) --------- */
 /* MLP: x[N,D] -> Linear(D,Hd)+ReLU -> Linear(Hd,C) -> softmax CE; backward; WeightDecay hook (grad += wd*p,
  * include/origin/optim/hooks.h:40-65); Adam step t (src/optim/adam.cpp:19-114). Parameters and Adam

@@ -513,6 +513,55 @@ def yolo_detect_forward(x, conv_w, conv_b, grid, anchor_grid, stride, num_anchor
     return out
 
 
+def _bn_dims(x, who):
+    if x.dim() not in (2, 4):
+        raise OdlInvalidArgument("%s: x must have 2 or 4 dimensions, but got shape %s" % (who, tuple(x.shape)))
+    return x.shape[0], x.shape[1], (x.shape[2] * x.shape[3] if x.dim() == 4 else 1)
+
+
+def batch_norm_forward(x, gamma, beta, running_mean, running_var, training, eps=1e-5, want_x_norm=True):
+    """Mat::batch_norm_forward (src/mat/origin/cpu/normalization/batch_norm.cpp:31-258) -> (y, mean, var, x_norm);
+    want_x_norm=False is the y-only Mat::batch_norm (x_norm is None)."""
+    for name, t in (("x", x), ("gamma", gamma), ("beta", beta), ("running_mean", running_mean),
+                    ("running_var", running_var)):
+        _chk(t, name)
+    N, C, P = _bn_dims(x, "batch_norm")
+    for name, t in (("gamma", gamma), ("beta", beta), ("running_mean", running_mean), ("running_var", running_var)):
+        if tuple(t.shape) != (C,):
+            raise OdlInvalidArgument("batch_norm: gamma, beta, running_mean, running_var must have shape (%d)" % C)
+    y, mean, var = _empty(x.shape), _empty((C,)), _empty((C,))
+    xn = _empty(x.shape) if want_x_norm else None
+    ws, nb = _ws(lib().query("odl_hip_batch_norm_workspace_bytes", N, C, P) if training else 0)
+    lib().call("odl_hip_batch_norm_forward", _p(x), _p(gamma), _p(beta), _p(running_mean), _p(running_var),
+               1 if training else 0, float(eps), N, C, P, _p(y), _p(mean), _p(var), _p(xn), _p(ws), nb, _stream())
+    return y, mean, var, xn
+
+
+def batch_norm_backward(gy, gamma, saved_var, saved_x_norm, eps=1e-5):
+    """Mat::batch_norm_backward (batch_norm.cpp:279-418) -> (gx, dgamma, dbeta)."""
+    for name, t in (("gy", gy), ("gamma", gamma), ("saved_var", saved_var), ("saved_x_norm", saved_x_norm)):
+        _chk(t, name)
+    N, C, P = _bn_dims(gy, "batch_norm_backward")
+    if saved_x_norm.shape != gy.shape or tuple(gamma.shape) != (C,) or tuple(saved_var.shape) != (C,):
+        raise OdlInvalidArgument("batch_norm_backward: shape mismatch")
+    gx, dg, db = _empty(gy.shape), _empty((C,)), _empty((C,))
+    ws, nb = _ws(lib().query("odl_hip_batch_norm_workspace_bytes", N, C, P))
+    lib().call("odl_hip_batch_norm_backward", _p(gy), _p(gamma), _p(saved_var), _p(saved_x_norm), float(eps), N, C, P,
+               _p(gx), _p(dg), _p(db), _p(ws), nb, _stream())
+    return gx, dg, db
+
+
+def axpby(a, x, b, y):
+    """a*x + b*y with each product rounded first: the running-statistics update of the BatchNorm layers
+    (src/nn/layers/batch_norm2d.cpp:77-80)."""
+    _chk(x, "x"), _chk(y, "y")
+    if x.shape != y.shape:
+        raise OdlInvalidArgument("axpby: shape mismatch")
+    out = _empty(x.shape)
+    lib().call("odl_hip_axpby", float(a), _p(x), float(b), _p(y), x.numel(), _p(out), _stream())
+    return out
+
+
 def adam_step(p, g, m, v, t, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8):
     """One fused Adam step (src/optim/adam.cpp:52-113): returns the new parameter, updates m and v in place.
     The bias-correction scales are computed in float32 on the host exactly as the reference computes them."""

@@ -42,6 +42,15 @@ void exp_(Tensor &x);
 void log_(Tensor &x);
 void square_(Tensor &x);
 void relu_(Tensor &x);
+// src/operators/normalization/batch_norm.cpp:16-139. num_dims 2 = [N, C], 4 = [N, C, H, W]; momentum is carried for
+// the interface only (the layers update their running statistics themselves).
+Tensor batch_norm(const Tensor &x, const Tensor &gamma, const Tensor &beta, const Tensor &running_mean,
+                  const Tensor &running_var, bool training = false, float eps = 1e-5f, float momentum = 0.1f,
+                  int num_dims = 4);
+// the same operator with all of its outputs: y, and in training mode the batch mean and variance
+std::vector<Tensor> batch_norm_outputs(const Tensor &x, const Tensor &gamma, const Tensor &beta,
+                                       const Tensor &running_mean, const Tensor &running_var, bool training, float eps,
+                                       float momentum, int num_dims);
 Tensor softmax(const Tensor &x, int axis = -1);
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &target);
 Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b = nullptr, std::pair<int, int> stride = {1, 1},

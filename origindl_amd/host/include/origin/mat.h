@@ -115,6 +115,20 @@ public:
     virtual std::unique_ptr<Mat> yolo_detect_forward(const Mat &conv_weight, const Mat *conv_bias, const Mat &grid,
                                                      const Mat &anchor_grid, float stride, int32_t num_anchors,
                                                      int32_t num_classes) const = 0;
+    // ---- batch normalisation (mat.h:584-649 of the reference); num_dims 2 = [N, C], 4 = [N, C, H, W]
+    struct BatchNormResult
+    {
+        std::unique_ptr<Mat> y, mean, var, x_norm;
+    };
+    virtual BatchNormResult batch_norm_forward(const Mat &gamma, const Mat &beta, const Mat &running_mean,
+                                               const Mat &running_var, bool training, float eps,
+                                               int num_dims) const = 0;
+    virtual std::unique_ptr<Mat> batch_norm(const Mat &gamma, const Mat &beta, const Mat &running_mean,
+                                            const Mat &running_var, bool training, float eps, float momentum,
+                                            int num_dims) const = 0;
+    virtual std::vector<std::unique_ptr<Mat>> batch_norm_backward(const Mat &gy, const Mat &gamma, const Mat &saved_mean,
+                                                                  const Mat &saved_var, const Mat &saved_x_norm,
+                                                                  float eps, int num_dims) const = 0;
     // ---- convolution / pooling
     virtual std::unique_ptr<Mat> im2col(std::pair<int, int> kernel_size, std::pair<int, int> stride,
                                         std::pair<int, int> pad, bool to_matrix = true) const = 0;
@@ -221,6 +235,13 @@ public:
                                              const Mat &anchor_grid, float stride, int32_t num_anchors,
                                              int32_t num_classes) const override;
 
+    BatchNormResult batch_norm_forward(const Mat &gamma, const Mat &beta, const Mat &running_mean, const Mat &running_var,
+                                       bool training, float eps, int num_dims) const override;
+    std::unique_ptr<Mat> batch_norm(const Mat &gamma, const Mat &beta, const Mat &running_mean, const Mat &running_var,
+                                    bool training, float eps, float momentum, int num_dims) const override;
+    std::vector<std::unique_ptr<Mat>> batch_norm_backward(const Mat &gy, const Mat &gamma, const Mat &saved_mean,
+                                                          const Mat &saved_var, const Mat &saved_x_norm, float eps,
+                                                          int num_dims) const override;
     std::unique_ptr<Mat> im2col(std::pair<int, int> kernel_size, std::pair<int, int> stride, std::pair<int, int> pad,
                                 bool to_matrix = true) const override;
     std::unique_ptr<Mat> col2im(const Shape &input_shape, std::pair<int, int> kernel_size, std::pair<int, int> stride,
@@ -254,6 +275,9 @@ public:
     std::unique_ptr<Mat> max_pool2d_backward_device(const Mat &gy, std::pair<int, int> kernel_size,
                                                     std::pair<int, int> stride, std::pair<int, int> pad,
                                                     const Storage &indices) const;
+    // a*this + b*other in one launch (each product rounded before the sum): the running-statistics update of the
+    // BatchNorm layers
+    std::unique_ptr<Mat> axpby(float a, float b, const Mat &other) const;
     // fused optimizer steps (one launch each; same per-element arithmetic as the op-by-op sequences of
     // src/optim/adam.cpp:52-113 and src/optim/sgd.cpp:18-75). m and v are updated in place.
     std::unique_ptr<Mat> adam_step(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, float m_hat_scale,

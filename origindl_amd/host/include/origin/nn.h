@@ -34,6 +34,8 @@ protected:
     bool training_;
 };
 
+using Layer = Module;  // the reference's layers derive from an empty Layer : Module
+
 class Sequential : public Module
 {
 public:
@@ -110,6 +112,49 @@ public:
 
 private:
     int start_, end_;
+};
+
+// gamma ones, beta zeros, running mean zeros, running variance ones (src/nn/layers/batch_norm2d.cpp:12-35). In
+// training mode each forward normalises with the batch statistics and then folds them into the running ones as
+// running = momentum * running + (1 - momentum) * batch (batch_norm2d.cpp:62-86: this order, not the usual one);
+// in evaluation mode the running statistics are used. The update is one device launch per statistic here; the
+// reference copies four vectors to the host and two back. Only gamma ("weight") and beta ("bias") are registered
+// parameters, as in the reference, but to(device) also moves the running statistics.
+class BatchNormBase : public Module
+{
+public:
+    Tensor forward(const Tensor &input) override;
+    Parameter *weight() { return &gamma_; }
+    Parameter *bias() { return &beta_; }
+    const Tensor &running_mean() const { return running_mean_; }
+    const Tensor &running_var() const { return running_var_; }
+    void reset_parameters();
+    void to(Device device) override;
+    using Module::to;
+
+protected:
+    BatchNormBase(const char *name, int num_dims, int num_features, float eps, float momentum);
+    const char *name_;
+    int num_dims_, num_features_;
+    float eps_, momentum_;
+    Parameter gamma_, beta_;
+    Tensor running_mean_, running_var_;
+};
+
+class BatchNorm1d : public BatchNormBase  // input [N, C] (src/nn/layers/batch_norm1d.cpp)
+{
+public:
+    explicit BatchNorm1d(int num_features, float eps = 1e-5f, float momentum = 0.1f)
+        : BatchNormBase("BatchNorm1d", 2, num_features, eps, momentum)
+    {}
+};
+
+class BatchNorm2d : public BatchNormBase  // input [N, C, H, W] (src/nn/layers/batch_norm2d.cpp)
+{
+public:
+    explicit BatchNorm2d(int num_features, float eps = 1e-5f, float momentum = 0.1f)
+        : BatchNormBase("BatchNorm2d", 4, num_features, eps, momentum)
+    {}
 };
 
 // MLP({784, 1000, 10}, relu): Linear layers with the activation between them, none after the last

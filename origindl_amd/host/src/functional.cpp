@@ -438,6 +438,50 @@ struct Upsample : Operator  // src/operators/nn/upsample.cpp:13-90
     }
 };
 
+struct BatchNorm : Operator  // src/operators/normalization/batch_norm.cpp:16-122
+{
+    bool training;
+    float eps, momentum;
+    int num_dims;
+    Tensor saved_mean, saved_var, saved_x_norm;
+    BatchNorm(bool t, float e, float m, int nd) : training(t), eps(e), momentum(m), num_dims(nd) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        if (xs.size() != 5)
+            THROW_RUNTIME_ERROR("BatchNorm operator requires exactly 5 inputs (x, gamma, beta, running_mean, "
+                                "running_var), but got {}", xs.size());
+        Tensor y;
+        if (xs[0].requires_grad() || xs[1].requires_grad() || xs[2].requires_grad())
+        {
+            auto r = mat(xs[0]).batch_norm_forward(mat(xs[1]), mat(xs[2]), mat(xs[3]), mat(xs[4]), training, eps, num_dims);
+            y = wrap(std::move(r.y));
+            saved_mean = wrap(std::move(r.mean)), saved_var = wrap(std::move(r.var));
+            saved_x_norm = wrap(std::move(r.x_norm));
+        }
+        else if (training)
+        {
+            // the layers read the batch statistics off the operator's outputs, so they are computed here too
+            auto r = mat(xs[0]).batch_norm_forward(mat(xs[1]), mat(xs[2]), mat(xs[3]), mat(xs[4]), training, eps, num_dims);
+            y = wrap(std::move(r.y));
+            saved_mean = wrap(std::move(r.mean)), saved_var = wrap(std::move(r.var));
+        }
+        else
+            y = wrap(mat(xs[0]).batch_norm(mat(xs[1]), mat(xs[2]), mat(xs[3]), mat(xs[4]), training, eps, momentum, num_dims));
+        if (training)
+            return {y, saved_mean, saved_var};
+        return {y};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        // the gradient of y only: the statistics outputs feed the running averages, outside the graph
+        auto r = mat(inputs_[0]).batch_norm_backward(mat(gys[0]), mat(inputs_[1]), mat(saved_mean), mat(saved_var),
+                                                     mat(saved_x_norm), eps, num_dims);
+        const auto opt = dtype(DataType::kFloat32).device(inputs_[0].device());
+        return {wrap(std::move(r[0])), wrap(std::move(r[1])), wrap(std::move(r[2])), Tensor::zeros(inputs_[3].shape(), opt),
+                Tensor::zeros(inputs_[4].shape(), opt)};
+    }
+};
+
 template <typename Op, typename... A>
 Tensor apply(const std::vector<Tensor> &xs, A &&...args)
 {
@@ -484,6 +528,17 @@ void exp_(Tensor &x) { writable(x).exp_inplace(); }
 void log_(Tensor &x) { writable(x).log_inplace(); }
 void square_(Tensor &x) { writable(x).square_inplace(); }
 void relu_(Tensor &x) { writable(x).relu_inplace(); }
+std::vector<Tensor> batch_norm_outputs(const Tensor &x, const Tensor &gamma, const Tensor &beta, const Tensor &rm,
+                                       const Tensor &rv, bool training, float eps, float momentum, int num_dims)
+{
+    auto op = std::make_shared<BatchNorm>(training, eps, momentum, num_dims);
+    return (*op)({x, gamma, beta, rm, rv});
+}
+Tensor batch_norm(const Tensor &x, const Tensor &gamma, const Tensor &beta, const Tensor &rm, const Tensor &rv,
+                  bool training, float eps, float momentum, int num_dims)
+{
+    return batch_norm_outputs(x, gamma, beta, rm, rv, training, eps, momentum, num_dims)[0];
+}
 Tensor softmax(const Tensor &x, int axis) { return apply<Softmax>({x}, axis); }
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &t) { return apply<SoftmaxCrossEntropy>({x, t}); }
 

@@ -524,6 +524,111 @@ std::unique_ptr<Mat> OriginMat::upsample_backward(const Mat &gym, const Shape &x
     return gx;
 }
 
+// ---- batch normalisation (src/mat/origin/cpu/normalization/batch_norm.cpp:31-258, 279-418: same checks, same text)
+namespace
+{
+struct BnShape
+{
+    int64_t N, C, P;
+};
+
+BnShape bn_check(const char *who, const OriginMat &x, int num_dims, const Mat &gamma, const Mat &beta, const Mat &rm,
+                 const Mat &rv)
+{
+    if (x.shape().size() != (size_t)num_dims)
+        THROW_INVALID_ARG("{}: x must have {} dimensions, but got shape {}", who, num_dims, x.shape().to_string());
+    if (num_dims != 2 && num_dims != 4)
+        THROW_INVALID_ARG("{}: num_dims must be 2 or 4, but got {}", who, num_dims);
+    const size_t C = x.shape()[1];
+    if (gamma.shape() != Shape({C}) || beta.shape() != Shape({C}) || rm.shape() != Shape({C}) || rv.shape() != Shape({C}))
+        THROW_INVALID_ARG("{}: gamma, beta, running_mean, running_var must have shape ({})", who, C);
+    if (x.dtype() != DataType::kFloat32 && x.dtype() != DataType::kFloat64)
+        THROW_INVALID_ARG("{}: input x must be float32 or float64, but got {}", who, static_cast<int>(x.dtype()));
+    if (gamma.dtype() != x.dtype() || beta.dtype() != x.dtype() || rm.dtype() != x.dtype() || rv.dtype() != x.dtype())
+        THROW_INVALID_ARG("{}: all inputs (x, gamma, beta, running_mean, running_var) must have the same "
+                          "floating-point dtype", who);
+    return BnShape{(int64_t)x.shape()[0], (int64_t)C,
+                   num_dims == 4 ? (int64_t)(x.shape()[2] * x.shape()[3]) : (int64_t)1};
+}
+}  // namespace
+
+Mat::BatchNormResult OriginMat::batch_norm_forward(const Mat &gamma, const Mat &beta, const Mat &running_mean,
+                                                   const Mat &running_var, bool training, float eps,
+                                                   int num_dims) const
+{
+    const BnShape s = bn_check("batch_norm", *this, num_dims, gamma, beta, running_mean, running_var);
+    const OriginMat &x = dev_f32(*this, "batch_norm");
+    const OriginMat &g = dev_f32(gamma, "batch_norm"), &b = dev_f32(beta, "batch_norm");
+    const OriginMat &rm = dev_f32(running_mean, "batch_norm"), &rv = dev_f32(running_var, "batch_norm");
+    BatchNormResult r;
+    auto y = new_like(x, shape_), xn = new_like(x, shape_);
+    auto mean = new_like(x, Shape({(size_t)s.C})), var = new_like(x, Shape({(size_t)s.C}));
+    Workspace ws(training ? odl_hip_batch_norm_workspace_bytes(s.N, s.C, s.P) : 0, device().index());
+    check(odl_hip_batch_norm_forward(fp(x), fp(g), fp(b), fp(rm), fp(rv), training ? 1 : 0, eps, s.N, s.C, s.P,
+                                     y->data_ptr<float>(), mean->data_ptr<float>(), var->data_ptr<float>(),
+                                     xn->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+    r.y = std::move(y), r.mean = std::move(mean), r.var = std::move(var), r.x_norm = std::move(xn);
+    return r;
+}
+
+std::unique_ptr<Mat> OriginMat::batch_norm(const Mat &gamma, const Mat &beta, const Mat &running_mean,
+                                           const Mat &running_var, bool training, float eps, float, int num_dims) const
+{
+    const BnShape s = bn_check("batch_norm", *this, num_dims, gamma, beta, running_mean, running_var);
+    const OriginMat &x = dev_f32(*this, "batch_norm");
+    const OriginMat &g = dev_f32(gamma, "batch_norm"), &b = dev_f32(beta, "batch_norm");
+    const OriginMat &rm = dev_f32(running_mean, "batch_norm"), &rv = dev_f32(running_var, "batch_norm");
+    auto y = new_like(x, shape_);
+    auto mean = new_like(x, Shape({(size_t)s.C})), var = new_like(x, Shape({(size_t)s.C}));
+    Workspace ws(training ? odl_hip_batch_norm_workspace_bytes(s.N, s.C, s.P) : 0, device().index());
+    check(odl_hip_batch_norm_forward(fp(x), fp(g), fp(b), fp(rm), fp(rv), training ? 1 : 0, eps, s.N, s.C, s.P,
+                                     y->data_ptr<float>(), mean->data_ptr<float>(), var->data_ptr<float>(), nullptr,
+                                     ws.ptr(), ws.bytes, nullptr));
+    return y;
+}
+
+std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward(const Mat &gym, const Mat &gamma, const Mat &saved_mean,
+                                                                 const Mat &saved_var, const Mat &saved_x_norm, float eps,
+                                                                 int num_dims) const
+{
+    if (shape_.size() != (size_t)num_dims)
+        THROW_INVALID_ARG("batch_norm_backward: x must have {} dimensions, but got shape {}", num_dims, shape_.to_string());
+    if (num_dims != 2 && num_dims != 4)
+        THROW_INVALID_ARG("batch_norm_backward: num_dims must be 2 or 4, but got {}", num_dims);
+    const size_t C = shape_[1];
+    if (gym.shape() != shape_ || gamma.shape() != Shape({C}) || saved_mean.shape() != Shape({C}) ||
+        saved_var.shape() != Shape({C}) || saved_x_norm.shape() != shape_)
+        THROW_INVALID_ARG("batch_norm_backward: shape mismatch");
+    if (dtype() != DataType::kFloat32 && dtype() != DataType::kFloat64)
+        THROW_INVALID_ARG("batch_norm_backward: input x must be float32 or float64, but got {}", static_cast<int>(dtype()));
+    if (gym.dtype() != dtype() || gamma.dtype() != dtype() || saved_mean.dtype() != dtype() ||
+        saved_var.dtype() != dtype() || saved_x_norm.dtype() != dtype())
+        THROW_INVALID_ARG("batch_norm_backward: all inputs (gy, x, gamma, saved_mean, saved_var, saved_x_norm) must "
+                          "have the same floating-point dtype");
+    const OriginMat &x = dev_f32(*this, "batch_norm_backward");
+    const OriginMat &gy = dev_f32(gym, "batch_norm_backward"), &g = dev_f32(gamma, "batch_norm_backward");
+    const OriginMat &sv = dev_f32(saved_var, "batch_norm_backward"), &xn = dev_f32(saved_x_norm, "batch_norm_backward");
+    const int64_t N = (int64_t)shape_[0], P = num_dims == 4 ? (int64_t)(shape_[2] * shape_[3]) : 1;
+    auto gx = new_like(x, shape_);
+    auto dgamma = new_like(x, Shape({C})), dbeta = new_like(x, Shape({C}));
+    Workspace ws(odl_hip_batch_norm_workspace_bytes(N, (int64_t)C, P), device().index());
+    check(odl_hip_batch_norm_backward(fp(gy), fp(g), fp(sv), fp(xn), eps, N, (int64_t)C, P, gx->data_ptr<float>(),
+                                      dgamma->data_ptr<float>(), dbeta->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+    std::vector<std::unique_ptr<Mat>> outs;
+    outs.push_back(std::move(gx)), outs.push_back(std::move(dgamma)), outs.push_back(std::move(dbeta));
+    return outs;
+}
+
+std::unique_ptr<Mat> OriginMat::axpby(float a, float b, const Mat &other) const
+{
+    const OriginMat &x = dev_f32(*this, "axpby"), &y = dev_f32(other, "axpby");
+    if (x.shape() != y.shape())
+        THROW_INVALID_ARG("axpby: shape mismatch {} vs {}", x.shape().to_string(), y.shape().to_string());
+    auto o = new_like(x, shape_);
+    check(odl_hip_axpby(a, fp(x), b, fp(y), (int64_t)elements(), o->data_ptr<float>(), nullptr));
+    return o;
+}
+
 std::vector<std::unique_ptr<Mat>> OriginMat::split(const std::vector<size_t> &sizes, int dim) const
 {
     const OriginMat &x = dev_f32(*this, "split");

@@ -54,6 +54,61 @@ void Module::zero_grad()
         p->clear_grad();
 }
 
+namespace nn
+{
+BatchNormBase::BatchNormBase(const char *name, int num_dims, int num_features, float eps, float momentum)
+    : name_(name), num_dims_(num_dims), num_features_(num_features), eps_(eps), momentum_(momentum)
+{
+    if (num_features <= 0)
+        THROW_INVALID_ARG("{}: num_features must be positive, but got {}", name, num_features);
+    reset_parameters();
+    register_parameter("weight", gamma_);
+    register_parameter("bias", beta_);
+}
+
+void BatchNormBase::reset_parameters()
+{
+    const Shape s{static_cast<size_t>(num_features_)};
+    gamma_ = Parameter(Tensor::ones(s, TensorOptions(DataType::kFloat32).requires_grad(true)));
+    beta_ = Parameter(Tensor::zeros(s, TensorOptions(DataType::kFloat32).requires_grad(true)));
+    running_mean_ = Tensor::zeros(s, TensorOptions(DataType::kFloat32));
+    running_var_ = Tensor::ones(s, TensorOptions(DataType::kFloat32));
+}
+
+void BatchNormBase::to(Device device)
+{
+    Module::to(device);
+    if (running_mean_.device() != device)
+        running_mean_ = running_mean_.to(device);
+    if (running_var_.device() != device)
+        running_var_ = running_var_.to(device);
+}
+
+Tensor BatchNormBase::forward(const Tensor &input)
+{
+    const Shape s = input.shape();
+    if (s.size() != static_cast<size_t>(num_dims_))
+        THROW_RUNTIME_ERROR("{} forward: input must be {}, but got shape {}", name_,
+                            num_dims_ == 4 ? "4D (N, C, H, W)" : "2D (N, C)", s.to_string());
+    if (s[1] != static_cast<size_t>(num_features_))
+        THROW_RUNTIME_ERROR("{} forward: input feature size {} does not match num_features {}", name_, s[1],
+                            num_features_);
+    auto outs = functional::batch_norm_outputs(input, static_cast<const Tensor &>(gamma_),
+                                               static_cast<const Tensor &>(beta_), running_mean_, running_var_,
+                                               is_training(), eps_, momentum_, num_dims_);
+    if (is_training() && outs.size() >= 3)
+    {
+        auto fold = [&](const Tensor &running, const Tensor &batch) {
+            const auto &r = static_cast<const OriginMat &>(*running.impl_->data_);
+            return Tensor(r.axpby(momentum_, 1.0f - momentum_, *batch.impl_->data_));
+        };
+        running_mean_ = fold(running_mean_, outs[1]);
+        running_var_ = fold(running_var_, outs[2]);
+    }
+    return outs[0];
+}
+}  // namespace nn
+
 Tensor Sequential::forward(const Tensor &input)
 {
     Tensor x = input;

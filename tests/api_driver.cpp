@@ -11,6 +11,8 @@
 #include <cstdint>
 #include <chrono>
 #include <cmath>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <random>
@@ -46,6 +48,9 @@
 #include "origin/operators/math/sub.h"
 #include "origin/operators/math/sum.h"
 #include "origin/operators/math/sum_to.h"
+#include "origin/nn/layers/batch_norm1d.h"
+#include "origin/nn/layers/batch_norm2d.h"
+#include "origin/operators/normalization/batch_norm.h"
 #include "origin/operators/pooling/max_pool2d.h"
 #include "origin/optim/adam.h"
 #include "origin/optim/hooks.h"
@@ -124,14 +129,53 @@ int guarded(Fn &&fn)
         fn();
         return 0;
     }
-    catch (const std::invalid_argument &)
+    catch (const std::invalid_argument &e)
     {
+        if (std::getenv("ODL_DRV_VERBOSE"))
+            std::fprintf(stderr, "driver: invalid_argument: %s\n", e.what());
         return -1;
     }
-    catch (const std::exception &)
+    catch (const std::exception &e)
     {
+        if (std::getenv("ODL_DRV_VERBOSE"))
+            std::fprintf(stderr, "driver: exception: %s\n", e.what());
         return -2;
     }
+}
+}  // namespace
+
+namespace
+{
+template <class L>
+void bn_layer_run(L &layer, const float *x, const Shape &xs, int64_t C, int steps, float scale, float *y_train,
+                  float *y_eval, float *grads, bool with_backward)
+{
+    layer.to(kDev);
+    layer.train(true);
+    Tensor X, Y;
+    for (int s = 0; s < steps; ++s)
+    {
+        std::vector<float> xv(x, x + xs.elements());
+        for (auto &v : xv)
+            v = v * (1.0f + scale * (float)s);
+        X = f32(xv.data(), xs, true);  // a leaf, so that its gradient survives backward
+        Y = layer.forward(X);
+    }
+    out(Y, y_train);
+    if (with_backward)
+    {
+        // The reference itself cannot do this step: its operator moves the saved batch statistics into its outputs
+        // (src/operators/normalization/batch_norm.cpp:78-83) and backward then finds them empty.
+        auto loss = F::sum(Y * Y);
+        layer.zero_grad();
+        loss.backward();
+        float *gp = grads;
+        out(X.grad(), gp), gp += xs.elements();
+        out(layer.weight()->grad(), gp), gp += C;
+        out(layer.bias()->grad(), gp);
+    }
+    layer.train(false);
+    out(layer.forward(f32(x, xs)), y_eval);
 }
 }  // namespace
 
@@ -422,6 +466,64 @@ int DRV(yolo_detect)(const float *x, const float *w, const float *b, const float
         auto gm = mat_f32(grid, Shape{1, A, (size_t)H, (size_t)W, 2});
         auto am = mat_f32(anchor_grid, Shape{1, A, (size_t)anchor_H, (size_t)anchor_W, 2});
         out(*xm->yolo_detect_forward(*wm, bm.get(), *gm, *am, stride, num_anchors, num_classes), o);
+    });
+}
+
+// ---- batch normalisation at the Mat interface (mat.h:584-649); H == 0 selects the two-dimensional [N, C] form
+int DRV(batch_norm_forward)(const float *x, const float *gamma, const float *beta, const float *rm, const float *rv,
+                            int training, float eps, int64_t N, int64_t C, int64_t H, int64_t W, float *y, float *mean,
+                            float *var, float *x_norm)
+{
+    return guarded([&] {
+        const int nd = H == 0 ? 2 : 4;
+        const Shape xs = nd == 2 ? Shape{(size_t)N, (size_t)C} : Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W};
+        auto xm = mat_f32(x, xs);
+        auto g = mat_f32(gamma, Shape{(size_t)C}), b = mat_f32(beta, Shape{(size_t)C});
+        auto m = mat_f32(rm, Shape{(size_t)C}), v = mat_f32(rv, Shape{(size_t)C});
+        if (x_norm)
+        {
+            auto r = xm->batch_norm_forward(*g, *b, *m, *v, training != 0, eps, nd);
+            out(*r.y, y), out(*r.mean, mean), out(*r.var, var), out(*r.x_norm, x_norm);
+        }
+        else
+            out(*xm->batch_norm(*g, *b, *m, *v, training != 0, eps, 0.1f, nd), y);
+    });
+}
+
+int DRV(batch_norm_backward)(const float *gy, const float *x, const float *gamma, const float *saved_mean,
+                             const float *saved_var, const float *saved_x_norm, float eps, int64_t N, int64_t C, int64_t H,
+                             int64_t W, float *gx, float *dgamma, float *dbeta)
+{
+    return guarded([&] {
+        const int nd = H == 0 ? 2 : 4;
+        const Shape xs = nd == 2 ? Shape{(size_t)N, (size_t)C} : Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W};
+        auto xm = mat_f32(x, xs), gm = mat_f32(gy, xs), xn = mat_f32(saved_x_norm, xs);
+        auto g = mat_f32(gamma, Shape{(size_t)C});
+        auto m = mat_f32(saved_mean, Shape{(size_t)C}), v = mat_f32(saved_var, Shape{(size_t)C});
+        auto r = xm->batch_norm_backward(*gm, *g, *m, *v, *xn, eps, nd);
+        out(*r[0], gx), out(*r[1], dgamma), out(*r[2], dbeta);
+    });
+}
+
+// nn::BatchNorm2d (H > 0) or nn::BatchNorm1d (H == 0) in training mode, `steps` forwards of x * (1 + scale*step):
+// the last output, with_backward: the gradients of sum(y*y) from that forward (the scaled input, then gamma, then
+// beta), and one evaluation-mode forward of x. Exercises the running-statistics update (batch_norm2d.cpp:62-86) and the operator's
+// backward through the autograd engine.
+int DRV(batch_norm_layer)(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int steps, float eps, float momentum,
+                          float scale, int with_backward, float *y_train, float *y_eval, float *grads)
+{
+    return guarded([&] {
+        if (H == 0)
+        {
+            nn::BatchNorm1d layer((int)C, eps, momentum);
+            bn_layer_run(layer, x, Shape{(size_t)N, (size_t)C}, C, steps, scale, y_train, y_eval, grads, with_backward != 0);
+        }
+        else
+        {
+            nn::BatchNorm2d layer((int)C, eps, momentum);
+            bn_layer_run(layer, x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W}, C, steps, scale, y_train, y_eval,
+                         grads, with_backward != 0);
+        }
     });
 }
 

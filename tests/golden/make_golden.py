@@ -272,6 +272,41 @@ def main():
         assert tuple(oshape[:nd[0]]) == tuple(shp)
     out["y5n64_x"], out["y5n64_out"] = xin, o
 
+    # --- batch normalisation: Mat-level forward (training and evaluation) and backward in both layouts, and the
+    # layers (running statistics over three training forwards, gradients through autograd, an evaluation forward) ---
+    rb = np.random.default_rng(11)
+    for nm, (N, C, H, W) in {"bnA": (6, 5, 0, 0), "bnB": (3, 4, 5, 6), "bnC": (1, 2, 3, 3), "bnD": (4, 3, 2, 2)}.items():
+        P = max(H * W, 1)
+        xs = (N, C) if H == 0 else (N, C, H, W)
+        x = (rb.standard_normal(xs, dtype=f32) * f32(2) + f32(0.5)).astype(f32)
+        gamma = (rb.random(C, dtype=f32) + f32(0.5)).astype(f32)
+        beta = rb.standard_normal(C, dtype=f32)
+        rm = rb.standard_normal(C, dtype=f32)
+        rv = (rb.random(C, dtype=f32) + f32(0.25)).astype(f32)
+        gy = rb.standard_normal(xs, dtype=f32)
+        out[f"{nm}_x"], out[f"{nm}_gamma"], out[f"{nm}_beta"], out[f"{nm}_rm"], out[f"{nm}_rv"], out[f"{nm}_gy"] = \
+            x, gamma, beta, rm, rv, gy
+        for mode, training in (("train", 1), ("eval", 0)):
+            y, xn = np.empty(xs, f32), np.empty(xs, f32)
+            mean, var = np.empty(C, f32), np.empty(C, f32)
+            assert r.odl_ref_batch_norm_forward(x, gamma, beta, rm, rv, training, 1e-5, N, C, H, W, y, mean, var, xn) == 0
+            out[f"{nm}_{mode}_y"], out[f"{nm}_{mode}_mean"], out[f"{nm}_{mode}_var"], out[f"{nm}_{mode}_xn"] = y, mean, var, xn
+            y_only = np.empty(xs, f32)
+            assert r.odl_ref_batch_norm_forward(x, gamma, beta, rm, rv, training, 1e-5, N, C, H, W, y_only, None, None,
+                                                None) == 0
+            assert np.array_equal(y_only, y)
+            if training:
+                gx, dg, db = np.empty(xs, f32), np.empty(C, f32), np.empty(C, f32)
+                assert r.odl_ref_batch_norm_backward(gy, x, gamma, mean, var, xn, 1e-5, N, C, H, W, gx, dg, db) == 0
+                out[f"{nm}_gx"], out[f"{nm}_dgamma"], out[f"{nm}_dbeta"] = gx, dg, db
+        # the reference's operator cannot run backward in training mode (it moves its saved statistics away,
+        # operators/normalization/batch_norm.cpp:78-83), so the layer fixture holds the two forwards only
+        yt, ye = np.empty(xs, f32), np.empty(xs, f32)
+        assert r.odl_ref_batch_norm_layer(x, N, C, H, W, 3, 1e-5, 0.1, 0.25, 0, yt, ye, None) == 0
+        assert r.odl_ref_batch_norm_layer(x, N, C, H, W, 3, 1e-5, 0.1, 0.25, 1, yt.copy(), ye.copy(),
+                                          np.empty(x.size + 2 * C, f32)) == -2
+        out[f"{nm}_layer_ytrain"], out[f"{nm}_layer_yeval"] = yt, ye
+
     path = os.path.join(HERE, "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

@@ -47,6 +47,8 @@ _ORC_SIGS = {
     "orc_upsample_nearest": "p" + "llllll" + "ii" + "p>i",
     "orc_cat": "ppillp>i",
     "orc_yolo_detect_forward": "pppplp" + "lll" + "llll" + "f" + "ii" + "p>i",
+    "orc_batch_norm_forward": "pppppif" + "lll" + "pppp>i",
+    "orc_batch_norm_backward": "ppppf" + "lll" + "ppp>i",
     "orc_mlp_train_step": "ppillll" + "p" * 12 + "ifffff" + "pppppp>i",
     "orc_cnn_train_step": "ppillllll" + "p" * 8 + "f" + "p" + "pp" + "p" * 8 + "p>i",
 }
@@ -81,6 +83,9 @@ _REF_SIGS = {
     "odl_ref_cat": "ppillp>i",
     "odl_ref_pnnx_forward": "ppplllliplppp>i",
     "odl_ref_yolo_detect": "ppppp" + "ll" + "llll" + "f" + "ii" + "p>i",
+    "odl_ref_batch_norm_forward": "pppppif" + "llll" + "pppp>i",
+    "odl_ref_batch_norm_backward": "ppppppf" + "llll" + "ppp>i",
+    "odl_ref_batch_norm_layer": "pllllifffi" + "ppp" + ">i",
     "odl_ref_mlp_train": "ppillll" + "pppp" + "ifffff" + "pppppp>i",
     "odl_ref_cnn_train": "ppillllll" + "p" * 8 + "f" + "p" + "p" * 8 + "p>i",
     "odl_ref_mlp_bench": "lllliipp>i",

@@ -708,6 +708,77 @@ def test_compare_masks_activation_backward_split_and_upsample_backward(api):
     assert np.array_equal(host(api.upsample_backward(dev(ones), (1, 2, 4, 4), 2)), np.full((1, 2, 4, 4), 4, f32))
 
 
+# ------------------------------------------------------------------ batch normalisation
+BN_CASES = ("bnA", "bnB", "bnC", "bnD")
+
+
+@pytest.mark.parametrize("name", BN_CASES)
+def test_batch_norm_fixtures(api, name):
+    # fixtures from the compiled reference: [N, C] and [N, C, H, W], training and evaluation, and the gradient.
+    # Statistics are sums in a different (parallel) order than the reference's sequential loop: a few ulps of the mean
+    # and variance, carried into y; everything downstream of given statistics is the same arithmetic.
+    g = lambda k: G[f"{name}_{k}"]
+    x, gamma, beta, rm, rv = (dev(g(k)) for k in ("x", "gamma", "beta", "rm", "rv"))
+    for mode, training in (("train", True), ("eval", False)):
+        y, mean, var, xn = api.batch_norm_forward(x, gamma, beta, rm, rv, training)
+        tol = dict(rtol=2e-5, atol=2e-6) if training else dict(rtol=0, atol=0)
+        for got, key in ((y, "y"), (mean, "mean"), (var, "var"), (xn, "xn")):
+            np.testing.assert_allclose(host(got), g(f"{mode}_{key}"), err_msg=f"{mode} {key}", **tol)
+        y_only = api.batch_norm_forward(x, gamma, beta, rm, rv, training, want_x_norm=False)[0]
+        assert np.array_equal(host(y_only), host(y))
+    gx, dg, db = api.batch_norm_backward(dev(g("gy")), gamma, dev(g("train_var")), dev(g("train_xn")))
+    np.testing.assert_allclose(host(dg), g("dgamma"), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(host(db), g("dbeta"), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(host(gx), g("gx"), rtol=2e-5, atol=2e-5)
+
+
+def test_batch_norm_vs_oracle_at_cnn_sizes(api, o):
+    # the BatchNorm layers of the reference's conv_mnist example: [256, 32, 28, 28] and [256, 64, 14, 14]
+    # (scaled down in N so that the scalar oracle stays quick), a plane that is not a multiple of four, and [N, C]
+    rng = np.random.default_rng(41)
+    for shape in ((32, 32, 28, 28), (32, 64, 14, 14), (5, 7, 5, 5), (512, 100)):
+        N, C = shape[:2]
+        P = int(np.prod(shape[2:])) if len(shape) == 4 else 1
+        x = (rng.standard_normal(shape, dtype=f32) * f32(1.5) + f32(0.3)).astype(f32)
+        gamma = (rng.random(C, dtype=f32) + f32(0.5)).astype(f32)
+        beta = rng.standard_normal(C, dtype=f32)
+        gy = rng.standard_normal(shape, dtype=f32)
+        wy, wxn, wm, wv = np.empty(shape, f32), np.empty(shape, f32), np.empty(C, f32), np.empty(C, f32)
+        zeros, ones = np.zeros(C, f32), np.ones(C, f32)
+        assert o.orc_batch_norm_forward(x, gamma, beta, zeros, ones, 1, 1e-5, N, C, P, wy, wm, wv, wxn) == 0
+        y, mean, var, xn = api.batch_norm_forward(dev(x), dev(gamma), dev(beta), dev(zeros), dev(ones), True)
+        x64 = x.astype(np.float64).reshape(N, C, P)
+        # against double precision: both sums are float sums over N*P terms, the parallel one the more accurate
+        np.testing.assert_allclose(host(mean), x64.mean(axis=(0, 2)), rtol=0, atol=1e-6 * np.sqrt(N * P))
+        np.testing.assert_allclose(host(var), x64.var(axis=(0, 2)), rtol=1e-6 * np.sqrt(N * P))
+        np.testing.assert_allclose(host(mean), wm, rtol=0, atol=2e-6 * np.sqrt(N * P))
+        np.testing.assert_allclose(host(var), wv, rtol=2e-6 * np.sqrt(N * P))
+        np.testing.assert_allclose(host(y), wy, rtol=1e-4, atol=1e-4)
+        # backward from the oracle's own saved statistics: the channel sums differ by summation order only
+        wgx, wdg, wdb = np.empty(shape, f32), np.empty(C, f32), np.empty(C, f32)
+        assert o.orc_batch_norm_backward(gy, gamma, wv, wxn, 1e-5, N, C, P, wgx, wdg, wdb) == 0
+        gx, dg, db = api.batch_norm_backward(dev(gy), dev(gamma), dev(wv), dev(wxn))
+        bound = 2e-6 * np.sqrt(N * P) * 4
+        np.testing.assert_allclose(host(db), wdb, rtol=0, atol=bound * np.sqrt(N * P))
+        np.testing.assert_allclose(host(dg), wdg, rtol=0, atol=bound * np.sqrt(N * P))
+        np.testing.assert_allclose(host(gx), wgx, rtol=1e-4, atol=1e-5)
+    # evaluation mode has no reduction: bit-exact against the oracle at any size
+    x = rng.standard_normal((16, 64, 14, 14), dtype=f32)
+    gamma, beta, rm = (rng.standard_normal(64, dtype=f32) for _ in range(3))
+    rv = (rng.random(64, dtype=f32) + f32(0.1)).astype(f32)
+    wy, wxn, wm, wv = np.empty_like(x), np.empty_like(x), np.empty(64, f32), np.empty(64, f32)
+    assert o.orc_batch_norm_forward(x, gamma, beta, rm, rv, 0, 1e-5, 16, 64, 196, wy, wm, wv, wxn) == 0
+    y, mean, var, xn = api.batch_norm_forward(dev(x), dev(gamma), dev(beta), dev(rm), dev(rv), False)
+    assert np.array_equal(host(y), wy) and np.array_equal(host(xn), wxn)
+    assert np.array_equal(host(mean), rm) and np.array_equal(host(var), rv)
+    # the running-statistics update: momentum*running + (1 - momentum)*batch, products rounded first
+    a, b = rng.standard_normal(1001, dtype=f32), rng.standard_normal(1001, dtype=f32)
+    m = f32(0.1)
+    assert np.array_equal(host(api.axpby(m, dev(a), f32(1.0) - m, dev(b))), m * a + (f32(1.0) - m) * b)
+    with pytest.raises(api.OdlInvalidArgument):
+        api.batch_norm_forward(dev(x), dev(gamma[:3].copy()), dev(beta), dev(rm), dev(rv), True)
+
+
 @pytest.mark.parametrize("name", ["detA", "detB"])
 def test_yolo_detect_fixtures(api, name):
     ag = G[f"{name}_anchor_grid"]

@@ -329,7 +329,115 @@ def test_against_compiled_reference_fresh_inputs():
     assert acc[0] == o.orc_accuracy(y, t, 50, 6)
 
 
+BN_CASES = {"bnA": (6, 5, 0, 0), "bnB": (3, 4, 5, 6), "bnC": (1, 2, 3, 3), "bnD": (4, 3, 2, 2)}
+
+
+def bn_forward(x, gamma, beta, rm, rv, training, eps=1e-5, want_xn=True):
+    N, C = x.shape[:2]
+    P = int(np.prod(x.shape[2:])) if x.ndim == 4 else 1
+    y, xn = np.empty_like(x), np.empty_like(x)
+    mean, var = np.empty(C, f32), np.empty(C, f32)
+    assert o.orc_batch_norm_forward(x, gamma, beta, rm, rv, training, eps, N, C, P, y, mean, var,
+                                    xn if want_xn else None) == 0
+    return y, mean, var, xn
+
+
+def bn_backward(gy, gamma, var, xn, eps=1e-5):
+    N, C = gy.shape[:2]
+    P = int(np.prod(gy.shape[2:])) if gy.ndim == 4 else 1
+    gx, dg, db = np.empty_like(gy), np.empty(C, f32), np.empty(C, f32)
+    assert o.orc_batch_norm_backward(gy, gamma, var, xn, eps, N, C, P, gx, dg, db) == 0
+    return gx, dg, db
+
+
+@pytest.mark.parametrize("name", list(BN_CASES))
+def test_batch_norm_fixtures_bit_exact(name):
+    # written from the compiled reference (Mat::batch_norm_forward / batch_norm / batch_norm_backward and the layers)
+    g = lambda k: G[f"{name}_{k}"]
+    x, gamma, beta, rm, rv = g("x"), g("gamma"), g("beta"), g("rm"), g("rv")
+    for mode, training in (("train", 1), ("eval", 0)):
+        y, mean, var, xn = bn_forward(x, gamma, beta, rm, rv, training)
+        for got, key in ((y, "y"), (mean, "mean"), (var, "var"), (xn, "xn")):
+            assert np.array_equal(got, g(f"{mode}_{key}")), (mode, key)
+        assert np.array_equal(bn_forward(x, gamma, beta, rm, rv, training, want_xn=False)[0], y)
+    gx, dg, db = bn_backward(g("gy"), gamma, g("train_var"), g("train_xn"))
+    assert np.array_equal(gx, g("gx")) and np.array_equal(dg, g("dgamma")) and np.array_equal(db, g("dbeta"))
+    # the layers: three training forwards of x*(1 + 0.25*step) from running mean 0 / variance 1, each folding the batch
+    # statistics in as running = 0.1*running + 0.9*batch (batch_norm2d.cpp:77-80), then an evaluation forward of x
+    C = x.shape[1]
+    ones, zeros = np.ones(C, f32), np.zeros(C, f32)
+    rmean, rvar = zeros.copy(), ones.copy()
+    for step in range(3):
+        xs = (x * f32(1.0 + 0.25 * step)).astype(f32)
+        y, mean, var, _ = bn_forward(xs, ones, zeros, rmean, rvar, 1)
+        rmean = f32(0.1) * rmean + (f32(1.0) - f32(0.1)) * mean
+        rvar = f32(0.1) * rvar + (f32(1.0) - f32(0.1)) * var
+    assert np.array_equal(y, g("layer_ytrain"))
+    assert np.array_equal(bn_forward(x, ones, zeros, rmean, rvar, 0)[0], g("layer_yeval"))
+
+
+@needs_ref
+def test_batch_norm_against_compiled_reference_fresh_inputs():
+    r = ol.ref()
+    rng = np.random.default_rng(17)
+    for N, C, H, W in ((7, 3, 0, 0), (2, 5, 4, 7), (5, 1, 1, 1), (3, 6, 9, 9)):
+        xs = (N, C) if H == 0 else (N, C, H, W)
+        x = rng.standard_normal(xs, dtype=f32)
+        gamma, beta, rm = (rng.standard_normal(C, dtype=f32) for _ in range(3))
+        rv = (rng.random(C, dtype=f32) + f32(0.1)).astype(f32)
+        gy = rng.standard_normal(xs, dtype=f32)
+        for training in (1, 0):
+            y, xn, mean, var = np.empty(xs, f32), np.empty(xs, f32), np.empty(C, f32), np.empty(C, f32)
+            assert r.odl_ref_batch_norm_forward(x, gamma, beta, rm, rv, training, 1e-3, N, C, H, W, y, mean, var, xn) == 0
+            y2, mean2, var2, xn2 = bn_forward(x, gamma, beta, rm, rv, training, eps=1e-3)
+            assert all(np.array_equal(a, b) for a, b in ((y, y2), (mean, mean2), (var, var2), (xn, xn2)))
+        gx, dg, db = np.empty(xs, f32), np.empty(C, f32), np.empty(C, f32)
+        assert r.odl_ref_batch_norm_backward(gy, x, gamma, mean2, var2, xn2, 1e-3, N, C, H, W, gx, dg, db) == 0
+        gx2, dg2, db2 = bn_backward(gy, gamma, var2, xn2, eps=1e-3)
+        assert np.array_equal(gx, gx2) and np.array_equal(dg, dg2) and np.array_equal(db, db2)
+
 # ------------------------------------------------------------------------ 3. independent mathematics
+def test_batch_norm_against_float64_and_finite_differences():
+    rng = np.random.default_rng(18)
+    x = (rng.standard_normal((8, 3, 5, 7)) * 3 + 1).astype(f32)
+    gamma, beta = rng.standard_normal(3).astype(f32), rng.standard_normal(3).astype(f32)
+    y, mean, var, xn = bn_forward(x, gamma, beta, np.zeros(3, f32), np.ones(3, f32), 1)
+    x64 = x.astype(np.float64)
+    np.testing.assert_allclose(mean, x64.mean(axis=(0, 2, 3)), rtol=1e-5)
+    np.testing.assert_allclose(var, x64.var(axis=(0, 2, 3)), rtol=1e-5)  # the biased (population) variance
+    # normalised activations have zero mean and (almost) unit variance per channel whatever the input's scale
+    assert np.abs(xn.astype(np.float64).mean(axis=(0, 2, 3))).max() < 1e-6
+    np.testing.assert_allclose(xn.astype(np.float64).var(axis=(0, 2, 3)), var / (var + 1e-5), rtol=1e-5)
+    np.testing.assert_allclose(y, gamma[None, :, None, None] * xn + beta[None, :, None, None], rtol=1e-6, atol=1e-6)
+
+    def loss64(xv, gv, bv, r):
+        m, v = xv.mean(axis=(0, 2, 3), keepdims=True), xv.var(axis=(0, 2, 3), keepdims=True)
+        return float((((xv - m) / np.sqrt(v + 1e-5) * gv[None, :, None, None] + bv[None, :, None, None]) * r).sum())
+
+    r = rng.standard_normal(x.shape)
+    gx, dg, db = bn_backward(r.astype(f32), gamma, var, xn)
+    g64, b64 = gamma.astype(np.float64), beta.astype(np.float64)
+    h = 1e-4
+    for idx in [(0, 0, 0, 0), (3, 1, 2, 5), (7, 2, 4, 6)]:  # the statistics depend on x: the full Jacobian is checked
+        xp, xm = x64.copy(), x64.copy()
+        xp[idx] += h
+        xm[idx] -= h
+        fd = (loss64(xp, g64, b64, r) - loss64(xm, g64, b64, r)) / (2 * h)
+        assert abs(gx[idx] - fd) <= 2e-3 * max(1.0, abs(fd)), (idx, gx[idx], fd)
+    for c in range(3):
+        gp, gm = g64.copy(), g64.copy()
+        gp[c] += h
+        gm[c] -= h
+        assert abs(dg[c] - (loss64(x64, gp, b64, r) - loss64(x64, gm, b64, r)) / (2 * h)) <= 1e-3 * max(1.0, abs(dg[c]))
+        np.testing.assert_allclose(db[c], r[:, c].sum(), rtol=1e-4, atol=1e-4)
+    # evaluation mode is a per-channel affine map of x with the running statistics
+    rm, rv = rng.standard_normal(3).astype(f32), (rng.random(3) + 0.5).astype(f32)
+    ye = bn_forward(x, gamma, beta, rm, rv, 0)[0]
+    want = (x64 - rm[None, :, None, None]) / np.sqrt(rv[None, :, None, None].astype(np.float64) + 1e-5)
+    np.testing.assert_allclose(ye, want * g64[None, :, None, None] + b64[None, :, None, None], rtol=1e-5, atol=1e-5)
+
+
+
 def test_matmul_against_float64():
     rng = np.random.default_rng(1)
     a, b = rng.standard_normal((37, 211), dtype=f32), rng.standard_normal((211, 19), dtype=f32)
