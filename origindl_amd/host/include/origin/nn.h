@@ -8,7 +8,10 @@
 #include <unordered_map>
 #include <vector>
 
+#include <any>
+
 #include "functional.h"
+#include "io.h"
 
 namespace origin
 {
@@ -22,6 +25,13 @@ public:
     virtual std::vector<Parameter *> parameters();
     void register_parameter(const std::string &name, Parameter &param);
     void register_module(const std::string &name, std::unique_ptr<Module> module);
+    // name -> tensor of every registered parameter, children prefixed "child." (src/nn/module.cpp:120-207)
+    using StateDict = std::unordered_map<std::string, Tensor>;
+    virtual StateDict state_dict() const;
+    virtual void load_state_dict(const StateDict &state_dict, bool strict = true);
+    void load(const std::string &filepath, bool strict = true);
+    std::unordered_map<std::string, Parameter *> named_parameters(const std::string &prefix = "");
+    std::unordered_map<std::string, const Parameter *> named_parameters(const std::string &prefix) const;
     void train(bool mode = true);
     void eval() { train(false); }
     bool is_training() const { return training_; }
@@ -182,6 +192,10 @@ public:
     void step();       // filter params with a gradient -> hooks -> step_one each (src/optim/optimizer.cpp:19-53)
     void zero_grad();
     void register_hook(std::function<void(std::vector<Parameter *> &)> hook) { hooks_.push_back(std::move(hook)); }
+    // settings as float / bool values, buffers as StateDict values keyed "<kind>_<parameter name>"
+    // (src/optim/adam.cpp:116-284, src/optim/sgd.cpp:77-157)
+    virtual std::unordered_map<std::string, std::any> state_dict() const = 0;
+    virtual void load_state_dict(const std::unordered_map<std::string, std::any> &state_dict) = 0;
 
 protected:
     virtual void step_one(Parameter &param) = 0;
@@ -194,6 +208,8 @@ class SGD : public Optimizer  // src/optim/sgd.cpp:18-75
 {
 public:
     SGD(Module &target, float lr, float momentum = 0.0f, float weight_decay = 0.0f, bool nesterov = false);
+    std::unordered_map<std::string, std::any> state_dict() const override;
+    void load_state_dict(const std::unordered_map<std::string, std::any> &state_dict) override;
 
 protected:
     void step_one(Parameter &param) override;
@@ -208,6 +224,8 @@ class Adam : public Optimizer  // src/optim/adam.cpp:19-114
 {
 public:
     Adam(Module &target, float lr = 0.001f, float beta1 = 0.9f, float beta2 = 0.999f, float eps = 1e-8f);
+    std::unordered_map<std::string, std::any> state_dict() const override;
+    void load_state_dict(const std::unordered_map<std::string, std::any> &state_dict) override;
 
 protected:
     void step_one(Parameter &param) override;

@@ -54,6 +54,63 @@ void Module::zero_grad()
         p->clear_grad();
 }
 
+std::unordered_map<std::string, Parameter *> Module::named_parameters(const std::string &prefix)
+{
+    std::unordered_map<std::string, Parameter *> named;
+    for (auto &p : parameters_)
+        named[prefix.empty() ? p.first : prefix + "." + p.first] = p.second;
+    for (auto &m : modules_)
+    {
+        auto sub = m.second->named_parameters(prefix.empty() ? m.first : prefix + "." + m.first);
+        named.insert(sub.begin(), sub.end());
+    }
+    return named;
+}
+
+std::unordered_map<std::string, const Parameter *> Module::named_parameters(const std::string &prefix) const
+{
+    std::unordered_map<std::string, const Parameter *> named;
+    for (auto &p : const_cast<Module *>(this)->named_parameters(prefix))
+        named[p.first] = p.second;
+    return named;
+}
+
+Module::StateDict Module::state_dict() const
+{
+    StateDict sd;
+    for (auto &p : named_parameters(""))
+        sd[p.first] = static_cast<const Tensor &>(*p.second);
+    return sd;
+}
+
+void Module::load_state_dict(const StateDict &state_dict, bool strict)
+{
+    std::unordered_map<std::string, bool> loaded;
+    for (auto &[name, param] : named_parameters())
+    {
+        auto it = state_dict.find(name);
+        if (it != state_dict.end())
+        {
+            if (param->shape() != it->second.shape())
+                THROW_RUNTIME_ERROR("Shape mismatch for parameter '{}': expected {}, got {}", name,
+                                    param->shape().to_string(), it->second.shape().to_string());
+            *param = Parameter(it->second);
+            loaded[name] = true;
+        }
+        else if (strict)
+            THROW_RUNTIME_ERROR("Missing parameter '{}' in state_dict (strict mode)", name);
+    }
+    if (strict)
+        for (const auto &kv : state_dict)
+            if (!loaded.count(kv.first))
+                THROW_RUNTIME_ERROR("Unexpected parameter '{}' in state_dict (strict mode)", kv.first);
+}
+
+void Module::load(const std::string &filepath, bool strict)
+{
+    load_state_dict(origin::load(filepath), strict);
+}
+
 namespace nn
 {
 BatchNormBase::BatchNormBase(const char *name, int num_dims, int num_features, float eps, float momentum)
@@ -221,7 +278,7 @@ MLP::MLP(const std::vector<int> &sizes, std::function<Tensor(const Tensor &)> ac
     {
         auto l = std::make_unique<Linear>(sizes[i], sizes[i + 1], true);
         layers_.push_back(l.get());
-        register_module("l" + std::to_string(i), std::move(l));
+        register_module("layer_" + std::to_string(i), std::move(l));  // the names state_dict() keys are built from
     }
 }
 
@@ -385,4 +442,115 @@ void synchronize()
         THROW_RUNTIME_ERROR("{}", odl_hip_last_error());
 }
 }  // namespace cuda
+}  // namespace origin
+
+// ---- optimizer state (src/optim/adam.cpp:116-284, src/optim/sgd.cpp:77-157)
+namespace origin
+{
+namespace
+{
+std::string name_of(const std::unordered_map<std::string, const Parameter *> &named, const Parameter *p)
+{
+    for (const auto &kv : named)
+        if (kv.second == p)
+            return kv.first;
+    return "";
+}
+
+template <typename T>
+void read_setting(const std::unordered_map<std::string, std::any> &sd, const char *key, T &dst)
+{
+    auto it = sd.find(key);
+    if (it != sd.end())
+        dst = std::any_cast<T>(it->second);
+}
+
+void read_buffers(const std::unordered_map<std::string, std::any> &sd, const char *key, const std::string &prefix,
+                  std::unordered_map<std::string, Parameter *> &named, std::unordered_map<Parameter *, Tensor> &dst)
+{
+    auto it = sd.find(key);
+    if (it == sd.end())
+        return;
+    const auto buffers = std::any_cast<StateDict>(it->second);
+    dst.clear();
+    for (const auto &kv : buffers)
+        if (kv.first.size() > prefix.size() && kv.first.compare(0, prefix.size(), prefix) == 0)
+        {
+            auto p = named.find(kv.first.substr(prefix.size()));
+            if (p != named.end())
+                dst[p->second] = kv.second;
+        }
+}
+}  // namespace
+
+std::unordered_map<std::string, std::any> Adam::state_dict() const
+{
+    std::unordered_map<std::string, std::any> state;
+    state["lr"] = lr_, state["beta1"] = beta1_, state["beta2"] = beta2_, state["eps"] = eps_;
+    const auto named = static_cast<const Module *>(target_)->named_parameters("");
+    StateDict m, v;
+    std::unordered_map<std::string, int> steps;
+    for (const auto &kv : m_buffers_)
+        if (const std::string n = name_of(named, kv.first); !n.empty())
+            m["m_" + n] = kv.second;
+    for (const auto &kv : v_buffers_)
+        if (const std::string n = name_of(named, kv.first); !n.empty())
+            v["v_" + n] = kv.second;
+    for (const auto &kv : step_counts_)
+        if (const std::string n = name_of(named, kv.first); !n.empty())
+            steps["step_" + n] = kv.second;
+    state["m_buffers"] = m, state["v_buffers"] = v, state["step_counts"] = steps;
+    return state;
+}
+
+void Adam::load_state_dict(const std::unordered_map<std::string, std::any> &sd)
+{
+    read_setting(sd, "lr", lr_), read_setting(sd, "beta1", beta1_), read_setting(sd, "beta2", beta2_);
+    read_setting(sd, "eps", eps_);
+    auto named = target_->named_parameters("");
+    read_buffers(sd, "m_buffers", "m_", named, m_buffers_);
+    read_buffers(sd, "v_buffers", "v_", named, v_buffers_);
+    auto it = sd.find("step_counts");
+    if (it != sd.end())
+    {
+        const auto steps = std::any_cast<std::unordered_map<std::string, int>>(it->second);
+        step_counts_.clear();
+        for (const auto &kv : steps)
+            if (kv.first.size() > 5 && kv.first.compare(0, 5, "step_") == 0)
+            {
+                auto p = named.find(kv.first.substr(5));
+                if (p != named.end())
+                    step_counts_[p->second] = kv.second;
+            }
+    }
+}
+
+std::unordered_map<std::string, std::any> SGD::state_dict() const
+{
+    std::unordered_map<std::string, std::any> state;
+    state["lr"] = lr_, state["momentum"] = momentum_, state["weight_decay"] = weight_decay_, state["nesterov"] = nesterov_;
+    if (momentum_ > 0.0f)
+    {
+        const auto named = static_cast<const Module *>(target_)->named_parameters("");
+        StateDict buffers;
+        for (const auto &kv : momentum_buffers_)
+            if (const std::string n = name_of(named, kv.first); !n.empty())
+                buffers["momentum_" + n] = kv.second;
+        state["momentum_buffers"] = buffers;
+    }
+    return state;
+}
+
+// The reference compares a ten-character prefix with the nine-character "momentum_" and so never restores a
+// momentum buffer (sgd.cpp:146-148); here the buffers written by state_dict() are read back.
+void SGD::load_state_dict(const std::unordered_map<std::string, std::any> &sd)
+{
+    read_setting(sd, "lr", lr_), read_setting(sd, "momentum", momentum_), read_setting(sd, "weight_decay", weight_decay_);
+    read_setting(sd, "nesterov", nesterov_);
+    if (momentum_ > 0.0f)
+    {
+        auto named = target_->named_parameters("");
+        read_buffers(sd, "momentum_buffers", "momentum_", named, momentum_buffers_);
+    }
+}
 }  // namespace origin

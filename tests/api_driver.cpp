@@ -8,6 +8,7 @@
 //     the GPU): the same calls then run on the gfx950 backend, which is what "drop-in behind the Tensor/Operator/
 //     Mat interfaces" means; tests compare its results with the fixtures and the oracle.
 // Every entry point returns 0, or -1 for std::invalid_argument, -2 for any other std::exception.
+#include <any>
 #include <cstdint>
 #include <chrono>
 #include <cmath>
@@ -48,7 +49,10 @@
 #include "origin/operators/math/sub.h"
 #include "origin/operators/math/sum.h"
 #include "origin/operators/math/sum_to.h"
+#include "origin/io/checkpoint.h"
+#include "origin/io/model_io.h"
 #include "origin/nn/layers/batch_norm1d.h"
+#include "origin/nn/models/mlp.h"
 #include "origin/nn/layers/batch_norm2d.h"
 #include "origin/operators/normalization/batch_norm.h"
 #include "origin/operators/pooling/max_pool2d.h"
@@ -176,6 +180,36 @@ void bn_layer_run(L &layer, const float *x, const Shape &xs, int64_t C, int step
     }
     layer.train(false);
     out(layer.forward(f32(x, xs)), y_eval);
+}
+}  // namespace
+
+// ---- model files and checkpoints (include/origin/io/model_io.h, checkpoint.h). An nn::MLP({4, 8, 2}) whose four
+// parameters are set from `params` (layer_0.weight [4,8], layer_0.bias, layer_1.weight [8,2], layer_1.bias: 58 floats).
+namespace
+{
+const char *const kMlpNames[4] = {"layer_0.weight", "layer_0.bias", "layer_1.weight", "layer_1.bias"};
+
+void set_mlp(nn::MLP &model, const float *params)
+{
+    auto named = model.named_parameters("");
+    const float *p = params;
+    for (const char *name : kMlpNames)
+    {
+        Parameter *dst = named.at(name);
+        *dst = Parameter(f32(p, dst->shape(), true));
+        p += dst->shape().elements();
+    }
+}
+
+void get_mlp(nn::MLP &model, float *params)
+{
+    auto named = model.named_parameters("");
+    float *p = params;
+    for (const char *name : kMlpNames)
+    {
+        out(static_cast<const Tensor &>(*named.at(name)), p);
+        p += named.at(name)->shape().elements();
+    }
 }
 }  // namespace
 
@@ -527,6 +561,62 @@ int DRV(batch_norm_layer)(const float *x, int64_t N, int64_t C, int64_t H, int64
     });
 }
 
+// writes the model's state_dict() to `path` in the .odl format
+int DRV(save_mlp)(const float *params, const char *path)
+{
+    return guarded([&] {
+        nn::MLP model({4, 8, 2});
+        set_mlp(model, params);
+        save(model.state_dict(), path);
+    });
+}
+
+// Module::load(path, strict) into a fresh model; the loaded parameters come back in `params`, and y = model(x[3,4])
+// after moving the model to the driver's device
+int DRV(load_mlp)(const char *path, int strict, const float *x, float *params, float *y)
+{
+    return guarded([&] {
+        nn::MLP model({4, 8, 2});
+        model.load(path, strict != 0);
+        get_mlp(model, params);
+        if (y)
+        {
+            model.to(kDev);
+            out(model(f32(x, Shape{3, 4})), y);
+        }
+    });
+}
+
+// save(Checkpoint) then load_checkpoint of the same path: the metadata read back, and the parameters
+int DRV(checkpoint_roundtrip)(const float *params, const char *path, int epoch, int step, float loss, float lr, float beta1,
+                              float beta2, float eps, int *epoch_step /*2*/, float *floats /* loss lr beta1 beta2 eps */,
+                              float *params_out)
+{
+    return guarded([&] {
+        nn::MLP model({4, 8, 2});
+        set_mlp(model, params);
+        Adam opt(model, lr, beta1, beta2, eps);
+        Checkpoint ck;
+        ck.model_state_dict = model.state_dict();
+        ck.optimizer_state_dict["adam"] = opt.state_dict();
+        ck.epoch = epoch, ck.step = step, ck.loss = loss, ck.optimizer_type = "Adam";
+        ck.optimizer_config["lr"] = lr, ck.optimizer_config["beta1"] = beta1;
+        ck.optimizer_config["beta2"] = beta2, ck.optimizer_config["eps"] = eps;
+        save(ck, path);
+        Checkpoint back = load_checkpoint(path);
+        epoch_step[0] = back.epoch, epoch_step[1] = back.step;
+        floats[0] = back.loss, floats[1] = back.optimizer_config.at("lr"), floats[2] = back.optimizer_config.at("beta1");
+        floats[3] = back.optimizer_config.at("beta2"), floats[4] = back.optimizer_config.at("eps");
+        if (back.optimizer_type != "Adam")
+            throw std::runtime_error("optimizer type lost");
+        nn::MLP fresh({4, 8, 2});
+        fresh.load_state_dict(back.model_state_dict);
+        get_mlp(fresh, params_out);
+        auto st = opt.state_dict();
+        if (std::any_cast<float>(st.at("lr")) != lr || std::any_cast<float>(st.at("eps")) != eps)
+            throw std::runtime_error("optimizer state_dict does not hold its settings");
+    });
+}
 // A PNNX model (`.pnnx.param` + `.pnnx.bin`) run forward `reps` times on x[N,C,H,W]; the first output of
 // `pnnx_output_0` is copied to out (capacity in floats) and its shape to out_shape[0..out_nd). ms = mean time of the
 // forwards after the first (which also loads weights), each complete on the device; the output is read back once, after.

@@ -307,6 +307,16 @@ def main():
                                           np.empty(x.size + 2 * C, f32)) == -2
         out[f"{nm}_layer_ytrain"], out[f"{nm}_layer_yeval"] = yt, ye
 
+    # --- a model file written by the reference itself (.odl, src/io/model_io.cpp:116-168): an MLP({4, 8, 2}) ---
+    mlp_params = np.random.default_rng(13).standard_normal(58).astype(f32)
+    assert r.odl_ref_save_mlp(mlp_params, os.path.join(HERE, "ref_mlp.odl").encode()) == 0
+    out["io_mlp_params"] = mlp_params
+    xio = np.random.default_rng(14).standard_normal((3, 4)).astype(f32)
+    back, yio = np.empty(58, f32), np.empty((3, 2), f32)
+    assert r.odl_ref_load_mlp(os.path.join(HERE, "ref_mlp.odl").encode(), 1, xio, back, yio) == 0
+    assert np.array_equal(back, mlp_params)
+    out["io_mlp_x"], out["io_mlp_y"] = xio, yio
+
     path = os.path.join(HERE, "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

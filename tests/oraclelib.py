@@ -86,6 +86,9 @@ _REF_SIGS = {
     "odl_ref_batch_norm_forward": "pppppif" + "llll" + "pppp>i",
     "odl_ref_batch_norm_backward": "ppppppf" + "llll" + "ppp>i",
     "odl_ref_batch_norm_layer": "pllllifffi" + "ppp" + ">i",
+    "odl_ref_save_mlp": "pp>i",
+    "odl_ref_load_mlp": "pippp>i",
+    "odl_ref_checkpoint_roundtrip": "ppiifffffppp>i",
     "odl_ref_mlp_train": "ppillll" + "pppp" + "ifffff" + "pppppp>i",
     "odl_ref_cnn_train": "ppillllll" + "p" * 8 + "f" + "p" + "p" * 8 + "p>i",
     "odl_ref_mlp_bench": "lllliipp>i",
