@@ -155,6 +155,26 @@ def extras(torch, capi, steps, warmup):
                                        stream), steps, warmup)
         nb = 8.0 * N * C + 8.0 * N
         out[name] = {"ms": ms, "gbs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
+    # batch normalisation at the shape of the first BatchNorm2d of the reference's conv_mnist example, batch 256.
+    # Algorithmic bytes: forward reads x and writes y and x_norm; backward reads gy and x_norm and writes gx (the
+    # statistics passes re-read what the first pass brought in; 51 MB fits the 256 MB last-level cache).
+    N, C, P = 256, 64, 28 * 28
+    x, gam, bet = rnd(N, C, P), rnd(C), rnd(C)
+    rmean, rvar = torch.zeros(C, device="cuda"), torch.ones(C, device="cuda")
+    y, xn, gx, gyb = empty(N, C, P), empty(N, C, P), empty(N, C, P), rnd(N, C, P)
+    mean, var, dg, dbt = empty(C), empty(C), empty(C), empty(C)
+    wbn, nbn = ws(L.query("odl_hip_batch_norm_workspace_bytes", N, C, P))
+    f = direct("odl_hip_batch_norm_forward", ptr(x), ptr(gam), ptr(bet), ptr(rmean), ptr(rvar), 1, ctypes.c_float(1e-5),
+               N, C, P, ptr(y), ptr(mean), ptr(var), ptr(xn), wbn, nbn, stream)
+    b = direct("odl_hip_batch_norm_backward", ptr(gyb), ptr(gam), ptr(var), ptr(xn), ctypes.c_float(1e-5), N, C, P,
+               ptr(gx), ptr(dg), ptr(dbt), wbn, nbn, stream)
+    ms_f, ms_b = time_region(torch, f, steps, warmup), time_region(torch, b, steps, warmup)
+    nb = 12.0 * N * C * P
+    out["batch_norm_256x64x28x28"] = {"fwd_ms": ms_f, "bwd_ms": ms_b, "fwd_gbs": nb / ms_f / 1e6,
+                                      "bwd_gbs": nb / ms_b / 1e6, "fwd_frac_hbm": nb / ms_f / 1e6 / PEAK_HBM_GBS,
+                                      "bwd_frac_hbm": nb / ms_b / 1e6 / PEAK_HBM_GBS}
+    del x, y, xn, gx, gyb
+    keep.clear()
     # config 2's other shapes: forward + both gradient GEMMs, 6*M*N*K FLOP per step
     for (M, K, N) in ((1024, 1024, 1024), (2048, 2048, 2048), (8192, 8192, 8192), (512, 784, 1000), (512, 1000, 10)):
         a, b, dc = rnd(M, K), rnd(K, N), rnd(M, N)
@@ -248,10 +268,10 @@ def yolo_forward(h, ref, reps):
     return res
 
 
-# HBM-side bytes of one 4096^3 sgemm_mfma_kernel launch: FETCH_SIZE (scaled 2.000x by the calibration copy) 805.2 MiB on
-# average over the NN / NT / TN variants (734 / 983 / 699) + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc`
+# HBM-side bytes of one 4096^3 sgemm_mfma_kernel launch: FETCH_SIZE (scaled 2.000x by the calibration copy) 808.6 MiB on
+# average over the NN / NT / TN variants (742 / 978 / 706) + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc`
 # runs of `--pmc-probe` summarised under profiles/.
-GEMM_4096_TRAFFIC_BYTES = int((805.2 + 64.0) * 1024 * 1024)
+GEMM_4096_TRAFFIC_BYTES = int((808.6 + 64.0) * 1024 * 1024)
 
 
 def pmc_probe(torch, capi, gemm_step):

@@ -111,20 +111,32 @@ __global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__rest
     const int np = (HW - p0 < 64) ? HW - p0 : 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float *src = conv + ((int64_t)(b * g.A + a) * g.CI) * HW + p0;
-    for (int c = wave; c < g.CI; c += kBlock / 64)
-        if (lane < np)
-        {
-            const float v = src[(int64_t)c * HW + lane];
-            sh_det[lane * LS + c] = 1.0f / (1.0f + expf(-v));  // the reference's -x, exp, 1 + ., 1 / . steps
-        }
-    __syncthreads();
-    float *dst = out + ((int64_t)(b * g.A + a) * HW + p0) * g.CI;
-    for (int e = threadIdx.x; e < np * g.CI; e += kBlock)
+    // four channels per wave in flight: the loads of a group are issued together, then the four sigmoids
+    for (int c0 = wave; c0 < g.CI; c0 += 4 * (kBlock / 64))
     {
-        const int pl = e / g.CI, c = e - pl * g.CI;
-        float v = sh_det[pl * LS + c];
-        if (c < 4)
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
         {
+            const int c = c0 + j * (kBlock / 64);
+            v[j] = (c < g.CI && lane < np) ? src[(int64_t)c * HW + lane] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const int c = c0 + j * (kBlock / 64);
+            if (c < g.CI && lane < np)
+                sh_det[lane * LS + c] = 1.0f / (1.0f + expf(-v[j]));  // the reference's -x, exp, 1 + ., 1 / . steps
+        }
+    }
+    __syncthreads();
+    // the four box channels of each pixel: one thread each (64 pixels x 4 = the whole workgroup), so the grid and
+    // anchor loads are issued once, outside the streaming loop below
+    {
+        const int pl = threadIdx.x >> 2, c = threadIdx.x & 3;
+        if (pl < np && c < g.CI)
+        {
+            float v = sh_det[pl * LS + c];
             const int p = p0 + pl;
             const int h = p / g.W, w = p - h * g.W;
             if (c < 2)
@@ -146,9 +158,15 @@ __global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__rest
                 const float t = v * 2.0f;
                 v = (t * t) * av;  // pow(2s, 2) * anchor
             }
+            sh_det[pl * LS + c] = v;
         }
-        dst[e] = v;
     }
+    __syncthreads();
+    // [pixel][channel] rows out of LDS, consecutive lanes along the output
+    float *dst = out + ((int64_t)(b * g.A + a) * HW + p0) * g.CI;
+    for (int pl = wave; pl < np; pl += kBlock / 64)
+        for (int c = lane; c < g.CI; c += 64)
+            dst[pl * g.CI + c] = sh_det[pl * LS + c];
 }
 }  // namespace
 
