@@ -237,6 +237,16 @@ Conv2d::Conv2d(int in_channels, int out_channels, std::pair<int, int> kernel_siz
     : in_channels_(in_channels), out_channels_(out_channels), kernel_(kernel_size), stride_(stride), pad_(pad),
       use_bias_(bias)
 {
+    if (in_channels <= 0)
+        THROW_INVALID_ARG("Conv2d: in_channels must be positive, but got {}", in_channels);
+    if (out_channels <= 0)
+        THROW_INVALID_ARG("Conv2d: out_channels must be positive, but got {}", out_channels);
+    if (kernel_size.first <= 0 || kernel_size.second <= 0)
+        THROW_INVALID_ARG("Conv2d: kernel_size must be positive, but got ({}, {})", kernel_size.first, kernel_size.second);
+    if (stride.first <= 0 || stride.second <= 0)
+        THROW_INVALID_ARG("Conv2d: stride must be positive, but got ({}, {})", stride.first, stride.second);
+    if (pad.first < 0 || pad.second < 0)
+        THROW_INVALID_ARG("Conv2d: pad must be non-negative, but got ({}, {})", pad.first, pad.second);
     const float fan_in = (float)(in_channels * kernel_.first * kernel_.second);
     weight_ = scaled_randn(Shape{(size_t)out_channels, (size_t)in_channels, (size_t)kernel_.first, (size_t)kernel_.second},
                            std::sqrt(2.0f / fan_in));
