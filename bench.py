@@ -229,6 +229,14 @@ def train_steps(steps, warmup, with_cpu):
                                        "gemm_flop_per_step": 6.0 * 512 * (784 * 1000 + 1000 * 10)}
     rc = h.odl_host_cnn_bench(256, steps, warmup, ms, loss)
     out["cnn_b256_sgd"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss": float(loss[0])}
+    # the same steps recorded once into a HIP graph and replayed (one submission per step instead of ~50 launches);
+    # the loss is still read back after every step
+    rc = h.odl_host_mlp_bench_graph(512, 784, 1000, 10, steps, warmup, 1, ms, loss)
+    out["mlp_512x784x1000x10_adam"].update({"graph_replay_rc": rc, "graph_replay_ms_per_step": float(ms[0]),
+                                            "graph_replay_loss": float(loss[0])})
+    rc = h.odl_host_cnn_bench_graph(256, steps, warmup, 1, ms, loss)
+    out["cnn_b256_sgd"].update({"graph_replay_rc": rc, "graph_replay_ms_per_step": float(ms[0]),
+                                "graph_replay_loss": float(loss[0])})
     out["yolov5n_forward_4x3x320x320"] = yolo_forward(h, ol.ref() if with_cpu and ol.have_ref() else None, steps)
     if with_cpu and ol.have_ref():
         r = ol.ref()

@@ -54,6 +54,21 @@ int odl_hip_memcpy_d2h(void *host_dst, const void *src, size_t bytes);
 int odl_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
 int odl_hip_memset(void *dst, int value, size_t bytes, void *stream);
 
+/* Streams and captured graphs. No counterpart in the reference, which launches everything on the null stream
+ * (SURVEY of src/mat/origin/cuda: no streams, events or graphs): they exist so that a caller can record a step of
+ * fixed shapes once and replay it with one submission. A created stream is non-blocking and has the default
+ * priority. Between capture_begin and capture_end every launch on that stream is recorded, not run; entry points
+ * that synchronise or copy to the host (odl_hip_synchronize, odl_hip_memcpy_d2h, odl_hip_softmax_ce_loss,
+ * odl_hip_gather, odl_hip_accuracy) must not be called in between. All entry points clear memory with fill kernels,
+ * never with memset nodes. capture_end returns an executable graph; launch replays it on a stream. */
+int odl_hip_stream_create(void **stream);
+int odl_hip_stream_destroy(void *stream);
+int odl_hip_stream_synchronize(void *stream);
+int odl_hip_graph_capture_begin(void *stream);
+int odl_hip_graph_capture_end(void *stream, void **graph_exec);
+int odl_hip_graph_launch(void *graph_exec, void *stream);
+int odl_hip_graph_destroy(void *graph_exec);
+
 /* ------------------------------------------------------------------ GEMM ---------------------------- */
 /* General row-major SGEMM on FP32 MFMA: C[M,N] = op(A)[M,K] . op(B)[K,N] (+ bias[N] broadcast over rows
  * when bias != NULL). trans_a: A is stored [K,M] (lda >= M) else [M,K] (lda >= K); trans_b: B is stored
@@ -158,6 +173,14 @@ size_t odl_hip_softmax_ce_loss_workspace_bytes(int64_t N);
  * gx = (softmax(x) - one_hot(t)) * (gy / N); gy is the host scalar the reference reads with .item<float>() */
 int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float gy, float *gx,
                             void *stream);
+/* The same two without a host round trip, for callers that record the step into a graph: the loss goes to
+ * device_loss2[0] (float) and the out-of-range-label flag to device_loss2[1] (int, nonzero = a bad label; the caller
+ * decides when to look at it), and the upstream gradient is read from device memory (device_gy[0]). Same kernels,
+ * same arithmetic: gy / N is formed in the kernel as the host forms it. */
+int odl_hip_softmax_ce_loss_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
+                                   float *device_loss2, void *workspace, size_t workspace_bytes, void *stream);
+int odl_hip_softmax_ce_grad_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
+                                   const float *device_gy, float *gx, void *stream);
 
 /* ------------------------------------------------------------------ pooling ------------------------- */
 /* Mat::max_pool2d / max_pool2d_backward (mat.h:560-578; src/mat/origin/cpu/pooling/max_pool2d.cpp:40-224).
@@ -245,6 +268,12 @@ int odl_hip_axpby(float a, const float *x, float b, const float *y, int64_t n, f
  * m and v are updated in place; p_out may be p. sgd_step: p_out = p - g*lr (no momentum, no weight decay). */
 int odl_hip_adam_step(const float *p, const float *g, float *m, float *v, int64_t n, float beta1, float beta2,
                       float m_hat_scale, float v_hat_scale, float eps, float lr, float *p_out, void *stream);
+/* the same step with m_hat_scale and v_hat_scale read from device memory (device_scales[0], [1]): for a step that
+ * is recorded into a graph once and replayed, where the step count changes between replays and the caller rewrites
+ * the two floats before each one */
+int odl_hip_adam_step_device_scales(const float *p, const float *g, float *m, float *v, int64_t n, float beta1,
+                                    float beta2, const float *device_scales, float eps, float lr, float *p_out,
+                                    void *stream);
 int odl_hip_sgd_step(const float *p, const float *g, int64_t n, float lr, float *p_out, void *stream);
 /* origin::cuda::{zeros,ones,full} (cuda/factory.cuh:23-50) */
 int odl_hip_fill(float *dst, int64_t n, float value, void *stream);

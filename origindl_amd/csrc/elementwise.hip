@@ -155,9 +155,14 @@ __device__ inline void adam_one(float p, float g, float &m, float &v, float &p_o
     m = mn, v = vn;
 }
 
+// `scales` (optional): the two bias-correction factors in device memory, for a step recorded once and replayed with
+// a different step count each time
 template <bool VEC>
-__global__ void adam_step_kernel(const float *p, const float *g, float *m, float *v, float *p_out, int64_t n, AdamScalars a)
+__global__ void adam_step_kernel(const float *p, const float *g, float *m, float *v, float *p_out, int64_t n, AdamScalars a,
+                                 const float *__restrict__ scales)
 {
+    if (scales)
+        a.m_hat_scale = scales[0], a.v_hat_scale = scales[1];
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (VEC)
     {
@@ -338,8 +343,9 @@ int odl_hip_pow_scalar(const float *a, int64_t n, float exponent, float *out, vo
     return ODL_OK;
 }
 
-int odl_hip_adam_step(const float *p, const float *g, float *m, float *v, int64_t n, float beta1, float beta2,
-                      float m_hat_scale, float v_hat_scale, float eps, float lr, float *p_out, void *stream)
+static int adam_launch(const float *p, const float *g, float *m, float *v, int64_t n, float beta1, float beta2,
+                       float m_hat_scale, float v_hat_scale, const float *scales, float eps, float lr, float *p_out,
+                       void *stream)
 {
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(n >= 0, "adam_step: negative size");
@@ -351,12 +357,26 @@ int odl_hip_adam_step(const float *p, const float *g, float *m, float *v, int64_
     hipStream_t st = odl::as_stream(stream);
     if (aligned(p) && aligned(g) && aligned(m) && aligned(v) && aligned(p_out))
         hipLaunchKernelGGL((adam_step_kernel<true>), dim3((unsigned)odl::ceil_div(odl::ceil_div(n, 4), kBlock)),
-                           dim3(kBlock), 0, st, p, g, m, v, p_out, n, a);
+                           dim3(kBlock), 0, st, p, g, m, v, p_out, n, a, scales);
     else
         hipLaunchKernelGGL((adam_step_kernel<false>), dim3((unsigned)odl::ceil_div(n, kBlock)), dim3(kBlock), 0, st, p, g,
-                           m, v, p_out, n, a);
+                           m, v, p_out, n, a, scales);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
+}
+
+int odl_hip_adam_step(const float *p, const float *g, float *m, float *v, int64_t n, float beta1, float beta2,
+                      float m_hat_scale, float v_hat_scale, float eps, float lr, float *p_out, void *stream)
+{
+    return adam_launch(p, g, m, v, n, beta1, beta2, m_hat_scale, v_hat_scale, nullptr, eps, lr, p_out, stream);
+}
+
+int odl_hip_adam_step_device_scales(const float *p, const float *g, float *m, float *v, int64_t n, float beta1,
+                                    float beta2, const float *device_scales, float eps, float lr, float *p_out,
+                                    void *stream)
+{
+    ODL_REQUIRE(device_scales != nullptr, "adam_step: null scales");
+    return adam_launch(p, g, m, v, n, beta1, beta2, 0.0f, 0.0f, device_scales, eps, lr, p_out, stream);
 }
 
 int odl_hip_sgd_step(const float *p, const float *g, int64_t n, float lr, float *p_out, void *stream)

@@ -154,8 +154,11 @@ __global__ void ce_finish_kernel(const float *__restrict__ logp, int64_t N, floa
 // between the max, the sum and the write, so the logits are read from memory once; longer rows re-read them.
 template <int REGS>
 __global__ __launch_bounds__(kBlock) void ce_grad_kernel(const float *__restrict__ x, const void *t, int is64, int64_t N,
-                                                          int64_t C, float scale, float *__restrict__ gx)
+                                                          int64_t C, float scale_in, const float *__restrict__ gy_dev,
+    float *__restrict__ gx)
 {
+    // the upstream gradient either as a host scalar already divided by N, or still in device memory
+    const float scale = gy_dev ? gy_dev[0] / (float)N : scale_in;
     const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
     if (row >= N)
         return;
@@ -208,8 +211,11 @@ __global__ __launch_bounds__(kBlock) void ce_grad_kernel(const float *__restrict
 // per access (QUADS float4 per lane, rows of up to 256*QUADS classes).
 template <int QUADS>
 __global__ __launch_bounds__(kBlock) void ce_grad_vec_kernel(const float *__restrict__ x, const void *t, int is64,
-                                                              int64_t N, int64_t C, float scale, float *__restrict__ gx)
+                                                              int64_t N, int64_t C, float scale_in, const float *__restrict__ gy_dev,
+    float *__restrict__ gx)
 {
+    // the upstream gradient either as a host scalar already divided by N, or still in device memory
+    const float scale = gy_dev ? gy_dev[0] / (float)N : scale_in;
     const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
     if (row >= N)
         return;
@@ -375,26 +381,47 @@ size_t odl_hip_softmax_ce_loss_workspace_bytes(int64_t N)
     return align256((size_t)(N > 0 ? N : 0) * sizeof(float)) + 256;
 }
 
-int odl_hip_softmax_ce_loss(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float *host_loss,
-                            void *workspace, size_t workspace_bytes, void *stream)
+// loss and out-of-range flag into two device words: [0] loss (float), [1] flag (int, nonzero = a bad label)
+static int ce_loss_launch(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, unsigned int *out2,
+                          void *workspace, size_t workspace_bytes, hipStream_t st)
 {
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(N > 0 && C > 0, "softmax_cross_entropy: empty input");
-    ODL_REQUIRE(host_loss != nullptr, "softmax_cross_entropy: null output");
     const size_t need = odl_hip_softmax_ce_loss_workspace_bytes(N);
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
                 "softmax_cross_entropy: workspace of %zu bytes required, got %zu", need, workspace_bytes);
-    hipStream_t st = odl::as_stream(stream);
     float *logp = static_cast<float *>(workspace);
-    // tail of the workspace: [0] loss (float), [1] out-of-range flag (int)
-    unsigned int *tail = reinterpret_cast<unsigned int *>(static_cast<char *>(workspace) + need - 256);
-    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, tail, 2);
+    hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, out2, 2);
     ODL_LAUNCH_CHECK();
     hipLaunchKernelGGL(ce_row_logp_kernel, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, st, x, t,
-                       idx_is_i64, N, C, logp, reinterpret_cast<int *>(tail + 1));
+                       idx_is_i64, N, C, logp, reinterpret_cast<int *>(out2 + 1));
     ODL_LAUNCH_CHECK();
-    hipLaunchKernelGGL(ce_finish_kernel, dim3(1), dim3(1024), 0, st, logp, N, reinterpret_cast<float *>(tail));
+    hipLaunchKernelGGL(ce_finish_kernel, dim3(1), dim3(1024), 0, st, logp, N, reinterpret_cast<float *>(out2));
     ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_softmax_ce_loss_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
+                                   float *device_loss2, void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE(device_loss2 != nullptr, "softmax_cross_entropy: null output");
+    return ce_loss_launch(x, t, idx_is_i64, N, C, reinterpret_cast<unsigned int *>(device_loss2), workspace,
+                          workspace_bytes, odl::as_stream(stream));
+}
+
+int odl_hip_softmax_ce_loss(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float *host_loss,
+                            void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE(host_loss != nullptr, "softmax_cross_entropy: null output");
+    hipStream_t st = odl::as_stream(stream);
+    const size_t need = odl_hip_softmax_ce_loss_workspace_bytes(N > 0 ? N : 1);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
+                "softmax_cross_entropy: workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    // tail of the workspace: [0] loss (float), [1] out-of-range flag (int)
+    unsigned int *tail = reinterpret_cast<unsigned int *>(static_cast<char *>(workspace) + need - 256);
+    const int rc = ce_loss_launch(x, t, idx_is_i64, N, C, tail, workspace, workspace_bytes, st);
+    if (rc != ODL_OK)
+        return rc;
     unsigned int host_tail[2] = {0, 0};
     ODL_HIP_CHECK(hipMemcpyAsync(host_tail, tail, sizeof(host_tail), hipMemcpyDeviceToHost, st));
     ODL_HIP_CHECK(hipStreamSynchronize(st));
@@ -406,8 +433,8 @@ int odl_hip_softmax_ce_loss(const float *x, const void *t, int idx_is_i64, int64
     return ODL_OK;
 }
 
-int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float gy, float *gx,
-                            void *stream)
+static int ce_grad_launch(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float gy,
+                          const float *gy_dev, float *gx, void *stream)
 {
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(N > 0 && C > 0, "softmax_cross_entropy backward: empty input");
@@ -418,22 +445,35 @@ int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64
     if (vec && C > 64 && C <= 1024)
     {
         if (C <= 256)
-            hipLaunchKernelGGL(ce_grad_vec_kernel<1>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+            hipLaunchKernelGGL(ce_grad_vec_kernel<1>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gy_dev, gx);
         else if (C <= 512)
-            hipLaunchKernelGGL(ce_grad_vec_kernel<2>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+            hipLaunchKernelGGL(ce_grad_vec_kernel<2>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gy_dev, gx);
         else
-            hipLaunchKernelGGL(ce_grad_vec_kernel<4>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+            hipLaunchKernelGGL(ce_grad_vec_kernel<4>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gy_dev, gx);
     }
     else if (C <= 64)
-        hipLaunchKernelGGL(ce_grad_kernel<1>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+        hipLaunchKernelGGL(ce_grad_kernel<1>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gy_dev, gx);
     else if (C <= 256)
-        hipLaunchKernelGGL(ce_grad_kernel<4>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+        hipLaunchKernelGGL(ce_grad_kernel<4>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gy_dev, gx);
     else if (C <= 1024)
-        hipLaunchKernelGGL(ce_grad_kernel<16>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+        hipLaunchKernelGGL(ce_grad_kernel<16>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gy_dev, gx);
     else
-        hipLaunchKernelGGL(ce_grad_kernel<0>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gx);
+        hipLaunchKernelGGL(ce_grad_kernel<0>, grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, scale, gy_dev, gx);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
+}
+
+int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float gy, float *gx,
+                            void *stream)
+{
+    return ce_grad_launch(x, t, idx_is_i64, N, C, gy, nullptr, gx, stream);
+}
+
+int odl_hip_softmax_ce_grad_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
+                                   const float *device_gy, float *gx, void *stream)
+{
+    ODL_REQUIRE(device_gy != nullptr, "softmax_cross_entropy backward: null upstream gradient");
+    return ce_grad_launch(x, t, idx_is_i64, N, C, 0.0f, device_gy, gx, stream);
 }
 
 int odl_hip_argmax_rows(const float *y, int64_t N, int64_t C, int64_t *out, void *stream)

@@ -168,4 +168,67 @@ int odl_hip_memset(void *dst, int value, size_t bytes, void *stream)
     return odl::fill_bytes_launch(dst, value, bytes, odl::as_stream(stream));
 }
 
+// ---- streams and captured graphs. A step whose shapes and pointers do not change from one iteration to the next
+// (a training step on a fixed batch shape, an inference forward) is dozens of launches of microsecond kernels; recorded
+// once into a graph and replayed, it costs one submission.
+int odl_hip_stream_create(void **stream)
+{
+    ODL_REQUIRE(stream != nullptr, "stream_create: null output");
+    hipStream_t s = nullptr;
+    ODL_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
+    *stream = s;
+    return ODL_OK;
+}
+
+int odl_hip_stream_destroy(void *stream)
+{
+    if (stream)
+        ODL_HIP_CHECK(hipStreamDestroy(odl::as_stream(stream)));
+    return ODL_OK;
+}
+
+int odl_hip_stream_synchronize(void *stream)
+{
+    ODL_HIP_CHECK(hipStreamSynchronize(odl::as_stream(stream)));
+    return ODL_OK;
+}
+
+int odl_hip_graph_capture_begin(void *stream)
+{
+    ODL_REQUIRE(stream != nullptr, "graph capture needs a created stream: the null stream cannot be captured");
+    ODL_HIP_CHECK(hipStreamBeginCapture(odl::as_stream(stream), hipStreamCaptureModeRelaxed));
+    return ODL_OK;
+}
+
+int odl_hip_graph_capture_end(void *stream, void **graph_exec)
+{
+    ODL_REQUIRE(stream != nullptr && graph_exec != nullptr, "graph_capture_end: null argument");
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    ODL_HIP_CHECK(hipStreamEndCapture(odl::as_stream(stream), &graph));
+    if (graph == nullptr)
+        return odl::fail(ODL_ERR_RUNTIME, "graph capture produced no graph (an operation that cannot be captured ended it)");
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess)
+        return odl::fail(ODL_ERR_RUNTIME, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    *graph_exec = exec;
+    return ODL_OK;
+}
+
+int odl_hip_graph_launch(void *graph_exec, void *stream)
+{
+    ODL_REQUIRE(graph_exec != nullptr, "graph_launch: null graph");
+    ODL_HIP_CHECK(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), odl::as_stream(stream)));
+    return ODL_OK;
+}
+
+int odl_hip_graph_destroy(void *graph_exec)
+{
+    if (graph_exec)
+        ODL_HIP_CHECK(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+    return ODL_OK;
+}
+
 }  // extern "C"

@@ -275,6 +275,20 @@ public:
     std::unique_ptr<Mat> max_pool2d_backward_device(const Mat &gy, std::pair<int, int> kernel_size,
                                                     std::pair<int, int> stride, std::pair<int, int> pad,
                                                     const Storage &indices) const;
+    // The loss and its gradient without the host round trip of the pair above: the loss stays a device scalar and the
+    // upstream gradient is read from device memory. For steps recorded into a graph; an out-of-range label is not
+    // reported here (the flag stays on the device).
+    std::unique_ptr<Mat> softmax_cross_entropy_device(const Mat &target) const;
+    std::unique_ptr<Mat> softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const;
+    // overwrites this tensor's elements from host memory (synchronises first: work in flight may still read them)
+    void upload(const void *host, size_t bytes);
+    // the fused Adam step written over this parameter, bias-correction factors read from device memory
+    void adam_step_inplace(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, const float *device_scales, float eps,
+                           float lr);
+    void sgd_step_inplace(const Mat &grad, float lr);
+    // overwrites this tensor's elements with another's of the same shape (a device-to-device copy on the current
+    // stream): how a recorded step stores a freshly computed tensor at the address later replays read it from
+    void copy_from(const Mat &src);
     // a*this + b*other in one launch (each product rounded before the sum): the running-statistics update of the
     // BatchNorm layers
     std::unique_ptr<Mat> axpby(float a, float b, const Mat &other) const;

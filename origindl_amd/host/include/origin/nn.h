@@ -196,6 +196,11 @@ public:
     // (src/optim/adam.cpp:116-284, src/optim/sgd.cpp:77-157)
     virtual std::unordered_map<std::string, std::any> state_dict() const = 0;
     virtual void load_state_dict(const std::unordered_map<std::string, std::any> &state_dict) = 0;
+    // Call before every replay of a graph that recorded step(): brings the host-side state the recorded kernels
+    // depend on (Adam's step counts and bias-correction factors) forward by one step. While a graph is being
+    // captured, step() writes parameters and buffers in place, so that replays find them at the recorded addresses;
+    // at least one ordinary step must have run before (the buffers must exist).
+    virtual void prepare_replay() {}
 
 protected:
     virtual void step_one(Parameter &param) = 0;
@@ -234,6 +239,11 @@ private:
     float lr_, beta1_, beta2_, eps_;
     std::unordered_map<Parameter *, Tensor> m_buffers_, v_buffers_;
     std::unordered_map<Parameter *, int> step_counts_;
+    Tensor replay_scales_;                      // [parameters, 2] on the device: 1/(1-b1^t), 1/(1-b2^t) per parameter
+    std::vector<Parameter *> replay_params_;    // the parameters the recorded step updates
+
+public:
+    void prepare_replay() override;
 };
 
 class WeightDecay  // include/origin/optim/hooks.h:37-66: grad += rate * param, for every parameter
@@ -255,5 +265,35 @@ int current_device();
 void set_device(int device);
 void device_info();
 void synchronize();
+
+// ---- beyond the reference (which queues everything on the null stream): a current stream per host thread, and a
+// step recorded once and replayed. Usage: `void *s = cuda::create_stream(); cuda::set_stream(s);` run the step a few
+// times (memory pool warm, optimizer buffers created), then `cuda::Graph g; g.begin_capture(); step(); g.end_capture();`
+// and per iteration: `x.upload(batch); optimizer.prepare_replay(); g.launch();` — the tensors made by the capture run
+// (the loss, the outputs) keep their addresses and hold the results of the latest replay. A captured step must not
+// move data to or from the host (no item(), no to_vector(), no tensors built from host values): such a call throws.
+// Memory allocated during the capture belongs to the graph until it is destroyed.
+void *create_stream();
+void destroy_stream(void *stream);
+void set_stream(void *stream);  // nullptr = the null stream; synchronises the device when the stream changes
+void *current_stream();
+bool is_capturing();
+
+class Graph
+{
+public:
+    Graph() = default;
+    ~Graph();
+    Graph(const Graph &) = delete;
+    Graph &operator=(const Graph &) = delete;
+    void begin_capture();
+    void end_capture();
+    void launch();  // on the current stream
+    bool captured() const { return exec_ != nullptr; }
+
+private:
+    void *exec_ = nullptr;
+    std::shared_ptr<void> arena_;
+};
 }  // namespace cuda
 }  // namespace origin

@@ -123,6 +123,9 @@ public:
         return static_cast<const OriginMat &>(*impl_->data_).to_vector<T>();
     }
 
+    // overwrites the elements in place from host memory (same byte count); the tensor keeps its address, which is
+    // what a recorded graph reads from
+    void upload(const void *host, size_t bytes);
     Tensor to(DataType target) const;
     Tensor to(Device device) const;
     Tensor to(const TensorOptions &options) const;

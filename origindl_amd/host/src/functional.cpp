@@ -1,6 +1,7 @@
 // Operators over Mat. Gradients restate the reference's backward rules (cited per operator); softmax and
 // softmax-cross-entropy go to the fused device kernels instead of the reference's chain of eight Mat ops.
 #include "origin/functional.h"
+#include "origin/nn.h"
 
 #include <cmath>
 #include <string>
@@ -291,15 +292,20 @@ struct SoftmaxCrossEntropy : Operator  // src/operators/loss/softmax_cross_entro
         if (x.shape()[0] != t.shape()[0])
             THROW_INVALID_ARG("SoftmaxCrossEntropy: batch size mismatch. x has {} samples, target has {} samples",
                               x.shape()[0], t.shape()[0]);
+        if (cuda::is_capturing())  // a recorded step cannot visit the host: the loss stays where it is computed
+            return {wrap(omat(x).softmax_cross_entropy_device(mat(t)))};
         const float loss = omat(x).softmax_cross_entropy(mat(t));  // synchronises, as the reference's .item() does
         return {Tensor({loss}, Shape{}, dtype(DataType::kFloat32).device(x.device()))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
         const Tensor &x = inputs_[0], &t = inputs_[1];
-        const float gy  = gys[0].item<float>();
-        auto gx         = omat(x).softmax_cross_entropy_backward(mat(t), gy);
-        auto gt         = Tensor::zeros(t.shape(), dtype(DataType::kFloat32).device(t.device()));
+        std::unique_ptr<Mat> gx;
+        if (cuda::is_capturing())
+            gx = omat(x).softmax_cross_entropy_backward_device(mat(t), mat(gys[0]));
+        else
+            gx = omat(x).softmax_cross_entropy_backward(mat(t), gys[0].item<float>());
+        auto gt = Tensor::zeros(t.shape(), dtype(DataType::kFloat32).device(t.device()));
         return {wrap(std::move(gx)), gt};
     }
 };

@@ -6,10 +6,13 @@
 #include <cmath>
 #include <cstring>
 #include <map>
+#include <memory>
+#include <unordered_map>
 #include <mutex>
 #include <random>
 
 #include "odl_hip.h"
+#include "origin/nn.h"
 
 namespace origin
 {
@@ -24,9 +27,31 @@ void check(int rc)
     throw std::runtime_error(odl_hip_last_error());
 }
 
+// ---- the stream every launch of this layer goes to, and graph capture (per host thread)
+thread_local void *t_stream = nullptr;     // nullptr = the null stream, as in the reference
+thread_local bool t_capturing = false;
+
+void *cur()
+{
+    return t_stream;
+}
+
+// host <-> device copies are synchronous; they cannot be part of a recorded step
+void no_capture(const char *what)
+{
+    if (t_capturing)
+        THROW_RUNTIME_ERROR("{} while a graph is being captured: a captured step may not move data to or from the host",
+                            what);
+}
+
 // Caching allocator for device memory: freed blocks are kept in size bins (powers of two from 256 B up to 1 MiB,
-// whole MiB above) and handed out again. Everything runs on the null stream, so a block freed by the host is
-// reused only by work queued after every kernel that touched it.
+// whole MiB above) and handed out again. All work of a thread is queued on one stream at a time (switching streams
+// synchronises the device), so a block freed by the host is reused only by work queued after every kernel that
+// touched it.
+// While a graph is being captured, blocks come from — and return to — an arena owned by that graph: the recorded
+// kernels keep their addresses for as long as the graph lives, so those blocks must never be handed to anyone
+// else, not even after the tensors of the capture run have died. Inside the capture they are reused freely (the
+// graph replays its nodes in recording order).
 class DevicePool
 {
 public:
@@ -48,31 +73,93 @@ public:
         }
         return (bytes + (1u << 20) - 1) & ~(size_t)((1u << 20) - 1);
     }
+    struct Arena
+    {
+        std::map<size_t, std::vector<void *>> free_;
+        ~Arena() { DevicePool::get().absorb(*this); }
+    };
     void *alloc(size_t cap)
     {
+        std::shared_ptr<Arena> arena;
         {
             std::lock_guard<std::mutex> lk(mu_);
-            auto it = free_.find(cap);
-            if (it != free_.end() && !it->second.empty())
+            arena = capture_arena_;
+            void *p = nullptr;
+            if (arena)
+                p = take(arena->free_, cap);
+            if (!p)
+                p = take(free_, cap);
+            if (p)
             {
-                void *p = it->second.back();
-                it->second.pop_back();
+                if (arena)
+                    owner_[p] = arena;
                 return p;
             }
         }
         void *p = nullptr;
         check(odl_hip_malloc(&p, cap));
+        if (arena)
+        {
+            std::lock_guard<std::mutex> lk(mu_);
+            owner_[p] = arena;
+        }
         return p;
     }
     void release(void *p, size_t cap)
     {
         std::lock_guard<std::mutex> lk(mu_);
+        auto it = owner_.find(p);
+        if (it != owner_.end())
+        {
+            if (auto arena = it->second.lock())
+            {
+                arena->free_[cap].push_back(p);
+                return;
+            }
+            owner_.erase(it);  // its graph is gone: an ordinary block again
+        }
         free_[cap].push_back(p);
+    }
+    std::shared_ptr<Arena> begin_capture()
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        if (capture_arena_)
+            THROW_RUNTIME_ERROR("a graph is already being captured");
+        capture_arena_ = std::make_shared<Arena>();
+        return capture_arena_;
+    }
+    void end_capture()
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        capture_arena_.reset();
     }
 
 private:
+    static void *take(std::map<size_t, std::vector<void *>> &bins, size_t cap)
+    {
+        auto it = bins.find(cap);
+        if (it == bins.end() || it->second.empty())
+            return nullptr;
+        void *p = it->second.back();
+        it->second.pop_back();
+        return p;
+    }
+    // a dying graph's free blocks become ordinary blocks; the ones still held by tensors follow when released
+    void absorb(Arena &a)
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        for (auto &bin : a.free_)
+            for (void *p : bin.second)
+            {
+                owner_.erase(p);
+                free_[bin.first].push_back(p);
+            }
+        a.free_.clear();
+    }
     std::mutex mu_;
     std::map<size_t, std::vector<void *>> free_;
+    std::shared_ptr<Arena> capture_arena_;
+    std::unordered_map<void *, std::weak_ptr<Arena>> owner_;
 };
 
 const OriginMat &as_origin(const Mat &m)
@@ -163,7 +250,7 @@ std::unique_ptr<Mat> binary(int op, const char *who, const OriginMat &a, const M
         THROW_INVALID_ARG("Output tensor mismatch. Expected shape={}, got shape={}", rs.to_string(),
                           dst->shape().to_string());
     check(odl_hip_binary(op, fp(x), (int64_t)x.elements(), fp(y), (int64_t)y.elements(), dst->data_ptr<float>(),
-                         nullptr));
+                         cur()));
     return fresh;
 }
 
@@ -177,7 +264,7 @@ std::unique_ptr<Mat> unary(int op, const char *who, const OriginMat &a, OriginMa
         fresh = new_like(x, x.shape());
         dst   = fresh.get();
     }
-    check(odl_hip_unary(op, fp(x), (int64_t)x.elements(), dst->data_ptr<float>(), nullptr));
+    check(odl_hip_unary(op, fp(x), (int64_t)x.elements(), dst->data_ptr<float>(), cur()));
     return fresh;
 }
 
@@ -236,12 +323,18 @@ std::shared_ptr<Storage> Storage::to_device(DeviceType type, int index) const
     if (type_ == DeviceType::kCPU && type == DeviceType::kCPU)
         std::memcpy(dst->data(), data_, size_);
     else if (type_ == DeviceType::kCPU)
+    {
+        no_capture("host-to-device copy");
         check(odl_hip_memcpy_h2d(dst->data(), data_, size_));
+    }
     else if (type == DeviceType::kCPU)
+    {
+        no_capture("device-to-host copy");
         check(odl_hip_memcpy_d2h(dst->data(), data_, size_));
+    }
     else
     {
-        check(odl_hip_memcpy_d2d(dst->data(), data_, size_, nullptr));
+        check(odl_hip_memcpy_d2d(dst->data(), data_, size_, cur()));
     }
     return dst;
 }
@@ -288,7 +381,7 @@ double load_as(const void *src, DataType dt, size_t i)
     }
 }
 
-std::unique_ptr<Mat> upload(const void *host, DataType dt, const Shape &shape, Device dev)
+std::unique_ptr<Mat> upload_new(const void *host, DataType dt, const Shape &shape, Device dev)
 {
     auto m = std::make_unique<OriginMat>(shape, dt, dev);
     const size_t bytes = shape.elements() * dtype_size(dt);
@@ -297,7 +390,10 @@ std::unique_ptr<Mat> upload(const void *host, DataType dt, const Shape &shape, D
     if (dev.type() == DeviceType::kCPU)
         std::memcpy(m->data_ptr(), host, bytes);
     else
+    {
+        no_capture("host-to-device copy");
         check(odl_hip_memcpy_h2d(m->data_ptr(), host, bytes));
+    }
     return m;
 }
 }  // namespace
@@ -307,13 +403,13 @@ std::unique_ptr<Mat> OriginMat::from_memory(const void *data, DataType user_dtyp
 {
     const size_t n = shape.elements();
     if (user_dtype == options.dtype())
-        return upload(data, user_dtype, shape, options.device());
+        return upload_new(data, user_dtype, shape, options.device());
     std::vector<double> tmp(n);
     for (size_t i = 0; i < n; ++i)
         tmp[i] = load_as(data, user_dtype, i);
     std::vector<char> conv(n * dtype_size(options.dtype()));
     store_as(conv.data(), options.dtype(), tmp.data(), n);
-    return upload(conv.data(), options.dtype(), shape, options.device());
+    return upload_new(conv.data(), options.dtype(), shape, options.device());
 }
 
 std::unique_ptr<Mat> OriginMat::from_scalar(const Scalar &scalar, const Shape &shape, const TensorOptions &options)
@@ -322,13 +418,13 @@ std::unique_ptr<Mat> OriginMat::from_scalar(const Scalar &scalar, const Shape &s
     if (options.device().type() == DeviceType::kCUDA && options.dtype() == DataType::kFloat32)
     {
         auto m = std::make_unique<OriginMat>(shape, DataType::kFloat32, options.device());
-        check(odl_hip_fill(m->data_ptr<float>(), (int64_t)n, scalar.to_float32(), nullptr));
+        check(odl_hip_fill(m->data_ptr<float>(), (int64_t)n, scalar.to_float32(), cur()));
         return m;
     }
     std::vector<double> tmp(n, scalar.to_float64());
     std::vector<char> conv(n * dtype_size(options.dtype()));
     store_as(conv.data(), options.dtype(), tmp.data(), n);
-    return upload(conv.data(), options.dtype(), shape, options.device());
+    return upload_new(conv.data(), options.dtype(), shape, options.device());
 }
 
 std::unique_ptr<Mat> OriginMat::randn(const Shape &shape, const TensorOptions &options)
@@ -395,7 +491,7 @@ std::unique_ptr<Mat> OriginMat::transpose() const
     std::swap(d[d.size() - 2], d[d.size() - 1]);
     auto out = new_like(x, Shape(d));
     const int64_t outer = (int64_t)(shape_.elements() / ((rows * cols) != 0 ? rows * cols : 1));
-    check(odl_hip_transpose(fp(x), out->data_ptr<float>(), outer, (int64_t)rows, (int64_t)cols, nullptr));
+    check(odl_hip_transpose(fp(x), out->data_ptr<float>(), outer, (int64_t)rows, (int64_t)cols, cur()));
     return out;
 }
 
@@ -410,6 +506,7 @@ std::vector<double> OriginMat::to_doubles() const
     if (storage_->device_type() != DeviceType::kCPU)
     {
         host.resize(n * dtype_size(dtype_));
+        no_capture("device-to-host copy");
         check(odl_hip_memcpy_d2h(host.data(), storage_->data(), host.size()));
         src = host.data();
     }
@@ -440,7 +537,7 @@ std::unique_ptr<Mat> OriginMat::to(DataType target) const
     const std::vector<double> d = to_doubles();
     std::vector<char> conv(d.size() * dtype_size(target));
     store_as(conv.data(), target, d.data(), d.size());
-    return upload(conv.data(), target, shape_, device());
+    return upload_new(conv.data(), target, shape_, device());
 }
 
 std::unique_ptr<Mat> OriginMat::to_device(Device dev) const
@@ -520,7 +617,7 @@ std::unique_ptr<Mat> OriginMat::upsample_backward(const Mat &gym, const Shape &x
     auto gx = new_like(gy, xs);
     check(odl_hip_upsample_nearest_backward(fp(gy), (int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3],
                                             (int64_t)gy.shape()[2], (int64_t)gy.shape()[3], scale_h, scale_w,
-                                            gx->data_ptr<float>(), nullptr));
+                                            gx->data_ptr<float>(), cur()));
     return gx;
 }
 
@@ -566,7 +663,7 @@ Mat::BatchNormResult OriginMat::batch_norm_forward(const Mat &gamma, const Mat &
     Workspace ws(training ? odl_hip_batch_norm_workspace_bytes(s.N, s.C, s.P) : 0, device().index());
     check(odl_hip_batch_norm_forward(fp(x), fp(g), fp(b), fp(rm), fp(rv), training ? 1 : 0, eps, s.N, s.C, s.P,
                                      y->data_ptr<float>(), mean->data_ptr<float>(), var->data_ptr<float>(),
-                                     xn->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+                                     xn->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
     r.y = std::move(y), r.mean = std::move(mean), r.var = std::move(var), r.x_norm = std::move(xn);
     return r;
 }
@@ -583,7 +680,7 @@ std::unique_ptr<Mat> OriginMat::batch_norm(const Mat &gamma, const Mat &beta, co
     Workspace ws(training ? odl_hip_batch_norm_workspace_bytes(s.N, s.C, s.P) : 0, device().index());
     check(odl_hip_batch_norm_forward(fp(x), fp(g), fp(b), fp(rm), fp(rv), training ? 1 : 0, eps, s.N, s.C, s.P,
                                      y->data_ptr<float>(), mean->data_ptr<float>(), var->data_ptr<float>(), nullptr,
-                                     ws.ptr(), ws.bytes, nullptr));
+                                     ws.ptr(), ws.bytes, cur()));
     return y;
 }
 
@@ -613,7 +710,7 @@ std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward(const Mat &gym,
     auto dgamma = new_like(x, Shape({C})), dbeta = new_like(x, Shape({C}));
     Workspace ws(odl_hip_batch_norm_workspace_bytes(N, (int64_t)C, P), device().index());
     check(odl_hip_batch_norm_backward(fp(gy), fp(g), fp(sv), fp(xn), eps, N, (int64_t)C, P, gx->data_ptr<float>(),
-                                      dgamma->data_ptr<float>(), dbeta->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+                                      dgamma->data_ptr<float>(), dbeta->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
     std::vector<std::unique_ptr<Mat>> outs;
     outs.push_back(std::move(gx)), outs.push_back(std::move(dgamma)), outs.push_back(std::move(dbeta));
     return outs;
@@ -625,7 +722,7 @@ std::unique_ptr<Mat> OriginMat::axpby(float a, float b, const Mat &other) const
     if (x.shape() != y.shape())
         THROW_INVALID_ARG("axpby: shape mismatch {} vs {}", x.shape().to_string(), y.shape().to_string());
     auto o = new_like(x, shape_);
-    check(odl_hip_axpby(a, fp(x), b, fp(y), (int64_t)elements(), o->data_ptr<float>(), nullptr));
+    check(odl_hip_axpby(a, fp(x), b, fp(y), (int64_t)elements(), o->data_ptr<float>(), cur()));
     return o;
 }
 
@@ -648,7 +745,7 @@ std::vector<std::unique_ptr<Mat>> OriginMat::split(const std::vector<size_t> &si
         std::vector<size_t> d = shape_.dims();
         d[dim] = sz;
         auto piece = new_like(x, Shape(d));
-        check(odl_hip_slice_axis(fp(x), outer, ax, inner, off, (int64_t)sz, piece->data_ptr<float>(), nullptr));
+        check(odl_hip_slice_axis(fp(x), outer, ax, inner, off, (int64_t)sz, piece->data_ptr<float>(), cur()));
         off += (int64_t)sz;
         parts.push_back(std::move(piece));
     }
@@ -666,7 +763,7 @@ std::unique_ptr<Mat> OriginMat::upsample(const Shape &output_shape, int scale_h,
     auto y = new_like(x, output_shape);
     check(odl_hip_upsample_nearest(fp(x), (int64_t)shape_[0], (int64_t)shape_[1], (int64_t)shape_[2], (int64_t)shape_[3],
                                    (int64_t)output_shape[2], (int64_t)output_shape[3], scale_h, scale_w,
-                                   y->data_ptr<float>(), nullptr));
+                                   y->data_ptr<float>(), cur()));
     return y;
 }
 
@@ -706,7 +803,7 @@ std::unique_ptr<Mat> OriginMat::cat(const std::vector<const Mat *> &others, int 
     int64_t outer, ax, inner;
     split_axis(os, dim, outer, ax, inner);
     auto y = new_like(*in[0], os);
-    check(odl_hip_cat(ptrs.data(), sizes.data(), (int)ptrs.size(), outer, inner, y->data_ptr<float>(), nullptr));
+    check(odl_hip_cat(ptrs.data(), sizes.data(), (int)ptrs.size(), outer, inner, y->data_ptr<float>(), cur()));
     return y;
 }
 
@@ -733,7 +830,7 @@ std::unique_ptr<Mat> OriginMat::yolo_detect_forward(const Mat &conv_weight, cons
     Workspace ws(odl_hip_yolo_detect_workspace_bytes(N, C, H, W, num_anchors, num_classes), device().index());
     check(odl_hip_yolo_detect_forward(fp(x), fp(w), b ? fp(*b) : nullptr, fp(g), (int64_t)g.elements(), fp(ag),
                                       (int64_t)ag.elements(), aH, aW, N, C, H, W, stride, num_anchors, num_classes,
-                                      y->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+                                      y->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
     return y;
 }
 
@@ -741,7 +838,7 @@ std::unique_ptr<Mat> OriginMat::pow(const Scalar &exponent) const
 {
     const OriginMat &x = dev_f32(*this, "pow");
     auto out = new_like(x, shape_);
-    check(odl_hip_pow_scalar(fp(x), (int64_t)elements(), exponent.to_float32(), out->data_ptr<float>(), nullptr));
+    check(odl_hip_pow_scalar(fp(x), (int64_t)elements(), exponent.to_float32(), out->data_ptr<float>(), cur()));
     return out;
 }
 
@@ -781,7 +878,7 @@ std::unique_ptr<Mat> OriginMat::matmul(const Mat &other) const
                           as.to_string(), bs.to_string());
     auto c = new_like(a, rs);
     Workspace ws(odl_hip_matmul_workspace_bytes(batch, M, N, K, b_batched), device().index());
-    check(odl_hip_matmul(fp(a), fp(b), c->data_ptr<float>(), batch, M, N, K, b_batched, ws.ptr(), ws.bytes, nullptr));
+    check(odl_hip_matmul(fp(a), fp(b), c->data_ptr<float>(), batch, M, N, K, b_batched, ws.ptr(), ws.bytes, cur()));
     return c;
 }
 
@@ -792,7 +889,7 @@ std::unique_ptr<Mat> OriginMat::broadcast_to(const Shape &shape) const
     auto out = new_like(x, shape);
     const auto sd = dims64(shape_), dd = dims64(shape);
     check(odl_hip_broadcast_to(fp(x), sd.data(), (int)shape_.size(), dd.data(), (int)shape.size(),
-                               out->data_ptr<float>(), nullptr));
+                               out->data_ptr<float>(), cur()));
     return out;
 }
 
@@ -806,7 +903,7 @@ std::unique_ptr<Mat> OriginMat::sum_to(const Shape &shape) const
                  device().index());
     auto out = new_like(x, shape);
     check(odl_hip_sum_to(fp(x), sd.data(), (int)shape_.size(), td.data(), (int)shape.size(), out->data_ptr<float>(),
-                         ws.ptr(), ws.bytes, nullptr));
+                         ws.ptr(), ws.bytes, cur()));
     return out;
 }
 
@@ -818,7 +915,7 @@ std::unique_ptr<Mat> OriginMat::sum(int axis, bool keepdim) const
         const Shape rs = keepdim ? Shape(std::vector<size_t>(shape_.size(), 1)) : Shape{1};
         auto out = new_like(x, rs);
         Workspace ws(odl_hip_sum_all_workspace_bytes((int64_t)elements()), device().index());
-        check(odl_hip_sum_all(fp(x), (int64_t)elements(), out->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+        check(odl_hip_sum_all(fp(x), (int64_t)elements(), out->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
         return out;
     }
     if (axis < 0 || axis >= (int)shape_.size())
@@ -835,7 +932,7 @@ std::unique_ptr<Mat> OriginMat::sum(int axis, bool keepdim) const
     split_axis(shape_, axis, outer, ax, inner);
     auto out = new_like(x, Shape(rd));
     Workspace ws(odl_hip_sum_axis_workspace_bytes(outer, ax, inner), device().index());
-    check(odl_hip_sum_axis(fp(x), outer, ax, inner, out->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+    check(odl_hip_sum_axis(fp(x), outer, ax, inner, out->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
     return out;
 }
 
@@ -845,7 +942,7 @@ std::unique_ptr<Mat> OriginMat::max(int axis) const
     if (axis == -1)
     {
         auto out = new_like(x, Shape{1});
-        check(odl_hip_max_all(fp(x), (int64_t)elements(), out->data_ptr<float>(), nullptr));
+        check(odl_hip_max_all(fp(x), (int64_t)elements(), out->data_ptr<float>(), cur()));
         return out;
     }
     if (axis < 0 || axis >= (int)shape_.size())
@@ -857,7 +954,7 @@ std::unique_ptr<Mat> OriginMat::max(int axis) const
     int64_t outer, ax, inner;
     split_axis(shape_, axis, outer, ax, inner);
     auto out = new_like(x, Shape(rd));
-    check(odl_hip_max_axis(fp(x), outer, ax, inner, out->data_ptr<float>(), nullptr));
+    check(odl_hip_max_axis(fp(x), outer, ax, inner, out->data_ptr<float>(), cur()));
     return out;
 }
 
@@ -877,7 +974,7 @@ std::unique_ptr<Mat> OriginMat::im2col(std::pair<int, int> k, std::pair<int, int
                                : Shape{(size_t)N, (size_t)C, (size_t)k.first, (size_t)k.second, (size_t)OH, (size_t)OW};
     auto col = new_like(x, cs);
     check(odl_hip_im2col(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
-                         col->data_ptr<float>(), nullptr));
+                         col->data_ptr<float>(), cur()));
     return col;
 }
 
@@ -896,7 +993,7 @@ std::unique_ptr<Mat> OriginMat::col2im(const Shape &is, std::pair<int, int> k, s
         THROW_INVALID_ARG("col2im: invalid col shape {} for input_shape {}", shape_.to_string(), is.to_string());
     auto img = new_like(col, is);
     check(odl_hip_col2im(fp(col), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
-                         img->data_ptr<float>(), nullptr));
+                         img->data_ptr<float>(), cur()));
     return img;
 }
 
@@ -935,7 +1032,7 @@ std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pa
     Workspace ws(odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
                  device().index());
     check(odl_hip_conv2d_act(fp(x), fp(w), bias, N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
-                             activation, y->data_ptr<float>(), ws.ptr(), ws.bytes, nullptr));
+                             activation, y->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
     return y;
 }
 
@@ -963,7 +1060,7 @@ std::vector<std::unique_ptr<Mat>> OriginMat::conv2d_backward(const Mat &gym, con
                  device().index());
     check(odl_hip_conv2d_backward(fp(gy), fp(x), fp(w), N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
                                   gx->data_ptr<float>(), gw->data_ptr<float>(), gb ? gb->data_ptr<float>() : nullptr,
-                                  ws.ptr(), ws.bytes, nullptr));
+                                  ws.ptr(), ws.bytes, cur()));
     std::vector<std::unique_ptr<Mat>> grads;  // {gx, gW, [gb]}
     grads.push_back(std::move(gx));
     grads.push_back(std::move(gw));
@@ -988,7 +1085,7 @@ std::unique_ptr<Mat> OriginMat::max_pool2d_device(std::pair<int, int> k, std::pa
     if (indices)
         idx = Storage::create(y->elements() * sizeof(uint64_t), DeviceType::kCUDA, device().index());
     check(odl_hip_max_pool2d(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second,
-                             y->data_ptr<float>(), idx ? static_cast<uint64_t *>(idx->data()) : nullptr, nullptr));
+                             y->data_ptr<float>(), idx ? static_cast<uint64_t *>(idx->data()) : nullptr, cur()));
     if (indices)
         *indices = idx;
     return y;
@@ -1004,6 +1101,7 @@ std::unique_ptr<Mat> OriginMat::max_pool2d(std::pair<int, int> k, std::pair<int,
         // the interface hands the window-local indices to the caller as a host vector (mat.h:560-566)
         static_assert(sizeof(size_t) == sizeof(uint64_t), "size_t must be 64-bit");
         indices->resize(y->elements());
+        no_capture("device-to-host copy");
         check(odl_hip_memcpy_d2h(indices->data(), idx->data(), y->elements() * sizeof(uint64_t)));
     }
     return y;
@@ -1021,7 +1119,7 @@ std::unique_ptr<Mat> OriginMat::max_pool2d_backward_device(const Mat &gym, std::
     const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
     auto gx = new_like(gy, shape_);
     check(odl_hip_max_pool2d_backward(fp(gy), static_cast<const uint64_t *>(indices.data()), N, C, H, W, k.first, k.second,
-                                      s.first, s.second, p.first, p.second, gx->data_ptr<float>(), nullptr));
+                                      s.first, s.second, p.first, p.second, gx->data_ptr<float>(), cur()));
     return gx;
 }
 
@@ -1033,6 +1131,7 @@ std::unique_ptr<Mat> OriginMat::max_pool2d_backward(const Mat &gym, std::pair<in
         THROW_INVALID_ARG("max_pool2d_backward: indices size mismatch. Expected {}, got {}", gy.elements(),
                           indices.size());
     auto idx = Storage::create(indices.size() * sizeof(uint64_t), DeviceType::kCUDA, gy.device().index());
+    no_capture("host-to-device copy");
     check(odl_hip_memcpy_h2d(idx->data(), indices.data(), indices.size() * sizeof(uint64_t)));
     return max_pool2d_backward_device(gym, k, s, p, *idx);
 }
@@ -1054,7 +1153,7 @@ std::unique_ptr<Mat> OriginMat::gather(const Mat &indices) const
     const int is64 = label_kind(idx, "gather");
     auto out = new_like(x, Shape{shape_[0]});
     check(odl_hip_gather(fp(x), idx.storage()->data(), is64, (int64_t)shape_[0], (int64_t)shape_[1],
-                         out->data_ptr<float>(), nullptr));
+                         out->data_ptr<float>(), cur()));
     return out;
 }
 
@@ -1070,7 +1169,7 @@ std::unique_ptr<Mat> OriginMat::one_hot(const Mat &indices, int num_classes) con
     const int is64 = label_kind(idx, "one_hot");
     auto out = std::make_unique<OriginMat>(Shape{idx.shape()[0], (size_t)num_classes}, DataType::kFloat32, idx.device());
     check(odl_hip_one_hot(idx.storage()->data(), is64, (int64_t)idx.shape()[0], num_classes, out->data_ptr<float>(),
-                          nullptr));
+                          cur()));
     return out;
 }
 
@@ -1081,7 +1180,7 @@ std::unique_ptr<Mat> OriginMat::softmax(int axis) const
     int64_t outer, ax, inner;
     split_axis(shape_, axis, outer, ax, inner);
     auto y = new_like(x, shape_);
-    check(odl_hip_softmax(fp(x), outer, ax, inner, y->data_ptr<float>(), nullptr));
+    check(odl_hip_softmax(fp(x), outer, ax, inner, y->data_ptr<float>(), cur()));
     return y;
 }
 
@@ -1093,7 +1192,7 @@ float OriginMat::softmax_cross_entropy(const Mat &target) const
     const int64_t N = shape_[0], C = shape_[1];
     Workspace ws(odl_hip_softmax_ce_loss_workspace_bytes(N), device().index());
     float loss = 0.f;
-    check(odl_hip_softmax_ce_loss(fp(x), t.storage()->data(), is64, N, C, &loss, ws.ptr(), ws.bytes, nullptr));
+    check(odl_hip_softmax_ce_loss(fp(x), t.storage()->data(), is64, N, C, &loss, ws.ptr(), ws.bytes, cur()));
     return loss;
 }
 
@@ -1104,8 +1203,85 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_backward(const Mat &target
     const int is64     = label_kind(t, "one_hot");
     auto gx = new_like(x, shape_);
     check(odl_hip_softmax_ce_grad(fp(x), t.storage()->data(), is64, (int64_t)shape_[0], (int64_t)shape_[1], gy,
-                                  gx->data_ptr<float>(), nullptr));
+                                  gx->data_ptr<float>(), cur()));
     return gx;
+}
+
+std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) const
+{
+    const OriginMat &x = dev_f32(*this, "softmax_cross_entropy");
+    const OriginMat &t = as_origin(target);
+    const int is64     = label_kind(t, "gather");
+    const int64_t N = shape_[0], C = shape_[1];
+    Workspace ws(odl_hip_softmax_ce_loss_workspace_bytes(N), device().index());
+    // two words: the loss, and the bad-label flag behind it; the Mat is the scalar in front
+    auto storage = Storage::create(2 * sizeof(float), DeviceType::kCUDA, device().index());
+    check(odl_hip_softmax_ce_loss_device(fp(x), t.storage()->data(), is64, N, C, static_cast<float *>(storage->data()),
+                                         ws.ptr(), ws.bytes, cur()));
+    return std::make_unique<OriginMat>(std::move(storage), Shape{}, DataType::kFloat32);
+}
+
+std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const
+{
+    const OriginMat &x = dev_f32(*this, "softmax_cross_entropy");
+    const OriginMat &t = as_origin(target);
+    const OriginMat &g = dev_f32(gy, "softmax_cross_entropy");
+    const int is64     = label_kind(t, "one_hot");
+    auto gx = new_like(x, shape_);
+    check(odl_hip_softmax_ce_grad_device(fp(x), t.storage()->data(), is64, (int64_t)shape_[0], (int64_t)shape_[1], fp(g),
+                                         gx->data_ptr<float>(), cur()));
+    return gx;
+}
+
+void OriginMat::upload(const void *host, size_t bytes)
+{
+    if (bytes != elements() * dtype_size(dtype_))
+        THROW_INVALID_ARG("upload: {} bytes given for a tensor of {} bytes", bytes, elements() * dtype_size(dtype_));
+    if (bytes == 0)
+        return;
+    if (device().type() == DeviceType::kCPU)
+    {
+        std::memcpy(storage_->data(), host, bytes);
+        return;
+    }
+    no_capture("host-to-device copy");
+    check(odl_hip_synchronize());
+    check(odl_hip_memcpy_h2d(storage_->data(), host, bytes));
+}
+
+void OriginMat::adam_step_inplace(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, const float *device_scales,
+                                  float eps, float lr)
+{
+    const OriginMat &p = dev_f32(*this, "adam_step");
+    const OriginMat &g = dev_f32(grad, "adam_step");
+    const OriginMat &mm = dev_f32(m, "adam_step");
+    const OriginMat &vv = dev_f32(v, "adam_step");
+    if (g.shape() != shape_ || mm.shape() != shape_ || vv.shape() != shape_)
+        THROW_INVALID_ARG("adam_step: parameter, gradient and moments must have one shape");
+    float *pp = const_cast<float *>(fp(p));
+    check(odl_hip_adam_step_device_scales(pp, fp(g), const_cast<float *>(fp(mm)), const_cast<float *>(fp(vv)),
+                                          (int64_t)elements(), beta1, beta2, device_scales, eps, lr, pp, cur()));
+}
+
+void OriginMat::copy_from(const Mat &src)
+{
+    const OriginMat &o = as_origin(src);
+    if (o.shape() != shape_ || o.dtype() != dtype_ || o.device() != device())
+        THROW_INVALID_ARG("copy_from: shape, dtype and device must match");
+    if (device().type() == DeviceType::kCPU)
+        std::memcpy(storage_->data(), o.storage()->data(), elements() * dtype_size(dtype_));
+    else
+        check(odl_hip_memcpy_d2d(storage_->data(), o.storage()->data(), elements() * dtype_size(dtype_), cur()));
+}
+
+void OriginMat::sgd_step_inplace(const Mat &grad, float lr)
+{
+    const OriginMat &p = dev_f32(*this, "sgd_step");
+    const OriginMat &g = dev_f32(grad, "sgd_step");
+    if (g.shape() != shape_)
+        THROW_INVALID_ARG("sgd_step: parameter and gradient must have one shape");
+    float *pp = const_cast<float *>(fp(p));
+    check(odl_hip_sgd_step(pp, fp(g), (int64_t)elements(), lr, pp, cur()));
 }
 
 std::unique_ptr<Mat> OriginMat::adam_step(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, float m_hat_scale,
@@ -1119,7 +1295,7 @@ std::unique_ptr<Mat> OriginMat::adam_step(const Mat &grad, Mat &m, Mat &v, float
         THROW_INVALID_ARG("adam_step: parameter, gradient and moment sizes differ");
     auto out = new_like(p, shape_);
     check(odl_hip_adam_step(fp(p), fp(g), const_cast<float *>(fp(mm)), const_cast<float *>(fp(vv)), (int64_t)elements(),
-                            beta1, beta2, m_hat_scale, v_hat_scale, eps, lr, out->data_ptr<float>(), nullptr));
+                            beta1, beta2, m_hat_scale, v_hat_scale, eps, lr, out->data_ptr<float>(), cur()));
     return out;
 }
 
@@ -1130,7 +1306,7 @@ std::unique_ptr<Mat> OriginMat::sgd_step(const Mat &grad, float lr) const
     if (g.elements() != elements())
         THROW_INVALID_ARG("sgd_step: parameter and gradient sizes differ");
     auto out = new_like(p, shape_);
-    check(odl_hip_sgd_step(fp(p), fp(g), (int64_t)elements(), lr, out->data_ptr<float>(), nullptr));
+    check(odl_hip_sgd_step(fp(p), fp(g), (int64_t)elements(), lr, out->data_ptr<float>(), cur()));
     return out;
 }
 
@@ -1147,7 +1323,7 @@ std::pair<std::unique_ptr<Mat>, std::unique_ptr<Mat>> OriginMat::matmul_backward
     auto gw = new_like(w, ws_);
     Workspace ws(odl_hip_matmul_backward_workspace_bytes(M, K, N), x.device().index());
     check(odl_hip_matmul_backward(fp(x), fp(w), fp(gy), gx->data_ptr<float>(), gw->data_ptr<float>(), M, K, N, ws.ptr(),
-                                  ws.bytes, nullptr));
+                                  ws.bytes, cur()));
     return {std::move(gx), std::move(gw)};
 }
 
@@ -1160,7 +1336,93 @@ float OriginMat::accuracy(const Mat &target_int32) const
     Workspace ws(odl_hip_accuracy_workspace_bytes((int64_t)shape_[0]), device().index());
     float acc = 0.f;
     check(odl_hip_accuracy(fp(y), t.data_ptr<int32_t>(), (int64_t)shape_[0], (int64_t)shape_[1], &acc, ws.ptr(),
-                           ws.bytes, nullptr));
+                           ws.bytes, cur()));
     return acc;
 }
+
+// ----------------------------------------------------------------------------------- streams and graphs
+namespace cuda
+{
+void *create_stream()
+{
+    void *s = nullptr;
+    check(odl_hip_stream_create(&s));
+    return s;
+}
+
+void destroy_stream(void *stream)
+{
+    if (stream && stream == t_stream)
+        set_stream(nullptr);
+    check(odl_hip_stream_destroy(stream));
+}
+
+void set_stream(void *stream)
+{
+    if (t_capturing)
+        THROW_RUNTIME_ERROR("the stream cannot be changed while a graph is being captured");
+    if (stream == t_stream)
+        return;
+    check(odl_hip_synchronize());  // memory freed under the old stream may be handed out under the new one
+    t_stream = stream;
+}
+
+void *current_stream()
+{
+    return t_stream;
+}
+
+bool is_capturing()
+{
+    return t_capturing;
+}
+
+Graph::~Graph()
+{
+    if (exec_)
+    {
+        (void)odl_hip_synchronize();  // no replay may still be running when its memory is handed back
+        (void)odl_hip_graph_destroy(exec_);
+    }
+}
+
+void Graph::begin_capture()
+{
+    if (exec_)
+        THROW_RUNTIME_ERROR("this graph has been captured already");
+    if (!t_stream)
+        THROW_RUNTIME_ERROR("graph capture needs a created stream (cuda::set_stream): the null stream cannot be captured");
+    check(odl_hip_stream_synchronize(t_stream));
+    arena_ = DevicePool::get().begin_capture();
+    if (odl_hip_graph_capture_begin(t_stream) != ODL_OK)
+    {
+        DevicePool::get().end_capture();
+        arena_.reset();
+        THROW_RUNTIME_ERROR("{}", odl_hip_last_error());
+    }
+    t_capturing = true;
+}
+
+void Graph::end_capture()
+{
+    if (!t_capturing)
+        THROW_RUNTIME_ERROR("end_capture without begin_capture");
+    t_capturing = false;
+    DevicePool::get().end_capture();
+    void *exec = nullptr;
+    if (odl_hip_graph_capture_end(t_stream, &exec) != ODL_OK)
+    {
+        arena_.reset();
+        THROW_RUNTIME_ERROR("{}", odl_hip_last_error());
+    }
+    exec_ = exec;
+}
+
+void Graph::launch()
+{
+    if (!exec_)
+        THROW_RUNTIME_ERROR("this graph has not been captured");
+    check(odl_hip_graph_launch(exec_, t_stream));
+}
+}  // namespace cuda
 }  // namespace origin

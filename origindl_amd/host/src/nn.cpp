@@ -362,16 +362,28 @@ void SGD::step_one(Parameter &param)
         if (it == momentum_buffers_.end())
             it = momentum_buffers_.emplace(&param, Tensor::zeros(grad.shape(), TensorOptions(grad.dtype()).device(grad.device()))).first;
         Tensor &buf = it->second;
-        buf  = buf * Scalar(momentum_) + grad;
+        if (cuda::is_capturing())
+            const_cast<OriginMat &>(origin_mat(buf)).copy_from(*(buf * Scalar(momentum_) + grad).impl_->data_);
+        else
+            buf = buf * Scalar(momentum_) + grad;
         grad = nesterov_ ? grad + buf * Scalar(momentum_) : buf;
     }
+    // While a graph is being captured every persistent tensor is written where it lies (a later replay reads it
+    // from that address), instead of being rebound to a new one.
+    const bool in_place = cuda::is_capturing();
     if (weight_decay_ <= 0.0f && momentum_ <= 0.0f)
     {
         // plain step: one launch computing the same two roundings as param - grad * lr
-        param = as_leaf(Tensor(origin_mat(param).sgd_step(*grad.impl_->data_, lr_)));
+        if (in_place)
+            const_cast<OriginMat &>(origin_mat(param)).sgd_step_inplace(*grad.impl_->data_, lr_);
+        else
+            param = as_leaf(Tensor(origin_mat(param).sgd_step(*grad.impl_->data_, lr_)));
         return;
     }
-    param = as_leaf(param - grad * Scalar(lr_));
+    if (in_place)
+        const_cast<OriginMat &>(origin_mat(param)).copy_from(*(param - grad * Scalar(lr_)).impl_->data_);
+    else
+        param = as_leaf(param - grad * Scalar(lr_));
 }
 
 Adam::Adam(Module &target, float lr, float beta1, float beta2, float eps)
@@ -387,9 +399,25 @@ void Adam::step_one(Parameter &param)
         m_buffers_.emplace(&param, zeros());
     if (!v_buffers_.count(&param))
         v_buffers_.emplace(&param, zeros());
+    Tensor &m = m_buffers_.at(&param), &v = v_buffers_.at(&param);
+    if (!replay_scales_.defined())  // two floats per parameter, read by recorded steps (see prepare_replay)
+        replay_scales_ = Tensor::zeros(Shape{parameters_.size(), 2}, TensorOptions(DataType::kFloat32).device(grad.device()));
+    if (cuda::is_capturing())
+    {
+        // recorded, not run: the step count moves in prepare_replay(), and the factors come from device memory
+        if (!step_counts_.count(&param))
+            THROW_RUNTIME_ERROR("Adam: run one ordinary step before capturing (the moment buffers must exist)");
+        size_t index = 0;
+        while (index < parameters_.size() && parameters_[index] != &param)
+            ++index;
+        const float *scales = static_cast<const OriginMat &>(*replay_scales_.impl_->data_).data_ptr<float>() + 2 * index;
+        const_cast<OriginMat &>(origin_mat(param))
+            .adam_step_inplace(*grad.impl_->data_, *m.impl_->data_, *v.impl_->data_, beta1_, beta2_, scales, eps_, lr_);
+        replay_params_.push_back(&param);
+        return;
+    }
     int &t = step_counts_[&param];
     ++t;
-    Tensor &m = m_buffers_.at(&param), &v = v_buffers_.at(&param);
     // same sequence of elementwise steps, each rounded to float, as src/optim/adam.cpp:52-113
     //   m = m*b1 + grad*(1-b1);  v = v*b2 + (grad*grad)*(1-b2);  m_hat = m*s1;  v_hat = v*s2;
     //   param = param - (m_hat / (pow(v_hat, 0.5) + eps)) * lr
@@ -398,6 +426,23 @@ void Adam::step_one(Parameter &param)
     const float m_hat_scale = 1.0f / (1.0f - b1p), v_hat_scale = 1.0f / (1.0f - b2p);
     param = as_leaf(Tensor(origin_mat(param).adam_step(*grad.impl_->data_, *m.impl_->data_, *v.impl_->data_, beta1_, beta2_,
                                                        m_hat_scale, v_hat_scale, eps_, lr_)));
+}
+
+void Adam::prepare_replay()
+{
+    if (replay_params_.empty())
+        return;
+    std::vector<float> host(parameters_.size() * 2, 0.0f);
+    for (Parameter *p : replay_params_)
+    {
+        size_t index = 0;
+        while (index < parameters_.size() && parameters_[index] != p)
+            ++index;
+        const int t = ++step_counts_[p];
+        const float b1p = std::pow(beta1_, static_cast<float>(t)), b2p = std::pow(beta2_, static_cast<float>(t));
+        host[2 * index] = 1.0f / (1.0f - b1p), host[2 * index + 1] = 1.0f / (1.0f - b2p);
+    }
+    replay_scales_.upload(host.data(), host.size() * sizeof(float));
 }
 
 std::function<void(std::vector<Parameter *> &)> WeightDecay::hook() const

@@ -149,6 +149,12 @@ Tensor Tensor::full(const Shape &s, const Scalar &v, const TensorOptions &o)
     return t;
 }
 
+void Tensor::upload(const void *host, size_t bytes)
+{
+    check_defined("upload");
+    static_cast<OriginMat &>(*impl_->data_).upload(host, bytes);
+}
+
 Shape Tensor::shape() const
 {
     return defined() ? impl_->data_->shape() : Shape();

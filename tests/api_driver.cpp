@@ -125,6 +125,20 @@ void out(const origin::Mat &m, float *dst)
     std::memcpy(dst, v.data(), v.size() * sizeof(float));
 }
 
+#ifdef DRV_ON_DEVICE
+// a created stream made current for the scope (graph capture needs one: the null stream cannot be captured)
+struct StreamScope
+{
+    void *s;
+    StreamScope() : s(origin::cuda::create_stream()) { origin::cuda::set_stream(s); }
+    ~StreamScope()
+    {
+        origin::cuda::set_stream(nullptr);
+        origin::cuda::destroy_stream(s);
+    }
+};
+#endif
+
 template <typename Fn>
 int guarded(Fn &&fn)
 {
@@ -656,6 +670,58 @@ int DRV(pnnx_forward)(const char *param_path, const char *bin_path, const float 
     });
 }
 
+#ifdef DRV_ON_DEVICE
+// The same model with its forward recorded into a graph: two ordinary forwards (weights uploaded, pool warm), the
+// capture, then `reps` replays. Before every replay the input tensor is rewritten in place with x scaled by
+// (1 + 0.125 * replay), the last replay with x itself, so the output returned is the one of x and a replay that
+// ignored its input would be caught. ms = mean time of a replay, complete on the device.
+int DRV(pnnx_forward_graph)(const char *param_path, const char *bin_path, const float *x, int64_t N, int64_t C, int64_t H,
+                            int64_t W, int reps, float *o, int64_t capacity, int64_t *out_shape, int *out_nd, float *ms)
+{
+    return guarded([&] {
+        StreamScope stream;
+        origin::pnnx::PNNXGraph graph(param_path, bin_path);
+        graph.build();
+        const Shape xs{(size_t)N, (size_t)C, (size_t)H, (size_t)W};
+        auto X = f32(x, xs);
+        graph.set_inputs("pnnx_input_0", {X});
+        for (int r = 0; r < 2; ++r)
+            graph.forward();
+        origin::cuda::Graph recorded;
+        recorded.begin_capture();
+        graph.forward();
+        recorded.end_capture();
+        std::vector<Tensor> outs = graph.get_outputs("pnnx_output_0");
+        if (outs.empty())
+            throw std::runtime_error("pnnx_forward: the graph produced no output");
+        const int n = reps < 1 ? 1 : reps;
+        std::vector<float> scaled(xs.elements());
+        float total_ms = 0.0f;
+        for (int r = 0; r < n; ++r)
+        {
+            const float f = r + 1 == n ? 1.0f : 1.0f + 0.125f * (float)(r + 1);
+            for (size_t i = 0; i < scaled.size(); ++i)
+                scaled[i] = x[i] * f;
+            X.upload(scaled.data(), scaled.size() * sizeof(float));
+            const auto t0 = std::chrono::steady_clock::now();
+            recorded.launch();
+            origin::cuda::synchronize();
+            total_ms += std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        }
+        const Shape shp         = outs[0].shape();
+        std::vector<float> last = outs[0].to_vector<float>();
+        if (ms)
+            *ms = total_ms / (float)n;
+        if ((int64_t)last.size() > capacity)
+            throw std::invalid_argument("pnnx_forward: output larger than the buffer");
+        std::memcpy(o, last.data(), last.size() * sizeof(float));
+        *out_nd = (int)shp.size();
+        for (size_t i = 0; i < shp.size(); ++i)
+            out_shape[i] = (int64_t)shp[i];
+    });
+}
+#endif
+
 int DRV(pow_scalar)(const float *a, int64_t n, float e, float *o)
 {
     return guarded([&] { out(F::pow(f32(a, Shape{(size_t)n}), Scalar(e)), o); });
@@ -663,11 +729,25 @@ int DRV(pow_scalar)(const float *a, int64_t n, float e, float *o)
 
 // MLP D -> Hd -> C (Linear, ReLU, Linear), softmax CE, WeightDecay hook, Adam; `steps` steps on the same batch.
 // Parameters are read and written in place; loss/grads/logits of the LAST step are returned.
-int DRV(mlp_train)(const float *x, const void *t, int is64, int64_t N, int64_t D, int64_t Hd, int64_t C, float *W1,
-                      float *b1, float *W2, float *b2, int steps, float lr, float beta1, float beta2, float eps,
-                      float wd, float *loss, float *gW1, float *gb1, float *gW2, float *gb2, float *logits)
+}  // extern "C"
+
+namespace
+{
+// use_graph (device build only): the first step runs ordinarily, then one step is recorded into a graph and the
+// remaining steps are replays of it — the results must be the ones of `steps` ordinary steps, bit for bit.
+int mlp_train_impl(const float *x, const void *t, int is64, int64_t N, int64_t D, int64_t Hd, int64_t C, float *W1,
+                   float *b1, float *W2, float *b2, int steps, float lr, float beta1, float beta2, float eps, float wd,
+                   float *loss, float *gW1, float *gb1, float *gW2, float *gb2, float *logits, bool use_graph)
 {
     return guarded([&] {
+#ifdef DRV_ON_DEVICE
+        std::unique_ptr<StreamScope> stream;
+        if (use_graph)
+            stream = std::make_unique<StreamScope>();
+#else
+        if (use_graph)
+            throw std::runtime_error("graph replay is only available on the device build of this driver");
+#endif
         Sequential model;
         model.add(std::make_unique<nn::Linear>((int)D, (int)Hd, true));
         model.add(std::make_unique<nn::ReLU>());
@@ -684,7 +764,7 @@ int DRV(mlp_train)(const float *x, const void *t, int is64, int64_t N, int64_t D
         auto X = f32(x, Shape{(size_t)N, (size_t)D});
         auto T = labels(t, is64, N);
         model.train();
-        for (int s = 0; s < steps; ++s)
+        for (int s = 0; s < (use_graph ? 1 : steps); ++s)
         {
             opt.zero_grad();
             auto y = model(X);
@@ -698,12 +778,62 @@ int DRV(mlp_train)(const float *x, const void *t, int is64, int64_t N, int64_t D
             out(l2.bias()->grad(), gb2);
             opt.step();
         }
+#ifdef DRV_ON_DEVICE
+        if (use_graph && steps > 1)
+        {
+            origin::cuda::Graph graph;
+            graph.begin_capture();
+            opt.zero_grad();
+            auto y = model(X);
+            auto L = F::softmax_cross_entropy(y, T);
+            L.backward();
+            opt.step();
+            graph.end_capture();
+            for (int s = 1; s < steps; ++s)
+            {
+                opt.prepare_replay();
+                graph.launch();
+                // ordinary work between the replays, on memory the graph does not own: a replay must not depend on
+                // what ran in between
+                auto scratch = (X * Scalar(2.0f)).to_vector<float>();
+                (void)scratch;
+            }
+            *loss = L.item<float>();
+            out(y, logits);
+            // the gradients of the last replay, after the weight-decay hook of the recorded step (the ordinary loop
+            // above reports them before the hook): equal to it only when wd == 0
+            out(l1.weight()->grad(), gW1);
+            out(l1.bias()->grad(), gb1);
+            out(l2.weight()->grad(), gW2);
+            out(l2.bias()->grad(), gb2);
+        }
+#endif
         out(*l1.weight(), W1);
         out(*l1.bias(), b1);
         out(*l2.weight(), W2);
         out(*l2.bias(), b2);
     });
 }
+}  // namespace
+
+extern "C" {
+int DRV(mlp_train)(const float *x, const void *t, int is64, int64_t N, int64_t D, int64_t Hd, int64_t C, float *W1,
+                      float *b1, float *W2, float *b2, int steps, float lr, float beta1, float beta2, float eps,
+                      float wd, float *loss, float *gW1, float *gb1, float *gW2, float *gb2, float *logits)
+{
+    return mlp_train_impl(x, t, is64, N, D, Hd, C, W1, b1, W2, b2, steps, lr, beta1, beta2, eps, wd, loss, gW1, gb1, gW2,
+                          gb2, logits, false);
+}
+
+#ifdef DRV_ON_DEVICE
+int DRV(mlp_train_graph)(const float *x, const void *t, int is64, int64_t N, int64_t D, int64_t Hd, int64_t C, float *W1,
+                         float *b1, float *W2, float *b2, int steps, float lr, float beta1, float beta2, float eps,
+                         float wd, float *loss, float *gW1, float *gb1, float *gW2, float *gb2, float *logits)
+{
+    return mlp_train_impl(x, t, is64, N, D, Hd, C, W1, b1, W2, b2, steps, lr, beta1, beta2, eps, wd, loss, gW1, gb1, gW2,
+                          gb2, logits, true);
+}
+#endif
 
 // CNN of BASELINE config 4 (no BatchNorm), SGD without momentum/weight decay, one step.
 int DRV(cnn_train)(const float *x, const void *t, int is64, int64_t N, int64_t S, int64_t C1, int64_t C2, int64_t Hd,
@@ -824,11 +954,77 @@ void timed_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T, int s
     const auto t1 = std::chrono::steady_clock::now();
     *ms = std::chrono::duration<float, std::milli>(t1 - t0).count() / (float)(steps > 0 ? steps : 1);
 }
+
+#ifdef DRV_ON_DEVICE
+// The same step recorded once into a graph and replayed (this backend only: the reference has no streams or
+// graphs). Two ordinary steps first (memory pool warm, optimizer buffers made), then the capture, then `steps`
+// replays; the loss is read back after every replay when read_loss != 0, as the loop above does, or once at the end.
+
+template <typename Model, typename Opt>
+void timed_graph_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T, int steps, int warmup, int read_loss,
+                       float *ms, float *loss)
+{
+    StreamScope stream;
+    model.train();
+    for (int i = 0; i < (warmup > 2 ? warmup : 2); ++i)
+    {
+        opt.zero_grad();
+        auto L = F::softmax_cross_entropy(model(X), T);
+        L.backward();
+        opt.step();
+        *loss = L.template item<float>();
+    }
+    origin::cuda::Graph graph;
+    Tensor L;
+    graph.begin_capture();
+    opt.zero_grad();
+    L = F::softmax_cross_entropy(model(X), T);
+    L.backward();
+    opt.step();
+    graph.end_capture();
+    for (int i = 0; i < 2; ++i)  // untimed replays
+    {
+        opt.prepare_replay();
+        graph.launch();
+    }
+    *loss = L.template item<float>();
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; ++i)
+    {
+        opt.prepare_replay();
+        graph.launch();
+        if (read_loss)
+            *loss = L.template item<float>();
+    }
+    *loss = L.template item<float>();  // synchronises: every replay is complete
+    const auto t1 = std::chrono::steady_clock::now();
+    *ms = std::chrono::duration<float, std::milli>(t1 - t0).count() / (float)(steps > 0 ? steps : 1);
+}
+#endif
 }  // namespace
 
 extern "C" {
 
-int DRV(mlp_bench)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, float *ms_per_step, float *loss)
+}  // extern "C"
+
+namespace
+{
+// graph_mode 0: ordinary steps; 1: a recorded step replayed, loss read back every step; 2: read back at the end only
+template <typename Model, typename Opt>
+void run_timed(Model &model, Opt &opt, const Tensor &X, const Tensor &T, int steps, int warmup, int graph_mode, float *ms,
+               float *loss)
+{
+#ifdef DRV_ON_DEVICE
+    if (graph_mode != 0)
+        return timed_graph_steps(model, opt, X, T, steps, warmup, graph_mode == 1, ms, loss);
+#endif
+    if (graph_mode != 0)
+        throw std::runtime_error("graph replay is only available on the device build of this driver");
+    timed_steps(model, opt, X, T, steps, warmup, ms, loss);
+}
+
+int mlp_bench_impl(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, int graph_mode, float *ms_per_step,
+                   float *loss)
 {
     return guarded([&] {
         std::mt19937 gen(1234);
@@ -850,11 +1046,11 @@ int DRV(mlp_bench)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int w
         for (auto &e : tv)
             e = (int64_t)(gen() % (uint32_t)C);
         auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt64).device(kDev));
-        timed_steps(model, opt, X, T, steps, warmup, ms_per_step, loss);
+        run_timed(model, opt, X, T, steps, warmup, graph_mode, ms_per_step, loss);
     });
 }
 
-int DRV(cnn_bench)(int64_t N, int steps, int warmup, float *ms_per_step, float *loss)
+int cnn_bench_impl(int64_t N, int steps, int warmup, int graph_mode, float *ms_per_step, float *loss)
 {
     return guarded([&] {
         std::mt19937 gen(4321);
@@ -889,8 +1085,32 @@ int DRV(cnn_bench)(int64_t N, int steps, int warmup, float *ms_per_step, float *
         for (auto &e : tv)
             e = (int64_t)(gen() % (uint32_t)Cc);
         auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt64).device(kDev));
-        timed_steps(model, opt, X, T, steps, warmup, ms_per_step, loss);
+        run_timed(model, opt, X, T, steps, warmup, graph_mode, ms_per_step, loss);
     });
 }
+}  // namespace
 
+extern "C" {
+int DRV(mlp_bench)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, float *ms_per_step, float *loss)
+{
+    return mlp_bench_impl(N, D, Hd, C, steps, warmup, 0, ms_per_step, loss);
+}
+
+int DRV(cnn_bench)(int64_t N, int steps, int warmup, float *ms_per_step, float *loss)
+{
+    return cnn_bench_impl(N, steps, warmup, 0, ms_per_step, loss);
+}
+
+#ifdef DRV_ON_DEVICE
+int DRV(mlp_bench_graph)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, int read_loss_each_step,
+                         float *ms_per_step, float *loss)
+{
+    return mlp_bench_impl(N, D, Hd, C, steps, warmup, read_loss_each_step ? 1 : 2, ms_per_step, loss);
+}
+
+int DRV(cnn_bench_graph)(int64_t N, int steps, int warmup, int read_loss_each_step, float *ms_per_step, float *loss)
+{
+    return cnn_bench_impl(N, steps, warmup, read_loss_each_step ? 1 : 2, ms_per_step, loss);
+}
+#endif
 }  // extern "C"

@@ -96,6 +96,15 @@ _REF_SIGS = {
 }
 
 
+# entry points only the device build of the driver has (streams and recorded graphs do not exist in the reference)
+_DEVICE_ONLY_SIGS = {
+    "odl_host_mlp_train_graph": _REF_SIGS["odl_ref_mlp_train"],
+    "odl_host_mlp_bench_graph": "lllliiipp>i",
+    "odl_host_cnn_bench_graph": "liiipp>i",
+    "odl_host_pnnx_forward_graph": _REF_SIGS["odl_ref_pnnx_forward"],
+}
+
+
 def _ret(c):
     return {"v": None, "i": ctypes.c_int, "f": ctypes.c_float, "l": ctypes.c_int64}[c]
 
@@ -173,6 +182,8 @@ def host_driver(cpu=False):
     if key not in _host:
         prefix = "odl_%s_" % key
         sigs = {k.replace("odl_ref_", prefix): v for k, v in _REF_SIGS.items()}
+        if not cpu:
+            sigs.update(_DEVICE_ONLY_SIGS)
         _host[key] = _Lib(HOST_CPU_DRIVER_SO if cpu else HOST_DRIVER_SO, sigs)
     return _host[key]
 

@@ -203,6 +203,34 @@ def test_mlp_training_step_matches_the_reference(h, steps):
         assert np.abs(a - ref).max() <= 2.1e-3 * steps
 
 
+@pytest.mark.parametrize("wd", [1e-4, 0.0])
+def test_recorded_training_step_replays_bit_for_bit(h, wd):
+    """The MLP step (forward, softmax-CE, backward, weight-decay hook, Adam) recorded once into a graph and replayed
+    must leave exactly what the same number of ordinary steps leaves: same kernels, same arithmetic, the loss and the
+    upstream gradient read from device memory instead of passing through the host, Adam's bias-correction factors
+    rewritten before every replay. Ordinary work runs between the replays (the driver queues an unrelated kernel and
+    reads its result back), so a replay that depended on leftover state would show."""
+    x, t = G["mlp_x"], G["mlp_t"]
+    N, D = x.shape
+    p0 = [G[f"mlp_{k}"] for k in ("W1", "b1", "W2", "b2")]
+    Hd, C = p0[0].shape[1], p0[2].shape[1]
+    for steps in (2, 5):
+        res = {}
+        for name in ("odl_host_mlp_train", "odl_host_mlp_train_graph"):
+            p = [a.copy() for a in p0]
+            g = [np.empty_like(a) for a in p]
+            loss, logits = np.zeros(1, f32), np.empty((N, C), f32)
+            assert getattr(h, name)(x, t, 1, N, D, Hd, C, *p, steps, 1e-3, 0.9, 0.999, 1e-8, wd, loss, *g, logits) == 0
+            res[name] = (loss, logits, p, g)
+        (le, ye, pe, ge), (lg, yg, pg, gg) = res["odl_host_mlp_train"], res["odl_host_mlp_train_graph"]
+        assert le[0] == lg[0] and np.array_equal(ye, yg), steps
+        for a, b in zip(pe, pg):
+            assert np.array_equal(a, b), steps
+        if wd == 0.0:  # with the hook the two drivers report the gradients at different moments
+            for a, b in zip(ge, gg):
+                assert np.array_equal(a, b), steps
+
+
 def test_cnn_training_step_matches_the_reference(h):
     names = ("Wc1", "bc1", "Wc2", "bc2", "Wl1", "bl1", "Wl2", "bl2")
     x, t = G["cnn_x"], G["cnn_t"]
@@ -374,12 +402,11 @@ def test_batch_norm_layer_rejects_wrong_inputs(h):
                                              1e-5, 2, 3, 4, 4, buf, buf, buf, buf) == -2
 
 
-def _run_pnnx(drv, prefix, param, binp, x, out_shape, reps=1):
+def _run_pnnx(drv, prefix, param, binp, x, out_shape, reps=1, entry="pnnx_forward"):
     out = np.empty(out_shape, f32)
     oshape, nd, ms = np.zeros(8, np.int64), np.zeros(1, np.int32), np.zeros(1, f32)
     N, C, H, W = x.shape
-    rc = getattr(drv, prefix + "pnnx_forward")(param.encode(), binp.encode(), x, N, C, H, W, reps, out, out.size, oshape,
-                                               nd, ms)
+    rc = getattr(drv, prefix + entry)(param.encode(), binp.encode(), x, N, C, H, W, reps, out, out.size, oshape, nd, ms)
     return rc, out, tuple(oshape[:nd[0]]), float(ms[0])
 
 
@@ -417,6 +444,20 @@ def test_pnnx_runner_rejects_bad_files(h, tmp_path):
     trunc.write_bytes(open(binp, "rb").read()[:4000])
     assert _run_pnnx(h, "odl_host_", param, str(trunc), x, shp)[0] == -2
     assert _run_pnnx(h, "odl_host_", param, binp, x, shp)[0] == 0
+
+
+def test_recorded_detector_forward_replays_bit_for_bit(h, tmp_path):
+    """The YOLOv5n-architecture forward recorded into a graph: every replay reads the input tensor in place, and the
+    last one (on the fixture's input) must give exactly the ordinary forward's output."""
+    import pnnx_synth
+    param, binp, shp = pnnx_synth.write(str(tmp_path / "y5n"), seed=3, batch=1, size=64, num_classes=80)
+    x = G["y5n64_x"]
+    rc, eager, _, _ = _run_pnnx(h, "odl_host_", param, binp, x, shp, reps=2)
+    assert rc == 0
+    rc, replayed, _, ms = _run_pnnx(h, "odl_host_", param, binp, x, shp, reps=4, entry="pnnx_forward_graph")
+    assert rc == 0 and ms > 0
+    assert np.array_equal(replayed, eager)
+    np.testing.assert_allclose(replayed, G["y5n64_out"], rtol=1e-4, atol=1e-4)
 
 
 def test_the_references_own_operator_unit_tests_pass_on_this_backend():
