@@ -202,7 +202,8 @@ size_t odl_hip_accuracy_workspace_bytes(int64_t N);
 /* ------------------------------------------------------------------ elementwise --------------------- */
 /* origin::cuda::{add,subtract,multiply,divide,gt,eq,ne,lt,le,ge} (cuda_ops.cuh:57-140): op 0 add, 1 sub, 2 mul, 3 div,
  * 4 greater-than, 5 equal, 6 not-equal, 7 less, 8 less-equal, 9 greater-equal (masks of 1.0f / 0.0f);
- * 10 sigmoid_backward(a = gy, b = y) = gy*y*(1-y) (mat.h:399), 11 silu_backward(a = gy, b = x) (mat.h:413).
+ * 10 sigmoid_backward(a = gy, b = y) = gy*y*(1-y) (mat.h:399), 11 silu_backward(a = gy, b = x) (mat.h:413),
+ * 12 relu_backward(a = gy, b = x) = gy * (x > 0 ? 1 : 0): ReLU::backward's mask and product (relu.cpp:23-52) in one pass.
  * na == nb, or one side has a single element; anything else is the
  * reference's "complex broadcasting" runtime_error. out may alias a or b (add_inplace). */
 int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t nb, float *out, void *stream);

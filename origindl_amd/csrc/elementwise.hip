@@ -30,6 +30,8 @@ __device__ inline float bin(float a, float b)
         const float t = a * b;
         return t * (1.0f - b);
     }
+    if (OP == 12)  // relu: b = x; gy * (x > 0 ? 1 : 0), a product as in the reference (relu.cpp:23-29, 45-52)
+        return a * ((b > 0.f) ? 1.f : 0.f);
     // silu: b = x; gy*(s + x*s*(1-s)) with s = sigmoid(x) (cpu/activation/silu.cpp:87-90)
     const float sg = 1.0f / (1.0f + expf(-b));
     const float xs = b * sg;
@@ -274,7 +276,7 @@ extern "C" {
 int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t nb, float *out, void *stream)
 {
     ODL_REQUIRE_DEVICE();
-    ODL_REQUIRE(op >= 0 && op <= 11, "binary: unknown op %d", op);
+    ODL_REQUIRE(op >= 0 && op <= 12, "binary: unknown op %d", op);
     ODL_REQUIRE(na >= 0 && nb >= 0, "binary: negative extent");
     if (!(na == nb || na == 1 || nb == 1))
         return odl::fail(ODL_ERR_RUNTIME, "Complex broadcasting not yet implemented (%lld vs %lld elements)",
@@ -295,7 +297,8 @@ int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t n
         case 8: return launch_binary<8>(a, na, b, nb, out, st);
         case 9: return launch_binary<9>(a, na, b, nb, out, st);
         case 10: return launch_binary<10>(a, na, b, nb, out, st);
-        default: return launch_binary<11>(a, na, b, nb, out, st);
+        case 11: return launch_binary<11>(a, na, b, nb, out, st);
+        default: return launch_binary<12>(a, na, b, nb, out, st);
     }
 }
 

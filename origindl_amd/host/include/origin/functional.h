@@ -51,6 +51,8 @@ Tensor batch_norm(const Tensor &x, const Tensor &gamma, const Tensor &beta, cons
 std::vector<Tensor> batch_norm_outputs(const Tensor &x, const Tensor &gamma, const Tensor &beta,
                                        const Tensor &running_mean, const Tensor &running_var, bool training, float eps,
                                        float momentum, int num_dims);
+// x[M,K] . w[K,N] + b (b of N elements) in one kernel; what nn::Linear::forward uses for 2-D inputs
+Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b);
 Tensor softmax(const Tensor &x, int axis = -1);
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &target);
 Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b = nullptr, std::pair<int, int> stride = {1, 1},

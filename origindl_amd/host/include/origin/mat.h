@@ -289,6 +289,13 @@ public:
     // overwrites this tensor's elements with another's of the same shape (a device-to-device copy on the current
     // stream): how a recorded step stores a freshly computed tensor at the address later replays read it from
     void copy_from(const Mat &src);
+    // gy (this) times the mask x > 0, in one launch: the two kernels of ReLU::backward, same products
+    std::unique_ptr<Mat> relu_backward(const Mat &x) const;
+    // x (this) . W + b with the bias added in the product's epilogue: the three kernels of Linear::forward
+    // (matmul, broadcast_to, add), same rounding (the sum is rounded to float before the bias is added)
+    std::unique_ptr<Mat> linear(const Mat &W, const Mat &b) const;
+    // this += b*other, one launch (the weight-decay hook's multiply and accumulate)
+    void axpy_inplace(float b, const Mat &other);
     // a*this + b*other in one launch (each product rounded before the sum): the running-statistics update of the
     // BatchNorm layers
     std::unique_ptr<Mat> axpby(float a, float b, const Mat &other) const;

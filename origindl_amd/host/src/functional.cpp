@@ -233,16 +233,31 @@ struct Transpose : Operator
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override { return {wrap(mat(gys[0]).transpose())}; }
 };
 
-struct ReLU : Operator  // src/operators/activation/relu.cpp:13-54: mask = x > 0, gx = gy * mask
+// src/operators/activation/relu.cpp:13-54: mask = x > 0, gx = gy * mask. The mask is not kept: backward forms it from
+// the input again inside the one kernel that also multiplies (same 0/1 factor, same product).
+struct ReLU : Operator
 {
-    Tensor mask;
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).relu())}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        return {wrap(omat(gys[0]).relu_backward(mat(inputs_[0])))};
+    }
+};
+
+// Linear::forward's matmul + broadcast_to + add (src/nn/layers/linear.cpp:88-104) as one operator for 2-D inputs:
+// the bias is added in the product's epilogue, and backward is the three gradients those operators would produce
+// (gx = gy.W^T, gW = x^T.gy, gb = gy summed to the bias's shape).
+struct LinearOp : Operator
+{
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
-        if (xs[0].requires_grad())
-            mask = wrap(mat(xs[0]) > mat(scalar_like(Scalar(0.0f), xs[0])));
-        return {wrap(mat(xs[0]).relu())};
+        return {wrap(omat(xs[0]).linear(mat(xs[1]), mat(xs[2])))};
     }
-    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override { return {wrap(mat(gys[0]) * mat(mask))}; }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        auto g = OriginMat::matmul_backward_2d(mat(inputs_[0]), mat(inputs_[1]), mat(gys[0]));
+        return {wrap(std::move(g.first)), wrap(std::move(g.second)), wrap(mat(gys[0]).sum_to(inputs_[2].shape()))};
+    }
 };
 
 struct Softmax : Operator  // src/operators/activation/softmax.cpp:14-129
@@ -545,6 +560,7 @@ Tensor batch_norm(const Tensor &x, const Tensor &gamma, const Tensor &beta, cons
 {
     return batch_norm_outputs(x, gamma, beta, rm, rv, training, eps, momentum, num_dims)[0];
 }
+Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b) { return apply<LinearOp>({x, w, b}); }
 Tensor softmax(const Tensor &x, int axis) { return apply<Softmax>({x}, axis); }
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &t) { return apply<SoftmaxCrossEntropy>({x, t}); }
 

@@ -716,6 +716,33 @@ std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward(const Mat &gym,
     return outs;
 }
 
+std::unique_ptr<Mat> OriginMat::relu_backward(const Mat &x) const
+{
+    return binary(12, "relu_backward", dev_f32(*this, "relu_backward"), x);
+}
+
+std::unique_ptr<Mat> OriginMat::linear(const Mat &W_, const Mat &b_) const
+{
+    const OriginMat &x = dev_f32(*this, "linear"), &W = dev_f32(W_, "linear"), &b = dev_f32(b_, "linear");
+    if (shape_.size() != 2 || W.shape().size() != 2 || shape_[1] != W.shape()[0] || b.elements() != W.shape()[1])
+        THROW_INVALID_ARG("linear: x {} . W {} + b {} do not fit", shape_.to_string(), W.shape().to_string(),
+                          b.shape().to_string());
+    const int64_t M = shape_[0], K = shape_[1], N = W.shape()[1];
+    auto y = new_like(x, Shape{(size_t)M, (size_t)N});
+    Workspace ws(odl_hip_sgemm_workspace_bytes(0, 0, M, N, K, 0), device().index());
+    check(odl_hip_sgemm(0, 0, M, N, K, fp(x), K, fp(W), N, y->data_ptr<float>(), N, fp(b), 0, ws.ptr(), ws.bytes, cur()));
+    return y;
+}
+
+void OriginMat::axpy_inplace(float b, const Mat &other)
+{
+    const OriginMat &x = dev_f32(*this, "axpy"), &y = dev_f32(other, "axpy");
+    if (x.shape() != y.shape())
+        THROW_INVALID_ARG("axpy: shape mismatch {} vs {}", x.shape().to_string(), y.shape().to_string());
+    float *p = const_cast<float *>(fp(x));
+    check(odl_hip_axpby(1.0f, p, b, fp(y), (int64_t)elements(), p, cur()));
+}
+
 std::unique_ptr<Mat> OriginMat::axpby(float a, float b, const Mat &other) const
 {
     const OriginMat &x = dev_f32(*this, "axpby"), &y = dev_f32(other, "axpby");

@@ -226,6 +226,8 @@ Tensor Linear::forward(const Tensor &input)
 {
     if (weight_.shape().elements() == 0)
         THROW_RUNTIME_ERROR("Weight is empty in forward! weight_.shape() = {}", weight_.shape().to_string());
+    if (use_bias_ && input.shape().size() == 2 && input.device().type() == DeviceType::kCUDA)
+        return functional::linear(input, static_cast<const Tensor &>(weight_), static_cast<const Tensor &>(bias_));
     auto output = functional::mat_mul(input, static_cast<const Tensor &>(weight_));
     if (use_bias_)
         output = output + functional::broadcast_to(bias_, output.shape());  // src/nn/layers/linear.cpp:96-102
@@ -451,8 +453,18 @@ std::function<void(std::vector<Parameter *> &)> WeightDecay::hook() const
     return [rate](std::vector<Parameter *> &params) {
         NoGradGuard guard;
         for (auto *p : params)
-            if (p)
+        {
+            if (!p)
+                continue;
+            // grad += rate * param: one launch when both live on the device (the product is rounded, then added —
+            // what the separate multiply and accumulate give)
+            Tensor g = p->grad();
+            if (g.defined() && g.device().type() == DeviceType::kCUDA && g.dtype() == DataType::kFloat32 &&
+                g.shape() == p->shape())
+                static_cast<OriginMat &>(*g.impl_->data_).axpy_inplace(rate, *p->impl_->data_);
+            else
                 p->accumulate_grad(static_cast<const Tensor &>(*p) * Scalar(rate));
+        }
     };
 }
 
