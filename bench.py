@@ -237,6 +237,14 @@ def train_steps(steps, warmup, with_cpu):
     rc = h.odl_host_cnn_bench_graph(256, steps, warmup, 1, ms, loss)
     out["cnn_b256_sgd"].update({"graph_replay_rc": rc, "graph_replay_ms_per_step": float(ms[0]),
                                 "graph_replay_loss": float(loss[0])})
+    # the network of the reference's own conv_mnist example (with its BatchNorm layers, Adam + WeightDecay), batch 256;
+    # device only: the reference's BatchNorm operator cannot run backward
+    losses = np.zeros(3, np.float32)
+    rc = h.odl_host_cnn_bn_bench(256, steps, warmup, 0, ms, losses)
+    out["cnn_batchnorm_b256_adam"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss_before": float(losses[0]),
+                                      "loss_last_step": float(losses[1]), "loss_eval_mode": float(losses[2])}
+    rc = h.odl_host_cnn_bn_bench(256, steps, warmup, 1, ms, losses)
+    out["cnn_batchnorm_b256_adam"].update({"graph_replay_rc": rc, "graph_replay_ms_per_step": float(ms[0])})
     out["yolov5n_forward_4x3x320x320"] = yolo_forward(h, ol.ref() if with_cpu and ol.have_ref() else None, steps)
     if with_cpu and ol.have_ref():
         r = ol.ref()

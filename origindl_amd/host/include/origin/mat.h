@@ -296,6 +296,8 @@ public:
     std::unique_ptr<Mat> linear(const Mat &W, const Mat &b) const;
     // this += b*other, one launch (the weight-decay hook's multiply and accumulate)
     void axpy_inplace(float b, const Mat &other);
+    // this = a*this + b*other, written where this lies
+    void axpby_inplace(float a, float b, const Mat &other);
     // a*this + b*other in one launch (each product rounded before the sum): the running-statistics update of the
     // BatchNorm layers
     std::unique_ptr<Mat> axpby(float a, float b, const Mat &other) const;

@@ -734,6 +734,15 @@ std::unique_ptr<Mat> OriginMat::linear(const Mat &W_, const Mat &b_) const
     return y;
 }
 
+void OriginMat::axpby_inplace(float a, float b, const Mat &other)
+{
+    const OriginMat &x = dev_f32(*this, "axpby"), &y = dev_f32(other, "axpby");
+    if (x.shape() != y.shape())
+        THROW_INVALID_ARG("axpby: shape mismatch {} vs {}", x.shape().to_string(), y.shape().to_string());
+    float *p = const_cast<float *>(fp(x));
+    check(odl_hip_axpby(a, p, b, fp(y), (int64_t)elements(), p, cur()));
+}
+
 void OriginMat::axpy_inplace(float b, const Mat &other)
 {
     const OriginMat &x = dev_f32(*this, "axpy"), &y = dev_f32(other, "axpy");

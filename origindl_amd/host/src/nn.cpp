@@ -159,8 +159,17 @@ Tensor BatchNormBase::forward(const Tensor &input)
             const auto &r = static_cast<const OriginMat &>(*running.impl_->data_);
             return Tensor(r.axpby(momentum_, 1.0f - momentum_, *batch.impl_->data_));
         };
-        running_mean_ = fold(running_mean_, outs[1]);
-        running_var_ = fold(running_var_, outs[2]);
+        if (cuda::is_capturing())
+        {
+            // a recorded step must find the statistics at the same address on every replay
+            static_cast<OriginMat &>(*running_mean_.impl_->data_).axpby_inplace(momentum_, 1.0f - momentum_, *outs[1].impl_->data_);
+            static_cast<OriginMat &>(*running_var_.impl_->data_).axpby_inplace(momentum_, 1.0f - momentum_, *outs[2].impl_->data_);
+        }
+        else
+        {
+            running_mean_ = fold(running_mean_, outs[1]);
+            running_var_ = fold(running_var_, outs[2]);
+        }
     }
     return outs[0];
 }

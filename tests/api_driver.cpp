@@ -1102,6 +1102,53 @@ int DRV(cnn_bench)(int64_t N, int steps, int warmup, float *ms_per_step, float *
 }
 
 #ifdef DRV_ON_DEVICE
+// The network of the reference's own tests/example/mnist/conv_mnist.cpp:16-104 (conv 1->64, BatchNorm, ReLU, pool,
+// conv 64->128, BatchNorm, ReLU, pool, 6272->128->10) with its optimizer (Adam 1e-4 + WeightDecay), on a fixed
+// synthetic batch. Device build only: the reference cannot run this step (its BatchNorm operator throws in
+// backward). losses[0] / losses[1] = the loss before training and at the last step: training must bring it down;
+// losses[2] = the loss of an evaluation-mode forward afterwards (it uses the running statistics the steps folded).
+int DRV(cnn_bn_bench)(int64_t N, int steps, int warmup, int graph_mode, float *ms_per_step, float *losses)
+{
+    return guarded([&] {
+        std::mt19937 gen(777);
+        Sequential model;
+        model.add(std::make_unique<nn::Conv2d>(1, 64, 3, 1, 1, true));
+        model.add(std::make_unique<nn::BatchNorm2d>(64));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::MaxPool2d>(2, 2, 0));
+        model.add(std::make_unique<nn::Conv2d>(64, 128, 3, 1, 1, true));
+        model.add(std::make_unique<nn::BatchNorm2d>(128));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::MaxPool2d>(2, 2, 0));
+        model.add(std::make_unique<nn::Flatten>());
+        model.add(std::make_unique<nn::Linear>(7 * 7 * 128, 128, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::Linear>(128, 10, true));
+        *dynamic_cast<nn::Conv2d &>(model[0]).weight() = kaiming_uniform(gen, Shape{64, 1, 3, 3}, 9);
+        *dynamic_cast<nn::Conv2d &>(model[4]).weight() = kaiming_uniform(gen, Shape{128, 64, 3, 3}, 9 * 64);
+        *dynamic_cast<nn::Linear &>(model[9]).weight() = kaiming_uniform(gen, Shape{6272, 128}, 6272);
+        *dynamic_cast<nn::Linear &>(model[11]).weight() = kaiming_uniform(gen, Shape{128, 10}, 128);
+        model.to(kDev);
+        Adam opt(model, 1e-4f);
+        opt.register_hook(WeightDecay(1e-4f).hook());
+        auto X = Tensor(uniform_vec(gen, (size_t)(N * 28 * 28), 0.0f, 1.0f), Shape{(size_t)N, 1, 28, 28},
+                        dtype(DataType::kFloat32).device(kDev));
+        std::vector<int64_t> tv((size_t)N);
+        for (auto &e : tv)
+            e = (int64_t)(gen() % 10u);
+        auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt64).device(kDev));
+        model.train();
+        {
+            auto guard = no_grad();
+            losses[0] = F::softmax_cross_entropy(model(X), T).item<float>();
+        }
+        run_timed(model, opt, X, T, steps, warmup, graph_mode, ms_per_step, &losses[1]);
+        model.eval();
+        auto guard = no_grad();
+        losses[2] = F::softmax_cross_entropy(model(X), T).item<float>();
+    });
+}
+
 int DRV(mlp_bench_graph)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, int read_loss_each_step,
                          float *ms_per_step, float *loss)
 {

@@ -101,6 +101,7 @@ _DEVICE_ONLY_SIGS = {
     "odl_host_mlp_train_graph": _REF_SIGS["odl_ref_mlp_train"],
     "odl_host_mlp_bench_graph": "lllliiipp>i",
     "odl_host_cnn_bench_graph": "liiipp>i",
+    "odl_host_cnn_bn_bench": "liiipp>i",
     "odl_host_pnnx_forward_graph": _REF_SIGS["odl_ref_pnnx_forward"],
 }
 

@@ -231,6 +231,18 @@ def test_recorded_training_step_replays_bit_for_bit(h, wd):
                 assert np.array_equal(a, b), steps
 
 
+def test_reference_example_network_with_batch_norm_trains_and_replays(h):
+    """The network of the reference's tests/example/mnist/conv_mnist.cpp (two conv + BatchNorm + ReLU + pool blocks,
+    two Linear layers, Adam + WeightDecay) at batch 16: eight ordinary steps, and two ordinary steps followed by six
+    replays of a recorded step, must end with the same training loss and the same evaluation-mode loss (which depends
+    on the running statistics every step folded in) bit for bit; and training must reduce the loss."""
+    ms, eager, replayed = np.zeros(1, f32), np.zeros(3, f32), np.zeros(3, f32)
+    assert h.odl_host_cnn_bn_bench(16, 6, 2, 0, ms, eager) == 0
+    assert h.odl_host_cnn_bn_bench(16, 4, 2, 2, ms, replayed) == 0
+    assert eager[1] < eager[0] and np.isfinite(eager).all()
+    assert np.array_equal(eager, replayed), (eager, replayed)
+
+
 def test_cnn_training_step_matches_the_reference(h):
     names = ("Wc1", "bc1", "Wc2", "bc2", "Wl1", "bl1", "Wl2", "bl2")
     x, t = G["cnn_x"], G["cnn_t"]
