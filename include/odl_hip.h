@@ -254,6 +254,13 @@ int odl_hip_batch_norm_forward(const float *x, const float *gamma, const float *
 int odl_hip_batch_norm_backward(const float *gy, const float *gamma, const float *saved_var, const float *saved_x_norm,
                                 float eps, int64_t N, int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta,
                                 void *workspace, size_t workspace_bytes, void *stream);
+/* The same gradients from x and the saved statistics instead of a saved x_norm: the normalised value is formed again
+ * in the kernel, (x - mean) / sqrt(var + eps), the expression — and so the float — of the forward pass. A caller that
+ * keeps x anyway (an autograd operator does) need not store x_norm at all and calls the forward with x_norm = NULL. */
+int odl_hip_batch_norm_backward_from_x(const float *gy, const float *x, const float *gamma, const float *saved_mean,
+                                       const float *saved_var, float eps, int64_t N, int64_t C, int64_t P, float *gx,
+                                       float *dgamma, float *dbeta, void *workspace, size_t workspace_bytes,
+                                       void *stream);
 /* workspace of either call (partial channel sums) */
 size_t odl_hip_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t P);
 /* out = a*x + b*y, each product rounded before the sum: the running-statistics update of the BatchNorm layers

@@ -551,6 +551,20 @@ def batch_norm_backward(gy, gamma, saved_var, saved_x_norm, eps=1e-5):
     return gx, dg, db
 
 
+def batch_norm_backward_from_x(gy, x, gamma, saved_mean, saved_var, eps=1e-5):
+    """The same gradients from x and the saved statistics (x_norm formed again in the kernel) -> (gx, dgamma, dbeta)."""
+    for name, t in (("gy", gy), ("x", x), ("gamma", gamma), ("saved_mean", saved_mean), ("saved_var", saved_var)):
+        _chk(t, name)
+    N, C, P = _bn_dims(gy, "batch_norm_backward")
+    if x.shape != gy.shape or any(tuple(t.shape) != (C,) for t in (gamma, saved_mean, saved_var)):
+        raise OdlInvalidArgument("batch_norm_backward: shape mismatch")
+    gx, dg, db = _empty(gy.shape), _empty((C,)), _empty((C,))
+    ws, nb = _ws(lib().query("odl_hip_batch_norm_workspace_bytes", N, C, P))
+    lib().call("odl_hip_batch_norm_backward_from_x", _p(gy), _p(x), _p(gamma), _p(saved_mean), _p(saved_var), float(eps),
+               N, C, P, _p(gx), _p(dg), _p(db), _p(ws), nb, _stream())
+    return gx, dg, db
+
+
 def axpby(a, x, b, y):
     """a*x + b*y with each product rounded first: the running-statistics update of the BatchNorm layers
     (src/nn/layers/batch_norm2d.cpp:77-80)."""

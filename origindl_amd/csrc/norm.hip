@@ -176,23 +176,36 @@ __global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float *__restric
     });
 }
 
-template <bool V4>
+// FROM_X: `xn` holds x itself and the normalised value is formed here, (x - mean) / sqrt(var + eps) — the expression
+// the forward pass used, so the same float — instead of being read back from a saved copy.
+template <bool V4, bool FROM_X>
 __global__ __launch_bounds__(kBlock) void bn_bwd_sums_kernel(const float *__restrict__ gy, const float *__restrict__ xn,
+                                                              const float *__restrict__ mean,
+                                                              const float *__restrict__ var, float eps,
                                                               float *__restrict__ part, BnGeom g)
 {
+    const float mu = FROM_X ? mean[blockIdx.y] : 0.f;
+    const float sd = FROM_X ? sqrtf(var[blockIdx.y] + eps) : 1.f;
     float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
     visit_chunk<V4>(g, [&](int64_t off, int j) {
         if (V4)
         {
             const f32x4 q = *reinterpret_cast<const f32x4 *>(gy + off);
-            const f32x4 r = *reinterpret_cast<const f32x4 *>(xn + off);
+            f32x4 r = *reinterpret_cast<const f32x4 *>(xn + off);
+            if (FROM_X)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    r[i] = (r[i] - mu) / sd;
+            }
             a[j] += (q[0] + q[1]) + (q[2] + q[3]);
             b[j] += (q[0] * r[0] + q[1] * r[1]) + (q[2] * r[2] + q[3] * r[3]);
         }
         else
         {
+            const float r = FROM_X ? (xn[off] - mu) / sd : xn[off];
             a[j] += gy[off];
-            b[j] += gy[off] * xn[off];
+            b[j] += gy[off] * r;
         }
     });
     const float sa = block_sum_all((a[0] + a[1]) + (a[2] + a[3]));
@@ -204,29 +217,34 @@ __global__ __launch_bounds__(kBlock) void bn_bwd_sums_kernel(const float *__rest
     }
 }
 
-template <bool V4>
+template <bool V4, bool FROM_X>
 __global__ __launch_bounds__(kBlock) void bn_bwd_apply_kernel(const float *__restrict__ gy, const float *__restrict__ xn,
                                                                const float *__restrict__ gamma,
+                                                               const float *__restrict__ mean,
                                                                const float *__restrict__ var,
                                                                const float *__restrict__ part, float *__restrict__ gx,
                                                                float *__restrict__ dgamma, float *__restrict__ dbeta,
                                                                BnGeom g, float count, float eps)
 {
     const unsigned c = blockIdx.y;
+    const float mu = FROM_X ? mean[c] : 0.f;
+    const float sd = sqrtf(var[c] + eps);
     const float sum_gy = channel_total(part, c, g.ns, 2, 0), sum_gy_xn = channel_total(part, c, g.ns, 2, 1);
     if (blockIdx.x == 0 && threadIdx.x == 0)
         dgamma[c] = sum_gy_xn, dbeta[c] = sum_gy;
     const float mean_gy = sum_gy / count, mean_gy_xn = sum_gy_xn / count;
-    const float scale = gamma[c] / sqrtf(var[c] + eps);
+    const float scale = gamma[c] / sd;
     visit_chunk<V4>(g, [&](int64_t off, int) {
         if (V4)
         {
             const f32x4 q = *reinterpret_cast<const f32x4 *>(gy + off);
-            const f32x4 r = *reinterpret_cast<const f32x4 *>(xn + off);
+            f32x4 r = *reinterpret_cast<const f32x4 *>(xn + off);
             f32x4 o;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
             {
+                if (FROM_X)
+                    r[i] = (r[i] - mu) / sd;
                 const float t = r[i] * mean_gy_xn;
                 o[i] = scale * ((q[i] - mean_gy) - t);
             }
@@ -234,7 +252,8 @@ __global__ __launch_bounds__(kBlock) void bn_bwd_apply_kernel(const float *__res
         }
         else
         {
-            const float t = xn[off] * mean_gy_xn;
+            const float r = FROM_X ? (xn[off] - mu) / sd : xn[off];
+            const float t = r * mean_gy_xn;
             gx[off] = scale * ((gy[off] - mean_gy) - t);
         }
     });
@@ -347,15 +366,16 @@ int odl_hip_batch_norm_forward(const float *x, const float *gamma, const float *
     return ODL_OK;
 }
 
-int odl_hip_batch_norm_backward(const float *gy, const float *gamma, const float *saved_var, const float *saved_x_norm,
-                                float eps, int64_t N, int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta,
-                                void *workspace, size_t workspace_bytes, void *stream)
+static int bn_backward_launch(const float *gy, const float *gamma, const float *saved_mean, const float *saved_var,
+                              const float *xn_or_x, bool from_x, float eps, int64_t N, int64_t C, int64_t P, float *gx,
+                              float *dgamma, float *dbeta, void *workspace, size_t workspace_bytes, void *stream)
 {
     ODL_REQUIRE_DEVICE();
     BnGeom g;
     ODL_REQUIRE(plan_bn(N, C, P, g), "batch_norm_backward: bad shape (N=%lld, C=%lld, P=%lld)", (long long)N,
                 (long long)C, (long long)P);
-    ODL_REQUIRE(gy && gamma && saved_var && saved_x_norm && gx && dgamma && dbeta, "batch_norm_backward: null operand");
+    ODL_REQUIRE(gy && gamma && saved_var && xn_or_x && gx && dgamma && dbeta && (!from_x || saved_mean),
+                "batch_norm_backward: null operand");
     hipStream_t st = odl::as_stream(stream);
     if (N == 0)  // nothing to sum: the parameter gradients are zero (batch_norm.cpp:337-339)
     {
@@ -366,24 +386,51 @@ int odl_hip_batch_norm_backward(const float *gy, const float *gamma, const float
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
                 "batch_norm_backward: workspace of %zu bytes required, got %zu", need, workspace_bytes);
     float *part = static_cast<float *>(workspace);
-    const bool v4 = P % 4 == 0 && aligned16(gy) && aligned16(saved_x_norm) && aligned16(gx);
+    const bool v4 = P % 4 == 0 && aligned16(gy) && aligned16(xn_or_x) && aligned16(gx);
     g.by_plane = odl::make_fastdiv((unsigned)(v4 ? P / 4 : P));
     const dim3 grid(g.ns, g.C), block(kBlock);
     const float count = (float)(N * P);
-    if (v4)
+#define ODL_BN_BWD(V4, FX)                                                                                          \
+    hipLaunchKernelGGL((bn_bwd_sums_kernel<V4, FX>), grid, block, 0, st, gy, xn_or_x, saved_mean, saved_var, eps, part, \
+                       g);                                                                                          \
+    hipLaunchKernelGGL((bn_bwd_apply_kernel<V4, FX>), grid, block, 0, st, gy, xn_or_x, gamma, saved_mean, saved_var,    \
+                       part, gx, dgamma, dbeta, g, count, eps)
+    if (v4 && from_x)
     {
-        hipLaunchKernelGGL((bn_bwd_sums_kernel<true>), grid, block, 0, st, gy, saved_x_norm, part, g);
-        hipLaunchKernelGGL((bn_bwd_apply_kernel<true>), grid, block, 0, st, gy, saved_x_norm, gamma, saved_var, part, gx,
-                           dgamma, dbeta, g, count, eps);
+        ODL_BN_BWD(true, true);
+    }
+    else if (v4)
+    {
+        ODL_BN_BWD(true, false);
+    }
+    else if (from_x)
+    {
+        ODL_BN_BWD(false, true);
     }
     else
     {
-        hipLaunchKernelGGL((bn_bwd_sums_kernel<false>), grid, block, 0, st, gy, saved_x_norm, part, g);
-        hipLaunchKernelGGL((bn_bwd_apply_kernel<false>), grid, block, 0, st, gy, saved_x_norm, gamma, saved_var, part, gx,
-                           dgamma, dbeta, g, count, eps);
+        ODL_BN_BWD(false, false);
     }
+#undef ODL_BN_BWD
     ODL_LAUNCH_CHECK();
     return ODL_OK;
+}
+
+int odl_hip_batch_norm_backward(const float *gy, const float *gamma, const float *saved_var, const float *saved_x_norm,
+                                float eps, int64_t N, int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta,
+                                void *workspace, size_t workspace_bytes, void *stream)
+{
+    return bn_backward_launch(gy, gamma, nullptr, saved_var, saved_x_norm, false, eps, N, C, P, gx, dgamma, dbeta,
+                              workspace, workspace_bytes, stream);
+}
+
+int odl_hip_batch_norm_backward_from_x(const float *gy, const float *x, const float *gamma, const float *saved_mean,
+                                       const float *saved_var, float eps, int64_t N, int64_t C, int64_t P, float *gx,
+                                       float *dgamma, float *dbeta, void *workspace, size_t workspace_bytes,
+                                       void *stream)
+{
+    return bn_backward_launch(gy, gamma, saved_mean, saved_var, x, true, eps, N, C, P, gx, dgamma, dbeta, workspace,
+                              workspace_bytes, stream);
 }
 
 int odl_hip_axpby(float a, const float *x, float b, const float *y, int64_t n, float *out, void *stream)

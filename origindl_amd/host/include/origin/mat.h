@@ -289,6 +289,13 @@ public:
     // overwrites this tensor's elements with another's of the same shape (a device-to-device copy on the current
     // stream): how a recorded step stores a freshly computed tensor at the address later replays read it from
     void copy_from(const Mat &src);
+    // Batch norm for an operator that keeps x anyway: the forward without the x_norm output (result.x_norm is null),
+    // and the backward that forms x_norm again from x (this) and the saved statistics — the same floats, 4 bytes per
+    // element less written in forward and one saved activation less.
+    BatchNormResult batch_norm_forward_no_xnorm(const Mat &gamma, const Mat &beta, const Mat &running_mean,
+                                                const Mat &running_var, bool training, float eps, int num_dims) const;
+    std::vector<std::unique_ptr<Mat>> batch_norm_backward_from_x(const Mat &gy, const Mat &gamma, const Mat &saved_mean,
+                                                                 const Mat &saved_var, float eps, int num_dims) const;
     // gy (this) times the mask x > 0, in one launch: the two kernels of ReLU::backward, same products
     std::unique_ptr<Mat> relu_backward(const Mat &x) const;
     // x (this) . W + b with the bias added in the product's epilogue: the three kernels of Linear::forward

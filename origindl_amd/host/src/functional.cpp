@@ -464,7 +464,7 @@ struct BatchNorm : Operator  // src/operators/normalization/batch_norm.cpp:16-12
     bool training;
     float eps, momentum;
     int num_dims;
-    Tensor saved_mean, saved_var, saved_x_norm;
+    Tensor saved_mean, saved_var;  // x_norm is not kept: backward forms it again from x and these two (same floats)
     BatchNorm(bool t, float e, float m, int nd) : training(t), eps(e), momentum(m), num_dims(nd) {}
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
@@ -472,17 +472,11 @@ struct BatchNorm : Operator  // src/operators/normalization/batch_norm.cpp:16-12
             THROW_RUNTIME_ERROR("BatchNorm operator requires exactly 5 inputs (x, gamma, beta, running_mean, "
                                 "running_var), but got {}", xs.size());
         Tensor y;
-        if (xs[0].requires_grad() || xs[1].requires_grad() || xs[2].requires_grad())
+        if (training || xs[0].requires_grad() || xs[1].requires_grad() || xs[2].requires_grad())
         {
-            auto r = mat(xs[0]).batch_norm_forward(mat(xs[1]), mat(xs[2]), mat(xs[3]), mat(xs[4]), training, eps, num_dims);
-            y = wrap(std::move(r.y));
-            saved_mean = wrap(std::move(r.mean)), saved_var = wrap(std::move(r.var));
-            saved_x_norm = wrap(std::move(r.x_norm));
-        }
-        else if (training)
-        {
-            // the layers read the batch statistics off the operator's outputs, so they are computed here too
-            auto r = mat(xs[0]).batch_norm_forward(mat(xs[1]), mat(xs[2]), mat(xs[3]), mat(xs[4]), training, eps, num_dims);
+            // in training mode the layers read the batch statistics off the operator's outputs even without a graph
+            auto r = omat(xs[0]).batch_norm_forward_no_xnorm(mat(xs[1]), mat(xs[2]), mat(xs[3]), mat(xs[4]), training, eps,
+                                                             num_dims);
             y = wrap(std::move(r.y));
             saved_mean = wrap(std::move(r.mean)), saved_var = wrap(std::move(r.var));
         }
@@ -495,8 +489,8 @@ struct BatchNorm : Operator  // src/operators/normalization/batch_norm.cpp:16-12
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
         // the gradient of y only: the statistics outputs feed the running averages, outside the graph
-        auto r = mat(inputs_[0]).batch_norm_backward(mat(gys[0]), mat(inputs_[1]), mat(saved_mean), mat(saved_var),
-                                                     mat(saved_x_norm), eps, num_dims);
+        auto r = omat(inputs_[0]).batch_norm_backward_from_x(mat(gys[0]), mat(inputs_[1]), mat(saved_mean), mat(saved_var),
+                                                             eps, num_dims);
         const auto opt = dtype(DataType::kFloat32).device(inputs_[0].device());
         return {wrap(std::move(r[0])), wrap(std::move(r[1])), wrap(std::move(r[2])), Tensor::zeros(inputs_[3].shape(), opt),
                 Tensor::zeros(inputs_[4].shape(), opt)};

@@ -668,6 +668,51 @@ Mat::BatchNormResult OriginMat::batch_norm_forward(const Mat &gamma, const Mat &
     return r;
 }
 
+Mat::BatchNormResult OriginMat::batch_norm_forward_no_xnorm(const Mat &gamma, const Mat &beta, const Mat &running_mean,
+                                                            const Mat &running_var, bool training, float eps,
+                                                            int num_dims) const
+{
+    const BnShape s = bn_check("batch_norm", *this, num_dims, gamma, beta, running_mean, running_var);
+    const OriginMat &x = dev_f32(*this, "batch_norm");
+    const OriginMat &g = dev_f32(gamma, "batch_norm"), &b = dev_f32(beta, "batch_norm");
+    const OriginMat &rm = dev_f32(running_mean, "batch_norm"), &rv = dev_f32(running_var, "batch_norm");
+    BatchNormResult r;
+    auto y = new_like(x, shape_);
+    auto mean = new_like(x, Shape({(size_t)s.C})), var = new_like(x, Shape({(size_t)s.C}));
+    Workspace ws(training ? odl_hip_batch_norm_workspace_bytes(s.N, s.C, s.P) : 0, device().index());
+    check(odl_hip_batch_norm_forward(fp(x), fp(g), fp(b), fp(rm), fp(rv), training ? 1 : 0, eps, s.N, s.C, s.P,
+                                     y->data_ptr<float>(), mean->data_ptr<float>(), var->data_ptr<float>(), nullptr,
+                                     ws.ptr(), ws.bytes, cur()));
+    r.y = std::move(y), r.mean = std::move(mean), r.var = std::move(var);
+    return r;
+}
+
+std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward_from_x(const Mat &gym, const Mat &gamma,
+                                                                        const Mat &saved_mean, const Mat &saved_var,
+                                                                        float eps, int num_dims) const
+{
+    if (shape_.size() != (size_t)num_dims || (num_dims != 2 && num_dims != 4))
+        THROW_INVALID_ARG("batch_norm_backward: x must have {} dimensions (2 or 4), but got shape {}", num_dims,
+                          shape_.to_string());
+    const size_t C = shape_[1];
+    if (gym.shape() != shape_ || gamma.shape() != Shape({C}) || saved_mean.shape() != Shape({C}) ||
+        saved_var.shape() != Shape({C}))
+        THROW_INVALID_ARG("batch_norm_backward: shape mismatch");
+    const OriginMat &x = dev_f32(*this, "batch_norm_backward");
+    const OriginMat &gy = dev_f32(gym, "batch_norm_backward"), &g = dev_f32(gamma, "batch_norm_backward");
+    const OriginMat &sm = dev_f32(saved_mean, "batch_norm_backward"), &sv = dev_f32(saved_var, "batch_norm_backward");
+    const int64_t N = (int64_t)shape_[0], P = num_dims == 4 ? (int64_t)(shape_[2] * shape_[3]) : 1;
+    auto gx = new_like(x, shape_);
+    auto dgamma = new_like(x, Shape({C})), dbeta = new_like(x, Shape({C}));
+    Workspace ws(odl_hip_batch_norm_workspace_bytes(N, (int64_t)C, P), device().index());
+    check(odl_hip_batch_norm_backward_from_x(fp(gy), fp(x), fp(g), fp(sm), fp(sv), eps, N, (int64_t)C, P,
+                                             gx->data_ptr<float>(), dgamma->data_ptr<float>(), dbeta->data_ptr<float>(),
+                                             ws.ptr(), ws.bytes, cur()));
+    std::vector<std::unique_ptr<Mat>> outs;
+    outs.push_back(std::move(gx)), outs.push_back(std::move(dgamma)), outs.push_back(std::move(dbeta));
+    return outs;
+}
+
 std::unique_ptr<Mat> OriginMat::batch_norm(const Mat &gamma, const Mat &beta, const Mat &running_mean,
                                            const Mat &running_var, bool training, float eps, float, int num_dims) const
 {

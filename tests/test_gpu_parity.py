@@ -762,6 +762,11 @@ def test_batch_norm_vs_oracle_at_cnn_sizes(api, o):
         np.testing.assert_allclose(host(db), wdb, rtol=0, atol=bound * np.sqrt(N * P))
         np.testing.assert_allclose(host(dg), wdg, rtol=0, atol=bound * np.sqrt(N * P))
         np.testing.assert_allclose(host(gx), wgx, rtol=1e-4, atol=1e-5)
+        # the backward that forms x_norm again from x and the statistics gives the same bits as the one reading the
+        # saved x_norm of the same forward
+        gx1, dg1, db1 = api.batch_norm_backward(dev(gy), dev(gamma), var, xn)
+        gx2, dg2, db2 = api.batch_norm_backward_from_x(dev(gy), dev(x), dev(gamma), mean, var)
+        assert all(np.array_equal(host(a), host(b)) for a, b in ((gx1, gx2), (dg1, dg2), (db1, db2))), shape
     # evaluation mode has no reduction: bit-exact against the oracle at any size
     x = rng.standard_normal((16, 64, 14, 14), dtype=f32)
     gamma, beta, rm = (rng.standard_normal(64, dtype=f32) for _ in range(3))
