@@ -169,6 +169,52 @@ __global__ __launch_bounds__(256) void max_pool_bwd_plane_kernel(const float *__
     }
 }
 
+// Windows that tile the image exactly (stride = window, no padding, H = OH*K, W = OW*K — the 2x2/2 pooling of the
+// networks on this path): every input cell belongs to one window, so the gradient is written from the output's side.
+// A thread owns one pooled output: it reads its index and its gradient (two independent, coalesced loads — the
+// gather kernel above chains the index load and the gradient load, and with one cell per thread that chain is all a
+// wave ever does) and writes the K x K cells of its window, gy at the indexed cell and zero elsewhere. The stored
+// values are the gather kernel's: 0.f + gy, or 0.f.
+template <int K>
+__global__ __launch_bounds__(256) void max_pool_bwd_tiled_kernel(const float *__restrict__ gy,
+                                                                 const uint64_t *__restrict__ idx,
+                                                                 float *__restrict__ gx, unsigned total, int OW,
+                                                                 unsigned oplane)
+{
+    const unsigned o = blockIdx.x * 256u + threadIdx.x;
+    if (o >= total)
+        return;
+    const int hit = (int)idx[o];  // the reference decodes the index with int arithmetic (max_pool2d.cpp:203-205)
+    const float v = 0.f + gy[o];
+    const unsigned nc = o / oplane, r = o - nc * oplane;
+    const int oh = (int)(r / (unsigned)OW), ow = (int)r - oh * OW;
+    const int W = OW * K;
+    float *dst = gx + ((int64_t)nc * oplane * (K * K)) + (int64_t)(oh * K) * W + ow * K;
+#pragma unroll
+    for (int kh = 0; kh < K; ++kh)
+    {
+        if (K == 2)
+        {
+            float2 row;
+            row.x = hit == kh * K ? v : 0.f;
+            row.y = hit == kh * K + 1 ? v : 0.f;
+            *reinterpret_cast<float2 *>(dst + kh * W) = row;  // W and the window start are even: 8-byte aligned
+        }
+        else
+        {
+#pragma unroll
+            for (int kw = 0; kw < K; ++kw)
+                dst[kh * W + kw] = hit == kh * K + kw ? v : 0.f;
+        }
+    }
+}
+
+bool tiles_exactly(const PoolGeom &g)
+{
+    return g.KH == g.KW && g.SH == g.KH && g.SW == g.KW && g.PH == 0 && g.PW == 0 && g.H == g.OH * g.KH &&
+           g.W == g.OW * g.KW && (g.KH == 2 || g.KH == 3);
+}
+
 // the 32-bit kernels take everything whose element counts fit
 bool plane_ok(const PoolGeom &g)
 {
@@ -250,7 +296,18 @@ int odl_hip_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N,
     if (total == 0)
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
-    if (plane_ok(g))
+    if (plane_ok(g) && tiles_exactly(g) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0)
+    {
+        const unsigned outputs = (unsigned)(N * C * g.OH * g.OW);
+        const dim3 grid((unsigned)odl::ceil_div((int64_t)outputs, 256));
+        if (g.KH == 2)
+            hipLaunchKernelGGL((max_pool_bwd_tiled_kernel<2>), grid, dim3(256), 0, st, gy, idx, gx, outputs, (int)g.OW,
+                               (unsigned)(g.OH * g.OW));
+        else
+            hipLaunchKernelGGL((max_pool_bwd_tiled_kernel<3>), grid, dim3(256), 0, st, gy, idx, gx, outputs, (int)g.OW,
+                               (unsigned)(g.OH * g.OW));
+    }
+    else if (plane_ok(g))
     {
         const dim3 grid = plane_grid(H * W, N * C);
         ODL_POOL_DISPATCH(max_pool_bwd_plane_kernel, gy, idx, gx, g);

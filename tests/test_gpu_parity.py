@@ -527,6 +527,21 @@ def test_max_pool_cnn_shapes_vs_oracle_bit_exact(api, o):
         yd, idxd = api.max_pool2d(dev(x), 2, 2, 0)
         assert np.array_equal(host(yd), y) and np.array_equal(host(idxd).view(np.uint64), idx)
         assert np.array_equal(host(api.max_pool2d_backward(dev(gy), idxd, x.shape, 2, 2, 0)), gx)
+    # windows that tile the image exactly take the output-side backward kernel (2x2/2 above, 3x3/3 here), everything
+    # else the gather (an odd size whose last row and column no window covers; overlapping windows); gradients with
+    # negative zeros keep their sign rules (0.f + -0.f = +0.f in both)
+    for N, C, H, W, K, S in ((3, 5, 9, 12, 3, 3), (2, 4, 9, 9, 2, 2), (2, 3, 8, 8, 3, 2), (1, 2, 6, 6, 2, 2)):
+        x = np.maximum(rng.standard_normal((N, C, H, W), dtype=f32), 0)
+        OH, OW = (H - K) // S + 1, (W - K) // S + 1
+        y, idx = np.empty((N, C, OH, OW), f32), np.empty((N, C, OH, OW), np.uint64)
+        assert o.orc_max_pool2d(x, N, C, H, W, K, K, S, S, 0, 0, y, idx) == 0
+        gy = rng.standard_normal(y.shape, dtype=f32)
+        gy.ravel()[::7] = -0.0
+        gx = np.empty_like(x)
+        assert o.orc_max_pool2d_backward(gy, idx, N, C, H, W, K, K, S, S, 0, 0, gx) == 0
+        yd, idxd = api.max_pool2d(dev(x), K, S, 0)
+        got = host(api.max_pool2d_backward(dev(gy), idxd, x.shape, K, S, 0))
+        assert np.array_equal(got, gx) and np.array_equal(np.signbit(got), np.signbit(gx)), (N, C, H, W, K, S)
     # tests/unit_test/operator/test_max_pool2d.cpp:20-45
     y, _ = api.max_pool2d(dev(np.arange(1, 17, dtype=f32).reshape(1, 1, 4, 4)), 2, 2, 0)
     assert host(y).ravel().tolist() == [6, 8, 14, 16]
