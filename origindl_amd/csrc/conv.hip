@@ -37,6 +37,23 @@ int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, i
 int conv_implicit_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W,
                         int64_t OC, int KH, int KW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
                         size_t workspace_bytes, hipStream_t st);
+// the first layer of an image network (1 or 3 input channels): direct kernels, one thread per pixel (conv_small.hip)
+bool conv_small_forward_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
+int conv_small_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H, int64_t W,
+                       int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW, int act,
+                       hipStream_t st);
+bool conv_small_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
+                         int64_t OW);
+size_t conv_small_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
+int conv_small_wgrad(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                     int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
+                     size_t workspace_bytes, hipStream_t st);
+bool conv_small_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
+                         int64_t OW);
+size_t conv_small_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW);
+int conv_small_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                     int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
+                     size_t workspace_bytes, hipStream_t st);
 int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
                              size_t workspace_bytes, hipStream_t st);
 size_t sum_nchw_channels_workspace(int64_t N, int64_t OC, int64_t P);
@@ -802,6 +819,8 @@ size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W
     const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
     if (OH <= 0 || OW <= 0)
         return 0;
+    if (odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, OH, OW))
+        return 0;
     if (odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW))
         return align256(odl::conv_implicit_forward_workspace(N, C, H, W, OC, KH, KW, OH, OW));  // no im2col matrix; K-slice
                                                                                           // partials for small outputs
@@ -825,6 +844,8 @@ int odl_hip_conv2d_act(const float *x, const float *w, const float *b, int64_t N
     if (M == 0)
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
+    if (odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, g.OH, g.OW))
+        return odl::conv_small_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, act, st);
     if (odl::conv_implicit_forward_ok(w, N, C, H, W, OC, KH, KW, g.OH, g.OW))
         return odl::conv_implicit_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, act, workspace,
                                           workspace_bytes, st);
@@ -852,6 +873,7 @@ namespace
 // workspace regions of conv2d_backward, in order: [col][split-K partials][permuted weights][bias partials]
 struct BwdPlan
 {
+    bool wgrad_small, dgrad_small;  // few input channels: the direct kernels, no matrices at all
     bool wgrad_implicit, dgrad_implicit;
     size_t col_bytes, splitk_bytes, wp_bytes, red_bytes;
     size_t total() const { return col_bytes + splitk_bytes + wp_bytes + red_bytes; }
@@ -862,12 +884,18 @@ BwdPlan plan_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t 
 {
     BwdPlan p{};
     const int64_t M = N * OH * OW, K = C * KH * KW;
-    p.wgrad_implicit = odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
-    p.dgrad_implicit = odl::conv_implicit_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW);
-    p.col_bytes = (p.wgrad_implicit && p.dgrad_implicit) ? 0 : align256((size_t)(M * K) * sizeof(float));
-    p.splitk_bytes = align256(p.wgrad_implicit ? odl::conv_implicit_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
-                                               : odl::sgemm_workspace(OC, K, M, 0));
-    p.wp_bytes = p.dgrad_implicit ? align256(odl::conv_implicit_dgrad_workspace(C, OC, KH, KW, N * H * W)) : 0;
+    p.wgrad_small = odl::conv_small_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
+    p.dgrad_small = odl::conv_small_dgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
+    p.wgrad_implicit = !p.wgrad_small && odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
+    p.dgrad_implicit = !p.dgrad_small && odl::conv_implicit_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW);
+    const bool no_col = (p.wgrad_small || p.wgrad_implicit) && (p.dgrad_small || p.dgrad_implicit);
+    p.col_bytes = no_col ? 0 : align256((size_t)(M * K) * sizeof(float));
+    p.splitk_bytes = align256(p.wgrad_small      ? odl::conv_small_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
+                              : p.wgrad_implicit ? odl::conv_implicit_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
+                                                 : odl::sgemm_workspace(OC, K, M, 0));
+    p.wp_bytes = p.dgrad_small      ? align256(odl::conv_small_dgrad_workspace(C, OC, KH, KW))
+                 : p.dgrad_implicit ? align256(odl::conv_implicit_dgrad_workspace(C, OC, KH, KW, N * H * W))
+                                    : 0;
     p.red_bytes = align256(odl::sum_nchw_channels_workspace(N, OC, OH * OW));
     return p;
 }
@@ -911,7 +939,10 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
     // gy2d: gy's NCHW buffer read as a row-major [M, OC] matrix exactly as it lies (conv2d.cpp:548)
     if (gw)
     {
-        if (p.wgrad_implicit)
+        if (p.wgrad_small)
+            rc = odl::conv_small_wgrad(gy, x, gw, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, splitk_ws,
+                                       p.splitk_bytes, st);
+        else if (p.wgrad_implicit)
             rc = odl::conv_implicit_wgrad(gy, x, gw, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, splitk_ws,
                                           p.splitk_bytes, st);
         else
@@ -932,7 +963,9 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
     }
     if (gx)
     {
-        if (p.dgrad_implicit)
+        if (p.dgrad_small)
+            rc = odl::conv_small_dgrad(gy, w, gx, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, wp_ws, p.wp_bytes, st);
+        else if (p.dgrad_implicit)
             rc = odl::conv_implicit_dgrad(gy, w, gx, N, C, H, W, OC, KH, KW, PH, PW, g.OH, g.OW, wp_ws, p.wp_bytes, st);
         else
         {

@@ -1,0 +1,396 @@
+// Convolutions over an image with very few channels — the first layer of an image network (1 or 3 channels under a
+// 3x3 to 6x6 window). Their GEMM has a reduction of 9 to 27 terms (or, for the input gradient, 1 to 3 output rows): a
+// 64- or 128-row MFMA tile would spend nearly all of its multiplies on padding, and the im2col matrix would be written
+// and read for nothing. Here one thread owns one pixel and walks the few terms itself on the vector ALU; the filter is
+// read through wave-uniform addresses, so it lives in scalar registers, and the kernels move the activations exactly
+// once. Results follow src/mat/origin/cpu/conv/conv2d.cpp:404-599 like the GEMM path does: the output gradient is read
+// as the row-major [N*OH*OW, OC] matrix that its NCHW buffer spells out as it lies (conv2d.cpp:548).
+#include "odl_common.h"
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace
+{
+struct SmallGeom
+{
+    int N, C, H, W, OC, OH, OW, SH, SW, PH, PW;
+    unsigned total;            // pixels the grid covers: N*OH*OW (forward, weight gradient) or N*H*W (input gradient)
+    odl::FastDiv by_w, by_h;   // the pixel decode: by (OW, OH) or by (W, H)
+};
+
+constexpr int kThreads = 256;
+
+// y[n][oc][oh][ow] = act(sum_{c,kh,kw} x[n][c][oh*SH-PH+kh][ow*SW-PW+kw] * w[oc][c][kh][kw] + b[oc]); one thread per
+// output pixel, OCB output channels per thread (blockIdx.y picks the group). The KH*KW window of one input channel is
+// held in registers and reused by all OCB channels.
+template <int KH, int KW, int OCB>
+__global__ __launch_bounds__(kThreads) void conv_small_fwd_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                                 const float *__restrict__ bias, float *__restrict__ y,
+                                                                 SmallGeom g, int act)
+{
+    const unsigned pix = blockIdx.x * kThreads + threadIdx.x;
+    if (pix >= g.total)
+        return;
+    const unsigned t = odl::fastdiv(pix, g.by_w), ow = pix - t * g.OW;
+    const unsigned n = odl::fastdiv(t, g.by_h), oh = t - n * g.OH;
+    const int oc0 = blockIdx.y * OCB;
+    const int ih0 = (int)oh * g.SH - g.PH, iw0 = (int)ow * g.SW - g.PW;
+    float acc[OCB];
+#pragma unroll
+    for (int o = 0; o < OCB; ++o)
+        acc[o] = 0.f;
+    for (int c = 0; c < g.C; ++c)
+    {
+        const float *xp = x + ((size_t)n * g.C + c) * g.H * g.W;
+        float xr[KH * KW];
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < KW; ++kw)
+            {
+                const int ih = ih0 + kh, iw = iw0 + kw;
+                const bool in = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+                xr[kh * KW + kw] = in ? xp[ih * g.W + iw] : 0.f;
+            }
+        const float *wc = w + ((size_t)oc0 * g.C + c) * (KH * KW);
+#pragma unroll
+        for (int o = 0; o < OCB; ++o)
+        {
+            const float *wo = wc + (size_t)o * g.C * (KH * KW);  // the same address in every lane
+#pragma unroll
+            for (int j = 0; j < KH * KW; ++j)
+                acc[o] = fmaf(xr[j], wo[j], acc[o]);
+        }
+    }
+    const size_t plane = (size_t)g.OH * g.OW;
+    float *yp = y + ((size_t)n * g.OC + oc0) * plane + (size_t)oh * g.OW + ow;
+#pragma unroll
+    for (int o = 0; o < OCB; ++o)
+    {
+        float v = acc[o];
+        if (bias)
+            v = v + bias[oc0 + o];
+        yp[o * plane] = odl::apply_act(v, act);
+    }
+}
+
+// gW[oc][k] = sum_m gy2d[m][oc] * col[m][k], col[m][(c,kh,kw)] = x[n][c][oh*SH-PH+kh][ow*SW-PW+kw] for m = (n,oh,ow).
+// A thread owns 8 consecutive channels of gy2d's rows m = first + i*rows_per_pass and all K = C*KH*KW columns: 8*K
+// private sums. G = OC/8 neighbouring lanes share a row, so a wave reads whole rows of gy2d, 16 bytes a lane. At the
+// end the lanes of equal channel group are added across the wave, the four waves across the workgroup, and the
+// workgroup writes one [OC][K] partial; conv_small_partial_sum_kernel adds the partials in a fixed order.
+template <int C, int KH, int KW>
+__global__ __launch_bounds__(kThreads) void conv_small_wgrad_kernel(const float *__restrict__ gy, const float *__restrict__ x,
+                                                                   float *__restrict__ part, SmallGeom g, int lgG,
+                                                                   unsigned rows_per_block)
+{
+    constexpr int K = C * KH * KW;
+    extern __shared__ float red[];  // [4][OC*K]
+    const int G = 1 << lgG;
+    const int ocg = threadIdx.x & (G - 1);
+    const unsigned rows_per_pass = kThreads >> lgG;
+    const unsigned m_begin = blockIdx.x * rows_per_block;
+    const unsigned m_end = (m_begin + rows_per_block < g.total) ? m_begin + rows_per_block : g.total;
+    float acc[8][K];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < K; ++j)
+            acc[i][j] = 0.f;
+    for (unsigned m = m_begin + (threadIdx.x >> lgG); m < m_end; m += rows_per_pass)
+    {
+        const unsigned t = odl::fastdiv(m, g.by_w), ow = m - t * g.OW;
+        const unsigned n = odl::fastdiv(t, g.by_h), oh = t - n * g.OH;
+        const int ih0 = (int)oh * g.SH - g.PH, iw0 = (int)ow * g.SW - g.PW;
+        const float *xp = x + (size_t)n * C * g.H * g.W;
+        float xr[K];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int kh = 0; kh < KH; ++kh)
+#pragma unroll
+                for (int kw = 0; kw < KW; ++kw)
+                {
+                    const int ih = ih0 + kh, iw = iw0 + kw;
+                    const bool in = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+                    xr[(c * KH + kh) * KW + kw] = in ? xp[((size_t)c * g.H + ih) * g.W + iw] : 0.f;
+                }
+        const f32x4 *gp = reinterpret_cast<const f32x4 *>(gy + (size_t)m * g.OC + ocg * 8);
+        const f32x4 g0 = gp[0], g1 = gp[1];
+        const float gv[8] = {g0[0], g0[1], g0[2], g0[3], g1[0], g1[1], g1[2], g1[3]};
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < K; ++j)
+                acc[i][j] = fmaf(gv[i], xr[j], acc[i][j]);
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int EK = g.OC * K;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < K; ++j)
+        {
+            float v = acc[i][j];
+            for (int off = G; off < 64; off <<= 1)
+                v += __shfl_xor(v, off);
+            if (lane < G)
+                red[wave * EK + (ocg * 8 + i) * K + j] = v;
+        }
+    __syncthreads();
+    float *out = part + (size_t)blockIdx.x * EK;
+    for (int e = threadIdx.x; e < EK; e += kThreads)
+        out[e] = (red[e] + red[EK + e]) + (red[2 * EK + e] + red[3 * EK + e]);
+}
+
+// out[e] = sum_p part[p][e]: one wave per element, lane l adds partials l, l+64, ... in ascending order, then the
+// lanes are added pairwise — the same order on every run
+__global__ __launch_bounds__(kThreads) void conv_small_partial_sum_kernel(const float *__restrict__ part, int nparts, int E,
+                                                                         float *__restrict__ out)
+{
+    const int e = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (e >= E)
+        return;
+    const int lane = threadIdx.x & 63;
+    float s = 0.f;
+    for (int p = lane; p < nparts; p += 64)
+        s += part[(size_t)p * E + e];
+    for (int off = 32; off > 0; off >>= 1)
+        s += __shfl_xor(s, off);
+    if (lane == 0)
+        out[e] = s;
+}
+
+// wp[(tap*C + c)*OC + oc] = w[oc][c][tap]: for one tap and input channel the OC factors lie side by side
+__global__ void conv_small_permute_kernel(const float *__restrict__ w, float *__restrict__ wp, int OC, int C, int KHW)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= OC * C * KHW)
+        return;
+    const int oc = t % OC, c = (t / OC) % C, tap = t / (OC * C);
+    wp[t] = w[((size_t)oc * C + c) * KHW + tap];
+}
+
+// gx[n][c][ih][iw] = sum over the taps (kh,kw) that reach the pixel, in ascending (kh,kw) order, of
+// gx_col[m][(c,kh,kw)] = sum_oc gy2d[m][oc] * w[oc][c][kh][kw], m = (n, (ih+PH-kh)/SH, (iw+PW-kw)/SW) — the
+// reference's GEMM followed by its col2im, without the matrix between them. One thread per image pixel, all C channels.
+template <int C, int KH, int KW>
+__global__ __launch_bounds__(kThreads) void conv_small_dgrad_kernel(const float *__restrict__ gy, const float *__restrict__ wp,
+                                                                   float *__restrict__ gx, SmallGeom g)
+{
+    const unsigned pix = blockIdx.x * kThreads + threadIdx.x;
+    if (pix >= g.total)
+        return;
+    const unsigned t = odl::fastdiv(pix, g.by_w), iw = pix - t * g.W;
+    const unsigned n = odl::fastdiv(t, g.by_h), ih = t - n * g.H;
+    float acc[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+        acc[c] = 0.f;
+    const bool unit = g.SH == 1 && g.SW == 1;
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh)
+    {
+        const int th = (int)ih + g.PH - kh;
+        if (th < 0)
+            continue;
+        const int oh = unit ? th : th / g.SH;
+        if (oh >= g.OH || (!unit && oh * g.SH != th))
+            continue;
+#pragma unroll
+        for (int kw = 0; kw < KW; ++kw)
+        {
+            const int tw = (int)iw + g.PW - kw;
+            if (tw < 0)
+                continue;
+            const int ow = unit ? tw : tw / g.SW;
+            if (ow >= g.OW || (!unit && ow * g.SW != tw))
+                continue;
+            const size_t m = ((size_t)n * g.OH + oh) * g.OW + ow;
+            const f32x4 *gp = reinterpret_cast<const f32x4 *>(gy + m * g.OC);
+            const float *wt = wp + (size_t)(kh * KW + kw) * C * g.OC;  // the same address in every lane
+            float s[C];
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+                s[c] = 0.f;
+#pragma unroll 2
+            for (int q = 0; q < g.OC / 4; ++q)
+            {
+                const f32x4 v = gp[q];
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    const float *wc = wt + c * g.OC + q * 4;
+                    s[c] = fmaf(v[0], wc[0], s[c]);
+                    s[c] = fmaf(v[1], wc[1], s[c]);
+                    s[c] = fmaf(v[2], wc[2], s[c]);
+                    s[c] = fmaf(v[3], wc[3], s[c]);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+                acc[c] += s[c];
+        }
+    }
+    float *gp = gx + (size_t)n * C * g.H * g.W + (size_t)ih * g.W + iw;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+        gp[(size_t)c * g.H * g.W] = acc[c];
+}
+
+bool aligned16(const void *p)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+
+// the (C, KH, KW) triples the backward kernels are instantiated for
+bool backward_shape(int64_t C, int KH, int KW)
+{
+    return KH == KW && ((C == 1 && (KH == 3 || KH == 5)) || (C == 3 && KH == 3));
+}
+
+SmallGeom make_small(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int SH, int SW, int PH, int PW, int64_t OH,
+                     int64_t OW, bool over_image)
+{
+    SmallGeom g;
+    g.N = (int)N, g.C = (int)C, g.H = (int)H, g.W = (int)W, g.OC = (int)OC, g.OH = (int)OH, g.OW = (int)OW;
+    g.SH = SH, g.SW = SW, g.PH = PH, g.PW = PW;
+    g.total = (unsigned)(over_image ? N * H * W : N * OH * OW);
+    g.by_w = odl::make_fastdiv((unsigned)(over_image ? W : OW));
+    g.by_h = odl::make_fastdiv((unsigned)(over_image ? H : OH));
+    return g;
+}
+
+// sizes all of these kernels index with 32 bits
+bool small_sizes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t OH, int64_t OW)
+{
+    return N * OH * OW < (1ll << 31) && N * H * W < (1ll << 31) && C * H * W < (1ll << 31) && OC <= 4096 && H > 0 && W > 0 &&
+           OH > 0 && OW > 0;
+}
+
+struct WgradPlan
+{
+    int lgG;
+    unsigned rows_per_block, nblocks;
+};
+
+WgradPlan plan_wgrad(int64_t M, int64_t OC)
+{
+    WgradPlan p;
+    p.lgG = OC == 8 ? 0 : (OC == 16 ? 1 : (OC == 32 ? 2 : 3));
+    const unsigned rpp = (unsigned)kThreads >> p.lgG;
+    // about three workgroups per compute unit, each at least two passes deep
+    unsigned rows = (unsigned)odl::ceil_div(M, 768);
+    rows = (unsigned)odl::ceil_div(rows, rpp) * rpp;
+    if (rows < 2 * rpp)
+        rows = 2 * rpp;
+    p.rows_per_block = rows;
+    p.nblocks = (unsigned)odl::ceil_div(M, rows);
+    return p;
+}
+}  // namespace
+
+namespace odl
+{
+bool conv_small_forward_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH, int64_t OW)
+{
+    if (!(KH == KW && (KH == 3 || KH == 5 || KH == 6)) || OC % 16 != 0 || OC > 128)
+        return false;
+    // few enough terms that the matrix units would mostly multiply padding: a short reduction, or a narrow output
+    if (!(C * KH * KW <= 32 || (OC <= 16 && C <= 4)))
+        return false;
+    return small_sizes(N, C, H, W, OC, OH, OW);
+}
+
+int conv_small_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H, int64_t W,
+                       int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW, int act,
+                       hipStream_t st)
+{
+    const SmallGeom g = make_small(N, C, H, W, OC, SH, SW, PH, PW, OH, OW, false);
+    const dim3 grid((unsigned)ceil_div(g.total, kThreads), (unsigned)(OC / 16));
+    if (KH == 3)
+        hipLaunchKernelGGL((conv_small_fwd_kernel<3, 3, 16>), grid, dim3(kThreads), 0, st, x, w, b, y, g, act);
+    else if (KH == 5)
+        hipLaunchKernelGGL((conv_small_fwd_kernel<5, 5, 16>), grid, dim3(kThreads), 0, st, x, w, b, y, g, act);
+    else
+        hipLaunchKernelGGL((conv_small_fwd_kernel<6, 6, 16>), grid, dim3(kThreads), 0, st, x, w, b, y, g, act);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+bool conv_small_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
+                         int64_t OW)
+{
+    return backward_shape(C, KH, KW) && (OC == 8 || OC == 16 || OC == 32 || OC == 64) && aligned16(gy) &&
+           small_sizes(N, C, H, W, OC, OH, OW);
+}
+
+size_t conv_small_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW)
+{
+    return (size_t)plan_wgrad(N * OH * OW, OC).nblocks * (size_t)(OC * C * KH * KW) * sizeof(float);
+}
+
+int conv_small_wgrad(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                     int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
+                     size_t workspace_bytes, hipStream_t st)
+{
+    const SmallGeom g = make_small(N, C, H, W, OC, SH, SW, PH, PW, OH, OW, false);
+    const WgradPlan p = plan_wgrad(N * OH * OW, OC);
+    const int EK = (int)(OC * C * KH * KW);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= (size_t)p.nblocks * EK * sizeof(float),
+                "conv2d_backward: the weight-gradient partials need %zu bytes, got %zu",
+                (size_t)p.nblocks * EK * sizeof(float), workspace_bytes);
+    float *part = static_cast<float *>(workspace);
+    const size_t lds = (size_t)4 * EK * sizeof(float);
+#define ODL_SMALL_WGRAD(CV, KV)                                                                                         \
+    hipLaunchKernelGGL((conv_small_wgrad_kernel<CV, KV, KV>), dim3(p.nblocks), dim3(kThreads), lds, st, gy, x, part, g, \
+                       p.lgG, p.rows_per_block)
+    if (C == 1 && KH == 3)
+        ODL_SMALL_WGRAD(1, 3);
+    else if (C == 1)
+        ODL_SMALL_WGRAD(1, 5);
+    else
+        ODL_SMALL_WGRAD(3, 3);
+#undef ODL_SMALL_WGRAD
+    ODL_LAUNCH_CHECK();
+    hipLaunchKernelGGL(conv_small_partial_sum_kernel, dim3((unsigned)ceil_div(EK, kThreads / 64)), dim3(kThreads), 0, st,
+                       part, (int)p.nblocks, EK, gw);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+bool conv_small_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
+                         int64_t OW)
+{
+    return backward_shape(C, KH, KW) && OC % 4 == 0 && OC <= 128 && aligned16(gy) && small_sizes(N, C, H, W, OC, OH, OW);
+}
+
+size_t conv_small_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW)
+{
+    return (size_t)(OC * C * KH * KW) * sizeof(float);
+}
+
+int conv_small_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                     int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
+                     size_t workspace_bytes, hipStream_t st)
+{
+    const SmallGeom g = make_small(N, C, H, W, OC, SH, SW, PH, PW, OH, OW, true);
+    const int EK = (int)(OC * C * KH * KW);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= (size_t)EK * sizeof(float) && aligned16(workspace),
+                "conv2d_backward: the reordered filter needs %zu bytes at a 16-byte boundary, got %zu",
+                (size_t)EK * sizeof(float), workspace_bytes);
+    float *wp = static_cast<float *>(workspace);
+    hipLaunchKernelGGL(conv_small_permute_kernel, dim3((unsigned)ceil_div(EK, 256)), dim3(256), 0, st, w, wp, (int)OC,
+                       (int)C, KH * KW);
+    ODL_LAUNCH_CHECK();
+    const dim3 grid((unsigned)ceil_div(g.total, kThreads));
+    if (C == 1 && KH == 3)
+        hipLaunchKernelGGL((conv_small_dgrad_kernel<1, 3, 3>), grid, dim3(kThreads), 0, st, gy, wp, gx, g);
+    else if (C == 1)
+        hipLaunchKernelGGL((conv_small_dgrad_kernel<1, 5, 5>), grid, dim3(kThreads), 0, st, gy, wp, gx, g);
+    else
+        hipLaunchKernelGGL((conv_small_dgrad_kernel<3, 3, 3>), grid, dim3(kThreads), 0, st, gy, wp, gx, g);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace odl

@@ -87,18 +87,7 @@ struct GemmArgs
     float *tail_ws;
 };
 
-// the activations a convolution's epilogue can apply; the expressions are those of the standalone unary kernels
-__device__ inline float apply_act(float v, int act)
-{
-    if (act == 1)
-        return v > 0.f ? v : 0.f;
-    if (act == 2)
-    {
-        const float s = 1.0f / (1.0f + expf(-v));
-        return v * s;
-    }
-    return v;
-}
+using odl::apply_act;
 
 __device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
 {

@@ -52,6 +52,20 @@ __device__ inline unsigned fastdiv(unsigned m, const FastDiv &f)
     const unsigned t = __umulhi(m, f.mul);
     return (t + ((m - t) >> f.sh1)) >> f.sh2;
 }
+
+// the activations a convolution's epilogue can apply (0 none, 1 relu, 2 silu); the expressions are those of the
+// standalone unary kernels
+__device__ inline float apply_act(float v, int act)
+{
+    if (act == 1)
+        return v > 0.f ? v : 0.f;
+    if (act == 2)
+    {
+        const float s = 1.0f / (1.0f + expf(-v));
+        return v * s;
+    }
+    return v;
+}
 }  // namespace odl
 
 #define ODL_HIP_CHECK(expr)                                                                          \

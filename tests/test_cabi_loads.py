@@ -40,8 +40,12 @@ def test_workspace_queries_need_no_gpu():
     assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 3, 3, 1, 1, 1, 1) == wp
     # a 1x1 window's weights are in tap order as they are
     assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 1, 1, 1, 1, 0, 0) == 0
-    # C*KH*KW = 9 is not a multiple of 4: explicit im2col path, workspace = the col matrix [N*OH*OW, 9]
-    assert l.query("odl_hip_conv2d_workspace_bytes", 256, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1) == 256 * 28 * 28 * 9 * 4
+    # one input channel under a 3x3 window: the direct kernel, no matrix and no workspace
+    assert l.query("odl_hip_conv2d_workspace_bytes", 256, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1) == 0
+    # its backward: the weight-gradient partials (one [32][9] block per workgroup) and the reordered filter
+    assert 0 < l.query("odl_hip_conv2d_backward_workspace_bytes", 256, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1) < 2 * 1024 * 1024
+    # C*KH*KW = 45 is not a multiple of 4: explicit im2col path, workspace = the col matrix [N*OH*OW, 45]
+    assert l.query("odl_hip_conv2d_workspace_bytes", 16, 5, 28, 28, 32, 3, 3, 1, 1, 1, 1) == 16 * 28 * 28 * 45 * 4
     assert l.query("odl_hip_conv2d_backward_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) < 100352 * 576 * 4
     assert l.query("odl_hip_conv2d_workspace_bytes", 1, 1, 2, 2, 1, 3, 3, 1, 1, 0, 0) == 0  # no valid output
     assert l.query("odl_hip_sum_axis_workspace_bytes", 4096, 10, 1) == 0

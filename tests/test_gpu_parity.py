@@ -265,7 +265,14 @@ CONV_SEEDED = [
     # N, C, H, W, OC, KH, KW, s, p
     (2, 16, 14, 14, 24, 3, 3, 1, 1),   # fwd + wgrad implicit, dgrad explicit
     (3, 8, 13, 13, 12, 3, 3, 2, 1),    # stride 2
-    (2, 1, 28, 28, 32, 3, 3, 1, 1),    # C*9 = 9: explicit forward; implicit wgrad/dgrad
+    (2, 1, 28, 28, 32, 3, 3, 1, 1),    # one input channel: the direct (one thread per pixel) kernels, all three
+    (3, 1, 28, 28, 64, 3, 3, 1, 1),    # the reference's MNIST stem, 64 filters: eight channel groups per gy row
+    (2, 3, 17, 19, 16, 3, 3, 1, 1),    # three channels, W != H, two channel groups
+    (2, 1, 20, 20, 8, 5, 5, 1, 2),     # 5x5 window, a single channel group
+    (2, 1, 15, 15, 16, 3, 3, 2, 1),    # direct kernels at stride 2: the input gradient skips taps between outputs
+    (2, 3, 12, 12, 32, 3, 3, 2, 0),    # stride 2 without padding, last row and column outside every window
+    (2, 1, 9, 9, 48, 3, 3, 1, 1),      # 48 filters: direct forward and input gradient, weight gradient by GEMM
+    (300, 1, 28, 28, 32, 3, 3, 1, 1),  # more pixels than one pass of the weight-gradient grid: several rows a thread
     (2, 16, 12, 10, 32, 3, 3, 1, 1),   # all three implicit, 64-row tiles, W != H
     (1, 32, 9, 9, 144, 3, 3, 1, 1),    # all three implicit, 128-row tiles with a ragged second tile
     (2, 8, 11, 11, 16, 1, 1, 1, 0),    # 1x1
@@ -273,7 +280,7 @@ CONV_SEEDED = [
     (2, 6, 10, 9, 16, 2, 3, 1, 1),     # rectangular kernel, K = 36
     (2, 16, 15, 15, 20, 3, 3, 2, 0),   # stride 2 without padding
     (5, 64, 7, 7, 48, 3, 3, 1, 1),     # more pixels than one tile column, C = 64
-    (2, 3, 64, 64, 16, 6, 6, 2, 2),    # the detector's stem: 6x6, stride 2, pad 2, three channels
+    (2, 3, 64, 64, 16, 6, 6, 2, 2),    # the detector's stem: 6x6, stride 2, pad 2, three channels (direct forward)
     (2, 32, 40, 40, 64, 3, 3, 2, 1),   # its down-sampling convolutions
     (2, 64, 20, 20, 128, 1, 1, 1, 0),  # its 1x1 bottleneck convolutions
 ]
@@ -830,7 +837,8 @@ def test_yolo_detect_at_detector_size_vs_oracle(api, o):
 
 @pytest.mark.parametrize("N,C,H,OC,k,s,p", [
     (2, 16, 14, 24, 3, 1, 1),     # implicit forward, one pass
-    (2, 1, 28, 32, 3, 1, 1),      # C*9 = 9: explicit im2col + GEMM
+    (2, 1, 28, 32, 3, 1, 1),      # one input channel: the direct kernel
+    (2, 5, 12, 24, 3, 1, 1),      # C*9 = 45, not a multiple of 4: explicit im2col + GEMM
     (8, 128, 14, 256, 3, 2, 1),   # few tiles: K slices summed by the reduction kernel
     (4, 64, 56, 128, 3, 1, 1),    # tile count just over a multiple of the CU count: tail pieces and their fix-up
     (2, 64, 20, 128, 1, 1, 0),    # 1x1
