@@ -20,6 +20,19 @@ struct SmallGeom
 
 constexpr int kThreads = 256;
 
+// v + (v of another lane of the same row of 16), the other lane picked by a DPP control; a lane whose source falls
+// outside its row adds zero
+template <int CTRL>
+__device__ inline float dpp_add(float v)
+{
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kRowShl = 0x100;         // row_shl:n — lane i reads lane i+n of its row
+constexpr int kQuadSwap1 = 0xB1;       // quad_perm:[1,0,3,2] — lane i reads lane i^1
+constexpr int kQuadSwap2 = 0x4E;       // quad_perm:[2,3,0,1] — lane i reads lane i^2
+constexpr int kRowHalfMirror = 0x141;  // lane i reads lane 7-i of its half row
+constexpr int kRowMirror = 0x140;      // lane i reads lane 15-i of its row
+
 // y[n][oc][oh][ow] = act(sum_{c,kh,kw} x[n][c][oh*SH-PH+kh][ow*SW-PW+kw] * w[oc][c][kh][kw] + b[oc]); one thread per
 // output pixel, OCB output channels per thread (blockIdx.y picks the group). The KH*KW window of one input channel is
 // held in registers and reused by all OCB channels.
@@ -76,17 +89,21 @@ __global__ __launch_bounds__(kThreads) void conv_small_fwd_kernel(const float *_
 
 // gW[oc][k] = sum_m gy2d[m][oc] * col[m][k], col[m][(c,kh,kw)] = x[n][c][oh*SH-PH+kh][ow*SW-PW+kw] for m = (n,oh,ow).
 // A thread owns 8 consecutive channels of gy2d's rows m = first + i*rows_per_pass and all K = C*KH*KW columns: 8*K
-// private sums. G = OC/8 neighbouring lanes share a row, so a wave reads whole rows of gy2d, 16 bytes a lane. At the
-// end the lanes of equal channel group are added across the wave, the four waves across the workgroup, and the
-// workgroup writes one [OC][K] partial; conv_small_partial_sum_kernel adds the partials in a fixed order.
-template <int C, int KH, int KW>
+// private sums. G = OC/8 = 2^LGG neighbouring lanes share a row, so a wave reads whole rows of gy2d, 16 bytes a lane. At
+// the end the lanes of equal channel group are added — inside a row of 16 lanes by DPP moves, across rows and waves
+// through LDS — and the workgroup writes one [OC][K] partial; conv_small_partial_sum_kernel adds the partials in a
+// fixed order.
+template <int C, int KH, int KW, int LGG>
 __global__ __launch_bounds__(kThreads) void conv_small_wgrad_kernel(const float *__restrict__ gy, const float *__restrict__ x,
-                                                                   float *__restrict__ part, SmallGeom g, int lgG,
+                                                                   float *__restrict__ part, SmallGeom g,
                                                                    unsigned rows_per_block)
 {
     constexpr int K = C * KH * KW;
-    extern __shared__ float red[];  // [4][OC*K]
-    const int G = 1 << lgG;
+    constexpr int G = 1 << LGG, lgG = LGG;
+    constexpr int EK = 8 * G * K;
+    // partial sums kept per row of 16 lanes (16 of them in the workgroup) when that fits, else per wave (4)
+    constexpr int NR = (16 * EK * 4 <= 48 * 1024) ? 16 : 4;
+    __shared__ float red[NR * EK];
     const int ocg = threadIdx.x & (G - 1);
     const unsigned rows_per_pass = kThreads >> lgG;
     const unsigned m_begin = blockIdx.x * rows_per_block;
@@ -97,50 +114,88 @@ __global__ __launch_bounds__(kThreads) void conv_small_wgrad_kernel(const float 
 #pragma unroll
         for (int j = 0; j < K; ++j)
             acc[i][j] = 0.f;
-    for (unsigned m = m_begin + (threadIdx.x >> lgG); m < m_end; m += rows_per_pass)
+    // U rows at a time, their loads issued together; a row past the end contributes zeros
+    constexpr int U = K <= 9 ? 4 : 1;
+    for (unsigned mb = m_begin + (threadIdx.x >> lgG); mb < m_end; mb += U * rows_per_pass)
     {
-        const unsigned t = odl::fastdiv(m, g.by_w), ow = m - t * g.OW;
-        const unsigned n = odl::fastdiv(t, g.by_h), oh = t - n * g.OH;
-        const int ih0 = (int)oh * g.SH - g.PH, iw0 = (int)ow * g.SW - g.PW;
-        const float *xp = x + (size_t)n * C * g.H * g.W;
-        float xr[K];
+        float xr[U][K];
+        f32x4 gr[U][2];
 #pragma unroll
-        for (int c = 0; c < C; ++c)
+        for (int u = 0; u < U; ++u)
+        {
+            const unsigned m = mb + u * rows_per_pass;
+            const bool live = m < m_end;
+            const unsigned mm = live ? m : mb;
+            const unsigned t = odl::fastdiv(mm, g.by_w), ow = mm - t * g.OW;
+            const unsigned n = odl::fastdiv(t, g.by_h), oh = t - n * g.OH;
+            const int ih0 = (int)oh * g.SH - g.PH, iw0 = (int)ow * g.SW - g.PW;
+            const float *xp = x + (size_t)n * C * g.H * g.W;
 #pragma unroll
-            for (int kh = 0; kh < KH; ++kh)
+            for (int c = 0; c < C; ++c)
 #pragma unroll
-                for (int kw = 0; kw < KW; ++kw)
-                {
-                    const int ih = ih0 + kh, iw = iw0 + kw;
-                    const bool in = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
-                    xr[(c * KH + kh) * KW + kw] = in ? xp[((size_t)c * g.H + ih) * g.W + iw] : 0.f;
-                }
-        const f32x4 *gp = reinterpret_cast<const f32x4 *>(gy + (size_t)m * g.OC + ocg * 8);
-        const f32x4 g0 = gp[0], g1 = gp[1];
-        const float gv[8] = {g0[0], g0[1], g0[2], g0[3], g1[0], g1[1], g1[2], g1[3]};
+                for (int kh = 0; kh < KH; ++kh)
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+                    for (int kw = 0; kw < KW; ++kw)
+                    {
+                        const int ih = ih0 + kh, iw = iw0 + kw;
+                        const bool in = live && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+                        xr[u][(c * KH + kh) * KW + kw] = in ? xp[((size_t)c * g.H + ih) * g.W + iw] : 0.f;
+                    }
+            const f32x4 *gp = reinterpret_cast<const f32x4 *>(gy + (size_t)mm * g.OC + ocg * 8);
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            gr[u][0] = live ? gp[0] : zero;
+            gr[u][1] = live ? gp[1] : zero;
+        }
 #pragma unroll
-            for (int j = 0; j < K; ++j)
-                acc[i][j] = fmaf(gv[i], xr[j], acc[i][j]);
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j)
+                    acc[i][j] = fmaf(gr[u][i / 4][i % 4], xr[u][j], acc[i][j]);
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int EK = g.OC * K;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < K; ++j)
         {
             float v = acc[i][j];
-            for (int off = G; off < 64; off <<= 1)
-                v += __shfl_xor(v, off);
-            if (lane < G)
-                red[wave * EK + (ocg * 8 + i) * K + j] = v;
+            if (LGG <= 0)
+                v = dpp_add<kRowShl + 1>(v);
+            if (LGG <= 1)
+                v = dpp_add<kRowShl + 2>(v);
+            if (LGG <= 2)
+                v = dpp_add<kRowShl + 4>(v);
+            v = dpp_add<kRowShl + 8>(v);  // lanes 0..G-1 of each row now hold the row's sums
+            if (NR == 16)
+            {
+                if ((lane & 15) < G)
+                    red[(wave * 4 + (lane >> 4)) * EK + (ocg * 8 + i) * K + j] = v;
+            }
+            else
+            {
+                v += __shfl_xor(v, 16);
+                v += __shfl_xor(v, 32);
+                if (lane < G)
+                    red[wave * EK + (ocg * 8 + i) * K + j] = v;
+            }
         }
     __syncthreads();
     float *out = part + (size_t)blockIdx.x * EK;
     for (int e = threadIdx.x; e < EK; e += kThreads)
-        out[e] = (red[e] + red[EK + e]) + (red[2 * EK + e] + red[3 * EK + e]);
+    {
+        float r[NR];
+#pragma unroll
+        for (int q = 0; q < NR; ++q)
+            r[q] = red[q * EK + e];
+#pragma unroll
+        for (int w = NR / 2; w > 0; w /= 2)
+#pragma unroll
+            for (int q = 0; q < w; ++q)
+                r[q] = r[q] + r[q + w];
+        out[e] = r[0];
+    }
 }
 
 // out[e] = sum_p part[p][e]: one wave per element, lane l adds partials l, l+64, ... in ascending order, then the
@@ -171,71 +226,83 @@ __global__ void conv_small_permute_kernel(const float *__restrict__ w, float *__
     wp[t] = w[((size_t)oc * C + c) * KHW + tap];
 }
 
-// gx[n][c][ih][iw] = sum over the taps (kh,kw) that reach the pixel, in ascending (kh,kw) order, of
-// gx_col[m][(c,kh,kw)] = sum_oc gy2d[m][oc] * w[oc][c][kh][kw], m = (n, (ih+PH-kh)/SH, (iw+PW-kw)/SW) — the
-// reference's GEMM followed by its col2im, without the matrix between them. One thread per image pixel, all C channels.
-template <int C, int KH, int KW>
-__global__ __launch_bounds__(kThreads) void conv_small_dgrad_kernel(const float *__restrict__ gy, const float *__restrict__ wp,
-                                                                   float *__restrict__ gx, SmallGeom g)
+// gx[n][c][ih][iw] = sum over the taps (kh,kw) that reach the pixel of gx_col[m][(c,kh,kw)] =
+// sum_oc gy2d[m][oc] * w[oc][c][kh][kw], m = (n, (ih+PH-kh)/SH, (iw+PW-kw)/SW) — the reference's GEMM followed by its
+// col2im, without the matrix between them. L = OC/4 = 2^LGL neighbouring lanes share a pixel: lane `sub` holds
+// channels 4*sub..4*sub+3 of every tap's factors in registers and reads those 16 bytes of each gy2d row, so a wave
+// reads whole rows; the L partial sums meet through DPP moves. A thread walks kDgPixels pixels with the same factors.
+// Every tap's row is loaded whether the tap reaches the pixel or not (row 0 stands in), so that the loads of all
+// taps are in flight together; a tap that does not reach the pixel is left out of the sum.
+constexpr int kDgThreads = 512, kDgPixels = 4;
+template <int C, int KH, int KW, int LGL>
+__global__ __launch_bounds__(kDgThreads) void conv_small_dgrad_kernel(const float *__restrict__ gy, const float *__restrict__ wp,
+                                                                     float *__restrict__ gx, SmallGeom g)
 {
-    const unsigned pix = blockIdx.x * kThreads + threadIdx.x;
-    if (pix >= g.total)
-        return;
-    const unsigned t = odl::fastdiv(pix, g.by_w), iw = pix - t * g.W;
-    const unsigned n = odl::fastdiv(t, g.by_h), ih = t - n * g.H;
-    float acc[C];
+    constexpr int L = 1 << LGL;
+    constexpr int kPer = kDgThreads >> LGL;  // pixels per pass of the workgroup
+    const int sub = threadIdx.x & (L - 1);
+    const f32x4 *gy4 = reinterpret_cast<const f32x4 *>(gy);
+    f32x4 wv[KH * KW][C];
 #pragma unroll
-    for (int c = 0; c < C; ++c)
-        acc[c] = 0.f;
+    for (int tap = 0; tap < KH * KW; ++tap)
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+            wv[tap][c] = reinterpret_cast<const f32x4 *>(wp)[(tap * C + c) * L + sub];
     const bool unit = g.SH == 1 && g.SW == 1;
-#pragma unroll
-    for (int kh = 0; kh < KH; ++kh)
+#pragma unroll 1
+    for (int it = 0; it < kDgPixels; ++it)
     {
-        const int th = (int)ih + g.PH - kh;
-        if (th < 0)
-            continue;
-        const int oh = unit ? th : th / g.SH;
-        if (oh >= g.OH || (!unit && oh * g.SH != th))
-            continue;
+        const unsigned pix = (blockIdx.x * kDgPixels + it) * kPer + (threadIdx.x >> LGL);
+        const bool live = pix < g.total;  // the same in all lanes of a pixel
+        const unsigned pp = live ? pix : g.total - 1;
+        const unsigned t = odl::fastdiv(pp, g.by_w), iw = pp - t * g.W;
+        const unsigned n = odl::fastdiv(t, g.by_h), ih = t - n * g.H;
+        float acc[C];
 #pragma unroll
-        for (int kw = 0; kw < KW; ++kw)
+        for (int c = 0; c < C; ++c)
+            acc[c] = 0.f;
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh)
         {
-            const int tw = (int)iw + g.PW - kw;
-            if (tw < 0)
-                continue;
-            const int ow = unit ? tw : tw / g.SW;
-            if (ow >= g.OW || (!unit && ow * g.SW != tw))
-                continue;
-            const size_t m = ((size_t)n * g.OH + oh) * g.OW + ow;
-            const f32x4 *gp = reinterpret_cast<const f32x4 *>(gy + m * g.OC);
-            const float *wt = wp + (size_t)(kh * KW + kw) * C * g.OC;  // the same address in every lane
-            float s[C];
+            const int th = (int)ih + g.PH - kh;
+            const int oh = unit ? th : th / g.SH;
+            const bool hit_h = th >= 0 && oh < g.OH && (unit || oh * g.SH == th);
 #pragma unroll
-            for (int c = 0; c < C; ++c)
-                s[c] = 0.f;
-#pragma unroll 2
-            for (int q = 0; q < g.OC / 4; ++q)
+            for (int kw = 0; kw < KW; ++kw)
             {
-                const f32x4 v = gp[q];
+                const int tw = (int)iw + g.PW - kw;
+                const int ow = unit ? tw : tw / g.SW;
+                const bool hit = hit_h && tw >= 0 && ow < g.OW && (unit || ow * g.SW == tw);
+                const size_t m = hit ? ((size_t)n * g.OH + oh) * g.OW + ow : 0;
+                const f32x4 v = gy4[m * L + sub];
 #pragma unroll
                 for (int c = 0; c < C; ++c)
                 {
-                    const float *wc = wt + c * g.OC + q * 4;
-                    s[c] = fmaf(v[0], wc[0], s[c]);
-                    s[c] = fmaf(v[1], wc[1], s[c]);
-                    s[c] = fmaf(v[2], wc[2], s[c]);
-                    s[c] = fmaf(v[3], wc[3], s[c]);
+                    const f32x4 wq = wv[kh * KW + kw][c];
+                    float s = v[0] * wq[0];
+                    s = fmaf(v[1], wq[1], s);
+                    s = fmaf(v[2], wq[2], s);
+                    s = fmaf(v[3], wq[3], s);
+                    acc[c] += hit ? s : 0.f;
                 }
             }
+        }
 #pragma unroll
-            for (int c = 0; c < C; ++c)
-                acc[c] += s[c];
+        for (int c = 0; c < C; ++c)
+        {
+            float v = acc[c];
+            if (LGL >= 1)
+                v = dpp_add<kQuadSwap1>(v);
+            if (LGL >= 2)
+                v = dpp_add<kQuadSwap2>(v);
+            if (LGL >= 3)
+                v = dpp_add<kRowHalfMirror>(v);  // the quads are uniform by now, so 7-i stands for i^4
+            if (LGL >= 4)
+                v = dpp_add<kRowMirror>(v);      // and 15-i for i^8
+            if (sub == 0 && live)
+                gx[((size_t)n * C + c) * g.H * g.W + (size_t)ih * g.W + iw] = v;
         }
     }
-    float *gp = gx + (size_t)n * C * g.H * g.W + (size_t)ih * g.W + iw;
-#pragma unroll
-    for (int c = 0; c < C; ++c)
-        gp[(size_t)c * g.H * g.W] = acc[c];
 }
 
 bool aligned16(const void *p)
@@ -279,11 +346,9 @@ WgradPlan plan_wgrad(int64_t M, int64_t OC)
     WgradPlan p;
     p.lgG = OC == 8 ? 0 : (OC == 16 ? 1 : (OC == 32 ? 2 : 3));
     const unsigned rpp = (unsigned)kThreads >> p.lgG;
-    // about three workgroups per compute unit, each at least two passes deep
+    // about three workgroups per compute unit at most, each a whole number of four-row rounds
     unsigned rows = (unsigned)odl::ceil_div(M, 768);
-    rows = (unsigned)odl::ceil_div(rows, rpp) * rpp;
-    if (rows < 2 * rpp)
-        rows = 2 * rpp;
+    rows = (unsigned)odl::ceil_div(rows, 4 * rpp) * 4 * rpp;
     p.rows_per_block = rows;
     p.nblocks = (unsigned)odl::ceil_div(M, rows);
     return p;
@@ -341,16 +406,28 @@ int conv_small_wgrad(const float *gy, const float *x, float *gw, int64_t N, int6
                 "conv2d_backward: the weight-gradient partials need %zu bytes, got %zu",
                 (size_t)p.nblocks * EK * sizeof(float), workspace_bytes);
     float *part = static_cast<float *>(workspace);
-    const size_t lds = (size_t)4 * EK * sizeof(float);
-#define ODL_SMALL_WGRAD(CV, KV)                                                                                         \
-    hipLaunchKernelGGL((conv_small_wgrad_kernel<CV, KV, KV>), dim3(p.nblocks), dim3(kThreads), lds, st, gy, x, part, g, \
-                       p.lgG, p.rows_per_block)
+#define ODL_SMALL_WGRAD(CV, KV, LG)                                                                                \
+    hipLaunchKernelGGL((conv_small_wgrad_kernel<CV, KV, KV, LG>), dim3(p.nblocks), dim3(kThreads), 0, st, gy, x, part, g, \
+                       p.rows_per_block)
+#define ODL_SMALL_WGRAD_G(CV, KV)     \
+    do                                \
+    {                                 \
+        if (p.lgG == 0)               \
+            ODL_SMALL_WGRAD(CV, KV, 0); \
+        else if (p.lgG == 1)          \
+            ODL_SMALL_WGRAD(CV, KV, 1); \
+        else if (p.lgG == 2)          \
+            ODL_SMALL_WGRAD(CV, KV, 2); \
+        else                          \
+            ODL_SMALL_WGRAD(CV, KV, 3); \
+    } while (0)
     if (C == 1 && KH == 3)
-        ODL_SMALL_WGRAD(1, 3);
+        ODL_SMALL_WGRAD_G(1, 3);
     else if (C == 1)
-        ODL_SMALL_WGRAD(1, 5);
+        ODL_SMALL_WGRAD_G(1, 5);
     else
-        ODL_SMALL_WGRAD(3, 3);
+        ODL_SMALL_WGRAD_G(3, 3);
+#undef ODL_SMALL_WGRAD_G
 #undef ODL_SMALL_WGRAD
     ODL_LAUNCH_CHECK();
     hipLaunchKernelGGL(conv_small_partial_sum_kernel, dim3((unsigned)ceil_div(EK, kThreads / 64)), dim3(kThreads), 0, st,
@@ -362,7 +439,8 @@ int conv_small_wgrad(const float *gy, const float *x, float *gw, int64_t N, int6
 bool conv_small_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
                          int64_t OW)
 {
-    return backward_shape(C, KH, KW) && OC % 4 == 0 && OC <= 128 && aligned16(gy) && small_sizes(N, C, H, W, OC, OH, OW);
+    return backward_shape(C, KH, KW) && (OC == 8 || OC == 16 || OC == 32 || OC == 64) && aligned16(gy) &&
+           small_sizes(N, C, H, W, OC, OH, OW);
 }
 
 size_t conv_small_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW)
@@ -383,13 +461,30 @@ int conv_small_dgrad(const float *gy, const float *w, float *gx, int64_t N, int6
     hipLaunchKernelGGL(conv_small_permute_kernel, dim3((unsigned)ceil_div(EK, 256)), dim3(256), 0, st, w, wp, (int)OC,
                        (int)C, KH * KW);
     ODL_LAUNCH_CHECK();
-    const dim3 grid((unsigned)ceil_div(g.total, kThreads));
+    const int lgL = OC == 8 ? 1 : (OC == 16 ? 2 : (OC == 32 ? 3 : 4));
+    const dim3 grid((unsigned)ceil_div(g.total, (int64_t)kDgPixels * (kDgThreads >> lgL)));
+#define ODL_SMALL_DGRAD(CV, KV, LG) \
+    hipLaunchKernelGGL((conv_small_dgrad_kernel<CV, KV, KV, LG>), grid, dim3(kDgThreads), 0, st, gy, wp, gx, g)
+#define ODL_SMALL_DGRAD_OC(CV, KV)      \
+    do                                  \
+    {                                   \
+        if (lgL == 1)                   \
+            ODL_SMALL_DGRAD(CV, KV, 1); \
+        else if (lgL == 2)              \
+            ODL_SMALL_DGRAD(CV, KV, 2); \
+        else if (lgL == 3)              \
+            ODL_SMALL_DGRAD(CV, KV, 3); \
+        else                            \
+            ODL_SMALL_DGRAD(CV, KV, 4); \
+    } while (0)
     if (C == 1 && KH == 3)
-        hipLaunchKernelGGL((conv_small_dgrad_kernel<1, 3, 3>), grid, dim3(kThreads), 0, st, gy, wp, gx, g);
+        ODL_SMALL_DGRAD_OC(1, 3);
     else if (C == 1)
-        hipLaunchKernelGGL((conv_small_dgrad_kernel<1, 5, 5>), grid, dim3(kThreads), 0, st, gy, wp, gx, g);
+        ODL_SMALL_DGRAD_OC(1, 5);
     else
-        hipLaunchKernelGGL((conv_small_dgrad_kernel<3, 3, 3>), grid, dim3(kThreads), 0, st, gy, wp, gx, g);
+        ODL_SMALL_DGRAD_OC(3, 3);
+#undef ODL_SMALL_DGRAD_OC
+#undef ODL_SMALL_DGRAD
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
