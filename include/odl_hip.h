@@ -283,6 +283,19 @@ int odl_hip_adam_step_device_scales(const float *p, const float *g, float *m, fl
                                     float beta2, const float *device_scales, float eps, float lr, float *p_out,
                                     void *stream);
 int odl_hip_sgd_step(const float *p, const float *g, int64_t n, float lr, float *p_out, void *stream);
+/* The same steps over a whole list of parameters in one launch (Optimizer::step, src/optim/optimizer.cpp:19-53, walks
+ * the parameters one by one; most of them are biases of a few hundred floats, so the walk is launch-bound). The
+ * arguments are host arrays of `count` device pointers and sizes; entry i gets exactly what the one-tensor call
+ * gives. adam_step_multi: m_hat_scale[i], v_hat_scale[i] from the host arrays, unless device_scales (an array, or
+ * NULL) holds a non-NULL device pointer for entry i (two floats, as in odl_hip_adam_step_device_scales).
+ * axpy_multi: y[i] += alpha * x[i], the product rounded before the sum — the WeightDecay hook
+ * (include/origin/optim/hooks.h: grad += rate * param) over all parameters. Empty tensors are skipped. */
+int odl_hip_adam_step_multi(int count, const float *const *p, const float *const *g, float *const *m, float *const *v,
+                            const int64_t *n, float beta1, float beta2, const float *m_hat_scale, const float *v_hat_scale,
+                            const float *const *device_scales, float eps, float lr, float *const *p_out, void *stream);
+int odl_hip_sgd_step_multi(int count, const float *const *p, const float *const *g, const int64_t *n, float lr,
+                           float *const *p_out, void *stream);
+int odl_hip_axpy_multi(int count, float alpha, const float *const *x, float *const *y, const int64_t *n, void *stream);
 /* origin::cuda::{zeros,ones,full} (cuda/factory.cuh:23-50) */
 int odl_hip_fill(float *dst, int64_t n, float value, void *stream);
 

@@ -598,6 +598,56 @@ def sgd_step(p, g, lr):
     return out
 
 
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() if t is not None else None for t in tensors])
+
+
+def _size_array(tensors):
+    return (ctypes.c_int64 * len(tensors))(*[t.numel() for t in tensors])
+
+
+def adam_step_multi(ps, gs, ms, vs, ts, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, device_scales=None):
+    """One launch over a list of parameters (Optimizer::step, src/optim/optimizer.cpp:19-53, walks them one by one):
+    entry i gets what adam_step gives at step count ts[i]. Returns the new parameters; ms and vs are updated in place.
+    device_scales: optional list whose non-None entries are device tensors of two floats used instead of ts[i]."""
+    for group in (ps, gs, ms, vs):
+        for x in group:
+            _chk(x, "adam_step_multi operand")
+    f = np.float32
+    s1 = [f(1.0) / (f(1.0) - f(np.power(f(beta1), f(t)))) for t in ts]
+    s2 = [f(1.0) / (f(1.0) - f(np.power(f(beta2), f(t)))) for t in ts]
+    outs = [_empty(p.shape) for p in ps]
+    n = len(ps)
+    lib().call("odl_hip_adam_step_multi", n, _ptr_array(ps), _ptr_array(gs), _ptr_array(ms), _ptr_array(vs),
+               _size_array(ps), float(f(beta1)), float(f(beta2)), (ctypes.c_float * n)(*s1), (ctypes.c_float * n)(*s2),
+               _ptr_array(device_scales) if device_scales is not None else None, float(f(eps)), float(f(lr)),
+               _ptr_array(outs), _stream())
+    return outs
+
+
+def sgd_step_multi(ps, gs, lr):
+    """p - g*lr for every pair of the lists in one launch."""
+    for group in (ps, gs):
+        for x in group:
+            _chk(x, "sgd_step_multi operand")
+    outs = [_empty(p.shape) for p in ps]
+    lib().call("odl_hip_sgd_step_multi", len(ps), _ptr_array(ps), _ptr_array(gs), _size_array(ps), float(np.float32(lr)),
+               _ptr_array(outs), _stream())
+    return outs
+
+
+def axpy_multi(alpha, xs, ys):
+    """ys[i] += alpha * xs[i] in place, one launch (the WeightDecay hook over all parameters)."""
+    for group in (xs, ys):
+        for x in group:
+            _chk(x, "axpy_multi operand")
+    for x, y in zip(xs, ys):
+        if x.shape != y.shape:
+            raise OdlInvalidArgument("axpy_multi: shape mismatch")
+    lib().call("odl_hip_axpy_multi", len(xs), float(np.float32(alpha)), _ptr_array(xs), _ptr_array(ys), _size_array(xs),
+               _stream())
+
+
 def fill(shape, value):
     out = _empty(shape)
     lib().call("odl_hip_fill", _p(out), out.numel(), ctypes.c_float(value), _stream())

@@ -203,6 +203,103 @@ __global__ void sgd_step_kernel(const float *p, const float *g, float *p_out, in
     }
 }
 
+// ---- one launch over several tensors (all the parameters of a model): the launch count of an optimizer step stops
+// growing with the number of parameters, most of which are biases of a few hundred floats
+constexpr int kMultiMax = 24;                   // tensors per launch; longer lists go out in several launches
+constexpr int kMultiChunk = kBlock * 4;         // elements per workgroup
+struct MultiArgs
+{
+    const float *a[kMultiMax];      // adam, sgd: parameter; axpy: x
+    const float *b[kMultiMax];      // adam, sgd: gradient
+    float *m[kMultiMax];            // adam: first moment
+    float *v[kMultiMax];            // adam: second moment
+    float *out[kMultiMax];          // adam, sgd: updated parameter; axpy: y (updated in place)
+    const float *scales[kMultiMax]; // adam: the two bias-correction factors in device memory, or null
+    float m_hat_scale[kMultiMax], v_hat_scale[kMultiMax];
+    int64_t n[kMultiMax];
+    unsigned first_block[kMultiMax + 1];  // workgroups [first_block[t], first_block[t+1]) belong to tensor t
+    int count;
+};
+
+// OP 0: Adam step, 1: SGD step, 2: out += alpha * a — per element the same float operations as the one-tensor kernels
+template <int OP>
+__global__ __launch_bounds__(kBlock) void multi_tensor_kernel(MultiArgs q, AdamScalars s, float alpha)
+{
+    int t = 0;
+    while (t + 1 < q.count && blockIdx.x >= q.first_block[t + 1])  // the same in every lane
+        ++t;
+    const int64_t n = q.n[t];
+    const int64_t i = ((int64_t)(blockIdx.x - q.first_block[t]) * kBlock + threadIdx.x) * 4;
+    if (i >= n)
+        return;
+    const float *a = q.a[t], *b = q.b[t];
+    float *m = q.m[t], *v = q.v[t], *out = q.out[t];
+    if (OP == 0)
+    {
+        s.m_hat_scale = q.m_hat_scale[t], s.v_hat_scale = q.v_hat_scale[t];
+        if (q.scales[t])
+            s.m_hat_scale = q.scales[t][0], s.v_hat_scale = q.scales[t][1];
+    }
+    auto aligned = [](const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; };
+    const bool vec = i + 3 < n && aligned(a) && aligned(out) && (OP == 2 || aligned(b)) && (OP != 0 || (aligned(m) && aligned(v)));
+    if (vec)
+    {
+        const f32x4 av = *reinterpret_cast<const f32x4 *>(a + i);
+        f32x4 ov;
+        if (OP == 0)
+        {
+            const f32x4 gv = *reinterpret_cast<const f32x4 *>(b + i);
+            f32x4 mv = *reinterpret_cast<f32x4 *>(m + i), vv = *reinterpret_cast<f32x4 *>(v + i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                float mj = mv[j], vj = vv[j], oj;
+                adam_one(av[j], gv[j], mj, vj, oj, s);
+                mv[j] = mj, vv[j] = vj, ov[j] = oj;
+            }
+            *reinterpret_cast<f32x4 *>(m + i) = mv;
+            *reinterpret_cast<f32x4 *>(v + i) = vv;
+        }
+        else if (OP == 1)
+        {
+            const f32x4 gv = *reinterpret_cast<const f32x4 *>(b + i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                const float step = gv[j] * s.lr;
+                ov[j] = av[j] - step;
+            }
+        }
+        else
+        {
+            const f32x4 yv = *reinterpret_cast<const f32x4 *>(out + i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                const float step = alpha * av[j];
+                ov[j] = yv[j] + step;
+            }
+        }
+        *reinterpret_cast<f32x4 *>(out + i) = ov;
+        return;
+    }
+    for (int64_t k = i; k < n && k < i + 4; ++k)
+    {
+        if (OP == 0)
+            adam_one(a[k], b[k], m[k], v[k], out[k], s);
+        else if (OP == 1)
+        {
+            const float step = b[k] * s.lr;
+            out[k] = a[k] - step;
+        }
+        else
+        {
+            const float step = alpha * a[k];
+            out[k] = out[k] + step;
+        }
+    }
+}
+
 __global__ void fill_kernel(float *dst, int64_t n, float v)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -269,6 +366,59 @@ int fill_bytes_launch(void *dst, int value, size_t bytes, hipStream_t st)
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
+// the list goes out kMultiMax tensors at a time; empty tensors are skipped
+template <int OP>
+int multi_launch(const char *what, int count, const float *const *a, const float *const *b, float *const *m,
+                        float *const *v, float *const *out, const float *const *scales, const float *m_hat,
+                        const float *v_hat, const int64_t *n, const AdamScalars &s, float alpha, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(count >= 0, "%s: negative count", what);
+    if (count == 0)
+        return ODL_OK;
+    ODL_REQUIRE(a && out && n && (OP == 2 || b) && (OP != 0 || (m && v && (scales || (m_hat && v_hat)))),
+                "%s: null argument list", what);
+    MultiArgs q;
+    int used = 0;
+    uint64_t blocks = 0;
+    auto flush = [&]() -> int {
+        if (used == 0)
+            return ODL_OK;
+        q.count = used;
+        q.first_block[used] = (unsigned)blocks;
+        hipLaunchKernelGGL((multi_tensor_kernel<OP>), dim3((unsigned)blocks), dim3(kBlock), 0, odl::as_stream(stream), q, s,
+                           alpha);
+        ODL_LAUNCH_CHECK();
+        used = 0, blocks = 0;
+        return ODL_OK;
+    };
+    for (int i = 0; i < count; ++i)
+    {
+        ODL_REQUIRE(n[i] >= 0, "%s: tensor %d has a negative size", what, i);
+        if (n[i] == 0)
+            continue;
+        ODL_REQUIRE(a[i] && out[i] && (OP == 2 || b[i]) && (OP != 0 || (m[i] && v[i])), "%s: tensor %d has a null operand",
+                    what, i);
+        const uint64_t nb = (uint64_t)odl::ceil_div(n[i], kMultiChunk);
+        ODL_REQUIRE(nb < (1ull << 31), "%s: tensor %d is too large", what, i);
+        if (used == kMultiMax || blocks + nb >= (1ull << 31))
+        {
+            const int rc = flush();
+            if (rc != ODL_OK)
+                return rc;
+        }
+        q.a[used] = a[i], q.b[used] = b ? b[i] : nullptr, q.m[used] = m ? m[i] : nullptr, q.v[used] = v ? v[i] : nullptr;
+        q.out[used] = out[i], q.scales[used] = scales ? scales[i] : nullptr;
+        q.m_hat_scale[used] = m_hat ? m_hat[i] : 0.0f, q.v_hat_scale[used] = v_hat ? v_hat[i] : 0.0f;
+        ODL_REQUIRE(OP != 0 || q.scales[used] || (m_hat && v_hat), "%s: tensor %d has no bias-correction factors", what, i);
+        q.n[used] = n[i];
+        q.first_block[used] = (unsigned)blocks;
+        blocks += nb;
+        ++used;
+    }
+    return flush();
+}
+
 }  // namespace odl
 
 extern "C" {
@@ -380,6 +530,30 @@ int odl_hip_adam_step_device_scales(const float *p, const float *g, float *m, fl
 {
     ODL_REQUIRE(device_scales != nullptr, "adam_step: null scales");
     return adam_launch(p, g, m, v, n, beta1, beta2, 0.0f, 0.0f, device_scales, eps, lr, p_out, stream);
+}
+
+int odl_hip_adam_step_multi(int count, const float *const *p, const float *const *g, float *const *m, float *const *v,
+                            const int64_t *n, float beta1, float beta2, const float *m_hat_scale, const float *v_hat_scale,
+                            const float *const *device_scales, float eps, float lr, float *const *p_out, void *stream)
+{
+    const AdamScalars s{beta1, 1.0f - beta1, beta2, 1.0f - beta2, 0.0f, 0.0f, eps, lr, 0.5f};
+    return odl::multi_launch<0>("adam_step_multi", count, p, g, m, v, p_out, device_scales, m_hat_scale, v_hat_scale, n, s, 0.0f,
+                           stream);
+}
+
+int odl_hip_sgd_step_multi(int count, const float *const *p, const float *const *g, const int64_t *n, float lr,
+                           float *const *p_out, void *stream)
+{
+    const AdamScalars s{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, lr, 0.5f};
+    return odl::multi_launch<1>("sgd_step_multi", count, p, g, nullptr, nullptr, p_out, nullptr, nullptr, nullptr, n, s, 0.0f,
+                           stream);
+}
+
+int odl_hip_axpy_multi(int count, float alpha, const float *const *x, float *const *y, const int64_t *n, void *stream)
+{
+    const AdamScalars s{};
+    return odl::multi_launch<2>("axpy_multi", count, x, nullptr, nullptr, nullptr, y, nullptr, nullptr, nullptr, n, s, alpha,
+                           stream);
 }
 
 int odl_hip_sgd_step(const float *p, const float *g, int64_t n, float lr, float *p_out, void *stream)

@@ -313,6 +313,23 @@ public:
     std::unique_ptr<Mat> adam_step(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, float m_hat_scale,
                                    float v_hat_scale, float eps, float lr) const;
     std::unique_ptr<Mat> sgd_step(const Mat &grad, float lr) const;
+    // The same steps over a whole list of parameters in one launch (the walk over the parameters is launch-bound: most
+    // are biases of a few hundred floats). Every tensor must be float32 on the device (device_f32 tells); in_place
+    // writes each parameter where it lies and returns nothing, otherwise entry i of the result is the updated parameter.
+    struct AdamItem
+    {
+        const Mat *param, *grad;
+        Mat *m, *v;
+        float m_hat_scale, v_hat_scale;
+        const float *device_scales;  // the two factors in device memory instead (recorded steps), or null
+    };
+    static std::vector<std::unique_ptr<Mat>> adam_step_multi(const std::vector<AdamItem> &items, float beta1, float beta2,
+                                                             float eps, float lr, bool in_place);
+    static std::vector<std::unique_ptr<Mat>> sgd_step_multi(const std::vector<std::pair<const Mat *, const Mat *>> &param_grad,
+                                                            float lr, bool in_place);
+    // y += a*x for every (x, y) of the list
+    static void axpy_multi(float a, const std::vector<std::pair<const Mat *, Mat *>> &x_y);
+    static bool device_f32(const Mat &m);
     // {gy . w^T, x^T . gy} for 2-D operands, reading w and x in place (no transposed copies)
     static std::pair<std::unique_ptr<Mat>, std::unique_ptr<Mat>> matmul_backward_2d(const Mat &x, const Mat &w,
                                                                                    const Mat &gy);

@@ -204,6 +204,12 @@ public:
 
 protected:
     virtual void step_one(Parameter &param) = 0;
+    // all parameters that have a gradient, after the hooks: one by one unless the optimizer knows better
+    virtual void step_all(std::vector<Parameter *> &params)
+    {
+        for (auto *p : params)
+            step_one(*p);
+    }
     Module *target_;
     std::vector<Parameter *> parameters_;
     std::vector<std::function<void(std::vector<Parameter *> &)>> hooks_;
@@ -218,6 +224,7 @@ public:
 
 protected:
     void step_one(Parameter &param) override;
+    void step_all(std::vector<Parameter *> &params) override;
 
 private:
     float lr_, momentum_, weight_decay_;
@@ -234,6 +241,7 @@ public:
 
 protected:
     void step_one(Parameter &param) override;
+    void step_all(std::vector<Parameter *> &params) override;
 
 private:
     float lr_, beta1_, beta2_, eps_;

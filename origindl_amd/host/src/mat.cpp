@@ -1380,6 +1380,87 @@ std::unique_ptr<Mat> OriginMat::adam_step(const Mat &grad, Mat &m, Mat &v, float
     return out;
 }
 
+bool OriginMat::device_f32(const Mat &m)
+{
+    const auto *o = dynamic_cast<const OriginMat *>(&m);
+    return o && o->device().type() == DeviceType::kCUDA && o->dtype() == DataType::kFloat32;
+}
+
+std::vector<std::unique_ptr<Mat>> OriginMat::adam_step_multi(const std::vector<AdamItem> &items, float beta1, float beta2,
+                                                             float eps, float lr, bool in_place)
+{
+    const size_t count = items.size();
+    std::vector<const float *> p(count), g(count), scales(count);
+    std::vector<float *> m(count), v(count), out(count);
+    std::vector<float> s1(count), s2(count);
+    std::vector<int64_t> n(count);
+    std::vector<std::unique_ptr<Mat>> results;
+    for (size_t i = 0; i < count; ++i)
+    {
+        const OriginMat &pm = dev_f32(*items[i].param, "adam_step"), &gm = dev_f32(*items[i].grad, "adam_step");
+        const OriginMat &mm = dev_f32(*items[i].m, "adam_step"), &vm = dev_f32(*items[i].v, "adam_step");
+        if (gm.elements() != pm.elements() || mm.elements() != pm.elements() || vm.elements() != pm.elements())
+            THROW_INVALID_ARG("adam_step: parameter, gradient and moment sizes differ");
+        p[i] = fp(pm), g[i] = fp(gm), m[i] = const_cast<float *>(fp(mm)), v[i] = const_cast<float *>(fp(vm));
+        s1[i] = items[i].m_hat_scale, s2[i] = items[i].v_hat_scale, scales[i] = items[i].device_scales;
+        n[i] = (int64_t)pm.elements();
+        if (in_place)
+            out[i] = const_cast<float *>(p[i]);
+        else
+        {
+            auto o = new_like(pm, pm.shape());
+            out[i] = o->data_ptr<float>();
+            results.push_back(std::move(o));
+        }
+    }
+    check(odl_hip_adam_step_multi((int)count, p.data(), g.data(), m.data(), v.data(), n.data(), beta1, beta2, s1.data(),
+                                  s2.data(), scales.data(), eps, lr, out.data(), cur()));
+    return results;
+}
+
+std::vector<std::unique_ptr<Mat>> OriginMat::sgd_step_multi(const std::vector<std::pair<const Mat *, const Mat *>> &param_grad,
+                                                            float lr, bool in_place)
+{
+    const size_t count = param_grad.size();
+    std::vector<const float *> p(count), g(count);
+    std::vector<float *> out(count);
+    std::vector<int64_t> n(count);
+    std::vector<std::unique_ptr<Mat>> results;
+    for (size_t i = 0; i < count; ++i)
+    {
+        const OriginMat &pm = dev_f32(*param_grad[i].first, "sgd_step"), &gm = dev_f32(*param_grad[i].second, "sgd_step");
+        if (gm.elements() != pm.elements())
+            THROW_INVALID_ARG("sgd_step: parameter and gradient sizes differ");
+        p[i] = fp(pm), g[i] = fp(gm), n[i] = (int64_t)pm.elements();
+        if (in_place)
+            out[i] = const_cast<float *>(p[i]);
+        else
+        {
+            auto o = new_like(pm, pm.shape());
+            out[i] = o->data_ptr<float>();
+            results.push_back(std::move(o));
+        }
+    }
+    check(odl_hip_sgd_step_multi((int)count, p.data(), g.data(), n.data(), lr, out.data(), cur()));
+    return results;
+}
+
+void OriginMat::axpy_multi(float a, const std::vector<std::pair<const Mat *, Mat *>> &x_y)
+{
+    const size_t count = x_y.size();
+    std::vector<const float *> x(count);
+    std::vector<float *> y(count);
+    std::vector<int64_t> n(count);
+    for (size_t i = 0; i < count; ++i)
+    {
+        const OriginMat &xm = dev_f32(*x_y[i].first, "axpy"), &ym = dev_f32(*x_y[i].second, "axpy");
+        if (xm.shape() != ym.shape())
+            THROW_INVALID_ARG("axpy: shape mismatch {} vs {}", xm.shape().to_string(), ym.shape().to_string());
+        x[i] = fp(xm), y[i] = const_cast<float *>(fp(ym)), n[i] = (int64_t)xm.elements();
+    }
+    check(odl_hip_axpy_multi((int)count, a, x.data(), y.data(), n.data(), cur()));
+}
+
 std::unique_ptr<Mat> OriginMat::sgd_step(const Mat &grad, float lr) const
 {
     const OriginMat &p = dev_f32(*this, "sgd_step");

@@ -327,8 +327,7 @@ void Optimizer::step()
             with_grad.push_back(p);
     for (auto &h : hooks_)
         h(with_grad);
-    for (auto *p : with_grad)
-        step_one(*p);
+    step_all(with_grad);
 }
 
 void Optimizer::zero_grad()
@@ -397,6 +396,32 @@ void SGD::step_one(Parameter &param)
         param = as_leaf(param - grad * Scalar(lr_));
 }
 
+// The plain step (no momentum, no weight decay) over device parameters: one launch for the whole list.
+void SGD::step_all(std::vector<Parameter *> &params)
+{
+    bool fused = weight_decay_ <= 0.0f && momentum_ <= 0.0f && params.size() > 1;
+    for (auto *p : params)
+        fused = fused && OriginMat::device_f32(*p->impl_->data_) && OriginMat::device_f32(*p->grad().impl_->data_);
+    if (!fused)
+    {
+        Optimizer::step_all(params);
+        return;
+    }
+    NoGradGuard guard;
+    std::vector<std::pair<const Mat *, const Mat *>> list;
+    std::vector<Tensor> grads;  // keeps the gradients alive until the launch is queued
+    for (auto *p : params)
+    {
+        grads.push_back(p->grad());
+        list.emplace_back(p->impl_->data_.get(), grads.back().impl_->data_.get());
+    }
+    const bool in_place = cuda::is_capturing();
+    auto updated = OriginMat::sgd_step_multi(list, lr_, in_place);
+    if (!in_place)
+        for (size_t i = 0; i < params.size(); ++i)
+            *params[i] = as_leaf(Tensor(std::move(updated[i])));
+}
+
 Adam::Adam(Module &target, float lr, float beta1, float beta2, float eps)
     : Optimizer(target), lr_(lr), beta1_(beta1), beta2_(beta2), eps_(eps)
 {}
@@ -439,6 +464,61 @@ void Adam::step_one(Parameter &param)
                                                        m_hat_scale, v_hat_scale, eps_, lr_)));
 }
 
+// Device parameters take one launch for the whole list; the bookkeeping per parameter (buffers, step counts, factors)
+// is that of step_one.
+void Adam::step_all(std::vector<Parameter *> &params)
+{
+    bool fused = params.size() > 1;
+    for (auto *p : params)
+        fused = fused && OriginMat::device_f32(*p->impl_->data_) && OriginMat::device_f32(*p->grad().impl_->data_);
+    if (!fused)
+    {
+        Optimizer::step_all(params);
+        return;
+    }
+    NoGradGuard guard;
+    const bool capturing = cuda::is_capturing();
+    std::vector<OriginMat::AdamItem> items;
+    std::vector<Tensor> grads;
+    for (auto *pp : params)
+    {
+        Parameter &param = *pp;
+        grads.push_back(param.grad());
+        const Tensor &grad = grads.back();
+        auto zeros = [&] { return Tensor::zeros(grad.shape(), TensorOptions(grad.dtype()).device(grad.device())); };
+        if (!m_buffers_.count(&param))
+            m_buffers_.emplace(&param, zeros());
+        if (!v_buffers_.count(&param))
+            v_buffers_.emplace(&param, zeros());
+        if (!replay_scales_.defined())
+            replay_scales_ = Tensor::zeros(Shape{parameters_.size(), 2}, TensorOptions(DataType::kFloat32).device(grad.device()));
+        OriginMat::AdamItem it{};
+        it.param = param.impl_->data_.get(), it.grad = grad.impl_->data_.get();
+        it.m = m_buffers_.at(&param).impl_->data_.get(), it.v = v_buffers_.at(&param).impl_->data_.get();
+        if (capturing)
+        {
+            if (!step_counts_.count(&param))
+                THROW_RUNTIME_ERROR("Adam: run one ordinary step before capturing (the moment buffers must exist)");
+            size_t index = 0;
+            while (index < parameters_.size() && parameters_[index] != &param)
+                ++index;
+            it.device_scales = static_cast<const OriginMat &>(*replay_scales_.impl_->data_).data_ptr<float>() + 2 * index;
+            replay_params_.push_back(&param);
+        }
+        else
+        {
+            const int t = ++step_counts_[&param];
+            const float b1p = std::pow(beta1_, static_cast<float>(t)), b2p = std::pow(beta2_, static_cast<float>(t));
+            it.m_hat_scale = 1.0f / (1.0f - b1p), it.v_hat_scale = 1.0f / (1.0f - b2p);
+        }
+        items.push_back(it);
+    }
+    auto updated = OriginMat::adam_step_multi(items, beta1_, beta2_, eps_, lr_, capturing);
+    if (!capturing)
+        for (size_t i = 0; i < params.size(); ++i)
+            *params[i] = as_leaf(Tensor(std::move(updated[i])));
+}
+
 void Adam::prepare_replay()
 {
     if (replay_params_.empty())
@@ -461,19 +541,26 @@ std::function<void(std::vector<Parameter *> &)> WeightDecay::hook() const
     const float rate = rate_;
     return [rate](std::vector<Parameter *> &params) {
         NoGradGuard guard;
+        // grad += rate * param: one launch for all parameters that live on the device (the product is rounded, then
+        // added — what the separate multiply and accumulate give)
+        std::vector<std::pair<const Mat *, Mat *>> on_device;
+        std::vector<Tensor> grads;
         for (auto *p : params)
         {
             if (!p)
                 continue;
-            // grad += rate * param: one launch when both live on the device (the product is rounded, then added —
-            // what the separate multiply and accumulate give)
             Tensor g = p->grad();
-            if (g.defined() && g.device().type() == DeviceType::kCUDA && g.dtype() == DataType::kFloat32 &&
+            if (g.defined() && OriginMat::device_f32(*g.impl_->data_) && OriginMat::device_f32(*p->impl_->data_) &&
                 g.shape() == p->shape())
-                static_cast<OriginMat &>(*g.impl_->data_).axpy_inplace(rate, *p->impl_->data_);
+            {
+                grads.push_back(g);
+                on_device.emplace_back(p->impl_->data_.get(), g.impl_->data_.get());
+            }
             else
                 p->accumulate_grad(static_cast<const Tensor &>(*p) * Scalar(rate));
         }
+        if (!on_device.empty())
+            OriginMat::axpy_multi(rate, on_device);
     };
 }
 

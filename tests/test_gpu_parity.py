@@ -642,6 +642,55 @@ def test_fused_optimizer_steps_match_the_op_by_op_sequence(api, o):
     np.testing.assert_allclose(out, b64 - 1e-3 * b64 / (np.abs(b64) + 1e-8), rtol=0, atol=3e-7)
 
 
+def test_multi_tensor_optimizer_steps_are_the_single_tensor_steps(api):
+    """One launch over a list of parameters gives, tensor by tensor, the bits of the one-tensor entry points: sizes from
+    one element to more than one workgroup's share, odd sizes (scalar tails), more tensors than one launch carries, and
+    an empty tensor in the list."""
+    import torch
+    rng = np.random.default_rng(29)
+    sizes = [1, 3, 10, 128, 1000, 1024, 1025, 784 * 100, 4097, 0, 7] + [33 + i for i in range(30)]
+    p = [rng.standard_normal(n, dtype=f32) for n in sizes]
+    g = [rng.standard_normal(n, dtype=f32) * f32(0.1) for n in sizes]
+    m = [rng.standard_normal(n, dtype=f32) * f32(0.05) for n in sizes]
+    v = [np.abs(rng.standard_normal(n, dtype=f32)) * f32(0.01) for n in sizes]
+    ts = [1 + (i % 5) for i in range(len(sizes))]
+    live = [i for i, n in enumerate(sizes) if n > 0]
+    # Adam
+    dm, dv = [dev(x) for x in m], [dev(x) for x in v]
+    outs = api.adam_step_multi([dev(x) for x in p], [dev(x) for x in g], dm, dv, ts, lr=2e-3)
+    for i in live:
+        sm, sv = dev(m[i]), dev(v[i])
+        want = api.adam_step(dev(p[i]), dev(g[i]), sm, sv, ts[i], lr=2e-3)
+        assert np.array_equal(host(outs[i]), host(want)), sizes[i]
+        assert np.array_equal(host(dm[i]), host(sm)) and np.array_equal(host(dv[i]), host(sv)), sizes[i]
+    # the factors read from device memory for some entries, from the host arrays for the others
+    fac = lambda t, b: f32(1.0) / (f32(1.0) - f32(np.power(f32(b), f32(t))))  # noqa: E731
+    scales = [dev(np.array([fac(3, 0.9), fac(3, 0.999)], f32)) if i % 2 == 0 else None for i in range(len(sizes))]
+    dm, dv = [dev(x) for x in m], [dev(x) for x in v]
+    outs = api.adam_step_multi([dev(x) for x in p], [dev(x) for x in g], dm, dv, ts, device_scales=scales)
+    for i in live[:12]:
+        want = api.adam_step(dev(p[i]), dev(g[i]), dev(m[i]), dev(v[i]), 3 if i % 2 == 0 else ts[i])
+        assert np.array_equal(host(outs[i]), host(want)), sizes[i]
+    # unaligned operands: views one float into their buffers take the scalar path
+    odd = [torch.empty(n + 1, dtype=torch.float32, device="cuda")[1:] for n in sizes]
+    for t, x in zip(odd, p):
+        t.copy_(torch.from_numpy(x))
+    outs = api.sgd_step_multi(odd, [dev(x) for x in g], 0.05)
+    for i in live:
+        assert np.array_equal(host(outs[i]), p[i] - g[i] * f32(0.05)), sizes[i]
+    outs = api.sgd_step_multi([dev(x) for x in p], [dev(x) for x in g], 0.05)
+    for i in live:
+        assert np.array_equal(host(outs[i]), host(api.sgd_step(dev(p[i]), dev(g[i]), 0.05))), sizes[i]
+    # weight decay: grad += rate * param
+    dg = [dev(x) for x in g]
+    api.axpy_multi(1e-4, [dev(x) for x in p], dg)
+    for i in live:
+        assert np.array_equal(host(dg[i]), g[i] + f32(1e-4) * p[i]), sizes[i]
+        assert np.array_equal(host(dg[i]), host(api.axpby(1.0, dev(g[i]), 1e-4, dev(p[i])))), sizes[i]
+    with pytest.raises(api.OdlInvalidArgument):
+        api.axpy_multi(0.5, [dev(p[3])], [dev(p[4])])
+
+
 # ------------------------------------------------------------------ detector forward path (config 5's operators)
 def test_sigmoid_silu_vs_oracle_and_fixtures(api, o):
     x = G["det_act_x"]
