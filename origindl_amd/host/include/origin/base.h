@@ -83,6 +83,14 @@ enum class DataType
     kUInt8   = 5,
 };
 
+// short names, as include/origin/mat/basic_types.h:29-34
+constexpr auto Float32 = DataType::kFloat32;
+constexpr auto Float64 = DataType::kFloat64;
+constexpr auto Int8    = DataType::kInt8;
+constexpr auto Int32   = DataType::kInt32;
+constexpr auto Int64   = DataType::kInt64;
+constexpr auto UInt8   = DataType::kUInt8;
+
 inline size_t dtype_size(DataType t)
 {
     switch (t)
@@ -163,6 +171,7 @@ public:
         return n;
     }
     const std::vector<size_t> &dims() const { return dims_; }
+    bool is_scalar() const { return dims_.empty(); }  // a 0-dim shape
     bool operator==(const Shape &o) const { return dims_ == o.dims_; }
     bool operator!=(const Shape &o) const { return dims_ != o.dims_; }
     std::string to_string() const
@@ -197,6 +206,11 @@ public:
     double to_float64() const { return is_float() ? f_ : (double)i_; }
     int32_t to_int32() const { return is_float() ? (int32_t)f_ : (int32_t)i_; }
     int64_t to_int64() const { return is_float() ? (int64_t)f_ : i_; }
+    template <typename T>
+    T to() const
+    {
+        return is_float() ? static_cast<T>(f_) : static_cast<T>(i_);
+    }
     bool is_float() const { return dtype_ == DataType::kFloat32 || dtype_ == DataType::kFloat64; }
 
 private:
@@ -234,6 +248,11 @@ public:
     DataType dtype() const { return dtype_; }
     Device device() const { return device_; }
     bool requires_grad() const { return requires_grad_; }
+    bool operator==(const TensorOptions &o) const
+    {
+        return dtype_ == o.dtype_ && device_ == o.device_ && requires_grad_ == o.requires_grad_;
+    }
+    bool operator!=(const TensorOptions &o) const { return !(*this == o); }
 
 private:
     DataType dtype_     = DataType::kFloat32;

@@ -5,12 +5,61 @@
 #pragma once
 #include <string>
 
+#include <initializer_list>
+#include <type_traits>
+
 #include "tensor.h"
+#include "utils/size_array_ref.h"
 
 namespace origin
 {
 namespace functional
 {
+// src/operators/shape/split.cpp: pieces of x along dim — either the listed sizes (which must add up to the dimension)
+// or equal pieces of split_size with a shorter last one; backward concatenates the pieces' gradients.
+class Split : public Operator
+{
+public:
+    int dim_;
+    std::vector<size_t> split_sizes_;
+    explicit Split(SizeArrayRef split_sizes, int dim = 0) : dim_(dim), split_sizes_(split_sizes.to_vector()) {}
+    explicit Split(size_t split_size, int dim = 0) : dim_(dim), split_sizes_{split_size} {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override;
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override;
+};
+std::vector<Tensor> split(const Tensor &x, SizeArrayRef split_sizes, int dim = 0);
+std::vector<Tensor> split(const Tensor &x, size_t split_size, int dim = 0);
+// braced lists of another integer type (split(x, {1, 2, 3}, 0) deduces int)
+template <typename T, typename = std::enable_if_t<std::is_integral<T>::value && !std::is_same<T, bool>::value &&
+                                                  !std::is_same<T, size_t>::value>>
+inline std::vector<Tensor> split(const Tensor &x, std::initializer_list<T> split_sizes, int dim = 0)
+{
+    std::vector<size_t> sizes;
+    for (const auto &v : split_sizes)
+        sizes.push_back(static_cast<size_t>(v));
+    return split(x, SizeArrayRef(sizes), dim);
+}
+
+// src/operators/custom/linear.cpp: y = flatten(x) . weight^T (+ bias) with weight laid out [out_features, in_features],
+// the layout of an imported model's fully connected layers. Forward only (backward throws, as there).
+class LinearOp : public Operator
+{
+public:
+    int in_features_, out_features_;
+    bool use_bias_;
+    LinearOp(int in_features, int out_features, bool use_bias = true)
+        : in_features_(in_features), out_features_(out_features), use_bias_(use_bias)
+    {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override;
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override;
+};
+Tensor custom_linear(const Tensor &x, const Tensor &weight, const Tensor &bias, int in_features, int out_features,
+                     bool use_bias = true);
+Tensor custom_linear(const Tensor &x, const Tensor &weight, int in_features, int out_features);
+
+// src/operators/activation/leaky_relu.cpp: x where x > 0, alpha*x elsewhere; gx = gy * (alpha + mask*(1-alpha))
+Tensor leaky_relu(const Tensor &x, float alpha = 0.01f);
+
 Tensor add(const Tensor &lhs, const Tensor &rhs);
 Tensor sub(const Tensor &lhs, const Tensor &rhs);
 Tensor mul(const Tensor &lhs, const Tensor &rhs);

@@ -146,6 +146,10 @@ public:
                                                      std::pair<int, int> stride, std::pair<int, int> pad,
                                                      const std::vector<size_t> &indices) const = 0;
     // ---- indexing
+    // one element by its coordinates (src/mat/origin/origin_mat.cpp:970-1039): on the device a synchronising copy of
+    // that element alone
+    virtual Scalar index(std::initializer_list<size_t> indices) const                   = 0;
+    virtual void index_put(std::initializer_list<size_t> indices, const Scalar &value) = 0;
     virtual std::unique_ptr<Mat> gather(const Mat &indices) const                   = 0;
     virtual std::unique_ptr<Mat> one_hot(const Mat &indices, int num_classes) const = 0;
 };
@@ -175,6 +179,8 @@ public:
     Shape shape() const override { return shape_; }
     size_t elements() const override { return shape_.elements(); }
     bool is_scalar() const override { return shape_.elements() == 1; }
+    Scalar index(std::initializer_list<size_t> indices) const override;
+    void index_put(std::initializer_list<size_t> indices, const Scalar &value) override;
     Scalar scalar_value() const override;
     void *data_ptr() override { return storage_->data(); }
     int backend_type() const override { return ORIGIN_BACKEND_TYPE; }

@@ -71,6 +71,7 @@ public:
         if (data.size() != shape.elements())
             throw std::invalid_argument("Data size (" + std::to_string(data.size()) + ") does not match shape elements (" +
                                         std::to_string(shape.elements()) + ")");
+        check_extents(shape);
         init(Mat_t::from_memory(data.data(), DataTypeTraits<T>::type, shape, options), options);
     }
     template <typename T>
@@ -91,6 +92,7 @@ public:
     {}
     Tensor(const Scalar &scalar, const Shape &shape, const TensorOptions &options)
     {
+        check_extents(shape);
         init(Mat_t::from_scalar(scalar, shape, options), options);
     }
 
@@ -98,11 +100,34 @@ public:
     static Tensor ones(const Shape &shape, const TensorOptions &options = TensorOptions());
     static Tensor randn(const Shape &shape, const TensorOptions &options = TensorOptions());
     static Tensor full(const Shape &shape, const Scalar &value, const TensorOptions &options = TensorOptions());
+    // a tensor holding a copy of shape.elements() values of options.dtype() read from host memory (src/core/tensor.cpp:72-78)
+    static Tensor from_blob(void *data, const Shape &shape, const TensorOptions &options = TensorOptions());
 
     Shape shape() const;
     size_t ndim() const { return shape().size(); }
     size_t elements() const { return shape().elements(); }
     size_t numel() const { return elements(); }
+    size_t element_size() const { return dtype_size(dtype()); }
+    size_t nbytes() const { return elements() * element_size(); }
+    // the element buffer as it lies: host memory for a CPU tensor, device memory for a device tensor
+    template <typename T>
+    T *data_ptr()
+    {
+        check_defined("data_ptr");
+        return static_cast<T *>(impl_->data_->data_ptr());
+    }
+    // one element by its coordinates; on the device a synchronising copy of that element
+    template <typename T>
+    T index(std::initializer_list<size_t> indices) const
+    {
+        check_defined("index");
+        return impl_->data_->index(indices).template to<T>();
+    }
+    void index_put(std::initializer_list<size_t> indices, const Scalar &value)
+    {
+        check_defined("index_put");
+        impl_->data_->index_put(indices, value);
+    }
     DataType dtype() const;
     Device device() const;
     bool defined() const { return impl_ && impl_->data_; }
@@ -149,6 +174,14 @@ private:
     {
         impl_                 = std::make_shared<TensorImpl>(std::move(m));
         impl_->requires_grad_ = options.requires_grad();
+    }
+    // a 0-dim shape is a scalar tensor; an extent of zero is refused (src/core/tensor.cpp:399-437)
+    static void check_extents(const Shape &shape)
+    {
+        for (size_t i = 0; i < shape.size(); ++i)
+            if (shape[i] == 0)
+                THROW_INVALID_ARG("Tensor shape cannot have zero dimensions. Dimension {} is zero in shape {}", i,
+                                  shape.to_string());
     }
     void check_defined(const char *who) const
     {

@@ -247,7 +247,7 @@ struct ReLU : Operator
 // Linear::forward's matmul + broadcast_to + add (src/nn/layers/linear.cpp:88-104) as one operator for 2-D inputs:
 // the bias is added in the product's epilogue, and backward is the three gradients those operators would produce
 // (gx = gy.W^T, gW = x^T.gy, gb = gy summed to the bias's shape).
-struct LinearOp : Operator
+struct FusedLinear : Operator
 {
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
@@ -257,6 +257,35 @@ struct LinearOp : Operator
     {
         auto g = OriginMat::matmul_backward_2d(mat(inputs_[0]), mat(inputs_[1]), mat(gys[0]));
         return {wrap(std::move(g.first)), wrap(std::move(g.second)), wrap(mat(gys[0]).sum_to(inputs_[2].shape()))};
+    }
+};
+
+// src/operators/activation/leaky_relu.cpp:17-72. Forward from the operations at hand, exact in both branches:
+// r = relu(x); y = r + alpha*(x - r) — where x > 0 that is x + alpha*0, elsewhere 0 + alpha*x. Backward as there:
+// gy * (alpha + mask*(1-alpha)) with mask = (x > 0).
+struct LeakyReLU : Operator
+{
+    float alpha;
+    explicit LeakyReLU(float a) : alpha(a) {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        if (xs.size() != 1)
+            THROW_RUNTIME_ERROR("LeakyReLU operator requires exactly 1 input, but got {}", xs.size());
+        const Mat &x = mat(xs[0]);
+        auto r       = x.relu();
+        auto rest    = x - *r;
+        auto scaled  = *rest * mat(scalar_like(Scalar(alpha), xs[0]));
+        return {wrap(*r + *scaled)};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        if (gys.size() != 1)
+            THROW_RUNTIME_ERROR("LeakyReLU backward requires exactly 1 gradient, but got {}", gys.size());
+        const Tensor &x = inputs_[0];
+        auto mask   = mat(x) > mat(scalar_like(Scalar(0.0f), x));
+        auto scaled = *mask * mat(scalar_like(Scalar(1.0f - alpha), x));
+        auto slope  = *scaled + mat(scalar_like(Scalar(alpha), x));
+        return {wrap(mat(gys[0]) * *slope)};
     }
 };
 
@@ -505,6 +534,130 @@ Tensor apply(const std::vector<Tensor> &xs, A &&...args)
 }
 }  // namespace
 
+// ---- Split (src/operators/shape/split.cpp:14-128)
+std::vector<Tensor> Split::forward(const std::vector<Tensor> &xs)
+{
+    if (xs.size() != 1)
+        THROW_RUNTIME_ERROR("Split operator requires exactly 1 input, but got {}", xs.size());
+    const Shape shape = xs[0].shape();
+    if (dim_ < 0 || (size_t)dim_ >= shape.size())
+        THROW_INVALID_ARG("Split: dim {} is out of range for input shape {}", dim_, shape.to_string());
+    const size_t extent = shape[dim_];
+    std::vector<size_t> sizes;
+    if (split_sizes_.size() == 1 && split_sizes_[0] > 0)
+    {
+        // equal pieces, the last one takes what is left
+        const size_t piece = split_sizes_[0], count = (extent + piece - 1) / piece;
+        for (size_t i = 0; i < count; ++i)
+            sizes.push_back(i + 1 < count ? piece : extent - (count - 1) * piece);
+    }
+    else
+    {
+        sizes = split_sizes_;
+        size_t total = 0;
+        for (size_t s : sizes)
+            total += s;
+        if (total != extent)
+            THROW_INVALID_ARG("Split: sum of split_sizes {} does not match dimension size {} at dim {}", total, extent, dim_);
+    }
+    std::vector<Tensor> out;
+    for (auto &piece : mat(xs[0]).split(sizes, dim_))
+        out.push_back(wrap(std::move(piece)));
+    return out;
+}
+
+std::vector<Tensor> Split::backward(const std::vector<Tensor> &gys)
+{
+    if (gys.empty())
+        THROW_RUNTIME_ERROR("Split backward requires at least 1 gradient, but got 0");
+    if (gys.size() == 1)
+        return gys;
+    const Shape first = gys[0].shape();
+    std::vector<const Mat *> others;
+    for (size_t i = 1; i < gys.size(); ++i)
+    {
+        const Shape s = gys[i].shape();
+        if (s.size() != first.size())
+            THROW_RUNTIME_ERROR("Split backward: all gradients must have same number of dimensions");
+        for (size_t d = 0; d < s.size(); ++d)
+            if (d != (size_t)dim_ && s[d] != first[d])
+                THROW_RUNTIME_ERROR("Split backward: dimension {} mismatch: {} vs {}", d, s[d], first[d]);
+        if (gys[i].device() != gys[0].device())
+            THROW_RUNTIME_ERROR("Split backward: device mismatch at gradient {}, expected {}, got {}", i,
+                                gys[0].device().to_string(), gys[i].device().to_string());
+        others.push_back(&mat(gys[i]));
+    }
+    return {wrap(mat(gys[0]).cat(others, dim_))};
+}
+
+std::vector<Tensor> split(const Tensor &x, SizeArrayRef split_sizes, int dim)
+{
+    auto op = std::make_shared<Split>(split_sizes, dim);
+    return (*op)(std::vector<Tensor>{x});
+}
+
+std::vector<Tensor> split(const Tensor &x, size_t split_size, int dim)
+{
+    auto op = std::make_shared<Split>(split_size, dim);
+    return (*op)(std::vector<Tensor>{x});
+}
+
+// ---- LinearOp (src/operators/custom/linear.cpp:12-110)
+std::vector<Tensor> LinearOp::forward(const std::vector<Tensor> &xs)
+{
+    const size_t expected = use_bias_ ? 3 : 2;
+    if (xs.size() != expected)
+        THROW_RUNTIME_ERROR("Linear operator requires {} inputs (x, weight{}), but got {}", expected,
+                            use_bias_ ? ", bias" : "", xs.size());
+    const Shape xs0 = xs[0].shape(), ws = xs[1].shape();
+    std::unique_ptr<Mat> flat;  // [batch, everything else]
+    const Mat *x2 = &mat(xs[0]);
+    if (xs0.size() > 2)
+    {
+        size_t features = 1;
+        for (size_t i = 1; i < xs0.size(); ++i)
+            features *= xs0[i];
+        flat = x2->reshape(Shape{xs0[0], features});
+        x2   = flat.get();
+    }
+    if (x2->shape().size() != 2)
+        THROW_RUNTIME_ERROR("Linear forward: x must be 2D after flattening, but got shape {}", x2->shape().to_string());
+    if (ws.size() != 2)
+        THROW_RUNTIME_ERROR("Linear forward: weight must be 2D (out_features, in_features), but got shape {}", ws.to_string());
+    if (x2->shape()[1] != ws[1])
+        THROW_RUNTIME_ERROR("Linear forward: feature mismatch - x has {} features, but weight expects {} features",
+                            x2->shape()[1], ws[1]);
+    if (ws[0] != (size_t)out_features_)
+        THROW_RUNTIME_ERROR("Linear forward: output feature mismatch - weight has {} out_features, but expected {}", ws[0],
+                            out_features_);
+    auto wt = mat(xs[1]).transpose();
+    auto y  = x2->matmul(*wt);
+    if (use_bias_)
+    {
+        auto b = mat(xs[2]).broadcast_to(y->shape());
+        y      = *y + *b;
+    }
+    return {wrap(std::move(y))};
+}
+
+std::vector<Tensor> LinearOp::backward(const std::vector<Tensor> &)
+{
+    THROW_RUNTIME_ERROR("LinearOp backward is not implemented");
+}
+
+Tensor custom_linear(const Tensor &x, const Tensor &weight, const Tensor &bias, int in_features, int out_features, bool use_bias)
+{
+    auto op = std::make_shared<LinearOp>(in_features, out_features, use_bias);
+    return use_bias ? (*op)(std::vector<Tensor>{x, weight, bias})[0] : (*op)(std::vector<Tensor>{x, weight})[0];
+}
+
+Tensor custom_linear(const Tensor &x, const Tensor &weight, int in_features, int out_features)
+{
+    return custom_linear(x, weight, Tensor(), in_features, out_features, false);
+}
+
+Tensor leaky_relu(const Tensor &x, float alpha) { return apply<LeakyReLU>({x}, alpha); }
+
 Tensor add(const Tensor &a, const Tensor &b) { return apply<Add>({a, b}); }
 Tensor sub(const Tensor &a, const Tensor &b) { return apply<Sub>({a, b}); }
 Tensor mul(const Tensor &a, const Tensor &b) { return apply<Mul>({a, b}); }
@@ -554,7 +707,7 @@ Tensor batch_norm(const Tensor &x, const Tensor &gamma, const Tensor &beta, cons
 {
     return batch_norm_outputs(x, gamma, beta, rm, rv, training, eps, momentum, num_dims)[0];
 }
-Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b) { return apply<LinearOp>({x, w, b}); }
+Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b) { return apply<FusedLinear>({x, w, b}); }
 Tensor softmax(const Tensor &x, int axis) { return apply<Softmax>({x}, axis); }
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &t) { return apply<SoftmaxCrossEntropy>({x, t}); }
 

@@ -529,6 +529,73 @@ Scalar OriginMat::scalar_value() const
     }
 }
 
+namespace
+{
+// element offset of a coordinate list in a contiguous tensor; the checks and messages of origin_mat.cpp:970-990
+size_t element_offset(const Shape &shape, std::initializer_list<size_t> indices)
+{
+    if (indices.size() != shape.size())
+        THROW_INVALID_ARG("Index count ({}) does not match tensor dimension ({}). Shape: {}", indices.size(), shape.size(),
+                          shape.to_string());
+    size_t offset = 0, i = 0;
+    for (size_t idx : indices)
+    {
+        if (idx >= shape[i])
+            THROW_INVALID_ARG("Index {} out of range for dimension {} (size: {}). Shape: {}", idx, i, shape[i],
+                              shape.to_string());
+        offset = offset * shape[i] + idx;
+        ++i;
+    }
+    return offset;
+}
+}  // namespace
+
+Scalar OriginMat::index(std::initializer_list<size_t> indices) const
+{
+    const size_t offset = element_offset(shape_, indices), width = dtype_size(dtype_);
+    alignas(8) char element[8];
+    const char *src = static_cast<const char *>(storage_->data()) + offset * width;
+    if (storage_->device_type() == DeviceType::kCPU)
+        std::memcpy(element, src, width);
+    else
+    {
+        no_capture("device-to-host copy");
+        check(odl_hip_synchronize());
+        check(odl_hip_memcpy_d2h(element, src, width));
+    }
+    const double v = load_as(element, dtype_, 0);
+    switch (dtype_)
+    {
+        case DataType::kFloat32: return Scalar((float)v);
+        case DataType::kFloat64: return Scalar(v);
+        case DataType::kInt64: return Scalar((int64_t)v);
+        default: return Scalar((int)v);
+    }
+}
+
+void OriginMat::index_put(std::initializer_list<size_t> indices, const Scalar &value)
+{
+    const size_t offset = element_offset(shape_, indices), width = dtype_size(dtype_);
+    alignas(8) char element[8];
+    const double v = value.to_float64();
+    if (dtype_ == DataType::kInt64)  // keeps all 64 bits
+    {
+        const int64_t w = value.to_int64();
+        std::memcpy(element, &w, sizeof(w));
+    }
+    else
+        store_as(element, dtype_, &v, 1);
+    char *dst = static_cast<char *>(storage_->data()) + offset * width;
+    if (storage_->device_type() == DeviceType::kCPU)
+        std::memcpy(dst, element, width);
+    else
+    {
+        no_capture("host-to-device copy");
+        check(odl_hip_synchronize());
+        check(odl_hip_memcpy_h2d(dst, element, width));
+    }
+}
+
 std::unique_ptr<Mat> OriginMat::to(DataType target) const
 {
     if (target == dtype_)

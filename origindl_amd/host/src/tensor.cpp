@@ -149,6 +149,15 @@ Tensor Tensor::full(const Shape &s, const Scalar &v, const TensorOptions &o)
     return t;
 }
 
+Tensor Tensor::from_blob(void *data, const Shape &s, const TensorOptions &o)
+{
+    if (!data)
+        THROW_INVALID_ARG("from_blob: null data");
+    Tensor t(Mat_t::from_memory(data, o.dtype(), s, o));
+    t.impl_->requires_grad_ = o.requires_grad();
+    return t;
+}
+
 void Tensor::upload(const void *host, size_t bytes)
 {
     check_defined("upload");
@@ -157,7 +166,8 @@ void Tensor::upload(const void *host, size_t bytes)
 
 Shape Tensor::shape() const
 {
-    return defined() ? impl_->data_->shape() : Shape();
+    check_defined("shape");  // src/core/tensor.cpp:82-86: metadata of an undefined tensor throws
+    return impl_->data_->shape();
 }
 DataType Tensor::dtype() const
 {
