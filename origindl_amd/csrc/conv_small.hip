@@ -87,6 +87,95 @@ __global__ __launch_bounds__(kThreads) void conv_small_fwd_kernel(const float *_
     }
 }
 
+// The same convolution for the larger windows (5x5, 6x6): there the filter no longer fits the scalar registers, and
+// reading it through them in pieces leaves the wave waiting on one short load after another. The workgroup stages its
+// OCB channels' filter in LDS once, as [c][tap][oc], and every lane reads it from there 16 bytes at a time (one address
+// for the whole wave); a thread computes two output pixels, half the grid apart, so that each filter read feeds two
+// multiply-adds. Per output the terms are added in the same order as in the kernel above.
+template <int KH, int KW, int OCB>
+__global__ __launch_bounds__(kThreads) void conv_small_fwd_lds_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                                     const float *__restrict__ bias, float *__restrict__ y,
+                                                                     SmallGeom g, int act, unsigned half)
+{
+    constexpr int KK = KH * KW;
+    extern __shared__ __attribute__((aligned(16))) float wl[];  // [C][KK][OCB]
+    const int oc0 = blockIdx.y * OCB;
+    for (int e = threadIdx.x; e < g.C * KK * OCB; e += kThreads)
+    {
+        const int o = e % OCB, ck = e / OCB;
+        wl[e] = w[(size_t)(oc0 + o) * g.C * KK + ck];
+    }
+    __syncthreads();
+    const unsigned first = blockIdx.x * kThreads + threadIdx.x;
+    bool live[2];
+    unsigned n[2], oh[2], ow[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+    {
+        const unsigned pix = first + p * half;
+        live[p] = first < half && pix < g.total;
+        const unsigned pp = live[p] ? pix : 0;
+        const unsigned t = odl::fastdiv(pp, g.by_w);
+        ow[p] = pp - t * g.OW;
+        n[p] = odl::fastdiv(t, g.by_h);
+        oh[p] = t - n[p] * g.OH;
+    }
+    float acc[2][OCB];
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int o = 0; o < OCB; ++o)
+            acc[p][o] = 0.f;
+    for (int c = 0; c < g.C; ++c)
+    {
+        float xr[2][KK];
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+        {
+            const float *xp = x + ((size_t)n[p] * g.C + c) * g.H * g.W;
+            const int ih0 = (int)oh[p] * g.SH - g.PH, iw0 = (int)ow[p] * g.SW - g.PW;
+#pragma unroll
+            for (int kh = 0; kh < KH; ++kh)
+#pragma unroll
+                for (int kw = 0; kw < KW; ++kw)
+                {
+                    const int ih = ih0 + kh, iw = iw0 + kw;
+                    const bool in = live[p] && (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+                    xr[p][kh * KW + kw] = in ? xp[ih * g.W + iw] : 0.f;
+                }
+        }
+        const f32x4 *wc = reinterpret_cast<const f32x4 *>(wl + (size_t)c * KK * OCB);
+#pragma unroll
+        for (int k = 0; k < KK; ++k)
+#pragma unroll
+            for (int q = 0; q < OCB / 4; ++q)
+            {
+                const f32x4 wv = wc[k * (OCB / 4) + q];
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        acc[p][q * 4 + j] = fmaf(xr[p][k], wv[j], acc[p][q * 4 + j]);
+            }
+    }
+    const size_t plane = (size_t)g.OH * g.OW;
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+    {
+        if (!live[p])
+            continue;
+        float *yp = y + ((size_t)n[p] * g.OC + oc0) * plane + (size_t)oh[p] * g.OW + ow[p];
+#pragma unroll
+        for (int o = 0; o < OCB; ++o)
+        {
+            float v = acc[p][o];
+            if (bias)
+                v = v + bias[oc0 + o];
+            yp[o * plane] = odl::apply_act(v, act);
+        }
+    }
+}
+
 // gW[oc][k] = sum_m gy2d[m][oc] * col[m][k], col[m][(c,kh,kw)] = x[n][c][oh*SH-PH+kh][ow*SW-PW+kw] for m = (n,oh,ow).
 // A thread owns 8 consecutive channels of gy2d's rows m = first + i*rows_per_pass and all K = C*KH*KW columns: 8*K
 // private sums. G = OC/8 = 2^LGG neighbouring lanes share a row, so a wave reads whole rows of gy2d, 16 bytes a lane. At
@@ -364,6 +453,8 @@ bool conv_small_forward_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t O
     // few enough terms that the matrix units would mostly multiply padding: a short reduction, or a narrow output
     if (!(C * KH * KW <= 32 || (OC <= 16 && C <= 4)))
         return false;
+    if (C * KH * KW * 16 * 4 > 48 * 1024)  // the staged filter of the larger windows
+        return false;
     return small_sizes(N, C, H, W, OC, OH, OW);
 }
 
@@ -372,13 +463,22 @@ int conv_small_forward(const float *x, const float *w, const float *b, float *y,
                        hipStream_t st)
 {
     const SmallGeom g = make_small(N, C, H, W, OC, SH, SW, PH, PW, OH, OW, false);
-    const dim3 grid((unsigned)ceil_div(g.total, kThreads), (unsigned)(OC / 16));
     if (KH == 3)
+    {
+        const dim3 grid((unsigned)ceil_div(g.total, kThreads), (unsigned)(OC / 16));
         hipLaunchKernelGGL((conv_small_fwd_kernel<3, 3, 16>), grid, dim3(kThreads), 0, st, x, w, b, y, g, act);
-    else if (KH == 5)
-        hipLaunchKernelGGL((conv_small_fwd_kernel<5, 5, 16>), grid, dim3(kThreads), 0, st, x, w, b, y, g, act);
+    }
     else
-        hipLaunchKernelGGL((conv_small_fwd_kernel<6, 6, 16>), grid, dim3(kThreads), 0, st, x, w, b, y, g, act);
+    {
+        // two pixels a thread: the second one `half` pixels after the first
+        const unsigned half = (unsigned)ceil_div(g.total, 2);
+        const dim3 grid((unsigned)ceil_div(half, kThreads), (unsigned)(OC / 16));
+        const size_t lds = (size_t)C * KH * KW * 16 * sizeof(float);
+        if (KH == 5)
+            hipLaunchKernelGGL((conv_small_fwd_lds_kernel<5, 5, 16>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
+        else
+            hipLaunchKernelGGL((conv_small_fwd_lds_kernel<6, 6, 16>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
+    }
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
