@@ -140,6 +140,35 @@ def extras(torch, capi, steps, warmup):
         out[name + "_bias_grad"] = {"ms": ms_gb, "gbs": nb / ms_gb / 1e6, "frac_hbm": nb / ms_gb / 1e6 / PEAK_HBM_GBS}
         del x, w, b, gy, col, img, y, gx, gw
         keep.clear()
+    # The first layer of the CNN (config 4): one input channel, 32 filters — direct kernels, HBM bound. Algorithmic
+    # bytes: forward reads x and writes y; backward reads gy and x once and writes gx and gW.
+    N, C, H, OC = 256, 1, 28, 32
+    x, w, b, gy = rnd(N, C, H, H), rnd(OC, C, 3, 3) / 3.0, rnd(OC), rnd(N, OC, H, H)
+    geom = (N, C, H, H, OC, 3, 3, 1, 1, 1, 1)
+    y, gx, gw, gb = empty(N, OC, H, H), empty(N, C, H, H), empty(OC, C, 3, 3), empty(OC)
+    wf, nf = ws(L.query("odl_hip_conv2d_workspace_bytes", *geom))
+    wb, nbb = ws(L.query("odl_hip_conv2d_backward_workspace_bytes", *geom))
+    fwd = direct("odl_hip_conv2d", ptr(x), ptr(w), ptr(b), *geom, ptr(y), wf, nf, stream)
+    bwd = direct("odl_hip_conv2d_backward", ptr(gy), ptr(x), ptr(w), *geom, ptr(gx), ptr(gw), None, wb, nbb, stream)
+    ms_f, ms_b = time_region(torch, fwd, steps, warmup), time_region(torch, bwd, steps, warmup)
+    nb_f, nb_b = 4.0 * (x.numel() + y.numel()), 4.0 * (gy.numel() + 2 * x.numel() + gw.numel())
+    out["conv_first_layer_256x1x28x28_to_32"] = {
+        "fwd_ms": ms_f, "bwd_ms": ms_b, "fwd_gbs": nb_f / ms_f / 1e6, "bwd_gbs": nb_b / ms_b / 1e6,
+        "fwd_frac_hbm": nb_f / ms_f / 1e6 / PEAK_HBM_GBS, "bwd_frac_hbm": nb_b / ms_b / 1e6 / PEAK_HBM_GBS}
+    # its 2x2 max-pool: forward reads x, writes y and the uint64 indices; backward reads gy and the indices, writes gx
+    OHp = H // 2
+    yp, idx = empty(N, OC, OHp, OHp), torch.empty((N, OC, OHp, OHp), dtype=torch.int64, device="cuda")
+    gyp, gxp = rnd(N, OC, OHp, OHp), empty(N, OC, H, H)
+    pg = (N, OC, H, H, 2, 2, 2, 2, 0, 0)
+    pf = direct("odl_hip_max_pool2d", ptr(y), *pg, ptr(yp), ptr(idx), stream)
+    pb = direct("odl_hip_max_pool2d_backward", ptr(gyp), ptr(idx), *pg, ptr(gxp), stream)
+    ms_pf, ms_pb = time_region(torch, pf, steps, warmup), time_region(torch, pb, steps, warmup)
+    nb_p = 4.0 * y.numel() + 12.0 * yp.numel()
+    out["max_pool_2x2_256x32x28x28"] = {
+        "fwd_ms": ms_pf, "bwd_ms": ms_pb, "fwd_gbs": nb_p / ms_pf / 1e6, "bwd_gbs": nb_p / ms_pb / 1e6,
+        "fwd_frac_hbm": nb_p / ms_pf / 1e6 / PEAK_HBM_GBS, "bwd_frac_hbm": nb_p / ms_pb / 1e6 / PEAK_HBM_GBS}
+    del x, w, b, gy, y, gx, gw, yp, idx, gyp, gxp
+    keep.clear()
     # gradient reductions: the MLP's own shapes (launch-bound) and scaled shapes that can saturate HBM
     for name, shape in (("bias_grad_512x1000", (512, 1000)), ("bias_grad_16384x4096_scaled", (16384, 4096))):
         x, o = rnd(*shape), empty(1, shape[1])
