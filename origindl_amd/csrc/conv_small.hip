@@ -394,6 +394,129 @@ __global__ __launch_bounds__(kDgThreads) void conv_small_dgrad_kernel(const floa
     }
 }
 
+// The input gradient at stride 1, row-stationary: a workgroup owns a band of image rows of one image. First every row
+// of gy2d the band needs (the band's rows plus KH-1 rows of halo) is read exactly once — L lanes a row, 16 bytes each —
+// and turned into its KH*KW*C products gx_col[m][(c,kh,kw)] (per lane four multiply-adds a product, the L partial
+// products joined by DPP moves), which go to LDS; then one thread per image pixel adds the pixel's taps from LDS in
+// ascending (kh, kw) order, as col2im does. The per-pixel kernel above reads every gy2d row KH*KW times instead.
+constexpr int kBandThreads = 256, kBandRows = 4;  // rows in flight per lane group
+template <int C, int KH, int KW, int LGL>
+__global__ __launch_bounds__(kBandThreads) void conv_small_dgrad_band_kernel(const float *__restrict__ gy,
+                                                                            const float *__restrict__ wp,
+                                                                            float *__restrict__ gx, SmallGeom g, int band_h,
+                                                                            int nbands, int ldr)
+{
+    constexpr int L = 1 << LGL, KK = KH * KW;
+    constexpr int kPer = kBandThreads >> LGL;  // gy2d rows per pass of the workgroup
+    extern __shared__ float prod[];            // [rows of the band][ldr], ldr >= KK*C and odd
+    const int n = blockIdx.x / nbands, band = blockIdx.x - n * nbands;
+    const int h0 = band * band_h, h1 = (h0 + band_h < g.H) ? h0 + band_h : g.H;
+    // output rows that reach the band: oh = ih + PH - kh
+    const int r0 = (h0 + g.PH - (KH - 1) > 0) ? h0 + g.PH - (KH - 1) : 0;
+    const int r1 = (h1 + g.PH < g.OH) ? h1 + g.PH : g.OH;
+    const int nrows = (r1 > r0 ? r1 - r0 : 0) * g.OW;
+    const int sub = threadIdx.x & (L - 1), grp = threadIdx.x >> LGL;
+    const f32x4 *gy4 = reinterpret_cast<const f32x4 *>(gy) + ((size_t)n * g.OH + r0) * g.OW * L;
+    f32x4 wv[KK][C];
+#pragma unroll
+    for (int tap = 0; tap < KK; ++tap)
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+            wv[tap][c] = reinterpret_cast<const f32x4 *>(wp)[(tap * C + c) * L + sub];
+    for (int rb = grp; rb < nrows; rb += kPer * kBandRows)
+    {
+        f32x4 v[kBandRows];
+#pragma unroll
+        for (int u = 0; u < kBandRows; ++u)
+        {
+            const int r = rb + u * kPer;
+            v[u] = gy4[(size_t)(r < nrows ? r : rb) * L + sub];
+        }
+#pragma unroll
+        for (int u = 0; u < kBandRows; ++u)
+        {
+            const int r = rb + u * kPer;
+#pragma unroll
+            for (int tap = 0; tap < KK; ++tap)
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                {
+                    const f32x4 wq = wv[tap][c];
+                    float s = v[u][0] * wq[0];
+                    s = fmaf(v[u][1], wq[1], s);
+                    s = fmaf(v[u][2], wq[2], s);
+                    s = fmaf(v[u][3], wq[3], s);
+                    if (LGL >= 1)
+                        s = dpp_add<kQuadSwap1>(s);
+                    if (LGL >= 2)
+                        s = dpp_add<kQuadSwap2>(s);
+                    if (LGL >= 3)
+                        s = dpp_add<kRowHalfMirror>(s);
+                    if (LGL >= 4)
+                        s = dpp_add<kRowMirror>(s);
+                    if (sub == 0 && r < nrows)
+                        prod[r * ldr + tap * C + c] = s;
+                }
+        }
+    }
+    __syncthreads();
+    const int npix = (h1 - h0) * g.W;
+    for (int p = threadIdx.x; p < npix; p += kBandThreads)
+    {
+        const int hl = (int)odl::fastdiv((unsigned)p, g.by_w), iw = p - hl * g.W;
+        const int ih = h0 + hl;
+        float acc[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+            acc[c] = 0.f;
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh)
+        {
+            const int oh = ih + g.PH - kh;
+            if (oh < r0 || oh >= r1)
+                continue;
+#pragma unroll
+            for (int kw = 0; kw < KW; ++kw)
+            {
+                const int ow = iw + g.PW - kw;
+                if (ow < 0 || ow >= g.OW)
+                    continue;
+                const float *q = prod + ((oh - r0) * g.OW + ow) * ldr + (kh * KW + kw) * C;
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                    acc[c] += q[c];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+            gx[(((size_t)n * C + c) * g.H + ih) * g.W + iw] = acc[c];
+    }
+}
+
+// band height for the kernel above (0: use the per-pixel kernel): about 512 workgroups, and a band's products within
+// 48 KB of LDS
+int band_height(const SmallGeom &g, int C, int KH, int KW, int &nbands, int &ldr)
+{
+    if (g.SH != 1 || g.SW != 1)
+        return 0;
+    ldr = (KH * KW * C) | 1;
+    int want = (int)odl::ceil_div(512, g.N);
+    if (want < 1)
+        want = 1;
+    if (want > g.H)
+        want = g.H;
+    for (nbands = want; nbands <= g.H; ++nbands)
+    {
+        const int bh = (int)odl::ceil_div(g.H, nbands);
+        if ((int64_t)(bh + KH - 1) * g.OW * ldr * (int64_t)sizeof(float) <= 48 * 1024)
+        {
+            nbands = (int)odl::ceil_div(g.H, bh);
+            return bh;
+        }
+    }
+    return 0;
+}
+
 bool aligned16(const void *p)
 {
     return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
@@ -563,8 +686,19 @@ int conv_small_dgrad(const float *gy, const float *w, float *gx, int64_t N, int6
     ODL_LAUNCH_CHECK();
     const int lgL = OC == 8 ? 1 : (OC == 16 ? 2 : (OC == 32 ? 3 : 4));
     const dim3 grid((unsigned)ceil_div(g.total, (int64_t)kDgPixels * (kDgThreads >> lgL)));
-#define ODL_SMALL_DGRAD(CV, KV, LG) \
-    hipLaunchKernelGGL((conv_small_dgrad_kernel<CV, KV, KV, LG>), grid, dim3(kDgThreads), 0, st, gy, wp, gx, g)
+    int nbands = 0, ldr = 0;
+    const int band_h = band_height(g, (int)C, KH, KW, nbands, ldr);
+    const dim3 band_grid((unsigned)(N * (band_h > 0 ? nbands : 1)));
+    const size_t band_lds = band_h > 0 ? (size_t)(band_h + KH - 1) * OW * ldr * sizeof(float) : 0;
+#define ODL_SMALL_DGRAD(CV, KV, LG)                                                                                     \
+    do                                                                                                                  \
+    {                                                                                                                   \
+        if (band_h > 0)                                                                                                 \
+            hipLaunchKernelGGL((conv_small_dgrad_band_kernel<CV, KV, KV, LG>), band_grid, dim3(kBandThreads), band_lds, \
+                               st, gy, wp, gx, g, band_h, nbands, ldr);                                                 \
+        else                                                                                                            \
+            hipLaunchKernelGGL((conv_small_dgrad_kernel<CV, KV, KV, LG>), grid, dim3(kDgThreads), 0, st, gy, wp, gx, g);  \
+    } while (0)
 #define ODL_SMALL_DGRAD_OC(CV, KV)      \
     do                                  \
     {                                   \

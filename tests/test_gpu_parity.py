@@ -307,12 +307,17 @@ def test_conv_vs_oracle_seeded(api, o, N, C, H, W, OC, KH, KW, s, p):
     np.testing.assert_allclose(host(gb), gbo, atol=1e-5 * np.sqrt(N * OH * OW) * np.abs(gy).max() * np.sqrt(N * OH * OW))
 
 
-def test_conv_full_size_c2_properties(api, o):
-    # BASELINE config C2: x[32,128,28,28] -> 256 channels, 3x3, stride 2, pad 1. The oracle checks a sample of
-    # output pixels (each is one dot product of a col row with a weight row); im2col/col2im adjointness and the
-    # bias-gradient identity hold at any size.
-    print("\n[case] conv C2 full size", flush=True)
-    N, C, H, OC, s, p = 32, 128, 28, 256, 2, 1
+@pytest.mark.parametrize("N,C,H,OC,s,p", [
+    (32, 64, 56, 128, 1, 1),    # BASELINE config C1
+    (32, 128, 28, 256, 2, 1),   # BASELINE config C2
+    (256, 1, 28, 32, 1, 1),     # the CNN's first layer at its batch size: the direct kernels
+    (256, 32, 14, 64, 1, 1),    # the CNN's second layer
+])
+def test_conv_full_size_properties(api, o, N, C, H, OC, s, p):
+    # BASELINE's convolutions at full size. The oracle checks a sample of output pixels (each is one dot product of a
+    # col row with a weight row); im2col/col2im adjointness and the bias-gradient identity hold at any size; the two
+    # gradients are checked against float64 GEMMs over the reference's reinterpreted gy.
+    print("\n[case] conv full size", N, C, H, OC, s, p, flush=True)
     g = torch.Generator(device="cuda").manual_seed(3)
     x = torch.randn((N, C, H, H), device="cuda", generator=g)
     w = torch.randn((OC, C, 3, 3), device="cuda", generator=g) * float(np.sqrt(2.0 / (C * 9)))
