@@ -285,6 +285,9 @@ public:
     // upstream gradient is read from device memory. For steps recorded into a graph; an out-of-range label is not
     // reported here (the flag stays on the device).
     std::unique_ptr<Mat> softmax_cross_entropy_device(const Mat &target) const;
+    // the device-resident loss, with the out-of-range-label flag read back and turned into the reference's exception
+    // (one small device-to-host copy; no upload of the loss afterwards)
+    std::unique_ptr<Mat> softmax_cross_entropy_checked(const Mat &target) const;
     std::unique_ptr<Mat> softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const;
     // overwrites this tensor's elements from host memory (synchronises first: work in flight may still read them)
     void upload(const void *host, size_t bytes);

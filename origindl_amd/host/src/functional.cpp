@@ -338,14 +338,17 @@ struct SoftmaxCrossEntropy : Operator  // src/operators/loss/softmax_cross_entro
                               x.shape()[0], t.shape()[0]);
         if (cuda::is_capturing())  // a recorded step cannot visit the host: the loss stays where it is computed
             return {wrap(omat(x).softmax_cross_entropy_device(mat(t)))};
-        const float loss = omat(x).softmax_cross_entropy(mat(t));  // synchronises, as the reference's .item() does
-        return {Tensor({loss}, Shape{}, dtype(DataType::kFloat32).device(x.device()))};
+        // synchronises once, as the reference's .item() does, to report an out-of-range label; the loss is not sent
+        // back up afterwards: it is the device scalar the kernel wrote
+        return {wrap(omat(x).softmax_cross_entropy_checked(mat(t)))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
         const Tensor &x = inputs_[0], &t = inputs_[1];
         std::unique_ptr<Mat> gx;
-        if (cuda::is_capturing())
+        // the upstream gradient is read where it lies when it is a float32 device scalar (no host round trip; gy/N
+        // is formed in the kernel as the host would form it)
+        if (cuda::is_capturing() || (OriginMat::device_f32(mat(gys[0])) && gys[0].elements() == 1))
             gx = omat(x).softmax_cross_entropy_backward_device(mat(t), mat(gys[0]));
         else
             gx = omat(x).softmax_cross_entropy_backward(mat(t), gys[0].item<float>());

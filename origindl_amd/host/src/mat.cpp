@@ -1369,6 +1369,19 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) 
     return std::make_unique<OriginMat>(std::move(storage), Shape{}, DataType::kFloat32);
 }
 
+std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target) const
+{
+    auto loss = softmax_cross_entropy_device(target);
+    // the loss word and the bad-label flag behind it come back together (this synchronises, as the reference's host-side
+    // divide does); the loss itself stays on the device for the operators that follow
+    unsigned words[2] = {0, 0};
+    no_capture("device-to-host copy");
+    check(odl_hip_memcpy_d2h(words, as_origin(*loss).storage()->data(), sizeof(words)));
+    if (words[1] != 0)
+        THROW_INVALID_ARG("gather: index out of range [0, {})", shape_[1]);
+    return loss;
+}
+
 std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const
 {
     const OriginMat &x = dev_f32(*this, "softmax_cross_entropy");
