@@ -282,6 +282,10 @@ CONV_SEEDED = [
     (5, 64, 7, 7, 48, 3, 3, 1, 1),     # more pixels than one tile column, C = 64
     (2, 3, 64, 64, 16, 6, 6, 2, 2),    # the detector's stem: 6x6, stride 2, pad 2, three channels (direct forward)
     (2, 32, 40, 40, 64, 3, 3, 2, 1),   # its down-sampling convolutions
+    (2, 16, 15, 13, 32, 3, 3, 2, 1),   # stride 2 over odd extents
+    (3, 8, 14, 14, 16, 3, 3, 2, 0),    # stride 2 without padding
+    (1, 4, 2, 2, 16, 3, 3, 2, 1),      # a 2x2 image under a 3x3 window at stride 2
+    (5, 130, 12, 12, 48, 3, 3, 2, 1),  # stride 2, more input channels than two row tiles hold
     (2, 64, 20, 20, 128, 1, 1, 1, 0),  # its 1x1 bottleneck convolutions
 ]
 
