@@ -698,6 +698,21 @@ def test_multi_tensor_optimizer_steps_are_the_single_tensor_steps(api):
         assert np.array_equal(host(dg[i]), host(api.axpby(1.0, dev(g[i]), 1e-4, dev(p[i])))), sizes[i]
     with pytest.raises(api.OdlInvalidArgument):
         api.axpy_multi(0.5, [dev(p[3])], [dev(p[4])])
+    # argument errors of the entry points themselves: a negative count, missing lists, a null tensor, a negative size
+    import ctypes
+    from origindl_amd import _lib
+    L = _lib.lib()
+    one = dev(p[4])
+    ptrs, sizes = (ctypes.c_void_p * 1)(one.data_ptr()), (ctypes.c_int64 * 1)(one.numel())
+    nulls, neg = (ctypes.c_void_p * 1)(None), (ctypes.c_int64 * 1)(-1)
+    for args in ((-1, ctypes.c_float(1.0), ptrs, ptrs, sizes, None), (1, ctypes.c_float(1.0), None, ptrs, sizes, None),
+                 (1, ctypes.c_float(1.0), nulls, ptrs, sizes, None), (1, ctypes.c_float(1.0), ptrs, ptrs, neg, None)):
+        assert L.cdll.odl_hip_axpy_multi(*args) == _lib.ODL_ERR_INVALID_ARG, args[0]
+    assert L.cdll.odl_hip_sgd_step_multi(1, ptrs, None, sizes, ctypes.c_float(0.1), ptrs, None) == _lib.ODL_ERR_INVALID_ARG
+    assert L.cdll.odl_hip_adam_step_multi(1, ptrs, ptrs, ptrs, ptrs, sizes, ctypes.c_float(0.9), ctypes.c_float(0.999), None,
+                                          None, None, ctypes.c_float(1e-8), ctypes.c_float(1e-3), ptrs,
+                                          None) == _lib.ODL_ERR_INVALID_ARG  # no bias-correction factors at all
+    assert L.cdll.odl_hip_axpy_multi(0, ctypes.c_float(1.0), None, None, None, None) == 0  # an empty list is a no-op
 
 
 # ------------------------------------------------------------------ detector forward path (config 5's operators)
