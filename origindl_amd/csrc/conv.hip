@@ -296,6 +296,9 @@ bool plan_im2col_tile(const ConvGeom &g, Im2colTile &t)
         CT = (int)g.C;
     if (CT >= 4)
         CT &= ~3;  // a multiple of four channels keeps every tile's columns 16-byte aligned
+    // a small problem gets narrower tiles: more workgroups in flight matter more than longer runs per store
+    while (CT >= 8 && odl::ceil_div(M, 64) * odl::ceil_div(g.C, CT) < 1536)
+        CT = (CT / 2) & ~3;
     t.CT = CT;
     t.ctiles = (int)odl::ceil_div(g.C, CT);
     t.LS = (int)(CT * KHW) | 1;
