@@ -116,6 +116,18 @@ int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, in
 int odl_hip_conv2d_act(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
                        int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int activation, float *y,
                        void *workspace, size_t workspace_bytes, void *stream);
+/* The same forward for weights that do not change between calls (inference): some shapes read the filter in another
+ * order, [OC][tap][C], and odl_hip_conv2d / _act write that copy into the workspace on every call. A caller that keeps
+ * its weights can make the copy once — packed_weights_bytes says how large it is for a shape (0: this shape reads the
+ * filter as it lies and `packed` is ignored), pack_weights fills it — and pass it to conv2d_act_packed, which then
+ * skips the copy. packed = NULL is odl_hip_conv2d_act. No counterpart in the reference (its runner re-uploads the
+ * weights on every forward, src/pnnx/pnnx_graph.cpp:341-405). */
+size_t odl_hip_conv2d_packed_weights_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                                           int SW, int PH, int PW);
+int odl_hip_conv2d_pack_weights(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, void *stream);
+int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packed, const float *b, int64_t N, int64_t C,
+                              int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW,
+                              int activation, float *y, void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
                                       int SH, int SW, int PH, int PW);
 /* Mat::conv2d_backward (mat.h:505; conv2d.cpp:514-599) -> gx, gW and (when gb != NULL) gb.

@@ -184,7 +184,21 @@ def col2im(col, input_shape, kernel_size, stride, pad, to_matrix=True):
     return img
 
 
-def conv2d(x, w, b=None, stride=1, pad=0, activation=None):
+def conv2d_pack_weights(x_shape, w, stride=1, pad=0):
+    """The filter copy, in the order the forward kernel for inputs of x_shape reads it, for weights that stay the same
+    from call to call; None when that kernel reads the filter as it lies. Pass it to conv2d(packed=...)."""
+    _chk(w, "W")
+    N, C, H, W = (int(d) for d in x_shape)
+    OC, _, KH, KW = w.shape
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    if lib().query("odl_hip_conv2d_packed_weights_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW) == 0:
+        return None
+    packed = _empty(w.shape)
+    lib().call("odl_hip_conv2d_pack_weights", _p(w), C, OC, KH, KW, _p(packed), _stream())
+    return packed
+
+
+def conv2d(x, w, b=None, stride=1, pad=0, activation=None, packed=None):
     """Mat::conv2d (src/mat/origin/cpu/conv/conv2d.cpp:404-512); activation "relu" / "silu" runs in the epilogue."""
     _chk(x, "x"), _chk(w, "W")
     if x.dim() != 4:
@@ -202,8 +216,8 @@ def conv2d(x, w, b=None, stride=1, pad=0, activation=None):
     y = _empty((N, OC, _builtins.max(OH, 0), _builtins.max(OW, 0)))
     ws, nb = _ws(lib().query("odl_hip_conv2d_workspace_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW))
     act = -1 if activation is None else _UN[activation]
-    lib().call("odl_hip_conv2d_act", _p(x), _p(w), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, act, _p(y), _p(ws),
-               nb, _stream())
+    lib().call("odl_hip_conv2d_act_packed", _p(x), _p(w), _p(packed), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, act,
+               _p(y), _p(ws), nb, _stream())
     return y
 
 

@@ -28,7 +28,9 @@ size_t conv_implicit_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, i
 size_t conv_implicit_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW, int64_t pixels);
 int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
-                          int act, void *workspace, size_t workspace_bytes, hipStream_t st);
+                          int act, void *workspace, size_t workspace_bytes, hipStream_t st, const float *packed = nullptr);
+size_t conv_implicit_forward_packed_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW);
+int conv_implicit_forward_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, hipStream_t st);
 size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
                                        int64_t OH, int64_t OW);
 int conv_implicit_wgrad(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W,
@@ -834,6 +836,33 @@ int odl_hip_conv2d_act(const float *x, const float *w, const float *b, int64_t N
                        int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int activation, float *y,
                        void *workspace, size_t workspace_bytes, void *stream)
 {
+    return odl_hip_conv2d_act_packed(x, w, nullptr, b, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, activation, y, workspace,
+                                     workspace_bytes, stream);
+}
+
+size_t odl_hip_conv2d_packed_weights_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                                           int SW, int PH, int PW)
+{
+    if (KH <= 0 || KW <= 0 || SH <= 0 || SW <= 0)
+        return 0;
+    const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
+    if (OH <= 0 || OW <= 0 || odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, OH, OW) ||
+        !odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW))
+        return 0;
+    return odl::conv_implicit_forward_packed_bytes(N, C, H, W, OC, KH, KW);
+}
+
+int odl_hip_conv2d_pack_weights(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(w && packed && C > 0 && OC > 0 && KH > 0 && KW > 0, "conv2d_pack_weights: bad argument");
+    return odl::conv_implicit_forward_pack(w, C, OC, KH, KW, packed, odl::as_stream(stream));
+}
+
+int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packed, const float *b, int64_t N, int64_t C,
+                              int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW,
+                              int activation, float *y, void *workspace, size_t workspace_bytes, void *stream)
+{
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(activation == -1 || activation == 0 || activation == 7,
                 "conv2d: activation must be -1 (none), 0 (relu) or 7 (silu), the unary operator numbers; got %d", activation);
@@ -851,7 +880,8 @@ int odl_hip_conv2d_act(const float *x, const float *w, const float *b, int64_t N
         return odl::conv_small_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, act, st);
     if (odl::conv_implicit_forward_ok(w, N, C, H, W, OC, KH, KW, g.OH, g.OW))
         return odl::conv_implicit_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, act, workspace,
-                                          workspace_bytes, st);
+                                          workspace_bytes, st,
+                                          (packed && reinterpret_cast<uintptr_t>(packed) % 16 == 0) ? packed : nullptr);
     // explicit path: col = im2col(x), then y^T[OC, M] = W2d[OC,K] . col[M,K]^T stored as y[n][oc][p] (+ bias per channel)
     const size_t need = align256((size_t)(M * K) * sizeof(float));
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,

@@ -1147,9 +1147,26 @@ size_t conv_implicit_forward_workspace(int64_t N, int64_t C, int64_t H, int64_t 
 }
 
 // y[n][oc][p] = sum_k W2d[oc][k] * x_gathered[(n,p)][k] + b[oc]
+// the bytes of the re-ordered filter copy the forward makes for this shape (0: it reads the filter as it lies)
+size_t conv_implicit_forward_packed_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW)
+{
+    return (forward_tap_ok(N, C, H, W, KH, KW) && KH > 1) ? (size_t)OC * C * KH * KW * sizeof(float) : 0;
+}
+
+// packed[oc][tap*C + c] = w[oc][c][tap]
+int conv_implicit_forward_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, hipStream_t st)
+{
+    const int64_t total = OC * C * KH * KW;
+    ODL_REQUIRE(total < (1ll << 31), "conv2d: filter too large");
+    hipLaunchKernelGGL(permute_weight_tap_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, w, packed, (int)C,
+                       KH * KW, total);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
 int conv_implicit_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW,
-                          int act, void *workspace, size_t workspace_bytes, hipStream_t st)
+                          int act, void *workspace, size_t workspace_bytes, hipStream_t st, const float *packed)
 {
     GemmArgs g{};
     g.A = w, g.B = x, g.C = y, g.bias = b, g.act = act;
@@ -1158,7 +1175,9 @@ int conv_implicit_forward(const float *x, const float *w, const float *b, float 
     g.k_per_split = ceil_div(g.K, kBK) * kBK, g.c_split_stride = 0;
     const ConvSrc cv = make_src(C, H, W, OH, OW, OC, KH, KW, SH, SW, PH, PW);
     bool tap = forward_tap_ok(N, C, H, W, KH, KW);
-    if (tap && KH > 1)
+    if (tap && KH > 1 && packed != nullptr)
+        g.A = packed;  // the caller keeps the re-ordered copy (weights that do not change between calls)
+    else if (tap && KH > 1)
     {
         const size_t wp_bytes = forward_wp_bytes(N, C, H, W, OC, KH, KW);
         if (workspace != nullptr && workspace_bytes >= wp_bytes)

@@ -271,6 +271,11 @@ public:
     std::unique_ptr<Mat> softmax_cross_entropy_backward(const Mat &target, float gy) const;
     // conv2d with an activation applied in the kernel's epilogue: -1 none, 0 relu, 7 silu. Bit-identical to conv2d()
     // followed by relu() / silu().
+    // `packed` (optional): the filter copy conv2d_packed_weights made for an input of this shape — for weights that stay
+    // the same from call to call, so that the forward does not re-order them every time
+    std::unique_ptr<Mat> conv2d_packed_weights(const Mat &W, std::pair<int, int> stride, std::pair<int, int> pad) const;
+    std::unique_ptr<Mat> conv2d_act(const Mat &W, const Mat *b, std::pair<int, int> stride, std::pair<int, int> pad,
+                                    int activation, const Mat *packed) const;
     std::unique_ptr<Mat> conv2d_act(const Mat &W, const Mat *b, std::pair<int, int> stride, std::pair<int, int> pad,
                                     int activation) const;
     // Max pooling with the window-local indices kept in device memory (uint64 per output). The Mat interface above

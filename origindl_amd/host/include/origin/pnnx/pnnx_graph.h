@@ -22,6 +22,10 @@ struct Attribute  // a weight blob: `@name=(d0,d1,...)f32` in the param file, ra
     std::vector<int> shape;
     std::vector<float> data;
     std::shared_ptr<Mat> device_mat;  // uploaded copy, created on first use
+    // a convolution filter's re-ordered copy for inputs of shape packed_for (made on the first forward over that shape;
+    // null when the forward reads the filter as it lies)
+    std::shared_ptr<Mat> packed_mat;
+    std::vector<size_t> packed_for;
 };
 
 struct PNNXNode

@@ -1153,6 +1153,31 @@ std::unique_ptr<Mat> OriginMat::conv2d(const Mat &Wm, const Mat *bm, std::pair<i
 std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pair<int, int> s, std::pair<int, int> p,
                                            int activation) const
 {
+    return conv2d_act(Wm, bm, s, p, activation, nullptr);
+}
+
+// null when a forward over an input of this shape reads the filter as it lies
+std::unique_ptr<Mat> OriginMat::conv2d_packed_weights(const Mat &Wm, std::pair<int, int> s, std::pair<int, int> p) const
+{
+    const OriginMat &x = dev_f32(*this, "conv2d");
+    const OriginMat &w = dev_f32(Wm, "conv2d");
+    if (shape_.size() != 4 || w.shape().size() != 4)
+        return nullptr;
+    const int64_t OC = w.shape()[0], C = w.shape()[1];
+    const int KH = (int)w.shape()[2], KW = (int)w.shape()[3];
+    const size_t bytes = odl_hip_conv2d_packed_weights_bytes((int64_t)shape_[0], (int64_t)shape_[1], (int64_t)shape_[2],
+                                                             (int64_t)shape_[3], OC, KH, KW, s.first, s.second, p.first,
+                                                             p.second);
+    if (bytes == 0 || (int64_t)shape_[1] != C)
+        return nullptr;
+    auto packed = new_like(x, w.shape());
+    check(odl_hip_conv2d_pack_weights(fp(w), C, OC, KH, KW, packed->data_ptr<float>(), cur()));
+    return packed;
+}
+
+std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pair<int, int> s, std::pair<int, int> p,
+                                           int activation, const Mat *packed_m) const
+{
     const OriginMat &x = dev_f32(*this, "conv2d");
     const OriginMat &w = dev_f32(Wm, "conv2d");
     if (shape_.size() != 4)
@@ -1179,8 +1204,16 @@ std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pa
     auto y = new_like(x, Shape{(size_t)N, (size_t)OC, (size_t)OH, (size_t)OW});
     Workspace ws(odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
                  device().index());
-    check(odl_hip_conv2d_act(fp(x), fp(w), bias, N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
-                             activation, y->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
+    const float *packed = nullptr;
+    if (packed_m)
+    {
+        const OriginMat &pk = dev_f32(*packed_m, "conv2d");
+        if (pk.elements() != w.elements())
+            THROW_INVALID_ARG("conv2d: the packed filter has {} elements, the filter {}", pk.elements(), w.elements());
+        packed = fp(pk);
+    }
+    check(odl_hip_conv2d_act_packed(fp(x), fp(w), packed, bias, N, C, H, W, OC, KH, KW, s.first, s.second, p.first,
+                                    p.second, activation, y->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
     return y;
 }
 

@@ -406,8 +406,16 @@ void PNNXGraph::run(PNNXNode &node)
         if (!w)
             THROW_RUNTIME_ERROR("PNNX: node {} has no weight", node.name);
         auto b = weight("bias");
-        out = origin_of(*in[0]).conv2d_act(*w, b.get(), int_pair(node, "stride", {1, 1}), int_pair(node, "padding", {0, 0}),
-                                          node.fused_activation);
+        const auto stride = int_pair(node, "stride", {1, 1}), padding = int_pair(node, "padding", {0, 0});
+        // the weights never change: the filter order this input shape's kernel wants is made once and kept
+        Attribute &wa = node.attributes.find("weight")->second;
+        const std::vector<size_t> in_dims = in[0]->shape().dims();
+        if (wa.packed_for != in_dims)
+        {
+            wa.packed_mat = origin_of(*in[0]).conv2d_packed_weights(*w, stride, padding);
+            wa.packed_for = in_dims;
+        }
+        out = origin_of(*in[0]).conv2d_act(*w, b.get(), stride, padding, node.fused_activation, wa.packed_mat.get());
     }
     else if (t == "nn.SiLU")
         out = in[0]->silu();

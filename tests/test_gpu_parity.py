@@ -928,3 +928,12 @@ def test_conv_with_fused_activation_is_conv_then_activation(api, N, C, H, OC, k,
         assert np.array_equal(host(api.conv2d(x, w, b, s, p, activation=act)), host(api.unary(act, plain))), act
     with pytest.raises(api.OdlInvalidArgument):
         api.conv2d(x, w, b, s, p, activation="exp")
+    # weights that do not change between calls: the filter copy made once gives the same bits as the per-call copy, and
+    # shapes whose kernel reads the filter as it lies have no such copy
+    packed = api.conv2d_pack_weights(x.shape, w, s, p)
+    assert (packed is not None) == (k == 3 and C % 16 == 0)
+    if packed is not None:
+        assert np.array_equal(host(packed), host(w).reshape(OC, C, k * k).transpose(0, 2, 1).reshape(w.shape))
+    for act in (None, "silu"):
+        assert np.array_equal(host(api.conv2d(x, w, b, s, p, activation=act, packed=packed)),
+                              host(api.conv2d(x, w, b, s, p, activation=act))), act
