@@ -55,7 +55,7 @@ int odl_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
 int odl_hip_memset(void *dst, int value, size_t bytes, void *stream);
 
 /* Streams and captured graphs. No counterpart in the reference, which launches everything on the null stream
- * (src/mat/origin/cuda/** creates no stream, event or graph): they exist so that a caller can record a step of
+ * (the files under src/mat/origin/cuda create no stream, event or graph): they exist so that a caller can record a step of
  * fixed shapes once and replay it with one submission. A created stream is non-blocking and has the default
  * priority. Between capture_begin and capture_end every launch on that stream is recorded, not run; entry points
  * that synchronise or copy to the host (odl_hip_synchronize, odl_hip_memcpy_d2h, odl_hip_softmax_ce_loss,

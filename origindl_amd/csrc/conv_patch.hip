@@ -1,0 +1,430 @@
+// 3x3, stride 1, padding 1 convolution on the matrix cores (v_mfma_f32_32x32x2_f32) with the input patch held in LDS.
+//
+// The implicit-GEMM kernels gather one [16 k, 128 pixel] operand tile per 16 values of K, so every input element
+// travels from L2 to LDS once per filter tap. Here a workgroup stages, per slab of 16 input channels, the image rows
+// its 128 output pixels touch (plus one halo row above and below and one zero column left and right) once, and the
+// nine taps read that patch at shifted LDS addresses: nine times fewer loads and one barrier pair per 144 values of K.
+//
+// One kernel serves two products of a 3x3/s1/p1 layer (src/operators/conv/conv2d.cpp:458-560 in the reference):
+//   forward         y[n,oc,h,w]  = b[oc] + sum_{c,t} x[n,c,h+dy,w+dx] * w[oc,c,t]                (source read as NCHW)
+//   input gradient  gx[n,c,h,w]  = sum_{oc,t} gy2d[pix(n,h+dy,w+dx)][oc] * w[oc,c,8-t]
+// where gy2d is the gradient buffer read as a row-major [N*OH*OW, OC] matrix exactly as it lies, the reference's
+// reading (conv2d.cpp:548) — for this kernel a channel-minor source.
+#include "odl_common.h"
+
+#include <cstdlib>
+
+namespace
+{
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kPixTile = 128;    // output pixels per workgroup, consecutive in (n, h, w) order
+constexpr int kSlab = 16;        // input channels per staging step
+constexpr int kPosPerThread = 2; // patch positions (row, column) one thread stages
+constexpr int kLdp = kSlab + 4;  // floats per patch position in LDS: 16-byte aligned, an odd number of 16-byte units
+constexpr int kLda = 9 * kSlab + 4;  // floats per filter row in LDS, likewise
+constexpr size_t kLdsCap = 80 * 1024;  // two workgroups per compute unit
+
+struct PatchGeom
+{
+    const float *src, *wp, *bias;
+    float *dst;
+    int Cin, M, Mpad, NH, H, W, HW;  // NH = N*H image rows in the batch
+    int PW, plane;                   // patch width W + 2 and positions per patch (rows * PW)
+    int pixels, mtiles, act;
+    odl::FastDiv by_w, by_h, by_hw, by_pw;
+};
+
+// wp[(m*nslab + slab)*144 + tap*16 + cc]: the zero-padded filter copy the kernel stages with 16-byte copies
+__global__ void conv_patch_pack_kernel(const float *__restrict__ w, float *__restrict__ wp, int Cin, int M, int Mpad,
+                                       int flipped)
+{
+    const int total = Cin * 9 * Mpad, nslab = Cin / kSlab;
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x)
+    {
+        const int rem = idx % (9 * kSlab), rest = idx / (9 * kSlab);
+        const int slab = rest % nslab, m = rest / nslab;
+        const int tap = rem / kSlab, ch = slab * kSlab + rem % kSlab;
+        float v = 0.f;
+        if (m < M)
+            v = flipped ? w[((int64_t)ch * M + m) * 9 + 8 - tap] : w[((int64_t)m * Cin + ch) * 9 + tap];
+        wp[idx] = v;
+    }
+}
+
+template <int BM, bool CH_MINOR>
+__global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
+{
+    constexpr int KS = 9 * kSlab;
+    constexpr int WM = BM >= 64 ? 2 : 1, WN = 4 / WM;
+    constexpr int TM = BM / WM, TN = kPixTile / WN;
+    constexpr int RB = TM / 32, CB = TN / 32;
+    extern __shared__ float lds[];
+    float *As = lds;              // [BM][kLda]
+    float *Bs = lds + BM * kLda;  // [plane + 3][kLdp]; the last three positions stay zero
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int mt = blockIdx.x % g.mtiles, nt = blockIdx.x / g.mtiles;
+    const int m0 = mt * BM, p0 = nt * kPixTile;
+    const int wm = (wave % WM) * TM, wn = (wave / WM) * TN;
+    const int gr0 = (int)odl::fastdiv((unsigned)p0, g.by_w);  // first image row (of the whole batch) of the tile
+
+    // ---- where this thread's patch positions come from: patch row r is batch row gr0 - 1 + r
+    int src_off[kPosPerThread];
+#pragma unroll
+    for (int i = 0; i < kPosPerThread; ++i)
+    {
+        const int pos = t + i * kThreads;
+        const int r = (int)odl::fastdiv((unsigned)pos, g.by_pw), col = pos - r * g.PW;
+        const int gr = gr0 - 1 + r;
+        const bool ok = pos < g.plane && col >= 1 && col <= g.W && gr >= 0 && gr < g.NH;
+        int off = -1;
+        if (ok)
+        {
+            if (CH_MINOR)
+                off = (gr * g.W + col - 1) * g.Cin;
+            else
+            {
+                const int n = (int)odl::fastdiv((unsigned)gr, g.by_h), h = gr - n * g.H;
+                off = (n * g.Cin * g.H + h) * g.W + col - 1;
+            }
+        }
+        src_off[i] = off;
+    }
+    if (t < 3 * kLdp)
+        Bs[g.plane * kLdp + t] = 0.f;
+
+    // ---- where this lane's output pixels sit in the patch, one base per tap row; a tap row that falls outside the
+    // pixel's own image points at the zero positions instead
+    int base[CB][3];
+#pragma unroll
+    for (int j = 0; j < CB; ++j)
+    {
+        int p = p0 + wn + j * 32 + l32;
+        p = p < g.pixels ? p : g.pixels - 1;
+        const int grow = (int)odl::fastdiv((unsigned)p, g.by_w), w = p - grow * g.W;
+        const int n = (int)odl::fastdiv((unsigned)grow, g.by_h), h = grow - n * g.H;
+        // the position left of the pixel, so that the three taps of a row sit at offsets 0, 1 and 2 positions
+        const int left = (grow - gr0 + 1) * g.PW + w;
+        const int zero = g.plane;
+        base[j][0] = (h > 0 ? left - g.PW : zero) * kLdp + 4 * lh;
+        base[j][1] = left * kLdp + 4 * lh;
+        base[j][2] = (h < g.H - 1 ? left + g.PW : zero) * kLdp + 4 * lh;
+    }
+
+    f32x16 acc[RB][CB];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < CB; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0.f;
+
+    const int nslab = g.Cin / kSlab;
+    const int ch_stride = CH_MINOR ? 1 : g.HW;
+
+    // one slab travels global memory -> registers -> LDS; the loads of slab s + 1 are issued before the matrix
+    // instructions of slab s and land while those run
+    constexpr int A_VECS = KS * BM / 4, A_PER_T = (A_VECS + kThreads - 1) / kThreads;
+    f32x4 ra[A_PER_T];
+    float rb[kPosPerThread][kSlab];
+    auto load_slab = [&](int s)
+    {
+        const float *wsrc = g.wp + ((int64_t)m0 * nslab + s) * KS;
+#pragma unroll
+        for (int q = 0; q < A_PER_T; ++q)
+        {
+            const int e = t + q * kThreads;
+            if (A_VECS % kThreads == 0 || e < A_VECS)
+            {
+                const int m = e / (KS / 4), k4 = e % (KS / 4);
+                ra[q] = *reinterpret_cast<const f32x4 *>(wsrc + (int64_t)m * nslab * KS + k4 * 4);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kPosPerThread; ++i)
+        {
+            if (src_off[i] < 0)
+            {
+#pragma unroll
+                for (int cc = 0; cc < kSlab; ++cc)
+                    rb[i][cc] = 0.f;
+            }
+            else if (CH_MINOR)
+            {
+                const f32x4 *in = reinterpret_cast<const f32x4 *>(g.src + src_off[i] + s * kSlab);
+#pragma unroll
+                for (int q = 0; q < kSlab / 4; ++q)
+                {
+                    const f32x4 v = in[q];
+                    rb[i][q * 4 + 0] = v[0], rb[i][q * 4 + 1] = v[1], rb[i][q * 4 + 2] = v[2], rb[i][q * 4 + 3] = v[3];
+                }
+            }
+            else
+            {
+                const float *in = g.src + src_off[i] + (int64_t)s * kSlab * ch_stride;
+#pragma unroll
+                for (int cc = 0; cc < kSlab; ++cc)
+                    rb[i][cc] = in[(int64_t)cc * ch_stride];
+            }
+        }
+    };
+    auto store_slab = [&]()
+    {
+#pragma unroll
+        for (int q = 0; q < A_PER_T; ++q)
+        {
+            const int e = t + q * kThreads;
+            if (A_VECS % kThreads == 0 || e < A_VECS)
+            {
+                const int m = e / (KS / 4), k4 = e % (KS / 4);
+                *reinterpret_cast<f32x4 *>(As + m * kLda + k4 * 4) = ra[q];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kPosPerThread; ++i)
+        {
+            const int pos = t + i * kThreads;
+            if (pos < g.plane)
+            {
+#pragma unroll
+                for (int q = 0; q < kSlab / 4; ++q)
+                {
+                    f32x4 v;
+                    v[0] = rb[i][q * 4 + 0], v[1] = rb[i][q * 4 + 1], v[2] = rb[i][q * 4 + 2], v[3] = rb[i][q * 4 + 3];
+                    *reinterpret_cast<f32x4 *>(Bs + pos * kLdp + q * 4) = v;
+                }
+            }
+        }
+    };
+
+    load_slab(0);
+    for (int s = 0; s < nslab; ++s)
+    {
+        __syncthreads();  // the previous slab has been read
+        store_slab();
+        __syncthreads();
+        if (s + 1 < nslab)
+            load_slab(s + 1);
+
+        // ---- 144 values of K: nine taps x two groups of eight channels. One 16-byte read per operand block brings four
+        // channels; instruction e of a group takes channel e from lanes 0-31 and channel 4 + e from lanes 32-63. The
+        // operands of group q + 1 are read while the instructions of group q run.
+        constexpr int NG = 9 * (kSlab / 8);
+        f32x4 a[2][RB], b[2][CB];
+        auto read_group = [&](int q, int buf)
+        {
+            const int tap = q / (kSlab / 8), g8 = q % (kSlab / 8);
+            const int dyi = tap / 3, dxi = tap % 3;
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+                a[buf][i] =
+                    *reinterpret_cast<const f32x4 *>(As + (wm + i * 32 + l32) * kLda + tap * kSlab + g8 * 8 + 4 * lh);
+#pragma unroll
+            for (int j = 0; j < CB; ++j)
+                b[buf][j] = *reinterpret_cast<const f32x4 *>(Bs + base[j][dyi] + dxi * kLdp + g8 * 8);
+        };
+        read_group(0, 0);
+#pragma unroll
+        for (int q = 0; q < NG; ++q)
+        {
+            if (q + 1 < NG)
+                read_group(q + 1, (q + 1) & 1);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int i = 0; i < RB; ++i)
+#pragma unroll
+                    for (int j = 0; j < CB; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q & 1][i][e], b[q & 1][j][e], acc[i][j], 0, 0, 0);
+            // issue order for the instruction scheduler: the next group's LDS reads go between this group's first
+            // matrix instructions instead of after its last
+            if (q + 1 < NG)
+            {
+#pragma unroll
+                for (int r = 0; r < RB + CB; ++r)
+                {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one matrix instruction
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 4 * RB * CB - (RB + CB), 0);
+            }
+            else
+                __builtin_amdgcn_sched_group_barrier(0x008, 4 * RB * CB, 0);
+        }
+    }
+
+    // ---- accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
+#pragma unroll
+    for (int j = 0; j < CB; ++j)
+    {
+        const int p = p0 + wn + j * 32 + l32;
+        if (p >= g.pixels)
+            continue;
+        const int n = (int)odl::fastdiv((unsigned)p, g.by_hw), hw = p - n * g.HW;
+        float *out = g.dst + (int64_t)n * g.M * g.HW + hw;
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+                if (row >= g.M)
+                    continue;
+                float v = acc[i][j][r];
+                if (g.bias)
+                    v = v + g.bias[row];
+                out[(int64_t)row * g.HW] = odl::apply_act(v, g.act);
+            }
+    }
+}
+
+inline int patch_rows(int64_t W)
+{
+    return (int)((W - 1 + kPixTile - 1) / W) + 1 + 2;
+}
+
+inline int tile_bm(int64_t M)
+{
+    return M <= 32 ? 32 : 64;
+}
+
+inline size_t lds_bytes(int bm, int plane)
+{
+    return ((size_t)bm * kLda + (size_t)(plane + 3) * kLdp) * sizeof(float);
+}
+
+// more dynamic LDS than the default limit of 64 KB, asked for once per kernel
+template <int BM, bool CH_MINOR>
+hipError_t allow_lds_of()
+{
+    static const hipError_t rc =
+        hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_patch_kernel<BM, CH_MINOR>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsCap);
+    return rc;
+}
+
+hipError_t allow_lds(int bm, bool ch_minor)
+{
+    if (bm == 32)
+        return ch_minor ? allow_lds_of<32, true>() : allow_lds_of<32, false>();
+    return ch_minor ? allow_lds_of<64, true>() : allow_lds_of<64, false>();
+}
+
+bool shape_ok(const float *src, int64_t N, int64_t Cin, int64_t H, int64_t W, int64_t M, int KH, int KW, int SH, int SW,
+              int PH, int PW)
+{
+    if (!(KH == 3 && KW == 3 && SH == 1 && SW == 1 && PH == 1 && PW == 1))
+        return false;
+    if (Cin < kSlab || Cin % kSlab != 0 || M < 1 || reinterpret_cast<uintptr_t>(src) % 16 != 0)
+        return false;
+    const int64_t plane = (int64_t)patch_rows(W) * (W + 2);
+    if (plane > kPosPerThread * kThreads || lds_bytes(tile_bm(M), (int)plane) > kLdsCap)
+        return false;
+    // fewer workgroups than compute units: the implicit kernels, which slice K, do better
+    // (ODL_CONV_PATCH_MIN_WGS overrides the threshold, so that small shapes can be sent through this kernel)
+    int64_t min_wgs = 256;
+    if (const char *e = getenv("ODL_CONV_PATCH_MIN_WGS"))
+        min_wgs = atoll(e);
+    if (odl::ceil_div(N * H * W, kPixTile) * odl::ceil_div(M, tile_bm(M)) < min_wgs)
+        return false;
+    // 32-bit element offsets inside the kernel
+    return N * Cin * H * W < (1ll << 31) && N * M * H * W < (1ll << 40) && N * H * W < (1ll << 31) - kPixTile &&
+           Cin * 9 * (M + 64) < (1ll << 31);
+}
+
+size_t packed_bytes(int64_t Cin, int64_t M)
+{
+    const int bm = tile_bm(M);
+    const int64_t mpad = odl::ceil_div(M, bm) * bm;
+    return (((size_t)Cin * 9 * mpad * sizeof(float)) + 255) & ~(size_t)255;
+}
+
+int launch(const float *src, const float *w, const float *bias, float *dst, int64_t N, int64_t Cin, int64_t H, int64_t W,
+           int64_t M, bool ch_minor, int act, void *workspace, size_t workspace_bytes, hipStream_t st, const char *who)
+{
+    const size_t need = packed_bytes(Cin, M);
+    if (!workspace || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return odl::fail(ODL_ERR_INVALID_ARG, "%s: needs a 16-byte aligned workspace of %zu bytes, got %zu", who, need,
+                         workspace_bytes);
+    const int bm = tile_bm(M);
+    PatchGeom g{};
+    g.src = src, g.bias = bias, g.dst = dst;
+    g.Cin = (int)Cin, g.M = (int)M, g.Mpad = (int)(odl::ceil_div(M, bm) * bm);
+    g.NH = (int)(N * H), g.H = (int)H, g.W = (int)W, g.HW = (int)(H * W);
+    g.PW = (int)W + 2, g.plane = patch_rows(W) * g.PW;
+    g.pixels = (int)(N * H * W), g.mtiles = g.Mpad / bm, g.act = act;
+    g.by_w = odl::make_fastdiv((unsigned)W), g.by_h = odl::make_fastdiv((unsigned)H);
+    g.by_hw = odl::make_fastdiv((unsigned)(H * W)), g.by_pw = odl::make_fastdiv((unsigned)g.PW);
+    float *wp = static_cast<float *>(workspace);
+    g.wp = wp;
+    const int total = g.Cin * 9 * g.Mpad;
+    hipLaunchKernelGGL(conv_patch_pack_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, w, wp, g.Cin,
+                       g.M, g.Mpad, ch_minor ? 1 : 0);
+    ODL_LAUNCH_CHECK();
+    const dim3 grid((unsigned)(odl::ceil_div(g.pixels, kPixTile) * g.mtiles));
+    const size_t lds = lds_bytes(bm, g.plane);
+    ODL_HIP_CHECK(allow_lds(bm, ch_minor));
+    if (bm == 32)
+    {
+        if (ch_minor)
+            hipLaunchKernelGGL((conv_patch_kernel<32, true>), grid, dim3(kThreads), lds, st, g);
+        else
+            hipLaunchKernelGGL((conv_patch_kernel<32, false>), grid, dim3(kThreads), lds, st, g);
+    }
+    else
+    {
+        if (ch_minor)
+            hipLaunchKernelGGL((conv_patch_kernel<64, true>), grid, dim3(kThreads), lds, st, g);
+        else
+            hipLaunchKernelGGL((conv_patch_kernel<64, false>), grid, dim3(kThreads), lds, st, g);
+    }
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace
+
+namespace odl
+{
+bool conv_patch_forward_ok(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                           int SW, int PH, int PW)
+{
+    // measured on the 3x3 layers of the benchmark networks: from 64 input channels on (K >= 576) the implicit-GEMM
+    // forward, whose K loop is software-pipelined over many short slabs, is as fast or faster; below that its fixed
+    // cost per workgroup dominates and this kernel wins. The threshold override lifts this rule too.
+    if (C > 48 && !getenv("ODL_CONV_PATCH_MIN_WGS"))
+        return false;
+    return shape_ok(x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
+}
+
+size_t conv_patch_forward_workspace(int64_t C, int64_t OC)
+{
+    return packed_bytes(C, OC);
+}
+
+int conv_patch_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
+                       int64_t W, int64_t OC, int act, void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    return launch(x, w, b, y, N, C, H, W, OC, false, act, workspace, workspace_bytes, st, "conv2d");
+}
+
+bool conv_patch_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                         int SW, int PH, int PW)
+{
+    return shape_ok(gy, N, OC, H, W, C, KH, KW, SH, SW, PH, PW);
+}
+
+size_t conv_patch_dgrad_workspace(int64_t C, int64_t OC)
+{
+    return packed_bytes(OC, C);
+}
+
+int conv_patch_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                     void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    return launch(gy, w, nullptr, gx, N, OC, H, W, C, true, 0, workspace, workspace_bytes, st, "conv2d_backward");
+}
+}  // namespace odl

@@ -289,12 +289,31 @@ CONV_SEEDED = [
     (1, 4, 2, 2, 16, 3, 3, 2, 1),      # a 2x2 image under a 3x3 window at stride 2
     (5, 130, 12, 12, 48, 3, 3, 2, 1),  # stride 2, more input channels than two row tiles hold
     (2, 64, 20, 20, 128, 1, 1, 1, 0),  # its 1x1 bottleneck convolutions
+    (3, 48, 9, 30, 33, 3, 3, 1, 1),    # LDS-patch forward with a ragged filter tile; three channel slabs
+    (1, 16, 1, 1, 80, 3, 3, 1, 1),     # a single pixel: every tap row but the centre falls outside the image
+    (2, 32, 3, 100, 16, 3, 3, 1, 1),   # the widest rows the LDS patch holds, two patch positions per thread
+    (7, 16, 5, 6, 64, 3, 3, 1, 1),     # tiles that start and end in the middle of an image; 64 gradient channels
 ]
 
 
 @pytest.mark.parametrize("N,C,H,W,OC,KH,KW,s,p", CONV_SEEDED)
 def test_conv_vs_oracle_seeded(api, o, N, C, H, W, OC, KH, KW, s, p):
     print("\n[case] conv seeded", N, C, H, W, OC, KH, KW, s, p, flush=True)
+    check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p)
+
+
+@pytest.mark.parametrize("N,C,H,W,OC,KH,KW,s,p",
+                         [c for c in CONV_SEEDED if c[5:] == (3, 3, 1, 1) and (c[1] % 16 == 0 or c[4] % 16 == 0)])
+def test_conv_lds_patch_kernel_vs_oracle_seeded(api, o, monkeypatch, N, C, H, W, OC, KH, KW, s, p):
+    # The kernel that keeps the input patch in LDS takes 3x3/s1/p1 layers whose channel count is a multiple of 16
+    # (forward: input channels; input gradient: filters) once they fill the chip; the override sends the small
+    # seeded shapes through it as well.
+    print("\n[case] conv seeded, LDS patch", N, C, H, W, OC, flush=True)
+    monkeypatch.setenv("ODL_CONV_PATCH_MIN_WGS", "0")
+    check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p)
+
+
+def check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p):
     rng = np.random.default_rng(N * 100 + C + OC)
     x = rng.standard_normal((N, C, H, W), dtype=f32)
     w = (rng.standard_normal((OC, C, KH, KW), dtype=f32) * f32(np.sqrt(2.0 / (C * KH * KW)))).astype(f32)
