@@ -293,6 +293,8 @@ CONV_SEEDED = [
     (1, 16, 1, 1, 80, 3, 3, 1, 1),     # a single pixel: every tap row but the centre falls outside the image
     (2, 32, 3, 100, 16, 3, 3, 1, 1),   # the widest rows the LDS patch holds, two patch positions per thread
     (7, 16, 5, 6, 64, 3, 3, 1, 1),     # tiles that start and end in the middle of an image; 64 gradient channels
+    (3, 16, 8, 8, 24, 3, 3, 1, 1),     # W a multiple of 4: the LDS patch is staged with 16-byte row loads
+    (2, 48, 6, 28, 40, 3, 3, 1, 1),    # the same over three channel slabs and rows shared between tiles
 ]
 
 
