@@ -107,7 +107,7 @@ def extras(torch, capi, steps, warmup):
         L.check(fn(*args))  # argument errors surface here, once
         return lambda: fn(*args)
 
-    # conv2d forward + weight-grad + input-grad at BASELINE's C1 and C2
+    # conv2d forward + weight-grad + input-grad at the benchmark's convolution configurations C1 and C2
     for name, (N, C, H, OC, s, p) in {"conv_c1": (32, 64, 56, 128, 1, 1), "conv_c2": (32, 128, 28, 256, 2, 1)}.items():
         x, w, b = rnd(N, C, H, H), rnd(OC, C, 3, 3) * (2.0 / (C * 9)) ** 0.5, rnd(OC)
         OH = (H + 2 * p - 3) // s + 1

@@ -137,7 +137,7 @@ int orc_mlp_train_step(const float *x, const void *t, int idx_is_i64, int64_t N,
                        float eps, float wd, float *loss, float *gW1, float *gb1, float *gW2, float *gb2,
                        float *logits);
 
-/* CNN (BASELINE config 4): x[N,1,S,S] -> conv(1->C1,3x3,p1) ReLU maxpool2 -> conv(C1->C2,3x3,p1) ReLU maxpool2
+/* CNN (the benchmark's CNN training configuration): x[N,1,S,S] -> conv(1->C1,3x3,p1) ReLU maxpool2 -> conv(C1->C2,3x3,p1) ReLU maxpool2
  * -> flatten -> Linear(F,Hd) ReLU -> Linear(Hd,Cc) -> softmax CE; backward; SGD (src/optim/sgd.cpp:18-75,
  * no momentum, no weight decay). Parameters updated in place. Returns loss, pool indices and all grads. */
 int orc_cnn_train_step(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t S, int64_t C1, int64_t C2,

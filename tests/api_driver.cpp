@@ -835,7 +835,7 @@ int DRV(mlp_train_graph)(const float *x, const void *t, int is64, int64_t N, int
 }
 #endif
 
-// CNN of BASELINE config 4 (no BatchNorm), SGD without momentum/weight decay, one step.
+// CNN of the benchmark's CNN training configuration (no BatchNorm), SGD without momentum/weight decay, one step.
 int DRV(cnn_train)(const float *x, const void *t, int is64, int64_t N, int64_t S, int64_t C1, int64_t C2, int64_t Hd,
                       int64_t Cc, float *Wc1, float *bc1, float *Wc2, float *bc2, float *Wl1, float *bl1, float *Wl2,
                       float *bl2, float lr, float *loss, float *gWc1, float *gbc1, float *gWc2, float *gbc2,

@@ -149,7 +149,7 @@ def test_sgemm_all_layouts_split_k_and_bias(api, ta, tb):
 
 @pytest.mark.parametrize("size", [4096])
 def test_matmul_full_size_sampled_rows_and_linearity(api, o, size):
-    # BASELINE's 4096^3: the oracle runs a seeded sample of rows (rows are independent in its loop);
+    # the headline 4096^3 products: the oracle runs a seeded sample of rows (rows are independent in its loop);
     # plus a size-independent property: (a1 + a2) @ b == a1 @ b + a2 @ b within the GEMM bound.
     print("\n[case] full size", size, flush=True)
     g = torch.Generator(device="cuda").manual_seed(1)
@@ -335,13 +335,13 @@ def check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p):
 
 
 @pytest.mark.parametrize("N,C,H,OC,s,p", [
-    (32, 64, 56, 128, 1, 1),    # BASELINE config C1
-    (32, 128, 28, 256, 2, 1),   # BASELINE config C2
+    (32, 64, 56, 128, 1, 1),    # benchmark configuration C1
+    (32, 128, 28, 256, 2, 1),   # benchmark configuration C2
     (256, 1, 28, 32, 1, 1),     # the CNN's first layer at its batch size: the direct kernels
     (256, 32, 14, 64, 1, 1),    # the CNN's second layer
 ])
 def test_conv_full_size_properties(api, o, N, C, H, OC, s, p):
-    # BASELINE's convolutions at full size. The oracle checks a sample of output pixels (each is one dot product of a
+    # The benchmark's convolutions at full size. The oracle checks a sample of output pixels (each is one dot product of a
     # col row with a weight row); im2col/col2im adjointness and the bias-gradient identity hold at any size; the two
     # gradients are checked against float64 GEMMs over the reference's reinterpreted gy.
     print("\n[case] conv full size", N, C, H, OC, s, p, flush=True)
