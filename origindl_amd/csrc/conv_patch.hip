@@ -392,10 +392,12 @@ namespace odl
 bool conv_patch_forward_ok(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
                            int SW, int PH, int PW)
 {
-    // measured on the 3x3 layers of the benchmark networks: from 64 input channels on (K >= 576) the implicit-GEMM
-    // forward, whose K loop is software-pipelined over many short slabs, is as fast or faster; below that its fixed
-    // cost per workgroup dominates and this kernel wins. The threshold override lifts this rule too.
-    if (C > 48 && !getenv("ODL_CONV_PATCH_MIN_WGS"))
+    // measured on the 3x3 layers of the benchmark networks: with few input channels (K < 576) the implicit-GEMM
+    // forward's fixed cost per workgroup dominates and this kernel wins; with more it still wins on short image rows
+    // (64 -> 128 channels at 14x14: 96 against 109 us), but on long rows, where the patch with its halo rows holds
+    // more than twice the pixels the tile produces (W = 56: 6 rows for 2.3), the implicit kernel is as fast or
+    // faster (172 against 175 us). The threshold override lifts this rule too.
+    if (C > 48 && (int64_t)patch_rows(W) * W > 2 * kPixTile && !getenv("ODL_CONV_PATCH_MIN_WGS"))
         return false;
     return shape_ok(x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
 }
