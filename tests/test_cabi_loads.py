@@ -48,6 +48,13 @@ def test_workspace_queries_need_no_gpu():
     assert l.query("odl_hip_conv2d_workspace_bytes", 16, 5, 28, 28, 32, 3, 3, 1, 1, 1, 1) == 16 * 28 * 28 * 45 * 4
     assert l.query("odl_hip_conv2d_backward_workspace_bytes", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) < 100352 * 576 * 4
     assert l.query("odl_hip_conv2d_workspace_bytes", 1, 1, 2, 2, 1, 3, 3, 1, 1, 0, 0) == 0  # no valid output
+    # 3x3/s1/p1 over 32 input channels with enough pixels to fill the chip: the LDS-patch kernel's re-ordered filter
+    # copy (9*C*OC floats, rows padded to the 64-row tile) bounds the forward's need from below; a batch too small
+    # for it (fewer than 256 workgroups) asks for less
+    assert l.query("odl_hip_conv2d_workspace_bytes", 256, 32, 14, 14, 64, 3, 3, 1, 1, 1, 1) >= 9 * 32 * 64 * 4
+    assert l.query("odl_hip_conv2d_workspace_bytes", 256, 32, 14, 14, 64, 3, 3, 1, 1, 1, 1) < 256 * 196 * 288 * 4
+    assert (l.query("odl_hip_conv2d_backward_workspace_bytes", 256, 32, 14, 14, 64, 3, 3, 1, 1, 1, 1) >=
+            9 * 64 * 32 * 4)
     assert l.query("odl_hip_sum_axis_workspace_bytes", 4096, 10, 1) == 0
     assert l.query("odl_hip_sum_axis_workspace_bytes", 1, 16384, 4096) > 0
     src = (ctypes.c_int64 * 2)(512, 1000)
