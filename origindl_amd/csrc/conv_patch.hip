@@ -12,10 +12,13 @@
 // reading (conv2d.cpp:548) — for this kernel a channel-minor source.
 #include "odl_common.h"
 
-#include <cstdlib>
+#include <atomic>
 
 namespace
 {
+// least number of workgroups for which this kernel is chosen; negative = one per compute unit of the device
+std::atomic<int64_t> g_min_wgs{-1};
+
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -325,11 +328,9 @@ bool shape_ok(const float *src, int64_t N, int64_t Cin, int64_t H, int64_t W, in
     if (plane > kPosPerThread * kThreads || lds_bytes(tile_bm(M), (int)plane) > kLdsCap)
         return false;
     // fewer workgroups than compute units: the implicit kernels, which slice K, do better
-    // (ODL_CONV_PATCH_MIN_WGS overrides the threshold, so that small shapes can be sent through this kernel)
-    int64_t min_wgs = 256;
-    if (const char *e = getenv("ODL_CONV_PATCH_MIN_WGS"))
-        min_wgs = atoll(e);
-    if (odl::ceil_div(N * H * W, kPixTile) * odl::ceil_div(M, tile_bm(M)) < min_wgs)
+    // (odl_hip_set_conv_patch_min_workgroups replaces the threshold, so that small shapes can be sent through this kernel)
+    const int64_t min_wgs = g_min_wgs.load(std::memory_order_relaxed);
+    if (odl::ceil_div(N * H * W, kPixTile) * odl::ceil_div(M, tile_bm(M)) < (min_wgs < 0 ? odl::device_cus() : min_wgs))
         return false;
     // 32-bit element offsets inside the kernel
     return N * Cin * H * W < (1ll << 31) && N * M * H * W < (1ll << 40) && N * H * W < (1ll << 31) - kPixTile &&
@@ -402,7 +403,7 @@ bool conv_patch_forward_ok(const float *x, int64_t N, int64_t C, int64_t H, int6
     // (64 -> 128 channels at 14x14: 96 against 109 us), but on long rows, where the patch with its halo rows holds
     // more than twice the pixels the tile produces (W = 56: 6 rows for 2.3), the implicit kernel is as fast or
     // faster (172 against 175 us). The threshold override lifts this rule too.
-    if (C > 48 && (int64_t)patch_rows(W) * W > 2 * kPixTile && !getenv("ODL_CONV_PATCH_MIN_WGS"))
+    if (C > 48 && (int64_t)patch_rows(W) * W > 2 * kPixTile && g_min_wgs.load(std::memory_order_relaxed) < 0)
         return false;
     return shape_ok(x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
 }
@@ -435,3 +436,9 @@ int conv_patch_dgrad(const float *gy, const float *w, float *gx, int64_t N, int6
     return launch(gy, w, nullptr, gx, N, OC, H, W, C, true, 0, workspace, workspace_bytes, st, "conv2d_backward");
 }
 }  // namespace odl
+
+extern "C" int odl_hip_set_conv_patch_min_workgroups(int64_t min_workgroups)
+{
+    g_min_wgs.store(min_workgroups < 0 ? -1 : min_workgroups, std::memory_order_relaxed);
+    return ODL_OK;
+}

@@ -31,7 +31,6 @@ inline bool aligned16(const void *p)
 {
     return reinterpret_cast<uintptr_t>(p) % 16 == 0;
 }
-constexpr int kXcds    = 8;
 constexpr int kGroupM  = 8;
 
 enum : int
@@ -79,6 +78,7 @@ struct GemmArgs
     int act;                 // EPI_NCHW_ROWB: activation applied after the bias (0 none, 1 relu, 2 silu)
     int tiles_m, tiles_n;
     int splits;              // K slices (grid = tiles_m * tiles_n * splits workgroups)
+    int xcds;                // XCDs of the device: consecutive workgroup ids are dealt round-robin over them
     // Tail split (splits == 1 only): when the tile count is a little over a multiple of the CU count, the last
     // `nt - tail_first` tiles would run alone after everything else. They are cut into tail_splits K pieces
     // each — workgroups main_blocks.. — which write tile-local partials to tail_ws; tail_fixup_kernel sums them.
@@ -151,13 +151,14 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
         }
         else
         {
-            const int64_t total = g.tail_splits > 0 ? (int64_t)g.main_blocks : (int64_t)nt * g.splits;
-            const int64_t bid = blockIdx.x;
-            const int64_t xcd = bid % kXcds, loc = bid / kXcds;
-            const int64_t full = total / kXcds, rem = total % kXcds;
-            const int64_t v = xcd * full + (xcd < rem ? xcd : rem) + loc;
-            kz = (int)(v / nt);
-            t = (int)(v % nt);
+            // (the workgroup count of a launch is below 2^31: 32-bit arithmetic)
+            const unsigned total = g.tail_splits > 0 ? (unsigned)g.main_blocks : (unsigned)nt * (unsigned)g.splits;
+            const unsigned bid = blockIdx.x, nx = (unsigned)g.xcds;
+            const unsigned loc = bid / nx, xcd = bid - loc * nx;
+            const unsigned full = total / nx, rem = total - full * nx;
+            const unsigned v = xcd * full + (xcd < rem ? xcd : rem) + loc;
+            kz = (int)(v / (unsigned)nt);
+            t = (int)(v - (unsigned)kz * (unsigned)nt);
             kbeg = (int64_t)kz * g.k_per_split;
             kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
         }
@@ -728,7 +729,7 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(GemmArgs g, int BM, int
     }
 }
 
-// Whether (and how) to split the last tiles: nt tiles over 256 CUs run in ceil(nt/256) rounds, and a last round of
+// Whether (and how) to split the last tiles: nt tiles over the chip's CUs (256) run in ceil(nt/256) rounds, and a last round of
 // only a few tiles leaves most CUs idle for a whole tile's time. Those few tiles are cut into K pieces instead.
 struct TailPlan
 {
@@ -741,10 +742,11 @@ TailPlan plan_tail(int64_t nt, int64_t K, int BM, int BN)
 {
     TailPlan p;
     const int64_t kt = odl::ceil_div(K, 16);
-    const int64_t r = nt % 256;
-    if (nt <= 256 || nt > 256 * 8 || r == 0 || r > 128 || kt < 16)
+    const int64_t cus = odl::device_cus();
+    const int64_t r = nt % cus;
+    if (nt <= cus || nt > cus * 8 || r == 0 || r > cus / 2 || kt < 16)
         return p;
-    int64_t s = 256 / r;
+    int64_t s = cus / r;
     if (s > kt / 2)
         s = kt / 2;
     if (s > 32)
@@ -763,6 +765,7 @@ unsigned apply_tail(GemmArgs &g, int BM, int BN, void *tail_ws, size_t tail_byte
 {
     const int64_t nt = (int64_t)g.tiles_m * g.tiles_n;
     g.main_blocks = 0, g.tail_first = (int)nt, g.tail_splits = 0, g.tail_kps = 0, g.tail_ws = nullptr;
+    g.xcds = odl::chip().xcds;
     if (g.splits != 1 || tail_ws == nullptr || reinterpret_cast<uintptr_t>(tail_ws) % 16 != 0)
         return (unsigned)(nt * g.splits);
     const TailPlan p = plan_tail(nt, g.K, BM, BN);
@@ -837,7 +840,7 @@ constexpr int kBK = 16;
 // that more workgroups exist.
 int pick_tile(int64_t M, int64_t N)
 {
-    return (odl::ceil_div(M, 128) * odl::ceil_div(N, 128) >= 256) ? 128 : 64;
+    return (odl::ceil_div(M, 128) * odl::ceil_div(N, 128) >= odl::device_cus()) ? 128 : 64;
 }
 
 // K slices for problems whose tiles alone cannot fill the chip: aim at ~512 workgroups, at least 4 K slabs each.
@@ -848,9 +851,9 @@ int pick_splits(int64_t M, int64_t N, int64_t K, int requested)
     const int tile      = pick_tile(M, N);
     const int64_t tiles = odl::ceil_div(M, tile) * odl::ceil_div(N, tile);
     const int64_t kt    = odl::ceil_div(K, kBK);
-    if (tiles >= 256 || kt < 8)
+    if (tiles >= odl::device_cus() || kt < 8)
         return 1;
-    int64_t s = odl::ceil_div(512, tiles);
+    int64_t s = odl::ceil_div(2 * odl::device_cus(), tiles);
     if (s > kt / 4)
         s = kt / 4;
     if (s > 128)
@@ -865,6 +868,7 @@ int launch_small_tile_wide_slab(bool ta, bool tb, GemmArgs g, hipStream_t st)
 {
     g.splits = 1;
     g.main_blocks = 0, g.tail_first = g.tiles_m * g.tiles_n, g.tail_splits = 0, g.tail_kps = 0, g.tail_ws = nullptr;
+    g.xcds = odl::chip().xcds;
     const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(kThreads);
 #define ODL_WIDE_CASE(TA, TB)                                                                                  \
     if (ta == TA && tb == TB)                                                                                  \
@@ -968,7 +972,7 @@ namespace
 {
 bool conv_tile_bm64(int64_t M, int64_t N, int splits)
 {
-    return M <= 64 || odl::ceil_div(M, 128) * odl::ceil_div(N, 128) * splits < 256;
+    return M <= 64 || odl::ceil_div(M, 128) * odl::ceil_div(N, 128) * splits < odl::device_cus();
 }
 
 template <int SB, bool TA, int EPI>
@@ -1035,9 +1039,10 @@ int pick_conv_splits(int64_t tiles, int64_t kt, int64_t slots, int64_t max_split
 {
     int best = 1;
     double best_cost = 0;
+    const int64_t cus = odl::device_cus();
     for (int64_t s = 1; s <= max_splits && tiles * s <= slots; ++s)
     {
-        const int64_t per_cu = odl::ceil_div(tiles * s, 256);
+        const int64_t per_cu = odl::ceil_div(tiles * s, cus);
         const double overlap = per_cu == 1 ? 1.25 : (per_cu == 2 ? 1.0 : 0.95);
         const double cost = (double)per_cu * (double)(odl::ceil_div(kt, s) + 3) * overlap + 0.014 * (double)tiles * (double)s;
         if (s == 1 || cost < best_cost)
@@ -1051,7 +1056,7 @@ int wgrad_splits(int64_t OC, int64_t K, int64_t M)
     const int64_t tiles = odl::ceil_div(OC, OC <= 64 ? 64 : 128) * odl::ceil_div(K, 128);
     const int64_t kt = odl::ceil_div(M, kBK);
     const int64_t cap = kt / 8 < 256 ? kt / 8 : 256;
-    return pick_conv_splits(tiles, kt, OC <= 64 ? 1024 : 768, cap);
+    return pick_conv_splits(tiles, kt, (OC <= 64 ? 4 : 3) * (int64_t)odl::device_cus(), cap);
 }
 }  // namespace
 
@@ -1118,7 +1123,7 @@ static int forward_splits(int64_t OC, int64_t M, int64_t K)
     if (tiles128 >= 200 || tiles >= 200 || kt < 8)
         return 1;
     const int64_t cap = kt / 4 < 32 ? kt / 4 : 32;
-    return pick_conv_splits(tiles, kt, OC <= 64 ? 1024 : 768, cap);
+    return pick_conv_splits(tiles, kt, (OC <= 64 ? 4 : 3) * (int64_t)odl::device_cus(), cap);
 }
 
 // The tap-ordered gather: square 1x1 / 3x3 windows over a channel count that fills whole K slabs, image addressed

@@ -15,6 +15,19 @@ int fail(int code, const char *fmt, ...);
 // true when the current device is a gfx950 part; the kernels in this library are built for nothing else
 int require_device();
 
+// Compute units and XCDs (one L2 each) of the current device, read once per device from its properties: a whole
+// MI355X has 256 and 8, a partition of it fewer. Without a visible device the whole chip's figures are returned, so
+// that the workspace-size queries answer on any machine.
+struct Chip
+{
+    int cus, xcds;
+};
+Chip chip();
+inline int device_cus()
+{
+    return chip().cus;
+}
+
 // small fills as kernels (a memset node inside a captured graph is avoided on purpose)
 int fill_launch(float *dst, int64_t n, float value, hipStream_t st);
 int fill_bytes_launch(void *dst, int value, size_t bytes, hipStream_t st);

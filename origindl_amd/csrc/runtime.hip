@@ -53,6 +53,30 @@ int require_device()
         checked[dev] = 1;
     return ODL_OK;
 }
+
+Chip chip()
+{
+    static Chip known[64] = {};
+    const Chip whole{256, 8};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    {
+        (void)hipGetLastError();
+        return whole;
+    }
+    if (known[dev].cus > 0)
+        return known[dev];
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess || prop.multiProcessorCount <= 0)
+    {
+        (void)hipGetLastError();
+        return whole;
+    }
+    // gfx950 exposes 32 compute units per XCD
+    Chip c{prop.multiProcessorCount, prop.multiProcessorCount >= 64 ? prop.multiProcessorCount / 32 : 1};
+    known[dev] = c;
+    return c;
+}
 }  // namespace odl
 
 extern "C" {

@@ -320,7 +320,39 @@ def main():
     path = os.path.join(HERE, "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")
+    detector_at_benchmark_size(r)
+
+
+Y5N320_SEED, Y5N320_INPUT_SEED, Y5N320_ROW_STEP = 3, 8, 16
+
+
+def y5n320_input():
+    """The [4,3,320,320] uniform[0,1) input of the detector benchmark configuration, from a fixed seed (the test
+    regenerates it instead of storing 4.9 MB; the fixture keeps its float64 sum as a guard)."""
+    return np.random.default_rng(Y5N320_INPUT_SEED).random((4, 3, 320, 320), dtype=f32)
+
+
+def detector_at_benchmark_size(r):
+    """tests/golden/ref_y5n320.npz: the YOLOv5n-architecture forward at the benchmark's own size, [4,3,320,320], through
+    the reference's PNNX runner (about a minute on one core here). The output is [4, 6300, 85]; every 16th of the 6300
+    rows of each image is kept (394 rows an image: all three detection scales are sampled, 0.5 MB)."""
+    import tempfile
+    import pnnx_synth
+    with tempfile.TemporaryDirectory() as tmp:
+        param, binp, shp = pnnx_synth.write(os.path.join(tmp, "y5n"), seed=Y5N320_SEED, batch=4, size=320, num_classes=80)
+        xin = y5n320_input()
+        o = np.empty(shp, f32)
+        oshape, nd, ms = np.zeros(8, np.int64), np.zeros(1, np.int32), np.zeros(1, f32)
+        assert r.odl_ref_pnnx_forward(param.encode(), binp.encode(), xin, 4, 3, 320, 320, 1, o, o.size, oshape, nd, ms) == 0
+        assert tuple(oshape[:nd[0]]) == tuple(shp) == (4, 6300, 85)
+    path = os.path.join(HERE, "ref_y5n320.npz")
+    np.savez_compressed(path, rows=np.ascontiguousarray(o[:, ::Y5N320_ROW_STEP, :]), row_step=np.int64(Y5N320_ROW_STEP),
+                        x_sum=np.float64(xin.astype(np.float64).sum()), out_shape=np.asarray(shp, np.int64))
+    print("wrote", path, os.path.getsize(path), "bytes")
 
 
 if __name__ == "__main__":
-    main()
+    if "--detector-only" in sys.argv:
+        detector_at_benchmark_size(ol.ref())
+    else:
+        main()

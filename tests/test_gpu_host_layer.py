@@ -313,6 +313,87 @@ def test_cnn_step_at_reduced_batch_against_the_oracle(h, o):
         np.testing.assert_allclose(a, b, atol=1e-6 + 0.01 * 2e-5 * 10, rtol=0)
 
 
+def test_cnn_step_at_batch_256_against_the_oracle_with_pool_indices_in_full(h, o):
+    """The CNN training configuration at its real batch of 256: the whole step (forward, loss, backward, SGD) against
+    the oracle's step, and both pools' uint64 argmax indices compared in full.
+
+    The indices are compared twice. (1) On identical inputs, bit for bit: the oracle's own post-ReLU activations
+    ([256,32,28,28] and [256,64,14,14], full of exact ties at 0) go through the device pool, whose values and indices
+    must equal the oracle's for every one of the 1 605 632 + 802 816 windows
+    (src/mat/origin/cpu/pooling/max_pool2d.cpp:110-139: first maximum under strict >). (2) End to end: the device's own
+    conv -> ReLU -> pool chain against the oracle's chain. There the pool inputs differ in the last bits (two GEMM
+    summation orders), so an index may differ only where the window's two candidates are closer than the convolution's
+    own bound; every differing window is checked for that and they must be rare."""
+    import torch
+    from origindl_amd import capi
+    rng = np.random.default_rng(6)
+    N, S, C1, C2, Hd, Cc = 256, 28, 32, 64, 128, 10
+    Fd = C2 * (S // 4) ** 2
+    x = rng.random((N, 1, S, S), dtype=f32)
+    t = rng.integers(0, Cc, size=N).astype(np.int32)
+    shapes = ((C1, 1, 3, 3), (C1,), (C2, C1, 3, 3), (C2,), (Fd, Hd), (1, Hd), (Hd, Cc), (1, Cc))
+    fans = (9, 0, 9 * C1, 0, Fd, 0, Hd, 0)
+    params = [(rng.standard_normal(s, dtype=f32) * f32(np.sqrt(2.0 / f) if f else 0.05)).astype(f32)
+              for s, f in zip(shapes, fans)]
+    po = [a.copy() for a in params]
+    go = [np.empty_like(a) for a in po]
+    loss_o, logits_o = np.zeros(1, f32), np.empty((N, Cc), f32)
+    idx1 = np.empty((N, C1, S // 2, S // 2), np.uint64)
+    idx2 = np.empty((N, C2, S // 4, S // 4), np.uint64)
+    print("\n[case] cnn step batch 256: oracle", flush=True)
+    assert o.orc_cnn_train_step(x, t, 0, N, S, C1, C2, Hd, Cc, *po, 0.01, loss_o, idx1, idx2, *go, logits_o) == 0
+    print("[case] cnn step batch 256: device", flush=True)
+    ph = [a.copy() for a in params]
+    gh = [np.empty_like(a) for a in ph]
+    loss_h, logits_h = np.zeros(1, f32), np.empty((N, Cc), f32)
+    assert h.odl_host_cnn_train(x, t, 0, N, S, C1, C2, Hd, Cc, *ph, 0.01, loss_h, *gh, logits_h) == 0
+    assert abs(loss_h[0] - loss_o[0]) <= 1e-4 * abs(loss_o[0])
+    np.testing.assert_allclose(logits_h, logits_o, atol=5e-4)
+    for a, b, s in zip(gh, go, shapes):
+        np.testing.assert_allclose(a, b, atol=2e-5 * max(np.abs(b).max(), 1.0), rtol=0, err_msg=str(s))
+    for a, b in zip(ph, po):
+        np.testing.assert_allclose(a, b, atol=1e-6 + 0.01 * 2e-5 * 10, rtol=0)
+
+    def dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    def oracle_layer(inp, w, b, C, H, OC):
+        a = np.empty((N, OC, H, H), f32)
+        assert o.orc_conv2d(inp, w, b, N, C, H, H, OC, 3, 3, 1, 1, 1, 1, a) == 0
+        o.orc_unary(0, a, a.size, a)  # ReLU in place
+        y, idx = np.empty((N, OC, H // 2, H // 2), f32), np.empty((N, OC, H // 2, H // 2), np.uint64)
+        assert o.orc_max_pool2d(a, N, OC, H, H, 2, 2, 2, 2, 0, 0, y, idx) == 0
+        return a, y, idx
+
+    def near_tie_only(act_dev, idx_dev, idx_ref, act_ref, slack):
+        """every window whose index differs holds, in the device's own activation, two candidates within `slack`"""
+        bad = np.argwhere(idx_dev != idx_ref)
+        for n, c, i, j in bad:
+            cand = lambda a, k: a[n, c, 2 * i + int(k) // 2, 2 * j + int(k) % 2]  # noqa: E731
+            kd, kr = idx_dev[n, c, i, j], idx_ref[n, c, i, j]
+            assert abs(cand(act_dev, kd) - cand(act_dev, kr)) <= slack and abs(cand(act_ref, kd) - cand(act_ref, kr)) <= slack
+        return len(bad)
+
+    inp_o, inp_d = x, dev(x)
+    for li, (w, b, C, H, OC, idx_step) in enumerate(((params[0], params[1], 1, S, C1, idx1),
+                                                     (params[2], params[3], C1, S // 2, C2, idx2))):
+        print("[case] cnn step batch 256: pool", li + 1, flush=True)
+        a_o, y_o, idx_o = oracle_layer(inp_o, w, b, C, H, OC)
+        assert np.array_equal(idx_o, idx_step)  # the layer-by-layer oracle is the oracle's training step
+        # (1) identical inputs: values and all indices bit-exact
+        y_d, idx_d = capi.max_pool2d(dev(a_o), 2, 2, 0)
+        assert np.array_equal(y_d.cpu().numpy(), y_o)
+        assert np.array_equal(idx_d.cpu().numpy().view(np.uint64), idx_o)
+        # (2) the device's own chain
+        a_d = capi.unary("relu", capi.conv2d(inp_d, dev(w), dev(b), 1, 1))
+        p_d, idx_own = capi.max_pool2d(a_d, 2, 2, 0)
+        slack = 1e-5 * float(np.sqrt(9 * C)) * float(np.abs(inp_o).max()) * float(np.linalg.norm(w.reshape(OC, -1), axis=1).max())
+        differing = near_tie_only(a_d.cpu().numpy(), idx_own.cpu().numpy().view(np.uint64), idx_o, a_o, slack)
+        print("[case] windows whose argmax differs end to end: %d of %d" % (differing, idx_o.size), flush=True)
+        assert differing <= idx_o.size * 1e-4
+        inp_o, inp_d = y_o, p_d
+
+
 def test_reference_example_nn_linear_runs_unchanged_on_the_gpu():
     """oracle/_ref/example_nn_linear_hip is the reference's tests/example/linear_regression/nn_linear.cpp compiled,
     unmodified, against origindl_amd/host/include and linked to the gfx950 backend (make -C oracle ref-examples; built
@@ -439,6 +520,32 @@ def test_yolov5n_pnnx_forward_matches_the_reference(h, tmp_path):
     # a second forward on the same graph object reuses the uploaded weights and gives the same answer
     rc, out2, _, _ = _run_pnnx(h, "odl_host_", param, binp, G["y5n64_x"], shp, reps=3)
     assert rc == 0 and np.array_equal(out, out2)
+
+
+def test_yolov5n_pnnx_forward_at_the_benchmark_size_matches_the_reference(h, tmp_path):
+    """The detector benchmark configuration itself — batch 4 at 320x320 — against the reference's PNNX runner: the fixture
+    ref_y5n320.npz (tests/golden/make_golden.py) holds every 16th of the 6300 output rows of each image, all three
+    detection scales among them. Same bar as at 64x64."""
+    import pnnx_synth
+    sys_path_golden = os.path.join(os.path.dirname(__file__), "golden")
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(sys_path_golden, "make_golden.py"))
+    mg = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mg)
+    F = np.load(os.path.join(sys_path_golden, "ref_y5n320.npz"))
+    x = mg.y5n320_input()
+    assert float(x.astype(np.float64).sum()) == float(F["x_sum"])  # the seeded input is the one the fixture was made from
+    param, binp, shp = pnnx_synth.write(str(tmp_path / "y5n"), seed=mg.Y5N320_SEED, batch=4, size=320, num_classes=80)
+    assert tuple(shp) == tuple(int(v) for v in F["out_shape"]) == (4, 6300, 85)
+    print("\n[case] yolov5n 4x3x320x320", flush=True)
+    rc, out, oshape, _ = _run_pnnx(h, "odl_host_", param, binp, x, shp)
+    assert rc == 0 and oshape == (4, 6300, 85)
+    got, want = out[:, ::int(F["row_step"]), :], F["rows"]
+    assert got.shape == want.shape
+    err = np.abs(got - want) / (np.abs(want) + 1.0)
+    print("[yolov5n 320x320, batch 4] max scaled deviation %.3g over %d values" % (err.max(), want.size), flush=True)
+    assert err.max() < 1e-5
+    assert np.isfinite(out).all()
 
 
 def test_pnnx_runner_rejects_bad_files(h, tmp_path):

@@ -329,6 +329,26 @@ def test_against_compiled_reference_fresh_inputs():
     assert acc[0] == o.orc_accuracy(y, t, 50, 6)
 
 
+def test_argmax_rows_is_the_first_maximum():
+    # src/utils/metrics.cpp:40-53: the scan starts at column 0 and moves on strict > only, so among equal maxima the
+    # first wins — which is numpy's argmax; accuracy is then the mean of (argmax == label) in float
+    o = ol.oracle()
+    rng = np.random.default_rng(77)
+    y = rng.integers(0, 3, size=(400, 7)).astype(f32)  # three distinct values in seven columns: ties in every row
+    y[::5, 0] = 2  # maximum in the first column
+    y[1::5, :] = -1.5  # a whole row of equal values
+    y[2::5, 6] = 9  # maximum in the last column only
+    am = np.full(400, -1, np.int64)
+    o.orc_argmax_rows(y, 400, 7, am)
+    assert np.array_equal(am, np.argmax(y, axis=1))
+    assert (am[1::5] == 0).all() and (am[2::5] == 6).all()
+    t = rng.integers(0, 7, size=400).astype(np.int32)
+    assert o.orc_accuracy(y, t, 400, 7) == f32((np.argmax(y, axis=1) == t).sum()) / f32(400)
+    one = np.array([[3.0]], f32)
+    o.orc_argmax_rows(one, 1, 1, am)
+    assert am[0] == 0
+
+
 BN_CASES = {"bnA": (6, 5, 0, 0), "bnB": (3, 4, 5, 6), "bnC": (1, 2, 3, 3), "bnD": (4, 3, 2, 2)}
 
 
