@@ -154,6 +154,17 @@ int odl_hip_set_conv_patch_min_workgroups(int64_t min_workgroups);
 int odl_hip_sum_axis(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *workspace,
                      size_t workspace_bytes, void *stream);
 size_t odl_hip_sum_axis_workspace_bytes(int64_t outer, int64_t axis, int64_t inner);
+/* odl_hip_sum_axis for callers that cannot allocate device memory and so cannot bring a workspace: code running under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. The
+ * partial sums go to an array that is part of the library's device image (8 MiB, held by every GPU the library runs on
+ * until the process ends; odl_hip_sum_axis_noalloc_max_bytes returns the size) instead of a workspace; kernels, plan
+ * and order of additions are those of odl_hip_sum_axis, so results are bit-identical to it. The call allocates nothing
+ * and frees nothing. A reduction whose partial sums (odl_hip_sum_axis_workspace_bytes) do not fit the array is refused
+ * with ODL_ERR_INVALID_ARG; the [16384, 4096] -> [4096] bias gradient fits exactly. All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU (two streams, two threads) race, so order them. The first call on
+ * each device resolves the array's address and must come outside stream capture (ODL_ERR_RUNTIME otherwise). */
+int odl_hip_sum_axis_noalloc(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *stream);
+size_t odl_hip_sum_axis_noalloc_max_bytes(void);
 /* Mat::sum(-1): all elements -> dst[0] (operation_templates.h:342-357) */
 int odl_hip_sum_all(const float *src, int64_t n, float *dst, void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_sum_all_workspace_bytes(int64_t n);

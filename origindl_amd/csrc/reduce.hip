@@ -9,6 +9,8 @@
 
 #include "odl_common.h"
 
+#include <mutex>
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace
@@ -571,6 +573,71 @@ int odl_hip_sum_axis(const float *src, int64_t outer, int64_t axis, int64_t inne
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, "sum: negative extent");
     return sum_axis_launch(src, outer, axis, inner, dst, workspace, workspace_bytes, odl::as_stream(stream));
+}
+
+// ---- the same reduction for callers that cannot allocate (and so cannot bring a workspace): the partial sums go to
+// an array that is part of the library's device image. Every device holds its own copy at its own address; the name
+// `scratch` is only the host-side handle of that symbol, so launches get the address hipGetSymbolAddress reports.
+}  // extern "C"
+
+namespace
+{
+constexpr size_t kScratchBytes = (size_t)8 << 20;
+// (kept in the device image although no kernel names it: kernels receive its address as an argument)
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kScratchBytes];
+
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[64] = {nullptr};  // per device, resolved on the first call with that device current
+
+int scratch_of_current_device(hipStream_t st, void **out)
+{
+    int dev = -1;
+    ODL_HIP_CHECK(hipGetDevice(&dev));
+    ODL_REQUIRE(dev >= 0 && dev < 64, "sum_axis_noalloc: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr)
+    {
+        // resolving the symbol may load the device image: not something to do while a stream is recording
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        ODL_HIP_CHECK(hipStreamIsCapturing(st, &cap));
+        if (cap != hipStreamCaptureStatusNone)
+            return odl::fail(ODL_ERR_RUNTIME, "sum_axis_noalloc: the first call on a device must come outside stream capture");
+        void *ptr = nullptr;
+        ODL_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (ptr == nullptr)
+            return odl::fail(ODL_ERR_RUNTIME, "sum_axis_noalloc: the scratch array has no device address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return ODL_OK;
+}
+}  // namespace
+
+extern "C" {
+size_t odl_hip_sum_axis_noalloc_max_bytes(void)
+{
+    return kScratchBytes;
+}
+
+int odl_hip_sum_axis_noalloc(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, "sum: negative extent");
+    const size_t need = (outer > 0 && axis > 0 && inner > 0) ? plan_sum(outer, axis, inner).ws_bytes : 0;
+    if (need > kScratchBytes)
+        return odl::fail(ODL_ERR_INVALID_ARG,
+                         "sum_axis_noalloc: [%lld, %lld, %lld] needs %zu bytes of partial sums, the built-in scratch holds %zu; "
+                         "use odl_hip_sum_axis with a workspace",
+                         (long long)outer, (long long)axis, (long long)inner, need, kScratchBytes);
+    void *ws = nullptr;
+    if (need > 0)
+    {
+        const int rc = scratch_of_current_device(odl::as_stream(stream), &ws);
+        if (rc != ODL_OK)
+            return rc;
+    }
+    // every partial the fold reads is written by the pass before it in the same call: nothing has to start at zero
+    return sum_axis_launch(src, outer, axis, inner, dst, ws, need, odl::as_stream(stream));
 }
 
 size_t odl_hip_sum_all_workspace_bytes(int64_t n)
