@@ -48,8 +48,13 @@ const char *odl_hip_last_error(void);
 int odl_hip_malloc(void **ptr, size_t bytes);
 int odl_hip_free(void *ptr);
 int odl_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
-/* src/mat/origin/memory/storage.cpp:69-145 — synchronous copies, device-synchronised before D2H */
-int odl_hip_memcpy_h2d(void *dst, const void *host_src, size_t bytes);
+/* src/mat/origin/memory/storage.cpp:69-145 — synchronous copies, device-synchronised before D2H.
+ * h2d: the reference copies on the null stream, where all its kernels run too, so a copy into recycled memory waits for
+ * the kernels that last used it. Created streams here are non-blocking — they and the null stream do not wait for each
+ * other — so a caller that launches on a created stream passes that stream: the copy is queued behind everything
+ * already on it and the call returns when the data has landed. stream = NULL is the reference's plain blocking copy,
+ * ordered only against null-stream work. */
+int odl_hip_memcpy_h2d(void *dst, const void *host_src, size_t bytes, void *stream);
 int odl_hip_memcpy_d2h(void *host_dst, const void *src, size_t bytes);
 int odl_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
 int odl_hip_memset(void *dst, int value, size_t bytes, void *stream);
@@ -66,6 +71,10 @@ int odl_hip_stream_destroy(void *stream);
 int odl_hip_stream_synchronize(void *stream);
 int odl_hip_graph_capture_begin(void *stream);
 int odl_hip_graph_capture_end(void *stream, void **graph_exec);
+/* gives up a capture (after an error in the middle of the step being recorded): the stream leaves capture mode,
+ * whatever was recorded is discarded, the stream can be used and captured again. A no-op on a stream that is not
+ * capturing. */
+int odl_hip_graph_capture_abort(void *stream);
 int odl_hip_graph_launch(void *graph_exec, void *stream);
 int odl_hip_graph_destroy(void *graph_exec);
 

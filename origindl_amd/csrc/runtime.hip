@@ -163,10 +163,20 @@ int odl_hip_mem_info(size_t *free_bytes, size_t *total_bytes)
     return ODL_OK;
 }
 
-int odl_hip_memcpy_h2d(void *dst, const void *host_src, size_t bytes)
+int odl_hip_memcpy_h2d(void *dst, const void *host_src, size_t bytes, void *stream)
 {
-    if (bytes)
+    if (!bytes)
+        return ODL_OK;
+    if (stream == nullptr)
+    {
         ODL_HIP_CHECK(hipMemcpy(dst, host_src, bytes, hipMemcpyHostToDevice));
+        return ODL_OK;
+    }
+    // A created stream does not wait for the null stream nor the null stream for it: the copy goes onto the stream
+    // itself, behind every kernel queued there (one of them may still be using the block `dst` was recycled from),
+    // and the call returns when it has landed, so the host buffer can be reused at once.
+    ODL_HIP_CHECK(hipMemcpyAsync(dst, host_src, bytes, hipMemcpyHostToDevice, odl::as_stream(stream)));
+    ODL_HIP_CHECK(hipStreamSynchronize(odl::as_stream(stream)));
     return ODL_OK;
 }
 
@@ -238,6 +248,23 @@ int odl_hip_graph_capture_end(void *stream, void **graph_exec)
     if (e != hipSuccess)
         return odl::fail(ODL_ERR_RUNTIME, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
     *graph_exec = exec;
+    return ODL_OK;
+}
+
+int odl_hip_graph_capture_abort(void *stream)
+{
+    ODL_REQUIRE(stream != nullptr, "graph_capture_abort: null stream");
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(odl::as_stream(stream), &status) != hipSuccess)
+        (void)hipGetLastError();
+    if (status == hipStreamCaptureStatusNone)
+        return ODL_OK;
+    // ending an invalidated capture reports an error and hands back no graph: both are what is wanted here
+    hipGraph_t graph = nullptr;
+    if (hipStreamEndCapture(odl::as_stream(stream), &graph) != hipSuccess)
+        (void)hipGetLastError();
+    if (graph)
+        (void)hipGraphDestroy(graph);
     return ODL_OK;
 }
 

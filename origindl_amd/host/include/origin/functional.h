@@ -104,6 +104,10 @@ std::vector<Tensor> batch_norm_outputs(const Tensor &x, const Tensor &gamma, con
 Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b);
 Tensor softmax(const Tensor &x, int axis = -1);
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &target);
+// After replaying a recorded step on new labels: whether the loss kernel met an out-of-range label (the ordinary call
+// throws std::invalid_argument for one, as the reference's gather does; a recorded step cannot). `loss` is the tensor
+// softmax_cross_entropy returned while the step was recorded. Reads two words back from the device.
+bool softmax_cross_entropy_bad_label(const Tensor &loss);
 Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b = nullptr, std::pair<int, int> stride = {1, 1},
               std::pair<int, int> pad = {0, 0});
 Tensor conv2d(const Tensor &x, const Tensor &W, const Tensor *b, int stride, int pad);

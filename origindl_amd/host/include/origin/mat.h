@@ -294,7 +294,13 @@ public:
     // (one small device-to-host copy; no upload of the loss afterwards)
     std::unique_ptr<Mat> softmax_cross_entropy_checked(const Mat &target) const;
     std::unique_ptr<Mat> softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const;
-    // overwrites this tensor's elements from host memory (synchronises first: work in flight may still read them)
+    // on a loss made by softmax_cross_entropy_device / _checked: the out-of-range-label flag that lies behind the loss
+    // in device memory, read back now (one small device-to-host copy; synchronises). A recorded step cannot raise the
+    // reference's exception for a bad label — it contributes nothing to the loss — so a caller that replays a graph on
+    // new labels looks here after the replay. False for any other tensor.
+    bool loss_bad_label_flag() const;
+    // overwrites this tensor's elements from host memory (the copy is queued behind the work already on the current
+    // stream, which may still read them, and has landed when the call returns)
     void upload(const void *host, size_t bytes);
     // the fused Adam step written over this parameter, bias-correction factors read from device memory
     void adam_step_inplace(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, const float *device_scales, float eps,

@@ -286,6 +286,8 @@ void destroy_stream(void *stream);
 void set_stream(void *stream);  // nullptr = the null stream; synchronises the device when the stream changes
 void *current_stream();
 bool is_capturing();
+// hands every cached block of the device memory pool that no tensor holds back to the driver (synchronises first)
+void empty_cache();
 
 class Graph
 {
@@ -295,12 +297,14 @@ public:
     Graph(const Graph &) = delete;
     Graph &operator=(const Graph &) = delete;
     void begin_capture();
-    void end_capture();
+    void end_capture();    // only the Graph that began the capture may end it
+    void abort_capture();  // gives the capture up: the thread, its stream and the memory pool are as before begin_capture
     void launch();  // on the current stream
     bool captured() const { return exec_ != nullptr; }
 
 private:
     void *exec_ = nullptr;
+    bool began_ = false;  // between this object's begin_capture and its end_capture / abort_capture
     std::shared_ptr<void> arena_;
 };
 }  // namespace cuda

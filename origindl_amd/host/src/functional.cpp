@@ -322,6 +322,7 @@ struct Softmax : Operator  // src/operators/activation/softmax.cpp:14-129
 
 struct SoftmaxCrossEntropy : Operator  // src/operators/loss/softmax_cross_entropy.cpp:17-111
 {
+    static bool bad_label(const Tensor &loss) { return omat(loss).loss_bad_label_flag(); }
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
         if (xs.size() != 2)
@@ -713,6 +714,7 @@ Tensor batch_norm(const Tensor &x, const Tensor &gamma, const Tensor &beta, cons
 Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b) { return apply<FusedLinear>({x, w, b}); }
 Tensor softmax(const Tensor &x, int axis) { return apply<Softmax>({x}, axis); }
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &t) { return apply<SoftmaxCrossEntropy>({x, t}); }
+bool softmax_cross_entropy_bad_label(const Tensor &loss) { return SoftmaxCrossEntropy::bad_label(loss); }
 
 Tensor flatten(const Tensor &x, int start_dim, int end_dim)  // src/operators/shape/flatten.cpp
 {

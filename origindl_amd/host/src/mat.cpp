@@ -9,6 +9,7 @@
 #include <memory>
 #include <unordered_map>
 #include <mutex>
+#include <thread>
 #include <random>
 
 #include "odl_hip.h"
@@ -83,7 +84,8 @@ public:
         std::shared_ptr<Arena> arena;
         {
             std::lock_guard<std::mutex> lk(mu_);
-            arena = capture_arena_;
+            if (capture_arena_ && capture_thread_ == std::this_thread::get_id())
+                arena = capture_arena_;  // only the recording thread's blocks belong to the graph
             void *p = nullptr;
             if (arena)
                 p = take(arena->free_, cap);
@@ -97,7 +99,14 @@ public:
             }
         }
         void *p = nullptr;
-        check(odl_hip_malloc(&p, cap));
+        if (odl_hip_malloc(&p, cap) != ODL_OK)
+        {
+            // out of device memory with blocks parked in the bins: give them back and try once more
+            if (!arena && odl_hip_synchronize() == ODL_OK && trim() > 0)
+                check(odl_hip_malloc(&p, cap));
+            else
+                check(ODL_ERR_RUNTIME);
+        }
         if (arena)
         {
             std::lock_guard<std::mutex> lk(mu_);
@@ -126,7 +135,25 @@ public:
         if (capture_arena_)
             THROW_RUNTIME_ERROR("a graph is already being captured");
         capture_arena_ = std::make_shared<Arena>();
+        capture_thread_ = std::this_thread::get_id();
         return capture_arena_;
+    }
+    // frees every block of the ordinary bins (the caller has synchronised the device); returns how many
+    size_t trim()
+    {
+        std::map<size_t, std::vector<void *>> bins;
+        {
+            std::lock_guard<std::mutex> lk(mu_);
+            bins.swap(free_);
+        }
+        size_t n = 0;
+        for (auto &bin : bins)
+            for (void *p : bin.second)
+            {
+                (void)odl_hip_free(p);
+                ++n;
+            }
+        return n;
     }
     void end_capture()
     {
@@ -159,6 +186,7 @@ private:
     std::mutex mu_;
     std::map<size_t, std::vector<void *>> free_;
     std::shared_ptr<Arena> capture_arena_;
+    std::thread::id capture_thread_;
     std::unordered_map<void *, std::weak_ptr<Arena>> owner_;
 };
 
@@ -325,7 +353,7 @@ std::shared_ptr<Storage> Storage::to_device(DeviceType type, int index) const
     else if (type_ == DeviceType::kCPU)
     {
         no_capture("host-to-device copy");
-        check(odl_hip_memcpy_h2d(dst->data(), data_, size_));
+        check(odl_hip_memcpy_h2d(dst->data(), data_, size_, cur()));
     }
     else if (type == DeviceType::kCPU)
     {
@@ -392,7 +420,7 @@ std::unique_ptr<Mat> upload_new(const void *host, DataType dt, const Shape &shap
     else
     {
         no_capture("host-to-device copy");
-        check(odl_hip_memcpy_h2d(m->data_ptr(), host, bytes));
+        check(odl_hip_memcpy_h2d(m->data_ptr(), host, bytes, cur()));
     }
     return m;
 }
@@ -592,7 +620,7 @@ void OriginMat::index_put(std::initializer_list<size_t> indices, const Scalar &v
     {
         no_capture("host-to-device copy");
         check(odl_hip_synchronize());
-        check(odl_hip_memcpy_h2d(dst, element, width));
+        check(odl_hip_memcpy_h2d(dst, element, width, cur()));
     }
 }
 
@@ -1313,7 +1341,7 @@ std::unique_ptr<Mat> OriginMat::max_pool2d_backward(const Mat &gym, std::pair<in
                           indices.size());
     auto idx = Storage::create(indices.size() * sizeof(uint64_t), DeviceType::kCUDA, gy.device().index());
     no_capture("host-to-device copy");
-    check(odl_hip_memcpy_h2d(idx->data(), indices.data(), indices.size() * sizeof(uint64_t)));
+    check(odl_hip_memcpy_h2d(idx->data(), indices.data(), indices.size() * sizeof(uint64_t), cur()));
     return max_pool2d_backward_device(gym, k, s, p, *idx);
 }
 
@@ -1415,6 +1443,17 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target)
     return loss;
 }
 
+bool OriginMat::loss_bad_label_flag() const
+{
+    if (device().type() != DeviceType::kCUDA || dtype_ != DataType::kFloat32 || elements() != 1 || !storage_ ||
+        storage_->size() != 2 * sizeof(float))
+        return false;
+    unsigned words[2] = {0, 0};
+    no_capture("device-to-host copy");
+    check(odl_hip_memcpy_d2h(words, storage_->data(), sizeof(words)));
+    return words[1] != 0;
+}
+
 std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const
 {
     const OriginMat &x = dev_f32(*this, "softmax_cross_entropy");
@@ -1439,8 +1478,8 @@ void OriginMat::upload(const void *host, size_t bytes)
         return;
     }
     no_capture("host-to-device copy");
-    check(odl_hip_synchronize());
-    check(odl_hip_memcpy_h2d(storage_->data(), host, bytes));
+    // queued behind everything on the current stream that still reads the old contents
+    check(odl_hip_memcpy_h2d(storage_->data(), host, bytes, cur()));
 }
 
 void OriginMat::adam_step_inplace(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, const float *device_scales,
@@ -1652,8 +1691,17 @@ bool is_capturing()
     return t_capturing;
 }
 
+void empty_cache()
+{
+    check(odl_hip_synchronize());
+    DevicePool::get().trim();
+}
+
 Graph::~Graph()
 {
+    // a Graph destroyed in the middle of its capture (an exception unwound past it) must not leave the thread recording
+    if (began_)
+        abort_capture();
     if (exec_)
     {
         (void)odl_hip_synchronize();  // no replay may still be running when its memory is handed back
@@ -1676,12 +1724,28 @@ void Graph::begin_capture()
         THROW_RUNTIME_ERROR("{}", odl_hip_last_error());
     }
     t_capturing = true;
+    began_ = true;
+}
+
+void Graph::abort_capture()
+{
+    if (!began_)
+        return;
+    began_ = false;
+    t_capturing = false;
+    DevicePool::get().end_capture();
+    (void)odl_hip_graph_capture_abort(t_stream);
+    (void)odl_hip_stream_synchronize(t_stream);
+    arena_.reset();  // the blocks of the capture run return to the ordinary pool as their tensors die
 }
 
 void Graph::end_capture()
 {
     if (!t_capturing)
         THROW_RUNTIME_ERROR("end_capture without begin_capture");
+    if (!began_)
+        THROW_RUNTIME_ERROR("end_capture on a Graph that did not begin the capture in progress");
+    began_ = false;
     t_capturing = false;
     DevicePool::get().end_capture();
     void *exec = nullptr;

@@ -835,6 +835,138 @@ int DRV(mlp_train_graph)(const float *x, const void *t, int is64, int64_t N, int
 }
 #endif
 
+#ifdef DRV_ON_DEVICE
+// Uploads into recycled device memory must wait for the kernels that still read it. On a created (non-blocking) stream:
+// `reps` products of an all-ones [n,n] matrix are queued, the matrix is dropped while they are still running — its block
+// returns to the pool — and a host array of the same size is uploaded at once, which the pool serves from that block.
+// wrong[0] counts product elements that are not n (a product that read the overwritten operand), wrong[1] elements of
+// the uploaded tensor that did not arrive.
+int DRV(upload_ordering)(int64_t n, int reps, int64_t *wrong)
+{
+    return guarded([&] {
+        StreamScope stream;
+        const Shape shp{(size_t)n, (size_t)n};
+        std::vector<float> ones((size_t)(n * n), 1.0f), twos((size_t)(n * n), 2.0f);
+        auto w = mat_f32(ones.data(), shp);
+        auto x = mat_f32(ones.data(), shp);
+        std::vector<std::unique_ptr<origin::Mat>> ys;
+        for (int r = 0; r < reps; ++r)
+            ys.push_back(x->matmul(*w));
+        x.reset();
+        auto b = mat_f32(twos.data(), shp);
+        wrong[0] = wrong[1] = 0;
+        for (auto &y : ys)
+            for (float v : static_cast<const OriginMat &>(*y).to_vector<float>())
+                wrong[0] += v != (float)n;
+        for (float v : static_cast<const OriginMat &>(*b).to_vector<float>())
+            wrong[1] += v != 2.0f;
+    });
+}
+
+// A capture that fails in the middle must leave the thread usable. stage[0] counts how far the scenario got:
+// 1 the exception of a host read inside a capture arrived, 2 an ordinary step ran afterwards, 3 a fresh capture and a
+// replay ran and the replayed loss equals the ordinary one of the same step, 4 end_capture from a Graph that did not begin
+// the capture was refused (and that capture given up cleanly), 5 ordinary work still runs. After a replay on labels with
+// an out-of-range entry flags[0] holds the loss's bad-label flag, after a replay on the good labels again flags[1].
+int DRV(graph_abort_recovery)(const float *x, const int32_t *t, int64_t N, int64_t D, int64_t C, int *stage, int *flags)
+{
+    return guarded([&] {
+        StreamScope stream;
+        *stage = 0;
+        auto run = [&](int steps, bool replay_last, float *loss_out) {
+            Sequential model;
+            model.add(std::make_unique<nn::Linear>((int)D, (int)C, true));
+            auto &l = dynamic_cast<nn::Linear &>(model[0]);
+            std::vector<float> w((size_t)(D * C));
+            for (size_t i = 0; i < w.size(); ++i)
+                w[i] = 0.01f * (float)((int)(i % 7) - 3);
+            *l.weight() = Parameter(f32(w.data(), Shape{(size_t)D, (size_t)C}, true));
+            std::vector<float> zeros((size_t)C, 0.0f);
+            *l.bias() = Parameter(f32(zeros.data(), Shape{1, (size_t)C}, true));
+            SGD opt(model, 0.1f);
+            auto X = f32(x, Shape{(size_t)N, (size_t)D});
+            auto T = labels(t, 0, N);
+            model.train();
+            auto step = [&] {
+                opt.zero_grad();
+                auto L = F::softmax_cross_entropy(model(X), T);
+                L.backward();
+                opt.step();
+                return L;
+            };
+            for (int s = 0; s + 1 < steps; ++s)
+                step();
+            if (!replay_last)
+            {
+                *loss_out = step().item<float>();
+                return;
+            }
+            origin::cuda::Graph g;
+            g.begin_capture();
+            auto L = step();
+            g.end_capture();
+            // the capture run itself executed nothing: the replay is step number `steps`
+            g.launch();
+            *loss_out = L.item<float>();
+            if (flags)
+            {
+                std::vector<int32_t> bad(t, t + N);
+                bad[(size_t)(N / 2)] = (int32_t)C;  // one past the last class
+                T.upload(bad.data(), bad.size() * sizeof(int32_t));
+                g.launch();
+                flags[0] = F::softmax_cross_entropy_bad_label(L) ? 1 : 0;
+                T.upload(t, (size_t)N * sizeof(int32_t));
+                g.launch();
+                flags[1] = F::softmax_cross_entropy_bad_label(L) ? 1 : 0;
+            }
+        };
+        try
+        {
+            origin::cuda::Graph g;
+            g.begin_capture();
+            auto X = f32(x, Shape{(size_t)N, (size_t)D});  // a host-to-device copy: not allowed while recording
+            (void)X;
+            g.end_capture();
+        }
+        catch (const std::runtime_error &)
+        {
+            *stage = 1;
+        }
+        if (*stage != 1 || origin::cuda::is_capturing())
+            return;
+        float eager = 0.f, replayed = 0.f;
+        run(3, false, &eager);
+        *stage = 2;
+        run(3, true, &replayed);
+        if (eager != replayed)
+            return;
+        *stage = 3;
+        {
+            origin::cuda::Graph a, b;
+            a.begin_capture();
+            bool refused = false;
+            try
+            {
+                b.end_capture();
+            }
+            catch (const std::runtime_error &)
+            {
+                refused = true;
+            }
+            a.abort_capture();
+            if (!refused || origin::cuda::is_capturing())
+                return;
+        }
+        *stage = 4;
+        float again = 0.f;
+        flags = nullptr;
+        run(3, false, &again);
+        if (again == eager)
+            *stage = 5;
+    });
+}
+#endif
+
 // CNN of the benchmark's CNN training configuration (no BatchNorm), SGD without momentum/weight decay, one step.
 int DRV(cnn_train)(const float *x, const void *t, int is64, int64_t N, int64_t S, int64_t C1, int64_t C2, int64_t Hd,
                       int64_t Cc, float *Wc1, float *bc1, float *Wc2, float *bc2, float *Wl1, float *bl1, float *Wl2,

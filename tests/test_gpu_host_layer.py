@@ -231,6 +231,31 @@ def test_recorded_training_step_replays_bit_for_bit(h, wd):
                 assert np.array_equal(a, b), steps
 
 
+def test_upload_into_recycled_memory_waits_for_the_kernels_still_reading_it(h):
+    """On a created stream (which the null stream does not wait for), five 2048^3 products of an all-ones matrix are
+    queued, the matrix is dropped and a host array of its size uploaded straight away — the pool serves the upload from
+    the block the products are still reading. The copy must queue behind them: every product element is still 2048
+    and the uploaded tensor arrived whole."""
+    wrong = np.full(2, -1, np.int64)
+    assert h.odl_host_upload_ordering(2048, 5, wrong) == 0
+    assert wrong.tolist() == [0, 0]
+
+
+def test_a_failed_capture_leaves_the_thread_usable_and_replays_report_bad_labels(h):
+    """An exception in the middle of a capture (here: a host-to-device copy, which a recorded step may not contain) unwinds
+    past the Graph object; its destructor gives the capture up. Afterwards ordinary steps run, a fresh capture records and
+    replays bit for bit, a Graph that did not begin a capture cannot end it, and after a replay on labels with an
+    out-of-range entry the loss's flag word says so (the ordinary call would have thrown)."""
+    rng = np.random.default_rng(44)
+    N, D, C = 64, 32, 10
+    x = rng.standard_normal((N, D), dtype=f32)
+    t = rng.integers(0, C, size=N).astype(np.int32)
+    stage, flags = np.zeros(1, np.int32), np.full(2, -1, np.int32)
+    assert h.odl_host_graph_abort_recovery(x, t, N, D, C, stage, flags) == 0
+    assert stage[0] == 5, stage[0]
+    assert flags.tolist() == [1, 0]
+
+
 def test_reference_example_network_with_batch_norm_trains_and_replays(h):
     """The network of the reference's tests/example/mnist/conv_mnist.cpp (two conv + BatchNorm + ReLU + pool blocks,
     two Linear layers, Adam + WeightDecay) at batch 16: eight ordinary steps, and two ordinary steps followed by six
