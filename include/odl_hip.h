@@ -253,6 +253,33 @@ int odl_hip_binary(int op, const float *a, int64_t na, const float *b, int64_t n
 int odl_hip_unary(int op, const float *a, int64_t n, float *out, void *stream);
 /* origin::cuda::pow with a float32 scalar exponent (src/mat/origin/cpu/math/pow.cpp:35-43) */
 int odl_hip_pow_scalar(const float *a, int64_t n, float exponent, float *out, void *stream);
+/* ------------------------------------------------------------------ element types besides float32 -- */
+/* The reference dispatches its elementwise, reduction and conversion operators over six element types
+ * (include/origin/mat/origin/device_common/type_dispatcher.h:26-88). Type codes here are its DataType enumerators
+ * (include/origin/mat/basic_types.h:19-27): 0 float32, 1 float64, 2 int8, 3 int32, 4 int64, 5 uint8. float32 is what the
+ * hot path computes in; with code 0 these entry points forward to the float32 ones above. */
+size_t odl_hip_dtype_size(int dtype);
+/* origin::cuda::convert_datatype (src/mat/origin/cuda/type_conversion.cu; include/origin/mat/origin/cuda/cuda_kernels.cuh
+ * type_conversion_kernel): dst[i] = static_cast<Dst>(src[i]) on the device, any pair of types */
+int odl_hip_convert(const void *src, int src_dtype, void *dst, int dst_dtype, int64_t n, void *stream);
+/* odl_hip_binary ops 0-9 in any element type; integer arithmetic wraps, an integer division by zero gives 0,
+ * comparisons give 0/1 in the operands' type (operation_templates.h:177-240). Same broadcasting rule. */
+int odl_hip_binary_dtype(int op, int dtype, const void *a, int64_t na, const void *b, int64_t nb, void *out, void *stream);
+/* odl_hip_unary: relu, neg, square in any type; exp, log, sqrt, sigmoid, silu in the floating-point types only
+ * (ODL_ERR_INVALID_ARG otherwise — the reference throws for integer inputs, e.g. src/mat/origin/cpu/math/log.cpp) */
+int odl_hip_unary_dtype(int op, int dtype, const void *a, int64_t n, void *out, void *stream);
+/* pow with a scalar exponent for float32 / float64 (src/mat/origin/cpu/math/pow.cpp:14-44; the operator promotes integer
+ * tensors to float32 before it gets here, src/operators/math/pow.cpp) */
+int odl_hip_pow_scalar_dtype(int dtype, const void *a, int64_t n, double exponent, void *out, void *stream);
+/* origin::cuda::{zeros,ones,full}, from_scalar in any type: host_value points at ONE element of that type on the host */
+int odl_hip_fill_dtype(void *dst, int dtype, int64_t n, const void *host_value, void *stream);
+/* Mat::sum over [outer, axis, inner] in any type (operation_templates.h:270-357): integers sum with wrap-around in their
+ * own width, float64 in a fixed parallel order. through_float != 0 passes each result through a float on its way back
+ * into the element type, which is what the reference's whole-tensor sum does (src/mat/origin/cpu/math/sum.cpp:18-35,83-90). */
+int odl_hip_sum_axis_dtype(int dtype, const void *src, int64_t outer, int64_t axis, int64_t inner, int through_float,
+                           void *dst, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_sum_axis_dtype_workspace_bytes(int dtype, int64_t outer, int64_t axis, int64_t inner);
+
 /* ------------------------------------------------------------------ detector forward path ------------ */
 /* Mat::upsample, mode "nearest" (mat.h:770; src/mat/origin/cpu/nn/upsample.cpp:22-75):
  * y[n,c,oh,ow] = x[n,c,oh/scale_h,ow/scale_w]. Unlike the reference, an output that would index past x is refused. */

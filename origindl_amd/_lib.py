@@ -27,7 +27,7 @@ def _ctype(decl):
         return ctypes.c_char_p if re.match(r"const\s+char\s*\*$", decl) else ctypes.c_void_p
     base = re.sub(r"\bconst\b", "", decl).split()
     kind = base[0] if base else "void"
-    return {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "size_t": ctypes.c_size_t, "float": ctypes.c_float,
+    return {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "size_t": ctypes.c_size_t, "float": ctypes.c_float, "double": ctypes.c_double,
             "void": None}[kind]
 
 

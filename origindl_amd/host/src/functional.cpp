@@ -14,10 +14,30 @@ namespace
 {
 Tensor scalar_like(const Scalar &s, const Tensor &ref)
 {
-    // a Scalar operand becomes a 0-dim tensor on the other operand's device (src/operators/math/add.cpp:110-114);
-    // device tensors are float32 here, so the scalar is materialised as float32
-    const DataType dt = ref.device().type() == DeviceType::kCUDA ? DataType::kFloat32 : s.dtype();
-    return Tensor(s, Shape({}), dtype(dt).device(ref.device()));
+    // a constant inside an operator's own arithmetic: a 0-dim tensor of the other operand's element type and device
+    return Tensor(s, Shape({}), dtype(ref.dtype()).device(ref.device()));
+}
+
+// include/origin/mat/type_promotion.h:76-102: float64 > float32 > int64 > int32 > int8 > uint8
+DataType promote_types(DataType a, DataType b)
+{
+    if (a == b)
+        return a;
+    for (DataType t : {DataType::kFloat64, DataType::kFloat32, DataType::kInt64, DataType::kInt32, DataType::kInt8,
+                       DataType::kUInt8})
+        if (a == t || b == t)
+            return t;
+    return a;
+}
+
+// both operands in the promoted type; an operand that already has it is passed through untouched
+// (src/mat/type_promotion.cpp promote_tensors)
+std::pair<Tensor, Tensor> promoted(const Tensor &a, const Tensor &b)
+{
+    if (a.dtype() == b.dtype())
+        return {a, b};
+    const DataType t = promote_types(a.dtype(), b.dtype());
+    return {a.dtype() == t ? a : a.to(t), b.dtype() == t ? b : b.to(t)};
 }
 
 // gradient of a broadcasting binary op: reduce back to the operand's shape (left-aligned sum_to, as the reference)
@@ -43,7 +63,8 @@ struct Add : BinaryBase  // src/operators/math/add.cpp:12-55
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
         remember(xs, "Add");
-        return {wrap(mat(xs[0]) + mat(xs[1]))};
+        auto [x0, x1] = promoted(xs[0], xs[1]);
+        return {wrap(mat(x0) + mat(x1))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
@@ -56,7 +77,8 @@ struct Sub : BinaryBase  // src/operators/math/sub.cpp
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
         remember(xs, "Sub");
-        return {wrap(mat(xs[0]) - mat(xs[1]))};
+        auto [x0, x1] = promoted(xs[0], xs[1]);
+        return {wrap(mat(x0) - mat(x1))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
@@ -69,12 +91,14 @@ struct Mul : BinaryBase  // src/operators/math/mul.cpp:12-53
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
         remember(xs, "Mul");
-        return {wrap(mat(xs[0]) * mat(xs[1]))};
+        auto [x0, x1] = promoted(xs[0], xs[1]);
+        return {wrap(mat(x0) * mat(x1))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
         const Mat &gy = mat(gys[0]);
-        return {fit(wrap(gy * mat(inputs_[1])), s0), fit(wrap(gy * mat(inputs_[0])), s1)};
+        auto [x0, x1] = promoted(inputs_[0], inputs_[1]);  // the gradient has the promoted type (mul.cpp:36-44)
+        return {fit(wrap(gy * mat(x1)), s0), fit(wrap(gy * mat(x0)), s1)};
     }
 };
 
@@ -83,11 +107,13 @@ struct Div : BinaryBase  // src/operators/math/div.cpp:28-60
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
         remember(xs, "Div");
-        return {wrap(mat(xs[0]) / mat(xs[1]))};
+        auto [x0, x1] = promoted(xs[0], xs[1]);
+        return {wrap(mat(x0) / mat(x1))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
-        const Mat &gy = mat(gys[0]), &x0 = mat(inputs_[0]), &x1 = mat(inputs_[1]);
+        auto [p0, p1] = promoted(inputs_[0], inputs_[1]);
+        const Mat &gy = mat(gys[0]), &x0 = mat(p0), &x1 = mat(p1);
         auto gx0 = gy / x1;
         auto sq  = x1 * x1;
         auto gx1 = gy * x0;
@@ -105,14 +131,18 @@ struct Neg : Operator
 
 struct Pow : Operator  // src/operators/math/pow.cpp
 {
+    // the exponent arrives already in the result's type: float32 or float64 (pow.cpp:88-110; integers become float32)
     Scalar e;
     explicit Pow(const Scalar &s) : e(s) {}
-    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(xs[0]).pow(e))}; }
+    Tensor base(const Tensor &x) const { return x.dtype() == e.dtype() ? x : x.to(e.dtype()); }
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override { return {wrap(mat(base(xs[0])).pow(e))}; }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
-        auto tmp = mat(inputs_[0]).pow(Scalar(e.to_float32() - 1.0f));
+        const Tensor x = base(inputs_[0]);
+        const Scalar minus_one = e.dtype() == DataType::kFloat64 ? Scalar(e.to_float64() - 1.0) : Scalar(e.to_float32() - 1.0f);
+        auto tmp = mat(x).pow(minus_one);
         tmp->mul_inplace(mat(gys[0]));
-        tmp->mul_inplace(mat(scalar_like(Scalar(e.to_float32()), inputs_[0])));
+        tmp->mul_inplace(mat(scalar_like(e, x)));
         return {wrap(std::move(tmp))};
     }
 };
@@ -198,7 +228,8 @@ struct MatMul : Operator  // src/operators/math/mat_mul.cpp:12-182
     {
         if (xs.size() != 2)
             THROW_RUNTIME_ERROR("MatMul operator requires exactly 2 inputs, but got {}", xs.size());
-        return {wrap(mat(xs[0]).matmul(mat(xs[1])))};
+        auto [x0, x1] = promoted(xs[0], xs[1]);  // mat_mul.cpp promotes too; the product itself is a float32 kernel
+        return {wrap(mat(x0).matmul(mat(x1)))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
@@ -667,7 +698,15 @@ Tensor sub(const Tensor &a, const Tensor &b) { return apply<Sub>({a, b}); }
 Tensor mul(const Tensor &a, const Tensor &b) { return apply<Mul>({a, b}); }
 Tensor div(const Tensor &a, const Tensor &b) { return apply<Div>({a, b}); }
 Tensor neg(const Tensor &x) { return apply<Neg>({x}); }
-Tensor pow(const Tensor &x, const Scalar &e) { return apply<Pow>({x}, e); }
+Tensor pow(const Tensor &x, const Scalar &e)
+{
+    // src/operators/math/pow.cpp:88-110: base and exponent promote as two operands would, and a result that would be an
+    // integer type becomes float32; the exponent is stored in that type
+    DataType t = promote_types(x.dtype(), e.dtype());
+    if (t != DataType::kFloat32 && t != DataType::kFloat64)
+        t = DataType::kFloat32;
+    return apply<Pow>({x}, t == DataType::kFloat64 ? Scalar(e.to_float64()) : Scalar(e.to_float32()));
+}
 Tensor exp(const Tensor &x) { return apply<Exp>({x}); }
 Tensor log(const Tensor &x) { return apply<Log>({x}); }
 Tensor square(const Tensor &x) { return apply<Square>({x}); }
@@ -759,10 +798,16 @@ Tensor max_pool2d(const Tensor &x, int k, int s, int p)
 namespace F = functional;
 namespace
 {
+// a Scalar operand of an arithmetic operator: a 0-dim tensor of the scalar's own element type on the other operand's
+// device; the operator then promotes the two (src/operators/math/add.cpp:110-114)
 Tensor scalar_of(const Scalar &s, const Tensor &ref)
 {
-    const DataType dt = ref.device().type() == DeviceType::kCUDA ? DataType::kFloat32 : s.dtype();
-    return Tensor(s, Shape({}), dtype(dt).device(ref.device()));
+    return Tensor(s, Shape({}), dtype(s.dtype()).device(ref.device()));
+}
+// in a comparison or a compound assignment the tensor's type stands: the scalar is brought to it
+Tensor scalar_as(const Scalar &s, const Tensor &ref)
+{
+    return Tensor(s, Shape({}), dtype(ref.dtype()).device(ref.device()));
 }
 }  // namespace
 
@@ -781,10 +826,10 @@ Tensor operator/(const Scalar &a, const Tensor &b) { return F::div(scalar_of(a, 
 Tensor operator-(const Tensor &x) { return F::neg(x); }
 Tensor operator^(const Tensor &x, const Scalar &e) { return F::pow(x, e); }
 Tensor operator>(const Tensor &a, const Tensor &b) { return Tensor(*a.impl_->data_ > *b.impl_->data_); }
-Tensor operator>(const Tensor &a, const Scalar &b) { return a > scalar_of(b, a); }
+Tensor operator>(const Tensor &a, const Scalar &b) { return a > scalar_as(b, a); }
 #define ODL_COMPARE(OP)                                                                                     \
     Tensor operator OP(const Tensor &a, const Tensor &b) { return Tensor(*a.impl_->data_ OP * b.impl_->data_); } \
-    Tensor operator OP(const Tensor &a, const Scalar &b) { return a OP scalar_of(b, a); }
+    Tensor operator OP(const Tensor &a, const Scalar &b) { return a OP scalar_as(b, a); }
 ODL_COMPARE(==)
 ODL_COMPARE(!=)
 ODL_COMPARE(<)
@@ -796,10 +841,10 @@ Tensor &operator+=(Tensor &a, const Tensor &b) { F::add_(a, b); return a; }
 Tensor &operator-=(Tensor &a, const Tensor &b) { F::sub_(a, b); return a; }
 Tensor &operator*=(Tensor &a, const Tensor &b) { F::mul_(a, b); return a; }
 Tensor &operator/=(Tensor &a, const Tensor &b) { F::div_(a, b); return a; }
-Tensor &operator+=(Tensor &a, const Scalar &b) { F::add_(a, scalar_of(b, a)); return a; }
-Tensor &operator-=(Tensor &a, const Scalar &b) { F::sub_(a, scalar_of(b, a)); return a; }
-Tensor &operator*=(Tensor &a, const Scalar &b) { F::mul_(a, scalar_of(b, a)); return a; }
-Tensor &operator/=(Tensor &a, const Scalar &b) { F::div_(a, scalar_of(b, a)); return a; }
+Tensor &operator+=(Tensor &a, const Scalar &b) { F::add_(a, scalar_as(b, a)); return a; }
+Tensor &operator-=(Tensor &a, const Scalar &b) { F::sub_(a, scalar_as(b, a)); return a; }
+Tensor &operator*=(Tensor &a, const Scalar &b) { F::mul_(a, scalar_as(b, a)); return a; }
+Tensor &operator/=(Tensor &a, const Scalar &b) { F::div_(a, scalar_as(b, a)); return a; }
 
 Tensor Tensor::reshape(const Shape &shape) const { return F::reshape(*this, shape); }
 Tensor Tensor::transpose() const { return F::transpose(*this); }

@@ -215,6 +215,22 @@ const float *fp(const OriginMat &m)
     return m.data_ptr<float>();
 }
 
+// a Mat of any element type living on the device: the elementwise, conversion and sum kernels take all six types
+const OriginMat &dev_any(const Mat &m, const char *who)
+{
+    const OriginMat &o = as_origin(m);
+    if (o.device().type() != DeviceType::kCUDA)
+        THROW_RUNTIME_ERROR("{}: tensor is on {}; this backend computes on the GPU only (move it with .to(device))", who,
+                            o.device().to_string());
+    return o;
+}
+
+// the C ABI's element type codes are the DataType enumerators
+int code(DataType dt)
+{
+    return static_cast<int>(dt);
+}
+
 std::unique_ptr<OriginMat> new_like(const OriginMat &ref, const Shape &shape, DataType dt = DataType::kFloat32)
 {
     return std::make_unique<OriginMat>(shape, dt, ref.device());
@@ -263,36 +279,45 @@ Shape broadcast_shape(const OriginMat &a, const OriginMat &b, const char *who)
 
 std::unique_ptr<Mat> binary(int op, const char *who, const OriginMat &a, const Mat &other, OriginMat *out = nullptr)
 {
-    const OriginMat &x = dev_f32(a, who);
-    const OriginMat &y = dev_f32(other, who);
+    // arithmetic and comparisons run in any element type; the fused activation gradients (op > 9) are float32 kernels
+    const OriginMat &x = op <= 9 ? dev_any(a, who) : dev_f32(a, who);
+    const OriginMat &y = op <= 9 ? dev_any(other, who) : dev_f32(other, who);
     same_dtype_device(x, y, who);
     const Shape rs = broadcast_shape(x, y, who);
     std::unique_ptr<OriginMat> fresh;
     OriginMat *dst = out;
     if (!dst)
     {
-        fresh = new_like(x, rs);
+        fresh = new_like(x, rs, x.dtype());
         dst   = fresh.get();
     }
     else if (dst->shape() != rs)
         THROW_INVALID_ARG("Output tensor mismatch. Expected shape={}, got shape={}", rs.to_string(),
                           dst->shape().to_string());
-    check(odl_hip_binary(op, fp(x), (int64_t)x.elements(), fp(y), (int64_t)y.elements(), dst->data_ptr<float>(),
-                         cur()));
+    else if (dst->dtype() != x.dtype())
+        THROW_INVALID_ARG("Output tensor mismatch. Expected dtype={}, got dtype={}", dtype_to_string(x.dtype()),
+                          dtype_to_string(dst->dtype()));
+    check(odl_hip_binary_dtype(op, code(x.dtype()), x.storage()->data(), (int64_t)x.elements(), y.storage()->data(),
+                               (int64_t)y.elements(), dst->storage()->data(), cur()));
     return fresh;
 }
 
 std::unique_ptr<Mat> unary(int op, const char *who, const OriginMat &a, OriginMat *out = nullptr)
 {
-    const OriginMat &x = dev_f32(a, who);
+    const OriginMat &x = dev_any(a, who);
+    // exp, log, sqrt, sigmoid and silu exist for the floating-point types only, as in the reference
+    const bool floating = x.dtype() == DataType::kFloat32 || x.dtype() == DataType::kFloat64;
+    if (!floating && !(op == 0 || op == 3 || op == 4))
+        THROW_INVALID_ARG("{}: only floating-point tensors are supported, got {}", who, dtype_to_string(x.dtype()));
     std::unique_ptr<OriginMat> fresh;
     OriginMat *dst = out;
     if (!dst)
     {
-        fresh = new_like(x, x.shape());
+        fresh = new_like(x, x.shape(), x.dtype());
         dst   = fresh.get();
     }
-    check(odl_hip_unary(op, fp(x), (int64_t)x.elements(), dst->data_ptr<float>(), cur()));
+    check(odl_hip_unary_dtype(op, code(x.dtype()), x.storage()->data(), (int64_t)x.elements(), dst->storage()->data(),
+                              cur()));
     return fresh;
 }
 
@@ -443,10 +468,20 @@ std::unique_ptr<Mat> OriginMat::from_memory(const void *data, DataType user_dtyp
 std::unique_ptr<Mat> OriginMat::from_scalar(const Scalar &scalar, const Shape &shape, const TensorOptions &options)
 {
     const size_t n = shape.elements();
-    if (options.device().type() == DeviceType::kCUDA && options.dtype() == DataType::kFloat32)
+    if (options.device().type() == DeviceType::kCUDA)
     {
-        auto m = std::make_unique<OriginMat>(shape, DataType::kFloat32, options.device());
-        check(odl_hip_fill(m->data_ptr<float>(), (int64_t)n, scalar.to_float32(), cur()));
+        // one element converted on the host the way the host path below converts all of them, then a fill kernel
+        auto m = std::make_unique<OriginMat>(shape, options.dtype(), options.device());
+        const double v = scalar.to_float64();
+        char element[8];
+        if (options.dtype() == DataType::kInt64)
+        {
+            const int64_t w = scalar.to_int64();
+            std::memcpy(element, &w, sizeof(w));
+        }
+        else
+            store_as(element, options.dtype(), &v, 1);
+        check(odl_hip_fill_dtype(m->storage()->data(), code(options.dtype()), (int64_t)n, element, cur()));
         return m;
     }
     std::vector<double> tmp(n, scalar.to_float64());
@@ -628,7 +663,14 @@ std::unique_ptr<Mat> OriginMat::to(DataType target) const
 {
     if (target == dtype_)
         return std::make_unique<OriginMat>(*this);
-    // dtype conversion is host-side plumbing (labels, metrics); it is not a device kernel of this backend
+    if (device().type() == DeviceType::kCUDA)
+    {
+        // a cast kernel on the current stream: no host round trip, so it can sit inside a recorded step
+        auto out = std::make_unique<OriginMat>(shape_, target, device());
+        check(odl_hip_convert(storage_->data(), code(dtype_), out->storage()->data(), code(target), (int64_t)elements(),
+                              cur()));
+        return out;
+    }
     const std::vector<double> d = to_doubles();
     std::vector<char> conv(d.size() * dtype_size(target));
     store_as(conv.data(), target, d.data(), d.size());
@@ -1012,9 +1054,14 @@ std::unique_ptr<Mat> OriginMat::yolo_detect_forward(const Mat &conv_weight, cons
 
 std::unique_ptr<Mat> OriginMat::pow(const Scalar &exponent) const
 {
-    const OriginMat &x = dev_f32(*this, "pow");
-    auto out = new_like(x, shape_);
-    check(odl_hip_pow_scalar(fp(x), (int64_t)elements(), exponent.to_float32(), out->data_ptr<float>(), cur()));
+    const OriginMat &x = dev_any(*this, "pow");
+    if (x.dtype() != DataType::kFloat32 && x.dtype() != DataType::kFloat64)
+        THROW_INVALID_ARG("pow: only floating-point tensors are supported on the device, got {}", dtype_to_string(x.dtype()));
+    auto out = new_like(x, shape_, x.dtype());
+    // float32: powf with the exponent rounded to float, as the reference's float kernel sees it
+    const double e = x.dtype() == DataType::kFloat32 ? (double)exponent.to_float32() : exponent.to_float64();
+    check(odl_hip_pow_scalar_dtype(code(x.dtype()), x.storage()->data(), (int64_t)elements(), e, out->storage()->data(),
+                                   cur()));
     return out;
 }
 
@@ -1085,13 +1132,16 @@ std::unique_ptr<Mat> OriginMat::sum_to(const Shape &shape) const
 
 std::unique_ptr<Mat> OriginMat::sum(int axis, bool keepdim) const
 {
-    const OriginMat &x = dev_f32(*this, "sum");
+    const OriginMat &x = dev_any(*this, "sum");
+    const int dt = code(x.dtype());
     if (axis == -1)
     {
         const Shape rs = keepdim ? Shape(std::vector<size_t>(shape_.size(), 1)) : Shape{1};
-        auto out = new_like(x, rs);
-        Workspace ws(odl_hip_sum_all_workspace_bytes((int64_t)elements()), device().index());
-        check(odl_hip_sum_all(fp(x), (int64_t)elements(), out->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
+        auto out = new_like(x, rs, x.dtype());
+        // the reference's whole-tensor sum goes back into the element type through a float (sum.cpp:18-35)
+        Workspace ws(odl_hip_sum_axis_dtype_workspace_bytes(dt, 1, (int64_t)elements(), 1), device().index());
+        check(odl_hip_sum_axis_dtype(dt, x.storage()->data(), 1, (int64_t)elements(), 1, 1, out->storage()->data(), ws.ptr(),
+                                     ws.bytes, cur()));
         return out;
     }
     if (axis < 0 || axis >= (int)shape_.size())
@@ -1106,9 +1156,10 @@ std::unique_ptr<Mat> OriginMat::sum(int axis, bool keepdim) const
     }
     int64_t outer, ax, inner;
     split_axis(shape_, axis, outer, ax, inner);
-    auto out = new_like(x, Shape(rd));
-    Workspace ws(odl_hip_sum_axis_workspace_bytes(outer, ax, inner), device().index());
-    check(odl_hip_sum_axis(fp(x), outer, ax, inner, out->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
+    auto out = new_like(x, Shape(rd), x.dtype());
+    Workspace ws(odl_hip_sum_axis_dtype_workspace_bytes(dt, outer, ax, inner), device().index());
+    check(odl_hip_sum_axis_dtype(dt, x.storage()->data(), outer, ax, inner, 0, out->storage()->data(), ws.ptr(), ws.bytes,
+                                 cur()));
     return out;
 }
 

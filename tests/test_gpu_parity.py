@@ -968,3 +968,113 @@ def test_conv_with_fused_activation_is_conv_then_activation(api, N, C, H, OC, k,
     for act in (None, "silu"):
         assert np.array_equal(host(api.conv2d(x, w, b, s, p, activation=act, packed=packed)),
                               host(api.conv2d(x, w, b, s, p, activation=act))), act
+
+
+# ------------------------------------------------------------------ element types besides float32
+DT = {"f32": (0, np.float32), "f64": (1, np.float64), "i8": (2, np.int8), "i32": (3, np.int32), "i64": (4, np.int64),
+      "u8": (5, np.uint8)}
+
+
+def _typed_values(rng, np_t, n, positive=False):
+    if np_t in (np.float32, np.float64):
+        v = rng.standard_normal(n) * 40
+        return (np.abs(v) if positive else v).astype(np_t)
+    hi = {np.int8: 100, np.uint8: 200}.get(np_t, 100000)
+    lo = 0 if (positive or np_t is np.uint8) else -hi
+    return rng.integers(lo, hi, size=n).astype(np_t)
+
+
+def test_convert_between_all_element_types_is_a_static_cast(api):
+    # src/mat/origin/cuda/type_conversion.cu: dst[i] = static_cast<Dst>(src[i]); numpy's astype is the same conversion
+    # wherever C++ defines it (values inside the destination's range; float -> integer truncates towards zero)
+    L = api.lib()
+    rng = np.random.default_rng(51)
+    n = 100_003
+    for sname, (scode, s_t) in DT.items():
+        for dname, (dcode, d_t) in DT.items():
+            small = d_t in (np.int8, np.uint8) or s_t in (np.int8, np.uint8)
+            src = _typed_values(rng, s_t, n, positive=(d_t is np.uint8))
+            if small:
+                src = (src % 100).astype(s_t) if s_t not in (np.float32, np.float64) else np.clip(src, 0 if d_t is np.uint8 else -100, 100).astype(s_t)
+            d_src = dev(src)
+            d_dst = torch.empty(n, dtype=getattr(torch, np.dtype(d_t).name), device="cuda")
+            L.call("odl_hip_convert", d_src.data_ptr(), scode, d_dst.data_ptr(), dcode, n, None)
+            assert np.array_equal(host(d_dst), src.astype(d_t)), (sname, dname)
+    assert [L.query("odl_hip_dtype_size", c) for c in range(7)] == [4, 8, 1, 4, 8, 1, 0]
+    with pytest.raises(api.OdlInvalidArgument):
+        L.call("odl_hip_convert", d_src.data_ptr(), 9, d_dst.data_ptr(), 0, 4, None)
+
+
+@pytest.mark.parametrize("name", ["f64", "i8", "i32", "i64", "u8"])
+def test_elementwise_fill_and_sum_in_every_element_type(api, name):
+    L = api.lib()
+    code, t = DT[name]
+    tt = getattr(torch, np.dtype(t).name)
+    rng = np.random.default_rng(52 + code)
+    n = 70_001
+    a, b = _typed_values(rng, t, n), _typed_values(rng, t, n)
+    b[b == 0] = 3
+    is_float = t is np.float64
+
+    def run_binary(op, x, y):
+        out = torch.empty(max(x.size, y.size), dtype=tt, device="cuda")
+        dx, dy = dev(x), dev(y)  # both kept alive until the call has been made
+        L.call("odl_hip_binary_dtype", op, code, dx.data_ptr(), x.size, dy.data_ptr(), y.size, out.data_ptr(), None)
+        return host(out)
+
+    with np.errstate(over="ignore"):
+        wide = np.float64 if is_float else np.int64
+        quotient = a / b if is_float else np.trunc(a.astype(np.float64) / b.astype(np.float64)).astype(np.int64).astype(t)
+        want = [a + b, a - b, a * b, quotient] + [f(a, b).astype(t) for f in (np.greater, np.equal, np.not_equal, np.less,
+                                                                              np.less_equal, np.greater_equal)]
+        for op, w in enumerate(want):
+            assert np.array_equal(run_binary(op, a, b), w.astype(t)), (name, op)  # integer arithmetic wraps in numpy too
+        one = np.array([3], t)
+        assert np.array_equal(run_binary(0, a, one), (a + one).astype(t))
+        assert np.array_equal(run_binary(1, one, a), (one - a).astype(t))
+        # unary: relu, negate, square everywhere
+        da = dev(a)
+        for op, w in ((0, np.maximum(a, 0)), (3, (0 - a.astype(wide)).astype(t) if not is_float else -a),
+                      (4, (a.astype(wide) * a.astype(wide)).astype(t) if not is_float else a * a)):
+            out = torch.empty(n, dtype=tt, device="cuda")
+            L.call("odl_hip_unary_dtype", op, code, da.data_ptr(), n, out.data_ptr(), None)
+            assert np.array_equal(host(out), w.astype(t)), (name, "unary", op)
+    out = torch.empty(n, dtype=tt, device="cuda")
+    if is_float:
+        pos = np.abs(a) + 0.5
+        for op, f in ((1, lambda v: np.exp(v / 40)), (2, np.log), (5, np.sqrt)):
+            src = a / 40 if op == 1 else pos
+            dsrc = dev(src)
+            L.call("odl_hip_unary_dtype", op, code, dsrc.data_ptr(), n, out.data_ptr(), None)
+            np.testing.assert_allclose(host(out), np.exp(src) if op == 1 else f(src), rtol=1e-14)
+        dpos = dev(pos)
+        L.call("odl_hip_pow_scalar_dtype", code, dpos.data_ptr(), n, 2.5, out.data_ptr(), None)
+        np.testing.assert_allclose(host(out), pos ** 2.5, rtol=1e-14)
+    else:
+        for op in (1, 2, 5, 6, 7):  # the reference throws for integer inputs (tests/unit_test/operator/test_log.cpp:210-225)
+            with pytest.raises(api.OdlInvalidArgument):
+                L.call("odl_hip_unary_dtype", op, code, da.data_ptr(), n, out.data_ptr(), None)
+        with pytest.raises(api.OdlInvalidArgument):
+            L.call("odl_hip_pow_scalar_dtype", code, da.data_ptr(), n, 2.0, out.data_ptr(), None)
+    # fill
+    v = np.array([7], t)
+    L.call("odl_hip_fill_dtype", out.data_ptr(), code, n, v.ctypes.data, None)
+    assert (host(out) == v[0]).all()
+    # sums: [outer, axis, inner] in both layouts and the whole tensor (which passes through a float, as the reference's)
+    for outer, axis, inner in ((1, n, 1), (3, 1000, 1), (4, 300, 50), (1, 5000, 3), (2, 7, 1), (1, 4096 * 64, 1)):
+        x = _typed_values(rng, t, outer * axis * inner).reshape(outer, axis, inner)
+        nb = L.query("odl_hip_sum_axis_dtype_workspace_bytes", code, outer, axis, inner)
+        ws = torch.empty(max(nb, 8), dtype=torch.uint8, device="cuda")
+        res = torch.empty(outer * inner, dtype=tt, device="cuda")
+        dx = dev(x)
+        for through_float in (0, 1):
+            L.call("odl_hip_sum_axis_dtype", code, dx.data_ptr(), outer, axis, inner, through_float, res.data_ptr(),
+                   ws.data_ptr(), nb, None)
+            if is_float:
+                w = x.sum(axis=1).reshape(-1)
+                w = w.astype(np.float32).astype(t) if through_float else w
+                np.testing.assert_allclose(host(res), w, rtol=1e-6 if through_float else 1e-12, atol=1e-9)
+            else:
+                w = x.astype(np.int64).sum(axis=1).reshape(-1).astype(t)  # the wrapped sum in the type's own width
+                w = w.astype(np.float32).astype(t) if through_float else w
+                assert np.array_equal(host(res), w), (name, outer, axis, inner, through_float)
