@@ -150,6 +150,52 @@ __global__ void ce_finish_kernel(const float *__restrict__ logp, int64_t N, floa
     }
 }
 
+// The whole loss of a small batch of short rows in ONE launch (the three-launch schedule above is bound by launch latency
+// there): one workgroup, a thread per row — max, sum of exponentials and the label's probability in the order the
+// reference's loops take them (src/operators/loss/softmax_cross_entropy.cpp:30-70) — then the block sum of ce_finish_kernel.
+// Writes both words: out2[0] = loss, out2[1] = 1 when a label is out of range.
+__global__ __launch_bounds__(1024) void ce_loss_small_kernel(const float *__restrict__ x, const void *t, int is64, int N,
+                                                             int C, unsigned int *out2)
+{
+    __shared__ float part[1024 / 64];
+    __shared__ int bad;
+    if (threadIdx.x == 0)
+        bad = 0;
+    __syncthreads();
+    float acc = 0.f;
+    for (int row = threadIdx.x; row < N; row += 1024)
+    {
+        const float *xr = x + (int64_t)row * C;
+        float m = -FLT_MAX;
+        for (int j = 0; j < C; ++j)
+            m = (m < xr[j]) ? xr[j] : m;
+        float s = 0.f;
+        for (int j = 0; j < C; ++j)
+            s += expf(xr[j] - m);
+        const int64_t lab = label_at(t, is64, row);
+        if (lab < 0 || lab >= C)
+            bad = 1;  // every writer stores the same value
+        else
+        {
+            const float p = expf(xr[lab] - m) / s;
+            acc += logf(p + 1e-8f);
+        }
+    }
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        float s = 0.f;
+        for (int i = 0; i < 1024 / 64; ++i)
+            s += part[i];
+        const float loss = -s / (float)N;
+        out2[0] = __float_as_uint(loss);
+        out2[1] = bad ? 1u : 0u;
+    }
+}
+
 // gx = (softmax(x) - one_hot(t)) * scale, one wave per row. Rows of up to 64*REGS classes stay in registers
 // between the max, the sum and the write, so the logits are read from memory once; longer rows re-read them.
 template <int REGS>
@@ -390,6 +436,12 @@ static int ce_loss_launch(const float *x, const void *t, int idx_is_i64, int64_t
     const size_t need = odl_hip_softmax_ce_loss_workspace_bytes(N);
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
                 "softmax_cross_entropy: workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    if (N <= 2048 && C <= 64)
+    {
+        hipLaunchKernelGGL(ce_loss_small_kernel, dim3(1), dim3(1024), 0, st, x, t, idx_is_i64, (int)N, (int)C, out2);
+        ODL_LAUNCH_CHECK();
+        return ODL_OK;
+    }
     float *logp = static_cast<float *>(workspace);
     hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, out2, 2);
     ODL_LAUNCH_CHECK();

@@ -153,6 +153,71 @@ __global__ __launch_bounds__(kBlock) void col_sum_kernel(const float *__restrict
         d[e] = acc[e];
 }
 
+// ---- columns of a small tensor in ONE launch (a bias gradient of a few MB is bound by launch latency, not by HBM: the
+// two-pass schedule above costs two launches and the gap between them). A workgroup owns CW*VEC adjacent columns of one
+// `outer` slice; its 256 threads are CW column lanes x (256/CW) row groups, group g adds rows g, g+G, ... (eight loads
+// in flight), the group sums meet in LDS and are added in group order.
+template <int VEC, int CW>
+__global__ __launch_bounds__(kBlock) void col_sum_small_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                                int64_t axis, int64_t inner)
+{
+    constexpr int G = kBlock / CW;
+    __shared__ float sh[G][CW * VEC + 1];
+    const int lane = threadIdx.x % CW, grp = threadIdx.x / CW;
+    const int64_t o = blockIdx.y;
+    const int64_t col = ((int64_t)blockIdx.x * CW + lane) * VEC;
+    const bool live = col < inner;
+    const float *p = src + (o * axis) * inner + col;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+        acc[e] = 0.f;
+    if (live)
+    {
+        int64_t a = grp;
+        for (; a + 7 * G < axis; a += 8 * G)
+        {
+            float v[8][VEC];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+            {
+                if (VEC == 4)
+                {
+                    const f32x4 q = *reinterpret_cast<const f32x4 *>(p + (a + u * G) * inner);
+                    v[u][0] = q[0], v[u][1 % VEC] = q[1], v[u][2 % VEC] = q[2], v[u][3 % VEC] = q[3];
+                }
+                else
+                    v[u][0] = p[(a + u * G) * inner];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    acc[e] += v[u][e];
+        }
+        for (; a < axis; a += G)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                acc[e] += p[a * inner + e];
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+        sh[grp][lane * VEC + e] = acc[e];
+    __syncthreads();
+    if (threadIdx.x < CW * VEC)
+    {
+        const int64_t c = (int64_t)blockIdx.x * CW * VEC + threadIdx.x;
+        if (c < inner)
+        {
+            float t = sh[0][threadIdx.x];
+#pragma unroll 4
+            for (int g = 1; g < G; ++g)
+                t += sh[g][threadIdx.x];
+            dst[o * inner + c] = t;
+        }
+    }
+}
+
 // dst[i] = sum over s of part[s*n + i]. 64 columns x 16 slice groups per workgroup: group g adds slices
 // g, g+16, ... (coalesced along i), the group sums meet in LDS and are added in group order — a fixed order.
 constexpr int kFoldGroups = 16;
@@ -338,6 +403,12 @@ struct SumPlan
     size_t ws_bytes;
 };
 
+// column sums small enough to be bound by launch latency: one launch (col_sum_small_kernel)
+bool small_cols(int64_t outer, int64_t axis, int64_t inner)
+{
+    return inner > 1 && axis >= 16 && outer <= 1024 && outer * axis * inner <= (1 << 20);
+}
+
 SumPlan plan_sum(int64_t outer, int64_t axis, int64_t inner)
 {
     SumPlan p{};
@@ -359,6 +430,12 @@ SumPlan plan_sum(int64_t outer, int64_t axis, int64_t inner)
         p.chunk = odl::ceil_div(odl::ceil_div(axis, s), 4) * 4;
         p.splits = (int)odl::ceil_div(axis, p.chunk);
         p.ws_bytes = p.splits > 1 ? (size_t)(outer * p.splits) * sizeof(float) : 0;
+        return p;
+    }
+    if (small_cols(outer, axis, inner))
+    {
+        p.splits = 1;
+        p.chunk = axis;
         return p;
     }
     const int64_t vec = (inner % 4 == 0) ? 4 : 1;
@@ -416,6 +493,17 @@ int sum_axis_launch(const float *src, int64_t outer, int64_t axis, int64_t inner
         return ODL_OK;
     }
     const bool v4 = (inner % 4 == 0) && (reinterpret_cast<uintptr_t>(src) % 16 == 0);
+    if (small_cols(outer, axis, inner))
+    {
+        if (v4)
+            hipLaunchKernelGGL((col_sum_small_kernel<4, 8>), dim3((unsigned)odl::ceil_div(inner, 32), (unsigned)outer),
+                               dim3(kBlock), 0, st, src, dst, axis, inner);
+        else
+            hipLaunchKernelGGL((col_sum_small_kernel<1, 16>), dim3((unsigned)odl::ceil_div(inner, 16), (unsigned)outer),
+                               dim3(kBlock), 0, st, src, dst, axis, inner);
+        ODL_LAUNCH_CHECK();
+        return ODL_OK;
+    }
     const int64_t cols = outer * (v4 ? inner / 4 : inner);
     float *part = p.splits > 1 ? static_cast<float *>(workspace) : dst;
     const dim3 grid((unsigned)odl::ceil_div(cols, kBlock), (unsigned)p.splits);

@@ -12,6 +12,8 @@
 #include <utility>
 #include <vector>
 
+#include <cstring>
+
 #include "base.h"
 
 namespace origin
@@ -27,8 +29,32 @@ public:
     ~Storage();
     Storage(const Storage &)            = delete;
     Storage &operator=(const Storage &) = delete;
-    void *data() const { return data_; }
+    // Handing out the address ends the validity of the host copy below: whoever holds the pointer may write through it.
+    void *data() const
+    {
+        host_copy_valid_ = false;
+        return data_;
+    }
     size_t size() const { return size_; }
+    // A host copy of the first bytes of a small device buffer, kept by code that has just read them back anyway (the loss
+    // scalar comes to the host once, for the bad-label check, and item() is then served from here instead of a second
+    // synchronising copy). Valid until the next data() call.
+    void set_host_copy(const void *bytes, size_t n) const
+    {
+        if (n <= sizeof(host_copy_))
+        {
+            std::memcpy(host_copy_, bytes, n);
+            host_copy_bytes_ = n;
+            host_copy_valid_ = true;
+        }
+    }
+    bool host_copy(void *dst, size_t n) const
+    {
+        if (!host_copy_valid_ || n > host_copy_bytes_)
+            return false;
+        std::memcpy(dst, host_copy_, n);
+        return true;
+    }
     DeviceType device_type() const { return type_; }
     int device_index() const { return index_; }
     std::shared_ptr<Storage> to_device(DeviceType type, int index) const;  // synchronous copy, like the reference
@@ -39,6 +65,9 @@ private:
     size_t size_, capacity_;
     DeviceType type_;
     int index_;
+    mutable bool host_copy_valid_ = false;
+    mutable size_t host_copy_bytes_ = 0;
+    mutable unsigned char host_copy_[8] = {0};
 };
 
 class Mat

@@ -564,9 +564,17 @@ std::vector<double> OriginMat::to_doubles() const
     std::vector<double> out(n);
     if (n == 0)
         return out;
-    const void *src = storage_->data();
     std::vector<char> host;
-    if (storage_->device_type() != DeviceType::kCPU)
+    const void *src = nullptr;
+    if (storage_->device_type() != DeviceType::kCPU && n == 1)
+    {
+        host.resize(dtype_size(dtype_));
+        if (storage_->host_copy(host.data(), host.size()))  // a scalar that has been read back already
+            src = host.data();
+    }
+    if (!src)
+        src = storage_->data();
+    if (storage_->device_type() != DeviceType::kCPU && src != host.data())
     {
         host.resize(n * dtype_size(dtype_));
         no_capture("device-to-host copy");
@@ -1488,9 +1496,11 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target)
     // divide does); the loss itself stays on the device for the operators that follow
     unsigned words[2] = {0, 0};
     no_capture("device-to-host copy");
-    check(odl_hip_memcpy_d2h(words, as_origin(*loss).storage()->data(), sizeof(words)));
+    const auto &st = as_origin(*loss).storage();
+    check(odl_hip_memcpy_d2h(words, st->data(), sizeof(words)));
     if (words[1] != 0)
         THROW_INVALID_ARG("gather: index out of range [0, {})", shape_[1]);
+    st->set_host_copy(words, sizeof(words));  // item() on the loss needs no second trip
     return loss;
 }
 

@@ -37,9 +37,10 @@ def test_sum_axis_without_allocation_matches_the_workspace_entry_point():
     assert limit == 8 << 20
     g = torch.Generator(device="cuda").manual_seed(11)
     # two calls in a row on column sums whose partials go through the scratch array: the bias gradient of the scaled
-    # benchmark shape (the whole 8 MiB), then the MLP's own [512, 1000] -> [1000] (128 KB of the same array)
-    shapes = [(1, 16384, 4096), (1, 512, 1000),
-              (1, 512, 10), (3, 700, 36), (1, 300000, 1),    # unaligned columns; a middle axis; one long row cut in pieces
+    # benchmark shape (the whole 8 MiB), then a smaller one ([4096, 1000] -> [1000], a part of the same array); after them
+    # shapes that need no partial sums at all (one launch), a middle axis, one long row cut in pieces, an empty axis
+    shapes = [(1, 16384, 4096), (1, 4096, 1000),
+              (1, 512, 1000), (1, 512, 10), (3, 700, 36), (1, 300000, 1), (2, 3000, 512),
               (8, 300, 7), (5000, 3, 1), (2, 0, 5), (1, 40000, 64)]
     used_scratch = 0
     for outer, axis, inner in shapes:
