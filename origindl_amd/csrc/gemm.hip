@@ -99,9 +99,16 @@ __device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int
     tn = in_g / gm;
 }
 
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI, int SB = SB_PLAIN, int CK = 0>
-__global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_CONV_WGRAD ? 4 : 1)) void sgemm_mfma_kernel(GemmArgs g, ConvSrc cv)
+// WS = 2: the workgroup has a second set of four waves on the same tile. Both sets stage the operands together; of the
+// 8-wide K steps of a slab each set multiplies every other one, and the second set's accumulators join the first's
+// through LDS before the epilogue. For products with at most one workgroup per compute unit: a lone set of four waves
+// (one per SIMD) leaves the matrix pipe idle whenever it waits for LDS, memory or the barrier; the second set fills
+// those gaps without changing the tile shape.
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI, int SB = SB_PLAIN, int CK = 0, int WS = 1>
+__global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && VEC && SB != SB_CONV_WGRAD ? 4 : 1)) void sgemm_mfma_kernel(GemmArgs g, ConvSrc cv)
 {
+    constexpr int NT = kThreads * WS;
+    static_assert(WS == 1 || (WS == 2 && SB == SB_PLAIN && VEC && (BK / 8) % 2 == 0), "the second wave set: plain operands only");
     // A tile: !TA -> memory is [M][K] (K-contiguous) -> LDS K-major; TA -> memory [K][M] -> LDS row-major.
     // B tile: !TB -> memory is [K][N] (row-contiguous) -> LDS row-major; TB -> memory [N][K] -> LDS K-major.
     // A gathered B is laid out in LDS the way its gather runs: the forward gather has lanes along the pixels
@@ -117,15 +124,17 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
     constexpr int B_SIZE    = B_KMAJOR ? BN * LDB_S : BK * LDB_S;
     constexpr int WM = BM / 2, WN = BN / 2;  // wave tile
     constexpr int RB = WM / 32, CB = WN / 32;
-    constexpr int A_PER_T = BM * BK / kThreads;  // floats staged per thread
-    constexpr int B_PER_T = BN * BK / kThreads;
+    constexpr int A_PER_T = BM * BK / NT;  // floats staged per thread
+    constexpr int B_PER_T = BN * BK / NT;
     static_assert(BK % 8 == 0 && A_PER_T % 4 == 0 && B_PER_T % 4 == 0, "tile shape");
 
     __shared__ __attribute__((aligned(16))) float As[2][A_SIZE];
     __shared__ __attribute__((aligned(16))) float Bs[2][B_SIZE];
+    // (the second wave set's accumulators pass through the A buffers at the end)
+    static_assert(WS == 1 || 2 * A_SIZE >= 4 * 16 * 64, "the A buffers hold one accumulator block of four waves");
 
     const int tid  = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = WS > 1 ? ((tid >> 6) & 3) : (tid >> 6), kset = WS > 1 ? (tid >> 8) : 0;  // kset: which wave set (0 when WS == 1)
     const int l32 = lane & 31, lh = lane >> 5;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
@@ -176,7 +185,7 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
         {
             for (int u = 0; u < per_t / 4; ++u)
             {
-                const int f = tid + u * kThreads;
+                const int f = tid + u * NT;
                 int64_t r, k;
                 if (kmajor)
                 {
@@ -201,7 +210,7 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
         {
             for (int u = 0; u < per_t; ++u)
             {
-                const int e = tid + u * kThreads;
+                const int e = tid + u * NT;
                 int64_t r, k;
                 if (kmajor)
                 {
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
         {
             for (int u = 0; u < per_t / 4; ++u)
             {
-                const int f = tid + u * kThreads;
+                const int f = tid + u * NT;
                 int off;
                 if (kmajor)
                     off = (f / (BK / 4)) * lds_ld + 4 * (f % (BK / 4));
@@ -237,7 +246,7 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
         {
             for (int u = 0; u < per_t; ++u)
             {
-                const int e = tid + u * kThreads;
+                const int e = tid + u * NT;
                 const int off = kmajor ? (e / BK) * lds_ld + e % BK : (e / brows) * lds_ld + e % brows;
                 lds[off] = regs[u];
             }
@@ -470,20 +479,12 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
     }
     __syncthreads();
 
-    for (int kt = 0; kt < nkt; ++kt)
-    {
-        const int cur = kt & 1;
-        if (kt + 1 < nkt)
-        {
-            const int64_t k0 = kbeg + (int64_t)(kt + 1) * BK;
-            load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra, A_PER_T);
-            load_b(k0);
-        }
-        const float *as = As[cur];
-        const float *bs = Bs[cur];
+    // the matrix instructions of one K slab out of LDS
+    auto mma = [&](const float *as, const float *bs) {
 #pragma unroll
-        for (int ks = 0; ks < BK / 8; ++ks)
+        for (int ks0 = 0; ks0 < BK / 8; ks0 += WS)
         {
+            const int ks = ks0 + (WS > 1 ? kset : 0);
             float a[RB][4], b[CB][4];
 #pragma unroll
             for (int i = 0; i < RB; ++i)
@@ -525,14 +526,99 @@ __global__ __launch_bounds__(kThreads, (BM * BN >= 128 * 128 && VEC && SB != SB_
                     for (int j = 0; j < CB; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < nkt)
+    };
+
+    if constexpr (WS > 1)
+    {
+        // One workgroup per compute unit has nobody to cover its memory latency, and a K slab's worth of matrix
+        // instructions (0.85 us) is shorter than a load's round trip: operands are fetched TWO slabs ahead into two
+        // register sets, so that each load has two slab times to land before it is stored to LDS.
+        float ra2[A_PER_T], rb2[B_PER_T];
+        if (nkt > 1)
         {
-            store_tile(As[cur ^ 1], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
-            store_b(Bs[cur ^ 1]);
+            load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, kbeg + BK, BM, ra2, A_PER_T);
+            load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, kbeg + BK, BN, rb2, B_PER_T);
         }
-        __syncthreads();
+        for (int kt = 0; kt < nkt; kt += 2)
+        {
+            if (kt + 2 < nkt)
+            {
+                const int64_t k0 = kbeg + (int64_t)(kt + 2) * BK;
+                load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra, A_PER_T);
+                load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, k0, BN, rb_, B_PER_T);
+            }
+            mma(As[0], Bs[0]);
+            if (kt + 1 < nkt)
+            {
+                store_tile(As[1], LDA_S, A_KMAJOR, BM, ra2, A_PER_T);
+                store_tile(Bs[1], LDB_S, B_KMAJOR, BN, rb2, B_PER_T);
+            }
+            __syncthreads();
+            if (kt + 1 >= nkt)
+                break;
+            if (kt + 3 < nkt)
+            {
+                const int64_t k0 = kbeg + (int64_t)(kt + 3) * BK;
+                load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra2, A_PER_T);
+                load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, k0, BN, rb2, B_PER_T);
+            }
+            mma(As[1], Bs[1]);
+            if (kt + 2 < nkt)
+            {
+                store_tile(As[0], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
+                store_tile(Bs[0], LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
+            }
+            __syncthreads();
+        }
+    }
+    else
+    {
+        for (int kt = 0; kt < nkt; ++kt)
+        {
+            const int cur = kt & 1;
+            if (kt + 1 < nkt)
+            {
+                const int64_t k0 = kbeg + (int64_t)(kt + 1) * BK;
+                load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra, A_PER_T);
+                load_b(k0);
+            }
+            mma(As[cur], Bs[cur]);
+            if (kt + 1 < nkt)
+            {
+                store_tile(As[cur ^ 1], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
+                store_b(Bs[cur ^ 1]);
+            }
+            __syncthreads();
+        }
     }
 
+    if constexpr (WS > 1)
+    {
+        // the second wave set hands its accumulators to the first, one 32x32 block of each wave at a time
+        float *xch = &As[0][0] + (wave * 16) * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int j = 0; j < CB; ++j)
+            {
+                if (kset == 1)
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        xch[r * 64] = acc[i][j][r];
+                }
+                __syncthreads();
+                if (kset == 0)
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[i][j][r] += xch[r * 64];
+                }
+                __syncthreads();
+            }
+        if (kset == 1)
+            return;
+    }
     // ---- epilogue: accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
     if (tail_out)
     {
@@ -785,6 +871,13 @@ void launch_tail_fixup(const GemmArgs &g, int BM, int BN, int epi, hipStream_t s
     hipLaunchKernelGGL(tail_fixup_kernel, dim3((unsigned)odl::ceil_div(threads, 256)), dim3(256), 0, st, g, BM, BN, epi);
 }
 
+// tile counts up to which a launch puts about one workgroup on a compute unit
+int64_t lone_workgroup_limit()
+{
+    const int64_t cus = odl::device_cus();
+    return cus + cus / 4;
+}
+
 __global__ void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows, int64_t cols)
 {
     __shared__ float tile[32][33];
@@ -814,6 +907,25 @@ int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g_in, int splits, vo
     g.splits = splits;
     dim3 grid(apply_tail(g, BM, BN, tail_ws, tail_bytes));
     dim3 block(kThreads);
+    if constexpr (BM == 128 && BN == 128)
+    {
+        // at most about one workgroup per compute unit: a second set of four waves on every tile
+        if (vec && splits == 1 && g.tail_splits == 0 && (int64_t)g.tiles_m * g.tiles_n <= lone_workgroup_limit())
+        {
+#define ODL_GEMM_TWO_SETS(TA, TB)                                                                                   \
+    if (ta == TA && tb == TB)                                                                                       \
+    {                                                                                                               \
+        hipLaunchKernelGGL((sgemm_mfma_kernel<BM, BN, 32, TA, TB, true, EPI, SB_PLAIN, 0, 2>), grid, dim3(2 * kThreads), \
+                           0, st, g, ConvSrc{});                                                                    \
+        return ODL_OK;                                                                                              \
+    }
+            ODL_GEMM_TWO_SETS(false, false)
+            ODL_GEMM_TWO_SETS(false, true)
+            ODL_GEMM_TWO_SETS(true, false)
+            ODL_GEMM_TWO_SETS(true, true)
+#undef ODL_GEMM_TWO_SETS
+        }
+    }
 #define ODL_GEMM_CASE(TA, TB, V)                                                                      \
     if (ta == TA && tb == TB && vec == V)                                                             \
     {                                                                                                 \
@@ -870,10 +982,15 @@ int launch_small_tile_wide_slab(bool ta, bool tb, GemmArgs g, hipStream_t st)
     g.main_blocks = 0, g.tail_first = g.tiles_m * g.tiles_n, g.tail_splits = 0, g.tail_kps = 0, g.tail_ws = nullptr;
     g.xcds = odl::chip().xcds;
     const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(kThreads);
+    const bool two_sets = (int64_t)g.tiles_m * g.tiles_n <= lone_workgroup_limit();
 #define ODL_WIDE_CASE(TA, TB)                                                                                  \
     if (ta == TA && tb == TB)                                                                                  \
     {                                                                                                          \
-        hipLaunchKernelGGL((sgemm_mfma_kernel<64, 64, 32, TA, TB, true, EPI>), grid, block, 0, st, g, ConvSrc{}); \
+        if (two_sets)                                                                                          \
+            hipLaunchKernelGGL((sgemm_mfma_kernel<64, 64, 32, TA, TB, true, EPI, SB_PLAIN, 0, 2>), grid,       \
+                               dim3(2 * kThreads), 0, st, g, ConvSrc{});                                       \
+        else                                                                                                   \
+            hipLaunchKernelGGL((sgemm_mfma_kernel<64, 64, 32, TA, TB, true, EPI>), grid, block, 0, st, g, ConvSrc{}); \
         return ODL_OK;                                                                                         \
     }
     ODL_WIDE_CASE(false, false)

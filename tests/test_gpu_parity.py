@@ -58,7 +58,10 @@ def assert_gemm_close(got, want, a, b, what):
 GEMM_SHAPES = [(128, 128, 128), (256, 384, 128), (64, 100, 10), (33, 47, 29), (512, 784, 1000), (512, 1000, 10),
                (1, 5, 1), (130, 16, 260), (4, 1000, 4), (257, 129, 131),
                # one dimension of at most 16 (the classifier layer's products), ragged against the tile edges
-               (256, 3136, 10), (70, 65, 1), (300, 200, 4), (129, 64, 5), (67, 333, 9), (65, 129, 13), (128, 1000, 16)]
+               (256, 3136, 10), (70, 65, 1), (300, 200, 4), (129, 64, 5), (67, 333, 9), (65, 129, 13), (128, 1000, 16),
+               # about one workgroup per compute unit: the variants with a second wave set and operands fetched two
+               # slabs ahead, ragged against the tile edges and with a last K slab that is not whole
+               (2052, 1000, 2044), (1000, 1056, 1020)]
 
 
 @pytest.mark.parametrize("m,k,n", GEMM_SHAPES)
