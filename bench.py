@@ -40,6 +40,15 @@ def time_region(torch, fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
+def time_region_auto(torch, fn, target_ms=40.0, warmup=3):
+    """ms per call for the short kernels of `extras`: a probe of ten calls sizes the timed run to about `target_ms` of
+    device time (at least 10, at most 4000 calls), so that a kernel of a few microseconds is timed over thousands of
+    back-to-back launches and not over the clock ramp of the first ten."""
+    probe = time_region(torch, fn, 10, warmup)
+    n = int(min(4000, max(10, target_ms / max(probe, 1e-4))))
+    return time_region(torch, fn, n, 2)
+
+
 def cpu_baseline_gemm(size, budget_s=18.0):
     """Reference CPU algorithm on a row slice of each of the three products; rows are independent in its loop
     (src/mat/origin/cpu/math/matmul.cpp:27-41), so time scales linearly with the number of rows."""
@@ -120,22 +129,21 @@ def extras(torch, capi, steps, warmup):
         fwd = direct("odl_hip_conv2d", ptr(x), ptr(w), ptr(b), *geom, ptr(y), wf, nf, stream)
         bwd = direct("odl_hip_conv2d_backward", ptr(gy), ptr(x), ptr(w), *geom, ptr(gx), ptr(gw), ptr(gb), wb, nbb,
                      stream)
-        ms_f = time_region(torch, fwd, steps, warmup)
-        ms_b = time_region(torch, bwd, steps, warmup)
+        ms_f = time_region_auto(torch, fwd)
+        ms_b = time_region_auto(torch, bwd)
         flop = 6.0 * M * K * OC
         tf = flop / (ms_f + ms_b) / 1e9
         out[name] = {"fwd_ms": ms_f, "bwd_ms": ms_b, "tflops": tf, "frac_mfma_peak": tf / PEAK_FP32_MFMA_TFLOPS,
                      "flop": flop}
         col, img = empty(M, K), empty(N, C, H, H)
         ig = (N, C, H, H, 3, 3, s, s, p, p, 1)
-        ms_i = time_region(torch, direct("odl_hip_im2col", ptr(x), *ig, ptr(col), stream), steps, warmup)
-        ms_c = time_region(torch, direct("odl_hip_col2im", ptr(col), *ig, ptr(img), stream), steps, warmup)
+        ms_i = time_region_auto(torch, direct("odl_hip_im2col", ptr(x), *ig, ptr(col), stream))
+        ms_c = time_region_auto(torch, direct("odl_hip_col2im", ptr(col), *ig, ptr(img), stream))
         nbytes = 4.0 * (x.numel() + M * K)
         out[name + "_im2col"] = {"ms": ms_i, "gbs": nbytes / ms_i / 1e6, "frac_hbm": nbytes / ms_i / 1e6 / PEAK_HBM_GBS}
         out[name + "_col2im"] = {"ms": ms_c, "gbs": nbytes / ms_c / 1e6, "frac_hbm": nbytes / ms_c / 1e6 / PEAK_HBM_GBS}
         wr, nr = ws(L.query("odl_hip_sum_nchw_channels_workspace_bytes", N, OC, OH * OH))
-        ms_gb = time_region(torch, direct("odl_hip_sum_nchw_channels", ptr(gy), N, OC, OH * OH, ptr(gb), wr, nr, stream),
-                            steps, warmup)
+        ms_gb = time_region_auto(torch, direct("odl_hip_sum_nchw_channels", ptr(gy), N, OC, OH * OH, ptr(gb), wr, nr, stream))
         nb = 4.0 * (gy.numel() + OC)
         out[name + "_bias_grad"] = {"ms": ms_gb, "gbs": nb / ms_gb / 1e6, "frac_hbm": nb / ms_gb / 1e6 / PEAK_HBM_GBS}
         del x, w, b, gy, col, img, y, gx, gw
@@ -150,7 +158,7 @@ def extras(torch, capi, steps, warmup):
     wb, nbb = ws(L.query("odl_hip_conv2d_backward_workspace_bytes", *geom))
     fwd = direct("odl_hip_conv2d", ptr(x), ptr(w), ptr(b), *geom, ptr(y), wf, nf, stream)
     bwd = direct("odl_hip_conv2d_backward", ptr(gy), ptr(x), ptr(w), *geom, ptr(gx), ptr(gw), None, wb, nbb, stream)
-    ms_f, ms_b = time_region(torch, fwd, steps, warmup), time_region(torch, bwd, steps, warmup)
+    ms_f, ms_b = time_region_auto(torch, fwd), time_region_auto(torch, bwd)
     nb_f, nb_b = 4.0 * (x.numel() + y.numel()), 4.0 * (gy.numel() + 2 * x.numel() + gw.numel())
     out["conv_first_layer_256x1x28x28_to_32"] = {
         "fwd_ms": ms_f, "bwd_ms": ms_b, "fwd_gbs": nb_f / ms_f / 1e6, "bwd_gbs": nb_b / ms_b / 1e6,
@@ -162,7 +170,7 @@ def extras(torch, capi, steps, warmup):
     pg = (N, OC, H, H, 2, 2, 2, 2, 0, 0)
     pf = direct("odl_hip_max_pool2d", ptr(y), *pg, ptr(yp), ptr(idx), stream)
     pb = direct("odl_hip_max_pool2d_backward", ptr(gyp), ptr(idx), *pg, ptr(gxp), stream)
-    ms_pf, ms_pb = time_region(torch, pf, steps, warmup), time_region(torch, pb, steps, warmup)
+    ms_pf, ms_pb = time_region_auto(torch, pf), time_region_auto(torch, pb)
     nb_p = 4.0 * y.numel() + 12.0 * yp.numel()
     out["max_pool_2x2_256x32x28x28"] = {
         "fwd_ms": ms_pf, "bwd_ms": ms_pb, "fwd_gbs": nb_p / ms_pf / 1e6, "bwd_gbs": nb_p / ms_pb / 1e6,
@@ -174,14 +182,14 @@ def extras(torch, capi, steps, warmup):
         x, o = rnd(*shape), empty(1, shape[1])
         ss, ts = (ctypes.c_int64 * 2)(*shape), (ctypes.c_int64 * 2)(1, shape[1])
         wr, nr = ws(L.query("odl_hip_sum_to_workspace_bytes", ss, 2, ts, 2))
-        ms = time_region(torch, direct("odl_hip_sum_to", ptr(x), ss, 2, ts, 2, ptr(o), wr, nr, stream), steps, warmup)
+        ms = time_region_auto(torch, direct("odl_hip_sum_to", ptr(x), ss, 2, ts, 2, ptr(o), wr, nr, stream))
         nb = 4.0 * (x.numel() + shape[1])
         out[name] = {"ms": ms, "gbs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
     for name, (N, C) in (("softmax_ce_grad_512x10", (512, 10)), ("softmax_ce_grad_16384x1000_scaled", (16384, 1000))):
         x, gx = rnd(N, C), empty(N, C)
         t = torch.randint(0, C, (N,), device="cuda", generator=g)
-        ms = time_region(torch, direct("odl_hip_softmax_ce_grad", ptr(x), ptr(t), 1, N, C, ctypes.c_float(1.0), ptr(gx),
-                                       stream), steps, warmup)
+        ms = time_region_auto(torch, direct("odl_hip_softmax_ce_grad", ptr(x), ptr(t), 1, N, C, ctypes.c_float(1.0), ptr(gx),
+                                            stream))
         nb = 8.0 * N * C + 8.0 * N
         out[name] = {"ms": ms, "gbs": nb / ms / 1e6, "frac_hbm": nb / ms / 1e6 / PEAK_HBM_GBS}
     # batch normalisation at the shape of the first BatchNorm2d of the reference's conv_mnist example, batch 256.
@@ -197,7 +205,7 @@ def extras(torch, capi, steps, warmup):
                N, C, P, ptr(y), ptr(mean), ptr(var), ptr(xn), wbn, nbn, stream)
     b = direct("odl_hip_batch_norm_backward", ptr(gyb), ptr(gam), ptr(var), ptr(xn), ctypes.c_float(1e-5), N, C, P,
                ptr(gx), ptr(dg), ptr(dbt), wbn, nbn, stream)
-    ms_f, ms_b = time_region(torch, f, steps, warmup), time_region(torch, b, steps, warmup)
+    ms_f, ms_b = time_region_auto(torch, f), time_region_auto(torch, b)
     nb = 12.0 * N * C * P
     out["batch_norm_256x64x28x28"] = {"fwd_ms": ms_f, "bwd_ms": ms_b, "fwd_gbs": nb / ms_f / 1e6,
                                       "bwd_gbs": nb / ms_b / 1e6, "fwd_frac_hbm": nb / ms_f / 1e6 / PEAK_HBM_GBS,
@@ -213,13 +221,11 @@ def extras(torch, capi, steps, warmup):
         wp, nw = ws(wsz)
         fwd = direct("odl_hip_matmul", ptr(a), ptr(b), ptr(c), 1, M, N, K, 0, wp, nw, stream)
         bwd = direct("odl_hip_matmul_backward", ptr(a), ptr(b), ptr(dc), ptr(da), ptr(db), M, K, N, wp, nw, stream)
-        n = 3 if M >= 8192 else steps
-
         def both():
             fwd()
             bwd()
 
-        ms = time_region(torch, both, n, 1 if M >= 8192 else warmup)
+        ms = time_region(torch, both, 3, 1) if M >= 8192 else time_region_auto(torch, both)
         flop = 6.0 * M * N * K
         tf = flop / ms / 1e9
         out["gemm_fwd_bwd_%dx%dx%d" % (M, K, N)] = {"ms": ms, "tflops": tf, "frac_mfma_peak": tf / PEAK_FP32_MFMA_TFLOPS,
@@ -236,7 +242,7 @@ def extras(torch, capi, steps, warmup):
         capi.mat_mul_backward(x2, w2, g2)
         capi.mat_mul_backward(x1, w1, g1)
 
-    ms = time_region(torch, mlp_gemms, steps, warmup)
+    ms = time_region_auto(torch, mlp_gemms)
     flop = 6.0 * 512 * (784 * 1000 + 1000 * 10)
     out["mlp_gemms_fwd_bwd"] = {"ms": ms, "tflops": flop / ms / 1e9, "flop": flop}
     return out

@@ -151,9 +151,8 @@ size_t odl_hip_conv2d_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, 
 /* Kernel selection of the 3x3 / stride 1 / padding 1 convolutions. The kernel that keeps the input patch in LDS is
  * chosen for the forward and the input gradient only when it would launch at least `min_workgroups` workgroups (default:
  * one per compute unit of the device; smaller layers go to the K-sliced implicit kernels, which fill the chip better).
- * This call replaces that threshold for the whole process, and any value >= 0 also lifts the rule that sends layers of more
- * than 48 input channels on long image rows to the implicit kernel; a negative value restores the default. It exists so
- * that tests can send small shapes through the LDS-patch kernel. The choice enters the workspace sizes: never change it
+ * This call replaces that threshold for the whole process; a negative value restores the default. It exists so that
+ * tests can send small shapes through the LDS-patch kernel. The choice enters the workspace sizes: never change it
  * between a *_workspace_bytes query and the call the query was made for. No counterpart in the reference. */
 int odl_hip_set_conv_patch_min_workgroups(int64_t min_workgroups);
 

@@ -49,12 +49,13 @@ int conv_small_forward(const float *x, const float *w, const float *b, float *y,
 // 3x3, stride 1, padding 1 with the input channels a multiple of 16: the input patch stays in LDS (conv_patch.hip)
 bool conv_patch_forward_ok(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
                            int SW, int PH, int PW);
-size_t conv_patch_forward_workspace(int64_t C, int64_t OC);
+size_t conv_patch_forward_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC);
 int conv_patch_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
                        int64_t W, int64_t OC, int act, void *workspace, size_t workspace_bytes, hipStream_t st);
 bool conv_patch_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
                          int SW, int PH, int PW);
-size_t conv_patch_dgrad_workspace(int64_t C, int64_t OC);
+size_t conv_patch_dgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC);
+
 int conv_patch_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
                      void *workspace, size_t workspace_bytes, hipStream_t st);
 bool conv_small_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
@@ -844,7 +845,7 @@ size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W
         // no im2col matrix: K-slice partials for small outputs, or the filter copy of the LDS-patch kernel
         size_t need = odl::conv_implicit_forward_workspace(N, C, H, W, OC, KH, KW, OH, OW);
         if (odl::conv_patch_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, SH, SW, PH, PW))
-            need = std::max(need, odl::conv_patch_forward_workspace(C, OC));
+            need = std::max(need, odl::conv_patch_forward_workspace(N, C, H, W, OC));
         return align256(need);
     }
     return align256((size_t)(N * OH * OW * C * KH * KW) * sizeof(float));
@@ -897,7 +898,7 @@ int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packe
     if (odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, g.OH, g.OW))
         return odl::conv_small_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, act, st);
     if (odl::conv_patch_forward_ok(x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW) &&
-        workspace_bytes >= odl::conv_patch_forward_workspace(C, OC) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+        workspace_bytes >= odl::conv_patch_forward_workspace(N, C, H, W, OC) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
         workspace)
         return odl::conv_patch_forward(x, w, b, y, N, C, H, W, OC, act, workspace, workspace_bytes, st);
     if (odl::conv_implicit_forward_ok(w, N, C, H, W, OC, KH, KW, g.OH, g.OW))
@@ -942,9 +943,9 @@ BwdPlan plan_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t 
     const int64_t M = N * OH * OW, K = C * KH * KW;
     p.wgrad_small = odl::conv_small_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
     p.dgrad_small = odl::conv_small_dgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
-    p.wgrad_implicit = !p.wgrad_small && odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
     // 3x3 at stride 1 keeps the image size only with a padding of 1
     const int pad = (OH == H && OW == W) ? 1 : -1;
+    p.wgrad_implicit = !p.wgrad_small && odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
     p.dgrad_patch = !p.dgrad_small && odl::conv_patch_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW, pad, pad);
     p.dgrad_implicit = !p.dgrad_small && !p.dgrad_patch && odl::conv_implicit_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW);
     const bool no_col = (p.wgrad_small || p.wgrad_implicit) && (p.dgrad_small || p.dgrad_patch || p.dgrad_implicit);
@@ -953,7 +954,7 @@ BwdPlan plan_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t 
                               : p.wgrad_implicit ? odl::conv_implicit_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
                                                  : odl::sgemm_workspace(OC, K, M, 0));
     p.wp_bytes = p.dgrad_small      ? align256(odl::conv_small_dgrad_workspace(C, OC, KH, KW))
-                 : p.dgrad_patch    ? align256(odl::conv_patch_dgrad_workspace(C, OC))
+                 : p.dgrad_patch    ? align256(odl::conv_patch_dgrad_workspace(N, C, H, W, OC))
                  : p.dgrad_implicit ? align256(odl::conv_implicit_dgrad_workspace(C, OC, KH, KW, N * H * W))
                                     : 0;
     p.red_bytes = align256(odl::sum_nchw_channels_workspace(N, OC, OH * OW));

@@ -38,6 +38,12 @@ struct PatchGeom
     int PW, plane;                   // patch width W + 2 and positions per patch (rows * PW)
     int pixels, mtiles, act;
     odl::FastDiv by_w, by_h, by_hw, by_pw;
+    // Tail split. The launch runs in rounds of as many workgroups as the chip holds; when the last round would be a
+    // handful of tiles, those tiles (numbers tail_first..) are cut into tail_pieces runs of channel slabs instead —
+    // workgroups main_blocks.. — which write their raw accumulators to tail_ws, one [BM][128] block per (tile, piece);
+    // conv_patch_tail_kernel adds the pieces in order and finishes the tile.
+    int main_blocks, tail_first, tail_pieces, slabs_per_piece;
+    float *tail_ws;
 };
 
 // wp[(m*nslab + slab)*144 + tap*16 + cc]: the zero-padded filter copy the kernel stages with 16-byte copies
@@ -69,7 +75,14 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
     float *Bs = lds + BM * kLda;  // [plane + 3][kLdp]; the last three positions stay zero
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l32 = lane & 31, lh = lane >> 5;
-    const int mt = blockIdx.x % g.mtiles, nt = blockIdx.x / g.mtiles;
+    int tile = blockIdx.x, piece = -1;
+    if (g.tail_pieces > 0 && (int)blockIdx.x >= g.main_blocks)
+    {
+        const int u = (int)blockIdx.x - g.main_blocks;
+        tile = g.tail_first + u / g.tail_pieces;
+        piece = u % g.tail_pieces;
+    }
+    const int mt = tile % g.mtiles, nt = tile / g.mtiles;
     const int m0 = mt * BM, p0 = nt * kPixTile;
     const int wm = (wave % WM) * TM, wn = (wave / WM) * TN;
     const int gr0 = (int)odl::fastdiv((unsigned)p0, g.by_w);  // first image row (of the whole batch) of the tile
@@ -128,6 +141,8 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
 
     const int nslab = g.Cin / kSlab;
     const int ch_stride = CH_MINOR ? 1 : g.HW;
+    const int s_beg = piece < 0 ? 0 : piece * g.slabs_per_piece;
+    const int s_end = piece < 0 ? nslab : (s_beg + g.slabs_per_piece < nslab ? s_beg + g.slabs_per_piece : nslab);
 
     // one slab travels global memory -> registers -> LDS; the loads of slab s + 1 are issued before the matrix
     // instructions of slab s and land while those run
@@ -204,13 +219,13 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
         }
     };
 
-    load_slab(0);
-    for (int s = 0; s < nslab; ++s)
+    load_slab(s_beg);
+    for (int s = s_beg; s < s_end; ++s)
     {
         __syncthreads();  // the previous slab has been read
         store_slab();
         __syncthreads();
-        if (s + 1 < nslab)
+        if (s + 1 < s_end)
             load_slab(s + 1);
 
         // ---- 144 values of K: nine taps x two groups of eight channels. One 16-byte read per operand block brings four
@@ -261,6 +276,19 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
     }
 
     // ---- accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
+    if (piece >= 0)
+    {
+        // a piece of a tail tile: the raw sums, tile-local (rows or pixels past the end hold whatever the padding gave)
+        float *out = g.tail_ws + ((int64_t)(tile - g.tail_first) * g.tail_pieces + piece) * (BM * kPixTile);
+#pragma unroll
+        for (int j = 0; j < CB; ++j)
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    out[(wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4)) * kPixTile + wn + j * 32 + l32] = acc[i][j][r];
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < CB; ++j)
     {
@@ -283,6 +311,31 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
                 out[(int64_t)row * g.HW] = odl::apply_act(v, g.act);
             }
     }
+}
+
+// Adds the pieces of each tail tile in piece order and stores the tile the way the main kernel does (bias, activation,
+// NCHW). One thread per output element, lanes along the pixels.
+__global__ __launch_bounds__(kThreads) void conv_patch_tail_kernel(const PatchGeom g, int BM)
+{
+    const int per_tile = BM * kPixTile;
+    const int idx = blockIdx.x * kThreads + threadIdx.x;
+    const int ti = idx / per_tile, e = idx - ti * per_tile;
+    const int tile = g.tail_first + ti;
+    if (tile >= g.mtiles * (int)((g.pixels + kPixTile - 1) / kPixTile))
+        return;
+    const int row_l = e / kPixTile, px = e - row_l * kPixTile;
+    const int mt = tile % g.mtiles, nt = tile / g.mtiles;
+    const int row = mt * BM + row_l, p = nt * kPixTile + px;
+    if (row >= g.M || p >= g.pixels)
+        return;
+    const float *src = g.tail_ws + (int64_t)ti * g.tail_pieces * per_tile + e;
+    float v = src[0];
+    for (int z = 1; z < g.tail_pieces; ++z)
+        v += src[(int64_t)z * per_tile];
+    if (g.bias)
+        v = v + g.bias[row];
+    const int n = (int)odl::fastdiv((unsigned)p, g.by_hw), hw = p - n * g.HW;
+    g.dst[((int64_t)n * g.M + row) * g.HW + hw] = odl::apply_act(v, g.act);
 }
 
 inline int patch_rows(int64_t W)
@@ -344,6 +397,70 @@ size_t packed_bytes(int64_t Cin, int64_t M)
     return (((size_t)Cin * 9 * mpad * sizeof(float)) + 255) & ~(size_t)255;
 }
 
+// the channel-minor kernel runs a 33..64-row product of many pixel tiles as two 32-row tiles
+bool use_halves(int64_t pixels, int64_t M, bool ch_minor)
+{
+    return ch_minor && tile_bm(M) == 64 && M <= 64 && odl::ceil_div(pixels, kPixTile) >= 512;
+}
+
+// Workgroups of a variant that one compute unit holds at once: what the runtime reports for the kernel (registers and
+// LDS together), or, on a machine without a device — where only the workspace-size queries run — the same figure from
+// the kernels' register counts (96 / 156 / 138 / 198 of 512 per SIMD) and the LDS size.
+int wgs_per_cu(int bm, bool ch_minor, size_t lds)
+{
+    int n = 0;
+    const void *fn = bm == 32 ? (ch_minor ? reinterpret_cast<const void *>(&conv_patch_kernel<32, true>)
+                                          : reinterpret_cast<const void *>(&conv_patch_kernel<32, false>))
+                              : (ch_minor ? reinterpret_cast<const void *>(&conv_patch_kernel<64, true>)
+                                          : reinterpret_cast<const void *>(&conv_patch_kernel<64, false>));
+    (void)allow_lds(bm, ch_minor);
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, kThreads, lds) == hipSuccess && n > 0)
+        return n;
+    (void)hipGetLastError();
+    const int by_regs = bm == 32 ? (ch_minor ? 5 : 3) : (ch_minor ? 3 : 2);
+    const int by_lds = (int)((160 * 1024) / (lds > 0 ? lds : 1));
+    n = by_regs < by_lds ? by_regs : by_lds;
+    return n > 0 ? n : 1;
+}
+
+struct TailPlan
+{
+    int tiles = 0, pieces = 0, slabs_per_piece = 0;
+    size_t bytes = 0;
+};
+
+// A launch runs in rounds of `slots` workgroups. When the last round would hold at most half of that, its tiles are
+// cut into runs of channel slabs so that the round is short.
+TailPlan plan_tail(int64_t n_wg, int nslab, int bm, bool ch_minor, size_t lds)
+{
+    TailPlan p;
+    const int64_t slots = (int64_t)wgs_per_cu(bm, ch_minor, lds) * odl::device_cus();
+    const int64_t r = n_wg % slots;
+    if (n_wg <= slots || r == 0 || r > slots / 2 || nslab < 2)
+        return p;
+    int64_t pieces = slots / r;
+    if (pieces > nslab)
+        pieces = nslab;
+    if (pieces > 8)
+        pieces = 8;
+    if (pieces < 2)
+        return p;
+    p.slabs_per_piece = (int)odl::ceil_div(nslab, pieces);
+    p.pieces = (int)odl::ceil_div(nslab, p.slabs_per_piece);
+    p.tiles = (int)r;
+    p.bytes = (size_t)p.tiles * p.pieces * bm * kPixTile * sizeof(float);
+    return p;
+}
+
+TailPlan plan_tail_for(int64_t N, int64_t Cin, int64_t H, int64_t W, int64_t M, bool ch_minor)
+{
+    const int bm_pad = tile_bm(M);
+    const int bm = use_halves(N * H * W, M, ch_minor) ? 32 : bm_pad;
+    const int64_t mtiles = odl::ceil_div(M, bm_pad) * bm_pad / bm;
+    const int plane = patch_rows(W) * ((int)W + 2);
+    return plan_tail(odl::ceil_div(N * H * W, kPixTile) * mtiles, (int)(Cin / kSlab), bm, ch_minor, lds_bytes(bm, plane));
+}
+
 int launch(const float *src, const float *w, const float *bias, float *dst, int64_t N, int64_t Cin, int64_t H, int64_t W,
            int64_t M, bool ch_minor, int act, void *workspace, size_t workspace_bytes, hipStream_t st, const char *who)
 {
@@ -355,7 +472,7 @@ int launch(const float *src, const float *w, const float *bias, float *dst, int6
     // tiles as two 32-row tiles: twice the workgroups at half the length leave a shorter tail when the last
     // workgroups of the launch drain (64 rows x 784 pixel tiles: 170 -> 162 us).
     const int bm_pad = tile_bm(M);
-    const bool halves = ch_minor && bm_pad == 64 && M <= 64 && odl::ceil_div(N * H * W, kPixTile) >= 512;
+    const bool halves = use_halves(N * H * W, M, ch_minor);
     const int bm = halves ? 32 : bm_pad;
     PatchGeom g{};
     g.src = src, g.bias = bias, g.dst = dst;
@@ -371,9 +488,19 @@ int launch(const float *src, const float *w, const float *bias, float *dst, int6
     hipLaunchKernelGGL(conv_patch_pack_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, w, wp, g.Cin,
                        g.M, g.Mpad, ch_minor ? 1 : 0);
     ODL_LAUNCH_CHECK();
-    const dim3 grid((unsigned)(odl::ceil_div(g.pixels, kPixTile) * g.mtiles));
     const size_t lds = lds_bytes(bm, g.plane);
     ODL_HIP_CHECK(allow_lds(bm, ch_minor));
+    // the tiles of a short last round go out as runs of channel slabs (when the workspace has room for their sums)
+    const int64_t n_wg = odl::ceil_div(g.pixels, kPixTile) * g.mtiles;
+    const TailPlan tp = plan_tail(n_wg, g.Cin / kSlab, bm, ch_minor, lds);
+    g.main_blocks = (int)n_wg, g.tail_first = (int)n_wg, g.tail_pieces = 0, g.slabs_per_piece = 0, g.tail_ws = nullptr;
+    if (tp.pieces > 0 && workspace_bytes >= need + tp.bytes)
+    {
+        g.tail_first = (int)(n_wg - tp.tiles), g.main_blocks = g.tail_first;
+        g.tail_pieces = tp.pieces, g.slabs_per_piece = tp.slabs_per_piece;
+        g.tail_ws = reinterpret_cast<float *>(static_cast<char *>(workspace) + need);
+    }
+    const dim3 grid((unsigned)(g.main_blocks + (g.tail_pieces > 0 ? tp.tiles * tp.pieces : 0)));
     if (bm == 32)
     {
         if (ch_minor)
@@ -389,6 +516,13 @@ int launch(const float *src, const float *w, const float *bias, float *dst, int6
             hipLaunchKernelGGL((conv_patch_kernel<64, false>), grid, dim3(kThreads), lds, st, g);
     }
     ODL_LAUNCH_CHECK();
+    if (g.tail_pieces > 0)
+    {
+        const int64_t threads = (int64_t)tp.tiles * bm * kPixTile;
+        hipLaunchKernelGGL(conv_patch_tail_kernel, dim3((unsigned)odl::ceil_div(threads, kThreads)), dim3(kThreads), 0, st, g,
+                           bm);
+        ODL_LAUNCH_CHECK();
+    }
     return ODL_OK;
 }
 }  // namespace
@@ -398,19 +532,16 @@ namespace odl
 bool conv_patch_forward_ok(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
                            int SW, int PH, int PW)
 {
-    // measured on the 3x3 layers of the benchmark networks: with few input channels (K < 576) the implicit-GEMM
-    // forward's fixed cost per workgroup dominates and this kernel wins; with more it still wins on short image rows
-    // (64 -> 128 channels at 14x14: 96 against 109 us), but on long rows, where the patch with its halo rows holds
-    // more than twice the pixels the tile produces (W = 56: 6 rows for 2.3), the implicit kernel is as fast or
-    // faster (172 against 175 us). The threshold override lifts this rule too.
-    if (C > 48 && (int64_t)patch_rows(W) * W > 2 * kPixTile && g_min_wgs.load(std::memory_order_relaxed) < 0)
-        return false;
+    // Measured on the 3x3 layers of the benchmark networks, this kernel is the faster forward whenever it fills the chip:
+    // few input channels (K < 576: the implicit-GEMM kernel's fixed cost per workgroup dominates there), short image
+    // rows (64 -> 128 channels at 14x14: 96 against 109 us), and — since the tiles of a short last round are cut into
+    // runs of channel slabs — long rows too (64 -> 128 channels at 56x56: 165 against 176 us).
     return shape_ok(x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
 }
 
-size_t conv_patch_forward_workspace(int64_t C, int64_t OC)
+size_t conv_patch_forward_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC)
 {
-    return packed_bytes(C, OC);
+    return packed_bytes(C, OC) + plan_tail_for(N, C, H, W, OC, false).bytes;
 }
 
 int conv_patch_forward(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t H,
@@ -425,9 +556,9 @@ bool conv_patch_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64
     return shape_ok(gy, N, OC, H, W, C, KH, KW, SH, SW, PH, PW);
 }
 
-size_t conv_patch_dgrad_workspace(int64_t C, int64_t OC)
+size_t conv_patch_dgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC)
 {
-    return packed_bytes(OC, C);
+    return packed_bytes(OC, C) + plan_tail_for(N, OC, H, W, C, true).bytes;
 }
 
 int conv_patch_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,

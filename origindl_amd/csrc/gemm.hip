@@ -104,8 +104,8 @@ __device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int
 // through LDS before the epilogue. For products with at most one workgroup per compute unit: a lone set of four waves
 // (one per SIMD) leaves the matrix pipe idle whenever it waits for LDS, memory or the barrier; the second set fills
 // those gaps without changing the tile shape.
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI, int SB = SB_PLAIN, int CK = 0, int WS = 1>
-__global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && VEC && SB != SB_CONV_WGRAD ? 4 : 1)) void sgemm_mfma_kernel(GemmArgs g, ConvSrc cv)
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, int EPI, int SB = SB_PLAIN, int CK = 0, int WS = 1, bool PF2 = false>
+__global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && VEC && SB != SB_CONV_WGRAD ? (PF2 ? 3 : 4) : 1)) void sgemm_mfma_kernel(GemmArgs g, ConvSrc cv)
 {
     constexpr int NT = kThreads * WS;
     static_assert(WS == 1 || (WS == 2 && SB == SB_PLAIN && VEC && (BK / 8) % 2 == 0), "the second wave set: plain operands only");
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int nkt = (int)((kend - kbeg + BK - 1) / BK);
 
-    float ra[A_PER_T], rb_[B_PER_T];
+    float ra[A_PER_T], rb_main[B_PER_T];
 
     auto load_tile = [&](const float *__restrict__ src, int64_t ld, bool kmajor, int64_t row0, int64_t rows,
                          int64_t k0, int brows, float *regs, int per_t) {
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
         }
     }
 
-    auto load_b = [&](int64_t k0) {
+    auto load_b = [&](int64_t k0, float *rb_) {
         if constexpr (SB == SB_PLAIN)
         {
             load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, k0, BN, rb_, B_PER_T);
@@ -432,7 +432,7 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
         }
     };
 
-    auto store_b = [&](float *lds) {
+    auto store_b = [&](float *lds, const float *rb_) {
         if constexpr (SB == SB_PLAIN)
         {
             store_tile(lds, LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
@@ -473,9 +473,9 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
     if (nkt > 0)
     {
         load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, kbeg, BM, ra, A_PER_T);
-        load_b(kbeg);
+        load_b(kbeg, rb_main);
         store_tile(As[0], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
-        store_b(Bs[0]);
+        store_b(Bs[0], rb_main);
     }
     __syncthreads();
 
@@ -528,16 +528,17 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
         }
     };
 
-    if constexpr (WS > 1)
+    if constexpr (WS > 1 || PF2)
     {
         // One workgroup per compute unit has nobody to cover its memory latency, and a K slab's worth of matrix
         // instructions (0.85 us) is shorter than a load's round trip: operands are fetched TWO slabs ahead into two
-        // register sets, so that each load has two slab times to land before it is stored to LDS.
+        // register sets, so that each load has two slab times to land before it is stored to LDS. The gathered
+        // convolution operands, whose loads wait longer still, can ask for the same (PF2).
         float ra2[A_PER_T], rb2[B_PER_T];
         if (nkt > 1)
         {
             load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, kbeg + BK, BM, ra2, A_PER_T);
-            load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, kbeg + BK, BN, rb2, B_PER_T);
+            load_b(kbeg + BK, rb2);
         }
         for (int kt = 0; kt < nkt; kt += 2)
         {
@@ -545,13 +546,13 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
             {
                 const int64_t k0 = kbeg + (int64_t)(kt + 2) * BK;
                 load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra, A_PER_T);
-                load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, k0, BN, rb_, B_PER_T);
+                load_b(k0, rb_main);
             }
             mma(As[0], Bs[0]);
             if (kt + 1 < nkt)
             {
                 store_tile(As[1], LDA_S, A_KMAJOR, BM, ra2, A_PER_T);
-                store_tile(Bs[1], LDB_S, B_KMAJOR, BN, rb2, B_PER_T);
+                store_b(Bs[1], rb2);
             }
             __syncthreads();
             if (kt + 1 >= nkt)
@@ -560,13 +561,13 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
             {
                 const int64_t k0 = kbeg + (int64_t)(kt + 3) * BK;
                 load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra2, A_PER_T);
-                load_tile(g.B, g.ldb, B_KMAJOR, n0, g.N, k0, BN, rb2, B_PER_T);
+                load_b(k0, rb2);
             }
             mma(As[1], Bs[1]);
             if (kt + 2 < nkt)
             {
                 store_tile(As[0], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
-                store_tile(Bs[0], LDB_S, B_KMAJOR, BN, rb_, B_PER_T);
+                store_b(Bs[0], rb_main);
             }
             __syncthreads();
         }
@@ -580,13 +581,13 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
             {
                 const int64_t k0 = kbeg + (int64_t)(kt + 1) * BK;
                 load_tile(g.A, g.lda, A_KMAJOR, m0, g.M, k0, BM, ra, A_PER_T);
-                load_b(k0);
+                load_b(k0, rb_main);
             }
             mma(As[cur], Bs[cur]);
             if (kt + 1 < nkt)
             {
                 store_tile(As[cur ^ 1], LDA_S, A_KMAJOR, BM, ra, A_PER_T);
-                store_b(Bs[cur ^ 1]);
+                store_b(Bs[cur ^ 1], rb_main);
             }
             __syncthreads();
         }
@@ -1092,6 +1093,10 @@ bool conv_tile_bm64(int64_t M, int64_t N, int splits)
     return M <= 64 || odl::ceil_div(M, 128) * odl::ceil_div(N, 128) * splits < odl::device_cus();
 }
 
+// Fetching the gathered operands two K slabs ahead was measured and lost: the second register set costs the 128x128
+// kernels their fourth wave per SIMD (C1 forward 175 -> 254 us, C2 forward 58 -> 91 us).
+constexpr bool kConvPF2 = false;
+
 template <int SB, bool TA, int EPI>
 int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, void *tail_ws, size_t tail_bytes, hipStream_t st)
 {
@@ -1105,8 +1110,8 @@ int launch_conv_tile(GemmArgs g, const ConvSrc &cv, int splits, void *tail_ws, s
     if constexpr (SB != SB_CONV_FWD_TAP || CKV > 0)                                                              \
         if (bm64 == (BMV == 64) && ck == CKV)                                                                    \
         {                                                                                                        \
-            hipLaunchKernelGGL((sgemm_mfma_kernel<BMV, 128, 16, TA, false, true, EPI, SB, CKV>), grid, block, 0, \
-                               st, g, cv);                                                                       \
+            hipLaunchKernelGGL((sgemm_mfma_kernel<BMV, 128, 16, TA, false, true, EPI, SB, CKV, 1, kConvPF2>), grid,  \
+                               block, 0, st, g, cv);                                                             \
             launch_tail_fixup(g, BMV, 128, EPI, st);                                                             \
             return ODL_OK;                                                                                       \
         }

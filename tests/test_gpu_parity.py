@@ -299,6 +299,13 @@ CONV_SEEDED = [
     (7, 16, 5, 6, 64, 3, 3, 1, 1),     # tiles that start and end in the middle of an image; 64 gradient channels
     (3, 16, 8, 8, 24, 3, 3, 1, 1),     # W a multiple of 4: the LDS patch is staged with 16-byte row loads
     (2, 48, 6, 28, 40, 3, 3, 1, 1),    # the same over three channel slabs and rows shared between tiles
+    # more 3x3/s1/p1 layers with channels in groups of 32 and 64 or more filters: two filter tiles with a ragged second
+    # one, three channel groups, rows wider than a pixel tile, a single pixel, tiles that cross image boundaries
+    (3, 64, 10, 12, 128, 3, 3, 1, 1),
+    (2, 32, 9, 70, 64, 3, 3, 1, 1),
+    (4, 96, 6, 5, 192, 3, 3, 1, 1),
+    (2, 32, 1, 1, 64, 3, 3, 1, 1),
+    (5, 32, 7, 9, 68, 3, 3, 1, 1),
 ]
 
 
