@@ -272,6 +272,11 @@ int odl_hip_unary_dtype(int op, int dtype, const void *a, int64_t n, void *out, 
 int odl_hip_pow_scalar_dtype(int dtype, const void *a, int64_t n, double exponent, void *out, void *stream);
 /* origin::cuda::{zeros,ones,full}, from_scalar in any type: host_value points at ONE element of that type on the host */
 int odl_hip_fill_dtype(void *dst, int dtype, int64_t n, const void *host_value, void *stream);
+/* OriginMat::permute (include/origin/mat/origin/origin_mat.h:75; src/mat/origin/cuda/shape/permute.cu,
+ * src/mat/origin/cpu/shape/permute.cpp:22-110): a dense copy whose dimension d is the input's dimension host_perm[d],
+ * any element type, up to 8 dimensions. ODL_ERR_INVALID_ARG for an order that is not a permutation. */
+int odl_hip_permute(const void *src, int dtype, const int64_t *host_shape, int ndim, const int *host_perm, void *dst,
+                    void *stream);
 /* Mat::sum over [outer, axis, inner] in any type (operation_templates.h:270-357): integers sum with wrap-around in their
  * own width, float64 in a fixed parallel order. through_float != 0 passes each result through a float on its way back
  * into the element type, which is what the reference's whole-tensor sum does (src/mat/origin/cpu/math/sum.cpp:18-35,83-90). */

@@ -269,6 +269,30 @@ __global__ void fold_kernel(const typename Acc<T>::type *__restrict__ part, T *_
     dst[c] = v;
 }
 
+// permute: out[o0..] = in[..] with output dimension d taken from input dimension perm[d]; one thread per output
+// element (lanes along the output's last dimension: coalesced writes), the input offset rebuilt from the output index
+struct PermuteDims
+{
+    int nd;
+    int64_t oshape[8];
+    int64_t istride[8];  // stride in the input of the dimension that became output dimension d
+};
+
+template <typename T>
+__global__ void permute_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t total, PermuteDims d)
+{
+    for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (int64_t)gridDim.x * blockDim.x)
+    {
+        int64_t r = t, si = 0;
+        for (int k = d.nd - 1; k >= 0; --k)
+        {
+            si += (r % d.oshape[k]) * d.istride[k];
+            r /= d.oshape[k];
+        }
+        dst[t] = src[si];
+    }
+}
+
 struct SumPlan
 {
     int64_t slices, chunk;
@@ -404,6 +428,56 @@ int odl_hip_fill_dtype(void *dst, int dtype, int64_t n, const void *host_value, 
         ODL_LAUNCH_CHECK();
         return ODL_OK;
     });
+}
+
+int odl_hip_permute(const void *src, int dtype, const int64_t *host_shape, int ndim, const int *host_perm, void *dst,
+                    void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(ndim >= 0 && ndim <= 8, "permute: up to 8 dimensions, got %d", ndim);
+    ODL_REQUIRE(dtype >= 0 && dtype < DT_COUNT, "permute: unknown element type code %d", dtype);
+    ODL_REQUIRE(ndim == 0 || (host_shape && host_perm), "permute: null shape or order");
+    PermuteDims d{};
+    d.nd = ndim;
+    bool used[8] = {false};
+    int64_t istr[8], total = 1;
+    for (int i = ndim - 1; i >= 0; --i)
+    {
+        ODL_REQUIRE(host_shape[i] >= 0, "permute: negative extent");
+        istr[i] = total;
+        total *= host_shape[i];
+    }
+    for (int k = 0; k < ndim; ++k)
+    {
+        const int p = host_perm[k];
+        // the reference's messages (src/mat/origin/cpu/shape/permute.cpp:33-45)
+        ODL_REQUIRE(p >= 0 && p < ndim, "permute: invalid dimension %d (must be in [0, %d))", p, ndim);
+        ODL_REQUIRE(!used[p], "permute: duplicate dimension %d", p);
+        used[p] = true;
+        d.oshape[k] = host_shape[p];
+        d.istride[k] = istr[p];
+    }
+    if (total == 0)
+        return ODL_OK;
+    ODL_REQUIRE(src && dst, "permute: null operand");
+    hipStream_t st = odl::as_stream(stream);
+    // elements of equal width move alike: 1, 4 or 8 bytes
+    switch (dtype_bytes(dtype))
+    {
+        case 1:
+            hipLaunchKernelGGL((permute_kernel<uint8_t>), dim3(grid_for(total)), dim3(kBlock), 0, st,
+                               static_cast<const uint8_t *>(src), static_cast<uint8_t *>(dst), total, d);
+            break;
+        case 8:
+            hipLaunchKernelGGL((permute_kernel<uint64_t>), dim3(grid_for(total)), dim3(kBlock), 0, st,
+                               static_cast<const uint64_t *>(src), static_cast<uint64_t *>(dst), total, d);
+            break;
+        default:
+            hipLaunchKernelGGL((permute_kernel<uint32_t>), dim3(grid_for(total)), dim3(kBlock), 0, st,
+                               static_cast<const uint32_t *>(src), static_cast<uint32_t *>(dst), total, d);
+    }
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
 }
 
 size_t odl_hip_sum_axis_dtype_workspace_bytes(int dtype, int64_t outer, int64_t axis, int64_t inner)

@@ -1093,8 +1093,9 @@ bool conv_tile_bm64(int64_t M, int64_t N, int splits)
     return M <= 64 || odl::ceil_div(M, 128) * odl::ceil_div(N, 128) * splits < odl::device_cus();
 }
 
-// Fetching the gathered operands two K slabs ahead was measured and lost: the second register set costs the 128x128
-// kernels their fourth wave per SIMD (C1 forward 175 -> 254 us, C2 forward 58 -> 91 us).
+// Fetching the gathered operands two K slabs ahead was measured and lost, on full launches (the second register set
+// costs the 128x128 kernels their fourth wave per SIMD: C1 forward 175 -> 254 us) and on sparse ones alike (C2 forward,
+// one or two workgroups per compute unit: 57 -> 90 us).
 constexpr bool kConvPF2 = false;
 
 template <int SB, bool TA, int EPI>

@@ -323,6 +323,8 @@ public:
     // (one small device-to-host copy; no upload of the loss afterwards)
     std::unique_ptr<Mat> softmax_cross_entropy_checked(const Mat &target) const;
     std::unique_ptr<Mat> softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const;
+    // include/origin/mat/origin/origin_mat.h:75: a dense copy with the dimensions in the order `dims`
+    std::unique_ptr<Mat> permute(const std::vector<int> &dims) const;
     // on a loss made by softmax_cross_entropy_device / _checked: the out-of-range-label flag that lies behind the loss
     // in device memory, read back now (one small device-to-host copy; synchronises). A recorded step cannot raise the
     // reference's exception for a bad label — it contributes nothing to the loss — so a caller that replays a graph on

@@ -1504,6 +1504,25 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target)
     return loss;
 }
 
+std::unique_ptr<Mat> OriginMat::permute(const std::vector<int> &dims) const
+{
+    if (dims.size() != shape_.size())
+        THROW_INVALID_ARG("permute: dims size {} does not match input dimension {}", dims.size(), shape_.size());
+    std::vector<size_t> od;
+    for (int d : dims)
+    {
+        if (d < 0 || d >= (int)shape_.size())
+            THROW_INVALID_ARG("permute: invalid dimension {} (must be in [0, {}))", d, shape_.size());
+        od.push_back(shape_[d]);
+    }
+    const OriginMat &x = dev_any(*this, "permute");
+    auto out = new_like(x, Shape(od), dtype_);
+    const std::vector<int64_t> in = dims64(shape_);
+    check(odl_hip_permute(x.storage()->data(), code(dtype_), in.data(), (int)shape_.size(), dims.data(),
+                          out->storage()->data(), cur()));
+    return out;
+}
+
 bool OriginMat::loss_bad_label_flag() const
 {
     if (device().type() != DeviceType::kCUDA || dtype_ != DataType::kFloat32 || elements() != 1 || !storage_ ||

@@ -1088,3 +1088,23 @@ def test_elementwise_fill_and_sum_in_every_element_type(api, name):
                 w = x.astype(np.int64).sum(axis=1).reshape(-1).astype(t)  # the wrapped sum in the type's own width
                 w = w.astype(np.float32).astype(t) if through_float else w
                 assert np.array_equal(host(res), w), (name, outer, axis, inner, through_float)
+
+
+def test_permute_is_numpy_transpose_in_every_element_width(api):
+    # src/mat/origin/cpu/shape/permute.cpp:22-110: output dimension d is input dimension dims[d]
+    import ctypes
+    L = api.lib()
+    rng = np.random.default_rng(61)
+    for name, shape, perm in (("f32", (4, 3, 5, 7), (0, 2, 3, 1)), ("f32", (2, 3, 85, 6, 5), (0, 1, 3, 4, 2)),
+                              ("f64", (6, 5), (1, 0)), ("u8", (3, 4, 5), (2, 0, 1)), ("i64", (7,), (0,)),
+                              ("i32", (2, 1, 3, 1, 4), (4, 3, 2, 1, 0))):
+        code, t = DT[name]
+        x = _typed_values(rng, t, int(np.prod(shape))).reshape(shape)
+        dx = dev(x)
+        out = torch.empty(tuple(shape[p] for p in perm), dtype=getattr(torch, np.dtype(t).name), device="cuda")
+        sh, pm = (ctypes.c_int64 * len(shape))(*shape), (ctypes.c_int * len(perm))(*perm)
+        L.call("odl_hip_permute", dx.data_ptr(), code, sh, len(shape), pm, out.data_ptr(), None)
+        assert np.array_equal(host(out), np.transpose(x, perm)), (name, shape, perm)
+    sh, pm = (ctypes.c_int64 * 2)(3, 4), (ctypes.c_int * 2)(0, 0)
+    with pytest.raises(api.OdlInvalidArgument):
+        L.call("odl_hip_permute", dx.data_ptr(), 0, sh, 2, pm, out.data_ptr(), None)
