@@ -44,6 +44,7 @@ struct PatchGeom
     // conv_patch_tail_kernel adds the pieces in order and finishes the tile.
     int main_blocks, tail_first, tail_pieces, slabs_per_piece;
     float *tail_ws;
+    int xcds;  // consecutive workgroup ids are dealt round-robin over this many XCDs, each with an L2 of its own
 };
 
 // wp[(m*nslab + slab)*144 + tap*16 + cc]: the zero-padded filter copy the kernel stages with 16-byte copies
@@ -81,6 +82,15 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
         const int u = (int)blockIdx.x - g.main_blocks;
         tile = g.tail_first + u / g.tail_pieces;
         piece = u % g.tail_pieces;
+    }
+    else
+    {
+        // a contiguous band of tiles per XCD: the output-channel tiles of one pixel tile read the same patch, and the
+        // next pixel tile shares two of its rows, so they should meet in one L2
+        const unsigned total = (unsigned)g.main_blocks, nx = (unsigned)g.xcds;
+        const unsigned loc = blockIdx.x / nx, xcd = blockIdx.x - loc * nx;
+        const unsigned full = total / nx, rem = total - full * nx;
+        tile = (int)(xcd * full + (xcd < rem ? xcd : rem) + loc);
     }
     const int mt = tile % g.mtiles, nt = tile / g.mtiles;
     const int m0 = mt * BM, p0 = nt * kPixTile;
@@ -493,6 +503,7 @@ int launch(const float *src, const float *w, const float *bias, float *dst, int6
     // the tiles of a short last round go out as runs of channel slabs (when the workspace has room for their sums)
     const int64_t n_wg = odl::ceil_div(g.pixels, kPixTile) * g.mtiles;
     const TailPlan tp = plan_tail(n_wg, g.Cin / kSlab, bm, ch_minor, lds);
+    g.xcds = odl::chip().xcds;
     g.main_blocks = (int)n_wg, g.tail_first = (int)n_wg, g.tail_pieces = 0, g.slabs_per_piece = 0, g.tail_ws = nullptr;
     if (tp.pieces > 0 && workspace_bytes >= need + tp.bytes)
     {

@@ -974,16 +974,37 @@ int pick_splits(int64_t M, int64_t N, int64_t K, int requested)
     return s < 1 ? 1 : (int)s;
 }
 
-// A long K walked by few 64x64 tiles (one workgroup per CU, nothing to overlap with): a 32-wide K slab halves the number
-// of barrier-and-refill bubbles per tile (1024^3: 34 -> 31 us). 16-byte loads only, one K slice.
-template <int EPI>
-int launch_small_tile_wide_slab(bool ta, bool tb, GemmArgs g, hipStream_t st)
+// K slices for 64x64 tiles read with 16-byte loads: about one workgroup of eight waves per compute unit, each slice at
+// least 8 slabs of 32 long. 0: the product does not suit that variant.
+int pick_splits_two_sets(int64_t tiles, int64_t K)
 {
-    g.splits = 1;
+    const int64_t cus = odl::device_cus();
+    if (tiles > lone_workgroup_limit() || K < 256)
+        return 0;
+    // cost of s slices in slab times: rounds of workgroups over the compute units, each walking its slabs plus about
+    // four slab times of prologue and epilogue, plus the fold's share, which grows with the slices
+    const int64_t slabs = odl::ceil_div(K, 32);
+    int64_t best = 1, best_cost = 0;
+    for (int64_t s = 1; s <= 128 && (s == 1 || K / s >= 256); ++s)
+    {
+        const int64_t cost = 4 * odl::ceil_div(tiles * s, cus) * (odl::ceil_div(slabs, s) + 4) + s;
+        if (s == 1 || cost < best_cost)
+            best = s, best_cost = cost;
+    }
+    // whole slabs per slice, and no empty slice
+    return (int)odl::ceil_div(slabs, odl::ceil_div(slabs, best));
+}
+
+// A long K walked by few 64x64 tiles (one workgroup per CU, nothing to overlap with): a 32-wide K slab halves the number
+// of barrier-and-refill bubbles per tile (1024^3: 34 -> 31 us). 16-byte loads only.
+template <int EPI>
+int launch_small_tile_wide_slab(bool ta, bool tb, GemmArgs g, int splits, hipStream_t st)
+{
+    g.splits = splits;
     g.main_blocks = 0, g.tail_first = g.tiles_m * g.tiles_n, g.tail_splits = 0, g.tail_kps = 0, g.tail_ws = nullptr;
     g.xcds = odl::chip().xcds;
-    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n)), block(kThreads);
-    const bool two_sets = (int64_t)g.tiles_m * g.tiles_n <= lone_workgroup_limit();
+    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n * splits)), block(kThreads);
+    const bool two_sets = (int64_t)g.tiles_m * g.tiles_n * splits <= lone_workgroup_limit();
 #define ODL_WIDE_CASE(TA, TB)                                                                                  \
     if (ta == TA && tb == TB)                                                                                  \
     {                                                                                                          \
@@ -1009,8 +1030,9 @@ int launch_any_tile(int tile, bool ta, bool tb, bool vec, const GemmArgs &g, int
     if (tile == 128)
         return launch_tile<128, 128, kBK, EPI>(ta, tb, vec, g, splits, tail_ws, tail_bytes, st);
     if constexpr (EPI != EPI_NCHW_ROWB)
-        if (vec && splits == 1 && g.K >= 1024 && g.K % 32 == 0)
-            return launch_small_tile_wide_slab<EPI>(ta, tb, g, st);
+        if (vec && ((splits == 1 && g.K >= 1024 && g.K % 32 == 0) ||
+                    splits == pick_splits_two_sets((int64_t)g.tiles_m * g.tiles_n, g.K)))
+            return launch_small_tile_wide_slab<EPI>(ta, tb, g, splits, st);
     return launch_tile<64, 64, kBK, EPI>(ta, tb, vec, g, splits, nullptr, 0, st);
 }
 }  // namespace
@@ -1042,6 +1064,12 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
                      ldb % 4 == 0 && (trans_a ? M : K) % 4 == 0 && (trans_b ? K : N) % 4 == 0;
 
     int splits = (epi == EPI_NCHW_ROWB) ? 1 : pick_splits(M, N, K, split_k);
+    if (epi != EPI_NCHW_ROWB && split_k < 1 && tile == 64 && vec)
+    {
+        const int s2 = pick_splits_two_sets((int64_t)g.tiles_m * g.tiles_n, K);
+        if (s2 > 0 && s2 <= splits)  // never more slices than the workspace query promised room for
+            splits = s2;
+    }
     const int64_t kt = ceil_div(K > 0 ? K : 1, kBK);
     if (splits > kt)
         splits = (int)kt;
@@ -1056,7 +1084,9 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
             splits = 1;  // automatic choice falls back to a single pass
         }
     }
-    g.k_per_split    = ceil_div(kt, splits) * kBK;
+    const bool slab32 = epi != EPI_NCHW_ROWB && tile == 64 && vec && splits > 1 &&
+                        splits == pick_splits_two_sets((int64_t)g.tiles_m * g.tiles_n, K);
+    g.k_per_split    = slab32 ? ceil_div(ceil_div(K, 32), splits) * 32 : ceil_div(kt, splits) * kBK;
     g.c_split_stride = 0;
     int rc;
     if (splits > 1)
