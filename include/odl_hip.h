@@ -69,6 +69,10 @@ int odl_hip_memset(void *dst, int value, size_t bytes, void *stream);
 int odl_hip_stream_create(void **stream);
 int odl_hip_stream_destroy(void *stream);
 int odl_hip_stream_synchronize(void *stream);
+int odl_hip_device_synchronize(void); /* every stream of the current device */
+/* pinned host memory that kernels can write (hipHostMalloc): for the few words a caller polls after a synchronise */
+int odl_hip_host_alloc(void **ptr, size_t bytes);
+int odl_hip_host_free(void *ptr);
 int odl_hip_graph_capture_begin(void *stream);
 int odl_hip_graph_capture_end(void *stream, void **graph_exec);
 /* gives up a capture (after an error in the middle of the step being recorded): the stream leaves capture mode,
@@ -90,6 +94,12 @@ int odl_hip_sgemm(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, con
                   const float *B, int64_t ldb, float *C, int64_t ldc, const float *bias, int split_k,
                   void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_sgemm_workspace_bytes(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, int split_k);
+/* Linear::forward (src/nn/layers/linear.cpp:80-106) with the activation that follows it applied in the product's epilogue:
+ * y[M,N] = act(x[M,K] . w[K,N] + b[N]), activation -1 none, 0 relu, 7 silu (the odl_hip_unary operator numbers).
+ * Bit-identical to odl_hip_sgemm with a bias followed by odl_hip_unary; the reference runs Linear and ReLU as separate
+ * modules (tests/example/mnist/mlp_mnist.cpp). Workspace: odl_hip_sgemm_workspace_bytes(0, 0, M, N, K, 0). */
+int odl_hip_linear_act(const float *x, const float *w, const float *b, int64_t M, int64_t N, int64_t K, int activation,
+                       float *y, void *workspace, size_t workspace_bytes, void *stream);
 
 /* Mat::matmul — 2-D x 2-D (batch = 1), 3-D x 2-D (b_is_batched = 0), 3-D x 3-D (b_is_batched = 1);
  * src/mat/origin/cpu/math/matmul.cpp:113-218. The workspace (may be NULL) lets small products be split along K
@@ -216,9 +226,12 @@ int odl_hip_softmax_ce_grad(const float *x, const void *t, int idx_is_i64, int64
 /* The same two without a host round trip, for callers that record the step into a graph: the loss goes to
  * device_loss2[0] (float) and the out-of-range-label flag to device_loss2[1] (int, nonzero = a bad label; the caller
  * decides when to look at it), and the upstream gradient is read from device memory (device_gy[0]). Same kernels,
- * same arithmetic: gy / N is formed in the kernel as the host forms it. */
+ * same arithmetic: gy / N is formed in the kernel as the host forms it. host_mirror2 (may be NULL): 8 bytes of pinned
+ * host memory from odl_hip_host_alloc that the loss kernel fills with the same two words, so that a caller who has
+ * synchronised the stream reads them without queueing a copy. */
 int odl_hip_softmax_ce_loss_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
-                                   float *device_loss2, void *workspace, size_t workspace_bytes, void *stream);
+                                   float *device_loss2, void *host_mirror2, void *workspace, size_t workspace_bytes,
+                                   void *stream);
 int odl_hip_softmax_ce_grad_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
                                    const float *device_gy, float *gx, void *stream);
 

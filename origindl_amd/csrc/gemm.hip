@@ -75,7 +75,7 @@ struct GemmArgs
     int64_t k_per_split;     // K range of one grid.y slice (multiple of BK)
     int64_t c_split_stride;  // elements between the partial outputs of consecutive slices (0 = none)
     int64_t P;               // EPI_NCHW_ROWB: OH*OW
-    int act;                 // EPI_NCHW_ROWB: activation applied after the bias (0 none, 1 relu, 2 silu)
+    int act;                 // EPI_NCHW_ROWB, EPI_BIAS_COL: activation applied after the bias (0 none, 1 relu, 2 silu)
     int tiles_m, tiles_n;
     int splits;              // K slices (grid = tiles_m * tiles_n * splits workgroups)
     int xcds;                // XCDs of the device: consecutive workgroup ids are dealt round-robin over them
@@ -667,7 +667,7 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
                 else
                 {
                     if (EPI == EPI_BIAS_COL)
-                        v = v + bcol;
+                        v = apply_act(v + bcol, g.act);
                     Cout[row * g.ldc + col] = v;
                 }
             }
@@ -710,7 +710,7 @@ __global__ __launch_bounds__(64 * kRedGroups) void splitk_reduce_kernel(const fl
         else
         {
             if (bias)
-                s = s + bias[c];
+                s = apply_act(s + bias[c], act);
             out[r * ldc + c] = s;
         }
     }
@@ -749,7 +749,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_vec_kernel(const float *__r
         if (bias)
         {
             const f32x4 b = *reinterpret_cast<const f32x4 *>(bias + c);
-            acc[0] = acc[0] + b[0], acc[1] = acc[1] + b[1], acc[2] = acc[2] + b[2], acc[3] = acc[3] + b[3];
+            acc[0] = apply_act(acc[0] + b[0], act), acc[1] = apply_act(acc[1] + b[1], act);
+            acc[2] = apply_act(acc[2] + b[2], act), acc[3] = apply_act(acc[3] + b[3], act);
         }
         *reinterpret_cast<f32x4 *>(out + r * ldc + c) = acc;
     }
@@ -810,7 +811,7 @@ __global__ __launch_bounds__(256) void tail_fixup_kernel(GemmArgs g, int BM, int
         else
         {
             if (epi == EPI_BIAS_COL && g.bias)
-                v = v + g.bias[col];
+                v = apply_act(v + g.bias[col], g.act);
             g.C[row * g.ldc + col] = v;
         }
     }
@@ -1098,7 +1099,7 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
             return fail(rc, "sgemm: no kernel variant");
         ODL_LAUNCH_CHECK();
         launch_splitk_reduce(static_cast<const float *>(workspace), splits, M * N, C, M, N, ldc,
-                             epi == EPI_BIAS_COL ? bias : nullptr, 0, st);
+                             epi == EPI_BIAS_COL ? bias : nullptr, 0, st, epi == EPI_BIAS_COL && bias ? act : 0);
         ODL_LAUNCH_CHECK();
         return ODL_OK;
     }
@@ -1455,6 +1456,18 @@ int odl_hip_sgemm(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, con
     ODL_REQUIRE_DEVICE();
     return odl::sgemm_launch(trans_a, trans_b, M, N, K, A, lda, B, ldb, C, ldc, bias, bias ? EPI_BIAS_COL : EPI_PLAIN,
                              0, split_k, workspace, workspace_bytes, odl::as_stream(stream));
+}
+
+int odl_hip_linear_act(const float *x, const float *w, const float *b, int64_t M, int64_t N, int64_t K, int activation,
+                       float *y, void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(b != nullptr, "linear: null bias");
+    ODL_REQUIRE(activation == -1 || activation == 0 || activation == 7,
+                "linear: activation must be -1 (none), 0 (relu) or 7 (silu), the unary operator numbers; got %d", activation);
+    const int act = activation == 0 ? 1 : (activation == 7 ? 2 : 0);
+    return odl::sgemm_launch(0, 0, M, N, K, x, K, w, N, y, N, b, EPI_BIAS_COL, 0, 0, workspace, workspace_bytes,
+                             odl::as_stream(stream), act);
 }
 
 size_t odl_hip_sgemm_workspace_bytes(int, int, int64_t M, int64_t N, int64_t K, int split_k)

@@ -131,7 +131,8 @@ __global__ void ce_row_logp_kernel(const float *__restrict__ x, const void *t, i
 }
 
 // out[0] = -(sum of logp) / N   (softmax_cross_entropy.cpp:67-70); one workgroup
-__global__ void ce_finish_kernel(const float *__restrict__ logp, int64_t N, float *out)
+// mirror (may be null): pinned host memory that receives the loss word and the flag word behind it as well
+__global__ void ce_finish_kernel(const float *__restrict__ logp, int64_t N, float *out, unsigned int *mirror)
 {
     __shared__ float part[1024 / 64];
     float acc = 0.f;
@@ -146,7 +147,13 @@ __global__ void ce_finish_kernel(const float *__restrict__ logp, int64_t N, floa
         float s = 0.f;
         for (unsigned i = 0; i < blockDim.x / 64; ++i)
             s += part[i];
-        out[0] = -s / (float)N;
+        const float loss = -s / (float)N;
+        out[0] = loss;
+        if (mirror)
+        {
+            mirror[0] = __float_as_uint(loss);
+            mirror[1] = reinterpret_cast<const unsigned int *>(out)[1];  // set by the kernel that ran before this one
+        }
     }
 }
 
@@ -155,7 +162,7 @@ __global__ void ce_finish_kernel(const float *__restrict__ logp, int64_t N, floa
 // reference's loops take them (src/operators/loss/softmax_cross_entropy.cpp:30-70) — then the block sum of ce_finish_kernel.
 // Writes both words: out2[0] = loss, out2[1] = 1 when a label is out of range.
 __global__ __launch_bounds__(1024) void ce_loss_small_kernel(const float *__restrict__ x, const void *t, int is64, int N,
-                                                             int C, unsigned int *out2)
+                                                             int C, unsigned int *out2, unsigned int *mirror)
 {
     __shared__ float part[1024 / 64];
     __shared__ int bad;
@@ -193,6 +200,8 @@ __global__ __launch_bounds__(1024) void ce_loss_small_kernel(const float *__rest
         const float loss = -s / (float)N;
         out2[0] = __float_as_uint(loss);
         out2[1] = bad ? 1u : 0u;
+        if (mirror)
+            mirror[0] = __float_as_uint(loss), mirror[1] = bad ? 1u : 0u;
     }
 }
 
@@ -429,7 +438,7 @@ size_t odl_hip_softmax_ce_loss_workspace_bytes(int64_t N)
 
 // loss and out-of-range flag into two device words: [0] loss (float), [1] flag (int, nonzero = a bad label)
 static int ce_loss_launch(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, unsigned int *out2,
-                          void *workspace, size_t workspace_bytes, hipStream_t st)
+                          unsigned int *mirror, void *workspace, size_t workspace_bytes, hipStream_t st)
 {
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(N > 0 && C > 0, "softmax_cross_entropy: empty input");
@@ -438,7 +447,8 @@ static int ce_loss_launch(const float *x, const void *t, int idx_is_i64, int64_t
                 "softmax_cross_entropy: workspace of %zu bytes required, got %zu", need, workspace_bytes);
     if (N <= 2048 && C <= 64)
     {
-        hipLaunchKernelGGL(ce_loss_small_kernel, dim3(1), dim3(1024), 0, st, x, t, idx_is_i64, (int)N, (int)C, out2);
+        hipLaunchKernelGGL(ce_loss_small_kernel, dim3(1), dim3(1024), 0, st, x, t, idx_is_i64, (int)N, (int)C, out2,
+                           mirror);
         ODL_LAUNCH_CHECK();
         return ODL_OK;
     }
@@ -448,16 +458,19 @@ static int ce_loss_launch(const float *x, const void *t, int idx_is_i64, int64_t
     hipLaunchKernelGGL(ce_row_logp_kernel, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, st, x, t,
                        idx_is_i64, N, C, logp, reinterpret_cast<int *>(out2 + 1));
     ODL_LAUNCH_CHECK();
-    hipLaunchKernelGGL(ce_finish_kernel, dim3(1), dim3(1024), 0, st, logp, N, reinterpret_cast<float *>(out2));
+    hipLaunchKernelGGL(ce_finish_kernel, dim3(1), dim3(1024), 0, st, logp, N, reinterpret_cast<float *>(out2),
+                       mirror);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
 
 int odl_hip_softmax_ce_loss_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
-                                   float *device_loss2, void *workspace, size_t workspace_bytes, void *stream)
+                                   float *device_loss2, void *host_mirror2, void *workspace, size_t workspace_bytes,
+                                   void *stream)
 {
     ODL_REQUIRE(device_loss2 != nullptr, "softmax_cross_entropy: null output");
-    return ce_loss_launch(x, t, idx_is_i64, N, C, reinterpret_cast<unsigned int *>(device_loss2), workspace,
+    return ce_loss_launch(x, t, idx_is_i64, N, C, reinterpret_cast<unsigned int *>(device_loss2),
+                          static_cast<unsigned int *>(host_mirror2), workspace,
                           workspace_bytes, odl::as_stream(stream));
 }
 
@@ -471,7 +484,7 @@ int odl_hip_softmax_ce_loss(const float *x, const void *t, int idx_is_i64, int64
                 "softmax_cross_entropy: workspace of %zu bytes required, got %zu", need, workspace_bytes);
     // tail of the workspace: [0] loss (float), [1] out-of-range flag (int)
     unsigned int *tail = reinterpret_cast<unsigned int *>(static_cast<char *>(workspace) + need - 256);
-    const int rc = ce_loss_launch(x, t, idx_is_i64, N, C, tail, workspace, workspace_bytes, st);
+    const int rc = ce_loss_launch(x, t, idx_is_i64, N, C, tail, nullptr, workspace, workspace_bytes, st);
     if (rc != ODL_OK)
         return rc;
     unsigned int host_tail[2] = {0, 0};

@@ -221,6 +221,27 @@ int odl_hip_stream_destroy(void *stream)
     return ODL_OK;
 }
 
+int odl_hip_device_synchronize(void)
+{
+    ODL_HIP_CHECK(hipDeviceSynchronize());
+    return ODL_OK;
+}
+
+int odl_hip_host_alloc(void **ptr, size_t bytes)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(ptr != nullptr && bytes > 0, "host_alloc: null result pointer or zero size");
+    ODL_HIP_CHECK(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+    return ODL_OK;
+}
+
+int odl_hip_host_free(void *ptr)
+{
+    if (ptr)
+        ODL_HIP_CHECK(hipHostFree(ptr));
+    return ODL_OK;
+}
+
 int odl_hip_stream_synchronize(void *stream)
 {
     ODL_HIP_CHECK(hipStreamSynchronize(odl::as_stream(stream)));

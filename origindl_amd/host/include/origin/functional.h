@@ -102,6 +102,9 @@ std::vector<Tensor> batch_norm_outputs(const Tensor &x, const Tensor &gamma, con
                                        float momentum, int num_dims);
 // x[M,K] . w[K,N] + b (b of N elements) in one kernel; what nn::Linear::forward uses for 2-D inputs
 Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b);
+// relu(linear(x, w, b)) and relu(conv2d(x, W, b)) as one operator each, for device tensors (float32)
+Tensor linear_relu(const Tensor &x, const Tensor &w, const Tensor &b);
+Tensor conv2d_relu(const Tensor &x, const Tensor &W, const Tensor *b, std::pair<int, int> stride, std::pair<int, int> pad);
 Tensor softmax(const Tensor &x, int axis = -1);
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &target);
 // After replaying a recorded step on new labels: whether the loss kernel met an out-of-range label (the ordinary call

@@ -33,6 +33,7 @@ public:
     void *data() const
     {
         host_copy_valid_ = false;
+        mirror_valid_    = false;
         return data_;
     }
     size_t size() const { return size_; }
@@ -55,6 +56,16 @@ public:
         std::memcpy(dst, host_copy_, n);
         return true;
     }
+    // Pinned host words that the kernel which fills this buffer also writes (the loss and its bad-label flag): once the
+    // device has been synchronised the host reads them there, with no copy queued. Set after the data() call that handed
+    // the buffer to that kernel; like the host copy above it stops being trusted at the next data() call. A kernel
+    // recorded into a graph keeps writing the words on every replay, so they are never given back (`recorded`).
+    void set_mirror(void *pinned_words, bool recorded) const
+    {
+        mirror_ = pinned_words, mirror_recorded_ = recorded, mirror_valid_ = pinned_words != nullptr;
+    }
+    // the device is synchronised and `n` bytes are read from the mirror; false when there is none to trust
+    bool read_mirror(void *dst, size_t n) const;
     DeviceType device_type() const { return type_; }
     int device_index() const { return index_; }
     std::shared_ptr<Storage> to_device(DeviceType type, int index) const;  // synchronous copy, like the reference
@@ -68,6 +79,8 @@ private:
     mutable bool host_copy_valid_ = false;
     mutable size_t host_copy_bytes_ = 0;
     mutable unsigned char host_copy_[8] = {0};
+    mutable void *mirror_ = nullptr;
+    mutable bool mirror_valid_ = false, mirror_recorded_ = false;
 };
 
 class Mat
@@ -349,6 +362,8 @@ public:
                                                                  const Mat &saved_var, float eps, int num_dims) const;
     // gy (this) times the mask x > 0, in one launch: the two kernels of ReLU::backward, same products
     std::unique_ptr<Mat> relu_backward(const Mat &x) const;
+    // x . W + b with the activation applied in the product's epilogue (-1 none, 0 relu): what linear() then relu() give
+    std::unique_ptr<Mat> linear_act(const Mat &W, const Mat &b, int activation) const;
     // x (this) . W + b with the bias added in the product's epilogue: the three kernels of Linear::forward
     // (matmul, broadcast_to, add), same rounding (the sum is rounded to float before the bias is added)
     std::unique_ptr<Mat> linear(const Mat &W, const Mat &b) const;

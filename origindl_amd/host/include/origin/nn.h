@@ -69,6 +69,8 @@ class Linear : public Module
 public:
     Linear(int in_features, int out_features, bool bias = true);
     Tensor forward(const Tensor &input) override;
+    // relu(forward(input)); Sequential calls it for a Linear that a ReLU follows, and on the device the two run as one
+    Tensor forward_relu(const Tensor &input);
     Parameter *weight() { return &weight_; }
     Parameter *bias() { return use_bias_ ? &bias_ : nullptr; }
     void reset_parameters();
@@ -87,6 +89,7 @@ public:
            std::pair<int, int> pad = {0, 0}, bool bias = true);
     Conv2d(int in_channels, int out_channels, int kernel_size, int stride = 1, int pad = 0, bool bias = true);
     Tensor forward(const Tensor &input) override;
+    Tensor forward_relu(const Tensor &input);  // relu(forward(input)), as Linear::forward_relu
     Parameter *weight() { return &weight_; }
     Parameter *bias() { return use_bias_ ? &bias_ : nullptr; }
 

@@ -291,6 +291,27 @@ struct FusedLinear : Operator
     }
 };
 
+// A layer followed by ReLU as one operator (Sequential pairs them up): the activation runs in the layer's epilogue, so the
+// pre-activation tensor is never written, and backward first masks the incoming gradient with (y > 0) — the same
+// elements as the (x > 0) of ReLU's own backward (src/operators/activation/relu.cpp), since y = max(x, 0) — and then
+// does what the layer's backward does. The values are those of the two operators run one after the other.
+struct FusedLinearRelu : Operator
+{
+    std::shared_ptr<Mat> y;  // the output's data (not its tensor: that would own this operator in turn)
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        Tensor out = wrap(omat(xs[0]).linear_act(mat(xs[1]), mat(xs[2]), 0));
+        y = out.impl_->data_;
+        return {out};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        auto g0 = omat(gys[0]).relu_backward(*y);
+        auto g  = OriginMat::matmul_backward_2d(mat(inputs_[0]), mat(inputs_[1]), *g0);
+        return {wrap(std::move(g.first)), wrap(std::move(g.second)), wrap(g0->sum_to(inputs_[2].shape()))};
+    }
+};
+
 // src/operators/activation/leaky_relu.cpp:17-72. Forward from the operations at hand, exact in both branches:
 // r = relu(x); y = r + alpha*(x - r) — where x > 0 that is x + alpha*0, elsewhere 0 + alpha*x. Backward as there:
 // gy * (alpha + mask*(1-alpha)) with mask = (x > 0).
@@ -393,7 +414,7 @@ struct Conv2dOp : Operator  // src/operators/conv/conv2d.cpp:14-89
 {
     std::pair<int, int> stride, pad;
     Conv2dOp(std::pair<int, int> s, std::pair<int, int> p) : stride(s), pad(p) {}
-    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    static void validate(const std::vector<Tensor> &xs)
     {
         if (xs.size() < 2 || xs.size() > 3)
             THROW_RUNTIME_ERROR("Conv2d operator requires 2 or 3 inputs (x, W, [b]), but got {}", xs.size());
@@ -405,6 +426,10 @@ struct Conv2dOp : Operator  // src/operators/conv/conv2d.cpp:14-89
         if (xs[0].shape()[1] != xs[1].shape()[1])
             THROW_RUNTIME_ERROR("Conv2d forward: channel mismatch - x has {} channels, but W expects {} channels",
                                 xs[0].shape()[1], xs[1].shape()[1]);
+    }
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        validate(xs);
         const Mat *b = xs.size() == 3 ? &mat(xs[2]) : nullptr;
         return {wrap(mat(xs[0]).conv2d(mat(xs[1]), b, stride, pad))};
     }
@@ -413,6 +438,31 @@ struct Conv2dOp : Operator  // src/operators/conv/conv2d.cpp:14-89
         const Mat &gy = mat(gys[0]);
         const Mat *b  = inputs_.size() == 3 ? &mat(inputs_[2]) : nullptr;
         auto grads    = gy.conv2d_backward(gy, mat(inputs_[0]), mat(inputs_[1]), b, stride, pad);
+        std::vector<Tensor> out;
+        for (auto &g : grads)
+            out.push_back(wrap(std::move(g)));
+        return out;
+    }
+};
+
+// Conv2d followed by ReLU as one operator, as FusedLinearRelu above
+struct Conv2dReluOp : Conv2dOp
+{
+    std::shared_ptr<Mat> y;
+    using Conv2dOp::Conv2dOp;
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        validate(xs);
+        const Mat *b = xs.size() == 3 ? &mat(xs[2]) : nullptr;
+        Tensor out   = wrap(omat(xs[0]).conv2d_act(mat(xs[1]), b, stride, pad, 0));
+        y            = out.impl_->data_;
+        return {out};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        auto g0 = omat(gys[0]).relu_backward(*y);
+        const Mat *b  = inputs_.size() == 3 ? &mat(inputs_[2]) : nullptr;
+        auto grads    = g0->conv2d_backward(*g0, mat(inputs_[0]), mat(inputs_[1]), b, stride, pad);
         std::vector<Tensor> out;
         for (auto &g : grads)
             out.push_back(wrap(std::move(g)));
@@ -751,6 +801,14 @@ Tensor batch_norm(const Tensor &x, const Tensor &gamma, const Tensor &beta, cons
     return batch_norm_outputs(x, gamma, beta, rm, rv, training, eps, momentum, num_dims)[0];
 }
 Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b) { return apply<FusedLinear>({x, w, b}); }
+Tensor linear_relu(const Tensor &x, const Tensor &w, const Tensor &b) { return apply<FusedLinearRelu>({x, w, b}); }
+Tensor conv2d_relu(const Tensor &x, const Tensor &W, const Tensor *b, std::pair<int, int> stride, std::pair<int, int> pad)
+{
+    std::vector<Tensor> in{x, W};
+    if (b)
+        in.push_back(*b);
+    return apply<Conv2dReluOp>(in, stride, pad);
+}
 Tensor softmax(const Tensor &x, int axis) { return apply<Softmax>({x}, axis); }
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &t) { return apply<SoftmaxCrossEntropy>({x, t}); }
 bool softmax_cross_entropy_bad_label(const Tensor &loss) { return SoftmaxCrossEntropy::bad_label(loss); }

@@ -358,8 +358,53 @@ std::shared_ptr<Storage> Storage::create(size_t bytes, DeviceType type, int inde
     return std::shared_ptr<Storage>(new Storage(p, bytes, cap, type, index));
 }
 
+// 16-byte slots of pinned host memory, carved from 4 KiB pieces that live as long as the process
+class MirrorPool
+{
+public:
+    static MirrorPool &get()
+    {
+        static MirrorPool *pool = new MirrorPool();
+        return *pool;
+    }
+    void *take()
+    {
+        std::lock_guard<std::mutex> lock(mutex_);
+        if (free_.empty())
+        {
+            void *piece = nullptr;
+            check(odl_hip_host_alloc(&piece, 4096));
+            for (size_t off = 0; off < 4096; off += 16)
+                free_.push_back(static_cast<char *>(piece) + off);
+        }
+        void *slot = free_.back();
+        free_.pop_back();
+        return slot;
+    }
+    void give(void *slot)
+    {
+        std::lock_guard<std::mutex> lock(mutex_);
+        free_.push_back(slot);
+    }
+
+private:
+    std::mutex mutex_;
+    std::vector<void *> free_;
+};
+
+bool Storage::read_mirror(void *dst, size_t n) const
+{
+    if (!mirror_valid_ || n > 8)
+        return false;
+    check(odl_hip_device_synchronize());
+    std::memcpy(dst, mirror_, n);
+    return true;
+}
+
 Storage::~Storage()
 {
+    if (mirror_ && !mirror_recorded_)
+        MirrorPool::get().give(mirror_);
     if (!data_)
         return;
     if (type_ == DeviceType::kCPU)
@@ -569,7 +614,8 @@ std::vector<double> OriginMat::to_doubles() const
     if (storage_->device_type() != DeviceType::kCPU && n == 1)
     {
         host.resize(dtype_size(dtype_));
-        if (storage_->host_copy(host.data(), host.size()))  // a scalar that has been read back already
+        // a scalar that has been read back already, or one whose kernel also wrote it to pinned host memory
+        if (storage_->host_copy(host.data(), host.size()) || (!t_capturing && storage_->read_mirror(host.data(), host.size())))
             src = host.data();
     }
     if (!src)
@@ -913,6 +959,11 @@ std::unique_ptr<Mat> OriginMat::relu_backward(const Mat &x) const
 
 std::unique_ptr<Mat> OriginMat::linear(const Mat &W_, const Mat &b_) const
 {
+    return linear_act(W_, b_, -1);
+}
+
+std::unique_ptr<Mat> OriginMat::linear_act(const Mat &W_, const Mat &b_, int activation) const
+{
     const OriginMat &x = dev_f32(*this, "linear"), &W = dev_f32(W_, "linear"), &b = dev_f32(b_, "linear");
     if (shape_.size() != 2 || W.shape().size() != 2 || shape_[1] != W.shape()[0] || b.elements() != W.shape()[1])
         THROW_INVALID_ARG("linear: x {} . W {} + b {} do not fit", shape_.to_string(), W.shape().to_string(),
@@ -920,7 +971,7 @@ std::unique_ptr<Mat> OriginMat::linear(const Mat &W_, const Mat &b_) const
     const int64_t M = shape_[0], K = shape_[1], N = W.shape()[1];
     auto y = new_like(x, Shape{(size_t)M, (size_t)N});
     Workspace ws(odl_hip_sgemm_workspace_bytes(0, 0, M, N, K, 0), device().index());
-    check(odl_hip_sgemm(0, 0, M, N, K, fp(x), K, fp(W), N, y->data_ptr<float>(), N, fp(b), 0, ws.ptr(), ws.bytes, cur()));
+    check(odl_hip_linear_act(fp(x), fp(W), fp(b), M, N, K, activation, y->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
     return y;
 }
 
@@ -1484,8 +1535,10 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) 
     Workspace ws(odl_hip_softmax_ce_loss_workspace_bytes(N), device().index());
     // two words: the loss, and the bad-label flag behind it; the Mat is the scalar in front
     auto storage = Storage::create(2 * sizeof(float), DeviceType::kCUDA, device().index());
+    void *mirror = MirrorPool::get().take();
     check(odl_hip_softmax_ce_loss_device(fp(x), t.storage()->data(), is64, N, C, static_cast<float *>(storage->data()),
-                                         ws.ptr(), ws.bytes, cur()));
+                                         mirror, ws.ptr(), ws.bytes, cur()));
+    storage->set_mirror(mirror, t_capturing);
     return std::make_unique<OriginMat>(std::move(storage), Shape{}, DataType::kFloat32);
 }
 
@@ -1497,7 +1550,8 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target)
     unsigned words[2] = {0, 0};
     no_capture("device-to-host copy");
     const auto &st = as_origin(*loss).storage();
-    check(odl_hip_memcpy_d2h(words, st->data(), sizeof(words)));
+    if (!st->read_mirror(words, sizeof(words)))
+        check(odl_hip_memcpy_d2h(words, st->data(), sizeof(words)));
     if (words[1] != 0)
         THROW_INVALID_ARG("gather: index out of range [0, {})", shape_[1]);
     st->set_host_copy(words, sizeof(words));  // item() on the loss needs no second trip
@@ -1530,7 +1584,8 @@ bool OriginMat::loss_bad_label_flag() const
         return false;
     unsigned words[2] = {0, 0};
     no_capture("device-to-host copy");
-    check(odl_hip_memcpy_d2h(words, storage_->data(), sizeof(words)));
+    if (!storage_->read_mirror(words, sizeof(words)))
+        check(odl_hip_memcpy_d2h(words, storage_->data(), sizeof(words)));
     return words[1] != 0;
 }
 

@@ -1,6 +1,8 @@
 // Host glue above the operators: modules, layers, optimizers, device API (see origin/nn.h).
 #include "origin/nn.h"
 
+#include <typeinfo>
+
 #include <cmath>
 #include <random>
 
@@ -177,9 +179,29 @@ Tensor BatchNormBase::forward(const Tensor &input)
 
 Tensor Sequential::forward(const Tensor &input)
 {
+    // A Linear or Conv2d that a ReLU follows runs together with it (the tensor between the two is not visible from
+    // outside a Sequential); the values are those of the two modules run in turn.
     Tensor x = input;
-    for (auto &l : layers_)
-        x = l->forward(x);
+    for (size_t i = 0; i < layers_.size(); ++i)
+    {
+        Module &l = *layers_[i];
+        if (i + 1 < layers_.size() && typeid(*layers_[i + 1]) == typeid(nn::ReLU))
+        {
+            if (typeid(l) == typeid(nn::Linear))
+            {
+                x = static_cast<nn::Linear &>(l).forward_relu(x);
+                ++i;
+                continue;
+            }
+            if (typeid(l) == typeid(nn::Conv2d))
+            {
+                x = static_cast<nn::Conv2d &>(l).forward_relu(x);
+                ++i;
+                continue;
+            }
+        }
+        x = l.forward(x);
+    }
     return x;
 }
 
@@ -243,6 +265,14 @@ Tensor Linear::forward(const Tensor &input)
     return output;
 }
 
+Tensor Linear::forward_relu(const Tensor &input)
+{
+    if (weight_.shape().elements() != 0 && use_bias_ && input.shape().size() == 2 &&
+        input.device().type() == DeviceType::kCUDA && input.dtype() == DataType::kFloat32)
+        return functional::linear_relu(input, static_cast<const Tensor &>(weight_), static_cast<const Tensor &>(bias_));
+    return functional::relu(forward(input));
+}
+
 Conv2d::Conv2d(int in_channels, int out_channels, std::pair<int, int> kernel_size, std::pair<int, int> stride,
                std::pair<int, int> pad, bool bias)
     : in_channels_(in_channels), out_channels_(out_channels), kernel_(kernel_size), stride_(stride), pad_(pad),
@@ -282,6 +312,15 @@ Tensor Conv2d::forward(const Tensor &input)
                             input.shape()[1], in_channels_);
     const Tensor *b = use_bias_ ? &static_cast<const Tensor &>(bias_) : nullptr;
     return functional::conv2d(input, static_cast<const Tensor &>(weight_), b, stride_, pad_);
+}
+
+Tensor Conv2d::forward_relu(const Tensor &input)
+{
+    if (input.shape().size() != 4 || input.shape()[1] != (size_t)in_channels_ ||
+        input.device().type() != DeviceType::kCUDA || input.dtype() != DataType::kFloat32)
+        return functional::relu(forward(input));
+    const Tensor *b = use_bias_ ? &static_cast<const Tensor &>(bias_) : nullptr;
+    return functional::conv2d_relu(input, static_cast<const Tensor &>(weight_), b, stride_, pad_);
 }
 
 MaxPool2d::MaxPool2d(std::pair<int, int> kernel_size, std::pair<int, int> stride, std::pair<int, int> pad)

@@ -1108,3 +1108,25 @@ def test_permute_is_numpy_transpose_in_every_element_width(api):
     sh, pm = (ctypes.c_int64 * 2)(3, 4), (ctypes.c_int * 2)(0, 0)
     with pytest.raises(api.OdlInvalidArgument):
         L.call("odl_hip_permute", dx.data_ptr(), 0, sh, 2, pm, out.data_ptr(), None)
+
+
+def test_linear_with_the_activation_in_the_epilogue_equals_linear_then_relu(api):
+    # src/nn/layers/linear.cpp:80-106 followed by src/operators/activation/relu.cpp: the fused entry must give the bits
+    # of the two run in turn, for the single-pass, K-sliced and tail-split schedules of the product
+    L = api.lib()
+    rng = np.random.default_rng(77)
+    for M, K, N in ((512, 784, 1000), (64, 100, 10), (300, 1024, 1024), (1536, 640, 2304), (33, 17, 5)):
+        x, w = dev(rng.standard_normal((M, K), dtype=np.float32)), dev(rng.standard_normal((K, N), dtype=np.float32))
+        b = dev(rng.standard_normal((N,), dtype=np.float32))
+        nb = L.query("odl_hip_sgemm_workspace_bytes", 0, 0, M, N, K, 0)
+        ws = torch.empty(max(nb, 16), dtype=torch.uint8, device="cuda")
+        plain, fused = torch.empty((M, N), device="cuda"), torch.empty((M, N), device="cuda")
+        L.call("odl_hip_sgemm", 0, 0, M, N, K, x.data_ptr(), K, w.data_ptr(), N, plain.data_ptr(), N, b.data_ptr(), 0,
+               ws.data_ptr(), nb, None)
+        for act, f in ((-1, lambda v: v), (0, lambda v: np.maximum(v, np.float32(0)))):
+            L.call("odl_hip_linear_act", x.data_ptr(), w.data_ptr(), b.data_ptr(), M, N, K, act, fused.data_ptr(),
+                   ws.data_ptr(), nb, None)
+            assert np.array_equal(host(fused), f(host(plain))), (M, K, N, act)
+    with pytest.raises(api.OdlInvalidArgument):
+        L.call("odl_hip_linear_act", x.data_ptr(), w.data_ptr(), b.data_ptr(), M, N, K, 3, fused.data_ptr(), ws.data_ptr(),
+               nb, None)
