@@ -22,7 +22,7 @@ constexpr int ORIGIN_BACKEND_TYPE = 0;
 
 // Owning buffer on the host or on the device (device memory comes from a caching pool over odl_hip_malloc,
 // as the reference's Storage sits on its MemoryPool, src/mat/origin/memory/*).
-class Storage
+class Storage : public std::enable_shared_from_this<Storage>
 {
 public:
     static std::shared_ptr<Storage> create(size_t bytes, DeviceType type, int index = 0);
@@ -34,7 +34,22 @@ public:
     {
         host_copy_valid_ = false;
         mirror_valid_    = false;
+        if (fill_pending_)
+            run_pending_fill();
         return data_;
+    }
+    // A device buffer that is to hold one value in all of its `n` elements (zeros, ones, full): the fill kernel is not
+    // queued until the first data() call. Code that only needs to know the value (a gradient seed of ones read as a
+    // scalar, zeros added to zeros) asks pending_fill() and never causes the launch.
+    void set_pending_fill(int dtype_code, int64_t n, const void *element, size_t element_bytes) const;
+    // true while the fill has not run; *dtype_code and the element's bytes (8 at most) are returned when asked for
+    bool pending_fill(int *dtype_code = nullptr, void *element = nullptr) const
+    {
+        if (fill_pending_ && dtype_code)
+            *dtype_code = fill_dtype_;
+        if (fill_pending_ && element)
+            std::memcpy(element, fill_element_, sizeof(fill_element_));
+        return fill_pending_;
     }
     size_t size() const { return size_; }
     // A host copy of the first bytes of a small device buffer, kept by code that has just read them back anyway (the loss
@@ -79,6 +94,11 @@ private:
     mutable bool host_copy_valid_ = false;
     mutable size_t host_copy_bytes_ = 0;
     mutable unsigned char host_copy_[8] = {0};
+    void run_pending_fill() const;
+    mutable bool fill_pending_ = false, fill_set_while_capturing_ = false;
+    mutable int fill_dtype_ = 0;
+    mutable int64_t fill_n_ = 0;
+    mutable unsigned char fill_element_[8] = {0};
     mutable void *mirror_ = nullptr;
     mutable bool mirror_valid_ = false, mirror_recorded_ = false;
 };
@@ -338,6 +358,16 @@ public:
     std::unique_ptr<Mat> softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const;
     // include/origin/mat/origin/origin_mat.h:75: a dense copy with the dimensions in the order `dims`
     std::unique_ptr<Mat> permute(const std::vector<int> &dims) const;
+    // a float32 tensor made by zeros / ones / full whose fill has not been queued yet: its one value, known on the host
+    bool unwritten_constant(float *value) const
+    {
+        int code = -1;
+        unsigned char element[8];
+        if (!storage_ || dtype_ != DataType::kFloat32 || !storage_->pending_fill(&code, element) || code != 0)
+            return false;
+        std::memcpy(value, element, sizeof(float));
+        return true;
+    }
     // on a loss made by softmax_cross_entropy_device / _checked: the out-of-range-label flag that lies behind the loss
     // in device memory, read back now (one small device-to-host copy; synchronises). A recorded step cannot raise the
     // reference's exception for a bad label — it contributes nothing to the loss — so a caller that replays a graph on

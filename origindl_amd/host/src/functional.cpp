@@ -401,7 +401,10 @@ struct SoftmaxCrossEntropy : Operator  // src/operators/loss/softmax_cross_entro
         std::unique_ptr<Mat> gx;
         // the upstream gradient is read where it lies when it is a float32 device scalar (no host round trip; gy/N
         // is formed in the kernel as the host would form it)
-        if (cuda::is_capturing() || (OriginMat::device_f32(mat(gys[0])) && gys[0].elements() == 1))
+        float seed = 0.f;
+        if (gys[0].elements() == 1 && omat(gys[0]).unwritten_constant(&seed))
+            gx = omat(x).softmax_cross_entropy_backward(mat(t), seed);  // the ones backward() starts from: no read at all
+        else if (cuda::is_capturing() || (OriginMat::device_f32(mat(gys[0])) && gys[0].elements() == 1))
             gx = omat(x).softmax_cross_entropy_backward_device(mat(t), mat(gys[0]));
         else
             gx = omat(x).softmax_cross_entropy_backward(mat(t), gys[0].item<float>());

@@ -392,6 +392,49 @@ private:
     std::vector<void *> free_;
 };
 
+// The buffers of this thread whose fill may still be pending. A capture must not record the fill of a buffer that was
+// made before it (a replay would then reset the buffer every time), so begin_capture queues those fills first.
+thread_local std::vector<std::weak_ptr<const Storage>> t_pending_fills;
+
+void Storage::set_pending_fill(int dtype_code, int64_t n, const void *element, size_t element_bytes) const
+{
+    std::memset(fill_element_, 0, sizeof(fill_element_));
+    std::memcpy(fill_element_, element, element_bytes < sizeof(fill_element_) ? element_bytes : sizeof(fill_element_));
+    fill_dtype_ = dtype_code, fill_n_ = n;
+    fill_pending_ = n > 0;
+    if (!fill_pending_ || t_capturing)
+        return;
+    if (t_pending_fills.size() >= 4096)
+    {
+        // drop the entries that are gone or done
+        size_t kept = 0;
+        for (auto &w : t_pending_fills)
+        {
+            auto st = w.lock();
+            if (st && st->pending_fill())
+                t_pending_fills[kept++] = w;
+        }
+        t_pending_fills.resize(kept);
+    }
+    t_pending_fills.push_back(weak_from_this());
+}
+
+void Storage::run_pending_fill() const
+{
+    fill_pending_ = false;
+    check(odl_hip_fill_dtype(data_, fill_dtype_, fill_n_, fill_element_, cur()));
+}
+
+static void run_pending_fills_of_this_thread()
+{
+    std::vector<std::weak_ptr<const Storage>> list;
+    list.swap(t_pending_fills);
+    for (auto &w : list)
+        if (auto st = w.lock())
+            if (st->pending_fill())
+                (void)st->data();
+}
+
 bool Storage::read_mirror(void *dst, size_t n) const
 {
     if (!mirror_valid_ || n > 8)
@@ -418,6 +461,8 @@ std::shared_ptr<Storage> Storage::to_device(DeviceType type, int index) const
     auto dst = Storage::create(size_, type, index);
     if (size_ == 0)
         return dst;
+    if (fill_pending_)
+        run_pending_fill();
     if (type_ == DeviceType::kCPU && type == DeviceType::kCPU)
         std::memcpy(dst->data(), data_, size_);
     else if (type_ == DeviceType::kCPU)
@@ -518,7 +563,7 @@ std::unique_ptr<Mat> OriginMat::from_scalar(const Scalar &scalar, const Shape &s
         // one element converted on the host the way the host path below converts all of them, then a fill kernel
         auto m = std::make_unique<OriginMat>(shape, options.dtype(), options.device());
         const double v = scalar.to_float64();
-        char element[8];
+        char element[8] = {0};
         if (options.dtype() == DataType::kInt64)
         {
             const int64_t w = scalar.to_int64();
@@ -526,7 +571,8 @@ std::unique_ptr<Mat> OriginMat::from_scalar(const Scalar &scalar, const Shape &s
         }
         else
             store_as(element, options.dtype(), &v, 1);
-        check(odl_hip_fill_dtype(m->storage()->data(), code(options.dtype()), (int64_t)n, element, cur()));
+        // the kernel is queued when the buffer is first asked for
+        m->storage()->set_pending_fill(code(options.dtype()), (int64_t)n, element, dtype_size(options.dtype()));
         return m;
     }
     std::vector<double> tmp(n, scalar.to_float64());
@@ -761,7 +807,21 @@ std::unique_ptr<Mat> OriginMat::operator<=(const Mat &o) const { return binary(8
 std::unique_ptr<Mat> OriginMat::operator>=(const Mat &o) const { return binary(9, "ge", *this, o); }
 std::unique_ptr<Mat> OriginMat::operator-() const { return unary(3, "negate", *this); }
 
-void OriginMat::add_inplace(const Mat &o) { binary(0, "add", *this, o, this); }
+void OriginMat::add_inplace(const Mat &o)
+{
+    // zeros that have not been written yet, added to zeros that have not been written yet, are just that
+    if (const auto *other = dynamic_cast<const OriginMat *>(&o))
+    {
+        int ca = 0, cb = 0;
+        unsigned char ea[8], eb[8];
+        const unsigned char none[8] = {0};
+        if (storage_ && other->storage_ && shape_ == other->shape_ && dtype_ == other->dtype_ &&
+            storage_->pending_fill(&ca, ea) && other->storage_->pending_fill(&cb, eb) && ca == cb &&
+            std::memcmp(ea, none, 8) == 0 && std::memcmp(eb, none, 8) == 0)
+            return;
+    }
+    binary(0, "add", *this, o, this);
+}
 void OriginMat::sub_inplace(const Mat &o) { binary(1, "subtract", *this, o, this); }
 void OriginMat::mul_inplace(const Mat &o) { binary(2, "multiply", *this, o, this); }
 void OriginMat::div_inplace(const Mat &o) { binary(3, "divide", *this, o, this); }
@@ -1850,6 +1910,7 @@ void Graph::begin_capture()
         THROW_RUNTIME_ERROR("this graph has been captured already");
     if (!t_stream)
         THROW_RUNTIME_ERROR("graph capture needs a created stream (cuda::set_stream): the null stream cannot be captured");
+    run_pending_fills_of_this_thread();
     check(odl_hip_stream_synchronize(t_stream));
     arena_ = DevicePool::get().begin_capture();
     if (odl_hip_graph_capture_begin(t_stream) != ODL_OK)

@@ -1063,8 +1063,11 @@ void timed_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T, int s
     model.train();
     auto one = [&] {
         opt.zero_grad();
-        auto y = model(X);
-        auto L = F::softmax_cross_entropy(y, T);
+        // a new handle on the batch every step, as a data loader hands out new tensors (mlp_mnist.cpp's loop): the
+        // gradients the step leaves on its inputs are assigned, not accumulated over the steps
+        const Tensor x = X.detach(), t = T.detach();
+        auto y = model(x);
+        auto L = F::softmax_cross_entropy(y, t);
         L.backward();
         opt.step();
         return L.template item<float>();
@@ -1101,7 +1104,7 @@ void timed_graph_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T,
     for (int i = 0; i < (warmup > 2 ? warmup : 2); ++i)
     {
         opt.zero_grad();
-        auto L = F::softmax_cross_entropy(model(X), T);
+        auto L = F::softmax_cross_entropy(model(X.detach()), T.detach());  // new handles on the batch, as in timed_steps
         L.backward();
         opt.step();
         *loss = L.template item<float>();
@@ -1110,7 +1113,7 @@ void timed_graph_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T,
     Tensor L;
     graph.begin_capture();
     opt.zero_grad();
-    L = F::softmax_cross_entropy(model(X), T);
+    L = F::softmax_cross_entropy(model(X.detach()), T.detach());
     L.backward();
     opt.step();
     graph.end_capture();
@@ -1223,6 +1226,61 @@ int cnn_bench_impl(int64_t N, int steps, int warmup, int graph_mode, float *ms_p
 }  // namespace
 
 extern "C" {
+#ifdef DRV_ON_DEVICE
+// zeros / ones / full on the device queue their fill kernel only when the buffer is first asked for. What must hold:
+// out[0] the sum of a ones tensor that went to the host untouched (n); out[1] an accumulator made with zeros BEFORE a
+// capture and first touched inside it, after three replays of `acc += ones` (3 in every element: its fill ran before
+// the capture and is not part of the replays), read as the sum / n; out[2] the sum of zeros + zeros added in place,
+// neither written before (0); out[3] element 0 of -0.0f filled then added to zeros (+0.0, sign bit clear -> 0, the
+// addition may not be skipped); out[4] x.grad of sum(x * full(2.5)) (2.5 * n) / n.
+int DRV(pending_fill_semantics)(int64_t n, double *out)
+{
+    return guarded([&] {
+        StreamScope stream;
+        const auto opt = dtype(DataType::kFloat32).device(kDev);
+        const Shape shp{(size_t)n};
+        auto total = [](const Tensor &t) {
+            double s = 0;
+            for (float v : t.to_vector<float>())
+                s += v;
+            return s;
+        };
+        out[0] = total(Tensor::ones(shp, opt).to(Device(DeviceType::kCPU)));
+        {
+            Tensor acc = Tensor::zeros(shp, opt), one = Tensor::ones(shp, opt);
+            one.to_vector<float>();  // written now
+            origin::cuda::Graph graph;
+            graph.begin_capture();
+            acc += one;
+            graph.end_capture();
+            for (int i = 0; i < 3; ++i)
+                graph.launch();
+            out[1] = total(acc) / (double)n;
+        }
+        {
+            Tensor a = Tensor::zeros(shp, opt), b = Tensor::zeros(shp, opt);
+            a += b;
+            out[2] = total(a);
+        }
+        {
+            Tensor a = Tensor::full(shp, -0.0f, opt), b = Tensor::zeros(shp, opt);
+            a += b;
+            const float v = a.to_vector<float>()[0];
+            uint32_t bits;
+            std::memcpy(&bits, &v, sizeof(bits));
+            out[3] = (double)(bits >> 31);
+        }
+        {
+            std::vector<float> h((size_t)n, 1.0f);
+            Tensor x = f32(h.data(), shp, true);
+            auto y = F::sum(x * Tensor::full(shp, 2.5f, opt));
+            y.backward();
+            out[4] = total(x.grad()) / (double)n;
+        }
+    });
+}
+#endif
+
 int DRV(mlp_bench)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, float *ms_per_step, float *loss)
 {
     return mlp_bench_impl(N, D, Hd, C, steps, warmup, 0, ms_per_step, loss);

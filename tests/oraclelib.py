@@ -105,6 +105,7 @@ _DEVICE_ONLY_SIGS = {
     "odl_host_pnnx_forward_graph": _REF_SIGS["odl_ref_pnnx_forward"],
     "odl_host_upload_ordering": "lip>i",
     "odl_host_graph_abort_recovery": "pplllpp>i",
+    "odl_host_pending_fill_semantics": "lp>i",
 }
 
 

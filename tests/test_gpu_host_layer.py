@@ -256,6 +256,16 @@ def test_a_failed_capture_leaves_the_thread_usable_and_replays_report_bad_labels
     assert flags.tolist() == [1, 0]
 
 
+def test_deferred_fills_behave_like_fills_at_creation(h):
+    """zeros / ones / full queue their kernel at the first use of the buffer. Seen from outside nothing may change:
+    a copy to the host sees the values, a buffer made before a capture is filled before it (not on every replay),
+    zeros += zeros stays zeros, -0.0 += zeros becomes +0.0 (src/mat/origin/cpu/math/add.cpp adds every element), and a
+    constant operand takes part in backward."""
+    out = np.full(5, -1.0)
+    assert h.odl_host_pending_fill_semantics(4096, out) == 0
+    assert out.tolist() == [4096.0, 3.0, 0.0, 0.0, 2.5], out
+
+
 def test_reference_example_network_with_batch_norm_trains_and_replays(h):
     """The network of the reference's tests/example/mnist/conv_mnist.cpp (two conv + BatchNorm + ReLU + pool blocks,
     two Linear layers, Adam + WeightDecay) at batch 16: eight ordinary steps, and two ordinary steps followed by six
