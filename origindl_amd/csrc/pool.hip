@@ -209,6 +209,45 @@ __global__ __launch_bounds__(256) void max_pool_bwd_tiled_kernel(const float *__
     }
 }
 
+// Forward of the 2x2 / stride 2 / no padding pooling over an image whose rows hold a multiple of four floats: a thread
+// owns two neighbouring outputs, reads the four cells under them from each of the two image rows with one 16-byte load
+// and stores the two maxima (8 bytes) and the two indices (16 bytes) together. The comparisons are those of the general
+// kernel: window cells in row-major order, a later cell wins only when it is greater (max_pool2d.cpp:110-139).
+__global__ __launch_bounds__(256) void max_pool_fwd_pair_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                uint64_t *__restrict__ idx, unsigned pairs, int OW2,
+                                                                unsigned oplane2)
+{
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+    const unsigned t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= pairs)
+        return;
+    const unsigned nc = t / oplane2, r = t - nc * oplane2;
+    const int oh = (int)(r / (unsigned)OW2), op = (int)r - oh * OW2;  // op: which pair of the output row
+    const int W = OW2 * 4;
+    const float *p = x + (int64_t)nc * oplane2 * 8 + (int64_t)(2 * oh) * W + 4 * op;
+    const f32x4 top = *reinterpret_cast<const f32x4 *>(p), bot = *reinterpret_cast<const f32x4 *>(p + W);
+    f32x2 mv;
+    u64x2 mi;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+    {
+        float m = top[2 * j];
+        int w = 0;
+        if (top[2 * j + 1] > m)
+            m = top[2 * j + 1], w = 1;
+        if (bot[2 * j] > m)
+            m = bot[2 * j], w = 2;
+        if (bot[2 * j + 1] > m)
+            m = bot[2 * j + 1], w = 3;
+        mv[j] = m, mi[j] = (unsigned long long)w;
+    }
+    *reinterpret_cast<f32x2 *>(y + 2 * (int64_t)t) = mv;
+    if (idx)
+        *reinterpret_cast<u64x2 *>(idx + 2 * (int64_t)t) = mi;
+}
+
 bool tiles_exactly(const PoolGeom &g)
 {
     return g.KH == g.KW && g.SH == g.KH && g.SW == g.KW && g.PH == 0 && g.PW == 0 && g.H == g.OH * g.KH &&
@@ -271,7 +310,14 @@ int odl_hip_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t 
     if (total == 0)
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
-    if (plane_ok(g))
+    if (plane_ok(g) && tiles_exactly(g) && g.KH == 2 && g.W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+        (reinterpret_cast<uintptr_t>(y) & 7) == 0 && (reinterpret_cast<uintptr_t>(idx) & 15) == 0)
+    {
+        const unsigned pairs = (unsigned)(total / 2);
+        hipLaunchKernelGGL(max_pool_fwd_pair_kernel, dim3((unsigned)odl::ceil_div((int64_t)pairs, 256)), dim3(256), 0, st,
+                           x, y, idx, pairs, (int)(g.OW / 2), (unsigned)(g.OH * g.OW / 2));
+    }
+    else if (plane_ok(g))
     {
         const dim3 grid = plane_grid(g.OH * g.OW, N * C);
         ODL_POOL_DISPATCH(max_pool_fwd_plane_kernel, x, y, idx, g);
