@@ -18,6 +18,7 @@
 //     8 XCDs) on a contiguous band of tiles, walked in groups of 8 tile-rows so A and B panels are reused
 //     from that XCD's L2;
 //   * split-K (grid.y) writes partial tiles that a second kernel sums in slice order — deterministic.
+#include "gemm_dma.h"
 #include "odl_common.h"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -873,6 +874,18 @@ void launch_tail_fixup(const GemmArgs &g, int BM, int BN, int epi, hipStream_t s
     hipLaunchKernelGGL(tail_fixup_kernel, dim3((unsigned)odl::ceil_div(threads, 256)), dim3(256), 0, st, g, BM, BN, epi);
 }
 
+// the same product for the variant whose operands go from global memory straight into LDS
+odl::DmaGemmArgs dma_args(const GemmArgs &g, int epi)
+{
+    odl::DmaGemmArgs d;
+    d.A = g.A, d.B = g.B, d.bias = g.bias, d.C = g.C;
+    d.M = g.M, d.N = g.N, d.K = g.K, d.lda = g.lda, d.ldb = g.ldb, d.ldc = g.ldc;
+    d.tiles_m = g.tiles_m, d.tiles_n = g.tiles_n, d.splits = g.splits;
+    d.k_per_split = g.k_per_split, d.c_split_stride = g.c_split_stride;
+    d.epi = epi == EPI_BIAS_COL ? 1 : 0, d.act = g.act, d.xcds = g.xcds;
+    return d;
+}
+
 // tile counts up to which a launch puts about one workgroup on a compute unit
 int64_t lone_workgroup_limit()
 {
@@ -914,6 +927,12 @@ int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g_in, int splits, vo
         // at most about one workgroup per compute unit: a second set of four waves on every tile
         if (vec && splits == 1 && g.tail_splits == 0 && (int64_t)g.tiles_m * g.tiles_n <= lone_workgroup_limit())
         {
+            if constexpr (EPI != EPI_NCHW_ROWB)
+            {
+                const odl::DmaGemmArgs d = dma_args(g, EPI);
+                if (odl::sgemm_dma_fits(ta, tb, d))
+                    return odl::sgemm_dma_launch(128, ta, tb, d, st);
+            }
 #define ODL_GEMM_TWO_SETS(TA, TB)                                                                                   \
     if (ta == TA && tb == TB)                                                                                       \
     {                                                                                                               \
@@ -1006,6 +1025,12 @@ int launch_small_tile_wide_slab(bool ta, bool tb, GemmArgs g, int splits, hipStr
     g.xcds = odl::chip().xcds;
     const dim3 grid((unsigned)(g.tiles_m * g.tiles_n * splits)), block(kThreads);
     const bool two_sets = (int64_t)g.tiles_m * g.tiles_n * splits <= lone_workgroup_limit();
+    if (two_sets)
+    {
+        const odl::DmaGemmArgs d = dma_args(g, EPI);
+        if (odl::sgemm_dma_fits(ta, tb, d))
+            return odl::sgemm_dma_launch(64, ta, tb, d, st);
+    }
 #define ODL_WIDE_CASE(TA, TB)                                                                                  \
     if (ta == TA && tb == TB)                                                                                  \
     {                                                                                                          \

@@ -1,0 +1,27 @@
+// C = A . B for products whose tiles leave about one workgroup per compute unit: operands go from global memory straight
+// into LDS (no registers in between), four K slabs deep. Declared here for gemm.hip, which picks the variant.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace odl
+{
+struct DmaGemmArgs
+{
+    const float *A, *B, *bias;
+    float *C;
+    int64_t M, N, K, lda, ldb, ldc;
+    int tiles_m, tiles_n, splits;
+    int64_t k_per_split;     // K range of one slice (a multiple of 32)
+    int64_t c_split_stride;  // distance between the partial outputs of two slices (0 when splits == 1)
+    int epi;                 // 0 plain, 1 bias by column then the activation
+    int act;                 // 0 none, 1 relu, 2 silu
+    int xcds;
+};
+
+// true when the shape suits the variant (16-byte aligned rows, offsets within 31 bits)
+bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g);
+// tile: 64 (64x64 tiles) or 128 (128x128 tiles); the grid is tiles_m * tiles_n * splits workgroups of 512 threads
+int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st);
+}  // namespace odl

@@ -1,0 +1,341 @@
+// FP32 GEMM on v_mfma_f32_32x32x2_f32 whose operands travel from global memory into LDS without passing through
+// registers (buffer_load ... lds, 16 bytes per lane), four K slabs deep.
+//
+// For products with about one workgroup per compute unit. There nothing else runs on the compute unit while a workgroup
+// waits: with operands staged through registers, every slab costs the wait for its loads plus the LDS stores in front of
+// the barrier, and the matrix pipe idles through both (1024x1024x4096: 99 us with staging, 72 us with the staging taken
+// out). Here a slab's loads are queued three slabs ahead and land in LDS on their own; a wave only waits for loads that
+// were queued three barriers ago, then reads its fragments and issues its matrix instructions.
+//
+//   * 512 threads: two sets of four waves on the tile; of the 8-wide K steps of a slab each set multiplies every other
+//     one, and the second set's accumulators join the first's through LDS before the epilogue.
+//   * LDS holds the operand tiles exactly as the loads deliver them: lane i of a wave's load lands at base + 16*i.
+//       K-contiguous operand (A of A.B, B of A.B^T): tile [rows][BK], a row's 16-byte pieces permuted by
+//         piece ^ (row & (BK/4-1)) — chosen on the global side, so that the 8 rows one ds_read_b128 phase touches fall
+//         into 8 different bank groups;
+//       row-contiguous operand (A of A^T.B, B of A.B): tile [BK][cols], read back with ds_read_b32, lanes along cols.
+//   * Rows, columns and K positions outside the matrix: the lane's offset is set past the buffer's size and the load
+//     delivers zeros.
+#include "gemm_dma.h"
+#include "odl_common.h"
+
+namespace
+{
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kNT     = 512;
+constexpr int kStages = 4;
+constexpr int kEpiBiasCol = 1;
+constexpr unsigned kOutside = 0x80000000u;  // beyond the 2^31 - 1 bytes every buffer descriptor here declares
+
+__device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
+{
+    const int gsz = 8 * tiles_n;  // groups of 8 tile-rows
+    const int grp = t / gsz, in_g = t % gsz;
+    const int first_m = grp * 8;
+    const int gm = (tiles_m - first_m) < 8 ? (tiles_m - first_m) : 8;
+    tm = first_m + in_g % gm;
+    tn = in_g / gm;
+}
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// One 16-byte load per lane from a buffer into LDS: lane i's data lands at lds_byte_address + 16*i. Written as an
+// instruction rather than through the compiler's builtin: the compiler cannot tell which stage a queued load writes
+// and would wait for ALL queued loads before every LDS read, which is exactly the wait this kernel exists to avoid.
+// The waits are placed by hand (wait_vmcnt below). The LDS address travels in M0, which nothing else here uses.
+__device__ inline void load_to_lds_16(i32x4 rsrc, unsigned lds_byte_address, unsigned lane_offset)
+{
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_byte_address), "v"(lane_offset), "s"(rsrc)
+                 : "memory", "m0");
+}
+
+__device__ inline i32x4 buffer_of(const float *base)
+{
+    const uint64_t p = reinterpret_cast<uint64_t>(base);
+    i32x4 r;
+    // (the address is the same in every lane; readfirstlane tells the compiler so, and the descriptor stays in SGPRs)
+    r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)p);
+    r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(p >> 32));  // stride 0: a raw buffer
+    r[2] = 0x7fffffff;                                          // bytes; offsets at or past it deliver zeros
+    r[3] = 0x00020000;
+    return r;
+}
+
+// s_waitcnt that only waits for the vector-memory counter to drop to n (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+template <int N>
+__device__ inline void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <int BM, int BN, int BK, bool TA, bool TB>
+__global__ __launch_bounds__(kNT, 1) void sgemm_dma_kernel(const odl::DmaGemmArgs g)
+{
+    constexpr bool A_KMAJOR = !TA, B_KMAJOR = TB;
+    constexpr int PIECES = BK / 4;                       // 16-byte pieces in a K-contiguous row of a slab
+    constexpr int A_U = BM * BK / 4 / kNT, B_U = BN * BK / 4 / kNT;  // loads per thread and slab
+    static_assert((BM * BK / 4) % kNT == 0 && (BN * BK / 4) % kNT == 0 && (PIECES & (PIECES - 1)) == 0, "tile shape");
+    constexpr int PER_SLAB = A_U + B_U;
+    constexpr int RB = BM / 64, CB = BN / 64;            // 32x32 blocks per wave
+    constexpr int STEPS = BK / 16;                       // 8-wide K steps per wave and slab (two wave sets)
+    __shared__ __attribute__((aligned(16))) float As[kStages][BM * BK];
+    __shared__ __attribute__((aligned(16))) float Bs[kStages][BN * BK];
+    static_assert(kStages * BM * BK >= 4 * 16 * 64, "the A buffers hold one accumulator block of four waves");
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = wave8 & 3, kset = wave8 >> 2;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+
+    // workgroup -> (K slice, tile): a contiguous band of workgroups per XCD, tiles in groups of 8 tile-rows
+    int tm, tn, kz;
+    {
+        const unsigned nt = (unsigned)(g.tiles_m * g.tiles_n), total = nt * (unsigned)g.splits;
+        const unsigned bid = blockIdx.x, nx = (unsigned)g.xcds;
+        const unsigned loc = bid / nx, xcd = bid - loc * nx;
+        const unsigned full = total / nx, rem = total - full * nx;
+        const unsigned v = xcd * full + (xcd < rem ? xcd : rem) + loc;
+        kz = (int)(v / nt);
+        tile_coords((int)(v - (unsigned)kz * nt), g.tiles_m, g.tiles_n, tm, tn);
+    }
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t kbeg = (int64_t)kz * g.k_per_split;
+    const int64_t kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
+    const int nkt = (int)((kend - kbeg + BK - 1) / BK);
+    const int klen = (int)(kend - kbeg);
+
+    // buffer descriptors based at this workgroup's corner of each operand; every lane offset is relative to it
+    const float *abase = g.A + (A_KMAJOR ? m0 * g.lda + kbeg : kbeg * g.lda + m0);
+    const float *bbase = g.B + (B_KMAJOR ? n0 * g.ldb + kbeg : kbeg * g.ldb + n0);
+    const i32x4 ra = buffer_of(abase), rb = buffer_of(bbase);
+    const unsigned as_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) float *)&As[0][0];
+    const unsigned bs_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) float *)&Bs[0][0];
+
+    // per load of this thread: byte offset inside slab 0, the K position it covers inside a slab, and whether its row
+    // (or column quad) is inside the matrix
+    unsigned a_off[A_U], b_off[B_U];
+    int a_k[A_U], b_k[B_U];
+    bool a_in[A_U], b_in[B_U];
+#pragma unroll
+    for (int u = 0; u < A_U; ++u)
+    {
+        const int f = tid + u * kNT;
+        if (A_KMAJOR)
+        {
+            const int row = f / PIECES, piece = (f % PIECES) ^ (row & (PIECES - 1));
+            a_off[u] = (unsigned)((row * g.lda + 4 * piece) * 4), a_k[u] = 4 * piece, a_in[u] = m0 + row < g.M;
+        }
+        else
+        {
+            const int k = f / (BM / 4), c4 = f % (BM / 4);
+            a_off[u] = (unsigned)((k * g.lda + 4 * c4) * 4), a_k[u] = k, a_in[u] = m0 + 4 * c4 < g.M;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < B_U; ++u)
+    {
+        const int f = tid + u * kNT;
+        if (B_KMAJOR)
+        {
+            const int row = f / PIECES, piece = (f % PIECES) ^ (row & (PIECES - 1));
+            b_off[u] = (unsigned)((row * g.ldb + 4 * piece) * 4), b_k[u] = 4 * piece, b_in[u] = n0 + row < g.N;
+        }
+        else
+        {
+            const int k = f / (BN / 4), c4 = f % (BN / 4);
+            b_off[u] = (unsigned)((k * g.ldb + 4 * c4) * 4), b_k[u] = k, b_in[u] = n0 + 4 * c4 < g.N;
+        }
+    }
+    const unsigned a_step = (unsigned)((A_KMAJOR ? (int64_t)BK : (int64_t)BK * g.lda) * 4);
+    const unsigned b_step = (unsigned)((B_KMAJOR ? (int64_t)BK : (int64_t)BK * g.ldb) * 4);
+
+    // queue the loads of slab kt into a stage (slabs past the end deliver zeros into a stage nobody reads: the count of
+    // loads in flight stays the same for every slab, which is what the waits below rely on)
+    auto issue = [&](int stage, int kt) {
+        const int k0 = kt * BK;
+#pragma unroll
+        for (int u = 0; u < A_U; ++u)
+        {
+            const bool ok = a_in[u] && k0 + a_k[u] < klen;
+            load_to_lds_16(ra, as_lds + (unsigned)((stage * BM * BK + (u * kNT + wave8 * 64) * 4) * 4),
+                           ok ? a_off[u] + (unsigned)kt * a_step : kOutside);
+        }
+#pragma unroll
+        for (int u = 0; u < B_U; ++u)
+        {
+            const bool ok = b_in[u] && k0 + b_k[u] < klen;
+            load_to_lds_16(rb, bs_lds + (unsigned)((stage * BN * BK + (u * kNT + wave8 * 64) * 4) * 4),
+                           ok ? b_off[u] + (unsigned)kt * b_step : kOutside);
+        }
+    };
+
+    f32x16 acc[RB][CB];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < CB; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0.f;
+
+    auto mma = [&](const float *as, const float *bs) {
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st)
+        {
+            const int ks = 2 * st + kset;
+            float a[RB][4], b[CB][4];
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
+            {
+                const int r = wm + i * 32 + l32;
+                if (A_KMAJOR)
+                {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(as + (r * PIECES + ((2 * ks + lh) ^ (r & (PIECES - 1)))) * 4);
+                    a[i][0] = v[0], a[i][1] = v[1], a[i][2] = v[2], a[i][3] = v[3];
+                }
+                else
+                {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        a[i][s] = as[(ks * 8 + 4 * lh + s) * BM + r];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < CB; ++j)
+            {
+                const int c = wn + j * 32 + l32;
+                if (B_KMAJOR)
+                {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(bs + (c * PIECES + ((2 * ks + lh) ^ (c & (PIECES - 1)))) * 4);
+                    b[j][0] = v[0], b[j][1] = v[1], b[j][2] = v[2], b[j][3] = v[3];
+                }
+                else
+                {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+                        b[j][s] = bs[(ks * 8 + 4 * lh + s) * BN + c];
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int i = 0; i < RB; ++i)
+#pragma unroll
+                    for (int j = 0; j < CB; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][s], b[j][s], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    // slabs 0..2 are on their way before the loop; in the loop, slab kt's loads were queued three barriers ago
+#pragma unroll
+    for (int s = 0; s < kStages - 1; ++s)
+        issue(s, s);
+    for (int kt = 0; kt < nkt; kt += kStages)
+    {
+#pragma unroll
+        for (int s = 0; s < kStages; ++s)
+        {
+            if (kt + s < nkt)
+            {
+                wait_vmcnt<(kStages - 2) * PER_SLAB>();  // this thread's loads of slab kt+s have landed
+                __syncthreads();                         // ... and everybody else's; slab kt+s-1 has been read by all
+                issue((s + kStages - 1) % kStages, kt + s + kStages - 1);
+                mma(As[s], Bs[s]);
+            }
+        }
+    }
+    wait_vmcnt<0>();  // the zero-filled slabs past the end are still landing in the stages
+    __syncthreads();
+
+    // the second wave set hands its accumulators to the first, one 32x32 block of each wave at a time
+    {
+        float *xch = &As[0][0] + (wave * 16) * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int j = 0; j < CB; ++j)
+            {
+                if (kset == 1)
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        xch[r * 64] = acc[i][j][r];
+                }
+                __syncthreads();
+                if (kset == 0)
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[i][j][r] += xch[r * 64];
+                }
+                __syncthreads();
+            }
+        if (kset == 1)
+            return;
+    }
+
+    // accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
+    float *Cout = g.C + (int64_t)kz * g.c_split_stride;
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
+#pragma unroll
+        for (int j = 0; j < CB; ++j)
+        {
+            const int64_t col = n0 + wn + j * 32 + l32;
+            if (col >= g.N)
+                continue;
+            const bool with_bias = g.epi == kEpiBiasCol && g.bias != nullptr;
+            const float bcol = with_bias ? g.bias[col] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                const int64_t row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+                if (row >= g.M)
+                    continue;
+                float v = acc[i][j][r];
+                if (with_bias)
+                    v = odl::apply_act(v + bcol, g.act);
+                Cout[row * g.ldc + col] = v;
+            }
+        }
+}
+}  // namespace
+
+namespace odl
+{
+bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g)
+{
+    const bool aligned = ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) % 16 == 0) &&
+                         g.lda % 4 == 0 && g.ldb % 4 == 0 && (ta ? g.M : g.K) % 4 == 0 && (tb ? g.K : g.N) % 4 == 0 &&
+                         (g.splits == 1 || g.k_per_split % 32 == 0);
+    // lane offsets are 32-bit and must stay below 2^31: the rows of a tile, or the K range of a slice, times the row length
+    const int64_t a_span = (ta ? g.k_per_split + 64 : 128) * g.lda * 4, b_span = (tb ? 128 : g.k_per_split + 64) * g.ldb * 4;
+    return aligned && a_span < (1ll << 31) && b_span < (1ll << 31) && g.M > 0 && g.N > 0 && g.K > 0;
+}
+
+int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st)
+{
+    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n * g.splits)), block(kNT);
+#define ODL_DMA_CASE(TA, TB)                                                                          \
+    if (ta == TA && tb == TB)                                                                         \
+    {                                                                                                 \
+        if (tile == 64)                                                                               \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB>), grid, block, 0, st, g);        \
+        else                                                                                          \
+            hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 32, TA, TB>), grid, block, 0, st, g);      \
+        return ODL_OK;                                                                                \
+    }
+    ODL_DMA_CASE(false, false)
+    ODL_DMA_CASE(false, true)
+    ODL_DMA_CASE(true, false)
+    ODL_DMA_CASE(true, true)
+#undef ODL_DMA_CASE
+    return ODL_ERR_RUNTIME;
+}
+}  // namespace odl

@@ -1130,3 +1130,30 @@ def test_linear_with_the_activation_in_the_epilogue_equals_linear_then_relu(api)
     with pytest.raises(api.OdlInvalidArgument):
         L.call("odl_hip_linear_act", x.data_ptr(), w.data_ptr(), b.data_ptr(), M, N, K, 3, fused.data_ptr(), ws.data_ptr(),
                nb, None)
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 256), (200, 136, 520), (512, 1000, 784), (1024, 1024, 1024), (260, 2052, 4100),
+                                   (1536, 1536, 512)])
+def test_products_with_about_one_workgroup_per_compute_unit_in_all_four_layouts(api, M, N, K):
+    # The variant whose operands go from global memory straight into LDS (64x64 and 128x128 tiles, K in slices or whole):
+    # ragged edges in M, N and K (zero-filled by the loads), the four operand layouts of
+    # src/mat/origin/cpu/math/matmul.cpp:113-218 and src/operators/math/mat_mul.cpp:123-182, bias in the epilogue.
+    L = api.lib()
+    rng = np.random.default_rng(M + N + K)
+    a, b = rng.standard_normal((M, K), dtype=np.float32), rng.standard_normal((K, N), dtype=np.float32)
+    bias = rng.standard_normal((N,), dtype=np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    bound = gemm_bound(a, b)
+    for ta in (0, 1):
+        for tb in (0, 1):
+            da, db = dev(a.T if ta else a), dev(b.T if tb else b)
+            c = torch.full((M, N), float("nan"), device="cuda")
+            nb = L.query("odl_hip_sgemm_workspace_bytes", ta, tb, M, N, K, 0)
+            ws = torch.empty(max(nb, 16), dtype=torch.uint8, device="cuda")
+            L.call("odl_hip_sgemm", ta, tb, M, N, K, da.data_ptr(), da.shape[1], db.data_ptr(), db.shape[1], c.data_ptr(), N,
+                   None, 0, ws.data_ptr(), nb, None)
+            got = host(c).astype(np.float64)
+            assert (np.abs(got - want) <= bound).all(), (ta, tb, np.abs(got - want).max())
+            L.call("odl_hip_sgemm", ta, tb, M, N, K, da.data_ptr(), da.shape[1], db.data_ptr(), db.shape[1], c.data_ptr(), N,
+                   dev(bias).data_ptr(), 0, ws.data_ptr(), nb, None)
+            assert np.array_equal(host(c), (got.astype(np.float32) + bias)), (ta, tb, "bias")
