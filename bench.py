@@ -434,7 +434,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                      "traffic": GEMM_4096_TRAFFIC_BYTES if S == 4096 else None,
-                     "kernel": "sgemm_mfma_kernel<128,128,16> (NN, NT, TN)", "launch_ms": launch_ms},
+                     "kernel": "sgemm_dma_kernel<128,128,16,TA,TB,2> (NN, NT, TN)", "launch_ms": launch_ms},
         "device": capi.device_info(0),
     }
     if not args.no_extras:

@@ -947,6 +947,17 @@ int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g_in, int splits, vo
 #undef ODL_GEMM_TWO_SETS
         }
     }
+    if constexpr (BM == 128 && BN == 128 && EPI != EPI_NCHW_ROWB)
+    {
+        // whole rounds of many tiles: operands straight into LDS, two workgroups of eight waves per compute unit
+        // (4096^3: 82 -> 88 % of the matrix peak). Launches with a split tail keep the kernel below, which has the fix-up.
+        if (vec && splits == 1 && g.tail_splits == 0)
+        {
+            const odl::DmaGemmArgs d = dma_args(g, EPI);
+            if (odl::sgemm_dma_fits(ta, tb, d))
+                return odl::sgemm_dma_launch(129, ta, tb, d, st);
+        }
+    }
 #define ODL_GEMM_CASE(TA, TB, V)                                                                      \
     if (ta == TA && tb == TB && vec == V)                                                             \
     {                                                                                                 \

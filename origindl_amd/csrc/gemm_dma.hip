@@ -73,8 +73,17 @@ __device__ inline void wait_vmcnt()
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-template <int BM, int BN, int BK, bool TA, bool TB>
-__global__ __launch_bounds__(kNT, 1) void sgemm_dma_kernel(const odl::DmaGemmArgs g)
+// which 16-byte slot of its LDS row a K-contiguous row's piece goes to: piece ^ swizzle(row). Eight consecutive rows,
+// read 16 bytes each at the same piece, must fall into eight different bank groups: rows that share a 128-byte line of
+// LDS (8/PIECES of them) get the same value, consecutive lines different ones.
+template <int PIECES>
+__device__ inline int swizzle(int row)
+{
+    return PIECES >= 8 ? (row & (PIECES - 1)) : ((row / (8 / PIECES)) & (PIECES - 1));
+}
+
+template <int BM, int BN, int BK, bool TA, bool TB, int WGS_PER_CU>
+__global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::DmaGemmArgs g)
 {
     constexpr bool A_KMAJOR = !TA, B_KMAJOR = TB;
     constexpr int PIECES = BK / 4;                       // 16-byte pieces in a K-contiguous row of a slab
@@ -128,7 +137,7 @@ __global__ __launch_bounds__(kNT, 1) void sgemm_dma_kernel(const odl::DmaGemmArg
         const int f = tid + u * kNT;
         if (A_KMAJOR)
         {
-            const int row = f / PIECES, piece = (f % PIECES) ^ (row & (PIECES - 1));
+            const int row = f / PIECES, piece = (f % PIECES) ^ swizzle<PIECES>(row);
             a_off[u] = (unsigned)((row * g.lda + 4 * piece) * 4), a_k[u] = 4 * piece, a_in[u] = m0 + row < g.M;
         }
         else
@@ -143,7 +152,7 @@ __global__ __launch_bounds__(kNT, 1) void sgemm_dma_kernel(const odl::DmaGemmArg
         const int f = tid + u * kNT;
         if (B_KMAJOR)
         {
-            const int row = f / PIECES, piece = (f % PIECES) ^ (row & (PIECES - 1));
+            const int row = f / PIECES, piece = (f % PIECES) ^ swizzle<PIECES>(row);
             b_off[u] = (unsigned)((row * g.ldb + 4 * piece) * 4), b_k[u] = 4 * piece, b_in[u] = n0 + row < g.N;
         }
         else
@@ -196,7 +205,7 @@ __global__ __launch_bounds__(kNT, 1) void sgemm_dma_kernel(const odl::DmaGemmArg
                 const int r = wm + i * 32 + l32;
                 if (A_KMAJOR)
                 {
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(as + (r * PIECES + ((2 * ks + lh) ^ (r & (PIECES - 1)))) * 4);
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(as + (r * PIECES + ((2 * ks + lh) ^ swizzle<PIECES>(r))) * 4);
                     a[i][0] = v[0], a[i][1] = v[1], a[i][2] = v[2], a[i][3] = v[3];
                 }
                 else
@@ -212,7 +221,7 @@ __global__ __launch_bounds__(kNT, 1) void sgemm_dma_kernel(const odl::DmaGemmArg
                 const int c = wn + j * 32 + l32;
                 if (B_KMAJOR)
                 {
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(bs + (c * PIECES + ((2 * ks + lh) ^ (c & (PIECES - 1)))) * 4);
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(bs + (c * PIECES + ((2 * ks + lh) ^ swizzle<PIECES>(c))) * 4);
                     b[j][0] = v[0], b[j][1] = v[1], b[j][2] = v[2], b[j][3] = v[3];
                 }
                 else
@@ -326,9 +335,11 @@ int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream
     if (ta == TA && tb == TB)                                                                         \
     {                                                                                                 \
         if (tile == 64)                                                                               \
-            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB>), grid, block, 0, st, g);        \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 1>), grid, block, 0, st, g);     \
+        else if (tile == 128)                                                                         \
+            hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 32, TA, TB, 1>), grid, block, 0, st, g);   \
         else                                                                                          \
-            hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 32, TA, TB>), grid, block, 0, st, g);      \
+            hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 16, TA, TB, 2>), grid, block, 0, st, g);   \
         return ODL_OK;                                                                                \
     }
     ODL_DMA_CASE(false, false)
