@@ -319,10 +319,11 @@ def yolo_forward(h, ref, reps):
     return res
 
 
-# HBM-side bytes of one 4096^3 sgemm_mfma_kernel launch: FETCH_SIZE (scaled 2.000x by the calibration copy) 808.6 MiB on
-# average over the NN / NT / TN variants (742 / 978 / 706) + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc`
-# runs of `--pmc-probe` summarised under profiles/.
-GEMM_4096_TRAFFIC_BYTES = int((808.6 + 64.0) * 1024 * 1024)
+# HBM-side bytes of one 4096^3 GEMM launch, a recorded constant (counters cannot be read from inside this process):
+# FETCH_SIZE (scaled 2.000x by the calibration copy) 729.5 MiB on average over the NN / NT / TN variants
+# (725 / 723 / 740) + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc` runs of `--pmc-probe` summarised in
+# profiles/hot_kernels_hbm_traffic.md.
+GEMM_4096_TRAFFIC_BYTES = int((729.5 + 64.0) * 1024 * 1024)
 
 
 def pmc_probe(torch, capi, gemm_step):
@@ -434,6 +435,8 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                      "traffic": GEMM_4096_TRAFFIC_BYTES if S == 4096 else None,
+                     "traffic_source": ("recorded constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py "
+                                        "--pmc-probe`, profiles/hot_kernels_hbm_traffic.md" if S == 4096 else None),
                      "kernel": "sgemm_dma_kernel<128,128,16,TA,TB,2> (NN, NT, TN)", "launch_ms": launch_ms},
         "device": capi.device_info(0),
     }
