@@ -22,7 +22,7 @@ struct DmaGemmArgs
 
 // true when the shape suits the variant (16-byte aligned rows, offsets within 31 bits)
 bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g);
-// tile: 64 (64x64 tiles, one workgroup per compute unit), 128 (128x128 tiles, one per compute unit) or 129 (128x128
+// tile: 32 (64x32 tiles in 64-wide slabs, four wave sets), 64 (64x64 tiles, one workgroup per compute unit), 128 (128x128 tiles, one per compute unit) or 129 (128x128
 // tiles in 16-wide slabs, two workgroups per compute unit: for launches of many tiles); the grid is
 // tiles_m * tiles_n * splits workgroups of 512 threads
 int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st);

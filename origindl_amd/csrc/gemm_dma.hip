@@ -82,7 +82,10 @@ __device__ inline int swizzle(int row)
     return PIECES >= 8 ? (row & (PIECES - 1)) : ((row / (8 / PIECES)) & (PIECES - 1));
 }
 
-template <int BM, int BN, int BK, bool TA, bool TB, int WGS_PER_CU>
+// KSETS wave sets share a tile: the eight waves are WAVES_N columns x (8 / KSETS / WAVES_N) rows of wave tiles, times
+// KSETS sets that each multiply every KSETS-th 8-wide K step (2 sets for square tiles; 4 sets on a 64x32 tile, whose
+// two 32x32 blocks could not occupy eight waves otherwise).
+template <int BM, int BN, int BK, bool TA, bool TB, int WGS_PER_CU, int KSETS = 2>
 __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::DmaGemmArgs g)
 {
     constexpr bool A_KMAJOR = !TA, B_KMAJOR = TB;
@@ -90,17 +93,20 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     constexpr int A_U = BM * BK / 4 / kNT, B_U = BN * BK / 4 / kNT;  // loads per thread and slab
     static_assert((BM * BK / 4) % kNT == 0 && (BN * BK / 4) % kNT == 0 && (PIECES & (PIECES - 1)) == 0, "tile shape");
     constexpr int PER_SLAB = A_U + B_U;
-    constexpr int RB = BM / 64, CB = BN / 64;            // 32x32 blocks per wave
-    constexpr int STEPS = BK / 16;                       // 8-wide K steps per wave and slab (two wave sets)
+    constexpr int WAVES_N = KSETS == 2 ? 2 : 1, WAVES_M = 8 / KSETS / WAVES_N;
+    constexpr int RB = BM / WAVES_M / 32, CB = BN / WAVES_N / 32;  // 32x32 blocks per wave
+    constexpr int STEPS = BK / 8 / KSETS;                          // 8-wide K steps per wave and slab
+    static_assert(RB >= 1 && CB >= 1 && STEPS >= 1 && RB * WAVES_M * 32 == BM && CB * WAVES_N * 32 == BN, "wave layout");
     __shared__ __attribute__((aligned(16))) float As[kStages][BM * BK];
     __shared__ __attribute__((aligned(16))) float Bs[kStages][BN * BK];
-    static_assert(kStages * BM * BK >= 4 * 16 * 64, "the A buffers hold one accumulator block of four waves");
+    static_assert(kStages * BM * BK >= (KSETS - 1) * (8 / KSETS) * 16 * 64, "the A buffers hold one accumulator block of every wave of the other sets");
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave = wave8 & 3, kset = wave8 >> 2;
+    constexpr int TILE_WAVES = 8 / KSETS;
+    const int wave = wave8 % TILE_WAVES, kset = wave8 / TILE_WAVES;
     const int l32 = lane & 31, lh = lane >> 5;
-    const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+    const int wm = (wave / WAVES_N) * (BM / WAVES_M), wn = (wave % WAVES_N) * (BN / WAVES_N);
 
     // workgroup -> (K slice, tile): a contiguous band of workgroups per XCD, tiles in groups of 8 tile-rows
     int tm, tn, kz;
@@ -197,7 +203,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
 #pragma unroll
         for (int st = 0; st < STEPS; ++st)
         {
-            const int ks = 2 * st + kset;
+            const int ks = KSETS * st + kset;
             float a[RB][4], b[CB][4];
 #pragma unroll
             for (int i = 0; i < RB; ++i)
@@ -262,30 +268,34 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     wait_vmcnt<0>();  // the zero-filled slabs past the end are still landing in the stages
     __syncthreads();
 
-    // the second wave set hands its accumulators to the first, one 32x32 block of each wave at a time
+    // the other wave sets hand their accumulators to the first, one 32x32 block of each wave at a time; the first adds
+    // them in set order
     {
         float *xch = &As[0][0] + (wave * 16) * 64 + lane;
+        constexpr int SET_STRIDE = TILE_WAVES * 16 * 64;
 #pragma unroll
         for (int i = 0; i < RB; ++i)
 #pragma unroll
             for (int j = 0; j < CB; ++j)
             {
-                if (kset == 1)
+                if (kset > 0)
                 {
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
-                        xch[r * 64] = acc[i][j][r];
+                        xch[(kset - 1) * SET_STRIDE + r * 64] = acc[i][j][r];
                 }
                 __syncthreads();
                 if (kset == 0)
                 {
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        acc[i][j][r] += xch[r * 64];
+                    for (int z = 0; z < KSETS - 1; ++z)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            acc[i][j][r] += xch[z * SET_STRIDE + r * 64];
                 }
                 __syncthreads();
             }
-        if (kset == 1)
+        if (kset > 0)
             return;
     }
 
@@ -336,6 +346,8 @@ int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream
     {                                                                                                 \
         if (tile == 64)                                                                               \
             hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 1>), grid, block, 0, st, g);     \
+        else if (tile == 32)                                                                          \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 32, 64, TA, TB, 1, 4>), grid, block, 0, st, g);  \
         else if (tile == 128)                                                                         \
             hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 32, TA, TB, 1>), grid, block, 0, st, g);   \
         else                                                                                          \
