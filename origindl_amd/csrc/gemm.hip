@@ -883,6 +883,8 @@ odl::DmaGemmArgs dma_args(const GemmArgs &g, int epi)
     d.tiles_m = g.tiles_m, d.tiles_n = g.tiles_n, d.splits = g.splits;
     d.k_per_split = g.k_per_split, d.c_split_stride = g.c_split_stride;
     d.epi = epi == EPI_BIAS_COL ? 1 : 0, d.act = g.act, d.xcds = g.xcds;
+    d.main_blocks = g.main_blocks, d.tail_first = g.tail_first, d.tail_splits = g.tail_splits, d.tail_kps = g.tail_kps;
+    d.tail_ws = g.tail_ws;
     return d;
 }
 
@@ -949,13 +951,18 @@ int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g_in, int splits, vo
     }
     if constexpr (BM == 128 && BN == 128 && EPI != EPI_NCHW_ROWB)
     {
-        // whole rounds of many tiles: operands straight into LDS, two workgroups of eight waves per compute unit
-        // (4096^3: 82 -> 88 % of the matrix peak). Launches with a split tail keep the kernel below, which has the fix-up.
-        if (vec && splits == 1 && g.tail_splits == 0)
+        // many tiles: operands straight into LDS, two workgroups of eight waves per compute unit (4096^3: 82 -> 88 % of
+        // the matrix peak); the K pieces of a split tail are finished by the fix-up kernel as below
+        if (vec && splits == 1)
         {
             const odl::DmaGemmArgs d = dma_args(g, EPI);
             if (odl::sgemm_dma_fits(ta, tb, d))
-                return odl::sgemm_dma_launch(129, ta, tb, d, st);
+            {
+                const int rc = odl::sgemm_dma_launch(129, ta, tb, d, st);
+                if (rc == ODL_OK)
+                    launch_tail_fixup(g, BM, BN, EPI, st);
+                return rc;
+            }
         }
     }
 #define ODL_GEMM_CASE(TA, TB, V)                                                                      \
@@ -1108,6 +1115,7 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
         GemmArgs h = g;
         h.tiles_n = (int)ceil_div(N, 32), h.splits = 1, h.k_per_split = ceil_div(K, 64) * 64, h.c_split_stride = 0;
         h.xcds = odl::chip().xcds;
+        h.main_blocks = 0, h.tail_first = h.tiles_m * h.tiles_n, h.tail_splits = 0, h.tail_kps = 0, h.tail_ws = nullptr;
         const odl::DmaGemmArgs d = dma_args(h, epi);
         if (odl::sgemm_dma_fits(trans_a, trans_b, d))
         {

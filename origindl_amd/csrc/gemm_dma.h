@@ -18,12 +18,18 @@ struct DmaGemmArgs
     int epi;                 // 0 plain, 1 bias by column then the activation
     int act;                 // 0 none, 1 relu, 2 silu
     int xcds;
+    // Tail split (0 pieces: none): the tiles from tail_first on are cut into tail_splits runs of tail_kps K values each,
+    // done by the workgroups from main_blocks on, which write their raw [BM][BN] accumulators to tail_ws, one block
+    // per (tile, piece); a fix-up kernel of the caller adds the pieces in order and finishes those tiles.
+    int main_blocks, tail_first, tail_splits;
+    int64_t tail_kps;
+    float *tail_ws;
 };
 
 // true when the shape suits the variant (16-byte aligned rows, offsets within 31 bits)
 bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g);
 // tile: 32 (64x32 tiles in 64-wide slabs, four wave sets), 64 (64x64 tiles, one workgroup per compute unit), 128 (128x128 tiles, one per compute unit) or 129 (128x128
 // tiles in 16-wide slabs, two workgroups per compute unit: for launches of many tiles); the grid is
-// tiles_m * tiles_n * splits workgroups of 512 threads
+// tiles_m * tiles_n * splits workgroups of 512 threads (main_blocks + tail tiles * tail_splits with a tail split)
 int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st);
 }  // namespace odl

@@ -109,19 +109,37 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     const int wm = (wave / WAVES_N) * (BM / WAVES_M), wn = (wave % WAVES_N) * (BN / WAVES_N);
 
     // workgroup -> (K slice, tile): a contiguous band of workgroups per XCD, tiles in groups of 8 tile-rows
-    int tm, tn, kz;
+    int tm, tn, kz = 0;
+    int64_t kbeg, kend;
+    float *tail_out = nullptr;
     {
-        const unsigned nt = (unsigned)(g.tiles_m * g.tiles_n), total = nt * (unsigned)g.splits;
-        const unsigned bid = blockIdx.x, nx = (unsigned)g.xcds;
-        const unsigned loc = bid / nx, xcd = bid - loc * nx;
-        const unsigned full = total / nx, rem = total - full * nx;
-        const unsigned v = xcd * full + (xcd < rem ? xcd : rem) + loc;
-        kz = (int)(v / nt);
-        tile_coords((int)(v - (unsigned)kz * nt), g.tiles_m, g.tiles_n, tm, tn);
+        const unsigned nt = (unsigned)(g.tiles_m * g.tiles_n);
+        int t;
+        if (g.tail_splits > 0 && (int)blockIdx.x >= g.main_blocks)
+        {
+            // pieces of the tail tiles keep the hardware's round-robin order: they are short and should spread over all XCDs
+            const int u = (int)blockIdx.x - g.main_blocks;
+            const int ti = u / g.tail_splits, piece = u - ti * g.tail_splits;
+            t = g.tail_first + ti;
+            kbeg = (int64_t)piece * g.tail_kps;
+            kend = (kbeg + g.tail_kps < g.K) ? kbeg + g.tail_kps : g.K;
+            tail_out = g.tail_ws + (int64_t)u * (BM * BN);
+        }
+        else
+        {
+            const unsigned total = g.tail_splits > 0 ? (unsigned)g.main_blocks : nt * (unsigned)g.splits;
+            const unsigned bid = blockIdx.x, nx = (unsigned)g.xcds;
+            const unsigned loc = bid / nx, xcd = bid - loc * nx;
+            const unsigned full = total / nx, rem = total - full * nx;
+            const unsigned v = xcd * full + (xcd < rem ? xcd : rem) + loc;
+            kz = (int)(v / nt);
+            t = (int)(v - (unsigned)kz * nt);
+            kbeg = (int64_t)kz * g.k_per_split;
+            kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
+        }
+        tile_coords(t, g.tiles_m, g.tiles_n, tm, tn);
     }
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-    const int64_t kbeg = (int64_t)kz * g.k_per_split;
-    const int64_t kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
     const int nkt = (int)((kend - kbeg + BK - 1) / BK);
     const int klen = (int)(kend - kbeg);
 
@@ -300,6 +318,18 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     }
 
     // accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
+    if (tail_out)
+    {
+        // K piece of a tail tile: the whole BM x BN partial, tile-local (rows or columns past the matrix hold zeros)
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int j = 0; j < CB; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    tail_out[(wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4)) * BN + wn + j * 32 + l32] = acc[i][j][r];
+        return;
+    }
     float *Cout = g.C + (int64_t)kz * g.c_split_stride;
 #pragma unroll
     for (int i = 0; i < RB; ++i)
@@ -332,7 +362,7 @@ bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g)
 {
     const bool aligned = ((reinterpret_cast<uintptr_t>(g.A) | reinterpret_cast<uintptr_t>(g.B)) % 16 == 0) &&
                          g.lda % 4 == 0 && g.ldb % 4 == 0 && (ta ? g.M : g.K) % 4 == 0 && (tb ? g.K : g.N) % 4 == 0 &&
-                         (g.splits == 1 || g.k_per_split % 32 == 0);
+                         (g.splits == 1 || g.k_per_split % 32 == 0) && (g.tail_splits == 0 || g.tail_kps % 16 == 0);
     // lane offsets are 32-bit and must stay below 2^31: the rows of a tile, or the K range of a slice, times the row length
     const int64_t a_span = (ta ? g.k_per_split + 64 : 128) * g.lda * 4, b_span = (tb ? 128 : g.k_per_split + 64) * g.ldb * 4;
     return aligned && a_span < (1ll << 31) && b_span < (1ll << 31) && g.M > 0 && g.N > 0 && g.K > 0;
@@ -340,7 +370,8 @@ bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g)
 
 int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st)
 {
-    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n * g.splits)), block(kNT);
+    const int64_t nt = (int64_t)g.tiles_m * g.tiles_n;
+    const dim3 grid((unsigned)(g.tail_splits > 0 ? g.main_blocks + (nt - g.tail_first) * g.tail_splits : nt * g.splits)), block(kNT);
 #define ODL_DMA_CASE(TA, TB)                                                                          \
     if (ta == TA && tb == TB)                                                                         \
     {                                                                                                 \
