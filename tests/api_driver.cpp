@@ -1227,6 +1227,64 @@ int cnn_bench_impl(int64_t N, int steps, int warmup, int graph_mode, float *ms_p
 
 extern "C" {
 #ifdef DRV_ON_DEVICE
+// A Linear or Conv2d that a ReLU follows inside a Sequential runs as one operator. The same network, the same input:
+// once through the Sequential, once module by module (nothing paired). diffs[0] counts output elements that differ in
+// any bit, diffs[1] the same over the gradients of all parameters and of the input.
+int DRV(paired_layers_match_separate_modules)(int64_t N, int64_t *diffs)
+{
+    return guarded([&] {
+        std::mt19937 gen(99);
+        Sequential model;
+        model.add(std::make_unique<nn::Conv2d>(3, 32, 3, 1, 1, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::MaxPool2d>(2, 2, 0));
+        model.add(std::make_unique<nn::Flatten>());
+        model.add(std::make_unique<nn::Linear>(32 * 8 * 8, 100, true));
+        model.add(std::make_unique<nn::ReLU>());
+        model.add(std::make_unique<nn::Linear>(100, 10, true));
+        *dynamic_cast<nn::Conv2d &>(model[0]).weight() = kaiming_uniform(gen, Shape{32, 3, 3, 3}, 27);
+        *dynamic_cast<nn::Linear &>(model[4]).weight() = kaiming_uniform(gen, Shape{32 * 8 * 8, 100}, 32 * 8 * 8);
+        *dynamic_cast<nn::Linear &>(model[6]).weight() = kaiming_uniform(gen, Shape{100, 10}, 100);
+        model.to(kDev);
+        model.train();
+        auto xv = uniform_vec(gen, (size_t)(N * 3 * 16 * 16), -1.0f, 1.0f);
+        std::vector<int64_t> tv((size_t)N);
+        for (auto &e : tv)
+            e = (int64_t)(gen() % 10u);
+        auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt64).device(kDev));
+        auto run = [&](bool paired, std::vector<std::vector<float>> &out) {
+            auto X = Tensor(xv, Shape{(size_t)N, 3, 16, 16}, dtype(DataType::kFloat32).device(kDev).requires_grad(true));
+            for (auto *p : model.parameters())
+                p->clear_grad();
+            Tensor y = X;
+            if (paired)
+                y = model(X);
+            else
+                for (size_t i = 0; i < model.size(); ++i)
+                    y = model[i].forward(y);
+            auto L = F::softmax_cross_entropy(y, T);
+            L.backward();
+            out.push_back(y.to_vector<float>());
+            out.push_back(X.grad().to_vector<float>());
+            for (auto *p : model.parameters())
+                out.push_back(p->grad().to_vector<float>());
+        };
+        std::vector<std::vector<float>> a, b;
+        run(true, a);
+        run(false, b);
+        diffs[0] = diffs[1] = 0;
+        for (size_t k = 0; k < a.size(); ++k)
+        {
+            if (a[k].size() != b[k].size())
+                throw std::runtime_error("paired and separate runs gave tensors of different sizes");
+            for (size_t i = 0; i < a[k].size(); ++i)
+                diffs[k == 0 ? 0 : 1] += std::memcmp(&a[k][i], &b[k][i], sizeof(float)) != 0;
+        }
+    });
+}
+#endif
+
+#ifdef DRV_ON_DEVICE
 // zeros / ones / full on the device queue their fill kernel only when the buffer is first asked for. What must hold:
 // out[0] the sum of a ones tensor that went to the host untouched (n); out[1] an accumulator made with zeros BEFORE a
 // capture and first touched inside it, after three replays of `acc += ones` (3 in every element: its fill ran before

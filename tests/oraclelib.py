@@ -106,6 +106,7 @@ _DEVICE_ONLY_SIGS = {
     "odl_host_upload_ordering": "lip>i",
     "odl_host_graph_abort_recovery": "pplllpp>i",
     "odl_host_pending_fill_semantics": "lp>i",
+    "odl_host_paired_layers_match_separate_modules": "lp>i",
 }
 
 

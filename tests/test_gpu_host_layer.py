@@ -256,6 +256,15 @@ def test_a_failed_capture_leaves_the_thread_usable_and_replays_report_bad_labels
     assert flags.tolist() == [1, 0]
 
 
+def test_a_layer_paired_with_its_relu_gives_the_bits_of_the_two_modules_run_in_turn(h):
+    """Sequential runs Linear+ReLU and Conv2d+ReLU as one operator each (activation in the epilogue, backward masked
+    with the output). The network's output and every gradient — parameters and input — must equal, bit for bit, what
+    the modules give when called one after the other (src/nn/sequential.cpp, src/operators/activation/relu.cpp)."""
+    diffs = np.full(2, -1, np.int64)
+    assert h.odl_host_paired_layers_match_separate_modules(64, diffs) == 0
+    assert diffs.tolist() == [0, 0], diffs
+
+
 def test_deferred_fills_behave_like_fills_at_creation(h):
     """zeros / ones / full queue their kernel at the first use of the buffer. Seen from outside nothing may change:
     a copy to the host sees the values, a buffer made before a capture is filled before it (not on every replay),
