@@ -1133,9 +1133,10 @@ def test_linear_with_the_activation_in_the_epilogue_equals_linear_then_relu(api)
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 64, 256), (200, 136, 520), (512, 1000, 784), (1024, 1024, 1024), (260, 2052, 4100),
-                                   (1536, 1536, 512)])
-def test_products_with_about_one_workgroup_per_compute_unit_in_all_four_layouts(api, M, N, K):
-    # The variant whose operands go from global memory straight into LDS (64x64 and 128x128 tiles, K in slices or whole):
+                                   (1536, 1536, 512), (2304, 2304, 512), (2560, 3072, 256)])
+def test_the_straight_to_lds_gemm_in_all_four_layouts_over_ragged_edges(api, M, N, K):
+    # The variant whose operands go from global memory straight into LDS (64x32, 64x64 and 128x128 tiles, K in slices or
+    # whole, 324 tiles whose last 68 are cut into K pieces, 480 tiles at two workgroups per compute unit):
     # ragged edges in M, N and K (zero-filled by the loads), the four operand layouts of
     # src/mat/origin/cpu/math/matmul.cpp:113-218 and src/operators/math/mat_mul.cpp:123-182, bias in the epilogue.
     L = api.lib()
