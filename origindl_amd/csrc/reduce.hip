@@ -280,11 +280,16 @@ __host__ inline ChannelSumPlan plan_channel_sum(int64_t N, int64_t OC, int64_t P
     return p;
 }
 
-// one workgroup per channel: channels for at least half the compute units, planes of whole quads, and enough elements
-// per channel that the single launch is the cheaper schedule
+// one workgroup per channel when the single launch is the cheaper schedule: channels for at least half the compute
+// units, or fewer channels (32 and up) of at most 400 KB each, which one compute unit reads in the time the second
+// launch of the two-pass schedule would take; planes of whole quads
 __host__ inline bool channel_sum_whole(int64_t N, int64_t OC, int64_t P)
 {
-    return OC * 2 >= odl::device_cus() && P % 4 == 0 && N * P >= 32 * 1024 && N * P < (1ll << 31);
+    const int64_t per_channel = N * P;
+    if (P % 4 != 0 || per_channel >= (1ll << 31))
+        return false;
+    return (OC * 2 >= odl::device_cus() && per_channel >= 32 * 1024) ||
+           (OC >= 32 && per_channel >= 16 * 1024 && per_channel <= 100 * 1024);
 }
 
 template <bool V4>
