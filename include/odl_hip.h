@@ -348,6 +348,15 @@ int odl_hip_batch_norm_backward_from_x(const float *gy, const float *x, const fl
                                        void *stream);
 /* workspace of either call (partial channel sums) */
 size_t odl_hip_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t P);
+/* The same on float64 tensors (src/mat/origin/cuda/normalization/batch_norm.cu:497-560 accepts float32 and float64): one
+ * workgroup per channel, no workspace. x_norm may be NULL. backward: x_norm_or_x is the saved normalised input
+ * (from_x = 0), or x itself with saved_mean (from_x != 0). */
+int odl_hip_batch_norm_forward_f64(const double *x, const double *gamma, const double *beta, const double *running_mean,
+                                   const double *running_var, int training, double eps, int64_t N, int64_t C, int64_t P,
+                                   double *y, double *mean, double *var, double *x_norm, void *stream);
+int odl_hip_batch_norm_backward_f64(const double *gy, const double *x_norm_or_x, int from_x, const double *gamma,
+                                    const double *saved_mean, const double *saved_var, double eps, int64_t N, int64_t C,
+                                    int64_t P, double *gx, double *dgamma, double *dbeta, void *stream);
 /* out = a*x + b*y, each product rounded before the sum: the running-statistics update of the BatchNorm layers
  * (src/nn/layers/batch_norm2d.cpp:77-80, batch_norm1d.cpp), which the reference does on the host after four
  * device-to-host copies. out may be x or y. */

@@ -433,6 +433,133 @@ int odl_hip_batch_norm_backward_from_x(const float *gy, const float *x, const fl
                               workspace_bytes, stream);
 }
 
+// ---- float64 (src/mat/origin/cuda/normalization/batch_norm.cu:497-560 runs the same algorithm on doubles). Not a hot
+// path: one workgroup per channel walks the channel's N*P elements three times (sum, squared deviations, apply), the
+// sums reduced in a fixed order.
+}  // extern "C"
+
+namespace
+{
+__device__ inline double block_sum_f64(double v, double *sh)
+{
+    for (int off = 32; off > 0; off >>= 1)
+        v += __shfl_down(v, off, 64);
+    if ((threadIdx.x & 63) == 0)
+        sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    double s = 0.0;
+    for (int i = 0; i < kBlock / 64; ++i)
+        s += sh[i];
+    __syncthreads();
+    return s;  // the same value in every thread
+}
+
+__global__ __launch_bounds__(kBlock) void bn_forward_f64_kernel(const double *__restrict__ x, const double *__restrict__ gamma,
+                                                                const double *__restrict__ beta,
+                                                                const double *__restrict__ running_mean,
+                                                                const double *__restrict__ running_var, int training,
+                                                                double eps, int64_t N, int64_t C, int64_t P,
+                                                                double *__restrict__ y, double *__restrict__ mean_out,
+                                                                double *__restrict__ var_out, double *__restrict__ x_norm)
+{
+    __shared__ double sh[kBlock / 64];
+    const int64_t c = blockIdx.x, total = N * P;
+    auto at = [&](int64_t i) { return ((i / P) * C + c) * P + i % P; };
+    double mean, var;
+    if (training)
+    {
+        double acc = 0.0;
+        for (int64_t i = threadIdx.x; i < total; i += kBlock)
+            acc += x[at(i)];
+        mean = block_sum_f64(acc, sh) / (double)total;
+        acc = 0.0;
+        for (int64_t i = threadIdx.x; i < total; i += kBlock)
+        {
+            const double d = x[at(i)] - mean;
+            acc += d * d;
+        }
+        var = block_sum_f64(acc, sh) / (double)total;
+    }
+    else
+        mean = running_mean[c], var = running_var[c];
+    if (threadIdx.x == 0)
+        mean_out[c] = mean, var_out[c] = var;
+    const double stdv = sqrt(var + eps), ga = gamma[c], be = beta[c];
+    for (int64_t i = threadIdx.x; i < total; i += kBlock)
+    {
+        const int64_t off = at(i);
+        const double xn = (x[off] - mean) / stdv;
+        if (x_norm)
+            x_norm[off] = xn;
+        y[off] = ga * xn + be;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void bn_backward_f64_kernel(const double *__restrict__ gy, const double *__restrict__ xn_or_x,
+                                                                 int from_x, const double *__restrict__ gamma,
+                                                                 const double *__restrict__ mean,
+                                                                 const double *__restrict__ var, double eps, int64_t N,
+                                                                 int64_t C, int64_t P, double *__restrict__ gx,
+                                                                 double *__restrict__ dgamma, double *__restrict__ dbeta)
+{
+    __shared__ double sh[kBlock / 64];
+    const int64_t c = blockIdx.x, total = N * P;
+    auto at = [&](int64_t i) { return ((i / P) * C + c) * P + i % P; };
+    const double mu = from_x ? mean[c] : 0.0, sd = sqrt(var[c] + eps);
+    auto norm = [&](int64_t off) { return from_x ? (xn_or_x[off] - mu) / sd : xn_or_x[off]; };
+    double a = 0.0, b = 0.0;
+    for (int64_t i = threadIdx.x; i < total; i += kBlock)
+    {
+        const int64_t off = at(i);
+        a += gy[off];
+        b += gy[off] * norm(off);
+    }
+    const double sum_gy = block_sum_f64(a, sh), sum_gy_xn = block_sum_f64(b, sh);
+    if (threadIdx.x == 0)
+        dgamma[c] = sum_gy_xn, dbeta[c] = sum_gy;
+    const double mean_gy = sum_gy / (double)total, mean_gy_xn = sum_gy_xn / (double)total, scale = gamma[c] / sd;
+    for (int64_t i = threadIdx.x; i < total; i += kBlock)
+    {
+        const int64_t off = at(i);
+        gx[off] = scale * ((gy[off] - mean_gy) - norm(off) * mean_gy_xn);
+    }
+}
+}  // namespace
+
+extern "C" {
+
+int odl_hip_batch_norm_forward_f64(const double *x, const double *gamma, const double *beta, const double *running_mean,
+                                   const double *running_var, int training, double eps, int64_t N, int64_t C, int64_t P,
+                                   double *y, double *mean, double *var, double *x_norm, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C > 0 && P > 0 && C < (1ll << 31), "batch_norm: bad shape (N=%lld, C=%lld, P=%lld)", (long long)N,
+                (long long)C, (long long)P);
+    ODL_REQUIRE(x && gamma && beta && y && mean && var, "batch_norm: null operand");
+    ODL_REQUIRE(training || (running_mean && running_var), "batch_norm: evaluation mode needs the running statistics");
+    if (N == 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(bn_forward_f64_kernel, dim3((unsigned)C), dim3(kBlock), 0, odl::as_stream(stream), x, gamma, beta,
+                       running_mean, running_var, training, eps, N, C, P, y, mean, var, x_norm);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_batch_norm_backward_f64(const double *gy, const double *x_norm_or_x, int from_x, const double *gamma,
+                                    const double *saved_mean, const double *saved_var, double eps, int64_t N, int64_t C,
+                                    int64_t P, double *gx, double *dgamma, double *dbeta, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N > 0 && C > 0 && P > 0 && C < (1ll << 31), "batch_norm_backward: bad shape (N=%lld, C=%lld, P=%lld)",
+                (long long)N, (long long)C, (long long)P);
+    ODL_REQUIRE(gy && gamma && saved_var && x_norm_or_x && gx && dgamma && dbeta && (!from_x || saved_mean),
+                "batch_norm_backward: null operand");
+    hipLaunchKernelGGL(bn_backward_f64_kernel, dim3((unsigned)C), dim3(kBlock), 0, odl::as_stream(stream), gy, x_norm_or_x,
+                       from_x, gamma, saved_mean, saved_var, eps, N, C, P, gx, dgamma, dbeta);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
 int odl_hip_axpby(float a, const float *x, float b, const float *y, int64_t n, float *out, void *stream)
 {
     ODL_REQUIRE_DEVICE();

@@ -898,6 +898,54 @@ BnShape bn_check(const char *who, const OriginMat &x, int num_dims, const Mat &g
     return BnShape{(int64_t)x.shape()[0], (int64_t)C,
                    num_dims == 4 ? (int64_t)(x.shape()[2] * x.shape()[3]) : (int64_t)1};
 }
+
+const double *dp(const OriginMat &m)
+{
+    return static_cast<const double *>(m.storage()->data());
+}
+double *dp(OriginMat &m)
+{
+    return static_cast<double *>(m.storage()->data());
+}
+
+// float64 tensors take the same path on doubles (src/mat/origin/cuda/normalization/batch_norm.cu:497-560)
+Mat::BatchNormResult bn_forward_f64(const OriginMat &self, const BnShape &s, const Mat &gamma, const Mat &beta,
+                                    const Mat &rm_, const Mat &rv_, bool training, float eps, bool with_x_norm)
+{
+    const OriginMat &x = dev_any(self, "batch_norm"), &g = dev_any(gamma, "batch_norm"), &b = dev_any(beta, "batch_norm");
+    const OriginMat &rm = dev_any(rm_, "batch_norm"), &rv = dev_any(rv_, "batch_norm");
+    Mat::BatchNormResult r;
+    auto y = new_like(x, x.shape(), DataType::kFloat64);
+    auto mean = new_like(x, Shape({(size_t)s.C}), DataType::kFloat64), var = new_like(x, Shape({(size_t)s.C}), DataType::kFloat64);
+    std::unique_ptr<OriginMat> xn;
+    if (with_x_norm)
+        xn = new_like(x, x.shape(), DataType::kFloat64);
+    check(odl_hip_batch_norm_forward_f64(dp(x), dp(g), dp(b), dp(rm), dp(rv), training ? 1 : 0, (double)eps, s.N, s.C, s.P,
+                                         dp(*y), dp(*mean), dp(*var), xn ? dp(*xn) : nullptr, cur()));
+    r.y = std::move(y), r.mean = std::move(mean), r.var = std::move(var);
+    if (xn)
+        r.x_norm = std::move(xn);
+    return r;
+}
+
+std::vector<std::unique_ptr<Mat>> bn_backward_f64(const OriginMat &self, const Mat &gym, const Mat &xn_or_x, bool from_x,
+                                                  const Mat &gamma, const Mat &saved_mean, const Mat &saved_var, float eps,
+                                                  int num_dims)
+{
+    const OriginMat &x = dev_any(self, "batch_norm_backward"), &gy = dev_any(gym, "batch_norm_backward");
+    const OriginMat &src = dev_any(xn_or_x, "batch_norm_backward"), &g = dev_any(gamma, "batch_norm_backward");
+    const OriginMat &sm = dev_any(saved_mean, "batch_norm_backward"), &sv = dev_any(saved_var, "batch_norm_backward");
+    const size_t C = x.shape()[1];
+    const int64_t N = (int64_t)x.shape()[0], P = num_dims == 4 ? (int64_t)(x.shape()[2] * x.shape()[3]) : 1;
+    auto gx = new_like(x, x.shape(), DataType::kFloat64);
+    auto dgamma = new_like(x, Shape({C}), DataType::kFloat64), dbeta = new_like(x, Shape({C}), DataType::kFloat64);
+    if (N > 0)
+        check(odl_hip_batch_norm_backward_f64(dp(gy), dp(src), from_x ? 1 : 0, dp(g), dp(sm), dp(sv), (double)eps, N,
+                                              (int64_t)C, P, dp(*gx), dp(*dgamma), dp(*dbeta), cur()));
+    std::vector<std::unique_ptr<Mat>> outs;
+    outs.push_back(std::move(gx)), outs.push_back(std::move(dgamma)), outs.push_back(std::move(dbeta));
+    return outs;
+}
 }  // namespace
 
 Mat::BatchNormResult OriginMat::batch_norm_forward(const Mat &gamma, const Mat &beta, const Mat &running_mean,
@@ -905,6 +953,8 @@ Mat::BatchNormResult OriginMat::batch_norm_forward(const Mat &gamma, const Mat &
                                                    int num_dims) const
 {
     const BnShape s = bn_check("batch_norm", *this, num_dims, gamma, beta, running_mean, running_var);
+    if (dtype_ == DataType::kFloat64)
+        return bn_forward_f64(*this, s, gamma, beta, running_mean, running_var, training, eps, true);
     const OriginMat &x = dev_f32(*this, "batch_norm");
     const OriginMat &g = dev_f32(gamma, "batch_norm"), &b = dev_f32(beta, "batch_norm");
     const OriginMat &rm = dev_f32(running_mean, "batch_norm"), &rv = dev_f32(running_var, "batch_norm");
@@ -924,6 +974,8 @@ Mat::BatchNormResult OriginMat::batch_norm_forward_no_xnorm(const Mat &gamma, co
                                                             int num_dims) const
 {
     const BnShape s = bn_check("batch_norm", *this, num_dims, gamma, beta, running_mean, running_var);
+    if (dtype_ == DataType::kFloat64)
+        return bn_forward_f64(*this, s, gamma, beta, running_mean, running_var, training, eps, false);
     const OriginMat &x = dev_f32(*this, "batch_norm");
     const OriginMat &g = dev_f32(gamma, "batch_norm"), &b = dev_f32(beta, "batch_norm");
     const OriginMat &rm = dev_f32(running_mean, "batch_norm"), &rv = dev_f32(running_var, "batch_norm");
@@ -949,6 +1001,8 @@ std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward_from_x(const Ma
     if (gym.shape() != shape_ || gamma.shape() != Shape({C}) || saved_mean.shape() != Shape({C}) ||
         saved_var.shape() != Shape({C}))
         THROW_INVALID_ARG("batch_norm_backward: shape mismatch");
+    if (dtype_ == DataType::kFloat64)
+        return bn_backward_f64(*this, gym, *this, true, gamma, saved_mean, saved_var, eps, num_dims);
     const OriginMat &x = dev_f32(*this, "batch_norm_backward");
     const OriginMat &gy = dev_f32(gym, "batch_norm_backward"), &g = dev_f32(gamma, "batch_norm_backward");
     const OriginMat &sm = dev_f32(saved_mean, "batch_norm_backward"), &sv = dev_f32(saved_var, "batch_norm_backward");
@@ -968,6 +1022,8 @@ std::unique_ptr<Mat> OriginMat::batch_norm(const Mat &gamma, const Mat &beta, co
                                            const Mat &running_var, bool training, float eps, float, int num_dims) const
 {
     const BnShape s = bn_check("batch_norm", *this, num_dims, gamma, beta, running_mean, running_var);
+    if (dtype_ == DataType::kFloat64)
+        return std::move(bn_forward_f64(*this, s, gamma, beta, running_mean, running_var, training, eps, false).y);
     const OriginMat &x = dev_f32(*this, "batch_norm");
     const OriginMat &g = dev_f32(gamma, "batch_norm"), &b = dev_f32(beta, "batch_norm");
     const OriginMat &rm = dev_f32(running_mean, "batch_norm"), &rv = dev_f32(running_var, "batch_norm");
@@ -998,6 +1054,8 @@ std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward(const Mat &gym,
         saved_var.dtype() != dtype() || saved_x_norm.dtype() != dtype())
         THROW_INVALID_ARG("batch_norm_backward: all inputs (gy, x, gamma, saved_mean, saved_var, saved_x_norm) must "
                           "have the same floating-point dtype");
+    if (dtype_ == DataType::kFloat64)
+        return bn_backward_f64(*this, gym, saved_x_norm, false, gamma, saved_mean, saved_var, eps, num_dims);
     const OriginMat &x = dev_f32(*this, "batch_norm_backward");
     const OriginMat &gy = dev_f32(gym, "batch_norm_backward"), &g = dev_f32(gamma, "batch_norm_backward");
     const OriginMat &sv = dev_f32(saved_var, "batch_norm_backward"), &xn = dev_f32(saved_x_norm, "batch_norm_backward");

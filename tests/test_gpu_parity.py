@@ -1158,3 +1158,50 @@ def test_the_straight_to_lds_gemm_in_all_four_layouts_over_ragged_edges(api, M, 
             L.call("odl_hip_sgemm", ta, tb, M, N, K, da.data_ptr(), da.shape[1], db.data_ptr(), db.shape[1], c.data_ptr(), N,
                    dev(bias).data_ptr(), 0, ws.data_ptr(), nb, None)
             assert np.array_equal(host(c), (got.astype(np.float32) + bias)), (ta, tb, "bias")
+
+
+def test_float64_batch_norm_matches_float64_numpy(api):
+    # src/mat/origin/cuda/normalization/batch_norm.cu:497-560 and its backward: the float32 algorithm on doubles
+    # (two-pass statistics, biased variance); checked against numpy in float64, [N,C] and [N,C,H,W], both forms of backward
+    import ctypes
+    L = api.lib()
+    rng = np.random.default_rng(5)
+    for N, C, P in ((6, 5, 1), (4, 3, 35), (2, 2, 1)):
+        x = rng.standard_normal((N, C, P)) * 2 + 1
+        gamma, beta = rng.standard_normal(C) + 1.5, rng.standard_normal(C)
+        rm, rv = rng.standard_normal(C), rng.random(C) + 0.5
+        gy = rng.standard_normal((N, C, P))
+        eps = 1e-5
+        d = {k: dev(v) for k, v in dict(x=x, gamma=gamma, beta=beta, rm=rm, rv=rv, gy=gy).items()}
+        y, xn = torch.empty_like(d["x"]), torch.empty_like(d["x"])
+        mean, var = torch.empty(C, dtype=torch.float64, device="cuda"), torch.empty(C, dtype=torch.float64, device="cuda")
+        for training in (1, 0):
+            L.call("odl_hip_batch_norm_forward_f64", d["x"].data_ptr(), d["gamma"].data_ptr(), d["beta"].data_ptr(),
+                   d["rm"].data_ptr(), d["rv"].data_ptr(), training, ctypes.c_double(eps), N, C, P, y.data_ptr(),
+                   mean.data_ptr(), var.data_ptr(), xn.data_ptr(), None)
+            m = x.mean(axis=(0, 2)) if training else rm
+            v = ((x - m[None, :, None]) ** 2).mean(axis=(0, 2)) if training else rv
+            want_xn = (x - m[None, :, None]) / np.sqrt(v + eps)[None, :, None]
+            np.testing.assert_allclose(host(mean), m, rtol=1e-13, atol=1e-14)
+            np.testing.assert_allclose(host(var), v, rtol=1e-12, atol=1e-14)
+            np.testing.assert_allclose(host(xn), want_xn, rtol=1e-11, atol=1e-12)
+            np.testing.assert_allclose(host(y), gamma[None, :, None] * want_xn + beta[None, :, None], rtol=1e-11, atol=1e-12)
+        # backward with the batch statistics of the training forward
+        m = x.mean(axis=(0, 2))
+        v = ((x - m[None, :, None]) ** 2).mean(axis=(0, 2))
+        sd = np.sqrt(v + eps)
+        want_xn = (x - m[None, :, None]) / sd[None, :, None]
+        dm, dv = dev(m), dev(v)
+        dxn = dev(want_xn)
+        gx = torch.empty_like(d["x"])
+        dgamma, dbeta = torch.empty(C, dtype=torch.float64, device="cuda"), torch.empty(C, dtype=torch.float64, device="cuda")
+        want_dgamma, want_dbeta = (gy * want_xn).sum(axis=(0, 2)), gy.sum(axis=(0, 2))
+        cnt = N * P
+        want_gx = (gamma / sd)[None, :, None] * (gy - (want_dbeta / cnt)[None, :, None] - want_xn * (want_dgamma / cnt)[None, :, None])
+        for from_x, src in ((0, dxn), (1, d["x"])):
+            L.call("odl_hip_batch_norm_backward_f64", d["gy"].data_ptr(), src.data_ptr(), from_x, d["gamma"].data_ptr(),
+                   dm.data_ptr(), dv.data_ptr(), ctypes.c_double(eps), N, C, P, gx.data_ptr(), dgamma.data_ptr(),
+                   dbeta.data_ptr(), None)
+            np.testing.assert_allclose(host(dgamma), want_dgamma, rtol=1e-11, atol=1e-12)
+            np.testing.assert_allclose(host(dbeta), want_dbeta, rtol=1e-11, atol=1e-12)
+            np.testing.assert_allclose(host(gx), want_gx, rtol=1e-10, atol=1e-11)
