@@ -10,6 +10,7 @@
 //             [N*OH*OW, OC] matrix exactly as it lies (conv2d.cpp:548) — free on the GPU: it is the same pointer.
 //   col2im is a gather: one thread owns one image pixel and adds its taps in ascending (kh, kw) order, which
 //   is the order in which the reference's scatter loop reaches that pixel — bit-identical sums, no atomics.
+#include "gemm_dma.h"
 #include "odl_common.h"
 
 #include <algorithm>
@@ -895,6 +896,10 @@ int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packe
     if (M == 0)
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
+    // a 1x1 window at stride 1 is a plain product per image, y[n] = W . x[n]: operands straight into LDS, bias and
+    // activation in the epilogue, the output already NCHW (no K slices, no second launch)
+    if (KH == 1 && KW == 1 && SH == 1 && SW == 1 && PH == 0 && PW == 0 && odl::conv1x1_dma_ok(x, w, N, C, H * W, OC))
+        return odl::conv1x1_dma(x, w, b, y, N, C, H * W, OC, act, st);
     if (odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, g.OH, g.OW))
         return odl::conv_small_forward(x, w, b, y, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, act, st);
     if (odl::conv_patch_forward_ok(x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW) &&

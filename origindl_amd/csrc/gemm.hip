@@ -885,6 +885,7 @@ odl::DmaGemmArgs dma_args(const GemmArgs &g, int epi)
     d.epi = epi == EPI_BIAS_COL ? 1 : 0, d.act = g.act, d.xcds = g.xcds;
     d.main_blocks = g.main_blocks, d.tail_first = g.tail_first, d.tail_splits = g.tail_splits, d.tail_kps = g.tail_kps;
     d.tail_ws = g.tail_ws;
+    d.batch = 1, d.a_batch = d.b_batch = d.c_batch = 0;
     return d;
 }
 

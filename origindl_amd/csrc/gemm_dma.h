@@ -15,7 +15,7 @@ struct DmaGemmArgs
     int tiles_m, tiles_n, splits;
     int64_t k_per_split;     // K range of one slice (a multiple of 32)
     int64_t c_split_stride;  // distance between the partial outputs of two slices (0 when splits == 1)
-    int epi;                 // 0 plain, 1 bias by column then the activation
+    int epi;                 // 0 plain, 1 bias by column then the activation, 2 bias by row then the activation
     int act;                 // 0 none, 1 relu, 2 silu
     int xcds;
     // Tail split (0 pieces: none): the tiles from tail_first on are cut into tail_splits runs of tail_kps K values each,
@@ -24,6 +24,10 @@ struct DmaGemmArgs
     int main_blocks, tail_first, tail_splits;
     int64_t tail_kps;
     float *tail_ws;
+    // `batch` independent products in one launch (1: a single product): product z reads A + z*a_batch, B + z*b_batch
+    // and writes C + z*c_batch (elements). Not combined with K slices or a split tail.
+    int batch;
+    int64_t a_batch, b_batch, c_batch;
 };
 
 // true when the shape suits the variant (16-byte aligned rows, offsets within 31 bits)
@@ -32,4 +36,10 @@ bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g);
 // tiles in 16-wide slabs, two workgroups per compute unit: for launches of many tiles); the grid is
 // tiles_m * tiles_n * splits workgroups of 512 threads (main_blocks + tail tiles * tail_splits with a tail split)
 int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st);
+
+// 1x1 / stride 1 / unpadded convolution as `N` products y[n] = act(W[OC,C] . x[n][C, H*W] + b[oc]) in one launch; false
+// when the shape does not suit (rows of H*W or C floats that are not multiples of four, unaligned pointers)
+bool conv1x1_dma_ok(const float *x, const float *w, int64_t N, int64_t C, int64_t HW, int64_t OC);
+int conv1x1_dma(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t HW, int64_t OC,
+                int act, hipStream_t st);
 }  // namespace odl

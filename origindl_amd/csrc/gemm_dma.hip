@@ -26,7 +26,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kNT     = 512;
 constexpr int kStages = 4;
-constexpr int kEpiBiasCol = 1;
+constexpr int kEpiBiasCol = 1, kEpiBiasRow = 2;
 constexpr unsigned kOutside = 0x80000000u;  // beyond the 2^31 - 1 bytes every buffer descriptor here declares
 
 __device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     const int wm = (wave / WAVES_N) * (BM / WAVES_M), wn = (wave % WAVES_N) * (BN / WAVES_N);
 
     // workgroup -> (K slice, tile): a contiguous band of workgroups per XCD, tiles in groups of 8 tile-rows
-    int tm, tn, kz = 0;
+    int tm, tn, kz = 0, bz = 0;
     int64_t kbeg, kend;
     float *tail_out = nullptr;
     {
@@ -127,11 +127,16 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
         }
         else
         {
-            const unsigned total = g.tail_splits > 0 ? (unsigned)g.main_blocks : nt * (unsigned)g.splits;
+            const unsigned total = g.tail_splits > 0 ? (unsigned)g.main_blocks : nt * (unsigned)g.splits * (unsigned)g.batch;
             const unsigned bid = blockIdx.x, nx = (unsigned)g.xcds;
             const unsigned loc = bid / nx, xcd = bid - loc * nx;
             const unsigned full = total / nx, rem = total - full * nx;
-            const unsigned v = xcd * full + (xcd < rem ? xcd : rem) + loc;
+            unsigned v = xcd * full + (xcd < rem ? xcd : rem) + loc;
+            if (g.batch > 1)
+            {
+                bz = (int)(v / nt);  // one K slice per product when there are several
+                v -= (unsigned)bz * nt;
+            }
             kz = (int)(v / nt);
             t = (int)(v - (unsigned)kz * nt);
             kbeg = (int64_t)kz * g.k_per_split;
@@ -144,8 +149,8 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     const int klen = (int)(kend - kbeg);
 
     // buffer descriptors based at this workgroup's corner of each operand; every lane offset is relative to it
-    const float *abase = g.A + (A_KMAJOR ? m0 * g.lda + kbeg : kbeg * g.lda + m0);
-    const float *bbase = g.B + (B_KMAJOR ? n0 * g.ldb + kbeg : kbeg * g.ldb + n0);
+    const float *abase = g.A + (int64_t)bz * g.a_batch + (A_KMAJOR ? m0 * g.lda + kbeg : kbeg * g.lda + m0);
+    const float *bbase = g.B + (int64_t)bz * g.b_batch + (B_KMAJOR ? n0 * g.ldb + kbeg : kbeg * g.ldb + n0);
     const i32x4 ra = buffer_of(abase), rb = buffer_of(bbase);
     const unsigned as_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) float *)&As[0][0];
     const unsigned bs_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) float *)&Bs[0][0];
@@ -330,7 +335,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
                     tail_out[(wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4)) * BN + wn + j * 32 + l32] = acc[i][j][r];
         return;
     }
-    float *Cout = g.C + (int64_t)kz * g.c_split_stride;
+    float *Cout = g.C + (int64_t)kz * g.c_split_stride + (int64_t)bz * g.c_batch;
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
@@ -350,6 +355,8 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
                 float v = acc[i][j][r];
                 if (with_bias)
                     v = odl::apply_act(v + bcol, g.act);
+                else if (g.epi == kEpiBiasRow)
+                    v = odl::apply_act(g.bias ? v + g.bias[row] : v, g.act);
                 Cout[row * g.ldc + col] = v;
             }
         }
@@ -371,12 +378,16 @@ bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g)
 int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st)
 {
     const int64_t nt = (int64_t)g.tiles_m * g.tiles_n;
-    const dim3 grid((unsigned)(g.tail_splits > 0 ? g.main_blocks + (nt - g.tail_first) * g.tail_splits : nt * g.splits)), block(kNT);
+    const dim3 grid((unsigned)(g.tail_splits > 0 ? g.main_blocks + (nt - g.tail_first) * g.tail_splits
+                                                 : nt * g.splits * (g.batch > 1 ? g.batch : 1))),
+        block(kNT);
 #define ODL_DMA_CASE(TA, TB)                                                                          \
     if (ta == TA && tb == TB)                                                                         \
     {                                                                                                 \
         if (tile == 64)                                                                               \
             hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 1>), grid, block, 0, st, g);     \
+        else if (tile == 65)                                                                          \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 2>), grid, block, 0, st, g);     \
         else if (tile == 32)                                                                          \
             hipLaunchKernelGGL((sgemm_dma_kernel<64, 32, 64, TA, TB, 1, 4>), grid, block, 0, st, g);  \
         else if (tile == 128)                                                                         \
@@ -391,5 +402,32 @@ int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream
     ODL_DMA_CASE(true, true)
 #undef ODL_DMA_CASE
     return ODL_ERR_RUNTIME;
+}
+
+bool conv1x1_dma_ok(const float *x, const float *w, int64_t N, int64_t C, int64_t HW, int64_t OC)
+{
+    return N >= 1 && N < 65536 && C >= 4 && C % 4 == 0 && HW >= 4 && HW % 4 == 0 && OC >= 1 &&
+           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0) &&
+           (C + 64) * HW * 4 < (1ll << 31) && 128 * C * 4 < (1ll << 31) &&
+           ceil_div(OC, 64) * ceil_div(HW, 32) * N < (1ll << 31);
+}
+
+int conv1x1_dma(const float *x, const float *w, const float *b, float *y, int64_t N, int64_t C, int64_t HW, int64_t OC,
+                int act, hipStream_t st)
+{
+    DmaGemmArgs g{};
+    g.A = w, g.B = x, g.bias = b, g.C = y;
+    g.M = OC, g.N = HW, g.K = C, g.lda = C, g.ldb = HW, g.ldc = HW;
+    g.splits = 1, g.k_per_split = ceil_div(C, 64) * 64, g.c_split_stride = 0;
+    g.epi = 2, g.act = act, g.xcds = chip().xcds;
+    g.tail_splits = 0, g.main_blocks = 0, g.tail_kps = 0, g.tail_ws = nullptr;
+    g.batch = (int)N, g.a_batch = 0, g.b_batch = C * HW, g.c_batch = OC * HW;
+    // 64x64 tiles when they occupy the chip (two workgroups per compute unit once there are more than the chip holds
+    // singly), 64x32 tiles for the small images
+    const int64_t t64 = ceil_div(OC, 64) * ceil_div(HW, 64) * N, cus = device_cus();
+    int tile = t64 >= cus / 2 ? (t64 > cus + cus / 4 ? 65 : 64) : 32;
+    g.tiles_m = (int)ceil_div(OC, 64), g.tiles_n = (int)ceil_div(HW, tile == 32 ? 32 : 64);
+    g.tail_first = g.tiles_m * g.tiles_n;
+    return sgemm_dma_launch(tile, false, false, g, st);
 }
 }  // namespace odl
