@@ -1,21 +1,25 @@
 // FP32 GEMM on v_mfma_f32_32x32x2_f32 whose operands travel from global memory into LDS without passing through
 // registers (buffer_load ... lds, 16 bytes per lane), four K slabs deep.
 //
-// For products with about one workgroup per compute unit. There nothing else runs on the compute unit while a workgroup
-// waits: with operands staged through registers, every slab costs the wait for its loads plus the LDS stores in front of
-// the barrier, and the matrix pipe idles through both (1024x1024x4096: 99 us with staging, 72 us with the staging taken
-// out). Here a slab's loads are queued three slabs ahead and land in LDS on their own; a wave only waits for loads that
-// were queued three barriers ago, then reads its fragments and issues its matrix instructions.
+// Why. With operands staged through registers, every K slab costs the wait for its loads plus the LDS stores in front
+// of the barrier, and the staging instructions compete with the matrix instructions for issue slots. A workgroup that is
+// alone on its compute unit idles the matrix pipe through all of that (1024x1024x4096: 99 us with staging, 72 us with the
+// staging taken out as an experiment, 73 us here); on launches of many tiles the difference is 82 -> 88 % of the matrix
+// peak at 4096^3. Here a slab's loads are queued three slabs ahead and land in LDS on their own; a wave only waits for
+// loads that were queued three barriers ago, then reads its fragments and issues its matrix instructions.
 //
-//   * 512 threads: two sets of four waves on the tile; of the 8-wide K steps of a slab each set multiplies every other
-//     one, and the second set's accumulators join the first's through LDS before the epilogue.
+//   * 512 threads: KSETS sets of waves share one tile (2 sets of four waves on square tiles, 4 sets of two waves on the
+//     64x32 tile); of the 8-wide K steps of a slab each set multiplies every KSETS-th one, and the other sets'
+//     accumulators join the first's through LDS before the epilogue, added in set order.
 //   * LDS holds the operand tiles exactly as the loads deliver them: lane i of a wave's load lands at base + 16*i.
 //       K-contiguous operand (A of A.B, B of A.B^T): tile [rows][BK], a row's 16-byte pieces permuted by
-//         piece ^ (row & (BK/4-1)) — chosen on the global side, so that the 8 rows one ds_read_b128 phase touches fall
-//         into 8 different bank groups;
+//         piece ^ swizzle(row) — chosen on the global side, so that the 8 rows one ds_read_b128 phase touches fall into
+//         8 different bank groups although the rows are not padded;
 //       row-contiguous operand (A of A^T.B, B of A.B): tile [BK][cols], read back with ds_read_b32, lanes along cols.
 //   * Rows, columns and K positions outside the matrix: the lane's offset is set past the buffer's size and the load
-//     delivers zeros.
+//     delivers zeros, so ragged edges need no separate code.
+//   * Instances: 128x128x16 at two workgroups per compute unit (many tiles; a short last round as K pieces), 128x128x32,
+//     64x64x32 and 64x32x64 at one (few tiles), 64x64x32 at two (batches of small products: 1x1 convolutions).
 #include "gemm_dma.h"
 #include "odl_common.h"
 
