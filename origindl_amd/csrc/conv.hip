@@ -646,6 +646,125 @@ __global__ __launch_bounds__(256) void col2im_tile_kernel(const float *__restric
     }
 }
 
+// Matrix layout, 3x3 / stride 1 / padding 1, the streaming form. The tile kernel above re-reads the col rows of a
+// tile's halo and reads 144-byte runs that straddle 128-byte lines: about 2.3 times the matrix passes from L2 to LDS.
+// Here a workgroup owns one image, eight channels (288 bytes of every col row: 18 whole 16-byte pieces) and a band
+// of image rows, and walks down the band: LDS keeps four rows of output positions ([W positions][72 floats] each, as
+// the loads deliver them); while image row h is summed from position rows h-1, h, h+1, the rows h+2 and h+3 are on
+// their way in registers. Every col row of the band is read once, plus one halo row above and below the band. Lanes
+// run along (pixel, channel) with the channel fastest: the LDS addresses w*72 + c*9 + tap of a wave fall into 32
+// different banks. Taps are added in ascending (kh, kw), absent ones as +0.0f — the sums of the tile kernel, bit for bit.
+constexpr int kRowsCT = 8, kRowsRun = kRowsCT * 9, kRowsNT = 512, kRowsQ = 2;  // quads of a position row per thread: W * 18 <= 2 * 512
+
+__global__ __launch_bounds__(kRowsNT, 2) void col2im_rows3x3_kernel(const float *__restrict__ col, float *__restrict__ img, int N,
+                                                             int C, int H, int W, int band, int nbands, unsigned xcds)
+{
+    extern __shared__ float sh_rows[];
+    const int t = threadIdx.x;
+    const int slot_floats = W * kRowsRun, quads = W * (kRowsRun / 4), K = C * 9;
+    unsigned vb;
+    {
+        const unsigned nb = gridDim.x, bid = blockIdx.x;
+        const unsigned loc = bid / xcds, xcd = bid - loc * xcds, full = nb / xcds, rem = nb - full * xcds;
+        vb = xcd * full + (xcd < rem ? xcd : rem) + loc;
+    }
+    const int cchunks = C / kRowsCT;
+    const int cc = (int)(vb % (unsigned)cchunks);
+    vb /= (unsigned)cchunks;
+    const int b = (int)(vb % (unsigned)nbands), n = (int)(vb / (unsigned)nbands);
+    const int h0 = b * band, h1 = (h0 + band < H) ? h0 + band : H, c0 = cc * kRowsCT;
+    const float *src = col + (int64_t)n * H * W * K + c0 * 9;
+
+    f32x4 r0[kRowsQ], r1[kRowsQ];
+    int roff[kRowsQ];  // this thread's quads of a position row: offset inside the row, -1 past its end
+#pragma unroll
+    for (int q = 0; q < kRowsQ; ++q)
+    {
+        const int e = t + q * kRowsNT;
+        const int pos = e / (kRowsRun / 4), qq = e - pos * (kRowsRun / 4);
+        roff[q] = e < quads ? pos * K + qq * 4 : -1;
+        r0[q] = r1[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    auto load_row = [&](int oh, f32x4 (&r)[kRowsQ]) {
+        // position rows outside the image, or below the band's halo, are never read back: skip them
+        const bool live = oh >= 0 && oh < H && oh <= h1;
+        const float *row = src + (int64_t)oh * W * K;
+#pragma unroll
+        for (int q = 0; q < kRowsQ; ++q)
+            if (live && roff[q] >= 0)
+                r[q] = *reinterpret_cast<const f32x4 *>(row + roff[q]);
+    };
+    auto store_row = [&](int oh, const f32x4 (&r)[kRowsQ]) {
+        float *dst = sh_rows + (oh & 3) * slot_floats;
+#pragma unroll
+        for (int q = 0; q < kRowsQ; ++q)
+            if (roff[q] >= 0)
+                *reinterpret_cast<f32x4 *>(dst + (t + q * kRowsNT) * 4) = r[q];
+    };
+    auto sum_row = [&](int h) {
+#pragma unroll 1
+        for (int idx = t; idx < kRowsCT * W; idx += kRowsNT)
+        {
+            const int c = idx & (kRowsCT - 1), w = idx >> 3;
+            float v[9];
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh)
+            {
+                const int oh = h + 1 - kh;
+#pragma unroll
+                for (int kw = 0; kw < 3; ++kw)
+                {
+                    const int ow = w + 1 - kw;
+                    const bool ok = (unsigned)oh < (unsigned)H && (unsigned)ow < (unsigned)W;
+                    const int at = ok ? (oh & 3) * slot_floats + ow * kRowsRun + c * 9 + kh * 3 + kw : 0;
+                    const float x = sh_rows[at];
+                    v[kh * 3 + kw] = ok ? x : 0.f;
+                }
+            }
+            float acc = 0.f;
+#pragma unroll
+            for (int q = 0; q < 9; ++q)
+                acc += v[q];
+            img[((int64_t)(n * C + c0 + c) * H + h) * W + w] = acc;
+        }
+    };
+
+    // the three position rows the first image row needs, then two more on their way
+    load_row(h0 - 1, r0);
+    load_row(h0, r1);
+    if (h0 - 1 >= 0)
+        store_row(h0 - 1, r0);
+    load_row(h0 + 1, r0);
+    store_row(h0, r1);
+    load_row(h0 + 2, r1);
+    store_row(h0 + 1, r0);
+    load_row(h0 + 3, r0);
+    __syncthreads();
+    // invariant at the top of an iteration for image row h: LDS holds position rows h-1, h, h+1; the registers hold
+    // h+2 (first set of the pair in flight) and h+3. Row h+2 goes into the slot row h-2 left, which nobody reads.
+#pragma unroll 1
+    for (int h = h0; h < h1; h += 2)
+    {
+        store_row(h + 2, r1);
+        load_row(h + 4, r1);
+        sum_row(h);
+        __syncthreads();
+        if (h + 1 >= h1)
+            break;
+        store_row(h + 3, r0);
+        load_row(h + 5, r0);
+        sum_row(h + 1);
+        __syncthreads();
+    }
+}
+
+bool col2im_rows3x3_ok(const ConvGeom &g, const float *col)
+{
+    return g.KH == 3 && g.KW == 3 && g.SH == 1 && g.SW == 1 && g.PH == 1 && g.PW == 1 && g.C % kRowsCT == 0 && g.W <= 56 &&
+           g.W >= 4 && g.H >= 2 && reinterpret_cast<uintptr_t>(col) % 16 == 0 && g.N * g.C * g.H * g.W < (1ll << 31) &&
+           g.N * (g.C / kRowsCT) * g.H < (1ll << 31);
+}
+
 // Tile shape for col2im_tile_kernel: the staged rectangle must fit in a third of a CU's LDS, there should be enough
 // workgroups to fill the chip, and among those the tile that re-reads the fewest col rows wins. False when the
 // shape needs the general kernel (64-bit offsets, windows too large to stage).
@@ -759,6 +878,23 @@ int col2im_launch(const float *col, float *img, const ConvGeom &g, int to_matrix
     if (to_matrix)
     {
         const int cs = (g.SH == g.SW && (g.SH == 1 || g.SH == 2)) ? g.SH : 0;
+        if (col2im_rows3x3_ok(g, col))
+        {
+            // bands of image rows: enough workgroups for four per compute unit where the image allows, seven rows or more
+            const int64_t per_band = g.N * (g.C / kRowsCT);
+            int64_t nbands = odl::ceil_div((int64_t)4 * odl::device_cus(), per_band);
+            if (nbands > g.H / 7)
+                nbands = g.H / 7;
+            if (nbands < 1)
+                nbands = 1;
+            const int band = (int)odl::ceil_div(g.H, nbands);
+            nbands = odl::ceil_div(g.H, band);
+            const size_t lds = (size_t)4 * g.W * kRowsRun * sizeof(float);
+            hipLaunchKernelGGL(col2im_rows3x3_kernel, dim3((unsigned)(per_band * nbands)), dim3(kRowsNT), lds, st, col, img,
+                               (int)g.N, (int)g.C, (int)g.H, (int)g.W, band, (int)nbands, (unsigned)odl::chip().xcds);
+            ODL_LAUNCH_CHECK();
+            return ODL_OK;
+        }
         Col2imTile t;
         // the staged kernel pays off at stride 1, where neighbouring pixels share most of their col rows
         if (cs == 1 && plan_col2im_tile(g, t))

@@ -1205,3 +1205,16 @@ def test_float64_batch_norm_matches_float64_numpy(api):
             np.testing.assert_allclose(host(dgamma), want_dgamma, rtol=1e-11, atol=1e-12)
             np.testing.assert_allclose(host(dbeta), want_dbeta, rtol=1e-11, atol=1e-12)
             np.testing.assert_allclose(host(gx), want_gx, rtol=1e-10, atol=1e-11)
+
+
+@pytest.mark.parametrize("N,C,H,W", [(3, 16, 23, 13), (2, 8, 2, 4), (1, 24, 57, 56), (5, 32, 14, 14), (2, 64, 9, 37)])
+def test_col2im_3x3_streaming_rows_is_bit_identical_to_the_scatter_loop(api, o, N, C, H, W):
+    # src/mat/origin/cpu/conv/conv2d.cpp:320-349 adds a pixel's taps in ascending (kh, kw); the kernel that walks down a band
+    # of image rows with four position rows in LDS must give the same float: bands that do not divide H, one-band images,
+    # rows of 4 to 56 pixels, channel counts of one to eight 8-channel chunks
+    rng = np.random.default_rng(N * 1000 + C * 10 + H + W)
+    col = rng.standard_normal((N * H * W, C * 9), dtype=f32)
+    want = np.empty((N, C, H, W), f32)
+    o.orc_col2im(col, N, C, H, W, 3, 3, 1, 1, 1, 1, 1, want)
+    got = host(api.col2im(dev(col), (N, C, H, W), 3, 1, 1, True))
+    assert np.array_equal(got, want)
