@@ -646,22 +646,83 @@ __global__ __launch_bounds__(256) void col2im_tile_kernel(const float *__restric
     }
 }
 
-// Matrix layout, 3x3 / stride 1 / padding 1, the streaming form. The tile kernel above re-reads the col rows of a
+// Matrix layout, 3x3 / padding 1 / stride 1 or 2, the streaming form. The tile kernel above re-reads the col rows of a
 // tile's halo and reads 144-byte runs that straddle 128-byte lines: about 2.3 times the matrix passes from L2 to LDS.
 // Here a workgroup owns one image, eight channels (288 bytes of every col row: 18 whole 16-byte pieces) and a band
-// of image rows, and walks down the band: LDS keeps four rows of output positions ([W positions][72 floats] each, as
-// the loads deliver them); while image row h is summed from position rows h-1, h, h+1, the rows h+2 and h+3 are on
-// their way in registers. Every col row of the band is read once, plus one halo row above and below the band. Lanes
-// run along (pixel, channel) with the channel fastest: the LDS addresses w*72 + c*9 + tap of a wave fall into 32
-// different banks. Taps are added in ascending (kh, kw), absent ones as +0.0f — the sums of the tile kernel, bit for bit.
-constexpr int kRowsCT = 8, kRowsRun = kRowsCT * 9, kRowsNT = 512, kRowsQ = 2;  // quads of a position row per thread: W * 18 <= 2 * 512
+// of rows of output positions, and walks down the band: LDS keeps four position rows ([OW positions][72 floats] each,
+// as the loads deliver them); while the image rows under position row r are summed (row r itself from position rows
+// r-1, r, r+1 at stride 1; rows 2r and 2r+1 from position rows r and r+1 at stride 2), the rows r+2 and r+3 are on their
+// way in registers. Every col row of the band is read once, plus one halo row above and below the band. Lanes run along
+// (pixel, channel) with the channel fastest: the LDS addresses ow*72 + c*9 + tap of a wave fall into 32 different banks.
+// Taps are added in ascending (kh, kw), absent ones left out — the sums of the other col2im kernels, bit for bit.
+constexpr int kRowsCT = 8, kRowsRun = kRowsCT * 9, kRowsNT = 512, kRowsQ = 2;  // quads of a position row per thread: OW * 18 <= 2 * 512
 
+// The lanes of the summing phase: a wave takes eight pixels of one image row (lane = pixel * 8 + channel), so the row and
+// with it the position rows of its taps are the same for the whole wave (scalar work), and what depends on the pixel and
+// the channel (the offsets of the three kw inside a position row, which of them exist) is worked out once per thread.
+// Images up to 64 pixels wide put 8 / ceil(W / 8) rows side by side on the eight waves; wider ones go through a row in
+// steps of 64 pixels.
+struct RowsLanes
+{
+    int wave, c, wl, wpr, rpp, rip, wg0;
+    __device__ RowsLanes(int t, int W)
+    {
+        wave = __builtin_amdgcn_readfirstlane(t >> 6);
+        c = t & (kRowsCT - 1);
+        wl = (t & 63) >> 3;
+        wpr = (W + 7) / 8;
+        rpp = wpr <= 8 ? 8 / wpr : 1;
+        rip = wpr <= 8 ? wave / wpr : 0;
+        wg0 = wpr <= 8 ? wave - rip * wpr : wave;
+    }
+};
+
+// one pixel's sum: taps in ascending (kh, kw); a tap that does not exist would add +0.0f to a sum that is never -0.0f,
+// so leaving it out gives the same float. `row_of(oh)` is the offset of position row `oh` in LDS.
+template <int S, typename RowOf>
+__device__ __forceinline__ float col2im_pixel3x3(const float *sh, RowOf row_of, int h, int OH, const int (&off)[3],
+                                                 const bool (&wok)[3])
+{
+    float acc = 0.f;
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh)
+    {
+        const int hp = h + 1 - kh, oh = S == 1 ? hp : hp >> 1;
+        if (hp >= 0 && (S == 1 || (hp & 1) == 0) && oh < OH)
+        {
+            const float *row = sh + row_of(oh) + kh * 3;
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw)
+            {
+                const float x = row[off[kw]];
+                acc += wok[kw] ? x : 0.f;
+            }
+        }
+    }
+    return acc;
+}
+
+// the three kw of pixel column `w`: offset inside a position row (0 where the tap does not exist) and whether it exists
+template <int S>
+__device__ __forceinline__ void col2im_taps_of_column(int w, int c, int W, int OW, int (&off)[3], bool (&wok)[3])
+{
+#pragma unroll
+    for (int kw = 0; kw < 3; ++kw)
+    {
+        const int wp = w + 1 - kw, ow = S == 1 ? wp : wp >> 1;
+        wok[kw] = w < W && wp >= 0 && (S == 1 || (wp & 1) == 0) && ow < OW;
+        off[kw] = wok[kw] ? ow * kRowsRun + c * 9 + kw : 0;
+    }
+}
+
+template <int S>
 __global__ __launch_bounds__(kRowsNT, 2) void col2im_rows3x3_kernel(const float *__restrict__ col, float *__restrict__ img, int N,
-                                                             int C, int H, int W, int band, int nbands, unsigned xcds)
+                                                                     int C, int H, int W, int OH, int OW, int band,
+                                                                     int nbands, unsigned xcds)
 {
     extern __shared__ float sh_rows[];
     const int t = threadIdx.x;
-    const int slot_floats = W * kRowsRun, quads = W * (kRowsRun / 4), K = C * 9;
+    const int slot_floats = OW * kRowsRun, quads = OW * (kRowsRun / 4), K = C * 9;
     unsigned vb;
     {
         const unsigned nb = gridDim.x, bid = blockIdx.x;
@@ -672,10 +733,12 @@ __global__ __launch_bounds__(kRowsNT, 2) void col2im_rows3x3_kernel(const float 
     const int cc = (int)(vb % (unsigned)cchunks);
     vb /= (unsigned)cchunks;
     const int b = (int)(vb % (unsigned)nbands), n = (int)(vb / (unsigned)nbands);
-    const int h0 = b * band, h1 = (h0 + band < H) ? h0 + band : H, c0 = cc * kRowsCT;
-    const float *src = col + (int64_t)n * H * W * K + c0 * 9;
+    // the band in rows of output positions; the last band also takes the image rows below the last position row's
+    const int r0 = b * band, r1 = (r0 + band < OH) ? r0 + band : OH, c0 = cc * kRowsCT;
+    const int h_end = (b == nbands - 1) ? H : S * r1;
+    const float *src = col + (int64_t)n * OH * OW * K + c0 * 9;
 
-    f32x4 r0[kRowsQ], r1[kRowsQ];
+    f32x4 ra[kRowsQ], rb[kRowsQ];
     int roff[kRowsQ];  // this thread's quads of a position row: offset inside the row, -1 past its end
 #pragma unroll
     for (int q = 0; q < kRowsQ; ++q)
@@ -683,12 +746,12 @@ __global__ __launch_bounds__(kRowsNT, 2) void col2im_rows3x3_kernel(const float 
         const int e = t + q * kRowsNT;
         const int pos = e / (kRowsRun / 4), qq = e - pos * (kRowsRun / 4);
         roff[q] = e < quads ? pos * K + qq * 4 : -1;
-        r0[q] = r1[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+        ra[q] = rb[q] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     auto load_row = [&](int oh, f32x4 (&r)[kRowsQ]) {
         // position rows outside the image, or below the band's halo, are never read back: skip them
-        const bool live = oh >= 0 && oh < H && oh <= h1;
-        const float *row = src + (int64_t)oh * W * K;
+        const bool live = oh >= 0 && oh < OH && oh <= r1;
+        const float *row = src + (int64_t)oh * OW * K;
 #pragma unroll
         for (int q = 0; q < kRowsQ; ++q)
             if (live && roff[q] >= 0)
@@ -701,68 +764,134 @@ __global__ __launch_bounds__(kRowsNT, 2) void col2im_rows3x3_kernel(const float 
             if (roff[q] >= 0)
                 *reinterpret_cast<f32x4 *>(dst + (t + q * kRowsNT) * 4) = r[q];
     };
-    auto sum_row = [&](int h) {
+    // the image rows under position row r
+    const RowsLanes ln(t, W);
+    auto sum_rows = [&](int r) {
+        if (ln.rip >= ln.rpp)
+            return;
 #pragma unroll 1
-        for (int idx = t; idx < kRowsCT * W; idx += kRowsNT)
+        for (int wg = ln.wg0; wg < ln.wpr; wg += 8)
         {
-            const int c = idx & (kRowsCT - 1), w = idx >> 3;
-            float v[9];
-#pragma unroll
-            for (int kh = 0; kh < 3; ++kh)
+            const int w = wg * 8 + ln.wl;
+            int off[3];
+            bool wok[3];
+            col2im_taps_of_column<S>(w, ln.c, W, OW, off, wok);
+#pragma unroll 1
+            for (int h = S * r + ln.rip; h < S * r + S && h < h_end; h += ln.rpp)
             {
-                const int oh = h + 1 - kh;
-#pragma unroll
-                for (int kw = 0; kw < 3; ++kw)
-                {
-                    const int ow = w + 1 - kw;
-                    const bool ok = (unsigned)oh < (unsigned)H && (unsigned)ow < (unsigned)W;
-                    const int at = ok ? (oh & 3) * slot_floats + ow * kRowsRun + c * 9 + kh * 3 + kw : 0;
-                    const float x = sh_rows[at];
-                    v[kh * 3 + kw] = ok ? x : 0.f;
-                }
+                const float acc = col2im_pixel3x3<S>(sh_rows, [&](int oh) { return (oh & 3) * slot_floats; }, h, OH, off, wok);
+                if (w < W)
+                    img[((int64_t)(n * C + c0 + ln.c) * H + h) * W + w] = acc;
             }
-            float acc = 0.f;
-#pragma unroll
-            for (int q = 0; q < 9; ++q)
-                acc += v[q];
-            img[((int64_t)(n * C + c0 + c) * H + h) * W + w] = acc;
         }
     };
 
-    // the three position rows the first image row needs, then two more on their way
-    load_row(h0 - 1, r0);
-    load_row(h0, r1);
-    if (h0 - 1 >= 0)
-        store_row(h0 - 1, r0);
-    load_row(h0 + 1, r0);
-    store_row(h0, r1);
-    load_row(h0 + 2, r1);
-    store_row(h0 + 1, r0);
-    load_row(h0 + 3, r0);
+    // the three position rows the first iteration needs, then two more on their way
+    load_row(r0 - 1, ra);
+    load_row(r0, rb);
+    if (r0 - 1 >= 0)
+        store_row(r0 - 1, ra);
+    load_row(r0 + 1, ra);
+    store_row(r0, rb);
+    load_row(r0 + 2, rb);
+    store_row(r0 + 1, ra);
+    load_row(r0 + 3, ra);
     __syncthreads();
-    // invariant at the top of an iteration for image row h: LDS holds position rows h-1, h, h+1; the registers hold
-    // h+2 (first set of the pair in flight) and h+3. Row h+2 goes into the slot row h-2 left, which nobody reads.
+    // invariant at the top of an iteration for position row r: LDS holds position rows r-1, r, r+1; the registers hold
+    // r+2 (the set stored first) and r+3. Row r+2 goes into the slot row r-2 left, which nobody reads any more.
 #pragma unroll 1
-    for (int h = h0; h < h1; h += 2)
+    for (int r = r0; r < r1; r += 2)
     {
-        store_row(h + 2, r1);
-        load_row(h + 4, r1);
-        sum_row(h);
+        store_row(r + 2, rb);
+        load_row(r + 4, rb);
+        sum_rows(r);
         __syncthreads();
-        if (h + 1 >= h1)
+        if (r + 1 >= r1)
             break;
-        store_row(h + 3, r0);
-        load_row(h + 5, r0);
-        sum_row(h + 1);
+        store_row(r + 3, ra);
+        load_row(r + 5, ra);
+        sum_rows(r + 1);
         __syncthreads();
+    }
+}
+
+// Matrix layout, 3x3 / stride 2 / padding 1, short rows of positions: the walk above keeps too few bytes in flight when a
+// position row is only a few KB. Here a workgroup takes its whole band of position rows (and the one below: image row
+// 2r+1 also reads position row r+1) into LDS at once, eight 16-byte loads deep per thread, and sums its image rows after
+// one barrier. Same lanes, same LDS layout, same order of the taps as the walk.
+constexpr int kBandLdsBytes = 64 * 1024;
+
+__global__ __launch_bounds__(kRowsNT, 2) void col2im_band3x3s2_kernel(const float *__restrict__ col, float *__restrict__ img, int N,
+                                                                       int C, int H, int W, int OH, int OW, int band,
+                                                                       int nbands, unsigned xcds)
+{
+    extern __shared__ float sh_rows[];
+    const int t = threadIdx.x;
+    const int K = C * 9;
+    unsigned vb;
+    {
+        const unsigned nb = gridDim.x, bid = blockIdx.x;
+        const unsigned loc = bid / xcds, xcd = bid - loc * xcds, full = nb / xcds, rem = nb - full * xcds;
+        vb = xcd * full + (xcd < rem ? xcd : rem) + loc;
+    }
+    const int cchunks = C / kRowsCT;
+    const int cc = (int)(vb % (unsigned)cchunks);
+    vb /= (unsigned)cchunks;
+    const int b = (int)(vb % (unsigned)nbands), n = (int)(vb / (unsigned)nbands);
+    const int r0 = b * band, r1 = (r0 + band < OH) ? r0 + band : OH, c0 = cc * kRowsCT;
+    const int rows_in = (r1 < OH ? r1 + 1 : OH) - r0;  // with the row below the band where the image has one
+    const int h0 = 2 * r0, h_end = (b == nbands - 1) ? H : 2 * r1;
+    const float *src = col + ((int64_t)n * OH + r0) * OW * K + c0 * 9;
+    const int quads = rows_in * OW * (kRowsRun / 4);
+    constexpr int kDeep = 8;
+#pragma unroll 1
+    for (int e0 = t; e0 < quads; e0 += kDeep * kRowsNT)
+    {
+        f32x4 r[kDeep];
+#pragma unroll
+        for (int q = 0; q < kDeep; ++q)
+        {
+            const int e = e0 + q * kRowsNT;
+            const int pos = e / (kRowsRun / 4), qq = e - pos * (kRowsRun / 4);
+            if (e < quads)
+                r[q] = *reinterpret_cast<const f32x4 *>(src + (int64_t)pos * K + qq * 4);
+        }
+#pragma unroll
+        for (int q = 0; q < kDeep; ++q)
+        {
+            const int e = e0 + q * kRowsNT;
+            if (e < quads)
+                *reinterpret_cast<f32x4 *>(sh_rows + e * 4) = r[q];
+        }
+    }
+    __syncthreads();
+    const RowsLanes ln(t, W);
+    if (ln.rip >= ln.rpp)
+        return;
+    const int row_floats = OW * kRowsRun;
+#pragma unroll 1
+    for (int wg = ln.wg0; wg < ln.wpr; wg += 8)
+    {
+        const int w = wg * 8 + ln.wl;
+        int off[3];
+        bool wok[3];
+        col2im_taps_of_column<2>(w, ln.c, W, OW, off, wok);
+#pragma unroll 1
+        for (int h = h0 + ln.rip; h < h_end; h += ln.rpp)
+        {
+            const float acc = col2im_pixel3x3<2>(sh_rows, [&](int oh) { return (oh - r0) * row_floats; }, h, OH, off, wok);
+            if (w < W)
+                img[((int64_t)(n * C + c0 + ln.c) * H + h) * W + w] = acc;
+        }
     }
 }
 
 bool col2im_rows3x3_ok(const ConvGeom &g, const float *col)
 {
-    return g.KH == 3 && g.KW == 3 && g.SH == 1 && g.SW == 1 && g.PH == 1 && g.PW == 1 && g.C % kRowsCT == 0 && g.W <= 56 &&
-           g.W >= 4 && g.H >= 2 && reinterpret_cast<uintptr_t>(col) % 16 == 0 && g.N * g.C * g.H * g.W < (1ll << 31) &&
-           g.N * (g.C / kRowsCT) * g.H < (1ll << 31);
+    return g.KH == 3 && g.KW == 3 && g.SH == g.SW && (g.SH == 1 || g.SH == 2) && g.PH == 1 && g.PW == 1 &&
+           g.C % kRowsCT == 0 && g.OW <= 56 && g.OW >= 2 && g.OH >= 2 && g.W >= 4 && reinterpret_cast<uintptr_t>(col) % 16 == 0 &&
+           g.N * g.C * g.H * g.W < (1ll << 31) && g.N * (g.C / kRowsCT) * g.OH < (1ll << 31) &&
+           g.OH * g.OW * g.C * 9 < (1ll << 31);
 }
 
 // Tile shape for col2im_tile_kernel: the staged rectangle must fit in a third of a CU's LDS, there should be enough
@@ -880,18 +1009,42 @@ int col2im_launch(const float *col, float *img, const ConvGeom &g, int to_matrix
         const int cs = (g.SH == g.SW && (g.SH == 1 || g.SH == 2)) ? g.SH : 0;
         if (col2im_rows3x3_ok(g, col))
         {
-            // bands of image rows: enough workgroups for four per compute unit where the image allows, seven rows or more
             const int64_t per_band = g.N * (g.C / kRowsCT);
+            const int64_t row_bytes = g.OW * kRowsRun * (int64_t)sizeof(float);
+            const unsigned xcds = (unsigned)odl::chip().xcds;
+            if (g.SH == 2 && 5 * row_bytes <= kBandLdsBytes)
+            {
+                // whole bands in LDS: four position rows or more a band (the row below it is read twice)
+                const int64_t most = kBandLdsBytes / row_bytes - 1;
+                int64_t nbands = odl::ceil_div((int64_t)2 * odl::device_cus(), per_band);
+                if (nbands > g.OH / 4)
+                    nbands = g.OH / 4;
+                if (nbands < odl::ceil_div(g.OH, most))
+                    nbands = odl::ceil_div(g.OH, most);
+                const int band = (int)odl::ceil_div(g.OH, nbands);
+                nbands = odl::ceil_div(g.OH, band);
+                const size_t lds = (size_t)((band + 1 < g.OH ? band + 1 : g.OH) * row_bytes);
+                hipLaunchKernelGGL(col2im_band3x3s2_kernel, dim3((unsigned)(per_band * nbands)), dim3(kRowsNT), lds, st, col, img,
+                                   (int)g.N, (int)g.C, (int)g.H, (int)g.W, (int)g.OH, (int)g.OW, band, (int)nbands, xcds);
+                ODL_LAUNCH_CHECK();
+                return ODL_OK;
+            }
+            // bands of position rows: enough workgroups for four per compute unit where the image allows, seven rows or more
             int64_t nbands = odl::ceil_div((int64_t)4 * odl::device_cus(), per_band);
-            if (nbands > g.H / 7)
-                nbands = g.H / 7;
+            if (nbands > g.OH / 7)
+                nbands = g.OH / 7;
             if (nbands < 1)
                 nbands = 1;
-            const int band = (int)odl::ceil_div(g.H, nbands);
-            nbands = odl::ceil_div(g.H, band);
-            const size_t lds = (size_t)4 * g.W * kRowsRun * sizeof(float);
-            hipLaunchKernelGGL(col2im_rows3x3_kernel, dim3((unsigned)(per_band * nbands)), dim3(kRowsNT), lds, st, col, img,
-                               (int)g.N, (int)g.C, (int)g.H, (int)g.W, band, (int)nbands, (unsigned)odl::chip().xcds);
+            const int band = (int)odl::ceil_div(g.OH, nbands);
+            nbands = odl::ceil_div(g.OH, band);
+            const size_t lds = (size_t)(4 * row_bytes);
+            const dim3 grid((unsigned)(per_band * nbands)), block(kRowsNT);
+            if (g.SH == 1)
+                hipLaunchKernelGGL(col2im_rows3x3_kernel<1>, grid, block, lds, st, col, img, (int)g.N, (int)g.C, (int)g.H,
+                                   (int)g.W, (int)g.OH, (int)g.OW, band, (int)nbands, xcds);
+            else
+                hipLaunchKernelGGL(col2im_rows3x3_kernel<2>, grid, block, lds, st, col, img, (int)g.N, (int)g.C, (int)g.H,
+                                   (int)g.W, (int)g.OH, (int)g.OW, band, (int)nbands, xcds);
             ODL_LAUNCH_CHECK();
             return ODL_OK;
         }

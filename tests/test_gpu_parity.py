@@ -1207,14 +1207,17 @@ def test_float64_batch_norm_matches_float64_numpy(api):
             np.testing.assert_allclose(host(gx), want_gx, rtol=1e-10, atol=1e-11)
 
 
-@pytest.mark.parametrize("N,C,H,W", [(3, 16, 23, 13), (2, 8, 2, 4), (1, 24, 57, 56), (5, 32, 14, 14), (2, 64, 9, 37)])
-def test_col2im_3x3_streaming_rows_is_bit_identical_to_the_scatter_loop(api, o, N, C, H, W):
+@pytest.mark.parametrize("N,C,H,W,S", [(3, 16, 23, 13, 1), (2, 8, 2, 4, 1), (1, 24, 57, 56, 1), (5, 32, 14, 14, 1),
+                                       (2, 64, 9, 37, 1), (3, 16, 28, 28, 2), (2, 8, 27, 13, 2), (1, 24, 112, 111, 2),
+                                       (4, 128, 28, 28, 2), (2, 8, 4, 4, 2), (1, 16, 31, 6, 2)])
+def test_col2im_3x3_streaming_rows_is_bit_identical_to_the_scatter_loop(api, o, N, C, H, W, S):
     # src/mat/origin/cpu/conv/conv2d.cpp:320-349 adds a pixel's taps in ascending (kh, kw); the kernel that walks down a band
-    # of image rows with four position rows in LDS must give the same float: bands that do not divide H, one-band images,
-    # rows of 4 to 56 pixels, channel counts of one to eight 8-channel chunks
-    rng = np.random.default_rng(N * 1000 + C * 10 + H + W)
-    col = rng.standard_normal((N * H * W, C * 9), dtype=f32)
+    # of position rows with four of them in LDS must give the same float at stride 1 and 2: bands that do not divide the
+    # rows, one-band images, odd and even heights and widths, rows of 2 to 56 positions, one to sixteen 8-channel chunks
+    rng = np.random.default_rng(N * 1000 + C * 10 + H + W + S)
+    OH, OW = (H + 2 - 3) // S + 1, (W + 2 - 3) // S + 1
+    col = rng.standard_normal((N * OH * OW, C * 9), dtype=f32)
     want = np.empty((N, C, H, W), f32)
-    o.orc_col2im(col, N, C, H, W, 3, 3, 1, 1, 1, 1, 1, want)
-    got = host(api.col2im(dev(col), (N, C, H, W), 3, 1, 1, True))
+    o.orc_col2im(col, N, C, H, W, 3, 3, S, S, 1, 1, 1, want)
+    got = host(api.col2im(dev(col), (N, C, H, W), 3, S, 1, True))
     assert np.array_equal(got, want)
