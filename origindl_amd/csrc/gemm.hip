@@ -877,7 +877,7 @@ void launch_tail_fixup(const GemmArgs &g, int BM, int BN, int epi, hipStream_t s
 // the same product for the variant whose operands go from global memory straight into LDS
 odl::DmaGemmArgs dma_args(const GemmArgs &g, int epi)
 {
-    odl::DmaGemmArgs d;
+    odl::DmaGemmArgs d{};
     d.A = g.A, d.B = g.B, d.bias = g.bias, d.C = g.C;
     d.M = g.M, d.N = g.N, d.K = g.K, d.lda = g.lda, d.ldb = g.ldb, d.ldc = g.ldc;
     d.tiles_m = g.tiles_m, d.tiles_n = g.tiles_n, d.splits = g.splits;
@@ -1044,12 +1044,15 @@ int launch_small_tile_wide_slab(bool ta, bool tb, GemmArgs g, int splits, hipStr
     g.xcds = odl::chip().xcds;
     const dim3 grid((unsigned)(g.tiles_m * g.tiles_n * splits)), block(kThreads);
     const bool two_sets = (int64_t)g.tiles_m * g.tiles_n * splits <= lone_workgroup_limit();
-    if (two_sets)
     {
+        // straight-to-LDS loads: one workgroup per compute unit while the launch is about that size, two beyond it
+        // (6272x256x1152: 51 -> 43 us, 3136x512x2304: 98 -> 78 us against the register-staged kernel)
         const odl::DmaGemmArgs d = dma_args(g, EPI);
         if (odl::sgemm_dma_fits(ta, tb, d))
-            return odl::sgemm_dma_launch(64, ta, tb, d, st);
+            return odl::sgemm_dma_launch(two_sets ? 64 : 65, ta, tb, d, st);
     }
+    if (g.K % 32 != 0)  // the register-staged kernel below walks whole 32-wide slabs only
+        return launch_tile<64, 64, kBK, EPI>(ta, tb, true, g, splits, nullptr, 0, st);
 #define ODL_WIDE_CASE(TA, TB)                                                                                  \
     if (ta == TA && tb == TB)                                                                                  \
     {                                                                                                          \
@@ -1076,6 +1079,7 @@ int launch_any_tile(int tile, bool ta, bool tb, bool vec, const GemmArgs &g, int
         return launch_tile<128, 128, kBK, EPI>(ta, tb, vec, g, splits, tail_ws, tail_bytes, st);
     if constexpr (EPI != EPI_NCHW_ROWB)
         if (vec && ((splits == 1 && g.K >= 1024 && g.K % 32 == 0) ||
+                    (splits == 1 && g.K >= 128 && (int64_t)g.tiles_m * g.tiles_n > lone_workgroup_limit()) ||
                     splits == pick_splits_two_sets((int64_t)g.tiles_m * g.tiles_n, g.K)))
             return launch_small_tile_wide_slab<EPI>(ta, tb, g, splits, st);
     return launch_tile<64, 64, kBK, EPI>(ta, tb, vec, g, splits, nullptr, 0, st);
