@@ -212,6 +212,38 @@ def extras(torch, capi, steps, warmup):
                                       "bwd_frac_hbm": nb / ms_b / 1e6 / PEAK_HBM_GBS}
     del x, y, xn, gx, gyb
     keep.clear()
+    # The streaming operators of the path at sizes that can saturate HBM (the MLP's and CNN's own shapes are a few
+    # microseconds of launch latency each). Algorithmic bytes: every input read once, every output written once.
+    def hbm_row(name, fn, nbytes):
+        ms = time_region_auto(torch, fn)
+        out[name] = {"ms": ms, "gbs": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / PEAK_HBM_GBS}
+
+    R, Cc = 16384, 4096
+    big, big2, res = rnd(R, Cc), rnd(R, Cc), empty(R, Cc)
+    nbig = 4.0 * R * Cc
+    hbm_row("transpose_16384x4096", direct("odl_hip_transpose", ptr(big), ptr(res), 1, R, Cc, stream), 2 * nbig)
+    shp, perm = (ctypes.c_int64 * 5)(32, 3, 85, 80, 80), (ctypes.c_int * 5)(0, 1, 3, 4, 2)
+    npm = 4.0 * 32 * 3 * 85 * 80 * 80
+    hbm_row("permute_detect_head_32x3x85x80x80", direct("odl_hip_permute", ptr(big), 0, shp, 5, perm, ptr(res), stream), 2 * npm)
+    hbm_row("relu_64Mi", direct("odl_hip_unary", 0, ptr(big), R * Cc, ptr(res), stream), 2 * nbig)
+    hbm_row("add_64Mi", direct("odl_hip_binary", 0, ptr(big), R * Cc, ptr(big2), R * Cc, ptr(res), stream), 3 * nbig)
+    row = rnd(1, Cc)
+    ss, ts = (ctypes.c_int64 * 2)(1, Cc), (ctypes.c_int64 * 2)(R, Cc)
+    hbm_row("broadcast_to_1x4096_to_16384x4096", direct("odl_hip_broadcast_to", ptr(row), ss, 2, ts, 2, ptr(res), stream),
+            nbig + 4.0 * Cc)
+    rs = empty(R)
+    wr, nr = ws(L.query("odl_hip_sum_axis_workspace_bytes", R, Cc, 1))
+    hbm_row("row_sums_16384x4096", direct("odl_hip_sum_axis", ptr(big), R, Cc, 1, ptr(rs), wr, nr, stream), nbig + 4.0 * R)
+    sm_in, sm_out = rnd(R, 1000), empty(R, 1000)
+    hbm_row("softmax_16384x1000", direct("odl_hip_softmax", ptr(sm_in), R, 1000, 1, ptr(sm_out), stream), 8.0 * R * 1000)
+    am = torch.empty((R,), dtype=torch.int64, device="cuda")
+    hbm_row("argmax_rows_16384x1000", direct("odl_hip_argmax_rows", ptr(sm_in), R, 1000, ptr(am), stream), 4.0 * R * 1000 + 8.0 * R)
+    pm_, gm_, mm_, vm_ = rnd(R * 1024), rnd(R * 1024), torch.zeros(R * 1024, device="cuda"), torch.zeros(R * 1024, device="cuda")
+    f32c = ctypes.c_float
+    hbm_row("adam_step_16Mi", direct("odl_hip_adam_step", ptr(pm_), ptr(gm_), ptr(mm_), ptr(vm_), R * 1024, f32c(0.9), f32c(0.999),
+                                     f32c(10.0), f32c(1000.0), f32c(1e-8), f32c(1e-3), ptr(pm_), stream), 7 * 4.0 * R * 1024)
+    del big, big2, res, row, rs, sm_in, sm_out, am, pm_, gm_, mm_, vm_
+    keep.clear()
     # config 2's other shapes: forward + both gradient GEMMs, 6*M*N*K FLOP per step
     for (M, K, N) in ((1024, 1024, 1024), (2048, 2048, 2048), (8192, 8192, 8192), (512, 784, 1000), (512, 1000, 10)):
         a, b, dc = rnd(M, K), rnd(K, N), rnd(M, N)

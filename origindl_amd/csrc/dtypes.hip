@@ -293,6 +293,175 @@ __global__ void permute_kernel(const T *__restrict__ src, T *__restrict__ dst, i
     }
 }
 
+// Batched 2-D transposition dst[o][c][r] = src[o][r][c] through 64x64 tiles in LDS (rows padded to 65: the column-wise
+// reads of the second phase hit 32 different banks). Lanes run along the contiguous side in both phases: a wave reads
+// 64 consecutive elements of a source row and writes 64 consecutive elements of a destination row. One workgroup of 256
+// threads per tile, tiles numbered with the source's column tiles fastest.
+struct TransposeGeom
+{
+    int64_t rows, cols;
+    unsigned tiles_c, tiles_r;
+    odl::FastDiv d_tiles, d_group;  // by tiles_r * tiles_c, by kTileGroup * tiles_c
+};
+
+// Tile order inside one matrix: groups of 16 tile-rows, inside a group down the rows first. The couple of thousand
+// workgroups in flight then read runs of many KB of each source row and write 4 KB runs of each destination row; with
+// the source's column tiles fastest every workgroup's 64 destination rows had their DRAM pages to themselves
+// (16384 x 4096: 58 % of HBM).
+constexpr unsigned kTileGroup = 16;
+
+__device__ inline void transpose_tile_of(const TransposeGeom &g, unsigned bid, unsigned &o, unsigned &tr, unsigned &tc)
+{
+    o = odl::fastdiv(bid, g.d_tiles);
+    const unsigned t = bid - o * (g.tiles_r * g.tiles_c);
+    const unsigned grp = odl::fastdiv(t, g.d_group), in_g = t - grp * (kTileGroup * g.tiles_c);
+    const unsigned first = grp * kTileGroup;
+    const unsigned gm = g.tiles_r - first < kTileGroup ? g.tiles_r - first : kTileGroup;
+    tc = gm == kTileGroup ? in_g / kTileGroup : in_g / gm;
+    tr = first + (in_g - tc * gm);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_tile_kernel(const T *__restrict__ src, T *__restrict__ dst, TransposeGeom g)
+{
+    __shared__ T tile[64][65];
+    unsigned o, tr, tc;
+    transpose_tile_of(g, blockIdx.x, o, tr, tc);
+    const int64_t r0 = (int64_t)tr * 64, c0 = (int64_t)tc * 64;
+    const T *s = src + (int64_t)o * g.rows * g.cols;
+    T *d = dst + (int64_t)o * g.rows * g.cols;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll 4
+    for (int i = wave; i < 64; i += 4)
+    {
+        const int64_t r = r0 + i, c = c0 + lane;
+        if (r < g.rows && c < g.cols)
+            tile[i][lane] = s[r * g.cols + c];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int i = wave; i < 64; i += 4)
+    {
+        const int64_t c = c0 + i, r = r0 + lane;
+        if (r < g.rows && c < g.cols)
+            d[c * g.rows + r] = tile[lane][i];
+    }
+}
+
+// A matrix with at most 128 rows (the detection head's [85][H*W] planes): a workgroup takes all rows of 64 columns, whose
+// transposed image is one contiguous run of the destination. Lanes along the columns while reading, along that run
+// while writing; LDS rows padded to an odd length.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_few_rows_kernel(const T *__restrict__ src, T *__restrict__ dst, int rows,
+                                                                  int64_t cols, unsigned tiles_c, odl::FastDiv d_tc,
+                                                                  odl::FastDiv d_rows)
+{
+    extern __shared__ unsigned char few_raw[];
+    T *tile = reinterpret_cast<T *>(few_raw);
+    const int ld = rows | 1;
+    const unsigned o = odl::fastdiv(blockIdx.x, d_tc), tc = blockIdx.x - o * tiles_c;
+    const int64_t c0 = (int64_t)tc * 64;
+    const int ncols = cols - c0 < 64 ? (int)(cols - c0) : 64;
+    const T *s = src + (int64_t)o * rows * cols;
+    T *d = dst + (int64_t)o * rows * cols + c0 * rows;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane < ncols)
+    {
+#pragma unroll 4
+        for (int r = wave; r < rows; r += 4)
+            tile[lane * ld + r] = s[(int64_t)r * cols + c0 + lane];
+    }
+    __syncthreads();
+    const int n = ncols * rows;
+#pragma unroll 4
+    for (int e = threadIdx.x; e < n; e += 256)
+    {
+        const unsigned c = odl::fastdiv((unsigned)e, d_rows);
+        d[e] = tile[c * ld + (e - c * rows)];
+    }
+}
+
+// The mirror image: at most 128 columns. 64 source rows are one contiguous run; lanes along it while reading, along the
+// rows (the destination's contiguous side) while writing.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_few_cols_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t rows,
+                                                                  int cols, unsigned tiles_r, odl::FastDiv d_tr,
+                                                                  odl::FastDiv d_cols)
+{
+    __shared__ T tile[128 * 65];
+    const unsigned o = odl::fastdiv(blockIdx.x, d_tr), tr = blockIdx.x - o * tiles_r;
+    const int64_t r0 = (int64_t)tr * 64;
+    const int nrows = rows - r0 < 64 ? (int)(rows - r0) : 64;
+    const T *s = src + (int64_t)o * rows * cols + r0 * cols;
+    T *d = dst + (int64_t)o * rows * cols;
+    const int n = nrows * cols;
+#pragma unroll 4
+    for (int e = threadIdx.x; e < n; e += 256)
+    {
+        const unsigned r = odl::fastdiv((unsigned)e, d_cols);
+        tile[(e - r * cols) * 65 + r] = s[e];
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane < nrows)
+    {
+#pragma unroll 4
+        for (int c = wave; c < cols; c += 4)
+            d[(int64_t)c * rows + r0 + lane] = tile[c * 65 + lane];
+    }
+}
+
+// The same for 4-byte elements when rows and cols are multiples of 4 and both bases are 16-byte aligned: 16 bytes per
+// lane on both sides (a wave reads 4 source rows x 256 bytes and writes 4 destination rows x 256 bytes); in LDS the lanes
+// of a wave touch (4*cq + r) mod 32 = 32 different banks, twice each.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void transpose_tile_vec_kernel(const unsigned *__restrict__ src, unsigned *__restrict__ dst,
+                                                                  TransposeGeom g)
+{
+    constexpr int TR = 64, TC = 64;  // (128x64 and 64x128 tiles measured the same)
+    __shared__ unsigned tile[TC][TR + 1];
+    unsigned o, tr, tc;
+    transpose_tile_of(g, blockIdx.x, o, tr, tc);
+    const int64_t r0 = (int64_t)tr * TR, c0 = (int64_t)tc * TC;
+    const unsigned *s = src + (int64_t)o * g.rows * g.cols;
+    unsigned *d = dst + (int64_t)o * g.rows * g.cols;
+    {
+        constexpr int QPR = TC / 4, LINES = 256 / QPR;  // quads across a source row of the tile, rows per pass
+        const int quad = threadIdx.x % QPR, line = threadIdx.x / QPR;
+#pragma unroll
+        for (int i = 0; i < TR / LINES; ++i)
+        {
+            const int rr = line + LINES * i;
+            const int64_t r = r0 + rr, c = c0 + 4 * quad;
+            if (r < g.rows && c < g.cols)
+            {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(s + r * g.cols + c);
+                tile[4 * quad + 0][rr] = v[0], tile[4 * quad + 1][rr] = v[1];
+                tile[4 * quad + 2][rr] = v[2], tile[4 * quad + 3][rr] = v[3];
+            }
+        }
+    }
+    __syncthreads();
+    {
+        constexpr int QPR = TR / 4, LINES = 256 / QPR;
+        const int quad = threadIdx.x % QPR, line = threadIdx.x / QPR;
+#pragma unroll
+        for (int i = 0; i < TC / LINES; ++i)
+        {
+            const int cc = line + LINES * i;
+            const int64_t c = c0 + cc, r = r0 + 4 * quad;
+            if (r < g.rows && c < g.cols)
+            {
+                u32x4 v;
+                v[0] = tile[cc][4 * quad + 0], v[1] = tile[cc][4 * quad + 1];
+                v[2] = tile[cc][4 * quad + 2], v[3] = tile[cc][4 * quad + 3];
+                *reinterpret_cast<u32x4 *>(d + c * g.rows + r) = v;
+            }
+        }
+    }
+}
+
 struct SumPlan
 {
     int64_t slices, chunk;
@@ -319,6 +488,60 @@ SumPlan plan_sum(int64_t outer, int64_t axis, int64_t inner)
     return p;
 }
 }  // namespace
+
+namespace odl
+{
+// dst[o][c][r] = src[o][r][c] for elements of 1, 4 or 8 bytes; ODL_ERR_INVALID_ARG when the tile count does not fit a grid
+int transpose_launch(const void *src, void *dst, int elem_bytes, int64_t outer, int64_t rows, int64_t cols, hipStream_t st)
+{
+    if (outer * rows * cols == 0)
+        return ODL_OK;
+    const bool vec = elem_bytes == 4 && rows % 4 == 0 && cols % 4 == 0 &&
+                     ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+    if (elem_bytes == 4 && (rows <= 128) != (cols <= 128))
+    {
+        // one narrow side: whole rows (or columns) of 64 columns (rows) per workgroup
+        const bool few_rows = rows <= 128;
+        const int64_t tiles = ceil_div(few_rows ? cols : rows, 64);
+        if (tiles < (1ll << 31) && outer * tiles < (1ll << 31))
+        {
+            const dim3 grid((unsigned)(outer * tiles));
+            if (few_rows)
+                hipLaunchKernelGGL((transpose_few_rows_kernel<uint32_t>), grid, dim3(256), (size_t)64 * ((int)rows | 1) * 4, st,
+                                   static_cast<const uint32_t *>(src), static_cast<uint32_t *>(dst), (int)rows, cols,
+                                   (unsigned)tiles, make_fastdiv((unsigned)tiles), make_fastdiv((unsigned)rows));
+            else
+                hipLaunchKernelGGL((transpose_few_cols_kernel<uint32_t>), grid, dim3(256), 0, st,
+                                   static_cast<const uint32_t *>(src), static_cast<uint32_t *>(dst), rows, (int)cols,
+                                   (unsigned)tiles, make_fastdiv((unsigned)tiles), make_fastdiv((unsigned)cols));
+            ODL_LAUNCH_CHECK();
+            return ODL_OK;
+        }
+    }
+    const int64_t tr = ceil_div(rows, 64), tc = ceil_div(cols, 64);
+    if (tr >= (1ll << 31) || tc >= (1ll << 31) || outer * tr * tc >= (1ll << 31))
+        return fail(ODL_ERR_INVALID_ARG, "transpose: too many tiles");
+    if (tr * tc >= (1ll << 31) || kTileGroup * tc >= (1ll << 31))
+        return fail(ODL_ERR_INVALID_ARG, "transpose: too many tiles");
+    const TransposeGeom g{rows, cols, (unsigned)tc, (unsigned)tr, make_fastdiv((unsigned)(tr * tc)),
+                          make_fastdiv((unsigned)(kTileGroup * tc))};
+    const dim3 grid((unsigned)(outer * tr * tc)), block(256);
+    if (vec)
+        hipLaunchKernelGGL(transpose_tile_vec_kernel, grid, block, 0, st, static_cast<const unsigned *>(src),
+                           static_cast<unsigned *>(dst), g);
+    else if (elem_bytes == 1)
+        hipLaunchKernelGGL((transpose_tile_kernel<uint8_t>), grid, block, 0, st, static_cast<const uint8_t *>(src),
+                           static_cast<uint8_t *>(dst), g);
+    else if (elem_bytes == 8)
+        hipLaunchKernelGGL((transpose_tile_kernel<uint64_t>), grid, block, 0, st, static_cast<const uint64_t *>(src),
+                           static_cast<uint64_t *>(dst), g);
+    else
+        hipLaunchKernelGGL((transpose_tile_kernel<uint32_t>), grid, block, 0, st, static_cast<const uint32_t *>(src),
+                           static_cast<uint32_t *>(dst), g);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace odl
 
 extern "C" {
 
@@ -461,6 +684,33 @@ int odl_hip_permute(const void *src, int dtype, const int64_t *host_shape, int n
         return ODL_OK;
     ODL_REQUIRE(src && dst, "permute: null operand");
     hipStream_t st = odl::as_stream(stream);
+    {
+        // Extents of 1 dropped and output dimensions that are neighbours in the input too taken as one, many orders are
+        // a copy, or a batched 2-D transposition [o][r][c] -> [o][c][r] (the detection head's (0,1,3,4,2) is one): those
+        // go through LDS tiles, with lanes along the contiguous side of both tensors.
+        int64_t mshape[8], mstride[8];  // merged output dimensions: extent, stride in the input
+        int m = 0;
+        for (int k = 0; k < ndim; ++k)
+        {
+            if (d.oshape[k] == 1)
+                continue;
+            if (m > 0 && mstride[m - 1] == d.oshape[k] * d.istride[k])
+                mshape[m - 1] *= d.oshape[k], mstride[m - 1] = d.istride[k];
+            else
+                mshape[m] = d.oshape[k], mstride[m] = d.istride[k], ++m;
+        }
+        const int eb = (int)dtype_bytes(dtype);
+        if (m <= 1)
+        {
+            ODL_HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)total * eb, hipMemcpyDeviceToDevice, st));
+            return ODL_OK;
+        }
+        // [c][r] from [r][c]: output (c, r) with input strides (1, cols); batched: output (o, c, r) with (rows*cols, 1, cols)
+        if (m == 2 && mstride[0] == 1 && mstride[1] == mshape[0] && total < (1ll << 40))
+            return odl::transpose_launch(src, dst, eb, 1, mshape[1], mshape[0], st);
+        if (m == 3 && mstride[1] == 1 && mstride[2] == mshape[1] && mstride[0] == mshape[1] * mshape[2] && total < (1ll << 40))
+            return odl::transpose_launch(src, dst, eb, mshape[0], mshape[2], mshape[1], st);
+    }
     // elements of equal width move alike: 1, 4 or 8 bytes
     switch (dtype_bytes(dtype))
     {

@@ -896,27 +896,6 @@ int64_t lone_workgroup_limit()
     return cus + cus / 4;
 }
 
-__global__ void transpose_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t rows, int64_t cols)
-{
-    __shared__ float tile[32][33];
-    const int64_t o   = blockIdx.z;
-    const float *s    = src + o * rows * cols;
-    float *d          = dst + o * rows * cols;
-    const int64_t c0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
-    for (int i = threadIdx.y; i < 32; i += 8)
-    {
-        const int64_t r = r0 + i, c = c0 + threadIdx.x;
-        tile[i][threadIdx.x] = (r < rows && c < cols) ? s[r * cols + c] : 0.f;
-    }
-    __syncthreads();
-    for (int i = threadIdx.y; i < 32; i += 8)
-    {
-        const int64_t c = c0 + i, r = r0 + threadIdx.x;
-        if (r < rows && c < cols)
-            d[c * rows + r] = tile[threadIdx.x][i];
-    }
-}
-
 template <int BM, int BN, int BK, int EPI>
 int launch_tile(bool ta, bool tb, bool vec, const GemmArgs &g_in, int splits, void *tail_ws, size_t tail_bytes,
                 hipStream_t st)
@@ -1598,11 +1577,8 @@ int odl_hip_transpose(const float *src, float *dst, int64_t outer, int64_t rows,
     ODL_REQUIRE_DEVICE();
     if (outer * rows * cols == 0)
         return ODL_OK;
-    ODL_REQUIRE(outer > 0 && rows > 0 && cols > 0 && outer < 65536, "transpose: bad dimensions");
-    dim3 grid((unsigned)odl::ceil_div(cols, 32), (unsigned)odl::ceil_div(rows, 32), (unsigned)outer);
-    hipLaunchKernelGGL(transpose_kernel, grid, dim3(32, 8), 0, odl::as_stream(stream), src, dst, rows, cols);
-    ODL_LAUNCH_CHECK();
-    return ODL_OK;
+    ODL_REQUIRE(outer > 0 && rows > 0 && cols > 0, "transpose: bad dimensions");
+    return odl::transpose_launch(src, dst, 4, outer, rows, cols, odl::as_stream(stream));
 }
 
 }  // extern "C"

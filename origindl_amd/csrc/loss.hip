@@ -65,6 +65,62 @@ __global__ void softmax_rows_kernel(const float *__restrict__ x, float *__restri
         y[row * C + j] = expf(x[row * C + j] - m) / s;
 }
 
+// Rows whose length is a multiple of 4 and whose bases are 16-byte aligned: a wave keeps its row in registers (QUADS
+// float4 per lane, rows of up to 256*QUADS values), so the row is read once and written once.
+template <int QUADS>
+__global__ __launch_bounds__(kBlock) void softmax_rows_vec_kernel(const float *__restrict__ x, float *__restrict__ y, int64_t N,
+                                                                   int64_t C)
+{
+    const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (row >= N)
+        return;
+    const int lane = threadIdx.x & 63;
+    const f32x4 *xr = reinterpret_cast<const f32x4 *>(x + row * C);
+    f32x4 *yr = reinterpret_cast<f32x4 *>(y + row * C);
+    const int64_t cq = C / 4;
+    f32x4 v[QUADS];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u)
+    {
+        const int64_t q = lane + 64 * u;
+        if (q < cq)
+            v[u] = xr[q];
+        else
+            v[u] = f32x4{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            m = (m < v[u][e]) ? v[u][e] : m;
+    }
+    m = wave_max(m);
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u)
+    {
+        const bool in = lane + 64 * u < cq;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+        {
+            v[u][e] = in ? expf(v[u][e] - m) : 0.f;
+            s += v[u][e];
+        }
+    }
+    s = wave_sum(s);
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u)
+    {
+        const int64_t q = lane + 64 * u;
+        if (q < cq)
+        {
+            f32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                o[e] = v[u][e] / s;
+            yr[q] = o;
+        }
+    }
+}
+
 // softmax along the middle axis of [outer, axis, inner], one thread per (outer, inner) pair
 __global__ void softmax_strided_kernel(const float *__restrict__ x, float *__restrict__ y, int64_t outer, int64_t axis,
                                        int64_t inner)
@@ -340,6 +396,87 @@ __global__ void argmax_rows_kernel(const float *__restrict__ y, int64_t N, int64
     out[i] = mi;
 }
 
+// The same answer for wide rows with a wave per row: every lane scans its strided share in ascending order (a NaN is
+// never greater than anything, as in the sequential scan), the lanes' (value, index) pairs meet by "greater value, or
+// equal value at the smaller index"; a row that starts with a NaN keeps index 0 like the sequential scan, where nothing
+// compares greater than it.
+template <bool VEC>
+__device__ inline int64_t wave_first_argmax(const float *p, int64_t C, int lane)
+{
+    float mv = 0.f;
+    int64_t mi = 0;
+    bool has = false;
+    if (VEC)
+    {
+        // 16 bytes per lane and load, four loads in flight; a lane still meets its elements in ascending order
+        const f32x4 *pv = reinterpret_cast<const f32x4 *>(p);
+        const int64_t cq = C / 4;
+        for (int64_t q0 = lane; q0 < cq; q0 += 256)
+        {
+            f32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (q0 + 64 * u < cq)
+                    v[u] = pv[q0 + 64 * u];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (q0 + 64 * u < cq)
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (v[u][e] == v[u][e] && (!has || v[u][e] > mv))
+                            mv = v[u][e], mi = 4 * (q0 + 64 * u) + e, has = true;
+                }
+        }
+    }
+    else
+    {
+        for (int64_t j = lane; j < C; j += 64)
+        {
+            const float v = p[j];
+            if (v == v && (!has || v > mv))
+                mv = v, mi = j, has = true;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        const float ov = __shfl_xor(mv, o, 64);
+        const int64_t oi = __shfl_xor(mi, o, 64);
+        const int oh = __shfl_xor((int)has, o, 64);
+        if (oh && (!has || ov > mv || (ov == mv && oi < mi)))
+            mv = ov, mi = oi, has = true;
+    }
+    const float first = p[0];
+    return (has && first == first) ? mi : 0;
+}
+
+template <bool VEC>
+__global__ void argmax_rows_wave_kernel(const float *__restrict__ y, int64_t N, int64_t C, int64_t *__restrict__ out)
+{
+    const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (row >= N)
+        return;
+    const int lane = threadIdx.x & 63;
+    const int64_t mi = wave_first_argmax<VEC>(y + row * C, C, lane);
+    if (lane == 0)
+        out[row] = mi;
+}
+
+template <bool VEC>
+__global__ void accuracy_count_wave_kernel(const float *__restrict__ y, const int32_t *__restrict__ t, int64_t N, int64_t C,
+                                           unsigned int *count)
+{
+    const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (row >= N)
+        return;
+    const int lane = threadIdx.x & 63;
+    const int64_t mi = wave_first_argmax<VEC>(y + row * C, C, lane);
+    const int32_t lab = t[row];
+    if (lane == 0 && lab >= 0 && lab < (int32_t)C && (int64_t)lab == mi)
+        atomicAdd(count, 1u);
+}
+
 __global__ void accuracy_count_kernel(const float *__restrict__ y, const int32_t *__restrict__ t, int64_t N, int64_t C,
                                       unsigned int *count)
 {
@@ -381,9 +518,21 @@ int odl_hip_softmax(const float *x, int64_t outer, int64_t axis, int64_t inner, 
     if (outer * axis * inner == 0)
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
-    if (inner == 1)
-        hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)odl::ceil_div(outer, kWaves)), dim3(kBlock), 0, st, x, y,
-                           outer, axis);
+    const bool vec = axis % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    const dim3 rows_grid((unsigned)odl::ceil_div(outer, kWaves));
+    if (inner == 1 && vec && axis > 64 && axis <= 2048)
+    {
+        if (axis <= 256)
+            hipLaunchKernelGGL(softmax_rows_vec_kernel<1>, rows_grid, dim3(kBlock), 0, st, x, y, outer, axis);
+        else if (axis <= 512)
+            hipLaunchKernelGGL(softmax_rows_vec_kernel<2>, rows_grid, dim3(kBlock), 0, st, x, y, outer, axis);
+        else if (axis <= 1024)
+            hipLaunchKernelGGL(softmax_rows_vec_kernel<4>, rows_grid, dim3(kBlock), 0, st, x, y, outer, axis);
+        else
+            hipLaunchKernelGGL(softmax_rows_vec_kernel<8>, rows_grid, dim3(kBlock), 0, st, x, y, outer, axis);
+    }
+    else if (inner == 1)
+        hipLaunchKernelGGL(softmax_rows_kernel, rows_grid, dim3(kBlock), 0, st, x, y, outer, axis);
     else
         hipLaunchKernelGGL(softmax_strided_kernel, dim3((unsigned)odl::ceil_div(outer * inner, kBlock)), dim3(kBlock), 0,
                            st, x, y, outer, axis, inner);
@@ -547,8 +696,16 @@ int odl_hip_argmax_rows(const float *y, int64_t N, int64_t C, int64_t *out, void
     ODL_REQUIRE(N >= 0 && C > 0, "argmax: bad shape");
     if (N == 0)
         return ODL_OK;
-    hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)odl::ceil_div(N, kBlock)), dim3(kBlock), 0,
-                       odl::as_stream(stream), y, N, C, out);
+    const bool vec = C % 4 == 0 && C >= 256 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    if (vec)
+        hipLaunchKernelGGL(argmax_rows_wave_kernel<true>, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0,
+                           odl::as_stream(stream), y, N, C, out);
+    else if (C >= 32)  // a wave per row once a row is worth 64 lanes; a thread per row for a handful of classes
+        hipLaunchKernelGGL(argmax_rows_wave_kernel<false>, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0,
+                           odl::as_stream(stream), y, N, C, out);
+    else
+        hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)odl::ceil_div(N, kBlock)), dim3(kBlock), 0,
+                           odl::as_stream(stream), y, N, C, out);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
@@ -569,8 +726,15 @@ int odl_hip_accuracy(const float *y, const int32_t *t, int64_t N, int64_t C, flo
     unsigned int *count = static_cast<unsigned int *>(workspace);
     hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, count, 1);
     ODL_LAUNCH_CHECK();
-    hipLaunchKernelGGL(accuracy_count_kernel, dim3((unsigned)odl::ceil_div(N, kBlock)), dim3(kBlock), 0, st, y, t, N, C,
-                       count);
+    if (C % 4 == 0 && C >= 256 && (reinterpret_cast<uintptr_t>(y) & 15) == 0)
+        hipLaunchKernelGGL(accuracy_count_wave_kernel<true>, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, st, y,
+                           t, N, C, count);
+    else if (C >= 32)
+        hipLaunchKernelGGL(accuracy_count_wave_kernel<false>, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, st, y,
+                           t, N, C, count);
+    else
+        hipLaunchKernelGGL(accuracy_count_kernel, dim3((unsigned)odl::ceil_div(N, kBlock)), dim3(kBlock), 0, st, y, t, N, C,
+                           count);
     ODL_LAUNCH_CHECK();
     unsigned int host_count = 0;
     ODL_HIP_CHECK(hipMemcpyAsync(&host_count, count, sizeof(host_count), hipMemcpyDeviceToHost, st));

@@ -32,6 +32,9 @@ inline int device_cus()
 int fill_launch(float *dst, int64_t n, float value, hipStream_t st);
 int fill_bytes_launch(void *dst, int value, size_t bytes, hipStream_t st);
 
+// dst[o][c][r] = src[o][r][c] for elements of 1, 4 or 8 bytes (LDS tiles, lanes along the contiguous side of both)
+int transpose_launch(const void *src, void *dst, int elem_bytes, int64_t outer, int64_t rows, int64_t cols, hipStream_t st);
+
 inline hipStream_t as_stream(void *s)
 {
     return reinterpret_cast<hipStream_t>(s);

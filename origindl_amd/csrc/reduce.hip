@@ -445,6 +445,43 @@ __global__ void broadcast_kernel(const float *__restrict__ src, float *__restric
     dst[t] = src[si];
 }
 
+// The same over merged dimensions, four consecutive outputs per thread: neighbouring target dimensions that are both
+// copied or both repeated count as one, the innermost merged extent is a multiple of 4, all counts fit 32 bits. A repeated
+// innermost dimension splats one source value, a copied one loads 16 bytes.
+struct BcastQuads
+{
+    int nd;
+    unsigned dshape[8];  // merged target extents, the innermost in quads
+    odl::FastDiv div[8];
+    unsigned sstride[8];  // in elements; 0 where the source is repeated
+};
+
+__global__ __launch_bounds__(256) void broadcast_quads_kernel(const float *__restrict__ src, float *__restrict__ dst,
+                                                               unsigned quads, BcastQuads d)
+{
+    const unsigned t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= quads)
+        return;
+    const int last = d.nd - 1;
+    unsigned r = odl::fastdiv(t, d.div[last]);
+    unsigned si = (t - r * d.dshape[last]) * 4u * d.sstride[last];
+    for (int k = last - 1; k >= 0; --k)
+    {
+        const unsigned q = odl::fastdiv(r, d.div[k]);
+        si += (r - q * d.dshape[k]) * d.sstride[k];
+        r = q;
+    }
+    f32x4 v;
+    if (d.sstride[last])
+        v = *reinterpret_cast<const f32x4 *>(src + si);
+    else
+    {
+        const float x = src[si];
+        v = f32x4{x, x, x, x};
+    }
+    reinterpret_cast<f32x4 *>(dst)[t] = v;
+}
+
 int64_t prod(const int64_t *s, int n)
 {
     int64_t p = 1;
@@ -919,6 +956,41 @@ int odl_hip_broadcast_to(const float *src, const int64_t *host_src_shape, int sr
     const int64_t total = prod(host_dst_shape, dst_ndim);
     if (total == 0)
         return ODL_OK;
+    {
+        // merged dimensions, innermost first in the scan: extents of 1 dropped, neighbours of the same kind multiplied
+        BcastQuads q{};
+        int64_t mshape[8], mstride[8];
+        int m = 0;
+        for (int k = 0; k < dst_ndim; ++k)
+        {
+            if (d.dshape[k] == 1)
+                continue;
+            const bool rep = d.sstride[k] == 0;
+            if (m > 0 && ((rep && mstride[m - 1] == 0) || (!rep && mstride[m - 1] == d.dshape[k] * d.sstride[k])))
+                mshape[m - 1] *= d.dshape[k], mstride[m - 1] = d.sstride[k];
+            else
+                mshape[m] = d.dshape[k], mstride[m] = d.sstride[k], ++m;
+        }
+        const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+        bool ok = m >= 1 && total < (1ll << 32) && mshape[m - 1] % 4 == 0 && aligned;
+        for (int k = 0; ok && k < m; ++k)
+            ok = mshape[k] < (1ll << 31) && mstride[k] < (1ll << 31) && (k == m - 1 || mstride[k] % 4 == 0);
+        if (ok)
+        {
+            q.nd = m;
+            for (int k = 0; k < m; ++k)
+            {
+                q.dshape[k] = (unsigned)(k == m - 1 ? mshape[k] / 4 : mshape[k]);
+                q.div[k] = odl::make_fastdiv(q.dshape[k]);
+                q.sstride[k] = (unsigned)mstride[k];
+            }
+            const unsigned quads = (unsigned)(total / 4);
+            hipLaunchKernelGGL(broadcast_quads_kernel, dim3((unsigned)odl::ceil_div(quads, 256)), dim3(256), 0,
+                               odl::as_stream(stream), src, dst, quads, q);
+            ODL_LAUNCH_CHECK();
+            return ODL_OK;
+        }
+    }
     hipLaunchKernelGGL(broadcast_kernel, dim3((unsigned)odl::ceil_div(total, kBlock)), dim3(kBlock), 0,
                        odl::as_stream(stream), src, dst, total, d);
     ODL_LAUNCH_CHECK();

@@ -184,7 +184,9 @@ def test_matmul_full_size_sampled_rows_and_linearity(api, o, size):
 
 def test_transpose(api, o):
     rng = np.random.default_rng(3)
-    for shape in ((37, 53), (2, 3, 5), (128, 64), (1, 7)):
+    # tiles of 64x64: ragged edges on both sides, whole tiles read and written 16 bytes per lane, batches, single rows
+    for shape in ((37, 53), (2, 3, 5), (128, 64), (1, 7), (3, 132, 68), (200, 260), (5, 64, 192), (130, 1), (257, 129),
+                  (2, 4, 1000)):
         x = rng.standard_normal(shape, dtype=f32)
         want = np.empty(shape[:-2] + (shape[-1], shape[-2]), f32)
         o.orc_transpose(x, want, int(np.prod(shape[:-2])) if len(shape) > 2 else 1, shape[-2], shape[-1])
@@ -494,20 +496,30 @@ def test_broadcast_fixtures(api):
             np.testing.assert_allclose(got, G[f"{name}_gx"], atol=1e-5)
     x = np.arange(3, dtype=f32).reshape(3, 1)
     assert np.array_equal(host(api.broadcast_to(dev(x), (2, 3, 4))), np.broadcast_to(x, (2, 3, 4)))
+    # src/mat/origin/cpu/math/broadcast.cpp (right-aligned, extent 1 repeats): rows, columns, scalars, repeated and copied
+    # dimensions in turn, innermost extents that are and are not multiples of four
+    rng = np.random.default_rng(5)
+    for ss, ds in (((1, 4096), (33, 4096)), ((64, 1), (64, 100)), ((1,), (7, 12)), ((3, 1, 8), (5, 3, 6, 8)),
+                   ((2, 1, 3, 1, 4), (2, 5, 3, 7, 4)), ((6, 10), (4, 6, 10)), ((5, 1, 1), (5, 4, 8)), ((1, 7), (9, 7)),
+                   ((4, 1, 2), (4, 6, 2)), ((), (3, 4))):
+        x = rng.standard_normal(ss, dtype=f32)
+        assert np.array_equal(host(api.broadcast_to(dev(x), ds)), np.broadcast_to(x, ds)), (ss, ds)
 
 
 # ------------------------------------------------------------------------------------ softmax / CE
 def test_softmax_and_ce_vs_oracle(api, o):
     rng = np.random.default_rng(14)
     for N, C, is64 in ((512, 10, 1), (256, 10, 0), (7, 1000, 1), (1, 3, 0), (300, 65, 1), (33, 128, 0), (9, 400, 1),
-                       (5, 2000, 0)):
+                       (5, 2000, 0), (130, 256, 1), (67, 516, 0), (31, 1028, 1), (19, 2048, 0), (3, 2052, 1)):
         x = (rng.standard_normal((N, C), dtype=f32) * 3).astype(f32)
         t = rng.integers(0, C, size=N).astype(np.int64 if is64 else np.int32)
         p, gx, loss = np.empty_like(x), np.empty_like(x), np.zeros(1, f32)
         o.orc_softmax(x, N, C, 1, p)
         assert o.orc_softmax_ce_loss(x, t, is64, N, C, loss) == 0
         assert o.orc_softmax_ce_grad(x, t, is64, N, C, 1.0, gx) == 0
-        np.testing.assert_allclose(host(api.softmax(dev(x))), p, atol=1e-6, rtol=0)
+        # the denominator is a sum of C exponentials taken in another order than the reference's loop: about
+        # sqrt(C) * 2^-24 relative (2.7e-6 at C = 2048), well inside the 1e-5 of the reference's strict tolerance
+        np.testing.assert_allclose(host(api.softmax(dev(x))), p, atol=1e-6, rtol=4e-6)
         got_loss = api.softmax_cross_entropy(dev(x), dev(t))
         assert abs(got_loss - loss[0]) <= 1e-4 * abs(loss[0]) + 1e-6
         np.testing.assert_allclose(host(api.softmax_cross_entropy_backward(dev(x), dev(t), 1.0)), gx, atol=1e-6, rtol=0)
@@ -615,6 +627,19 @@ def test_argmax_and_accuracy_bit_exact(api, o):
     o.orc_argmax_rows(y, 1000, 10, am)
     assert np.array_equal(host(api.argmax_rows(dev(y))), am)
     assert api.accuracy(dev(y), dev(t)) == o.orc_accuracy(y, t, 1000, 10)
+    # wide rows take a wave per row: ties at every distance, a NaN at the head of a row (src/utils/metrics.cpp:42-53 never
+    # finds anything greater than it: index 0), NaNs and infinities further in, widths around the multiples of 64
+    for N, C in ((300, 32), (257, 63), (129, 64), (100, 65), (64, 1000), (5, 4097), (37, 256), (9, 1028), (3, 5000)):
+        y = rng.integers(0, 3, size=(N, C)).astype(f32)
+        y[rng.integers(0, N, N // 4), rng.integers(0, C, N // 4)] = np.nan
+        y[rng.integers(0, N, N // 8), 0] = np.nan
+        y[rng.integers(0, N, N // 8), rng.integers(0, C, N // 8)] = np.inf
+        y[N - 1, :] = -np.inf
+        t = rng.integers(0, C, size=N).astype(np.int32)
+        am = np.empty(N, np.int64)
+        o.orc_argmax_rows(y, N, C, am)
+        assert np.array_equal(host(api.argmax_rows(dev(y))), am), (N, C)
+        assert api.accuracy(dev(y), dev(t)) == o.orc_accuracy(y, t, N, C), (N, C)
 
 
 # ------------------------------------------------------------------------------------- elementwise
@@ -1097,7 +1122,10 @@ def test_permute_is_numpy_transpose_in_every_element_width(api):
     rng = np.random.default_rng(61)
     for name, shape, perm in (("f32", (4, 3, 5, 7), (0, 2, 3, 1)), ("f32", (2, 3, 85, 6, 5), (0, 1, 3, 4, 2)),
                               ("f64", (6, 5), (1, 0)), ("u8", (3, 4, 5), (2, 0, 1)), ("i64", (7,), (0,)),
-                              ("i32", (2, 1, 3, 1, 4), (4, 3, 2, 1, 0))):
+                              ("i32", (2, 1, 3, 1, 4), (4, 3, 2, 1, 0)), ("f32", (3, 2, 85, 12, 20), (0, 1, 3, 4, 2)),
+                              ("f32", (130, 70), (1, 0)), ("f32", (64, 128), (1, 0)), ("u8", (5, 67, 130), (0, 2, 1)),
+                              ("i64", (3, 65, 66), (0, 2, 1)), ("f64", (2, 3, 4, 5), (0, 1, 2, 3)),
+                              ("i32", (6, 1, 9), (2, 1, 0)), ("f32", (4, 5, 6, 7), (2, 3, 0, 1))):
         code, t = DT[name]
         x = _typed_values(rng, t, int(np.prod(shape))).reshape(shape)
         dx = dev(x)
