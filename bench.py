@@ -238,6 +238,28 @@ def extras(torch, capi, steps, warmup):
     hbm_row("softmax_16384x1000", direct("odl_hip_softmax", ptr(sm_in), R, 1000, 1, ptr(sm_out), stream), 8.0 * R * 1000)
     am = torch.empty((R,), dtype=torch.int64, device="cuda")
     hbm_row("argmax_rows_16384x1000", direct("odl_hip_argmax_rows", ptr(sm_in), R, 1000, ptr(am), stream), 4.0 * R * 1000 + 8.0 * R)
+    tot = empty(1)
+    wr, nr = ws(L.query("odl_hip_sum_all_workspace_bytes", R * Cc))
+    hbm_row("sum_all_64Mi", direct("odl_hip_sum_all", ptr(big), R * Cc, ptr(tot), wr, nr, stream), nbig)
+    cm = empty(Cc)
+    hbm_row("max_over_rows_16384x4096", direct("odl_hip_max_axis", ptr(big), 1, R, Cc, ptr(cm), stream), nbig + 4.0 * Cc)
+    hbm_row("max_along_rows_16384x4096", direct("odl_hip_max_axis", ptr(big), R, Cc, 1, ptr(rs), stream), nbig + 4.0 * R)
+    # the detector's shape operators at batch 32: 2x nearest upsample of a P4 map, the concatenation that follows it,
+    # SiLU over a P3 map, and the float32 -> float64 conversion of the same map
+    up_in, up_out = rnd(32, 128, 40, 40), empty(32, 128, 80, 80)
+    hbm_row("upsample2x_32x128x40x40", direct("odl_hip_upsample_nearest", ptr(up_in), 32, 128, 40, 40, 80, 80, 2, 2, ptr(up_out),
+                                              stream), 4.0 * (up_in.numel() + up_out.numel()))
+    cat_b, cat_out = rnd(32, 64, 80, 80), empty(32, 192, 80, 80)
+    ins = (ctypes.c_void_p * 2)(up_out.data_ptr(), cat_b.data_ptr())
+    szs = (ctypes.c_int64 * 2)(128, 64)
+    keep.extend([ins, szs])
+    hbm_row("cat_channels_128+64_at_32x80x80", direct("odl_hip_cat", ins, szs, 2, 32, 6400, ptr(cat_out), stream),
+            8.0 * cat_out.numel())
+    hbm_row("silu_32x192x80x80", direct("odl_hip_unary", 7, ptr(cat_out), cat_out.numel(), ptr(cat_out), stream), 8.0 * cat_out.numel())
+    f64 = torch.empty(cat_b.shape, dtype=torch.float64, device="cuda")
+    hbm_row("convert_f32_to_f64_13Mi", direct("odl_hip_convert", ptr(cat_b), 0, ptr(f64), 1, cat_b.numel(), stream),
+            12.0 * cat_b.numel())
+    del up_in, up_out, cat_b, cat_out, f64
     pm_, gm_, mm_, vm_ = rnd(R * 1024), rnd(R * 1024), torch.zeros(R * 1024, device="cuda"), torch.zeros(R * 1024, device="cuda")
     f32c = ctypes.c_float
     hbm_row("adam_step_16Mi", direct("odl_hip_adam_step", ptr(pm_), ptr(gm_), ptr(mm_), ptr(vm_), R * 1024, f32c(0.9), f32c(0.999),

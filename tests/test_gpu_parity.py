@@ -434,6 +434,27 @@ def test_sum_all_and_max_all(api, o):
     assert tuple(api.sum(dev(rng.standard_normal((3, 4), dtype=f32)), -1, keepdim=True).shape) == (1, 1)
     with pytest.raises(api.OdlInvalidArgument):
         api.sum(dev(np.ones((2, 2), f32)), 2)
+    # src/mat/origin/cpu/math/max.cpp:25-40, 58-117 on the shapes that split the scan over workgroups: a long axis over
+    # few columns (chunks merged with integer atomics), whole tensors of a million elements; infinities, NaNs that the
+    # comparison skips, a NaN first element (the whole-tensor maximum then stays NaN), all-negative and all -inf data
+    for outer, axis, inner in ((1, 5000, 300), (3, 700, 40), (2, 4096, 1028), (1, 100000, 7)):
+        x = (rng.standard_normal((outer, axis, inner), dtype=f32) - 2.0).astype(f32)
+        x[0, axis // 2, 0] = np.inf
+        x[0, 3, inner - 1] = np.nan
+        x[outer - 1, :, 1] = -np.inf
+        want = np.empty((outer, inner), f32)
+        o.orc_max_axis(x, outer, axis, inner, want)
+        assert np.array_equal(host(api.max(dev(x), 1)).reshape(outer, inner), want), (outer, axis, inner)
+    for n, edit in ((300_001, None), (1 << 20, "nan_first"), (70_000, "neg_inf"), (1_000_000, "nan_inside")):
+        x = (rng.standard_normal(n, dtype=f32) - 5.0).astype(f32)
+        if edit == "nan_first":
+            x[0] = np.nan
+        elif edit == "neg_inf":
+            x[:] = -np.inf
+        elif edit == "nan_inside":
+            x[12345] = np.nan
+        got, want = host(api.max(dev(x)))[0], o.orc_max_all(x, n)
+        assert got == want or (np.isnan(got) and np.isnan(want)), (n, edit)
 
 
 def test_sum_to_fixtures_and_errors(api, o):
@@ -811,6 +832,13 @@ def test_upsample_and_cat_bit_exact(api, o):
     assert np.array_equal(up, want)
     cat = host(api.cat([dev(up), dev(b)], 1))
     assert np.array_equal(cat, np.concatenate([up, b], axis=1))
+    # cpu/nn/upsample.cpp:62-63 (ih = oh / scale) over scales and row lengths that do and do not fill 16-byte quads
+    for (N, C, H, W, sh, sw) in ((2, 3, 5, 6, 2, 2), (1, 2, 7, 4, 3, 1), (2, 2, 3, 4, 1, 3), (1, 1, 4, 3, 2, 4), (3, 1, 2, 5, 2, 2),
+                                 (1, 4, 9, 2, 1, 2)):
+        xs = rng.standard_normal((N, C, H, W), dtype=f32)
+        want = np.empty((N, C, H * sh, W * sw), f32)
+        assert o.orc_upsample_nearest(xs, N, C, H, W, H * sh, W * sw, sh, sw, want) == 0
+        assert np.array_equal(host(api.upsample(dev(xs), (sh, sw))), want), (N, C, H, W, sh, sw)
     odd = [rng.standard_normal((3, c, 5), dtype=f32) for c in (3, 1, 7)]  # runs that are not multiples of four floats
     assert np.array_equal(host(api.cat([dev(p) for p in odd], 1)), np.concatenate(odd, axis=1))
     same = [rng.standard_normal((2, 4, 6), dtype=f32) for _ in range(3)]
