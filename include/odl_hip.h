@@ -186,7 +186,11 @@ size_t odl_hip_sum_axis_noalloc_max_bytes(void);
 /* Mat::sum(-1): all elements -> dst[0] (operation_templates.h:342-357) */
 int odl_hip_sum_all(const float *src, int64_t n, float *dst, void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_sum_all_workspace_bytes(int64_t n);
-/* Mat::max(axis) / Mat::max(-1) (src/mat/origin/cpu/math/max.cpp:20-121) */
+/* Mat::max(axis) / Mat::max(-1) (src/mat/origin/cpu/math/max.cpp:20-121): NaNs never win (`max_val < v` is false for
+ * them), except that the whole-tensor maximum starts from the first element and stays NaN when that is one. A long axis
+ * over few columns, and a whole tensor of 65536 elements or more, are scanned by many workgroups whose partial maxima
+ * meet through integer atomics: the value is the reference's, but where the maximum is a zero and zeros of both signs
+ * occur the result is +0.0f whatever their order (the reference keeps the first one it meets). */
 int odl_hip_max_axis(const float *src, int64_t outer, int64_t axis, int64_t inner, float *dst, void *stream);
 int odl_hip_max_all(const float *src, int64_t n, float *dst, void *stream);
 /* Mat::sum_to (mat.h:217; src/mat/origin/cpu/math/sum_to.cpp:11-76): LEFT-aligned shape comparison, one

@@ -106,10 +106,10 @@ __device__ inline int64_t xcd_contiguous_block(int64_t bid, int64_t nb)
     return xcd * full + (xcd < rem ? xcd : rem) + loc;
 }
 
-__device__ inline unsigned xcd_contiguous_block32(unsigned bid, unsigned nb)
+__device__ inline unsigned xcd_contiguous_block32(unsigned bid, unsigned nb, unsigned xcds)
 {
-    const unsigned xcd = bid % 8u, loc = bid / 8u;
-    const unsigned full = nb / 8u, rem = nb % 8u;
+    const unsigned loc = bid / xcds, xcd = bid - loc * xcds;
+    const unsigned full = nb / xcds, rem = nb - full * xcds;
     return xcd * full + (xcd < rem ? xcd : rem) + loc;
 }
 
@@ -201,6 +201,7 @@ struct Im2colTile
     int CT, ctiles, LS;      // channels per tile, channel tiles, LDS row stride (floats, odd)
     unsigned mtiles;         // pixel tiles
     unsigned q4_magic;       // ceil(2^32 / q4) for q4 = CT*KH*KW/4
+    unsigned xcds;           // L2 domains the hardware deals workgroups over
 };
 
 template <int CK>
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(256) void im2col_tile_kernel(const float *__restric
     float *sh = sh_i2c;
     const int KH = CK > 0 ? CK : g.KH, KW = CK > 0 ? CK : g.KW;
     const int KHW = KH * KW;
-    const unsigned vb = xcd_contiguous_block32(blockIdx.x, t.mtiles * (unsigned)t.ctiles);
+    const unsigned vb = xcd_contiguous_block32(blockIdx.x, t.mtiles * (unsigned)t.ctiles, t.xcds);
     const unsigned mt = vb / (unsigned)t.ctiles;
     const int ct = (int)(vb - mt * (unsigned)t.ctiles);
     const int lane = threadIdx.x & 63;
@@ -324,6 +325,7 @@ bool plan_im2col_tile(const ConvGeom &g, Im2colTile &t)
         return false;
     const unsigned q4 = (unsigned)(CT * KHW / 4);
     t.q4_magic = q4 > 1 ? (unsigned)(((1ull << 32) + q4 - 1) / q4) : 0u;  // 0: the kernel divides directly
+    t.xcds = (unsigned)odl::chip().xcds;
     return true;
 }
 
@@ -499,6 +501,7 @@ struct Col2imTile
     int LS;                  // LDS row stride in floats (odd)
     unsigned q4_magic;       // ceil(2^32 / (CT*KH*KW/4)), 0 = divide directly
     unsigned owr_magic;      // ceil(2^32 / owr)
+    unsigned xcds;           // L2 domains the hardware deals workgroups over
 };
 
 __device__ inline int ceil_div_signed(int a, int d)  // d > 0
@@ -516,7 +519,7 @@ __global__ __launch_bounds__(256) void col2im_tile_kernel(const float *__restric
     const int SH = CS > 0 ? CS : g.SH, SW = CS > 0 ? CS : g.SW;
     const int KHW = KH * KW;
     const int H = (int)g.H, W = (int)g.W, OH = (int)g.OH, OW = (int)g.OW, C = (int)g.C;
-    unsigned vb = xcd_contiguous_block32(blockIdx.x, (unsigned)g.N * t.htiles * t.wtiles * t.ctiles);
+    unsigned vb = xcd_contiguous_block32(blockIdx.x, (unsigned)g.N * t.htiles * t.wtiles * t.ctiles, t.xcds);
     const int ct = (int)(vb % (unsigned)t.ctiles);
     vb /= (unsigned)t.ctiles;
     const int wt = (int)(vb % (unsigned)t.wtiles);
@@ -945,6 +948,7 @@ bool plan_col2im_tile(const ConvGeom &g, Col2imTile &best)
     const unsigned q4 = (unsigned)(best.CT * KHW / 4);
     best.q4_magic = q4 > 1 ? (unsigned)(((1ull << 32) + q4 - 1) / q4) : 0u;
     best.owr_magic = best.owr > 1 ? (unsigned)(((1ull << 32) + best.owr - 1) / best.owr) : 0u;
+    best.xcds = (unsigned)odl::chip().xcds;
     return true;
 }
 
