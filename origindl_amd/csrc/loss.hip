@@ -132,11 +132,14 @@ __global__ void softmax_strided_kernel(const float *__restrict__ x, float *__res
     const float *p = x + o * axis * inner + i;
     float *q = y + o * axis * inner + i;
     float m = -FLT_MAX;
+#pragma unroll 8
     for (int64_t a = 0; a < axis; ++a)
         m = (m < p[a * inner]) ? p[a * inner] : m;
     float s = 0.f;
+#pragma unroll 8
     for (int64_t a = 0; a < axis; ++a)
         s += expf(p[a * inner] - m);
+#pragma unroll 8
     for (int64_t a = 0; a < axis; ++a)
         q[a * inner] = expf(p[a * inner] - m) / s;
 }
@@ -160,6 +163,18 @@ __global__ void one_hot_kernel(const void *idx, int is64, int64_t N, int64_t C, 
     out[e] = (label_at(idx, is64, i) == j) ? 1.f : 0.f;  // out-of-range labels match no column (gather.cpp:134)
 }
 
+// rows of a multiple of four classes, 16-byte aligned output: one 16-byte store per thread, the label read once per quad
+__global__ void one_hot_quads_kernel(const void *idx, int is64, unsigned quads, unsigned cq, odl::FastDiv d_cq,
+                                     float *__restrict__ out)
+{
+    const unsigned q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= quads)
+        return;
+    const unsigned i = odl::fastdiv(q, d_cq), j = (q - i * cq) * 4u;
+    const int64_t d = label_at(idx, is64, i) - (int64_t)j;  // the quad's element that is set, if 0 <= d < 4
+    reinterpret_cast<f32x4 *>(out)[q] = f32x4{d == 0 ? 1.f : 0.f, d == 1 ? 1.f : 0.f, d == 2 ? 1.f : 0.f, d == 3 ? 1.f : 0.f};
+}
+
 // logp[i] = log(softmax(x)[i, t_i] + 1e-8); flag[0] |= 1 when a label is out of range
 __global__ void ce_row_logp_kernel(const float *__restrict__ x, const void *t, int is64, int64_t N, int64_t C,
                                    float *__restrict__ logp, int *flag)
@@ -170,6 +185,59 @@ __global__ void ce_row_logp_kernel(const float *__restrict__ x, const void *t, i
     const int lane = threadIdx.x & 63;
     float m, s;
     row_stats(x + row * C, C, lane, m, s);
+    if (lane == 0)
+    {
+        const int64_t lab = label_at(t, is64, row);
+        if (lab < 0 || lab >= C)
+        {
+            atomicOr(flag, 1);
+            logp[row] = 0.f;
+        }
+        else
+        {
+            const float p = expf(x[row * C + lab] - m) / s;
+            logp[row] = logf(p + 1e-8f);
+        }
+    }
+}
+
+// The same with the row in registers (lengths that are multiples of 4, 16-byte aligned base, up to 256*QUADS classes):
+// one read of x instead of two.
+template <int QUADS>
+__global__ __launch_bounds__(kBlock) void ce_row_logp_vec_kernel(const float *__restrict__ x, const void *t, int is64, int64_t N,
+                                                                  int64_t C, float *__restrict__ logp, int *flag)
+{
+    const int64_t row = (int64_t)blockIdx.x * kWaves + (threadIdx.x >> 6);
+    if (row >= N)
+        return;
+    const int lane = threadIdx.x & 63;
+    const f32x4 *xr = reinterpret_cast<const f32x4 *>(x + row * C);
+    const int64_t cq = C / 4;
+    f32x4 v[QUADS];
+    float m = -FLT_MAX;
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u)
+    {
+        const int64_t q = lane + 64 * u;
+        if (q < cq)
+            v[u] = xr[q];
+        else
+            v[u] = f32x4{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            m = (m < v[u][e]) ? v[u][e] : m;
+    }
+    m = wave_max(m);
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < QUADS; ++u)
+    {
+        const bool in = lane + 64 * u < cq;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            s += in ? expf(v[u][e] - m) : 0.f;
+    }
+    s = wave_sum(s);
     if (lane == 0)
     {
         const int64_t lab = label_at(t, is64, row);
@@ -574,8 +642,15 @@ int odl_hip_one_hot(const void *idx, int idx_is_i64, int64_t N, int64_t C, float
     ODL_REQUIRE(C > 0, "one_hot: num_classes must be positive, but got %lld", (long long)C);
     if (N == 0)
         return ODL_OK;
-    hipLaunchKernelGGL(one_hot_kernel, dim3((unsigned)odl::ceil_div(N * C, kBlock)), dim3(kBlock), 0,
-                       odl::as_stream(stream), idx, idx_is_i64, N, C, out);
+    if (C % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 && N * C < (1ll << 33) && N < (1ll << 31))
+    {
+        const unsigned quads = (unsigned)(N * C / 4), cq = (unsigned)(C / 4);
+        hipLaunchKernelGGL(one_hot_quads_kernel, dim3((unsigned)odl::ceil_div(quads, kBlock)), dim3(kBlock), 0,
+                           odl::as_stream(stream), idx, idx_is_i64, quads, cq, odl::make_fastdiv(cq), out);
+    }
+    else
+        hipLaunchKernelGGL(one_hot_kernel, dim3((unsigned)odl::ceil_div(N * C, kBlock)), dim3(kBlock), 0,
+                           odl::as_stream(stream), idx, idx_is_i64, N, C, out);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
@@ -604,8 +679,21 @@ static int ce_loss_launch(const float *x, const void *t, int idx_is_i64, int64_t
     float *logp = static_cast<float *>(workspace);
     hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, out2, 2);
     ODL_LAUNCH_CHECK();
-    hipLaunchKernelGGL(ce_row_logp_kernel, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, st, x, t,
-                       idx_is_i64, N, C, logp, reinterpret_cast<int *>(out2 + 1));
+    const dim3 rows_grid((unsigned)odl::ceil_div(N, kWaves));
+    int *flag = reinterpret_cast<int *>(out2 + 1);
+    if (C % 4 == 0 && C > 64 && C <= 2048 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
+    {
+        if (C <= 256)
+            hipLaunchKernelGGL(ce_row_logp_vec_kernel<1>, rows_grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, logp, flag);
+        else if (C <= 512)
+            hipLaunchKernelGGL(ce_row_logp_vec_kernel<2>, rows_grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, logp, flag);
+        else if (C <= 1024)
+            hipLaunchKernelGGL(ce_row_logp_vec_kernel<4>, rows_grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, logp, flag);
+        else
+            hipLaunchKernelGGL(ce_row_logp_vec_kernel<8>, rows_grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, logp, flag);
+    }
+    else
+        hipLaunchKernelGGL(ce_row_logp_kernel, rows_grid, dim3(kBlock), 0, st, x, t, idx_is_i64, N, C, logp, flag);
     ODL_LAUNCH_CHECK();
     hipLaunchKernelGGL(ce_finish_kernel, dim3(1), dim3(1024), 0, st, logp, N, reinterpret_cast<float *>(out2),
                        mirror);

@@ -549,10 +549,22 @@ def test_softmax_and_ce_vs_oracle(api, o):
         o.orc_one_hot(t, is64, N, C, oh)
         assert np.array_equal(host(api.gather(dev(p), dev(t))), sel)  # integer indexing: bit-exact
         assert np.array_equal(host(api.one_hot(dev(t), C)), oh)
+    # one_hot in 16-byte quads: labels at every position of a quad, out of range on both sides (gather.cpp:134 leaves the
+    # row zero), 32- and 64-bit labels
+    for C in (4, 8, 36):
+        for dt in (np.int32, np.int64):
+            t = np.concatenate([np.arange(-2, C + 3), rng.integers(0, C, 50)]).astype(dt)
+            oh = np.empty((t.size, C), f32)
+            o.orc_one_hot(t, int(dt is np.int64), t.size, C, oh)
+            assert np.array_equal(host(api.one_hot(dev(t), C)), oh), (C, dt)
     x3 = rng.standard_normal((4, 6, 5), dtype=f32)
     p3 = np.empty_like(x3)
     o.orc_softmax(x3, 4, 6, 5, p3)
     np.testing.assert_allclose(host(api.softmax(dev(x3), 1)), p3, atol=1e-6, rtol=0)
+    x4 = rng.standard_normal((3, 70, 9, 11), dtype=f32)  # a channel axis longer than the unrolled stretch of the scan
+    p4 = np.empty_like(x4)
+    o.orc_softmax(x4, 3, 70, 99, p4)
+    np.testing.assert_allclose(host(api.softmax(dev(x4), 1)), p4, atol=1e-6, rtol=2e-6)
 
 
 def test_ce_reference_unit_test_vectors_and_errors(api):
