@@ -651,6 +651,27 @@ def test_max_pool_cnn_shapes_vs_oracle_bit_exact(api, o):
     assert host(y).ravel().tolist() == [6, 8, 14, 16]
 
 
+def test_max_pool_overlapping_padded_windows_staged_in_lds_bit_exact(api, o):
+    # max_pool2d.cpp:40-224 with padding cells counted as 0.0 and first maximum on strict >: the kernels that keep whole
+    # planes in LDS, over the windows with compile-time sizes (3x3/2, 3x3/1, 5x5/1, 2x2/2 on a width that is not a multiple
+    # of four) and run-time ones (4x4/2, 3x2 windows), one and several planes per workgroup with a ragged last workgroup
+    rng = np.random.default_rng(151)
+    for N, C, H, W, KH, KW, S, P in ((2, 3, 13, 9, 3, 3, 2, 1), (1, 5, 10, 10, 5, 5, 1, 2), (2, 2, 7, 8, 3, 3, 1, 1),
+                                     (3, 2, 9, 10, 4, 4, 2, 1), (2, 3, 8, 7, 3, 2, 1, 1), (3, 1, 6, 6, 2, 2, 2, 1),
+                                     (9, 251, 6, 7, 3, 3, 2, 1), (5, 500, 5, 5, 5, 5, 1, 2)):
+        x = np.maximum(rng.standard_normal((N, C, H, W), dtype=f32), -0.2).astype(f32)  # ties at the clamp, some below the padding's 0
+        OH, OW = (H + 2 * P - KH) // S + 1, (W + 2 * P - KW) // S + 1
+        y, idx = np.empty((N, C, OH, OW), f32), np.empty((N, C, OH, OW), np.uint64)
+        assert o.orc_max_pool2d(x, N, C, H, W, KH, KW, S, S, P, P, y, idx) == 0
+        gy = rng.standard_normal(y.shape, dtype=f32)
+        gx = np.empty_like(x)
+        assert o.orc_max_pool2d_backward(gy, idx, N, C, H, W, KH, KW, S, S, P, P, gx) == 0
+        yd, idxd = api.max_pool2d(dev(x), (KH, KW), S, P)
+        assert np.array_equal(host(yd), y) and np.array_equal(host(idxd).view(np.uint64), idx), (N, C, H, W, KH, KW, S, P)
+        got = host(api.max_pool2d_backward(dev(gy), idxd, x.shape, (KH, KW), S, P))
+        assert np.array_equal(got, gx), (N, C, H, W, KH, KW, S, P)
+
+
 # ----------------------------------------------------------------------------------------- metrics
 def test_argmax_and_accuracy_bit_exact(api, o):
     rng = np.random.default_rng(16)
