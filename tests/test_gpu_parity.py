@@ -1310,3 +1310,19 @@ def test_col2im_3x3_streaming_rows_is_bit_identical_to_the_scatter_loop(api, o, 
     o.orc_col2im(col, N, C, H, W, 3, 3, S, S, 1, 1, 1, want)
     got = host(api.col2im(dev(col), (N, C, H, W), 3, S, 1, True))
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("N,C,H,W,S", [(3, 16, 23, 13, 1), (2, 8, 2, 4, 1), (1, 24, 57, 56, 1), (5, 32, 14, 14, 1), (2, 64, 9, 37, 1),
+                                       (3, 16, 28, 28, 2), (2, 8, 27, 13, 2), (1, 24, 112, 111, 2), (2, 8, 4, 4, 2),
+                                       (1, 16, 31, 6, 2), (1, 8, 1, 1, 1), (1, 8, 3, 200, 1), (2, 8, 130, 5, 2)])
+def test_im2col_3x3_matrix_layout_is_bit_identical_to_the_gather_loop(api, o, N, C, H, W, S):
+    # src/mat/origin/cpu/conv/conv2d.cpp:39-207 copies x[n, c, oh*S-1+kh, ow*S-1+kw] (zero outside the image) to
+    # col[(n, oh, ow)][(c, kh, kw)]; the tiled kernel must give the same matrix at stride 1 and 2: pixel tiles that cross
+    # image rows and images, one-row and one-pixel images, very wide and very tall images, odd and even sizes
+    rng = np.random.default_rng(N * 1000 + C * 10 + H + W + S)
+    x = rng.standard_normal((N, C, H, W), dtype=f32)
+    OH, OW = (H + 2 - 3) // S + 1, (W + 2 - 3) // S + 1
+    want = np.empty((N * OH * OW, C * 9), f32)
+    o.orc_im2col(x, N, C, H, W, 3, 3, S, S, 1, 1, 1, want)
+    got = host(api.im2col(dev(x), 3, S, 1, True))
+    assert np.array_equal(got, want)
