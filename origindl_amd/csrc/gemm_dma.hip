@@ -97,7 +97,12 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     constexpr int A_U = BM * BK / 4 / kNT, B_U = BN * BK / 4 / kNT;  // loads per thread and slab
     static_assert((BM * BK / 4) % kNT == 0 && (BN * BK / 4) % kNT == 0 && (PIECES & (PIECES - 1)) == 0, "tile shape");
     constexpr int PER_SLAB = A_U + B_U;
-    constexpr int WAVES_N = KSETS == 2 ? 2 : 1, WAVES_M = 8 / KSETS / WAVES_N;
+    // Row-contiguous B on a 128-wide tile: a wave takes the whole tile width, and lane l32 of its four column blocks owns
+    // the four ADJACENT columns 4*l32 .. 4*l32+3 (block j = column 4*l32 + j). One 16-byte LDS read of a K row then feeds
+    // the four blocks' matrix instructions of one K pair, where the plain layout (block j = columns 32*j + l32) needs a
+    // 4-byte read per block and K value; the output leaves in 16-byte stores as well.
+    constexpr bool QUADB = !B_KMAJOR && BN == 128 && BM == 128 && KSETS == 2;
+    constexpr int WAVES_N = QUADB ? 1 : (KSETS == 2 ? 2 : 1), WAVES_M = 8 / KSETS / WAVES_N;
     constexpr int RB = BM / WAVES_M / 32, CB = BN / WAVES_N / 32;  // 32x32 blocks per wave
     constexpr int STEPS = BK / 8 / KSETS;                          // 8-wide K steps per wave and slab
     static_assert(RB >= 1 && CB >= 1 && STEPS >= 1 && RB * WAVES_M * 32 == BM && CB * WAVES_N * 32 == BN, "wave layout");
@@ -255,11 +260,22 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
                 const f32x4 v = *reinterpret_cast<const f32x4 *>(bs + (c * PIECES + ((2 * ks + lh) ^ swizzle<PIECES>(c))) * 4);
                 b[j][0] = v[0], b[j][1] = v[1], b[j][2] = v[2], b[j][3] = v[3];
             }
-            else
+            else if (!QUADB)
             {
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
                     b[j][s] = bs[(ks * 8 + 4 * lh + s) * BN + c];
+            }
+        }
+        if (QUADB)
+        {
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+            {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(bs + (ks * 8 + 4 * lh + s) * BN + 4 * l32);
+#pragma unroll
+                for (int j = 0; j < CB; ++j)
+                    b[j][s] = v[j % 4];
             }
         }
     };
@@ -393,7 +409,55 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
             return;
     }
 
-    // accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4, column l32
+    // accumulator register r of lane (l32, lh) holds row 8*(r/4) + 4*lh + r%4 and the lane's column of block j
+    if constexpr (QUADB)
+    {
+        // the lane's four blocks are four adjacent columns: one 16-byte store per row where the row's base allows
+        const int64_t col0 = n0 + 4 * l32;
+        float *Cout = tail_out ? tail_out : g.C + (int64_t)kz * g.c_split_stride + (int64_t)bz * g.c_batch;
+        const int64_t ld = tail_out ? BN : g.ldc, cbase = tail_out ? 4 * l32 : col0;
+        const int64_t rbase = tail_out ? 0 : m0;
+        const bool whole = (reinterpret_cast<uintptr_t>(Cout) & 15) == 0 && (tail_out || (col0 + 3 < g.N && g.ldc % 4 == 0));
+        const bool with_bias = !tail_out && g.epi == kEpiBiasCol && g.bias != nullptr;
+        float bcol[4] = {0.f, 0.f, 0.f, 0.f};
+        if (with_bias)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                bcol[e] = col0 + e < g.N ? g.bias[col0 + e] : 0.f;
+#pragma unroll
+        for (int i = 0; i < RB; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+            {
+                const int64_t row = rbase + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+                if (!tail_out && row >= g.M)
+                    continue;
+                f32x4 v = {acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+                if (with_bias)
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        v[e] = odl::apply_act(v[e] + bcol[e], g.act);
+                }
+                else if (!tail_out && g.epi == kEpiBiasRow)
+                {
+                    const float br = g.bias ? g.bias[row] : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        v[e] = odl::apply_act(g.bias ? v[e] + br : v[e], g.act);
+                }
+                if (whole)
+                    *reinterpret_cast<f32x4 *>(Cout + row * ld + cbase) = v;
+                else
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (tail_out || col0 + e < g.N)
+                            Cout[row * ld + cbase + e] = v[e];
+                }
+            }
+        return;
+    }
     if (tail_out)
     {
         // K piece of a tail tile: the whole BM x BN partial, tile-local (rows or columns past the matrix hold zeros)
