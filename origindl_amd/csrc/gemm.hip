@@ -882,7 +882,8 @@ odl::DmaGemmArgs dma_args(const GemmArgs &g, int epi)
     d.M = g.M, d.N = g.N, d.K = g.K, d.lda = g.lda, d.ldb = g.ldb, d.ldc = g.ldc;
     d.tiles_m = g.tiles_m, d.tiles_n = g.tiles_n, d.splits = g.splits;
     d.k_per_split = g.k_per_split, d.c_split_stride = g.c_split_stride;
-    d.epi = epi == EPI_BIAS_COL ? 1 : 0, d.act = g.act, d.xcds = g.xcds;
+    d.epi = epi == EPI_BIAS_COL ? 1 : (epi == EPI_NCHW_ROWB ? 2 : 0), d.act = g.act, d.xcds = g.xcds;
+    d.c_p = epi == EPI_NCHW_ROWB ? g.P : 0;
     d.main_blocks = g.main_blocks, d.tail_first = g.tail_first, d.tail_splits = g.tail_splits, d.tail_kps = g.tail_kps;
     d.tail_ws = g.tail_ws;
     d.batch = 1, d.a_batch = d.b_batch = d.c_batch = 0;
@@ -1057,10 +1058,22 @@ int launch_any_tile(int tile, bool ta, bool tb, bool vec, const GemmArgs &g, int
     if (tile == 128)
         return launch_tile<128, 128, kBK, EPI>(ta, tb, vec, g, splits, tail_ws, tail_bytes, st);
     if constexpr (EPI != EPI_NCHW_ROWB)
+    {
         if (vec && ((splits == 1 && g.K >= 1024 && g.K % 32 == 0) ||
                     (splits == 1 && g.K >= 128 && (int64_t)g.tiles_m * g.tiles_n > lone_workgroup_limit()) ||
                     splits == pick_splits_two_sets((int64_t)g.tiles_m * g.tiles_n, g.K)))
             return launch_small_tile_wide_slab<EPI>(ta, tb, g, splits, st);
+    }
+    else if (vec && splits == 1 && g.K >= 128 && g.N < (1ll << 32) && g.P < (1ll << 32))
+    {
+        // the explicit convolution forward (y^T = W . col^T, stored NCHW): straight-to-LDS loads when the shape allows
+        GemmArgs h = g;
+        h.splits = 1, h.xcds = odl::chip().xcds;
+        h.main_blocks = 0, h.tail_first = h.tiles_m * h.tiles_n, h.tail_splits = 0, h.tail_kps = 0, h.tail_ws = nullptr;
+        const odl::DmaGemmArgs d = dma_args(h, EPI);
+        if (odl::sgemm_dma_fits(ta, tb, d))
+            return odl::sgemm_dma_launch((int64_t)h.tiles_m * h.tiles_n <= lone_workgroup_limit() ? 64 : 65, ta, tb, d, st);
+    }
     return launch_tile<64, 64, kBK, EPI>(ta, tb, vec, g, splits, nullptr, 0, st);
 }
 }  // namespace
@@ -1324,6 +1337,15 @@ static int forward_splits(int64_t OC, int64_t M, int64_t K)
         return 1;
     const int64_t cap = kt / 4 < 32 ? kt / 4 : 32;
     return pick_conv_splits(tiles, kt, (OC <= 64 ? 4 : 3) * (int64_t)odl::device_cus(), cap);
+}
+
+}  // namespace odl
+namespace odl
+{
+// K slices the gathered forward would cut this product into (1: none)
+int conv_implicit_forward_splits(int64_t OC, int64_t M, int64_t K)
+{
+    return forward_splits(OC, M, K);
 }
 
 // The tap-ordered gather: square 1x1 / 3x3 windows over a channel count that fills whole K slabs, image addressed

@@ -28,6 +28,9 @@ struct DmaGemmArgs
     // and writes C + z*c_batch (elements). Not combined with K slices or a split tail.
     int batch;
     int64_t a_batch, b_batch, c_batch;
+    // c_p > 0 (64-wide tiles only, with epi == 2): column n of the product is (image n / c_p, position n % c_p) and goes to
+    // C[(image * M + row) * c_p + position] — an NCHW tensor of M channels, the bias by row
+    int64_t c_p;
 };
 
 // true when the shape suits the variant (16-byte aligned rows, offsets within 31 bits)

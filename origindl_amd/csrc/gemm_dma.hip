@@ -481,6 +481,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
                 continue;
             const bool with_bias = g.epi == kEpiBiasCol && g.bias != nullptr;
             const float bcol = with_bias ? g.bias[col] : 0.f;
+            const int64_t img = g.c_p > 0 ? (int64_t)((unsigned)col / (unsigned)g.c_p) : 0, pos = col - img * g.c_p;
 #pragma unroll
             for (int r = 0; r < 16; ++r)
             {
@@ -488,6 +489,11 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
                 if (row >= g.M)
                     continue;
                 float v = acc[i][j][r];
+                if (g.c_p > 0)
+                {
+                    Cout[(img * g.M + row) * g.c_p + pos] = odl::apply_act(g.bias ? v + g.bias[row] : v, g.act);
+                    continue;
+                }
                 if (with_bias)
                     v = odl::apply_act(v + bcol, g.act);
                 else if (g.epi == kEpiBiasRow)
@@ -512,6 +518,8 @@ bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g)
 
 int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st)
 {
+    if (g.c_p > 0 && !(tile == 64 || tile == 65 || tile == 32))
+        return fail(ODL_ERR_RUNTIME, "sgemm: the NCHW output exists for the 64-wide tiles only");
     const int64_t nt = (int64_t)g.tiles_m * g.tiles_n;
     const dim3 grid((unsigned)(g.tail_splits > 0 ? g.main_blocks + (nt - g.tail_first) * g.tail_splits
                                                  : nt * g.splits * (g.batch > 1 ? g.batch : 1))),
