@@ -1133,8 +1133,9 @@ static const float *const kAlignedProbe = reinterpret_cast<const float *>(uintpt
 static bool forward_by_col_matrix(int64_t N, int64_t C, int64_t OC, int KH, int KW, int SH, int SW, int64_t OH, int64_t OW)
 {
     const int64_t M = N * OH * OW, K = C * KH * KW;
+    // (from about a GFLOP on: below that both ways are a few launch latencies and the extra launch loses)
     return (SH > 1 || SW > 1) && K % 4 == 0 && K >= 128 && M * K * (int64_t)sizeof(float) <= (256ll << 20) &&
-           odl::conv_implicit_forward_splits(OC, M, K) >= 4;
+           2 * M * K * OC >= (1ll << 30) && odl::conv_implicit_forward_splits(OC, M, K) >= 4;
 }
 
 size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
