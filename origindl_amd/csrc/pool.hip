@@ -169,7 +169,8 @@ __global__ __launch_bounds__(256) void max_pool_bwd_plane_kernel(const float *__
     }
 }
 
-// Overlapping windows (3x3/2, 5x5/1 ...) over planes that fit LDS: a workgroup copies `ppw` whole (n, c) planes into LDS
+// Overlapping windows (3x3/2, 5x5/1 ...: a cell is read by several outputs; windows that do not overlap gain nothing from
+// the staging and keep the kernels above) over planes that fit LDS: a workgroup copies `ppw` whole (n, c) planes into LDS
 // with coalesced loads and scans the windows there — the K*K reads per output (per input pixel, in the backward, an
 // 8-byte index and a gradient each) then cost LDS bandwidth instead of K*K trips through the vector cache (5x5/1 over
 // [64,256,40,40]: forward 175 us, backward 788 us with the kernels above). Scan order and comparisons are theirs.
@@ -409,9 +410,7 @@ dim3 plane_grid(int64_t plane, int64_t ncount)
     do                                                                                   \
     {                                                                                    \
         const bool sq = g.KH == g.KW && g.SH == g.SW;                                    \
-        if (sq && g.KH == 2 && g.SH == 2)                                                \
-            hipLaunchKernelGGL((KERNEL<2, 2>), grid, dim3(256), LDS, st, __VA_ARGS__);   \
-        else if (sq && g.KH == 3 && g.SH == 2)                                           \
+        if (sq && g.KH == 3 && g.SH == 2)                                                \
             hipLaunchKernelGGL((KERNEL<3, 2>), grid, dim3(256), LDS, st, __VA_ARGS__);   \
         else if (sq && g.KH == 3 && g.SH == 1)                                           \
             hipLaunchKernelGGL((KERNEL<3, 1>), grid, dim3(256), LDS, st, __VA_ARGS__);   \
@@ -455,7 +454,7 @@ int odl_hip_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t 
         hipLaunchKernelGGL(max_pool_fwd_pair_kernel, dim3((unsigned)odl::ceil_div((int64_t)pairs, 256)), dim3(256), 0, st,
                            x, y, idx, pairs, (int)(g.OW / 2), (unsigned)(g.OH * g.OW / 2));
     }
-    else if (plane_ok(g) && (int64_t)g.KH * g.KW >= 4 && N * C < (1ll << 31) && planes_per_workgroup(N * C, H * W, 4) > 0)
+    else if (plane_ok(g) && (g.KH > g.SH || g.KW > g.SW) && N * C < (1ll << 31) && planes_per_workgroup(N * C, H * W, 4) > 0)
     {
         const int ppw = planes_per_workgroup(N * C, H * W, 4);
         const dim3 grid((unsigned)odl::ceil_div(N * C, ppw));
@@ -498,7 +497,7 @@ int odl_hip_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N,
             hipLaunchKernelGGL((max_pool_bwd_tiled_kernel<3>), grid, dim3(256), 0, st, gy, idx, gx, outputs, (int)g.OW,
                                (unsigned)(g.OH * g.OW));
     }
-    else if (plane_ok(g) && (int64_t)g.KH * g.KW >= 4 && N * C < (1ll << 31) &&
+    else if (plane_ok(g) && (g.KH > g.SH || g.KW > g.SW) && N * C < (1ll << 31) &&
              planes_per_workgroup(N * C, g.OH * g.OW, 8) > 0)
     {
         const int ppw = planes_per_workgroup(N * C, g.OH * g.OW, 8);

@@ -653,8 +653,9 @@ def test_max_pool_cnn_shapes_vs_oracle_bit_exact(api, o):
 
 def test_max_pool_overlapping_padded_windows_staged_in_lds_bit_exact(api, o):
     # max_pool2d.cpp:40-224 with padding cells counted as 0.0 and first maximum on strict >: the kernels that keep whole
-    # planes in LDS, over the windows with compile-time sizes (3x3/2, 3x3/1, 5x5/1, 2x2/2 on a width that is not a multiple
-    # of four) and run-time ones (4x4/2, 3x2 windows), one and several planes per workgroup with a ragged last workgroup
+    # planes in LDS, over the overlapping windows with compile-time sizes (3x3/2, 3x3/1, 5x5/1) and run-time ones (4x4/2,
+    # 3x2 windows), one and several planes per workgroup with a ragged last workgroup; a padded 2x2/2, which does not
+    # overlap, stays with the plain kernels
     rng = np.random.default_rng(151)
     for N, C, H, W, KH, KW, S, P in ((2, 3, 13, 9, 3, 3, 2, 1), (1, 5, 10, 10, 5, 5, 1, 2), (2, 2, 7, 8, 3, 3, 1, 1),
                                      (3, 2, 9, 10, 4, 4, 2, 1), (2, 3, 8, 7, 3, 2, 1, 1), (3, 1, 6, 6, 2, 2, 2, 1),
