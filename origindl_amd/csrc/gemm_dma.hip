@@ -90,6 +90,9 @@ __device__ inline int swizzle(int row)
 // KSETS sets that each multiply every KSETS-th 8-wide K step (2 sets for square tiles; 4 sets on a 64x32 tile, whose
 // two 32x32 blocks could not occupy eight waves otherwise).
 template <int BM, int BN, int BK, bool TA, bool TB, int WGS_PER_CU, int KSETS = 2>
+// (The second launch bound counts waves per SIMD, of which a workgroup of 512 threads brings two: WGS_PER_CU there only
+// keeps the register budget generous — the kernels use under 128 registers and fit two workgroups per compute unit
+// anyway. Bounds of 2 * WGS_PER_CU changed the compiler's schedule for the worse: 2048^3 dA = dC.B^T 133 -> 142 us.)
 __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::DmaGemmArgs g)
 {
     constexpr bool A_KMAJOR = !TA, B_KMAJOR = TB;
@@ -298,8 +301,10 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     // while the matrix instructions of the current one run — the first half of a step's instructions is issued, then (when
     // the next step opens a new slab) the wait for that slab, the barrier and the queueing of the slab four ahead, then the
     // reads of the next fragments, then the second half, so neither the barrier nor the LDS latency leaves the matrix pipe
-    // idle (4096^3 dA = dC.B^T: 994 -> 955 us). With a row-contiguous operand (four 4-byte reads per block) the same
-    // order measured slower than reading right after the barrier (NN 1005 -> 1047 us, TN 992 -> 1026 us): those keep it.
+    // idle (4096^3 dA = dC.B^T: 994 -> 955 us). With a row-contiguous operand the same order measured slower than reading
+    // right after the barrier (4-byte reads: NN 1005 -> 1047 us, TN 992 -> 1026 us) or no faster (B in 16-byte quads: the
+    // second fragment set takes the kernel past 128 registers and with that to one workgroup per compute unit; held to
+    // 128 registers it runs 969 against 972 us): those keep the plain order.
     constexpr bool PIPE = A_KMAJOR && B_KMAJOR;
     if constexpr (PIPE)
     {
