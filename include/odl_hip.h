@@ -247,6 +247,13 @@ int odl_hip_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t 
                        int PH, int PW, float *y, uint64_t *idx, void *stream);
 int odl_hip_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N, int64_t C, int64_t H, int64_t W,
                                 int KH, int KW, int SH, int SW, int PH, int PW, float *gx, void *stream);
+/* max_pool2d_backward followed by the backward of the ReLU whose output x was pooled, in one pass:
+ * gx = pool_backward(gy, idx) * (x > 0 ? 1 : 0), the product of src/operators/activation/relu.cpp:23-29 applied to the
+ * pooling gradient (MaxPool2d::backward then ReLU::backward, src/operators/pooling/max_pool2d.cpp:60-86), same floats
+ * as the two calls in turn. Windows that tile the image exactly (2x2/2, 3x3/3) write each cell once, masked; other
+ * windows run the two steps. x has the shape of gx. */
+int odl_hip_max_pool2d_backward_relu(const float *gy, const uint64_t *idx, const float *x, int64_t N, int64_t C, int64_t H,
+                                     int64_t W, int KH, int KW, int SH, int SW, int PH, int PW, float *gx, void *stream);
 
 /* ------------------------------------------------------------------ metrics ------------------------- */
 /* argmax per row, first maximum (src/utils/metrics.cpp:40-53), and accuracy() (metrics.cpp:11-70) with

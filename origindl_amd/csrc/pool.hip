@@ -332,6 +332,52 @@ __global__ __launch_bounds__(256) void max_pool_bwd_tiled_kernel(const float *__
     }
 }
 
+// The same with the gradient of the ReLU that produced the pooled tensor folded in: every cell is multiplied by
+// (x > 0 ? 1 : 0) as it is written — the product src/operators/activation/relu.cpp:23-29 forms on the pooling gradient
+// in a pass of its own (the sign of a zero included).
+template <int K>
+__global__ __launch_bounds__(256) void max_pool_bwd_tiled_relu_kernel(const float *__restrict__ gy,
+                                                                      const uint64_t *__restrict__ idx,
+                                                                      const float *__restrict__ x, float *__restrict__ gx,
+                                                                      unsigned total, int OW, unsigned oplane)
+{
+    const unsigned o = blockIdx.x * 256u + threadIdx.x;
+    if (o >= total)
+        return;
+    const int hit = (int)idx[o];
+    const float v = 0.f + gy[o];
+    const unsigned nc = o / oplane, r = o - nc * oplane;
+    const int oh = (int)(r / (unsigned)OW), ow = (int)r - oh * OW;
+    const int W = OW * K;
+    const int64_t at = ((int64_t)nc * oplane * (K * K)) + (int64_t)(oh * K) * W + ow * K;
+#pragma unroll
+    for (int kh = 0; kh < K; ++kh)
+    {
+        if (K == 2)
+        {
+            const float2 xr = *reinterpret_cast<const float2 *>(x + at + kh * W);
+            float2 row;
+            row.x = (hit == kh * K ? v : 0.f) * ((xr.x > 0.f) ? 1.f : 0.f);
+            row.y = (hit == kh * K + 1 ? v : 0.f) * ((xr.y > 0.f) ? 1.f : 0.f);
+            *reinterpret_cast<float2 *>(gx + at + kh * W) = row;
+        }
+        else
+        {
+#pragma unroll
+            for (int kw = 0; kw < K; ++kw)
+                gx[at + kh * W + kw] = (hit == kh * K + kw ? v : 0.f) * ((x[at + kh * W + kw] > 0.f) ? 1.f : 0.f);
+        }
+    }
+}
+
+// gx[i] *= (x[i] > 0 ? 1 : 0) for the window shapes without a fused kernel
+__global__ __launch_bounds__(256) void relu_mask_inplace_kernel(float *__restrict__ gx, const float *__restrict__ x, int64_t n)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n)
+        gx[i] = gx[i] * ((x[i] > 0.f) ? 1.f : 0.f);
+}
+
 // Forward of the 2x2 / stride 2 / no padding pooling over an image whose rows hold a multiple of four floats: a thread
 // owns two neighbouring outputs, reads the four cells under them from each of the two image rows with one 16-byte load
 // and stores the two maxima (8 bytes) and the two indices (16 bytes) together. The comparisons are those of the general
@@ -513,6 +559,40 @@ int odl_hip_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N,
     else
         hipLaunchKernelGGL(max_pool_bwd_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, gy, idx, gx,
                            g);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_max_pool2d_backward_relu(const float *gy, const uint64_t *idx, const float *x, int64_t N, int64_t C, int64_t H,
+                                     int64_t W, int KH, int KW, int SH, int SW, int PH, int PW, float *gx, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    PoolGeom g;
+    int rc = make_geom(g, "max_pool2d_backward_relu", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(idx != nullptr && x != nullptr, "max_pool2d_backward_relu: indices or pooled input missing");
+    const int64_t total = N * C * H * W;
+    if (total == 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    if (plane_ok(g) && tiles_exactly(g) && ((reinterpret_cast<uintptr_t>(gx) | reinterpret_cast<uintptr_t>(x)) & 7) == 0)
+    {
+        const unsigned outputs = (unsigned)(N * C * g.OH * g.OW);
+        const dim3 grid((unsigned)odl::ceil_div((int64_t)outputs, 256));
+        if (g.KH == 2)
+            hipLaunchKernelGGL((max_pool_bwd_tiled_relu_kernel<2>), grid, dim3(256), 0, st, gy, idx, x, gx, outputs, (int)g.OW,
+                               (unsigned)(g.OH * g.OW));
+        else
+            hipLaunchKernelGGL((max_pool_bwd_tiled_relu_kernel<3>), grid, dim3(256), 0, st, gy, idx, x, gx, outputs, (int)g.OW,
+                               (unsigned)(g.OH * g.OW));
+        ODL_LAUNCH_CHECK();
+        return ODL_OK;
+    }
+    rc = odl_hip_max_pool2d_backward(gy, idx, N, C, H, W, KH, KW, SH, SW, PH, PW, gx, stream);
+    if (rc != ODL_OK)
+        return rc;
+    hipLaunchKernelGGL(relu_mask_inplace_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, gx, x, total);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

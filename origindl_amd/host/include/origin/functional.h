@@ -105,6 +105,11 @@ Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b);
 // relu(linear(x, w, b)) and relu(conv2d(x, W, b)) as one operator each, for device tensors (float32)
 Tensor linear_relu(const Tensor &x, const Tensor &w, const Tensor &b);
 Tensor conv2d_relu(const Tensor &x, const Tensor &W, const Tensor *b, std::pair<int, int> stride, std::pair<int, int> pad);
+// max_pool2d(relu(conv2d(x, W, b)), ...) as one operator: same values, and in backward the pooling gradient is masked by
+// the ReLU as it is written
+Tensor conv2d_relu_max_pool2d(const Tensor &x, const Tensor &W, const Tensor *b, std::pair<int, int> stride,
+                              std::pair<int, int> pad, std::pair<int, int> pool_kernel, std::pair<int, int> pool_stride,
+                              std::pair<int, int> pool_pad);
 Tensor softmax(const Tensor &x, int axis = -1);
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &target);
 // After replaying a recorded step on new labels: whether the loss kernel met an out-of-range label (the ordinary call

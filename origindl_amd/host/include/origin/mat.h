@@ -348,6 +348,11 @@ public:
     std::unique_ptr<Mat> max_pool2d_backward_device(const Mat &gy, std::pair<int, int> kernel_size,
                                                     std::pair<int, int> stride, std::pair<int, int> pad,
                                                     const Storage &indices) const;
+    // ... and with the backward of the ReLU that produced this (the pooled) tensor applied in the same pass:
+    // max_pool2d_backward_device(...)->relu_backward(*this), same floats
+    std::unique_ptr<Mat> max_pool2d_backward_relu_device(const Mat &gy, std::pair<int, int> kernel_size,
+                                                         std::pair<int, int> stride, std::pair<int, int> pad,
+                                                         const Storage &indices) const;
     // The loss and its gradient without the host round trip of the pair above: the loss stays a device scalar and the
     // upstream gradient is read from device memory. For steps recorded into a graph; an out-of-range label is not
     // reported here (the flag stays on the device).

@@ -90,6 +90,9 @@ public:
     Conv2d(int in_channels, int out_channels, int kernel_size, int stride = 1, int pad = 0, bool bias = true);
     Tensor forward(const Tensor &input) override;
     Tensor forward_relu(const Tensor &input);  // relu(forward(input)), as Linear::forward_relu
+    // max_pool2d(relu(forward(input)), ...) as one operator
+    Tensor forward_relu_pool(const Tensor &input, std::pair<int, int> pool_kernel, std::pair<int, int> pool_stride,
+                             std::pair<int, int> pool_pad);
     Parameter *weight() { return &weight_; }
     Parameter *bias() { return use_bias_ ? &bias_ : nullptr; }
 
@@ -106,6 +109,9 @@ public:
     MaxPool2d(std::pair<int, int> kernel_size, std::pair<int, int> stride = {0, 0}, std::pair<int, int> pad = {0, 0});
     MaxPool2d(int kernel_size, int stride = 0, int pad = 0);
     Tensor forward(const Tensor &input) override { return functional::max_pool2d(input, kernel_, stride_, pad_); }
+    std::pair<int, int> kernel_size() const { return kernel_; }
+    std::pair<int, int> stride() const { return stride_; }
+    std::pair<int, int> pad() const { return pad_; }
 
 private:
     std::pair<int, int> kernel_, stride_, pad_;

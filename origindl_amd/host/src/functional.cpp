@@ -497,6 +497,39 @@ struct MaxPool2d : Operator  // src/operators/pooling/max_pool2d.cpp:14-86
     }
 };
 
+// Conv2d -> ReLU -> MaxPool2d as one operator (the two tensors in between are not visible from outside): the activation
+// in the convolution's epilogue, and in backward the pooling gradient masked by the ReLU as it is written. The values are
+// those of the three operators run in turn (src/operators/conv/conv2d.cpp, activation/relu.cpp, pooling/max_pool2d.cpp).
+struct Conv2dReluPoolOp : Conv2dOp
+{
+    std::pair<int, int> pk, ps, pp;
+    std::shared_ptr<Mat> y;            // relu(conv(x)), the pooled tensor
+    std::shared_ptr<Storage> indices;  // window-local argmax per output, uint64, kept on the device
+    Conv2dReluPoolOp(std::pair<int, int> st, std::pair<int, int> pd, std::pair<int, int> k, std::pair<int, int> s,
+                     std::pair<int, int> p)
+        : Conv2dOp(st, pd), pk(k), ps(s), pp(p)
+    {}
+    std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
+    {
+        validate(xs);
+        const Mat *b = xs.size() == 3 ? &mat(xs[2]) : nullptr;
+        y            = std::shared_ptr<Mat>(omat(xs[0]).conv2d_act(mat(xs[1]), b, stride, pad, 0));
+        const auto *yo = dynamic_cast<const OriginMat *>(y.get());
+        return {wrap(yo->max_pool2d_device(pk, ps, pp, &indices))};
+    }
+    std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
+    {
+        const auto *yo = dynamic_cast<const OriginMat *>(y.get());
+        auto g0        = yo->max_pool2d_backward_relu_device(mat(gys[0]), pk, ps, pp, *indices);
+        const Mat *b   = inputs_.size() == 3 ? &mat(inputs_[2]) : nullptr;
+        auto grads     = g0->conv2d_backward(*g0, mat(inputs_[0]), mat(inputs_[1]), b, stride, pad);
+        std::vector<Tensor> out;
+        for (auto &g : grads)
+            out.push_back(wrap(std::move(g)));
+        return out;
+    }
+};
+
 struct Sigmoid : Operator  // src/operators/activation/sigmoid.cpp:13-44: keeps y, gx = gy*y*(1-y)
 {
     Tensor y;
@@ -811,6 +844,15 @@ Tensor conv2d_relu(const Tensor &x, const Tensor &W, const Tensor *b, std::pair<
     if (b)
         in.push_back(*b);
     return apply<Conv2dReluOp>(in, stride, pad);
+}
+Tensor conv2d_relu_max_pool2d(const Tensor &x, const Tensor &W, const Tensor *b, std::pair<int, int> stride,
+                              std::pair<int, int> pad, std::pair<int, int> pool_kernel, std::pair<int, int> pool_stride,
+                              std::pair<int, int> pool_pad)
+{
+    std::vector<Tensor> in{x, W};
+    if (b)
+        in.push_back(*b);
+    return apply<Conv2dReluPoolOp>(in, stride, pad, pool_kernel, pool_stride, pool_pad);
 }
 Tensor softmax(const Tensor &x, int axis) { return apply<Softmax>({x}, axis); }
 Tensor softmax_cross_entropy(const Tensor &x, const Tensor &t) { return apply<SoftmaxCrossEntropy>({x, t}); }

@@ -1560,6 +1560,23 @@ std::unique_ptr<Mat> OriginMat::max_pool2d_backward_device(const Mat &gym, std::
     return gx;
 }
 
+std::unique_ptr<Mat> OriginMat::max_pool2d_backward_relu_device(const Mat &gym, std::pair<int, int> k, std::pair<int, int> s,
+                                                                std::pair<int, int> p, const Storage &indices) const
+{
+    const OriginMat &gy = dev_f32(gym, "max_pool2d_backward");
+    const OriginMat &x  = dev_f32(*this, "max_pool2d_backward");
+    if (gy.shape().size() != 4)
+        THROW_INVALID_ARG("max_pool2d_backward: gy must be 4D (N, C, OH, OW), but got shape {}", gy.shape().to_string());
+    if (indices.size() < gy.elements() * sizeof(uint64_t) || indices.device_type() != DeviceType::kCUDA)
+        THROW_INVALID_ARG("max_pool2d_backward: indices size mismatch. Expected {}, got {}", gy.elements(),
+                          indices.size() / sizeof(uint64_t));
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
+    auto gx = new_like(gy, shape_);
+    check(odl_hip_max_pool2d_backward_relu(fp(gy), static_cast<const uint64_t *>(indices.data()), fp(x), N, C, H, W, k.first,
+                                           k.second, s.first, s.second, p.first, p.second, gx->data_ptr<float>(), cur()));
+    return gx;
+}
+
 std::unique_ptr<Mat> OriginMat::max_pool2d_backward(const Mat &gym, std::pair<int, int> k, std::pair<int, int> s,
                                                     std::pair<int, int> p, const std::vector<size_t> &indices) const
 {

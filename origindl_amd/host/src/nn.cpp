@@ -195,6 +195,14 @@ Tensor Sequential::forward(const Tensor &input)
             }
             if (typeid(l) == typeid(nn::Conv2d))
             {
+                if (i + 2 < layers_.size() && typeid(*layers_[i + 2]) == typeid(nn::MaxPool2d))
+                {
+                    // ... and a MaxPool2d after the pair joins it: its gradient is masked by the ReLU as it is written
+                    const auto &pool = static_cast<const nn::MaxPool2d &>(*layers_[i + 2]);
+                    x = static_cast<nn::Conv2d &>(l).forward_relu_pool(x, pool.kernel_size(), pool.stride(), pool.pad());
+                    i += 2;
+                    continue;
+                }
                 x = static_cast<nn::Conv2d &>(l).forward_relu(x);
                 ++i;
                 continue;
@@ -321,6 +329,17 @@ Tensor Conv2d::forward_relu(const Tensor &input)
         return functional::relu(forward(input));
     const Tensor *b = use_bias_ ? &static_cast<const Tensor &>(bias_) : nullptr;
     return functional::conv2d_relu(input, static_cast<const Tensor &>(weight_), b, stride_, pad_);
+}
+
+Tensor Conv2d::forward_relu_pool(const Tensor &input, std::pair<int, int> pool_kernel, std::pair<int, int> pool_stride,
+                                 std::pair<int, int> pool_pad)
+{
+    if (input.shape().size() != 4 || input.shape()[1] != (size_t)in_channels_ ||
+        input.device().type() != DeviceType::kCUDA || input.dtype() != DataType::kFloat32)
+        return functional::max_pool2d(functional::relu(forward(input)), pool_kernel, pool_stride, pool_pad);
+    const Tensor *b = use_bias_ ? &static_cast<const Tensor &>(bias_) : nullptr;
+    return functional::conv2d_relu_max_pool2d(input, static_cast<const Tensor &>(weight_), b, stride_, pad_, pool_kernel,
+                                              pool_stride, pool_pad);
 }
 
 MaxPool2d::MaxPool2d(std::pair<int, int> kernel_size, std::pair<int, int> stride, std::pair<int, int> pad)

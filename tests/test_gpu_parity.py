@@ -1330,3 +1330,27 @@ def test_im2col_3x3_matrix_layout_is_bit_identical_to_the_gather_loop(api, o, N,
     o.orc_im2col(x, N, C, H, W, 3, 3, S, S, 1, 1, 1, want)
     got = host(api.im2col(dev(x), 3, S, 1, True))
     assert np.array_equal(got, want)
+
+
+def test_max_pool_backward_with_the_relu_mask_folded_in_equals_the_two_steps(api):
+    # src/operators/pooling/max_pool2d.cpp:60-86 then src/operators/activation/relu.cpp:23-29 (gy * (x > 0 ? 1 : 0)): the
+    # fused entry must give the bits of the two calls in turn, signed zeros included — windows that tile the image exactly
+    # (one masked write per cell) and windows that do not (the two steps behind one call)
+    import ctypes
+    L = api.lib()
+    rng = np.random.default_rng(171)
+    for N, C, H, W, K, S, P in ((3, 5, 8, 12, 2, 2, 0), (2, 4, 9, 9, 3, 3, 0), (2, 3, 9, 10, 3, 2, 1), (1, 2, 7, 7, 2, 2, 0),
+                                (4, 16, 28, 28, 2, 2, 0)):
+        x = np.maximum(rng.standard_normal((N, C, H, W), dtype=f32), 0)  # a ReLU output: zeros where the mask is 0
+        xd = dev(x)
+        y, idx = api.max_pool2d(xd, K, S, P)
+        gy = rng.standard_normal(tuple(y.shape), dtype=f32)
+        gy.ravel()[::5] = -0.0
+        gyd = dev(gy)
+        gx_pool = api.max_pool2d_backward(gyd, idx, x.shape, K, S, P)
+        want = host(gx_pool) * (x > 0).astype(f32)  # the product, so that -g * 0 keeps its sign
+        got = torch.empty_like(xd)
+        L.call("odl_hip_max_pool2d_backward_relu", gyd.data_ptr(), idx.data_ptr(), xd.data_ptr(), N, C, H, W, K, K, S, S, P, P,
+               got.data_ptr(), None)
+        g = host(got)
+        assert np.array_equal(g, want) and np.array_equal(np.signbit(g), np.signbit(want)), (N, C, H, W, K, S, P)
