@@ -357,7 +357,22 @@ int odl_hip_batch_norm_backward_from_x(const float *gy, const float *x, const fl
                                        const float *saved_var, float eps, int64_t N, int64_t C, int64_t P, float *gx,
                                        float *dgamma, float *dbeta, void *workspace, size_t workspace_bytes,
                                        void *stream);
-/* workspace of either call (partial channel sums) */
+/* A batch normalisation whose output goes straight into a ReLU, as in the reference's CNN example
+ * (tests/example/mnist/conv_mnist.cpp: Conv2d, BatchNorm2d, ReLU, MaxPool2d): y = relu(gamma * x_norm + beta) is
+ * written once instead of the normalised tensor and then its ReLU; mean / var as in the plain forward, no x_norm.
+ * The backward takes the gradient of the ReLU's OUTPUT: the mask gamma * x_norm + beta > 0 is formed again from x and
+ * the saved statistics (the floats of the forward pass), gy is multiplied by 1 or 0 as the separate ReLU backward
+ * does (relu.cpp:45-52), and the sums and gx follow from that product. Results equal the two separate steps bit
+ * for bit. */
+int odl_hip_batch_norm_relu_forward(const float *x, const float *gamma, const float *beta, const float *running_mean,
+                                    const float *running_var, int training, float eps, int64_t N, int64_t C, int64_t P,
+                                    float *y, float *mean, float *var, void *workspace, size_t workspace_bytes,
+                                    void *stream);
+int odl_hip_batch_norm_relu_backward_from_x(const float *gy, const float *x, const float *gamma, const float *beta,
+                                            const float *saved_mean, const float *saved_var, float eps, int64_t N,
+                                            int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta,
+                                            void *workspace, size_t workspace_bytes, void *stream);
+/* workspace of any of these calls (partial channel sums) */
 size_t odl_hip_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t P);
 /* The same on float64 tensors (src/mat/origin/cuda/normalization/batch_norm.cu:497-560 accepts float32 and float64): one
  * workgroup per channel, no workspace. x_norm may be NULL. backward: x_norm_or_x is the saved normalised input

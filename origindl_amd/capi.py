@@ -423,7 +423,7 @@ def accuracy(y, t):
 
 # -------------------------------------------------------------------------------------- elementwise
 _BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "gt": 4, "eq": 5, "ne": 6, "lt": 7, "le": 8, "ge": 9,
-        "sigmoid_backward": 10, "silu_backward": 11}
+        "sigmoid_backward": 10, "silu_backward": 11, "relu_backward": 12}
 _UN = {"relu": 0, "exp": 1, "log": 2, "neg": 3, "square": 4, "sqrt": 5, "sigmoid": 6, "silu": 7}
 
 
@@ -576,6 +576,39 @@ def batch_norm_backward_from_x(gy, x, gamma, saved_mean, saved_var, eps=1e-5):
     ws, nb = _ws(lib().query("odl_hip_batch_norm_workspace_bytes", N, C, P))
     lib().call("odl_hip_batch_norm_backward_from_x", _p(gy), _p(x), _p(gamma), _p(saved_mean), _p(saved_var), float(eps),
                N, C, P, _p(gx), _p(dg), _p(db), _p(ws), nb, _stream())
+    return gx, dg, db
+
+
+def batch_norm_relu_forward(x, gamma, beta, running_mean, running_var, training, eps=1e-5):
+    """relu(batch_norm(x)) written once (the BatchNorm2d + ReLU pair of tests/example/mnist/conv_mnist.cpp)
+    -> (y, mean, var)."""
+    for name, t in (("x", x), ("gamma", gamma), ("beta", beta), ("running_mean", running_mean),
+                    ("running_var", running_var)):
+        _chk(t, name)
+    N, C, P = _bn_dims(x, "batch_norm")
+    for t in (gamma, beta, running_mean, running_var):
+        if tuple(t.shape) != (C,):
+            raise OdlInvalidArgument("batch_norm: gamma, beta, running_mean, running_var must have shape (%d)" % C)
+    y, mean, var = _empty(x.shape), _empty((C,)), _empty((C,))
+    ws, nb = _ws(lib().query("odl_hip_batch_norm_workspace_bytes", N, C, P) if training else 0)
+    lib().call("odl_hip_batch_norm_relu_forward", _p(x), _p(gamma), _p(beta), _p(running_mean), _p(running_var),
+               1 if training else 0, float(eps), N, C, P, _p(y), _p(mean), _p(var), _p(ws), nb, _stream())
+    return y, mean, var
+
+
+def batch_norm_relu_backward_from_x(gy, x, gamma, beta, saved_mean, saved_var, eps=1e-5):
+    """Backward of the pair: gy is the gradient of the ReLU's output; the mask is formed again from x and the saved
+    statistics -> (gx, dgamma, dbeta)."""
+    for name, t in (("gy", gy), ("x", x), ("gamma", gamma), ("beta", beta), ("saved_mean", saved_mean),
+                    ("saved_var", saved_var)):
+        _chk(t, name)
+    N, C, P = _bn_dims(gy, "batch_norm_backward")
+    if x.shape != gy.shape or any(tuple(t.shape) != (C,) for t in (gamma, beta, saved_mean, saved_var)):
+        raise OdlInvalidArgument("batch_norm_backward: shape mismatch")
+    gx, dg, db = _empty(gy.shape), _empty((C,)), _empty((C,))
+    ws, nb = _ws(lib().query("odl_hip_batch_norm_workspace_bytes", N, C, P))
+    lib().call("odl_hip_batch_norm_relu_backward_from_x", _p(gy), _p(x), _p(gamma), _p(beta), _p(saved_mean),
+               _p(saved_var), float(eps), N, C, P, _p(gx), _p(dg), _p(db), _p(ws), nb, _stream())
     return gx, dg, db
 
 

@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kBlock) void bn_sqdiff_kernel(const float *__restri
 
 // mean / variance either from the batch (sqsums != nullptr: variance = its total / count, mean as already stored) or
 // from the running statistics; writes the statistics used, x_norm (when asked for) and y
-template <bool V4>
+template <bool V4, bool RELU>
 __global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                            const float *__restrict__ beta,
                                                            const float *__restrict__ mean_src,
@@ -161,6 +161,8 @@ __global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float *__restric
             {
                 xn[i] = (q[i] - mean) / stdv;
                 o[i] = ga * xn[i] + be;
+                if (RELU)
+                    o[i] = odl::apply_act(o[i], 1);
             }
             if (x_norm)
                 *reinterpret_cast<f32x4 *>(x_norm + off) = xn;
@@ -171,26 +173,35 @@ __global__ __launch_bounds__(kBlock) void bn_apply_kernel(const float *__restric
             const float xn = (x[off] - mean) / stdv;
             if (x_norm)
                 x_norm[off] = xn;
-            y[off] = ga * xn + be;
+            const float o = ga * xn + be;
+            y[off] = RELU ? odl::apply_act(o, 1) : o;
         }
     });
 }
 
 // FROM_X: `xn` holds x itself and the normalised value is formed here, (x - mean) / sqrt(var + eps) — the expression
 // the forward pass used, so the same float — instead of being read back from a saved copy.
-template <bool V4, bool FROM_X>
+//
+// RELU: the layer's output went through a ReLU before anything else saw it, and `gy` is the gradient of THAT output.
+// The ReLU's mask is formed again from the expression the forward pass evaluated, gamma * xn + beta > 0, and gy is
+// multiplied by 1 or 0 as the separate ReLU backward would (relu.cpp:45-52), so both kernels see the masked gradient
+// without it ever being stored.
+template <bool V4, bool FROM_X, bool RELU>
 __global__ __launch_bounds__(kBlock) void bn_bwd_sums_kernel(const float *__restrict__ gy, const float *__restrict__ xn,
+                                                              const float *__restrict__ gamma,
+                                                              const float *__restrict__ beta,
                                                               const float *__restrict__ mean,
                                                               const float *__restrict__ var, float eps,
                                                               float *__restrict__ part, BnGeom g)
 {
     const float mu = FROM_X ? mean[blockIdx.y] : 0.f;
     const float sd = FROM_X ? sqrtf(var[blockIdx.y] + eps) : 1.f;
+    const float ga = RELU ? gamma[blockIdx.y] : 0.f, be = RELU ? beta[blockIdx.y] : 0.f;
     float a[4] = {0.f, 0.f, 0.f, 0.f}, b[4] = {0.f, 0.f, 0.f, 0.f};
     visit_chunk<V4>(g, [&](int64_t off, int j) {
         if (V4)
         {
-            const f32x4 q = *reinterpret_cast<const f32x4 *>(gy + off);
+            f32x4 q = *reinterpret_cast<const f32x4 *>(gy + off);
             f32x4 r = *reinterpret_cast<const f32x4 *>(xn + off);
             if (FROM_X)
             {
@@ -198,14 +209,21 @@ __global__ __launch_bounds__(kBlock) void bn_bwd_sums_kernel(const float *__rest
                 for (int i = 0; i < 4; ++i)
                     r[i] = (r[i] - mu) / sd;
             }
+            if (RELU)
+            {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    q[i] = q[i] * (ga * r[i] + be > 0.f ? 1.f : 0.f);
+            }
             a[j] += (q[0] + q[1]) + (q[2] + q[3]);
             b[j] += (q[0] * r[0] + q[1] * r[1]) + (q[2] * r[2] + q[3] * r[3]);
         }
         else
         {
             const float r = FROM_X ? (xn[off] - mu) / sd : xn[off];
-            a[j] += gy[off];
-            b[j] += gy[off] * r;
+            const float q = RELU ? gy[off] * (ga * r + be > 0.f ? 1.f : 0.f) : gy[off];
+            a[j] += q;
+            b[j] += q * r;
         }
     });
     const float sa = block_sum_all((a[0] + a[1]) + (a[2] + a[3]));
@@ -217,9 +235,10 @@ __global__ __launch_bounds__(kBlock) void bn_bwd_sums_kernel(const float *__rest
     }
 }
 
-template <bool V4, bool FROM_X>
+template <bool V4, bool FROM_X, bool RELU>
 __global__ __launch_bounds__(kBlock) void bn_bwd_apply_kernel(const float *__restrict__ gy, const float *__restrict__ xn,
                                                                const float *__restrict__ gamma,
+                                                               const float *__restrict__ beta,
                                                                const float *__restrict__ mean,
                                                                const float *__restrict__ var,
                                                                const float *__restrict__ part, float *__restrict__ gx,
@@ -234,10 +253,11 @@ __global__ __launch_bounds__(kBlock) void bn_bwd_apply_kernel(const float *__res
         dgamma[c] = sum_gy_xn, dbeta[c] = sum_gy;
     const float mean_gy = sum_gy / count, mean_gy_xn = sum_gy_xn / count;
     const float scale = gamma[c] / sd;
+    const float ga = gamma[c], be = RELU ? beta[c] : 0.f;
     visit_chunk<V4>(g, [&](int64_t off, int) {
         if (V4)
         {
-            const f32x4 q = *reinterpret_cast<const f32x4 *>(gy + off);
+            f32x4 q = *reinterpret_cast<const f32x4 *>(gy + off);
             f32x4 r = *reinterpret_cast<const f32x4 *>(xn + off);
             f32x4 o;
 #pragma unroll
@@ -245,6 +265,8 @@ __global__ __launch_bounds__(kBlock) void bn_bwd_apply_kernel(const float *__res
             {
                 if (FROM_X)
                     r[i] = (r[i] - mu) / sd;
+                if (RELU)
+                    q[i] = q[i] * (ga * r[i] + be > 0.f ? 1.f : 0.f);
                 const float t = r[i] * mean_gy_xn;
                 o[i] = scale * ((q[i] - mean_gy) - t);
             }
@@ -253,8 +275,9 @@ __global__ __launch_bounds__(kBlock) void bn_bwd_apply_kernel(const float *__res
         else
         {
             const float r = FROM_X ? (xn[off] - mu) / sd : xn[off];
+            const float q = RELU ? gy[off] * (ga * r + be > 0.f ? 1.f : 0.f) : gy[off];
             const float t = r * mean_gy_xn;
-            gx[off] = scale * ((gy[off] - mean_gy) - t);
+            gx[off] = scale * ((q - mean_gy) - t);
         }
     });
 }
@@ -318,10 +341,10 @@ size_t odl_hip_batch_norm_workspace_bytes(int64_t N, int64_t C, int64_t P)
     return (size_t)C * g.ns * 2 * sizeof(float);
 }
 
-int odl_hip_batch_norm_forward(const float *x, const float *gamma, const float *beta, const float *running_mean,
-                               const float *running_var, int training, float eps, int64_t N, int64_t C, int64_t P,
-                               float *y, float *mean, float *var, float *x_norm, void *workspace,
-                               size_t workspace_bytes, void *stream)
+static int bn_forward_launch(const float *x, const float *gamma, const float *beta, const float *running_mean,
+                             const float *running_var, int training, float eps, int64_t N, int64_t C, int64_t P, float *y,
+                             float *mean, float *var, float *x_norm, bool relu, void *workspace, size_t workspace_bytes,
+                             void *stream)
 {
     ODL_REQUIRE_DEVICE();
     BnGeom g;
@@ -356,18 +379,42 @@ int odl_hip_batch_norm_forward(const float *x, const float *gamma, const float *
         ODL_LAUNCH_CHECK();
     }
     const float *mean_src = training ? mean : running_mean;
-    if (v4)
-        hipLaunchKernelGGL((bn_apply_kernel<true>), grid, block, 0, st, x, gamma, beta, mean_src, running_var, sqsums,
-                           mean, var, y, x_norm, g, count, eps);
+#define ODL_BN_APPLY(V4, RELU)                                                                                       \
+    hipLaunchKernelGGL((bn_apply_kernel<V4, RELU>), grid, block, 0, st, x, gamma, beta, mean_src, running_var, sqsums, \
+                       mean, var, y, x_norm, g, count, eps)
+    if (v4 && relu)
+        ODL_BN_APPLY(true, true);
+    else if (v4)
+        ODL_BN_APPLY(true, false);
+    else if (relu)
+        ODL_BN_APPLY(false, true);
     else
-        hipLaunchKernelGGL((bn_apply_kernel<false>), grid, block, 0, st, x, gamma, beta, mean_src, running_var, sqsums,
-                           mean, var, y, x_norm, g, count, eps);
+        ODL_BN_APPLY(false, false);
+#undef ODL_BN_APPLY
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
 
-static int bn_backward_launch(const float *gy, const float *gamma, const float *saved_mean, const float *saved_var,
-                              const float *xn_or_x, bool from_x, float eps, int64_t N, int64_t C, int64_t P, float *gx,
+int odl_hip_batch_norm_forward(const float *x, const float *gamma, const float *beta, const float *running_mean,
+                               const float *running_var, int training, float eps, int64_t N, int64_t C, int64_t P,
+                               float *y, float *mean, float *var, float *x_norm, void *workspace,
+                               size_t workspace_bytes, void *stream)
+{
+    return bn_forward_launch(x, gamma, beta, running_mean, running_var, training, eps, N, C, P, y, mean, var, x_norm,
+                             false, workspace, workspace_bytes, stream);
+}
+
+int odl_hip_batch_norm_relu_forward(const float *x, const float *gamma, const float *beta, const float *running_mean,
+                                    const float *running_var, int training, float eps, int64_t N, int64_t C, int64_t P,
+                                    float *y, float *mean, float *var, void *workspace, size_t workspace_bytes,
+                                    void *stream)
+{
+    return bn_forward_launch(x, gamma, beta, running_mean, running_var, training, eps, N, C, P, y, mean, var, nullptr,
+                             true, workspace, workspace_bytes, stream);
+}
+
+static int bn_backward_launch(const float *gy, const float *gamma, const float *beta_for_relu, const float *saved_mean,
+                              const float *saved_var, const float *xn_or_x, bool from_x, float eps, int64_t N, int64_t C, int64_t P, float *gx,
                               float *dgamma, float *dbeta, void *workspace, size_t workspace_bytes, void *stream)
 {
     ODL_REQUIRE_DEVICE();
@@ -390,26 +437,37 @@ static int bn_backward_launch(const float *gy, const float *gamma, const float *
     g.by_plane = odl::make_fastdiv((unsigned)(v4 ? P / 4 : P));
     const dim3 grid(g.ns, g.C), block(kBlock);
     const float count = (float)(N * P);
-#define ODL_BN_BWD(V4, FX)                                                                                          \
-    hipLaunchKernelGGL((bn_bwd_sums_kernel<V4, FX>), grid, block, 0, st, gy, xn_or_x, saved_mean, saved_var, eps, part, \
-                       g);                                                                                          \
-    hipLaunchKernelGGL((bn_bwd_apply_kernel<V4, FX>), grid, block, 0, st, gy, xn_or_x, gamma, saved_mean, saved_var,    \
-                       part, gx, dgamma, dbeta, g, count, eps)
-    if (v4 && from_x)
+#define ODL_BN_BWD(V4, FX, RELU)                                                                                    \
+    hipLaunchKernelGGL((bn_bwd_sums_kernel<V4, FX, RELU>), grid, block, 0, st, gy, xn_or_x, gamma, beta_for_relu,       \
+                       saved_mean, saved_var, eps, part, g);                                                        \
+    hipLaunchKernelGGL((bn_bwd_apply_kernel<V4, FX, RELU>), grid, block, 0, st, gy, xn_or_x, gamma, beta_for_relu,      \
+                       saved_mean, saved_var, part, gx, dgamma, dbeta, g, count, eps)
+    if (beta_for_relu)  // the fused layer keeps x, never x_norm
     {
-        ODL_BN_BWD(true, true);
+        if (v4)
+        {
+            ODL_BN_BWD(true, true, true);
+        }
+        else
+        {
+            ODL_BN_BWD(false, true, true);
+        }
+    }
+    else if (v4 && from_x)
+    {
+        ODL_BN_BWD(true, true, false);
     }
     else if (v4)
     {
-        ODL_BN_BWD(true, false);
+        ODL_BN_BWD(true, false, false);
     }
     else if (from_x)
     {
-        ODL_BN_BWD(false, true);
+        ODL_BN_BWD(false, true, false);
     }
     else
     {
-        ODL_BN_BWD(false, false);
+        ODL_BN_BWD(false, false, false);
     }
 #undef ODL_BN_BWD
     ODL_LAUNCH_CHECK();
@@ -420,7 +478,7 @@ int odl_hip_batch_norm_backward(const float *gy, const float *gamma, const float
                                 float eps, int64_t N, int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta,
                                 void *workspace, size_t workspace_bytes, void *stream)
 {
-    return bn_backward_launch(gy, gamma, nullptr, saved_var, saved_x_norm, false, eps, N, C, P, gx, dgamma, dbeta,
+    return bn_backward_launch(gy, gamma, nullptr, nullptr, saved_var, saved_x_norm, false, eps, N, C, P, gx, dgamma, dbeta,
                               workspace, workspace_bytes, stream);
 }
 
@@ -429,7 +487,18 @@ int odl_hip_batch_norm_backward_from_x(const float *gy, const float *x, const fl
                                        float *dgamma, float *dbeta, void *workspace, size_t workspace_bytes,
                                        void *stream)
 {
-    return bn_backward_launch(gy, gamma, saved_mean, saved_var, x, true, eps, N, C, P, gx, dgamma, dbeta, workspace,
+    return bn_backward_launch(gy, gamma, nullptr, saved_mean, saved_var, x, true, eps, N, C, P, gx, dgamma, dbeta, workspace,
+                              workspace_bytes, stream);
+}
+
+int odl_hip_batch_norm_relu_backward_from_x(const float *gy, const float *x, const float *gamma, const float *beta,
+                                            const float *saved_mean, const float *saved_var, float eps, int64_t N,
+                                            int64_t C, int64_t P, float *gx, float *dgamma, float *dbeta,
+                                            void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!beta)
+        return odl::fail(ODL_ERR_INVALID_ARG, "batch_norm_relu_backward: null operand");
+    return bn_backward_launch(gy, gamma, beta, saved_mean, saved_var, x, true, eps, N, C, P, gx, dgamma, dbeta, workspace,
                               workspace_bytes, stream);
 }
 

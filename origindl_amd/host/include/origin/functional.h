@@ -100,6 +100,10 @@ Tensor batch_norm(const Tensor &x, const Tensor &gamma, const Tensor &beta, cons
 std::vector<Tensor> batch_norm_outputs(const Tensor &x, const Tensor &gamma, const Tensor &beta,
                                        const Tensor &running_mean, const Tensor &running_var, bool training, float eps,
                                        float momentum, int num_dims);
+// ... with a ReLU applied to y before it leaves the operator (float32 device tensors): what batch_norm then relu give
+std::vector<Tensor> batch_norm_relu_outputs(const Tensor &x, const Tensor &gamma, const Tensor &beta,
+                                            const Tensor &running_mean, const Tensor &running_var, bool training,
+                                            float eps, float momentum, int num_dims);
 // x[M,K] . w[K,N] + b (b of N elements) in one kernel; what nn::Linear::forward uses for 2-D inputs
 Tensor linear(const Tensor &x, const Tensor &w, const Tensor &b);
 // relu(linear(x, w, b)) and relu(conv2d(x, W, b)) as one operator each, for device tensors (float32)

@@ -391,10 +391,14 @@ public:
     // Batch norm for an operator that keeps x anyway: the forward without the x_norm output (result.x_norm is null),
     // and the backward that forms x_norm again from x (this) and the saved statistics — the same floats, 4 bytes per
     // element less written in forward and one saved activation less.
+    // relu / beta_for_relu (float32 only): the layer's output passes through a ReLU on its way out, and the backward
+    // takes the gradient of that ReLU's output, forming the mask again from gamma * x_norm + beta.
     BatchNormResult batch_norm_forward_no_xnorm(const Mat &gamma, const Mat &beta, const Mat &running_mean,
-                                                const Mat &running_var, bool training, float eps, int num_dims) const;
+                                                const Mat &running_var, bool training, float eps, int num_dims,
+                                                bool relu = false) const;
     std::vector<std::unique_ptr<Mat>> batch_norm_backward_from_x(const Mat &gy, const Mat &gamma, const Mat &saved_mean,
-                                                                 const Mat &saved_var, float eps, int num_dims) const;
+                                                                 const Mat &saved_var, float eps, int num_dims,
+                                                                 const Mat *beta_for_relu = nullptr) const;
     // gy (this) times the mask x > 0, in one launch: the two kernels of ReLU::backward, same products
     std::unique_ptr<Mat> relu_backward(const Mat &x) const;
     // x . W + b with the activation applied in the product's epilogue (-1 none, 0 relu): what linear() then relu() give

@@ -143,6 +143,9 @@ class BatchNormBase : public Module
 {
 public:
     Tensor forward(const Tensor &input) override;
+    // relu(forward(input)) as one operator on a float32 device tensor: the normalised tensor is never stored, and in
+    // backward the ReLU's mask is formed again inside the normalisation's own kernels (same values either way)
+    Tensor forward_relu(const Tensor &input);
     Parameter *weight() { return &gamma_; }
     Parameter *bias() { return &beta_; }
     const Tensor &running_mean() const { return running_mean_; }
@@ -153,6 +156,7 @@ public:
 
 protected:
     BatchNormBase(const char *name, int num_dims, int num_features, float eps, float momentum);
+    Tensor run(const Tensor &input, bool relu);
     const char *name_;
     int num_dims_, num_features_;
     float eps_, momentum_;

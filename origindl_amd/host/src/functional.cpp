@@ -614,19 +614,20 @@ struct BatchNorm : Operator  // src/operators/normalization/batch_norm.cpp:16-12
     bool training;
     float eps, momentum;
     int num_dims;
+    bool relu;  // the output passes through a ReLU before leaving (the layer pair BatchNorm, ReLU folded into one)
     Tensor saved_mean, saved_var;  // x_norm is not kept: backward forms it again from x and these two (same floats)
-    BatchNorm(bool t, float e, float m, int nd) : training(t), eps(e), momentum(m), num_dims(nd) {}
+    BatchNorm(bool t, float e, float m, int nd, bool r = false) : training(t), eps(e), momentum(m), num_dims(nd), relu(r) {}
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
         if (xs.size() != 5)
             THROW_RUNTIME_ERROR("BatchNorm operator requires exactly 5 inputs (x, gamma, beta, running_mean, "
                                 "running_var), but got {}", xs.size());
         Tensor y;
-        if (training || xs[0].requires_grad() || xs[1].requires_grad() || xs[2].requires_grad())
+        if (relu || training || xs[0].requires_grad() || xs[1].requires_grad() || xs[2].requires_grad())
         {
             // in training mode the layers read the batch statistics off the operator's outputs even without a graph
             auto r = omat(xs[0]).batch_norm_forward_no_xnorm(mat(xs[1]), mat(xs[2]), mat(xs[3]), mat(xs[4]), training, eps,
-                                                             num_dims);
+                                                             num_dims, relu);
             y = wrap(std::move(r.y));
             saved_mean = wrap(std::move(r.mean)), saved_var = wrap(std::move(r.var));
         }
@@ -640,7 +641,7 @@ struct BatchNorm : Operator  // src/operators/normalization/batch_norm.cpp:16-12
     {
         // the gradient of y only: the statistics outputs feed the running averages, outside the graph
         auto r = omat(inputs_[0]).batch_norm_backward_from_x(mat(gys[0]), mat(inputs_[1]), mat(saved_mean), mat(saved_var),
-                                                             eps, num_dims);
+                                                             eps, num_dims, relu ? &mat(inputs_[2]) : nullptr);
         const auto opt = dtype(DataType::kFloat32).device(inputs_[0].device());
         return {wrap(std::move(r[0])), wrap(std::move(r[1])), wrap(std::move(r[2])), Tensor::zeros(inputs_[3].shape(), opt),
                 Tensor::zeros(inputs_[4].shape(), opt)};
@@ -825,6 +826,13 @@ void exp_(Tensor &x) { writable(x).exp_inplace(); }
 void log_(Tensor &x) { writable(x).log_inplace(); }
 void square_(Tensor &x) { writable(x).square_inplace(); }
 void relu_(Tensor &x) { writable(x).relu_inplace(); }
+std::vector<Tensor> batch_norm_relu_outputs(const Tensor &x, const Tensor &gamma, const Tensor &beta, const Tensor &rm,
+                                            const Tensor &rv, bool training, float eps, float momentum, int num_dims)
+{
+    auto op = std::make_shared<BatchNorm>(training, eps, momentum, num_dims, true);
+    return (*op)({x, gamma, beta, rm, rv});
+}
+
 std::vector<Tensor> batch_norm_outputs(const Tensor &x, const Tensor &gamma, const Tensor &beta, const Tensor &rm,
                                        const Tensor &rv, bool training, float eps, float momentum, int num_dims)
 {

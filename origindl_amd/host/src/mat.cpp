@@ -971,11 +971,15 @@ Mat::BatchNormResult OriginMat::batch_norm_forward(const Mat &gamma, const Mat &
 
 Mat::BatchNormResult OriginMat::batch_norm_forward_no_xnorm(const Mat &gamma, const Mat &beta, const Mat &running_mean,
                                                             const Mat &running_var, bool training, float eps,
-                                                            int num_dims) const
+                                                            int num_dims, bool relu) const
 {
     const BnShape s = bn_check("batch_norm", *this, num_dims, gamma, beta, running_mean, running_var);
     if (dtype_ == DataType::kFloat64)
+    {
+        if (relu)
+            THROW_RUNTIME_ERROR("batch_norm: the form with the ReLU folded in takes float32 tensors only");
         return bn_forward_f64(*this, s, gamma, beta, running_mean, running_var, training, eps, false);
+    }
     const OriginMat &x = dev_f32(*this, "batch_norm");
     const OriginMat &g = dev_f32(gamma, "batch_norm"), &b = dev_f32(beta, "batch_norm");
     const OriginMat &rm = dev_f32(running_mean, "batch_norm"), &rv = dev_f32(running_var, "batch_norm");
@@ -983,16 +987,22 @@ Mat::BatchNormResult OriginMat::batch_norm_forward_no_xnorm(const Mat &gamma, co
     auto y = new_like(x, shape_);
     auto mean = new_like(x, Shape({(size_t)s.C})), var = new_like(x, Shape({(size_t)s.C}));
     Workspace ws(training ? odl_hip_batch_norm_workspace_bytes(s.N, s.C, s.P) : 0, device().index());
-    check(odl_hip_batch_norm_forward(fp(x), fp(g), fp(b), fp(rm), fp(rv), training ? 1 : 0, eps, s.N, s.C, s.P,
-                                     y->data_ptr<float>(), mean->data_ptr<float>(), var->data_ptr<float>(), nullptr,
-                                     ws.ptr(), ws.bytes, cur()));
+    if (relu)
+        check(odl_hip_batch_norm_relu_forward(fp(x), fp(g), fp(b), fp(rm), fp(rv), training ? 1 : 0, eps, s.N, s.C, s.P,
+                                              y->data_ptr<float>(), mean->data_ptr<float>(), var->data_ptr<float>(),
+                                              ws.ptr(), ws.bytes, cur()));
+    else
+        check(odl_hip_batch_norm_forward(fp(x), fp(g), fp(b), fp(rm), fp(rv), training ? 1 : 0, eps, s.N, s.C, s.P,
+                                         y->data_ptr<float>(), mean->data_ptr<float>(), var->data_ptr<float>(), nullptr,
+                                         ws.ptr(), ws.bytes, cur()));
     r.y = std::move(y), r.mean = std::move(mean), r.var = std::move(var);
     return r;
 }
 
 std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward_from_x(const Mat &gym, const Mat &gamma,
                                                                         const Mat &saved_mean, const Mat &saved_var,
-                                                                        float eps, int num_dims) const
+                                                                        float eps, int num_dims,
+                                                                        const Mat *beta_for_relu) const
 {
     if (shape_.size() != (size_t)num_dims || (num_dims != 2 && num_dims != 4))
         THROW_INVALID_ARG("batch_norm_backward: x must have {} dimensions (2 or 4), but got shape {}", num_dims,
@@ -1001,8 +1011,14 @@ std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward_from_x(const Ma
     if (gym.shape() != shape_ || gamma.shape() != Shape({C}) || saved_mean.shape() != Shape({C}) ||
         saved_var.shape() != Shape({C}))
         THROW_INVALID_ARG("batch_norm_backward: shape mismatch");
+    if (beta_for_relu && beta_for_relu->shape() != Shape({C}))
+        THROW_INVALID_ARG("batch_norm_backward: shape mismatch");
     if (dtype_ == DataType::kFloat64)
+    {
+        if (beta_for_relu)
+            THROW_RUNTIME_ERROR("batch_norm_backward: the form with the ReLU folded in takes float32 tensors only");
         return bn_backward_f64(*this, gym, *this, true, gamma, saved_mean, saved_var, eps, num_dims);
+    }
     const OriginMat &x = dev_f32(*this, "batch_norm_backward");
     const OriginMat &gy = dev_f32(gym, "batch_norm_backward"), &g = dev_f32(gamma, "batch_norm_backward");
     const OriginMat &sm = dev_f32(saved_mean, "batch_norm_backward"), &sv = dev_f32(saved_var, "batch_norm_backward");
@@ -1010,9 +1026,15 @@ std::vector<std::unique_ptr<Mat>> OriginMat::batch_norm_backward_from_x(const Ma
     auto gx = new_like(x, shape_);
     auto dgamma = new_like(x, Shape({C})), dbeta = new_like(x, Shape({C}));
     Workspace ws(odl_hip_batch_norm_workspace_bytes(N, (int64_t)C, P), device().index());
-    check(odl_hip_batch_norm_backward_from_x(fp(gy), fp(x), fp(g), fp(sm), fp(sv), eps, N, (int64_t)C, P,
-                                             gx->data_ptr<float>(), dgamma->data_ptr<float>(), dbeta->data_ptr<float>(),
-                                             ws.ptr(), ws.bytes, cur()));
+    if (beta_for_relu)
+        check(odl_hip_batch_norm_relu_backward_from_x(fp(gy), fp(x), fp(g), fp(dev_f32(*beta_for_relu, "batch_norm_backward")),
+                                                      fp(sm), fp(sv), eps, N, (int64_t)C, P, gx->data_ptr<float>(),
+                                                      dgamma->data_ptr<float>(), dbeta->data_ptr<float>(), ws.ptr(),
+                                                      ws.bytes, cur()));
+    else
+        check(odl_hip_batch_norm_backward_from_x(fp(gy), fp(x), fp(g), fp(sm), fp(sv), eps, N, (int64_t)C, P,
+                                                 gx->data_ptr<float>(), dgamma->data_ptr<float>(),
+                                                 dbeta->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
     std::vector<std::unique_ptr<Mat>> outs;
     outs.push_back(std::move(gx)), outs.push_back(std::move(dgamma)), outs.push_back(std::move(dbeta));
     return outs;

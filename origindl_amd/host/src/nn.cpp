@@ -145,6 +145,18 @@ void BatchNormBase::to(Device device)
 
 Tensor BatchNormBase::forward(const Tensor &input)
 {
+    return run(input, false);
+}
+
+Tensor BatchNormBase::forward_relu(const Tensor &input)
+{
+    if (input.device().type() != DeviceType::kCUDA || input.dtype() != DataType::kFloat32)
+        return functional::relu(run(input, false));
+    return run(input, true);
+}
+
+Tensor BatchNormBase::run(const Tensor &input, bool relu)
+{
     const Shape s = input.shape();
     if (s.size() != static_cast<size_t>(num_dims_))
         THROW_RUNTIME_ERROR("{} forward: input must be {}, but got shape {}", name_,
@@ -152,9 +164,9 @@ Tensor BatchNormBase::forward(const Tensor &input)
     if (s[1] != static_cast<size_t>(num_features_))
         THROW_RUNTIME_ERROR("{} forward: input feature size {} does not match num_features {}", name_, s[1],
                             num_features_);
-    auto outs = functional::batch_norm_outputs(input, static_cast<const Tensor &>(gamma_),
-                                               static_cast<const Tensor &>(beta_), running_mean_, running_var_,
-                                               is_training(), eps_, momentum_, num_dims_);
+    auto outs = (relu ? functional::batch_norm_relu_outputs : functional::batch_norm_outputs)(
+        input, static_cast<const Tensor &>(gamma_), static_cast<const Tensor &>(beta_), running_mean_, running_var_,
+        is_training(), eps_, momentum_, num_dims_);
     if (is_training() && outs.size() >= 3)
     {
         auto fold = [&](const Tensor &running, const Tensor &batch) {
@@ -179,7 +191,7 @@ Tensor BatchNormBase::forward(const Tensor &input)
 
 Tensor Sequential::forward(const Tensor &input)
 {
-    // A Linear or Conv2d that a ReLU follows runs together with it (the tensor between the two is not visible from
+    // A Linear, Conv2d or batch normalisation that a ReLU follows runs together with it (the tensor between the two is not visible from
     // outside a Sequential); the values are those of the two modules run in turn.
     Tensor x = input;
     for (size_t i = 0; i < layers_.size(); ++i)
@@ -190,6 +202,12 @@ Tensor Sequential::forward(const Tensor &input)
             if (typeid(l) == typeid(nn::Linear))
             {
                 x = static_cast<nn::Linear &>(l).forward_relu(x);
+                ++i;
+                continue;
+            }
+            if (typeid(l) == typeid(nn::BatchNorm2d) || typeid(l) == typeid(nn::BatchNorm1d))
+            {
+                x = static_cast<nn::BatchNormBase &>(l).forward_relu(x);
                 ++i;
                 continue;
             }

@@ -1227,7 +1227,8 @@ int cnn_bench_impl(int64_t N, int steps, int warmup, int graph_mode, float *ms_p
 
 extern "C" {
 #ifdef DRV_ON_DEVICE
-// A Linear or Conv2d that a ReLU follows inside a Sequential runs as one operator. The same network, the same input:
+// A Linear, Conv2d or BatchNorm2d that a ReLU follows inside a Sequential runs as one operator (Conv2d, ReLU, MaxPool2d
+// as one too). The same network, the same input:
 // once through the Sequential, once module by module (nothing paired). diffs[0] counts output elements that differ in
 // any bit, diffs[1] the same over the gradients of all parameters and of the input.
 int DRV(paired_layers_match_separate_modules)(int64_t N, int64_t *diffs)
@@ -1238,13 +1239,20 @@ int DRV(paired_layers_match_separate_modules)(int64_t N, int64_t *diffs)
         model.add(std::make_unique<nn::Conv2d>(3, 32, 3, 1, 1, true));
         model.add(std::make_unique<nn::ReLU>());
         model.add(std::make_unique<nn::MaxPool2d>(2, 2, 0));
+        model.add(std::make_unique<nn::Conv2d>(32, 32, 3, 1, 1, true));
+        model.add(std::make_unique<nn::BatchNorm2d>(32));
+        model.add(std::make_unique<nn::ReLU>());
         model.add(std::make_unique<nn::Flatten>());
         model.add(std::make_unique<nn::Linear>(32 * 8 * 8, 100, true));
         model.add(std::make_unique<nn::ReLU>());
         model.add(std::make_unique<nn::Linear>(100, 10, true));
         *dynamic_cast<nn::Conv2d &>(model[0]).weight() = kaiming_uniform(gen, Shape{32, 3, 3, 3}, 27);
-        *dynamic_cast<nn::Linear &>(model[4]).weight() = kaiming_uniform(gen, Shape{32 * 8 * 8, 100}, 32 * 8 * 8);
-        *dynamic_cast<nn::Linear &>(model[6]).weight() = kaiming_uniform(gen, Shape{100, 10}, 100);
+        *dynamic_cast<nn::Conv2d &>(model[3]).weight() = kaiming_uniform(gen, Shape{32, 32, 3, 3}, 288);
+        // scale and shift away from 1 and 0, so that the ReLU's mask depends on both
+        *dynamic_cast<nn::BatchNorm2d &>(model[4]).weight() = kaiming_uniform(gen, Shape{32}, 3);
+        *dynamic_cast<nn::BatchNorm2d &>(model[4]).bias() = kaiming_uniform(gen, Shape{32}, 24);
+        *dynamic_cast<nn::Linear &>(model[7]).weight() = kaiming_uniform(gen, Shape{32 * 8 * 8, 100}, 32 * 8 * 8);
+        *dynamic_cast<nn::Linear &>(model[9]).weight() = kaiming_uniform(gen, Shape{100, 10}, 100);
         model.to(kDev);
         model.train();
         auto xv = uniform_vec(gen, (size_t)(N * 3 * 16 * 16), -1.0f, 1.0f);

@@ -257,8 +257,8 @@ def test_a_failed_capture_leaves_the_thread_usable_and_replays_report_bad_labels
 
 
 def test_a_layer_paired_with_its_relu_gives_the_bits_of_the_two_modules_run_in_turn(h):
-    """Sequential runs Linear+ReLU and Conv2d+ReLU as one operator each (activation in the epilogue, backward masked
-    with the output). The network's output and every gradient — parameters and input — must equal, bit for bit, what
+    """Sequential runs Linear+ReLU, Conv2d+ReLU(+MaxPool2d) and BatchNorm2d+ReLU as one operator each (activation in
+    the epilogue, backward masked with the output or, for the normalisation, with the mask formed again). The network's output and every gradient — parameters and input — must equal, bit for bit, what
     the modules give when called one after the other (src/nn/sequential.cpp, src/operators/activation/relu.cpp)."""
     diffs = np.full(2, -1, np.int64)
     assert h.odl_host_paired_layers_match_separate_modules(64, diffs) == 0

@@ -1354,3 +1354,35 @@ def test_max_pool_backward_with_the_relu_mask_folded_in_equals_the_two_steps(api
                got.data_ptr(), None)
         g = host(got)
         assert np.array_equal(g, want) and np.array_equal(np.signbit(g), np.signbit(want)), (N, C, H, W, K, S, P)
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(64, 32, 14, 14), (5, 7, 3, 3), (33, 19), (256, 64, 14, 14)])
+@pytest.mark.parametrize("training", [True, False])
+def test_batch_norm_with_the_relu_folded_in_equals_the_two_steps(api, shape, training):
+    """relu(batch_norm(x)) in one call, and its backward from the gradient of the ReLU's output, give the bits of
+    batch_norm_forward, relu, relu's backward (gy * (y > 0), relu.cpp:45-52) and batch_norm_backward run in turn:
+    the mask is the one expression gamma * x_norm + beta > 0 either way, and the channel sums add the same products
+    in the same order."""
+    rng = np.random.default_rng(hash(shape) % 1000 + training)
+    C = shape[1]
+    x = rng.standard_normal(shape, dtype=f32)
+    gy = rng.standard_normal(shape, dtype=f32)
+    gamma = rng.standard_normal(C, dtype=f32)  # both signs: a negative scale flips which side of the mean survives
+    beta = (rng.standard_normal(C, dtype=f32) * f32(0.5)).astype(f32)
+    rm = rng.standard_normal(C, dtype=f32)
+    rv = (rng.random(C, dtype=f32) + f32(0.1)).astype(f32)
+    y0, mean0, var0, _ = api.batch_norm_forward(dev(x), dev(gamma), dev(beta), dev(rm), dev(rv), training,
+                                                want_x_norm=False)
+    want_y = api.unary("relu", y0)
+    y, mean, var = api.batch_norm_relu_forward(dev(x), dev(gamma), dev(beta), dev(rm), dev(rv), training)
+    assert np.array_equal(host(y), host(want_y))
+    assert np.array_equal(host(mean), host(mean0)) and np.array_equal(host(var), host(var0))
+    assert 0.2 < float((host(y) > 0).mean()) < 0.8  # the mask is neither empty nor full
+    masked = api.binary("relu_backward", dev(gy), y0)
+    want = api.batch_norm_backward_from_x(masked, dev(x), dev(gamma), mean0, var0)
+    got = api.batch_norm_relu_backward_from_x(dev(gy), dev(x), dev(gamma), dev(beta), mean, var)
+    for a, b, name in zip(got, want, ("gx", "dgamma", "dbeta")):
+        assert np.array_equal(host(a), host(b)), name
+    with pytest.raises(api.OdlInvalidArgument):
+        api.batch_norm_relu_backward_from_x(dev(gy), dev(x), dev(gamma), dev(beta[:1].copy()), mean, var)
+
+
