@@ -31,6 +31,11 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kNT     = 512;
 constexpr int kStages = 4;
 constexpr int kEpiBiasCol = 1, kEpiBiasRow = 2;
+template <int V>
+struct IntTag  // a compile-time integer passed to a generic lambda
+{
+    static constexpr int value = V;
+};
 constexpr unsigned kOutside = 0x80000000u;  // beyond the 2^31 - 1 bytes every buffer descriptor here declares
 
 __device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
@@ -476,36 +481,68 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
         return;
     }
     float *Cout = g.C + (int64_t)kz * g.c_split_stride + (int64_t)bz * g.c_batch;
+    // The kind of epilogue is the same for the whole launch: it is decided once, outside the sixteen-element loops, whose
+    // bodies are then an addition, the activation as a constant, and a store (with the tests inside, a 64x32 tile spent
+    // 1.7 us of a 13 us product here). BIAS: 0 none (a column bias that is absent also means no activation), 1 by
+    // column, 2 by row (an absent row bias still applies the activation). With c_p > 0 the product's columns are
+    // (image, position) pairs of an NCHW tensor of M channels: rows are then c_p elements apart, the bias goes by row.
+    auto store_blocks = [&](auto bias_tag, auto act_tag) {
+        constexpr int BIAS = decltype(bias_tag)::value, ACT = decltype(act_tag)::value;
 #pragma unroll
-    for (int i = 0; i < RB; ++i)
+        for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int j = 0; j < CB; ++j)
-        {
-            const int64_t col = n0 + wn + j * 32 + l32;
-            if (col >= g.N)
-                continue;
-            const bool with_bias = g.epi == kEpiBiasCol && g.bias != nullptr;
-            const float bcol = with_bias ? g.bias[col] : 0.f;
-            const int64_t img = g.c_p > 0 ? (int64_t)((unsigned)col / (unsigned)g.c_p) : 0, pos = col - img * g.c_p;
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
+            for (int j = 0; j < CB; ++j)
             {
-                const int64_t row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-                if (row >= g.M)
+                const int64_t col = n0 + wn + j * 32 + l32;
+                if (col >= g.N)
                     continue;
-                float v = acc[i][j][r];
+                const int64_t row0 = m0 + wm + i * 32 + 4 * lh;
+                const int rows_left = (int)(g.M - row0 < 32 ? g.M - row0 : 32);  // rows from row0 on inside the matrix
+                int64_t stride = g.ldc;
+                float *out = Cout + row0 * g.ldc + col;
                 if (g.c_p > 0)
                 {
-                    Cout[(img * g.M + row) * g.c_p + pos] = odl::apply_act(g.bias ? v + g.bias[row] : v, g.act);
-                    continue;
+                    const int64_t img = (int64_t)((unsigned)col / (unsigned)g.c_p), pos = col - img * g.c_p;
+                    stride = g.c_p, out = Cout + (img * g.M + row0) * g.c_p + pos;
                 }
-                if (with_bias)
-                    v = odl::apply_act(v + bcol, g.act);
-                else if (g.epi == kEpiBiasRow)
-                    v = odl::apply_act(g.bias ? v + g.bias[row] : v, g.act);
-                Cout[row * g.ldc + col] = v;
+                const float bcol = BIAS == 1 ? g.bias[col] : 0.f;
+                const bool row_bias = BIAS == 2 && g.bias != nullptr;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                {
+                    const int dr = 8 * (r / 4) + (r % 4);
+                    if (dr >= rows_left)
+                        continue;
+                    float v = acc[i][j][r];
+                    if (BIAS == 1)
+                        v = odl::apply_act(v + bcol, ACT);
+                    else if (BIAS == 2)
+                        v = odl::apply_act(row_bias ? v + g.bias[row0 + dr] : v, ACT);
+                    out[(int64_t)dr * stride] = v;
+                }
             }
-        }
+    };
+    const int bias_kind = g.c_p > 0 ? 2 : (g.epi == kEpiBiasCol && g.bias != nullptr) ? 1 : (g.epi == kEpiBiasRow ? 2 : 0);
+    if (bias_kind == 0)
+        store_blocks(IntTag<0>{}, IntTag<0>{});
+    else if (bias_kind == 1)
+    {
+        if (g.act == 1)
+            store_blocks(IntTag<1>{}, IntTag<1>{});
+        else if (g.act == 2)
+            store_blocks(IntTag<1>{}, IntTag<2>{});
+        else
+            store_blocks(IntTag<1>{}, IntTag<0>{});
+    }
+    else
+    {
+        if (g.act == 1)
+            store_blocks(IntTag<2>{}, IntTag<1>{});
+        else if (g.act == 2)
+            store_blocks(IntTag<2>{}, IntTag<2>{});
+        else
+            store_blocks(IntTag<2>{}, IntTag<0>{});
+    }
 }
 }  // namespace
 
