@@ -36,6 +36,32 @@ struct IntTag  // a compile-time integer passed to a generic lambda
 {
     static constexpr int value = V;
 };
+// calls f(IntTag<bias kind>, IntTag<activation>) for the launch's epilogue: bias kind 0 none (and no activation), 1 by
+// column, 2 by row; the activation 0 none, 1 relu, 2 silu
+template <typename F>
+__device__ inline void with_epilogue_kind(int bias_kind, int act, F &&f)
+{
+    if (bias_kind == 0)
+        f(IntTag<0>{}, IntTag<0>{});
+    else if (bias_kind == 1)
+    {
+        if (act == 1)
+            f(IntTag<1>{}, IntTag<1>{});
+        else if (act == 2)
+            f(IntTag<1>{}, IntTag<2>{});
+        else
+            f(IntTag<1>{}, IntTag<0>{});
+    }
+    else
+    {
+        if (act == 1)
+            f(IntTag<2>{}, IntTag<1>{});
+        else if (act == 2)
+            f(IntTag<2>{}, IntTag<2>{});
+        else
+            f(IntTag<2>{}, IntTag<0>{});
+    }
+}
 constexpr unsigned kOutside = 0x80000000u;  // beyond the 2^31 - 1 bytes every buffer descriptor here declares
 
 __device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
@@ -428,44 +454,55 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
         const int64_t ld = tail_out ? BN : g.ldc, cbase = tail_out ? 4 * l32 : col0;
         const int64_t rbase = tail_out ? 0 : m0;
         const bool whole = (reinterpret_cast<uintptr_t>(Cout) & 15) == 0 && (tail_out || (col0 + 3 < g.N && g.ldc % 4 == 0));
-        const bool with_bias = !tail_out && g.epi == kEpiBiasCol && g.bias != nullptr;
-        float bcol[4] = {0.f, 0.f, 0.f, 0.f};
-        if (with_bias)
+        // (the kind of epilogue decided once per launch, as for the plain layout below)
+        auto store_rows = [&](auto bias_tag, auto act_tag) {
+            constexpr int BIAS = decltype(bias_tag)::value, ACT = decltype(act_tag)::value;
+            float bcol[4] = {0.f, 0.f, 0.f, 0.f};
+            if (BIAS == 1)
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                bcol[e] = col0 + e < g.N ? g.bias[col0 + e] : 0.f;
+                for (int e = 0; e < 4; ++e)
+                    bcol[e] = col0 + e < g.N ? g.bias[col0 + e] : 0.f;
+            const bool row_bias = BIAS == 2 && g.bias != nullptr;
 #pragma unroll
-        for (int i = 0; i < RB; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
+            for (int i = 0; i < RB; ++i)
             {
-                const int64_t row = rbase + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-                if (!tail_out && row >= g.M)
-                    continue;
-                f32x4 v = {acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
-                if (with_bias)
-                {
+                const int64_t row0 = rbase + wm + i * 32 + 4 * lh;
+                const int rows_left = tail_out ? 32 : (int)(g.M - row0 < 32 ? g.M - row0 : 32);
+                float *out = Cout + row0 * ld + cbase;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        v[e] = odl::apply_act(v[e] + bcol[e], g.act);
-                }
-                else if (!tail_out && g.epi == kEpiBiasRow)
+                for (int r = 0; r < 16; ++r)
                 {
-                    const float br = g.bias ? g.bias[row] : 0.f;
+                    const int dr = 8 * (r / 4) + (r % 4);
+                    if (dr >= rows_left)
+                        continue;
+                    f32x4 v = {acc[i][0][r], acc[i][1][r], acc[i][2][r], acc[i][3][r]};
+                    if (BIAS == 1)
+                    {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        v[e] = odl::apply_act(g.bias ? v[e] + br : v[e], g.act);
-                }
-                if (whole)
-                    *reinterpret_cast<f32x4 *>(Cout + row * ld + cbase) = v;
-                else
-                {
+                        for (int e = 0; e < 4; ++e)
+                            v[e] = odl::apply_act(v[e] + bcol[e], ACT);
+                    }
+                    else if (BIAS == 2)
+                    {
+                        const float br = row_bias ? g.bias[row0 + dr] : 0.f;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (tail_out || col0 + e < g.N)
-                            Cout[row * ld + cbase + e] = v[e];
+                        for (int e = 0; e < 4; ++e)
+                            v[e] = odl::apply_act(row_bias ? v[e] + br : v[e], ACT);
+                    }
+                    if (whole)
+                        *reinterpret_cast<f32x4 *>(out + (int64_t)dr * ld) = v;
+                    else
+                    {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (tail_out || col0 + e < g.N)
+                                out[(int64_t)dr * ld + e] = v[e];
+                    }
                 }
             }
+        };
+        const int bias_kind = tail_out ? 0 : (g.epi == kEpiBiasCol && g.bias != nullptr) ? 1 : (g.epi == kEpiBiasRow ? 2 : 0);
+        with_epilogue_kind(bias_kind, g.act, store_rows);
         return;
     }
     if (tail_out)
@@ -523,26 +560,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
             }
     };
     const int bias_kind = g.c_p > 0 ? 2 : (g.epi == kEpiBiasCol && g.bias != nullptr) ? 1 : (g.epi == kEpiBiasRow ? 2 : 0);
-    if (bias_kind == 0)
-        store_blocks(IntTag<0>{}, IntTag<0>{});
-    else if (bias_kind == 1)
-    {
-        if (g.act == 1)
-            store_blocks(IntTag<1>{}, IntTag<1>{});
-        else if (g.act == 2)
-            store_blocks(IntTag<1>{}, IntTag<2>{});
-        else
-            store_blocks(IntTag<1>{}, IntTag<0>{});
-    }
-    else
-    {
-        if (g.act == 1)
-            store_blocks(IntTag<2>{}, IntTag<1>{});
-        else if (g.act == 2)
-            store_blocks(IntTag<2>{}, IntTag<2>{});
-        else
-            store_blocks(IntTag<2>{}, IntTag<0>{});
-    }
+    with_epilogue_kind(bias_kind, g.act, store_blocks);
 }
 }  // namespace
 
