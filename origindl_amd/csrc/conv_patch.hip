@@ -22,6 +22,12 @@ std::atomic<int64_t> g_min_wgs{-1};
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+template <int V>
+struct ActTag  // the activation as a compile-time value for a generic lambda
+{
+    static constexpr int value = V;
+};
+
 constexpr int kThreads = 256;
 constexpr int kPixTile = 128;    // output pixels per workgroup, consecutive in (n, h, w) order
 constexpr int kSlab = 16;        // input channels per staging step
@@ -299,28 +305,53 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
                     out[(wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4)) * kPixTile + wn + j * 32 + l32] = acc[i][j][r];
         return;
     }
+    // The lane's bias values are fetched together before the first store (sixteen loads in flight instead of one before
+    // every store), and the activation is a constant inside the store loop.
+    const bool has_bias = g.bias != nullptr;
+    float bv[RB][16];
 #pragma unroll
-    for (int j = 0; j < CB; ++j)
-    {
-        const int p = p0 + wn + j * 32 + l32;
-        if (p >= g.pixels)
-            continue;
-        const int n = (int)odl::fastdiv((unsigned)p, g.by_hw), hw = p - n * g.HW;
-        float *out = g.dst + (int64_t)n * g.M * g.HW + hw;
+    for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int i = 0; i < RB; ++i)
+        for (int r = 0; r < 16; ++r)
+        {
+            const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+            bv[i][r] = (has_bias && row < g.M) ? g.bias[row] : 0.f;
+        }
+    auto store_all = [&](auto act_tag) {
+        constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
+        for (int j = 0; j < CB; ++j)
+        {
+            const int p = p0 + wn + j * 32 + l32;
+            if (p >= g.pixels)
+                continue;
+            const int n = (int)odl::fastdiv((unsigned)p, g.by_hw), hw = p - n * g.HW;
+#pragma unroll
+            for (int i = 0; i < RB; ++i)
             {
-                const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-                if (row >= g.M)
-                    continue;
-                float v = acc[i][j][r];
-                if (g.bias)
-                    v = v + g.bias[row];
-                out[(int64_t)row * g.HW] = odl::apply_act(v, g.act);
+                const int row0 = m0 + wm + i * 32 + 4 * lh;
+                const int rows_left = g.M - row0;
+                float *out = g.dst + ((int64_t)n * g.M + row0) * g.HW + hw;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                {
+                    const int dr = 8 * (r / 4) + (r % 4);
+                    if (dr >= rows_left)
+                        continue;
+                    float v = acc[i][j][r];
+                    if (has_bias)
+                        v = v + bv[i][r];
+                    out[(int64_t)dr * g.HW] = odl::apply_act(v, ACT);
+                }
             }
-    }
+        }
+    };
+    if (g.act == 1)
+        store_all(ActTag<1>{});
+    else if (g.act == 2)
+        store_all(ActTag<2>{});
+    else
+        store_all(ActTag<0>{});
 }
 
 // Adds the pieces of each tail tile in piece order and stores the tile the way the main kernel does (bias, activation,
