@@ -80,6 +80,7 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
     extern __shared__ float lds[];
     float *As = lds;              // [BM][kLda]
     float *Bs = lds + BM * kLda;  // [plane + 3][kLdp]; the last three positions stay zero
+    float *bias_s = Bs + (g.plane + 3) * kLdp;  // [BM]: the bias of the tile's rows (zeros without one)
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l32 = lane & 31, lh = lane >> 5;
     int tile = blockIdx.x, piece = -1;
@@ -127,6 +128,12 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
     }
     if (t < 3 * kLdp)
         Bs[g.plane * kLdp + t] = 0.f;
+    // The bias of the tile's rows waits in LDS from here on (the first barrier of the slab loop publishes it): fetched
+    // after the last slab it cost every workgroup a trip to memory before its first store — 4.3 us of a 28 us
+    // workgroup by in-kernel timestamps — and held in registers it took the 64-row kernel past 256 registers.
+    const bool has_bias = g.bias != nullptr && piece < 0;
+    if (t < BM)
+        bias_s[t] = (has_bias && m0 + t < g.M) ? g.bias[m0 + t] : 0.f;
 
     // ---- where this lane's output pixels sit in the patch, one base per tap row; a tap row that falls outside the
     // pixel's own image points at the zero positions instead
@@ -305,17 +312,14 @@ __global__ __launch_bounds__(kThreads) void conv_patch_kernel(const PatchGeom g)
                     out[(wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4)) * kPixTile + wn + j * 32 + l32] = acc[i][j][r];
         return;
     }
-    // The lane's bias values are fetched together before the first store (sixteen loads in flight instead of one before
-    // every store), and the activation is a constant inside the store loop.
-    const bool has_bias = g.bias != nullptr;
     float bv[RB][16];
 #pragma unroll
     for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
+        for (int q = 0; q < 4; ++q)
         {
-            const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-            bv[i][r] = (has_bias && row < g.M) ? g.bias[row] : 0.f;
+            const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bias_s + wm + i * 32 + 8 * q + 4 * lh);
+            bv[i][4 * q + 0] = b4[0], bv[i][4 * q + 1] = b4[1], bv[i][4 * q + 2] = b4[2], bv[i][4 * q + 3] = b4[3];
         }
     auto store_all = [&](auto act_tag) {
         constexpr int ACT = decltype(act_tag)::value;
@@ -391,7 +395,7 @@ inline int tile_bm(int64_t M)
 
 inline size_t lds_bytes(int bm, int plane)
 {
-    return ((size_t)bm * kLda + (size_t)(plane + 3) * kLdp) * sizeof(float);
+    return ((size_t)bm * kLda + (size_t)(plane + 3) * kLdp + (size_t)bm) * sizeof(float);  // filters, patch, the tile's bias
 }
 
 // more dynamic LDS than the default limit of 64 KB, asked for once per kernel
