@@ -64,14 +64,28 @@ __device__ inline void with_epilogue_kind(int bias_kind, int act, F &&f)
 }
 constexpr unsigned kOutside = 0x80000000u;  // beyond the 2^31 - 1 bytes every buffer descriptor here declares
 
-__device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
+// What the workgroup -> tile mapping divides by, as multiply-and-shift constants worked out by the launcher: done with
+// the machine's integer division (a reciprocal on the vector unit and a trip back to the scalar one, six times) the
+// mapping was a fifth of the 1 us a workgroup spends before its first load, which a 13 us product notices.
+struct DmaTileMap
 {
-    const int gsz = 8 * tiles_n;  // groups of 8 tile-rows
-    const int grp = t / gsz, in_g = t % gsz;
-    const int first_m = grp * 8;
-    const int gm = (tiles_m - first_m) < 8 ? (tiles_m - first_m) : 8;
-    tm = first_m + in_g % gm;
-    tn = in_g / gm;
+    odl::FastDiv by_xcds, by_nt, by_gsz, by_gm_last;
+    unsigned xcds, xcd_full, xcd_rem;  // XCDs, workgroups every XCD gets, and how many XCDs get one more
+};
+
+// tiles in groups of 8 tile-rows; inside a group down the rows first
+__device__ inline void tile_coords(unsigned t, int tiles_m, int tiles_n, const DmaTileMap &map, int &tm, int &tn)
+{
+    const unsigned gsz = 8u * (unsigned)tiles_n;
+    const unsigned grp = odl::fastdiv(t, map.by_gsz), in_g = t - grp * gsz;
+    const int first_m = (int)grp * 8;
+    if (tiles_m - first_m >= 8)
+        tm = first_m + (int)(in_g & 7u), tn = (int)(in_g >> 3);
+    else
+    {
+        const unsigned gm = (unsigned)(tiles_m - first_m), q = odl::fastdiv(in_g, map.by_gm_last);
+        tm = first_m + (int)(in_g - q * gm), tn = (int)q;
+    }
 }
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -124,7 +138,7 @@ template <int BM, int BN, int BK, bool TA, bool TB, int WGS_PER_CU, int KSETS = 
 // (The second launch bound counts waves per SIMD, of which a workgroup of 512 threads brings two: WGS_PER_CU there only
 // keeps the register budget generous — the kernels use under 128 registers and fit two workgroups per compute unit
 // anyway. Bounds of 2 * WGS_PER_CU changed the compiler's schedule for the worse: 2048^3 dA = dC.B^T 133 -> 142 us.)
-__global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::DmaGemmArgs g)
+__global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::DmaGemmArgs g, const DmaTileMap map)
 {
     constexpr bool A_KMAJOR = !TA, B_KMAJOR = TB;
     constexpr int PIECES = BK / 4;                       // 16-byte pieces in a K-contiguous row of a slab
@@ -157,35 +171,33 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     float *tail_out = nullptr;
     {
         const unsigned nt = (unsigned)(g.tiles_m * g.tiles_n);
-        int t;
+        unsigned t;
         if (g.tail_splits > 0 && (int)blockIdx.x >= g.main_blocks)
         {
             // pieces of the tail tiles keep the hardware's round-robin order: they are short and should spread over all XCDs
             const int u = (int)blockIdx.x - g.main_blocks;
             const int ti = u / g.tail_splits, piece = u - ti * g.tail_splits;
-            t = g.tail_first + ti;
+            t = (unsigned)(g.tail_first + ti);
             kbeg = (int64_t)piece * g.tail_kps;
             kend = (kbeg + g.tail_kps < g.K) ? kbeg + g.tail_kps : g.K;
             tail_out = g.tail_ws + (int64_t)u * (BM * BN);
         }
         else
         {
-            const unsigned total = g.tail_splits > 0 ? (unsigned)g.main_blocks : nt * (unsigned)g.splits * (unsigned)g.batch;
-            const unsigned bid = blockIdx.x, nx = (unsigned)g.xcds;
-            const unsigned loc = bid / nx, xcd = bid - loc * nx;
-            const unsigned full = total / nx, rem = total - full * nx;
-            unsigned v = xcd * full + (xcd < rem ? xcd : rem) + loc;
+            const unsigned bid = blockIdx.x, nx = map.xcds;
+            const unsigned loc = odl::fastdiv(bid, map.by_xcds), xcd = bid - loc * nx;
+            unsigned v = xcd * map.xcd_full + (xcd < map.xcd_rem ? xcd : map.xcd_rem) + loc;
             if (g.batch > 1)
             {
-                bz = (int)(v / nt);  // one K slice per product when there are several
+                bz = (int)odl::fastdiv(v, map.by_nt);  // one K slice per product when there are several
                 v -= (unsigned)bz * nt;
             }
-            kz = (int)(v / nt);
-            t = (int)(v - (unsigned)kz * nt);
+            kz = (int)odl::fastdiv(v, map.by_nt);
+            t = v - (unsigned)kz * nt;
             kbeg = (int64_t)kz * g.k_per_split;
             kend = (kbeg + g.k_per_split < g.K) ? kbeg + g.k_per_split : g.K;
         }
-        tile_coords(t, g.tiles_m, g.tiles_n, tm, tn);
+        tile_coords(t, g.tiles_m, g.tiles_n, map, tm, tn);
     }
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     const int nkt = __builtin_amdgcn_readfirstlane((int)((kend - kbeg + BK - 1) / BK));
@@ -584,19 +596,28 @@ int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream
     const dim3 grid((unsigned)(g.tail_splits > 0 ? g.main_blocks + (nt - g.tail_first) * g.tail_splits
                                                  : nt * g.splits * (g.batch > 1 ? g.batch : 1))),
         block(kNT);
+    DmaTileMap map;
+    {
+        const unsigned total = (unsigned)(g.tail_splits > 0 ? g.main_blocks : nt * g.splits * (g.batch > 1 ? g.batch : 1));
+        const unsigned nx = (unsigned)(g.xcds > 0 ? g.xcds : 1);
+        map.by_xcds = make_fastdiv(nx), map.by_nt = make_fastdiv((unsigned)nt);
+        map.by_gsz = make_fastdiv(8u * (unsigned)g.tiles_n);
+        map.by_gm_last = make_fastdiv((unsigned)(g.tiles_m % 8 ? g.tiles_m % 8 : 8));
+        map.xcds = nx, map.xcd_full = total / nx, map.xcd_rem = total % nx;
+    }
 #define ODL_DMA_CASE(TA, TB)                                                                          \
     if (ta == TA && tb == TB)                                                                         \
     {                                                                                                 \
         if (tile == 64)                                                                               \
-            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 1>), grid, block, 0, st, g);     \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 1>), grid, block, 0, st, g, map);     \
         else if (tile == 65)                                                                          \
-            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 2>), grid, block, 0, st, g);     \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 2>), grid, block, 0, st, g, map);     \
         else if (tile == 32)                                                                          \
-            hipLaunchKernelGGL((sgemm_dma_kernel<64, 32, 64, TA, TB, 1, 4>), grid, block, 0, st, g);  \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 32, 64, TA, TB, 1, 4>), grid, block, 0, st, g, map);  \
         else if (tile == 128)                                                                         \
-            hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 32, TA, TB, 1>), grid, block, 0, st, g);   \
+            hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 32, TA, TB, 1>), grid, block, 0, st, g, map);   \
         else                                                                                          \
-            hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 16, TA, TB, 2>), grid, block, 0, st, g);   \
+            hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 16, TA, TB, 2>), grid, block, 0, st, g, map);   \
         return ODL_OK;                                                                                \
     }
     ODL_DMA_CASE(false, false)
