@@ -90,6 +90,12 @@ struct GemmArgs
 
 using odl::apply_act;
 
+template <int V>
+struct ActTag  // the activation as a compile-time value for a generic lambda
+{
+    static constexpr int value = V;
+};
+
 __device__ __host__ inline void tile_coords(int t, int tiles_m, int tiles_n, int &tm, int &tn)
 {
     const int gsz = 8 * tiles_n;  // groups of 8 tile-rows
@@ -635,44 +641,64 @@ __global__ __launch_bounds__(kThreads * WS, (WS == 1 && BM * BN >= 128 * 128 && 
         return;
     }
     float *Cout = g.C + (int64_t)kz * g.c_split_stride;
+    // The activation is a constant inside the store loops, the addresses are a base per block plus a row stride, and
+    // the bias values of a block's rows are fetched together before its first store.
+    auto store_blocks = [&](auto act_tag) {
+        constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-    for (int i = 0; i < RB; ++i)
+        for (int i = 0; i < RB; ++i)
 #pragma unroll
-        for (int j = 0; j < CB; ++j)
-        {
-            const int64_t col = n0 + wn + j * 32 + l32;
-            if (col >= g.N)
-                continue;
-            float bcol = 0.f;
-            if (EPI == EPI_BIAS_COL && g.bias)
-                bcol = g.bias[col];
-            int64_t nchw_base = 0;
-            if (EPI == EPI_NCHW_ROWB)
+            for (int j = 0; j < CB; ++j)
             {
-                const int64_t n = col / g.P, p = col % g.P;
-                nchw_base = n * g.M * g.P + p;  // + oc * P
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-            {
-                const int64_t row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-                if (row >= g.M)
+                const int64_t col = n0 + wn + j * 32 + l32;
+                if (col >= g.N)
                     continue;
-                float v = acc[i][j][r];
+                const int64_t row0 = m0 + wm + i * 32 + 4 * lh;
+                const int rows_left = (int)(g.M - row0 < 32 ? g.M - row0 : 32);
+                float bcol = 0.f;
+                if (EPI == EPI_BIAS_COL && g.bias)
+                    bcol = g.bias[col];
+                float *out = Cout + row0 * g.ldc + col;
+                int64_t stride = g.ldc;
+                float brow[16];
                 if (EPI == EPI_NCHW_ROWB)
                 {
-                    if (g.bias)
-                        v = v + g.bias[row];
-                    Cout[nchw_base + row * g.P] = apply_act(v, g.act);
+                    const int64_t n = col / g.P, p = col % g.P;
+                    out = Cout + (n * g.M + row0) * g.P + p, stride = g.P;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                    {
+                        const int dr = 8 * (r / 4) + (r % 4);
+                        brow[r] = (g.bias && dr < rows_left) ? g.bias[row0 + dr] : 0.f;
+                    }
                 }
-                else
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
                 {
-                    if (EPI == EPI_BIAS_COL)
-                        v = apply_act(v + bcol, g.act);
-                    Cout[row * g.ldc + col] = v;
+                    const int dr = 8 * (r / 4) + (r % 4);
+                    if (dr >= rows_left)
+                        continue;
+                    float v = acc[i][j][r];
+                    if (EPI == EPI_NCHW_ROWB)
+                    {
+                        if (g.bias)
+                            v = v + brow[r];
+                        v = apply_act(v, ACT);
+                    }
+                    else if (EPI == EPI_BIAS_COL)
+                        v = apply_act(v + bcol, ACT);
+                    out[(int64_t)dr * stride] = v;
                 }
             }
-        }
+    };
+    if (EPI == 0 || g.act == 0)
+        store_blocks(ActTag<0>{});
+    else if (g.act == 1)
+        store_blocks(ActTag<1>{});
+    else if (g.act == 2)
+        store_blocks(ActTag<2>{});
+    else
+        store_blocks(ActTag<0>{});
 }
 
 // out[i] = sum over slices of part[s*stride + i] (+ bias by column). 64 outputs x 16 slice groups per workgroup:
