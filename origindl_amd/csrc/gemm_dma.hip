@@ -348,7 +348,9 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     // right after the barrier (4-byte reads: NN 1005 -> 1047 us, TN 992 -> 1026 us) or no faster (B in 16-byte quads: the
     // second fragment set takes the kernel past 128 registers and with that to one workgroup per compute unit; held to
     // 128 registers it runs 969 against 972 us): those keep the plain order.
-    constexpr bool PIPE = A_KMAJOR && B_KMAJOR;
+    // (On the 64-row tiles, whose waves hold one block each, the order also pays with a row-contiguous B — 1024^3 22.0
+    // -> 21.3 us, 6272x256x1152 41.2 -> 40.2 us against the plain order on one box — but not with a row-contiguous A.)
+    constexpr bool PIPE = A_KMAJOR && (B_KMAJOR || BM <= 64);
     if constexpr (PIPE)
     {
         if (nkt > 0)
