@@ -416,6 +416,16 @@ int odl_hip_adam_step_multi(int count, const float *const *p, const float *const
 int odl_hip_sgd_step_multi(int count, const float *const *p, const float *const *g, const int64_t *n, float lr,
                            float *const *p_out, void *stream);
 int odl_hip_axpy_multi(int count, float alpha, const float *const *x, float *const *y, const int64_t *n, void *stream);
+/* The WeightDecay hook and the step it precedes (Optimizer::step runs the hooks, then the steps) in one pass over the
+ * parameters: g[i] += weight_decay * p[i] (product rounded, then the sum, as axpy_multi) is written back to g[i] — the
+ * caller's gradients hold the decayed values afterwards, as after the hook — and the step uses that g. The floats of
+ * axpy_multi followed by adam_step_multi / sgd_step_multi. */
+int odl_hip_adam_step_multi_decay(int count, const float *const *p, float *const *g, float *const *m, float *const *v,
+                                  const int64_t *n, float weight_decay, float beta1, float beta2, const float *m_hat_scale,
+                                  const float *v_hat_scale, const float *const *device_scales, float eps, float lr,
+                                  float *const *p_out, void *stream);
+int odl_hip_sgd_step_multi_decay(int count, const float *const *p, float *const *g, const int64_t *n, float weight_decay,
+                                 float lr, float *const *p_out, void *stream);
 /* origin::cuda::{zeros,ones,full} (cuda/factory.cuh:23-50) */
 int odl_hip_fill(float *dst, int64_t n, float value, void *stream);
 

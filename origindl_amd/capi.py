@@ -653,10 +653,11 @@ def _size_array(tensors):
     return (ctypes.c_int64 * len(tensors))(*[t.numel() for t in tensors])
 
 
-def adam_step_multi(ps, gs, ms, vs, ts, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, device_scales=None):
+def adam_step_multi(ps, gs, ms, vs, ts, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, device_scales=None, weight_decay=0.0):
     """One launch over a list of parameters (Optimizer::step, src/optim/optimizer.cpp:19-53, walks them one by one):
     entry i gets what adam_step gives at step count ts[i]. Returns the new parameters; ms and vs are updated in place.
-    device_scales: optional list whose non-None entries are device tensors of two floats used instead of ts[i]."""
+    device_scales: optional list whose non-None entries are device tensors of two floats used instead of ts[i].
+    weight_decay != 0: gs[i] += weight_decay * ps[i] first, in place and in the same launch (the WeightDecay hook)."""
     for group in (ps, gs, ms, vs):
         for x in group:
             _chk(x, "adam_step_multi operand")
@@ -665,6 +666,12 @@ def adam_step_multi(ps, gs, ms, vs, ts, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-
     s2 = [f(1.0) / (f(1.0) - f(np.power(f(beta2), f(t)))) for t in ts]
     outs = [_empty(p.shape) for p in ps]
     n = len(ps)
+    if weight_decay != 0.0:
+        lib().call("odl_hip_adam_step_multi_decay", n, _ptr_array(ps), _ptr_array(gs), _ptr_array(ms), _ptr_array(vs),
+                   _size_array(ps), float(f(weight_decay)), float(f(beta1)), float(f(beta2)), (ctypes.c_float * n)(*s1),
+                   (ctypes.c_float * n)(*s2), _ptr_array(device_scales) if device_scales is not None else None,
+                   float(f(eps)), float(f(lr)), _ptr_array(outs), _stream())
+        return outs
     lib().call("odl_hip_adam_step_multi", n, _ptr_array(ps), _ptr_array(gs), _ptr_array(ms), _ptr_array(vs),
                _size_array(ps), float(f(beta1)), float(f(beta2)), (ctypes.c_float * n)(*s1), (ctypes.c_float * n)(*s2),
                _ptr_array(device_scales) if device_scales is not None else None, float(f(eps)), float(f(lr)),
@@ -672,12 +679,16 @@ def adam_step_multi(ps, gs, ms, vs, ts, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-
     return outs
 
 
-def sgd_step_multi(ps, gs, lr):
-    """p - g*lr for every pair of the lists in one launch."""
+def sgd_step_multi(ps, gs, lr, weight_decay=0.0):
+    """p - g*lr for every pair of the lists in one launch (weight_decay != 0: g += weight_decay * p first, in place)."""
     for group in (ps, gs):
         for x in group:
             _chk(x, "sgd_step_multi operand")
     outs = [_empty(p.shape) for p in ps]
+    if weight_decay != 0.0:
+        lib().call("odl_hip_sgd_step_multi_decay", len(ps), _ptr_array(ps), _ptr_array(gs), _size_array(ps),
+                   float(np.float32(weight_decay)), float(np.float32(lr)), _ptr_array(outs), _stream())
+        return outs
     lib().call("odl_hip_sgd_step_multi", len(ps), _ptr_array(ps), _ptr_array(gs), _size_array(ps), float(np.float32(lr)),
                _ptr_array(outs), _stream())
     return outs

@@ -221,10 +221,14 @@ struct MultiArgs
     int count;
 };
 
-// OP 0: Adam step, 1: SGD step, 2: out += alpha * a — per element the same float operations as the one-tensor kernels
-template <int OP>
+// OP 0: Adam step, 1: SGD step, 2: out += alpha * a — per element the same float operations as the one-tensor kernels.
+// OP 3 / 4: the Adam / SGD step with the WeightDecay hook in front of it in the same pass: g += alpha * p (the product
+// rounded, then the sum: what OP 2 does) is written back to g, and the step uses that g.
+template <int OPX>
 __global__ __launch_bounds__(kBlock) void multi_tensor_kernel(MultiArgs q, AdamScalars s, float alpha)
 {
+    constexpr bool DECAY = OPX >= 3;
+    constexpr int OP = OPX == 3 ? 0 : (OPX == 4 ? 1 : OPX);
     int t = 0;
     while (t + 1 < q.count && blockIdx.x >= q.first_block[t + 1])  // the same in every lane
         ++t;
@@ -248,7 +252,17 @@ __global__ __launch_bounds__(kBlock) void multi_tensor_kernel(MultiArgs q, AdamS
         f32x4 ov;
         if (OP == 0)
         {
-            const f32x4 gv = *reinterpret_cast<const f32x4 *>(b + i);
+            f32x4 gv = *reinterpret_cast<const f32x4 *>(b + i);
+            if (DECAY)
+            {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    const float step = alpha * av[j];
+                    gv[j] = gv[j] + step;
+                }
+                *reinterpret_cast<f32x4 *>(const_cast<float *>(b) + i) = gv;
+            }
             f32x4 mv = *reinterpret_cast<f32x4 *>(m + i), vv = *reinterpret_cast<f32x4 *>(v + i);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
@@ -262,7 +276,17 @@ __global__ __launch_bounds__(kBlock) void multi_tensor_kernel(MultiArgs q, AdamS
         }
         else if (OP == 1)
         {
-            const f32x4 gv = *reinterpret_cast<const f32x4 *>(b + i);
+            f32x4 gv = *reinterpret_cast<const f32x4 *>(b + i);
+            if (DECAY)
+            {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    const float step = alpha * av[j];
+                    gv[j] = gv[j] + step;
+                }
+                *reinterpret_cast<f32x4 *>(const_cast<float *>(b) + i) = gv;
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j)
             {
@@ -285,11 +309,18 @@ __global__ __launch_bounds__(kBlock) void multi_tensor_kernel(MultiArgs q, AdamS
     }
     for (int64_t k = i; k < n && k < i + 4; ++k)
     {
+        float gk = OP == 2 ? 0.f : b[k];
+        if (DECAY)
+        {
+            const float step = alpha * a[k];
+            gk = gk + step;
+            const_cast<float *>(b)[k] = gk;
+        }
         if (OP == 0)
-            adam_one(a[k], b[k], m[k], v[k], out[k], s);
+            adam_one(a[k], gk, m[k], v[k], out[k], s);
         else if (OP == 1)
         {
-            const float step = b[k] * s.lr;
+            const float step = gk * s.lr;
             out[k] = a[k] - step;
         }
         else
@@ -367,11 +398,12 @@ int fill_bytes_launch(void *dst, int value, size_t bytes, hipStream_t st)
     return ODL_OK;
 }
 // the list goes out kMultiMax tensors at a time; empty tensors are skipped
-template <int OP>
+template <int OPX>
 int multi_launch(const char *what, int count, const float *const *a, const float *const *b, float *const *m,
                         float *const *v, float *const *out, const float *const *scales, const float *m_hat,
                         const float *v_hat, const int64_t *n, const AdamScalars &s, float alpha, void *stream)
 {
+    constexpr int OP = OPX == 3 ? 0 : (OPX == 4 ? 1 : OPX);
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(count >= 0, "%s: negative count", what);
     if (count == 0)
@@ -386,7 +418,7 @@ int multi_launch(const char *what, int count, const float *const *a, const float
             return ODL_OK;
         q.count = used;
         q.first_block[used] = (unsigned)blocks;
-        hipLaunchKernelGGL((multi_tensor_kernel<OP>), dim3((unsigned)blocks), dim3(kBlock), 0, odl::as_stream(stream), q, s,
+        hipLaunchKernelGGL((multi_tensor_kernel<OPX>), dim3((unsigned)blocks), dim3(kBlock), 0, odl::as_stream(stream), q, s,
                            alpha);
         ODL_LAUNCH_CHECK();
         used = 0, blocks = 0;
@@ -547,6 +579,24 @@ int odl_hip_sgd_step_multi(int count, const float *const *p, const float *const 
     const AdamScalars s{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, lr, 0.5f};
     return odl::multi_launch<1>("sgd_step_multi", count, p, g, nullptr, nullptr, p_out, nullptr, nullptr, nullptr, n, s, 0.0f,
                            stream);
+}
+
+int odl_hip_adam_step_multi_decay(int count, const float *const *p, float *const *g, float *const *m, float *const *v,
+                                  const int64_t *n, float weight_decay, float beta1, float beta2, const float *m_hat_scale,
+                                  const float *v_hat_scale, const float *const *device_scales, float eps, float lr,
+                                  float *const *p_out, void *stream)
+{
+    const AdamScalars s{beta1, 1.0f - beta1, beta2, 1.0f - beta2, 0.0f, 0.0f, eps, lr, 0.5f};
+    return odl::multi_launch<3>("adam_step_multi_decay", count, p, g, m, v, p_out, device_scales, m_hat_scale, v_hat_scale, n,
+                                s, weight_decay, stream);
+}
+
+int odl_hip_sgd_step_multi_decay(int count, const float *const *p, float *const *g, const int64_t *n, float weight_decay,
+                                 float lr, float *const *p_out, void *stream)
+{
+    const AdamScalars s{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, lr, 0.5f};
+    return odl::multi_launch<4>("sgd_step_multi_decay", count, p, g, nullptr, nullptr, p_out, nullptr, nullptr, nullptr, n, s,
+                                weight_decay, stream);
 }
 
 int odl_hip_axpy_multi(int count, float alpha, const float *const *x, float *const *y, const int64_t *n, void *stream)

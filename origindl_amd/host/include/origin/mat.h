@@ -428,10 +428,12 @@ public:
         float m_hat_scale, v_hat_scale;
         const float *device_scales;  // the two factors in device memory instead (recorded steps), or null
     };
+    // weight_decay != 0: the WeightDecay hook in the same pass — every gradient becomes g + weight_decay * p first (and
+    // keeps that value), then the step runs on it
     static std::vector<std::unique_ptr<Mat>> adam_step_multi(const std::vector<AdamItem> &items, float beta1, float beta2,
-                                                             float eps, float lr, bool in_place);
+                                                             float eps, float lr, bool in_place, float weight_decay = 0.0f);
     static std::vector<std::unique_ptr<Mat>> sgd_step_multi(const std::vector<std::pair<const Mat *, const Mat *>> &param_grad,
-                                                            float lr, bool in_place);
+                                                            float lr, bool in_place, float weight_decay = 0.0f);
     // y += a*x for every (x, y) of the list
     static void axpy_multi(float a, const std::vector<std::pair<const Mat *, Mat *>> &x_y);
     static bool device_f32(const Mat &m);

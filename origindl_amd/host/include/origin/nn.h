@@ -223,6 +223,10 @@ protected:
         for (auto *p : params)
             step_one(*p);
     }
+    // true when step_all will update this list in one launch that can apply a WeightDecay hook on its way: step() then
+    // hands the hook's rate over in hook_decay_ instead of running the hook as a launch of its own (same floats)
+    virtual bool step_all_takes_decay(const std::vector<Parameter *> &) const { return false; }
+    float hook_decay_ = 0.0f;
     Module *target_;
     std::vector<Parameter *> parameters_;
     std::vector<std::function<void(std::vector<Parameter *> &)>> hooks_;
@@ -238,6 +242,7 @@ public:
 protected:
     void step_one(Parameter &param) override;
     void step_all(std::vector<Parameter *> &params) override;
+    bool step_all_takes_decay(const std::vector<Parameter *> &params) const override;
 
 private:
     float lr_, momentum_, weight_decay_;
@@ -255,6 +260,7 @@ public:
 protected:
     void step_one(Parameter &param) override;
     void step_all(std::vector<Parameter *> &params) override;
+    bool step_all_takes_decay(const std::vector<Parameter *> &params) const override;
 
 private:
     float lr_, beta1_, beta2_, eps_;
@@ -265,6 +271,13 @@ private:
 
 public:
     void prepare_replay() override;
+};
+
+// what WeightDecay::hook() wraps: a named type, so that Optimizer::step can recognise the hook and its rate
+struct WeightDecayHook
+{
+    float rate;
+    void operator()(std::vector<Parameter *> &params) const;
 };
 
 class WeightDecay  // include/origin/optim/hooks.h:37-66: grad += rate * param, for every parameter

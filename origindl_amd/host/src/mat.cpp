@@ -1831,7 +1831,7 @@ bool OriginMat::device_f32(const Mat &m)
 }
 
 std::vector<std::unique_ptr<Mat>> OriginMat::adam_step_multi(const std::vector<AdamItem> &items, float beta1, float beta2,
-                                                             float eps, float lr, bool in_place)
+                                                             float eps, float lr, bool in_place, float weight_decay)
 {
     const size_t count = items.size();
     std::vector<const float *> p(count), g(count), scales(count);
@@ -1857,13 +1857,18 @@ std::vector<std::unique_ptr<Mat>> OriginMat::adam_step_multi(const std::vector<A
             results.push_back(std::move(o));
         }
     }
-    check(odl_hip_adam_step_multi((int)count, p.data(), g.data(), m.data(), v.data(), n.data(), beta1, beta2, s1.data(),
-                                  s2.data(), scales.data(), eps, lr, out.data(), cur()));
+    if (weight_decay != 0.0f)
+        check(odl_hip_adam_step_multi_decay((int)count, p.data(), const_cast<float *const *>(g.data()), m.data(), v.data(),
+                                            n.data(), weight_decay, beta1, beta2, s1.data(), s2.data(), scales.data(), eps,
+                                            lr, out.data(), cur()));
+    else
+        check(odl_hip_adam_step_multi((int)count, p.data(), g.data(), m.data(), v.data(), n.data(), beta1, beta2, s1.data(),
+                                      s2.data(), scales.data(), eps, lr, out.data(), cur()));
     return results;
 }
 
 std::vector<std::unique_ptr<Mat>> OriginMat::sgd_step_multi(const std::vector<std::pair<const Mat *, const Mat *>> &param_grad,
-                                                            float lr, bool in_place)
+                                                            float lr, bool in_place, float weight_decay)
 {
     const size_t count = param_grad.size();
     std::vector<const float *> p(count), g(count);
@@ -1885,7 +1890,11 @@ std::vector<std::unique_ptr<Mat>> OriginMat::sgd_step_multi(const std::vector<st
             results.push_back(std::move(o));
         }
     }
-    check(odl_hip_sgd_step_multi((int)count, p.data(), g.data(), n.data(), lr, out.data(), cur()));
+    if (weight_decay != 0.0f)
+        check(odl_hip_sgd_step_multi_decay((int)count, p.data(), const_cast<float *const *>(g.data()), n.data(), weight_decay,
+                                           lr, out.data(), cur()));
+    else
+        check(odl_hip_sgd_step_multi((int)count, p.data(), g.data(), n.data(), lr, out.data(), cur()));
     return results;
 }
 

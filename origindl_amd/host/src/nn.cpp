@@ -401,6 +401,23 @@ void Optimizer::step()
     for (auto *p : parameters_)
         if (p->defined() && p->grad().defined())
             with_grad.push_back(p);
+    // a lone WeightDecay hook in front of a one-launch step rides along in that launch
+    const WeightDecayHook *decay = hooks_.size() == 1 ? hooks_[0].target<WeightDecayHook>() : nullptr;
+    if (decay && decay->rate != 0.0f && step_all_takes_decay(with_grad))
+    {
+        hook_decay_ = decay->rate;
+        try
+        {
+            step_all(with_grad);
+        }
+        catch (...)
+        {
+            hook_decay_ = 0.0f;
+            throw;
+        }
+        hook_decay_ = 0.0f;
+        return;
+    }
     for (auto &h : hooks_)
         h(with_grad);
     step_all(with_grad);
@@ -472,6 +489,30 @@ void SGD::step_one(Parameter &param)
         param = as_leaf(param - grad * Scalar(lr_));
 }
 
+namespace
+{
+// every parameter and its gradient float32 on the device, of one shape: what the one-launch steps and the hook's own
+// one-launch form both ask for
+bool all_on_device(const std::vector<Parameter *> &params)
+{
+    for (auto *p : params)
+        if (!OriginMat::device_f32(*p->impl_->data_) || !OriginMat::device_f32(*p->grad().impl_->data_) ||
+            p->grad().shape() != p->shape())
+            return false;
+    return true;
+}
+}  // namespace
+
+bool SGD::step_all_takes_decay(const std::vector<Parameter *> &params) const
+{
+    return weight_decay_ <= 0.0f && momentum_ <= 0.0f && params.size() > 1 && all_on_device(params);
+}
+
+bool Adam::step_all_takes_decay(const std::vector<Parameter *> &params) const
+{
+    return params.size() > 1 && all_on_device(params);
+}
+
 // The plain step (no momentum, no weight decay) over device parameters: one launch for the whole list.
 void SGD::step_all(std::vector<Parameter *> &params)
 {
@@ -492,7 +533,7 @@ void SGD::step_all(std::vector<Parameter *> &params)
         list.emplace_back(p->impl_->data_.get(), grads.back().impl_->data_.get());
     }
     const bool in_place = cuda::is_capturing();
-    auto updated = OriginMat::sgd_step_multi(list, lr_, in_place);
+    auto updated = OriginMat::sgd_step_multi(list, lr_, in_place, hook_decay_);
     if (!in_place)
         for (size_t i = 0; i < params.size(); ++i)
             *params[i] = as_leaf(Tensor(std::move(updated[i])));
@@ -589,7 +630,7 @@ void Adam::step_all(std::vector<Parameter *> &params)
         }
         items.push_back(it);
     }
-    auto updated = OriginMat::adam_step_multi(items, beta1_, beta2_, eps_, lr_, capturing);
+    auto updated = OriginMat::adam_step_multi(items, beta1_, beta2_, eps_, lr_, capturing, hook_decay_);
     if (!capturing)
         for (size_t i = 0; i < params.size(); ++i)
             *params[i] = as_leaf(Tensor(std::move(updated[i])));
@@ -614,8 +655,12 @@ void Adam::prepare_replay()
 
 std::function<void(std::vector<Parameter *> &)> WeightDecay::hook() const
 {
-    const float rate = rate_;
-    return [rate](std::vector<Parameter *> &params) {
+    return WeightDecayHook{rate_};
+}
+
+void WeightDecayHook::operator()(std::vector<Parameter *> &params) const
+{
+    {
         NoGradGuard guard;
         // grad += rate * param: one launch for all parameters that live on the device (the product is rounded, then
         // added — what the separate multiply and accumulate give)
@@ -637,7 +682,7 @@ std::function<void(std::vector<Parameter *> &)> WeightDecay::hook() const
         }
         if (!on_device.empty())
             OriginMat::axpy_multi(rate, on_device);
-    };
+    }
 }
 
 // ----------------------------------------------------------------------------------------- device API

@@ -819,6 +819,30 @@ def test_multi_tensor_optimizer_steps_are_the_single_tensor_steps(api):
     for i in live:
         assert np.array_equal(host(dg[i]), g[i] + f32(1e-4) * p[i]), sizes[i]
         assert np.array_equal(host(dg[i]), host(api.axpby(1.0, dev(g[i]), 1e-4, dev(p[i])))), sizes[i]
+    # the hook and the step in one launch: the bits of the hook's launch followed by the step's, gradients included
+    for unaligned in (False, True):
+        def fresh(arrs):
+            if not unaligned:
+                return [dev(x) for x in arrs]
+            views = [torch.empty(x.size + 1, dtype=torch.float32, device="cuda")[1:] for x in arrs]
+            for t, x in zip(views, arrs):
+                t.copy_(torch.from_numpy(x))
+            return views
+        dp, dg2, dm2, dv2 = fresh(p), fresh(g), fresh(m), fresh(v)
+        api.axpy_multi(1e-4, dp, dg2)
+        want = api.adam_step_multi(dp, dg2, dm2, dv2, ts, lr=2e-3)
+        fp_, fg, fm, fv = fresh(p), fresh(g), fresh(m), fresh(v)
+        got = api.adam_step_multi(fp_, fg, fm, fv, ts, lr=2e-3, weight_decay=1e-4)
+        for i in live:
+            assert np.array_equal(host(got[i]), host(want[i])), (sizes[i], unaligned)
+            assert np.array_equal(host(fg[i]), host(dg2[i])) and np.array_equal(host(fm[i]), host(dm2[i])), sizes[i]
+            assert np.array_equal(host(fv[i]), host(dv2[i])) and np.array_equal(host(fp_[i]), p[i]), sizes[i]
+        dg2, fg = fresh(g), fresh(g)
+        api.axpy_multi(1e-4, dp, dg2)
+        want = api.sgd_step_multi(dp, dg2, 0.05)
+        got = api.sgd_step_multi(fp_, fg, 0.05, weight_decay=1e-4)
+        for i in live:
+            assert np.array_equal(host(got[i]), host(want[i])) and np.array_equal(host(fg[i]), host(dg2[i])), sizes[i]
     with pytest.raises(api.OdlInvalidArgument):
         api.axpy_multi(0.5, [dev(p[3])], [dev(p[4])])
     # argument errors of the entry points themselves: a negative count, missing lists, a null tensor, a negative size
