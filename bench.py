@@ -312,20 +312,22 @@ def train_steps(steps, warmup, with_cpu):
     if not os.path.exists(ol.HOST_DRIVER_SO):
         return {"error": "host layer not built"}
     h = ol.host_driver()
-    ms, loss = np.zeros(1, np.float32), np.zeros(1, np.float32)
+    # loss = [loss of the first step from the initial parameters, loss of the last step]: the first is the number to
+    # compare between the ordinary run, the replayed run and the CPU reference (they take different numbers of steps)
+    ms, loss = np.zeros(1, np.float32), np.zeros(2, np.float32)
     rc = h.odl_host_mlp_bench(512, 784, 1000, 10, steps, warmup, ms, loss)
-    out["mlp_512x784x1000x10_adam"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss": float(loss[0]),
+    out["mlp_512x784x1000x10_adam"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss_step_1": float(loss[0]),
                                        "gemm_flop_per_step": 6.0 * 512 * (784 * 1000 + 1000 * 10)}
     rc = h.odl_host_cnn_bench(256, steps, warmup, ms, loss)
-    out["cnn_b256_sgd"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss": float(loss[0])}
+    out["cnn_b256_sgd"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss_step_1": float(loss[0])}
     # the same steps recorded once into a HIP graph and replayed (one submission per step instead of ~50 launches);
     # the loss is still read back after every step
     rc = h.odl_host_mlp_bench_graph(512, 784, 1000, 10, steps, warmup, 1, ms, loss)
     out["mlp_512x784x1000x10_adam"].update({"graph_replay_rc": rc, "graph_replay_ms_per_step": float(ms[0]),
-                                            "graph_replay_loss": float(loss[0])})
+                                            "graph_replay_loss_step_1": float(loss[0])})
     rc = h.odl_host_cnn_bench_graph(256, steps, warmup, 1, ms, loss)
     out["cnn_b256_sgd"].update({"graph_replay_rc": rc, "graph_replay_ms_per_step": float(ms[0]),
-                                "graph_replay_loss": float(loss[0])})
+                                "graph_replay_loss_step_1": float(loss[0])})
     # the network of the reference's own conv_mnist example (with its BatchNorm layers, Adam + WeightDecay), batch 256;
     # device only: the reference's BatchNorm operator cannot run backward
     losses = np.zeros(3, np.float32)
@@ -339,9 +341,10 @@ def train_steps(steps, warmup, with_cpu):
         r = ol.ref()
         rc = r.odl_ref_mlp_bench(512, 784, 1000, 10, 1, 0, ms, loss)
         out["mlp_512x784x1000x10_adam"]["cpu_reference_ms_per_step"] = float(ms[0])
-        out["mlp_512x784x1000x10_adam"]["cpu_reference_loss"] = float(loss[0])
+        out["mlp_512x784x1000x10_adam"]["cpu_reference_loss_step_1"] = float(loss[0])
         rc = r.odl_ref_cnn_bench(4, 1, 0, ms, loss)
         out["cnn_b256_sgd"]["cpu_reference_ms_per_step_extrapolated_from_batch_4"] = float(ms[0]) * 64.0
+        out["cnn_b256_sgd"]["cpu_reference_loss_step_1_at_batch_4"] = float(loss[0])
     return out
 
 

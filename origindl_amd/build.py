@@ -57,34 +57,24 @@ def build(verbose=False):
 
 HOST_DIR = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIB_DIR, "liborigin_host.so")
-HOST_DRIVER_LIB = os.path.join(LIB_DIR, "libodl_host_driver.so")
-HOST_CPU_DRIVER_LIB = os.path.join(LIB_DIR, "libodl_hostcpu_driver.so")  # same driver, tensors left on the CPU
 CXX = os.environ.get("CXX", "g++")
 
 
 def build_host(verbose=False):
-    """C++ host layer (Mat / Tensor / operators / nn / optim over the C ABI) -> lib/liborigin_host.so, and the API
-    driver of tests/api_driver.cpp compiled against it -> lib/libodl_host_driver.so. Plain g++: no device code."""
+    """C++ host layer (Mat / Tensor / operators / nn / optim over the C ABI) -> lib/liborigin_host.so.
+    Plain g++: no device code."""
     os.makedirs(LIB_DIR, exist_ok=True)
     inc = ["-I" + os.path.join(HOST_DIR, "include"), "-I" + os.path.join(os.path.dirname(HERE), "include")]
     common = [CXX, "-std=c++17", "-O2", "-fPIC", "-Wall", "-Wno-unused-variable"] + inc
     srcs = sorted(glob.glob(os.path.join(HOST_DIR, "src", "*.cpp")))
     link = ["-L" + LIB_DIR, "-lodl_hip", "-Wl,-rpath,$ORIGIN"]
-    for cmd in (
-        common + ["-shared", "-o", HOST_LIB] + srcs + link,
-        common + ["-shared", "-DDRV_ON_DEVICE", "-DDRV_PREFIX=odl_host_", "-o", HOST_DRIVER_LIB,
-                  os.path.join(os.path.dirname(HERE), "tests", "api_driver.cpp"), "-L" + LIB_DIR, "-lorigin_host",
-                  "-lodl_hip", "-Wl,-rpath,$ORIGIN"],
-        common + ["-shared", "-DDRV_PREFIX=odl_hostcpu_", "-o", HOST_CPU_DRIVER_LIB,
-                  os.path.join(os.path.dirname(HERE), "tests", "api_driver.cpp"), "-L" + LIB_DIR, "-lorigin_host",
-                  "-lodl_hip", "-Wl,-rpath,$ORIGIN"],
-    ):
-        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-        if verbose and res.stdout.strip():
-            print(res.stdout)
-        if res.returncode != 0:
-            raise RuntimeError("host build failed:\n" + " ".join(cmd) + "\n" + res.stdout)
-    return HOST_LIB, HOST_DRIVER_LIB
+    cmd = common + ["-shared", "-o", HOST_LIB] + srcs + link
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose and res.stdout.strip():
+        print(res.stdout)
+    if res.returncode != 0:
+        raise RuntimeError("host build failed:\n" + " ".join(cmd) + "\n" + res.stdout)
+    return HOST_LIB
 
 
 if __name__ == "__main__":

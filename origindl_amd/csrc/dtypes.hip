@@ -204,14 +204,15 @@ __device__ inline typename Acc<T>::type widen(T v)
         return (uint64_t)(int64_t)v;
 }
 
-// rows: src[outer][axis] (inner == 1). One workgroup per (row, slice); partial[slice * outer + row].
+// rows: src[outer][axis] (inner == 1). One workgroup per (row, slice), both folded into the grid's first
+// dimension (its 2^31 limit, not the 65535 of the second, bounds the row count); partial[slice * outer + row].
 template <typename T>
 __global__ __launch_bounds__(kBlock) void row_partial_kernel(const T *__restrict__ src, typename Acc<T>::type *__restrict__ part,
-                                                             int64_t outer, int64_t axis, int64_t chunk)
+                                                             int64_t outer, int64_t axis, int64_t chunk, int slices)
 {
     using A = typename Acc<T>::type;
     __shared__ A red[kBlock];
-    const int64_t row = blockIdx.y, slice = blockIdx.x;
+    const int64_t row = blockIdx.x / (unsigned)slices, slice = blockIdx.x % (unsigned)slices;
     const int64_t k0 = slice * chunk, k1 = (k0 + chunk < axis) ? k0 + chunk : axis;
     A s = 0;
     for (int64_t k = k0 + threadIdx.x; k < k1; k += kBlock)
@@ -759,14 +760,14 @@ int odl_hip_sum_axis_dtype(int dtype, const void *src, int64_t outer, int64_t ax
     const SumPlan p = plan_sum(outer, axis, inner);
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= p.ws_bytes && reinterpret_cast<uintptr_t>(workspace) % 8 == 0,
                 "sum: an 8-byte aligned workspace of %zu bytes required, got %zu", p.ws_bytes, workspace_bytes);
-    ODL_REQUIRE(outer < 65536 || inner > 1, "sum: too many rows for the row schedule");
+    ODL_REQUIRE(inner > 1 || outer * p.slices < (1ll << 31), "sum: too many rows for one launch");
     return with_type(dtype, [&](auto t) {
         using T = decltype(t);
         using A = typename Acc<T>::type;
         A *part = static_cast<A *>(workspace);
         if (inner == 1)
-            hipLaunchKernelGGL((row_partial_kernel<T>), dim3((unsigned)p.slices, (unsigned)outer), dim3(kBlock), 0, st,
-                               static_cast<const T *>(src), part, outer, axis, p.chunk);
+            hipLaunchKernelGGL((row_partial_kernel<T>), dim3((unsigned)(p.slices * outer)), dim3(kBlock), 0, st,
+                               static_cast<const T *>(src), part, outer, axis, p.chunk, (int)p.slices);
         else
             hipLaunchKernelGGL((col_partial_kernel<T>), dim3((unsigned)odl::ceil_div(nout, kBlock), (unsigned)p.slices),
                                dim3(kBlock), 0, st, static_cast<const T *>(src), part, outer, axis, inner, p.chunk);

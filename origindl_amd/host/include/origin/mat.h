@@ -12,6 +12,7 @@
 #include <utility>
 #include <vector>
 
+#include <atomic>
 #include <cstring>
 
 #include "base.h"
@@ -75,9 +76,10 @@ public:
     // device has been synchronised the host reads them there, with no copy queued. Set after the data() call that handed
     // the buffer to that kernel; like the host copy above it stops being trusted at the next data() call. A kernel
     // recorded into a graph keeps writing the words on every replay, so they are never given back (`recorded`).
-    void set_mirror(void *pinned_words, bool recorded) const
+    // `stream` is the stream of the kernel that writes the words: the slot goes back to that stream's free list only.
+    void set_mirror(void *pinned_words, bool recorded, void *stream) const
     {
-        mirror_ = pinned_words, mirror_recorded_ = recorded, mirror_valid_ = pinned_words != nullptr;
+        mirror_ = pinned_words, mirror_stream_ = stream, mirror_recorded_ = recorded, mirror_valid_ = pinned_words != nullptr;
     }
     // the device is synchronised and `n` bytes are read from the mirror; false when there is none to trust
     bool read_mirror(void *dst, size_t n) const;
@@ -91,16 +93,19 @@ private:
     size_t size_, capacity_;
     DeviceType type_;
     int index_;
-    mutable bool host_copy_valid_ = false;
+    // the three flags below are flipped inside const accessors that other host threads may call on a shared buffer
+    mutable std::atomic<bool> host_copy_valid_{false};
     mutable size_t host_copy_bytes_ = 0;
     mutable unsigned char host_copy_[8] = {0};
     void run_pending_fill() const;
-    mutable bool fill_pending_ = false, fill_set_while_capturing_ = false;
+    mutable std::atomic<bool> fill_pending_{false};
+    mutable bool fill_set_while_capturing_ = false;
     mutable int fill_dtype_ = 0;
     mutable int64_t fill_n_ = 0;
     mutable unsigned char fill_element_[8] = {0};
-    mutable void *mirror_ = nullptr;
-    mutable bool mirror_valid_ = false, mirror_recorded_ = false;
+    mutable void *mirror_ = nullptr, *mirror_stream_ = nullptr;
+    mutable std::atomic<bool> mirror_valid_{false};
+    mutable bool mirror_recorded_ = false;
 };
 
 class Mat

@@ -358,7 +358,9 @@ std::shared_ptr<Storage> Storage::create(size_t bytes, DeviceType type, int inde
     return std::shared_ptr<Storage>(new Storage(p, bytes, cap, type, index));
 }
 
-// 16-byte slots of pinned host memory, carved from 4 KiB pieces that live as long as the process
+// 16-byte slots of pinned host memory, carved from 4 KiB pieces that live as long as the process. A slot is given back
+// while the kernel that writes it may still be queued, so free slots are kept per stream: the next kernel to get the
+// slot is then queued behind that one, and a stale write can never land after a newer one.
 class MirrorPool
 {
 public:
@@ -367,29 +369,36 @@ public:
         static MirrorPool *pool = new MirrorPool();
         return *pool;
     }
-    void *take()
+    void *take(void *stream)
     {
         std::lock_guard<std::mutex> lock(mutex_);
-        if (free_.empty())
+        auto &mine = free_[stream];
+        if (mine.empty())
         {
-            void *piece = nullptr;
-            check(odl_hip_host_alloc(&piece, 4096));
-            for (size_t off = 0; off < 4096; off += 16)
-                free_.push_back(static_cast<char *>(piece) + off);
+            if (fresh_.empty())
+            {
+                void *piece = nullptr;
+                check(odl_hip_host_alloc(&piece, 4096));
+                for (size_t off = 0; off < 4096; off += 16)
+                    fresh_.push_back(static_cast<char *>(piece) + off);
+            }
+            mine.push_back(fresh_.back());
+            fresh_.pop_back();
         }
-        void *slot = free_.back();
-        free_.pop_back();
+        void *slot = mine.back();
+        mine.pop_back();
         return slot;
     }
-    void give(void *slot)
+    void give(void *slot, void *stream)
     {
         std::lock_guard<std::mutex> lock(mutex_);
-        free_.push_back(slot);
+        free_[stream].push_back(slot);
     }
 
 private:
     std::mutex mutex_;
-    std::vector<void *> free_;
+    std::vector<void *> fresh_;                    // never handed to a kernel yet
+    std::map<void *, std::vector<void *>> free_;   // by the stream of the kernel that last wrote the slot
 };
 
 // The buffers of this thread whose fill may still be pending. A capture must not record the fill of a buffer that was
@@ -401,6 +410,7 @@ void Storage::set_pending_fill(int dtype_code, int64_t n, const void *element, s
     std::memset(fill_element_, 0, sizeof(fill_element_));
     std::memcpy(fill_element_, element, element_bytes < sizeof(fill_element_) ? element_bytes : sizeof(fill_element_));
     fill_dtype_ = dtype_code, fill_n_ = n;
+    fill_set_while_capturing_ = t_capturing;
     fill_pending_ = n > 0;
     if (!fill_pending_ || t_capturing)
         return;
@@ -421,6 +431,11 @@ void Storage::set_pending_fill(int dtype_code, int64_t n, const void *element, s
 
 void Storage::run_pending_fill() const
 {
+    // begin_capture runs the fills this thread had pending; one that is still pending here was made by another thread
+    // (or dropped from the list). Recording it would make every replay reset the buffer.
+    if (t_capturing && !fill_set_while_capturing_)
+        THROW_RUNTIME_ERROR("a zeros/ones/full buffer made before the capture began (on another thread?) is first used "
+                            "inside it: touch it before begin_capture");
     fill_pending_ = false;
     check(odl_hip_fill_dtype(data_, fill_dtype_, fill_n_, fill_element_, cur()));
 }
@@ -447,7 +462,7 @@ bool Storage::read_mirror(void *dst, size_t n) const
 Storage::~Storage()
 {
     if (mirror_ && !mirror_recorded_)
-        MirrorPool::get().give(mirror_);
+        MirrorPool::get().give(mirror_, mirror_stream_);
     if (!data_)
         return;
     if (type_ == DeviceType::kCPU)
@@ -1692,10 +1707,10 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) 
     Workspace ws(odl_hip_softmax_ce_loss_workspace_bytes(N), device().index());
     // two words: the loss, and the bad-label flag behind it; the Mat is the scalar in front
     auto storage = Storage::create(2 * sizeof(float), DeviceType::kCUDA, device().index());
-    void *mirror = MirrorPool::get().take();
+    void *mirror = MirrorPool::get().take(cur());
     check(odl_hip_softmax_ce_loss_device(fp(x), t.storage()->data(), is64, N, C, static_cast<float *>(storage->data()),
                                          mirror, ws.ptr(), ws.bytes, cur()));
-    storage->set_mirror(mirror, t_capturing);
+    storage->set_mirror(mirror, t_capturing, cur());
     return std::make_unique<OriginMat>(std::move(storage), Shape{}, DataType::kFloat32);
 }
 

@@ -41,6 +41,7 @@
 #include "origin/operators/math/div.h"
 #include "origin/operators/math/exp.h"
 #include "origin/operators/math/log.h"
+#include "origin/utils/log.h"
 #include "origin/operators/math/mat_mul.h"
 #include "origin/operators/math/mul.h"
 #include "origin/operators/math/neg.h"
@@ -231,6 +232,11 @@ extern "C" {
 
 int DRV(ping)()
 {
+#ifdef origin_logger
+    // the reference's logger opens its file sink relative to the working directory when first used; touching it here
+    // lets the loader choose that directory
+    (void)origin_logger;
+#endif
     return 1;
 }
 
@@ -1072,11 +1078,20 @@ void timed_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T, int s
         opt.step();
         return L.template item<float>();
     };
+    // loss[0]: the loss of the first step taken from the initial parameters (the same number whichever way the steps
+    // are run afterwards, so the runs can be compared); loss[1]: the loss of the last step
+    bool first = true;
+    auto note = [&](float v) {
+        if (first)
+            loss[0] = v;
+        first   = false;
+        loss[1] = v;
+    };
     for (int i = 0; i < warmup; ++i)
-        *loss = one();
+        note(one());
     const auto t0 = std::chrono::steady_clock::now();
     for (int i = 0; i < steps; ++i)
-        *loss = one();
+        note(one());
     // the parameters of the last step are still in flight: reading the smallest one back drains the queue
     // (a large one would add its own copy time to the steps)
     auto params = model.parameters();
@@ -1107,7 +1122,9 @@ void timed_graph_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T,
         auto L = F::softmax_cross_entropy(model(X.detach()), T.detach());  // new handles on the batch, as in timed_steps
         L.backward();
         opt.step();
-        *loss = L.template item<float>();
+        loss[1] = L.template item<float>();
+        if (i == 0)
+            loss[0] = loss[1];  // the first step from the initial parameters, as in timed_steps
     }
     origin::cuda::Graph graph;
     Tensor L;
@@ -1122,16 +1139,16 @@ void timed_graph_steps(Model &model, Opt &opt, const Tensor &X, const Tensor &T,
         opt.prepare_replay();
         graph.launch();
     }
-    *loss = L.template item<float>();
+    loss[1] = L.template item<float>();
     const auto t0 = std::chrono::steady_clock::now();
     for (int i = 0; i < steps; ++i)
     {
         opt.prepare_replay();
         graph.launch();
         if (read_loss)
-            *loss = L.template item<float>();
+            loss[1] = L.template item<float>();
     }
-    *loss = L.template item<float>();  // synchronises: every replay is complete
+    loss[1] = L.template item<float>();  // synchronises: every replay is complete
     const auto t1 = std::chrono::steady_clock::now();
     *ms = std::chrono::duration<float, std::milli>(t1 - t0).count() / (float)(steps > 0 ? steps : 1);
 }
@@ -1398,7 +1415,9 @@ int DRV(cnn_bn_bench)(int64_t N, int steps, int warmup, int graph_mode, float *m
             auto guard = no_grad();
             losses[0] = F::softmax_cross_entropy(model(X), T).item<float>();
         }
-        run_timed(model, opt, X, T, steps, warmup, graph_mode, ms_per_step, &losses[1]);
+        float first_last[2] = {0.0f, 0.0f};
+        run_timed(model, opt, X, T, steps, warmup, graph_mode, ms_per_step, first_last);
+        losses[1] = first_last[1];
         model.eval();
         auto guard = no_grad();
         losses[2] = F::softmax_cross_entropy(model(X), T).item<float>();

@@ -1,9 +1,12 @@
 """ctypes bindings of the CPU oracle (oracle/liboracle.so) and, where it was built, of the compiled
 reference CPU backend (oracle/_ref/libodl_ref.so). Test infrastructure only: imported by tests, by the
 smoke check and by the CPU-baseline leg of the benchmark, never by the shipped package."""
+import atexit
 import ctypes
 import os
+import shutil
 import subprocess
+import tempfile
 
 import numpy as np
 
@@ -166,16 +169,71 @@ def have_ref():
     return os.path.exists(REF_SO)
 
 
+REF_MANIFEST = os.path.join(ORACLE_DIR, "_ref", "MANIFEST")
+
+
+def write_ref_manifest(names):
+    """Called by the build once the reference-side binaries exist: the tests that run them then FAIL when one is
+    missing; without a manifest (a tree that never had the reference beside it) they skip."""
+    with open(REF_MANIFEST, "w") as f:
+        f.write("\n".join(names) + "\n")
+
+
+def ref_binary(name):
+    """Path of oracle/_ref/<name>, or None when it is absent and nothing says that it was built. Raises when the build
+    recorded it (oracle/_ref/MANIFEST, or ODL_REQUIRE_REF=1 in the environment) and the file is not there."""
+    path = os.path.join(ORACLE_DIR, "_ref", name)
+    if os.path.exists(path):
+        return path
+    promised = os.environ.get("ODL_REQUIRE_REF") == "1"
+    if os.path.exists(REF_MANIFEST):
+        with open(REF_MANIFEST) as f:
+            promised = promised or name in f.read().split()
+    if promised:
+        raise FileNotFoundError("oracle/_ref/%s was built with this tree but is missing now" % name)
+    return None
+
+
 def ref():
     """The compiled reference CPU backend; only present where oracle/Makefile's `ref` target was built."""
     global _ref
     if _ref is None:
-        _ref = _Lib(REF_SO, _REF_SIGS)
+        lib = _Lib(REF_SO, _REF_SIGS)
+        # the reference's logger creates originlog/origin.txt under the working directory the first time it is used:
+        # let that happen in a scratch directory, not in the tree the tests run from
+        here, scratch = os.getcwd(), tempfile.mkdtemp(prefix="odl_ref_log_")
+        os.chdir(scratch)
+        try:
+            lib.odl_ref_ping()
+        finally:
+            os.chdir(here)
+        atexit.register(shutil.rmtree, scratch, True)
+        _ref = lib
     return _ref
 
 
-HOST_DRIVER_SO = os.path.join(ROOT, "origindl_amd", "lib", "libodl_host_driver.so")
-HOST_CPU_DRIVER_SO = os.path.join(ROOT, "origindl_amd", "lib", "libodl_hostcpu_driver.so")
+DRIVER_DIR = os.path.join(ROOT, "tests", "lib")
+HOST_DRIVER_SO = os.path.join(DRIVER_DIR, "libodl_host_driver.so")
+HOST_CPU_DRIVER_SO = os.path.join(DRIVER_DIR, "libodl_hostcpu_driver.so")
+
+
+def build_drivers():
+    """tests/api_driver.cpp compiled against the C++ host layer (origindl_amd/lib/liborigin_host.so, which must exist)
+    -> tests/lib/libodl_host_driver.so (tensors on the device) and tests/lib/libodl_hostcpu_driver.so (tensors left
+    on the CPU). Plain g++, no device code; the benchmark's whole-step rows and the host-layer tests load them."""
+    pkg = os.path.join(ROOT, "origindl_amd")
+    os.makedirs(DRIVER_DIR, exist_ok=True)
+    common = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-fPIC", "-Wall", "-Wno-unused-variable", "-shared",
+              "-I" + os.path.join(pkg, "host", "include"), "-I" + os.path.join(ROOT, "include")]
+    link = [os.path.join(ROOT, "tests", "api_driver.cpp"), "-L" + os.path.join(pkg, "lib"), "-lorigin_host", "-lodl_hip",
+            "-Wl,-rpath,$ORIGIN/../../origindl_amd/lib"]
+    for defs, out in ((["-DDRV_ON_DEVICE", "-DDRV_PREFIX=odl_host_"], HOST_DRIVER_SO),
+                      (["-DDRV_PREFIX=odl_hostcpu_"], HOST_CPU_DRIVER_SO)):
+        cmd = common + defs + ["-o", out] + link
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("driver build failed:\n" + " ".join(cmd) + "\n" + res.stdout)
+    return HOST_DRIVER_SO, HOST_CPU_DRIVER_SO
 _host = {}
 
 

@@ -445,8 +445,8 @@ def test_reference_example_nn_linear_runs_unchanged_on_the_gpu():
     own integration test accepts |w-2| < 0.1 and |b-5| < 0.1 (tests/unit_test/autograd/test_linear_regression.cpp:47-101)."""
     import re
     import subprocess
-    exe = os.path.join(ol.ORACLE_DIR, "_ref", "example_nn_linear_hip")
-    if not os.path.exists(exe):
+    exe = ol.ref_binary("example_nn_linear_hip")  # raises when the build recorded the binary and it is gone
+    if exe is None:
         pytest.skip("the example binary is built only where the reference checkout is present")
     out = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert out.returncode == 0, out.stdout[-2000:]
@@ -640,8 +640,8 @@ def test_the_references_own_operator_unit_tests_pass_on_this_backend():
     for every type, batch norm for both floating-point types. No case is left out by name."""
     import re
     import subprocess
-    exe = os.path.join(ol.ORACLE_DIR, "_ref", "reference_operator_tests_hip")
-    if not os.path.exists(exe):
+    exe = ol.ref_binary("reference_operator_tests_hip")  # raises when the build recorded the binary and it is gone
+    if exe is None:
         pytest.skip("the unit-test binary is built only where the reference checkout is present")
     out = subprocess.run([exe, "--gtest_filter=*CUDA*:TensorCreateTest.*:MultiTypeTensorTest.*:TensorOptionsTest.*",
                           "--gtest_brief=1"],

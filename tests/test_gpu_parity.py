@@ -398,6 +398,40 @@ def test_conv_full_size_properties(api, o, N, C, H, OC, s, p):
     assert bool(((gw.double() - want_gw).abs() <= bnd).all())
     want_gx = api.col2im((gy2d @ w.reshape(OC, K).double()).float(), x.shape, 3, s, p, True)
     assert float((gx - want_gx).abs().max()) <= 9 * 1e-5 * float(gy2d.norm(dim=1).max() * w.reshape(OC, K).norm(dim=0).max())
+    # The same two gradients against the oracle alone, on samples (nothing of the device's own output enters): three rows
+    # gW[oc] = gy2d^T[oc, :] . col with col from the oracle's im2col and the reference's k-ascending sums
+    # (conv2d.cpp:548-562), and twenty pixels of gx = col2im(gy2d . W2d) (conv2d.cpp:584-596), each from the nine col rows
+    # that reach it, folded by the oracle's col2im on that image alone.
+    gyh, gwh, gxh = host(gy), host(gw), host(gx)
+    gy2dh, w2d = gyh.reshape(M, OC), np.ascontiguousarray(wh.reshape(OC, K))
+    colh = np.empty((M, K), f32)
+    assert o.orc_im2col(xh, N, C, H, H, 3, 3, s, s, p, p, 1, colh) == 0
+    col_norm = np.linalg.norm(colh.astype(np.float64), axis=0)
+    for oc in sorted({0, OC - 1, int(rng.integers(0, OC))}):
+        row = np.ascontiguousarray(gy2dh[:, oc]).reshape(1, M)
+        want = np.empty((1, K), f32)
+        o.orc_matmul(row, colh, want, 1, K, M)
+        bound = 1e-5 * np.linalg.norm(row.astype(np.float64)) * col_norm + 1e-7
+        assert (np.abs(gwh[oc].reshape(-1) - want[0]) <= bound).all(), ("gW row", oc)
+    del colh
+    wcol_norm = np.linalg.norm(w2d.astype(np.float64), axis=0)
+    for _ in range(20):
+        n, c, h, wx = (int(rng.integers(0, d)) for d in (N, C, H, H))
+        gcol = np.zeros((OH * OH, K), f32)
+        bound = 1e-6
+        for kh in range(3):
+            for kw in range(3):
+                hh, ww = h + p - kh, wx + p - kw
+                if hh % s or ww % s or not (0 <= hh // s < OH and 0 <= ww // s < OH):
+                    continue
+                m = (hh // s) * OH + ww // s
+                out = np.empty((1, K), f32)
+                o.orc_matmul(np.ascontiguousarray(gy2dh[n * OH * OH + m]).reshape(1, OC), w2d, out, 1, K, OC)
+                gcol[m] = out[0]
+                bound += 1e-5 * np.linalg.norm(gy2dh[n * OH * OH + m].astype(np.float64)) * wcol_norm[(c * 3 + kh) * 3 + kw]
+        img = np.empty((1, C, H, H), f32)
+        assert o.orc_col2im(gcol, 1, C, H, H, 3, 3, s, s, p, p, 1, img) == 0
+        assert abs(gxh[n, c, h, wx] - img[0, c, h, wx]) <= bound, ("gx pixel", n, c, h, wx)
 
 
 # ------------------------------------------------------------------------------- reductions / broadcast
@@ -1185,7 +1219,8 @@ def test_elementwise_fill_and_sum_in_every_element_type(api, name):
     L.call("odl_hip_fill_dtype", out.data_ptr(), code, n, v.ctypes.data, None)
     assert (host(out) == v[0]).all()
     # sums: [outer, axis, inner] in both layouts and the whole tensor (which passes through a float, as the reference's)
-    for outer, axis, inner in ((1, n, 1), (3, 1000, 1), (4, 300, 50), (1, 5000, 3), (2, 7, 1), (1, 4096 * 64, 1)):
+    for outer, axis, inner in ((1, n, 1), (3, 1000, 1), (4, 300, 50), (1, 5000, 3), (2, 7, 1), (1, 4096 * 64, 1),
+                               (70000, 8, 1)):  # more rows than a grid's second dimension holds
         x = _typed_values(rng, t, outer * axis * inner).reshape(outer, axis, inner)
         nb = L.query("odl_hip_sum_axis_dtype_workspace_bytes", code, outer, axis, inner)
         ws = torch.empty(max(nb, 8), dtype=torch.uint8, device="cuda")
