@@ -1200,6 +1200,69 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
     return ODL_OK;
 }
 
+// The two gradients of y = x.w in one launch (gx[M,K] = gy[M,N].w[K,N]^T and gw[K,N] = x[M,K]^T.gy[M,N]) when each of
+// them alone would be a single launch of about one workgroup per compute unit on the straight-to-LDS kernel: together
+// they put two workgroups on every compute unit. Returns 1 when launched, 0 when the shapes do not suit (the caller then
+// launches them one after the other), a negative error code on failure.
+namespace
+{
+// the tile class a product would take as a launch of its own, when that launch is one the pair kernel can stand in for
+// (whole K per workgroup, 16-byte loads): 128, 64 or 32; 0 otherwise
+int pair_tile_class(bool vec, int64_t M, int64_t N, int64_t K)
+{
+    if (!vec || K < 128)
+        return 0;
+    if (pick_tile(M, N) == 128)
+        return ceil_div(M, 128) * ceil_div(N, 128) <= lone_workgroup_limit() ? 128 : 0;
+    const int64_t tiles = ceil_div(M, 64) * ceil_div(N, 64);
+    const int s2 = pick_splits_two_sets(tiles, K);
+    if (s2 == 2 && ceil_div(M, 64) * ceil_div(N, 32) <= lone_workgroup_limit())
+        return 32;
+    if (s2 == 1)  // (which already says: at most about one 64x64 tile per compute unit, K of 256 or more)
+        return 64;
+    return 0;
+}
+
+odl::DmaGemmArgs pair_product(int cls, const float *A, int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc,
+                              int64_t M, int64_t N, int64_t K)
+{
+    odl::DmaGemmArgs d{};
+    d.A = A, d.B = B, d.bias = nullptr, d.C = C;
+    d.M = M, d.N = N, d.K = K, d.lda = lda, d.ldb = ldb, d.ldc = ldc;
+    d.tiles_m = (int)ceil_div(M, cls == 128 ? 128 : 64), d.tiles_n = (int)ceil_div(N, cls == 128 ? 128 : (cls == 32 ? 32 : 64));
+    d.splits = 1, d.k_per_split = ceil_div(K, 64) * 64, d.c_split_stride = 0;
+    d.epi = 0, d.act = 0, d.xcds = odl::chip().xcds, d.c_p = 0;
+    d.main_blocks = 0, d.tail_first = d.tiles_m * d.tiles_n, d.tail_splits = 0, d.tail_kps = 0, d.tail_ws = nullptr;
+    d.batch = 1, d.a_batch = d.b_batch = d.c_batch = 0;
+    return d;
+}
+}  // namespace
+
+int matmul_backward_pair(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M, int64_t K,
+                         int64_t N, hipStream_t st)
+{
+    if (M <= 0 || K <= 0 || N <= 0 || M >= (1ll << 31) || K >= (1ll << 31) || N >= (1ll << 31))
+        return 0;
+    // 16-byte loads: every row of x [M,K], w [K,N] and gy [M,N] starts on a 16-byte boundary and M is a multiple of four
+    // (x^T's rows are read four columns of x at a time)
+    const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(gy)) % 16 == 0) &&
+                     K % 4 == 0 && N % 4 == 0;
+    const int c0 = pair_tile_class(vec, M, K, N), c1 = pair_tile_class(vec, K, N, M);
+    if (c0 == 0 || c1 == 0 || (c0 == 128) != (c1 == 128))
+        return 0;
+    const odl::DmaGemmArgs d0 = pair_product(c0, gy, N, w, N, gx, K, M, K, N);  // gx = gy . w^T
+    const odl::DmaGemmArgs d1 = pair_product(c1, x, K, gy, N, gw, N, K, N, M);  // gw = x^T . gy
+    // all workgroups resident at once, two per compute unit
+    if ((int64_t)d0.tiles_m * d0.tiles_n + (int64_t)d1.tiles_m * d1.tiles_n > 2 * (int64_t)odl::device_cus())
+        return 0;
+    if (!odl::sgemm_dma_fits(false, true, d0) || !odl::sgemm_dma_fits(true, false, d1))
+        return 0;
+    const int rc = odl::sgemm_dma_pair_launch(c0, d0, c1, d1, st);
+    if (rc != ODL_OK)
+        return rc;  // (error codes are negative)
+    return 1;
+}
+
 // ------------------------------------------------------------------------------------------------------
 // Convolution as implicit GEMM: the same kernel, its B operand gathered from the image / upstream gradient.
 namespace
@@ -1603,6 +1666,17 @@ int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, flo
 {
     ODL_REQUIRE_DEVICE();
     hipStream_t st = odl::as_stream(stream);
+    if (gx && gw && x && w && gy)
+    {
+        const int paired = odl::matmul_backward_pair(x, w, gy, gx, gw, M, K, N, st);
+        if (paired < 0)
+            return paired;
+        if (paired == 1)
+        {
+            ODL_LAUNCH_CHECK();
+            return ODL_OK;
+        }
+    }
     if (gx)  // gx[M,K] = gy[M,N] . w[K,N]^T
     {
         int rc = odl::sgemm_launch(0, 1, M, K, N, gy, N, w, N, gx, K, nullptr, EPI_PLAIN, 0, 0, workspace,

@@ -40,6 +40,11 @@ bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g);
 // tiles_m * tiles_n * splits workgroups of 512 threads (main_blocks + tail tiles * tail_splits with a tail split)
 int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st);
 
+// Two whole products in one launch, two workgroups per compute unit: g0 = X.Y^T (A [M,K] and B [N,K] row-major) on tiles
+// of class tile0, g1 = X^T.Y (A [K,M] and B [K,N] row-major) on tiles of class tile1. Classes: 64 (64x64 tiles), 32 (64x32
+// tiles) — these two mix freely — or 128 for both (128x128 tiles). tiles_m / tiles_n of each product count its own tiles.
+int sgemm_dma_pair_launch(int tile0, const DmaGemmArgs &g0, int tile1, const DmaGemmArgs &g1, hipStream_t st);
+
 // 1x1 / stride 1 / unpadded convolution as `N` products y[n] = act(W[OC,C] . x[n][C, H*W] + b[oc]) in one launch; false
 // when the shape does not suit (rows of H*W or C floats that are not multiples of four, unaligned pointers)
 bool conv1x1_dma_ok(const float *x, const float *w, int64_t N, int64_t C, int64_t HW, int64_t OC);

@@ -29,7 +29,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kNT     = 512;
-constexpr int kStages = 4;
 constexpr int kEpiBiasCol = 1, kEpiBiasRow = 2;
 template <int V>
 struct IntTag  // a compile-time integer passed to a generic lambda
@@ -134,11 +133,11 @@ __device__ inline int swizzle(int row)
 // KSETS wave sets share a tile: the eight waves are WAVES_N columns x (8 / KSETS / WAVES_N) rows of wave tiles, times
 // KSETS sets that each multiply every KSETS-th 8-wide K step (2 sets for square tiles; 4 sets on a 64x32 tile, whose
 // two 32x32 blocks could not occupy eight waves otherwise).
-template <int BM, int BN, int BK, bool TA, bool TB, int WGS_PER_CU, int KSETS = 2>
-// (The second launch bound counts waves per SIMD, of which a workgroup of 512 threads brings two: WGS_PER_CU there only
-// keeps the register budget generous — the kernels use under 128 registers and fit two workgroups per compute unit
-// anyway. Bounds of 2 * WGS_PER_CU changed the compiler's schedule for the worse: 2048^3 dA = dC.B^T 133 -> 142 us.)
-__global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::DmaGemmArgs g, const DmaTileMap map)
+// The whole product of one workgroup. `bid` is the workgroup's number inside its product (a launch may hold two
+// products, below); As / Bs are the LDS stages, kStages x BM*BK and kStages x BN*BK floats.
+template <int BM, int BN, int BK, bool TA, bool TB, int KSETS, int kStages>
+__device__ __forceinline__ void sgemm_dma_body(const odl::DmaGemmArgs &g, const DmaTileMap &map, const unsigned bid,
+                                               float *const As0, float *const Bs0)
 {
     constexpr bool A_KMAJOR = !TA, B_KMAJOR = TB;
     constexpr int PIECES = BK / 4;                       // 16-byte pieces in a K-contiguous row of a slab
@@ -154,8 +153,8 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     constexpr int RB = BM / WAVES_M / 32, CB = BN / WAVES_N / 32;  // 32x32 blocks per wave
     constexpr int STEPS = BK / 8 / KSETS;                          // 8-wide K steps per wave and slab
     static_assert(RB >= 1 && CB >= 1 && STEPS >= 1 && RB * WAVES_M * 32 == BM && CB * WAVES_N * 32 == BN, "wave layout");
-    __shared__ __attribute__((aligned(16))) float As[kStages][BM * BK];
-    __shared__ __attribute__((aligned(16))) float Bs[kStages][BN * BK];
+    auto As = [&](int stage) { return As0 + stage * (BM * BK); };
+    auto Bs = [&](int stage) { return Bs0 + stage * (BN * BK); };
     static_assert(kStages * BM * BK >= (KSETS - 1) * (8 / KSETS) * 16 * 64, "the A buffers hold one accumulator block of every wave of the other sets");
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -172,10 +171,10 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     {
         const unsigned nt = (unsigned)(g.tiles_m * g.tiles_n);
         unsigned t;
-        if (g.tail_splits > 0 && (int)blockIdx.x >= g.main_blocks)
+        if (g.tail_splits > 0 && (int)bid >= g.main_blocks)
         {
             // pieces of the tail tiles keep the hardware's round-robin order: they are short and should spread over all XCDs
-            const int u = (int)blockIdx.x - g.main_blocks;
+            const int u = (int)bid - g.main_blocks;
             const int ti = u / g.tail_splits, piece = u - ti * g.tail_splits;
             t = (unsigned)(g.tail_first + ti);
             kbeg = (int64_t)piece * g.tail_kps;
@@ -184,7 +183,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
         }
         else
         {
-            const unsigned bid = blockIdx.x, nx = map.xcds;
+            const unsigned nx = map.xcds;
             const unsigned loc = odl::fastdiv(bid, map.by_xcds), xcd = bid - loc * nx;
             unsigned v = xcd * map.xcd_full + (xcd < map.xcd_rem ? xcd : map.xcd_rem) + loc;
             if (g.batch > 1)
@@ -207,8 +206,8 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     const float *abase = g.A + (int64_t)bz * g.a_batch + (A_KMAJOR ? m0 * g.lda + kbeg : kbeg * g.lda + m0);
     const float *bbase = g.B + (int64_t)bz * g.b_batch + (B_KMAJOR ? n0 * g.ldb + kbeg : kbeg * g.ldb + n0);
     const i32x4 ra = buffer_of(abase), rb = buffer_of(bbase);
-    const unsigned as_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) float *)&As[0][0];
-    const unsigned bs_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) float *)&Bs[0][0];
+    const unsigned as_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) float *)As0;
+    const unsigned bs_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) float *)Bs0;
 
     // per load of this thread: byte offset inside slab 0, the K position it covers inside a slab, and whether its row
     // (or column quad) is inside the matrix
@@ -358,7 +357,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
             wait_vmcnt<(kStages - 2) * PER_SLAB>();
             __syncthreads();
             issue(kStages - 1, kStages - 1);
-            read_frags(As[0], Bs[0], 0, fa[0], fb[0]);
+            read_frags(As(0), Bs(0), 0, fa[0], fb[0]);
         }
         // all K steps of slab j, which lies in stage s; `more`: a slab follows it
         auto slab = [&](int s, int j, bool more) {
@@ -371,7 +370,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
                 mfma_part(fa[cur], fb[cur], 0, 2);
                 __builtin_amdgcn_sched_barrier(0);
                 if (st + 1 < STEPS)
-                    read_frags(As[s], Bs[s], st + 1, fa[nxt], fb[nxt]);
+                    read_frags(As(s), Bs(s), st + 1, fa[nxt], fb[nxt]);
                 else
                 {
                     if (more)
@@ -382,7 +381,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
                     }
                     // (read without a condition: after the last slab the values are never used, and a read inside a
                     // branch would have to be waited for at the branch's end)
-                    read_frags(As[(s + 1) % kStages], Bs[(s + 1) % kStages], 0, fa[nxt], fb[nxt]);
+                    read_frags(As((s + 1) % kStages), Bs((s + 1) % kStages), 0, fa[nxt], fb[nxt]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 mfma_part(fa[cur], fb[cur], 2, 4);
@@ -418,7 +417,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
 #pragma unroll
                     for (int st = 0; st < STEPS; ++st)
                     {
-                        read_frags(As[s], Bs[s], st, fa[0], fb[0]);
+                        read_frags(As(s), Bs(s), st, fa[0], fb[0]);
                         mfma_part(fa[0], fb[0], 0, 4);
                     }
                 }
@@ -431,7 +430,7 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     // the other wave sets hand their accumulators to the first, one 32x32 block of each wave at a time; the first adds
     // them in set order
     {
-        float *xch = &As[0][0] + (wave * 16) * 64 + lane;
+        float *xch = As0 + (wave * 16) * 64 + lane;
         constexpr int SET_STRIDE = TILE_WAVES * 16 * 64;
 #pragma unroll
         for (int i = 0; i < RB; ++i)
@@ -576,6 +575,37 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
     const int bias_kind = g.c_p > 0 ? 2 : (g.epi == kEpiBiasCol && g.bias != nullptr) ? 1 : (g.epi == kEpiBiasRow ? 2 : 0);
     with_epilogue_kind(bias_kind, g.act, store_blocks);
 }
+
+template <int BM, int BN, int BK, bool TA, bool TB, int WGS_PER_CU, int KSETS = 2, int kStages = 4>
+// (The second launch bound counts waves per SIMD, of which a workgroup of 512 threads brings two: WGS_PER_CU there only
+// keeps the register budget generous — the kernels use under 128 registers and fit two workgroups per compute unit
+// anyway. Bounds of 2 * WGS_PER_CU changed the compiler's schedule for the worse: 2048^3 dA = dC.B^T 133 -> 142 us.)
+__global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::DmaGemmArgs g, const DmaTileMap map)
+{
+    __shared__ __attribute__((aligned(16))) float As[kStages * BM * BK];
+    __shared__ __attribute__((aligned(16))) float Bs[kStages * BN * BK];
+    sgemm_dma_body<BM, BN, BK, TA, TB, KSETS, kStages>(g, map, blockIdx.x, As, Bs);
+}
+
+// Two independent products in one launch: workgroups [0, first) run product 0 = X.Y^T, the others product 1 = X^T.Y —
+// the two gradients of a matrix product (gx = gy.w^T, gw = x^T.gy), each on its own tile shape. Two workgroups, one of
+// each product as a rule, share a compute unit: the prologue, barriers and epilogue of one are covered by the matrix
+// instructions of the other, and the second launch's start-up is gone. Same tile code as the single launches, so the
+// same bits.
+template <int BM0, int BN0, int BK0, int KSETS0, int ST0, int BM1, int BN1, int BK1, int KSETS1, int ST1>
+__global__ __launch_bounds__(kNT, 2) void sgemm_dma_pair_kernel(const odl::DmaGemmArgs g0, const DmaTileMap map0,
+                                                                const odl::DmaGemmArgs g1, const DmaTileMap map1,
+                                                                const unsigned first, const unsigned first_padded)
+{
+    constexpr int F0 = ST0 * (BM0 + BN0) * BK0, F1 = ST1 * (BM1 + BN1) * BK1;
+    static_assert(F0 * 4 <= 80 * 1024 && F1 * 4 <= 80 * 1024, "two workgroups must fit the LDS of a compute unit");
+    __shared__ __attribute__((aligned(16))) float stages[F0 > F1 ? F0 : F1];
+    const unsigned bid = blockIdx.x;
+    if (bid < first)
+        sgemm_dma_body<BM0, BN0, BK0, false, true, KSETS0, ST0>(g0, map0, bid, stages, stages + ST0 * BM0 * BK0);
+    else if (bid >= first_padded)  // (the gap keeps product 1's workgroup numbers congruent to the XCD they run on)
+        sgemm_dma_body<BM1, BN1, BK1, true, false, KSETS1, ST1>(g1, map1, bid - first_padded, stages, stages + ST1 * BM1 * BK1);
+}
 }  // namespace
 
 namespace odl
@@ -590,6 +620,50 @@ bool sgemm_dma_fits(bool ta, bool tb, const DmaGemmArgs &g)
     return aligned && a_span < (1ll << 31) && b_span < (1ll << 31) && g.M > 0 && g.N > 0 && g.K > 0;
 }
 
+static DmaTileMap tile_map_of(const DmaGemmArgs &g)
+{
+    DmaTileMap map;
+    const int64_t nt = (int64_t)g.tiles_m * g.tiles_n;
+    const unsigned total = (unsigned)(g.tail_splits > 0 ? g.main_blocks : nt * g.splits * (g.batch > 1 ? g.batch : 1));
+    const unsigned nx = (unsigned)(g.xcds > 0 ? g.xcds : 1);
+    map.by_xcds = make_fastdiv(nx), map.by_nt = make_fastdiv((unsigned)nt);
+    map.by_gsz = make_fastdiv(8u * (unsigned)g.tiles_n);
+    map.by_gm_last = make_fastdiv((unsigned)(g.tiles_m % 8 ? g.tiles_m % 8 : 8));
+    map.xcds = nx, map.xcd_full = total / nx, map.xcd_rem = total % nx;
+    return map;
+}
+
+int sgemm_dma_pair_launch(int tile0, const DmaGemmArgs &g0, int tile1, const DmaGemmArgs &g1, hipStream_t st)
+{
+    if (g0.splits != 1 || g1.splits != 1 || g0.tail_splits > 0 || g1.tail_splits > 0 || g0.batch > 1 || g1.batch > 1 ||
+        g0.c_p > 0 || g1.c_p > 0)
+        return fail(ODL_ERR_RUNTIME, "sgemm: a pair launch takes two whole, unbatched products");
+    const unsigned n0 = (unsigned)(g0.tiles_m * g0.tiles_n), n1 = (unsigned)(g1.tiles_m * g1.tiles_n);
+    const unsigned nx = (unsigned)(g0.xcds > 0 ? g0.xcds : 1), n0p = (n0 + nx - 1) / nx * nx;
+    const DmaTileMap m0 = tile_map_of(g0), m1 = tile_map_of(g1);
+    const dim3 grid(n0p + n1), block(kNT);
+    // per class: tile rows, tile columns, slab width, wave sets, stages (two workgroups of 64 to 72 KB per compute unit)
+#define ODL_PAIR_64 64, 64, 32, 2, 4
+#define ODL_PAIR_32 64, 32, 64, 4, 3
+#define ODL_PAIR_128 128, 128, 16, 2, 4
+#define ODL_PAIR_CASE(T0, C0, T1, C1)                                                                                   \
+    if (tile0 == T0 && tile1 == T1)                                                                                     \
+    {                                                                                                                   \
+        hipLaunchKernelGGL((sgemm_dma_pair_kernel<C0, C1>), grid, block, 0, st, g0, m0, g1, m1, n0, n0p);               \
+        return ODL_OK;                                                                                                  \
+    }
+    ODL_PAIR_CASE(64, ODL_PAIR_64, 64, ODL_PAIR_64)
+    ODL_PAIR_CASE(64, ODL_PAIR_64, 32, ODL_PAIR_32)
+    ODL_PAIR_CASE(32, ODL_PAIR_32, 64, ODL_PAIR_64)
+    ODL_PAIR_CASE(32, ODL_PAIR_32, 32, ODL_PAIR_32)
+    ODL_PAIR_CASE(128, ODL_PAIR_128, 128, ODL_PAIR_128)
+#undef ODL_PAIR_CASE
+#undef ODL_PAIR_64
+#undef ODL_PAIR_32
+#undef ODL_PAIR_128
+    return fail(ODL_ERR_RUNTIME, "sgemm: no pair kernel for tile classes %d and %d", tile0, tile1);
+}
+
 int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream_t st)
 {
     if (g.c_p > 0 && !(tile == 64 || tile == 65 || tile == 32))
@@ -598,24 +672,16 @@ int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream
     const dim3 grid((unsigned)(g.tail_splits > 0 ? g.main_blocks + (nt - g.tail_first) * g.tail_splits
                                                  : nt * g.splits * (g.batch > 1 ? g.batch : 1))),
         block(kNT);
-    DmaTileMap map;
-    {
-        const unsigned total = (unsigned)(g.tail_splits > 0 ? g.main_blocks : nt * g.splits * (g.batch > 1 ? g.batch : 1));
-        const unsigned nx = (unsigned)(g.xcds > 0 ? g.xcds : 1);
-        map.by_xcds = make_fastdiv(nx), map.by_nt = make_fastdiv((unsigned)nt);
-        map.by_gsz = make_fastdiv(8u * (unsigned)g.tiles_n);
-        map.by_gm_last = make_fastdiv((unsigned)(g.tiles_m % 8 ? g.tiles_m % 8 : 8));
-        map.xcds = nx, map.xcd_full = total / nx, map.xcd_rem = total % nx;
-    }
+    const DmaTileMap map = tile_map_of(g);
 #define ODL_DMA_CASE(TA, TB)                                                                          \
     if (ta == TA && tb == TB)                                                                         \
     {                                                                                                 \
         if (tile == 64)                                                                               \
-            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 1>), grid, block, 0, st, g, map);     \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 1, 2, 4>), grid, block, 0, st, g, map); \
         else if (tile == 65)                                                                          \
             hipLaunchKernelGGL((sgemm_dma_kernel<64, 64, 32, TA, TB, 2>), grid, block, 0, st, g, map);     \
         else if (tile == 32)                                                                          \
-            hipLaunchKernelGGL((sgemm_dma_kernel<64, 32, 64, TA, TB, 1, 4>), grid, block, 0, st, g, map);  \
+            hipLaunchKernelGGL((sgemm_dma_kernel<64, 32, 64, TA, TB, 1, 4, 4>), grid, block, 0, st, g, map); \
         else if (tile == 128)                                                                         \
             hipLaunchKernelGGL((sgemm_dma_kernel<128, 128, 32, TA, TB, 1>), grid, block, 0, st, g, map);   \
         else                                                                                          \

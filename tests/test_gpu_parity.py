@@ -92,6 +92,31 @@ def test_matmul_forward_backward_vs_oracle(api, o, m, k, n):
     assert_gemm_close(gw[krows], gwo, xT[krows], gy, "dB")
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 784, 1000), (1024, 1024, 1024), (2048, 2048, 2048), (516, 780, 1004),
+                                   (772, 1028, 520), (1000, 1000, 1000), (260, 516, 772), (2044, 2052, 1996)])
+def test_matmul_backward_in_one_launch_equals_the_two_gradients_launched_alone(api, m, k, n):
+    # Both gradients asked for together may run as one launch of two products (two workgroups per compute unit); asked
+    # for one at a time they are launches of their own. The tile code is shared and K is walked in the same order, so the
+    # results must agree bit for bit, whatever tile classes the two products fall into (64x64, 64x32, 128x128, ragged).
+    print("\n[case] matmul backward pair", m, k, n, flush=True)
+    import ctypes
+    L = api.lib()
+    g = torch.Generator(device="cuda").manual_seed(m + k + n)
+    x, w, gy = (torch.randn(s, device="cuda", generator=g) for s in ((m, k), (k, n), (m, n)))
+    nb = L.query("odl_hip_matmul_backward_workspace_bytes", m, k, n)
+    ws = torch.empty(max(nb, 16) // 4, dtype=torch.int32, device="cuda")
+    P = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    gx2, gw2, gx1, gw1 = (torch.full(s, float("nan"), device="cuda") for s in ((m, k), (k, n), (m, k), (k, n)))
+    L.call("odl_hip_matmul_backward", P(x), P(w), P(gy), P(gx2), P(gw2), m, k, n, P(ws), nb, None)
+    L.call("odl_hip_matmul_backward", P(x), P(w), P(gy), P(gx1), None, m, k, n, P(ws), nb, None)
+    L.call("odl_hip_matmul_backward", P(x), P(w), P(gy), None, P(gw1), m, k, n, P(ws), nb, None)
+    assert torch.equal(gx2, gx1) and torch.equal(gw2, gw1)
+    want_gx, want_gw = gy.double() @ w.double().t(), x.double().t() @ gy.double()
+    bx = 1e-5 * torch.outer(gy.double().norm(dim=1), w.double().norm(dim=1))
+    bw = 1e-5 * torch.outer(x.double().norm(dim=0), gy.double().norm(dim=0))
+    assert bool(((gx2.double() - want_gx).abs() <= bx).all()) and bool(((gw2.double() - want_gw).abs() <= bw).all())
+
+
 def test_matmul_reference_unit_test_vectors(api):
     # tests/unit_test/operator/test_matmul.cpp:19-64, 119-143, 213-229
     x, w = dev(np.array([[1, 2], [3, 4]], f32)), dev(np.array([[5, 6], [7, 8]], f32))
