@@ -10,6 +10,7 @@
 //             [N*OH*OW, OC] matrix exactly as it lies (conv2d.cpp:548) — free on the GPU: it is the same pointer.
 //   col2im is a gather: one thread owns one image pixel and adds its taps in ascending (kh, kw) order, which
 //   is the order in which the reference's scatter loop reaches that pixel — bit-identical sums, no atomics.
+#include "conv_side.h"
 #include "gemm_dma.h"
 #include "odl_common.h"
 
@@ -59,7 +60,8 @@ bool conv_patch_dgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64
 size_t conv_patch_dgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC);
 
 int conv_patch_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
-                     void *workspace, size_t workspace_bytes, hipStream_t st);
+                     void *workspace, size_t workspace_bytes, hipStream_t st, bool packed);
+SidePack conv_patch_dgrad_pack(const float *w, int64_t C, int64_t OC, void *workspace);
 bool conv_small_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
                          int64_t OW);
 size_t conv_small_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
@@ -72,6 +74,13 @@ size_t conv_small_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW);
 int conv_small_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
                      int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
                      size_t workspace_bytes, hipStream_t st);
+// conv_wgrad.hip: 3x3 / padding 1 / stride 1 or 2, walking the output rows with the input rows staged in LDS
+bool conv_wgrad_rows_ok(const float *gy, const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH,
+                        int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW);
+size_t conv_wgrad_rows_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW,
+                                 int PH, int PW, int64_t OH, int64_t OW);
+int conv_wgrad_rows(const float *gy, const float *x, float *gw, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                    int S, int64_t OH, int64_t OW, void *workspace, size_t workspace_bytes, hipStream_t st, SideFold *fold);
 int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
                              size_t workspace_bytes, hipStream_t st);
 size_t sum_nchw_channels_workspace(int64_t N, int64_t OC, int64_t P);
@@ -1245,18 +1254,42 @@ int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, in
 
 namespace
 {
+// The small jobs of a backward pass in one launch: workgroups [0, n_bias) sum a channel of gy each (the longest job
+// first), the next n_fold add the weight gradient's partial tiles, the last n_pack make the input-gradient kernel's
+// filter copy. Any of the three counts may be zero.
+struct SideJobs
+{
+    odl::SideBias bias;
+    odl::SideFold fold;
+    odl::SidePack pack;
+    unsigned n_bias, n_fold, n_pack;
+};
+
+__global__ __launch_bounds__(1024) void conv_backward_side_kernel(const SideJobs j)
+{
+    __shared__ odl::side_f32x4 lds[1024];
+    const unsigned b = blockIdx.x;
+    if (b < j.n_bias)
+        odl::side_bias(j.bias, b, reinterpret_cast<float *>(lds));
+    else if (b < j.n_bias + j.n_fold)
+        odl::side_fold(j.fold, b - j.n_bias, lds);
+    else
+        odl::side_pack(j.pack, b - j.n_bias - j.n_fold, j.n_pack);
+}
+
 // workspace regions of conv2d_backward, in order: [col][split-K partials][permuted weights][bias partials]
 struct BwdPlan
 {
     bool wgrad_small, dgrad_small;  // few input channels: the direct kernels, no matrices at all
+    bool wgrad_rows;                // 3x3/p1 at stride 1 or 2: output rows walked with the input rows in LDS
     bool dgrad_patch;               // 3x3/s1/p1: the gradient patch stays in LDS
     bool wgrad_implicit, dgrad_implicit;
     size_t col_bytes, splitk_bytes, wp_bytes, red_bytes;
     size_t total() const { return col_bytes + splitk_bytes + wp_bytes + red_bytes; }
 };
 
-BwdPlan plan_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
-                      int SW, int64_t OH, int64_t OW)
+BwdPlan plan_backward(const float *gy, const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                      int SH, int SW, int PH, int PW, int64_t OH, int64_t OW)
 {
     BwdPlan p{};
     const int64_t M = N * OH * OW, K = C * KH * KW;
@@ -1264,12 +1297,14 @@ BwdPlan plan_backward(const float *gy, int64_t N, int64_t C, int64_t H, int64_t 
     p.dgrad_small = odl::conv_small_dgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
     // 3x3 at stride 1 keeps the image size only with a padding of 1
     const int pad = (OH == H && OW == W) ? 1 : -1;
-    p.wgrad_implicit = !p.wgrad_small && odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
+    p.wgrad_rows = !p.wgrad_small && odl::conv_wgrad_rows_ok(gy, x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW);
+    p.wgrad_implicit = !p.wgrad_small && !p.wgrad_rows && odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
     p.dgrad_patch = !p.dgrad_small && odl::conv_patch_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW, pad, pad);
     p.dgrad_implicit = !p.dgrad_small && !p.dgrad_patch && odl::conv_implicit_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW);
-    const bool no_col = (p.wgrad_small || p.wgrad_implicit) && (p.dgrad_small || p.dgrad_patch || p.dgrad_implicit);
+    const bool no_col = (p.wgrad_small || p.wgrad_rows || p.wgrad_implicit) && (p.dgrad_small || p.dgrad_patch || p.dgrad_implicit);
     p.col_bytes = no_col ? 0 : align256((size_t)(M * K) * sizeof(float));
     p.splitk_bytes = align256(p.wgrad_small      ? odl::conv_small_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
+                              : p.wgrad_rows     ? odl::conv_wgrad_rows_workspace(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW)
                               : p.wgrad_implicit ? odl::conv_implicit_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
                                                  : odl::sgemm_workspace(OC, K, M, 0));
     p.wp_bytes = p.dgrad_small      ? align256(odl::conv_small_dgrad_workspace(C, OC, KH, KW))
@@ -1289,7 +1324,7 @@ size_t odl_hip_conv2d_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, 
     const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
     if (OH <= 0 || OW <= 0)
         return 0;
-    return plan_backward(kAlignedProbe, N, C, H, W, OC, KH, KW, SH, SW, OH, OW).total();
+    return plan_backward(kAlignedProbe, kAlignedProbe, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW).total();
 }
 
 int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int64_t N, int64_t C, int64_t H, int64_t W,
@@ -1305,7 +1340,7 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
     const int64_t M = N * g.OH * g.OW, K = C * KH * KW;
     if (M == 0)
         return ODL_OK;
-    const BwdPlan p = plan_backward(gy, N, C, H, W, OC, KH, KW, SH, SW, g.OH, g.OW);
+    const BwdPlan p = plan_backward(gy, x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW);
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= p.total(),
                 "conv2d_backward: this shape/alignment needs a workspace of %zu bytes, got %zu", p.total(),
                 workspace_bytes);
@@ -1317,7 +1352,33 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
     void *red_ws = ws + p.col_bytes + p.splitk_bytes + p.wp_bytes;
 
     // gy2d: gy's NCHW buffer read as a row-major [M, OC] matrix exactly as it lies (conv2d.cpp:548)
-    if (gw)
+    // With the row-walking weight gradient, the jobs that follow it — the sum of its partial tiles, the bias gradient,
+    // the filter copy of the LDS-patch input gradient — run side by side in one launch.
+    const int64_t P = g.OH * g.OW;
+    const bool side = gw && p.wgrad_rows;
+    const bool side_bias = side && gb && P % 4 == 0 && N * P < (1ll << 31) && OC <= 4096 && reinterpret_cast<uintptr_t>(gy) % 16 == 0;
+    const bool side_pack = side && gx && p.dgrad_patch;
+    if (side)
+    {
+        SideJobs j{};
+        rc = odl::conv_wgrad_rows(gy, x, gw, N, C, H, W, OC, SH, g.OH, g.OW, splitk_ws, p.splitk_bytes, st, &j.fold);
+        if (rc != ODL_OK)
+            return rc;
+        j.n_fold = (unsigned)odl::ceil_div(j.fold.n4, 256);
+        if (side_bias)
+        {
+            j.bias = odl::SideBias{gy, gb, (unsigned)(N * P), (unsigned)P, (unsigned)OC, odl::make_fastdiv((unsigned)(P / 4))};
+            j.n_bias = (unsigned)OC;
+        }
+        if (side_pack)
+        {
+            j.pack = odl::conv_patch_dgrad_pack(w, C, OC, wp_ws);
+            j.n_pack = (unsigned)std::min<int64_t>(odl::ceil_div((int64_t)j.pack.Cin * 9 * j.pack.Mpad, 1024), 128);
+        }
+        hipLaunchKernelGGL(conv_backward_side_kernel, dim3(j.n_bias + j.n_fold + j.n_pack), dim3(1024), 0, st, j);
+        ODL_LAUNCH_CHECK();
+    }
+    else if (gw)
     {
         if (p.wgrad_small)
             rc = odl::conv_small_wgrad(gy, x, gw, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, splitk_ws,
@@ -1335,7 +1396,7 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
         if (rc != ODL_OK)
             return rc;
     }
-    if (gb)
+    if (gb && !side_bias)
     {
         rc = odl::sum_nchw_channels_launch(gy, N, OC, g.OH * g.OW, gb, red_ws, p.red_bytes, st);
         if (rc != ODL_OK)
@@ -1346,7 +1407,7 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
         if (p.dgrad_small)
             rc = odl::conv_small_dgrad(gy, w, gx, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, wp_ws, p.wp_bytes, st);
         else if (p.dgrad_patch)
-            rc = odl::conv_patch_dgrad(gy, w, gx, N, C, H, W, OC, wp_ws, p.wp_bytes, st);
+            rc = odl::conv_patch_dgrad(gy, w, gx, N, C, H, W, OC, wp_ws, p.wp_bytes, st, side_pack);
         else if (p.dgrad_implicit)
             rc = odl::conv_implicit_dgrad(gy, w, gx, N, C, H, W, OC, KH, KW, PH, PW, g.OH, g.OW, wp_ws, p.wp_bytes, st);
         else

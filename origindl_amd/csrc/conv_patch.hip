@@ -10,6 +10,7 @@
 //   input gradient  gx[n,c,h,w]  = sum_{oc,t} gy2d[pix(n,h+dy,w+dx)][oc] * w[oc,c,8-t]
 // where gy2d is the gradient buffer read as a row-major [N*OH*OW, OC] matrix exactly as it lies, the reference's
 // reading (conv2d.cpp:548) — for this kernel a channel-minor source.
+#include "conv_side.h"
 #include "odl_common.h"
 
 #include <atomic>
@@ -54,20 +55,9 @@ struct PatchGeom
 };
 
 // wp[(m*nslab + slab)*144 + tap*16 + cc]: the zero-padded filter copy the kernel stages with 16-byte copies
-__global__ void conv_patch_pack_kernel(const float *__restrict__ w, float *__restrict__ wp, int Cin, int M, int Mpad,
-                                       int flipped)
+__global__ void conv_patch_pack_kernel(const odl::SidePack p)
 {
-    const int total = Cin * 9 * Mpad, nslab = Cin / kSlab;
-    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x)
-    {
-        const int rem = idx % (9 * kSlab), rest = idx / (9 * kSlab);
-        const int slab = rest % nslab, m = rest / nslab;
-        const int tap = rem / kSlab, ch = slab * kSlab + rem % kSlab;
-        float v = 0.f;
-        if (m < M)
-            v = flipped ? w[((int64_t)ch * M + m) * 9 + 8 - tap] : w[((int64_t)m * Cin + ch) * 9 + tap];
-        wp[idx] = v;
-    }
+    odl::side_pack(p, blockIdx.x, gridDim.x);
 }
 
 template <int BM, bool CH_MINOR>
@@ -506,8 +496,10 @@ TailPlan plan_tail_for(int64_t N, int64_t Cin, int64_t H, int64_t W, int64_t M, 
     return plan_tail(odl::ceil_div(N * H * W, kPixTile) * mtiles, (int)(Cin / kSlab), bm, ch_minor, lds_bytes(bm, plane));
 }
 
+// packed: the filter copy at the head of the workspace has been made already (by the caller's own launch of side_pack)
 int launch(const float *src, const float *w, const float *bias, float *dst, int64_t N, int64_t Cin, int64_t H, int64_t W,
-           int64_t M, bool ch_minor, int act, void *workspace, size_t workspace_bytes, hipStream_t st, const char *who)
+           int64_t M, bool ch_minor, int act, void *workspace, size_t workspace_bytes, hipStream_t st, const char *who,
+           bool packed = false)
 {
     const size_t need = packed_bytes(Cin, M);
     if (!workspace || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
@@ -529,10 +521,13 @@ int launch(const float *src, const float *w, const float *bias, float *dst, int6
     g.by_hw = odl::make_fastdiv((unsigned)(H * W)), g.by_pw = odl::make_fastdiv((unsigned)g.PW);
     float *wp = static_cast<float *>(workspace);
     g.wp = wp;
-    const int total = g.Cin * 9 * g.Mpad;
-    hipLaunchKernelGGL(conv_patch_pack_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, w, wp, g.Cin,
-                       g.M, g.Mpad, ch_minor ? 1 : 0);
-    ODL_LAUNCH_CHECK();
+    if (!packed)
+    {
+        const int total = g.Cin * 9 * g.Mpad;
+        hipLaunchKernelGGL(conv_patch_pack_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st,
+                           odl::SidePack{w, wp, g.Cin, g.M, g.Mpad, ch_minor ? 1 : 0});
+        ODL_LAUNCH_CHECK();
+    }
     const size_t lds = lds_bytes(bm, g.plane);
     ODL_HIP_CHECK(allow_lds(bm, ch_minor));
     // the tiles of a short last round go out as runs of channel slabs (when the workspace has room for their sums)
@@ -608,9 +603,16 @@ size_t conv_patch_dgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, in
 }
 
 int conv_patch_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
-                     void *workspace, size_t workspace_bytes, hipStream_t st)
+                     void *workspace, size_t workspace_bytes, hipStream_t st, bool packed)
 {
-    return launch(gy, w, nullptr, gx, N, OC, H, W, C, true, 0, workspace, workspace_bytes, st, "conv2d_backward");
+    return launch(gy, w, nullptr, gx, N, OC, H, W, C, true, 0, workspace, workspace_bytes, st, "conv2d_backward", packed);
+}
+
+// the filter copy conv_patch_dgrad stages from, as a job for a launch of the caller's (then `packed` above)
+SidePack conv_patch_dgrad_pack(const float *w, int64_t C, int64_t OC, void *workspace)
+{
+    const int bm_pad = tile_bm(C);
+    return SidePack{w, static_cast<float *>(workspace), (int)OC, (int)C, (int)(ceil_div(C, bm_pad) * bm_pad), 1};
 }
 }  // namespace odl
 
