@@ -336,6 +336,18 @@ def train_steps(steps, warmup, with_cpu):
                                       "loss_last_step": float(losses[1]), "loss_eval_mode": float(losses[2])}
     rc = h.odl_host_cnn_bn_bench(256, steps, warmup, 1, ms, losses)
     out["cnn_batchnorm_b256_adam"].update({"graph_replay_rc": rc, "graph_replay_ms_per_step": float(ms[0])})
+    # the same two steps run by the REFERENCE's own Tensor / Operator / nn / optim object code over binding/ (its
+    # op-by-op graph: no fused layers, no recorded step; built only where the reference checkout was present)
+    if os.path.exists(ol.BIND_DRIVER_SO):
+        bd = ol.binding_driver()
+        rc = bd.odl_bind_mlp_bench(512, 784, 1000, 10, steps, warmup, ms, loss)
+        out["mlp_512x784x1000x10_adam"].update({"reference_classes_over_binding_rc": rc,
+                                                "reference_classes_over_binding_ms_per_step": float(ms[0]),
+                                                "reference_classes_over_binding_loss_step_1": float(loss[0])})
+        rc = bd.odl_bind_cnn_bench(256, steps, warmup, ms, loss)
+        out["cnn_b256_sgd"].update({"reference_classes_over_binding_rc": rc,
+                                    "reference_classes_over_binding_ms_per_step": float(ms[0]),
+                                    "reference_classes_over_binding_loss_step_1": float(loss[0])})
     out["yolov5n_forward_4x3x320x320"] = yolo_forward(h, ol.ref() if with_cpu and ol.have_ref() else None, steps)
     if with_cpu and ol.have_ref():
         r = ol.ref()

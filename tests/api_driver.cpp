@@ -74,7 +74,9 @@ namespace F = origin::functional;
 
 namespace
 {
-#ifdef DRV_ON_DEVICE
+#if defined(DRV_ON_DEVICE) || defined(DRV_DEVICE_TENSORS)
+// (DRV_DEVICE_TENSORS alone: tensors on the device, but only calls the reference's own API has - the build against the
+// reference's headers and objects with the gfx950 binding underneath)
 const Device kDev(DeviceType::kCUDA, 0);
 #else
 const Device kDev(DeviceType::kCPU, 0);
@@ -122,7 +124,9 @@ void out(const Tensor &t, float *dst)
 
 void out(const origin::Mat &m, float *dst)
 {
-    auto v = static_cast<const OriginMat &>(m).to_vector<float>();
+    // (the reference's OriginMat::to_vector<T>() reads the storage in place: a device Mat comes to the host first)
+    const auto host = m.device().type() == DeviceType::kCPU ? nullptr : m.to_device(Device(DeviceType::kCPU, 0));
+    auto v = static_cast<const OriginMat &>(host ? *host : m).to_vector<float>();
     std::memcpy(dst, v.data(), v.size() * sizeof(float));
 }
 

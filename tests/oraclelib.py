@@ -251,6 +251,29 @@ def host_driver(cpu=False):
     return _host[key]
 
 
+BIND_DRIVER_SO = os.path.join(ORACLE_DIR, "_ref", "libodl_bind_driver.so")
+_bind = None
+
+
+def binding_driver():
+    """tests/api_driver.cpp compiled against the REFERENCE's own headers and linked to the reference's own Tensor /
+    Operator / nn / optim objects, with the gfx950 binding (binding/src) underneath instead of the reference's device
+    dispatcher and memory layer; tensors on the device (odl_bind_*). Built by `make -C oracle ref-binding`."""
+    global _bind
+    if _bind is None:
+        sigs = {k.replace("odl_ref_", "odl_bind_"): v for k, v in _REF_SIGS.items()}
+        lib = _Lib(BIND_DRIVER_SO, sigs)
+        here, scratch = os.getcwd(), tempfile.mkdtemp(prefix="odl_bind_log_")  # (the reference's logger, as in ref())
+        os.chdir(scratch)
+        try:
+            lib.odl_bind_ping()
+        finally:
+            os.chdir(here)
+        atexit.register(shutil.rmtree, scratch, True)
+        _bind = lib
+    return _bind
+
+
 def ptr_arr(arrays):
     """Host array of the data addresses of `arrays` (for entry points that take a pointer table)."""
     return np.asarray([a.ctypes.data for a in arrays], dtype=np.uint64)
