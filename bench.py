@@ -318,6 +318,10 @@ def train_steps(steps, warmup, with_cpu):
     rc = h.odl_host_mlp_bench(512, 784, 1000, 10, steps, warmup, ms, loss)
     out["mlp_512x784x1000x10_adam"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss_step_1": float(loss[0]),
                                        "gemm_flop_per_step": 6.0 * 512 * (784 * 1000 + 1000 * 10)}
+    # the same step with the network as one nn::MLP object, the way the reference's own training loop builds it
+    rc = h.odl_host_mlp_model_bench(512, 784, 1000, 10, steps, warmup, 0, ms, loss)
+    out["mlp_512x784x1000x10_adam"].update({"nn_MLP_object_rc": rc, "nn_MLP_object_ms_per_step": float(ms[0]),
+                                            "nn_MLP_object_loss_step_1": float(loss[0])})
     rc = h.odl_host_cnn_bench(256, steps, warmup, ms, loss)
     out["cnn_b256_sgd"] = {"rc": rc, "ms_per_step": float(ms[0]), "loss_step_1": float(loss[0])}
     # the same steps recorded once into a HIP graph and replayed (one submission per step instead of ~50 launches);

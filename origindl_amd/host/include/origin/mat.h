@@ -72,6 +72,18 @@ public:
         std::memcpy(dst, host_copy_, n);
         return true;
     }
+    // The least and greatest element of an integer buffer that was uploaded from the host (found by a scan of the host
+    // data on its way up): whoever needs to know whether class labels lie in range then needs no trip to the device.
+    // Every in-place writer of the buffer calls forget_int_range().
+    void set_int_range(int64_t lo, int64_t hi) const { int_lo_ = lo, int_hi_ = hi, int_range_valid_ = true; }
+    void forget_int_range() const { int_range_valid_ = false; }
+    bool int_range(int64_t *lo, int64_t *hi) const
+    {
+        if (!int_range_valid_)
+            return false;
+        *lo = int_lo_, *hi = int_hi_;
+        return true;
+    }
     // Pinned host words that the kernel which fills this buffer also writes (the loss and its bad-label flag): once the
     // device has been synchronised the host reads them there, with no copy queued. Set after the data() call that handed
     // the buffer to that kernel; like the host copy above it stops being trusted at the next data() call. A kernel
@@ -103,6 +115,8 @@ private:
     mutable int fill_dtype_ = 0;
     mutable int64_t fill_n_ = 0;
     mutable unsigned char fill_element_[8] = {0};
+    mutable std::atomic<bool> int_range_valid_{false};
+    mutable int64_t int_lo_ = 0, int_hi_ = 0;
     mutable void *mirror_ = nullptr, *mirror_stream_ = nullptr;
     mutable std::atomic<bool> mirror_valid_{false};
     mutable bool mirror_recorded_ = false;

@@ -193,6 +193,7 @@ public:
 private:
     std::vector<Linear *> layers_;
     std::function<Tensor(const Tensor &)> activation_;
+    bool default_relu_ = false;  // no activation was given: the ReLU between the layers rides in their epilogues
 };
 }  // namespace nn
 

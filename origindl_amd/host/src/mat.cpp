@@ -297,6 +297,7 @@ std::unique_ptr<Mat> binary(int op, const char *who, const OriginMat &a, const M
     else if (dst->dtype() != x.dtype())
         THROW_INVALID_ARG("Output tensor mismatch. Expected dtype={}, got dtype={}", dtype_to_string(x.dtype()),
                           dtype_to_string(dst->dtype()));
+    dst->storage()->forget_int_range();
     check(odl_hip_binary_dtype(op, code(x.dtype()), x.storage()->data(), (int64_t)x.elements(), y.storage()->data(),
                                (int64_t)y.elements(), dst->storage()->data(), cur()));
     return fresh;
@@ -316,6 +317,7 @@ std::unique_ptr<Mat> unary(int op, const char *who, const OriginMat &a, OriginMa
         fresh = new_like(x, x.shape(), x.dtype());
         dst   = fresh.get();
     }
+    dst->storage()->forget_int_range();
     check(odl_hip_unary_dtype(op, code(x.dtype()), x.storage()->data(), (int64_t)x.elements(), dst->storage()->data(),
                               cur()));
     return fresh;
@@ -539,6 +541,20 @@ double load_as(const void *src, DataType dt, size_t i)
     }
 }
 
+// class labels come up from the host as int32 / int64: their range is noted on the way
+void note_int_range(const Storage &st, const void *host, DataType dt, size_t n)
+{
+    if ((dt != DataType::kInt32 && dt != DataType::kInt64) || n == 0)
+        return;
+    int64_t lo = INT64_MAX, hi = INT64_MIN;
+    for (size_t i = 0; i < n; ++i)
+    {
+        const int64_t v = dt == DataType::kInt64 ? static_cast<const int64_t *>(host)[i] : static_cast<const int32_t *>(host)[i];
+        lo = v < lo ? v : lo, hi = v > hi ? v : hi;
+    }
+    st.set_int_range(lo, hi);
+}
+
 std::unique_ptr<Mat> upload_new(const void *host, DataType dt, const Shape &shape, Device dev)
 {
     auto m = std::make_unique<OriginMat>(shape, dt, dev);
@@ -551,6 +567,7 @@ std::unique_ptr<Mat> upload_new(const void *host, DataType dt, const Shape &shap
     {
         no_capture("host-to-device copy");
         check(odl_hip_memcpy_h2d(m->data_ptr(), host, bytes, cur()));
+        note_int_range(*m->storage(), host, dt, shape.elements());
     }
     return m;
 }
@@ -763,6 +780,7 @@ void OriginMat::index_put(std::initializer_list<size_t> indices, const Scalar &v
     }
     else
         store_as(element, dtype_, &v, 1);
+    storage_->forget_int_range();
     char *dst = static_cast<char *>(storage_->data()) + offset * width;
     if (storage_->device_type() == DeviceType::kCPU)
         std::memcpy(dst, element, width);
@@ -796,7 +814,10 @@ std::unique_ptr<Mat> OriginMat::to_device(Device dev) const
 {
     if (dev == device())
         return std::make_unique<OriginMat>(*this);
-    return std::make_unique<OriginMat>(storage_->to_device(dev.type(), dev.index()), shape_, dtype_);
+    auto moved = storage_->to_device(dev.type(), dev.index());
+    if (storage_->device_type() == DeviceType::kCPU && dev.type() == DeviceType::kCUDA)
+        note_int_range(*moved, storage_->data(), dtype_, elements());
+    return std::make_unique<OriginMat>(std::move(moved), shape_, dtype_);
 }
 
 void OriginMat::print(const std::string &desc) const
@@ -1716,6 +1737,15 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) 
 
 std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target) const
 {
+    // labels that came up from the host carry their range: an out-of-range label is reported without asking the device,
+    // and a batch in range needs no check at all (the step then has no stop in its middle)
+    int64_t lo = 0, hi = 0;
+    if (as_origin(target).storage()->int_range(&lo, &hi))
+    {
+        if (lo < 0 || hi >= (int64_t)shape_[1])
+            THROW_INVALID_ARG("gather: index out of range [0, {})", shape_[1]);
+        return softmax_cross_entropy_device(target);
+    }
     auto loss = softmax_cross_entropy_device(target);
     // the loss word and the bad-label flag behind it come back together (this synchronises, as the reference's host-side
     // divide does); the loss itself stays on the device for the operators that follow
@@ -1787,6 +1817,8 @@ void OriginMat::upload(const void *host, size_t bytes)
     no_capture("host-to-device copy");
     // queued behind everything on the current stream that still reads the old contents
     check(odl_hip_memcpy_h2d(storage_->data(), host, bytes, cur()));
+    storage_->forget_int_range();
+    note_int_range(*storage_, host, dtype_, elements());
 }
 
 void OriginMat::adam_step_inplace(const Mat &grad, Mat &m, Mat &v, float beta1, float beta2, const float *device_scales,
@@ -1808,6 +1840,7 @@ void OriginMat::copy_from(const Mat &src)
     const OriginMat &o = as_origin(src);
     if (o.shape() != shape_ || o.dtype() != dtype_ || o.device() != device())
         THROW_INVALID_ARG("copy_from: shape, dtype and device must match");
+    storage_->forget_int_range();
     if (device().type() == DeviceType::kCPU)
         std::memcpy(storage_->data(), o.storage()->data(), elements() * dtype_size(dtype_));
     else

@@ -367,7 +367,8 @@ MaxPool2d::MaxPool2d(std::pair<int, int> kernel_size, std::pair<int, int> stride
 MaxPool2d::MaxPool2d(int kernel_size, int stride, int pad) : MaxPool2d(pair(kernel_size), pair(stride), pair(pad)) {}
 
 MLP::MLP(const std::vector<int> &sizes, std::function<Tensor(const Tensor &)> activation)
-    : activation_(activation ? std::move(activation) : [](const Tensor &x) { return functional::relu(x); })
+    : activation_(activation ? std::move(activation) : [](const Tensor &x) { return functional::relu(x); }),
+      default_relu_(!activation)
 {
     if (sizes.size() < 2)
         THROW_INVALID_ARG("MLP needs at least an input and an output size");
@@ -384,9 +385,16 @@ Tensor MLP::forward(const Tensor &input)
     Tensor x = input;
     for (size_t i = 0; i < layers_.size(); ++i)
     {
-        x = layers_[i]->forward(x);
-        if (i + 1 < layers_.size())
-            x = activation_(x);
+        // src/nn/models/mlp.cpp:43-61: every layer but the last is followed by the activation. With the default ReLU
+        // the pair runs as one operator, as a Linear followed by a ReLU inside a Sequential does (the same bits).
+        if (i + 1 < layers_.size() && default_relu_)
+            x = layers_[i]->forward_relu(x);
+        else
+        {
+            x = layers_[i]->forward(x);
+            if (i + 1 < layers_.size())
+                x = activation_(x);
+        }
     }
     return x;
 }

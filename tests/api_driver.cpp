@@ -1206,6 +1206,32 @@ int mlp_bench_impl(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int w
     });
 }
 
+// The same step with the network built as the reference's own loop builds it (tests/example/mnist/mlp_mnist.cpp:227):
+// one nn::MLP({D, Hd, C}) object instead of a Sequential of layers. Same seed, same draws in the same order, so the
+// first step's loss is the Sequential's.
+int mlp_model_bench_impl(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, int graph_mode,
+                         float *ms_per_step, float *loss)
+{
+    return guarded([&] {
+        std::mt19937 gen(1234);
+        nn::MLP model({(int)D, (int)Hd, (int)C});
+        Adam opt(model, 1e-3f, 0.9f, 0.999f, 1e-8f);
+        opt.register_hook(WeightDecay(1e-4f).hook());
+        auto named = model.named_parameters("");
+        *named.at("layer_0.weight") = kaiming_uniform(gen, Shape{(size_t)D, (size_t)Hd}, (size_t)D);
+        *named.at("layer_0.bias")   = zeros_param(Shape{1, (size_t)Hd});
+        *named.at("layer_1.weight") = kaiming_uniform(gen, Shape{(size_t)Hd, (size_t)C}, (size_t)Hd);
+        *named.at("layer_1.bias")   = zeros_param(Shape{1, (size_t)C});
+        auto X = Tensor(uniform_vec(gen, (size_t)(N * D), 0.0f, 1.0f), Shape{(size_t)N, (size_t)D},
+                        dtype(DataType::kFloat32).device(kDev));
+        std::vector<int64_t> tv((size_t)N);
+        for (auto &e : tv)
+            e = (int64_t)(gen() % (uint32_t)C);
+        auto T = Tensor(tv, Shape{(size_t)N}, dtype(DataType::kInt64).device(kDev));
+        run_timed(model, opt, X, T, steps, warmup, graph_mode, ms_per_step, loss);
+    });
+}
+
 int cnn_bench_impl(int64_t N, int steps, int warmup, int graph_mode, float *ms_per_step, float *loss)
 {
     return guarded([&] {
@@ -1371,6 +1397,13 @@ int DRV(pending_fill_semantics)(int64_t n, double *out)
 int DRV(mlp_bench)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, float *ms_per_step, float *loss)
 {
     return mlp_bench_impl(N, D, Hd, C, steps, warmup, 0, ms_per_step, loss);
+}
+
+// graph_mode: 0 ordinary steps; 1 / 2: a recorded step replayed (device build of this repository's host layer only)
+int DRV(mlp_model_bench)(int64_t N, int64_t D, int64_t Hd, int64_t C, int steps, int warmup, int graph_mode,
+                         float *ms_per_step, float *loss)
+{
+    return mlp_model_bench_impl(N, D, Hd, C, steps, warmup, graph_mode, ms_per_step, loss);
 }
 
 int DRV(cnn_bench)(int64_t N, int steps, int warmup, float *ms_per_step, float *loss)

@@ -96,6 +96,7 @@ _REF_SIGS = {
     "odl_ref_cnn_train": "ppillllll" + "p" * 8 + "f" + "p" + "p" * 8 + "p>i",
     "odl_ref_mlp_bench": "lllliipp>i",
     "odl_ref_cnn_bench": "liipp>i",
+    "odl_ref_mlp_model_bench": "lllliiipp>i",
 }
 
 
