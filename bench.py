@@ -381,10 +381,28 @@ def yolo_forward(h, ref, reps):
             t0 = time.perf_counter()
             rc = getattr(drv, name)(param.encode(), binp.encode(), x, batch, 3, 320, 320, n, o, o.size, oshape, nd, ms)
             return rc, float(ms[0]), time.perf_counter() - t0, o
-        rc, ms, _, o = run(h, "odl_host_pnnx_forward", 4, max(3, reps) + 1)
+        n = max(10, reps) + 1
+        rc, ms, _, o = run(h, "odl_host_pnnx_forward", 4, n)
         gflop = pnnx_synth.flops(4, 320) / 1e9
         res.update({"rc": rc, "ms_per_forward": ms, "conv_gflop": gflop, "tflops": gflop / ms if ms > 0 else None,
                     "output_shape": list(o.shape), "output_mean": float(o.mean())})
+        # the same forward recorded into a graph and replayed, and how many launches it holds
+        nodes = np.zeros(1, np.int64)
+        rc, ms_g, _, og = run(h, "odl_host_pnnx_forward_graph", 4, n)
+        h.odl_host_pnnx_last_graph_nodes(nodes)
+        res.update({"graph_replay_rc": rc, "graph_replay_ms_per_forward": ms_g, "launches_per_forward": int(nodes[0]),
+                    "graph_replay_equals_eager": bool(np.array_equal(o, og))})
+        # every node on its own, as the reference's runner goes through the graph (no add / concatenation / pool chain
+        # folded into its producer): same kernels for the convolutions, same floats
+        h.odl_host_pnnx_set_fusion(0)
+        try:
+            rc, ms_p, _, op = run(h, "odl_host_pnnx_forward", 4, n)
+            rc2, _, _, _ = run(h, "odl_host_pnnx_forward_graph", 4, 2)
+            h.odl_host_pnnx_last_graph_nodes(nodes)
+        finally:
+            h.odl_host_pnnx_set_fusion(1)
+        res.update({"node_by_node_rc": rc, "node_by_node_ms_per_forward": ms_p, "node_by_node_launches_per_forward": int(nodes[0]),
+                    "node_by_node_equals_folded": bool(np.array_equal(o, op))})
         if ref is not None:
             rc, _, wall, _ = run(ref, "odl_ref_pnnx_forward", 1, 1)
             res["cpu_reference_ms_per_forward_batch_1"] = wall * 1e3

@@ -75,6 +75,8 @@ int odl_hip_host_alloc(void **ptr, size_t bytes);
 int odl_hip_host_free(void *ptr);
 int odl_hip_graph_capture_begin(void *stream);
 int odl_hip_graph_capture_end(void *stream, void **graph_exec);
+/* how many nodes (launches) the graph that this thread ended last holds */
+int odl_hip_graph_last_node_count(int64_t *nodes);
 /* gives up a capture (after an error in the middle of the step being recorded): the stream leaves capture mode,
  * whatever was recorded is discarded, the stream can be used and captured again. A no-op on a stream that is not
  * capturing. */
@@ -136,14 +138,16 @@ int odl_hip_conv2d_act(const float *x, const float *w, const float *b, int64_t N
                        int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int activation, float *y,
                        void *workspace, size_t workspace_bytes, void *stream);
 /* The same forward for weights that do not change between calls (inference): some shapes read the filter in another
- * order, [OC][tap][C], and odl_hip_conv2d / _act write that copy into the workspace on every call. A caller that keeps
- * its weights can make the copy once — packed_weights_bytes says how large it is for a shape (0: this shape reads the
- * filter as it lies and `packed` is ignored), pack_weights fills it — and pass it to conv2d_act_packed, which then
- * skips the copy. packed = NULL is odl_hip_conv2d_act. No counterpart in the reference (its runner re-uploads the
+ * order ([OC][tap][C], or blocks of 32 output channels x 8 channels per tap for the small-problem kernel), and
+ * odl_hip_conv2d / _act write that copy into the workspace on every call. A caller that keeps its weights can make
+ * the copy once — packed_weights_bytes says how large it is for a shape (0: this shape reads the filter as it lies and
+ * `packed` is ignored), pack_weights fills it in the order that shape's kernel reads — and pass it to
+ * conv2d_act_packed, which then skips the copy. packed = NULL is odl_hip_conv2d_act. No counterpart in the reference (its runner re-uploads the
  * weights on every forward, src/pnnx/pnnx_graph.cpp:341-405). */
 size_t odl_hip_conv2d_packed_weights_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
                                            int SW, int PH, int PW);
-int odl_hip_conv2d_pack_weights(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, void *stream);
+int odl_hip_conv2d_pack_weights(const float *w, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                                int SW, int PH, int PW, float *packed, void *stream);
 int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packed, const float *b, int64_t N, int64_t C,
                               int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW,
                               int activation, float *y, void *workspace, size_t workspace_bytes, void *stream);
@@ -165,6 +169,30 @@ size_t odl_hip_conv2d_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, 
  * tests can send small shapes through the LDS-patch kernel. The choice enters the workspace sizes: never change it
  * between a *_workspace_bytes query and the call the query was made for. No counterpart in the reference. */
 int odl_hip_set_conv_patch_min_workgroups(int64_t min_workgroups);
+/* A convolution node of the reference's graph runner together with the nodes that follow it
+ * (src/pnnx/pnnx_graph.cpp:286-528 runs nn.Conv2d, nn.SiLU, pnnx.Expression add and torch.cat one by one;
+ * src/mat/origin/cpu/shape/cat.cpp:81-123 then copies every input of the concatenation):
+ *   y[n, oc] = residual[n, oc] + act(conv(x)[n, oc] + b[oc])
+ * where x, residual and y are NCHW tensors whose images lie x_image_stride / residual_image_stride / y_image_stride
+ * floats apart (0: dense), so that each may be a run of channels inside a wider tensor: a convolution writes straight
+ * into its part of a concatenation's destination and reads an input that lives in one. residual may be NULL.
+ * packed: the filter as odl_hip_conv2d_pack_weights lays it out for this shape (required). Covers small problems only (channels a
+ * multiple of 8, square stride and padding, up to about 1.6 GFLOP): odl_hip_conv2d_fused_ok answers 1 for a shape
+ * this entry point takes, and a shape it does not take is refused with ODL_ERR_INVALID_ARG — the caller then runs
+ * the nodes one by one. The sums are formed in another order than odl_hip_conv2d's large-problem kernels form them
+ * (float32 rounding differs in the last bits); odl_hip_conv2d itself sends the shapes covered here through the
+ * same kernel. */
+int odl_hip_conv2d_fused_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH,
+                            int PW);
+int odl_hip_conv2d_fused(const float *x, int64_t x_image_stride, const float *packed, const float *b, int64_t N, int64_t C,
+                         int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int activation,
+                         const float *residual, int64_t residual_image_stride, float *y, int64_t y_image_stride,
+                         void *stream);
+/* Measurement switches, for the whole process (same caveat as above: never between a query and its call):
+ * set_conv_direct(0) sends the small problems to the tiled kernels again; set_conv_direct_plan(k_shares, pixel_tiles)
+ * fixes how a workgroup of the small-problem kernel is cut (0, 0: its own rule). No counterpart in the reference. */
+int odl_hip_set_conv_direct(int enabled);
+int odl_hip_set_conv_direct_plan(int k_shares, int pixel_tiles);
 
 /* ------------------------------------------------------------------ reductions / broadcast ---------- */
 /* Mat::sum(axis) seen as [outer, axis, inner] -> [outer, inner]
@@ -334,6 +362,27 @@ int odl_hip_yolo_detect_forward(const float *x, const float *conv_w, const float
                                 int64_t anchor_W, int64_t N, int64_t C, int64_t H, int64_t W, float stride, int num_anchors,
                                 int num_classes, float *out, void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_yolo_detect_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int num_anchors, int num_classes);
+
+/* Operators of the detector's graph for tensors that are runs of channels inside a wider NCHW tensor — the inputs of a
+ * torch.cat written where the concatenation would copy them (src/mat/origin/cpu/shape/cat.cpp:81-123), and read from
+ * there by the nodes that follow. An image stride is the distance in floats from one image of the view to the next
+ * (0: dense). Values are those of the dense entry points. No counterpart in the reference, whose runner materialises
+ * every node's output (src/pnnx/pnnx_graph.cpp:286-528).
+ *  upsample_nearest_view: odl_hip_upsample_nearest; OW and the output stride multiples of 4, y 16-byte aligned.
+ *  max_pool2d_chain: `count` K x K / stride 1 / padding K/2 max pools applied one after the other (a detector's SPPF
+ *    block); stage j's result goes to channels [(j-1)*C, j*C) of y. One launch, the plane stays in LDS (H*W <= 8192).
+ *  copy_images: dst[n][j] = src[n][j] for j < count — one input of a concatenation, or a view made dense.
+ *  yolo_decode: the second half of odl_hip_yolo_detect_forward (sigmoid + box decoding of conv[N, A*(classes+5), H, W])
+ *    with the stage's rows written out_image_stride floats apart, i.e. straight into the concatenation of the stages. */
+int odl_hip_upsample_nearest_view(const float *x, int64_t x_image_stride, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
+                                  int64_t OW, int scale_h, int scale_w, float *y, int64_t y_image_stride, void *stream);
+int odl_hip_max_pool2d_chain(const float *x, int64_t x_image_stride, int64_t N, int64_t C, int64_t H, int64_t W, int K,
+                             int count, float *y, int64_t y_image_stride, void *stream);
+int odl_hip_copy_images(const float *src, int64_t src_image_stride, float *dst, int64_t dst_image_stride, int64_t N,
+                        int64_t count, void *stream);
+int odl_hip_yolo_decode(const float *conv, const float *grid, int64_t grid_elems, const float *anchor_grid, int64_t anchor_elems,
+                        int64_t anchor_H, int64_t anchor_W, int64_t N, int64_t H, int64_t W, float stride, int num_anchors,
+                        int num_classes, float *out, int64_t out_image_stride, void *stream);
 
 /* Mat::batch_norm_forward / Mat::batch_norm (mat.h:603-631; src/mat/origin/cpu/normalization/batch_norm.cpp:31-258)
  * over x[N, C, P]: P = H*W for num_dims 4, P = 1 for num_dims 2. training != 0: per-channel mean and biased variance

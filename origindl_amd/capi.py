@@ -191,10 +191,11 @@ def conv2d_pack_weights(x_shape, w, stride=1, pad=0):
     N, C, H, W = (int(d) for d in x_shape)
     OC, _, KH, KW = w.shape
     (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
-    if lib().query("odl_hip_conv2d_packed_weights_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW) == 0:
+    nbytes = lib().query("odl_hip_conv2d_packed_weights_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW)
+    if nbytes == 0:
         return None
-    packed = _empty(w.shape)
-    lib().call("odl_hip_conv2d_pack_weights", _p(w), C, OC, KH, KW, _p(packed), _stream())
+    packed = _empty((nbytes // 4,))  # rounded up to whole tiles of output channels for some kernels
+    lib().call("odl_hip_conv2d_pack_weights", _p(w), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, _p(packed), _stream())
     return packed
 
 
@@ -525,6 +526,84 @@ def yolo_detect_forward(x, conv_w, conv_b, grid, anchor_grid, stride, num_anchor
                anchor_grid.numel(), aH, aW, N, C, H, W, float(stride), num_anchors, num_classes, _p(out), _p(ws), nb,
                _stream())
     return out
+
+
+# ------------------------------------------------------------------ runs of channels inside wider NCHW tensors
+def _run(t, name):
+    """A 4-D float32 device tensor that is dense, or a run of channels of one (`buf[:, c0:c1]`): -> its image stride."""
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == _f32 and t.dim() == 4):
+        raise OdlInvalidArgument("%s must be a 4D float32 device tensor (or a run of channels of one)" % name)
+    N, C, H, W = t.shape
+    s = t.stride()
+    if (s[1], s[2], s[3]) != (H * W, W, 1) or (N > 1 and s[0] < C * H * W):
+        raise OdlInvalidArgument("%s must be NCHW with only the images spaced apart, got strides %s" % (name, tuple(s)))
+    return int(s[0]) if N > 1 else C * H * W
+
+
+def conv2d_fused_ok(x_shape, w_shape, stride=1, pad=0):
+    N, C, H, W = (int(d) for d in x_shape)
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    return lib().query("odl_hip_conv2d_fused_ok", N, C, H, W, int(w_shape[0]), int(w_shape[2]), int(w_shape[3]), SH, SW, PH, PW) == 1
+
+
+def conv2d_fused(x, w_shape, packed, b, y, stride=1, pad=0, activation=None, residual=None):
+    """y = residual + act(conv(x, W) + b) where x, y and residual may each be a run of channels of a wider tensor
+    (a torch view `buf[:, c0:c1]`); packed = conv2d_pack_weights(x.shape, W, ...). The nodes nn.Conv2d, nn.SiLU,
+    pnnx.Expression add and the copy of torch.cat of the reference's graph runner (src/pnnx/pnnx_graph.cpp:286-528)."""
+    xs, ys = _run(x, "x"), _run(y, "y")
+    rs = _run(residual, "residual") if residual is not None else 0
+    N, C, H, W = x.shape
+    OC, _, KH, KW = (int(d) for d in w_shape)
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    if tuple(y.shape) != (N, OC, OH, OW) or (residual is not None and tuple(residual.shape) != tuple(y.shape)):
+        raise OdlInvalidArgument("conv2d_fused: y (and residual) must be [%d, %d, %d, %d]" % (N, OC, OH, OW))
+    act = -1 if activation is None else _UN[activation]
+    lib().call("odl_hip_conv2d_fused", _p(x), xs, _p(packed), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, act,
+               _p(residual), rs, _p(y), ys, _stream())
+    return y
+
+
+def upsample_view(x, y, scale):
+    sh, sw = _pair(scale)
+    xs, ys = _run(x, "x"), _run(y, "y")
+    N, C, H, W = x.shape
+    lib().call("odl_hip_upsample_nearest_view", _p(x), xs, N, C, H, W, y.shape[2], y.shape[3], sh, sw, _p(y), ys, _stream())
+    return y
+
+
+def max_pool2d_chain(x, K, count, y):
+    """y[:, (j-1)*C : j*C] = the K x K / stride 1 / padding K/2 max pool applied j times to x, j = 1..count."""
+    xs, ys = _run(x, "x"), _run(y, "y")
+    N, C, H, W = x.shape
+    if tuple(y.shape) != (N, count * C, H, W):
+        raise OdlInvalidArgument("max_pool2d_chain: y must hold %d stages of x's shape" % count)
+    lib().call("odl_hip_max_pool2d_chain", _p(x), xs, N, C, H, W, K, count, _p(y), ys, _stream())
+    return y
+
+
+def copy_images(src, dst):
+    ss, ds = _run(src, "src"), _run(dst, "dst")
+    if tuple(src.shape) != tuple(dst.shape):
+        raise OdlInvalidArgument("copy_images: shapes differ")
+    N, C, H, W = src.shape
+    lib().call("odl_hip_copy_images", _p(src), ss, _p(dst), ds, N, C * H * W, _stream())
+    return dst
+
+
+def yolo_decode(conv, grid, anchor_grid, stride, num_anchors, num_classes, out_rows):
+    """The decoding half of yolo_detect_forward: conv[N, A*(classes+5), H, W] -> out_rows, the stage's rows
+    `out[:, r0 : r0 + A*H*W, :]` of the tensor that concatenates the stages."""
+    _chk(conv, "conv"), _chk(grid, "grid"), _chk(anchor_grid, "anchor_grid")
+    N, _, H, W = conv.shape
+    CI = num_classes + 5
+    if tuple(out_rows.shape) != (N, num_anchors * H * W, CI) or out_rows.stride()[1:] != (CI, 1):
+        raise OdlInvalidArgument("yolo_decode: out_rows must be [%d, %d, %d] rows of a dense tensor" % (N, num_anchors * H * W, CI))
+    aH = anchor_grid.shape[2] if anchor_grid.dim() >= 3 else H
+    aW = anchor_grid.shape[3] if anchor_grid.dim() >= 4 else W
+    lib().call("odl_hip_yolo_decode", _p(conv), _p(grid), grid.numel(), _p(anchor_grid), anchor_grid.numel(), aH, aW, N, H, W,
+               float(stride), num_anchors, num_classes, _p(out_rows), int(out_rows.stride()[0]) if N > 1 else 0, _stream())
+    return out_rows
 
 
 def _bn_dims(x, who):

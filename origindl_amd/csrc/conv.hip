@@ -15,6 +15,7 @@
 #include "odl_common.h"
 
 #include <algorithm>
+#include <atomic>
 
 namespace odl
 {
@@ -84,6 +85,15 @@ int conv_wgrad_rows(const float *gy, const float *x, float *gw, int64_t N, int64
 int sum_nchw_channels_launch(const float *gy, int64_t N, int64_t OC, int64_t P, float *gb, void *workspace,
                              size_t workspace_bytes, hipStream_t st);
 size_t sum_nchw_channels_workspace(int64_t N, int64_t OC, int64_t P);
+// conv_direct.hip: small problems, operands straight from global memory, K shared between the waves of a workgroup;
+// input, output and residual may be channel slices of wider tensors
+bool conv_direct_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW,
+                    int64_t OH, int64_t OW);
+size_t conv_direct_packed_bytes(int64_t C, int64_t OC, int KH, int KW);
+int conv_direct_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, hipStream_t st);
+int conv_direct(const float *x, int64_t x_bs, const float *packed, const float *b, const float *res, int64_t res_bs, float *y,
+                int64_t y_bs, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int S, int P, int64_t OH,
+                int64_t OW, int act, hipStream_t st);
 }  // namespace odl
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -1131,6 +1141,9 @@ int odl_hip_col2im(const float *col, int64_t N, int64_t C, int64_t H, int64_t W,
     return col2im_launch(col, img, g, to_matrix, odl::as_stream(stream));
 }
 
+// whether small problems go to the direct kernel (odl_hip_set_conv_direct; on unless switched off for a measurement)
+static std::atomic<int> g_direct{1};
+
 // 16-byte aligned stand-in used by the workspace queries, which see shapes only
 static const float *const kAlignedProbe = reinterpret_cast<const float *>(uintptr_t(256));
 
@@ -1155,6 +1168,8 @@ size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W
     const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
     if (OH <= 0 || OW <= 0)
         return 0;
+    if (g_direct.load(std::memory_order_relaxed) && odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW))
+        return align256(odl::conv_direct_packed_bytes(C, OC, KH, KW));  // the filter copy of a caller that keeps none
     if (odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, OH, OW))
         return 0;
     if (odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW))
@@ -1184,6 +1199,9 @@ size_t odl_hip_conv2d_packed_weights_bytes(int64_t N, int64_t C, int64_t H, int6
     if (KH <= 0 || KW <= 0 || SH <= 0 || SW <= 0)
         return 0;
     const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
+    if (OH > 0 && OW > 0 && g_direct.load(std::memory_order_relaxed) &&
+        odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW))
+        return odl::conv_direct_packed_bytes(C, OC, KH, KW);
     if (OH <= 0 || OW <= 0 || odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, OH, OW) ||
         !odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW) ||
         forward_by_col_matrix(N, C, OC, KH, KW, SH, SW, OH, OW))
@@ -1191,10 +1209,16 @@ size_t odl_hip_conv2d_packed_weights_bytes(int64_t N, int64_t C, int64_t H, int6
     return odl::conv_implicit_forward_packed_bytes(N, C, H, W, OC, KH, KW);
 }
 
-int odl_hip_conv2d_pack_weights(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, void *stream)
+int odl_hip_conv2d_pack_weights(const float *w, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                                int SW, int PH, int PW, float *packed, void *stream)
 {
     ODL_REQUIRE_DEVICE();
-    ODL_REQUIRE(w && packed && C > 0 && OC > 0 && KH > 0 && KW > 0, "conv2d_pack_weights: bad argument");
+    ODL_REQUIRE(w && packed && C > 0 && OC > 0 && KH > 0 && KW > 0 && SH > 0 && SW > 0, "conv2d_pack_weights: bad argument");
+    ODL_REQUIRE(odl_hip_conv2d_packed_weights_bytes(N, C, H, W, OC, KH, KW, SH, SW, PH, PW) > 0,
+                "conv2d_pack_weights: a forward over this shape reads the filter as it lies");
+    const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
+    if (g_direct.load(std::memory_order_relaxed) && odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW))
+        return odl::conv_direct_pack(w, C, OC, KH, KW, packed, odl::as_stream(stream));
     return odl::conv_implicit_forward_pack(w, C, OC, KH, KW, packed, odl::as_stream(stream));
 }
 
@@ -1215,6 +1239,22 @@ int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packe
     if (M == 0)
         return ODL_OK;
     hipStream_t st = odl::as_stream(stream);
+    // small problems: one launch whatever the window, no workspace (the same shape always takes the same kernel)
+    if (g_direct.load(std::memory_order_relaxed) && odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW))
+    {
+        if (packed == nullptr)
+        {
+            // a caller that keeps no filter copy: one is made in the workspace first
+            const size_t need = odl::conv_direct_packed_bytes(C, OC, KH, KW);
+            ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0,
+                        "conv2d: this shape needs a 16-byte aligned workspace of %zu bytes, got %zu", need, workspace_bytes);
+            rc = odl::conv_direct_pack(w, C, OC, KH, KW, static_cast<float *>(workspace), st);
+            if (rc != ODL_OK)
+                return rc;
+            packed = static_cast<const float *>(workspace);
+        }
+        return odl::conv_direct(x, 0, packed, b, nullptr, 0, y, 0, N, C, H, W, OC, KH, KW, SH, PH, g.OH, g.OW, act, st);
+    }
     // a 1x1 window at stride 1 is a plain product per image, y[n] = W . x[n]: operands straight into LDS, bias and
     // activation in the epilogue, the output already NCHW (no K slices, no second launch)
     if (KH == 1 && KW == 1 && SH == 1 && SW == 1 && PH == 0 && PW == 0 && odl::conv1x1_dma_ok(x, w, N, C, H * W, OC))
@@ -1243,6 +1283,47 @@ int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packe
         return rc;
     return odl::sgemm_launch(0, 1, OC, M, K, w, K, col, K, y, 0, b, /*EPI_NCHW_ROWB*/ 2, g.OH * g.OW, 1, nullptr, 0,
                              st, act);
+}
+
+int odl_hip_set_conv_direct(int enabled)
+{
+    g_direct.store(enabled ? 1 : 0, std::memory_order_relaxed);
+    return ODL_OK;
+}
+
+int odl_hip_conv2d_fused_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH,
+                            int PW)
+{
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || KH <= 0 || KW <= 0 || SH <= 0 || SW <= 0 || PH < 0 || PW < 0)
+        return 0;
+    const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
+    return OH > 0 && OW > 0 && odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW) ? 1 : 0;
+}
+
+int odl_hip_conv2d_fused(const float *x, int64_t x_image_stride, const float *packed, const float *b, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW,
+                         int activation, const float *residual, int64_t residual_image_stride, float *y,
+                         int64_t y_image_stride, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(activation == -1 || activation == 0 || activation == 7,
+                "conv2d: activation must be -1 (none), 0 (relu) or 7 (silu), the unary operator numbers; got %d", activation);
+    ConvGeom g;
+    int rc = make_geom(g, "conv2d", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(OC > 0 && x && packed && y, "conv2d_fused: null operand or OC <= 0");
+    if (N == 0)
+        return ODL_OK;
+    ODL_REQUIRE(odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW),
+                "conv2d_fused: shape not covered (ask odl_hip_conv2d_fused_ok first)");
+    ODL_REQUIRE((x_image_stride == 0 || x_image_stride >= C * H * W) && (y_image_stride == 0 || y_image_stride >= OC * g.OH * g.OW) &&
+                    (residual_image_stride == 0 || residual_image_stride >= OC * g.OH * g.OW),
+                "conv2d_fused: an image stride is shorter than the image it strides over");
+    ODL_REQUIRE(x_image_stride < (1ll << 40) && y_image_stride < (1ll << 40) && residual_image_stride < (1ll << 40),
+                "conv2d_fused: image stride too large");
+    const int act = activation == 0 ? 1 : (activation == 7 ? 2 : 0);
+    return odl::conv_direct(x, x_image_stride, packed, b, residual, residual_image_stride, y, y_image_stride, N, C, H, W, OC,
+                            KH, KW, SH, PH, g.OH, g.OW, act, odl::as_stream(stream));
 }
 
 int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,

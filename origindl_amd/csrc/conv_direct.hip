@@ -1,0 +1,336 @@
+// Convolution forward for small problems (a detector's layers at batch 1-8: a few hundred MFLOP, outputs of a few
+// hundred KB), where a tiled GEMM spends its time in launch, prologue and a K-slice reduction rather than in arithmetic.
+//   y[n, oc, oh, ow] = act(b[oc] + sum_{c,kh,kw} x[n, c, oh*s-p+kh, ow*s-p+kw] * W[oc, c, kh, kw]) (+ r[n, oc, oh, ow])
+// the reference's forward (src/mat/origin/cpu/nn/conv2d.cpp:230-300 through im2col + matmul; the detector's runner calls it
+// per node, src/pnnx/pnnx_graph.cpp:286-528, then its SiLU / add / cat nodes one by one).
+//
+// One wave owns a 32 (output channels) x 32 (output pixels) tile on v_mfma_f32_32x32x2_f32 and reads its operands
+// straight from global memory (the whole layer lives in L2): per step a lane loads four consecutive channels of one
+// filter row (16 bytes) and the four matching input values of its pixel, which feed four MFMAs. The filter is read
+// from a copy laid out for exactly this access — per (tile of 32 output channels, tap, group of 8 channels) one
+// contiguous 1 KB block [lane half][row][4 channels], so a wave's load is eight whole cache lines — made once per
+// set of weights (or into the workspace on every call for a caller that does not keep it). No LDS staging and no
+// barrier in the K loop. The waves of a workgroup are `pixel tiles` x `K shares`: a long K (3x3 over 128 channels)
+// is cut into shares of whole channel groups, one wave each, summed through LDS in share order in the epilogue,
+// which also adds the bias, applies the activation, adds a residual tensor and stores NCHW. Input, output and
+// residual each carry their own distance between images, so any of them can be a channel slice of a wider tensor
+// (the destination of a concatenation).
+#include "odl_common.h"
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+namespace
+{
+struct DirectArgs
+{
+    const float *x, *w, *bias, *res;
+    float *y;
+    int64_t x_bs, y_bs, res_bs;  // floats from one image to the next
+    int C, H, W, OC, OH, OW, KH, KW, S, P;
+    int M;             // N * OH * OW output pixels
+    int act;           // 0 none, 1 relu, 2 silu
+    int KS, WP;        // K shares and pixel tiles of a workgroup (KS * WP waves)
+    int chunks;        // channel groups of eight per K share
+    int octiles;
+    odl::FastDiv d_ohw, d_ow, d_chunks, d_kw;
+};
+
+#ifdef ODL_DIRECT_DBG
+__device__ unsigned long long g_direct_dbg[4096 * 8];
+#define ODL_DIRECT_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < 4096) g_direct_dbg[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define ODL_DIRECT_STAMP(i) do { } while (0)
+#endif
+
+constexpr int kPitch = 33;    // floats per row of a partial tile in LDS
+
+// wd[((tile * KHW + tap) * groups + grp) * 256 + (half * 32 + row) * 4 + j] = w[tile*32 + row][grp*8 + half*4 + j][tap]
+// (rows past OC are zero)
+__global__ void pack_direct_kernel(const float *__restrict__ w, float *__restrict__ wd, int C, int OC, int KHW, int64_t total)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    const int j = (int)(t & 3), row = (int)((t >> 2) & 31), half = (int)((t >> 7) & 1);
+    int64_t blk = t >> 8;
+    const int groups = C / 8;
+    const int grp = (int)(blk % groups);
+    blk /= groups;
+    const int tap = (int)(blk % KHW), tile = (int)(blk / KHW);
+    const int oc = tile * 32 + row, c = grp * 8 + half * 4 + j;
+    wd[t] = oc < OC ? w[((int64_t)oc * C + c) * KHW + tap] : 0.f;
+}
+
+// The sums of the workgroup's outputs over the K shares, then bias, activation, residual, store: E outputs per thread
+// (32 consecutive threads along the pixels of one output channel). Straight-line code: the residual loads first, the
+// stores last, nothing that waits for a store.
+template <int E, bool RES>
+__device__ __forceinline__ void direct_epilogue(const DirectArgs &g, const float *partial, const float *bias_s, int m_base,
+                                                int oc0, int OHW)
+{
+    const int nthreads = 64 * g.KS * g.WP;
+    int64_t off[E];
+    float res[E], v[E];
+    bool ok[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i)
+    {
+        const int e = threadIdx.x + i * nthreads;
+        const int tp = e >> 10, rr = (e >> 5) & 31, col = e & 31;
+        const int mm = m_base + tp * 32 + col, oc = oc0 + rr;
+        ok[i] = mm < g.M && oc < g.OC;
+        const unsigned mc = ok[i] ? (unsigned)mm : 0u;
+        const unsigned nn = odl::fastdiv(mc, g.d_ohw), px = mc - nn * (unsigned)OHW;
+        const int64_t o = (int64_t)(ok[i] ? oc : 0) * OHW + px;
+        off[i] = (int64_t)nn * g.y_bs + o;
+        if (RES)
+            res[i] = g.res[(int64_t)nn * g.res_bs + o];
+    }
+#pragma unroll
+    for (int i = 0; i < E; ++i)
+    {
+        const int e = threadIdx.x + i * nthreads;
+        const int tp = e >> 10, rr = (e >> 5) & 31, col = e & 31;
+        const float *src = partial + ((size_t)tp * g.KS * 32 + rr) * kPitch + col;
+        float a = src[0];
+        for (int s = 1; s < g.KS; ++s)
+            a += src[(size_t)s * 32 * kPitch];
+        v[i] = odl::apply_act(a + bias_s[rr], g.act);
+        if (RES)
+            v[i] = res[i] + v[i];
+    }
+#pragma unroll
+    for (int i = 0; i < E; ++i)
+        if (ok[i])
+            g.y[off[i]] = v[i];
+}
+
+// kDepth: operand groups in flight per wave. Every load instruction costs the compute unit's one address unit 16
+// clocks whether or not its data is used, so the depth divides the group count (3 for 3x3 windows, 4 otherwise) and no
+// group is loaded twice.
+template <int kDepth, bool RES>
+__global__ __launch_bounds__(1024) void conv_direct_kernel(DirectArgs g)
+{
+    extern __shared__ float lds[];  // bias[32], then partial[WP * KS][32][kPitch] when KS > 1
+    ODL_DIRECT_STAMP(0);
+    float *bias_s = lds, *partial = lds + 32;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int pt = wv / g.KS, ks = wv - pt * g.KS;
+    const unsigned bid = blockIdx.x;
+    const int oct = (int)(bid % (unsigned)g.octiles);
+    const int m_base = (int)(bid / (unsigned)g.octiles) * 32 * g.WP;
+    const int oc0 = oct * 32;
+    const int HW = g.H * g.W, OHW = g.OH * g.OW, KHW = g.KH * g.KW;
+    // the bias rows of the tile: asked for now, put into LDS after the K loop (no wait here)
+    const float bias_v = (threadIdx.x < 32 && g.bias && oc0 + (int)threadIdx.x < g.OC) ? g.bias[oc0 + threadIdx.x] : 0.f;
+    // a lane past the last pixel reads the last pixel's operands; its results are never stored
+    int m = m_base + pt * 32 + l32;
+    m = m < g.M ? m : g.M - 1;
+    const unsigned n = odl::fastdiv((unsigned)m, g.d_ohw), r = (unsigned)m - n * (unsigned)OHW;
+    const int oh = (int)odl::fastdiv(r, g.d_ow), ow = (int)r - oh * g.OW;
+    const int ih0 = oh * g.S - g.P, iw0 = ow * g.S - g.P;
+    const int groups = g.C >> 3;
+    const int grp0 = ks * g.chunks;
+    const float *xb = g.x + (int64_t)n * g.x_bs + (int64_t)(grp0 * 8 + 4 * half) * HW;
+    // this wave's first block of the filter copy; consecutive groups and then consecutive taps follow each other
+    const float *wb = g.w + ((int64_t)oct * KHW * groups + grp0) * 256 + lane * 4;
+
+    const int total = KHW * g.chunks;
+    ODL_DIRECT_STAMP(1);
+    // Operand groups are numbered tap-major, (tap, channel group); group q is loaded kDepth groups ahead of its use.
+    // Inside the K loop the loads are unconditional and their addresses come from q by arithmetic alone, so the loop
+    // body is one basic block and the loads of later groups stay in flight across the MFMAs of earlier ones; a q
+    // past the end (only when kDepth does not divide the group count) loads the last group again, unused.
+    f32x4 fa[kDepth], fb[kDepth];
+    bool fok[kDepth];  // a tap in the padding: its group is replaced by zeros when it is used
+    auto load = [&](int slot, int q) {
+        q = q < total ? q : total - 1;
+        const int tap = (int)odl::fastdiv((unsigned)q, g.d_chunks), cc = q - tap * g.chunks;
+        const int kh = (int)odl::fastdiv((unsigned)tap, g.d_kw), kw = tap - kh * g.KW;
+        const int ih = ih0 + kh, iw = iw0 + kw;
+        fok[slot] = (unsigned)ih < (unsigned)g.H && (unsigned)iw < (unsigned)g.W;
+        // (the padding tap reads the pixel's nearest valid neighbour)
+        const int ihc = ih < 0 ? 0 : (ih >= g.H ? g.H - 1 : ih), iwc = iw < 0 ? 0 : (iw >= g.W ? g.W - 1 : iw);
+        const float *px = xb + (ihc * g.W + iwc) + (int64_t)cc * 8 * HW;
+        fa[slot] = *reinterpret_cast<const f32x4 *>(wb + ((int64_t)tap * groups + cc) * 256);
+        fb[slot] = f32x4{px[0], px[HW], px[2 * HW], px[3 * HW]};
+    };
+    f32x16 acc = {0};
+    auto use = [&](int slot) {
+        const f32x4 a = fa[slot], b = fok[slot] ? fb[slot] : f32x4{0.f, 0.f, 0.f, 0.f};
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
+    };
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d)
+        if (d < total)
+            load(d, d);
+    int it = 0;
+    for (; it + kDepth < total; it += kDepth)
+    {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d)
+        {
+            use(d);
+            load(d, it + d + kDepth);
+            __builtin_amdgcn_sched_barrier(0);  // keep each group's loads where they are written: right behind its use
+        }
+    }
+    ODL_DIRECT_STAMP(2);
+    const int rem = total - it;  // groups left (1 .. kDepth), already loaded into slots 0 .. rem-1
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d)
+        if (d < rem)
+            use(d);
+    ODL_DIRECT_STAMP(3);
+    if (threadIdx.x < 32)
+        bias_s[threadIdx.x] = bias_v;
+    if (g.KS == 1)
+    {
+        // accumulator register q of a lane: row 8*(q/4) + 4*half + q%4, column l32
+        __syncthreads();  // the bias rows
+        const int mm = m_base + pt * 32 + l32;
+        if (mm < g.M)
+        {
+            const int64_t pix = (int64_t)r;
+            float *yp = g.y + (int64_t)n * g.y_bs + pix;
+            float rv[16];
+            if (RES)
+            {
+                // (a row past OC reads the last row's residual and is not stored)
+                const float *rp = g.res + (int64_t)n * g.res_bs + pix;
+#pragma unroll
+                for (int q = 0; q < 16; ++q)
+                {
+                    const int oc = oc0 + 8 * (q / 4) + 4 * half + (q % 4);
+                    rv[q] = rp[(int64_t)(oc < g.OC ? oc : g.OC - 1) * OHW];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 16; ++q)
+            {
+                const int rr = 8 * (q / 4) + 4 * half + (q % 4);
+                float v = odl::apply_act(acc[q] + bias_s[rr], g.act);
+                if (RES)
+                    v = rv[q] + v;
+                if (oc0 + rr < g.OC)
+                    yp[(int64_t)(oc0 + rr) * OHW] = v;
+            }
+        }
+        ODL_DIRECT_STAMP(5);
+        return;
+    }
+    float *mine = partial + (size_t)wv * 32 * kPitch;
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+        mine[(8 * (q / 4) + 4 * half + (q % 4)) * kPitch + l32] = acc[q];
+    __syncthreads();
+    ODL_DIRECT_STAMP(4);
+    // 1024 outputs a pixel tile over 64 * KS * WP threads: 16 / KS outputs a thread
+    if (g.KS == 2)
+        direct_epilogue<8, RES>(g, partial, bias_s, m_base, oc0, OHW);
+    else if (g.KS == 4)
+        direct_epilogue<4, RES>(g, partial, bias_s, m_base, oc0, OHW);
+    else if (g.KS == 8)
+        direct_epilogue<2, RES>(g, partial, bias_s, m_base, oc0, OHW);
+    else
+        direct_epilogue<1, RES>(g, partial, bias_s, m_base, oc0, OHW);
+    ODL_DIRECT_STAMP(5);
+}
+
+int g_force_ks = 0, g_force_wp = 0;  // measurement overrides (0: the rule below)
+
+// K shares and pixel tiles per workgroup: enough waves to give every SIMD of the chip one or two, shares of at least
+// one channel group, at most sixteen waves a workgroup
+void plan_direct(int64_t M, int64_t OC, int64_t C, int KHW, int &KS, int &WP, int &chunks)
+{
+    const int64_t tiles = odl::ceil_div(M, 32) * odl::ceil_div(OC, 32);
+    const int64_t want = (int64_t)odl::device_cus() * 4 * 2;
+    const int groups = (int)(C / 8);
+    int ks = 1;
+    while (ks < 16 && tiles * ks < want && groups % (2 * ks) == 0 && (int64_t)(groups / (2 * ks)) * KHW >= 2)
+        ks *= 2;
+    if (g_force_ks > 0 && groups % g_force_ks == 0)
+        ks = g_force_ks;
+    int wp = ks >= 4 ? 1 : 4 / ks;
+    if (g_force_wp > 0 && (ks == 1 || ks * g_force_wp <= 16) && (g_force_wp & (g_force_wp - 1)) == 0)
+        wp = g_force_wp;
+    while (wp > 1 && (int64_t)32 * (wp - 1) >= M)
+        --wp;
+    KS = ks, WP = wp, chunks = groups / ks;
+}
+}  // namespace
+
+namespace odl
+{
+// Shapes this kernel takes: channels in groups of eight (a lane's four consecutive channels, two lane halves), a
+// problem small enough that the tiled kernels' fixed costs dominate, 32-bit offsets within an image.
+bool conv_direct_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW,
+                    int64_t OH, int64_t OW)
+{
+    if (C <= 0 || C % 8 != 0 || SH != SW || PH != PW || KH <= 0 || KW <= 0 || KH * KW > 49 || OC <= 0)
+        return false;
+    const int64_t M = N * OH * OW, K = C * KH * KW;
+    if (M <= 0 || M >= (1ll << 30) || C * H * W >= (1ll << 30) || OC * OH * OW >= (1ll << 30) || OC * K >= (1ll << 30))
+        return false;
+    // (measured against the tiled kernels: ahead up to about 1.6 GFLOP, even with the filter copy made on every call)
+    return 2 * M * K * OC <= (3ll << 29);
+}
+
+size_t conv_direct_packed_bytes(int64_t C, int64_t OC, int KH, int KW)
+{
+    return (size_t)(ceil_div(OC, 32) * 32 * C * KH * KW) * sizeof(float);
+}
+
+int conv_direct_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, hipStream_t st)
+{
+    const int64_t total = ceil_div(OC, 32) * 32 * C * KH * KW;
+    ODL_REQUIRE(total < (1ll << 31) && C % 8 == 0, "conv2d: filter too large or channels not a multiple of 8");
+    hipLaunchKernelGGL(pack_direct_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, w, packed, (int)C, (int)OC,
+                       KH * KW, total);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+// x, y, residual: NCHW with x_bs / y_bs / res_bs floats from one image to the next (0: dense). packed: the filter as
+// conv_direct_pack lays it out (16-byte aligned).
+int conv_direct(const float *x, int64_t x_bs, const float *packed, const float *b, const float *res, int64_t res_bs, float *y,
+                int64_t y_bs, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int S, int P, int64_t OH,
+                int64_t OW, int act, hipStream_t st)
+{
+    ODL_REQUIRE(packed != nullptr && reinterpret_cast<uintptr_t>(packed) % 16 == 0, "conv2d: the filter copy must be 16-byte aligned");
+    DirectArgs g{};
+    g.x = x, g.w = packed, g.bias = b, g.res = res, g.y = y;
+    g.x_bs = x_bs ? x_bs : C * H * W, g.y_bs = y_bs ? y_bs : OC * OH * OW, g.res_bs = res_bs ? res_bs : OC * OH * OW;
+    g.C = (int)C, g.H = (int)H, g.W = (int)W, g.OC = (int)OC, g.OH = (int)OH, g.OW = (int)OW, g.KH = KH, g.KW = KW, g.S = S, g.P = P;
+    g.M = (int)(N * OH * OW), g.act = act;
+    plan_direct(g.M, OC, C, KH * KW, g.KS, g.WP, g.chunks);
+    g.octiles = (int)ceil_div(OC, 32);
+    g.d_ohw = make_fastdiv((unsigned)(OH * OW)), g.d_ow = make_fastdiv((unsigned)OW);
+    g.d_chunks = make_fastdiv((unsigned)g.chunks), g.d_kw = make_fastdiv((unsigned)KW);
+    const int64_t blocks = ceil_div(g.M, 32 * g.WP) * g.octiles;
+    ODL_REQUIRE(blocks < (1ll << 31), "conv2d: too many tiles");
+    const size_t lds = (32 + (g.KS > 1 ? (size_t)g.KS * g.WP * 32 * kPitch : 0)) * sizeof(float);
+    const dim3 grid((unsigned)blocks), block(64 * g.KS * g.WP);
+    if ((KH * KW) % 3 == 0 && res)
+        hipLaunchKernelGGL((conv_direct_kernel<3, true>), grid, block, lds, st, g);
+    else if ((KH * KW) % 3 == 0)
+        hipLaunchKernelGGL((conv_direct_kernel<3, false>), grid, block, lds, st, g);
+    else if (res)
+        hipLaunchKernelGGL((conv_direct_kernel<4, true>), grid, block, lds, st, g);
+    else
+        hipLaunchKernelGGL((conv_direct_kernel<4, false>), grid, block, lds, st, g);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace odl
+
+extern "C" int odl_hip_set_conv_direct_plan(int k_shares, int pixel_tiles)
+{
+    g_force_ks = k_shares, g_force_wp = pixel_tiles;
+    return ODL_OK;
+}

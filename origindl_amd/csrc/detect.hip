@@ -57,6 +57,25 @@ __global__ __launch_bounds__(kBlock) void upsample_nearest_quads_kernel(const fl
     reinterpret_cast<f32x4 *>(y)[t] = v;
 }
 
+// upsample_nearest_quads_kernel for tensors whose images lie x_bs / y_bs floats apart (channel runs of wider tensors)
+__global__ __launch_bounds__(kBlock) void upsample_nearest_view_kernel(const float *__restrict__ x, int64_t x_bs,
+                                                                       float *__restrict__ y, int64_t y_bs, unsigned quads,
+                                                                       int C, int H, int W, int OH, int OW, int sh, int sw,
+                                                                       odl::FastDiv d_qrow, odl::FastDiv d_oh, odl::FastDiv d_c)
+{
+    const unsigned t = blockIdx.x * (unsigned)kBlock + threadIdx.x;
+    if (t >= quads)
+        return;
+    const unsigned qrow = (unsigned)OW / 4u;
+    const unsigned line = odl::fastdiv(t, d_qrow), q = t - line * qrow;  // line = (n * C + c) * OH + oh
+    const unsigned nc = odl::fastdiv(line, d_oh), oh = line - nc * (unsigned)OH;
+    const unsigned n = odl::fastdiv(nc, d_c), c = nc - n * (unsigned)C;
+    const float *row = x + (int64_t)n * x_bs + ((int64_t)c * H + (int)oh / sh) * W;
+    const int ow = 4 * (int)q;
+    const f32x4 v{row[ow / sw], row[(ow + 1) / sw], row[(ow + 2) / sw], row[(ow + 3) / sw]};
+    *reinterpret_cast<f32x4 *>(y + (int64_t)n * y_bs + ((int64_t)c * OH + oh) * OW + ow) = v;
+}
+
 // dst[m*dst_stride + dst_off + j] = src[m*src_stride + src_off + j] for j < chunk: `outer` contiguous runs;
 // grid (run pieces, m). Concatenation scatters whole inputs (src_stride = chunk, src_off = 0); its backward, split,
 // gathers a slice (dst_stride = chunk, dst_off = 0).
@@ -118,6 +137,7 @@ struct DetectGeom
     int anchor_H, anchor_W;
     int64_t grid_elems, anchor_elems;
     float stride;
+    int64_t out_bs;  // floats from one image's rows of this stage to the next image's
 };
 
 __global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__restrict__ conv, const float *__restrict__ grid,
@@ -188,7 +208,7 @@ __global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__rest
     }
     __syncthreads();
     // [pixel][channel] rows out of LDS, consecutive lanes along the output
-    float *dst = out + ((int64_t)(b * g.A + a) * HW + p0) * g.CI;
+    float *dst = out + (int64_t)b * g.out_bs + ((int64_t)a * HW + p0) * g.CI;
     for (int pl = wave; pl < np; pl += kBlock / 64)
         for (int c = lane; c < g.CI; c += 64)
             dst[pl * g.CI + c] = sh_det[pl * LS + c];
@@ -320,6 +340,82 @@ int odl_hip_upsample_nearest_backward(const float *gy, int64_t N, int64_t C, int
     return ODL_OK;
 }
 
+int odl_hip_upsample_nearest_view(const float *x, int64_t x_image_stride, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
+                                  int64_t OW, int scale_h, int scale_w, float *y, int64_t y_image_stride, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(x && y && N >= 0 && C > 0 && H > 0 && W > 0 && OH > 0 && OW > 0, "upsample: bad shape or null operand");
+    ODL_REQUIRE(scale_h > 0 && scale_w > 0, "upsample: scale must be positive");
+    ODL_REQUIRE((OH - 1) / scale_h < H && (OW - 1) / scale_w < W,
+                "upsample: output (%lld,%lld) reaches past input (%lld,%lld) at scale (%d,%d)", (long long)OH,
+                (long long)OW, (long long)H, (long long)W, scale_h, scale_w);
+    const int64_t xs = x_image_stride ? x_image_stride : C * H * W, ys = y_image_stride ? y_image_stride : C * OH * OW;
+    ODL_REQUIRE(xs >= C * H * W && ys >= C * OH * OW, "upsample: an image stride is shorter than the image");
+    ODL_REQUIRE(OW % 4 == 0 && ys % 4 == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0,
+                "upsample_view: output rows must be a multiple of four floats and 16-byte aligned");
+    const int64_t total = N * C * OH * OW;
+    if (total == 0)
+        return ODL_OK;
+    ODL_REQUIRE(total < (1ll << 32) - kBlock && H * W < (1ll << 31) && OH * OW < (1ll << 31) && N * C * OH < (1ll << 31),
+                "upsample: too large");
+    const unsigned quads = (unsigned)(total / 4);
+    hipLaunchKernelGGL(upsample_nearest_view_kernel, dim3((unsigned)odl::ceil_div(quads, kBlock)), dim3(kBlock), 0,
+                       odl::as_stream(stream), x, xs, y, ys, quads, (int)C, (int)H, (int)W, (int)OH, (int)OW, scale_h, scale_w,
+                       odl::make_fastdiv((unsigned)(OW / 4)), odl::make_fastdiv((unsigned)OH), odl::make_fastdiv((unsigned)C));
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_copy_images(const float *src, int64_t src_image_stride, float *dst, int64_t dst_image_stride, int64_t N,
+                        int64_t count, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && count >= 0 && src_image_stride >= count && dst_image_stride >= count, "copy_images: bad extents");
+    if (N == 0 || count == 0)
+        return ODL_OK;
+    ODL_REQUIRE(src && dst, "copy_images: null operand");
+    hipStream_t st = odl::as_stream(stream);
+    const bool vec = count % 4 == 0 && src_image_stride % 4 == 0 && dst_image_stride % 4 == 0 &&
+                     reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
+    for (int64_t m0 = 0; m0 < N; m0 += 65535)
+    {
+        const int64_t ms = N - m0 < 65535 ? N - m0 : 65535;
+        const float *s = src + m0 * src_image_stride;
+        float *d = dst + m0 * dst_image_stride;
+        if (vec)
+            hipLaunchKernelGGL((cat_copy_kernel<true>), dim3((unsigned)odl::ceil_div(count / 4, kBlock), (unsigned)ms), dim3(kBlock),
+                               0, st, s, d, count, src_image_stride, (int64_t)0, dst_image_stride, (int64_t)0);
+        else
+            hipLaunchKernelGGL((cat_copy_kernel<false>), dim3((unsigned)odl::ceil_div(count, kBlock), (unsigned)ms), dim3(kBlock), 0,
+                               st, s, d, count, src_image_stride, (int64_t)0, dst_image_stride, (int64_t)0);
+        ODL_LAUNCH_CHECK();
+    }
+    return ODL_OK;
+}
+
+int odl_hip_yolo_decode(const float *conv, const float *grid, int64_t grid_elems, const float *anchor_grid, int64_t anchor_elems,
+                        int64_t anchor_H, int64_t anchor_W, int64_t N, int64_t H, int64_t W, float stride, int num_anchors,
+                        int num_classes, float *out, int64_t out_image_stride, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && H > 0 && W > 0 && num_anchors > 0 && num_classes >= 0, "yolo_decode: bad shape");
+    ODL_REQUIRE(conv && grid && anchor_grid && out, "yolo_decode: null operand");
+    ODL_REQUIRE(grid_elems >= 0 && anchor_elems >= 0 && anchor_H > 0 && anchor_W > 0, "yolo_decode: bad grid sizes");
+    if (N == 0)
+        return ODL_OK;
+    const int CI = num_classes + 5;
+    ODL_REQUIRE(N * num_anchors * odl::ceil_div(H * W, 64) < (1ll << 31) && H * W < (1ll << 30) && CI < 8192, "yolo_decode: too large");
+    const int64_t os = out_image_stride ? out_image_stride : (int64_t)num_anchors * H * W * CI;
+    ODL_REQUIRE(os >= (int64_t)num_anchors * H * W * CI, "yolo_decode: the output image stride is shorter than a stage's rows");
+    const int ptiles = (int)odl::ceil_div(H * W, 64);
+    const DetectGeom g{num_anchors, CI, (int)H, (int)W, (int)anchor_H, (int)anchor_W, grid_elems, anchor_elems, stride, os};
+    const size_t lds = (size_t)64 * (CI | 1) * sizeof(float);
+    hipLaunchKernelGGL(yolo_decode_kernel, dim3((unsigned)(N * num_anchors * ptiles)), dim3(kBlock), lds, odl::as_stream(stream),
+                       conv, grid, anchor_grid, out, g, ptiles);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
 size_t odl_hip_yolo_detect_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int num_anchors, int num_classes)
 {
     if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || num_anchors <= 0 || num_classes < 0)
@@ -355,7 +451,8 @@ int odl_hip_yolo_detect_forward(const float *x, const float *conv_w, const float
     if (rc != ODL_OK)
         return rc;
     const int ptiles = (int)odl::ceil_div(H * W, 64);
-    const DetectGeom g{num_anchors, CI, (int)H, (int)W, (int)anchor_H, (int)anchor_W, grid_elems, anchor_elems, stride};
+    const DetectGeom g{num_anchors, CI, (int)H, (int)W, (int)anchor_H, (int)anchor_W, grid_elems, anchor_elems, stride,
+                       (int64_t)num_anchors * H * W * CI};
     const size_t lds = (size_t)64 * (CI | 1) * sizeof(float);
     hipLaunchKernelGGL(yolo_decode_kernel, dim3((unsigned)(N * num_anchors * ptiles)), dim3(kBlock), lds,
                        odl::as_stream(stream), conv, grid, anchor_grid, out, g, ptiles);

@@ -477,9 +477,74 @@ int make_geom(PoolGeom &g, const char *who, int64_t N, int64_t C, int64_t H, int
                 (long long)g.OW);
     return ODL_OK;
 }
+// `count` K x K / stride 1 / padding K/2 max pools one after the other over an (n, c) plane that stays in LDS: stage j reads
+// the plane stage j-1 wrote and writes its own both to LDS and to y[n, (j-1)*C + c] (a detector's SPPF block:
+// y1 = pool(x), y2 = pool(y1), y3 = pool(y2), all three concatenated). Each stage scans its windows exactly as
+// max_pool_fwd_lds_kernel does (first cell, then strict >, padding cells 0.0), so the values are those of `count`
+// separate calls. x and y carry their own distance between images: either may be a run of channels of a wider tensor.
+__global__ __launch_bounds__(256) void max_pool_chain_kernel(const float *__restrict__ x, int64_t x_bs, float *__restrict__ y,
+                                                              int64_t y_bs, int C, int H, int W, int K, int count)
+{
+    extern __shared__ float chain_sh[];  // two planes
+    const int plane = H * W, P = K / 2;
+    const int n = blockIdx.x / C, c = blockIdx.x - n * C;
+    const float *src = x + (int64_t)n * x_bs + (int64_t)c * plane;
+    float *cur = chain_sh, *nxt = chain_sh + plane;
+    for (int e = threadIdx.x; e < plane; e += 256)
+        cur[e] = src[e];
+    __syncthreads();
+    for (int j = 0; j < count; ++j)
+    {
+        float *dst = y + (int64_t)n * y_bs + ((int64_t)j * C + c) * plane;
+        for (int t = threadIdx.x; t < plane; t += 256)
+        {
+            const int oh = t / W, ow = t - oh * W;
+            float mv = 0.f;
+            for (int kh = 0; kh < K; ++kh)
+            {
+                const int h = oh - P + kh;
+                for (int kw = 0; kw < K; ++kw)
+                {
+                    const int w = ow - P + kw;
+                    const bool in = (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W;
+                    const float v = in ? cur[h * W + w] : 0.f;
+                    if ((kh | kw) == 0)
+                        mv = v;
+                    else if (v > mv)
+                        mv = v;
+                }
+            }
+            nxt[t] = mv;
+            dst[t] = mv;
+        }
+        __syncthreads();
+        float *tmp = cur;
+        cur = nxt, nxt = tmp;
+    }
+}
 }  // namespace
 
 extern "C" {
+
+int odl_hip_max_pool2d_chain(const float *x, int64_t x_image_stride, int64_t N, int64_t C, int64_t H, int64_t W, int K,
+                             int count, float *y, int64_t y_image_stride, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(x && y && N >= 0 && C > 0 && H > 0 && W > 0, "max_pool2d_chain: bad shape or null operand");
+    ODL_REQUIRE(K >= 1 && K % 2 == 1 && K <= 15 && count >= 1 && count <= 8, "max_pool2d_chain: odd window up to 15, 1 to 8 stages");
+    ODL_REQUIRE(H * W * 2 * (int64_t)sizeof(float) <= 64 * 1024, "max_pool2d_chain: the plane must fit LDS twice (%lld x %lld)",
+                (long long)H, (long long)W);
+    ODL_REQUIRE((x_image_stride == 0 || x_image_stride >= C * H * W) && (y_image_stride == 0 || y_image_stride >= count * C * H * W),
+                "max_pool2d_chain: an image stride is shorter than the image");
+    ODL_REQUIRE(N * C < (1ll << 31), "max_pool2d_chain: too many planes");
+    if (N == 0)
+        return ODL_OK;
+    hipLaunchKernelGGL(max_pool_chain_kernel, dim3((unsigned)(N * C)), dim3(256), (size_t)(2 * H * W) * sizeof(float),
+                       odl::as_stream(stream), x, x_image_stride ? x_image_stride : C * H * W, y,
+                       y_image_stride ? y_image_stride : count * C * H * W, (int)C, (int)H, (int)W, K, count);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
 
 int odl_hip_max_pool2d(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
                        int PH, int PW, float *y, uint64_t *idx, void *stream)

@@ -255,6 +255,15 @@ int odl_hip_graph_capture_begin(void *stream)
     return ODL_OK;
 }
 
+static thread_local int64_t t_last_graph_nodes = 0;
+
+int odl_hip_graph_last_node_count(int64_t *nodes)
+{
+    ODL_REQUIRE(nodes != nullptr, "graph_last_node_count: null argument");
+    *nodes = t_last_graph_nodes;
+    return ODL_OK;
+}
+
 int odl_hip_graph_capture_end(void *stream, void **graph_exec)
 {
     ODL_REQUIRE(stream != nullptr && graph_exec != nullptr, "graph_capture_end: null argument");
@@ -263,6 +272,10 @@ int odl_hip_graph_capture_end(void *stream, void **graph_exec)
     ODL_HIP_CHECK(hipStreamEndCapture(odl::as_stream(stream), &graph));
     if (graph == nullptr)
         return odl::fail(ODL_ERR_RUNTIME, "graph capture produced no graph (an operation that cannot be captured ended it)");
+    size_t nodes = 0;
+    if (hipGraphGetNodes(graph, nullptr, &nodes) != hipSuccess)
+        (void)hipGetLastError(), nodes = 0;
+    t_last_graph_nodes = (int64_t)nodes;
     hipGraphExec_t exec = nullptr;
     const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);

@@ -355,10 +355,36 @@ public:
     // `packed` (optional): the filter copy conv2d_packed_weights made for an input of this shape — for weights that stay
     // the same from call to call, so that the forward does not re-order them every time
     std::unique_ptr<Mat> conv2d_packed_weights(const Mat &W, std::pair<int, int> stride, std::pair<int, int> pad) const;
+    static std::unique_ptr<Mat> conv2d_packed_weights_for(const Shape &x_shape, const Mat &W, std::pair<int, int> stride,
+                                                          std::pair<int, int> pad);
     std::unique_ptr<Mat> conv2d_act(const Mat &W, const Mat *b, std::pair<int, int> stride, std::pair<int, int> pad,
                                     int activation, const Mat *packed) const;
     std::unique_ptr<Mat> conv2d_act(const Mat &W, const Mat *b, std::pair<int, int> stride, std::pair<int, int> pad,
                                     int activation) const;
+    // A run of channels [c0, c0 + channels) of an NCHW float32 device tensor: one input of a concatenation, written where
+    // the concatenation would copy it and read from there by what follows. The operators below take and fill such
+    // runs (a whole tensor is the run {t, 0, C}); their values are those of the dense operators.
+    struct ChannelRun
+    {
+        const OriginMat *tensor;
+        size_t c0, channels;
+    };
+    static ChannelRun whole(const Mat &m);
+    // whether conv2d_fused covers a convolution over an input run of this [N, C, H, W]
+    static bool conv2d_fused_ok(const Shape &x_run_shape, const Shape &w_shape, std::pair<int, int> stride,
+                                std::pair<int, int> pad);
+    // y = residual + act(conv(x, W) + b), W given as the copy conv2d_packed_weights made for this input shape
+    static void conv2d_fused(const ChannelRun &x, const Mat &packed, const Shape &w_shape, const Mat *b,
+                             std::pair<int, int> stride, std::pair<int, int> pad, int activation, const ChannelRun *residual,
+                             const ChannelRun &y);
+    static void upsample_run(const ChannelRun &x, const ChannelRun &y, int scale_h, int scale_w);
+    // y's channels [(j-1)*C, j*C) = the K x K / stride 1 / padding K/2 max pool applied j times to x, j = 1..count
+    static void max_pool_chain(const ChannelRun &x, int K, int count, const ChannelRun &y);
+    static void copy_run(const ChannelRun &src, const ChannelRun &dst);
+    // the convolution of a detect stage (this = its output [N, A*(classes+5), H, W]) decoded into rows
+    // [row0, row0 + A*H*W) of out[N, rows, classes+5]: the second half of yolo_detect_forward
+    void yolo_decode_into(const Mat &grid, const Mat &anchor_grid, float stride, int32_t num_anchors, int32_t num_classes,
+                          Mat &out, size_t row0) const;
     // Max pooling with the window-local indices kept in device memory (uint64 per output). The Mat interface above
     // hands them to the caller as a host vector, which costs a device-to-host copy in forward and a host-to-device
     // copy in backward (the reference's device backend pays both); the pooling operator uses this pair instead.

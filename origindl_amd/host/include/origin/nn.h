@@ -328,9 +328,11 @@ public:
     void abort_capture();  // gives the capture up: the thread, its stream and the memory pool are as before begin_capture
     void launch();  // on the current stream
     bool captured() const { return exec_ != nullptr; }
+    size_t node_count() const { return nodes_; }  // launches recorded
 
 private:
     void *exec_ = nullptr;
+    size_t nodes_ = 0;
     bool began_ = false;  // between this object's begin_capture and its end_capture / abort_capture
     std::shared_ptr<void> arena_;
 };

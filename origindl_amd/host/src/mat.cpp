@@ -1287,6 +1287,124 @@ std::unique_ptr<Mat> OriginMat::yolo_detect_forward(const Mat &conv_weight, cons
     return y;
 }
 
+namespace
+{
+struct RunPtr
+{
+    float *data;
+    int64_t image_stride, N, C, H, W;
+};
+
+RunPtr run_ptr(const OriginMat::ChannelRun &r, const char *who)
+{
+    if (!r.tensor)
+        THROW_INVALID_ARG("{}: null tensor in a channel run", who);
+    const OriginMat &t = dev_f32(*r.tensor, who);
+    const Shape &s = t.shape();
+    if (s.size() != 4 || r.c0 + r.channels > s[1] || r.channels == 0)
+        THROW_INVALID_ARG("{}: channels [{}, {}) do not lie in a 4D tensor of shape {}", who, r.c0, r.c0 + r.channels, s.to_string());
+    const int64_t plane = (int64_t)(s[2] * s[3]);
+    return RunPtr{const_cast<float *>(fp(t)) + (int64_t)r.c0 * plane, (int64_t)s[1] * plane, (int64_t)s[0], (int64_t)r.channels,
+                  (int64_t)s[2], (int64_t)s[3]};
+}
+}  // namespace
+
+OriginMat::ChannelRun OriginMat::whole(const Mat &m)
+{
+    const OriginMat &t = as_origin(m);
+    return ChannelRun{&t, 0, t.shape().size() == 4 ? t.shape()[1] : 0};
+}
+
+bool OriginMat::conv2d_fused_ok(const Shape &xs, const Shape &ws, std::pair<int, int> s, std::pair<int, int> p)
+{
+    if (xs.size() != 4 || ws.size() != 4 || xs[1] != ws[1])
+        return false;
+    return odl_hip_conv2d_fused_ok((int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3], (int64_t)ws[0], (int)ws[2],
+                                   (int)ws[3], s.first, s.second, p.first, p.second) == 1;
+}
+
+void OriginMat::conv2d_fused(const ChannelRun &xr, const Mat &packed_m, const Shape &ws, const Mat *bm, std::pair<int, int> s,
+                             std::pair<int, int> p, int activation, const ChannelRun *rr, const ChannelRun &yr)
+{
+    const RunPtr x = run_ptr(xr, "conv2d"), y = run_ptr(yr, "conv2d");
+    if (ws.size() != 4 || (int64_t)ws[1] != x.C || (int64_t)ws[0] != y.C)
+        THROW_INVALID_ARG("conv2d: filter {} does not map {} channels to {}", ws.to_string(), x.C, y.C);
+    const int KH = (int)ws[2], KW = (int)ws[3];
+    const int OH = get_conv_outsize((int)x.H, KH, s.first, p.first), OW = get_conv_outsize((int)x.W, KW, s.second, p.second);
+    if (y.N != x.N || y.H != OH || y.W != OW)
+        THROW_INVALID_ARG("conv2d: the output run is [{}, {}, {}, {}], the convolution gives [{}, {}, {}, {}]", y.N, y.C, y.H, y.W,
+                          x.N, y.C, OH, OW);
+    const OriginMat &pk = dev_f32(packed_m, "conv2d");
+    const size_t want = odl_hip_conv2d_packed_weights_bytes(x.N, x.C, x.H, x.W, y.C, KH, KW, s.first, s.second, p.first, p.second);
+    if (pk.elements() * sizeof(float) != want)
+        THROW_INVALID_ARG("conv2d: the packed filter has {} bytes, this shape's kernel reads {}", pk.elements() * sizeof(float), want);
+    const float *bias = nullptr;
+    if (bm)
+    {
+        const OriginMat &b = dev_f32(*bm, "conv2d");
+        if (b.shape().size() != 1 || (int64_t)b.shape()[0] != y.C)
+            THROW_INVALID_ARG("conv2d: b must be 1D with size {}, but got shape {}", y.C, b.shape().to_string());
+        bias = fp(b);
+    }
+    const float *res = nullptr;
+    int64_t res_stride = 0;
+    if (rr)
+    {
+        const RunPtr r = run_ptr(*rr, "conv2d");
+        if (r.N != y.N || r.C != y.C || r.H != y.H || r.W != y.W)
+            THROW_INVALID_ARG("conv2d: the residual run does not have the output's shape");
+        res = r.data, res_stride = r.image_stride;
+    }
+    check(odl_hip_conv2d_fused(x.data, x.image_stride, fp(pk), bias, x.N, x.C, x.H, x.W, y.C, KH, KW, s.first, s.second, p.first,
+                               p.second, activation, res, res_stride, y.data, y.image_stride, cur()));
+}
+
+void OriginMat::upsample_run(const ChannelRun &xr, const ChannelRun &yr, int sh, int sw)
+{
+    const RunPtr x = run_ptr(xr, "upsample"), y = run_ptr(yr, "upsample");
+    if (x.N != y.N || x.C != y.C)
+        THROW_INVALID_ARG("upsample: the runs differ in batch or channels");
+    check(odl_hip_upsample_nearest_view(x.data, x.image_stride, x.N, x.C, x.H, x.W, y.H, y.W, sh, sw, y.data, y.image_stride, cur()));
+}
+
+void OriginMat::max_pool_chain(const ChannelRun &xr, int K, int count, const ChannelRun &yr)
+{
+    const RunPtr x = run_ptr(xr, "max_pool2d"), y = run_ptr(yr, "max_pool2d");
+    if (x.N != y.N || x.C * count != y.C || x.H != y.H || x.W != y.W)
+        THROW_INVALID_ARG("max_pool2d: the output run must hold {} stages of the input run's shape", count);
+    check(odl_hip_max_pool2d_chain(x.data, x.image_stride, x.N, x.C, x.H, x.W, K, count, y.data, y.image_stride, cur()));
+}
+
+void OriginMat::copy_run(const ChannelRun &sr, const ChannelRun &dr)
+{
+    const RunPtr s = run_ptr(sr, "cat"), d = run_ptr(dr, "cat");
+    if (s.N != d.N || s.C != d.C || s.H != d.H || s.W != d.W)
+        THROW_INVALID_ARG("cat: the runs differ in shape");
+    check(odl_hip_copy_images(s.data, s.image_stride, d.data, d.image_stride, s.N, s.C * s.H * s.W, cur()));
+}
+
+void OriginMat::yolo_decode_into(const Mat &grid, const Mat &anchor_grid, float stride, int32_t num_anchors, int32_t num_classes,
+                                 Mat &out_m, size_t row0) const
+{
+    const OriginMat &conv = dev_f32(*this, "yolo_detect_forward");
+    const OriginMat &g = dev_f32(grid, "yolo_detect_forward");
+    const OriginMat &ag = dev_f32(anchor_grid, "yolo_detect_forward");
+    const OriginMat &out = dev_f32(out_m, "yolo_detect_forward");
+    const int64_t CI = num_classes + 5;
+    if (shape_.size() != 4 || (int64_t)shape_[1] != num_anchors * CI)
+        THROW_INVALID_ARG("yolo_detect_forward: the stage's convolution must be [N, {}, H, W], got {}", num_anchors * CI, shape_.to_string());
+    const int64_t N = shape_[0], H = shape_[2], W = shape_[3];
+    const Shape &os = out.shape();
+    if (os.size() != 3 || (int64_t)os[0] != N || (int64_t)os[2] != CI || row0 + (size_t)(num_anchors * H * W) > os[1])
+        THROW_INVALID_ARG("yolo_detect_forward: rows [{}, {}) do not lie in an output of shape {}", row0, row0 + num_anchors * H * W,
+                          os.to_string());
+    const Shape as = ag.shape();
+    const int64_t aH = as.size() >= 3 ? (int64_t)as[2] : H, aW = as.size() >= 4 ? (int64_t)as[3] : W;
+    check(odl_hip_yolo_decode(fp(conv), fp(g), (int64_t)g.elements(), fp(ag), (int64_t)ag.elements(), aH, aW, N, H, W, stride,
+                              num_anchors, num_classes, const_cast<float *>(fp(out)) + (int64_t)row0 * CI, (int64_t)(os[1] * os[2]),
+                              cur()));
+}
+
 std::unique_ptr<Mat> OriginMat::pow(const Scalar &exponent) const
 {
     const OriginMat &x = dev_any(*this, "pow");
@@ -1473,8 +1591,15 @@ std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pa
 // null when a forward over an input of this shape reads the filter as it lies
 std::unique_ptr<Mat> OriginMat::conv2d_packed_weights(const Mat &Wm, std::pair<int, int> s, std::pair<int, int> p) const
 {
-    const OriginMat &x = dev_f32(*this, "conv2d");
+    dev_f32(*this, "conv2d");
+    return conv2d_packed_weights_for(shape_, Wm, s, p);
+}
+
+std::unique_ptr<Mat> OriginMat::conv2d_packed_weights_for(const Shape &shape_, const Mat &Wm, std::pair<int, int> s,
+                                                          std::pair<int, int> p)
+{
     const OriginMat &w = dev_f32(Wm, "conv2d");
+    const OriginMat &x = w;  // the copy lives where the filter does
     if (shape_.size() != 4 || w.shape().size() != 4)
         return nullptr;
     const int64_t OC = w.shape()[0], C = w.shape()[1];
@@ -1484,8 +1609,9 @@ std::unique_ptr<Mat> OriginMat::conv2d_packed_weights(const Mat &Wm, std::pair<i
                                                              p.second);
     if (bytes == 0 || (int64_t)shape_[1] != C)
         return nullptr;
-    auto packed = new_like(x, w.shape());
-    check(odl_hip_conv2d_pack_weights(fp(w), C, OC, KH, KW, packed->data_ptr<float>(), cur()));
+    auto packed = new_like(x, Shape{bytes / sizeof(float)});  // whole tiles of output channels for some kernels
+    check(odl_hip_conv2d_pack_weights(fp(w), (int64_t)shape_[0], C, (int64_t)shape_[2], (int64_t)shape_[3], OC, KH, KW, s.first,
+                                      s.second, p.first, p.second, packed->data_ptr<float>(), cur()));
     return packed;
 }
 
@@ -1522,8 +1648,10 @@ std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pa
     if (packed_m)
     {
         const OriginMat &pk = dev_f32(*packed_m, "conv2d");
-        if (pk.elements() != w.elements())
-            THROW_INVALID_ARG("conv2d: the packed filter has {} elements, the filter {}", pk.elements(), w.elements());
+        const size_t want = odl_hip_conv2d_packed_weights_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second);
+        if (pk.elements() * sizeof(float) != want)
+            THROW_INVALID_ARG("conv2d: the packed filter has {} bytes, this shape's kernel reads {}", pk.elements() * sizeof(float),
+                              want);
         packed = fp(pk);
     }
     check(odl_hip_conv2d_act_packed(fp(x), fp(w), packed, bias, N, C, H, W, OC, KH, KW, s.first, s.second, p.first,
@@ -2105,6 +2233,9 @@ void Graph::end_capture()
         THROW_RUNTIME_ERROR("{}", odl_hip_last_error());
     }
     exec_ = exec;
+    int64_t nodes = 0;
+    if (odl_hip_graph_last_node_count(&nodes) == ODL_OK)
+        nodes_ = (size_t)nodes;
 }
 
 void Graph::launch()

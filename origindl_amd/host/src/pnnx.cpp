@@ -2,6 +2,7 @@
 // src/pnnx/internal/store_zip.cpp:20-100); operator set as in src/pnnx/operator_mapper.cpp:26-78.
 #include "origin/pnnx/pnnx_graph.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -333,7 +334,177 @@ void PNNXGraph::build()
         if (!ok)
             THROW_RUNTIME_ERROR("Unsupported operator type: {}", n->type);
     }
+    placed_.clear();
+    cat_channels_.clear();
+    if (fusion_)
+        plan_fusion();
     built_ = true;
+}
+
+namespace
+{
+// the tensor a node leaves behind once the nodes folded into it are counted in
+const std::string &final_output(const PNNXNode &n)
+{
+    return n.fused_output_name.empty() ? n.output_names[0] : n.fused_output_name;
+}
+
+bool same_pool(const PNNXNode &n, int &K)
+{
+    if (n.type != "nn.MaxPool2d" || n.input_names.size() != 1 || n.output_names.size() != 1)
+        return false;
+    const auto k = int_pair(n, "kernel_size", {2, 2});
+    auto s = int_pair(n, "stride", {0, 0});
+    if (s.first <= 0 || s.second <= 0)
+        s = k;
+    const auto p = int_pair(n, "padding", {0, 0});
+    K = k.first;
+    return k.first == k.second && k.first % 2 == 1 && s == std::make_pair(1, 1) && p == std::make_pair(k.first / 2, k.first / 2);
+}
+}  // namespace
+
+// Decides, from the graph alone, which adds fold into the convolution before them, which tensors are written
+// straight into a concatenation's output, and which max pools form one chain. What a kernel can take is only known
+// once the shapes are (at run time); a node that cannot honour a decision falls back to its own tensor and a copy.
+void PNNXGraph::plan_fusion()
+{
+    std::map<std::string, PNNXNode *> writer;  // tensor -> the node that leaves it behind
+    std::map<std::string, std::vector<PNNXNode *>> readers;
+    for (auto &n : plan_)
+    {
+        if (!n->folded_into_producer && !n->output_names.empty())
+            writer[final_output(*n)] = n.get();
+        if (!n->folded_into_producer)
+            for (auto &in : n->input_names)
+                readers[in].push_back(n.get());
+    }
+    for (auto &n : nodes_)
+        if (n->type == "pnnx.Output")
+            for (auto &in : n->input_names)
+                readers[in].push_back(n.get());
+    // 1. conv (+ activation) -> add: the add moves into the convolution when the convolution's result has no other
+    // reader and the other addend already exists when the convolution runs
+    for (auto &n : plan_)
+    {
+        if (n->type != "pnnx.Expression" || n->input_names.size() != 2 || n->output_names.size() != 1)
+            continue;
+        const std::string expr = n->params.count("expr") ? n->params.at("expr") : "";
+        if (expr.find("add") == std::string::npos || n->input_names[0] == n->input_names[1])
+            continue;
+        for (int side = 0; side < 2; ++side)
+        {
+            const std::string &t = n->input_names[side], &other = n->input_names[1 - side];
+            auto w = writer.find(t);
+            if (w == writer.end() || w->second->type != "nn.Conv2d" || !w->second->residual_name.empty() ||
+                readers[t].size() != 1)
+                continue;
+            auto ow = writer.find(other);
+            if (ow != writer.end() && ow->second->execution_order >= w->second->execution_order)
+                continue;
+            PNNXNode *conv = w->second;
+            writer.erase(t);
+            readers[other].push_back(conv);
+            conv->residual_name = other;
+            conv->fused_output_name = n->output_names[0];
+            n->folded_into_producer = true;
+            writer[n->output_names[0]] = conv;
+            auto &ro = readers[other];
+            ro.erase(std::remove(ro.begin(), ro.end(), n.get()), ro.end());
+            break;
+        }
+    }
+    // 2. channel counts that follow from the graph alone
+    std::map<std::string, size_t> channels;
+    for (auto &n : plan_)
+    {
+        if (n->folded_into_producer || n->output_names.size() != 1)
+            continue;
+        size_t c = 0;
+        if (n->type == "nn.Conv2d")
+        {
+            auto w = n->attributes.find("weight");
+            c = (w != n->attributes.end() && w->second.shape.size() == 4) ? (size_t)w->second.shape[0] : 0;
+        }
+        else if (n->type == "nn.SiLU" || n->type == "nn.ReLU" || n->type == "nn.MaxPool2d" || n->type == "nn.Upsample" ||
+                 n->type == "pnnx.Expression")
+            c = channels.count(n->input_names[0]) ? channels[n->input_names[0]] : 0;
+        else if (n->type == "torch.cat" && int_param(*n, "dim", 0) == 1)
+        {
+            for (auto &in : n->input_names)
+            {
+                const size_t ci = channels.count(in) ? channels[in] : 0;
+                if (ci == 0)
+                {
+                    c = 0;
+                    break;
+                }
+                c += ci;
+            }
+        }
+        if (c > 0)
+            channels[final_output(*n)] = c;
+    }
+    // 3. inputs of a channel concatenation whose writer can aim at a run of channels are placed in its output
+    for (auto &n : plan_)
+    {
+        if (n->type != "torch.cat" || int_param(*n, "dim", 0) != 1 || n->input_names.size() < 2 || n->output_names.size() != 1)
+            continue;
+        const std::string &out = n->output_names[0];
+        if (!channels.count(out))
+            continue;
+        cat_channels_[out] = channels[out];
+        size_t c0 = 0;
+        for (auto &in : n->input_names)
+        {
+            auto w = writer.find(in);
+            const bool can_aim = w != writer.end() && (w->second->type == "nn.Conv2d" || w->second->type == "nn.Upsample" ||
+                                                       w->second->type == "nn.MaxPool2d");
+            if (can_aim && !placed_.count(in))
+                placed_[in] = Placement{out, c0};
+            c0 += channels[in];
+        }
+    }
+    // 4. chains of same-size max pools (stride 1, padding K/2) whose stages lie side by side in one concatenation
+    for (auto &n : plan_)
+    {
+        int K = 0;
+        if (n->folded_into_producer || !same_pool(*n, K) || !placed_.count(n->output_names[0]))
+            continue;
+        const Placement first = placed_[n->output_names[0]];
+        const size_t C = channels.count(n->output_names[0]) ? channels[n->output_names[0]] : 0;
+        if (C == 0)
+            continue;
+        int count = 1;
+        PNNXNode *last = n.get();
+        for (;;)
+        {
+            PNNXNode *next = nullptr;
+            for (PNNXNode *r : readers[last->output_names[0]])
+            {
+                int K2 = 0;
+                if (same_pool(*r, K2) && K2 == K && !r->folded_into_producer && r->pool_chain == 0)
+                    next = r;
+            }
+            if (!next || !placed_.count(next->output_names[0]))
+                break;
+            const Placement &pl = placed_[next->output_names[0]];
+            if (pl.buffer != first.buffer || pl.c0 != first.c0 + (size_t)count * C || count >= 8)
+                break;
+            next->folded_into_producer = true;
+            ++count;
+            last = next;
+        }
+        n->pool_chain = count;
+    }
+}
+
+size_t PNNXGraph::launching_nodes() const
+{
+    size_t c = 0;
+    for (auto &n : plan_)
+        if (!n->folded_into_producer && n->type != "torch.flatten")
+            ++c;
+    return c;
 }
 
 void PNNXGraph::set_inputs(const std::string &input_name, const std::vector<Tensor> &inputs)
@@ -348,13 +519,28 @@ void PNNXGraph::set_inputs(const std::string &input_name, const std::vector<Tens
         THROW_RUNTIME_ERROR("Input count mismatch: input node has {} outputs, but {} inputs provided",
                             n.output_names.size(), inputs.size());
     for (size_t i = 0; i < inputs.size(); ++i)
-        blobs_[n.output_names[i]] = inputs[i].impl_->data_;
+    {
+        Value v;
+        v.mat = inputs[i].impl_->data_;
+        blobs_[n.output_names[i]] = v;
+        if (std::find(input_blobs_.begin(), input_blobs_.end(), n.output_names[i]) == input_blobs_.end())
+            input_blobs_.push_back(n.output_names[i]);
+    }
 }
 
 void PNNXGraph::forward()
 {
     if (!built_)
         THROW_RUNTIME_ERROR("Graph must be built before forward");
+    // the tensors of the previous forward go (a concatenation's output is made when its first input is written, so
+    // one left over from the last forward must not be mistaken for it)
+    for (auto it = blobs_.begin(); it != blobs_.end();)
+    {
+        if (std::find(input_blobs_.begin(), input_blobs_.end(), it->first) == input_blobs_.end())
+            it = blobs_.erase(it);
+        else
+            ++it;
+    }
     for (auto &n : plan_)
         run(*n);
 }
@@ -368,35 +554,118 @@ std::vector<Tensor> PNNXGraph::get_outputs(const std::string &output_name) const
     for (auto &in : it->second->input_names)
     {
         auto b = blobs_.find(in);
-        if (b == blobs_.end())
+        if (b == blobs_.end() || !b->second.mat)
             THROW_RUNTIME_ERROR("Output '{}' has not been computed: call forward() first", in);
-        out.emplace_back(std::make_shared<TensorImpl>(b->second));
+        const Value &v = b->second;
+        if (!v.run)
+            out.emplace_back(std::make_shared<TensorImpl>(v.mat));
+        else
+        {
+            // a graph output that lives inside a concatenation: handed out as a tensor of its own
+            const Shape bs = v.mat->shape();
+            std::shared_ptr<Mat> copy = std::make_shared<OriginMat>(Shape{bs[0], v.channels, bs[2], bs[3]}, DataType::kFloat32, v.mat->device());
+            OriginMat::copy_run(OriginMat::ChannelRun{&origin_of(*v.mat), v.c0, v.channels}, OriginMat::whole(*copy));
+            out.emplace_back(std::make_shared<TensorImpl>(copy));
+        }
     }
     return out;
+}
+
+PNNXGraph::Value &PNNXGraph::value(const std::string &name, const PNNXNode &reader)
+{
+    auto it = blobs_.find(name);
+    if (it == blobs_.end() || !it->second.mat)
+        THROW_RUNTIME_ERROR("PNNX: input '{}' of node {} has no value (set_inputs not called?)", name, reader.name);
+    return it->second;
+}
+
+// the tensor as one of its own: a run of channels inside a concatenation is copied out once, when first asked for
+std::shared_ptr<Mat> PNNXGraph::dense(const std::string &name, const PNNXNode &reader)
+{
+    Value &v = value(name, reader);
+    if (!v.run)
+        return v.mat;
+    if (!v.dense)
+    {
+        const Shape bs = v.mat->shape();
+        v.dense = std::make_shared<OriginMat>(Shape{bs[0], v.channels, bs[2], bs[3]}, DataType::kFloat32, v.mat->device());
+        OriginMat::copy_run(OriginMat::ChannelRun{&origin_of(*v.mat), v.c0, v.channels}, OriginMat::whole(*v.dense));
+    }
+    return v.dense;
+}
+
+std::shared_ptr<Mat> PNNXGraph::buffer_for(const std::string &cat_output, size_t N, size_t H, size_t W, const Device &dev)
+{
+    Value &v = blobs_[cat_output];
+    const Shape want{N, cat_channels_.at(cat_output), H, W};
+    if (!v.mat)
+        v.mat = std::make_shared<OriginMat>(want, DataType::kFloat32, dev);
+    else if (v.mat->shape() != want)
+        THROW_RUNTIME_ERROR("PNNX: inputs of the concatenation {} disagree about its shape ({} and {})", cat_output,
+                            v.mat->shape().to_string(), want.to_string());
+    return v.mat;
+}
+
+// a node's dense result: kept as it is, or — for a tensor that build() placed in a concatenation — copied to its place
+void PNNXGraph::store(const PNNXNode &node, std::shared_ptr<Mat> out)
+{
+    const std::string &name = final_output(node);
+    auto pl = placed_.find(name);
+    const Shape os = out->shape();
+    if (pl == placed_.end() || os.size() != 4 || out->dtype() != DataType::kFloat32)
+    {
+        if (pl != placed_.end())
+            placed_.erase(pl);  // not a 4D float tensor after all: the concatenation copies it like any other input
+        Value v;
+        v.mat = std::move(out);
+        blobs_[name] = v;
+        return;
+    }
+    auto buf = buffer_for(pl->second.buffer, os[0], os[2], os[3], out->device());
+    OriginMat::copy_run(OriginMat::whole(*out), OriginMat::ChannelRun{&origin_of(*buf), pl->second.c0, os[1]});
+    Value v;
+    v.mat = buf, v.c0 = pl->second.c0, v.channels = os[1], v.run = true, v.dense = std::move(out);
+    blobs_[name] = v;
 }
 
 void PNNXGraph::run(PNNXNode &node)
 {
     if (node.folded_into_producer)
         return;  // its producer already wrote this node's output
-    std::vector<std::shared_ptr<Mat>> in;
-    for (auto &name : node.input_names)
-    {
-        auto it = blobs_.find(name);
-        if (it == blobs_.end())
-            THROW_RUNTIME_ERROR("PNNX: input '{}' of node {} has no value (set_inputs not called?)", name, node.name);
-        in.push_back(it->second);
-    }
-    if (in.empty())
+    if (node.input_names.empty())
         THROW_RUNTIME_ERROR("PNNX: node {} ({}) has no inputs", node.name, node.type);
-    const Device dev = in[0]->device();
+    if (node.output_names.size() != 1)
+        THROW_RUNTIME_ERROR("PNNX: node {} declares {} outputs; this runner's operators produce one", node.name,
+                            node.output_names.size());
+    Value &first = value(node.input_names[0], node);
+    const Device dev = first.mat->device();
     auto weight = [&](const std::string &key) -> std::shared_ptr<Mat> {
         auto it = node.attributes.find(key);
         if (it == node.attributes.end())
             return nullptr;
         return upload(it->second, dev, node.name + "." + key);
     };
-    std::shared_ptr<Mat> out;
+    auto run_of = [&](const Value &v) {
+        return v.run ? OriginMat::ChannelRun{&origin_of(*v.mat), v.c0, v.channels} : OriginMat::whole(*v.mat);
+    };
+    auto run_shape = [&](const Value &v) {
+        const Shape s = v.mat->shape();
+        return (v.run && s.size() == 4) ? Shape{s[0], v.channels, s[2], s[3]} : s;
+    };
+    const std::string &out_name = final_output(node);
+    auto place = placed_.find(out_name);
+    // where a [N, C, H, W] result of this node goes: its run of the concatenation, or a tensor of its own
+    auto destination = [&](size_t N, size_t C, size_t H, size_t W) {
+        Value v;
+        if (place != placed_.end())
+        {
+            v.mat = buffer_for(place->second.buffer, N, H, W, dev);
+            v.c0 = place->second.c0, v.channels = C, v.run = true;
+        }
+        else
+            v.mat = std::make_shared<OriginMat>(Shape{N, C, H, W}, DataType::kFloat32, dev);
+        return v;
+    };
     const std::string &t = node.type;
     if (t == "nn.Conv2d")
     {
@@ -407,31 +676,76 @@ void PNNXGraph::run(PNNXNode &node)
             THROW_RUNTIME_ERROR("PNNX: node {} has no weight", node.name);
         auto b = weight("bias");
         const auto stride = int_pair(node, "stride", {1, 1}), padding = int_pair(node, "padding", {0, 0});
+        const Shape xs = run_shape(first), ws = w->shape();
         // the weights never change: the filter order this input shape's kernel wants is made once and kept
         Attribute &wa = node.attributes.find("weight")->second;
-        const std::vector<size_t> in_dims = in[0]->shape().dims();
-        if (wa.packed_for != in_dims)
+        if (wa.packed_for != xs.dims())
         {
-            wa.packed_mat = origin_of(*in[0]).conv2d_packed_weights(*w, stride, padding);
-            wa.packed_for = in_dims;
+            wa.packed_mat = OriginMat::conv2d_packed_weights_for(xs, *w, stride, padding);
+            wa.packed_for = xs.dims();
         }
-        out = origin_of(*in[0]).conv2d_act(*w, b.get(), stride, padding, node.fused_activation, wa.packed_mat.get());
+        if (fusion_ && wa.packed_mat && first.mat->dtype() == DataType::kFloat32 && OriginMat::conv2d_fused_ok(xs, ws, stride, padding))
+        {
+            const int OH = get_conv_outsize((int)xs[2], (int)ws[2], stride.first, padding.first);
+            const int OW = get_conv_outsize((int)xs[3], (int)ws[3], stride.second, padding.second);
+            Value out = destination(xs[0], ws[0], (size_t)OH, (size_t)OW);
+            OriginMat::ChannelRun res{};
+            if (!node.residual_name.empty())
+                res = run_of(value(node.residual_name, node));
+            OriginMat::conv2d_fused(run_of(first), *wa.packed_mat, ws, b.get(), stride, padding, node.fused_activation,
+                                    node.residual_name.empty() ? nullptr : &res, run_of(out));
+            blobs_[out_name] = out;
+            return;
+        }
+        auto x = dense(node.input_names[0], node);
+        std::shared_ptr<Mat> out = origin_of(*x).conv2d_act(*w, b.get(), stride, padding, node.fused_activation, wa.packed_mat.get());
+        if (!node.residual_name.empty())
+            out = *dense(node.residual_name, node) + *out;
+        store(node, std::move(out));
+        return;
     }
-    else if (t == "nn.SiLU")
-        out = in[0]->silu();
-    else if (t == "nn.ReLU")
-        out = in[0]->relu();
-    else if (t == "nn.MaxPool2d")
+    if (t == "nn.MaxPool2d")
     {
         const auto k = int_pair(node, "kernel_size", {2, 2});
         auto s = int_pair(node, "stride", {0, 0});
         if (s.first <= 0 || s.second <= 0)
             s = k;  // a missing stride means the kernel size
-        out = in[0]->max_pool2d(k, s, int_pair(node, "padding", {0, 0}), nullptr);
+        const Shape xs = run_shape(first);
+        // this pool and the pools folded into it, in order
+        std::vector<PNNXNode *> stages{&node};
+        for (int j = 1; j < node.pool_chain; ++j)
+            for (auto &n : plan_)
+                if (n->folded_into_producer && n->type == "nn.MaxPool2d" && n->input_names[0] == stages.back()->output_names[0])
+                {
+                    stages.push_back(n.get());
+                    break;
+                }
+        if ((int)stages.size() != (node.pool_chain > 0 ? node.pool_chain : 1))
+            THROW_RUNTIME_ERROR("PNNX: node {}: the chain of {} max pools planned at build() is not in the graph", node.name,
+                                node.pool_chain);
+        if (node.pool_chain > 0 && place != placed_.end() && xs.size() == 4 && first.mat->dtype() == DataType::kFloat32 &&
+            xs[2] * xs[3] <= 8192 && k.first <= 15)
+        {
+            // stage j goes to channels [c0 + (j-1)*C, c0 + j*C) of the concatenation: one launch for the whole chain
+            auto buf = buffer_for(place->second.buffer, xs[0], xs[2], xs[3], dev);
+            OriginMat::max_pool_chain(run_of(first), k.first, node.pool_chain,
+                                      OriginMat::ChannelRun{&origin_of(*buf), place->second.c0, xs[1] * (size_t)node.pool_chain});
+            for (size_t j = 0; j < stages.size(); ++j)
+            {
+                Value v;
+                v.mat = buf, v.c0 = place->second.c0 + j * xs[1], v.channels = xs[1], v.run = true;
+                blobs_[stages[j]->output_names[0]] = v;
+            }
+            return;
+        }
+        // one pool after the other, each result copied to its place
+        for (PNNXNode *stage : stages)
+            store(*stage, dense(stage->input_names[0], *stage)->max_pool2d(k, s, int_pair(node, "padding", {0, 0}), nullptr));
+        return;
     }
-    else if (t == "nn.Upsample")
+    if (t == "nn.Upsample")
     {
-        const Shape xs = in[0]->shape();
+        const Shape xs = run_shape(first);
         if (xs.size() != 4)
             THROW_RUNTIME_ERROR("Upsample forward: x must be 4D (N, C, H, W), but got shape {}", xs.to_string());
         size_t OH, OW;
@@ -450,15 +764,137 @@ void PNNXGraph::run(PNNXNode &node)
         const std::string mode = node.params.count("mode") ? node.params.at("mode") : "nearest";
         if (mode != "nearest")
             THROW_RUNTIME_ERROR("PNNX: node {}: upsample mode '{}' is not supported", node.name, mode);
-        out = in[0]->upsample(Shape{xs[0], xs[1], OH, OW}, (int)(OH / xs[2]), (int)(OW / xs[3]), mode);
+        const int sh = (int)(OH / xs[2]), sw = (int)(OW / xs[3]);
+        if ((first.run || place != placed_.end()) && first.mat->dtype() == DataType::kFloat32 && OW % 4 == 0 && sh > 0 && sw > 0)
+        {
+            Value out = destination(xs[0], xs[1], OH, OW);
+            OriginMat::upsample_run(run_of(first), run_of(out), sh, sw);
+            blobs_[out_name] = out;
+            return;
+        }
+        std::shared_ptr<Mat> out = dense(node.input_names[0], node)->upsample(Shape{xs[0], xs[1], OH, OW}, sh, sw, mode);
+        store(node, std::move(out));
+        return;
     }
-    else if (t == "torch.cat")
+    if (t == "torch.cat")
     {
+        const int dim = int_param(node, "dim", 0);
+        auto cc = cat_channels_.find(node.output_names[0]);
+        bool any_placed = false;
+        for (auto &in : node.input_names)
+        {
+            auto pl = placed_.find(in);
+            any_placed = any_placed || (pl != placed_.end() && pl->second.buffer == node.output_names[0]);
+        }
+        if (cc != cat_channels_.end() && any_placed)
+        {
+            // the output exists already, with the placed inputs in it; the others are copied to their channels
+            std::shared_ptr<Mat> buf;
+            size_t c0 = 0;
+            for (auto &in : node.input_names)
+            {
+                Value &v = value(in, node);
+                const Shape s = run_shape(v);
+                if (s.size() != 4)
+                    THROW_RUNTIME_ERROR("PNNX: node {}: input {} is not 4D", node.name, in);
+                if (!buf)
+                    buf = buffer_for(node.output_names[0], s[0], s[2], s[3], dev);
+                const bool in_place = v.run && v.mat == buf && v.c0 == c0;
+                if (!in_place)
+                    OriginMat::copy_run(run_of(v), OriginMat::ChannelRun{&origin_of(*buf), c0, s[1]});
+                c0 += s[1];
+            }
+            if (c0 != cc->second)
+                THROW_RUNTIME_ERROR("PNNX: node {}: the inputs hold {} channels, the plan expected {}", node.name, c0, cc->second);
+            return;  // blobs_[output] is the buffer
+        }
+        std::vector<std::shared_ptr<Mat>> in;
+        for (auto &name : node.input_names)
+            in.push_back(dense(name, node));
         std::vector<const Mat *> others;
         for (size_t i = 1; i < in.size(); ++i)
             others.push_back(in[i].get());
-        out = in[0]->cat(others, int_param(node, "dim", 0));
+        store(node, in[0]->cat(others, dim));
+        return;
     }
+    if (t == "models.yolo.Detect")
+    {
+        // attribute names as PNNX exports them for a three-stage head (operator_mapper.cpp:282-345):
+        // strides pnnx_5; anchor grids pnnx_4/2/0 and grids pnnx_6/3/1 for stages 0/1/2; convolutions m.<stage>.{weight,bias}
+        auto sit = node.attributes.find("pnnx_5");
+        if (sit == node.attributes.end())
+            THROW_RUNTIME_ERROR("YoloDetect: cannot find pnnx_5 (strides) attribute");
+        const std::vector<float> &strides = sit->second.data;
+        if (strides.size() != 3 || node.input_names.size() != 3)
+            THROW_RUNTIME_ERROR("YoloDetect: only supports 3 stages, but got {} strides and {} inputs", strides.size(),
+                                node.input_names.size());
+        static const char *anchor_names[3] = {"pnnx_4", "pnnx_2", "pnnx_0"}, *grid_names[3] = {"pnnx_6", "pnnx_3", "pnnx_1"};
+        std::shared_ptr<Mat> ws[3], bs[3], ags[3], gs[3];
+        size_t rows = 0, ci = 0;
+        bool direct = fusion_;
+        for (int s = 0; s < 3; ++s)
+        {
+            ws[s] = weight("m." + std::to_string(s) + ".weight"), bs[s] = weight("m." + std::to_string(s) + ".bias");
+            ags[s] = weight(anchor_names[s]), gs[s] = weight(grid_names[s]);
+            if (!ws[s] || !bs[s] || !ags[s] || !gs[s])
+                THROW_RUNTIME_ERROR("YoloDetect: stage {} lacks one of weight / bias / anchor grid / grid", s);
+            const int out_ch = (int)ws[s]->shape()[0];
+            if (out_ch % 3 != 0 || out_ch / 3 - 5 <= 0)
+                THROW_RUNTIME_ERROR("YoloDetect: out_channels ({}) must be 3 * (classes + 5)", out_ch);
+            const Shape xs = run_shape(value(node.input_names[s], node));
+            direct = direct && xs.size() == 4 && (ci == 0 || ci == (size_t)out_ch / 3);
+            ci = (size_t)out_ch / 3;
+            if (xs.size() == 4)
+                rows += 3 * xs[2] * xs[3];
+        }
+        if (direct)
+        {
+            // each stage: its 1x1 convolution, then the decoding straight into the stage's rows of the final tensor
+            const size_t N = run_shape(first)[0];
+            std::shared_ptr<Mat> out = std::make_shared<OriginMat>(Shape{N, rows, ci}, DataType::kFloat32, dev);
+            size_t row0 = 0;
+            for (int s = 0; s < 3; ++s)
+            {
+                Value &xv = value(node.input_names[s], node);
+                const Shape xs = run_shape(xv), wsh = ws[s]->shape();
+                Attribute &wa = node.attributes.find("m." + std::to_string(s) + ".weight")->second;
+                if (wa.packed_for != xs.dims())
+                {
+                    wa.packed_mat = OriginMat::conv2d_packed_weights_for(xs, *ws[s], {1, 1}, {0, 0});
+                    wa.packed_for = xs.dims();
+                }
+                std::shared_ptr<Mat> conv;
+                if (wa.packed_mat && OriginMat::conv2d_fused_ok(xs, wsh, {1, 1}, {0, 0}))
+                {
+                    conv = std::make_shared<OriginMat>(Shape{xs[0], wsh[0], xs[2], xs[3]}, DataType::kFloat32, dev);
+                    OriginMat::conv2d_fused(run_of(xv), *wa.packed_mat, wsh, bs[s].get(), {1, 1}, {0, 0}, -1, nullptr,
+                                            OriginMat::whole(*conv));
+                }
+                else
+                    conv = origin_of(*dense(node.input_names[s], node)).conv2d_act(*ws[s], bs[s].get(), {1, 1}, {0, 0}, -1, wa.packed_mat.get());
+                origin_of(*conv).yolo_decode_into(*gs[s], *ags[s], strides[s], 3, (int)ci - 5, *out, row0);
+                row0 += 3 * xs[2] * xs[3];
+            }
+            store(node, std::move(out));
+            return;
+        }
+        std::vector<std::unique_ptr<Mat>> stages;
+        for (int s = 0; s < 3; ++s)
+            stages.push_back(dense(node.input_names[s], node)->yolo_detect_forward(*ws[s], bs[s].get(), *gs[s], *ags[s], strides[s], 3,
+                                                                                  (int)ws[s]->shape()[0] / 3 - 5));
+        std::vector<const Mat *> others{stages[1].get(), stages[2].get()};
+        store(node, stages[0]->cat(others, 1));
+        return;
+    }
+    // the remaining operators work on tensors of their own
+    std::vector<std::shared_ptr<Mat>> in;
+    for (auto &name : node.input_names)
+        in.push_back(dense(name, node));
+    std::shared_ptr<Mat> out;
+    if (t == "nn.SiLU")
+        out = in[0]->silu();
+    else if (t == "nn.ReLU")
+        out = in[0]->relu();
     else if (t == "pnnx.Expression")
     {
         const std::string expr = node.params.count("expr") ? node.params.at("expr") : "unknown";
@@ -499,39 +935,9 @@ void PNNXGraph::run(PNNXNode &node)
         if (auto b = weight("bias"))
             out = *out + *b->broadcast_to(out->shape());
     }
-    else if (t == "models.yolo.Detect")
-    {
-        // attribute names as PNNX exports them for a three-stage head (operator_mapper.cpp:282-345):
-        // strides pnnx_5; anchor grids pnnx_4/2/0 and grids pnnx_6/3/1 for stages 0/1/2; convolutions m.<stage>.{weight,bias}
-        auto sit = node.attributes.find("pnnx_5");
-        if (sit == node.attributes.end())
-            THROW_RUNTIME_ERROR("YoloDetect: cannot find pnnx_5 (strides) attribute");
-        const std::vector<float> &strides = sit->second.data;
-        if (strides.size() != 3 || in.size() != 3)
-            THROW_RUNTIME_ERROR("YoloDetect: only supports 3 stages, but got {} strides and {} inputs", strides.size(),
-                                in.size());
-        static const char *anchor_names[3] = {"pnnx_4", "pnnx_2", "pnnx_0"}, *grid_names[3] = {"pnnx_6", "pnnx_3", "pnnx_1"};
-        std::vector<std::unique_ptr<Mat>> stages;
-        for (int s = 0; s < 3; ++s)
-        {
-            auto w = weight("m." + std::to_string(s) + ".weight"), b = weight("m." + std::to_string(s) + ".bias");
-            auto ag = weight(anchor_names[s]), g = weight(grid_names[s]);
-            if (!w || !b || !ag || !g)
-                THROW_RUNTIME_ERROR("YoloDetect: stage {} lacks one of weight / bias / anchor grid / grid", s);
-            const int out_ch = (int)w->shape()[0];
-            if (out_ch % 3 != 0 || out_ch / 3 - 5 <= 0)
-                THROW_RUNTIME_ERROR("YoloDetect: out_channels ({}) must be 3 * (classes + 5)", out_ch);
-            stages.push_back(in[s]->yolo_detect_forward(*w, b.get(), *g, *ag, strides[s], 3, out_ch / 3 - 5));
-        }
-        std::vector<const Mat *> others{stages[1].get(), stages[2].get()};
-        out = stages[0]->cat(others, 1);
-    }
     else
         THROW_RUNTIME_ERROR("Unsupported operator type: {}", t);
-    if (node.output_names.size() != 1)
-        THROW_RUNTIME_ERROR("PNNX: node {} declares {} outputs; this runner's operators produce one", node.name,
-                            node.output_names.size());
-    blobs_[node.fused_output_name.empty() ? node.output_names[0] : node.fused_output_name] = std::move(out);
+    store(node, std::move(out));
 }
 }  // namespace pnnx
 }  // namespace origin

@@ -644,11 +644,29 @@ int DRV(checkpoint_roundtrip)(const float *params, const char *path, int epoch, 
 // A PNNX model (`.pnnx.param` + `.pnnx.bin`) run forward `reps` times on x[N,C,H,W]; the first output of
 // `pnnx_output_0` is copied to out (capacity in floats) and its shape to out_shape[0..out_nd). ms = mean time of the
 // forwards after the first (which also loads weights), each complete on the device; the output is read back once, after.
+// 0: every node of a PNNX graph runs on its own, as in the reference's runner (only this repository's runner has the
+// switch; the reference's classes ignore it). The launches of the forward recorded last are read back below.
+static int g_pnnx_fusion = 1;
+static int64_t g_pnnx_graph_nodes = 0;
+int DRV(pnnx_set_fusion)(int on)
+{
+    g_pnnx_fusion = on;
+    return 0;
+}
+int DRV(pnnx_last_graph_nodes)(int64_t *nodes)
+{
+    *nodes = g_pnnx_graph_nodes;
+    return 0;
+}
+
 int DRV(pnnx_forward)(const char *param_path, const char *bin_path, const float *x, int64_t N, int64_t C, int64_t H,
                       int64_t W, int reps, float *o, int64_t capacity, int64_t *out_shape, int *out_nd, float *ms)
 {
     return guarded([&] {
         origin::pnnx::PNNXGraph graph(param_path, bin_path);
+#ifdef ORIGINDL_AMD_PNNX_FUSION
+        graph.set_fusion(g_pnnx_fusion != 0);
+#endif
         graph.build();
         auto X = f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
         std::vector<Tensor> outs;
@@ -691,6 +709,9 @@ int DRV(pnnx_forward_graph)(const char *param_path, const char *bin_path, const 
     return guarded([&] {
         StreamScope stream;
         origin::pnnx::PNNXGraph graph(param_path, bin_path);
+#ifdef ORIGINDL_AMD_PNNX_FUSION
+        graph.set_fusion(g_pnnx_fusion != 0);
+#endif
         graph.build();
         const Shape xs{(size_t)N, (size_t)C, (size_t)H, (size_t)W};
         auto X = f32(x, xs);
@@ -701,6 +722,7 @@ int DRV(pnnx_forward_graph)(const char *param_path, const char *bin_path, const 
         recorded.begin_capture();
         graph.forward();
         recorded.end_capture();
+        g_pnnx_graph_nodes = (int64_t)recorded.node_count();
         std::vector<Tensor> outs = graph.get_outputs("pnnx_output_0");
         if (outs.empty())
             throw std::runtime_error("pnnx_forward: the graph produced no output");

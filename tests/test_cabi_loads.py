@@ -39,7 +39,15 @@ def test_workspace_queries_need_no_gpu():
     # a tile count that is a multiple of the CU count needs no K pieces
     assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 3, 3, 1, 1, 1, 1) == wp
     # a 1x1 window's weights are in tap order as they are
-    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 1, 1, 1, 1, 0, 0) == 0
+    assert l.query("odl_hip_conv2d_workspace_bytes", 64, 128, 32, 32, 256, 1, 1, 1, 1, 0, 0) == 0
+    # a small problem (up to 1.6 GFLOP, channels in eights) goes to the kernel that reads its operands straight from
+    # global memory: the workspace holds the filter copy in that kernel's order, whole tiles of 32 filters
+    assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 1, 1, 1, 1, 0, 0) == 128 * 64 * 4
+    assert l.query("odl_hip_conv2d_workspace_bytes", 4, 64, 40, 40, 255, 1, 1, 1, 1, 0, 0) == 256 * 64 * 4
+    assert l.query("odl_hip_conv2d_packed_weights_bytes", 4, 128, 10, 10, 128, 3, 3, 1, 1, 1, 1) == 128 * 128 * 9 * 4
+    assert l.query("odl_hip_conv2d_fused_ok", 4, 128, 10, 10, 128, 3, 3, 1, 1, 1, 1) == 1
+    assert l.query("odl_hip_conv2d_fused_ok", 4, 3, 320, 320, 16, 6, 6, 2, 2, 2, 2) == 0
+    assert l.query("odl_hip_conv2d_fused_ok", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) == 0
     # one input channel under a 3x3 window: the direct kernel, no matrix and no workspace
     assert l.query("odl_hip_conv2d_workspace_bytes", 256, 1, 28, 28, 32, 3, 3, 1, 1, 1, 1) == 0
     # its backward: the weight-gradient partials (one [32][9] block per workgroup) and the reordered filter

@@ -592,6 +592,37 @@ def test_yolov5n_pnnx_forward_at_the_benchmark_size_matches_the_reference(h, tmp
     assert np.isfinite(out).all()
 
 
+def test_pnnx_runner_with_nodes_folded_together_gives_the_floats_of_running_them_one_by_one(h, tmp_path):
+    """The runner folds a residual add into the convolution before it, lets producers write straight into a
+    concatenation's output, runs SPPF's three pools as one launch and decodes each detect stage into its rows of the
+    final tensor. With all of that switched off every node runs on its own, as in the reference's runner
+    (src/pnnx/pnnx_graph.cpp:286-528); the convolutions are the same kernels either way, so the outputs must agree bit
+    for bit — at 64x64 (one image, planes down to 2x2) and at the benchmark's 4 x 320x320. The recorded forward holds
+    66 launches folded against 109 plain (57 + 3 convolutions either way)."""
+    import pnnx_synth
+    for batch, size, seed in ((1, 64, 3), (4, 320, 0)):
+        param, binp, shp = pnnx_synth.write(str(tmp_path / ("y5n%d" % size)), seed=seed, batch=batch, size=size, num_classes=80)
+        x = np.random.default_rng(size).random((batch, 3, size, size), dtype=f32)
+        nodes = {}
+        outs = {}
+        try:
+            for fusion in (1, 0):
+                assert h.odl_host_pnnx_set_fusion(fusion) == 0
+                rc, outs[fusion], _, _ = _run_pnnx(h, "odl_host_", param, binp, x, shp, reps=2)
+                assert rc == 0
+                rc, replayed, _, _ = _run_pnnx(h, "odl_host_", param, binp, x, shp, reps=2, entry="pnnx_forward_graph")
+                assert rc == 0 and np.array_equal(replayed, outs[fusion])
+                n = np.zeros(1, np.int64)
+                assert h.odl_host_pnnx_last_graph_nodes(n) == 0
+                nodes[fusion] = int(n[0])
+        finally:
+            h.odl_host_pnnx_set_fusion(1)
+        print("\n[yolov5n %dx%d] launches per forward: %d folded, %d node by node" % (size, size, nodes[1], nodes[0]), flush=True)
+        assert np.array_equal(outs[1], outs[0])
+        assert np.isfinite(outs[1]).all()
+        assert nodes[1] <= 70 and nodes[0] >= 100
+
+
 def test_pnnx_runner_rejects_bad_files(h, tmp_path):
     import pnnx_synth
     param, binp, shp = pnnx_synth.write(str(tmp_path / "y5n"), seed=1, batch=1, size=32, num_classes=3)

@@ -342,6 +342,19 @@ def test_conv_vs_oracle_seeded(api, o, N, C, H, W, OC, KH, KW, s, p):
     check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p)
 
 
+@pytest.mark.parametrize("N,C,H,W,OC,KH,KW,s,p", [c for c in CONV_SEEDED if c[1] % 8 == 0])
+def test_conv_tiled_forward_kernels_vs_oracle_seeded(api, o, N, C, H, W, OC, KH, KW, s, p):
+    # Small layers whose channels come in groups of eight take the small-problem forward kernel (operands straight from
+    # global memory, K shared between the waves of a workgroup); with it switched off the same shapes reach the tiled
+    # forward kernels that larger layers use (implicit GEMM with and without K slices, the 1x1 product, im2col + GEMM).
+    print("\n[case] conv seeded, tiled forward", N, C, H, W, OC, KH, KW, s, p, flush=True)
+    api.lib().call("odl_hip_set_conv_direct", 0)
+    try:
+        check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p)
+    finally:
+        api.lib().call("odl_hip_set_conv_direct", 1)
+
+
 @pytest.mark.parametrize("N,C,H,W,OC,KH,KW,s,p",
                          [c for c in CONV_SEEDED if c[5:] == (3, 3, 1, 1) and (c[1] % 16 == 0 or c[4] % 16 == 0)])
 def test_conv_lds_patch_kernel_vs_oracle_seeded(api, o, N, C, H, W, OC, KH, KW, s, p):
@@ -350,10 +363,12 @@ def test_conv_lds_patch_kernel_vs_oracle_seeded(api, o, N, C, H, W, OC, KH, KW, 
     # small seeded shapes through it as well.
     print("\n[case] conv seeded, LDS patch", N, C, H, W, OC, flush=True)
     api.lib().call("odl_hip_set_conv_patch_min_workgroups", 0)
+    api.lib().call("odl_hip_set_conv_direct", 0)  # (the small-problem kernel would take these forwards first)
     try:
         check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p)
     finally:
         api.lib().call("odl_hip_set_conv_patch_min_workgroups", -1)
+        api.lib().call("odl_hip_set_conv_direct", 1)
 
 
 def check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p):
@@ -1121,6 +1136,7 @@ def test_yolo_detect_at_detector_size_vs_oracle(api, o):
     np.testing.assert_allclose(got[..., :4], want[..., :4], rtol=2e-5, atol=2e-4)
 
 
+@pytest.mark.parametrize("direct", [1, 0])
 @pytest.mark.parametrize("N,C,H,OC,k,s,p", [
     (2, 16, 14, 24, 3, 1, 1),     # implicit forward, one pass
     (2, 1, 28, 32, 3, 1, 1),      # one input channel: the direct kernel
@@ -1131,26 +1147,172 @@ def test_yolo_detect_at_detector_size_vs_oracle(api, o):
     (4, 64, 56, 128, 3, 1, 1),    # tile count just over a multiple of the CU count: tail pieces and their fix-up
     (2, 64, 20, 128, 1, 1, 0),    # 1x1
 ])
-def test_conv_with_fused_activation_is_conv_then_activation(api, N, C, H, OC, k, s, p):
+def test_conv_with_fused_activation_is_conv_then_activation(api, N, C, H, OC, k, s, p, direct):
+    """direct = 1: the small shapes among these (channels in eights, under 1.6 GFLOP) go through the small-problem
+    kernel; direct = 0: every shape takes the tiled kernel named beside it."""
     rng = np.random.default_rng(41)
     x = dev(rng.standard_normal((N, C, H, H), dtype=f32))
     w = dev((rng.standard_normal((OC, C, k, k), dtype=f32) * f32(np.sqrt(2.0 / (C * k * k)))).astype(f32))
     b = dev(rng.standard_normal(OC, dtype=f32))
-    plain = api.conv2d(x, w, b, s, p)
-    for act in ("silu", "relu"):
-        assert np.array_equal(host(api.conv2d(x, w, b, s, p, activation=act)), host(api.unary(act, plain))), act
-    with pytest.raises(api.OdlInvalidArgument):
-        api.conv2d(x, w, b, s, p, activation="exp")
-    # weights that do not change between calls: the filter copy made once gives the same bits as the per-call copy, and
-    # shapes whose kernel reads the filter as it lies (here: 1x1, few channels, the strided case that goes through the
-    # col matrix) have no such copy
+    api.lib().call("odl_hip_set_conv_direct", direct)
+    try:
+        plain = api.conv2d(x, w, b, s, p)
+        for act in ("silu", "relu"):
+            assert np.array_equal(host(api.conv2d(x, w, b, s, p, activation=act)), host(api.unary(act, plain))), act
+        with pytest.raises(api.OdlInvalidArgument):
+            api.conv2d(x, w, b, s, p, activation="exp")
+        # weights that do not change between calls: the filter copy made once gives the same bits as the per-call copy,
+        # and shapes whose kernel reads the filter as it lies (with the tiled kernels: 1x1, few channels, the strided case
+        # that goes through the col matrix) have no such copy
+        small = C % 8 == 0 and 2 * N * ((H + 2 * p - k) // s + 1) ** 2 * C * k * k * OC <= 3 << 29
+        packed = api.conv2d_pack_weights(x.shape, w, s, p)
+        if direct and small:
+            assert packed is not None and packed.numel() == -(-OC // 32) * 32 * C * k * k
+            # blocks of [lane half][row][4 channels] per (tile of 32 filters, tap, group of 8 channels)
+            wp = np.zeros((-(-OC // 32) * 32, C, k * k), f32)
+            wp[:OC] = host(w).reshape(OC, C, k * k)
+            want = wp.reshape(-1, 32, C // 8, 2, 4, k * k).transpose(0, 5, 2, 3, 1, 4)
+            assert np.array_equal(host(packed), want.reshape(-1))
+        else:
+            assert (packed is not None) == (k == 3 and C % 16 == 0 and not (s == 2 and N == 64))
+            if packed is not None:
+                assert np.array_equal(host(packed), host(w).reshape(OC, C, k * k).transpose(0, 2, 1).reshape(-1))
+        for act in (None, "silu"):
+            assert np.array_equal(host(api.conv2d(x, w, b, s, p, activation=act, packed=packed)),
+                                  host(api.conv2d(x, w, b, s, p, activation=act))), act
+    finally:
+        api.lib().call("odl_hip_set_conv_direct", 1)
+
+
+@pytest.mark.parametrize("N,C,H,W,OC,k,s,p", [
+    (4, 64, 20, 20, 64, 1, 1, 0),     # K shared by four waves
+    (4, 256, 10, 10, 128, 1, 1, 0),   # sixteen K shares
+    (4, 32, 80, 80, 16, 1, 1, 0),     # half a filter tile, two pixel tiles a workgroup
+    (2, 64, 40, 40, 255, 1, 1, 0),    # a detect head: the last filter tile one row short
+    (4, 16, 160, 160, 32, 3, 2, 1),   # stride 2, two K shares of one channel group
+    (4, 128, 10, 10, 128, 3, 1, 1),   # long K over few pixels
+    (3, 24, 9, 13, 40, 3, 1, 1),      # three channel groups (no share divides them), ragged pixel and filter tiles
+    (1, 8, 5, 5, 8, 3, 1, 1),         # a single pixel tile, a single group per tap
+    (2, 16, 12, 12, 24, 5, 1, 2),     # 5x5: depth 4 over 25 taps x 2 groups
+    (2, 32, 14, 10, 48, 3, 2, 0),     # stride 2 without padding
+    (1, 1024, 4, 4, 64, 1, 1, 0),     # 128 channel groups: eight per share
+])
+def test_conv_fused_into_channel_runs_equals_the_nodes_one_by_one(api, o, N, C, H, W, OC, k, s, p):
+    """odl_hip_conv2d_fused with its input, output and residual each a run of channels of a wider tensor: the result
+    must be, bit for bit, what the nodes give one after the other on tensors of their own — convolution (the same
+    kernel, through odl_hip_conv2d), activation, add, and the copy into the concatenation — and must leave the rest of
+    the wider output untouched. The convolution itself is held to the oracle by the seeded cases above."""
+    print("\n[case] conv fused", N, C, H, W, OC, k, s, p, flush=True)
+    rng = np.random.default_rng(C * 7 + OC)
+    assert api.conv2d_fused_ok((N, C, H, W), (OC, C, k, k), s, p)
+    OH, OW = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+    xbuf = dev(rng.standard_normal((N, C + 24, H, W), dtype=f32))
+    rbuf = dev(rng.standard_normal((N, OC + 8, OH, OW), dtype=f32))
+    ybuf0 = rng.standard_normal((N, OC + 40, OH, OW), dtype=f32)
+    w = dev((rng.standard_normal((OC, C, k, k), dtype=f32) * f32(np.sqrt(2.0 / (C * k * k)))).astype(f32))
+    b = dev(rng.standard_normal(OC, dtype=f32))
+    xr, rr = xbuf[:, 16:16 + C], rbuf[:, 8:8 + OC]
+    x, r = xr.contiguous(), rr.contiguous()
     packed = api.conv2d_pack_weights(x.shape, w, s, p)
-    assert (packed is not None) == (k == 3 and C % 16 == 0 and not (s == 2 and N == 64))
-    if packed is not None:
-        assert np.array_equal(host(packed), host(w).reshape(OC, C, k * k).transpose(0, 2, 1).reshape(w.shape))
-    for act in (None, "silu"):
-        assert np.array_equal(host(api.conv2d(x, w, b, s, p, activation=act, packed=packed)),
-                              host(api.conv2d(x, w, b, s, p, activation=act))), act
+    for act in (None, "silu", "relu"):
+        for with_res in (False, True):
+            for with_bias in (True, False):
+                ybuf = dev(ybuf0)
+                api.conv2d_fused(xr, w.shape, packed, b if with_bias else None, ybuf[:, 32:32 + OC], s, p, act,
+                                 rr if with_res else None)
+                step = api.conv2d(x, w, b if with_bias else None, s, p)
+                if act:
+                    step = api.unary(act, step)
+                if with_res:
+                    step = api.binary("add", r, step)
+                want = ybuf0.copy()
+                want[:, 32:32 + OC] = host(step)
+                assert np.array_equal(host(ybuf), want), (act, with_res, with_bias)
+    # dense operands (image strides 0) are the same call
+    y = dev(np.zeros((N, OC, OH, OW), f32))
+    api.conv2d_fused(x, w.shape, packed, b, y, s, p, "silu", r)
+    assert np.array_equal(host(y), host(api.binary("add", r, api.unary("silu", api.conv2d(x, w, b, s, p)))))
+    # against the oracle too, so that this test stands on its own
+    yo = np.empty((N, OC, OH, OW), f32)
+    assert o.orc_conv2d(host(x), host(w), host(b), N, C, H, W, OC, k, k, s, s, p, p, yo) == 0
+    by, _, _ = conv_bounds(host(x), host(w), np.zeros((N, OC, OH, OW), f32), (s, s), (p, p), o)
+    assert (np.abs(host(api.conv2d(x, w, b, s, p)) - yo) <= by + 1e-6).all()
+
+
+def test_conv_fused_refuses_what_it_does_not_cover(api):
+    assert not api.conv2d_fused_ok((2, 3, 64, 64), (16, 3, 6, 6), 2, 2)        # three channels
+    assert not api.conv2d_fused_ok((32, 64, 56, 56), (128, 64, 3, 3), 1, 1)    # 14.8 GFLOP: the tiled kernels' work
+    x, y = dev(np.zeros((2, 12, 8, 8), f32)), dev(np.zeros((2, 16, 8, 8), f32))
+    with pytest.raises(api.OdlInvalidArgument):
+        api.conv2d_fused(x, (16, 12, 1, 1), dev(np.zeros(16 * 12, f32)), None, y, 1, 0)
+    x = dev(np.zeros((2, 16, 8, 8), f32))
+    w = dev(np.ones((16, 16, 1, 1), f32))
+    packed = api.conv2d_pack_weights(x.shape, w, 1, 0)
+    with pytest.raises(api.OdlInvalidArgument):  # an image stride shorter than the image
+        api.lib().call("odl_hip_conv2d_fused", x.data_ptr(), 100, packed.data_ptr(), None, 2, 16, 8, 8, 16, 1, 1, 1, 1, 0, 0, -1,
+                       None, 0, y.data_ptr(), 0, None)
+    with pytest.raises(api.OdlInvalidArgument):
+        api.conv2d_fused(x, w.shape, packed, None, y, 1, 0, "exp")
+
+
+def test_detector_operators_on_channel_runs_are_the_dense_operators(api, o):
+    """upsample, the SPPF chain of max pools, the image copy and the detect decoding, reading and writing runs of
+    channels (rows, for the decoding) of wider tensors: bit-identical to the dense entry points."""
+    rng = np.random.default_rng(77)
+    # upsample: [4, 128, 10, 10] out of a 160-channel tensor into channels 64.. of a 256-channel one
+    src = dev(rng.standard_normal((4, 160, 10, 10), dtype=f32))
+    dst0 = rng.standard_normal((4, 256, 20, 20), dtype=f32)
+    dst = dev(dst0)
+    api.upsample_view(src[:, 32:160], dst[:, 64:192], 2)
+    want = dst0.copy()
+    want[:, 64:192] = host(api.upsample(src[:, 32:160].contiguous(), 2))
+    assert np.array_equal(host(dst), want)
+    for (N, C, H, W, sh, sw) in ((2, 3, 5, 6, 2, 2), (1, 2, 7, 4, 3, 1), (3, 1, 2, 5, 2, 4)):
+        xs = dev(rng.standard_normal((N, C, H, W), dtype=f32))
+        ys = dev(np.zeros((N, C + 2, H * sh, W * sw), f32))
+        api.upsample_view(xs, ys[:, 1:1 + C], (sh, sw))
+        assert np.array_equal(host(ys)[:, 1:1 + C], host(api.upsample(xs, (sh, sw)))), (N, C, H, W, sh, sw)
+    # SPPF: x = channels 0..128 of the 512-channel concatenation itself, three 5x5 pools into channels 128..512
+    for (N, C, H, W, K, count) in ((4, 128, 10, 10, 5, 3), (2, 5, 7, 9, 3, 2), (1, 3, 20, 20, 9, 1), (2, 4, 1, 1, 5, 3)):
+        buf0 = rng.standard_normal((N, (count + 1) * C, H, W), dtype=f32)
+        buf = dev(buf0)
+        api.max_pool2d_chain(buf[:, :C], K, count, buf[:, C:])
+        want, cur = buf0.copy(), dev(np.ascontiguousarray(buf0[:, :C]))
+        for j in range(count):
+            cur, _ = api.max_pool2d(cur, K, 1, K // 2, with_indices=False)
+            want[:, (j + 1) * C:(j + 2) * C] = host(cur)
+        assert np.array_equal(host(buf), want), (N, C, H, W, K, count)
+    with pytest.raises(api.OdlInvalidArgument):
+        api.max_pool2d_chain(dev(np.zeros((1, 1, 8, 8), f32)), 4, 1, dev(np.zeros((1, 1, 8, 8), f32)))  # even window
+    with pytest.raises(api.OdlInvalidArgument):
+        api.max_pool2d_chain(dev(np.zeros((1, 1, 100, 100), f32)), 3, 1, dev(np.zeros((1, 1, 100, 100), f32)))  # plane too large
+    # image copy in both directions, runs that are and are not multiples of four floats
+    for (N, C, H, W) in ((4, 64, 20, 20), (3, 5, 3, 7)):
+        a0 = rng.standard_normal((N, C + 3, H, W), dtype=f32)
+        a, d = dev(a0), dev(np.zeros((N, C + 9, H, W), f32))
+        api.copy_images(a[:, 2:2 + C], d[:, 4:4 + C])
+        want = np.zeros((N, C + 9, H, W), f32)
+        want[:, 4:4 + C] = a0[:, 2:2 + C]
+        assert np.array_equal(host(d), want)
+        back = dev(np.zeros((N, C, H, W), f32))
+        api.copy_images(d[:, 4:4 + C], back)
+        assert np.array_equal(host(back), a0[:, 2:2 + C])
+    # detect: decoding into the stage's rows of the concatenated output = the dense call's decoding
+    N, C, H, W, A, NC = 4, 64, 20, 20, 3, 80
+    CI = NC + 5
+    x = dev(rng.standard_normal((N, C, H, W), dtype=f32))
+    w = dev((rng.standard_normal((A * CI, C, 1, 1), dtype=f32) * f32(0.2)).astype(f32))
+    b = dev(rng.standard_normal(A * CI, dtype=f32))
+    gyy, gxx = np.meshgrid(np.arange(H), np.arange(W), indexing="ij")
+    grid = dev(np.broadcast_to(np.stack([gxx, gyy], -1).astype(f32) - f32(0.5), (1, A, H, W, 2)).copy())
+    ag = dev(np.broadcast_to(np.array([[10, 13], [16, 30], [33, 23]], f32).reshape(1, A, 1, 1, 2), (1, A, H, W, 2)).copy())
+    dense = host(api.yolo_detect_forward(x, w, b, grid, ag, 16.0, A, NC))
+    out0 = rng.standard_normal((N, 500 + A * H * W + 70, CI), dtype=f32)
+    out = dev(out0)
+    api.yolo_decode(api.conv2d(x, w, b, 1, 0), grid, ag, 16.0, A, NC, out[:, 500:500 + A * H * W])
+    want = out0.copy()
+    want[:, 500:500 + A * H * W] = dense
+    assert np.array_equal(host(out), want)
 
 
 # ------------------------------------------------------------------ element types besides float32
