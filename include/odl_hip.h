@@ -188,6 +188,17 @@ int odl_hip_conv2d_fused(const float *x, int64_t x_image_stride, const float *pa
                          int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int activation,
                          const float *residual, int64_t residual_image_stride, float *y, int64_t y_image_stride,
                          void *stream);
+/* Two convolutions over the same input with the same window, stride, padding and activation (the cv1 / cv2 pair of a
+ * detector's C3 block: two nn.Conv2d nodes reading one tensor) run as one: `packed` and b hold the two filters and
+ * biases one after the other ([OC, C, KH, KW] packed by odl_hip_conv2d_pack_weights for OC filters, b[OC]); the outputs
+ * of filters [0, split) go to y_first [N, split, OH, OW], those of filters [split, OC) to y_second [N, OC - split, OH, OW],
+ * each with its own image stride. K is shared between waves as for the member with more filters alone, so two members
+ * of equal size (the C3 case) give the floats of two odl_hip_conv2d_fused calls, bit for bit. Covered shapes:
+ * odl_hip_conv2d_fused_ok(..., OC, ...). */
+int odl_hip_conv2d_fused_pair(const float *x, int64_t x_image_stride, const float *packed, const float *b, int64_t N, int64_t C,
+                              int64_t H, int64_t W, int64_t OC, int64_t split, int KH, int KW, int SH, int SW, int PH, int PW,
+                              int activation, float *y_first, int64_t y_first_image_stride, float *y_second,
+                              int64_t y_second_image_stride, void *stream);
 /* Measurement switches, for the whole process (same caveat as above: never between a query and its call):
  * set_conv_direct(0) sends the small problems to the tiled kernels again; set_conv_direct_plan(k_shares, pixel_tiles)
  * fixes how a workgroup of the small-problem kernel is cut (0, 0: its own rule). No counterpart in the reference. */

@@ -89,11 +89,11 @@ size_t sum_nchw_channels_workspace(int64_t N, int64_t OC, int64_t P);
 // input, output and residual may be channel slices of wider tensors
 bool conv_direct_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW,
                     int64_t OH, int64_t OW);
-size_t conv_direct_packed_bytes(int64_t C, int64_t OC, int KH, int KW);
-int conv_direct_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, hipStream_t st);
+size_t conv_direct_packed_bytes(int64_t C, int64_t OC, int KH, int KW, int P, int64_t W);
+int conv_direct_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, int P, int64_t W, float *packed, hipStream_t st);
 int conv_direct(const float *x, int64_t x_bs, const float *packed, const float *b, const float *res, int64_t res_bs, float *y,
                 int64_t y_bs, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int S, int P, int64_t OH,
-                int64_t OW, int act, hipStream_t st);
+                int64_t OW, int act, hipStream_t st, float *y2 = nullptr, int64_t y2_bs = 0, int64_t split = 0);
 }  // namespace odl
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -1169,7 +1169,7 @@ size_t odl_hip_conv2d_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W
     if (OH <= 0 || OW <= 0)
         return 0;
     if (g_direct.load(std::memory_order_relaxed) && odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW))
-        return align256(odl::conv_direct_packed_bytes(C, OC, KH, KW));  // the filter copy of a caller that keeps none
+        return align256(odl::conv_direct_packed_bytes(C, OC, KH, KW, PH, W));  // the filter copy of a caller that keeps none
     if (odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, OH, OW))
         return 0;
     if (odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW))
@@ -1201,7 +1201,7 @@ size_t odl_hip_conv2d_packed_weights_bytes(int64_t N, int64_t C, int64_t H, int6
     const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
     if (OH > 0 && OW > 0 && g_direct.load(std::memory_order_relaxed) &&
         odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW))
-        return odl::conv_direct_packed_bytes(C, OC, KH, KW);
+        return odl::conv_direct_packed_bytes(C, OC, KH, KW, PH, W);
     if (OH <= 0 || OW <= 0 || odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, OH, OW) ||
         !odl::conv_implicit_forward_ok(kAlignedProbe, N, C, H, W, OC, KH, KW, OH, OW) ||
         forward_by_col_matrix(N, C, OC, KH, KW, SH, SW, OH, OW))
@@ -1218,7 +1218,7 @@ int odl_hip_conv2d_pack_weights(const float *w, int64_t N, int64_t C, int64_t H,
                 "conv2d_pack_weights: a forward over this shape reads the filter as it lies");
     const int64_t OH = outsize(H, KH, SH, PH), OW = outsize(W, KW, SW, PW);
     if (g_direct.load(std::memory_order_relaxed) && odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW))
-        return odl::conv_direct_pack(w, C, OC, KH, KW, packed, odl::as_stream(stream));
+        return odl::conv_direct_pack(w, C, OC, KH, KW, PH, W, packed, odl::as_stream(stream));
     return odl::conv_implicit_forward_pack(w, C, OC, KH, KW, packed, odl::as_stream(stream));
 }
 
@@ -1245,10 +1245,10 @@ int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packe
         if (packed == nullptr)
         {
             // a caller that keeps no filter copy: one is made in the workspace first
-            const size_t need = odl::conv_direct_packed_bytes(C, OC, KH, KW);
+            const size_t need = odl::conv_direct_packed_bytes(C, OC, KH, KW, PH, W);
             ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0,
                         "conv2d: this shape needs a 16-byte aligned workspace of %zu bytes, got %zu", need, workspace_bytes);
-            rc = odl::conv_direct_pack(w, C, OC, KH, KW, static_cast<float *>(workspace), st);
+            rc = odl::conv_direct_pack(w, C, OC, KH, KW, PH, W, static_cast<float *>(workspace), st);
             if (rc != ODL_OK)
                 return rc;
             packed = static_cast<const float *>(workspace);
@@ -1324,6 +1324,36 @@ int odl_hip_conv2d_fused(const float *x, int64_t x_image_stride, const float *pa
     const int act = activation == 0 ? 1 : (activation == 7 ? 2 : 0);
     return odl::conv_direct(x, x_image_stride, packed, b, residual, residual_image_stride, y, y_image_stride, N, C, H, W, OC,
                             KH, KW, SH, PH, g.OH, g.OW, act, odl::as_stream(stream));
+}
+
+int odl_hip_conv2d_fused_pair(const float *x, int64_t x_image_stride, const float *packed, const float *b, int64_t N, int64_t C,
+                              int64_t H, int64_t W, int64_t OC, int64_t split, int KH, int KW, int SH, int SW, int PH, int PW,
+                              int activation, float *y_first, int64_t y_first_image_stride, float *y_second,
+                              int64_t y_second_image_stride, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(activation == -1 || activation == 0 || activation == 7,
+                "conv2d: activation must be -1 (none), 0 (relu) or 7 (silu), the unary operator numbers; got %d", activation);
+    ConvGeom g;
+    int rc = make_geom(g, "conv2d", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(x && packed && y_first && y_second, "conv2d_fused_pair: null operand");
+    ODL_REQUIRE(split > 0 && split < OC, "conv2d_fused_pair: the first convolution's filter count (%lld) must lie inside (0, %lld)",
+                (long long)split, (long long)OC);
+    if (N == 0)
+        return ODL_OK;
+    ODL_REQUIRE(odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW),
+                "conv2d_fused_pair: shape not covered (ask odl_hip_conv2d_fused_ok with the two filter counts added)");
+    const int64_t plane = g.OH * g.OW;
+    ODL_REQUIRE((x_image_stride == 0 || x_image_stride >= C * H * W) && (y_first_image_stride == 0 || y_first_image_stride >= split * plane) &&
+                    (y_second_image_stride == 0 || y_second_image_stride >= (OC - split) * plane),
+                "conv2d_fused_pair: an image stride is shorter than the image it strides over");
+    ODL_REQUIRE(x_image_stride < (1ll << 40) && y_first_image_stride < (1ll << 40) && y_second_image_stride < (1ll << 40),
+                "conv2d_fused_pair: image stride too large");
+    const int act = activation == 0 ? 1 : (activation == 7 ? 2 : 0);
+    return odl::conv_direct(x, x_image_stride, packed, b, nullptr, 0, y_first, y_first_image_stride, N, C, H, W, OC, KH, KW, SH, PH,
+                            g.OH, g.OW, act, odl::as_stream(stream), y_second, y_second_image_stride, split);
 }
 
 int odl_hip_conv2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,

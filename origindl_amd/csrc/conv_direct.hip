@@ -25,8 +25,9 @@ namespace
 struct DirectArgs
 {
     const float *x, *w, *bias, *res;
-    float *y;
-    int64_t x_bs, y_bs, res_bs;  // floats from one image to the next
+    float *y, *y2;               // filters [0, split) go to y, filters [split, OC) to y2 (two convolutions run as one)
+    int64_t x_bs, y_bs, y2_bs, res_bs;  // floats from one image to the next
+    int split;
     int C, H, W, OC, OH, OW, KH, KW, S, P;
     int M;             // N * OH * OW output pixels
     int act;           // 0 none, 1 relu, 2 silu
@@ -72,7 +73,7 @@ __device__ __forceinline__ void direct_epilogue(const DirectArgs &g, const float
     const int nthreads = 64 * g.KS * g.WP;
     int64_t off[E];
     float res[E], v[E];
-    bool ok[E];
+    bool ok[E], second[E];
 #pragma unroll
     for (int i = 0; i < E; ++i)
     {
@@ -83,7 +84,8 @@ __device__ __forceinline__ void direct_epilogue(const DirectArgs &g, const float
         const unsigned mc = ok[i] ? (unsigned)mm : 0u;
         const unsigned nn = odl::fastdiv(mc, g.d_ohw), px = mc - nn * (unsigned)OHW;
         const int64_t o = (int64_t)(ok[i] ? oc : 0) * OHW + px;
-        off[i] = (int64_t)nn * g.y_bs + o;
+        second[i] = oc >= g.split;
+        off[i] = second[i] ? (int64_t)nn * g.y2_bs + o - (int64_t)g.split * OHW : (int64_t)nn * g.y_bs + o;
         if (RES)
             res[i] = g.res[(int64_t)nn * g.res_bs + o];
     }
@@ -103,7 +105,69 @@ __device__ __forceinline__ void direct_epilogue(const DirectArgs &g, const float
 #pragma unroll
     for (int i = 0; i < E; ++i)
         if (ok[i])
-            g.y[off[i]] = v[i];
+            (second[i] ? g.y2 : g.y)[off[i]] = v[i];
+}
+
+// What follows the K loop: the tile's sums (this wave's share of K in acc) to their places in y.
+template <bool RES>
+__device__ __forceinline__ void direct_finish(const DirectArgs &g, const f32x16 &acc, float bias_v, float *bias_s, float *partial,
+                                              int wv, int pt, int l32, int half, int m_base, int oc0, int OHW, unsigned n, unsigned r)
+{
+    ODL_DIRECT_STAMP(3);
+    if (threadIdx.x < 32)
+        bias_s[threadIdx.x] = bias_v;
+    if (g.KS == 1)
+    {
+        // accumulator register q of a lane: row 8*(q/4) + 4*half + q%4, column l32
+        __syncthreads();  // the bias rows
+        const int mm = m_base + pt * 32 + l32;
+        if (mm < g.M)
+        {
+            const int64_t pix = (int64_t)r;
+            float *yp = g.y + (int64_t)n * g.y_bs + pix;
+            float *yp2 = g.y2 + (int64_t)n * g.y2_bs + pix - (int64_t)g.split * OHW;
+            float rv[16];
+            if (RES)
+            {
+                // (a row past OC reads the last row's residual and is not stored)
+                const float *rp = g.res + (int64_t)n * g.res_bs + pix;
+#pragma unroll
+                for (int q = 0; q < 16; ++q)
+                {
+                    const int oc = oc0 + 8 * (q / 4) + 4 * half + (q % 4);
+                    rv[q] = rp[(int64_t)(oc < g.OC ? oc : g.OC - 1) * OHW];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 16; ++q)
+            {
+                const int rr = 8 * (q / 4) + 4 * half + (q % 4);
+                float v = odl::apply_act(acc[q] + bias_s[rr], g.act);
+                if (RES)
+                    v = rv[q] + v;
+                if (oc0 + rr < g.OC)
+                    (oc0 + rr >= g.split ? yp2 : yp)[(int64_t)(oc0 + rr) * OHW] = v;
+            }
+        }
+        ODL_DIRECT_STAMP(5);
+        return;
+    }
+    float *mine = partial + (size_t)wv * 32 * kPitch;
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+        mine[(8 * (q / 4) + 4 * half + (q % 4)) * kPitch + l32] = acc[q];
+    __syncthreads();
+    ODL_DIRECT_STAMP(4);
+    // 1024 outputs a pixel tile over 64 * KS * WP threads: 16 / KS outputs a thread
+    if (g.KS == 2)
+        direct_epilogue<8, RES>(g, partial, bias_s, m_base, oc0, OHW);
+    else if (g.KS == 4)
+        direct_epilogue<4, RES>(g, partial, bias_s, m_base, oc0, OHW);
+    else if (g.KS == 8)
+        direct_epilogue<2, RES>(g, partial, bias_s, m_base, oc0, OHW);
+    else
+        direct_epilogue<1, RES>(g, partial, bias_s, m_base, oc0, OHW);
+    ODL_DIRECT_STAMP(5);
 }
 
 // kDepth: operand groups in flight per wave. Every load instruction costs the compute unit's one address unit 16
@@ -186,60 +250,112 @@ __global__ __launch_bounds__(1024) void conv_direct_kernel(DirectArgs g)
     for (int d = 0; d < kDepth; ++d)
         if (d < rem)
             use(d);
-    ODL_DIRECT_STAMP(3);
-    if (threadIdx.x < 32)
-        bias_s[threadIdx.x] = bias_v;
-    if (g.KS == 1)
+    direct_finish<RES>(g, acc, bias_v, bias_s, partial, wv, pt, l32, half, m_base, oc0, OHW, n, r);
+}
+
+// 3x3 windows with padding 1 (stride 1 or 2, rows of three pixels or more): the three taps of a window row are three
+// consecutive input floats, so a lane fetches them with one 12-byte load and they feed three MFMAs, whose filter
+// values — w[row][c][kh][0..2] — are one 16-byte load from a copy laid out [tile of 32 filters][channel pair][kh] x
+// [lane half][row][kw, one pad]. A lane half is one channel of the pair. Two load instructions per three MFMAs instead
+// of five per four: the compute unit's address unit, which every load occupies for 16 clocks, stops being the
+// limit. A window that hangs over the left or right edge loads the three floats next to it and shifts them.
+constexpr int kDepth3 = 6;
+typedef float f32x3 __attribute__((ext_vector_type(3)));
+
+template <bool RES>
+__global__ __launch_bounds__(1024) void conv_direct3_kernel(DirectArgs g)
+{
+    extern __shared__ float lds[];  // bias[32], then partial[WP * KS][32][kPitch] when KS > 1
+    float *bias_s = lds, *partial = lds + 32;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int pt = wv / g.KS, ks = wv - pt * g.KS;
+    const unsigned bid = blockIdx.x;
+    const int oct = (int)(bid % (unsigned)g.octiles);
+    const int m_base = (int)(bid / (unsigned)g.octiles) * 32 * g.WP;
+    const int oc0 = oct * 32;
+    const int HW = g.H * g.W, OHW = g.OH * g.OW;
+    const float bias_v = (threadIdx.x < 32 && g.bias && oc0 + (int)threadIdx.x < g.OC) ? g.bias[oc0 + threadIdx.x] : 0.f;
+    int m = m_base + pt * 32 + l32;
+    m = m < g.M ? m : g.M - 1;
+    const unsigned n = odl::fastdiv((unsigned)m, g.d_ohw), r = (unsigned)m - n * (unsigned)OHW;
+    const int oh = (int)odl::fastdiv(r, g.d_ow), ow = (int)r - oh * g.OW;
+    const int ih0 = oh * g.S - 1, iw0 = ow * g.S - 1;
+    // the window's three columns iw0 .. iw0+2: read from iwb .. iwb+2, which lie inside the row
+    const int shift = iw0 < 0 ? 1 : (iw0 + 2 >= g.W ? 2 : 0);
+    const int iwb = shift == 1 ? 0 : (shift == 2 ? g.W - 3 : iw0);
+    const int pairs = g.C >> 1;                 // channel pairs; this wave's are [pair0, pair0 + 4 * chunks)
+    const int pair0 = ks * g.chunks * 4;
+    const float *xb = g.x + (int64_t)n * g.x_bs + (int64_t)(2 * pair0 + half) * HW + iwb;
+    const float *wb = g.w + ((int64_t)oct * pairs + pair0) * 768 + lane * 4;
+    const int total = 12 * g.chunks;            // groups: (channel pair, window row)
+    f32x4 fa[kDepth3];
+    f32x3 fb[kDepth3];
+    bool fok[kDepth3];
+    auto load = [&](int slot, int q) {
+        q = q < total ? q : total - 1;
+        const int pr = (int)(((unsigned)q * 43691u) >> 17), kh = q - 3 * pr;  // q / 3 for q < 98304
+        const int ih = ih0 + kh;
+        fok[slot] = (unsigned)ih < (unsigned)g.H;
+        const int ihc = ih < 0 ? 0 : (ih >= g.H ? g.H - 1 : ih);
+        const float *px = xb + (int64_t)pr * 2 * HW + ihc * g.W;
+        fa[slot] = *reinterpret_cast<const f32x4 *>(wb + (int64_t)q * 256);
+        fb[slot] = f32x3{px[0], px[1], px[2]};
+    };
+    f32x16 acc = {0};
+    auto use = [&](int slot) {
+        const f32x4 a = fa[slot];
+        const f32x3 v = fb[slot];
+        const bool ok = fok[slot];
+        // the window's columns out of the three floats read (a column in the padding is zero)
+        const float b0 = (ok && shift != 1) ? (shift == 2 ? v.y : v.x) : 0.f;
+        const float b1 = ok ? (shift == 1 ? v.x : (shift == 2 ? v.z : v.y)) : 0.f;
+        const float b2 = (ok && shift != 2) ? (shift == 1 ? v.y : v.z) : 0.f;
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b1, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b2, acc, 0, 0, 0);
+    };
+#pragma unroll
+    for (int d = 0; d < kDepth3; ++d)
+        load(d, d);  // (total is a multiple of 12)
+    int it = 0;
+    for (; it + kDepth3 < total; it += kDepth3)
     {
-        // accumulator register q of a lane: row 8*(q/4) + 4*half + q%4, column l32
-        __syncthreads();  // the bias rows
-        const int mm = m_base + pt * 32 + l32;
-        if (mm < g.M)
+#pragma unroll
+        for (int d = 0; d < kDepth3; ++d)
         {
-            const int64_t pix = (int64_t)r;
-            float *yp = g.y + (int64_t)n * g.y_bs + pix;
-            float rv[16];
-            if (RES)
-            {
-                // (a row past OC reads the last row's residual and is not stored)
-                const float *rp = g.res + (int64_t)n * g.res_bs + pix;
-#pragma unroll
-                for (int q = 0; q < 16; ++q)
-                {
-                    const int oc = oc0 + 8 * (q / 4) + 4 * half + (q % 4);
-                    rv[q] = rp[(int64_t)(oc < g.OC ? oc : g.OC - 1) * OHW];
-                }
-            }
-#pragma unroll
-            for (int q = 0; q < 16; ++q)
-            {
-                const int rr = 8 * (q / 4) + 4 * half + (q % 4);
-                float v = odl::apply_act(acc[q] + bias_s[rr], g.act);
-                if (RES)
-                    v = rv[q] + v;
-                if (oc0 + rr < g.OC)
-                    yp[(int64_t)(oc0 + rr) * OHW] = v;
-            }
+            use(d);
+            load(d, it + d + kDepth3);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        ODL_DIRECT_STAMP(5);
-        return;
     }
-    float *mine = partial + (size_t)wv * 32 * kPitch;
 #pragma unroll
-    for (int q = 0; q < 16; ++q)
-        mine[(8 * (q / 4) + 4 * half + (q % 4)) * kPitch + l32] = acc[q];
-    __syncthreads();
-    ODL_DIRECT_STAMP(4);
-    // 1024 outputs a pixel tile over 64 * KS * WP threads: 16 / KS outputs a thread
-    if (g.KS == 2)
-        direct_epilogue<8, RES>(g, partial, bias_s, m_base, oc0, OHW);
-    else if (g.KS == 4)
-        direct_epilogue<4, RES>(g, partial, bias_s, m_base, oc0, OHW);
-    else if (g.KS == 8)
-        direct_epilogue<2, RES>(g, partial, bias_s, m_base, oc0, OHW);
-    else
-        direct_epilogue<1, RES>(g, partial, bias_s, m_base, oc0, OHW);
-    ODL_DIRECT_STAMP(5);
+    for (int d = 0; d < kDepth3; ++d)
+        use(d);
+    direct_finish<RES>(g, acc, bias_v, bias_s, partial, wv, pt, l32, half, m_base, oc0, OHW, n, r);
+}
+
+// wd[(((tile * pairs + pair) * 3 + kh) * 64 + half * 32 + row) * 4 + kw] = w[tile*32 + row][2*pair + half][kh][kw], kw < 3
+// (the fourth float of a lane and rows past OC are zero)
+__global__ void pack_direct3_kernel(const float *__restrict__ w, float *__restrict__ wd, int C, int OC, int64_t total)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    const int kw = (int)(t & 3), row = (int)((t >> 2) & 31), half = (int)((t >> 7) & 1);
+    int64_t blk = t >> 8;
+    const int kh = (int)(blk % 3);
+    blk /= 3;
+    const int pairs = C / 2;
+    const int pair = (int)(blk % pairs), tile = (int)(blk / pairs);
+    const int oc = tile * 32 + row, c = 2 * pair + half;
+    wd[t] = (oc < OC && kw < 3) ? w[(((int64_t)oc * C + c) * 3 + kh) * 3 + kw] : 0.f;
+}
+
+// the 3x3 kernel above takes windows of 3x3 with padding 1 over rows of at least three pixels
+inline bool direct_rows3(int KH, int KW, int P, int64_t W)
+{
+    return KH == 3 && KW == 3 && P == 1 && W >= 3;
 }
 
 int g_force_ks = 0, g_force_wp = 0;  // measurement overrides (0: the rule below)
@@ -281,34 +397,44 @@ bool conv_direct_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int 
     return 2 * M * K * OC <= (3ll << 29);
 }
 
-size_t conv_direct_packed_bytes(int64_t C, int64_t OC, int KH, int KW)
+size_t conv_direct_packed_bytes(int64_t C, int64_t OC, int KH, int KW, int P, int64_t W)
 {
-    return (size_t)(ceil_div(OC, 32) * 32 * C * KH * KW) * sizeof(float);
+    const int per_channel = direct_rows3(KH, KW, P, W) ? 12 : KH * KW;  // (window rows padded to four floats)
+    return (size_t)(ceil_div(OC, 32) * 32 * C * per_channel) * sizeof(float);
 }
 
-int conv_direct_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, float *packed, hipStream_t st)
+int conv_direct_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, int P, int64_t W, float *packed, hipStream_t st)
 {
-    const int64_t total = ceil_div(OC, 32) * 32 * C * KH * KW;
+    const int64_t total = (int64_t)(conv_direct_packed_bytes(C, OC, KH, KW, P, W) / sizeof(float));
     ODL_REQUIRE(total < (1ll << 31) && C % 8 == 0, "conv2d: filter too large or channels not a multiple of 8");
-    hipLaunchKernelGGL(pack_direct_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, w, packed, (int)C, (int)OC,
-                       KH * KW, total);
+    if (direct_rows3(KH, KW, P, W))
+        hipLaunchKernelGGL(pack_direct3_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, w, packed, (int)C, (int)OC, total);
+    else
+        hipLaunchKernelGGL(pack_direct_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, w, packed, (int)C, (int)OC,
+                           KH * KW, total);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }
 
 // x, y, residual: NCHW with x_bs / y_bs / res_bs floats from one image to the next (0: dense). packed: the filter as
-// conv_direct_pack lays it out (16-byte aligned).
+// conv_direct_pack lays it out (16-byte aligned). y2 (optional): the outputs of filters [split, OC) go there instead.
 int conv_direct(const float *x, int64_t x_bs, const float *packed, const float *b, const float *res, int64_t res_bs, float *y,
                 int64_t y_bs, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int S, int P, int64_t OH,
-                int64_t OW, int act, hipStream_t st)
+                int64_t OW, int act, hipStream_t st, float *y2, int64_t y2_bs, int64_t split)
 {
     ODL_REQUIRE(packed != nullptr && reinterpret_cast<uintptr_t>(packed) % 16 == 0, "conv2d: the filter copy must be 16-byte aligned");
     DirectArgs g{};
     g.x = x, g.w = packed, g.bias = b, g.res = res, g.y = y;
-    g.x_bs = x_bs ? x_bs : C * H * W, g.y_bs = y_bs ? y_bs : OC * OH * OW, g.res_bs = res_bs ? res_bs : OC * OH * OW;
+    // two convolutions run as one: filters [0, split) fill y, the rest y2 (otherwise split = OC and y2 is never chosen)
+    const int64_t first = y2 ? split : OC;
+    g.y2 = y2 ? y2 : y, g.split = (int)first;
+    g.x_bs = x_bs ? x_bs : C * H * W, g.y_bs = y_bs ? y_bs : first * OH * OW, g.res_bs = res_bs ? res_bs : OC * OH * OW;
+    g.y2_bs = y2_bs ? y2_bs : (OC - first) * OH * OW;
     g.C = (int)C, g.H = (int)H, g.W = (int)W, g.OC = (int)OC, g.OH = (int)OH, g.OW = (int)OW, g.KH = KH, g.KW = KW, g.S = S, g.P = P;
     g.M = (int)(N * OH * OW), g.act = act;
-    plan_direct(g.M, OC, C, KH * KW, g.KS, g.WP, g.chunks);
+    // a pair is cut into K shares as its larger member alone would be: each member then sums in the order of its own call
+    const int64_t oc_plan = y2 ? (first > OC - first ? first : OC - first) : OC;
+    plan_direct(g.M, oc_plan, C, KH * KW, g.KS, g.WP, g.chunks);
     g.octiles = (int)ceil_div(OC, 32);
     g.d_ohw = make_fastdiv((unsigned)(OH * OW)), g.d_ow = make_fastdiv((unsigned)OW);
     g.d_chunks = make_fastdiv((unsigned)g.chunks), g.d_kw = make_fastdiv((unsigned)KW);
@@ -316,7 +442,11 @@ int conv_direct(const float *x, int64_t x_bs, const float *packed, const float *
     ODL_REQUIRE(blocks < (1ll << 31), "conv2d: too many tiles");
     const size_t lds = (32 + (g.KS > 1 ? (size_t)g.KS * g.WP * 32 * kPitch : 0)) * sizeof(float);
     const dim3 grid((unsigned)blocks), block(64 * g.KS * g.WP);
-    if ((KH * KW) % 3 == 0 && res)
+    if (direct_rows3(KH, KW, P, W) && res)
+        hipLaunchKernelGGL((conv_direct3_kernel<true>), grid, block, lds, st, g);
+    else if (direct_rows3(KH, KW, P, W))
+        hipLaunchKernelGGL((conv_direct3_kernel<false>), grid, block, lds, st, g);
+    else if ((KH * KW) % 3 == 0 && res)
         hipLaunchKernelGGL((conv_direct_kernel<3, true>), grid, block, lds, st, g);
     else if ((KH * KW) % 3 == 0)
         hipLaunchKernelGGL((conv_direct_kernel<3, false>), grid, block, lds, st, g);

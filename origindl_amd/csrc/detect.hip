@@ -156,20 +156,22 @@ __global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__rest
     const int np = (HW - p0 < 64) ? HW - p0 : 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float *src = conv + ((int64_t)(b * g.A + a) * g.CI) * HW + p0;
-    // four channels per wave in flight: the loads of a group are issued together, then the four sigmoids
-    for (int c0 = wave; c0 < g.CI; c0 += 4 * (kBlock / 64))
+    // a wave takes every fourth channel; twelve of them in flight at a time: the loads of a batch are issued together,
+    // then its sigmoids (85 channels: two batches a wave)
+    constexpr int kBatch = 12, kWaves = kBlock / 64;
+    for (int c0 = wave; c0 < g.CI; c0 += kBatch * kWaves)
     {
-        float v[4];
+        float v[kBatch];
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < kBatch; ++j)
         {
-            const int c = c0 + j * (kBlock / 64);
+            const int c = c0 + j * kWaves;
             v[j] = (c < g.CI && lane < np) ? src[(int64_t)c * HW + lane] : 0.0f;
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < kBatch; ++j)
         {
-            const int c = c0 + j * (kBlock / 64);
+            const int c = c0 + j * kWaves;
             if (c < g.CI && lane < np)
                 sh_det[lane * LS + c] = 1.0f / (1.0f + expf(-v[j]));  // the reference's -x, exp, 1 + ., 1 / . steps
         }

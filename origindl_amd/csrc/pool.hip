@@ -482,10 +482,12 @@ int make_geom(PoolGeom &g, const char *who, int64_t N, int64_t C, int64_t H, int
 // y1 = pool(x), y2 = pool(y1), y3 = pool(y2), all three concatenated). Each stage scans its windows exactly as
 // max_pool_fwd_lds_kernel does (first cell, then strict >, padding cells 0.0), so the values are those of `count`
 // separate calls. x and y carry their own distance between images: either may be a run of channels of a wider tensor.
+template <int CK>
 __global__ __launch_bounds__(256) void max_pool_chain_kernel(const float *__restrict__ x, int64_t x_bs, float *__restrict__ y,
-                                                              int64_t y_bs, int C, int H, int W, int K, int count)
+                                                              int64_t y_bs, int C, int H, int W, int K_, int count)
 {
     extern __shared__ float chain_sh[];  // two planes
+    const int K = CK > 0 ? CK : K_;
     const int plane = H * W, P = K / 2;
     const int n = blockIdx.x / C, c = blockIdx.x - n * C;
     const float *src = x + (int64_t)n * x_bs + (int64_t)c * plane;
@@ -500,14 +502,17 @@ __global__ __launch_bounds__(256) void max_pool_chain_kernel(const float *__rest
         {
             const int oh = t / W, ow = t - oh * W;
             float mv = 0.f;
+#pragma unroll
             for (int kh = 0; kh < K; ++kh)
             {
                 const int h = oh - P + kh;
+#pragma unroll
                 for (int kw = 0; kw < K; ++kw)
                 {
                     const int w = ow - P + kw;
                     const bool in = (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W;
-                    const float v = in ? cur[h * W + w] : 0.f;
+                    const float xv = cur[in ? h * W + w : 0];
+                    const float v = in ? xv : 0.f;
                     if ((kh | kw) == 0)
                         mv = v;
                     else if (v > mv)
@@ -517,7 +522,8 @@ __global__ __launch_bounds__(256) void max_pool_chain_kernel(const float *__rest
             nxt[t] = mv;
             dst[t] = mv;
         }
-        __syncthreads();
+        // the next stage reads this one out of LDS: wait for the LDS writes only, not for the stores to memory
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         float *tmp = cur;
         cur = nxt, nxt = tmp;
     }
@@ -539,9 +545,15 @@ int odl_hip_max_pool2d_chain(const float *x, int64_t x_image_stride, int64_t N, 
     ODL_REQUIRE(N * C < (1ll << 31), "max_pool2d_chain: too many planes");
     if (N == 0)
         return ODL_OK;
-    hipLaunchKernelGGL(max_pool_chain_kernel, dim3((unsigned)(N * C)), dim3(256), (size_t)(2 * H * W) * sizeof(float),
-                       odl::as_stream(stream), x, x_image_stride ? x_image_stride : C * H * W, y,
-                       y_image_stride ? y_image_stride : count * C * H * W, (int)C, (int)H, (int)W, K, count);
+    const size_t lds = (size_t)(2 * H * W) * sizeof(float);
+    const int64_t xs = x_image_stride ? x_image_stride : C * H * W, ys = y_image_stride ? y_image_stride : count * C * H * W;
+    const dim3 grid((unsigned)(N * C)), block(256);
+    if (K == 5)
+        hipLaunchKernelGGL(max_pool_chain_kernel<5>, grid, block, lds, odl::as_stream(stream), x, xs, y, ys, (int)C, (int)H, (int)W, K, count);
+    else if (K == 3)
+        hipLaunchKernelGGL(max_pool_chain_kernel<3>, grid, block, lds, odl::as_stream(stream), x, xs, y, ys, (int)C, (int)H, (int)W, K, count);
+    else
+        hipLaunchKernelGGL(max_pool_chain_kernel<0>, grid, block, lds, odl::as_stream(stream), x, xs, y, ys, (int)C, (int)H, (int)W, K, count);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

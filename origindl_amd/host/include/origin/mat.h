@@ -377,6 +377,11 @@ public:
     static void conv2d_fused(const ChannelRun &x, const Mat &packed, const Shape &w_shape, const Mat *b,
                              std::pair<int, int> stride, std::pair<int, int> pad, int activation, const ChannelRun *residual,
                              const ChannelRun &y);
+    // two convolutions over x as one launch: `packed` and b hold both filters / biases one after the other (w_shape: the
+    // two together); the first y_first.channels filters fill y_first, the others y_second
+    static void conv2d_fused_pair(const ChannelRun &x, const Mat &packed, const Shape &w_shape, const Mat *b,
+                                  std::pair<int, int> stride, std::pair<int, int> pad, int activation, const ChannelRun &y_first,
+                                  const ChannelRun &y_second);
     static void upsample_run(const ChannelRun &x, const ChannelRun &y, int scale_h, int scale_w);
     // y's channels [(j-1)*C, j*C) = the K x K / stride 1 / padding K/2 max pool applied j times to x, j = 1..count
     static void max_pool_chain(const ChannelRun &x, int K, int count, const ChannelRun &y);

@@ -6,7 +6,8 @@
 // and so does the residual add that follows it alone; the inputs of a channel concatenation are written by their
 // producers straight into the concatenation's output (and read from there by their other readers), so the torch.cat
 // node copies only what could not be placed; a chain of same-size max pools whose stages are all concatenated (SPPF)
-// is one launch; the detect head decodes each stage into its rows of the final tensor. Weights are uploaded to the
+// is one launch; two convolutions that read the same tensor through the same window (the cv1 / cv2 pair of a C3 block)
+// are one launch; the detect head decodes each stage into its rows of the final tensor. Weights are uploaded to the
 // device once (at the first forward on that device) and kept, where the reference rebuilds every weight tensor from
 // host data on every forward (src/pnnx/pnnx_graph.cpp:341-405); nodes run on Mat objects directly, without building
 // an autograd graph. set_fusion(false) runs every node on its own, as the reference does.
@@ -51,6 +52,12 @@ struct PNNXNode
     std::string residual_name;
     // the first max pool of a chain of `pool_chain` same-size pools whose outputs lie side by side in one concatenation
     int pool_chain = 0;
+    // a convolution that also runs the convolution `pair_with` (same input, window, stride, padding and activation):
+    // the two filters follow each other in the attributes "pair.weight" / "pair.bias", made at the first forward
+    std::string pair_with;
+    // the node's numeric parameters, read out of `params` once (at the first forward)
+    bool parsed = false;
+    std::pair<int, int> kernel{1, 1}, stride{1, 1}, padding{0, 0};
 };
 
 class PNNXGraph
@@ -95,7 +102,9 @@ private:
     std::vector<std::string> input_blobs_;
     bool built_ = false, fusion_ = true;
     void run(PNNXNode &node);
+    void run_conv(PNNXNode &node);
     void plan_fusion();
+    Value destination(const std::string &tensor, size_t N, size_t C, size_t H, size_t W, const Device &dev);
     Value &value(const std::string &name, const PNNXNode &reader);
     std::shared_ptr<Mat> dense(const std::string &name, const PNNXNode &reader);
     std::shared_ptr<Mat> buffer_for(const std::string &cat_output, size_t N, size_t H, size_t W, const Device &dev);

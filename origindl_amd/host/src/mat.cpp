@@ -1359,6 +1359,33 @@ void OriginMat::conv2d_fused(const ChannelRun &xr, const Mat &packed_m, const Sh
                                p.second, activation, res, res_stride, y.data, y.image_stride, cur()));
 }
 
+void OriginMat::conv2d_fused_pair(const ChannelRun &xr, const Mat &packed_m, const Shape &ws, const Mat *bm, std::pair<int, int> s,
+                                  std::pair<int, int> p, int activation, const ChannelRun &y1r, const ChannelRun &y2r)
+{
+    const RunPtr x = run_ptr(xr, "conv2d"), y1 = run_ptr(y1r, "conv2d"), y2 = run_ptr(y2r, "conv2d");
+    if (ws.size() != 4 || (int64_t)ws[1] != x.C || (int64_t)ws[0] != y1.C + y2.C)
+        THROW_INVALID_ARG("conv2d: filters {} do not map {} channels to {} + {}", ws.to_string(), x.C, y1.C, y2.C);
+    const int KH = (int)ws[2], KW = (int)ws[3];
+    const int OH = get_conv_outsize((int)x.H, KH, s.first, p.first), OW = get_conv_outsize((int)x.W, KW, s.second, p.second);
+    if (y1.N != x.N || y1.H != OH || y1.W != OW || y2.N != x.N || y2.H != OH || y2.W != OW)
+        THROW_INVALID_ARG("conv2d: an output run does not have the convolution's [{}, *, {}, {}]", x.N, OH, OW);
+    const OriginMat &pk = dev_f32(packed_m, "conv2d");
+    const int64_t OC = (int64_t)ws[0];
+    const size_t want = odl_hip_conv2d_packed_weights_bytes(x.N, x.C, x.H, x.W, OC, KH, KW, s.first, s.second, p.first, p.second);
+    if (pk.elements() * sizeof(float) != want)
+        THROW_INVALID_ARG("conv2d: the packed filter has {} bytes, this shape's kernel reads {}", pk.elements() * sizeof(float), want);
+    const float *bias = nullptr;
+    if (bm)
+    {
+        const OriginMat &b = dev_f32(*bm, "conv2d");
+        if (b.shape().size() != 1 || (int64_t)b.shape()[0] != OC)
+            THROW_INVALID_ARG("conv2d: b must be 1D with size {}, but got shape {}", OC, b.shape().to_string());
+        bias = fp(b);
+    }
+    check(odl_hip_conv2d_fused_pair(x.data, x.image_stride, fp(pk), bias, x.N, x.C, x.H, x.W, OC, y1.C, KH, KW, s.first, s.second,
+                                    p.first, p.second, activation, y1.data, y1.image_stride, y2.data, y2.image_stride, cur()));
+}
+
 void OriginMat::upsample_run(const ChannelRun &xr, const ChannelRun &yr, int sh, int sw)
 {
     const RunPtr x = run_ptr(xr, "upsample"), y = run_ptr(yr, "upsample");

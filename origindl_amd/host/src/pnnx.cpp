@@ -413,11 +413,49 @@ void PNNXGraph::plan_fusion()
             break;
         }
     }
+    // 1b. two convolutions that read the same tensor through the same window with the same activation run as one
+    // launch over both filters (the later one folds into the earlier one)
+    {
+        auto same_params = [](const PNNXNode &a, const PNNXNode &b) {
+            for (const char *key : {"kernel_size", "stride", "padding", "dilation", "groups", "padding_mode"})
+            {
+                const bool ha = a.params.count(key) > 0, hb = b.params.count(key) > 0;
+                if (ha != hb || (ha && a.params.at(key) != b.params.at(key)))
+                    return false;
+            }
+            auto wa = a.attributes.find("weight"), wb = b.attributes.find("weight");
+            if (wa == a.attributes.end() || wb == b.attributes.end() || wa->second.shape.size() != 4 || wb->second.shape.size() != 4)
+                return false;
+            for (int d = 1; d < 4; ++d)
+                if (wa->second.shape[d] != wb->second.shape[d])
+                    return false;
+            return (a.attributes.count("bias") > 0) == (b.attributes.count("bias") > 0);
+        };
+        for (size_t i = 0; i < plan_.size(); ++i)
+        {
+            PNNXNode &a = *plan_[i];
+            if (a.type != "nn.Conv2d" || a.folded_into_producer || !a.pair_with.empty() || !a.residual_name.empty() ||
+                a.input_names.size() != 1 || a.output_names.size() != 1)
+                continue;
+            for (size_t j = i + 1; j < plan_.size(); ++j)
+            {
+                PNNXNode &b = *plan_[j];
+                if (b.type != "nn.Conv2d" || b.folded_into_producer || !b.pair_with.empty() || !b.residual_name.empty() ||
+                    b.input_names != a.input_names || b.output_names.size() != 1 || b.fused_activation != a.fused_activation ||
+                    !same_params(a, b))
+                    continue;
+                a.pair_with = b.name;
+                b.folded_into_producer = true;
+                break;
+            }
+        }
+    }
     // 2. channel counts that follow from the graph alone
     std::map<std::string, size_t> channels;
     for (auto &n : plan_)
     {
-        if (n->folded_into_producer || n->output_names.size() != 1)
+        const bool paired_conv = n->folded_into_producer && n->type == "nn.Conv2d";  // runs inside its partner
+        if ((n->folded_into_producer && !paired_conv) || n->output_names.size() != 1)
             continue;
         size_t c = 0;
         if (n->type == "nn.Conv2d")
@@ -628,6 +666,119 @@ void PNNXGraph::store(const PNNXNode &node, std::shared_ptr<Mat> out)
     blobs_[name] = v;
 }
 
+// where a [N, C, H, W] tensor goes: its run of the concatenation build() placed it in, or a tensor of its own
+PNNXGraph::Value PNNXGraph::destination(const std::string &tensor, size_t N, size_t C, size_t H, size_t W, const Device &dev)
+{
+    Value v;
+    auto place = placed_.find(tensor);
+    if (place != placed_.end())
+    {
+        v.mat = buffer_for(place->second.buffer, N, H, W, dev);
+        v.c0 = place->second.c0, v.channels = C, v.run = true;
+    }
+    else
+        v.mat = std::make_shared<OriginMat>(Shape{N, C, H, W}, DataType::kFloat32, dev);
+    return v;
+}
+
+void PNNXGraph::run_conv(PNNXNode &node)
+{
+    Value &first = value(node.input_names[0], node);
+    const Device dev = first.mat->device();
+    auto run_of = [&](const Value &v) {
+        return v.run ? OriginMat::ChannelRun{&origin_of(*v.mat), v.c0, v.channels} : OriginMat::whole(*v.mat);
+    };
+    if (!node.parsed)
+    {
+        if (int_pair(node, "dilation", {1, 1}) != std::make_pair(1, 1) || int_param(node, "groups", 1) != 1)
+            THROW_RUNTIME_ERROR("PNNX: node {}: dilated or grouped convolutions are not supported", node.name);
+        node.stride = int_pair(node, "stride", {1, 1}), node.padding = int_pair(node, "padding", {0, 0});
+        node.parsed = true;
+    }
+    auto wit = node.attributes.find("weight");
+    if (wit == node.attributes.end())
+        THROW_RUNTIME_ERROR("PNNX: node {} has no weight", node.name);
+    auto w = upload(wit->second, dev, node.name + ".weight");
+    auto bit = node.attributes.find("bias");
+    std::shared_ptr<Mat> b = bit == node.attributes.end() ? nullptr : upload(bit->second, dev, node.name + ".bias");
+    const auto stride = node.stride, padding = node.padding;
+    const Shape s0 = first.mat->shape();
+    const Shape xs = (first.run && s0.size() == 4) ? Shape{s0[0], first.channels, s0[2], s0[3]} : s0;
+    const Shape ws = w->shape();
+    const bool f32 = first.mat->dtype() == DataType::kFloat32;
+    const std::string &out_name = final_output(node);
+    // this convolution and the one paired with it as one launch over both filters
+    if (!node.pair_with.empty())
+    {
+        PNNXNode &other = *by_name_.at(node.pair_with);
+        auto owit = other.attributes.find("weight");
+        auto ow = upload(owit->second, dev, other.name + ".weight");
+        const Shape ows = ow->shape();
+        const Shape both{ws[0] + ows[0], ws[1], ws[2], ws[3]};
+        if (fusion_ && f32 && xs.size() == 4 && OriginMat::conv2d_fused_ok(xs, both, stride, padding))
+        {
+            Attribute &pw = node.attributes["pair.weight"];
+            if (!pw.device_mat || pw.device_mat->device() != dev)
+            {
+                pw.device_mat = w->cat({ow.get()}, 0);
+                pw.packed_for.clear();
+                if (b)
+                {
+                    auto ob = upload(other.attributes.find("bias")->second, dev, other.name + ".bias");
+                    node.attributes["pair.bias"].device_mat = b->cat({ob.get()}, 0);
+                }
+            }
+            if (pw.packed_for != xs.dims())
+            {
+                pw.packed_mat = OriginMat::conv2d_packed_weights_for(xs, *pw.device_mat, stride, padding);
+                pw.packed_for = xs.dims();
+            }
+            if (pw.packed_mat)
+            {
+                const int OH = get_conv_outsize((int)xs[2], (int)ws[2], stride.first, padding.first);
+                const int OW = get_conv_outsize((int)xs[3], (int)ws[3], stride.second, padding.second);
+                const std::string &other_out = final_output(other);
+                Value out = destination(out_name, xs[0], ws[0], (size_t)OH, (size_t)OW, dev);
+                Value out2 = destination(other_out, xs[0], ows[0], (size_t)OH, (size_t)OW, dev);
+                OriginMat::conv2d_fused_pair(run_of(first), *pw.packed_mat, both, b ? node.attributes["pair.bias"].device_mat.get() : nullptr,
+                                             stride, padding, node.fused_activation, run_of(out), run_of(out2));
+                blobs_[out_name] = out;
+                blobs_[other_out] = out2;
+                return;
+            }
+        }
+    }
+    // the weights never change: the filter order this input shape's kernel wants is made once and kept
+    Attribute &wa = wit->second;
+    if (wa.packed_for != xs.dims())
+    {
+        wa.packed_mat = OriginMat::conv2d_packed_weights_for(xs, *w, stride, padding);
+        wa.packed_for = xs.dims();
+    }
+    if (fusion_ && wa.packed_mat && f32 && OriginMat::conv2d_fused_ok(xs, ws, stride, padding))
+    {
+        const int OH = get_conv_outsize((int)xs[2], (int)ws[2], stride.first, padding.first);
+        const int OW = get_conv_outsize((int)xs[3], (int)ws[3], stride.second, padding.second);
+        Value out = destination(out_name, xs[0], ws[0], (size_t)OH, (size_t)OW, dev);
+        OriginMat::ChannelRun res{};
+        if (!node.residual_name.empty())
+            res = run_of(value(node.residual_name, node));
+        OriginMat::conv2d_fused(run_of(first), *wa.packed_mat, ws, b.get(), stride, padding, node.fused_activation,
+                                node.residual_name.empty() ? nullptr : &res, run_of(out));
+        blobs_[out_name] = out;
+    }
+    else
+    {
+        auto x = dense(node.input_names[0], node);
+        std::shared_ptr<Mat> out = origin_of(*x).conv2d_act(*w, b.get(), stride, padding, node.fused_activation, wa.packed_mat.get());
+        if (!node.residual_name.empty())
+            out = *dense(node.residual_name, node) + *out;
+        store(node, std::move(out));
+    }
+    if (!node.pair_with.empty())
+        run_conv(*by_name_.at(node.pair_with));  // the pair could not run as one: the partner on its own
+}
+
 void PNNXGraph::run(PNNXNode &node)
 {
     if (node.folded_into_producer)
@@ -654,62 +805,24 @@ void PNNXGraph::run(PNNXNode &node)
     };
     const std::string &out_name = final_output(node);
     auto place = placed_.find(out_name);
-    // where a [N, C, H, W] result of this node goes: its run of the concatenation, or a tensor of its own
-    auto destination = [&](size_t N, size_t C, size_t H, size_t W) {
-        Value v;
-        if (place != placed_.end())
-        {
-            v.mat = buffer_for(place->second.buffer, N, H, W, dev);
-            v.c0 = place->second.c0, v.channels = C, v.run = true;
-        }
-        else
-            v.mat = std::make_shared<OriginMat>(Shape{N, C, H, W}, DataType::kFloat32, dev);
-        return v;
-    };
     const std::string &t = node.type;
     if (t == "nn.Conv2d")
     {
-        if (int_pair(node, "dilation", {1, 1}) != std::make_pair(1, 1) || int_param(node, "groups", 1) != 1)
-            THROW_RUNTIME_ERROR("PNNX: node {}: dilated or grouped convolutions are not supported", node.name);
-        auto w = weight("weight");
-        if (!w)
-            THROW_RUNTIME_ERROR("PNNX: node {} has no weight", node.name);
-        auto b = weight("bias");
-        const auto stride = int_pair(node, "stride", {1, 1}), padding = int_pair(node, "padding", {0, 0});
-        const Shape xs = run_shape(first), ws = w->shape();
-        // the weights never change: the filter order this input shape's kernel wants is made once and kept
-        Attribute &wa = node.attributes.find("weight")->second;
-        if (wa.packed_for != xs.dims())
-        {
-            wa.packed_mat = OriginMat::conv2d_packed_weights_for(xs, *w, stride, padding);
-            wa.packed_for = xs.dims();
-        }
-        if (fusion_ && wa.packed_mat && first.mat->dtype() == DataType::kFloat32 && OriginMat::conv2d_fused_ok(xs, ws, stride, padding))
-        {
-            const int OH = get_conv_outsize((int)xs[2], (int)ws[2], stride.first, padding.first);
-            const int OW = get_conv_outsize((int)xs[3], (int)ws[3], stride.second, padding.second);
-            Value out = destination(xs[0], ws[0], (size_t)OH, (size_t)OW);
-            OriginMat::ChannelRun res{};
-            if (!node.residual_name.empty())
-                res = run_of(value(node.residual_name, node));
-            OriginMat::conv2d_fused(run_of(first), *wa.packed_mat, ws, b.get(), stride, padding, node.fused_activation,
-                                    node.residual_name.empty() ? nullptr : &res, run_of(out));
-            blobs_[out_name] = out;
-            return;
-        }
-        auto x = dense(node.input_names[0], node);
-        std::shared_ptr<Mat> out = origin_of(*x).conv2d_act(*w, b.get(), stride, padding, node.fused_activation, wa.packed_mat.get());
-        if (!node.residual_name.empty())
-            out = *dense(node.residual_name, node) + *out;
-        store(node, std::move(out));
+        run_conv(node);
         return;
     }
     if (t == "nn.MaxPool2d")
     {
-        const auto k = int_pair(node, "kernel_size", {2, 2});
-        auto s = int_pair(node, "stride", {0, 0});
-        if (s.first <= 0 || s.second <= 0)
-            s = k;  // a missing stride means the kernel size
+        if (!node.parsed)
+        {
+            node.kernel = int_pair(node, "kernel_size", {2, 2});
+            node.stride = int_pair(node, "stride", {0, 0});
+            if (node.stride.first <= 0 || node.stride.second <= 0)
+                node.stride = node.kernel;  // a missing stride means the kernel size
+            node.padding = int_pair(node, "padding", {0, 0});
+            node.parsed = true;
+        }
+        const auto k = node.kernel, s = node.stride;
         const Shape xs = run_shape(first);
         // this pool and the pools folded into it, in order
         std::vector<PNNXNode *> stages{&node};
@@ -740,7 +853,7 @@ void PNNXGraph::run(PNNXNode &node)
         }
         // one pool after the other, each result copied to its place
         for (PNNXNode *stage : stages)
-            store(*stage, dense(stage->input_names[0], *stage)->max_pool2d(k, s, int_pair(node, "padding", {0, 0}), nullptr));
+            store(*stage, dense(stage->input_names[0], *stage)->max_pool2d(k, s, node.padding, nullptr));
         return;
     }
     if (t == "nn.Upsample")
@@ -767,7 +880,7 @@ void PNNXGraph::run(PNNXNode &node)
         const int sh = (int)(OH / xs[2]), sw = (int)(OW / xs[3]);
         if ((first.run || place != placed_.end()) && first.mat->dtype() == DataType::kFloat32 && OW % 4 == 0 && sh > 0 && sw > 0)
         {
-            Value out = destination(xs[0], xs[1], OH, OW);
+            Value out = destination(out_name, xs[0], xs[1], OH, OW, dev);
             OriginMat::upsample_run(run_of(first), run_of(out), sh, sw);
             blobs_[out_name] = out;
             return;

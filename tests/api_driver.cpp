@@ -648,6 +648,7 @@ int DRV(checkpoint_roundtrip)(const float *params, const char *path, int epoch, 
 // switch; the reference's classes ignore it). The launches of the forward recorded last are read back below.
 static int g_pnnx_fusion = 1;
 static int64_t g_pnnx_graph_nodes = 0;
+static float g_pnnx_host_ms = 0.0f;  // mean time forward() took to return (its launches queued, not yet run)
 int DRV(pnnx_set_fusion)(int on)
 {
     g_pnnx_fusion = on;
@@ -656,6 +657,11 @@ int DRV(pnnx_set_fusion)(int on)
 int DRV(pnnx_last_graph_nodes)(int64_t *nodes)
 {
     *nodes = g_pnnx_graph_nodes;
+    return 0;
+}
+int DRV(pnnx_last_host_ms)(float *ms)
+{
+    *ms = g_pnnx_host_ms;
     return 0;
 }
 
@@ -670,13 +676,17 @@ int DRV(pnnx_forward)(const char *param_path, const char *bin_path, const float 
         graph.build();
         auto X = f32(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W});
         std::vector<Tensor> outs;
+        float host_ms = 0.0f;
         auto t0 = std::chrono::steady_clock::now();
         for (int r = 0; r < (reps < 1 ? 1 : reps); ++r)
         {
             if (r == 1)
                 t0 = std::chrono::steady_clock::now();
             graph.set_inputs("pnnx_input_0", {X});
+            const auto h0 = std::chrono::steady_clock::now();
             graph.forward();
+            if (r >= 1)
+                host_ms += std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - h0).count();
             outs = graph.get_outputs("pnnx_output_0");
 #ifdef DRV_ON_DEVICE
             origin::cuda::synchronize();  // the forward is complete on the device; the copy to the host comes after the loop
@@ -689,6 +699,7 @@ int DRV(pnnx_forward)(const char *param_path, const char *bin_path, const float 
         std::vector<float> last = outs[0].to_vector<float>();
         if (ms)
             *ms = reps > 1 ? std::chrono::duration<float, std::milli>(t1 - t0).count() / (float)(reps - 1) : 0.0f;
+        g_pnnx_host_ms = reps > 1 ? host_ms / (float)(reps - 1) : 0.0f;
         if ((int64_t)last.size() > capacity)
             throw std::invalid_argument("pnnx_forward: output larger than the buffer");
         std::memcpy(o, last.data(), last.size() * sizeof(float));

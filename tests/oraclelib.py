@@ -109,6 +109,7 @@ _DEVICE_ONLY_SIGS = {
     "odl_host_pnnx_forward_graph": _REF_SIGS["odl_ref_pnnx_forward"],
     "odl_host_pnnx_set_fusion": "i>i",
     "odl_host_pnnx_last_graph_nodes": "p>i",
+    "odl_host_pnnx_last_host_ms": "p>i",
     "odl_host_upload_ordering": "lip>i",
     "odl_host_graph_abort_recovery": "pplllpp>i",
     "odl_host_pending_fill_semantics": "lp>i",

@@ -1167,11 +1167,16 @@ def test_conv_with_fused_activation_is_conv_then_activation(api, N, C, H, OC, k,
         small = C % 8 == 0 and 2 * N * ((H + 2 * p - k) // s + 1) ** 2 * C * k * k * OC <= 3 << 29
         packed = api.conv2d_pack_weights(x.shape, w, s, p)
         if direct and small:
-            assert packed is not None and packed.numel() == -(-OC // 32) * 32 * C * k * k
-            # blocks of [lane half][row][4 channels] per (tile of 32 filters, tap, group of 8 channels)
             wp = np.zeros((-(-OC // 32) * 32, C, k * k), f32)
             wp[:OC] = host(w).reshape(OC, C, k * k)
-            want = wp.reshape(-1, 32, C // 8, 2, 4, k * k).transpose(0, 5, 2, 3, 1, 4)
+            if k == 3 and p == 1:
+                # 3x3 / padding 1: per (tile of 32 filters, channel pair, window row) a block [lane half][row][kw, one pad]
+                want = np.zeros((wp.shape[0] // 32, C // 2, 3, 2, 32, 4), f32)
+                want[..., :3] = wp.reshape(-1, 32, C // 2, 2, 3, 3).transpose(0, 2, 4, 3, 1, 5)
+            else:
+                # blocks of [lane half][row][4 channels] per (tile of 32 filters, tap, group of 8 channels)
+                want = wp.reshape(-1, 32, C // 8, 2, 4, k * k).transpose(0, 5, 2, 3, 1, 4)
+            assert packed is not None and packed.numel() == want.size
             assert np.array_equal(host(packed), want.reshape(-1))
         else:
             assert (packed is not None) == (k == 3 and C % 16 == 0 and not (s == 2 and N == 64))
@@ -1196,6 +1201,10 @@ def test_conv_with_fused_activation_is_conv_then_activation(api, N, C, H, OC, k,
     (2, 16, 12, 12, 24, 5, 1, 2),     # 5x5: depth 4 over 25 taps x 2 groups
     (2, 32, 14, 10, 48, 3, 2, 0),     # stride 2 without padding
     (1, 1024, 4, 4, 64, 1, 1, 0),     # 128 channel groups: eight per share
+    (2, 16, 7, 3, 32, 3, 1, 1),       # rows of three pixels: every window hangs over an edge or touches both
+    (2, 8, 6, 9, 16, 3, 2, 1),        # stride 2 over an odd width: the last window hangs over the right edge
+    (2, 8, 3, 2, 16, 3, 1, 1),        # rows of two pixels: the general kernel, not the three-floats-a-load one
+    (1, 32, 1, 5, 16, 3, 1, 1),       # a single image row: the windows' outer rows lie in the padding
 ])
 def test_conv_fused_into_channel_runs_equals_the_nodes_one_by_one(api, o, N, C, H, W, OC, k, s, p):
     """odl_hip_conv2d_fused with its input, output and residual each a run of channels of a wider tensor: the result
