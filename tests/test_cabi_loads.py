@@ -44,7 +44,9 @@ def test_workspace_queries_need_no_gpu():
     # global memory: the workspace holds the filter copy in that kernel's order, whole tiles of 32 filters
     assert l.query("odl_hip_conv2d_workspace_bytes", 32, 64, 32, 32, 128, 1, 1, 1, 1, 0, 0) == 128 * 64 * 4
     assert l.query("odl_hip_conv2d_workspace_bytes", 4, 64, 40, 40, 255, 1, 1, 1, 1, 0, 0) == 256 * 64 * 4
-    assert l.query("odl_hip_conv2d_packed_weights_bytes", 4, 128, 10, 10, 128, 3, 3, 1, 1, 1, 1) == 128 * 128 * 9 * 4
+    # (a 3x3 / padding 1 window's three rows are padded to four floats each in that copy; other windows are not)
+    assert l.query("odl_hip_conv2d_packed_weights_bytes", 4, 128, 10, 10, 128, 3, 3, 1, 1, 1, 1) == 128 * 128 * 12 * 4
+    assert l.query("odl_hip_conv2d_packed_weights_bytes", 4, 128, 10, 10, 128, 3, 3, 1, 1, 0, 0) == 128 * 128 * 9 * 4
     assert l.query("odl_hip_conv2d_fused_ok", 4, 128, 10, 10, 128, 3, 3, 1, 1, 1, 1) == 1
     assert l.query("odl_hip_conv2d_fused_ok", 4, 3, 320, 320, 16, 6, 6, 2, 2, 2, 2) == 0
     assert l.query("odl_hip_conv2d_fused_ok", 32, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1) == 0
