@@ -286,6 +286,24 @@ def extras(torch, capi, steps, warmup):
                                                       "flop": flop}
         del a, b, dc, c, da, db
         keep.clear()
+    # the same three products on float64 tensors (FP64 matrix cores, 78.6 TFLOP/s): C = A.B, dA = dC.B^T, dB = A^T.dC
+    for S in (2048, 4096):
+        a, b, dc = (torch.randn((S, S), device="cuda", dtype=torch.float64, generator=g) for _ in range(3))
+        c, da, db = (torch.empty((S, S), device="cuda", dtype=torch.float64) for _ in range(3))
+        calls = [direct("odl_hip_dgemm", 0, 0, S, S, S, ptr(a), S, ptr(b), S, ptr(c), S, 1, 0, 0, 0, stream),
+                 direct("odl_hip_dgemm", 0, 1, S, S, S, ptr(dc), S, ptr(b), S, ptr(da), S, 1, 0, 0, 0, stream),
+                 direct("odl_hip_dgemm", 1, 0, S, S, S, ptr(a), S, ptr(dc), S, ptr(db), S, 1, 0, 0, 0, stream)]
+
+        def all_three():
+            for f in calls:
+                f()
+
+        ms = time_region_auto(torch, all_three)
+        flop = 6.0 * S * S * S
+        out["gemm_f64_fwd_bwd_%d" % S] = {"ms": ms, "tflops": flop / ms / 1e9, "frac_fp64_mfma_peak": flop / ms / 1e9 / 78.6,
+                                            "flop": flop}
+        del a, b, dc, c, da, db
+        keep.clear()
     # the MLP's six GEMMs (config 1): 512x784x1000 and 512x1000x10, forward + backward
     x1, w1, g1 = rnd(512, 784), rnd(784, 1000), rnd(512, 1000)
     x2, w2, g2 = rnd(512, 1000), rnd(1000, 10), rnd(512, 10)

@@ -114,6 +114,14 @@ size_t odl_hip_matmul_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64
 int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M,
                             int64_t K, int64_t N, void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_matmul_backward_workspace_bytes(int64_t M, int64_t K, int64_t N);
+/* Mat::matmul and MatMul::backward for float64 tensors (the reference's device matmul is a template over the element
+ * type and serves double through the kernels it uses for float, src/mat/origin/cuda/math/mat_mul.cu:1911-1954; CPU form
+ * src/mat/origin/cpu/math/matmul.cpp:27-41): C[M,N] = op(A)[M,K] . op(B)[K,N] on the FP64 matrix cores, layouts as in
+ * odl_hip_sgemm (trans_a: A stored [K,M]; trans_b: B stored [N,K]), `batch` independent products stride_a / stride_b /
+ * stride_c doubles apart (stride_b = 0: one B for all, the 3-D x 2-D case). No workspace. */
+int odl_hip_dgemm(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const double *A, int64_t lda, const double *B,
+                  int64_t ldb, double *C, int64_t ldc, int64_t batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                  void *stream);
 /* Mat::transpose (src/mat/origin/cpu/shape/transpose.cpp:27-77): last two dims of [outer, rows, cols] */
 int odl_hip_transpose(const float *src, float *dst, int64_t outer, int64_t rows, int64_t cols, void *stream);
 

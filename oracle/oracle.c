@@ -35,6 +35,19 @@ void orc_matmul(const float *a, const float *b, float *c, int64_t m, int64_t n, 
 }
 
 /* matmul.cpp:55-76 (B shared) and 91-109 (B batched) */
+/* the same loops over doubles: the reference's matmul is a template over the element type (matmul.cpp:27-41) */
+void orc_matmul_f64(const double *a, const double *b, double *c, int64_t m, int64_t n, int64_t k)
+{
+    for (int64_t i = 0; i < m; ++i)
+        for (int64_t j = 0; j < n; ++j)
+        {
+            double sum = 0.0;
+            for (int64_t p = 0; p < k; ++p)
+                sum += a[i * k + p] * b[p * n + j];
+            c[i * n + j] = sum;
+        }
+}
+
 void orc_matmul_batched(const float *a, const float *b, float *c, int64_t batch, int64_t m, int64_t n, int64_t k,
                         int b_is_batched)
 {

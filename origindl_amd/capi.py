@@ -184,6 +184,25 @@ def col2im(col, input_shape, kernel_size, stride, pad, to_matrix=True):
     return img
 
 
+def matmul_f64(a, b, trans_a=False, trans_b=False):
+    """Mat::matmul on float64 tensors: 2-D x 2-D, 3-D x 2-D or 3-D x 3-D (src/mat/origin/cpu/math/matmul.cpp:113-218);
+    trans_a / trans_b read a 2-D operand as its transpose (the two products of MatMul::backward)."""
+    _chk(a, "a", torch.float64), _chk(b, "b", torch.float64)
+    batch, sa, sb = 1, 0, 0
+    if a.dim() == 3:
+        batch, sa = a.shape[0], a.shape[1] * a.shape[2]
+        sb = b.shape[1] * b.shape[2] if b.dim() == 3 else 0
+    ar, ac = a.shape[-2], a.shape[-1]
+    br, bc = b.shape[-2], b.shape[-1]
+    M, K = (ac, ar) if trans_a else (ar, ac)
+    Kb, N = (bc, br) if trans_b else (br, bc)
+    if K != Kb:
+        raise OdlInvalidArgument("matmul: inner dimensions differ (%d and %d)" % (K, Kb))
+    c = _empty(((batch, M, N) if a.dim() == 3 else (M, N)), torch.float64)
+    lib().call("odl_hip_dgemm", int(trans_a), int(trans_b), M, N, K, _p(a), ac, _p(b), bc, _p(c), N, batch, sa, sb, M * N, _stream())
+    return c
+
+
 def conv2d_pack_weights(x_shape, w, stride=1, pad=0):
     """The filter copy, in the order the forward kernel for inputs of x_shape reads it, for weights that stay the same
     from call to call; None when that kernel reads the filter as it lies. Pass it to conv2d(packed=...)."""

@@ -671,6 +671,15 @@ std::unique_ptr<Mat> OriginMat::transpose() const
 {
     if (shape_.size() < 2)
         return clone();
+    if (dtype_ != DataType::kFloat32)
+    {
+        // every other element type: the same copy as a permutation of the last two dimensions
+        std::vector<int> order(shape_.size());
+        for (size_t i = 0; i < order.size(); ++i)
+            order[i] = (int)i;
+        std::swap(order[order.size() - 2], order[order.size() - 1]);
+        return permute(order);
+    }
     const OriginMat &x = dev_f32(*this, "transpose");
     std::vector<size_t> d = shape_.dims();
     const size_t rows = d[d.size() - 2], cols = d[d.size() - 1];
@@ -1447,8 +1456,10 @@ std::unique_ptr<Mat> OriginMat::pow(const Scalar &exponent) const
 
 std::unique_ptr<Mat> OriginMat::matmul(const Mat &other) const
 {
-    const OriginMat &a = dev_f32(*this, "matmul");
-    const OriginMat &b = dev_f32(other, "matmul");
+    // float64 x float64 goes to the FP64 matrix cores; everything else is the float32 product
+    const bool f64 = dtype_ == DataType::kFloat64 && other.dtype() == DataType::kFloat64;
+    const OriginMat &a = f64 ? dev_any(*this, "matmul") : dev_f32(*this, "matmul");
+    const OriginMat &b = f64 ? dev_any(other, "matmul") : dev_f32(other, "matmul");
     const Shape as = a.shape(), bs = b.shape();
     if (as.size() < 2 || bs.size() < 2)
         THROW_INVALID_ARG("Matrix multiplication requires at least 2D tensors. A shape: {}, B shape: {}", as.to_string(),
@@ -1479,6 +1490,14 @@ std::unique_ptr<Mat> OriginMat::matmul(const Mat &other) const
     if ((int64_t)bs[bs.size() - 2] != K)
         THROW_INVALID_ARG("Matrix dimensions must be compatible for multiplication. A shape: {}, B shape: {}",
                           as.to_string(), bs.to_string());
+    if (f64)
+    {
+        auto c = new_like(a, rs, DataType::kFloat64);
+        check(odl_hip_dgemm(0, 0, M, N, K, static_cast<const double *>(a.storage()->data()), K,
+                            static_cast<const double *>(b.storage()->data()), N, static_cast<double *>(c->storage()->data()), N,
+                            batch, M * K, b_batched ? K * N : 0, M * N, cur()));
+        return c;
+    }
     auto c = new_like(a, rs);
     Workspace ws(odl_hip_matmul_workspace_bytes(batch, M, N, K, b_batched), device().index());
     check(odl_hip_matmul(fp(a), fp(b), c->data_ptr<float>(), batch, M, N, K, b_batched, ws.ptr(), ws.bytes, cur()));
@@ -2131,12 +2150,26 @@ std::unique_ptr<Mat> OriginMat::sgd_step(const Mat &grad, float lr) const
 std::pair<std::unique_ptr<Mat>, std::unique_ptr<Mat>> OriginMat::matmul_backward_2d(const Mat &x_, const Mat &w_,
                                                                                     const Mat &gy_)
 {
-    const OriginMat &x = dev_f32(x_, "matmul"), &w = dev_f32(w_, "matmul"), &gy = dev_f32(gy_, "matmul");
+    const bool f64 = x_.dtype() == DataType::kFloat64 && w_.dtype() == DataType::kFloat64 && gy_.dtype() == DataType::kFloat64;
+    const OriginMat &x = f64 ? dev_any(x_, "matmul") : dev_f32(x_, "matmul");
+    const OriginMat &w = f64 ? dev_any(w_, "matmul") : dev_f32(w_, "matmul");
+    const OriginMat &gy = f64 ? dev_any(gy_, "matmul") : dev_f32(gy_, "matmul");
     const Shape xs = x.shape(), ws_ = w.shape(), gs = gy.shape();
     if (xs.size() != 2 || ws_.size() != 2 || gs.size() != 2 || xs[1] != ws_[0] || gs[0] != xs[0] || gs[1] != ws_[1])
         THROW_INVALID_ARG("matmul backward: shapes {} {} {} do not form x[M,K] w[K,N] gy[M,N]", xs.to_string(),
                           ws_.to_string(), gs.to_string());
     const int64_t M = xs[0], K = xs[1], N = ws_[1];
+    if (f64)
+    {
+        // gx[M,K] = gy[M,N] . w[K,N]^T and gw[K,N] = x[M,K]^T . gy[M,N], both operands read where they lie
+        auto gx = new_like(x, xs, DataType::kFloat64);
+        auto gw = new_like(w, ws_, DataType::kFloat64);
+        const double *xp = static_cast<const double *>(x.storage()->data()), *wp = static_cast<const double *>(w.storage()->data());
+        const double *gp = static_cast<const double *>(gy.storage()->data());
+        check(odl_hip_dgemm(0, 1, M, K, N, gp, N, wp, N, static_cast<double *>(gx->storage()->data()), K, 1, 0, 0, 0, cur()));
+        check(odl_hip_dgemm(1, 0, K, N, M, xp, K, gp, N, static_cast<double *>(gw->storage()->data()), N, 1, 0, 0, 0, cur()));
+        return {std::move(gx), std::move(gw)};
+    }
     auto gx = new_like(x, xs);
     auto gw = new_like(w, ws_);
     Workspace ws(odl_hip_matmul_backward_workspace_bytes(M, K, N), x.device().index());

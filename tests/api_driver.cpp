@@ -279,6 +279,31 @@ int DRV(matmul_fwd_bwd)(const float *x, const float *w, const float *gy, float *
     });
 }
 
+// the same on float64 tensors: the product, and both gradients through the autograd graph
+int DRV(matmul_f64_fwd_bwd)(const double *x, const double *w, const double *gy, double *y, double *gx, double *gw, int64_t m,
+                            int64_t k, int64_t n)
+{
+    return guarded([&] {
+        auto f64 = [](const double *p, const Shape &s, bool grad) {
+            std::vector<double> v(p, p + s.elements());
+            return Tensor(v, s, dtype(DataType::kFloat64).requires_grad(grad).device(kDev));
+        };
+        auto put = [](const Tensor &t, double *dst) {
+            auto v = t.to_vector<double>();
+            std::memcpy(dst, v.data(), v.size() * sizeof(double));
+        };
+        auto X = f64(x, Shape{(size_t)m, (size_t)k}, true);
+        auto W = f64(w, Shape{(size_t)k, (size_t)n}, true);
+        auto G = f64(gy, Shape{(size_t)m, (size_t)n}, false);
+        auto Y = F::mat_mul(X, W);
+        auto Z = Y * G;
+        Z.backward();
+        put(Y, y);
+        put(X.grad(), gx);
+        put(W.grad(), gw);
+    });
+}
+
 int DRV(transpose)(const float *src, float *dst, const int64_t *shape, int nd)
 {
     return guarded([&] { out(f32(src, make_shape(shape, nd)).transpose(), dst); });

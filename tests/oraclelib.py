@@ -20,6 +20,7 @@ _T = {"p": ctypes.c_void_p, "l": ctypes.c_int64, "i": ctypes.c_int, "f": ctypes.
 # signature strings: p pointer, l int64, i int, f float; return type after '>' (i int, f float, l int64, v void)
 _ORC_SIGS = {
     "orc_matmul": "ppplll>v",
+    "orc_matmul_f64": "ppplll>v",
     "orc_matmul_batched": "ppplllli>v",
     "orc_matmul_rows": "pppllll>v",
     "orc_transpose": "pplll>v",
@@ -97,6 +98,7 @@ _REF_SIGS = {
     "odl_ref_mlp_bench": "lllliipp>i",
     "odl_ref_cnn_bench": "liipp>i",
     "odl_ref_mlp_model_bench": "lllliiipp>i",
+    "odl_ref_matmul_f64_fwd_bwd": "pppppplll>i",
 }
 
 

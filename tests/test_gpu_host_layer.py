@@ -592,6 +592,28 @@ def test_yolov5n_pnnx_forward_at_the_benchmark_size_matches_the_reference(h, tmp
     assert np.isfinite(out).all()
 
 
+def test_float64_matmul_and_its_gradients_through_the_tensor_api(h):
+    """F::mat_mul on float64 tensors, forward and backward through the autograd graph (MatMul::backward,
+    src/operators/math/mat_mul.cpp:123-182), on the FP64 matrix cores against the compiled reference on the CPU (where it
+    was built) and against numpy: within k * 2^-52 * sum |a||b| per element."""
+    rng = np.random.default_rng(12)
+    for (m, k, n) in ((5, 7, 3), (130, 257, 96), (64, 512, 200)):
+        x, w, gy = rng.standard_normal((m, k)), rng.standard_normal((k, n)), rng.standard_normal((m, n))
+        y, gx, gw = np.empty((m, n)), np.empty((m, k)), np.empty((k, n))
+        assert h.odl_host_matmul_f64_fwd_bwd(x, w, gy, y, gx, gw, m, k, n) == 0
+        eps = 2.0 ** -52
+        assert (np.abs(y - x @ w) <= k * eps * (np.abs(x) @ np.abs(w))).all()
+        assert (np.abs(gx - gy @ w.T) <= n * eps * (np.abs(gy) @ np.abs(w.T))).all()
+        assert (np.abs(gw - x.T @ gy) <= m * eps * (np.abs(x.T) @ np.abs(gy))).all()
+        if ol.have_ref():
+            r = ol.ref()
+            yr, gxr, gwr = np.empty((m, n)), np.empty((m, k)), np.empty((k, n))
+            assert r.odl_ref_matmul_f64_fwd_bwd(x, w, gy, yr, gxr, gwr, m, k, n) == 0
+            assert (np.abs(y - yr) <= k * eps * (np.abs(x) @ np.abs(w))).all()
+            assert (np.abs(gx - gxr) <= n * eps * (np.abs(gy) @ np.abs(w.T))).all()
+            assert (np.abs(gw - gwr) <= m * eps * (np.abs(x.T) @ np.abs(gy))).all()
+
+
 def test_pnnx_runner_with_nodes_folded_together_gives_the_floats_of_running_them_one_by_one(h, tmp_path):
     """The runner folds a residual add into the convolution before it, lets producers write straight into a
     concatenation's output, runs SPPF's three pools as one launch and decodes each detect stage into its rows of the

@@ -207,6 +207,44 @@ def test_matmul_full_size_sampled_rows_and_linearity(api, o, size):
     assert (np.abs(lhs - rhs) <= 3 * bound).all()
 
 
+@pytest.mark.parametrize("m,k,n", [(2, 2, 2), (64, 64, 64), (200, 136, 520), (129, 17, 257), (512, 1000, 784), (1024, 1024, 1024),
+                                   (1, 7, 1), (130, 1, 5)])
+def test_matmul_float64_all_layouts_vs_the_double_oracle(api, o, m, k, n):
+    """odl_hip_dgemm (FP64 matrix cores) against the double form of the reference's loops: every element within
+    k * 2^-52 * sum |a||b| of it (a different but fixed summation order), integer-valued operands bit for bit, in all four
+    layouts (NN; NT and TN are the two products of MatMul::backward; TT for completeness) and over ragged edges."""
+    print("\n[case] matmul float64", m, k, n, flush=True)
+    rng = np.random.default_rng(m * 7 + k + n)
+    a, b = rng.standard_normal((m, k)), rng.standard_normal((k, n))
+    want = np.empty((m, n), np.float64)
+    o.orc_matmul_f64(a, b, want, m, n, k)
+    bound = k * 2.0 ** -52 * (np.abs(a) @ np.abs(b)) + 1e-300
+    for ta, tb in ((0, 0), (0, 1), (1, 0), (1, 1)):
+        A = dev(np.ascontiguousarray(a.T) if ta else a)
+        B = dev(np.ascontiguousarray(b.T) if tb else b)
+        got = host(api.matmul_f64(A, B, bool(ta), bool(tb)))
+        assert got.shape == (m, n) and (np.abs(got - want) <= bound).all(), (ta, tb)
+    ai = rng.integers(-30, 30, (m, k)).astype(np.float64)
+    bi = rng.integers(-30, 30, (k, n)).astype(np.float64)
+    assert np.array_equal(host(api.matmul_f64(dev(ai), dev(bi))), ai @ bi)
+
+
+def test_matmul_float64_batched_and_errors(api, o):
+    rng = np.random.default_rng(5)
+    a, b2, b3 = rng.standard_normal((3, 70, 33)), rng.standard_normal((33, 45)), rng.standard_normal((3, 33, 45))
+    for b in (b2, b3):
+        got = host(api.matmul_f64(dev(a), dev(b)))
+        want = a @ b
+        assert (np.abs(got - want) <= 33 * 2.0 ** -52 * (np.abs(a) @ np.abs(b))).all()
+    with pytest.raises(api.OdlInvalidArgument):
+        api.matmul_f64(dev(a[0]), dev(rng.standard_normal((34, 45))))
+    with pytest.raises(api.OdlInvalidArgument):  # a leading dimension shorter than the row
+        api.lib().call("odl_hip_dgemm", 0, 0, 4, 4, 4, 8, 2, 8, 4, 8, 4, 1, 0, 0, 0, None)
+    # K = 0: an empty sum is 0
+    z = host(api.matmul_f64(dev(np.zeros((5, 0))), dev(np.zeros((0, 6)))))
+    assert z.shape == (5, 6) and (z == 0).all()
+
+
 def test_transpose(api, o):
     rng = np.random.default_rng(3)
     # tiles of 64x64: ragged edges on both sides, whole tiles read and written 16 bytes per lane, batches, single rows

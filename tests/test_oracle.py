@@ -59,6 +59,27 @@ def test_matmul_reference_vectors():
     a, b, c = np.ones((5, 1000), f32), np.ones((1000, 3), f32), np.empty((5, 3), f32)
     o.orc_matmul(a, b, c, 5, 3, 1000)
     assert (c == 1000).all()
+    # the float64 form of the same loops: the unit-test vectors above in double, integer-valued operands (every partial
+    # sum exact, so any order gives the same bits as numpy's), and random operands against numpy's own double product
+    for a, b, exp, (m, k, n) in [([1, 2, 3, 4], [5, 6, 7, 8], [19, 22, 43, 50], (2, 2, 2)),
+                                 ([1, 2, 3, 4, 5, 6], [7, 8, 9, 10, 11, 12], [58, 64, 139, 154], (2, 3, 2))]:
+        c = np.empty((m, n), np.float64)
+        o.orc_matmul_f64(np.array(a, np.float64), np.array(b, np.float64), c, m, n, k)
+        assert c.ravel().tolist() == exp
+    rng = np.random.default_rng(8)
+    ai, bi = rng.integers(-50, 50, (23, 41)).astype(np.float64), rng.integers(-50, 50, (41, 17)).astype(np.float64)
+    c = np.empty((23, 17), np.float64)
+    o.orc_matmul_f64(ai, bi, c, 23, 17, 41)
+    assert np.array_equal(c, ai @ bi)
+    ar, br = rng.standard_normal((23, 41)), rng.standard_normal((41, 17))
+    o.orc_matmul_f64(ar, br, c, 23, 17, 41)
+    bound = 1e-15 * 41 * (np.abs(ar) @ np.abs(br))
+    assert (np.abs(c - ar @ br) <= bound).all()
+    # a transposed operand or a dropped term would show: against the float32 oracle on float32-exact inputs
+    c32 = np.empty((23, 17), f32)
+    o.orc_matmul(ai.astype(f32), bi.astype(f32), c32, 23, 17, 41)
+    o.orc_matmul_f64(ai, bi, c, 23, 17, 41)
+    assert np.array_equal(c32.astype(np.float64), c)
 
 
 def test_conv2d_reference_vectors():
