@@ -24,6 +24,16 @@
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+namespace odl
+{
+// gemm_skinny.hip: products whose output has at most 16 columns (a classifier layer), on the vector ALUs
+bool skinny_ok(int64_t M, int64_t N, int64_t K);
+int skinny_forward(const float *x, const float *w, const float *bias, float *y, int64_t M, int64_t N, int64_t K, int64_t ldx,
+                   int64_t ldw, int64_t ldy, int act, hipStream_t st);
+int skinny_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M, int64_t K, int64_t N,
+                    hipStream_t st);
+}  // namespace odl
+
 namespace
 {
 constexpr int kThreads = 256;
@@ -1119,6 +1129,10 @@ int sgemm_launch(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, cons
     ODL_REQUIRE(lda >= (trans_a ? M : K) && ldb >= (trans_b ? K : N) && (epi == EPI_NCHW_ROWB || ldc >= N),
                 "sgemm: leading dimension smaller than the row length");
     ODL_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "sgemm: dimension exceeds 2^31");
+    // a classifier layer's handful of output columns: vector-ALU kernel, one launch, no K slices (gemm_skinny.hip)
+    if (!trans_a && !trans_b && epi != EPI_NCHW_ROWB && split_k < 1 && odl::skinny_ok(M, N, K))
+        return odl::skinny_forward(A, B, epi == EPI_BIAS_COL ? bias : nullptr, C, M, N, K, lda, ldb, ldc,
+                                   epi == EPI_BIAS_COL && bias ? act : 0, st);
     GemmArgs g;
     g.A = A, g.B = B, g.C = C, g.bias = bias;
     g.M = M, g.N = N, g.K = K, g.lda = lda, g.ldb = ldb, g.ldc = ldc, g.P = P, g.act = act;
@@ -1666,6 +1680,8 @@ int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, flo
 {
     ODL_REQUIRE_DEVICE();
     hipStream_t st = odl::as_stream(stream);
+    if ((gx || gw) && x && w && gy && M > 0 && odl::skinny_ok(M, N, K))
+        return odl::skinny_backward(x, w, gy, gx, gw, M, K, N, st);  // both gradients of a classifier layer in one launch
     if (gx && gw && x && w && gy)
     {
         const int paired = odl::matmul_backward_pair(x, w, gy, gx, gw, M, K, N, st);

@@ -92,6 +92,35 @@ def test_matmul_forward_backward_vs_oracle(api, o, m, k, n):
     assert_gemm_close(gw[krows], gwo, xT[krows], gy, "dB")
 
 
+@pytest.mark.parametrize("m,k,n", [(512, 1000, 10), (511, 1001, 10), (3, 128, 16), (1, 4100, 1), (1030, 130, 7), (64, 2049, 3)])
+def test_classifier_layer_products_on_the_vector_units(api, o, m, k, n):
+    """Outputs of at most 16 columns over a K of 128 or more take gemm_skinny.hip: forward with bias and activation in
+    one launch, both gradients in one launch, either gradient alone the same floats as both together."""
+    print("\n[case] classifier products", m, k, n, flush=True)
+    rng = np.random.default_rng(m + k + n)
+    x, w, gy, b = (rng.standard_normal(s, dtype=f32) for s in ((m, k), (k, n), (m, n), (n,)))
+    yo = np.empty((m, n), f32)
+    o.orc_matmul(x, w, yo, m, n, k)
+    assert_gemm_close(host(api.mat_mul(dev(x), dev(w))), yo, x, w, "C")
+    dx, dw, db = dev(x), dev(w), dev(b)
+    fused = torch.empty((m, n), device="cuda")
+    plain = api.binary("add", api.mat_mul(dx, dw), dev(np.broadcast_to(b, (m, n)).copy()))
+    for code, act in ((-1, None), (0, "relu"), (7, "silu")):
+        api.lib().call("odl_hip_linear_act", dx.data_ptr(), dw.data_ptr(), db.data_ptr(), m, n, k, code, fused.data_ptr(), None, 0,
+                       None)
+        want = host(api.unary(act, plain)) if act else host(plain)
+        assert np.array_equal(host(fused), want), act
+    gx, gw = (host(t) for t in api.mat_mul_backward(dev(x), dev(w), dev(gy)))
+    gxo, gwo = np.empty((m, k), f32), np.empty((k, n), f32)
+    o.orc_matmul_backward(x, w, gy, gxo, gwo, m, k, n)
+    assert_gemm_close(gx, gxo, gy, np.ascontiguousarray(w.T), "dA")
+    assert_gemm_close(gw, gwo, np.ascontiguousarray(x.T), gy, "dB")
+    gx1, none = api.mat_mul_backward(dev(x), dev(w), dev(gy), need_gw=False)
+    assert none is None and np.array_equal(host(gx1), gx)
+    none, gw1 = api.mat_mul_backward(dev(x), dev(w), dev(gy), need_gx=False)
+    assert none is None and np.array_equal(host(gw1), gw)
+
+
 @pytest.mark.parametrize("m,k,n", [(512, 784, 1000), (1024, 1024, 1024), (2048, 2048, 2048), (516, 780, 1004),
                                    (772, 1028, 520), (1000, 1000, 1000), (260, 516, 772), (2044, 2052, 1996)])
 def test_matmul_backward_in_one_launch_equals_the_two_gradients_launched_alone(api, m, k, n):
