@@ -73,6 +73,13 @@ int odl_hip_device_synchronize(void); /* every stream of the current device */
 /* pinned host memory that kernels can write (hipHostMalloc): for the few words a caller polls after a synchronise */
 int odl_hip_host_alloc(void **ptr, size_t bytes);
 int odl_hip_host_free(void *ptr);
+/* events: a point in a stream's queue the host can wait for without waiting for what was queued after it (the loss of a
+ * step is read while the step's backward pass is still running). Created without timing; not to be recorded into a
+ * capture. */
+int odl_hip_event_create(void **event);
+int odl_hip_event_destroy(void *event);
+int odl_hip_event_record(void *event, void *stream);
+int odl_hip_event_synchronize(void *event);
 int odl_hip_graph_capture_begin(void *stream);
 int odl_hip_graph_capture_end(void *stream, void **graph_exec);
 /* how many nodes (launches) the graph that this thread ended last holds */

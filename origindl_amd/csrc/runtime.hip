@@ -255,6 +255,36 @@ int odl_hip_graph_capture_begin(void *stream)
     return ODL_OK;
 }
 
+int odl_hip_event_create(void **event)
+{
+    ODL_REQUIRE(event != nullptr, "event_create: null argument");
+    hipEvent_t e = nullptr;
+    ODL_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    *event = e;
+    return ODL_OK;
+}
+
+int odl_hip_event_destroy(void *event)
+{
+    if (event)
+        ODL_HIP_CHECK(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return ODL_OK;
+}
+
+int odl_hip_event_record(void *event, void *stream)
+{
+    ODL_REQUIRE(event != nullptr, "event_record: null event");
+    ODL_HIP_CHECK(hipEventRecord(static_cast<hipEvent_t>(event), odl::as_stream(stream)));
+    return ODL_OK;
+}
+
+int odl_hip_event_synchronize(void *event)
+{
+    ODL_REQUIRE(event != nullptr, "event_synchronize: null event");
+    ODL_HIP_CHECK(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+    return ODL_OK;
+}
+
 static thread_local int64_t t_last_graph_nodes = 0;
 
 int odl_hip_graph_last_node_count(int64_t *nodes)

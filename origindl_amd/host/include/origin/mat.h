@@ -89,11 +89,15 @@ public:
     // the buffer to that kernel; like the host copy above it stops being trusted at the next data() call. A kernel
     // recorded into a graph keeps writing the words on every replay, so they are never given back (`recorded`).
     // `stream` is the stream of the kernel that writes the words: the slot goes back to that stream's free list only.
-    void set_mirror(void *pinned_words, bool recorded, void *stream) const
+    // `event` (may be null): recorded right behind that kernel; a reader then waits for it alone, not for the work queued
+    // after it.
+    void set_mirror(void *pinned_words, bool recorded, void *stream, void *event = nullptr) const
     {
-        mirror_ = pinned_words, mirror_stream_ = stream, mirror_recorded_ = recorded, mirror_valid_ = pinned_words != nullptr;
+        mirror_ = pinned_words, mirror_stream_ = stream, mirror_recorded_ = recorded, mirror_event_ = event;
+        mirror_valid_ = pinned_words != nullptr;
     }
-    // the device is synchronised and `n` bytes are read from the mirror; false when there is none to trust
+    // waits for the kernel that writes the mirror (its event, or the whole device when there is none) and reads `n`
+    // bytes from it; false when there is none to trust
     bool read_mirror(void *dst, size_t n) const;
     DeviceType device_type() const { return type_; }
     int device_index() const { return index_; }
@@ -117,7 +121,7 @@ private:
     mutable unsigned char fill_element_[8] = {0};
     mutable std::atomic<bool> int_range_valid_{false};
     mutable int64_t int_lo_ = 0, int_hi_ = 0;
-    mutable void *mirror_ = nullptr, *mirror_stream_ = nullptr;
+    mutable void *mirror_ = nullptr, *mirror_stream_ = nullptr, *mirror_event_ = nullptr;
     mutable std::atomic<bool> mirror_valid_{false};
     mutable bool mirror_recorded_ = false;
 };

@@ -391,6 +391,15 @@ public:
         mine.pop_back();
         return slot;
     }
+    // the event that goes with a slot (made when first asked for, kept for the life of the process)
+    void *event_of(void *slot)
+    {
+        std::lock_guard<std::mutex> lock(mutex_);
+        void *&e = events_[slot];
+        if (!e)
+            check(odl_hip_event_create(&e));
+        return e;
+    }
     void give(void *slot, void *stream)
     {
         std::lock_guard<std::mutex> lock(mutex_);
@@ -401,6 +410,7 @@ private:
     std::mutex mutex_;
     std::vector<void *> fresh_;                    // never handed to a kernel yet
     std::map<void *, std::vector<void *>> free_;   // by the stream of the kernel that last wrote the slot
+    std::map<void *, void *> events_;              // slot -> its event
 };
 
 // The buffers of this thread whose fill may still be pending. A capture must not record the fill of a buffer that was
@@ -456,7 +466,10 @@ bool Storage::read_mirror(void *dst, size_t n) const
 {
     if (!mirror_valid_ || n > 8)
         return false;
-    check(odl_hip_device_synchronize());
+    if (mirror_event_)
+        check(odl_hip_event_synchronize(mirror_event_));  // the loss kernel is done; what was queued after it may still run
+    else
+        check(odl_hip_device_synchronize());
     std::memcpy(dst, mirror_, n);
     return true;
 }
@@ -1905,7 +1918,14 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) 
     void *mirror = MirrorPool::get().take(cur());
     check(odl_hip_softmax_ce_loss_device(fp(x), t.storage()->data(), is64, N, C, static_cast<float *>(storage->data()),
                                          mirror, ws.ptr(), ws.bytes, cur()));
-    storage->set_mirror(mirror, t_capturing, cur());
+    // outside a capture an event behind the kernel lets the host read the loss without waiting for the backward pass
+    void *event = nullptr;
+    if (!t_capturing)
+    {
+        event = MirrorPool::get().event_of(mirror);
+        check(odl_hip_event_record(event, cur()));
+    }
+    storage->set_mirror(mirror, t_capturing, cur(), event);
     return std::make_unique<OriginMat>(std::move(storage), Shape{}, DataType::kFloat32);
 }
 
