@@ -429,10 +429,10 @@ def yolo_forward(h, ref, reps):
 
 
 # HBM-side bytes of one 4096^3 GEMM launch, a recorded constant (counters cannot be read from inside this process):
-# FETCH_SIZE (scaled 2.000x by the calibration copy) 739.0 MiB on average over the NN / NT / TN variants
-# (730 / 748 / 737; between 510 and 880 from run to run) + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc`
+# FETCH_SIZE (scaled 2.000x by the calibration copy) 738.0 MiB on average over the NN / NT / TN variants
+# (713 / 763 / 737; between 510 and 880 from run to run) + WRITE_SIZE (1.000x) 64.0 MiB, from the two `rocprofv3 --pmc`
 # runs of `--pmc-probe` summarised in profiles/hot_kernels_hbm_traffic.md.
-GEMM_4096_TRAFFIC_BYTES = int((739.0 + 64.0) * 1024 * 1024)
+GEMM_4096_TRAFFIC_BYTES = int((738.0 + 64.0) * 1024 * 1024)
 
 
 def pmc_probe(torch, capi, gemm_step):
