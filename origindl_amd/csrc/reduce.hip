@@ -441,11 +441,77 @@ __global__ __launch_bounds__(256) void col_max_chunk_kernel(const float *__restr
         const float v = *p;
         m = (m < v) ? v : m;
     }
-    // (four columns per thread with 16-byte loads measured slower: 60 against 55 us on [16384, 4096])
     if (chunks == 1)
         dst[(int64_t)o * inner + i] = m;
     else
         atomic_max_float(dst + (int64_t)o * inner + i, m);
+}
+
+// The same for columns in fours (inner % 4 == 0, 16-byte aligned rows): a wave reads 1 KB of a row per load and the
+// sixteen waves of a workgroup take every sixteenth row of the chunk; the waves' maxima meet in LDS and one merge per
+// column and workgroup goes to memory — the merges of one column are served one after the other by the L2, so their
+// number per column (the number of chunks), not the scan, was most of the kernel above on a long axis.
+constexpr int kMaxWaves = 16;
+__global__ __launch_bounds__(64 * kMaxWaves) void col_max_chunk4_kernel(const float *__restrict__ src, float *__restrict__ dst, int64_t axis,
+                                                              int64_t inner, unsigned tiles_i, unsigned chunks, int64_t chunk_len)
+{
+    __shared__ f32x4 part[kMaxWaves - 1][64];
+    unsigned b = blockIdx.x;
+    const unsigned ti = b % tiles_i;
+    b /= tiles_i;
+    const unsigned ch = b % chunks, o = b / chunks;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t i = (int64_t)ti * 256 + 4 * lane;
+    const bool live = i < inner;
+    const int64_t a0 = (int64_t)ch * chunk_len, a1 = a0 + chunk_len < axis ? a0 + chunk_len : axis;
+    f32x4 m = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+    if (live)
+    {
+        const float *p = src + ((int64_t)o * axis + a0 + wave) * inner + i;
+        const int64_t step = kMaxWaves * inner;
+        int64_t a = a0 + wave;
+        for (; a + 7 * kMaxWaves < a1; a += 8 * kMaxWaves, p += 8 * step)
+        {
+            f32x4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                v[u] = *reinterpret_cast<const f32x4 *>(p + u * step);
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    m[e] = (m[e] < v[u][e]) ? v[u][e] : m[e];
+        }
+        for (; a < a1; a += kMaxWaves, p += step)
+        {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(p);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                m[e] = (m[e] < v[e]) ? v[e] : m[e];
+        }
+    }
+    if (wave > 0)
+        part[wave - 1][lane] = m;
+    __syncthreads();
+    if (wave > 0 || !live)
+        return;
+#pragma unroll
+    for (int w = 0; w < kMaxWaves - 1; ++w)
+    {
+        const f32x4 v = part[w][lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            m[e] = (m[e] < v[e]) ? v[e] : m[e];
+    }
+    float *d = dst + (int64_t)o * inner + i;
+    if (chunks == 1)
+        *reinterpret_cast<f32x4 *>(d) = m;
+    else
+    {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            atomic_max_float(d + e, m[e]);
+    }
 }
 
 __global__ void max_fill_kernel(float *__restrict__ dst, int64_t n, const float *first)
@@ -951,7 +1017,9 @@ int odl_hip_max_axis(const float *src, int64_t outer, int64_t axis, int64_t inne
     {
         // too few columns to fill the chip with a thread each: chunks of the axis per workgroup
         const int64_t tiles_i = odl::ceil_div(inner, 256);
-        int64_t chunks = odl::ceil_div((int64_t)8 * odl::device_cus(), outer * tiles_i);
+        const bool quads = inner % 4 == 0 && (reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) % 16 == 0;
+        // workgroups of 256 threads, eight per compute unit; of 1024 threads (columns in fours), two
+        int64_t chunks = odl::ceil_div((int64_t)(quads ? 2 : 8) * odl::device_cus(), outer * tiles_i);
         if (chunks > axis / 32)
             chunks = axis / 32;
         if (chunks < 1)
@@ -965,8 +1033,12 @@ int odl_hip_max_axis(const float *src, int64_t outer, int64_t axis, int64_t inne
                                outer * inner, (const float *)nullptr);
             ODL_LAUNCH_CHECK();
         }
-        hipLaunchKernelGGL(col_max_chunk_kernel, dim3((unsigned)(outer * chunks * tiles_i)), dim3(256), 0, st, src, dst, axis,
-                           inner, (unsigned)tiles_i, (unsigned)chunks, chunk_len);
+        if (quads)
+            hipLaunchKernelGGL(col_max_chunk4_kernel, dim3((unsigned)(outer * chunks * tiles_i)), dim3(64 * kMaxWaves), 0, st, src, dst,
+                               axis, inner, (unsigned)tiles_i, (unsigned)chunks, chunk_len);
+        else
+            hipLaunchKernelGGL(col_max_chunk_kernel, dim3((unsigned)(outer * chunks * tiles_i)), dim3(256), 0, st, src, dst,
+                               axis, inner, (unsigned)tiles_i, (unsigned)chunks, chunk_len);
     }
     else
         hipLaunchKernelGGL(col_max_kernel, dim3((unsigned)odl::ceil_div(outer * inner, kBlock)), dim3(kBlock), 0, st,

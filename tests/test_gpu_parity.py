@@ -578,7 +578,7 @@ def test_sum_all_and_max_all(api, o):
     # src/mat/origin/cpu/math/max.cpp:25-40, 58-117 on the shapes that split the scan over workgroups: a long axis over
     # few columns (chunks merged with integer atomics), whole tensors of a million elements; infinities, NaNs that the
     # comparison skips, a NaN first element (the whole-tensor maximum then stays NaN), all-negative and all -inf data
-    for outer, axis, inner in ((1, 5000, 300), (3, 700, 40), (2, 4096, 1028), (1, 100000, 7)):
+    for outer, axis, inner in ((1, 5000, 300), (3, 700, 40), (2, 4096, 1028), (1, 100000, 7), (1, 70, 512), (5, 1001, 260)):
         x = (rng.standard_normal((outer, axis, inner), dtype=f32) - 2.0).astype(f32)
         x[0, axis // 2, 0] = np.inf
         x[0, 3, inner - 1] = np.nan
