@@ -393,6 +393,10 @@ CONV_SEEDED = [
     (7, 16, 5, 6, 64, 3, 3, 1, 1),     # tiles that start and end in the middle of an image; 64 gradient channels
     (3, 16, 8, 8, 24, 3, 3, 1, 1),     # W a multiple of 4: the LDS patch is staged with 16-byte row loads
     (2, 48, 6, 28, 40, 3, 3, 1, 1),    # the same over three channel slabs and rows shared between tiles
+    (3, 16, 8, 8, 40, 3, 3, 2, 1),     # stride 2 with channels in sixteens: several images per pixel tile, ragged filter tile
+    (5, 32, 6, 28, 96, 3, 3, 2, 1),    # the same with 14-pixel output rows and two filter tiles
+    (2, 48, 12, 52, 64, 3, 3, 2, 1),   # wide rows at stride 2
+    (7, 16, 2, 2, 33, 3, 3, 2, 1),     # 2x2 images at stride 2: the top tap row always outside
     # more 3x3/s1/p1 layers with channels in groups of 32 and 64 or more filters: two filter tiles with a ragged second
     # one, three channel groups, rows wider than a pixel tile, a single pixel, tiles that cross image boundaries
     (3, 64, 10, 12, 128, 3, 3, 1, 1),
