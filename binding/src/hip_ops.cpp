@@ -64,6 +64,32 @@ const float *fp(const OriginMat &m)
     return m.data_ptr<float>();
 }
 
+// float32 or float64: the convolution operators take both (src/mat/origin/cuda/conv/conv2d.cu:412-664)
+const OriginMat &real(const OriginMat &m, const char *who)
+{
+    on_device(m, who);
+    if (m.dtype() != DataType::kFloat32 && m.dtype() != DataType::kFloat64)
+        THROW_INVALID_ARG("{}: only float32 and float64 are supported on the device, got {}", who, dtype_to_string(m.dtype()));
+    return m;
+}
+
+void same_type(const OriginMat &a, const OriginMat &b, const char *who)
+{
+    if (a.dtype() != b.dtype())
+        THROW_INVALID_ARG("{}: operands of different element types ({} and {})", who, dtype_to_string(a.dtype()),
+                          dtype_to_string(b.dtype()));
+}
+
+const double *dp(const OriginMat &m)
+{
+    return m.data_ptr<double>();
+}
+
+double *dp(OriginMat &m)
+{
+    return m.data_ptr<double>();
+}
+
 float *fp(OriginMat &m)
 {
     return m.data_ptr<float>();
@@ -580,7 +606,7 @@ std::unique_ptr<Mat> sum_to(const OriginMat &mat, const Shape &target_shape)
 std::unique_ptr<Mat> im2col(const OriginMat &img, std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
                             bool to_matrix)
 {
-    const OriginMat &x = f32(img, "im2col");
+    const OriginMat &x = real(img, "im2col");
     const Shape xs = x.shape();
     if (xs.size() != 4)
         THROW_INVALID_ARG("im2col: input must be 4D (N, C, H, W), but got shape {}", xs.to_string());
@@ -591,16 +617,20 @@ std::unique_ptr<Mat> im2col(const OriginMat &img, std::pair<int, int> k, std::pa
         THROW_INVALID_ARG("im2col: invalid output size OH={}, OW={} for input H={}, W={}", OH, OW, H, W);
     const Shape cs = to_matrix ? Shape{(size_t)(N * OH * OW), (size_t)(C * k.first * k.second)}
                                : Shape{(size_t)N, (size_t)C, (size_t)k.first, (size_t)k.second, (size_t)OH, (size_t)OW};
-    auto col = fresh(x, cs);
-    check(odl_hip_im2col(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
-                         fp(*col), kStream));
+    auto col = fresh(x, cs, x.dtype());
+    if (x.dtype() == DataType::kFloat64)
+        check(odl_hip_im2col_f64(dp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
+                                 dp(*col), kStream));
+    else
+        check(odl_hip_im2col(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
+                             fp(*col), kStream));
     return col;
 }
 
 std::unique_ptr<Mat> col2im(const OriginMat &col_, const Shape &is, std::pair<int, int> k, std::pair<int, int> s,
                             std::pair<int, int> p, bool to_matrix)
 {
-    const OriginMat &col = f32(col_, "col2im");
+    const OriginMat &col = real(col_, "col2im");
     if (is.size() != 4)
         THROW_INVALID_ARG("col2im: input_shape must be 4D (N, C, H, W), but got shape {}", is.to_string());
     const int64_t N = is[0], C = is[1], H = is[2], W = is[3];
@@ -610,16 +640,22 @@ std::unique_ptr<Mat> col2im(const OriginMat &col_, const Shape &is, std::pair<in
                                  : Shape{(size_t)N, (size_t)C, (size_t)k.first, (size_t)k.second, (size_t)OH, (size_t)OW};
     if (OH <= 0 || OW <= 0 || col.shape() != want)
         THROW_INVALID_ARG("col2im: invalid col shape {} for input_shape {}", col.shape().to_string(), is.to_string());
-    auto img = fresh(col, is);
-    check(odl_hip_col2im(fp(col), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
-                         fp(*img), kStream));
+    auto img = fresh(col, is, col.dtype());
+    if (col.dtype() == DataType::kFloat64)
+        check(odl_hip_col2im_f64(dp(col), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
+                                 dp(*img), kStream));
+    else
+        check(odl_hip_col2im(fp(col), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
+                             fp(*img), kStream));
     return img;
 }
 
 std::unique_ptr<Mat> conv2d(const OriginMat &x_, const OriginMat &W_, const OriginMat *b, std::pair<int, int> s,
                             std::pair<int, int> p)
 {
-    const OriginMat &x = f32(x_, "conv2d"), &w = f32(W_, "conv2d");
+    const OriginMat &x = real(x_, "conv2d"), &w = real(W_, "conv2d");
+    same_type(x, w, "conv2d");
+    const bool f64 = x.dtype() == DataType::kFloat64;
     const Shape xs = x.shape(), wsh = w.shape();
     if (xs.size() != 4)
         THROW_INVALID_ARG("conv2d: x must be 4D (N, C, H, W), but got shape {}", xs.to_string());
@@ -634,14 +670,26 @@ std::unique_ptr<Mat> conv2d(const OriginMat &x_, const OriginMat &W_, const Orig
         THROW_INVALID_ARG("conv2d: invalid output size OH={}, OW={} for input H={}, W={}, kernel=({},{})", OH, OW, H, W, KH,
                           KW);
     const float *bias = nullptr;
+    const double *bias64 = nullptr;
     if (b)
     {
-        const OriginMat &bm = f32(*b, "conv2d");
+        const OriginMat &bm = real(*b, "conv2d");
+        same_type(x, bm, "conv2d");
         if (bm.shape().size() != 1 || (int64_t)bm.shape()[0] != OC)
             THROW_INVALID_ARG("conv2d: b must be 1D with size {}, but got shape {}", OC, bm.shape().to_string());
-        bias = fp(bm);
+        if (f64)
+            bias64 = dp(bm);
+        else
+            bias = fp(bm);
     }
-    auto y = fresh(x, Shape{(size_t)N, (size_t)OC, (size_t)OH, (size_t)OW});
+    auto y = fresh(x, Shape{(size_t)N, (size_t)OC, (size_t)OH, (size_t)OW}, x.dtype());
+    if (f64)
+    {
+        Workspace ws64(odl_hip_conv2d_f64_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second), x);
+        check(odl_hip_conv2d_f64(dp(x), dp(w), bias64, N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second, dp(*y),
+                                 ws64.ptr(), ws64.bytes, kStream));
+        return y;
+    }
     Workspace ws(odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second), x);
     check(odl_hip_conv2d(fp(x), fp(w), bias, N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second, fp(*y), ws.ptr(),
                          ws.bytes, kStream));
@@ -653,7 +701,9 @@ std::unique_ptr<Mat> conv2d(const OriginMat &x_, const OriginMat &W_, const Orig
 std::vector<std::unique_ptr<Mat>> conv2d_backward(const OriginMat &gy_, const OriginMat &x_, const OriginMat &W_,
                                                   const OriginMat *b, std::pair<int, int> s, std::pair<int, int> p)
 {
-    const OriginMat &gy = f32(gy_, "conv2d_backward"), &x = f32(x_, "conv2d_backward"), &w = f32(W_, "conv2d_backward");
+    const OriginMat &gy = real(gy_, "conv2d_backward"), &x = real(x_, "conv2d_backward"), &w = real(W_, "conv2d_backward");
+    same_type(x, gy, "conv2d_backward");
+    same_type(x, w, "conv2d_backward");
     if (gy.shape().size() != 4)
         THROW_INVALID_ARG("conv2d_backward: gy must be 4D (N, OC, OH, OW), but got shape {}", gy.shape().to_string());
     if (x.shape().size() != 4)
@@ -662,14 +712,23 @@ std::vector<std::unique_ptr<Mat>> conv2d_backward(const OriginMat &gy_, const Or
         THROW_INVALID_ARG("conv2d_backward: W must be 4D (OC, C, KH, KW), but got shape {}", w.shape().to_string());
     const int64_t N = x.shape()[0], C = x.shape()[1], H = x.shape()[2], W = x.shape()[3], OC = w.shape()[0];
     const int KH = (int)w.shape()[2], KW = (int)w.shape()[3];
-    auto gx = fresh(x, x.shape());
-    auto gw = fresh(x, w.shape());
+    auto gx = fresh(x, x.shape(), x.dtype());
+    auto gw = fresh(x, w.shape(), x.dtype());
     std::unique_ptr<OriginMat> gb;
     if (b)
-        gb = fresh(x, Shape{(size_t)OC});
-    Workspace ws(odl_hip_conv2d_backward_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second), x);
-    check(odl_hip_conv2d_backward(fp(gy), fp(x), fp(w), N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
-                                  fp(*gx), fp(*gw), gb ? fp(*gb) : nullptr, ws.ptr(), ws.bytes, kStream));
+        gb = fresh(x, Shape{(size_t)OC}, x.dtype());
+    if (x.dtype() == DataType::kFloat64)
+    {
+        Workspace ws64(odl_hip_conv2d_backward_f64_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second), x);
+        check(odl_hip_conv2d_backward_f64(dp(gy), dp(x), dp(w), N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
+                                          dp(*gx), dp(*gw), gb ? dp(*gb) : nullptr, ws64.ptr(), ws64.bytes, kStream));
+    }
+    else
+    {
+        Workspace ws(odl_hip_conv2d_backward_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second), x);
+        check(odl_hip_conv2d_backward(fp(gy), fp(x), fp(w), N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
+                                      fp(*gx), fp(*gw), gb ? fp(*gb) : nullptr, ws.ptr(), ws.bytes, kStream));
+    }
     std::vector<std::unique_ptr<Mat>> grads;
     grads.push_back(std::move(gx));
     grads.push_back(std::move(gw));
@@ -802,14 +861,6 @@ BnDims bn_dims(const char *who, const OriginMat &x, int num_dims, const OriginMa
     return BnDims{(int64_t)x.shape()[0], (int64_t)C, num_dims == 4 ? (int64_t)(x.shape()[2] * x.shape()[3]) : (int64_t)1};
 }
 
-const double *dp(const OriginMat &m)
-{
-    return static_cast<const double *>(m.storage()->data());
-}
-double *dp(OriginMat &m)
-{
-    return static_cast<double *>(m.storage()->data());
-}
 }  // namespace
 
 BatchNormForwardResult batch_norm_forward(const OriginMat &x, const OriginMat &gamma, const OriginMat &beta,

@@ -176,6 +176,25 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
                             float *gw, float *gb, void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_conv2d_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH,
                                                int KW, int SH, int SW, int PH, int PW);
+/* The same five operators on float64 tensors. The reference's device convolution dispatches over the element type
+ * (src/mat/origin/cuda/conv/conv2d.cu:412-664: im2col, col2im, conv2d, conv2d_backward) and runs the CPU algorithm
+ * (src/mat/origin/cpu/conv/conv2d.cpp:39-599) in that type; here the products run on the FP64 matrix cores
+ * (odl_hip_dgemm) with plain gather / scatter kernels around them. Same layouts, same reading of gy as a row-major
+ * [N*OH*OW, OC] matrix in the backward pass, same order of the taps in col2im. gx, gw, gb may each be NULL. */
+int odl_hip_im2col_f64(const double *img, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
+                       int PW, int to_matrix, double *col, void *stream);
+int odl_hip_col2im_f64(const double *col, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
+                       int PW, int to_matrix, double *img, void *stream);
+int odl_hip_conv2d_f64(const double *x, const double *w, const double *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                       int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, double *y, void *workspace,
+                       size_t workspace_bytes, void *stream);
+size_t odl_hip_conv2d_f64_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH,
+                                          int SW, int PH, int PW);
+int odl_hip_conv2d_backward_f64(const double *gy, const double *x, const double *w, int64_t N, int64_t C, int64_t H, int64_t W,
+                                int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, double *gx, double *gw, double *gb,
+                                void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_conv2d_backward_f64_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                                                   int SH, int SW, int PH, int PW);
 
 /* Kernel selection of the 3x3 / stride 1 / padding 1 convolutions. The kernel that keeps the input patch in LDS is
  * chosen for the forward and the input gradient only when it would launch at least `min_workgroups` workgroups (default:

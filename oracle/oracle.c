@@ -945,3 +945,175 @@ int orc_cnn_train_step(const float *x, const void *t, int is64, int64_t N, int64
     free(gr2); free(gy2); free(gp1); free(gr1); free(gy1); free(gx);
     return rc;
 }
+
+/* ============================================================== convolution on float64 tensors */
+/* The reference's device convolution dispatches over the element type (src/mat/origin/cuda/conv/conv2d.cu:412-664) and
+ * runs the algorithm of conv2d.cpp:404-599 in that type: the functions above over doubles, loop for loop. The compiled
+ * reference cannot pin these — its CPU im2col copies a float buffer into the double result (conv2d.cpp:87, 159), so a
+ * double convolution on the CPU returns garbage. They are pinned by the reference tests' known answers with integer
+ * data, by bit-equality with the float functions above on data both types hold exactly, and by numpy restatements of
+ * the mathematics (tests/test_oracle.py). */
+static double *pad_image_f64(const double *img, int64_t N, int64_t C, int64_t H, int64_t W, int PH, int PW)
+{
+    int64_t pH = H + 2 * PH, pW = W + 2 * PW;
+    double *p = (double *)calloc((size_t)(N * C * pH * pW), sizeof(double));
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < C; ++c)
+            for (int64_t h = 0; h < H; ++h)
+                for (int64_t w = 0; w < W; ++w)
+                    p[((n * C + c) * pH + h + PH) * pW + w + PW] = img[((n * C + c) * H + h) * W + w];
+    return p;
+}
+
+int orc_im2col_f64(const double *img, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
+               int PW, int to_matrix, double *col)
+{
+    int64_t OH = orc_conv_outsize(H, KH, SH, PH), OW = orc_conv_outsize(W, KW, SW, PW);
+    if (OH <= 0 || OW <= 0)
+        return ORC_ERR_INVALID_ARG; /* conv2d.cpp:69-75 */
+    int64_t pH = H + 2 * PH, pW = W + 2 * PW;
+    double *p = pad_image_f64(img, N, C, H, W, PH, PW);
+    memset(col, 0, sizeof(double) * (size_t)(N * C * KH * KW * OH * OW));
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < C; ++c)
+            for (int kh = 0; kh < KH; ++kh)
+                for (int kw = 0; kw < KW; ++kw)
+                    for (int64_t oh = 0; oh < OH; ++oh)
+                        for (int64_t ow = 0; ow < OW; ++ow)
+                        {
+                            int64_t hi = kh + SH * oh, wi = kw + SW * ow;
+                            if (hi < pH && wi < pW) /* conv2d.cpp:146, 186 */
+                            {
+                                double v = p[((n * C + c) * pH + hi) * pW + wi];
+                                if (to_matrix) /* conv2d.cpp:116-162 */
+                                    col[((n * OH + oh) * OW + ow) * (C * KH * KW) + (c * KH + kh) * KW + kw] = v;
+                                else /* conv2d.cpp:164-206 */
+                                    col[((((n * C + c) * KH + kh) * KW + kw) * OH + oh) * OW + ow] = v;
+                            }
+                        }
+    free(p);
+    return ORC_OK;
+}
+
+int orc_col2im_f64(const double *col, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH,
+               int PW, int to_matrix, double *img)
+{
+    int64_t OH = orc_conv_outsize(H, KH, SH, PH), OW = orc_conv_outsize(W, KW, SW, PW);
+    if (OH <= 0 || OW <= 0)
+        return ORC_ERR_INVALID_ARG;
+    int64_t pH = H + 2 * PH, pW = W + 2 * PW;
+    double *p = (double *)calloc((size_t)(N * C * pH * pW), sizeof(double));
+    /* conv2d.cpp:320-349 — accumulation order n, c, kh, kw, oh, ow ascending */
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < C; ++c)
+            for (int kh = 0; kh < KH; ++kh)
+                for (int kw = 0; kw < KW; ++kw)
+                    for (int64_t oh = 0; oh < OH; ++oh)
+                        for (int64_t ow = 0; ow < OW; ++ow)
+                        {
+                            int64_t hi = kh + SH * oh, wi = kw + SW * ow;
+                            if (hi < pH && wi < pW)
+                            {
+                                double v = to_matrix
+                                              ? col[((n * OH + oh) * OW + ow) * (C * KH * KW) + (c * KH + kh) * KW + kw]
+                                              : col[((((n * C + c) * KH + kh) * KW + kw) * OH + oh) * OW + ow];
+                                p[((n * C + c) * pH + hi) * pW + wi] += v;
+                            }
+                        }
+    /* conv2d.cpp:352-369 — strip the padding */
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t c = 0; c < C; ++c)
+            for (int64_t h = 0; h < H; ++h)
+                for (int64_t w = 0; w < W; ++w)
+                    img[((n * C + c) * H + h) * W + w] = p[((n * C + c) * pH + h + PH) * pW + w + PW];
+    free(p);
+    return ORC_OK;
+}
+
+void orc_transpose_f64(const double *src, double *dst, int64_t outer, int64_t rows, int64_t cols)
+{
+    for (int64_t o = 0; o < outer; ++o)
+    {
+        for (int64_t i = 0; i < rows; ++i)
+        {
+            for (int64_t j = 0; j < cols; ++j)
+            {
+                dst[o * rows * cols + j * rows + i] = src[o * rows * cols + i * cols + j];
+            }
+        }
+    }
+}
+
+void orc_sum_axis_f64(const double *src, int64_t outer, int64_t axis, int64_t inner, double *dst)
+{
+    for (int64_t o = 0; o < outer; ++o)
+        for (int64_t i = 0; i < inner; ++i)
+        {
+            double s = 0.0f;
+            for (int64_t a = 0; a < axis; ++a)
+                s += src[(o * axis + a) * inner + i];
+            dst[o * inner + i] = s;
+        }
+}
+
+int orc_conv2d_f64(const double *x, const double *w, const double *b, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+               int KH, int KW, int SH, int SW, int PH, int PW, double *y)
+{
+    int64_t OH = orc_conv_outsize(H, KH, SH, PH), OW = orc_conv_outsize(W, KW, SW, PW);
+    if (OH <= 0 || OW <= 0)
+        return ORC_ERR_INVALID_ARG; /* conv2d.cpp:438-444 */
+    int64_t M = N * OH * OW, K = C * KH * KW;
+    double *col = (double *)malloc(sizeof(double) * (size_t)(M * K));
+    double *wT = (double *)malloc(sizeof(double) * (size_t)(K * OC));
+    double *yf = (double *)malloc(sizeof(double) * (size_t)(M * OC));
+    orc_im2col_f64(x, N, C, H, W, KH, KW, SH, SW, PH, PW, 1, col); /* conv2d.cpp:460 */
+    orc_transpose_f64(w, wT, 1, OC, K);                             /* 463-464: W[OC,K] -> W_T[K,OC] */
+    orc_matmul_f64(col, wT, yf, M, OC, K);                          /* 469 */
+    if (b) /* 472-479: bias broadcast to [M,OC] then one double add per element */
+        for (int64_t i = 0; i < M; ++i)
+            for (int64_t oc = 0; oc < OC; ++oc)
+                yf[i * OC + oc] = yf[i * OC + oc] + b[oc];
+    /* 489-509: NHWC -> NCHW */
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t oc = 0; oc < OC; ++oc)
+            for (int64_t oh = 0; oh < OH; ++oh)
+                for (int64_t ow = 0; ow < OW; ++ow)
+                    y[((n * OC + oc) * OH + oh) * OW + ow] = yf[((n * OH + oh) * OW + ow) * OC + oc];
+    free(col);
+    free(wT);
+    free(yf);
+    return ORC_OK;
+}
+
+int orc_conv2d_backward_f64(const double *gy, const double *x, const double *w, int64_t N, int64_t C, int64_t H, int64_t W,
+                        int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, double *gx, double *gw, double *gb)
+{
+    int64_t OH = orc_conv_outsize(H, KH, SH, PH), OW = orc_conv_outsize(W, KW, SW, PW);
+    if (OH <= 0 || OW <= 0)
+        return ORC_ERR_INVALID_ARG;
+    int64_t M = N * OH * OW, K = C * KH * KW;
+    /* conv2d.cpp:548 — gy's NCHW buffer is *viewed* as a row-major [M, OC] matrix, no permutation. */
+    const double *gy2d = gy;
+    double *gyT = (double *)malloc(sizeof(double) * (size_t)(M * OC));
+    double *col = (double *)malloc(sizeof(double) * (size_t)(M * K));
+    orc_transpose_f64(gy2d, gyT, 1, M, OC);                         /* 550: [M,OC] -> [OC,M] */
+    orc_im2col_f64(x, N, C, H, W, KH, KW, SH, SW, PH, PW, 1, col); /* 554 */
+    orc_matmul_f64(gyT, col, gw, OC, K, M);                         /* 559: gW[OC,K] */
+    if (gb)
+    {
+        /* 571-575: gy.sum(2) -> [N,OC,OW]; .sum(2) -> [N,OC]; .sum(0) -> [OC], on the true NCHW gy */
+        double *s1 = (double *)malloc(sizeof(double) * (size_t)(N * OC * OW));
+        double *s2 = (double *)malloc(sizeof(double) * (size_t)(N * OC));
+        orc_sum_axis_f64(gy, N * OC, OH, OW, s1);
+        orc_sum_axis_f64(s1, N * OC, OW, 1, s2);
+        orc_sum_axis_f64(s2, 1, N, OC, gb);
+        free(s1);
+        free(s2);
+    }
+    /* 584-596: gx_col[M,K] = gy2d[M,OC] . W2d[OC,K]; gx = col2im(gx_col) */
+    orc_matmul_f64(gy2d, w, col, M, K, OC);
+    orc_col2im_f64(col, N, C, H, W, KH, KW, SH, SW, PH, PW, 1, gx);
+    free(gyT);
+    free(col);
+    return ORC_OK;
+}

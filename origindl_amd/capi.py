@@ -257,6 +257,69 @@ def conv2d_backward(gy, x, w, has_bias=True, stride=1, pad=0):
     return gx, gw, gb
 
 
+# ---- the same operators on float64 tensors (src/mat/origin/cuda/conv/conv2d.cu:412-664 dispatches over the element type)
+_f64 = torch.float64
+
+
+def im2col_f64(img, kernel_size, stride, pad, to_matrix=True):
+    _chk(img, "img", _f64)
+    if img.dim() != 4:
+        raise OdlInvalidArgument("im2col: input must be 4D (N, C, H, W)")
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = img.shape
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    shape = (N * OH * OW, C * KH * KW) if to_matrix else (N, C, KH, KW, OH, OW)
+    col = _empty([_builtins.max(s, 0) for s in shape], _f64)
+    lib().call("odl_hip_im2col_f64", _p(img), N, C, H, W, KH, KW, SH, SW, PH, PW, int(to_matrix), _p(col), _stream())
+    return col
+
+
+def col2im_f64(col, input_shape, kernel_size, stride, pad, to_matrix=True):
+    _chk(col, "col", _f64)
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = [int(s) for s in input_shape]
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    want = (N * OH * OW, C * KH * KW) if to_matrix else (N, C, KH, KW, OH, OW)
+    if tuple(col.shape) != want:
+        raise OdlInvalidArgument("col2im: invalid col shape %s for input_shape %s" % (tuple(col.shape), (N, C, H, W)))
+    img = _empty((N, C, H, W), _f64)
+    lib().call("odl_hip_col2im_f64", _p(col), N, C, H, W, KH, KW, SH, SW, PH, PW, int(to_matrix), _p(img), _stream())
+    return img
+
+
+def conv2d_f64(x, w, b=None, stride=1, pad=0):
+    """Mat::conv2d (conv2d.cpp:404-512) on float64 tensors."""
+    _chk(x, "x", _f64), _chk(w, "W", _f64)
+    if b is not None:
+        _chk(b, "b", _f64)
+    if x.dim() != 4 or w.dim() != 4 or x.shape[1] != w.shape[1]:
+        raise OdlInvalidArgument("conv2d: x must be (N, C, H, W) and W (OC, C, KH, KW) with the same C")
+    N, C, H, W = x.shape
+    OC, _, KH, KW = w.shape
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    if OH <= 0 or OW <= 0:
+        raise OdlInvalidArgument("conv2d: the window does not fit the padded image")
+    y = _empty((N, OC, OH, OW), _f64)
+    ws, nb = _ws(lib().query("odl_hip_conv2d_f64_workspace_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW))
+    lib().call("odl_hip_conv2d_f64", _p(x), _p(w), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, _p(y), _p(ws), nb, _stream())
+    return y
+
+
+def conv2d_backward_f64(gy, x, w, has_bias=True, stride=1, pad=0):
+    """Mat::conv2d_backward (conv2d.cpp:514-599) on float64 tensors -> (gx, gW, gb or None)."""
+    _chk(gy, "gy", _f64), _chk(x, "x", _f64), _chk(w, "W", _f64)
+    N, C, H, W = x.shape
+    OC, _, KH, KW = w.shape
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    gx, gw = _empty(x.shape, _f64), _empty(w.shape, _f64)
+    gb = _empty((OC,), _f64) if has_bias else None
+    ws, nb = _ws(lib().query("odl_hip_conv2d_backward_f64_workspace_bytes", N, C, H, W, OC, KH, KW, SH, SW, PH, PW))
+    lib().call("odl_hip_conv2d_backward_f64", _p(gy), _p(x), _p(w), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, _p(gx), _p(gw),
+               _p(gb), _p(ws), nb, _stream())
+    return gx, gw, gb
+
+
 # ------------------------------------------------------------------------------- reductions / broadcast
 def _split_axis(shape, axis):
     outer = int(np.prod(shape[:axis])) if axis > 0 else 1

@@ -100,6 +100,49 @@ __global__ __launch_bounds__(kBlock) void cat_copy_kernel(const float *__restric
         d[i] = s[i];
 }
 
+// Concatenation of up to kCatInputs inputs in one launch: dst[m][col0 + j] for j < cols, where the columns are the inputs'
+// chunks one after the other (end[i] = columns up to and including input i). Chunks, strides and bases are multiples of
+// four floats, so a 16-byte piece lies in one input. A workgroup moves 16 KB of one destination row, four loads in
+// flight per thread.
+constexpr int kCatInputs = 8;
+struct CatArgs
+{
+    const float *src[kCatInputs];
+    int64_t end[kCatInputs];
+    int count;
+};
+
+__global__ __launch_bounds__(kBlock) void cat_rows_kernel(const CatArgs a, float *__restrict__ dst, int64_t cols,
+                                                          int64_t dst_stride, int64_t dst_off)
+{
+    const int64_t m = blockIdx.y;
+    float *d = dst + m * dst_stride + dst_off;
+    const int64_t j0 = (int64_t)blockIdx.x * (16 * kBlock) + 4 * threadIdx.x;
+    f32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+    {
+        const int64_t j = j0 + (int64_t)u * 4 * kBlock;
+        if (j < cols)
+        {
+            int i = 0;
+            int64_t start = 0;
+#pragma unroll
+            for (int k = 0; k + 1 < kCatInputs; ++k)
+                if (k + 1 < a.count && j >= a.end[k])
+                    i = k + 1, start = a.end[k];
+            v[u] = *reinterpret_cast<const f32x4 *>(a.src[i] + m * (a.end[i] - start) + (j - start));
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+    {
+        const int64_t j = j0 + (int64_t)u * 4 * kBlock;
+        if (j < cols)
+            *reinterpret_cast<f32x4 *>(d + j) = v[u];
+    }
+}
+
 // gx[nc][h][w] = sum over the scale_h x scale_w block of gy it was copied to, rows then columns ascending — the order
 // in which the reference's loop over gy reaches that input pixel (nn/upsample.cpp:113-131)
 __global__ __launch_bounds__(kBlock) void upsample_nearest_bwd_kernel(const float *__restrict__ gy, float *__restrict__ gx,
@@ -264,6 +307,43 @@ int odl_hip_cat(const float *const *host_inputs, const int64_t *host_axis_sizes,
     }
     hipStream_t st = odl::as_stream(stream);
     int64_t off = 0;
+    // every input in 16-byte pieces: one launch for up to kCatInputs of them
+    bool all_vec = outer > 0 && outer < 65536 && (total_axis * inner) % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    for (int i = 0; i < count && all_vec; ++i)
+        all_vec = (host_axis_sizes[i] * inner) % 4 == 0 &&
+                  (host_axis_sizes[i] * inner == 0 || (host_inputs[i] && reinterpret_cast<uintptr_t>(host_inputs[i]) % 16 == 0));
+    if (all_vec && count >= 2)
+    {
+        const int64_t dst_stride = total_axis * inner;
+        int i = 0;
+        while (i < count)
+        {
+            CatArgs a{};
+            int64_t cols = 0;
+            const int64_t dst_off = off * inner;
+            while (i < count && a.count < kCatInputs)
+            {
+                const int64_t chunk = host_axis_sizes[i] * inner;
+                if (chunk > 0)
+                {
+                    cols += chunk;
+                    a.src[a.count] = host_inputs[i], a.end[a.count] = cols;
+                    ++a.count;
+                }
+                off += host_axis_sizes[i];
+                ++i;
+            }
+            if (cols == 0)
+                continue;
+            for (int k = a.count; k < kCatInputs; ++k)
+                a.src[k] = a.src[a.count - 1], a.end[k] = cols;
+            ODL_REQUIRE(odl::ceil_div(cols, 16 * kBlock) < (1ll << 31), "cat: rows too long");
+            hipLaunchKernelGGL(cat_rows_kernel, dim3((unsigned)odl::ceil_div(cols, 16 * kBlock), (unsigned)outer), dim3(kBlock), 0, st,
+                               a, out, cols, dst_stride, dst_off);
+            ODL_LAUNCH_CHECK();
+        }
+        return ODL_OK;
+    }
     for (int i = 0; i < count; ++i)
     {
         const int64_t chunk = host_axis_sizes[i] * inner;

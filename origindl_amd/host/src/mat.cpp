@@ -210,6 +210,25 @@ const OriginMat &dev_f32(const Mat &m, const char *who)
     return o;
 }
 
+// the convolution operators also run on float64 tensors, as the reference's do (src/mat/origin/cuda/conv/conv2d.cu:412-664)
+const OriginMat &dev_real(const Mat &m, const char *who)
+{
+    const OriginMat &o = as_origin(m);
+    if (o.device().type() != DeviceType::kCUDA)
+        THROW_RUNTIME_ERROR("{}: tensor is on {}; this backend computes on the GPU only (move it with .to(device))", who,
+                            o.device().to_string());
+    if (o.dtype() != DataType::kFloat32 && o.dtype() != DataType::kFloat64)
+        THROW_INVALID_ARG("{}: only float32 and float64 are supported on the device, got {}", who, dtype_to_string(o.dtype()));
+    return o;
+}
+
+void same_dtype(const OriginMat &a, const OriginMat &b, const char *who)
+{
+    if (a.dtype() != b.dtype())
+        THROW_INVALID_ARG("{}: operands of different element types ({} and {})", who, dtype_to_string(a.dtype()),
+                          dtype_to_string(b.dtype()));
+}
+
 const float *fp(const OriginMat &m)
 {
     return m.data_ptr<float>();
@@ -1601,7 +1620,7 @@ std::unique_ptr<Mat> OriginMat::max(int axis) const
 std::unique_ptr<Mat> OriginMat::im2col(std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
                                        bool to_matrix) const
 {
-    const OriginMat &x = dev_f32(*this, "im2col");
+    const OriginMat &x = dev_real(*this, "im2col");
     if (shape_.size() != 4)
         THROW_INVALID_ARG("im2col: input must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
     const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
@@ -1611,16 +1630,20 @@ std::unique_ptr<Mat> OriginMat::im2col(std::pair<int, int> k, std::pair<int, int
         THROW_INVALID_ARG("im2col: invalid output size OH={}, OW={} for input H={}, W={}", OH, OW, H, W);
     const Shape cs = to_matrix ? Shape{(size_t)(N * OH * OW), (size_t)(C * k.first * k.second)}
                                : Shape{(size_t)N, (size_t)C, (size_t)k.first, (size_t)k.second, (size_t)OH, (size_t)OW};
-    auto col = new_like(x, cs);
-    check(odl_hip_im2col(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
-                         col->data_ptr<float>(), cur()));
+    auto col = new_like(x, cs, x.dtype());
+    if (x.dtype() == DataType::kFloat64)
+        check(odl_hip_im2col_f64(x.data_ptr<double>(), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second,
+                                 to_matrix ? 1 : 0, col->data_ptr<double>(), cur()));
+    else
+        check(odl_hip_im2col(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
+                             col->data_ptr<float>(), cur()));
     return col;
 }
 
 std::unique_ptr<Mat> OriginMat::col2im(const Shape &is, std::pair<int, int> k, std::pair<int, int> s,
                                        std::pair<int, int> p, bool to_matrix) const
 {
-    const OriginMat &col = dev_f32(*this, "col2im");
+    const OriginMat &col = dev_real(*this, "col2im");
     if (is.size() != 4)
         THROW_INVALID_ARG("col2im: input_shape must be 4D (N, C, H, W), but got shape {}", is.to_string());
     const int64_t N = is[0], C = is[1], H = is[2], W = is[3];
@@ -1630,9 +1653,13 @@ std::unique_ptr<Mat> OriginMat::col2im(const Shape &is, std::pair<int, int> k, s
                                  : Shape{(size_t)N, (size_t)C, (size_t)k.first, (size_t)k.second, (size_t)OH, (size_t)OW};
     if (OH <= 0 || OW <= 0 || shape_ != want)
         THROW_INVALID_ARG("col2im: invalid col shape {} for input_shape {}", shape_.to_string(), is.to_string());
-    auto img = new_like(col, is);
-    check(odl_hip_col2im(fp(col), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
-                         img->data_ptr<float>(), cur()));
+    auto img = new_like(col, is, col.dtype());
+    if (col.dtype() == DataType::kFloat64)
+        check(odl_hip_col2im_f64(col.data_ptr<double>(), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second,
+                                 to_matrix ? 1 : 0, img->data_ptr<double>(), cur()));
+    else
+        check(odl_hip_col2im(fp(col), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second, to_matrix ? 1 : 0,
+                             img->data_ptr<float>(), cur()));
     return img;
 }
 
@@ -1677,8 +1704,10 @@ std::unique_ptr<Mat> OriginMat::conv2d_packed_weights_for(const Shape &shape_, c
 std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pair<int, int> s, std::pair<int, int> p,
                                            int activation, const Mat *packed_m) const
 {
-    const OriginMat &x = dev_f32(*this, "conv2d");
-    const OriginMat &w = dev_f32(Wm, "conv2d");
+    const OriginMat &x = dev_real(*this, "conv2d");
+    const OriginMat &w = dev_real(Wm, "conv2d");
+    same_dtype(x, w, "conv2d");
+    const bool f64 = x.dtype() == DataType::kFloat64;
     if (shape_.size() != 4)
         THROW_INVALID_ARG("conv2d: x must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
     if (w.shape().size() != 4)
@@ -1693,14 +1722,31 @@ std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pa
         THROW_INVALID_ARG("conv2d: invalid output size OH={}, OW={} for input H={}, W={}, kernel=({},{})", OH, OW, H, W,
                           KH, KW);
     const float *bias = nullptr;
+    const double *bias64 = nullptr;
     if (bm)
     {
-        const OriginMat &b = dev_f32(*bm, "conv2d");
+        const OriginMat &b = dev_real(*bm, "conv2d");
+        same_dtype(x, b, "conv2d");
         if (b.shape().size() != 1 || (int64_t)b.shape()[0] != OC)
             THROW_INVALID_ARG("conv2d: b must be 1D with size {}, but got shape {}", OC, b.shape().to_string());
-        bias = fp(b);
+        if (f64)
+            bias64 = b.data_ptr<double>();
+        else
+            bias = fp(b);
     }
-    auto y = new_like(x, Shape{(size_t)N, (size_t)OC, (size_t)OH, (size_t)OW});
+    auto y = new_like(x, Shape{(size_t)N, (size_t)OC, (size_t)OH, (size_t)OW}, x.dtype());
+    if (f64)
+    {
+        // float64: the products on the FP64 matrix cores, an activation that follows as a pass of its own
+        Workspace ws64(odl_hip_conv2d_f64_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
+                       device().index());
+        check(odl_hip_conv2d_f64(x.data_ptr<double>(), w.data_ptr<double>(), bias64, N, C, H, W, OC, KH, KW, s.first, s.second,
+                                 p.first, p.second, y->data_ptr<double>(), ws64.ptr(), ws64.bytes, cur()));
+        if (activation >= 0)
+            check(odl_hip_unary_dtype(activation, code(DataType::kFloat64), y->storage()->data(), (int64_t)y->elements(),
+                                      y->storage()->data(), cur()));
+        return y;
+    }
     Workspace ws(odl_hip_conv2d_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
                  device().index());
     const float *packed = nullptr;
@@ -1721,9 +1767,11 @@ std::unique_ptr<Mat> OriginMat::conv2d_act(const Mat &Wm, const Mat *bm, std::pa
 std::vector<std::unique_ptr<Mat>> OriginMat::conv2d_backward(const Mat &gym, const Mat &xm, const Mat &Wm, const Mat *bm,
                                                              std::pair<int, int> s, std::pair<int, int> p) const
 {
-    const OriginMat &gy = dev_f32(gym, "conv2d_backward");
-    const OriginMat &x  = dev_f32(xm, "conv2d_backward");
-    const OriginMat &w  = dev_f32(Wm, "conv2d_backward");
+    const OriginMat &gy = dev_real(gym, "conv2d_backward");
+    const OriginMat &x  = dev_real(xm, "conv2d_backward");
+    const OriginMat &w  = dev_real(Wm, "conv2d_backward");
+    same_dtype(x, gy, "conv2d_backward");
+    same_dtype(x, w, "conv2d_backward");
     if (gy.shape().size() != 4)
         THROW_INVALID_ARG("conv2d_backward: gy must be 4D (N, OC, OH, OW), but got shape {}", gy.shape().to_string());
     if (x.shape().size() != 4)
@@ -1733,16 +1781,28 @@ std::vector<std::unique_ptr<Mat>> OriginMat::conv2d_backward(const Mat &gym, con
     const int64_t N = x.shape()[0], C = x.shape()[1], H = x.shape()[2], W = x.shape()[3];
     const int64_t OC = w.shape()[0];
     const int KH = (int)w.shape()[2], KW = (int)w.shape()[3];
-    auto gx = new_like(x, x.shape());
-    auto gw = new_like(x, w.shape());
+    auto gx = new_like(x, x.shape(), x.dtype());
+    auto gw = new_like(x, w.shape(), x.dtype());
     std::unique_ptr<OriginMat> gb;
     if (bm)
-        gb = new_like(x, Shape{(size_t)OC});
-    Workspace ws(odl_hip_conv2d_backward_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
-                 device().index());
-    check(odl_hip_conv2d_backward(fp(gy), fp(x), fp(w), N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
-                                  gx->data_ptr<float>(), gw->data_ptr<float>(), gb ? gb->data_ptr<float>() : nullptr,
-                                  ws.ptr(), ws.bytes, cur()));
+        gb = new_like(x, Shape{(size_t)OC}, x.dtype());
+    if (x.dtype() == DataType::kFloat64)
+    {
+        Workspace ws64(odl_hip_conv2d_backward_f64_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
+                       device().index());
+        check(odl_hip_conv2d_backward_f64(gy.data_ptr<double>(), x.data_ptr<double>(), w.data_ptr<double>(), N, C, H, W, OC, KH,
+                                          KW, s.first, s.second, p.first, p.second, gx->data_ptr<double>(),
+                                          gw->data_ptr<double>(), gb ? gb->data_ptr<double>() : nullptr, ws64.ptr(), ws64.bytes,
+                                          cur()));
+    }
+    else
+    {
+        Workspace ws(odl_hip_conv2d_backward_workspace_bytes(N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second),
+                     device().index());
+        check(odl_hip_conv2d_backward(fp(gy), fp(x), fp(w), N, C, H, W, OC, KH, KW, s.first, s.second, p.first, p.second,
+                                      gx->data_ptr<float>(), gw->data_ptr<float>(), gb ? gb->data_ptr<float>() : nullptr,
+                                      ws.ptr(), ws.bytes, cur()));
+    }
     std::vector<std::unique_ptr<Mat>> grads;  // {gx, gW, [gb]}
     grads.push_back(std::move(gx));
     grads.push_back(std::move(gw));

@@ -304,6 +304,37 @@ int DRV(matmul_f64_fwd_bwd)(const double *x, const double *w, const double *gy, 
     });
 }
 
+// conv2d on float64 tensors through the whole operator path: y = conv2d(x, W, b); (y * gy).backward()
+int DRV(conv2d_f64_fwd_bwd)(const double *gy, const double *x, const double *w, const double *b, int64_t N, int64_t C, int64_t H,
+                            int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, double *y, double *gx,
+                            double *gw, double *gb)
+{
+    return guarded([&] {
+        auto f64 = [](const double *p, const Shape &s, bool grad) {
+            std::vector<double> v(p, p + s.elements());
+            return Tensor(v, s, dtype(DataType::kFloat64).requires_grad(grad).device(kDev));
+        };
+        auto put = [](const Tensor &t, double *dst) {
+            auto v = t.to_vector<double>();
+            std::memcpy(dst, v.data(), v.size() * sizeof(double));
+        };
+        auto X  = f64(x, Shape{(size_t)N, (size_t)C, (size_t)H, (size_t)W}, true);
+        auto Wt = f64(w, Shape{(size_t)OC, (size_t)C, (size_t)KH, (size_t)KW}, true);
+        Tensor B;
+        if (b)
+            B = f64(b, Shape{(size_t)OC}, true);
+        auto Y = F::conv2d(X, Wt, b ? &B : nullptr, {SH, SW}, {PH, PW});
+        auto G = f64(gy, Y.shape(), false);
+        auto Z = Y * G;
+        Z.backward();
+        put(Y, y);
+        put(X.grad(), gx);
+        put(Wt.grad(), gw);
+        if (b && gb)
+            put(B.grad(), gb);
+    });
+}
+
 int DRV(transpose)(const float *src, float *dst, const int64_t *shape, int nd)
 {
     return guarded([&] { out(f32(src, make_shape(shape, nd)).transpose(), dst); });

@@ -21,6 +21,10 @@ _T = {"p": ctypes.c_void_p, "l": ctypes.c_int64, "i": ctypes.c_int, "f": ctypes.
 _ORC_SIGS = {
     "orc_matmul": "ppplll>v",
     "orc_matmul_f64": "ppplll>v",
+    "orc_im2col_f64": "plllliiiiiiip>i",
+    "orc_col2im_f64": "plllliiiiiiip>i",
+    "orc_conv2d_f64": "ppplllll" + "iiiiii" + "p>i",
+    "orc_conv2d_backward_f64": "ppplllll" + "iiiiii" + "ppp>i",
     "orc_matmul_batched": "ppplllli>v",
     "orc_matmul_rows": "pppllll>v",
     "orc_transpose": "pplll>v",
@@ -99,6 +103,7 @@ _REF_SIGS = {
     "odl_ref_cnn_bench": "liipp>i",
     "odl_ref_mlp_model_bench": "lllliiipp>i",
     "odl_ref_matmul_f64_fwd_bwd": "pppppplll>i",
+    "odl_ref_conv2d_f64_fwd_bwd": "pppplllll" + "iiiiii" + "pppp>i",
 }
 
 

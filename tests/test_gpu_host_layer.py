@@ -614,6 +614,28 @@ def test_float64_matmul_and_its_gradients_through_the_tensor_api(h):
             assert (np.abs(gw - gwr) <= m * eps * (np.abs(x.T) @ np.abs(gy))).all()
 
 
+def test_float64_conv2d_and_its_gradients_through_the_tensor_api(h):
+    """F::conv2d on float64 tensors, forward and backward through the autograd graph (Conv2dOp, conv2d.cpp:404-599 in
+    doubles; the reference's device code dispatches over the element type, cuda/conv/conv2d.cu:412-664) against the double
+    oracle. (The compiled reference is no witness here: its CPU im2col returns garbage for doubles.)"""
+    o = ol.oracle()
+    rng = np.random.default_rng(21)
+    eps = 2.0 ** -52
+    for (N, C, H, W, OC, KH, KW, s, p) in ((2, 3, 7, 6, 4, 3, 3, 1, 1), (3, 4, 9, 9, 5, 3, 3, 2, 1), (4, 8, 16, 16, 12, 3, 3, 1, 1)):
+        OH, OW = (H + 2 * p - KH) // s + 1, (W + 2 * p - KW) // s + 1
+        x, gy = rng.standard_normal((N, C, H, W)), rng.standard_normal((N, OC, OH, OW))
+        w, b = rng.standard_normal((OC, C, KH, KW)), rng.standard_normal((OC,))
+        y, gx, gw, gb = np.empty((N, OC, OH, OW)), np.empty_like(x), np.empty_like(w), np.empty_like(b)
+        assert h.odl_host_conv2d_f64_fwd_bwd(gy, x, w, b, N, C, H, W, OC, KH, KW, s, s, p, p, y, gx, gw, gb) == 0
+        yo, gxo, gwo, gbo = np.empty_like(y), np.empty_like(x), np.empty_like(w), np.empty_like(b)
+        assert o.orc_conv2d_f64(x, w, b, N, C, H, W, OC, KH, KW, s, s, p, p, yo) == 0
+        assert o.orc_conv2d_backward_f64(gy, x, w, N, C, H, W, OC, KH, KW, s, s, p, p, gxo, gwo, gbo) == 0
+        terms = N * OH * OW * C * KH * KW  # a loose common bound: every output is a sum of at most this many products
+        for got, want in ((y, yo), (gx, gxo), (gw, gwo), (gb, gbo)):
+            assert np.abs(got - want).max() <= terms * eps * (1 + np.abs(want).max()), (N, C, H, W)
+        assert np.isfinite(y).all() and np.isfinite(gx).all() and np.isfinite(gw).all()
+
+
 def test_pnnx_runner_with_nodes_folded_together_gives_the_floats_of_running_them_one_by_one(h, tmp_path):
     """The runner folds a residual add into the convolution before it, lets producers write straight into a
     concatenation's output, runs SPPF's three pools as one launch and decodes each detect stage into its rows of the
@@ -642,7 +664,7 @@ def test_pnnx_runner_with_nodes_folded_together_gives_the_floats_of_running_them
         print("\n[yolov5n %dx%d] launches per forward: %d folded, %d node by node" % (size, size, nodes[1], nodes[0]), flush=True)
         assert np.array_equal(outs[1], outs[0])
         assert np.isfinite(outs[1]).all()
-        assert nodes[1] <= 70 and nodes[0] >= 100
+        assert nodes[1] <= 70 and nodes[0] >= 85
 
 
 def test_pnnx_runner_rejects_bad_files(h, tmp_path):

@@ -274,6 +274,75 @@ def test_matmul_float64_batched_and_errors(api, o):
     assert z.shape == (5, 6) and (z == 0).all()
 
 
+@pytest.mark.parametrize("N,C,H,W,OC,KH,KW,s,p", [
+    (2, 3, 7, 6, 4, 3, 3, 1, 1), (3, 4, 9, 9, 5, 3, 3, 2, 1), (2, 2, 8, 5, 3, 2, 3, 1, 0), (1, 1, 3, 3, 2, 2, 2, 1, 0),
+    (2, 5, 6, 6, 7, 1, 1, 1, 0), (2, 16, 14, 14, 24, 3, 3, 1, 1), (3, 1, 28, 28, 32, 3, 3, 1, 1),
+    (9, 8, 24, 20, 130, 3, 3, 1, 1),   # 4320 output pixels: the filter gradient's reduction in two runs, the second shorter
+    (2, 3, 64, 64, 16, 6, 6, 2, 2),    # 6x6 window, stride 2, padding 2
+])
+def test_conv_float64_vs_the_double_oracle(api, o, N, C, H, W, OC, KH, KW, s, p):
+    """The convolution operators on float64 tensors (products on the FP64 matrix cores) against the double form of the
+    reference's loops: im2col bit for bit in both layouts, col2im and every product within K * 2^-52 * sum |a||b| per
+    element (a fixed but different summation order), integer data bit for bit."""
+    print("\n[case] conv float64", N, C, H, W, OC, KH, KW, s, p, flush=True)
+    rng = np.random.default_rng(N + 10 * C + OC)
+    OH, OW = (H + 2 * p - KH) // s + 1, (W + 2 * p - KW) // s + 1
+    M, K = N * OH * OW, C * KH * KW
+    x, gy = rng.standard_normal((N, C, H, W)), rng.standard_normal((N, OC, OH, OW))
+    w, b = rng.standard_normal((OC, C, KH, KW)) * np.sqrt(2.0 / K), rng.standard_normal((OC,))
+    eps = 2.0 ** -52
+    # im2col / col2im, both layouts
+    for to_matrix, shape in ((1, (M, K)), (0, (N, C, KH, KW, OH, OW))):
+        col = np.empty(shape)
+        assert o.orc_im2col_f64(x, N, C, H, W, KH, KW, s, s, p, p, to_matrix, col) == 0
+        assert np.array_equal(host(api.im2col_f64(dev(x), (KH, KW), s, p, bool(to_matrix))), col)
+        img = np.empty_like(x)
+        assert o.orc_col2im_f64(col, N, C, H, W, KH, KW, s, s, p, p, to_matrix, img) == 0
+        assert np.array_equal(host(api.col2im_f64(dev(col), x.shape, (KH, KW), s, p, bool(to_matrix))), img)
+    col = np.empty((M, K))
+    o.orc_im2col_f64(x, N, C, H, W, KH, KW, s, s, p, p, 1, col)
+    # forward with and without a bias
+    y = np.empty((N, OC, OH, OW))
+    assert o.orc_conv2d_f64(x, w, b, N, C, H, W, OC, KH, KW, s, s, p, p, y) == 0
+    by = (K * eps * (np.abs(col) @ np.abs(w.reshape(OC, K)).T) + eps * np.abs(b)).reshape(N, OH, OW, OC).transpose(0, 3, 1, 2)
+    assert (np.abs(host(api.conv2d_f64(dev(x), dev(w), dev(b), s, p)) - y) <= by + 1e-300).all()
+    assert (np.abs(host(api.conv2d_f64(dev(x), dev(w), None, s, p)) - (y - b[None, :, None, None])) <= by + 4 * eps * np.abs(y)).all()
+    # backward: gy's buffer read as [M, OC]
+    gxo, gwo, gbo = np.empty_like(x), np.empty_like(w), np.empty_like(b)
+    assert o.orc_conv2d_backward_f64(gy, x, w, N, C, H, W, OC, KH, KW, s, s, p, p, gxo, gwo, gbo) == 0
+    gx, gw, gb = (host(t) for t in api.conv2d_backward_f64(dev(gy), dev(x), dev(w), True, s, p))
+    gy2d = gy.reshape(M, OC)
+    bgw = M * eps * (np.abs(gy2d).T @ np.abs(col)).reshape(w.shape)
+    assert (np.abs(gw - gwo) <= bgw + 1e-300).all()
+    bcol = OC * eps * (np.abs(gy2d) @ np.abs(w.reshape(OC, K)))
+    bgx = np.empty_like(x)
+    o.orc_col2im_f64(bcol, N, C, H, W, KH, KW, s, s, p, p, 1, bgx)
+    assert (np.abs(gx - gxo) <= bgx + KH * KW * eps * np.abs(gxo) + 1e-300).all()
+    assert (np.abs(gb - gbo) <= N * OH * OW * eps * np.abs(gy).sum((0, 2, 3))).all()
+    gx2, gw2, gb2 = api.conv2d_backward_f64(dev(gy), dev(x), dev(w), False, s, p)
+    assert gb2 is None and np.array_equal(host(gw2), gw) and np.array_equal(host(gx2), gx)
+    # integers: every sum exact, whatever its order
+    xi, wi = rng.integers(-8, 8, x.shape).astype(np.float64), rng.integers(-4, 4, w.shape).astype(np.float64)
+    bi, gi = rng.integers(-4, 4, b.shape).astype(np.float64), rng.integers(-4, 4, gy.shape).astype(np.float64)
+    assert o.orc_conv2d_f64(xi, wi, bi, N, C, H, W, OC, KH, KW, s, s, p, p, y) == 0
+    assert np.array_equal(host(api.conv2d_f64(dev(xi), dev(wi), dev(bi), s, p)), y)
+    assert o.orc_conv2d_backward_f64(gi, xi, wi, N, C, H, W, OC, KH, KW, s, s, p, p, gxo, gwo, gbo) == 0
+    for got, want in zip(api.conv2d_backward_f64(dev(gi), dev(xi), dev(wi), True, s, p), (gxo, gwo, gbo)):
+        assert np.array_equal(host(got), want)
+
+
+def test_conv_float64_argument_errors(api):
+    x, w = dev(np.zeros((1, 2, 4, 4))), dev(np.zeros((3, 2, 3, 3)))
+    with pytest.raises(api.OdlInvalidArgument):  # the window does not fit
+        api.conv2d_f64(dev(np.zeros((1, 2, 2, 2))), w)
+    with pytest.raises(api.OdlInvalidArgument):  # a float32 operand
+        api.conv2d_f64(x, dev(np.zeros((3, 2, 3, 3), f32)))
+    with pytest.raises(api.OdlInvalidArgument):  # too small a workspace
+        api.lib().call("odl_hip_conv2d_f64", x.data_ptr(), w.data_ptr(), None, 1, 2, 4, 4, 3, 3, 3, 1, 1, 0, 0, x.data_ptr(),
+                       x.data_ptr(), 8, None)
+    assert api.lib().query("odl_hip_conv2d_f64_workspace_bytes", 1, 2, 4, 4, 3, 3, 3, 1, 1, 0, 0) == 4 * 18 * 8 + (-4 * 18 * 8) % 256
+
+
 def test_transpose(api, o):
     rng = np.random.default_rng(3)
     # tiles of 64x64: ragged edges on both sides, whole tiles read and written 16 bytes per lane, batches, single rows

@@ -82,6 +82,83 @@ def test_matmul_reference_vectors():
     assert np.array_equal(c32.astype(np.float64), c)
 
 
+def _im2col_np(x, KH, KW, SH, SW, PH, PW):
+    """col[(n,oh,ow)][(c,kh,kw)] built from slices of the padded image (an independent restatement, any float type)"""
+    N, C, H, W = x.shape
+    OH, OW = (H + 2 * PH - KH) // SH + 1, (W + 2 * PW - KW) // SW + 1
+    xp = np.pad(x, ((0, 0), (0, 0), (PH, PH), (PW, PW)))
+    col = np.empty((N, OH, OW, C, KH, KW), x.dtype)
+    for kh in range(KH):
+        for kw in range(KW):
+            col[:, :, :, :, kh, kw] = xp[:, :, kh:kh + SH * OH:SH, kw:kw + SW * OW:SW].transpose(0, 2, 3, 1)
+    return col.reshape(N * OH * OW, C * KH * KW)
+
+
+def _col2im_np(col, shape, KH, KW, SH, SW, PH, PW):
+    N, C, H, W = shape
+    OH, OW = (H + 2 * PH - KH) // SH + 1, (W + 2 * PW - KW) // SW + 1
+    c6 = col.reshape(N, OH, OW, C, KH, KW)
+    xp = np.zeros((N, C, H + 2 * PH, W + 2 * PW), col.dtype)
+    for kh in range(KH):
+        for kw in range(KW):
+            xp[:, :, kh:kh + SH * OH:SH, kw:kw + SW * OW:SW] += c6[:, :, :, :, kh, kw].transpose(0, 3, 1, 2)
+    return xp[:, :, PH:PH + H, PW:PW + W]
+
+
+def test_conv2d_f64_restatement_is_pinned():
+    # The convolution over doubles. The compiled reference cannot pin it: its CPU im2col copies a float buffer into
+    # the double result (conv2d.cpp:87, 159), so a double convolution on the CPU returns garbage; the device code
+    # dispatches over the element type (cuda/conv/conv2d.cu:412-664) and is what the doubles here restate. Pinned by
+    # the reference's own known answers with integer data, by the float32 restatement (itself equal to the compiled
+    # reference bit for bit) on data both types hold exactly, and by the mathematics: a direct convolution, and the
+    # backward products written out with numpy on gy's buffer read as [N*OH*OW, OC].
+    rng = np.random.default_rng(20261125)
+    for (N, C, H, W, OC, KH, KW, SH, SW, PH, PW) in ((2, 3, 7, 6, 4, 3, 3, 1, 1, 1, 1), (3, 4, 9, 9, 5, 3, 3, 2, 2, 1, 1),
+                                                    (2, 2, 8, 5, 3, 2, 3, 2, 1, 0, 2)):
+        OH, OW = (H + 2 * PH - KH) // SH + 1, (W + 2 * PW - KW) // SW + 1
+        x, gy = rng.standard_normal((N, C, H, W)), rng.standard_normal((N, OC, OH, OW))
+        w, b = rng.standard_normal((OC, C, KH, KW)), rng.standard_normal((OC,))
+        y, gx, gw, gb = np.empty((N, OC, OH, OW)), np.empty_like(x), np.empty_like(w), np.empty_like(b)
+        assert o.orc_conv2d_f64(x, w, b, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, y) == 0
+        assert o.orc_conv2d_backward_f64(gy, x, w, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, gx, gw, gb) == 0
+        col = _im2col_np(x, KH, KW, SH, SW, PH, PW)
+        want_y = (col @ w.reshape(OC, -1).T + b).reshape(N, OH, OW, OC).transpose(0, 3, 1, 2)
+        gy2d = gy.reshape(N * OH * OW, OC)  # the buffer as it lies
+        want_gw = (gy2d.T @ col).reshape(w.shape)
+        want_gx = _col2im_np(gy2d @ w.reshape(OC, -1), x.shape, KH, KW, SH, SW, PH, PW)
+        for got, want in ((y, want_y), (gw, want_gw), (gx, want_gx), (gb, gy.sum((0, 2, 3)))):
+            assert np.abs(got - want).max() <= 1e-13 * (1 + np.abs(want).max())
+        got_col, got_img = np.empty_like(col), np.empty_like(x)
+        assert o.orc_im2col_f64(x, N, C, H, W, KH, KW, SH, SW, PH, PW, 1, got_col) == 0 and np.array_equal(got_col, col)
+        assert o.orc_col2im_f64(col, N, C, H, W, KH, KW, SH, SW, PH, PW, 1, got_img) == 0
+        assert np.abs(got_img - _col2im_np(col, x.shape, KH, KW, SH, SW, PH, PW)).max() <= 1e-13
+    # test_conv2d.cpp:21-48 and the reinterpreted filter gradient quoted below, in doubles
+    x9, ones = np.arange(1.0, 10.0).reshape(1, 1, 3, 3), np.ones((1, 1, 2, 2))
+    y4 = np.empty((1, 1, 2, 2))
+    assert o.orc_conv2d_f64(x9, ones, None, 1, 1, 3, 3, 1, 2, 2, 1, 1, 0, 0, y4) == 0
+    assert y4.ravel().tolist() == [12, 16, 24, 28]
+    gy8, w8 = np.arange(1.0, 9.0).reshape(1, 2, 2, 2), np.arange(1.0, 9.0).reshape(2, 1, 2, 2)
+    gx9, gw8 = np.empty_like(x9), np.empty_like(w8)
+    assert o.orc_conv2d_backward_f64(gy8, x9, w8, 1, 1, 3, 3, 2, 2, 2, 1, 1, 0, 0, gx9, gw8, None) == 0
+    assert gw8.ravel().tolist() == [62, 78, 110, 126, 74, 94, 134, 154]
+    # integers both element types hold exactly: the two restatements agree to the last bit
+    xi = rng.integers(-8, 8, (2, 3, 6, 5)).astype(np.float64)
+    wi = rng.integers(-4, 4, (4, 3, 3, 2)).astype(np.float64)
+    bi = rng.integers(-4, 4, (4,)).astype(np.float64)
+    OH, OW = (6 + 2 - 3) // 2 + 1, (5 + 0 - 2) // 1 + 1  # 3x2 window, stride 2x1, padding 1x0
+    gi = rng.integers(-4, 4, (2, 4, OH, OW)).astype(np.float64)
+    y64, y32 = np.empty((2, 4, OH, OW)), np.empty((2, 4, OH, OW), f32)
+    assert o.orc_conv2d_f64(xi, wi, bi, 2, 3, 6, 5, 4, 3, 2, 2, 1, 1, 0, y64) == 0
+    assert o.orc_conv2d(xi.astype(f32), wi.astype(f32), bi.astype(f32), 2, 3, 6, 5, 4, 3, 2, 2, 1, 1, 0, y32) == 0
+    assert np.array_equal(y64, y32.astype(np.float64))
+    g64 = [np.empty_like(xi), np.empty_like(wi), np.empty_like(bi)]
+    g32 = [np.empty(xi.shape, f32), np.empty(wi.shape, f32), np.empty(bi.shape, f32)]
+    assert o.orc_conv2d_backward_f64(gi, xi, wi, 2, 3, 6, 5, 4, 3, 2, 2, 1, 1, 0, *g64) == 0
+    assert o.orc_conv2d_backward(gi.astype(f32), xi.astype(f32), wi.astype(f32), 2, 3, 6, 5, 4, 3, 2, 2, 1, 1, 0, *g32) == 0
+    for a64, a32 in zip(g64, g32):
+        assert np.array_equal(a64, a32.astype(np.float64))
+
+
 def test_conv2d_reference_vectors():
     x9 = np.arange(1, 10, dtype=f32).reshape(1, 1, 3, 3)
     ones = np.ones((1, 1, 2, 2), f32)
