@@ -419,20 +419,21 @@ std::unique_ptr<Mat> cat(const std::vector<const OriginMat *> &inputs, int dim)
 {
     if (inputs.empty())
         THROW_RUNTIME_ERROR("cat: no input");
-    const OriginMat &first = f32(*inputs[0], "cat");
+    const OriginMat &first = on_device(*inputs[0], "cat");
     if (inputs.size() == 1)
         return clone(first);
     const Shape fs = first.shape();
     if (dim < 0 || (size_t)dim >= fs.size())
         THROW_RUNTIME_ERROR("cat: dimension {} out of range for {} dimensions", dim, fs.size());
     size_t total = 0;
-    std::vector<const float *> ptrs;
+    std::vector<const void *> ptrs;
     std::vector<int64_t> sizes;
     for (const OriginMat *m : inputs)
     {
         if (!m)
             THROW_RUNTIME_ERROR("cat: null input");
-        const Shape s = f32(*m, "cat").shape();
+        same_type(first, on_device(*m, "cat"), "cat");
+        const Shape s = m->shape();
         if (s.size() != fs.size())
             THROW_RUNTIME_ERROR("cat: all inputs must have same number of dimensions");
         for (size_t d = 0; d < s.size(); ++d)
@@ -441,7 +442,7 @@ std::unique_ptr<Mat> cat(const std::vector<const OriginMat *> &inputs, int dim)
         if (m->device() != first.device())
             THROW_INVALID_ARG("cat: inputs live on different devices");
         total += s[dim];
-        ptrs.push_back(fp(*m));
+        ptrs.push_back(vp(*m));
         sizes.push_back((int64_t)s[dim]);
     }
     std::vector<size_t> od = fs.dims();
@@ -449,14 +450,15 @@ std::unique_ptr<Mat> cat(const std::vector<const OriginMat *> &inputs, int dim)
     const Shape os(od);
     int64_t outer, ax, inner;
     split_axis(os, dim, outer, ax, inner);
-    auto y = fresh(first, os);
-    check(odl_hip_cat(ptrs.data(), sizes.data(), (int)ptrs.size(), outer, inner, fp(*y), kStream));
+    auto y = fresh(first, os, first.dtype());
+    check(odl_hip_cat_dtype(code(first.dtype()), ptrs.data(), sizes.data(), (int)ptrs.size(), outer, inner, y->storage()->data(),
+                            kStream));
     return y;
 }
 
 std::vector<std::unique_ptr<Mat>> split(const OriginMat &input, const std::vector<size_t> &split_sizes, int dim)
 {
-    const OriginMat &x = f32(input, "split");
+    const OriginMat &x = on_device(input, "split");
     const Shape s = x.shape();
     if (dim < 0 || (size_t)dim >= s.size())
         THROW_RUNTIME_ERROR("split: dimension {} out of range for {} dimensions", dim, s.size());
@@ -473,8 +475,8 @@ std::vector<std::unique_ptr<Mat>> split(const OriginMat &input, const std::vecto
     {
         std::vector<size_t> d = s.dims();
         d[dim] = z;
-        auto piece = fresh(x, Shape(d));
-        check(odl_hip_slice_axis(fp(x), outer, ax, inner, off, (int64_t)z, fp(*piece), kStream));
+        auto piece = fresh(x, Shape(d), x.dtype());
+        check(odl_hip_slice_axis_dtype(code(x.dtype()), vp(x), outer, ax, inner, off, (int64_t)z, piece->storage()->data(), kStream));
         off += (int64_t)z;
         parts.push_back(std::move(piece));
     }
@@ -557,12 +559,12 @@ std::unique_ptr<Mat> sum(const OriginMat &mat, int axis, bool keepdim)
 
 std::unique_ptr<Mat> max(const OriginMat &mat, int axis)
 {
-    const OriginMat &x = f32(mat, "max");
+    const OriginMat &x = on_device(mat, "max");
     const Shape s = x.shape();
     if (axis == -1)
     {
-        auto out = fresh(x, Shape{1});
-        check(odl_hip_max_all(fp(x), (int64_t)x.elements(), fp(*out), kStream));
+        auto out = fresh(x, Shape{1}, x.dtype());
+        check(odl_hip_max_all_dtype(code(x.dtype()), vp(x), (int64_t)x.elements(), out->storage()->data(), kStream));
         return out;
     }
     if (axis < 0 || axis >= (int)s.size())
@@ -573,18 +575,18 @@ std::unique_ptr<Mat> max(const OriginMat &mat, int axis)
             rd.push_back(s[i]);
     int64_t outer, ax, inner;
     split_axis(s, axis, outer, ax, inner);
-    auto out = fresh(x, Shape(rd));
-    check(odl_hip_max_axis(fp(x), outer, ax, inner, fp(*out), kStream));
+    auto out = fresh(x, Shape(rd), x.dtype());
+    check(odl_hip_max_axis_dtype(code(x.dtype()), vp(x), outer, ax, inner, out->storage()->data(), kStream));
     return out;
 }
 
 std::unique_ptr<Mat> broadcast_to(const OriginMat &mat, const Shape &target_shape)
 {
-    const OriginMat &x = f32(mat, "broadcast_to");
-    auto out = fresh(x, target_shape);
+    const OriginMat &x = on_device(mat, "broadcast_to");
+    auto out = fresh(x, target_shape, x.dtype());
     const auto sd = dims64(x.shape()), dd = dims64(target_shape);
-    check(odl_hip_broadcast_to(fp(x), sd.data(), (int)x.shape().size(), dd.data(), (int)target_shape.size(), fp(*out),
-                               kStream));
+    check(odl_hip_broadcast_to_dtype(code(x.dtype()), vp(x), sd.data(), (int)x.shape().size(), dd.data(), (int)target_shape.size(),
+                                     out->storage()->data(), kStream));
     return out;
 }
 
@@ -593,12 +595,13 @@ std::unique_ptr<Mat> sum_to(const OriginMat &mat, const Shape &target_shape)
 {
     if (mat.shape() == target_shape)
         return std::make_unique<OriginMat>(mat);
-    const OriginMat &x = f32(mat, "sum_to");
+    const OriginMat &x = on_device(mat, "sum_to");
+    const int dt = code(x.dtype());
     const auto sd = dims64(x.shape()), td = dims64(target_shape);
-    Workspace ws(odl_hip_sum_to_workspace_bytes(sd.data(), (int)x.shape().size(), td.data(), (int)target_shape.size()), x);
-    auto out = fresh(x, target_shape);
-    check(odl_hip_sum_to(fp(x), sd.data(), (int)x.shape().size(), td.data(), (int)target_shape.size(), fp(*out), ws.ptr(),
-                         ws.bytes, kStream));
+    Workspace ws(odl_hip_sum_to_dtype_workspace_bytes(dt, sd.data(), (int)x.shape().size(), td.data(), (int)target_shape.size()), x);
+    auto out = fresh(x, target_shape, x.dtype());
+    check(odl_hip_sum_to_dtype(dt, vp(x), sd.data(), (int)x.shape().size(), td.data(), (int)target_shape.size(),
+                               out->storage()->data(), ws.ptr(), ws.bytes, kStream));
     return out;
 }
 

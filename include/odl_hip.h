@@ -374,6 +374,25 @@ int odl_hip_fill_dtype(void *dst, int dtype, int64_t n, const void *host_value, 
  * any element type, up to 8 dimensions. ODL_ERR_INVALID_ARG for an order that is not a permutation. */
 int odl_hip_permute(const void *src, int dtype, const int64_t *host_shape, int ndim, const int *host_perm, void *dst,
                     void *stream);
+/* Mat::max, Mat::broadcast_to and Mat::sum_to in any element type (src/mat/origin/cuda/math/{max,broadcast_to,sum_to}.cu
+ * dispatch over the type; CPU forms src/mat/origin/cpu/math/max.cpp:20-121, operation_templates.h:433-493,
+ * src/mat/origin/cpu/math/sum_to.cpp:11-76): the semantics and errors of the float32 entry points above — max starts from
+ * the type's lowest value and takes v where `m < v`; the whole-tensor maximum starts from the first element; sum_to
+ * compares shapes from the LEFT, integers sum with wrap-around. Type code 0 forwards to the float32 kernels. */
+int odl_hip_max_axis_dtype(int dtype, const void *src, int64_t outer, int64_t axis, int64_t inner, void *dst, void *stream);
+int odl_hip_max_all_dtype(int dtype, const void *src, int64_t n, void *dst, void *stream);
+int odl_hip_broadcast_to_dtype(int dtype, const void *src, const int64_t *host_src_shape, int src_ndim,
+                               const int64_t *host_dst_shape, int dst_ndim, void *dst, void *stream);
+int odl_hip_sum_to_dtype(int dtype, const void *src, const int64_t *host_src_shape, int src_ndim, const int64_t *host_dst_shape,
+                         int dst_ndim, void *dst, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_sum_to_dtype_workspace_bytes(int dtype, const int64_t *host_src_shape, int src_ndim,
+                                            const int64_t *host_dst_shape, int dst_ndim);
+/* Mat::cat and one piece of Mat::split in any element type (src/mat/origin/cuda/shape/{cat,split}.cu dispatch over the
+ * type): odl_hip_cat and odl_hip_slice_axis for elements of odl_hip_dtype_size(dtype) bytes. */
+int odl_hip_cat_dtype(int dtype, const void *const *host_inputs, const int64_t *host_axis_sizes, int count, int64_t outer,
+                      int64_t inner, void *out, void *stream);
+int odl_hip_slice_axis_dtype(int dtype, const void *src, int64_t outer, int64_t axis_size, int64_t inner, int64_t offset,
+                             int64_t length, void *dst, void *stream);
 /* Mat::sum over [outer, axis, inner] in any type (operation_templates.h:270-357): integers sum with wrap-around in their
  * own width, float64 in a fixed parallel order. through_float != 0 passes each result through a float on its way back
  * into the element type, which is what the reference's whole-tensor sum does (src/mat/origin/cpu/math/sum.cpp:18-35,83-90). */

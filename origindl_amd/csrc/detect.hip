@@ -542,4 +542,97 @@ int odl_hip_yolo_detect_forward(const float *x, const float *conv_w, const float
     return ODL_OK;
 }
 
+// Mat::cat / Mat::split in the other element types (the reference dispatches both over the element type,
+// src/mat/origin/cuda/shape/{cat,split}.cu): pure copies, so elements of 4 or 8 bytes go through the float32 kernels as
+// one or two words each; 1-byte elements take a byte kernel.
+}  // extern "C"
+
+extern "C" size_t odl_hip_dtype_size(int dtype);
+
+namespace
+{
+// dst[m*dst_stride + dst_off + j] = src[m*src_stride + src_off + j] for j < chunk, in bytes; grid (pieces, m)
+__global__ __launch_bounds__(kBlock) void copy_runs_bytes_kernel(const unsigned char *__restrict__ src, unsigned char *__restrict__ dst,
+                                                                 int64_t chunk, int64_t src_stride, int64_t src_off,
+                                                                 int64_t dst_stride, int64_t dst_off)
+{
+    const int64_t m = blockIdx.y;
+    const int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (j < chunk)
+        dst[m * dst_stride + dst_off + j] = src[m * src_stride + src_off + j];
+}
+
+int copy_runs_bytes(const unsigned char *src, unsigned char *dst, int64_t outer, int64_t chunk, int64_t src_stride, int64_t src_off,
+                    int64_t dst_stride, int64_t dst_off, hipStream_t st)
+{
+    for (int64_t m0 = 0; m0 < outer; m0 += 65535)
+    {
+        const int64_t ms = outer - m0 < 65535 ? outer - m0 : 65535;
+        hipLaunchKernelGGL(copy_runs_bytes_kernel, dim3((unsigned)odl::ceil_div(chunk, kBlock), (unsigned)ms), dim3(kBlock), 0, st,
+                           src + m0 * src_stride, dst + m0 * dst_stride, chunk, src_stride, src_off, dst_stride, dst_off);
+        ODL_LAUNCH_CHECK();
+    }
+    return ODL_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int odl_hip_cat_dtype(int dtype, const void *const *host_inputs, const int64_t *host_axis_sizes, int count, int64_t outer,
+                      int64_t inner, void *out, void *stream)
+{
+    const size_t esz = odl_hip_dtype_size(dtype);
+    if (esz == 0)
+        return odl::fail(ODL_ERR_INVALID_ARG, "cat: unknown element type code %d", dtype);
+    if (esz % 4 == 0)
+        return odl_hip_cat(reinterpret_cast<const float *const *>(host_inputs), host_axis_sizes, count, outer,
+                           inner * (int64_t)(esz / 4), static_cast<float *>(out), stream);
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(count >= 1, "cat: requires at least 1 input");
+    ODL_REQUIRE(host_inputs && host_axis_sizes && out, "cat: null argument");
+    ODL_REQUIRE(outer >= 0 && inner >= 0 && outer < 65536 * 32768ll, "cat: bad outer/inner extents");
+    int64_t total_axis = 0;
+    for (int i = 0; i < count; ++i)
+    {
+        ODL_REQUIRE(host_axis_sizes[i] >= 0, "cat: negative axis size");
+        total_axis += host_axis_sizes[i];
+    }
+    int64_t off = 0;
+    for (int i = 0; i < count; ++i)
+    {
+        const int64_t chunk = host_axis_sizes[i] * inner;
+        if (chunk > 0 && outer > 0)
+        {
+            ODL_REQUIRE(host_inputs[i] != nullptr, "cat: input %d is null", i);
+            const int rc = copy_runs_bytes(static_cast<const unsigned char *>(host_inputs[i]), static_cast<unsigned char *>(out), outer,
+                                           chunk, chunk, 0, total_axis * inner, off * inner, odl::as_stream(stream));
+            if (rc != ODL_OK)
+                return rc;
+        }
+        off += host_axis_sizes[i];
+    }
+    return ODL_OK;
+}
+
+int odl_hip_slice_axis_dtype(int dtype, const void *src, int64_t outer, int64_t axis_size, int64_t inner, int64_t offset,
+                             int64_t length, void *dst, void *stream)
+{
+    const size_t esz = odl_hip_dtype_size(dtype);
+    if (esz == 0)
+        return odl::fail(ODL_ERR_INVALID_ARG, "slice: unknown element type code %d", dtype);
+    if (esz % 4 == 0)
+        return odl_hip_slice_axis(static_cast<const float *>(src), outer, axis_size, inner * (int64_t)(esz / 4), offset, length,
+                                  static_cast<float *>(dst), stream);
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(outer >= 0 && axis_size >= 0 && inner >= 0 && outer < 65536 * 32768ll, "slice: bad extents");
+    ODL_REQUIRE(offset >= 0 && length >= 0 && offset + length <= axis_size, "slice: [%lld, %lld) lies outside an axis of %lld",
+                (long long)offset, (long long)(offset + length), (long long)axis_size);
+    const int64_t chunk = length * inner;
+    if (chunk == 0 || outer == 0)
+        return ODL_OK;
+    ODL_REQUIRE(src && dst, "slice: null operand");
+    return copy_runs_bytes(static_cast<const unsigned char *>(src), static_cast<unsigned char *>(dst), outer, chunk, axis_size * inner,
+                           offset * inner, chunk, 0, odl::as_stream(stream));
+}
+
 }  // extern "C"

@@ -5,7 +5,9 @@
 // results do not depend on scheduling (no float atomics anywhere).
 // Behaviour matched: src/mat/origin/cpu/math/{sum,sum_to,max,broadcast}.cpp and
 // include/origin/mat/origin/device_common/operation_templates.h:259-495.
+#include <algorithm>
 #include <cfloat>
+#include <cstdint>
 
 #include "odl_common.h"
 
@@ -1190,6 +1192,256 @@ int odl_hip_broadcast_to(const float *src, const int64_t *host_src_shape, int sr
     hipLaunchKernelGGL(broadcast_kernel, dim3((unsigned)odl::ceil_div(total, kBlock)), dim3(kBlock), 0,
                        odl::as_stream(stream), src, dst, total, d);
     ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------ the same operators in the other element types
+// The reference dispatches max, broadcast_to and sum_to over its six element types
+// (src/mat/origin/cuda/math/{max,broadcast_to,sum_to}.cu through device_common/type_dispatcher.h). float32 takes the
+// kernels above; the other types take the plain forms below (one thread per output element).
+extern "C" size_t odl_hip_dtype_size(int dtype);
+extern "C" int odl_hip_sum_axis_dtype(int dtype, const void *src, int64_t outer, int64_t axis, int64_t inner, int through_float,
+                                      void *dst, void *workspace, size_t workspace_bytes, void *stream);
+extern "C" size_t odl_hip_sum_axis_dtype_workspace_bytes(int dtype, int64_t outer, int64_t axis, int64_t inner);
+
+namespace
+{
+// std::numeric_limits<T>::lowest()
+template <typename T>
+__device__ inline T lowest_of();
+template <>
+__device__ inline double lowest_of<double>()
+{
+    return -DBL_MAX;
+}
+template <>
+__device__ inline int8_t lowest_of<int8_t>()
+{
+    return INT8_MIN;
+}
+template <>
+__device__ inline int32_t lowest_of<int32_t>()
+{
+    return INT32_MIN;
+}
+template <>
+__device__ inline int64_t lowest_of<int64_t>()
+{
+    return INT64_MIN;
+}
+template <>
+__device__ inline uint8_t lowest_of<uint8_t>()
+{
+    return 0;
+}
+
+// max.cpp:58-117: every output starts from lowest() and takes v where `m < v`
+template <typename T>
+__global__ void max_axis_any_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t outer, int64_t axis, int64_t inner)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= outer * inner)
+        return;
+    const int64_t o = t / inner, i = t - o * inner;
+    const T *p = src + o * axis * inner + i;
+    T m = lowest_of<T>();
+    for (int64_t a = 0; a < axis; ++a)
+    {
+        const T v = p[a * inner];
+        m = (m < v) ? v : m;
+    }
+    dst[t] = m;
+}
+
+// max.cpp:25-40: the whole tensor, starting from its first element (a NaN there stays: nothing compares greater). One
+// workgroup; its threads' maxima are merged in thread order.
+template <typename T>
+__global__ __launch_bounds__(1024) void max_all_any_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t n)
+{
+    __shared__ T part[1024];
+    T m = src[0];
+    for (int64_t i = threadIdx.x; i < n; i += 1024)
+    {
+        const T v = src[i];
+        m = (m < v) ? v : m;
+    }
+    part[threadIdx.x] = m;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        for (int i = 1; i < 1024; ++i)
+            m = (m < part[i]) ? part[i] : m;
+        dst[0] = m;
+    }
+}
+
+template <typename T>
+__global__ void broadcast_any_kernel(const T *__restrict__ src, T *__restrict__ dst, int64_t total, BcastDims d)
+{
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total)
+        return;
+    int64_t r = t, si = 0;
+    for (int k = d.nd - 1; k >= 0; --k)
+    {
+        si += (r % d.dshape[k]) * d.sstride[k];
+        r /= d.dshape[k];
+    }
+    dst[t] = src[si];
+}
+
+// f(T{}) for the element type of a code (include/origin/mat/basic_types.h:19-27), float32 excluded
+template <typename F>
+int with_other_type(int dt, const char *who, F &&f)
+{
+    switch (dt)
+    {
+        case 1: return f(double{});
+        case 2: return f(int8_t{});
+        case 3: return f(int32_t{});
+        case 4: return f(int64_t{});
+        case 5: return f(uint8_t{});
+        default: return odl::fail(ODL_ERR_INVALID_ARG, "%s: unknown element type code %d", who, dt);
+    }
+}
+}  // namespace
+
+extern "C" {
+
+int odl_hip_max_axis_dtype(int dtype, const void *src, int64_t outer, int64_t axis, int64_t inner, void *dst, void *stream)
+{
+    if (dtype == 0)
+        return odl_hip_max_axis(static_cast<const float *>(src), outer, axis, inner, static_cast<float *>(dst), stream);
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(outer >= 0 && axis >= 0 && inner >= 0, "max: negative extent");
+    if (outer * inner == 0)
+        return ODL_OK;
+    return with_other_type(dtype, "max", [&](auto tag) {
+        using T = decltype(tag);
+        hipLaunchKernelGGL(max_axis_any_kernel<T>, dim3((unsigned)odl::ceil_div(outer * inner, kBlock)), dim3(kBlock), 0,
+                           odl::as_stream(stream), static_cast<const T *>(src), static_cast<T *>(dst), outer, axis, inner);
+        ODL_LAUNCH_CHECK();
+        return (int)ODL_OK;
+    });
+}
+
+int odl_hip_max_all_dtype(int dtype, const void *src, int64_t n, void *dst, void *stream)
+{
+    if (dtype == 0)
+        return odl_hip_max_all(static_cast<const float *>(src), n, static_cast<float *>(dst), stream);
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(n > 0, "max: empty input");
+    return with_other_type(dtype, "max", [&](auto tag) {
+        using T = decltype(tag);
+        hipLaunchKernelGGL(max_all_any_kernel<T>, dim3(1), dim3(1024), 0, odl::as_stream(stream), static_cast<const T *>(src),
+                           static_cast<T *>(dst), n);
+        ODL_LAUNCH_CHECK();
+        return (int)ODL_OK;
+    });
+}
+
+int odl_hip_broadcast_to_dtype(int dtype, const void *src, const int64_t *host_src_shape, int src_ndim,
+                               const int64_t *host_dst_shape, int dst_ndim, void *dst, void *stream)
+{
+    if (dtype == 0)
+        return odl_hip_broadcast_to(static_cast<const float *>(src), host_src_shape, src_ndim, host_dst_shape, dst_ndim,
+                                    static_cast<float *>(dst), stream);
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(src_ndim >= 0 && dst_ndim >= 0 && src_ndim <= 8 && dst_ndim <= 8, "broadcast_to: at most 8 dims");
+    ODL_REQUIRE(src_ndim <= dst_ndim, "broadcast_to: source has more dims than the target");
+    BcastDims d{};
+    d.nd = dst_ndim;
+    int64_t st = 1;
+    for (int i = 0; i < dst_ndim; ++i)
+    {
+        const int dd = dst_ndim - 1 - i, sd = src_ndim - 1 - i;
+        d.dshape[dd] = host_dst_shape[dd];
+        d.sstride[dd] = 0;
+        if (sd >= 0)
+        {
+            const int64_t ssz = host_src_shape[sd];
+            ODL_REQUIRE(ssz == 1 || ssz == host_dst_shape[dd], "broadcast_to: dim %d of size %lld cannot become %lld", sd,
+                        (long long)ssz, (long long)host_dst_shape[dd]);
+            d.sstride[dd] = (ssz == 1) ? 0 : st;
+            st *= ssz;
+        }
+    }
+    const int64_t total = prod(host_dst_shape, dst_ndim);
+    if (total == 0)
+        return ODL_OK;
+    return with_other_type(dtype, "broadcast_to", [&](auto tag) {
+        using T = decltype(tag);
+        hipLaunchKernelGGL(broadcast_any_kernel<T>, dim3((unsigned)odl::ceil_div(total, kBlock)), dim3(kBlock), 0,
+                           odl::as_stream(stream), static_cast<const T *>(src), static_cast<T *>(dst), total, d);
+        ODL_LAUNCH_CHECK();
+        return (int)ODL_OK;
+    });
+}
+
+size_t odl_hip_sum_to_dtype_workspace_bytes(int dtype, const int64_t *host_src_shape, int src_ndim, const int64_t *host_dst_shape,
+                                            int dst_ndim)
+{
+    if (dtype == 0)
+        return odl_hip_sum_to_workspace_bytes(host_src_shape, src_ndim, host_dst_shape, dst_ndim);
+    const SumToPlan p = plan_sum_to(host_src_shape, src_ndim, host_dst_shape, dst_ndim);
+    if (p.rc != ODL_OK || p.copy || p.npass == 0)
+        return 0;
+    size_t inter = 0, pass = 0;
+    for (int q = 0; q < p.npass; ++q)
+    {
+        inter = std::max(inter, (size_t)(p.outer[q] * p.inner[q]) * odl_hip_dtype_size(dtype));
+        pass = std::max(pass, odl_hip_sum_axis_dtype_workspace_bytes(dtype, p.outer[q], p.axis[q], p.inner[q]));
+    }
+    inter = (inter + 255) & ~(size_t)255;
+    return 2 * inter + ((pass + 255) & ~(size_t)255);
+}
+
+int odl_hip_sum_to_dtype(int dtype, const void *src, const int64_t *host_src_shape, int src_ndim, const int64_t *host_dst_shape,
+                         int dst_ndim, void *dst, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (dtype == 0)
+        return odl_hip_sum_to(static_cast<const float *>(src), host_src_shape, src_ndim, host_dst_shape, dst_ndim,
+                              static_cast<float *>(dst), workspace, workspace_bytes, stream);
+    ODL_REQUIRE_DEVICE();
+    const size_t esz = odl_hip_dtype_size(dtype);
+    ODL_REQUIRE(esz > 0, "sum_to: unknown element type code %d", dtype);
+    hipStream_t st = odl::as_stream(stream);
+    const SumToPlan p = plan_sum_to(host_src_shape, src_ndim, host_dst_shape, dst_ndim);
+    if (p.rc == ODL_ERR_RUNTIME)
+        return odl::fail(ODL_ERR_RUNTIME, "sum_to: Target shape cannot have more elements than source tensor");
+    if (p.rc != ODL_OK)
+        return odl::fail(p.rc, "sum_to: source shape cannot be reduced to the target shape (left-aligned rule)");
+    if (p.copy || p.npass == 0)  // equal shapes, or only size-1 dims differ: a copy
+    {
+        const int64_t n = prod(host_src_shape, src_ndim);
+        if (n && dst != src)
+            ODL_HIP_CHECK(hipMemcpyAsync(dst, src, (size_t)n * esz, hipMemcpyDeviceToDevice, st));
+        return ODL_OK;
+    }
+    const size_t need = odl_hip_sum_to_dtype_workspace_bytes(dtype, host_src_shape, src_ndim, host_dst_shape, dst_ndim);
+    ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need, "sum_to: workspace of %zu bytes required, got %zu", need,
+                workspace_bytes);
+    size_t inter = 0, pass = 0;
+    for (int q = 0; q < p.npass; ++q)
+    {
+        inter = std::max(inter, (size_t)(p.outer[q] * p.inner[q]) * esz);
+        pass = std::max(pass, odl_hip_sum_axis_dtype_workspace_bytes(dtype, p.outer[q], p.axis[q], p.inner[q]));
+    }
+    inter = (inter + 255) & ~(size_t)255;
+    char *ws = static_cast<char *>(workspace);
+    void *buf[2] = {ws, ws + inter};
+    void *pass_ws = ws + 2 * inter;
+    const void *cur = src;
+    for (int q = 0; q < p.npass; ++q)
+    {
+        void *out = (q == p.npass - 1) ? dst : buf[q & 1];
+        const int rc = odl_hip_sum_axis_dtype(dtype, cur, p.outer[q], p.axis[q], p.inner[q], 0, out, pass_ws, pass, stream);
+        if (rc != ODL_OK)
+            return rc;
+        cur = out;
+    }
     return ODL_OK;
 }
 

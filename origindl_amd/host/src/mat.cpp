@@ -1222,7 +1222,7 @@ std::unique_ptr<Mat> OriginMat::axpby(float a, float b, const Mat &other) const
 
 std::vector<std::unique_ptr<Mat>> OriginMat::split(const std::vector<size_t> &sizes, int dim) const
 {
-    const OriginMat &x = dev_f32(*this, "split");
+    const OriginMat &x = dev_any(*this, "split");
     if (dim < 0 || (size_t)dim >= shape_.size())
         THROW_RUNTIME_ERROR("split: dimension {} out of range for {} dimensions", dim, shape_.size());
     size_t total = 0;
@@ -1238,8 +1238,9 @@ std::vector<std::unique_ptr<Mat>> OriginMat::split(const std::vector<size_t> &si
     {
         std::vector<size_t> d = shape_.dims();
         d[dim] = sz;
-        auto piece = new_like(x, Shape(d));
-        check(odl_hip_slice_axis(fp(x), outer, ax, inner, off, (int64_t)sz, piece->data_ptr<float>(), cur()));
+        auto piece = new_like(x, Shape(d), x.dtype());
+        check(odl_hip_slice_axis_dtype(code(x.dtype()), x.storage()->data(), outer, ax, inner, off, (int64_t)sz,
+                                       piece->storage()->data(), cur()));
         off += (int64_t)sz;
         parts.push_back(std::move(piece));
     }
@@ -1263,19 +1264,22 @@ std::unique_ptr<Mat> OriginMat::upsample(const Shape &output_shape, int scale_h,
 
 std::unique_ptr<Mat> OriginMat::cat(const std::vector<const Mat *> &others, int dim) const
 {
-    std::vector<const OriginMat *> in{&dev_f32(*this, "cat")};
+    std::vector<const OriginMat *> in{&dev_any(*this, "cat")};
     for (const Mat *m : others)
     {
         if (!m)
             THROW_RUNTIME_ERROR("cat: null input");
-        in.push_back(&dev_f32(*m, "cat"));
+        in.push_back(&dev_any(*m, "cat"));
+        if (in.back()->dtype() != dtype())
+            THROW_INVALID_ARG("cat: inputs of different element types ({} and {})", dtype_to_string(dtype()),
+                              dtype_to_string(in.back()->dtype()));
     }
     if (in.size() == 1)
         return std::make_unique<OriginMat>(*this);  // shape/cat.cpp:29-33: a single input is returned as it is
     if (dim < 0 || (size_t)dim >= shape_.size())
         THROW_RUNTIME_ERROR("cat: dimension {} out of range for {} dimensions", dim, shape_.size());
     size_t total = 0;
-    std::vector<const float *> ptrs;
+    std::vector<const void *> ptrs;
     std::vector<int64_t> sizes;
     for (const OriginMat *m : in)
     {
@@ -1288,7 +1292,7 @@ std::unique_ptr<Mat> OriginMat::cat(const std::vector<const Mat *> &others, int 
         if (m->device() != device())
             THROW_INVALID_ARG("cat: inputs live on different devices");
         total += s[dim];
-        ptrs.push_back(fp(*m));
+        ptrs.push_back(m->storage()->data());
         sizes.push_back((int64_t)s[dim]);
     }
     std::vector<size_t> od = shape_.dims();
@@ -1296,8 +1300,8 @@ std::unique_ptr<Mat> OriginMat::cat(const std::vector<const Mat *> &others, int 
     const Shape os(od);
     int64_t outer, ax, inner;
     split_axis(os, dim, outer, ax, inner);
-    auto y = new_like(*in[0], os);
-    check(odl_hip_cat(ptrs.data(), sizes.data(), (int)ptrs.size(), outer, inner, y->data_ptr<float>(), cur()));
+    auto y = new_like(*in[0], os, dtype());
+    check(odl_hip_cat_dtype(code(dtype()), ptrs.data(), sizes.data(), (int)ptrs.size(), outer, inner, y->storage()->data(), cur()));
     return y;
 }
 
@@ -1539,11 +1543,11 @@ std::unique_ptr<Mat> OriginMat::matmul(const Mat &other) const
 // -------------------------------------------------------------------------------- reductions / broadcast
 std::unique_ptr<Mat> OriginMat::broadcast_to(const Shape &shape) const
 {
-    const OriginMat &x = dev_f32(*this, "broadcast_to");
-    auto out = new_like(x, shape);
+    const OriginMat &x = dev_any(*this, "broadcast_to");
+    auto out = new_like(x, shape, x.dtype());
     const auto sd = dims64(shape_), dd = dims64(shape);
-    check(odl_hip_broadcast_to(fp(x), sd.data(), (int)shape_.size(), dd.data(), (int)shape.size(),
-                               out->data_ptr<float>(), cur()));
+    check(odl_hip_broadcast_to_dtype(code(x.dtype()), x.storage()->data(), sd.data(), (int)shape_.size(), dd.data(),
+                                     (int)shape.size(), out->storage()->data(), cur()));
     return out;
 }
 
@@ -1551,13 +1555,14 @@ std::unique_ptr<Mat> OriginMat::sum_to(const Shape &shape) const
 {
     if (shape_ == shape)
         return std::make_unique<OriginMat>(*this);  // storage-sharing copy, src/mat/origin/cpu/math/sum_to.cpp:14-18
-    const OriginMat &x = dev_f32(*this, "sum_to");
+    const OriginMat &x = dev_any(*this, "sum_to");
+    const int dt = code(x.dtype());
     const auto sd = dims64(shape_), td = dims64(shape);
-    Workspace ws(odl_hip_sum_to_workspace_bytes(sd.data(), (int)shape_.size(), td.data(), (int)shape.size()),
+    Workspace ws(odl_hip_sum_to_dtype_workspace_bytes(dt, sd.data(), (int)shape_.size(), td.data(), (int)shape.size()),
                  device().index());
-    auto out = new_like(x, shape);
-    check(odl_hip_sum_to(fp(x), sd.data(), (int)shape_.size(), td.data(), (int)shape.size(), out->data_ptr<float>(),
-                         ws.ptr(), ws.bytes, cur()));
+    auto out = new_like(x, shape, x.dtype());
+    check(odl_hip_sum_to_dtype(dt, x.storage()->data(), sd.data(), (int)shape_.size(), td.data(), (int)shape.size(),
+                               out->storage()->data(), ws.ptr(), ws.bytes, cur()));
     return out;
 }
 
@@ -1596,11 +1601,12 @@ std::unique_ptr<Mat> OriginMat::sum(int axis, bool keepdim) const
 
 std::unique_ptr<Mat> OriginMat::max(int axis) const
 {
-    const OriginMat &x = dev_f32(*this, "max");
+    const OriginMat &x = dev_any(*this, "max");
+    const int dt = code(x.dtype());
     if (axis == -1)
     {
-        auto out = new_like(x, Shape{1});
-        check(odl_hip_max_all(fp(x), (int64_t)elements(), out->data_ptr<float>(), cur()));
+        auto out = new_like(x, Shape{1}, x.dtype());
+        check(odl_hip_max_all_dtype(dt, x.storage()->data(), (int64_t)elements(), out->storage()->data(), cur()));
         return out;
     }
     if (axis < 0 || axis >= (int)shape_.size())
@@ -1611,8 +1617,8 @@ std::unique_ptr<Mat> OriginMat::max(int axis) const
             rd.push_back(shape_[i]);
     int64_t outer, ax, inner;
     split_axis(shape_, axis, outer, ax, inner);
-    auto out = new_like(x, Shape(rd));
-    check(odl_hip_max_axis(fp(x), outer, ax, inner, out->data_ptr<float>(), cur()));
+    auto out = new_like(x, Shape(rd), x.dtype());
+    check(odl_hip_max_axis_dtype(dt, x.storage()->data(), outer, ax, inner, out->storage()->data(), cur()));
     return out;
 }
 
@@ -1935,6 +1941,18 @@ std::unique_ptr<Mat> OriginMat::one_hot(const Mat &indices, int num_classes) con
 // ------------------------------------------------------------------------ fused paths above the Mat set
 std::unique_ptr<Mat> OriginMat::softmax(int axis) const
 {
+    if (dtype() == DataType::kFloat64)
+    {
+        // float64: the reference's own composition (src/operators/activation/softmax.cpp:34-76) out of operators that
+        // take every element type — max along the axis, subtract, exp, sum along the axis, divide
+        dev_any(*this, "softmax");
+        std::vector<size_t> kd = shape_.dims();
+        kd[axis] = 1;
+        const Shape keep(kd);
+        auto shifted = *this - *max(axis)->reshape(keep)->broadcast_to(shape_);
+        auto e = shifted->exp();
+        return *e / *e->sum(axis, false)->reshape(keep)->broadcast_to(shape_);
+    }
     const OriginMat &x = dev_f32(*this, "softmax");
     int64_t outer, ax, inner;
     split_axis(shape_, axis, outer, ax, inner);

@@ -335,6 +335,23 @@ int DRV(conv2d_f64_fwd_bwd)(const double *gy, const double *x, const double *w, 
     });
 }
 
+// softmax on a float64 tensor, forward and backward: y = softmax(x, axis); (y * gy).backward()
+int DRV(softmax_f64_fwd_bwd)(const double *x, const double *gy, const int64_t *shape, int nd, int axis, double *y, double *gx)
+{
+    return guarded([&] {
+        const Shape s = make_shape(shape, nd);
+        std::vector<double> xv(x, x + s.elements()), gv(gy, gy + s.elements());
+        auto X = Tensor(xv, s, dtype(DataType::kFloat64).requires_grad(true).device(kDev));
+        auto G = Tensor(gv, s, dtype(DataType::kFloat64).device(kDev));
+        auto Y = F::softmax(X, axis);
+        auto Z = Y * G;
+        Z.backward();
+        auto yv = Y.to_vector<double>(), gxv = X.grad().to_vector<double>();
+        std::memcpy(y, yv.data(), yv.size() * sizeof(double));
+        std::memcpy(gx, gxv.data(), gxv.size() * sizeof(double));
+    });
+}
+
 int DRV(transpose)(const float *src, float *dst, const int64_t *shape, int nd)
 {
     return guarded([&] { out(f32(src, make_shape(shape, nd)).transpose(), dst); });

@@ -104,6 +104,7 @@ _REF_SIGS = {
     "odl_ref_mlp_model_bench": "lllliiipp>i",
     "odl_ref_matmul_f64_fwd_bwd": "pppppplll>i",
     "odl_ref_conv2d_f64_fwd_bwd": "pppplllll" + "iiiiii" + "pppp>i",
+    "odl_ref_softmax_f64_fwd_bwd": "pppiipp>i",
 }
 
 

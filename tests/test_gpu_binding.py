@@ -89,6 +89,10 @@ def test_conv2d_on_float64_tensors_through_the_references_operator(b):
     T.test_float64_conv2d_and_its_gradients_through_the_tensor_api(b)
 
 
+def test_softmax_on_float64_tensors_through_the_references_operator(b):
+    T.test_float64_softmax_through_the_tensor_api(b)
+
+
 @pytest.mark.parametrize("name", sorted(T.POOL_CASES))
 def test_max_pool_indices_bit_exact(b, name):
     T.test_max_pool_through_the_mat_interface_bit_exact(b, name)

@@ -636,6 +636,29 @@ def test_float64_conv2d_and_its_gradients_through_the_tensor_api(h):
         assert np.isfinite(y).all() and np.isfinite(gx).all() and np.isfinite(gw).all()
 
 
+def test_float64_softmax_through_the_tensor_api(h):
+    """F::softmax on float64 tensors, forward and backward: the reference composes it out of max, broadcast_to, subtract,
+    exp, sum and divide (src/operators/activation/softmax.cpp:34-129), each of which dispatches over the element type on
+    its device (src/mat/origin/cuda/math/{max,broadcast_to,sum}.cu). Against numpy in doubles, and against the compiled
+    reference on the CPU where it was built."""
+    rng = np.random.default_rng(33)
+    for shape, axis in (((5, 7), 1), ((4, 3, 6), 1), ((2, 3, 4, 5), -1), ((300, 1000), 1), ((6, 2), 0)):
+        x, gy = rng.standard_normal(shape) * 3, rng.standard_normal(shape)
+        y, gx = np.empty(shape), np.empty(shape)
+        sh = np.asarray(shape, np.int64)
+        assert h.odl_host_softmax_f64_fwd_bwd(x, gy, sh, len(shape), axis, y, gx) == 0
+        e = np.exp(x - x.max(axis=axis, keepdims=True))
+        want = e / e.sum(axis=axis, keepdims=True)
+        want_gx = want * (gy - (gy * want).sum(axis=axis, keepdims=True))
+        n = shape[axis]
+        assert np.abs(y - want).max() <= 4 * n * 2.0 ** -52
+        assert np.abs(gx - want_gx).max() <= 16 * n * 2.0 ** -52 * (1 + np.abs(gy).max())
+        if ol.have_ref():
+            yr, gxr = np.empty(shape), np.empty(shape)
+            assert ol.ref().odl_ref_softmax_f64_fwd_bwd(x, gy, sh, len(shape), axis, yr, gxr) == 0
+            assert np.abs(y - yr).max() <= 4 * n * 2.0 ** -52 and np.abs(gx - gxr).max() <= 16 * n * 2.0 ** -52 * (1 + np.abs(gy).max())
+
+
 def test_pnnx_runner_with_nodes_folded_together_gives_the_floats_of_running_them_one_by_one(h, tmp_path):
     """The runner folds a residual add into the convolution before it, lets producers write straight into a
     concatenation's output, runs SPPF's three pools as one launch and decodes each detect stage into its rows of the

@@ -6,6 +6,7 @@ Bars (from the benchmark contract): integer/index outputs bit-exact; FP32 GEMM-t
 |d| <= 1e-5 * ||a_row||_2 * ||b_col||_2 per element; plain sums within the same bound read as a dot product with
 a vector of ones; softmax/CE within 1e-6 absolute (exp/log of the device library vs glibc); copies, gathers,
 col2im and max-pool backward bit-exact (same additions in the same order)."""
+import ctypes
 import os
 
 import numpy as np
@@ -1497,6 +1498,84 @@ def test_convert_between_all_element_types_is_a_static_cast(api):
     assert [L.query("odl_hip_dtype_size", c) for c in range(7)] == [4, 8, 1, 4, 8, 1, 0]
     with pytest.raises(api.OdlInvalidArgument):
         L.call("odl_hip_convert", d_src.data_ptr(), 9, d_dst.data_ptr(), 0, 4, None)
+
+
+@pytest.mark.parametrize("name", ["f32", "f64", "i8", "i32", "i64", "u8"])
+def test_max_broadcast_sum_to_cat_split_in_every_element_type(api, name):
+    """Mat::max, broadcast_to, sum_to, cat and split dispatch over the element type in the reference
+    (src/mat/origin/cuda/math/{max,broadcast_to,sum_to}.cu, shape/{cat,split}.cu). Checked against numpy: max and the
+    copies bit for bit, sums of integers bit for bit (they wrap in the type's width), sums of doubles within n * 2^-52."""
+    L = api.lib()
+    code, t = DT[name]
+    tt = getattr(torch, np.dtype(t).name)
+    rng = np.random.default_rng(77 + code)
+    is_float = t in (np.float32, np.float64)
+
+    def shape_arr(shape):
+        return (ctypes.c_int64 * max(len(shape), 1))(*shape)
+
+    # ---- max over an axis of [outer, axis, inner] and over the whole tensor
+    for outer, axis, inner in ((1, 300, 1), (4, 37, 5), (3, 1, 7), (2, 513, 64)):
+        x = _typed_values(rng, t, outer * axis * inner).reshape(outer, axis, inner)
+        if is_float and axis > 1:
+            x[0, axis // 2, 0] = np.nan  # never wins: `m < v` is false for it
+        out = torch.empty((outer, inner), dtype=tt, device="cuda")
+        dx = dev(x)
+        L.call("odl_hip_max_axis_dtype", code, dx.data_ptr(), outer, axis, inner, out.data_ptr(), None)
+        want = np.fmax.reduce(x, axis=1) if is_float else x.max(axis=1)
+        assert np.array_equal(host(out), want.astype(t)), (name, outer, axis, inner)
+        one = torch.empty(1, dtype=tt, device="cuda")
+        L.call("odl_hip_max_all_dtype", code, dx.data_ptr(), x.size, one.data_ptr(), None)
+        assert host(one)[0] == (np.nanmax(x) if is_float else x.max())
+    # ---- broadcast_to (right-aligned)
+    for src, dst in (((1, 5), (7, 5)), ((3, 1), (3, 9)), ((4,), (2, 3, 4)), ((2, 1, 3), (2, 5, 3)), ((1,), (6,))):
+        x = _typed_values(rng, t, int(np.prod(src))).reshape(src)
+        out = torch.empty(dst, dtype=tt, device="cuda")
+        dx = dev(x)
+        L.call("odl_hip_broadcast_to_dtype", code, dx.data_ptr(), shape_arr(src), len(src), shape_arr(dst), len(dst),
+               out.data_ptr(), None)
+        assert np.array_equal(host(out), np.broadcast_to(x, dst)), (name, src, dst)
+    with pytest.raises(api.OdlInvalidArgument):
+        L.call("odl_hip_broadcast_to_dtype", code, dx.data_ptr(), shape_arr((3,)), 1, shape_arr((4,)), 1, out.data_ptr(), None)
+    # ---- sum_to (left-aligned): reduced where the target has a 1, trailing source dimensions summed away
+    for src, dst, axes in (((4, 5), (1, 5), (0,)), ((4, 5), (4, 1), (1,)), ((3, 4, 5), (3,), (1, 2)), ((2, 3, 4), (1, 3, 1), (0, 2)),
+                           ((6, 7), (6, 7), ())):
+        x = _typed_values(rng, t, int(np.prod(src))).reshape(src)
+        nb = L.query("odl_hip_sum_to_dtype_workspace_bytes", code, shape_arr(src), len(src), shape_arr(dst), len(dst))
+        ws = torch.empty(max(nb, 4), dtype=torch.uint8, device="cuda")
+        out = torch.empty(dst, dtype=tt, device="cuda")
+        dx = dev(x)
+        L.call("odl_hip_sum_to_dtype", code, dx.data_ptr(), shape_arr(src), len(src), shape_arr(dst), len(dst), out.data_ptr(),
+               ws.data_ptr(), nb, None)
+        with np.errstate(over="ignore"):
+            want = x.sum(axis=axes, dtype=t).reshape(dst) if axes else x
+        if is_float:
+            terms = x.size // max(int(np.prod(dst)), 1)
+            bound = terms * np.finfo(t).eps * np.abs(x).sum(axis=axes).reshape(dst) if axes else 0
+            assert (np.abs(host(out) - want) <= bound).all(), (name, src, dst)
+        else:
+            assert np.array_equal(host(out), want), (name, src, dst)
+    with pytest.raises(api.OdlRuntimeError):  # a larger target (sum_to.cpp:24-28)
+        L.call("odl_hip_sum_to_dtype", code, dx.data_ptr(), shape_arr((2, 2)), 2, shape_arr((3, 3)), 2, out.data_ptr(), None, 0, None)
+    # ---- cat along each dimension, and split (one piece at a time) back
+    for shapes, dim in ((((2, 3, 5), (2, 4, 5), (2, 1, 5)), 1), (((3, 4), (2, 4)), 0), (((2, 3, 2), (2, 3, 7)), 2), (((5,), (3,), (9,)), 0)):
+        xs = [_typed_values(rng, t, int(np.prod(sh))).reshape(sh) for sh in shapes]
+        want = np.concatenate(xs, axis=dim)
+        outer = int(np.prod(want.shape[:dim])) if dim else 1
+        inner = int(np.prod(want.shape[dim + 1:])) if dim + 1 < want.ndim else 1
+        dxs = [dev(x) for x in xs]
+        ptrs = (ctypes.c_void_p * len(xs))(*[d.data_ptr() for d in dxs])
+        sizes = (ctypes.c_int64 * len(xs))(*[sh[dim] for sh in shapes])
+        out = torch.empty(want.shape, dtype=tt, device="cuda")
+        L.call("odl_hip_cat_dtype", code, ptrs, sizes, len(xs), outer, inner, out.data_ptr(), None)
+        assert np.array_equal(host(out), want), (name, shapes, dim)
+        off = 0
+        for x in xs:
+            piece = torch.empty(x.shape, dtype=tt, device="cuda")
+            L.call("odl_hip_slice_axis_dtype", code, out.data_ptr(), outer, want.shape[dim], inner, off, x.shape[dim],
+                   piece.data_ptr(), None)
+            assert np.array_equal(host(piece), x)
+            off += x.shape[dim]
 
 
 @pytest.mark.parametrize("name", ["f64", "i8", "i32", "i64", "u8"])
