@@ -805,7 +805,7 @@ std::unique_ptr<Mat> adaptive_avg_pool2d_backward(const OriginMat &, const Origi
 // ------------------------------------------------------------------------------------------- labels
 std::unique_ptr<Mat> gather(const OriginMat &input, const OriginMat &indices)
 {
-    const OriginMat &x = f32(input, "gather");
+    const OriginMat &x = on_device(input, "gather");
     const Shape xs = x.shape();
     if (xs.size() != 2)
         THROW_INVALID_ARG("gather: input must be 2D (N, C), but got shape {}", xs.to_string());
@@ -817,10 +817,11 @@ std::unique_ptr<Mat> gather(const OriginMat &input, const OriginMat &indices)
     if (indices.device() != x.device())
         THROW_INVALID_ARG("gather: input and indices must be on the same device");
     const int is64 = label_kind(indices, "gather");
-    auto out = fresh(x, Shape{xs[0]});
+    auto out = fresh(x, Shape{xs[0]}, x.dtype());
     // (the labels are checked on the device; a label outside [0, C) comes back as ODL_ERR_INVALID_ARG ->
     // std::invalid_argument, the throw tests/unit_test/operator/test_softmax_cross_entropy.cpp:227-234 expects)
-    check(odl_hip_gather(fp(x), vp(indices), is64, (int64_t)xs[0], (int64_t)xs[1], fp(*out), kStream));
+    check(odl_hip_gather_dtype(code(x.dtype()), vp(x), vp(indices), is64, (int64_t)xs[0], (int64_t)xs[1], out->storage()->data(),
+                               kStream));
     return out;
 }
 
@@ -947,29 +948,30 @@ std::vector<std::unique_ptr<Mat>> rms_norm_backward(const OriginMat &, const Ori
 // ------------------------------------------------------------------------------------------- detector forward path
 std::unique_ptr<Mat> upsample(const OriginMat &x_, const Shape &output_shape, int scale_h, int scale_w, const std::string &)
 {
-    const OriginMat &x = f32(x_, "upsample");
+    const OriginMat &x = on_device(x_, "upsample");
     const Shape xs = x.shape();
     if (xs.size() != 4)
         THROW_INVALID_ARG("Upsample: input must be 4D (N, C, H, W), but got shape {}", xs.to_string());
     if (output_shape.size() != 4)
         THROW_INVALID_ARG("Upsample: output_shape must be 4D (N, C, OH, OW), but got shape {}", output_shape.to_string());
-    auto y = fresh(x, output_shape);
-    check(odl_hip_upsample_nearest(fp(x), (int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3],
-                                   (int64_t)output_shape[2], (int64_t)output_shape[3], scale_h, scale_w, fp(*y), kStream));
+    auto y = fresh(x, output_shape, x.dtype());
+    check(odl_hip_upsample_nearest_dtype(code(x.dtype()), vp(x), (int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3],
+                                         (int64_t)output_shape[2], (int64_t)output_shape[3], scale_h, scale_w,
+                                         y->storage()->data(), kStream));
     return y;
 }
 
 std::unique_ptr<Mat> upsample_backward(const OriginMat &gy_, const Shape &xs, int scale_h, int scale_w, const std::string &)
 {
-    const OriginMat &gy = f32(gy_, "upsample_backward");
+    const OriginMat &gy = on_device(gy_, "upsample_backward");
     if (gy.shape().size() != 4)
         THROW_INVALID_ARG("Upsample backward: gradient must be 4D (N, C, OH, OW), but got shape {}", gy.shape().to_string());
     if (xs.size() != 4)
         THROW_INVALID_ARG("Upsample backward: x_shape must be 4D (N, C, H, W), but got shape {}", xs.to_string());
-    auto gx = fresh(gy, xs);
-    check(odl_hip_upsample_nearest_backward(fp(gy), (int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3],
-                                            (int64_t)gy.shape()[2], (int64_t)gy.shape()[3], scale_h, scale_w, fp(*gx),
-                                            kStream));
+    auto gx = fresh(gy, xs, gy.dtype());
+    check(odl_hip_upsample_nearest_backward_dtype(code(gy.dtype()), vp(gy), (int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2],
+                                                  (int64_t)xs[3], (int64_t)gy.shape()[2], (int64_t)gy.shape()[3], scale_h,
+                                                  scale_w, gx->storage()->data(), kStream));
     return gx;
 }
 

@@ -393,6 +393,16 @@ int odl_hip_cat_dtype(int dtype, const void *const *host_inputs, const int64_t *
                       int64_t inner, void *out, void *stream);
 int odl_hip_slice_axis_dtype(int dtype, const void *src, int64_t outer, int64_t axis_size, int64_t inner, int64_t offset,
                              int64_t length, void *dst, void *stream);
+/* Mat::gather, Mat::upsample and Mat::upsample_backward in any element type (src/mat/origin/cuda/nn/gather.cu:189 and
+ * upsample.cu:176, 224 dispatch over the type): the semantics of the float32 entry points; gather and the forward are
+ * copies, the backward adds in the element type (integers wrap). one_hot gives float32 whatever the labels' type
+ * (gather.cu:234). */
+int odl_hip_gather_dtype(int dtype, const void *in, const void *idx, int idx_is_i64, int64_t N, int64_t C, void *out,
+                         void *stream);
+int odl_hip_upsample_nearest_dtype(int dtype, const void *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
+                                   int scale_h, int scale_w, void *y, void *stream);
+int odl_hip_upsample_nearest_backward_dtype(int dtype, const void *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
+                                            int64_t OW, int scale_h, int scale_w, void *gx, void *stream);
 /* Mat::sum over [outer, axis, inner] in any type (operation_templates.h:270-357): integers sum with wrap-around in their
  * own width, float64 in a fixed parallel order. through_float != 0 passes each result through a float on its way back
  * into the element type, which is what the reference's whole-tensor sum does (src/mat/origin/cpu/math/sum.cpp:18-35,83-90). */

@@ -635,4 +635,109 @@ int odl_hip_slice_axis_dtype(int dtype, const void *src, int64_t outer, int64_t 
                            offset * inner, chunk, 0, odl::as_stream(stream));
 }
 
+// Mat::upsample / upsample_backward in the other element types (src/mat/origin/cuda/nn/upsample.cu:176, 224 dispatch over
+// the type): the forward is a copy and goes by element width; the backward adds the scale_h x scale_w block of gy that
+// an input pixel was copied to, rows then columns ascending, in the element type (integers wrap).
+}  // extern "C"
+
+namespace
+{
+template <typename U>
+__global__ __launch_bounds__(kBlock) void upsample_nearest_words_kernel(const U *__restrict__ x, U *__restrict__ y, int64_t total,
+                                                                        int64_t H, int64_t W, int64_t OH, int64_t OW, int sh, int sw)
+{
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= total)
+        return;
+    const int64_t ow = t % OW, oh = (t / OW) % OH, nc = t / (OW * OH);
+    y[t] = x[(nc * H + oh / sh) * W + ow / sw];
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void upsample_nearest_bwd_any_kernel(const T *__restrict__ gy, T *__restrict__ gx, int64_t total,
+                                                                          int64_t H, int64_t W, int64_t OH, int64_t OW, int sh, int sw)
+{
+    const int64_t t = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= total)
+        return;
+    const int64_t w = t % W, h = (t / W) % H, nc = t / (W * H);
+    T acc = (T)0;
+    for (int64_t oh = h * sh; oh < (h + 1) * sh && oh < OH; ++oh)
+        for (int64_t ow = w * sw; ow < (w + 1) * sw && ow < OW; ++ow)
+        {
+            const T v = gy[(nc * OH + oh) * OW + ow];
+            if (sizeof(T) < 4)
+                acc = (T)((unsigned)acc + (unsigned)v);  // 8-bit integers wrap like the wider ones
+            else
+                acc = acc + v;
+        }
+    gx[t] = acc;
+}
+}  // namespace
+
+extern "C" {
+
+int odl_hip_upsample_nearest_dtype(int dtype, const void *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH, int64_t OW,
+                                   int scale_h, int scale_w, void *y, void *stream)
+{
+    if (dtype == 0)
+        return odl_hip_upsample_nearest(static_cast<const float *>(x), N, C, H, W, OH, OW, scale_h, scale_w, static_cast<float *>(y),
+                                        stream);
+    ODL_REQUIRE_DEVICE();
+    const size_t esz = odl_hip_dtype_size(dtype);
+    ODL_REQUIRE(esz > 0, "upsample: unknown element type code %d", dtype);
+    ODL_REQUIRE(N >= 0 && C >= 0 && H > 0 && W > 0 && OH > 0 && OW > 0, "upsample: bad shape");
+    ODL_REQUIRE(scale_h > 0 && scale_w > 0, "upsample: scale must be positive");
+    ODL_REQUIRE((OH - 1) / scale_h < H && (OW - 1) / scale_w < W,
+                "upsample: output (%lld,%lld) reaches past input (%lld,%lld) at scale (%d,%d)", (long long)OH, (long long)OW,
+                (long long)H, (long long)W, scale_h, scale_w);
+    const int64_t total = N * C * OH * OW;
+    if (total == 0)
+        return ODL_OK;
+    const dim3 grid((unsigned)odl::ceil_div(total, kBlock)), block(kBlock);
+    hipStream_t st = odl::as_stream(stream);
+    if (esz == 8)
+        hipLaunchKernelGGL(upsample_nearest_words_kernel<uint64_t>, grid, block, 0, st, static_cast<const uint64_t *>(x),
+                           static_cast<uint64_t *>(y), total, H, W, OH, OW, scale_h, scale_w);
+    else if (esz == 4)
+        hipLaunchKernelGGL(upsample_nearest_words_kernel<uint32_t>, grid, block, 0, st, static_cast<const uint32_t *>(x),
+                           static_cast<uint32_t *>(y), total, H, W, OH, OW, scale_h, scale_w);
+    else
+        hipLaunchKernelGGL(upsample_nearest_words_kernel<uint8_t>, grid, block, 0, st, static_cast<const uint8_t *>(x),
+                           static_cast<uint8_t *>(y), total, H, W, OH, OW, scale_h, scale_w);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_upsample_nearest_backward_dtype(int dtype, const void *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
+                                            int64_t OW, int scale_h, int scale_w, void *gx, void *stream)
+{
+    if (dtype == 0)
+        return odl_hip_upsample_nearest_backward(static_cast<const float *>(gy), N, C, H, W, OH, OW, scale_h, scale_w,
+                                                 static_cast<float *>(gx), stream);
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C >= 0 && H > 0 && W > 0 && OH > 0 && OW > 0, "upsample_backward: bad shape");
+    ODL_REQUIRE(scale_h > 0 && scale_w > 0, "upsample_backward: scale must be positive");
+    const int64_t total = N * C * H * W;
+    if (total == 0)
+        return ODL_OK;
+    const dim3 grid((unsigned)odl::ceil_div(total, kBlock)), block(kBlock);
+    hipStream_t st = odl::as_stream(stream);
+#define ODL_UPS_BWD(T)                                                                                                        \
+    hipLaunchKernelGGL(upsample_nearest_bwd_any_kernel<T>, grid, block, 0, st, static_cast<const T *>(gy), static_cast<T *>(gx), \
+                       total, H, W, OH, OW, scale_h, scale_w)
+    switch (dtype)
+    {
+        case 1: ODL_UPS_BWD(double); break;
+        case 2: ODL_UPS_BWD(int8_t); break;
+        case 3: ODL_UPS_BWD(int32_t); break;
+        case 4: ODL_UPS_BWD(int64_t); break;
+        case 5: ODL_UPS_BWD(uint8_t); break;
+        default: return odl::fail(ODL_ERR_INVALID_ARG, "upsample_backward: unknown element type code %d", dtype);
+    }
+#undef ODL_UPS_BWD
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
 }  // extern "C"

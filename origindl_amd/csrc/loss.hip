@@ -154,6 +154,17 @@ __global__ void gather_kernel(const float *__restrict__ in, const void *idx, int
     out[i] = (t >= 0 && t < C) ? in[i * C + t] : 0.f;
 }
 
+// the same for elements of another size (a copy: the element type does not matter beyond its width)
+template <typename U>
+__global__ void gather_words_kernel(const U *__restrict__ in, const void *idx, int is64, int64_t N, int64_t C, U *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= N)
+        return;
+    const int64_t t = label_at(idx, is64, i);
+    out[i] = (t >= 0 && t < C) ? in[i * C + t] : (U)0;
+}
+
 __global__ void one_hot_kernel(const void *idx, int is64, int64_t N, int64_t C, float *__restrict__ out)
 {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -577,6 +588,8 @@ inline size_t align256(size_t b)
 }
 }  // namespace
 
+extern "C" size_t odl_hip_dtype_size(int dtype);
+
 extern "C" {
 
 int odl_hip_softmax(const float *x, int64_t outer, int64_t axis, int64_t inner, float *y, void *stream)
@@ -608,15 +621,10 @@ int odl_hip_softmax(const float *x, int64_t outer, int64_t axis, int64_t inner, 
     return ODL_OK;
 }
 
-int odl_hip_gather(const float *in, const void *idx, int idx_is_i64, int64_t N, int64_t C, float *out, void *stream)
+// the labels are validated on the host before the launch, so that an out-of-range label can be reported the way the
+// reference reports it (gather.cpp:64-67; the CUDA backend does the same D2H copy)
+static int gather_check_labels(const void *idx, int idx_is_i64, int64_t N, int64_t C, hipStream_t st)
 {
-    ODL_REQUIRE_DEVICE();
-    ODL_REQUIRE(N >= 0 && C >= 0, "gather: negative extent");
-    if (N == 0)
-        return ODL_OK;
-    hipStream_t st = odl::as_stream(stream);
-    // the labels are validated on the host before the launch, so that an out-of-range label can be reported
-    // the way the reference reports it (gather.cpp:64-67; the CUDA backend does the same D2H copy)
     const size_t esz = idx_is_i64 ? 8 : 4;
     std::vector<char> host((size_t)N * esz);
     ODL_HIP_CHECK(hipMemcpyAsync(host.data(), idx, host.size(), hipMemcpyDeviceToHost, st));
@@ -629,8 +637,49 @@ int odl_hip_gather(const float *in, const void *idx, int idx_is_i64, int64_t N, 
             return odl::fail(ODL_ERR_INVALID_ARG, "gather: index %lld out of range [0, %lld)", (long long)t,
                              (long long)C);
     }
+    return ODL_OK;
+}
+
+int odl_hip_gather(const float *in, const void *idx, int idx_is_i64, int64_t N, int64_t C, float *out, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C >= 0, "gather: negative extent");
+    if (N == 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    const int rc = gather_check_labels(idx, idx_is_i64, N, C, st);
+    if (rc != ODL_OK)
+        return rc;
     hipLaunchKernelGGL(gather_kernel, dim3((unsigned)odl::ceil_div(N, kBlock)), dim3(kBlock), 0, st, in, idx, idx_is_i64,
                        N, C, out);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_gather_dtype(int dtype, const void *in, const void *idx, int idx_is_i64, int64_t N, int64_t C, void *out, void *stream)
+{
+    if (dtype == 0)
+        return odl_hip_gather(static_cast<const float *>(in), idx, idx_is_i64, N, C, static_cast<float *>(out), stream);
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(N >= 0 && C >= 0, "gather: negative extent");
+    const size_t esz = odl_hip_dtype_size(dtype);
+    ODL_REQUIRE(esz > 0, "gather: unknown element type code %d", dtype);
+    if (N == 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    const int rc = gather_check_labels(idx, idx_is_i64, N, C, st);
+    if (rc != ODL_OK)
+        return rc;
+    const dim3 grid((unsigned)odl::ceil_div(N, kBlock)), block(kBlock);
+    if (esz == 8)
+        hipLaunchKernelGGL(gather_words_kernel<uint64_t>, grid, block, 0, st, static_cast<const uint64_t *>(in), idx, idx_is_i64, N,
+                           C, static_cast<uint64_t *>(out));
+    else if (esz == 4)
+        hipLaunchKernelGGL(gather_words_kernel<uint32_t>, grid, block, 0, st, static_cast<const uint32_t *>(in), idx, idx_is_i64, N,
+                           C, static_cast<uint32_t *>(out));
+    else
+        hipLaunchKernelGGL(gather_words_kernel<uint8_t>, grid, block, 0, st, static_cast<const uint8_t *>(in), idx, idx_is_i64, N, C,
+                           static_cast<uint8_t *>(out));
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

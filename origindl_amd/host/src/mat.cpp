@@ -937,15 +937,15 @@ std::unique_ptr<Mat> OriginMat::silu_backward(const Mat &x) const
 std::unique_ptr<Mat> OriginMat::upsample_backward(const Mat &gym, const Shape &xs, int scale_h, int scale_w,
                                                   const std::string &) const
 {
-    const OriginMat &gy = dev_f32(gym, "upsample_backward");
+    const OriginMat &gy = dev_any(gym, "upsample_backward");
     if (gy.shape().size() != 4)
         THROW_INVALID_ARG("Upsample backward: gradient must be 4D (N, C, OH, OW), but got shape {}", gy.shape().to_string());
     if (xs.size() != 4)
         THROW_INVALID_ARG("Upsample backward: x_shape must be 4D (N, C, H, W), but got shape {}", xs.to_string());
-    auto gx = new_like(gy, xs);
-    check(odl_hip_upsample_nearest_backward(fp(gy), (int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3],
-                                            (int64_t)gy.shape()[2], (int64_t)gy.shape()[3], scale_h, scale_w,
-                                            gx->data_ptr<float>(), cur()));
+    auto gx = new_like(gy, xs, gy.dtype());
+    check(odl_hip_upsample_nearest_backward_dtype(code(gy.dtype()), gy.storage()->data(), (int64_t)xs[0], (int64_t)xs[1],
+                                                  (int64_t)xs[2], (int64_t)xs[3], (int64_t)gy.shape()[2], (int64_t)gy.shape()[3],
+                                                  scale_h, scale_w, gx->storage()->data(), cur()));
     return gx;
 }
 
@@ -1250,15 +1250,15 @@ std::vector<std::unique_ptr<Mat>> OriginMat::split(const std::vector<size_t> &si
 // ------------------------------------------------------------------------------------ detector forward path
 std::unique_ptr<Mat> OriginMat::upsample(const Shape &output_shape, int scale_h, int scale_w, const std::string &) const
 {
-    const OriginMat &x = dev_f32(*this, "upsample");
+    const OriginMat &x = dev_any(*this, "upsample");
     if (shape_.size() != 4)
         THROW_INVALID_ARG("Upsample: input must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
     if (output_shape.size() != 4)
         THROW_INVALID_ARG("Upsample: output_shape must be 4D (N, C, OH, OW), but got shape {}", output_shape.to_string());
-    auto y = new_like(x, output_shape);
-    check(odl_hip_upsample_nearest(fp(x), (int64_t)shape_[0], (int64_t)shape_[1], (int64_t)shape_[2], (int64_t)shape_[3],
-                                   (int64_t)output_shape[2], (int64_t)output_shape[3], scale_h, scale_w,
-                                   y->data_ptr<float>(), cur()));
+    auto y = new_like(x, output_shape, x.dtype());
+    check(odl_hip_upsample_nearest_dtype(code(x.dtype()), x.storage()->data(), (int64_t)shape_[0], (int64_t)shape_[1],
+                                         (int64_t)shape_[2], (int64_t)shape_[3], (int64_t)output_shape[2], (int64_t)output_shape[3],
+                                         scale_h, scale_w, y->storage()->data(), cur()));
     return y;
 }
 
@@ -1904,7 +1904,7 @@ std::unique_ptr<Mat> OriginMat::max_pool2d_backward(const Mat &gym, std::pair<in
 // -------------------------------------------------------------------------------------------- indexing
 std::unique_ptr<Mat> OriginMat::gather(const Mat &indices) const
 {
-    const OriginMat &x   = dev_f32(*this, "gather");
+    const OriginMat &x   = dev_any(*this, "gather");
     const OriginMat &idx = as_origin(indices);
     if (shape_.size() != 2)
         THROW_INVALID_ARG("gather: input must be 2D (N, C), but got shape {}", shape_.to_string());
@@ -1916,9 +1916,9 @@ std::unique_ptr<Mat> OriginMat::gather(const Mat &indices) const
     if (idx.device() != device())
         THROW_INVALID_ARG("gather: input and indices must be on the same device");
     const int is64 = label_kind(idx, "gather");
-    auto out = new_like(x, Shape{shape_[0]});
-    check(odl_hip_gather(fp(x), idx.storage()->data(), is64, (int64_t)shape_[0], (int64_t)shape_[1],
-                         out->data_ptr<float>(), cur()));
+    auto out = new_like(x, Shape{shape_[0]}, x.dtype());
+    check(odl_hip_gather_dtype(code(x.dtype()), x.storage()->data(), idx.storage()->data(), is64, (int64_t)shape_[0],
+                               (int64_t)shape_[1], out->storage()->data(), cur()));
     return out;
 }
 

@@ -1578,6 +1578,45 @@ def test_max_broadcast_sum_to_cat_split_in_every_element_type(api, name):
             off += x.shape[dim]
 
 
+@pytest.mark.parametrize("name", ["f32", "f64", "i8", "i32", "i64", "u8"])
+def test_gather_and_upsample_in_every_element_type(api, name):
+    """Mat::gather, upsample and upsample_backward dispatch over the element type in the reference
+    (src/mat/origin/cuda/nn/gather.cu:189, upsample.cu:176, 224): copies bit for bit; the backward sums in the type."""
+    L = api.lib()
+    code, t = DT[name]
+    tt = getattr(torch, np.dtype(t).name)
+    rng = np.random.default_rng(91 + code)
+    N, C = 37, 11
+    x = _typed_values(rng, t, N * C).reshape(N, C)
+    for is64, it in ((0, np.int32), (1, np.int64)):
+        idx = rng.integers(0, C, N).astype(it)
+        out = torch.empty(N, dtype=tt, device="cuda")
+        dx, di = dev(x), dev(idx)
+        L.call("odl_hip_gather_dtype", code, dx.data_ptr(), di.data_ptr(), is64, N, C, out.data_ptr(), None)
+        assert np.array_equal(host(out), x[np.arange(N), idx])
+        bad = idx.copy()
+        bad[5] = C
+        dbad = dev(bad)
+        with pytest.raises(api.OdlInvalidArgument):
+            L.call("odl_hip_gather_dtype", code, dx.data_ptr(), dbad.data_ptr(), is64, N, C, out.data_ptr(), None)
+    for (n, c, h, w, sh, sw) in ((2, 3, 4, 5, 2, 2), (1, 2, 3, 3, 3, 1), (2, 1, 5, 4, 1, 2)):
+        img = _typed_values(rng, t, n * c * h * w).reshape(n, c, h, w)
+        up = torch.empty((n, c, h * sh, w * sw), dtype=tt, device="cuda")
+        dimg = dev(img)
+        L.call("odl_hip_upsample_nearest_dtype", code, dimg.data_ptr(), n, c, h, w, h * sh, w * sw, sh, sw, up.data_ptr(), None)
+        assert np.array_equal(host(up), img.repeat(sh, axis=2).repeat(sw, axis=3))
+        gy = _typed_values(rng, t, n * c * h * sh * w * sw).reshape(n, c, h * sh, w * sw)
+        gx = torch.empty((n, c, h, w), dtype=tt, device="cuda")
+        dgy = dev(gy)
+        L.call("odl_hip_upsample_nearest_backward_dtype", code, dgy.data_ptr(), n, c, h, w, h * sh, w * sw, sh, sw, gx.data_ptr(), None)
+        with np.errstate(over="ignore"):
+            want = gy.reshape(n, c, h, sh, w, sw).sum(axis=(3, 5), dtype=t)
+        if t in (np.float32, np.float64):
+            np.testing.assert_allclose(host(gx), want, rtol=8 * np.finfo(t).eps, atol=8 * np.finfo(t).eps * np.abs(gy).max() * sh * sw)
+        else:
+            assert np.array_equal(host(gx), want)
+
+
 @pytest.mark.parametrize("name", ["f64", "i8", "i32", "i64", "u8"])
 def test_elementwise_fill_and_sum_in_every_element_type(api, name):
     L = api.lib()
