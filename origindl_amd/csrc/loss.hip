@@ -482,27 +482,29 @@ __global__ void argmax_rows_kernel(const float *__restrict__ y, int64_t N, int64
 template <bool VEC>
 __device__ inline int64_t wave_first_argmax(const float *p, int64_t C, int lane)
 {
+    // (the row's first element decides the NaN case below: its load goes out with the others, not behind the reduction)
+    const float first = p[0];
     float mv = 0.f;
-    int64_t mi = 0;
+    unsigned mi = 0;  // a row has fewer than 2^32 classes: 32-bit positions halve the cross-lane traffic of the reduction
     bool has = false;
     if (VEC)
     {
         // 16 bytes per lane and load, four loads in flight; a lane still meets its elements in ascending order
         const f32x4 *pv = reinterpret_cast<const f32x4 *>(p);
-        const int64_t cq = C / 4;
-        for (int64_t q0 = lane; q0 < cq; q0 += 256)
+        const unsigned cq = (unsigned)(C / 4);
+        for (unsigned q0 = (unsigned)lane; q0 < cq; q0 += 256)
         {
             f32x4 v[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (unsigned u = 0; u < 4; ++u)
                 if (q0 + 64 * u < cq)
                     v[u] = pv[q0 + 64 * u];
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (unsigned u = 0; u < 4; ++u)
                 if (q0 + 64 * u < cq)
                 {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
+                    for (unsigned e = 0; e < 4; ++e)
                         if (v[u][e] == v[u][e] && (!has || v[u][e] > mv))
                             mv = v[u][e], mi = 4 * (q0 + 64 * u) + e, has = true;
                 }
@@ -510,7 +512,7 @@ __device__ inline int64_t wave_first_argmax(const float *p, int64_t C, int lane)
     }
     else
     {
-        for (int64_t j = lane; j < C; j += 64)
+        for (unsigned j = (unsigned)lane; j < (unsigned)C; j += 64)
         {
             const float v = p[j];
             if (v == v && (!has || v > mv))
@@ -521,13 +523,12 @@ __device__ inline int64_t wave_first_argmax(const float *p, int64_t C, int lane)
     for (int o = 32; o > 0; o >>= 1)
     {
         const float ov = __shfl_xor(mv, o, 64);
-        const int64_t oi = __shfl_xor(mi, o, 64);
+        const unsigned oi = (unsigned)__shfl_xor((int)mi, o, 64);
         const int oh = __shfl_xor((int)has, o, 64);
         if (oh && (!has || ov > mv || (ov == mv && oi < mi)))
             mv = ov, mi = oi, has = true;
     }
-    const float first = p[0];
-    return (has && first == first) ? mi : 0;
+    return (has && first == first) ? (int64_t)mi : 0;
 }
 
 template <bool VEC>
@@ -833,11 +834,11 @@ int odl_hip_argmax_rows(const float *y, int64_t N, int64_t C, int64_t *out, void
     ODL_REQUIRE(N >= 0 && C > 0, "argmax: bad shape");
     if (N == 0)
         return ODL_OK;
-    const bool vec = C % 4 == 0 && C >= 256 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    const bool vec = C % 4 == 0 && C >= 256 && C < (1ll << 31) && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     if (vec)
         hipLaunchKernelGGL(argmax_rows_wave_kernel<true>, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0,
                            odl::as_stream(stream), y, N, C, out);
-    else if (C >= 32)  // a wave per row once a row is worth 64 lanes; a thread per row for a handful of classes
+    else if (C >= 32 && C < (1ll << 31))  // a wave per row once a row is worth 64 lanes; a thread per row for a handful of classes
         hipLaunchKernelGGL(argmax_rows_wave_kernel<false>, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0,
                            odl::as_stream(stream), y, N, C, out);
     else
@@ -863,10 +864,10 @@ int odl_hip_accuracy(const float *y, const int32_t *t, int64_t N, int64_t C, flo
     unsigned int *count = static_cast<unsigned int *>(workspace);
     hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, count, 1);
     ODL_LAUNCH_CHECK();
-    if (C % 4 == 0 && C >= 256 && (reinterpret_cast<uintptr_t>(y) & 15) == 0)
+    if (C % 4 == 0 && C >= 256 && C < (1ll << 31) && (reinterpret_cast<uintptr_t>(y) & 15) == 0)
         hipLaunchKernelGGL(accuracy_count_wave_kernel<true>, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, st, y,
                            t, N, C, count);
-    else if (C >= 32)
+    else if (C >= 32 && C < (1ll << 31))
         hipLaunchKernelGGL(accuracy_count_wave_kernel<false>, dim3((unsigned)odl::ceil_div(N, kWaves)), dim3(kBlock), 0, st, y,
                            t, N, C, count);
     else
