@@ -75,6 +75,19 @@ size_t conv_small_dgrad_workspace(int64_t C, int64_t OC, int KH, int KW);
 int conv_small_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
                      int KH, int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW, void *workspace,
                      size_t workspace_bytes, hipStream_t st);
+// conv_stem.hip: the whole backward pass of a one-channel 3x3 / stride 1 / padding 1 layer in one pass over gy
+bool conv_stem_backward_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW,
+                           int PH, int PW);
+size_t conv_stem_backward_workspace(int64_t N, int64_t OC);
+int conv_stem_backward(const float *gy, const float *x, const float *w, float *gx, float *gw, float *gb, int64_t N, int64_t H,
+                       int64_t W, int64_t OC, void *workspace, size_t workspace_bytes, hipStream_t st);
+// conv_image.hip: 3x3 / stride 1 / padding 1 over small images with few channels, an image at a time resident in LDS;
+// the weight and the bias gradient in one pass
+bool conv_image_wgrad_ok(const float *gy, const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW,
+                         int SH, int SW, int PH, int PW);
+size_t conv_image_wgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC);
+int conv_image_wgrad(const float *gy, const float *x, float *gw, float *gb, int64_t N, int64_t C, int64_t H, int64_t W,
+                     int64_t OC, void *workspace, size_t workspace_bytes, hipStream_t st);
 // conv_wgrad.hip: 3x3 / padding 1 / stride 1 or 2, walking the output rows with the input rows staged in LDS
 bool conv_wgrad_rows_ok(const float *gy, const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH,
                         int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW);
@@ -1391,8 +1404,10 @@ __global__ __launch_bounds__(1024) void conv_backward_side_kernel(const SideJobs
 // workspace regions of conv2d_backward, in order: [col][split-K partials][permuted weights][bias partials]
 struct BwdPlan
 {
+    bool stem;                      // one input channel, 3x3/s1/p1: all three gradients in one pass over gy
     bool wgrad_small, dgrad_small;  // few input channels: the direct kernels, no matrices at all
     bool wgrad_rows;                // 3x3/p1 at stride 1 or 2: output rows walked with the input rows in LDS
+    bool wgrad_image;               // 3x3/s1/p1 over small images with few channels: an image at a time resident in LDS
     bool dgrad_patch;               // 3x3/s1/p1: the gradient patch stays in LDS
     bool wgrad_implicit, dgrad_implicit;
     size_t col_bytes, splitk_bytes, wp_bytes, red_bytes;
@@ -1404,18 +1419,26 @@ BwdPlan plan_backward(const float *gy, const float *x, int64_t N, int64_t C, int
 {
     BwdPlan p{};
     const int64_t M = N * OH * OW, K = C * KH * KW;
+    if (odl::conv_stem_backward_ok(gy, N, C, H, W, OC, KH, KW, SH, SW, PH, PW))
+    {
+        p.stem = true;
+        p.splitk_bytes = align256(odl::conv_stem_backward_workspace(N, OC));
+        return p;
+    }
     p.wgrad_small = odl::conv_small_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
     p.dgrad_small = odl::conv_small_dgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
     // 3x3 at stride 1 keeps the image size only with a padding of 1
     const int pad = (OH == H && OW == W) ? 1 : -1;
     p.wgrad_rows = !p.wgrad_small && odl::conv_wgrad_rows_ok(gy, x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW);
-    p.wgrad_implicit = !p.wgrad_small && !p.wgrad_rows && odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
+    p.wgrad_image = !p.wgrad_small && !p.wgrad_rows && odl::conv_image_wgrad_ok(gy, x, N, C, H, W, OC, KH, KW, SH, SW, PH, PW);
+    p.wgrad_implicit = !p.wgrad_small && !p.wgrad_rows && !p.wgrad_image && odl::conv_implicit_wgrad_ok(gy, N, C, H, W, OC, KH, KW, OH, OW);
     p.dgrad_patch = !p.dgrad_small && odl::conv_patch_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW, pad, pad);
     p.dgrad_implicit = !p.dgrad_small && !p.dgrad_patch && odl::conv_implicit_dgrad_ok(gy, N, C, H, W, OC, KH, KW, SH, SW);
-    const bool no_col = (p.wgrad_small || p.wgrad_rows || p.wgrad_implicit) && (p.dgrad_small || p.dgrad_patch || p.dgrad_implicit);
+    const bool no_col = (p.wgrad_small || p.wgrad_rows || p.wgrad_image || p.wgrad_implicit) && (p.dgrad_small || p.dgrad_patch || p.dgrad_implicit);
     p.col_bytes = no_col ? 0 : align256((size_t)(M * K) * sizeof(float));
     p.splitk_bytes = align256(p.wgrad_small      ? odl::conv_small_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
                               : p.wgrad_rows     ? odl::conv_wgrad_rows_workspace(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, OH, OW)
+                              : p.wgrad_image    ? odl::conv_image_wgrad_workspace(N, C, H, W, OC)
                               : p.wgrad_implicit ? odl::conv_implicit_wgrad_workspace(N, C, OC, KH, KW, OH, OW)
                                                  : odl::sgemm_workspace(OC, K, M, 0));
     p.wp_bytes = p.dgrad_small      ? align256(odl::conv_small_dgrad_workspace(C, OC, KH, KW))
@@ -1462,6 +1485,8 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
     void *wp_ws = ws + p.col_bytes + p.splitk_bytes;
     void *red_ws = ws + p.col_bytes + p.splitk_bytes + p.wp_bytes;
 
+    if (p.stem)
+        return odl::conv_stem_backward(gy, x, w, gx, gw, gb, N, H, W, OC, splitk_ws, p.splitk_bytes, st);
     // gy2d: gy's NCHW buffer read as a row-major [M, OC] matrix exactly as it lies (conv2d.cpp:548)
     // With the row-walking weight gradient, the jobs that follow it — the sum of its partial tiles, the bias gradient,
     // the filter copy of the LDS-patch input gradient — run side by side in one launch.
@@ -1494,6 +1519,8 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
         if (p.wgrad_small)
             rc = odl::conv_small_wgrad(gy, x, gw, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, splitk_ws,
                                        p.splitk_bytes, st);
+        else if (p.wgrad_image)  // (with the bias gradient, if asked for)
+            rc = odl::conv_image_wgrad(gy, x, gw, gb, N, C, H, W, OC, splitk_ws, p.splitk_bytes, st);
         else if (p.wgrad_implicit)
             rc = odl::conv_implicit_wgrad(gy, x, gw, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, splitk_ws,
                                           p.splitk_bytes, st);
@@ -1507,7 +1534,7 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
         if (rc != ODL_OK)
             return rc;
     }
-    if (gb && !side_bias)
+    if (gb && !side_bias && !(gw && p.wgrad_image))
     {
         rc = odl::sum_nchw_channels_launch(gy, N, OC, g.OH * g.OW, gb, red_ws, p.red_bytes, st);
         if (rc != ODL_OK)

@@ -463,6 +463,13 @@ CONV_SEEDED = [
     (7, 16, 5, 6, 64, 3, 3, 1, 1),     # tiles that start and end in the middle of an image; 64 gradient channels
     (3, 16, 8, 8, 24, 3, 3, 1, 1),     # W a multiple of 4: the LDS patch is staged with 16-byte row loads
     (2, 48, 6, 28, 40, 3, 3, 1, 1),    # the same over three channel slabs and rows shared between tiles
+    (3, 1, 12, 10, 16, 3, 3, 1, 1),    # one channel, 3x3/s1/p1: the one-pass backward, 16 filters, W != H
+    (2, 1, 5, 7, 8, 3, 3, 1, 1),       # the same with 8 filters
+    (1, 1, 1, 1, 32, 3, 3, 1, 1),      # a single pixel: only the centre tap meets it
+    (700, 1, 6, 6, 32, 3, 3, 1, 1),    # more images than workgroups: several images a workgroup
+    (130, 32, 14, 14, 64, 3, 3, 1, 1), # small images, few channels: the weight gradient with an image at a time in LDS
+    (300, 16, 8, 6, 64, 3, 3, 1, 1),   # the same with more images than workgroups and W != H
+    (128, 10, 6, 10, 96, 3, 3, 1, 1),  # the same with 90 gW columns: the last MFMA tile ragged, three row blocks
     (3, 16, 8, 8, 40, 3, 3, 2, 1),     # stride 2 with channels in sixteens: several images per pixel tile, ragged filter tile
     (5, 32, 6, 28, 96, 3, 3, 2, 1),    # the same with 14-pixel output rows and two filter tiles
     (2, 48, 12, 52, 64, 3, 3, 2, 1),   # wide rows at stride 2
