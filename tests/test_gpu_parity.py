@@ -470,6 +470,8 @@ CONV_SEEDED = [
     (130, 32, 14, 14, 64, 3, 3, 1, 1), # small images, few channels: the weight gradient with an image at a time in LDS
     (300, 16, 8, 6, 64, 3, 3, 1, 1),   # the same with more images than workgroups and W != H
     (128, 10, 6, 10, 96, 3, 3, 1, 1),  # the same with 90 gW columns: the last MFMA tile ragged, three row blocks
+    (128, 12, 10, 10, 48, 3, 3, 1, 1), # image-resident forward: three filter tiles, the 27 steps of k in four uneven parts
+    (140, 16, 12, 16, 32, 3, 3, 1, 1), # image-resident forward and input gradient with twelve full pixel tiles
     (3, 16, 8, 8, 40, 3, 3, 2, 1),     # stride 2 with channels in sixteens: several images per pixel tile, ragged filter tile
     (5, 32, 6, 28, 96, 3, 3, 2, 1),    # the same with 14-pixel output rows and two filter tiles
     (2, 48, 12, 52, 64, 3, 3, 2, 1),   # wide rows at stride 2
