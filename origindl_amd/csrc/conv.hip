@@ -87,7 +87,7 @@ bool conv_image_wgrad_ok(const float *gy, const float *x, int64_t N, int64_t C, 
                          int SH, int SW, int PH, int PW);
 size_t conv_image_wgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC);
 int conv_image_wgrad(const float *gy, const float *x, float *gw, float *gb, int64_t N, int64_t C, int64_t H, int64_t W,
-                     int64_t OC, void *workspace, size_t workspace_bytes, hipStream_t st);
+                     int64_t OC, void *workspace, size_t workspace_bytes, hipStream_t st, const SidePack *pack, unsigned n_pack);
 // conv_wgrad.hip: 3x3 / padding 1 / stride 1 or 2, walking the output rows with the input rows staged in LDS
 bool conv_wgrad_rows_ok(const float *gy, const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH,
                         int KW, int SH, int SW, int PH, int PW, int64_t OH, int64_t OW);
@@ -1494,6 +1494,7 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
     const bool side = gw && p.wgrad_rows;
     const bool side_bias = side && gb && P % 4 == 0 && N * P < (1ll << 31) && OC <= 4096 && reinterpret_cast<uintptr_t>(gy) % 16 == 0;
     const bool side_pack = side && gx && p.dgrad_patch;
+    const bool image_pack = gw && !side && p.wgrad_image && !p.wgrad_small && gx && !p.dgrad_small && p.dgrad_patch;
     if (side)
     {
         SideJobs j{};
@@ -1519,8 +1520,15 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
         if (p.wgrad_small)
             rc = odl::conv_small_wgrad(gy, x, gw, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, splitk_ws,
                                        p.splitk_bytes, st);
-        else if (p.wgrad_image)  // (with the bias gradient, if asked for)
-            rc = odl::conv_image_wgrad(gy, x, gw, gb, N, C, H, W, OC, splitk_ws, p.splitk_bytes, st);
+        else if (p.wgrad_image)  // (with the bias gradient, if asked for, and the input gradient's filter copy)
+        {
+            odl::SidePack pack{};
+            if (image_pack)
+                pack = odl::conv_patch_dgrad_pack(w, C, OC, wp_ws);
+            const unsigned n_pack = (unsigned)std::min<int64_t>(odl::ceil_div((int64_t)pack.Cin * 9 * pack.Mpad, 1024), 128);
+            rc = odl::conv_image_wgrad(gy, x, gw, gb, N, C, H, W, OC, splitk_ws, p.splitk_bytes, st, image_pack ? &pack : nullptr,
+                                       n_pack);
+        }
         else if (p.wgrad_implicit)
             rc = odl::conv_implicit_wgrad(gy, x, gw, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, splitk_ws,
                                           p.splitk_bytes, st);
@@ -1545,7 +1553,7 @@ int odl_hip_conv2d_backward(const float *gy, const float *x, const float *w, int
         if (p.dgrad_small)
             rc = odl::conv_small_dgrad(gy, w, gx, N, C, H, W, OC, KH, KW, SH, SW, PH, PW, g.OH, g.OW, wp_ws, p.wp_bytes, st);
         else if (p.dgrad_patch)
-            rc = odl::conv_patch_dgrad(gy, w, gx, N, C, H, W, OC, wp_ws, p.wp_bytes, st, side_pack);
+            rc = odl::conv_patch_dgrad(gy, w, gx, N, C, H, W, OC, wp_ws, p.wp_bytes, st, side_pack || image_pack);
         else if (p.dgrad_implicit)
             rc = odl::conv_implicit_dgrad(gy, w, gx, N, C, H, W, OC, KH, KW, PH, PW, g.OH, g.OW, wp_ws, p.wp_bytes, st);
         else

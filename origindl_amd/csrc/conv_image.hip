@@ -12,6 +12,7 @@
 // by three MFMA tiles) and keeps it in registers across the workgroup's images; each workgroup writes one partial gW, and
 // a second launch adds the partials in workgroup order. The bias gradient (the NCHW reading of the same block,
 // conv2d.cpp:566-580) is summed from the pieces as they are staged and travels in the same partials.
+#include "conv_side.h"
 #include "odl_common.h"
 
 #include <map>
@@ -264,12 +265,19 @@ __global__ __launch_bounds__(kIT) void conv_image_wgrad_kernel(const ImageGeom g
 
 // gw, gb = sum over the workgroups' partials in workgroup order: sixteen 16-byte columns per workgroup, 64 threads a
 // column that each add every 64th partial from their own on; their sums are added four and then sixteen at a time in
-// thread order — the same order on every run.
+// thread order — the same order on every run. Workgroups past the fold's (n_fold of them) make the filter copy that the
+// LDS-patch input gradient stages from (conv_side.h), one launch less when that kernel follows.
 __global__ __launch_bounds__(1024) void conv_image_fold_kernel(const float *__restrict__ part, int nparts, int E4, int W4,
-                                                                float *gw, float *gb)
+                                                                float *gw, float *gb, unsigned n_fold, odl::SidePack pack,
+                                                                unsigned n_pack)
 {
     __shared__ f32x4 sums[64][16];
     __shared__ f32x4 sums2[16][16];
+    if (blockIdx.x >= n_fold)
+    {
+        odl::side_pack(pack, blockIdx.x - n_fold, n_pack);
+        return;
+    }
     const int t = threadIdx.x, col = t & 15, sub = t >> 4;
     const int i = blockIdx.x * 16 + col;
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
@@ -404,9 +412,10 @@ size_t conv_image_wgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, in
     return p.ok ? (size_t)p.nwg * (size_t)(OC * C * 9 + OC) * sizeof(float) : 0;
 }
 
-// gw and gb may each be null (the partials are computed either way)
+// gw and gb may each be null (the partials are computed either way). pack: a filter copy for the input gradient to be made
+// by n_pack more workgroups of the second launch, or null.
 int conv_image_wgrad(const float *gy, const float *x, float *gw, float *gb, int64_t N, int64_t C, int64_t H, int64_t W,
-                     int64_t OC, void *workspace, size_t workspace_bytes, hipStream_t st)
+                     int64_t OC, void *workspace, size_t workspace_bytes, hipStream_t st, const SidePack *pack, unsigned n_pack)
 {
     const ImagePlan p = plan_image(N, C, H, W, OC);
     if (!p.ok)
@@ -425,11 +434,14 @@ int conv_image_wgrad(const float *gy, const float *x, float *gw, float *gb, int6
     ODL_HIP_CHECK(allow_lds());
     hipLaunchKernelGGL(conv_image_wgrad_kernel, dim3(p.nwg), dim3(kIT), p.lds, st, g);
     ODL_LAUNCH_CHECK();
-    if (gw || gb)
+    if (gw || gb || pack)
     {
         const int E4 = g.E / 4;
-        hipLaunchKernelGGL(conv_image_fold_kernel, dim3((unsigned)ceil_div(E4, 16)), dim3(1024), 0, st, g.part, p.nwg, E4,
-                           (int)(OC * C * 9 / 4), gw, gb);
+        const unsigned n_fold = (gw || gb) ? (unsigned)ceil_div(E4, 16) : 0u;
+        if (!pack)
+            n_pack = 0;
+        hipLaunchKernelGGL(conv_image_fold_kernel, dim3(n_fold + n_pack), dim3(1024), 0, st, g.part, p.nwg, E4,
+                           (int)(OC * C * 9 / 4), gw, gb, n_fold, pack ? *pack : SidePack{}, n_pack);
         ODL_LAUNCH_CHECK();
     }
     return ODL_OK;
