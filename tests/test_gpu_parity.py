@@ -542,6 +542,52 @@ def check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p):
     assert (np.abs(host(gb) - gbo) <= gb_bound + 1e-6).all()
 
 
+@pytest.mark.parametrize("N,C,H,W,OC", [
+    (5, 1, 12, 10, 16),      # one input channel: the one-pass backward
+    (130, 32, 14, 14, 64),   # small images, few channels: the image-resident weight gradient
+    (3, 64, 8, 8, 64),       # the row-walking weight gradient with its side launch
+    (2, 16, 12, 10, 32),     # the implicit products
+])
+def test_conv_backward_with_gradients_left_out(api, N, C, H, W, OC):
+    # conv2d_backward writes only the gradients whose pointers are given (an operator whose input needs no gradient
+    # passes none for gx; a layer without bias none for gb): every subset must give the values of the full call.
+    # The kernels that compute several gradients in one pass skip the missing ones; the bias gradient alone takes
+    # another kernel than beside the weight gradient, so it is compared to a few ulp of its sum.
+    from origindl_amd import _lib
+    rng = np.random.default_rng(N + C + OC)
+    x, gy = rng.standard_normal((N, C, H, W), dtype=f32), rng.standard_normal((N, OC, H, W), dtype=f32)
+    w = (rng.standard_normal((OC, C, 3, 3), dtype=f32) * f32(0.2)).astype(f32)
+    dx, dgy, dw = dev(x), dev(gy), dev(w)
+    L = _lib.lib()
+    nb = L.query("odl_hip_conv2d_backward_workspace_bytes", N, C, H, W, OC, 3, 3, 1, 1, 1, 1)
+    ws = torch.empty(max(nb, 16) // 4 + 4, dtype=torch.float32, device="cuda")
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def run(want_gx, want_gw, want_gb):
+        outs = [torch.full(shape, float("nan"), dtype=torch.float32, device="cuda") if want else None
+                for shape, want in ((x.shape, want_gx), (w.shape, want_gw), ((OC,), want_gb))]
+        ptr = [ctypes.c_void_p(t.data_ptr()) if t is not None else None for t in outs]
+        print("[case] conv backward subset", N, C, H, W, OC, want_gx, want_gw, want_gb, flush=True)
+        L.call("odl_hip_conv2d_backward", ctypes.c_void_p(dgy.data_ptr()), ctypes.c_void_p(dx.data_ptr()),
+               ctypes.c_void_p(dw.data_ptr()), N, C, H, W, OC, 3, 3, 1, 1, 1, 1, ptr[0], ptr[1], ptr[2],
+               ctypes.c_void_p(ws.data_ptr()), nb, st)
+        return [host(t) if t is not None else None for t in outs]
+
+    full = run(True, True, True)
+    assert all(np.isfinite(t).all() for t in full)
+    gb_tol = 1e-5 * np.sqrt(N * H * W) * np.linalg.norm(gy.transpose(1, 0, 2, 3).reshape(OC, -1).astype(np.float64), axis=1)
+    for subset in ((True, False, False), (False, True, False), (False, False, True), (True, True, False),
+                   (False, True, True), (True, False, True)):
+        got = run(*subset)
+        for name, g, f in zip(("gx", "gW", "gb"), got, full):
+            if g is None:
+                continue
+            if name == "gb":
+                assert (np.abs(g - f) <= gb_tol + 1e-6).all(), (subset, name)
+            else:
+                np.testing.assert_array_equal(g, f, err_msg="%s %s" % (subset, name))
+
+
 @pytest.mark.parametrize("N,C,H,OC,s,p", [
     (32, 64, 56, 128, 1, 1),    # benchmark configuration C1
     (32, 128, 28, 256, 2, 1),   # benchmark configuration C2
