@@ -217,28 +217,36 @@ __global__ __launch_bounds__(kT) void conv_stem_backward_kernel(const StemGeom g
     ODL_STEM_STAMP(7);
 }
 
-// gw[e] / gb[e - OC*9] = sum over the workgroups' partials in workgroup order: a wave per element, lane l adds partials
-// l, l + 64, ..., then the lanes are added pairwise — the same order on every run
-__global__ __launch_bounds__(256) void conv_stem_fold_kernel(const float *__restrict__ part, int nparts, int OC, float *gw, float *gb)
+// gw[e] / gb[e - OC*9] = sum over the workgroups' partials in workgroup order. 64 elements x 16 groups of partials per
+// workgroup: a wave reads 64 neighbouring floats of one partial (whole lines), group q adds partials q, q + 16, ...,
+// and the groups' sums are added in group order — the same order on every run.
+__global__ __launch_bounds__(1024) void conv_stem_fold_kernel(const float *__restrict__ part, int nparts, int OC, float *gw, float *gb)
 {
-    const int E = OC * 10, e = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (e >= E)
-        return;
-    const int lane = threadIdx.x & 63;
+    __shared__ float sums[16][64];
+    const int E = OC * 10, lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int e = blockIdx.x * 64 + lane;
     float s = 0.f;
-    for (int p = lane; p < nparts; p += 64)
-        s += part[(int64_t)p * E + e];
-    for (int off = 32; off > 0; off >>= 1)
-        s += __shfl_xor(s, off);
-    if (lane == 0)
+    if (e < E)
     {
+#pragma unroll 4
+        for (int p = grp; p < nparts; p += 16)
+            s += part[(int64_t)p * E + e];
+    }
+    sums[grp][lane] = s;
+    __syncthreads();
+    if (grp == 0 && e < E)
+    {
+        float v = sums[0][lane];
+#pragma unroll
+        for (int q = 1; q < 16; ++q)
+            v += sums[q][lane];
         if (e < OC * 9)
         {
             if (gw)
-                gw[e] = s;
+                gw[e] = v;
         }
         else if (gb)
-            gb[e - OC * 9] = s;
+            gb[e - OC * 9] = v;
     }
 }
 
@@ -311,7 +319,7 @@ int conv_stem_backward(const float *gy, const float *x, const float *w, float *g
     ODL_LAUNCH_CHECK();
     if (gw || gb)
     {
-        hipLaunchKernelGGL(conv_stem_fold_kernel, dim3((unsigned)ceil_div(OC * 10, 4)), dim3(256), 0, st, g.part, nb, (int)OC, gw, gb);
+        hipLaunchKernelGGL(conv_stem_fold_kernel, dim3((unsigned)ceil_div(OC * 10, 64)), dim3(1024), 0, st, g.part, nb, (int)OC, gw, gb);
         ODL_LAUNCH_CHECK();
     }
     return ODL_OK;
