@@ -121,6 +121,13 @@ size_t odl_hip_matmul_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64
 int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M,
                             int64_t K, int64_t N, void *workspace, size_t workspace_bytes, void *stream);
 size_t odl_hip_matmul_backward_workspace_bytes(int64_t M, int64_t K, int64_t N);
+/* Backward of Linear::forward's matmul + broadcast_to + add for 2-D inputs (src/nn/layers/linear.cpp:88-104): the two
+ * gradients of odl_hip_matmul_backward and gb[N] = gy[M,N] summed over its rows — what Mat::sum_to to the bias's shape
+ * gives (src/mat/origin/cpu/math/sum_to.cpp), bit for bit the result of odl_hip_sum_axis(gy, 1, M, N). For a classifier
+ * layer (N <= 16, long K) the three are one launch. Any output may be NULL. */
+int odl_hip_linear_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, float *gb, int64_t M,
+                            int64_t K, int64_t N, void *workspace, size_t workspace_bytes, void *stream);
+size_t odl_hip_linear_backward_workspace_bytes(int64_t M, int64_t K, int64_t N);
 /* Mat::matmul and MatMul::backward for float64 tensors (the reference's device matmul is a template over the element
  * type and serves double through the kernels it uses for float, src/mat/origin/cuda/math/mat_mul.cu:1911-1954; CPU form
  * src/mat/origin/cpu/math/matmul.cpp:27-41): C[M,N] = op(A)[M,K] . op(B)[K,N] on the FP64 matrix cores, layouts as in

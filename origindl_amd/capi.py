@@ -144,6 +144,19 @@ def mat_mul_backward(x, w, gy, need_gx=True, need_gw=True):
     return gx, gw
 
 
+def linear_backward(x, w, gy, need_gx=True, need_gw=True, need_gb=True):
+    """Backward of Linear::forward for 2-D inputs (src/nn/layers/linear.cpp:88-104) -> (gx, gw, gb[1, N])."""
+    _chk(x, "x"), _chk(w, "w"), _chk(gy, "gy")
+    M, K = x.shape
+    N = w.shape[1]
+    gx = _empty((M, K)) if need_gx else None
+    gw = _empty((K, N)) if need_gw else None
+    gb = _empty((1, N)) if need_gb else None
+    ws, nb = _ws(lib().query("odl_hip_linear_backward_workspace_bytes", M, K, N))
+    lib().call("odl_hip_linear_backward", _p(x), _p(w), _p(gy), _p(gx), _p(gw), _p(gb), M, K, N, _p(ws), nb, _stream())
+    return gx, gw, gb
+
+
 def transpose(x):
     _chk(x, "x")
     if x.dim() < 2:

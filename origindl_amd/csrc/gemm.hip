@@ -30,8 +30,9 @@ namespace odl
 bool skinny_ok(int64_t M, int64_t N, int64_t K);
 int skinny_forward(const float *x, const float *w, const float *bias, float *y, int64_t M, int64_t N, int64_t K, int64_t ldx,
                    int64_t ldw, int64_t ldy, int act, hipStream_t st);
-int skinny_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M, int64_t K, int64_t N,
-                    hipStream_t st);
+bool skinny_bias_ok(int64_t M, int64_t N);
+int skinny_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, float *gb, int64_t M, int64_t K,
+                    int64_t N, hipStream_t st);
 }  // namespace odl
 
 namespace
@@ -1681,7 +1682,7 @@ int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, flo
     ODL_REQUIRE_DEVICE();
     hipStream_t st = odl::as_stream(stream);
     if ((gx || gw) && x && w && gy && M > 0 && odl::skinny_ok(M, N, K))
-        return odl::skinny_backward(x, w, gy, gx, gw, M, K, N, st);  // both gradients of a classifier layer in one launch
+        return odl::skinny_backward(x, w, gy, gx, gw, nullptr, M, K, N, st);  // both gradients of a classifier layer in one launch
     if (gx && gw && x && w && gy)
     {
         const int paired = odl::matmul_backward_pair(x, w, gy, gx, gw, M, K, N, st);
@@ -1707,6 +1708,32 @@ int odl_hip_matmul_backward(const float *x, const float *w, const float *gy, flo
         if (rc != ODL_OK)
             return rc;
     }
+    return ODL_OK;
+}
+
+size_t odl_hip_linear_backward_workspace_bytes(int64_t M, int64_t K, int64_t N)
+{
+    const size_t a = odl_hip_matmul_backward_workspace_bytes(M, K, N), b = odl_hip_sum_axis_workspace_bytes(1, M, N);
+    return a > b ? a : b;
+}
+
+int odl_hip_linear_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, float *gb, int64_t M,
+                            int64_t K, int64_t N, void *workspace, size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(M >= 0 && K >= 0 && N >= 0, "linear_backward: negative dimension");
+    ODL_REQUIRE(gy != nullptr || M * N == 0, "linear_backward: gy is null");
+    // a classifier layer: the three gradients in one launch
+    if (gb && (gx || gw) && x && w && gy && M > 0 && odl::skinny_ok(M, N, K) && odl::skinny_bias_ok(M, N))
+        return odl::skinny_backward(x, w, gy, gx, gw, gb, M, K, N, odl::as_stream(stream));
+    if (gx || gw)
+    {
+        const int rc = odl_hip_matmul_backward(x, w, gy, gx, gw, M, K, N, workspace, workspace_bytes, stream);
+        if (rc != ODL_OK)
+            return rc;
+    }
+    if (gb)  // (stream order: the workspace is free again)
+        return odl_hip_sum_axis(gy, 1, M, N, gb, workspace, workspace_bytes, stream);
     return ODL_OK;
 }
 

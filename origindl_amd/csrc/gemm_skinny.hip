@@ -8,6 +8,7 @@
 //   gw[k][n]  = sum_m x[m][k] gy[m][n]                        sixteen k a workgroup, its waves share the rows, summed in wave order
 // Sums are formed in a fixed order (strided partials, then fixed-order passes through LDS): deterministic.
 #include "odl_common.h"
+#include "reduce_small.h"
 
 namespace
 {
@@ -114,9 +115,11 @@ __global__ __launch_bounds__(256) void skinny_fwd_kernel(const float *__restrict
 struct SkinnyBwd
 {
     const float *x, *w, *gy;
-    float *gx, *gw;
+    float *gx, *gw, *gb;
     int M, K;
-    int gx_blocks;    // workgroups [0, gx_blocks) form gx, the rest gw
+    int gb_quads;     // the bias gradient's column sums take four columns a lane (N % 4 == 0 and gy 16-byte aligned)
+    int gw_blocks;    // workgroups [gx_blocks, gx_blocks + gw_blocks) form gw; one more, if gb is wanted, the bias gradient
+    int gx_blocks;    // workgroups [0, gx_blocks) form gx
     int gx_ktiles;    // tiles of 1024 k per row group
     int rows_per;     // rows of gx a workgroup walks
 };
@@ -134,6 +137,34 @@ __global__ __launch_bounds__(1024) void skinny_bwd_kernel(SkinnyBwd g)
     float(*part)[64][N] = reinterpret_cast<float(*)[64][N]>(buf);
     static_assert(kGyRows <= 16 * 64, "a block of gy rows must fit the buffer");
     const int bid = blockIdx.x;
+    if (bid >= g.gx_blocks + g.gw_blocks)
+    {
+        // the bias gradient of the layer, gb[n] = sum over the rows of gy[:, n]: the column sum Mat::sum_to would run as a
+        // launch of its own (reduce_small.h), here by this workgroup's first 256 threads — the same additions in the same
+        // order
+        static_assert(sizeof(buf) >= sizeof(odl::ColSumSmall<1, 16>::Sums), "the group sums must fit the buffer");
+        static_assert(N % 4 != 0 || sizeof(buf) >= sizeof(odl::ColSumSmall<4, 8>::Sums), "the group sums must fit the buffer");
+        const unsigned tid = threadIdx.x;
+        if (N % 4 == 0 && g.gb_quads)
+        {
+            auto &sh = *reinterpret_cast<typename odl::ColSumSmall<4, 8>::Sums *>(buf);
+            if (tid < 256)
+                odl::ColSumSmall<4, 8>::accumulate(g.gy, g.M, N, 0, 0, tid, sh);
+            __syncthreads();
+            if (tid < 256)
+                odl::ColSumSmall<4, 8>::finish(g.gb, N, 0, 0, tid, sh);
+        }
+        else
+        {
+            auto &sh = *reinterpret_cast<typename odl::ColSumSmall<1, 16>::Sums *>(buf);
+            if (tid < 256)
+                odl::ColSumSmall<1, 16>::accumulate(g.gy, g.M, N, 0, 0, tid, sh);
+            __syncthreads();
+            if (tid < 256)
+                odl::ColSumSmall<1, 16>::finish(g.gb, N, 0, 0, tid, sh);
+        }
+        return;
+    }
     if (bid < g.gx_blocks)
     {
         const int kt = bid % g.gx_ktiles, rg = bid / g.gx_ktiles;
@@ -247,8 +278,7 @@ void launch_fwd(const float *x, const float *w, const float *b, float *y, int64_
 template <int N>
 void launch_bwd(const SkinnyBwd &g, hipStream_t st)
 {
-    const int gw_blocks = g.gw ? (int)odl::ceil_div(g.K, 16) : 0;
-    hipLaunchKernelGGL(skinny_bwd_kernel<N>, dim3((unsigned)(g.gx_blocks + gw_blocks)), dim3(1024), 0, st, g);
+    hipLaunchKernelGGL(skinny_bwd_kernel<N>, dim3((unsigned)(g.gx_blocks + g.gw_blocks + (g.gb ? 1 : 0))), dim3(1024), 0, st, g);
 }
 }  // namespace
 
@@ -293,10 +323,23 @@ int skinny_forward(const float *x, const float *w, const float *bias, float *y, 
 }
 
 // gx[M,K] = gy[M,N] . w[K,N]^T and gw[K,N] = x[M,K]^T . gy[M,N] (dense operands), either output may be null
-int skinny_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M, int64_t K, int64_t N,
-                    hipStream_t st)
+// gb (may be null): the bias gradient gy summed over its rows, as one more workgroup of the launch; only for sizes that
+// Mat::sum_to would sum in one small launch (skinny_bias_ok), whose bits it then gives
+bool skinny_bias_ok(int64_t M, int64_t N)
 {
-    SkinnyBwd g{x, w, gy, gx, gw, (int)M, (int)K, 0, (int)ceil_div(K, 1024), 2};
+    return N <= 16 && small_cols(1, M, N);
+}
+
+int skinny_backward(const float *x, const float *w, const float *gy, float *gx, float *gw, float *gb, int64_t M, int64_t K,
+                    int64_t N, hipStream_t st)
+{
+    if (gb && !skinny_bias_ok(M, N))
+        return fail(ODL_ERR_RUNTIME, "linear_backward: the bias gradient of this size does not ride in the classifier launch");
+    SkinnyBwd g{};
+    g.x = x, g.w = w, g.gy = gy, g.gx = gx, g.gw = gw, g.gb = gb, g.M = (int)M, g.K = (int)K;
+    g.gb_quads = (N % 4 == 0 && reinterpret_cast<uintptr_t>(gy) % 16 == 0) ? 1 : 0;
+    g.gw_blocks = gw ? (int)ceil_div(K, 16) : 0;
+    g.gx_blocks = 0, g.gx_ktiles = (int)ceil_div(K, 1024), g.rows_per = 2;
     if (gx)
     {
         // a workgroup re-reads w once per group of rows: eight rows or more, and no more workgroups than two per compute unit

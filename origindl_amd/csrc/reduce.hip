@@ -10,6 +10,7 @@
 #include <cstdint>
 
 #include "odl_common.h"
+#include "reduce_small.h"
 
 #include <mutex>
 
@@ -165,61 +166,11 @@ template <int VEC, int CW>
 __global__ __launch_bounds__(kBlock) void col_sum_small_kernel(const float *__restrict__ src, float *__restrict__ dst,
                                                                 int64_t axis, int64_t inner)
 {
-    constexpr int G = kBlock / CW;
-    __shared__ float sh[G][CW * VEC + 1];
-    const int lane = threadIdx.x % CW, grp = threadIdx.x / CW;
-    const int64_t o = blockIdx.y;
-    const int64_t col = ((int64_t)blockIdx.x * CW + lane) * VEC;
-    const bool live = col < inner;
-    const float *p = src + (o * axis) * inner + col;
-    float acc[VEC];
-#pragma unroll
-    for (int e = 0; e < VEC; ++e)
-        acc[e] = 0.f;
-    if (live)
-    {
-        int64_t a = grp;
-        for (; a + 7 * G < axis; a += 8 * G)
-        {
-            float v[8][VEC];
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-            {
-                if (VEC == 4)
-                {
-                    const f32x4 q = *reinterpret_cast<const f32x4 *>(p + (a + u * G) * inner);
-                    v[u][0] = q[0], v[u][1 % VEC] = q[1], v[u][2 % VEC] = q[2], v[u][3 % VEC] = q[3];
-                }
-                else
-                    v[u][0] = p[(a + u * G) * inner];
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-#pragma unroll
-                for (int e = 0; e < VEC; ++e)
-                    acc[e] += v[u][e];
-        }
-        for (; a < axis; a += G)
-#pragma unroll
-            for (int e = 0; e < VEC; ++e)
-                acc[e] += p[a * inner + e];
-    }
-#pragma unroll
-    for (int e = 0; e < VEC; ++e)
-        sh[grp][lane * VEC + e] = acc[e];
+    // (the two halves live in reduce_small.h: the classifier layers' backward launch runs them as one of its jobs)
+    __shared__ typename odl::ColSumSmall<VEC, CW>::Sums sh;
+    odl::ColSumSmall<VEC, CW>::accumulate(src, axis, inner, blockIdx.x, blockIdx.y, threadIdx.x, sh);
     __syncthreads();
-    if (threadIdx.x < CW * VEC)
-    {
-        const int64_t c = (int64_t)blockIdx.x * CW * VEC + threadIdx.x;
-        if (c < inner)
-        {
-            float t = sh[0][threadIdx.x];
-#pragma unroll 4
-            for (int g = 1; g < G; ++g)
-                t += sh[g][threadIdx.x];
-            dst[o * inner + c] = t;
-        }
-    }
+    odl::ColSumSmall<VEC, CW>::finish(dst, inner, blockIdx.x, blockIdx.y, threadIdx.x, sh);
 }
 
 // dst[i] = sum over s of part[s*n + i]. 64 columns x 16 slice groups per workgroup: group g adds slices
@@ -661,11 +612,7 @@ struct SumPlan
     size_t ws_bytes;
 };
 
-// column sums small enough to be bound by launch latency: one launch (col_sum_small_kernel)
-bool small_cols(int64_t outer, int64_t axis, int64_t inner)
-{
-    return inner > 1 && axis >= 16 && outer <= 1024 && outer * axis * inner <= (1 << 20);
-}
+using odl::small_cols;  // (reduce_small.h)
 
 SumPlan plan_sum(int64_t outer, int64_t axis, int64_t inner)
 {

@@ -494,6 +494,9 @@ public:
     // {gy . w^T, x^T . gy} for 2-D operands, reading w and x in place (no transposed copies)
     static std::pair<std::unique_ptr<Mat>, std::unique_ptr<Mat>> matmul_backward_2d(const Mat &x, const Mat &w,
                                                                                    const Mat &gy);
+    // Backward of Linear for 2-D inputs: matmul_backward_2d's two gradients and gy summed to bias_shape ({N} or {1, N}),
+    // one library call (one launch for a classifier layer); the values of the separate operators
+    static std::vector<std::unique_ptr<Mat>> linear_backward_2d(const Mat &x, const Mat &w, const Mat &gy, const Shape &bias_shape);
     float accuracy(const Mat &target_int32) const;
 
     // ---- OriginMat-only helpers used by callers (origin_mat.h:442-559 in the reference)

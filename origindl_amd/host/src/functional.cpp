@@ -286,8 +286,8 @@ struct FusedLinear : Operator
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
-        auto g = OriginMat::matmul_backward_2d(mat(inputs_[0]), mat(inputs_[1]), mat(gys[0]));
-        return {wrap(std::move(g.first)), wrap(std::move(g.second)), wrap(mat(gys[0]).sum_to(inputs_[2].shape()))};
+        auto g = OriginMat::linear_backward_2d(mat(inputs_[0]), mat(inputs_[1]), mat(gys[0]), inputs_[2].shape());
+        return {wrap(std::move(g[0])), wrap(std::move(g[1])), wrap(std::move(g[2]))};
     }
 };
 
@@ -307,8 +307,8 @@ struct FusedLinearRelu : Operator
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
         auto g0 = omat(gys[0]).relu_backward(*y);
-        auto g  = OriginMat::matmul_backward_2d(mat(inputs_[0]), mat(inputs_[1]), *g0);
-        return {wrap(std::move(g.first)), wrap(std::move(g.second)), wrap(g0->sum_to(inputs_[2].shape()))};
+        auto g  = OriginMat::linear_backward_2d(mat(inputs_[0]), mat(inputs_[1]), *g0, inputs_[2].shape());
+        return {wrap(std::move(g[0])), wrap(std::move(g[1])), wrap(std::move(g[2]))};
     }
 };
 

@@ -2276,6 +2276,37 @@ std::pair<std::unique_ptr<Mat>, std::unique_ptr<Mat>> OriginMat::matmul_backward
     return {std::move(gx), std::move(gw)};
 }
 
+std::vector<std::unique_ptr<Mat>> OriginMat::linear_backward_2d(const Mat &x_, const Mat &w_, const Mat &gy_, const Shape &bias_shape)
+{
+    std::vector<std::unique_ptr<Mat>> out;
+    const bool f32 = x_.dtype() == DataType::kFloat32 && w_.dtype() == DataType::kFloat32 && gy_.dtype() == DataType::kFloat32;
+    const Shape gs = gy_.shape();
+    const bool row_bias = gs.size() == 2 && (bias_shape.size() == 1 || (bias_shape.size() == 2 && bias_shape[0] == 1)) &&
+                          bias_shape[bias_shape.size() - 1] == gs[1] && gs[0] > 0 && gs[1] > 0;
+    if (!f32 || !row_bias)
+    {
+        // other element types, or a bias of another shape: the operators one after the other
+        auto g = matmul_backward_2d(x_, w_, gy_);
+        out.push_back(std::move(g.first)), out.push_back(std::move(g.second));
+        out.push_back(gy_.sum_to(bias_shape));
+        return out;
+    }
+    const OriginMat &x = dev_f32(x_, "matmul"), &w = dev_f32(w_, "matmul"), &gy = dev_f32(gy_, "matmul");
+    const Shape xs = x.shape(), ws_ = w.shape();
+    if (xs.size() != 2 || ws_.size() != 2 || xs[1] != ws_[0] || gs[0] != xs[0] || gs[1] != ws_[1])
+        THROW_INVALID_ARG("matmul backward: shapes {} {} {} do not form x[M,K] w[K,N] gy[M,N]", xs.to_string(),
+                          ws_.to_string(), gs.to_string());
+    const int64_t M = xs[0], K = xs[1], N = ws_[1];
+    auto gx = new_like(x, xs);
+    auto gw = new_like(w, ws_);
+    auto gb = new_like(gy, bias_shape);
+    Workspace ws(odl_hip_linear_backward_workspace_bytes(M, K, N), x.device().index());
+    check(odl_hip_linear_backward(fp(x), fp(w), fp(gy), gx->data_ptr<float>(), gw->data_ptr<float>(), gb->data_ptr<float>(), M,
+                                  K, N, ws.ptr(), ws.bytes, cur()));
+    out.push_back(std::move(gx)), out.push_back(std::move(gw)), out.push_back(std::move(gb));
+    return out;
+}
+
 float OriginMat::accuracy(const Mat &target_int32) const
 {
     const OriginMat &y = dev_f32(*this, "accuracy");

@@ -147,6 +147,34 @@ def test_matmul_backward_in_one_launch_equals_the_two_gradients_launched_alone(a
     assert bool(((gx2.double() - want_gx).abs() <= bx).all()) and bool(((gw2.double() - want_gw).abs() <= bw).all())
 
 
+@pytest.mark.parametrize("m,k,n", [
+    (512, 1000, 10),     # the MLP's classifier layer: the three gradients in one launch, column sums one float a lane
+    (256, 128, 10),      # the CNN's
+    (300, 640, 16),      # sixteen classes: column sums in 16-byte pieces
+    (64, 200, 12), (33, 130, 1), (17, 256, 3),
+    (70000, 130, 16),    # more rows than the one-launch column sum takes: the sum as a launch of its own
+    (512, 784, 1000),    # a wide layer: paired matrix gradients, then the column sum
+    (5, 7, 3),
+])
+def test_linear_backward_equals_matmul_backward_and_sum_to(api, m, k, n):
+    # Linear's backward as one library call: gx and gw must be the bits of odl_hip_matmul_backward, gb the bits of
+    # Mat::sum_to of gy to the bias's shape — wherever the bias gradient rides in the classifier launch as well — and
+    # every subset of the three must give the same values.
+    print("\n[case] linear backward", m, k, n, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(m * 3 + k + n)
+    x, w, gy = (torch.randn(s, device="cuda", generator=g) for s in ((m, k), (k, n), (m, n)))
+    gx0, gw0 = api.mat_mul_backward(x, w, gy)
+    gb0 = api.sum_to(gy, (1, n))
+    gx, gw, gb = api.linear_backward(x, w, gy)
+    assert torch.equal(gx, gx0) and torch.equal(gw, gw0) and torch.equal(gb, gb0)
+    want = gy.double().sum(dim=0, keepdim=True)
+    assert bool(((gb.double() - want).abs() <= 1e-5 * np.sqrt(m) * gy.double().norm(dim=0) + 1e-6).all())
+    for need in ((True, False, True), (False, True, True), (False, False, True), (True, True, False)):
+        got = api.linear_backward(x, w, gy, *need)
+        for t, ref in zip(got, (gx0, gw0, gb0)):
+            assert t is None or torch.equal(t, ref), need
+
+
 def test_matmul_reference_unit_test_vectors(api):
     # tests/unit_test/operator/test_matmul.cpp:19-64, 119-143, 213-229
     x, w = dev(np.array([[1, 2], [3, 4]], f32)), dev(np.array([[5, 6], [7, 8]], f32))
