@@ -20,6 +20,7 @@
 //   * split-K (grid.y) writes partial tiles that a second kernel sums in slice order — deterministic.
 #include "gemm_dma.h"
 #include "odl_common.h"
+#include "reduce_small.h"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -1253,9 +1254,13 @@ odl::DmaGemmArgs pair_product(int cls, const float *A, int64_t lda, const float 
 }
 }  // namespace
 
+// gb (may be null): the bias gradient, gy summed over its rows, in the same launch when its size is one the small column
+// sum takes (*gb_done tells)
 int matmul_backward_pair(const float *x, const float *w, const float *gy, float *gx, float *gw, int64_t M, int64_t K,
-                         int64_t N, hipStream_t st)
+                         int64_t N, hipStream_t st, float *gb = nullptr, bool *gb_done = nullptr)
 {
+    if (gb_done)
+        *gb_done = false;
     if (M <= 0 || K <= 0 || N <= 0 || M >= (1ll << 31) || K >= (1ll << 31) || N >= (1ll << 31))
         return 0;
     // 16-byte loads: every row of x [M,K], w [K,N] and gy [M,N] starts on a 16-byte boundary and M is a multiple of four
@@ -1272,9 +1277,19 @@ int matmul_backward_pair(const float *x, const float *w, const float *gy, float 
         return 0;
     if (!odl::sgemm_dma_fits(false, true, d0) || !odl::sgemm_dma_fits(true, false, d1))
         return 0;
-    const int rc = odl::sgemm_dma_pair_launch(c0, d0, c1, d1, st);
+    odl::ColSumJob job{};
+    const bool with_sum = gb && gb_done && odl::small_cols(1, M, N);
+    if (with_sum)
+    {
+        job.src = gy, job.dst = gb, job.axis = M, job.inner = N;
+        job.quads = (N % 4 == 0 && reinterpret_cast<uintptr_t>(gy) % 16 == 0) ? 1 : 0;
+        job.blocks = (unsigned)odl::ceil_div(N, job.quads ? 32 : 16);
+    }
+    const int rc = odl::sgemm_dma_pair_launch(c0, d0, c1, d1, st, with_sum ? &job : nullptr);
     if (rc != ODL_OK)
         return rc;  // (error codes are negative)
+    if (with_sum)
+        *gb_done = true;
     return 1;
 }
 
@@ -1726,6 +1741,21 @@ int odl_hip_linear_backward(const float *x, const float *w, const float *gy, flo
     // a classifier layer: the three gradients in one launch
     if (gb && (gx || gw) && x && w && gy && M > 0 && odl::skinny_ok(M, N, K) && odl::skinny_bias_ok(M, N))
         return odl::skinny_backward(x, w, gy, gx, gw, gb, M, K, N, odl::as_stream(stream));
+    if (gb && gx && gw && x && w && gy && M > 0 && !odl::skinny_ok(M, N, K))
+    {
+        // both matrix gradients as one launch of two products, the column sum as a few more workgroups of it
+        bool gb_done = false;
+        const int paired = odl::matmul_backward_pair(x, w, gy, gx, gw, M, K, N, odl::as_stream(stream), gb, &gb_done);
+        if (paired < 0)
+            return paired;
+        if (paired == 1)
+        {
+            ODL_LAUNCH_CHECK();
+            if (gb_done)
+                return ODL_OK;
+            return odl_hip_sum_axis(gy, 1, M, N, gb, workspace, workspace_bytes, stream);
+        }
+    }
     if (gx || gw)
     {
         const int rc = odl_hip_matmul_backward(x, w, gy, gx, gw, M, K, N, workspace, workspace_bytes, stream);

@@ -43,7 +43,19 @@ int sgemm_dma_launch(int tile, bool ta, bool tb, const DmaGemmArgs &g, hipStream
 // Two whole products in one launch, two workgroups per compute unit: g0 = X.Y^T (A [M,K] and B [N,K] row-major) on tiles
 // of class tile0, g1 = X^T.Y (A [K,M] and B [K,N] row-major) on tiles of class tile1. Classes: 64 (64x64 tiles), 32 (64x32
 // tiles) — these two mix freely — or 128 for both (128x128 tiles). tiles_m / tiles_n of each product count its own tiles.
-int sgemm_dma_pair_launch(int tile0, const DmaGemmArgs &g0, int tile1, const DmaGemmArgs &g1, hipStream_t st);
+// `sums` (may be null): a small column sum (reduce_small.h) run by `blocks` more workgroups of the same launch — the bias
+// gradient beside a layer's two matrix gradients: dst[c] = sum over the `axis` rows of src[:, c], `inner` columns; quads:
+// four columns a lane (inner % 4 == 0, src 16-byte aligned), else one.
+struct ColSumJob
+{
+    const float *src;
+    float *dst;
+    int64_t axis, inner;
+    int quads;
+    unsigned blocks;
+};
+int sgemm_dma_pair_launch(int tile0, const DmaGemmArgs &g0, int tile1, const DmaGemmArgs &g1, hipStream_t st,
+                          const ColSumJob *sums = nullptr);
 
 // 1x1 / stride 1 / unpadded convolution as `N` products y[n] = act(W[OC,C] . x[n][C, H*W] + b[oc]) in one launch; false
 // when the shape does not suit (rows of H*W or C floats that are not multiples of four, unaligned pointers)

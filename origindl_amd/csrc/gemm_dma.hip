@@ -22,6 +22,7 @@
 //     64x64x32 and 64x32x64 at one (few tiles), 64x64x32 at two (batches of small products: 1x1 convolutions).
 #include "gemm_dma.h"
 #include "odl_common.h"
+#include "reduce_small.h"
 
 namespace
 {
@@ -595,7 +596,8 @@ __global__ __launch_bounds__(kNT, WGS_PER_CU) void sgemm_dma_kernel(const odl::D
 template <int BM0, int BN0, int BK0, int KSETS0, int ST0, int BM1, int BN1, int BK1, int KSETS1, int ST1>
 __global__ __launch_bounds__(kNT, 2) void sgemm_dma_pair_kernel(const odl::DmaGemmArgs g0, const DmaTileMap map0,
                                                                 const odl::DmaGemmArgs g1, const DmaTileMap map1,
-                                                                const unsigned first, const unsigned first_padded)
+                                                                const unsigned first, const unsigned first_padded,
+                                                                const unsigned n1, const odl::ColSumJob sums)
 {
     constexpr int F0 = ST0 * (BM0 + BN0) * BK0, F1 = ST1 * (BM1 + BN1) * BK1;
     static_assert(F0 * 4 <= 80 * 1024 && F1 * 4 <= 80 * 1024, "two workgroups must fit the LDS of a compute unit");
@@ -604,7 +606,34 @@ __global__ __launch_bounds__(kNT, 2) void sgemm_dma_pair_kernel(const odl::DmaGe
     if (bid < first)
         sgemm_dma_body<BM0, BN0, BK0, false, true, KSETS0, ST0>(g0, map0, bid, stages, stages + ST0 * BM0 * BK0);
     else if (bid >= first_padded)  // (the gap keeps product 1's workgroup numbers congruent to the XCD they run on)
-        sgemm_dma_body<BM1, BN1, BK1, true, false, KSETS1, ST1>(g1, map1, bid - first_padded, stages, stages + ST1 * BM1 * BK1);
+    {
+        if (bid - first_padded < n1)
+            sgemm_dma_body<BM1, BN1, BK1, true, false, KSETS1, ST1>(g1, map1, bid - first_padded, stages, stages + ST1 * BM1 * BK1);
+        else
+        {
+            // the column sum that rides along (the first 256 threads run reduce_small.h's two halves: the bits of the
+            // launch of its own)
+            const unsigned bx = bid - first_padded - n1, tid = threadIdx.x;
+            if (sums.quads)
+            {
+                auto &sh = *reinterpret_cast<typename odl::ColSumSmall<4, 8>::Sums *>(stages);
+                if (tid < 256)
+                    odl::ColSumSmall<4, 8>::accumulate(sums.src, sums.axis, sums.inner, bx, 0, tid, sh);
+                __syncthreads();
+                if (tid < 256)
+                    odl::ColSumSmall<4, 8>::finish(sums.dst, sums.inner, bx, 0, tid, sh);
+            }
+            else
+            {
+                auto &sh = *reinterpret_cast<typename odl::ColSumSmall<1, 16>::Sums *>(stages);
+                if (tid < 256)
+                    odl::ColSumSmall<1, 16>::accumulate(sums.src, sums.axis, sums.inner, bx, 0, tid, sh);
+                __syncthreads();
+                if (tid < 256)
+                    odl::ColSumSmall<1, 16>::finish(sums.dst, sums.inner, bx, 0, tid, sh);
+            }
+        }
+    }
 }
 }  // namespace
 
@@ -633,7 +662,8 @@ static DmaTileMap tile_map_of(const DmaGemmArgs &g)
     return map;
 }
 
-int sgemm_dma_pair_launch(int tile0, const DmaGemmArgs &g0, int tile1, const DmaGemmArgs &g1, hipStream_t st)
+int sgemm_dma_pair_launch(int tile0, const DmaGemmArgs &g0, int tile1, const DmaGemmArgs &g1, hipStream_t st,
+                          const ColSumJob *sums)
 {
     if (g0.splits != 1 || g1.splits != 1 || g0.tail_splits > 0 || g1.tail_splits > 0 || g0.batch > 1 || g1.batch > 1 ||
         g0.c_p > 0 || g1.c_p > 0)
@@ -641,7 +671,8 @@ int sgemm_dma_pair_launch(int tile0, const DmaGemmArgs &g0, int tile1, const Dma
     const unsigned n0 = (unsigned)(g0.tiles_m * g0.tiles_n), n1 = (unsigned)(g1.tiles_m * g1.tiles_n);
     const unsigned nx = (unsigned)(g0.xcds > 0 ? g0.xcds : 1), n0p = (n0 + nx - 1) / nx * nx;
     const DmaTileMap m0 = tile_map_of(g0), m1 = tile_map_of(g1);
-    const dim3 grid(n0p + n1), block(kNT);
+    const ColSumJob job = sums ? *sums : ColSumJob{};
+    const dim3 grid(n0p + n1 + job.blocks), block(kNT);
     // per class: tile rows, tile columns, slab width, wave sets, stages (two workgroups of 64 to 72 KB per compute unit)
 #define ODL_PAIR_64 64, 64, 32, 2, 4
 #define ODL_PAIR_32 64, 32, 64, 4, 3
@@ -649,7 +680,7 @@ int sgemm_dma_pair_launch(int tile0, const DmaGemmArgs &g0, int tile1, const Dma
 #define ODL_PAIR_CASE(T0, C0, T1, C1)                                                                                   \
     if (tile0 == T0 && tile1 == T1)                                                                                     \
     {                                                                                                                   \
-        hipLaunchKernelGGL((sgemm_dma_pair_kernel<C0, C1>), grid, block, 0, st, g0, m0, g1, m1, n0, n0p);               \
+        hipLaunchKernelGGL((sgemm_dma_pair_kernel<C0, C1>), grid, block, 0, st, g0, m0, g1, m1, n0, n0p, n1, job);      \
         return ODL_OK;                                                                                                  \
     }
     ODL_PAIR_CASE(64, ODL_PAIR_64, 64, ODL_PAIR_64)
