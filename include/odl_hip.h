@@ -334,6 +334,24 @@ int odl_hip_max_pool2d_backward(const float *gy, const uint64_t *idx, int64_t N,
  * windows run the two steps. x has the shape of gx. */
 int odl_hip_max_pool2d_backward_relu(const float *gy, const uint64_t *idx, const float *x, int64_t N, int64_t C, int64_t H,
                                      int64_t W, int KH, int KW, int SH, int SW, int PH, int PW, float *gx, void *stream);
+/* The same from the pooled tensor y [N, C, OH, OW] instead of the pooling's input x: the cell that receives a window's
+ * gradient is its maximum, so (x > 0) there is (y > 0), and every other cell gets the +0 it gets above — same floats.
+ * Only for windows that tile the image exactly (2x2/2, 3x3/3, no padding); for the layers whose pooled input was never
+ * written (odl_hip_conv2d_relu_max_pool2d). */
+int odl_hip_max_pool2d_backward_relu_pooled(const float *gy, const uint64_t *idx, const float *y, int64_t N, int64_t C,
+                                            int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH, int PW, float *gx,
+                                            void *stream);
+/* Conv2d + ReLU + MaxPool2d of a Sequential (src/nn/layers/conv2d.cpp, src/operators/activation/relu.cpp:13-21,
+ * src/operators/pooling/max_pool2d.cpp:25-58) in one pass for the layers odl_hip_conv2d_relu_max_pool2d_ok names (1 / 0):
+ * a 3x3 / stride 1 / padding 1 convolution with few input channels — a network's first layer — under a 2x2 / stride 2
+ * pooling, H and W even. y [N, OC, H/2, W/2] and idx (window-local argmax as in odl_hip_max_pool2d; may be NULL) hold
+ * the floats and indices of odl_hip_conv2d_act(relu) followed by odl_hip_max_pool2d; the tensor between them is never
+ * written. No workspace. */
+int odl_hip_conv2d_relu_max_pool2d_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW,
+                                      int PH, int PW, int PKH, int PKW, int PSH, int PSW, int PPH, int PPW);
+int odl_hip_conv2d_relu_max_pool2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                                   int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int PKH, int PKW, int PSH,
+                                   int PSW, int PPH, int PPW, float *y, uint64_t *idx, void *stream);
 
 /* ------------------------------------------------------------------ metrics ------------------------- */
 /* argmax per row, first maximum (src/utils/metrics.cpp:40-53), and accuracy() (metrics.cpp:11-70) with

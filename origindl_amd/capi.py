@@ -486,6 +486,53 @@ def max_pool2d(x, kernel_size, stride, pad, with_indices=True):
     return y, idx
 
 
+def conv2d_relu_max_pool2d_ok(x_shape, w_shape, stride=1, pad=1, pool_kernel=2, pool_stride=2, pool_pad=0):
+    """Whether Conv2d + ReLU + MaxPool2d of these shapes run as one pass (odl_hip_conv2d_relu_max_pool2d_ok)."""
+    N, C, H, W = [int(v) for v in x_shape]
+    OC, _, KH, KW = [int(v) for v in w_shape]
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    (PKH, PKW), (PSH, PSW), (PPH, PPW) = _pair(pool_kernel), _pair(pool_stride), _pair(pool_pad)
+    return lib().query("odl_hip_conv2d_relu_max_pool2d_ok", N, C, H, W, OC, KH, KW, SH, SW, PH, PW, PKH, PKW, PSH, PSW, PPH,
+                       PPW) == 1
+
+
+def conv2d_relu_max_pool2d(x, w, b=None, stride=1, pad=1, pool_kernel=2, pool_stride=2, pool_pad=0, with_indices=True):
+    """max_pool2d(relu(conv2d(x, w, b))) in one pass -> (pooled, indices); raises where there is no such kernel."""
+    _chk(x, "x"), _chk(w, "W")
+    if b is not None:
+        _chk(b, "b")
+    N, C, H, W = x.shape
+    OC, _, KH, KW = w.shape
+    (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
+    (PKH, PKW), (PSH, PSW), (PPH, PPW) = _pair(pool_kernel), _pair(pool_stride), _pair(pool_pad)
+    y = _empty((N, OC, H // 2, W // 2))
+    idx = torch.empty(y.shape, dtype=torch.int64, device="cuda") if with_indices else None  # uint64 bit pattern
+    lib().call("odl_hip_conv2d_relu_max_pool2d", _p(x), _p(w), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, PKH, PKW, PSH, PSW,
+               PPH, PPW, _p(y), _p(idx), _stream())
+    return y, idx
+
+
+def max_pool2d_backward_relu(gy, idx, x, kernel_size, stride, pad):
+    """MaxPool2d::backward then ReLU::backward, x the tensor that was pooled (odl_hip_max_pool2d_backward_relu)."""
+    _chk(gy, "gy"), _chk(x, "x")
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = x.shape
+    gx = _empty((N, C, H, W))
+    lib().call("odl_hip_max_pool2d_backward_relu", _p(gy), _p(idx), _p(x), N, C, H, W, KH, KW, SH, SW, PH, PW, _p(gx), _stream())
+    return gx
+
+
+def max_pool2d_backward_relu_pooled(gy, idx, y, input_shape, kernel_size, stride, pad):
+    """The same from the pooled tensor y (odl_hip_max_pool2d_backward_relu_pooled)."""
+    _chk(gy, "gy"), _chk(y, "y")
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = [int(v) for v in input_shape]
+    gx = _empty((N, C, H, W))
+    lib().call("odl_hip_max_pool2d_backward_relu_pooled", _p(gy), _p(idx), _p(y), N, C, H, W, KH, KW, SH, SW, PH, PW, _p(gx),
+               _stream())
+    return gx
+
+
 def max_pool2d_backward(gy, idx, input_shape, kernel_size, stride, pad):
     _chk(gy, "gy")
     if gy.dim() != 4:

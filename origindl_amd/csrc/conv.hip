@@ -63,6 +63,8 @@ size_t conv_patch_dgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, in
 int conv_patch_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
                      void *workspace, size_t workspace_bytes, hipStream_t st, bool packed);
 SidePack conv_patch_dgrad_pack(const float *w, int64_t C, int64_t OC, void *workspace);
+int conv_small_forward_pool(const float *x, const float *w, const float *b, float *y, uint64_t *idx, int64_t N, int64_t C,
+                            int64_t H, int64_t W, int64_t OC, int act, hipStream_t st);
 bool conv_small_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
                          int64_t OW);
 size_t conv_small_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
@@ -1296,6 +1298,33 @@ int odl_hip_conv2d_act_packed(const float *x, const float *w, const float *packe
         return rc;
     return odl::sgemm_launch(0, 1, OC, M, K, w, K, col, K, y, 0, b, /*EPI_NCHW_ROWB*/ 2, g.OH * g.OW, 1, nullptr, 0,
                              st, act);
+}
+
+int odl_hip_conv2d_relu_max_pool2d_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW,
+                                      int PH, int PW, int PKH, int PKW, int PSH, int PSW, int PPH, int PPW)
+{
+    if (!(KH == 3 && KW == 3 && SH == 1 && SW == 1 && PH == 1 && PW == 1))
+        return 0;
+    if (!(PKH == 2 && PKW == 2 && PSH == 2 && PSW == 2 && PPH == 0 && PPW == 0) || H < 2 || W < 2 || H % 2 != 0 || W % 2 != 0)
+        return 0;
+    if (N < 1 || C < 1 || OC < 1)
+        return 0;
+    // exactly the layers whose convolution alone runs as the thread-per-pixel kernel: the pooled values are then its bits
+    if (g_direct.load(std::memory_order_relaxed) && odl::conv_direct_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, H, W))
+        return 0;
+    return odl::conv_small_forward_ok(N, C, H, W, OC, KH, KW, H, W) ? 1 : 0;
+}
+
+int odl_hip_conv2d_relu_max_pool2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
+                                   int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int PKH, int PKW, int PSH,
+                                   int PSW, int PPH, int PPW, float *y, uint64_t *idx, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(x != nullptr && w != nullptr && y != nullptr, "conv2d_relu_max_pool2d: null tensor");
+    if (!odl_hip_conv2d_relu_max_pool2d_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, PKH, PKW, PSH, PSW, PPH, PPW))
+        return odl::fail(ODL_ERR_INVALID_ARG, "conv2d_relu_max_pool2d: this layer pair has no one-pass kernel (ask "
+                                              "odl_hip_conv2d_relu_max_pool2d_ok first)");
+    return odl::conv_small_forward_pool(x, w, b, y, idx, N, C, H, W, OC, /*relu*/ 1, odl::as_stream(stream));
 }
 
 int odl_hip_set_conv_direct(int enabled)

@@ -87,6 +87,93 @@ __global__ __launch_bounds__(kThreads) void conv_small_fwd_kernel(const float *_
     }
 }
 
+// The 3x3 / stride 1 / padding 1 convolution above with ReLU and a 2x2 / stride 2 max pooling behind it in one pass: a
+// thread owns one pooled pixel, computes the four convolution outputs under it (a 4x4 patch of each input channel in
+// registers) for OCB channels, applies bias and activation and keeps the maximum and its place in the window. Per
+// convolution output the terms are added in the order of conv_small_fwd_kernel, and the window is compared in the order
+// of the pooling kernels (row-major, a later cell wins only when it is greater, max_pool2d.cpp:110-139): the pooled
+// values and indices are those of the two kernels run one after the other — without the 4x larger tensor between them.
+template <int OCB>
+__global__ __launch_bounds__(kThreads) void conv_small_fwd_pool_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                                      const float *__restrict__ bias, float *__restrict__ y,
+                                                                      uint64_t *__restrict__ idx, SmallGeom g, int act)
+{
+    // (g.OH, g.OW: the pooled extents; g.total = N * OH * OW)
+    const unsigned pix = blockIdx.x * kThreads + threadIdx.x;
+    if (pix >= g.total)
+        return;
+    const unsigned t = odl::fastdiv(pix, g.by_w), pw = pix - t * g.OW;
+    const unsigned n = odl::fastdiv(t, g.by_h), ph = t - n * g.OH;
+    const int oc0 = blockIdx.y * OCB;
+    const int ih0 = 2 * (int)ph - 1, iw0 = 2 * (int)pw - 1;
+    float acc[4][OCB];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int o = 0; o < OCB; ++o)
+            acc[q][o] = 0.f;
+    for (int c = 0; c < g.C; ++c)
+    {
+        const float *xp = x + ((size_t)n * g.C + c) * g.H * g.W;
+        // the 4x4 patch: rows 2ph-1 .. 2ph+2, columns 2pw-1 .. 2pw+2. With H and W even only its first and last row and
+        // column can lie outside the image, and the two middle columns start at an even offset: one 8-byte load a row
+        // where the image allows it
+        float xr[4][4];
+        const bool left = pw > 0, right = (int)pw + 1 < g.OW, pair_ok = (reinterpret_cast<uintptr_t>(xp) & 7) == 0;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+        {
+            const int ih = ih0 + r;
+            const bool row = (r != 0 || ph > 0) && (r != 3 || (int)ph + 1 < g.OH);
+            const float *rp = xp + (row ? ih : 0) * g.W + 2 * (int)pw;
+            float2 mid;
+            if (pair_ok)
+                mid = *reinterpret_cast<const float2 *>(rp);
+            else
+                mid.x = rp[0], mid.y = rp[1];
+            const float l = left ? rp[-1] : 0.f, rr = right ? rp[2] : 0.f;
+            xr[r][0] = row ? l : 0.f, xr[r][1] = row ? mid.x : 0.f, xr[r][2] = row ? mid.y : 0.f, xr[r][3] = row ? rr : 0.f;
+        }
+        const float *wc = w + ((size_t)oc0 * g.C + c) * 9;
+#pragma unroll
+        for (int o = 0; o < OCB; ++o)
+        {
+            const float *wo = wc + (size_t)o * g.C * 9;  // the same address in every lane
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int j = 0; j < 9; ++j)
+                    acc[q][o] = fmaf(xr[q / 2 + j / 3][q % 2 + j % 3], wo[j], acc[q][o]);
+        }
+    }
+    const size_t plane = (size_t)g.OH * g.OW;
+    const size_t at = ((size_t)n * g.OC + oc0) * plane + (size_t)ph * g.OW + pw;
+#pragma unroll
+    for (int o = 0; o < OCB; ++o)
+    {
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            v[q] = acc[q][o];
+            if (bias)
+                v[q] = v[q] + bias[oc0 + o];
+            v[q] = odl::apply_act(v[q], act);
+        }
+        float m = v[0];
+        int win = 0;
+        if (v[1] > m)
+            m = v[1], win = 1;
+        if (v[2] > m)
+            m = v[2], win = 2;
+        if (v[3] > m)
+            m = v[3], win = 3;
+        y[at + o * plane] = m;
+        if (idx)
+            idx[at + o * plane] = (uint64_t)win;
+    }
+}
+
 // The same convolution for the larger windows (5x5, 6x6): there the filter no longer fits the scalar registers, and
 // reading it through them in pieces leaves the wave waiting on one short load after another. The workgroup stages its
 // OCB channels' filter in LDS once, as [c][tap][oc], and every lane reads it from there 16 bytes at a time (one address
@@ -602,6 +689,18 @@ int conv_small_forward(const float *x, const float *w, const float *b, float *y,
         else
             hipLaunchKernelGGL((conv_small_fwd_lds_kernel<6, 6, 16>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
     }
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+// 3x3 / stride 1 / padding 1 + activation + 2x2 / stride 2 pooling, H and W even; y [N, OC, H/2, W/2], idx may be null
+int conv_small_forward_pool(const float *x, const float *w, const float *b, float *y, uint64_t *idx, int64_t N, int64_t C,
+                            int64_t H, int64_t W, int64_t OC, int act, hipStream_t st)
+{
+    SmallGeom g = make_small(N, C, H, W, OC, 1, 1, 1, 1, H / 2, W / 2, false);
+    // four channels a thread: eight times the pooled pixels in threads, enough waves to hide each other's filter loads
+    const dim3 grid((unsigned)ceil_div(g.total, kThreads), (unsigned)(OC / 4));
+    hipLaunchKernelGGL((conv_small_fwd_pool_kernel<4>), grid, dim3(kThreads), 0, st, x, w, b, y, idx, g, act);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

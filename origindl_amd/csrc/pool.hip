@@ -370,6 +370,43 @@ __global__ __launch_bounds__(256) void max_pool_bwd_tiled_relu_kernel(const floa
     }
 }
 
+// The same from the pooled tensor y alone: the cell that receives the gradient is the window's maximum, whose value is
+// y[o], so (x > 0) there is (y[o] > 0); every other cell gets the +0 it gets above. The input of the pooling is not
+// read (and need not exist any more: conv_small.hip's one-pass convolution + ReLU + pooling never writes it).
+template <int K>
+__global__ __launch_bounds__(256) void max_pool_bwd_tiled_relu_pooled_kernel(const float *__restrict__ gy,
+                                                                             const uint64_t *__restrict__ idx,
+                                                                             const float *__restrict__ y, float *__restrict__ gx,
+                                                                             unsigned total, int OW, unsigned oplane)
+{
+    const unsigned o = blockIdx.x * 256u + threadIdx.x;
+    if (o >= total)
+        return;
+    const int hit = (int)idx[o];
+    const float v = (0.f + gy[o]) * ((y[o] > 0.f) ? 1.f : 0.f);
+    const unsigned nc = o / oplane, r = o - nc * oplane;
+    const int oh = (int)(r / (unsigned)OW), ow = (int)r - oh * OW;
+    const int W = OW * K;
+    const int64_t at = ((int64_t)nc * oplane * (K * K)) + (int64_t)(oh * K) * W + ow * K;
+#pragma unroll
+    for (int kh = 0; kh < K; ++kh)
+    {
+        if (K == 2)
+        {
+            float2 row;
+            row.x = hit == kh * K ? v : 0.f;
+            row.y = hit == kh * K + 1 ? v : 0.f;
+            *reinterpret_cast<float2 *>(gx + at + kh * W) = row;
+        }
+        else
+        {
+#pragma unroll
+            for (int kw = 0; kw < K; ++kw)
+                gx[at + kh * W + kw] = hit == kh * K + kw ? v : 0.f;
+        }
+    }
+}
+
 // gx[i] *= (x[i] > 0 ? 1 : 0) for the window shapes without a fused kernel
 __global__ __launch_bounds__(256) void relu_mask_inplace_kernel(float *__restrict__ gx, const float *__restrict__ x, int64_t n)
 {
@@ -670,6 +707,34 @@ int odl_hip_max_pool2d_backward_relu(const float *gy, const uint64_t *idx, const
     if (rc != ODL_OK)
         return rc;
     hipLaunchKernelGGL(relu_mask_inplace_kernel, dim3((unsigned)odl::ceil_div(total, 256)), dim3(256), 0, st, gx, x, total);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_max_pool2d_backward_relu_pooled(const float *gy, const uint64_t *idx, const float *y, int64_t N, int64_t C,
+                                            int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH, int PW, float *gx,
+                                            void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    PoolGeom g;
+    int rc = make_geom(g, "max_pool2d_backward_relu_pooled", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(idx != nullptr && y != nullptr && gy != nullptr && gx != nullptr, "max_pool2d_backward_relu_pooled: null tensor");
+    if (N * C * H * W == 0)
+        return ODL_OK;
+    // windows that tile the image: each cell belongs to one window, so the mask of the pooled value is the mask of the cell
+    ODL_REQUIRE(plane_ok(g) && tiles_exactly(g) && (reinterpret_cast<uintptr_t>(gx) & 7) == 0,
+                "max_pool2d_backward_relu_pooled: only for windows that tile the image (2x2/2, 3x3/3, no padding)");
+    const unsigned outputs = (unsigned)(N * C * g.OH * g.OW);
+    const dim3 grid((unsigned)odl::ceil_div((int64_t)outputs, 256));
+    hipStream_t st = odl::as_stream(stream);
+    if (g.KH == 2)
+        hipLaunchKernelGGL((max_pool_bwd_tiled_relu_pooled_kernel<2>), grid, dim3(256), 0, st, gy, idx, y, gx, outputs, (int)g.OW,
+                           (unsigned)(g.OH * g.OW));
+    else
+        hipLaunchKernelGGL((max_pool_bwd_tiled_relu_pooled_kernel<3>), grid, dim3(256), 0, st, gy, idx, y, gx, outputs, (int)g.OW,
+                           (unsigned)(g.OH * g.OW));
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

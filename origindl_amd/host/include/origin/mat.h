@@ -496,6 +496,17 @@ public:
                                                                                    const Mat &gy);
     // Backward of Linear for 2-D inputs: matmul_backward_2d's two gradients and gy summed to bias_shape ({N} or {1, N}),
     // one library call (one launch for a classifier layer); the values of the separate operators
+    // Conv2d + ReLU + MaxPool2d in one pass where the library has a kernel for the layer pair (conv_relu_pool_fused):
+    // the pooled tensor and the indices of conv2d_act(relu) followed by max_pool2d_device; backward of the pooling and
+    // the ReLU from the pooled tensor alone (this = the pooled tensor, input_shape = the shape of the convolution's output)
+    static bool conv_relu_pool_fused(const Mat &x, const Mat &W, std::pair<int, int> s, std::pair<int, int> p,
+                                     std::pair<int, int> pk, std::pair<int, int> ps, std::pair<int, int> pp);
+    std::unique_ptr<Mat> conv2d_relu_max_pool2d_device(const Mat &W, const Mat *b, std::pair<int, int> s, std::pair<int, int> p,
+                                                       std::pair<int, int> pk, std::pair<int, int> ps, std::pair<int, int> pp,
+                                                       std::shared_ptr<Storage> *indices) const;
+    std::unique_ptr<Mat> max_pool2d_backward_relu_pooled_device(const Mat &gy, const Shape &input_shape, std::pair<int, int> k,
+                                                                std::pair<int, int> s, std::pair<int, int> p,
+                                                                const Storage &indices) const;
     static std::vector<std::unique_ptr<Mat>> linear_backward_2d(const Mat &x, const Mat &w, const Mat &gy, const Shape &bias_shape);
     float accuracy(const Mat &target_int32) const;
 

@@ -503,7 +503,9 @@ struct MaxPool2d : Operator  // src/operators/pooling/max_pool2d.cpp:14-86
 struct Conv2dReluPoolOp : Conv2dOp
 {
     std::pair<int, int> pk, ps, pp;
-    std::shared_ptr<Mat> y;            // relu(conv(x)), the pooled tensor
+    std::shared_ptr<Mat> y;            // relu(conv(x)), the tensor that is pooled — or null after the one-pass forward
+    std::shared_ptr<Mat> pooled;       // then the output's data instead (not its tensor: that would own this operator)
+    Shape conv_shape;                  // and the shape relu(conv(x)) would have had
     std::shared_ptr<Storage> indices;  // window-local argmax per output, uint64, kept on the device
     Conv2dReluPoolOp(std::pair<int, int> st, std::pair<int, int> pd, std::pair<int, int> k, std::pair<int, int> s,
                      std::pair<int, int> p)
@@ -513,14 +515,29 @@ struct Conv2dReluPoolOp : Conv2dOp
     {
         validate(xs);
         const Mat *b = xs.size() == 3 ? &mat(xs[2]) : nullptr;
+        if (OriginMat::conv_relu_pool_fused(mat(xs[0]), mat(xs[1]), stride, pad, pk, ps, pp))
+        {
+            // a first layer under a 2x2 pooling: one pass, relu(conv(x)) is never written
+            const Shape xs0 = xs[0].shape();
+            conv_shape      = Shape{xs0[0], mat(xs[1]).shape()[0], xs0[2], xs0[3]};
+            Tensor out      = wrap(omat(xs[0]).conv2d_relu_max_pool2d_device(mat(xs[1]), b, stride, pad, pk, ps, pp, &indices));
+            pooled          = out.impl_->data_;
+            y.reset();
+            return {out};
+        }
+        pooled.reset();
         y            = std::shared_ptr<Mat>(omat(xs[0]).conv2d_act(mat(xs[1]), b, stride, pad, 0));
         const auto *yo = dynamic_cast<const OriginMat *>(y.get());
         return {wrap(yo->max_pool2d_device(pk, ps, pp, &indices))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
-        const auto *yo = dynamic_cast<const OriginMat *>(y.get());
-        auto g0        = yo->max_pool2d_backward_relu_device(mat(gys[0]), pk, ps, pp, *indices);
+        std::unique_ptr<Mat> g0;
+        if (y)
+            g0 = dynamic_cast<const OriginMat *>(y.get())->max_pool2d_backward_relu_device(mat(gys[0]), pk, ps, pp, *indices);
+        else
+            g0 = dynamic_cast<const OriginMat *>(pooled.get())
+                     ->max_pool2d_backward_relu_pooled_device(mat(gys[0]), conv_shape, pk, ps, pp, *indices);
         const Mat *b   = inputs_.size() == 3 ? &mat(inputs_[2]) : nullptr;
         auto grads     = g0->conv2d_backward(*g0, mat(inputs_[0]), mat(inputs_[1]), b, stride, pad);
         std::vector<Tensor> out;

@@ -1888,6 +1888,65 @@ std::unique_ptr<Mat> OriginMat::max_pool2d_backward_relu_device(const Mat &gym, 
     return gx;
 }
 
+bool OriginMat::conv_relu_pool_fused(const Mat &xm, const Mat &Wm, std::pair<int, int> s, std::pair<int, int> p,
+                                     std::pair<int, int> pk, std::pair<int, int> ps, std::pair<int, int> pp)
+{
+    if (!device_f32(xm) || !device_f32(Wm) || xm.shape().size() != 4 || Wm.shape().size() != 4 || xm.shape()[1] != Wm.shape()[1])
+        return false;
+    const Shape xs = xm.shape(), ws = Wm.shape();
+    return odl_hip_conv2d_relu_max_pool2d_ok((int64_t)xs[0], (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3], (int64_t)ws[0],
+                                             (int)ws[2], (int)ws[3], s.first, s.second, p.first, p.second, pk.first, pk.second,
+                                             ps.first, ps.second, pp.first, pp.second) == 1;
+}
+
+std::unique_ptr<Mat> OriginMat::conv2d_relu_max_pool2d_device(const Mat &Wm, const Mat *bm, std::pair<int, int> s,
+                                                              std::pair<int, int> p, std::pair<int, int> pk,
+                                                              std::pair<int, int> ps, std::pair<int, int> pp,
+                                                              std::shared_ptr<Storage> *indices) const
+{
+    const OriginMat &x = dev_f32(*this, "conv2d"), &w = dev_f32(Wm, "conv2d");
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3], OC = w.shape()[0];
+    const float *bias = nullptr;
+    if (bm)
+    {
+        const OriginMat &b = dev_f32(*bm, "conv2d");
+        if (b.shape().size() != 1 || (int64_t)b.shape()[0] != OC)
+            THROW_INVALID_ARG("conv2d: b must be 1D with size {}, but got shape {}", OC, b.shape().to_string());
+        bias = fp(b);
+    }
+    auto y = new_like(x, Shape{(size_t)N, (size_t)OC, (size_t)(H / 2), (size_t)(W / 2)});
+    std::shared_ptr<Storage> idx;
+    if (indices)
+        idx = Storage::create(y->elements() * sizeof(uint64_t), DeviceType::kCUDA, device().index());
+    check(odl_hip_conv2d_relu_max_pool2d(fp(x), fp(w), bias, N, C, H, W, OC, (int)w.shape()[2], (int)w.shape()[3], s.first,
+                                         s.second, p.first, p.second, pk.first, pk.second, ps.first, ps.second, pp.first,
+                                         pp.second, y->data_ptr<float>(), idx ? static_cast<uint64_t *>(idx->data()) : nullptr,
+                                         cur()));
+    if (indices)
+        *indices = idx;
+    return y;
+}
+
+std::unique_ptr<Mat> OriginMat::max_pool2d_backward_relu_pooled_device(const Mat &gym, const Shape &input_shape,
+                                                                       std::pair<int, int> k, std::pair<int, int> s,
+                                                                       std::pair<int, int> p, const Storage &indices) const
+{
+    const OriginMat &gy = dev_f32(gym, "max_pool2d_backward");
+    const OriginMat &y  = dev_f32(*this, "max_pool2d_backward");
+    if (gy.shape().size() != 4 || input_shape.size() != 4 || !(gy.shape() == y.shape()))
+        THROW_INVALID_ARG("max_pool2d_backward: gy {} and the pooled tensor {} must be 4D of one shape", gy.shape().to_string(),
+                          y.shape().to_string());
+    if (indices.size() < gy.elements() * sizeof(uint64_t) || indices.device_type() != DeviceType::kCUDA)
+        THROW_INVALID_ARG("max_pool2d_backward: indices size mismatch. Expected {}, got {}", gy.elements(),
+                          indices.size() / sizeof(uint64_t));
+    auto gx = new_like(gy, input_shape);
+    check(odl_hip_max_pool2d_backward_relu_pooled(fp(gy), static_cast<const uint64_t *>(indices.data()), fp(y),
+                                                  (int64_t)input_shape[0], (int64_t)input_shape[1], (int64_t)input_shape[2],
+                                                  (int64_t)input_shape[3], k.first, k.second, s.first, s.second, p.first,
+                                                  p.second, gx->data_ptr<float>(), cur()));
+    return gx;
+}
+
 std::unique_ptr<Mat> OriginMat::max_pool2d_backward(const Mat &gym, std::pair<int, int> k, std::pair<int, int> s,
                                                     std::pair<int, int> p, const std::vector<size_t> &indices) const
 {

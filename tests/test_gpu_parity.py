@@ -570,6 +570,55 @@ def check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p):
     assert (np.abs(host(gb) - gbo) <= gb_bound + 1e-6).all()
 
 
+@pytest.mark.parametrize("N,C,H,W,OC,bias", [
+    (256, 1, 28, 28, 32, True),   # the CNN's first layer under its pooling
+    (3, 1, 12, 10, 16, False),
+    (2, 3, 8, 6, 16, True),       # three input channels
+    (5, 2, 2, 2, 48, True),       # one pooled pixel an image: every window cell meets the border
+])
+def test_conv_relu_pool_in_one_pass_equals_the_three_operators(api, N, C, H, W, OC, bias):
+    # Conv2d + ReLU + MaxPool2d(2) of a first layer as one kernel: pooled values and window indices must be those of
+    # conv2d_act(relu) followed by max_pool2d bit for bit, and the backward of the pooling and the ReLU taken from the
+    # pooled tensor must give the floats of the one taken from the tensor that was pooled (zeros, negative zeros and the
+    # signs of masked gradients included).
+    print("\n[case] conv + relu + pool", N, C, H, W, OC, bias, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(N + C + H + OC)
+    x = torch.randn((N, C, H, W), device="cuda", generator=g)
+    w = torch.randn((OC, C, 3, 3), device="cuda", generator=g) * 0.3
+    b = torch.randn((OC,), device="cuda", generator=g) if bias else None
+    assert api.conv2d_relu_max_pool2d_ok(x.shape, w.shape)
+    y = api.conv2d(x, w, b, 1, 1, activation="relu")
+    want, want_idx = api.max_pool2d(y, 2, 2, 0)
+    got, got_idx = api.conv2d_relu_max_pool2d(x, w, b)
+    assert torch.equal(got, want) and torch.equal(got_idx, want_idx)
+    assert torch.equal(api.conv2d_relu_max_pool2d(x, w, b, with_indices=False)[0], want)
+    gy = torch.randn(want.shape, device="cuda", generator=g)
+    gy.view(-1)[::7] = 0.0
+    gy.view(-1)[3::11] = -0.0
+    a = api.max_pool2d_backward_relu(gy, want_idx, y, 2, 2, 0)
+    bq = api.max_pool2d_backward_relu_pooled(gy, got_idx, got, y.shape, 2, 2, 0)
+    assert torch.equal(a.view(torch.int32), bq.view(torch.int32))  # the bit patterns: signed zeros count
+
+
+def test_conv_relu_pool_one_pass_is_offered_only_where_it_gives_the_same_bits(api):
+    ok = api.conv2d_relu_max_pool2d_ok
+    assert ok((4, 1, 28, 28), (32, 1, 3, 3))
+    assert not ok((4, 1, 27, 28), (32, 1, 3, 3))            # an odd extent: the pooling drops a row
+    assert not ok((4, 1, 28, 28), (24, 1, 3, 3))            # filters not in sixteens
+    assert not ok((4, 32, 14, 14), (64, 32, 3, 3))          # many channels: the matrix kernels' layer
+    assert not ok((4, 1, 28, 28), (32, 1, 3, 3), stride=2)
+    assert not ok((4, 1, 28, 28), (32, 1, 3, 3), pool_kernel=3, pool_stride=3)
+    assert not ok((4, 1, 28, 28), (32, 1, 5, 5), pad=2)
+    x = torch.zeros((4, 32, 14, 14), device="cuda")
+    w = torch.zeros((64, 32, 3, 3), device="cuda")
+    with pytest.raises(api.OdlInvalidArgument):
+        api.conv2d_relu_max_pool2d(x, w)
+    with pytest.raises(api.OdlInvalidArgument):              # overlapping windows have no pooled-mask backward
+        api.max_pool2d_backward_relu_pooled(torch.zeros((1, 1, 3, 3), device="cuda"),
+                                            torch.zeros((1, 1, 3, 3), dtype=torch.int64, device="cuda"),
+                                            torch.zeros((1, 1, 3, 3), device="cuda"), (1, 1, 7, 7), 3, 2, 0)
+
+
 @pytest.mark.parametrize("N,C,H,W,OC", [
     (5, 1, 12, 10, 16),      # one input channel: the one-pass backward
     (130, 32, 14, 14, 64),   # small images, few channels: the image-resident weight gradient
