@@ -318,6 +318,15 @@ int odl_hip_softmax_ce_loss_device(const float *x, const void *t, int idx_is_i64
                                    void *stream);
 int odl_hip_softmax_ce_grad_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
                                    const float *device_gy, float *gx, void *stream);
+/* odl_hip_softmax_ce_loss_device that also writes unit_gx[N, C], the gradient for an upstream gradient of 1 — the seed
+ * Tensor::backward() starts from (src/core/tensor_impl.cpp:94-98) — in the same launch: bit for bit what
+ * odl_hip_softmax_ce_grad(x, t, ..., 1.0f) writes (for logits without NaN), so a caller whose upstream gradient is that
+ * constant needs no second launch. For the batches odl_hip_softmax_ce_loss_grad_ok names (1 / 0): up to 2048 rows of up to
+ * 64 classes. */
+int odl_hip_softmax_ce_loss_grad_ok(int64_t N, int64_t C);
+int odl_hip_softmax_ce_loss_grad_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
+                                        float *device_loss2, void *host_mirror2, float *unit_gx, void *workspace,
+                                        size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------ pooling ------------------------- */
 /* Mat::max_pool2d / max_pool2d_backward (mat.h:560-578; src/mat/origin/cpu/pooling/max_pool2d.cpp:40-224).

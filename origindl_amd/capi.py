@@ -472,6 +472,21 @@ def softmax_cross_entropy_backward(x, t, gy=1.0):
     return gx
 
 
+def softmax_cross_entropy_with_unit_grad(x, t):
+    """Loss and the gradient for an upstream gradient of 1 in one launch (odl_hip_softmax_ce_loss_grad_device)
+    -> (loss as a python float, bad-label flag, gx); raises where the library has no such kernel."""
+    t, is64 = _ce_check(x, t)
+    N, C = x.shape
+    if lib().query("odl_hip_softmax_ce_loss_grad_ok", N, C) != 1:
+        raise OdlInvalidArgument("softmax_cross_entropy: no one-launch loss and gradient for this batch")
+    ws, nb = _ws(lib().query("odl_hip_softmax_ce_loss_workspace_bytes", N))
+    out2 = torch.zeros(2, dtype=torch.float32, device="cuda")
+    gx = _empty(x.shape)
+    lib().call("odl_hip_softmax_ce_loss_grad_device", _p(x), _p(t), is64, N, C, _p(out2), None, _p(gx), _p(ws), nb, _stream())
+    words = out2.cpu()
+    return float(words[0]), int(words.view(torch.int32)[1]), gx
+
+
 # ----------------------------------------------------------------------------------------- pooling
 def max_pool2d(x, kernel_size, stride, pad, with_indices=True):
     _chk(x, "x")

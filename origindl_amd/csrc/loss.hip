@@ -340,6 +340,82 @@ __global__ __launch_bounds__(1024) void ce_loss_small_kernel(const float *__rest
     }
 }
 
+// The same launch with the gradient for an upstream gradient of one written beside the loss — what backward() asks for
+// right after (its seed is the constant 1), so that it needs no launch of its own. Per row the gradient is the float
+// ce_grad_kernel<1> would write: that kernel spreads a row over a wave's lanes and adds the exponentials by a butterfly
+// (lane l adds lane l ^ 32, then ^ 16, ...), which is a tree of sums a thread can walk alone — lanes past the row hold
+// zeros, and adding zero is exact. CMAX: the power of two the classes fit in (the tree's empty upper levels are skipped).
+template <int CMAX>
+__global__ __launch_bounds__(1024) void ce_loss_grad_small_kernel(const float *__restrict__ x, const void *t, int is64, int N,
+                                                                  int C, unsigned int *out2, unsigned int *mirror,
+                                                                  float *__restrict__ gx, float scale)
+{
+    __shared__ float part[1024 / 64];
+    __shared__ int bad;
+    if (threadIdx.x == 0)
+        bad = 0;
+    __syncthreads();
+    float acc = 0.f;
+    for (int row = threadIdx.x; row < N; row += 1024)
+    {
+        const float *xr = x + (int64_t)row * C;
+        float m = -FLT_MAX;
+        for (int j = 0; j < C; ++j)
+            m = (m < xr[j]) ? xr[j] : m;
+        float e[CMAX];
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < CMAX; ++j)
+        {
+            e[j] = 0.f;
+            if (j < C)  // (the same in every thread)
+            {
+                e[j] = expf(xr[j] - m);
+                s += e[j];
+            }
+        }
+        const int64_t lab = label_at(t, is64, row);
+        if (lab < 0 || lab >= C)
+            bad = 1;  // every writer stores the same value
+        else
+        {
+            const float p = expf(xr[lab] - m) / s;
+            acc += logf(p + 1e-8f);
+        }
+        // the wave's sum of the exponentials
+        float tree[CMAX];
+#pragma unroll
+        for (int j = 0; j < CMAX; ++j)
+            tree[j] = e[j];
+#pragma unroll
+        for (int o = CMAX / 2; o > 0; o >>= 1)
+#pragma unroll
+            for (int l = 0; l < o; ++l)
+                tree[l] = tree[l] + tree[l + o];
+        const float sw = tree[0];
+        float *gr = gx + (int64_t)row * C;
+#pragma unroll
+        for (int j = 0; j < CMAX; ++j)
+            if (j < C)
+                gr[j] = (e[j] / sw - ((j == lab) ? 1.f : 0.f)) * scale;
+    }
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0)
+        part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        float s = 0.f;
+        for (int i = 0; i < 1024 / 64; ++i)
+            s += part[i];
+        const float loss = -s / (float)N;
+        out2[0] = __float_as_uint(loss);
+        out2[1] = bad ? 1u : 0u;
+        if (mirror)
+            mirror[0] = __float_as_uint(loss), mirror[1] = bad ? 1u : 0u;
+    }
+}
+
 // gx = (softmax(x) - one_hot(t)) * scale, one wave per row. Rows of up to 64*REGS classes stay in registers
 // between the max, the sum and the write, so the logits are read from memory once; longer rows re-read them.
 template <int REGS>
@@ -712,13 +788,31 @@ size_t odl_hip_softmax_ce_loss_workspace_bytes(int64_t N)
 
 // loss and out-of-range flag into two device words: [0] loss (float), [1] flag (int, nonzero = a bad label)
 static int ce_loss_launch(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, unsigned int *out2,
-                          unsigned int *mirror, void *workspace, size_t workspace_bytes, hipStream_t st)
+                          unsigned int *mirror, void *workspace, size_t workspace_bytes, hipStream_t st,
+                          float *unit_gx = nullptr)
 {
     ODL_REQUIRE_DEVICE();
     ODL_REQUIRE(N > 0 && C > 0, "softmax_cross_entropy: empty input");
     const size_t need = odl_hip_softmax_ce_loss_workspace_bytes(N);
     ODL_REQUIRE(workspace != nullptr && workspace_bytes >= need,
                 "softmax_cross_entropy: workspace of %zu bytes required, got %zu", need, workspace_bytes);
+    if (N <= 2048 && C <= 64 && unit_gx)
+    {
+        const float scale = 1.0f / (float)N;  // an upstream gradient of 1 over N, as ce_grad_launch forms it
+        if (C <= 16)
+            hipLaunchKernelGGL(ce_loss_grad_small_kernel<16>, dim3(1), dim3(1024), 0, st, x, t, idx_is_i64, (int)N, (int)C, out2,
+                               mirror, unit_gx, scale);
+        else if (C <= 32)
+            hipLaunchKernelGGL(ce_loss_grad_small_kernel<32>, dim3(1), dim3(1024), 0, st, x, t, idx_is_i64, (int)N, (int)C, out2,
+                               mirror, unit_gx, scale);
+        else
+            hipLaunchKernelGGL(ce_loss_grad_small_kernel<64>, dim3(1), dim3(1024), 0, st, x, t, idx_is_i64, (int)N, (int)C, out2,
+                               mirror, unit_gx, scale);
+        ODL_LAUNCH_CHECK();
+        return ODL_OK;
+    }
+    ODL_REQUIRE(unit_gx == nullptr, "softmax_cross_entropy: no one-launch loss and gradient for %lld rows of %lld classes",
+                (long long)N, (long long)C);
     if (N <= 2048 && C <= 64)
     {
         hipLaunchKernelGGL(ce_loss_small_kernel, dim3(1), dim3(1024), 0, st, x, t, idx_is_i64, (int)N, (int)C, out2,
@@ -759,6 +853,20 @@ int odl_hip_softmax_ce_loss_device(const float *x, const void *t, int idx_is_i64
     return ce_loss_launch(x, t, idx_is_i64, N, C, reinterpret_cast<unsigned int *>(device_loss2),
                           static_cast<unsigned int *>(host_mirror2), workspace,
                           workspace_bytes, odl::as_stream(stream));
+}
+
+int odl_hip_softmax_ce_loss_grad_ok(int64_t N, int64_t C)
+{
+    return (N > 0 && N <= 2048 && C > 0 && C <= 64) ? 1 : 0;
+}
+
+int odl_hip_softmax_ce_loss_grad_device(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C,
+                                        float *device_loss2, void *host_mirror2, float *unit_gx, void *workspace,
+                                        size_t workspace_bytes, void *stream)
+{
+    ODL_REQUIRE(device_loss2 != nullptr && unit_gx != nullptr, "softmax_cross_entropy: null output");
+    return ce_loss_launch(x, t, idx_is_i64, N, C, reinterpret_cast<unsigned int *>(device_loss2),
+                          static_cast<unsigned int *>(host_mirror2), workspace, workspace_bytes, odl::as_stream(stream), unit_gx);
 }
 
 int odl_hip_softmax_ce_loss(const float *x, const void *t, int idx_is_i64, int64_t N, int64_t C, float *host_loss,

@@ -410,10 +410,12 @@ public:
     // The loss and its gradient without the host round trip of the pair above: the loss stays a device scalar and the
     // upstream gradient is read from device memory. For steps recorded into a graph; an out-of-range label is not
     // reported here (the flag stays on the device).
-    std::unique_ptr<Mat> softmax_cross_entropy_device(const Mat &target) const;
+    // unit_grad (may be null): receives the gradient for an upstream gradient of 1, written by the loss's own launch where
+    // the library has such a kernel (small batches of few classes), else stays empty
+    std::unique_ptr<Mat> softmax_cross_entropy_device(const Mat &target, std::unique_ptr<Mat> *unit_grad = nullptr) const;
     // the device-resident loss, with the out-of-range-label flag read back and turned into the reference's exception
     // (one small device-to-host copy; no upload of the loss afterwards)
-    std::unique_ptr<Mat> softmax_cross_entropy_checked(const Mat &target) const;
+    std::unique_ptr<Mat> softmax_cross_entropy_checked(const Mat &target, std::unique_ptr<Mat> *unit_grad = nullptr) const;
     std::unique_ptr<Mat> softmax_cross_entropy_backward_device(const Mat &target, const Mat &gy) const;
     // include/origin/mat/origin/origin_mat.h:75: a dense copy with the dimensions in the order `dims`
     std::unique_ptr<Mat> permute(const std::vector<int> &dims) const;

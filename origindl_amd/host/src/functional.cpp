@@ -375,6 +375,9 @@ struct Softmax : Operator  // src/operators/activation/softmax.cpp:14-129
 struct SoftmaxCrossEntropy : Operator  // src/operators/loss/softmax_cross_entropy.cpp:17-111
 {
     static bool bad_label(const Tensor &loss) { return omat(loss).loss_bad_label_flag(); }
+    // the gradient for an upstream gradient of 1, when the loss's launch wrote it along (small batches of few classes):
+    // backward() starts from that constant, and then has nothing to launch here
+    std::unique_ptr<Mat> unit_grad;
     std::vector<Tensor> forward(const std::vector<Tensor> &xs) override
     {
         if (xs.size() != 2)
@@ -389,11 +392,13 @@ struct SoftmaxCrossEntropy : Operator  // src/operators/loss/softmax_cross_entro
         if (x.shape()[0] != t.shape()[0])
             THROW_INVALID_ARG("SoftmaxCrossEntropy: batch size mismatch. x has {} samples, target has {} samples",
                               x.shape()[0], t.shape()[0]);
+        unit_grad.reset();
+        std::unique_ptr<Mat> *want = x.requires_grad() ? &unit_grad : nullptr;
         if (cuda::is_capturing())  // a recorded step cannot visit the host: the loss stays where it is computed
-            return {wrap(omat(x).softmax_cross_entropy_device(mat(t)))};
+            return {wrap(omat(x).softmax_cross_entropy_device(mat(t), want))};
         // synchronises once, as the reference's .item() does, to report an out-of-range label; the loss is not sent
         // back up afterwards: it is the device scalar the kernel wrote
-        return {wrap(omat(x).softmax_cross_entropy_checked(mat(t)))};
+        return {wrap(omat(x).softmax_cross_entropy_checked(mat(t), want))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {
@@ -402,7 +407,9 @@ struct SoftmaxCrossEntropy : Operator  // src/operators/loss/softmax_cross_entro
         // the upstream gradient is read where it lies when it is a float32 device scalar (no host round trip; gy/N
         // is formed in the kernel as the host would form it)
         float seed = 0.f;
-        if (gys[0].elements() == 1 && omat(gys[0]).unwritten_constant(&seed))
+        if (gys[0].elements() == 1 && omat(gys[0]).unwritten_constant(&seed) && seed == 1.0f && unit_grad)
+            gx = std::move(unit_grad);  // written by the loss's own launch
+        else if (gys[0].elements() == 1 && omat(gys[0]).unwritten_constant(&seed))
             gx = omat(x).softmax_cross_entropy_backward(mat(t), seed);  // the ones backward() starts from: no read at all
         else if (cuda::is_capturing() || (OriginMat::device_f32(mat(gys[0])) && gys[0].elements() == 1))
             gx = omat(x).softmax_cross_entropy_backward_device(mat(t), mat(gys[0]));

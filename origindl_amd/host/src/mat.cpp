@@ -2043,7 +2043,7 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_backward(const Mat &target
     return gx;
 }
 
-std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) const
+std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target, std::unique_ptr<Mat> *unit_grad) const
 {
     const OriginMat &x = dev_f32(*this, "softmax_cross_entropy");
     const OriginMat &t = as_origin(target);
@@ -2053,8 +2053,16 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) 
     // two words: the loss, and the bad-label flag behind it; the Mat is the scalar in front
     auto storage = Storage::create(2 * sizeof(float), DeviceType::kCUDA, device().index());
     void *mirror = MirrorPool::get().take(cur());
-    check(odl_hip_softmax_ce_loss_device(fp(x), t.storage()->data(), is64, N, C, static_cast<float *>(storage->data()),
-                                         mirror, ws.ptr(), ws.bytes, cur()));
+    if (unit_grad && odl_hip_softmax_ce_loss_grad_ok(N, C) == 1)
+    {
+        auto gx = new_like(x, shape_);
+        check(odl_hip_softmax_ce_loss_grad_device(fp(x), t.storage()->data(), is64, N, C, static_cast<float *>(storage->data()),
+                                                  mirror, gx->data_ptr<float>(), ws.ptr(), ws.bytes, cur()));
+        *unit_grad = std::move(gx);
+    }
+    else
+        check(odl_hip_softmax_ce_loss_device(fp(x), t.storage()->data(), is64, N, C, static_cast<float *>(storage->data()),
+                                             mirror, ws.ptr(), ws.bytes, cur()));
     // outside a capture an event behind the kernel lets the host read the loss without waiting for the backward pass
     void *event = nullptr;
     if (!t_capturing)
@@ -2066,7 +2074,7 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_device(const Mat &target) 
     return std::make_unique<OriginMat>(std::move(storage), Shape{}, DataType::kFloat32);
 }
 
-std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target) const
+std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target, std::unique_ptr<Mat> *unit_grad) const
 {
     // labels that came up from the host carry their range: an out-of-range label is reported without asking the device,
     // and a batch in range needs no check at all (the step then has no stop in its middle)
@@ -2075,9 +2083,9 @@ std::unique_ptr<Mat> OriginMat::softmax_cross_entropy_checked(const Mat &target)
     {
         if (lo < 0 || hi >= (int64_t)shape_[1])
             THROW_INVALID_ARG("gather: index out of range [0, {})", shape_[1]);
-        return softmax_cross_entropy_device(target);
+        return softmax_cross_entropy_device(target, unit_grad);
     }
-    auto loss = softmax_cross_entropy_device(target);
+    auto loss = softmax_cross_entropy_device(target, unit_grad);
     // the loss word and the bad-label flag behind it come back together (this synchronises, as the reference's host-side
     // divide does); the loss itself stays on the device for the operators that follow
     unsigned words[2] = {0, 0};

@@ -570,6 +570,27 @@ def check_conv_case(api, o, N, C, H, W, OC, KH, KW, s, p):
     assert (np.abs(host(gb) - gbo) <= gb_bound + 1e-6).all()
 
 
+@pytest.mark.parametrize("N,C", [(512, 10), (256, 10), (2048, 64), (7, 3), (1, 1), (100, 16), (33, 17), (1500, 33), (64, 48)])
+def test_ce_loss_with_unit_gradient_in_one_launch_equals_the_two_calls(api, N, C):
+    # the loss kernel that writes the gradient for an upstream gradient of 1 along: the loss is the float of the loss call
+    # and the gradient the floats of the gradient call with gy = 1, bit for bit, for int32 and int64 labels
+    print("\n[case] ce loss + unit gradient", N, C, flush=True)
+    g = torch.Generator(device="cuda").manual_seed(N * 7 + C)
+    x = torch.randn((N, C), device="cuda", generator=g) * 3.0
+    for dt in (torch.int32, torch.int64):
+        t = torch.randint(0, C, (N,), device="cuda", generator=g).to(dt)
+        loss, bad, gx = api.softmax_cross_entropy_with_unit_grad(x, t)
+        assert bad == 0
+        want_loss = api.softmax_cross_entropy(x, t)
+        assert np.float32(loss).tobytes() == np.float32(want_loss).tobytes()
+        assert torch.equal(gx.view(torch.int32), api.softmax_cross_entropy_backward(x, t, 1.0).view(torch.int32))
+    t_bad = torch.randint(0, C, (N,), device="cuda", generator=g).to(torch.int32)
+    t_bad[N // 2] = C
+    assert api.softmax_cross_entropy_with_unit_grad(x, t_bad)[1] == 1
+    with pytest.raises(api.OdlInvalidArgument):
+        api.softmax_cross_entropy_with_unit_grad(torch.zeros((4, 65), device="cuda"), torch.zeros(4, dtype=torch.int32, device="cuda"))
+
+
 @pytest.mark.parametrize("N,C,H,W,OC,bias", [
     (256, 1, 28, 28, 32, True),   # the CNN's first layer under its pooling
     (3, 1, 12, 10, 16, False),
