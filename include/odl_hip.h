@@ -361,6 +361,18 @@ int odl_hip_conv2d_relu_max_pool2d_ok(int64_t N, int64_t C, int64_t H, int64_t W
 int odl_hip_conv2d_relu_max_pool2d(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H, int64_t W,
                                    int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int PKH, int PKW, int PSH,
                                    int PSW, int PPH, int PPW, float *y, uint64_t *idx, void *stream);
+/* The three calls above with the window-local index in one byte instead of eight (windows of at most 256 cells), for a
+ * caller that keeps the indices to itself between a fused layer's forward and backward — the host layer's Conv2d + ReLU +
+ * MaxPool2d operator: the same index values, an eighth of their bytes written and read back. odl_hip_max_pool2d_compact
+ * takes every window odl_hip_max_pool2d takes as long as the sizes fit 32 bits. */
+int odl_hip_max_pool2d_compact(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+                               int PH, int PW, float *y, uint8_t *idx8, void *stream);
+int odl_hip_max_pool2d_backward_relu_pooled_compact(const float *gy, const uint8_t *idx8, const float *y, int64_t N, int64_t C,
+                                                    int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH, int PW,
+                                                    float *gx, void *stream);
+int odl_hip_conv2d_relu_max_pool2d_compact(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H,
+                                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int PKH,
+                                           int PKW, int PSH, int PSW, int PPH, int PPW, float *y, uint8_t *idx8, void *stream);
 
 /* ------------------------------------------------------------------ metrics ------------------------- */
 /* argmax per row, first maximum (src/utils/metrics.cpp:40-53), and accuracy() (metrics.cpp:11-70) with

@@ -521,9 +521,26 @@ def conv2d_relu_max_pool2d(x, w, b=None, stride=1, pad=1, pool_kernel=2, pool_st
     (SH, SW), (PH, PW) = _pair(stride), _pair(pad)
     (PKH, PKW), (PSH, PSW), (PPH, PPW) = _pair(pool_kernel), _pair(pool_stride), _pair(pool_pad)
     y = _empty((N, OC, H // 2, W // 2))
+    if with_indices == "bytes":
+        idx = torch.empty(y.shape, dtype=torch.uint8, device="cuda")
+        lib().call("odl_hip_conv2d_relu_max_pool2d_compact", _p(x), _p(w), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, PKH,
+                   PKW, PSH, PSW, PPH, PPW, _p(y), _p(idx), _stream())
+        return y, idx
     idx = torch.empty(y.shape, dtype=torch.int64, device="cuda") if with_indices else None  # uint64 bit pattern
     lib().call("odl_hip_conv2d_relu_max_pool2d", _p(x), _p(w), _p(b), N, C, H, W, OC, KH, KW, SH, SW, PH, PW, PKH, PKW, PSH, PSW,
                PPH, PPW, _p(y), _p(idx), _stream())
+    return y, idx
+
+
+def max_pool2d_compact(x, kernel_size, stride, pad):
+    """max_pool2d with the window-local indices as bytes (odl_hip_max_pool2d_compact) -> (y, idx uint8)."""
+    _chk(x, "x")
+    (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
+    N, C, H, W = x.shape
+    OH, OW = conv_outsize(H, KH, SH, PH), conv_outsize(W, KW, SW, PW)
+    y = _empty((N, C, _builtins.max(OH, 0), _builtins.max(OW, 0)))
+    idx = torch.empty(y.shape, dtype=torch.uint8, device="cuda")
+    lib().call("odl_hip_max_pool2d_compact", _p(x), N, C, H, W, KH, KW, SH, SW, PH, PW, _p(y), _p(idx), _stream())
     return y, idx
 
 
@@ -543,8 +560,8 @@ def max_pool2d_backward_relu_pooled(gy, idx, y, input_shape, kernel_size, stride
     (KH, KW), (SH, SW), (PH, PW) = _pair(kernel_size), _pair(stride), _pair(pad)
     N, C, H, W = [int(v) for v in input_shape]
     gx = _empty((N, C, H, W))
-    lib().call("odl_hip_max_pool2d_backward_relu_pooled", _p(gy), _p(idx), _p(y), N, C, H, W, KH, KW, SH, SW, PH, PW, _p(gx),
-               _stream())
+    name = "odl_hip_max_pool2d_backward_relu_pooled_compact" if idx.dtype == torch.uint8 else "odl_hip_max_pool2d_backward_relu_pooled"
+    lib().call(name, _p(gy), _p(idx), _p(y), N, C, H, W, KH, KW, SH, SW, PH, PW, _p(gx), _stream())
     return gx
 
 

@@ -63,8 +63,8 @@ size_t conv_patch_dgrad_workspace(int64_t N, int64_t C, int64_t H, int64_t W, in
 int conv_patch_dgrad(const float *gy, const float *w, float *gx, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
                      void *workspace, size_t workspace_bytes, hipStream_t st, bool packed);
 SidePack conv_patch_dgrad_pack(const float *w, int64_t C, int64_t OC, void *workspace);
-int conv_small_forward_pool(const float *x, const float *w, const float *b, float *y, uint64_t *idx, int64_t N, int64_t C,
-                            int64_t H, int64_t W, int64_t OC, int act, hipStream_t st);
+int conv_small_forward_pool(const float *x, const float *w, const float *b, float *y, uint64_t *idx, uint8_t *idx8, int64_t N,
+                            int64_t C, int64_t H, int64_t W, int64_t OC, int act, hipStream_t st);
 bool conv_small_wgrad_ok(const float *gy, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int64_t OH,
                          int64_t OW);
 size_t conv_small_wgrad_workspace(int64_t N, int64_t C, int64_t OC, int KH, int KW, int64_t OH, int64_t OW);
@@ -1324,7 +1324,19 @@ int odl_hip_conv2d_relu_max_pool2d(const float *x, const float *w, const float *
     if (!odl_hip_conv2d_relu_max_pool2d_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, PKH, PKW, PSH, PSW, PPH, PPW))
         return odl::fail(ODL_ERR_INVALID_ARG, "conv2d_relu_max_pool2d: this layer pair has no one-pass kernel (ask "
                                               "odl_hip_conv2d_relu_max_pool2d_ok first)");
-    return odl::conv_small_forward_pool(x, w, b, y, idx, N, C, H, W, OC, /*relu*/ 1, odl::as_stream(stream));
+    return odl::conv_small_forward_pool(x, w, b, y, idx, nullptr, N, C, H, W, OC, /*relu*/ 1, odl::as_stream(stream));
+}
+
+int odl_hip_conv2d_relu_max_pool2d_compact(const float *x, const float *w, const float *b, int64_t N, int64_t C, int64_t H,
+                                           int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW, int PKH,
+                                           int PKW, int PSH, int PSW, int PPH, int PPW, float *y, uint8_t *idx8, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(x != nullptr && w != nullptr && y != nullptr && idx8 != nullptr, "conv2d_relu_max_pool2d: null tensor");
+    if (!odl_hip_conv2d_relu_max_pool2d_ok(N, C, H, W, OC, KH, KW, SH, SW, PH, PW, PKH, PKW, PSH, PSW, PPH, PPW))
+        return odl::fail(ODL_ERR_INVALID_ARG, "conv2d_relu_max_pool2d: this layer pair has no one-pass kernel (ask "
+                                              "odl_hip_conv2d_relu_max_pool2d_ok first)");
+    return odl::conv_small_forward_pool(x, w, b, y, nullptr, idx8, N, C, H, W, OC, /*relu*/ 1, odl::as_stream(stream));
 }
 
 int odl_hip_set_conv_direct(int enabled)

@@ -93,10 +93,10 @@ __global__ __launch_bounds__(kThreads) void conv_small_fwd_kernel(const float *_
 // convolution output the terms are added in the order of conv_small_fwd_kernel, and the window is compared in the order
 // of the pooling kernels (row-major, a later cell wins only when it is greater, max_pool2d.cpp:110-139): the pooled
 // values and indices are those of the two kernels run one after the other — without the 4x larger tensor between them.
-template <int OCB>
+template <int OCB, typename IdxT>
 __global__ __launch_bounds__(kThreads) void conv_small_fwd_pool_kernel(const float *__restrict__ x, const float *__restrict__ w,
                                                                       const float *__restrict__ bias, float *__restrict__ y,
-                                                                      uint64_t *__restrict__ idx, SmallGeom g, int act)
+                                                                      IdxT *__restrict__ idx, SmallGeom g, int act)
 {
     // (g.OH, g.OW: the pooled extents; g.total = N * OH * OW)
     const unsigned pix = blockIdx.x * kThreads + threadIdx.x;
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(kThreads) void conv_small_fwd_pool_kernel(const flo
             m = v[3], win = 3;
         y[at + o * plane] = m;
         if (idx)
-            idx[at + o * plane] = (uint64_t)win;
+            idx[at + o * plane] = (IdxT)win;
     }
 }
 
@@ -694,13 +694,17 @@ int conv_small_forward(const float *x, const float *w, const float *b, float *y,
 }
 
 // 3x3 / stride 1 / padding 1 + activation + 2x2 / stride 2 pooling, H and W even; y [N, OC, H/2, W/2], idx may be null
-int conv_small_forward_pool(const float *x, const float *w, const float *b, float *y, uint64_t *idx, int64_t N, int64_t C,
-                            int64_t H, int64_t W, int64_t OC, int act, hipStream_t st)
+// (idx: 8-byte indices, or idx8: one byte each, or neither)
+int conv_small_forward_pool(const float *x, const float *w, const float *b, float *y, uint64_t *idx, uint8_t *idx8, int64_t N,
+                            int64_t C, int64_t H, int64_t W, int64_t OC, int act, hipStream_t st)
 {
     SmallGeom g = make_small(N, C, H, W, OC, 1, 1, 1, 1, H / 2, W / 2, false);
     // four channels a thread: eight times the pooled pixels in threads, enough waves to hide each other's filter loads
     const dim3 grid((unsigned)ceil_div(g.total, kThreads), (unsigned)(OC / 4));
-    hipLaunchKernelGGL((conv_small_fwd_pool_kernel<4>), grid, dim3(kThreads), 0, st, x, w, b, y, idx, g, act);
+    if (idx8)
+        hipLaunchKernelGGL((conv_small_fwd_pool_kernel<4, uint8_t>), grid, dim3(kThreads), 0, st, x, w, b, y, idx8, g, act);
+    else
+        hipLaunchKernelGGL((conv_small_fwd_pool_kernel<4, uint64_t>), grid, dim3(kThreads), 0, st, x, w, b, y, idx, g, act);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

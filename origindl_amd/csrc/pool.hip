@@ -84,9 +84,9 @@ __global__ void max_pool_bwd_kernel(const float *__restrict__ gy, const uint64_t
 // The same two kernels with 32-bit index arithmetic and (for the usual windows)
 // kernel size and stride fixed at compile time: on a 64-wide wave the 64-bit divisions and modulos of the general
 // kernels above cost several times the memory traffic they serve.
-template <int CK, int CS>
-__global__ __launch_bounds__(256) void max_pool_fwd_plane_kernel(const float *__restrict__ x, float *__restrict__ y,
-                                                                 uint64_t *__restrict__ idx, PoolGeom g)
+template <int CK, int CS, typename IdxT>
+__device__ inline void max_pool_fwd_plane_body(const float *__restrict__ x, float *__restrict__ y, IdxT *__restrict__ idx,
+                                               const PoolGeom &g)
 {
     const int KH = CK > 0 ? CK : g.KH, KW = CK > 0 ? CK : g.KW;
     const int SH = CS > 0 ? CS : g.SH, SW = CS > 0 ? CS : g.SW;
@@ -122,8 +122,24 @@ __global__ __launch_bounds__(256) void max_pool_fwd_plane_kernel(const float *__
         }
         y[t] = mv;
         if (idx)
-            idx[t] = (uint64_t)mi;
+            idx[t] = (IdxT)mi;
     }
+}
+
+template <int CK, int CS>
+__global__ __launch_bounds__(256) void max_pool_fwd_plane_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                 uint64_t *__restrict__ idx, PoolGeom g)
+{
+    max_pool_fwd_plane_body<CK, CS, uint64_t>(x, y, idx, g);
+}
+
+// The same with the window-local index in a byte (windows of up to 256 cells): for callers that keep the indices to
+// themselves — a fused layer's backward — an eighth of the index bytes written here and read back there.
+template <int CK, int CS>
+__global__ __launch_bounds__(256) void max_pool_fwd_plane_u8_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                    uint8_t *__restrict__ idx, PoolGeom g)
+{
+    max_pool_fwd_plane_body<CK, CS, uint8_t>(x, y, idx, g);
 }
 
 template <int CK, int CS>
@@ -373,9 +389,9 @@ __global__ __launch_bounds__(256) void max_pool_bwd_tiled_relu_kernel(const floa
 // The same from the pooled tensor y alone: the cell that receives the gradient is the window's maximum, whose value is
 // y[o], so (x > 0) there is (y[o] > 0); every other cell gets the +0 it gets above. The input of the pooling is not
 // read (and need not exist any more: conv_small.hip's one-pass convolution + ReLU + pooling never writes it).
-template <int K>
+template <int K, typename IdxT>
 __global__ __launch_bounds__(256) void max_pool_bwd_tiled_relu_pooled_kernel(const float *__restrict__ gy,
-                                                                             const uint64_t *__restrict__ idx,
+                                                                             const IdxT *__restrict__ idx,
                                                                              const float *__restrict__ y, float *__restrict__ gx,
                                                                              unsigned total, int OW, unsigned oplane)
 {
@@ -711,9 +727,11 @@ int odl_hip_max_pool2d_backward_relu(const float *gy, const uint64_t *idx, const
     return ODL_OK;
 }
 
-int odl_hip_max_pool2d_backward_relu_pooled(const float *gy, const uint64_t *idx, const float *y, int64_t N, int64_t C,
-                                            int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH, int PW, float *gx,
-                                            void *stream)
+}  // extern "C"
+
+template <typename IdxT>
+static int pool_backward_relu_pooled(const float *gy, const IdxT *idx, const float *y, int64_t N, int64_t C, int64_t H, int64_t W,
+                                     int KH, int KW, int SH, int SW, int PH, int PW, float *gx, void *stream)
 {
     ODL_REQUIRE_DEVICE();
     PoolGeom g;
@@ -730,11 +748,46 @@ int odl_hip_max_pool2d_backward_relu_pooled(const float *gy, const uint64_t *idx
     const dim3 grid((unsigned)odl::ceil_div((int64_t)outputs, 256));
     hipStream_t st = odl::as_stream(stream);
     if (g.KH == 2)
-        hipLaunchKernelGGL((max_pool_bwd_tiled_relu_pooled_kernel<2>), grid, dim3(256), 0, st, gy, idx, y, gx, outputs, (int)g.OW,
-                           (unsigned)(g.OH * g.OW));
+        hipLaunchKernelGGL((max_pool_bwd_tiled_relu_pooled_kernel<2, IdxT>), grid, dim3(256), 0, st, gy, idx, y, gx, outputs,
+                           (int)g.OW, (unsigned)(g.OH * g.OW));
     else
-        hipLaunchKernelGGL((max_pool_bwd_tiled_relu_pooled_kernel<3>), grid, dim3(256), 0, st, gy, idx, y, gx, outputs, (int)g.OW,
-                           (unsigned)(g.OH * g.OW));
+        hipLaunchKernelGGL((max_pool_bwd_tiled_relu_pooled_kernel<3, IdxT>), grid, dim3(256), 0, st, gy, idx, y, gx, outputs,
+                           (int)g.OW, (unsigned)(g.OH * g.OW));
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+extern "C" {
+
+int odl_hip_max_pool2d_backward_relu_pooled(const float *gy, const uint64_t *idx, const float *y, int64_t N, int64_t C,
+                                            int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH, int PW, float *gx,
+                                            void *stream)
+{
+    return pool_backward_relu_pooled<uint64_t>(gy, idx, y, N, C, H, W, KH, KW, SH, SW, PH, PW, gx, stream);
+}
+
+int odl_hip_max_pool2d_backward_relu_pooled_compact(const float *gy, const uint8_t *idx8, const float *y, int64_t N, int64_t C,
+                                                    int64_t H, int64_t W, int KH, int KW, int SH, int SW, int PH, int PW,
+                                                    float *gx, void *stream)
+{
+    return pool_backward_relu_pooled<uint8_t>(gy, idx8, y, N, C, H, W, KH, KW, SH, SW, PH, PW, gx, stream);
+}
+
+int odl_hip_max_pool2d_compact(const float *x, int64_t N, int64_t C, int64_t H, int64_t W, int KH, int KW, int SH, int SW,
+                               int PH, int PW, float *y, uint8_t *idx8, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    PoolGeom g;
+    int rc = make_geom(g, "max_pool2d", N, C, H, W, KH, KW, SH, SW, PH, PW);
+    if (rc != ODL_OK)
+        return rc;
+    ODL_REQUIRE(x != nullptr && y != nullptr && idx8 != nullptr, "max_pool2d_compact: null tensor");
+    ODL_REQUIRE((int64_t)KH * KW <= 256 && plane_ok(g), "max_pool2d_compact: a window of at most 256 cells and 32-bit sizes");
+    if (N * C * g.OH * g.OW == 0)
+        return ODL_OK;
+    hipStream_t st = odl::as_stream(stream);
+    const dim3 grid = plane_grid(g.OH * g.OW, N * C);
+    ODL_POOL_DISPATCH(max_pool_fwd_plane_u8_kernel, x, y, idx8, g);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

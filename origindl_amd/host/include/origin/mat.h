@@ -503,9 +503,12 @@ public:
     // the ReLU from the pooled tensor alone (this = the pooled tensor, input_shape = the shape of the convolution's output)
     static bool conv_relu_pool_fused(const Mat &x, const Mat &W, std::pair<int, int> s, std::pair<int, int> p,
                                      std::pair<int, int> pk, std::pair<int, int> ps, std::pair<int, int> pp);
+    // (the indices of these three are one byte each: they never leave the operator that asks for them)
     std::unique_ptr<Mat> conv2d_relu_max_pool2d_device(const Mat &W, const Mat *b, std::pair<int, int> s, std::pair<int, int> p,
                                                        std::pair<int, int> pk, std::pair<int, int> ps, std::pair<int, int> pp,
                                                        std::shared_ptr<Storage> *indices) const;
+    std::unique_ptr<Mat> max_pool2d_device_compact(std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
+                                                   std::shared_ptr<Storage> *indices) const;
     std::unique_ptr<Mat> max_pool2d_backward_relu_pooled_device(const Mat &gy, const Shape &input_shape, std::pair<int, int> k,
                                                                 std::pair<int, int> s, std::pair<int, int> p,
                                                                 const Storage &indices) const;

@@ -535,20 +535,22 @@ struct Conv2dReluPoolOp : Conv2dOp
         pooled.reset();
         y            = std::shared_ptr<Mat>(omat(xs[0]).conv2d_act(mat(xs[1]), b, stride, pad, 0));
         const auto *yo = dynamic_cast<const OriginMat *>(y.get());
-        Tensor out     = wrap(yo->max_pool2d_device(pk, ps, pp, &indices));
         // windows that tile the image (2x2/2, 3x3/3, no padding): the backward's mask can come from the pooled tensor, a
-        // quarter or a ninth of the reads, and relu(conv(x)) need not be kept until then
+        // quarter or a ninth of the reads, relu(conv(x)) need not be kept until then, and the indices — which never leave
+        // this operator — are kept as bytes
         const Shape ys = y->shape();
         const bool tiles = y->dtype() == DataType::kFloat32 && pk.first == pk.second && (pk.first == 2 || pk.first == 3) &&
                            ps == pk && pp.first == 0 && pp.second == 0 && ys[2] % pk.first == 0 && ys[3] % pk.second == 0 &&
-                           ys[2] > 0 && ys[3] > 0;
+                           ys[2] > 0 && ys[3] > 0 && ys.elements() < (size_t(1) << 31) - 256;
         if (tiles)
         {
+            Tensor out = wrap(yo->max_pool2d_device_compact(pk, ps, pp, &indices));
             conv_shape = ys;
             pooled     = out.impl_->data_;
             y.reset();
+            return {out};
         }
-        return {out};
+        return {wrap(yo->max_pool2d_device(pk, ps, pp, &indices))};
     }
     std::vector<Tensor> backward(const std::vector<Tensor> &gys) override
     {

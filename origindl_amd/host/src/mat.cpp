@@ -1917,13 +1917,18 @@ std::unique_ptr<Mat> OriginMat::conv2d_relu_max_pool2d_device(const Mat &Wm, con
     auto y = new_like(x, Shape{(size_t)N, (size_t)OC, (size_t)(H / 2), (size_t)(W / 2)});
     std::shared_ptr<Storage> idx;
     if (indices)
-        idx = Storage::create(y->elements() * sizeof(uint64_t), DeviceType::kCUDA, device().index());
-    check(odl_hip_conv2d_relu_max_pool2d(fp(x), fp(w), bias, N, C, H, W, OC, (int)w.shape()[2], (int)w.shape()[3], s.first,
-                                         s.second, p.first, p.second, pk.first, pk.second, ps.first, ps.second, pp.first,
-                                         pp.second, y->data_ptr<float>(), idx ? static_cast<uint64_t *>(idx->data()) : nullptr,
-                                         cur()));
-    if (indices)
+    {
+        idx = Storage::create(y->elements() * sizeof(uint8_t), DeviceType::kCUDA, device().index());
+        check(odl_hip_conv2d_relu_max_pool2d_compact(fp(x), fp(w), bias, N, C, H, W, OC, (int)w.shape()[2], (int)w.shape()[3],
+                                                     s.first, s.second, p.first, p.second, pk.first, pk.second, ps.first,
+                                                     ps.second, pp.first, pp.second, y->data_ptr<float>(),
+                                                     static_cast<uint8_t *>(idx->data()), cur()));
         *indices = idx;
+    }
+    else
+        check(odl_hip_conv2d_relu_max_pool2d(fp(x), fp(w), bias, N, C, H, W, OC, (int)w.shape()[2], (int)w.shape()[3], s.first,
+                                             s.second, p.first, p.second, pk.first, pk.second, ps.first, ps.second, pp.first,
+                                             pp.second, y->data_ptr<float>(), nullptr, cur()));
     return y;
 }
 
@@ -1936,15 +1941,33 @@ std::unique_ptr<Mat> OriginMat::max_pool2d_backward_relu_pooled_device(const Mat
     if (gy.shape().size() != 4 || input_shape.size() != 4 || !(gy.shape() == y.shape()))
         THROW_INVALID_ARG("max_pool2d_backward: gy {} and the pooled tensor {} must be 4D of one shape", gy.shape().to_string(),
                           y.shape().to_string());
-    if (indices.size() < gy.elements() * sizeof(uint64_t) || indices.device_type() != DeviceType::kCUDA)
-        THROW_INVALID_ARG("max_pool2d_backward: indices size mismatch. Expected {}, got {}", gy.elements(),
-                          indices.size() / sizeof(uint64_t));
+    if (indices.size() < gy.elements() * sizeof(uint8_t) || indices.device_type() != DeviceType::kCUDA)
+        THROW_INVALID_ARG("max_pool2d_backward: indices size mismatch. Expected {}, got {}", gy.elements(), indices.size());
     auto gx = new_like(gy, input_shape);
-    check(odl_hip_max_pool2d_backward_relu_pooled(fp(gy), static_cast<const uint64_t *>(indices.data()), fp(y),
-                                                  (int64_t)input_shape[0], (int64_t)input_shape[1], (int64_t)input_shape[2],
-                                                  (int64_t)input_shape[3], k.first, k.second, s.first, s.second, p.first,
-                                                  p.second, gx->data_ptr<float>(), cur()));
+    check(odl_hip_max_pool2d_backward_relu_pooled_compact(fp(gy), static_cast<const uint8_t *>(indices.data()), fp(y),
+                                                          (int64_t)input_shape[0], (int64_t)input_shape[1],
+                                                          (int64_t)input_shape[2], (int64_t)input_shape[3], k.first, k.second,
+                                                          s.first, s.second, p.first, p.second, gx->data_ptr<float>(), cur()));
     return gx;
+}
+
+std::unique_ptr<Mat> OriginMat::max_pool2d_device_compact(std::pair<int, int> k, std::pair<int, int> s, std::pair<int, int> p,
+                                                          std::shared_ptr<Storage> *indices) const
+{
+    const OriginMat &x = dev_f32(*this, "max_pool2d");
+    if (shape_.size() != 4)
+        THROW_INVALID_ARG("max_pool2d: x must be 4D (N, C, H, W), but got shape {}", shape_.to_string());
+    const int64_t N = shape_[0], C = shape_[1], H = shape_[2], W = shape_[3];
+    const int OH = get_conv_outsize((int)H, k.first, s.first, p.first);
+    const int OW = get_conv_outsize((int)W, k.second, s.second, p.second);
+    if (OH <= 0 || OW <= 0)
+        THROW_INVALID_ARG("max_pool2d: invalid output size OH={}, OW={} for input H={}, W={}", OH, OW, H, W);
+    auto y   = new_like(x, Shape{(size_t)N, (size_t)C, (size_t)OH, (size_t)OW});
+    auto idx = Storage::create(y->elements() * sizeof(uint8_t), DeviceType::kCUDA, device().index());
+    check(odl_hip_max_pool2d_compact(fp(x), N, C, H, W, k.first, k.second, s.first, s.second, p.first, p.second,
+                                     y->data_ptr<float>(), static_cast<uint8_t *>(idx->data()), cur()));
+    *indices = idx;
+    return y;
 }
 
 std::unique_ptr<Mat> OriginMat::max_pool2d_backward(const Mat &gym, std::pair<int, int> k, std::pair<int, int> s,

@@ -619,6 +619,23 @@ def test_conv_relu_pool_in_one_pass_equals_the_three_operators(api, N, C, H, W, 
     a = api.max_pool2d_backward_relu(gy, want_idx, y, 2, 2, 0)
     bq = api.max_pool2d_backward_relu_pooled(gy, got_idx, got, y.shape, 2, 2, 0)
     assert torch.equal(a.view(torch.int32), bq.view(torch.int32))  # the bit patterns: signed zeros count
+    # the same with the indices kept as bytes (what the host layer's fused operator does): equal index values, equal floats
+    got8, idx8 = api.conv2d_relu_max_pool2d(x, w, b, with_indices="bytes")
+    assert torch.equal(got8, want) and torch.equal(idx8.to(torch.int64), want_idx)
+    y8, i8 = api.max_pool2d_compact(y, 2, 2, 0)
+    assert torch.equal(y8, want) and torch.equal(i8.to(torch.int64), want_idx)
+    c8 = api.max_pool2d_backward_relu_pooled(gy, idx8, got8, y.shape, 2, 2, 0)
+    assert torch.equal(a.view(torch.int32), c8.view(torch.int32))
+
+
+@pytest.mark.parametrize("shape,k,st,p", [((3, 5, 9, 11), 3, 2, 1), ((2, 4, 12, 12), 3, 3, 0), ((2, 3, 10, 10), 5, 1, 2),
+                                          ((1, 2, 7, 9), (2, 3), (2, 1), (0, 1))])
+def test_max_pool_with_byte_indices_equals_the_eight_byte_ones(api, shape, k, st, p):
+    g = torch.Generator(device="cuda").manual_seed(sum(shape))
+    x = torch.randn(shape, device="cuda", generator=g)
+    y, idx = api.max_pool2d(x, k, st, p)
+    y8, idx8 = api.max_pool2d_compact(x, k, st, p)
+    assert torch.equal(y, y8) and torch.equal(idx, idx8.to(torch.int64))
 
 
 def test_conv_relu_pool_one_pass_is_offered_only_where_it_gives_the_same_bits(api):
