@@ -1021,7 +1021,9 @@ int pick_splits(int64_t M, int64_t N, int64_t K, int requested)
     const int tile      = pick_tile(M, N);
     const int64_t tiles = odl::ceil_div(M, tile) * odl::ceil_div(N, tile);
     const int64_t kt    = odl::ceil_div(K, kBK);
-    if (tiles >= odl::device_cus() || kt < 8)
+    // (a K of under 256 is a handful of slabs: slicing it saves less than the launch that adds the slices up costs —
+    // 256x3136x128, the CNN's hidden layer's input gradient: two slices 7.5 + 4.1 us)
+    if (tiles >= odl::device_cus() || kt < 16)
         return 1;
     int64_t s = odl::ceil_div(2 * odl::device_cus(), tiles);
     if (s > kt / 4)
