@@ -39,9 +39,10 @@ struct ImageGeom
     odl::FastDiv by_oc, by_p, by_w, by_cols;
 };
 
+// (time stamps of a workgroup's phases for a test harness that includes this file with ODL_IMAGE_DBG defined; nothing otherwise)
 #ifdef ODL_IMAGE_DBG
 __device__ unsigned long long g_image_dbg[256 * 16];
-#define ODL_IMAGE_STAMP(i) do { if (threadIdx.x == 0) g_image_dbg[blockIdx.x * 16 + (i)] = wall_clock64(); } while (0)
+#define ODL_IMAGE_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < 256) g_image_dbg[blockIdx.x * 16 + (i)] = wall_clock64(); } while (0)
 #else
 #define ODL_IMAGE_STAMP(i) do { } while (0)
 #endif

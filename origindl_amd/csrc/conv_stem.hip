@@ -28,9 +28,10 @@ struct StemGeom
     int N, H, W, P;    // P = H*W
 };
 
+// (time stamps of a workgroup's phases for a test harness that includes this file with ODL_STEM_DBG defined; nothing otherwise)
 #ifdef ODL_STEM_DBG
 __device__ unsigned long long g_stem_dbg[256 * 16];
-#define ODL_STEM_STAMP(i) do { if (threadIdx.x == 0) g_stem_dbg[blockIdx.x * 16 + (i)] = wall_clock64(); } while (0)
+#define ODL_STEM_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < 256) g_stem_dbg[blockIdx.x * 16 + (i)] = wall_clock64(); } while (0)
 #else
 #define ODL_STEM_STAMP(i) do { } while (0)
 #endif
