@@ -87,6 +87,193 @@ __global__ __launch_bounds__(kThreads) void conv_small_fwd_kernel(const float *_
     }
 }
 
+// A detector's stem — 6x6 / stride 2 / padding 2 over C input channels into 16 filters (YOLOv5's first layer,
+// [N,3,H,W] -> [N,16,H/2,W/2]) — on the matrix cores. As a thread-per-pixel kernel it was 216 bounds-tested loads and
+// 3456 multiply-adds in a row per thread (31 us at [4,3,320,320]). Here a workgroup takes one output row: the six input
+// rows under it, with their zero borders, go to LDS once in whole-row loads, and y[oc][pixel] = sum_k w[oc][k] *
+// patch[k][pixel] runs as 16x16x4 MFMAs over tiles of sixteen pixels — A, the filter, sits in registers for the whole
+// kernel (C*9 steps of four k), B is one LDS read a step at an offset that is constant per lane and step plus twice the
+// pixel. Rows of D are filters and columns pixels, so the stores are runs of sixteen pixels of one filter's plane.
+#ifdef ODL_STEM6_DBG
+__device__ unsigned long long g_stem6_dbg[1024 * 8];
+#define ODL_STEM6_STAMP(i) do { if (threadIdx.x == 0 && blockIdx.x < 1024) g_stem6_dbg[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
+#else
+#define ODL_STEM6_STAMP(i) do { } while (0)
+#endif
+template <int C>
+__global__ __launch_bounds__(kThreads) void conv_stem6_mfma_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                                  const float *__restrict__ bias, float *__restrict__ y, int H,
+                                                                  int W, int OH, int OW, int pitch, int act)
+{
+    constexpr int STEPS = C * 9;  // of four k = (c, kh, kw) each
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) float rows[];  // [C][6][pitch]: input columns -2 .. W+1 of six rows
+    const int n = blockIdx.x / OH, oh = blockIdx.x - n * OH;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, j = lane & 15, kq = lane >> 4;
+    ODL_STEM6_STAMP(0);
+    // the lane's four filters' biases, asked for now (a load in the epilogue is a trip to memory in the way of the stores)
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias)
+    {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            bv[r] = bias[4 * kq + r];
+    }
+    // the filter: lane (j, kq) holds w[j][4s + kq] for every step s
+    // (through LDS: read where it lies, every lane's 27 values are 27 loads of 64 scattered addresses a wave — more time
+    // in the address unit than the whole product takes on the matrix cores)
+    float *wl = rows + ((C * 6 * pitch + 3) & ~3);  // [16][C*36] (on a 16-byte boundary, and so is what follows it)
+    for (int e = t; e < 16 * C * 36; e += kThreads)
+        wl[e] = w[e];
+    int koff[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+    {
+        const int k = 4 * s + kq, c = k / 36, r = k - c * 36, kh = r / 6, kw = r - kh * 6;
+        koff[s] = (c * 6 + kh) * pitch + kw;
+    }
+    ODL_STEM6_STAMP(1);
+    // the six input rows: 2*oh - 2 .. 2*oh + 3 of each channel, zeros outside the image. All of a thread's loads are in
+    // flight together (one after the other, each waiting for the last, they were most of the kernel's time): 16-byte
+    // pieces where the rows allow it.
+    if (W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0)
+    {
+        const int quads = W / 4, total = C * 6 * quads;
+        constexpr int U = 6;
+        for (int e0 = t; e0 < total; e0 += U * kThreads)
+        {
+            f32x4 v[U];
+            int at[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+            {
+                const int e = e0 + u * kThreads, ec = e < total ? e : e0;
+                const int cr = ec / quads, q = ec - cr * quads, c = cr / 6, r = cr - c * 6;
+                const int ih = 2 * oh - 2 + r;
+                const bool in = e < total && (unsigned)ih < (unsigned)H;
+                v[u] = *reinterpret_cast<const f32x4 *>(x + ((size_t)(n * C + c) * H + (in ? ih : 0)) * W + 4 * q);
+                if (!in)
+                    v[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+                at[u] = e < total ? cr * pitch + 2 + 4 * q : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (at[u] >= 0)
+                {
+                    float *d = rows + at[u];
+                    d[0] = v[u][0], d[1] = v[u][1], d[2] = v[u][2], d[3] = v[u][3];
+                }
+        }
+        for (int e = t; e < C * 6 * 4; e += kThreads)  // the two border columns on either side
+        {
+            const int cr = e >> 2, b = e & 3;
+            rows[cr * pitch + (b < 2 ? b : W + b)] = 0.f;
+        }
+    }
+    else
+    {
+#pragma unroll 8
+        for (int e = t; e < C * 6 * pitch; e += kThreads)
+        {
+            const int cr = e / pitch, col = e - cr * pitch, c = cr / 6, r = cr - c * 6;
+            const int ih = 2 * oh - 2 + r, iw = col - 2;
+            const bool in = (unsigned)ih < (unsigned)H && (unsigned)iw < (unsigned)W;
+            rows[e] = in ? x[((size_t)(n * C + c) * H + ih) * W + iw] : 0.f;
+        }
+    }
+    __syncthreads();
+    float aw[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+        aw[s] = wl[j * (C * 36) + 4 * s + kq];
+    ODL_STEM6_STAMP(2);
+    const int tiles = (OW + 15) / 16;
+    constexpr int kWavesHere = kThreads / 64;
+    // A wave takes every fourth tile, starting from a tile that turns with the workgroup (the waves with one tile more
+    // than the others then fall on different SIMDs from one workgroup of a compute unit to the next), two tiles at a time
+    // where it has two: the MFMAs of one accumulator wait for each other, those of two take turns.
+    // The finished tiles meet in LDS (behind the rows and the filter) and leave as whole rows of one filter's plane: stored
+    // from the registers every instruction wrote four 64-byte pieces of four planes, and the stores took twice the time
+    // of the products.
+    float *outs = wl + 16 * C * 36;  // [16][opitch]
+    const int opitch = ((OW + 3) / 4 * 4) | 4;  // (4 mod 8: the four filters of a lane's store fall into different banks)
+    auto store_tile = [&](int pix, const f32x4 &acc) {
+        if (pix < OW)
+        {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+                const int oc = 4 * kq + r;
+                float v = acc[r];
+                if (bias)
+                    v = v + bv[r];
+                outs[oc * opitch + pix] = odl::apply_act(v, act);
+            }
+        }
+    };
+    const int first = (wave + (int)blockIdx.x) % kWavesHere;
+    for (int tile = first; tile < tiles; tile += 2 * kWavesHere)
+    {
+        const int tile1 = tile + kWavesHere;
+        const int pix0 = tile * 16 + j, pix1 = tile1 * 16 + j;
+        const float *bp0 = rows + 2 * (pix0 < OW ? pix0 : OW - 1);  // (pixels past the row compute a copy that is not stored)
+        f32x4 acc0 = {0.f, 0.f, 0.f, 0.f};
+        if (tile1 < tiles)
+        {
+            const float *bp1 = rows + 2 * (pix1 < OW ? pix1 : OW - 1);
+            f32x4 acc1 = {0.f, 0.f, 0.f, 0.f};
+            // every B operand of the pair asked for before the first MFMA: the reads' latency is paid once, not once a batch
+            float b0[STEPS], b1[STEPS];
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+                b0[s] = bp0[koff[s]], b1[s] = bp1[koff[s]];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+            {
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(aw[s], b0[s], acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(aw[s], b1[s], acc1, 0, 0, 0);
+            }
+            ODL_STEM6_STAMP(4);
+            store_tile(pix0, acc0);
+            store_tile(pix1, acc1);
+            ODL_STEM6_STAMP(5);
+        }
+        else
+        {
+            float b0[STEPS];
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+                b0[s] = bp0[koff[s]];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s)
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(aw[s], b0[s], acc0, 0, 0, 0);
+            store_tile(pix0, acc0);
+        }
+    }
+    __syncthreads();
+    float *yrow = y + ((size_t)n * 16 * OH + oh) * OW;  // filter oc's row lies oc * OH * OW floats further
+    if (OW % 4 == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0)
+    {
+        const int q = OW / 4;
+        for (int e = t; e < 16 * q; e += kThreads)
+        {
+            const int oc = e / q, c4 = e - oc * q;
+            *reinterpret_cast<f32x4 *>(yrow + (size_t)oc * OH * OW + 4 * c4) = *reinterpret_cast<const f32x4 *>(outs + oc * opitch + 4 * c4);
+        }
+    }
+    else
+    {
+        for (int e = t; e < 16 * OW; e += kThreads)
+        {
+            const int oc = e / OW, c = e - oc * OW;
+            yrow[(size_t)oc * OH * OW + c] = outs[oc * opitch + c];
+        }
+    }
+    ODL_STEM6_STAMP(3);
+}
+
 // The 3x3 / stride 1 / padding 1 convolution above with ReLU and a 2x2 / stride 2 max pooling behind it in one pass: a
 // thread owns one pooled pixel, computes the four convolution outputs under it (a 4x4 patch of each input channel in
 // registers) for OCB channels, applies bias and activation and keeps the maximum and its place in the window. Per
@@ -673,7 +860,16 @@ int conv_small_forward(const float *x, const float *w, const float *b, float *y,
                        hipStream_t st)
 {
     const SmallGeom g = make_small(N, C, H, W, OC, SH, SW, PH, PW, OH, OW, false);
-    if (KH == 3)
+    if (KH == 6 && KW == 6 && SH == 2 && SW == 2 && PH == 2 && PW == 2 && C == 3 && OC == 16 && N * OH < (1ll << 31) &&
+        ((W + 4) * 18 + 4 + 16 * 108 + 16 * (OW + 8)) * 4 <= 64 * 1024)
+    {
+        // a detector's stem: a workgroup per output row, the products on the matrix cores
+        const int pitch = (int)W + 4;
+        hipLaunchKernelGGL((conv_stem6_mfma_kernel<3>), dim3((unsigned)(N * OH)), dim3(kThreads),
+                           (size_t)(3 * 6 * pitch + 4 + 16 * 3 * 36 + 16 * ((((int)OW + 3) / 4 * 4) | 4)) * sizeof(float), st, x, w, b, y,
+                           (int)H, (int)W, (int)OH, (int)OW, pitch, act);
+    }
+    else if (KH == 3)
     {
         const dim3 grid((unsigned)ceil_div(g.total, kThreads), (unsigned)(OC / 16));
         hipLaunchKernelGGL((conv_small_fwd_kernel<3, 3, 16>), grid, dim3(kThreads), 0, st, x, w, b, y, g, act);
@@ -682,10 +878,19 @@ int conv_small_forward(const float *x, const float *w, const float *b, float *y,
     {
         // two pixels a thread: the second one `half` pixels after the first
         const unsigned half = (unsigned)ceil_div(g.total, 2);
-        const dim3 grid((unsigned)ceil_div(half, kThreads), (unsigned)(OC / 16));
-        const size_t lds = (size_t)C * KH * KW * 16 * sizeof(float);
-        if (KH == 5)
+        // sixteen channels a thread while that fills the chip; a launch of fewer workgroups than two per compute unit deals
+        // eight a thread instead (a detector's stem at batch 4: 200 workgroups whose threads each walked 3456
+        // multiply-adds in a row)
+        const bool eight = ceil_div(half, kThreads) * (OC / 16) < 2 * (int64_t)device_cus();
+        const int ocb = eight ? 8 : 16;
+        const dim3 grid((unsigned)ceil_div(half, kThreads), (unsigned)(OC / ocb));
+        const size_t lds = (size_t)C * KH * KW * ocb * sizeof(float);
+        if (KH == 5 && eight)
+            hipLaunchKernelGGL((conv_small_fwd_lds_kernel<5, 5, 8>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
+        else if (KH == 5)
             hipLaunchKernelGGL((conv_small_fwd_lds_kernel<5, 5, 16>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
+        else if (eight)
+            hipLaunchKernelGGL((conv_small_fwd_lds_kernel<6, 6, 8>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
         else
             hipLaunchKernelGGL((conv_small_fwd_lds_kernel<6, 6, 16>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
     }

@@ -478,7 +478,8 @@ CONV_SEEDED = [
     (2, 6, 10, 9, 16, 2, 3, 1, 1),     # rectangular kernel, K = 36
     (2, 16, 15, 15, 20, 3, 3, 2, 0),   # stride 2 without padding
     (5, 64, 7, 7, 48, 3, 3, 1, 1),     # more pixels than one tile column, C = 64
-    (2, 3, 64, 64, 16, 6, 6, 2, 2),    # the detector's stem: 6x6, stride 2, pad 2, three channels (direct forward)
+    (2, 3, 64, 64, 16, 6, 6, 2, 2),    # the detector's stem: 6x6, stride 2, pad 2, three channels (a row a workgroup, MFMA)
+    (3, 3, 37, 45, 16, 6, 6, 2, 2),    # the same over odd extents: a ragged last pixel tile, rows and columns past the image
     (2, 32, 40, 40, 64, 3, 3, 2, 1),   # its down-sampling convolutions
     (2, 16, 15, 13, 32, 3, 3, 2, 1),   # stride 2 over odd extents
     (3, 8, 14, 14, 16, 3, 3, 2, 0),    # stride 2 without padding
