@@ -183,7 +183,10 @@ struct DetectGeom
     int64_t out_bs;  // floats from one image's rows of this stage to the next image's
 };
 
-__global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__restrict__ conv, const float *__restrict__ grid,
+// (sixteen waves a workgroup: the kernel is a chain of a load, 85 x 64 sigmoids and a store, and the chain is as long as
+// one lane's share of the sigmoids)
+constexpr int kDecodeThreads = 1024;
+__global__ __launch_bounds__(kDecodeThreads) void yolo_decode_kernel(const float *__restrict__ conv, const float *__restrict__ grid,
                                                              const float *__restrict__ anchor_grid,
                                                              float *__restrict__ out, DetectGeom g, int ptiles)
 {
@@ -199,9 +202,35 @@ __global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__rest
     const int np = (HW - p0 < 64) ? HW - p0 : 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float *src = conv + ((int64_t)(b * g.A + a) * g.CI) * HW + p0;
-    // a wave takes every fourth channel; twelve of them in flight at a time: the loads of a batch are issued together,
-    // then its sigmoids (85 channels: two batches a wave)
-    constexpr int kBatch = 12, kWaves = kBlock / 64;
+    // the grid or anchor value of the thread's box channel (used after the first barrier), asked for before anything else:
+    // behind the barrier it was a trip to memory of its own in a kernel that is little else than such trips
+    float box_operand = 0.0f;
+    {
+        const int pl = threadIdx.x >> 2, c = threadIdx.x & 3;
+        if (pl < np && c < g.CI)
+        {
+            const int p = p0 + pl;
+            const int h = p / g.W, w = p - h * g.W;
+            if (c < 2)
+            {
+                const int64_t gi = ((int64_t)a * HW + (int64_t)h * g.W + w) * 2 + c;
+                box_operand = gi < g.grid_elems ? grid[gi] : 0.0f;
+            }
+            else
+            {
+                const int sh_ = (g.anchor_H > 0 && g.H > g.anchor_H) ? g.H / g.anchor_H : 1;
+                const int sw_ = (g.anchor_W > 0 && g.W > g.anchor_W) ? g.W / g.anchor_W : 1;
+                int ah = h / sh_, aw = w / sw_;
+                ah = ah < g.anchor_H - 1 ? ah : g.anchor_H - 1;
+                aw = aw < g.anchor_W - 1 ? aw : g.anchor_W - 1;
+                const int64_t ai = ((int64_t)a * g.anchor_H * g.anchor_W + (int64_t)ah * g.anchor_W + aw) * 2 + (c - 2);
+                box_operand = ai < g.anchor_elems ? anchor_grid[ai] : 1.0f;
+            }
+        }
+    }
+    // a wave takes every sixteenth channel; eight of them in flight at a time: the loads of a batch are issued together,
+    // then its sigmoids (85 channels: one batch a wave, one trip to memory, six sigmoids a lane)
+    constexpr int kBatch = 8, kWaves = kDecodeThreads / 64;
     for (int c0 = wave; c0 < g.CI; c0 += kBatch * kWaves)
     {
         float v[kBatch];
@@ -227,26 +256,15 @@ __global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__rest
         if (pl < np && c < g.CI)
         {
             float v = sh_det[pl * LS + c];
-            const int p = p0 + pl;
-            const int h = p / g.W, w = p - h * g.W;
             if (c < 2)
             {
-                const int64_t gi = ((int64_t)a * HW + (int64_t)h * g.W + w) * 2 + c;
-                const float gv = gi < g.grid_elems ? grid[gi] : 0.0f;
                 const float t = v * 2.0f;
-                v = (t + gv) * g.stride;
+                v = (t + box_operand) * g.stride;
             }
             else
             {
-                const int sh_ = (g.anchor_H > 0 && g.H > g.anchor_H) ? g.H / g.anchor_H : 1;
-                const int sw_ = (g.anchor_W > 0 && g.W > g.anchor_W) ? g.W / g.anchor_W : 1;
-                int ah = h / sh_, aw = w / sw_;
-                ah = ah < g.anchor_H - 1 ? ah : g.anchor_H - 1;
-                aw = aw < g.anchor_W - 1 ? aw : g.anchor_W - 1;
-                const int64_t ai = ((int64_t)a * g.anchor_H * g.anchor_W + (int64_t)ah * g.anchor_W + aw) * 2 + (c - 2);
-                const float av = ai < g.anchor_elems ? anchor_grid[ai] : 1.0f;
                 const float t = v * 2.0f;
-                v = (t * t) * av;  // pow(2s, 2) * anchor
+                v = (t * t) * box_operand;  // pow(2s, 2) * anchor
             }
             sh_det[pl * LS + c] = v;
         }
@@ -254,7 +272,8 @@ __global__ __launch_bounds__(kBlock) void yolo_decode_kernel(const float *__rest
     __syncthreads();
     // [pixel][channel] rows out of LDS, consecutive lanes along the output
     float *dst = out + (int64_t)b * g.out_bs + ((int64_t)a * HW + p0) * g.CI;
-    for (int pl = wave; pl < np; pl += kBlock / 64)
+    for (int pl = wave; pl < np; pl += kDecodeThreads / 64)
+#pragma unroll 2
         for (int c = lane; c < g.CI; c += 64)
             dst[pl * g.CI + c] = sh_det[pl * LS + c];
 }
@@ -492,7 +511,7 @@ int odl_hip_yolo_decode(const float *conv, const float *grid, int64_t grid_elems
     const int ptiles = (int)odl::ceil_div(H * W, 64);
     const DetectGeom g{num_anchors, CI, (int)H, (int)W, (int)anchor_H, (int)anchor_W, grid_elems, anchor_elems, stride, os};
     const size_t lds = (size_t)64 * (CI | 1) * sizeof(float);
-    hipLaunchKernelGGL(yolo_decode_kernel, dim3((unsigned)(N * num_anchors * ptiles)), dim3(kBlock), lds, odl::as_stream(stream),
+    hipLaunchKernelGGL(yolo_decode_kernel, dim3((unsigned)(N * num_anchors * ptiles)), dim3(kDecodeThreads), lds, odl::as_stream(stream),
                        conv, grid, anchor_grid, out, g, ptiles);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
@@ -536,7 +555,7 @@ int odl_hip_yolo_detect_forward(const float *x, const float *conv_w, const float
     const DetectGeom g{num_anchors, CI, (int)H, (int)W, (int)anchor_H, (int)anchor_W, grid_elems, anchor_elems, stride,
                        (int64_t)num_anchors * H * W * CI};
     const size_t lds = (size_t)64 * (CI | 1) * sizeof(float);
-    hipLaunchKernelGGL(yolo_decode_kernel, dim3((unsigned)(N * num_anchors * ptiles)), dim3(kBlock), lds,
+    hipLaunchKernelGGL(yolo_decode_kernel, dim3((unsigned)(N * num_anchors * ptiles)), dim3(kDecodeThreads), lds,
                        odl::as_stream(stream), conv, grid, anchor_grid, out, g, ptiles);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
