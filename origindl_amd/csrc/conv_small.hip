@@ -878,19 +878,10 @@ int conv_small_forward(const float *x, const float *w, const float *b, float *y,
     {
         // two pixels a thread: the second one `half` pixels after the first
         const unsigned half = (unsigned)ceil_div(g.total, 2);
-        // sixteen channels a thread while that fills the chip; a launch of fewer workgroups than two per compute unit deals
-        // eight a thread instead (a detector's stem at batch 4: 200 workgroups whose threads each walked 3456
-        // multiply-adds in a row)
-        const bool eight = ceil_div(half, kThreads) * (OC / 16) < 2 * (int64_t)device_cus();
-        const int ocb = eight ? 8 : 16;
-        const dim3 grid((unsigned)ceil_div(half, kThreads), (unsigned)(OC / ocb));
-        const size_t lds = (size_t)C * KH * KW * ocb * sizeof(float);
-        if (KH == 5 && eight)
-            hipLaunchKernelGGL((conv_small_fwd_lds_kernel<5, 5, 8>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
-        else if (KH == 5)
+        const dim3 grid((unsigned)ceil_div(half, kThreads), (unsigned)(OC / 16));
+        const size_t lds = (size_t)C * KH * KW * 16 * sizeof(float);
+        if (KH == 5)
             hipLaunchKernelGGL((conv_small_fwd_lds_kernel<5, 5, 16>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
-        else if (eight)
-            hipLaunchKernelGGL((conv_small_fwd_lds_kernel<6, 6, 8>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
         else
             hipLaunchKernelGGL((conv_small_fwd_lds_kernel<6, 6, 16>), grid, dim3(kThreads), lds, st, x, w, b, y, g, act, half);
     }
