@@ -493,7 +493,9 @@ size_t odl_hip_yolo_detect_workspace_bytes(int64_t N, int64_t C, int64_t H, int6
  *    block); stage j's result goes to channels [(j-1)*C, j*C) of y. One launch, the plane stays in LDS (H*W <= 8192).
  *  copy_images: dst[n][j] = src[n][j] for j < count — one input of a concatenation, or a view made dense.
  *  yolo_decode: the second half of odl_hip_yolo_detect_forward (sigmoid + box decoding of conv[N, A*(classes+5), H, W])
- *    with the stage's rows written out_image_stride floats apart, i.e. straight into the concatenation of the stages. */
+ *    with the stage's rows written out_image_stride floats apart, i.e. straight into the concatenation of the stages.
+ *  yolo_decode_stages: yolo_decode for 1 to 4 stages of one head (same N, anchors and classes) in one launch; the
+ *    arrays are host arrays with one entry per stage, out[s] the first row of stage s. Same values as one call a stage. */
 int odl_hip_upsample_nearest_view(const float *x, int64_t x_image_stride, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OH,
                                   int64_t OW, int scale_h, int scale_w, float *y, int64_t y_image_stride, void *stream);
 int odl_hip_max_pool2d_chain(const float *x, int64_t x_image_stride, int64_t N, int64_t C, int64_t H, int64_t W, int K,
@@ -503,6 +505,11 @@ int odl_hip_copy_images(const float *src, int64_t src_image_stride, float *dst, 
 int odl_hip_yolo_decode(const float *conv, const float *grid, int64_t grid_elems, const float *anchor_grid, int64_t anchor_elems,
                         int64_t anchor_H, int64_t anchor_W, int64_t N, int64_t H, int64_t W, float stride, int num_anchors,
                         int num_classes, float *out, int64_t out_image_stride, void *stream);
+int odl_hip_yolo_decode_stages(int stages, const float *const *host_conv, const float *const *host_grid, const int64_t *host_grid_elems,
+                               const float *const *host_anchor_grid, const int64_t *host_anchor_elems, const int64_t *host_anchor_H,
+                               const int64_t *host_anchor_W, int64_t N, const int64_t *host_H, const int64_t *host_W,
+                               const float *host_stride, int num_anchors, int num_classes, float *const *host_out,
+                               int64_t out_image_stride, void *stream);
 
 /* Mat::batch_norm_forward / Mat::batch_norm (mat.h:603-631; src/mat/origin/cpu/normalization/batch_norm.cpp:31-258)
  * over x[N, C, P]: P = H*W for num_dims 4, P = 1 for num_dims 2. training != 0: per-channel mean and biased variance

@@ -780,6 +780,36 @@ def yolo_decode(conv, grid, anchor_grid, stride, num_anchors, num_classes, out_r
     return out_rows
 
 
+def yolo_decode_stages(convs, grids, anchor_grids, strides, num_anchors, num_classes, out):
+    """yolo_decode for every stage of a head in one launch: stage s fills the rows of out[N, rows, classes+5] that follow
+    those of stage s - 1, from row 0 (the concatenation the reference's YoloDetect node makes,
+    src/pnnx/pnnx_graph.cpp:286-528)."""
+    S = len(convs)
+    if not (1 <= S <= 4) or len(grids) != S or len(anchor_grids) != S or len(strides) != S:
+        raise OdlInvalidArgument("yolo_decode_stages: 1 to 4 stages with a grid, an anchor grid and a stride each")
+    _chk(out, "out")
+    CI = num_classes + 5
+    N = out.shape[0]
+    outs, row0, aHs, aWs = [], 0, [], []
+    for c, g, a in zip(convs, grids, anchor_grids):
+        _chk(c, "conv"), _chk(g, "grid"), _chk(a, "anchor_grid")
+        if c.dim() != 4 or c.shape[0] != N or c.shape[1] != num_anchors * CI:
+            raise OdlInvalidArgument("yolo_decode_stages: a stage's convolution must be [%d, %d, H, W]" % (N, num_anchors * CI))
+        H, W = int(c.shape[2]), int(c.shape[3])
+        aHs.append(int(a.shape[2]) if a.dim() >= 3 else H), aWs.append(int(a.shape[3]) if a.dim() >= 4 else W)
+        outs.append(out.data_ptr() + row0 * CI * 4)
+        row0 += num_anchors * H * W
+    if out.dim() != 3 or out.shape[2] != CI or row0 > out.shape[1]:
+        raise OdlInvalidArgument("yolo_decode_stages: out must be [%d, >= %d, %d]" % (N, row0, CI))
+    ptr = lambda ts: (ctypes.c_void_p * S)(*[t.data_ptr() for t in ts])
+    i64 = lambda vs: (ctypes.c_int64 * S)(*[int(v) for v in vs])
+    lib().call("odl_hip_yolo_decode_stages", S, ptr(convs), ptr(grids), i64(g.numel() for g in grids), ptr(anchor_grids),
+               i64(a.numel() for a in anchor_grids), i64(aHs), i64(aWs), N, i64(c.shape[2] for c in convs),
+               i64(c.shape[3] for c in convs), (ctypes.c_float * S)(*[float(v) for v in strides]), num_anchors, num_classes,
+               (ctypes.c_void_p * S)(*outs), int(out.shape[1]) * CI, _stream())
+    return out
+
+
 def _bn_dims(x, who):
     if x.dim() not in (2, 4):
         raise OdlInvalidArgument("%s: x must have 2 or 4 dimensions, but got shape %s" % (who, tuple(x.shape)))

@@ -186,14 +186,13 @@ struct DetectGeom
 // (sixteen waves a workgroup: the kernel is a chain of a load, 85 x 64 sigmoids and a store, and the chain is as long as
 // one lane's share of the sigmoids)
 constexpr int kDecodeThreads = 1024;
-__global__ __launch_bounds__(kDecodeThreads) void yolo_decode_kernel(const float *__restrict__ conv, const float *__restrict__ grid,
-                                                             const float *__restrict__ anchor_grid,
-                                                             float *__restrict__ out, DetectGeom g, int ptiles)
+__device__ __forceinline__ void yolo_decode_tile(const float *__restrict__ conv, const float *__restrict__ grid,
+                                                 const float *__restrict__ anchor_grid, float *__restrict__ out,
+                                                 const DetectGeom &g, int ptiles, unsigned vb)
 {
     extern __shared__ float sh_det[];  // [64][CI | 1]
     const int LS = g.CI | 1;
     const int HW = g.H * g.W;
-    unsigned vb = blockIdx.x;
     const int pt = (int)(vb % (unsigned)ptiles);
     vb /= (unsigned)ptiles;
     const int a = (int)(vb % (unsigned)g.A);
@@ -276,6 +275,33 @@ __global__ __launch_bounds__(kDecodeThreads) void yolo_decode_kernel(const float
 #pragma unroll 2
         for (int c = lane; c < g.CI; c += 64)
             dst[pl * g.CI + c] = sh_det[pl * LS + c];
+}
+
+__global__ __launch_bounds__(kDecodeThreads) void yolo_decode_kernel(const float *__restrict__ conv, const float *__restrict__ grid,
+                                                             const float *__restrict__ anchor_grid,
+                                                             float *__restrict__ out, DetectGeom g, int ptiles)
+{
+    yolo_decode_tile(conv, grid, anchor_grid, out, g, ptiles, blockIdx.x);
+}
+
+// Up to kMaxStages stages of one detect head in one launch: workgroups [first[s], first[s + 1]) are stage s's, each doing
+// what yolo_decode_kernel's workgroup of the same number within the stage does.
+constexpr int kMaxStages = 4;
+struct DetectStages
+{
+    const float *conv[kMaxStages], *grid[kMaxStages], *anchor_grid[kMaxStages];
+    float *out[kMaxStages];
+    DetectGeom g[kMaxStages];
+    int ptiles[kMaxStages];
+    unsigned first[kMaxStages + 1];
+};
+
+__global__ __launch_bounds__(kDecodeThreads) void yolo_decode_stages_kernel(DetectStages d, int stages)
+{
+    int s = 0;
+    for (int j = 1; j < stages; ++j)
+        s = blockIdx.x >= d.first[j] ? j : s;
+    yolo_decode_tile(d.conv[s], d.grid[s], d.anchor_grid[s], d.out[s], d.g[s], d.ptiles[s], blockIdx.x - d.first[s]);
 }
 }  // namespace
 
@@ -513,6 +539,50 @@ int odl_hip_yolo_decode(const float *conv, const float *grid, int64_t grid_elems
     const size_t lds = (size_t)64 * (CI | 1) * sizeof(float);
     hipLaunchKernelGGL(yolo_decode_kernel, dim3((unsigned)(N * num_anchors * ptiles)), dim3(kDecodeThreads), lds, odl::as_stream(stream),
                        conv, grid, anchor_grid, out, g, ptiles);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+
+int odl_hip_yolo_decode_stages(int stages, const float *const *host_conv, const float *const *host_grid, const int64_t *host_grid_elems,
+                               const float *const *host_anchor_grid, const int64_t *host_anchor_elems, const int64_t *host_anchor_H,
+                               const int64_t *host_anchor_W, int64_t N, const int64_t *host_H, const int64_t *host_W,
+                               const float *host_stride, int num_anchors, int num_classes, float *const *host_out,
+                               int64_t out_image_stride, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(stages >= 1 && stages <= kMaxStages, "yolo_decode_stages: 1 to %d stages, got %d", kMaxStages, stages);
+    ODL_REQUIRE(host_conv && host_grid && host_grid_elems && host_anchor_grid && host_anchor_elems && host_anchor_H && host_anchor_W &&
+                    host_H && host_W && host_stride && host_out,
+                "yolo_decode_stages: null argument");
+    ODL_REQUIRE(N >= 0 && num_anchors > 0 && num_classes >= 0, "yolo_decode_stages: bad shape");
+    const int CI = num_classes + 5;
+    ODL_REQUIRE(CI < 8192, "yolo_decode_stages: too large");
+    DetectStages d{};
+    int64_t blocks = 0;
+    for (int s = 0; s < stages; ++s)
+    {
+        const int64_t H = host_H[s], W = host_W[s];
+        ODL_REQUIRE(H > 0 && W > 0 && H * W < (1ll << 30), "yolo_decode_stages: bad shape of stage %d", s);
+        ODL_REQUIRE(host_conv[s] && host_grid[s] && host_anchor_grid[s] && host_out[s], "yolo_decode_stages: null operand of stage %d", s);
+        ODL_REQUIRE(host_grid_elems[s] >= 0 && host_anchor_elems[s] >= 0 && host_anchor_H[s] > 0 && host_anchor_W[s] > 0,
+                    "yolo_decode_stages: bad grid sizes of stage %d", s);
+        const int64_t rows = (int64_t)num_anchors * H * W * CI;
+        const int64_t os = out_image_stride ? out_image_stride : rows;
+        ODL_REQUIRE(os >= rows, "yolo_decode_stages: the output image stride is shorter than the rows of stage %d", s);
+        d.conv[s] = host_conv[s], d.grid[s] = host_grid[s], d.anchor_grid[s] = host_anchor_grid[s], d.out[s] = host_out[s];
+        d.ptiles[s] = (int)odl::ceil_div(H * W, 64);
+        d.g[s] = DetectGeom{num_anchors, CI, (int)H, (int)W, (int)host_anchor_H[s], (int)host_anchor_W[s], host_grid_elems[s],
+                            host_anchor_elems[s], host_stride[s], os};
+        d.first[s] = (unsigned)blocks;
+        blocks += N * num_anchors * d.ptiles[s];
+        ODL_REQUIRE(blocks < (1ll << 31), "yolo_decode_stages: too large");
+    }
+    for (int s = stages; s <= kMaxStages; ++s)
+        d.first[s] = (unsigned)blocks;
+    if (blocks == 0)
+        return ODL_OK;
+    const size_t lds = (size_t)64 * (CI | 1) * sizeof(float);
+    hipLaunchKernelGGL(yolo_decode_stages_kernel, dim3((unsigned)blocks), dim3(kDecodeThreads), lds, odl::as_stream(stream), d, stages);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

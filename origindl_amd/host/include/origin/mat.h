@@ -394,6 +394,10 @@ public:
     // [row0, row0 + A*H*W) of out[N, rows, classes+5]: the second half of yolo_detect_forward
     void yolo_decode_into(const Mat &grid, const Mat &anchor_grid, float stride, int32_t num_anchors, int32_t num_classes,
                           Mat &out, size_t row0) const;
+    // the same for every stage of a head in one launch: conv[s] into the rows that follow those of conv[s - 1], from row 0
+    static void yolo_decode_stages_into(const std::vector<const Mat *> &conv, const std::vector<const Mat *> &grid,
+                                        const std::vector<const Mat *> &anchor_grid, const std::vector<float> &stride,
+                                        int32_t num_anchors, int32_t num_classes, Mat &out);
     // Max pooling with the window-local indices kept in device memory (uint64 per output). The Mat interface above
     // hands them to the caller as a host vector, which costs a device-to-host copy in forward and a host-to-device
     // copy in backward (the reference's device backend pays both); the pooling operator uses this pair instead.

@@ -1477,6 +1477,46 @@ void OriginMat::yolo_decode_into(const Mat &grid, const Mat &anchor_grid, float 
                               cur()));
 }
 
+void OriginMat::yolo_decode_stages_into(const std::vector<const Mat *> &conv_m, const std::vector<const Mat *> &grid,
+                                        const std::vector<const Mat *> &anchor_grid, const std::vector<float> &stride,
+                                        int32_t num_anchors, int32_t num_classes, Mat &out_m)
+{
+    const size_t S = conv_m.size();
+    if (S == 0 || S > 4 || grid.size() != S || anchor_grid.size() != S || stride.size() != S)
+        THROW_INVALID_ARG("yolo_detect_forward: 1 to 4 stages with a grid, an anchor grid and a stride each, got {}", S);
+    const OriginMat &out = dev_f32(out_m, "yolo_detect_forward");
+    const int64_t CI = num_classes + 5;
+    const Shape &os = out.shape();
+    if (os.size() != 3 || (int64_t)os[2] != CI)
+        THROW_INVALID_ARG("yolo_detect_forward: the output must be [N, rows, {}], got {}", CI, os.to_string());
+    const int64_t N = os[0];
+    const float *cp[4], *gp[4], *ap[4];
+    float *op[4];
+    int64_t ge[4], ae[4], aH[4], aW[4], H[4], W[4];
+    size_t row0 = 0;
+    for (size_t s = 0; s < S; ++s)
+    {
+        const OriginMat &conv = dev_f32(*conv_m[s], "yolo_detect_forward");
+        const OriginMat &g = dev_f32(*grid[s], "yolo_detect_forward");
+        const OriginMat &ag = dev_f32(*anchor_grid[s], "yolo_detect_forward");
+        const Shape &cs = conv.shape();
+        if (cs.size() != 4 || (int64_t)cs[0] != N || (int64_t)cs[1] != num_anchors * CI)
+            THROW_INVALID_ARG("yolo_detect_forward: the stage's convolution must be [{}, {}, H, W], got {}", N, num_anchors * CI,
+                              cs.to_string());
+        H[s] = cs[2], W[s] = cs[3];
+        if (row0 + (size_t)(num_anchors * H[s] * W[s]) > os[1])
+            THROW_INVALID_ARG("yolo_detect_forward: rows [{}, {}) do not lie in an output of shape {}", row0,
+                              row0 + num_anchors * H[s] * W[s], os.to_string());
+        const Shape as = ag.shape();
+        aH[s] = as.size() >= 3 ? (int64_t)as[2] : H[s], aW[s] = as.size() >= 4 ? (int64_t)as[3] : W[s];
+        cp[s] = fp(conv), gp[s] = fp(g), ap[s] = fp(ag), ge[s] = (int64_t)g.elements(), ae[s] = (int64_t)ag.elements();
+        op[s] = const_cast<float *>(fp(out)) + (int64_t)row0 * CI;
+        row0 += (size_t)(num_anchors * H[s] * W[s]);
+    }
+    check(odl_hip_yolo_decode_stages((int)S, cp, gp, ge, ap, ae, aH, aW, N, H, W, stride.data(), num_anchors, num_classes, op,
+                                     (int64_t)(os[1] * os[2]), cur()));
+}
+
 std::unique_ptr<Mat> OriginMat::pow(const Scalar &exponent) const
 {
     const OriginMat &x = dev_any(*this, "pow");

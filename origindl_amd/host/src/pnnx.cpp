@@ -962,10 +962,10 @@ void PNNXGraph::run(PNNXNode &node)
         }
         if (direct)
         {
-            // each stage: its 1x1 convolution, then the decoding straight into the stage's rows of the final tensor
+            // the stages' 1x1 convolutions, then their decoding straight into each stage's rows of the final tensor
             const size_t N = run_shape(first)[0];
             std::shared_ptr<Mat> out = std::make_shared<OriginMat>(Shape{N, rows, ci}, DataType::kFloat32, dev);
-            size_t row0 = 0;
+            std::shared_ptr<Mat> convs[3];
             for (int s = 0; s < 3; ++s)
             {
                 Value &xv = value(node.input_names[s], node);
@@ -985,9 +985,11 @@ void PNNXGraph::run(PNNXNode &node)
                 }
                 else
                     conv = origin_of(*dense(node.input_names[s], node)).conv2d_act(*ws[s], bs[s].get(), {1, 1}, {0, 0}, -1, wa.packed_mat.get());
-                origin_of(*conv).yolo_decode_into(*gs[s], *ags[s], strides[s], 3, (int)ci - 5, *out, row0);
-                row0 += 3 * xs[2] * xs[3];
+                convs[s] = std::move(conv);
             }
+            // (one launch for the three stages: each is a chain of a load, sigmoids and a store, shorter than a launch)
+            OriginMat::yolo_decode_stages_into({convs[0].get(), convs[1].get(), convs[2].get()}, {gs[0].get(), gs[1].get(), gs[2].get()},
+                                               {ags[0].get(), ags[1].get(), ags[2].get()}, strides, 3, (int)ci - 5, *out);
             store(node, std::move(out));
             return;
         }

@@ -1634,6 +1634,26 @@ def test_detector_operators_on_channel_runs_are_the_dense_operators(api, o):
     want = out0.copy()
     want[:, 500:500 + A * H * W] = dense
     assert np.array_equal(host(out), want)
+    # the stages of a head decoded in one launch = one call a stage (a stage with a ragged last pixel tile among them)
+    convs, grids, ags, wants = [], [], [], []
+    strides = (8.0, 16.0, 32.0)
+    for (H, W) in ((20, 20), (10, 13), (5, 5)):
+        convs.append(dev(rng.standard_normal((N, A * CI, H, W), dtype=f32) * f32(3)))
+        gyy, gxx = np.meshgrid(np.arange(H), np.arange(W), indexing="ij")
+        grids.append(dev(np.broadcast_to(np.stack([gxx, gyy], -1).astype(f32) - f32(0.5), (1, A, H, W, 2)).copy()))
+        ags.append(dev((rng.random((1, A, H, W, 2), dtype=f32) * f32(90) + f32(4)).astype(f32)))
+    rows = sum(A * c.shape[2] * c.shape[3] for c in convs)
+    one, each = dev(np.full((N, rows + 9, CI), 7, f32)), dev(np.full((N, rows + 9, CI), 7, f32))
+    api.yolo_decode_stages(convs, grids, ags, strides, A, NC, one)
+    r0 = 0
+    for c, g, a, st in zip(convs, grids, ags, strides):
+        r = A * c.shape[2] * c.shape[3]
+        api.yolo_decode(c, g, a, st, A, NC, each[:, r0:r0 + r])
+        r0 += r
+    assert np.array_equal(host(one), host(each))
+    assert np.all(host(one)[:, rows:] == 7)
+    with pytest.raises(api.OdlInvalidArgument):
+        api.yolo_decode_stages(convs, grids[:2], ags, strides, A, NC, one)
 
 
 # ------------------------------------------------------------------ element types besides float32
