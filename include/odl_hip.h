@@ -240,6 +240,18 @@ int odl_hip_conv2d_fused_pair(const float *x, int64_t x_image_stride, const floa
                               int64_t H, int64_t W, int64_t OC, int64_t split, int KH, int KW, int SH, int SW, int PH, int PW,
                               int activation, float *y_first, int64_t y_first_image_stride, float *y_second,
                               int64_t y_second_image_stride, void *stream);
+/* One to four convolutions with 1x1 windows (stride 1, no padding, no residual) over the same batch — the stage
+ * convolutions of a detect head, nn.Conv2d nodes that do not depend on each other — as one launch. Arrays are host
+ * arrays with one entry per member; host_b may be NULL (no member has a bias) or hold NULL entries. Each member gets
+ * the floats of its own odl_hip_conv2d_fused call, bit for bit. odl_hip_conv2d_fused_group_ok answers 1 for member shapes
+ * this entry point takes. No counterpart in the reference, whose runner executes the nodes one by one
+ * (src/pnnx/pnnx_graph.cpp:286-528). */
+int odl_hip_conv2d_fused_group_ok(int count, int64_t N, const int64_t *host_C, const int64_t *host_H, const int64_t *host_W,
+                                  const int64_t *host_OC);
+int odl_hip_conv2d_fused_group(int count, const float *const *host_x, const int64_t *host_x_image_stride, const float *const *host_packed,
+                               const float *const *host_b, int64_t N, const int64_t *host_C, const int64_t *host_H,
+                               const int64_t *host_W, const int64_t *host_OC, int activation, float *const *host_y,
+                               const int64_t *host_y_image_stride, void *stream);
 /* Measurement switches, for the whole process (same caveat as above: never between a query and its call):
  * set_conv_direct(0) sends the small problems to the tiled kernels again; set_conv_direct_plan(k_shares, pixel_tiles)
  * fixes how a workgroup of the small-problem kernel is cut (0, 0: its own rule). No counterpart in the reference. */

@@ -738,6 +738,38 @@ def conv2d_fused(x, w_shape, packed, b, y, stride=1, pad=0, activation=None, res
     return y
 
 
+def conv2d_fused_group_ok(x_shapes, w_shapes):
+    S = len(x_shapes)
+    if not (1 <= S <= 4) or len(w_shapes) != S:
+        return False
+    if any(len(w) != 4 or int(w[2]) != 1 or int(w[3]) != 1 or int(w[1]) != int(x[1]) or int(x[0]) != int(x_shapes[0][0])
+           for x, w in zip(x_shapes, w_shapes)):
+        return False
+    i64 = lambda vs: (ctypes.c_int64 * S)(*[int(v) for v in vs])
+    return lib().query("odl_hip_conv2d_fused_group_ok", S, int(x_shapes[0][0]), i64(x[1] for x in x_shapes), i64(x[2] for x in x_shapes),
+                       i64(x[3] for x in x_shapes), i64(w[0] for w in w_shapes)) == 1
+
+
+def conv2d_fused_group(xs, w_shapes, packeds, bs, ys, activation=None):
+    """One to four 1x1 convolutions (stride 1, no padding) of independent inputs as one launch: member i is
+    conv2d_fused(xs[i], w_shapes[i], packeds[i], bs[i], ys[i], 1, 0, activation), bit for bit. The stage convolutions of
+    the reference's YoloDetect node (src/pnnx/pnnx_graph.cpp:286-528)."""
+    S = len(xs)
+    if not (1 <= S <= 4) or len(w_shapes) != S or len(packeds) != S or len(bs) != S or len(ys) != S:
+        raise OdlInvalidArgument("conv2d_fused_group: 1 to 4 members with a filter shape, a filter copy, a bias (or None) and an output each")
+    xst, yst = [_run(x, "x") for x in xs], [_run(y, "y") for y in ys]
+    N = int(xs[0].shape[0])
+    for x, w, y in zip(xs, w_shapes, ys):
+        if tuple(y.shape) != (N, int(w[0]), x.shape[2], x.shape[3]) or x.shape[0] != N or int(w[1]) != x.shape[1] or tuple(w[2:]) != (1, 1):
+            raise OdlInvalidArgument("conv2d_fused_group: a member's x, filter shape and y do not belong together")
+    act = -1 if activation is None else _UN[activation]
+    ptr = lambda ts: (ctypes.c_void_p * S)(*[None if t is None else t.data_ptr() for t in ts])
+    i64 = lambda vs: (ctypes.c_int64 * S)(*[int(v) for v in vs])
+    lib().call("odl_hip_conv2d_fused_group", S, ptr(xs), i64(xst), ptr(packeds), ptr(bs), N, i64(x.shape[1] for x in xs),
+               i64(x.shape[2] for x in xs), i64(x.shape[3] for x in xs), i64(w[0] for w in w_shapes), act, ptr(ys), i64(yst), _stream())
+    return ys
+
+
 def upsample_view(x, y, scale):
     sh, sw = _pair(scale)
     xs, ys = _run(x, "x"), _run(y, "y")

@@ -106,6 +106,9 @@ bool conv_direct_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int 
                     int64_t OH, int64_t OW);
 size_t conv_direct_packed_bytes(int64_t C, int64_t OC, int KH, int KW, int P, int64_t W);
 int conv_direct_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, int P, int64_t W, float *packed, hipStream_t st);
+int conv_direct_group(int count, const float *const *x, const int64_t *x_bs, const float *const *packed, const float *const *b,
+                      float *const *y, const int64_t *y_bs, int64_t N, const int64_t *C, const int64_t *H, const int64_t *W,
+                      const int64_t *OC, int act, hipStream_t st);
 int conv_direct(const float *x, int64_t x_bs, const float *packed, const float *b, const float *res, int64_t res_bs, float *y,
                 int64_t y_bs, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int S, int P, int64_t OH,
                 int64_t OW, int act, hipStream_t st, float *y2 = nullptr, int64_t y2_bs = 0, int64_t split = 0);
@@ -1378,6 +1381,47 @@ int odl_hip_conv2d_fused(const float *x, int64_t x_image_stride, const float *pa
     const int act = activation == 0 ? 1 : (activation == 7 ? 2 : 0);
     return odl::conv_direct(x, x_image_stride, packed, b, residual, residual_image_stride, y, y_image_stride, N, C, H, W, OC,
                             KH, KW, SH, PH, g.OH, g.OW, act, odl::as_stream(stream));
+}
+
+int odl_hip_conv2d_fused_group_ok(int count, int64_t N, const int64_t *host_C, const int64_t *host_H, const int64_t *host_W,
+                                  const int64_t *host_OC)
+{
+    if (count < 1 || count > 4 || N <= 0 || !host_C || !host_H || !host_W || !host_OC)
+        return 0;
+    for (int s = 0; s < count; ++s)
+        if (host_C[s] <= 0 || host_H[s] <= 0 || host_W[s] <= 0 || host_OC[s] <= 0 ||
+            !odl::conv_direct_ok(N, host_C[s], host_H[s], host_W[s], host_OC[s], 1, 1, 1, 1, 0, 0, host_H[s], host_W[s]))
+            return 0;
+    return 1;
+}
+
+int odl_hip_conv2d_fused_group(int count, const float *const *host_x, const int64_t *host_x_image_stride, const float *const *host_packed,
+                               const float *const *host_b, int64_t N, const int64_t *host_C, const int64_t *host_H,
+                               const int64_t *host_W, const int64_t *host_OC, int activation, float *const *host_y,
+                               const int64_t *host_y_image_stride, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(activation == -1 || activation == 0 || activation == 7,
+                "conv2d: activation must be -1 (none), 0 (relu) or 7 (silu), the unary operator numbers; got %d", activation);
+    ODL_REQUIRE(count >= 1 && count <= 4, "conv2d_fused_group: 1 to 4 members, got %d", count);
+    ODL_REQUIRE(host_x && host_x_image_stride && host_packed && host_C && host_H && host_W && host_OC && host_y && host_y_image_stride,
+                "conv2d_fused_group: null argument");
+    ODL_REQUIRE(N >= 0, "conv2d_fused_group: N must not be negative");
+    if (N == 0)
+        return ODL_OK;
+    ODL_REQUIRE(odl_hip_conv2d_fused_group_ok(count, N, host_C, host_H, host_W, host_OC),
+                "conv2d_fused_group: shape not covered (ask odl_hip_conv2d_fused_group_ok first)");
+    for (int s = 0; s < count; ++s)
+    {
+        ODL_REQUIRE(host_x[s] && host_packed[s] && host_y[s], "conv2d_fused_group: null operand of member %d", s);
+        const int64_t xi = host_C[s] * host_H[s] * host_W[s], yi = host_OC[s] * host_H[s] * host_W[s];
+        ODL_REQUIRE((host_x_image_stride[s] == 0 || host_x_image_stride[s] >= xi) && (host_y_image_stride[s] == 0 || host_y_image_stride[s] >= yi),
+                    "conv2d_fused_group: an image stride of member %d is shorter than the image it strides over", s);
+        ODL_REQUIRE(host_x_image_stride[s] < (1ll << 40) && host_y_image_stride[s] < (1ll << 40), "conv2d_fused_group: image stride too large");
+    }
+    const int act = activation == 0 ? 1 : (activation == 7 ? 2 : 0);
+    return odl::conv_direct_group(count, host_x, host_x_image_stride, host_packed, host_b, host_y, host_y_image_stride, N, host_C, host_H,
+                                  host_W, host_OC, act, odl::as_stream(stream));
 }
 
 int odl_hip_conv2d_fused_pair(const float *x, int64_t x_image_stride, const float *packed, const float *b, int64_t N, int64_t C,

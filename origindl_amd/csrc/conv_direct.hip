@@ -174,7 +174,7 @@ __device__ __forceinline__ void direct_finish(const DirectArgs &g, const f32x16 
 // clocks whether or not its data is used, so the depth divides the group count (3 for 3x3 windows, 4 otherwise) and no
 // group is loaded twice.
 template <int kDepth, bool RES>
-__global__ __launch_bounds__(1024) void conv_direct_kernel(DirectArgs g)
+__device__ __forceinline__ void conv_direct_tile(const DirectArgs &g, const unsigned bid)
 {
     extern __shared__ float lds[];  // bias[32], then partial[WP * KS][32][kPitch] when KS > 1
     ODL_DIRECT_STAMP(0);
@@ -182,7 +182,6 @@ __global__ __launch_bounds__(1024) void conv_direct_kernel(DirectArgs g)
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int pt = wv / g.KS, ks = wv - pt * g.KS;
-    const unsigned bid = blockIdx.x;
     const int oct = (int)(bid % (unsigned)g.octiles);
     const int m_base = (int)(bid / (unsigned)g.octiles) * 32 * g.WP;
     const int oc0 = oct * 32;
@@ -251,6 +250,31 @@ __global__ __launch_bounds__(1024) void conv_direct_kernel(DirectArgs g)
         if (d < rem)
             use(d);
     direct_finish<RES>(g, acc, bias_v, bias_s, partial, wv, pt, l32, half, m_base, oc0, OHW, n, r);
+}
+
+template <int kDepth, bool RES>
+__global__ __launch_bounds__(1024) void conv_direct_kernel(DirectArgs g)
+{
+    conv_direct_tile<kDepth, RES>(g, blockIdx.x);
+}
+
+// Several convolutions with 1x1 windows in one launch (the stage convolutions of a detect head: small, independent, each
+// a launch's latency long on its own): workgroups [first[s], first[s + 1]) are member s's, each doing what
+// conv_direct_kernel's workgroup of the same number does for that member alone. Every member is cut into sixteen waves
+// a workgroup, its K shares as plan_direct gives them for the member alone, so its sums are formed in the same order.
+constexpr int kGroupMax = 4;
+struct DirectGroup
+{
+    DirectArgs g[kGroupMax];
+    unsigned first[kGroupMax + 1];
+};
+
+__global__ __launch_bounds__(1024) void conv_direct_group_kernel(DirectGroup d, int count)
+{
+    int s = 0;
+    for (int j = 1; j < count; ++j)
+        s = blockIdx.x >= d.first[j] ? j : s;
+    conv_direct_tile<4, false>(d.g[s], blockIdx.x - d.first[s]);
 }
 
 // 3x3 windows with padding 1 (stride 1 or 2, rows of three pixels or more): the three taps of a window row are three
@@ -454,6 +478,44 @@ int conv_direct(const float *x, int64_t x_bs, const float *packed, const float *
         hipLaunchKernelGGL((conv_direct_kernel<4, true>), grid, block, lds, st, g);
     else
         hipLaunchKernelGGL((conv_direct_kernel<4, false>), grid, block, lds, st, g);
+    ODL_LAUNCH_CHECK();
+    return ODL_OK;
+}
+}  // namespace odl
+
+namespace odl
+{
+int conv_direct_group(int count, const float *const *x, const int64_t *x_bs, const float *const *packed, const float *const *b,
+                      float *const *y, const int64_t *y_bs, int64_t N, const int64_t *C, const int64_t *H, const int64_t *W,
+                      const int64_t *OC, int act, hipStream_t st)
+{
+    ODL_REQUIRE(count >= 1 && count <= kGroupMax, "conv2d_fused_group: 1 to %d members, got %d", kGroupMax, count);
+    DirectGroup d{};
+    int64_t blocks = 0;
+    for (int s = 0; s < count; ++s)
+    {
+        ODL_REQUIRE(packed[s] != nullptr && reinterpret_cast<uintptr_t>(packed[s]) % 16 == 0,
+                    "conv2d: the filter copy must be 16-byte aligned");
+        DirectArgs &g = d.g[s];
+        g.x = x[s], g.w = packed[s], g.bias = b ? b[s] : nullptr, g.res = nullptr, g.y = y[s], g.y2 = y[s], g.split = (int)OC[s];
+        g.x_bs = x_bs[s] ? x_bs[s] : C[s] * H[s] * W[s], g.y_bs = y_bs[s] ? y_bs[s] : OC[s] * H[s] * W[s];
+        g.res_bs = g.y_bs, g.y2_bs = g.y_bs;
+        g.C = (int)C[s], g.H = (int)H[s], g.W = (int)W[s], g.OC = (int)OC[s], g.OH = (int)H[s], g.OW = (int)W[s];
+        g.KH = 1, g.KW = 1, g.S = 1, g.P = 0, g.M = (int)(N * H[s] * W[s]), g.act = act;
+        int wp_alone;
+        plan_direct(g.M, OC[s], C[s], 1, g.KS, wp_alone, g.chunks);
+        g.WP = 16 / g.KS;  // (pixel tiles past the last pixel compute on the last pixel's operands and store nothing)
+        g.octiles = (int)ceil_div(OC[s], 32);
+        g.d_ohw = make_fastdiv((unsigned)(H[s] * W[s])), g.d_ow = make_fastdiv((unsigned)W[s]);
+        g.d_chunks = make_fastdiv((unsigned)g.chunks), g.d_kw = make_fastdiv(1u);
+        d.first[s] = (unsigned)blocks;
+        blocks += ceil_div(g.M, 32 * g.WP) * g.octiles;
+        ODL_REQUIRE(blocks < (1ll << 31), "conv2d: too many tiles");
+    }
+    for (int s = count; s <= kGroupMax; ++s)
+        d.first[s] = (unsigned)blocks;
+    const size_t lds = (32 + (size_t)16 * 32 * kPitch) * sizeof(float);
+    hipLaunchKernelGGL(conv_direct_group_kernel, dim3((unsigned)blocks), dim3(1024), lds, st, d, count);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

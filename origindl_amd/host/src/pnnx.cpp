@@ -966,27 +966,50 @@ void PNNXGraph::run(PNNXNode &node)
             const size_t N = run_shape(first)[0];
             std::shared_ptr<Mat> out = std::make_shared<OriginMat>(Shape{N, rows, ci}, DataType::kFloat32, dev);
             std::shared_ptr<Mat> convs[3];
+            std::vector<Shape> xshapes, wshapes;
+            bool packed_all = true;
             for (int s = 0; s < 3; ++s)
             {
-                Value &xv = value(node.input_names[s], node);
-                const Shape xs = run_shape(xv), wsh = ws[s]->shape();
+                const Shape xs = run_shape(value(node.input_names[s], node));
                 Attribute &wa = node.attributes.find("m." + std::to_string(s) + ".weight")->second;
                 if (wa.packed_for != xs.dims())
                 {
                     wa.packed_mat = OriginMat::conv2d_packed_weights_for(xs, *ws[s], {1, 1}, {0, 0});
                     wa.packed_for = xs.dims();
                 }
-                std::shared_ptr<Mat> conv;
-                if (wa.packed_mat && OriginMat::conv2d_fused_ok(xs, wsh, {1, 1}, {0, 0}))
-                {
-                    conv = std::make_shared<OriginMat>(Shape{xs[0], wsh[0], xs[2], xs[3]}, DataType::kFloat32, dev);
-                    OriginMat::conv2d_fused(run_of(xv), *wa.packed_mat, wsh, bs[s].get(), {1, 1}, {0, 0}, -1, nullptr,
-                                            OriginMat::whole(*conv));
-                }
-                else
-                    conv = origin_of(*dense(node.input_names[s], node)).conv2d_act(*ws[s], bs[s].get(), {1, 1}, {0, 0}, -1, wa.packed_mat.get());
-                convs[s] = std::move(conv);
+                packed_all = packed_all && wa.packed_mat;
+                xshapes.push_back(xs), wshapes.push_back(ws[s]->shape());
             }
+            if (packed_all && OriginMat::conv2d_fused_group_ok(xshapes, wshapes))
+            {
+                // (the three convolutions do not depend on each other and each is a launch's latency long: one launch)
+                std::vector<OriginMat::ChannelRun> xr, yr;
+                std::vector<const Mat *> pk, bv;
+                for (int s = 0; s < 3; ++s)
+                {
+                    convs[s] = std::make_shared<OriginMat>(Shape{xshapes[s][0], wshapes[s][0], xshapes[s][2], xshapes[s][3]},
+                                                           DataType::kFloat32, dev);
+                    xr.push_back(run_of(value(node.input_names[s], node))), yr.push_back(OriginMat::whole(*convs[s]));
+                    pk.push_back(node.attributes.find("m." + std::to_string(s) + ".weight")->second.packed_mat.get());
+                    bv.push_back(bs[s].get());
+                }
+                OriginMat::conv2d_fused_group(xr, pk, wshapes, bv, -1, yr);
+            }
+            else
+                for (int s = 0; s < 3; ++s)
+                {
+                    Value &xv = value(node.input_names[s], node);
+                    const Shape &xs = xshapes[s], &wsh = wshapes[s];
+                    Attribute &wa = node.attributes.find("m." + std::to_string(s) + ".weight")->second;
+                    if (wa.packed_mat && OriginMat::conv2d_fused_ok(xs, wsh, {1, 1}, {0, 0}))
+                    {
+                        convs[s] = std::make_shared<OriginMat>(Shape{xs[0], wsh[0], xs[2], xs[3]}, DataType::kFloat32, dev);
+                        OriginMat::conv2d_fused(run_of(xv), *wa.packed_mat, wsh, bs[s].get(), {1, 1}, {0, 0}, -1, nullptr,
+                                                OriginMat::whole(*convs[s]));
+                    }
+                    else
+                        convs[s] = origin_of(*dense(node.input_names[s], node)).conv2d_act(*ws[s], bs[s].get(), {1, 1}, {0, 0}, -1, wa.packed_mat.get());
+                }
             // (one launch for the three stages: each is a chain of a load, sigmoids and a store, shorter than a launch)
             OriginMat::yolo_decode_stages_into({convs[0].get(), convs[1].get(), convs[2].get()}, {gs[0].get(), gs[1].get(), gs[2].get()},
                                                {ags[0].get(), ags[1].get(), ags[2].get()}, strides, 3, (int)ci - 5, *out);

@@ -1560,6 +1560,42 @@ def test_conv_fused_into_channel_runs_equals_the_nodes_one_by_one(api, o, N, C, 
     assert (np.abs(host(api.conv2d(x, w, b, s, p)) - yo) <= by + 1e-6).all()
 
 
+def test_conv_fused_group_gives_each_member_the_floats_of_its_own_call(api):
+    """The stage convolutions of a detect head as one launch: every member bit for bit what conv2d_fused gives it alone
+    (K shares from 1 to 16, a last pixel tile that is ragged or lies wholly past the last pixel, inputs and outputs that
+    are runs of wider tensors, a member without bias)."""
+    rng = np.random.default_rng(77)
+    for N, members, act in ((4, ((64, 40, 40, 255), (128, 20, 20, 255), (256, 10, 10, 255)), None),
+                            (2, ((8, 7, 9, 33), (512, 3, 5, 64)), "silu"),
+                            (1, ((16, 16, 16, 24), (32, 5, 5, 40), (64, 2, 2, 8), (128, 1, 1, 100)), "relu"),
+                            (3, ((24, 11, 6, 70),), None)):
+        xs, ws, pks, bs, ys, wants = [], [], [], [], [], []
+        for i, (C, H, W, OC) in enumerate(members):
+            xbuf = dev(rng.standard_normal((N, C + 8, H, W), dtype=f32))
+            x = xbuf[:, 8:] if i % 2 == 0 else dev(host(xbuf)[:, 8:].copy())
+            w = dev((rng.standard_normal((OC, C, 1, 1), dtype=f32) * f32(0.3)).astype(f32))
+            b = dev(rng.standard_normal(OC, dtype=f32)) if i != 1 else None
+            assert api.conv2d_fused_ok(x.shape, w.shape, 1, 0)
+            pk = api.conv2d_pack_weights(x.shape, w, 1, 0)
+            ybuf = dev(np.full((N, OC + 5, H, W), 3, f32))
+            y = ybuf[:, 2:2 + OC] if i % 2 == 1 else dev(np.full((N, OC, H, W), 3, f32))
+            alone = dev(np.zeros((N, OC, H, W), f32))
+            api.conv2d_fused(x, w.shape, pk, b, alone, 1, 0, act)
+            xs.append(x), ws.append(tuple(w.shape)), pks.append(pk), bs.append(b), ys.append((y, ybuf)), wants.append(host(alone))
+        assert api.conv2d_fused_group_ok([x.shape for x in xs], ws)
+        api.conv2d_fused_group(xs, ws, pks, bs, [y for y, _ in ys], act)
+        for i, ((y, ybuf), want) in enumerate(zip(ys, wants)):
+            assert np.array_equal(host(y), want), (N, members[i])
+            if i % 2 == 1:
+                assert np.all(host(ybuf)[:, :2] == 3) and np.all(host(ybuf)[:, 2 + want.shape[1]:] == 3)
+    assert not api.conv2d_fused_group_ok([(2, 12, 8, 8)], [(16, 12, 1, 1)])                    # channels not a multiple of 8
+    assert not api.conv2d_fused_group_ok([(2, 16, 8, 8)], [(16, 16, 3, 3)])                    # not a 1x1 window
+    assert not api.conv2d_fused_group_ok([(2, 16, 8, 8), (3, 16, 8, 8)], [(16, 16, 1, 1)] * 2)  # batches differ
+    x, y = dev(np.zeros((2, 12, 8, 8), f32)), dev(np.zeros((2, 16, 8, 8), f32))
+    with pytest.raises(api.OdlInvalidArgument):
+        api.conv2d_fused_group([x], [(16, 12, 1, 1)], [dev(np.zeros(16 * 12, f32))], [None], [y])
+
+
 def test_conv_fused_refuses_what_it_does_not_cover(api):
     assert not api.conv2d_fused_ok((2, 3, 64, 64), (16, 3, 6, 6), 2, 2)        # three channels
     assert not api.conv2d_fused_ok((32, 64, 56, 56), (128, 64, 3, 3), 1, 1)    # 14.8 GFLOP: the tiled kernels' work
