@@ -522,6 +522,20 @@ int odl_hip_yolo_decode_stages(int stages, const float *const *host_conv, const 
                                const int64_t *host_anchor_W, int64_t N, const int64_t *host_H, const int64_t *host_W,
                                const float *host_stride, int num_anchors, int num_classes, float *const *host_out,
                                int64_t out_image_stride, void *stream);
+/* Mat::yolo_detect_forward (src/mat/origin/cpu/custom/yolo_detect.cpp:28-166) for the 1 to 4 stages of a head in one
+ * launch: every stage's 1x1 convolution (x[s] a run with its image stride, packed[s] = odl_hip_conv2d_pack_weights of
+ * its filter, host_b NULL or with NULL entries) decoded in the convolution's epilogue and written to out[s], the
+ * stage's first row in the tensor that concatenates the stages (out_image_stride floats from image to image). The
+ * floats are those of odl_hip_conv2d_fused followed by odl_hip_yolo_decode. ..._ok answers 1 for shapes it takes. */
+int odl_hip_yolo_detect_stages_ok(int stages, int64_t N, const int64_t *host_C, const int64_t *host_H, const int64_t *host_W,
+                                  int num_anchors, int num_classes);
+int odl_hip_yolo_detect_stages_forward(int stages, const float *const *host_x, const int64_t *host_x_image_stride,
+                                       const float *const *host_packed, const float *const *host_b, const float *const *host_grid,
+                                       const int64_t *host_grid_elems, const float *const *host_anchor_grid,
+                                       const int64_t *host_anchor_elems, const int64_t *host_anchor_H, const int64_t *host_anchor_W,
+                                       int64_t N, const int64_t *host_C, const int64_t *host_H, const int64_t *host_W,
+                                       const float *host_stride, int num_anchors, int num_classes, float *const *host_out,
+                                       int64_t out_image_stride, void *stream);
 
 /* Mat::batch_norm_forward / Mat::batch_norm (mat.h:603-631; src/mat/origin/cpu/normalization/batch_norm.cpp:31-258)
  * over x[N, C, P]: P = H*W for num_dims 4, P = 1 for num_dims 2. training != 0: per-channel mean and biased variance

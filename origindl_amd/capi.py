@@ -842,6 +842,45 @@ def yolo_decode_stages(convs, grids, anchor_grids, strides, num_anchors, num_cla
     return out
 
 
+def yolo_detect_stages_ok(x_shapes, num_anchors, num_classes):
+    S = len(x_shapes)
+    if not (1 <= S <= 4) or any(len(x) != 4 or int(x[0]) != int(x_shapes[0][0]) for x in x_shapes):
+        return False
+    i64 = lambda vs: (ctypes.c_int64 * S)(*[int(v) for v in vs])
+    return lib().query("odl_hip_yolo_detect_stages_ok", S, int(x_shapes[0][0]), i64(x[1] for x in x_shapes), i64(x[2] for x in x_shapes),
+                       i64(x[3] for x in x_shapes), num_anchors, num_classes) == 1
+
+
+def yolo_detect_stages_forward(xs, packeds, bs, grids, anchor_grids, strides, num_anchors, num_classes, out):
+    """Mat::yolo_detect_forward (src/mat/origin/cpu/custom/yolo_detect.cpp:28-166) for every stage of a head in one
+    launch, stage s written behind stage s - 1 into out[N, rows, classes+5]: conv2d_fused then yolo_decode, bit for bit."""
+    S = len(xs)
+    if not (1 <= S <= 4) or any(len(v) != S for v in (packeds, bs, grids, anchor_grids, strides)):
+        raise OdlInvalidArgument("yolo_detect_stages_forward: 1 to 4 stages with a filter copy, a bias (or None), a grid, an anchor grid and a stride each")
+    _chk(out, "out")
+    CI = num_classes + 5
+    N = int(out.shape[0])
+    xst = [_run(x, "x") for x in xs]
+    outs, row0, aHs, aWs = [], 0, [], []
+    for x, a in zip(xs, anchor_grids):
+        if x.shape[0] != N:
+            raise OdlInvalidArgument("yolo_detect_stages_forward: a stage's batch differs from the output's")
+        H, W = int(x.shape[2]), int(x.shape[3])
+        aHs.append(int(a.shape[2]) if a.dim() >= 3 else H), aWs.append(int(a.shape[3]) if a.dim() >= 4 else W)
+        outs.append(out.data_ptr() + row0 * CI * 4)
+        row0 += num_anchors * H * W
+    if out.dim() != 3 or out.shape[2] != CI or row0 > out.shape[1]:
+        raise OdlInvalidArgument("yolo_detect_stages_forward: out must be [%d, >= %d, %d]" % (N, row0, CI))
+    ptr = lambda ts: (ctypes.c_void_p * S)(*[None if t is None else t.data_ptr() for t in ts])
+    i64 = lambda vs: (ctypes.c_int64 * S)(*[int(v) for v in vs])
+    lib().call("odl_hip_yolo_detect_stages_forward", S, ptr(xs), i64(xst), ptr(packeds), ptr(bs), ptr(grids),
+               i64(g.numel() for g in grids), ptr(anchor_grids), i64(a.numel() for a in anchor_grids), i64(aHs), i64(aWs), N,
+               i64(x.shape[1] for x in xs), i64(x.shape[2] for x in xs), i64(x.shape[3] for x in xs),
+               (ctypes.c_float * S)(*[float(v) for v in strides]), num_anchors, num_classes, (ctypes.c_void_p * S)(*outs),
+               int(out.shape[1]) * CI, _stream())
+    return out
+
+
 def _bn_dims(x, who):
     if x.dim() not in (2, 4):
         raise OdlInvalidArgument("%s: x must have 2 or 4 dimensions, but got shape %s" % (who, tuple(x.shape)))

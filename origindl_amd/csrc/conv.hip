@@ -106,9 +106,6 @@ bool conv_direct_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int 
                     int64_t OH, int64_t OW);
 size_t conv_direct_packed_bytes(int64_t C, int64_t OC, int KH, int KW, int P, int64_t W);
 int conv_direct_pack(const float *w, int64_t C, int64_t OC, int KH, int KW, int P, int64_t W, float *packed, hipStream_t st);
-int conv_direct_group(int count, const float *const *x, const int64_t *x_bs, const float *const *packed, const float *const *b,
-                      float *const *y, const int64_t *y_bs, int64_t N, const int64_t *C, const int64_t *H, const int64_t *W,
-                      const int64_t *OC, int act, hipStream_t st);
 int conv_direct(const float *x, int64_t x_bs, const float *packed, const float *b, const float *res, int64_t res_bs, float *y,
                 int64_t y_bs, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int S, int P, int64_t OH,
                 int64_t OW, int act, hipStream_t st, float *y2 = nullptr, int64_t y2_bs = 0, int64_t split = 0);

@@ -35,6 +35,14 @@ struct DirectArgs
     int chunks;        // channel groups of eight per K share
     int octiles;
     odl::FastDiv d_ohw, d_ow, d_chunks, d_kw;
+    // A detect stage (the DET kernels only): the filters are [anchor][classes + 5]; every output goes through the sigmoid
+    // and the box decoding and is stored to rows[n][anchor * OH * OW + pixel][channel] instead of y.
+    const float *det_grid, *det_anchor;
+    float *det_rows;
+    int64_t det_grid_elems, det_anchor_elems, det_rows_bs;
+    float det_stride;
+    int det_CI, det_aH, det_aW;
+    odl::FastDiv d_ci;
 };
 
 #ifdef ODL_DIRECT_DBG
@@ -108,14 +116,81 @@ __device__ __forceinline__ void direct_epilogue(const DirectArgs &g, const float
             (second[i] ? g.y2 : g.y)[off[i]] = v[i];
 }
 
+// The same sums for a detect stage: bias, then the steps of the decoding kernel (sigmoid as -x, exp, 1 + ., 1 / .; boxes
+// (2s + grid) * stride and (2s)^2 * anchor) on every output, stored as rows [pixel][channel]: 32 consecutive threads
+// along the channels of one pixel, so a store covers consecutive floats of a row.
+template <int E>
+__device__ __forceinline__ void direct_epilogue_detect(const DirectArgs &g, const float *partial, const float *bias_s, int m_base,
+                                                       int oc0, int OHW)
+{
+    const int nthreads = 64 * g.KS * g.WP;
+#pragma unroll
+    for (int i = 0; i < E; ++i)
+    {
+        const int e = threadIdx.x + i * nthreads;
+        const int tp = e >> 10, col = (e >> 5) & 31, rr = e & 31;
+        const int mm = m_base + tp * 32 + col, oc = oc0 + rr;
+        if (mm >= g.M || oc >= g.OC)
+            continue;
+        const float *src = partial + ((size_t)tp * g.KS * 32 + rr) * kPitch + col;
+        float a = src[0];
+        for (int s = 1; s < g.KS; ++s)
+            a += src[(size_t)s * 32 * kPitch];
+        float v = 1.0f / (1.0f + expf(-(a + bias_s[rr])));
+        const unsigned nn = odl::fastdiv((unsigned)mm, g.d_ohw), px = (unsigned)mm - nn * (unsigned)OHW;
+        const int anc = (int)odl::fastdiv((unsigned)oc, g.d_ci), c = oc - anc * g.det_CI;
+        if (c < 4)
+        {
+            const int h = (int)odl::fastdiv(px, g.d_ow), w = (int)px - h * g.OW;
+            const float t = v * 2.0f;
+            if (c < 2)
+            {
+                const int64_t gi = ((int64_t)anc * OHW + (int64_t)h * g.OW + w) * 2 + c;
+                v = (t + (gi < g.det_grid_elems ? g.det_grid[gi] : 0.0f)) * g.det_stride;
+            }
+            else
+            {
+                const int sh_ = (g.det_aH > 0 && g.OH > g.det_aH) ? g.OH / g.det_aH : 1;
+                const int sw_ = (g.det_aW > 0 && g.OW > g.det_aW) ? g.OW / g.det_aW : 1;
+                int ah = h / sh_, aw = w / sw_;
+                ah = ah < g.det_aH - 1 ? ah : g.det_aH - 1;
+                aw = aw < g.det_aW - 1 ? aw : g.det_aW - 1;
+                const int64_t ai = ((int64_t)anc * g.det_aH * g.det_aW + (int64_t)ah * g.det_aW + aw) * 2 + (c - 2);
+                v = (t * t) * (ai < g.det_anchor_elems ? g.det_anchor[ai] : 1.0f);
+            }
+        }
+        g.det_rows[(int64_t)nn * g.det_rows_bs + ((int64_t)anc * OHW + px) * g.det_CI + c] = v;
+    }
+}
+
 // What follows the K loop: the tile's sums (this wave's share of K in acc) to their places in y.
-template <bool RES>
+template <bool RES, bool DET = false>
 __device__ __forceinline__ void direct_finish(const DirectArgs &g, const f32x16 &acc, float bias_v, float *bias_s, float *partial,
                                               int wv, int pt, int l32, int half, int m_base, int oc0, int OHW, unsigned n, unsigned r)
 {
     ODL_DIRECT_STAMP(3);
     if (threadIdx.x < 32)
         bias_s[threadIdx.x] = bias_v;
+    if (DET)
+    {
+        // (through LDS whatever the number of K shares: the rows are written along the channels, the lanes hold pixels)
+        float *mine = partial + (size_t)wv * 32 * kPitch;
+#pragma unroll
+        for (int q = 0; q < 16; ++q)
+            mine[(8 * (q / 4) + 4 * half + (q % 4)) * kPitch + l32] = acc[q];
+        __syncthreads();
+        if (g.KS == 1)
+            direct_epilogue_detect<16>(g, partial, bias_s, m_base, oc0, OHW);
+        else if (g.KS == 2)
+            direct_epilogue_detect<8>(g, partial, bias_s, m_base, oc0, OHW);
+        else if (g.KS == 4)
+            direct_epilogue_detect<4>(g, partial, bias_s, m_base, oc0, OHW);
+        else if (g.KS == 8)
+            direct_epilogue_detect<2>(g, partial, bias_s, m_base, oc0, OHW);
+        else
+            direct_epilogue_detect<1>(g, partial, bias_s, m_base, oc0, OHW);
+        return;
+    }
     if (g.KS == 1)
     {
         // accumulator register q of a lane: row 8*(q/4) + 4*half + q%4, column l32
@@ -173,7 +248,7 @@ __device__ __forceinline__ void direct_finish(const DirectArgs &g, const f32x16 
 // kDepth: operand groups in flight per wave. Every load instruction costs the compute unit's one address unit 16
 // clocks whether or not its data is used, so the depth divides the group count (3 for 3x3 windows, 4 otherwise) and no
 // group is loaded twice.
-template <int kDepth, bool RES>
+template <int kDepth, bool RES, bool DET = false>
 __device__ __forceinline__ void conv_direct_tile(const DirectArgs &g, const unsigned bid)
 {
     extern __shared__ float lds[];  // bias[32], then partial[WP * KS][32][kPitch] when KS > 1
@@ -249,7 +324,7 @@ __device__ __forceinline__ void conv_direct_tile(const DirectArgs &g, const unsi
     for (int d = 0; d < kDepth; ++d)
         if (d < rem)
             use(d);
-    direct_finish<RES>(g, acc, bias_v, bias_s, partial, wv, pt, l32, half, m_base, oc0, OHW, n, r);
+    direct_finish<RES, DET>(g, acc, bias_v, bias_s, partial, wv, pt, l32, half, m_base, oc0, OHW, n, r);
 }
 
 template <int kDepth, bool RES>
@@ -269,12 +344,13 @@ struct DirectGroup
     unsigned first[kGroupMax + 1];
 };
 
+template <bool DET>
 __global__ __launch_bounds__(1024) void conv_direct_group_kernel(DirectGroup d, int count)
 {
     int s = 0;
     for (int j = 1; j < count; ++j)
         s = blockIdx.x >= d.first[j] ? j : s;
-    conv_direct_tile<4, false>(d.g[s], blockIdx.x - d.first[s]);
+    conv_direct_tile<4, false, DET>(d.g[s], blockIdx.x - d.first[s]);
 }
 
 // 3x3 windows with padding 1 (stride 1 or 2, rows of three pixels or more): the three taps of a window row are three
@@ -487,7 +563,7 @@ namespace odl
 {
 int conv_direct_group(int count, const float *const *x, const int64_t *x_bs, const float *const *packed, const float *const *b,
                       float *const *y, const int64_t *y_bs, int64_t N, const int64_t *C, const int64_t *H, const int64_t *W,
-                      const int64_t *OC, int act, hipStream_t st)
+                      const int64_t *OC, int act, hipStream_t st, const DetectRows *det)
 {
     ODL_REQUIRE(count >= 1 && count <= kGroupMax, "conv2d_fused_group: 1 to %d members, got %d", kGroupMax, count);
     DirectGroup d{};
@@ -497,8 +573,16 @@ int conv_direct_group(int count, const float *const *x, const int64_t *x_bs, con
         ODL_REQUIRE(packed[s] != nullptr && reinterpret_cast<uintptr_t>(packed[s]) % 16 == 0,
                     "conv2d: the filter copy must be 16-byte aligned");
         DirectArgs &g = d.g[s];
-        g.x = x[s], g.w = packed[s], g.bias = b ? b[s] : nullptr, g.res = nullptr, g.y = y[s], g.y2 = y[s], g.split = (int)OC[s];
-        g.x_bs = x_bs[s] ? x_bs[s] : C[s] * H[s] * W[s], g.y_bs = y_bs[s] ? y_bs[s] : OC[s] * H[s] * W[s];
+        g.x = x[s], g.w = packed[s], g.bias = b ? b[s] : nullptr, g.res = nullptr, g.split = (int)OC[s];
+        g.y = det ? nullptr : y[s], g.y2 = g.y;
+        g.x_bs = x_bs[s] ? x_bs[s] : C[s] * H[s] * W[s], g.y_bs = (!det && y_bs[s]) ? y_bs[s] : OC[s] * H[s] * W[s];
+        if (det)
+        {
+            g.det_grid = det[s].grid, g.det_anchor = det[s].anchor_grid, g.det_rows = det[s].rows;
+            g.det_grid_elems = det[s].grid_elems, g.det_anchor_elems = det[s].anchor_elems, g.det_rows_bs = det[s].rows_image_stride;
+            g.det_stride = det[s].stride, g.det_CI = det[s].CI, g.det_aH = det[s].anchor_H, g.det_aW = det[s].anchor_W;
+            g.d_ci = make_fastdiv((unsigned)det[s].CI);
+        }
         g.res_bs = g.y_bs, g.y2_bs = g.y_bs;
         g.C = (int)C[s], g.H = (int)H[s], g.W = (int)W[s], g.OC = (int)OC[s], g.OH = (int)H[s], g.OW = (int)W[s];
         g.KH = 1, g.KW = 1, g.S = 1, g.P = 0, g.M = (int)(N * H[s] * W[s]), g.act = act;
@@ -515,7 +599,10 @@ int conv_direct_group(int count, const float *const *x, const int64_t *x_bs, con
     for (int s = count; s <= kGroupMax; ++s)
         d.first[s] = (unsigned)blocks;
     const size_t lds = (32 + (size_t)16 * 32 * kPitch) * sizeof(float);
-    hipLaunchKernelGGL(conv_direct_group_kernel, dim3((unsigned)blocks), dim3(1024), lds, st, d, count);
+    if (det)
+        hipLaunchKernelGGL(conv_direct_group_kernel<true>, dim3((unsigned)blocks), dim3(1024), lds, st, d, count);
+    else
+        hipLaunchKernelGGL(conv_direct_group_kernel<false>, dim3((unsigned)blocks), dim3(1024), lds, st, d, count);
     ODL_LAUNCH_CHECK();
     return ODL_OK;
 }

@@ -587,6 +587,59 @@ int odl_hip_yolo_decode_stages(int stages, const float *const *host_conv, const 
     return ODL_OK;
 }
 
+int odl_hip_yolo_detect_stages_ok(int stages, int64_t N, const int64_t *host_C, const int64_t *host_H, const int64_t *host_W,
+                                  int num_anchors, int num_classes)
+{
+    if (stages < 1 || stages > kMaxStages || N <= 0 || num_anchors <= 0 || num_classes < 0 || !host_C || !host_H || !host_W)
+        return 0;
+    const int64_t OC = (int64_t)num_anchors * (num_classes + 5);
+    for (int s = 0; s < stages; ++s)
+        if (host_C[s] <= 0 || host_H[s] <= 0 || host_W[s] <= 0 ||
+            !odl::conv_direct_ok(N, host_C[s], host_H[s], host_W[s], OC, 1, 1, 1, 1, 0, 0, host_H[s], host_W[s]))
+            return 0;
+    return 1;
+}
+
+int odl_hip_yolo_detect_stages_forward(int stages, const float *const *host_x, const int64_t *host_x_image_stride,
+                                       const float *const *host_packed, const float *const *host_b, const float *const *host_grid,
+                                       const int64_t *host_grid_elems, const float *const *host_anchor_grid,
+                                       const int64_t *host_anchor_elems, const int64_t *host_anchor_H, const int64_t *host_anchor_W,
+                                       int64_t N, const int64_t *host_C, const int64_t *host_H, const int64_t *host_W,
+                                       const float *host_stride, int num_anchors, int num_classes, float *const *host_out,
+                                       int64_t out_image_stride, void *stream)
+{
+    ODL_REQUIRE_DEVICE();
+    ODL_REQUIRE(stages >= 1 && stages <= kMaxStages, "yolo_detect_stages_forward: 1 to %d stages, got %d", kMaxStages, stages);
+    ODL_REQUIRE(host_x && host_x_image_stride && host_packed && host_grid && host_grid_elems && host_anchor_grid && host_anchor_elems &&
+                    host_anchor_H && host_anchor_W && host_C && host_H && host_W && host_stride && host_out,
+                "yolo_detect_stages_forward: null argument");
+    ODL_REQUIRE(N >= 0 && num_anchors > 0 && num_classes >= 0, "yolo_detect_stages_forward: bad shape");
+    if (N == 0)
+        return ODL_OK;
+    ODL_REQUIRE(odl_hip_yolo_detect_stages_ok(stages, N, host_C, host_H, host_W, num_anchors, num_classes),
+                "yolo_detect_stages_forward: shape not covered (ask odl_hip_yolo_detect_stages_ok first)");
+    const int CI = num_classes + 5;
+    odl::DetectRows det[kMaxStages];
+    int64_t OC[kMaxStages];
+    for (int s = 0; s < stages; ++s)
+    {
+        ODL_REQUIRE(host_x[s] && host_packed[s] && host_grid[s] && host_anchor_grid[s] && host_out[s],
+                    "yolo_detect_stages_forward: null operand of stage %d", s);
+        ODL_REQUIRE(host_grid_elems[s] >= 0 && host_anchor_elems[s] >= 0 && host_anchor_H[s] > 0 && host_anchor_W[s] > 0,
+                    "yolo_detect_stages_forward: bad grid sizes of stage %d", s);
+        const int64_t rows = (int64_t)num_anchors * host_H[s] * host_W[s] * CI;
+        const int64_t os = out_image_stride ? out_image_stride : rows;
+        ODL_REQUIRE(os >= rows, "yolo_detect_stages_forward: the output image stride is shorter than the rows of stage %d", s);
+        ODL_REQUIRE(host_x_image_stride[s] == 0 || (host_x_image_stride[s] >= host_C[s] * host_H[s] * host_W[s] && host_x_image_stride[s] < (1ll << 40)),
+                    "yolo_detect_stages_forward: bad input image stride of stage %d", s);
+        det[s] = odl::DetectRows{host_grid[s], host_anchor_grid[s], host_out[s], host_grid_elems[s], host_anchor_elems[s], os,
+                                 host_stride[s], CI, (int)host_anchor_H[s], (int)host_anchor_W[s]};
+        OC[s] = (int64_t)num_anchors * CI;
+    }
+    return odl::conv_direct_group(stages, host_x, host_x_image_stride, host_packed, host_b, nullptr, nullptr, N, host_C, host_H, host_W,
+                                  OC, 0, odl::as_stream(stream), det);
+}
+
 size_t odl_hip_yolo_detect_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int num_anchors, int num_classes)
 {
     if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || num_anchors <= 0 || num_classes < 0)

@@ -69,6 +69,24 @@ __device__ inline unsigned fastdiv(unsigned m, const FastDiv &f)
     return (t + ((m - t) >> f.sh1)) >> f.sh2;
 }
 
+// A detect stage whose 1x1 convolution writes decoded rows: what decodes them (grid, anchor grid, stride; CI = classes
+// + 5 channels per anchor) and where they go (rows[n * rows_image_stride + (anchor * H * W + pixel) * CI + channel]).
+struct DetectRows
+{
+    const float *grid, *anchor_grid;
+    float *rows;
+    int64_t grid_elems, anchor_elems, rows_image_stride;
+    float stride;
+    int CI, anchor_H, anchor_W;
+};
+// One to four 1x1 convolutions in one launch (conv_direct.hip); with det, member s's outputs are decoded into det[s].rows
+// instead of stored to y[s] (y and y_bs are then not read).
+int conv_direct_group(int count, const float *const *x, const int64_t *x_bs, const float *const *packed, const float *const *b,
+                      float *const *y, const int64_t *y_bs, int64_t N, const int64_t *C, const int64_t *H, const int64_t *W,
+                      const int64_t *OC, int act, hipStream_t st, const DetectRows *det = nullptr);
+bool conv_direct_ok(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int KH, int KW, int SH, int SW, int PH, int PW,
+                    int64_t OH, int64_t OW);
+
 // the activations a convolution's epilogue can apply (0 none, 1 relu, 2 silu); the expressions are those of the
 // standalone unary kernels
 __device__ inline float apply_act(float v, int act)

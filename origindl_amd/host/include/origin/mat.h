@@ -400,6 +400,14 @@ public:
     // [row0, row0 + A*H*W) of out[N, rows, classes+5]: the second half of yolo_detect_forward
     void yolo_decode_into(const Mat &grid, const Mat &anchor_grid, float stride, int32_t num_anchors, int32_t num_classes,
                           Mat &out, size_t row0) const;
+    // yolo_detect_forward of every stage of a head in one launch: the stages' 1x1 convolutions (x[s] a run, packed[s] the
+    // filter copy conv2d_packed_weights made for it, b[s] a bias or null) decoded in their epilogues into out[N, rows,
+    // classes+5], stage s behind stage s - 1. stages_ok: whether the input shapes are covered
+    static bool yolo_detect_stages_ok(const std::vector<Shape> &x_run_shapes, int32_t num_anchors, int32_t num_classes);
+    static void yolo_detect_stages(const std::vector<ChannelRun> &x, const std::vector<const Mat *> &packed,
+                                   const std::vector<const Mat *> &b, const std::vector<const Mat *> &grid,
+                                   const std::vector<const Mat *> &anchor_grid, const std::vector<float> &stride, int32_t num_anchors,
+                                   int32_t num_classes, Mat &out);
     // the same for every stage of a head in one launch: conv[s] into the rows that follow those of conv[s - 1], from row 0
     static void yolo_decode_stages_into(const std::vector<const Mat *> &conv, const std::vector<const Mat *> &grid,
                                         const std::vector<const Mat *> &anchor_grid, const std::vector<float> &stride,

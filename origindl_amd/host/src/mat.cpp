@@ -1532,6 +1532,74 @@ void OriginMat::yolo_decode_into(const Mat &grid, const Mat &anchor_grid, float 
                               cur()));
 }
 
+bool OriginMat::yolo_detect_stages_ok(const std::vector<Shape> &xs, int32_t num_anchors, int32_t num_classes)
+{
+    const size_t S = xs.size();
+    if (S == 0 || S > 4)
+        return false;
+    int64_t C[4], H[4], W[4];
+    for (size_t s = 0; s < S; ++s)
+    {
+        if (xs[s].size() != 4 || xs[s][0] != xs[0][0])
+            return false;
+        C[s] = xs[s][1], H[s] = xs[s][2], W[s] = xs[s][3];
+    }
+    return odl_hip_yolo_detect_stages_ok((int)S, (int64_t)xs[0][0], C, H, W, num_anchors, num_classes) == 1;
+}
+
+void OriginMat::yolo_detect_stages(const std::vector<ChannelRun> &xr, const std::vector<const Mat *> &packed,
+                                   const std::vector<const Mat *> &bm, const std::vector<const Mat *> &grid,
+                                   const std::vector<const Mat *> &anchor_grid, const std::vector<float> &stride, int32_t num_anchors,
+                                   int32_t num_classes, Mat &out_m)
+{
+    const size_t S = xr.size();
+    if (S == 0 || S > 4 || packed.size() != S || bm.size() != S || grid.size() != S || anchor_grid.size() != S || stride.size() != S)
+        THROW_INVALID_ARG("yolo_detect_forward: 1 to 4 stages with a filter copy, a bias (or null), a grid, an anchor grid and a stride each, got {}", S);
+    const OriginMat &out = dev_f32(out_m, "yolo_detect_forward");
+    const int64_t CI = num_classes + 5, OC = num_anchors * CI;
+    const Shape &os = out.shape();
+    if (os.size() != 3 || (int64_t)os[2] != CI)
+        THROW_INVALID_ARG("yolo_detect_forward: the output must be [N, rows, {}], got {}", CI, os.to_string());
+    const int64_t N = os[0];
+    const float *xp[4], *pp[4], *bp[4], *gp[4], *ap[4];
+    float *op[4];
+    int64_t xs[4], ge[4], ae[4], aH[4], aW[4], C[4], H[4], W[4];
+    size_t row0 = 0;
+    for (size_t s = 0; s < S; ++s)
+    {
+        const RunPtr x = run_ptr(xr[s], "yolo_detect_forward");
+        if (x.N != N)
+            THROW_INVALID_ARG("yolo_detect_forward: stage {} has {} images, the output {}", s, x.N, N);
+        if (!packed[s] || !grid[s] || !anchor_grid[s])
+            THROW_INVALID_ARG("yolo_detect_forward: stage {} lacks one of filter copy / grid / anchor grid", s);
+        const OriginMat &pk = dev_f32(*packed[s], "yolo_detect_forward");
+        const size_t want = odl_hip_conv2d_packed_weights_bytes(x.N, x.C, x.H, x.W, OC, 1, 1, 1, 1, 0, 0);
+        if (want == 0 || pk.elements() * sizeof(float) != want)
+            THROW_INVALID_ARG("yolo_detect_forward: the packed filter has {} bytes, this shape's kernel reads {}", pk.elements() * sizeof(float), want);
+        bp[s] = nullptr;
+        if (bm[s])
+        {
+            const OriginMat &b = dev_f32(*bm[s], "yolo_detect_forward");
+            if (b.shape().size() != 1 || (int64_t)b.shape()[0] != OC)
+                THROW_INVALID_ARG("yolo_detect_forward: b must be 1D with size {}, but got shape {}", OC, b.shape().to_string());
+            bp[s] = fp(b);
+        }
+        const OriginMat &g = dev_f32(*grid[s], "yolo_detect_forward");
+        const OriginMat &ag = dev_f32(*anchor_grid[s], "yolo_detect_forward");
+        if (row0 + (size_t)(num_anchors * x.H * x.W) > os[1])
+            THROW_INVALID_ARG("yolo_detect_forward: rows [{}, {}) do not lie in an output of shape {}", row0,
+                              row0 + num_anchors * x.H * x.W, os.to_string());
+        const Shape as = ag.shape();
+        aH[s] = as.size() >= 3 ? (int64_t)as[2] : x.H, aW[s] = as.size() >= 4 ? (int64_t)as[3] : x.W;
+        xp[s] = x.data, xs[s] = x.image_stride, pp[s] = fp(pk), gp[s] = fp(g), ap[s] = fp(ag);
+        ge[s] = (int64_t)g.elements(), ae[s] = (int64_t)ag.elements(), C[s] = x.C, H[s] = x.H, W[s] = x.W;
+        op[s] = const_cast<float *>(fp(out)) + (int64_t)row0 * CI;
+        row0 += (size_t)(num_anchors * x.H * x.W);
+    }
+    check(odl_hip_yolo_detect_stages_forward((int)S, xp, xs, pp, bp, gp, ge, ap, ae, aH, aW, N, C, H, W, stride.data(), num_anchors,
+                                             num_classes, op, (int64_t)(os[1] * os[2]), cur()));
+}
+
 void OriginMat::yolo_decode_stages_into(const std::vector<const Mat *> &conv_m, const std::vector<const Mat *> &grid,
                                         const std::vector<const Mat *> &anchor_grid, const std::vector<float> &stride,
                                         int32_t num_anchors, int32_t num_classes, Mat &out_m)

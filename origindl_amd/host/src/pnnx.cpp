@@ -980,6 +980,23 @@ void PNNXGraph::run(PNNXNode &node)
                 packed_all = packed_all && wa.packed_mat;
                 xshapes.push_back(xs), wshapes.push_back(ws[s]->shape());
             }
+            if (packed_all && OriginMat::yolo_detect_stages_ok(xshapes, 3, (int)ci - 5))
+            {
+                // (the stages do not depend on each other and each is a launch's latency long: one launch for the three
+                // convolutions, which decode their sums themselves)
+                std::vector<OriginMat::ChannelRun> xr;
+                std::vector<const Mat *> pk, bv;
+                for (int s = 0; s < 3; ++s)
+                {
+                    xr.push_back(run_of(value(node.input_names[s], node)));
+                    pk.push_back(node.attributes.find("m." + std::to_string(s) + ".weight")->second.packed_mat.get());
+                    bv.push_back(bs[s].get());
+                }
+                OriginMat::yolo_detect_stages(xr, pk, bv, {gs[0].get(), gs[1].get(), gs[2].get()},
+                                              {ags[0].get(), ags[1].get(), ags[2].get()}, strides, 3, (int)ci - 5, *out);
+                store(node, std::move(out));
+                return;
+            }
             if (packed_all && OriginMat::conv2d_fused_group_ok(xshapes, wshapes))
             {
                 // (the three convolutions do not depend on each other and each is a launch's latency long: one launch)

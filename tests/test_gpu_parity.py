@@ -1596,6 +1596,49 @@ def test_conv_fused_group_gives_each_member_the_floats_of_its_own_call(api):
         api.conv2d_fused_group([x], [(16, 12, 1, 1)], [dev(np.zeros(16 * 12, f32))], [None], [y])
 
 
+def test_detect_head_in_one_launch_equals_convolution_then_decoding(api):
+    """Every stage of a detect head as one launch, the decoding in the convolutions' epilogues: the floats of
+    conv2d_fused followed by yolo_decode for each stage (K shares from 1 to 16, ragged pixel tiles, an anchor grid
+    coarser than the stage, inputs that are runs of wider tensors, a stage without bias, few and many classes)."""
+    rng = np.random.default_rng(78)
+    for N, A, NC, members in ((4, 3, 80, ((64, 40, 40), (128, 20, 20), (256, 10, 10))),
+                              (2, 2, 1, ((8, 7, 9), (512, 3, 5))),
+                              (1, 3, 6, ((16, 16, 16), (32, 6, 4), (64, 2, 2), (128, 1, 1))),
+                              (3, 1, 0, ((24, 11, 6),))):
+        CI = A * 0 + NC + 5
+        OC = A * CI
+        xs, pks, bs, grids, ags, strides, convs = [], [], [], [], [], [], []
+        for i, (C, H, W) in enumerate(members):
+            xbuf = dev(rng.standard_normal((N, C + 8, H, W), dtype=f32))
+            x = xbuf[:, 8:] if i % 2 == 0 else dev(host(xbuf)[:, 8:].copy())
+            w = dev((rng.standard_normal((OC, C, 1, 1), dtype=f32) * f32(0.3)).astype(f32))
+            b = dev(rng.standard_normal(OC, dtype=f32)) if i != 1 else None
+            pk = api.conv2d_pack_weights(x.shape, w, 1, 0)
+            conv = dev(np.zeros((N, OC, H, W), f32))
+            api.conv2d_fused(x, w.shape, pk, b, conv, 1, 0, None)
+            gyy, gxx = np.meshgrid(np.arange(H), np.arange(W), indexing="ij")
+            grids.append(dev(np.broadcast_to(np.stack([gxx, gyy], -1).astype(f32) - f32(0.5), (1, A, H, W, 2)).copy()))
+            aH, aW = (H, W) if i != 2 else (max(H // 2, 1), max(W // 2, 1))  # (one stage with an anchor grid at half the size)
+            ags.append(dev((rng.random((1, A, aH, aW, 2), dtype=f32) * f32(90) + f32(4)).astype(f32)))
+            xs.append(x), pks.append(pk), bs.append(b), strides.append(float(8 << i)), convs.append(conv)
+        assert api.yolo_detect_stages_ok([x.shape for x in xs], A, NC)
+        rows = sum(A * x.shape[2] * x.shape[3] for x in xs)
+        one, each = dev(np.full((N, rows + 9, CI), 7, f32)), dev(np.full((N, rows + 9, CI), 7, f32))
+        api.yolo_detect_stages_forward(xs, pks, bs, grids, ags, strides, A, NC, one)
+        r0 = 0
+        for c, g, a, st in zip(convs, grids, ags, strides):
+            r = A * c.shape[2] * c.shape[3]
+            api.yolo_decode(c, g, a, st, A, NC, each[:, r0:r0 + r])
+            r0 += r
+        assert np.array_equal(host(one), host(each)), (N, A, NC, members)
+    assert not api.yolo_detect_stages_ok([(2, 12, 8, 8)], 3, 80)                 # channels not a multiple of 8
+    assert not api.yolo_detect_stages_ok([(2, 16, 8, 8), (3, 16, 4, 4)], 3, 80)  # batches differ
+    with pytest.raises(api.OdlInvalidArgument):
+        api.yolo_detect_stages_forward([dev(np.zeros((2, 12, 8, 8), f32))], [dev(np.zeros(16 * 255, f32))], [None],
+                                       [dev(np.zeros((1, 3, 8, 8, 2), f32))], [dev(np.ones((1, 3, 8, 8, 2), f32))], [8.0], 3, 80,
+                                       dev(np.zeros((2, 192, 85), f32)))
+
+
 def test_conv_fused_refuses_what_it_does_not_cover(api):
     assert not api.conv2d_fused_ok((2, 3, 64, 64), (16, 3, 6, 6), 2, 2)        # three channels
     assert not api.conv2d_fused_ok((32, 64, 56, 56), (128, 64, 3, 3), 1, 1)    # 14.8 GFLOP: the tiled kernels' work
