@@ -123,43 +123,48 @@ template <int E>
 __device__ __forceinline__ void direct_epilogue_detect(const DirectArgs &g, const float *partial, const float *bias_s, int m_base,
                                                        int oc0, int OHW)
 {
-    const int nthreads = 64 * g.KS * g.WP;
+    // sixteen waves: a thread keeps its channel and its pixel column for all of its E outputs, one per pixel tile
+    const int col = (int)(threadIdx.x >> 5), rr = (int)(threadIdx.x & 31);
+    const int oc = oc0 + rr;
+    if (oc >= g.OC)
+        return;
+    const int anc = (int)odl::fastdiv((unsigned)oc, g.d_ci), c = oc - anc * g.det_CI;
+    const float bias = bias_s[rr];
+    const int sh_ = (g.det_aH > 0 && g.OH > g.det_aH) ? g.OH / g.det_aH : 1;
+    const int sw_ = (g.det_aW > 0 && g.OW > g.det_aW) ? g.OW / g.det_aW : 1;
+    float *rows = g.det_rows + (int64_t)anc * OHW * g.det_CI + c;
 #pragma unroll
     for (int i = 0; i < E; ++i)
     {
-        const int e = threadIdx.x + i * nthreads;
-        const int tp = e >> 10, col = (e >> 5) & 31, rr = e & 31;
-        const int mm = m_base + tp * 32 + col, oc = oc0 + rr;
-        if (mm >= g.M || oc >= g.OC)
-            continue;
-        const float *src = partial + ((size_t)tp * g.KS * 32 + rr) * kPitch + col;
-        float a = src[0];
-        for (int s = 1; s < g.KS; ++s)
-            a += src[(size_t)s * 32 * kPitch];
-        float v = 1.0f / (1.0f + expf(-(a + bias_s[rr])));
-        const unsigned nn = odl::fastdiv((unsigned)mm, g.d_ohw), px = (unsigned)mm - nn * (unsigned)OHW;
-        const int anc = (int)odl::fastdiv((unsigned)oc, g.d_ci), c = oc - anc * g.det_CI;
-        if (c < 4)
+        const int mm = m_base + i * 32 + col;
+        if (mm < g.M)
         {
-            const int h = (int)odl::fastdiv(px, g.d_ow), w = (int)px - h * g.OW;
-            const float t = v * 2.0f;
-            if (c < 2)
+            const float *src = partial + ((size_t)i * g.KS * 32 + rr) * kPitch + col;
+            float a = src[0];
+            for (int s = 1; s < g.KS; ++s)
+                a += src[(size_t)s * 32 * kPitch];
+            float v = 1.0f / (1.0f + expf(-(a + bias)));
+            const unsigned nn = odl::fastdiv((unsigned)mm, g.d_ohw), px = (unsigned)mm - nn * (unsigned)OHW;
+            if (c < 4)
             {
-                const int64_t gi = ((int64_t)anc * OHW + (int64_t)h * g.OW + w) * 2 + c;
-                v = (t + (gi < g.det_grid_elems ? g.det_grid[gi] : 0.0f)) * g.det_stride;
+                const int h = (int)odl::fastdiv(px, g.d_ow), w = (int)px - h * g.OW;
+                const float t = v * 2.0f;
+                if (c < 2)
+                {
+                    const int64_t gi = ((int64_t)anc * OHW + px) * 2 + c;
+                    v = (t + (gi < g.det_grid_elems ? g.det_grid[gi] : 0.0f)) * g.det_stride;
+                }
+                else
+                {
+                    int ah = h / sh_, aw = w / sw_;
+                    ah = ah < g.det_aH - 1 ? ah : g.det_aH - 1;
+                    aw = aw < g.det_aW - 1 ? aw : g.det_aW - 1;
+                    const int64_t ai = ((int64_t)anc * g.det_aH * g.det_aW + (int64_t)ah * g.det_aW + aw) * 2 + (c - 2);
+                    v = (t * t) * (ai < g.det_anchor_elems ? g.det_anchor[ai] : 1.0f);
+                }
             }
-            else
-            {
-                const int sh_ = (g.det_aH > 0 && g.OH > g.det_aH) ? g.OH / g.det_aH : 1;
-                const int sw_ = (g.det_aW > 0 && g.OW > g.det_aW) ? g.OW / g.det_aW : 1;
-                int ah = h / sh_, aw = w / sw_;
-                ah = ah < g.det_aH - 1 ? ah : g.det_aH - 1;
-                aw = aw < g.det_aW - 1 ? aw : g.det_aW - 1;
-                const int64_t ai = ((int64_t)anc * g.det_aH * g.det_aW + (int64_t)ah * g.det_aW + aw) * 2 + (c - 2);
-                v = (t * t) * (ai < g.det_anchor_elems ? g.det_anchor[ai] : 1.0f);
-            }
+            rows[(int64_t)nn * g.det_rows_bs + (int64_t)px * g.det_CI] = v;
         }
-        g.det_rows[(int64_t)nn * g.det_rows_bs + ((int64_t)anc * OHW + px) * g.det_CI + c] = v;
     }
 }
 
