@@ -143,12 +143,13 @@ void parse_line(const std::string &line, PNNXNode &node)
     }
 }
 
-std::shared_ptr<Mat> upload(Attribute &a, const Device &dev, const std::string &who)
+// (the weight's name is put together only for the error message: this runs for every weight of every node of every forward)
+std::shared_ptr<Mat> upload(Attribute &a, const Device &dev, const std::string &node_name, const char *key)
 {
     if (a.device_mat && a.device_mat->device() == dev)
         return a.device_mat;
     if (a.data.empty() || a.shape.empty())
-        THROW_RUNTIME_ERROR("PNNX: weight {} has no data (missing from the bin archive?)", who);
+        THROW_RUNTIME_ERROR("PNNX: weight {}.{} has no data (missing from the bin archive?)", node_name, key);
     std::vector<size_t> dims(a.shape.begin(), a.shape.end());
     a.device_mat = OriginMat::from_memory(a.data.data(), DataType::kFloat32, Shape(dims),
                                           TensorOptions(DataType::kFloat32).device(dev));
@@ -698,9 +699,9 @@ void PNNXGraph::run_conv(PNNXNode &node)
     auto wit = node.attributes.find("weight");
     if (wit == node.attributes.end())
         THROW_RUNTIME_ERROR("PNNX: node {} has no weight", node.name);
-    auto w = upload(wit->second, dev, node.name + ".weight");
+    auto w = upload(wit->second, dev, node.name, "weight");
     auto bit = node.attributes.find("bias");
-    std::shared_ptr<Mat> b = bit == node.attributes.end() ? nullptr : upload(bit->second, dev, node.name + ".bias");
+    std::shared_ptr<Mat> b = bit == node.attributes.end() ? nullptr : upload(bit->second, dev, node.name, "bias");
     const auto stride = node.stride, padding = node.padding;
     const Shape s0 = first.mat->shape();
     const Shape xs = (first.run && s0.size() == 4) ? Shape{s0[0], first.channels, s0[2], s0[3]} : s0;
@@ -712,7 +713,7 @@ void PNNXGraph::run_conv(PNNXNode &node)
     {
         PNNXNode &other = *by_name_.at(node.pair_with);
         auto owit = other.attributes.find("weight");
-        auto ow = upload(owit->second, dev, other.name + ".weight");
+        auto ow = upload(owit->second, dev, other.name, "weight");
         const Shape ows = ow->shape();
         const Shape both{ws[0] + ows[0], ws[1], ws[2], ws[3]};
         if (fusion_ && f32 && xs.size() == 4 && OriginMat::conv2d_fused_ok(xs, both, stride, padding))
@@ -724,7 +725,7 @@ void PNNXGraph::run_conv(PNNXNode &node)
                 pw.packed_for.clear();
                 if (b)
                 {
-                    auto ob = upload(other.attributes.find("bias")->second, dev, other.name + ".bias");
+                    auto ob = upload(other.attributes.find("bias")->second, dev, other.name, "bias");
                     node.attributes["pair.bias"].device_mat = b->cat({ob.get()}, 0);
                 }
             }
@@ -794,7 +795,7 @@ void PNNXGraph::run(PNNXNode &node)
         auto it = node.attributes.find(key);
         if (it == node.attributes.end())
             return nullptr;
-        return upload(it->second, dev, node.name + "." + key);
+        return upload(it->second, dev, node.name, key.c_str());
     };
     auto run_of = [&](const Value &v) {
         return v.run ? OriginMat::ChannelRun{&origin_of(*v.mat), v.c0, v.channels} : OriginMat::whole(*v.mat);
