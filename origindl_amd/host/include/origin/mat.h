@@ -386,12 +386,6 @@ public:
     static void conv2d_fused_pair(const ChannelRun &x, const Mat &packed, const Shape &w_shape, const Mat *b,
                                   std::pair<int, int> stride, std::pair<int, int> pad, int activation, const ChannelRun &y_first,
                                   const ChannelRun &y_second);
-    // one to four 1x1 convolutions (stride 1, no padding) of independent inputs as one launch, each with the floats of
-    // its own conv2d_fused call; a bias may be null. group_ok: whether the member shapes are covered
-    static bool conv2d_fused_group_ok(const std::vector<Shape> &x_run_shapes, const std::vector<Shape> &w_shapes);
-    static void conv2d_fused_group(const std::vector<ChannelRun> &x, const std::vector<const Mat *> &packed,
-                                   const std::vector<Shape> &w_shapes, const std::vector<const Mat *> &b, int activation,
-                                   const std::vector<ChannelRun> &y);
     static void upsample_run(const ChannelRun &x, const ChannelRun &y, int scale_h, int scale_w);
     // y's channels [(j-1)*C, j*C) = the K x K / stride 1 / padding K/2 max pool applied j times to x, j = 1..count
     static void max_pool_chain(const ChannelRun &x, int K, int count, const ChannelRun &y);

@@ -1404,61 +1404,6 @@ void OriginMat::conv2d_fused(const ChannelRun &xr, const Mat &packed_m, const Sh
                                p.second, activation, res, res_stride, y.data, y.image_stride, cur()));
 }
 
-bool OriginMat::conv2d_fused_group_ok(const std::vector<Shape> &xs, const std::vector<Shape> &ws)
-{
-    const size_t S = xs.size();
-    if (S == 0 || S > 4 || ws.size() != S)
-        return false;
-    int64_t C[4], H[4], W[4], OC[4];
-    for (size_t s = 0; s < S; ++s)
-    {
-        if (xs[s].size() != 4 || ws[s].size() != 4 || xs[s][1] != ws[s][1] || ws[s][2] != 1 || ws[s][3] != 1 || xs[s][0] != xs[0][0])
-            return false;
-        C[s] = xs[s][1], H[s] = xs[s][2], W[s] = xs[s][3], OC[s] = ws[s][0];
-    }
-    return odl_hip_conv2d_fused_group_ok((int)S, (int64_t)xs[0][0], C, H, W, OC) == 1;
-}
-
-void OriginMat::conv2d_fused_group(const std::vector<ChannelRun> &xr, const std::vector<const Mat *> &packed,
-                                   const std::vector<Shape> &ws, const std::vector<const Mat *> &bm, int activation,
-                                   const std::vector<ChannelRun> &yr)
-{
-    const size_t S = xr.size();
-    if (S == 0 || S > 4 || packed.size() != S || ws.size() != S || bm.size() != S || yr.size() != S)
-        THROW_INVALID_ARG("conv2d: a group has 1 to 4 members with a filter copy, a filter shape, a bias (or null) and an output each");
-    const float *xp[4], *pp[4], *bp[4];
-    float *yp[4];
-    int64_t xs[4], ys[4], C[4], H[4], W[4], OC[4], N = 0;
-    for (size_t s = 0; s < S; ++s)
-    {
-        const RunPtr x = run_ptr(xr[s], "conv2d"), y = run_ptr(yr[s], "conv2d");
-        if (ws[s].size() != 4 || (int64_t)ws[s][1] != x.C || (int64_t)ws[s][0] != y.C || ws[s][2] != 1 || ws[s][3] != 1)
-            THROW_INVALID_ARG("conv2d: filter {} is not a 1x1 filter that maps {} channels to {}", ws[s].to_string(), x.C, y.C);
-        if (s == 0)
-            N = x.N;
-        if (x.N != N || y.N != N || y.H != x.H || y.W != x.W)
-            THROW_INVALID_ARG("conv2d: the output run is [{}, {}, {}, {}], the convolution gives [{}, {}, {}, {}]", y.N, y.C, y.H, y.W, N,
-                              y.C, x.H, x.W);
-        if (!packed[s])
-            THROW_INVALID_ARG("conv2d: member {} has no filter copy", s);
-        const OriginMat &pk = dev_f32(*packed[s], "conv2d");
-        const size_t want = odl_hip_conv2d_packed_weights_bytes(x.N, x.C, x.H, x.W, y.C, 1, 1, 1, 1, 0, 0);
-        if (pk.elements() * sizeof(float) != want)
-            THROW_INVALID_ARG("conv2d: the packed filter has {} bytes, this shape's kernel reads {}", pk.elements() * sizeof(float), want);
-        bp[s] = nullptr;
-        if (bm[s])
-        {
-            const OriginMat &b = dev_f32(*bm[s], "conv2d");
-            if (b.shape().size() != 1 || (int64_t)b.shape()[0] != y.C)
-                THROW_INVALID_ARG("conv2d: b must be 1D with size {}, but got shape {}", y.C, b.shape().to_string());
-            bp[s] = fp(b);
-        }
-        xp[s] = x.data, pp[s] = fp(pk), yp[s] = y.data, xs[s] = x.image_stride, ys[s] = y.image_stride;
-        C[s] = x.C, H[s] = x.H, W[s] = x.W, OC[s] = y.C;
-    }
-    check(odl_hip_conv2d_fused_group((int)S, xp, xs, pp, bp, N, C, H, W, OC, activation, yp, ys, cur()));
-}
-
 void OriginMat::conv2d_fused_pair(const ChannelRun &xr, const Mat &packed_m, const Shape &ws, const Mat *bm, std::pair<int, int> s,
                                   std::pair<int, int> p, int activation, const ChannelRun &y1r, const ChannelRun &y2r)
 {

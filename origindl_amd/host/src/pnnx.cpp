@@ -998,36 +998,21 @@ void PNNXGraph::run(PNNXNode &node)
                 store(node, std::move(out));
                 return;
             }
-            if (packed_all && OriginMat::conv2d_fused_group_ok(xshapes, wshapes))
+            // (a head the one launch does not take: stage by stage, then one launch that decodes the three)
+            for (int s = 0; s < 3; ++s)
             {
-                // (the three convolutions do not depend on each other and each is a launch's latency long: one launch)
-                std::vector<OriginMat::ChannelRun> xr, yr;
-                std::vector<const Mat *> pk, bv;
-                for (int s = 0; s < 3; ++s)
+                Value &xv = value(node.input_names[s], node);
+                const Shape &xs = xshapes[s], &wsh = wshapes[s];
+                Attribute &wa = node.attributes.find("m." + std::to_string(s) + ".weight")->second;
+                if (wa.packed_mat && OriginMat::conv2d_fused_ok(xs, wsh, {1, 1}, {0, 0}))
                 {
-                    convs[s] = std::make_shared<OriginMat>(Shape{xshapes[s][0], wshapes[s][0], xshapes[s][2], xshapes[s][3]},
-                                                           DataType::kFloat32, dev);
-                    xr.push_back(run_of(value(node.input_names[s], node))), yr.push_back(OriginMat::whole(*convs[s]));
-                    pk.push_back(node.attributes.find("m." + std::to_string(s) + ".weight")->second.packed_mat.get());
-                    bv.push_back(bs[s].get());
+                    convs[s] = std::make_shared<OriginMat>(Shape{xs[0], wsh[0], xs[2], xs[3]}, DataType::kFloat32, dev);
+                    OriginMat::conv2d_fused(run_of(xv), *wa.packed_mat, wsh, bs[s].get(), {1, 1}, {0, 0}, -1, nullptr,
+                                            OriginMat::whole(*convs[s]));
                 }
-                OriginMat::conv2d_fused_group(xr, pk, wshapes, bv, -1, yr);
+                else
+                    convs[s] = origin_of(*dense(node.input_names[s], node)).conv2d_act(*ws[s], bs[s].get(), {1, 1}, {0, 0}, -1, wa.packed_mat.get());
             }
-            else
-                for (int s = 0; s < 3; ++s)
-                {
-                    Value &xv = value(node.input_names[s], node);
-                    const Shape &xs = xshapes[s], &wsh = wshapes[s];
-                    Attribute &wa = node.attributes.find("m." + std::to_string(s) + ".weight")->second;
-                    if (wa.packed_mat && OriginMat::conv2d_fused_ok(xs, wsh, {1, 1}, {0, 0}))
-                    {
-                        convs[s] = std::make_shared<OriginMat>(Shape{xs[0], wsh[0], xs[2], xs[3]}, DataType::kFloat32, dev);
-                        OriginMat::conv2d_fused(run_of(xv), *wa.packed_mat, wsh, bs[s].get(), {1, 1}, {0, 0}, -1, nullptr,
-                                                OriginMat::whole(*convs[s]));
-                    }
-                    else
-                        convs[s] = origin_of(*dense(node.input_names[s], node)).conv2d_act(*ws[s], bs[s].get(), {1, 1}, {0, 0}, -1, wa.packed_mat.get());
-                }
             // (one launch for the three stages: each is a chain of a load, sigmoids and a store, shorter than a launch)
             OriginMat::yolo_decode_stages_into({convs[0].get(), convs[1].get(), convs[2].get()}, {gs[0].get(), gs[1].get(), gs[2].get()},
                                                {ags[0].get(), ags[1].get(), ags[2].get()}, strides, 3, (int)ci - 5, *out);

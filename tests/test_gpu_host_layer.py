@@ -690,6 +690,25 @@ def test_pnnx_runner_with_nodes_folded_together_gives_the_floats_of_running_them
         assert nodes[1] <= 70 and nodes[0] >= 85
 
 
+def test_pnnx_runner_head_too_large_for_one_launch_runs_stage_by_stage_with_the_same_floats(h, tmp_path):
+    """At 8 x 640x640 the first detect stage's convolution (51200 pixels, 64 -> 255 channels: 1.67 GFLOP) is past what
+    the small-problem kernel takes, so the head is not one launch: its stages run one after the other and one launch
+    decodes the three. Every node on its own (fusion off) runs the same convolution kernels: same floats."""
+    import pnnx_synth
+    param, binp, shp = pnnx_synth.write(str(tmp_path / "y5n640"), seed=5, batch=8, size=640, num_classes=80)
+    x = np.random.default_rng(640).random((8, 3, 640, 640), dtype=f32)
+    outs = {}
+    try:
+        for fusion in (1, 0):
+            assert h.odl_host_pnnx_set_fusion(fusion) == 0
+            rc, outs[fusion], _, _ = _run_pnnx(h, "odl_host_", param, binp, x, shp, reps=1)
+            assert rc == 0
+    finally:
+        h.odl_host_pnnx_set_fusion(1)
+    assert outs[1].shape == (8, 25200, 85) and np.isfinite(outs[1]).all()
+    assert np.array_equal(outs[1], outs[0])
+
+
 def test_pnnx_runner_rejects_bad_files(h, tmp_path):
     import pnnx_synth
     param, binp, shp = pnnx_synth.write(str(tmp_path / "y5n"), seed=1, batch=1, size=32, num_classes=3)
