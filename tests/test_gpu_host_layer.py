@@ -661,11 +661,11 @@ def test_float64_softmax_through_the_tensor_api(h):
 
 def test_pnnx_runner_with_nodes_folded_together_gives_the_floats_of_running_them_one_by_one(h, tmp_path):
     """The runner folds a residual add into the convolution before it, lets producers write straight into a
-    concatenation's output, runs SPPF's three pools as one launch and decodes each detect stage into its rows of the
-    final tensor. With all of that switched off every node runs on its own, as in the reference's runner
+    concatenation's output, runs SPPF's three pools as one launch and the detect head (three convolutions that decode
+    their own sums into their rows of the final tensor) as one launch. With all of that switched off every node runs on its own, as in the reference's runner
     (src/pnnx/pnnx_graph.cpp:286-528); the convolutions are the same kernels either way, so the outputs must agree bit
     for bit — at 64x64 (one image, planes down to 2x2) and at the benchmark's 4 x 320x320. The recorded forward holds
-    66 launches folded against 109 plain (57 + 3 convolutions either way)."""
+    53 launches folded against 92 plain."""
     import pnnx_synth
     for batch, size, seed in ((1, 64, 3), (4, 320, 0)):
         param, binp, shp = pnnx_synth.write(str(tmp_path / ("y5n%d" % size)), seed=seed, batch=batch, size=size, num_classes=80)
