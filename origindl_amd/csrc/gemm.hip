@@ -1238,6 +1238,10 @@ int pair_tile_class(bool vec, int64_t M, int64_t N, int64_t K)
         return 32;
     if (s2 == 1)  // (which already says: at most about one 64x64 tile per compute unit, K of 256 or more)
         return 64;
+    // a K of 128 to 255 on its own is not worth this variant's prologue; next to its partner in one launch it is worth
+    // the launch it saves (a hidden layer of 128 units: its input gradient)
+    if (K < 256 && tiles <= lone_workgroup_limit())
+        return 64;
     return 0;
 }
 
