@@ -198,7 +198,7 @@ def test_sum_to_reference_vectors():
     assert st(list(range(1, 9)), (2, 2, 2), (1, 1, 1)) == (0, [36])
     # test_sum_to.cpp:53-60: a larger target throws runtime_error
     assert st([1, 2], (2,), (2, 2))[0] == ol.ctypes.c_int(-2).value
-    # the survey's probe of the compiled reference: x{2} broadcast to {2,2}, gy=[[1,2],[3,4]] -> x.grad=[3,7]
+    # a probe of the compiled reference: x{2} broadcast to {2,2}, gy=[[1,2],[3,4]] -> x.grad=[3,7]
     assert st([1, 2, 3, 4], (2, 2), (2,)) == (0, [3, 7])
 
 
